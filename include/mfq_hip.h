@@ -1,0 +1,220 @@
+/*
+ * mfq_hip.h -- C ABI of the MI355X (gfx950) MFQ packed-weight matmul kernels.
+ *
+ * Every entry point is `extern "C"`, takes plain device pointers and sizes, returns an
+ * int status (0 = MFQ_OK) and launches on the stream it is given without synchronising.
+ * No entry point allocates device memory: weights are written into caller-owned buffers
+ * whose size comes from the *_plan call, and kernels that need scratch take a workspace
+ * pointer whose size comes from the matching *_workspace_bytes query.
+ * mfq_hip_last_error() returns a thread-local message for the last non-zero status.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the
+ * reference tree).  Activations are bf16 or fp16 row-major [M, ldx]; outputs are fp32
+ * row-major [M, ldy].
+ */
+#ifndef MFQ_HIP_H
+#define MFQ_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *mfq_stream_t; /* a hipStream_t; NULL = the default stream */
+
+enum { MFQ_OK = 0, MFQ_ERR_INVALID = 1, MFQ_ERR_UNSUPPORTED = 2, MFQ_ERR_LAUNCH = 3, MFQ_ERR_WORKSPACE = 4 };
+enum { MFQ_X_BF16 = 0, MFQ_X_F16 = 1 };
+
+const char *mfq_hip_last_error(void);
+int mfq_hip_version(void);
+
+/* ------------------------------------------------------------------------------------
+ * NINT (neuron-anchored INT).  Device layout: row-blocks of 16 neurons; inside a block
+ * the groups of a neuron are spread over 4 lanes, 4 groups per lane per 16-group step,
+ * each step stored lane-interleaved so one wave load covers a contiguous span.
+ * Replaces NintWeight + to_device_nint (cpp_runtime/mfq_decode.cpp:2101-2165, 2268-2293).
+ * ---------------------------------------------------------------------------------- */
+typedef struct mfq_nint_desc {
+    int32_t bits, sub_bits, gs, out, neuron_len, ng;
+    int32_t kind;       /* 1 = paired-field fast unit, 0 = natural-order generic unit */
+    int32_t dwords;     /* full dwords of codes per (neuron, group) unit */
+    int32_t tail_bytes; /* 0 or 1 extra byte per unit */
+    int32_t ngp;        /* groups per neuron padded to a multiple of 16 */
+    int32_t nsteps;     /* ngp / 16 */
+    int32_t n_rowblocks;
+    int64_t step_bytes;     /* bytes of one 16-group step of one row-block */
+    int64_t rowblock_bytes; /* nsteps * step_bytes */
+    int64_t anchors_off;    /* float ns[16*n_rowblocks] then float nm[16*n_rowblocks] */
+    int64_t total_bytes;
+    int64_t payload_bytes;  /* compact MFQ payload (anchors + 3 bit streams), for GB/s accounting */
+} mfq_nint_desc;
+
+/* Fills `d` for a tensor of `out` neurons of length `neuron_len`. */
+int mfq_hip_nint_plan(int bits, int sub_bits, int gs, int out, int neuron_len, mfq_nint_desc *d);
+
+/* Load-time repack: `payload` is the device copy of the NINT blob body as pack_nint wrote
+ * it (mfq/formats/io.py:191-203) after the header: ns f16[out], nm f16[out], then the
+ * sub_scale, sub_min and q little-endian bit streams.  `legacy_bytes` != 0 selects the
+ * one-byte-per-value tail accepted by unpack_nint (mfq/formats/io.py:223-232). */
+int mfq_hip_nint_repack(const mfq_nint_desc *d, const void *payload, int64_t payload_bytes,
+                        int legacy_bytes, void *weight, mfq_stream_t stream);
+
+/* Bit-exact CPU-dequantizer twin: W[out, neuron_len] fp32 with the four separate roundings
+ * of nint_quant.dequantize (mfq/quantize/nint_quant.py:896-908); replaces
+ * nint_dequant_full_packed_compact_bits_cuda (cpp_runtime/mfq_decode.cpp:396-404). */
+int mfq_hip_nint_dequant_f32(const mfq_nint_desc *d, const void *weight, float *w_out, int64_t ld,
+                             mfq_stream_t stream);
+
+/* y[M, out] = x[M, neuron_len] . W^T, fp32 accumulate, for small M (decode).  Replaces
+ * nint_gemv_packed_ws_cuda / nint_gemv_packed_bits_ws_cuda (cpp_runtime/mfq_decode.cpp:421-435). */
+int mfq_hip_nint_gemv(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
+                      int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream);
+
+/* Prefill / large-M path (MFMA).  Replaces nint_mmq_f16_packed_cuda / nint_mmq_f32_packed_cuda
+ * and the dequant + cuBLAS fallback (cpp_runtime/mfq_decode.cpp:480-520, 8309-8314). */
+size_t mfq_hip_nint_gemm_workspace_bytes(const mfq_nint_desc *d, int M);
+int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
+                      int64_t ldx, int M, float *y, int64_t ldy, void *workspace,
+                      size_t workspace_bytes, mfq_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * NVQ-JSC, D4 family (NVQ3J = d4_256, NVQ3J-512 = d4_512; plain NVQ3 maps onto the
+ * analytic one-bank tables).  Replaces NvqWeight + to_device_nvq
+ * (cpp_runtime/mfq_decode.cpp:4019-4150).
+ * ---------------------------------------------------------------------------------- */
+typedef struct mfq_nvq_desc {
+    int32_t index_bits, entries, banks, out, neuron_len, ng, nvec, nsign;
+    int32_t ngp, nsteps, n_rowblocks;
+    int64_t step_bytes, rowblock_bytes;
+    int64_t tables_off;  /* float lut[16]; uint32 bank_for_state[16]; uint8 codebooks[banks*entries*4] */
+    int64_t anchors_off; /* float anchor[16*n_rowblocks] */
+    int64_t total_bytes;
+    int64_t payload_bytes; /* anchors + 3 streams + 64-byte JSC header + codebook banks */
+} mfq_nvq_desc;
+
+int mfq_hip_nvq_plan(int index_bits, int banks, int out, int neuron_len, mfq_nvq_desc *d);
+
+/* `payload` = device copy of the blob from the 64-byte JSC header on (mfq/formats/nvq.py:644-716):
+ * JSC header, codebook banks i8[banks, entries, 4], anchors f16[out], then the 4-bit state,
+ * index_bits-bit index and 7-bit sign streams, all tensor-contiguous. */
+int mfq_hip_nvq_repack(const mfq_nvq_desc *d, const void *payload, int64_t payload_bytes, void *weight,
+                       mfq_stream_t stream);
+/* Plain (non-JSC) NVQ3: payload starts at the anchors; `grid` is the device copy of the
+ * 256-entry int8 magnitude grid [256, 4]; state doubles as the integer relative scale. */
+int mfq_hip_nvq_repack_plain(const mfq_nvq_desc *d, const void *payload, int64_t payload_bytes,
+                             const void *grid, void *weight, mfq_stream_t stream);
+
+/* Bit-exact twin of dequantize_nvq_jsc (mfq/quantize/nvq_jsc.py:1053-1079); replaces
+ * nvq_dequant_cuda (cpp_runtime/mfq_decode.cpp:540-546). */
+int mfq_hip_nvq_dequant_f32(const mfq_nvq_desc *d, const void *weight, float *w_out, int64_t ld,
+                            mfq_stream_t stream);
+/* Replaces nvq_gemv_ws_cuda (cpp_runtime/mfq_decode.cpp:555-559). */
+int mfq_hip_nvq_gemv(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                     int M, float *y, int64_t ldy, mfq_stream_t stream);
+/* Replaces nvq_gemm_f16_cuda / dequant + cuBLAS (cpp_runtime/mfq_decode.cpp:561-575, 7928-7931). */
+size_t mfq_hip_nvq_gemm_workspace_bytes(const mfq_nvq_desc *d, int M);
+int mfq_hip_nvq_gemm(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                     int M, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                     mfq_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * NEPQ1-S / NEPQ1-L (cross-expert table pool, bank id per 96 weights).  Rows are the
+ * flattened [experts * out_per_expert] neurons.  Replaces NepqWeight
+ * (cpp_runtime/mfq_decode.cpp:4166-4463) and the Python nepq_matmul
+ * (mfq/kernels/cuda/nepq_matmul.py:215-280).
+ * ---------------------------------------------------------------------------------- */
+typedef struct mfq_nepq_desc {
+    int32_t profile; /* 2 = NEPQ1-S, 3 = NEPQ1-L */
+    int32_t state_bits, index_bits, banks, rows, neuron_len, ng, nvec, nsuper;
+    int32_t ngp, nsteps, n_rowblocks, table_entries; /* u16 entries per bank: 1024 (S) / 2048 (L) */
+    int64_t step_bytes, rowblock_bytes;
+    int64_t tables_off;  /* uint16 table[banks * table_entries] */
+    int64_t anchors_off; /* float anchor[16*n_rowblocks] */
+    int64_t total_bytes;
+    int64_t payload_bytes;
+} mfq_nepq_desc;
+
+int mfq_hip_nepq_plan(int profile, int banks, int rows, int neuron_len, mfq_nepq_desc *d);
+/* `payload` = device copy of the blob after the 40-byte header (mfq/formats/nepq.py:368-399):
+ * tables u8[banks, table_bytes], anchors f16[rows], state / index / aux bit streams, bank ids. */
+int mfq_hip_nepq_repack(const mfq_nepq_desc *d, const void *payload, int64_t payload_bytes, void *weight,
+                        mfq_stream_t stream);
+/* Bit-exact twin of dequantize_nepq (mfq/formats/nepq.py:492-544); replaces nepq_dequant_cuda. */
+int mfq_hip_nepq_dequant_f32(const mfq_nepq_desc *d, const void *weight, float *w_out, int64_t ld,
+                             mfq_stream_t stream);
+/* `row0`, `nrows` select one expert's neurons; replaces nepq_gemv_ws_cuda. */
+int mfq_hip_nepq_gemv(const mfq_nepq_desc *d, const void *weight, int row0, int nrows, const void *x,
+                      int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream);
+size_t mfq_hip_nepq_gemm_workspace_bytes(const mfq_nepq_desc *d, int nrows, int M);
+int mfq_hip_nepq_gemm(const mfq_nepq_desc *d, const void *weight, int row0, int nrows, const void *x,
+                      int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, void *workspace,
+                      size_t workspace_bytes, mfq_stream_t stream);
+/* x <- FWHT_block(x * signs) / sqrt(block), fp32 in LDS; replaces nepq_hadamard_input_cuda
+ * (mfq/kernels/cuda/nepq.cu:13-55).  `signs` int8[K] (+1/-1), block a power of two <= 4096. */
+int mfq_hip_nepq_hadamard(const void *x, int x_dtype, int64_t ldx, int rows, int K, int block,
+                          const int8_t *signs, void *x_out, int64_t ldo, mfq_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * MoE routing and the expert-grouped matmul ("mul_mat_id").
+ * ---------------------------------------------------------------------------------- */
+enum { MFQ_TOPK_SOFTMAX = 0, MFQ_TOPK_SIGMOID = 1, MFQ_TOPK_SQRT_SOFTPLUS = 2, MFQ_TOPK_DELAYED_SOFTMAX = 3 };
+
+/* Replaces moe_topk_cuda (mfq/kernels/cuda/moe.cu:3552-3637): ids int32[T,k], weights f32[T,k];
+ * tie -> lower expert id, NaN -> -FLT_MAX, bias (may be NULL) enters the selection score only. */
+int mfq_hip_moe_topk(const float *logits, const float *bias, int T, int E, int k, int mode, int normalize,
+                     float norm_floor, float scale, int32_t *ids, float *weights, mfq_stream_t stream);
+
+/* Replaces moe_build_expert_map_cuda (mfq/kernels/cuda/moe.cu:3082-3130) with a parallel
+ * prefix-sum bucketing.  counts[E], expert_bounds[E+1], tile_bounds[E+1], tile_experts[max_tiles],
+ * ids_dst[n_pairs] (pairs grouped by expert, ascending pair index inside an expert: deterministic).
+ * max_tiles >= ceil(n_pairs/tile_m) + E.  Pairs with an out-of-range expert id are dropped. */
+int mfq_hip_moe_route_map(const int32_t *ids, int n_pairs, int E, int tile_m, int32_t *counts,
+                          int32_t *expert_bounds, int32_t *tile_bounds, int32_t *tile_experts,
+                          int max_tiles, int32_t *ids_dst, mfq_stream_t stream);
+
+/* One cohort of experts sharing a NINT profile (NintMoePoolWeight,
+ * cpp_runtime/mfq_decode.cpp:2350-2365): `weight` holds n_local * out_per_expert neurons. */
+typedef struct mfq_moe_pool {
+    mfq_nint_desc desc;
+    const void *weight;
+} mfq_moe_pool;
+
+/* Device tables built once per NINTM tensor (initialize_nint_moe_dispatch,
+ * cpp_runtime/mfq_decode.cpp:3249-3343): expert_pool[E], expert_local[E] (int32, -1 = absent). */
+/* out[pair, :] = x[src(pair), :] . W[ids[pair]]^T for every (token, route) pair; src = pair when
+ * routed_input != 0 (x is [T*R, K]) else pair / R (x is [T, K]).  Invalid expert ids give zero rows.
+ * Replaces nint_moe_grouped_matmul_hetero_qx_cuda / _hetero_f16_cuda / _pool_ws_cuda
+ * (cpp_runtime/mfq_decode.cpp:248-290; mfq/kernels/cuda/moe.cu:3971-4345). */
+size_t mfq_hip_moe_grouped_workspace_bytes(int n_pairs, int K, int out_per_expert);
+int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools, const int32_t *expert_pool,
+                               const int32_t *expert_local, int E, int out_per_expert, int K,
+                               const void *x, int x_dtype, int64_t ldx, int routed_input,
+                               const int32_t *ids, int T, int R,
+                               const int32_t *ids_dst, const int32_t *expert_bounds, /* NULL when T*R small */
+                               float *out, int64_t ldo, void *workspace, size_t workspace_bytes,
+                               mfq_stream_t stream);
+
+/* hidden[r, c] = silu(gate_up[r, c]) * gate_up[r, W + c]  (moe_swiglu_split_cuda,
+ * mfq/kernels/cuda/moe.cu:2980-2996); output fp16 (x_dtype MFQ_X_F16) or bf16. */
+int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,
+                       int64_t ldh, mfq_stream_t stream);
+/* out[t, :] = sum_r w[t, r] * pair[t, r, :] (+ shared[t, :] when shared != NULL; ungated add,
+ * cpp_runtime/mfq_decode.cpp:11077-11080; with gate_logits != NULL: + sigmoid(gate_logits[t]) * shared).
+ * Replaces moe_weighted_reduce_cuda / moe_weighted_reduce_shared_gate_cuda. */
+int mfq_hip_moe_weighted_reduce(const float *pair, const float *weights, int T, int R, int H,
+                                const float *shared, const float *gate_logits, float *out,
+                                mfq_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * helpers shared by the GEMM paths
+ * ---------------------------------------------------------------------------------- */
+/* Plain fp16 x fp16 -> fp32 MFMA GEMM: y[M, N] = a[M, K] . b[N, K]^T (used after a full dequant). */
+int mfq_hip_gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K,
+                        float *y, int64_t ldy, mfq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MFQ_HIP_H */

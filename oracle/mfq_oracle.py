@@ -1,0 +1,930 @@
+"""CPU oracle for the MFQ packed-weight matmul path  --  TEST INFRASTRUCTURE ONLY.
+
+This module restates, in plain numpy, the reference's CPU algorithm for the hot
+path: the MFQ payload codecs, the CPU dequantizers, the fp32
+dequant-then-matmul linear, and the MoE routing / grouped-matmul reference loop.
+Nothing in the shipped product imports it: only tests/, __graft_entry__.smoke()
+and bench.py's cpu_baseline leg may.  It never touches a GPU.
+
+Each function cites the reference file:line it follows (paths relative to the
+reference tree).  Parity status of each function:
+
+  pinned (closed form / reference constants / brute force, see tests/test_oracle_*.py)
+    pack_bits / unpack_bits        mfq/formats/io.py:144-188, mfq/formats/nvq.py:556-581
+    pack_nint / unpack_nint        mfq/formats/io.py:191-248
+    dequantize_nint                mfq/quantize/nint_quant.py:896-908
+    pack_nvq_jsc / unpack_nvq      mfq/formats/nvq.py:586-820
+    dequantize_nvq_jsc             mfq/quantize/nvq_jsc.py:1053-1079
+    dequantize_nvq                 mfq/quantize/nvq_quant.py:591-626
+    pack_nepq / unpack_nepq        mfq/formats/nepq.py:368-474
+    dequantize_nepq (NEPQ1-S/L)    mfq/formats/nepq.py:492-544
+    pack_nint_moe / unpack_nint_moe  mfq/formats/io.py:251-446
+    dequantize_expertwise          mfq/quantize/expert_nint.py:605-615
+    linear_forward                 mfq/runtime/linear.py:37-42
+    moe_topk                       mfq/kernels/cuda/moe.cu:124-263
+    build_expert_map               mfq/kernels/cuda/moe.cu:472-542
+    moe_grouped_matmul / moe_ffn   tests/test_moe_kernels_cuda.py:58-68, cpp_runtime/mfq_decode.cpp:3394-3416
+    mfq_file_write / mfq_file_read mfq/formats/io.py:646-685
+
+  pinned by golden vectors written from the reference's own numpy quantizer
+  (tests/golden/nint_quant_vectors.npz, made by tests/golden/make_nint_quant_vectors.py)
+    make_qkx2 / quantize_nint      mfq/formats/nint.py:119-174, mfq/quantize/nint_quant.py:745-893
+    (weight-only branch, importance=None)
+"""
+from __future__ import annotations
+
+import math
+import struct
+from dataclasses import dataclass, field
+from pathlib import Path
+
+import numpy as np
+
+_DATA = Path(__file__).resolve().parents[1] / "tyloquant_amd" / "data"
+
+
+# ---------------------------------------------------------------------------
+# bit streams  (mfq/formats/io.py:144-188; mfq/formats/nvq.py:556-581;
+#               mfq/formats/nepq.py:217-255)
+# ---------------------------------------------------------------------------
+def pack_bits(values, bits: int) -> bytes:
+    """Little-endian bit stream: value i occupies bits [i*bits, (i+1)*bits)."""
+    v = np.ascontiguousarray(values).reshape(-1).astype(np.uint32)
+    if bits == 0:
+        return b""
+    if bits == 8:
+        return v.astype(np.uint8).tobytes()
+    shifts = np.arange(bits, dtype=np.uint32)
+    stream = ((v[:, None] >> shifts[None, :]) & 1).astype(np.uint8).reshape(-1)
+    return np.packbits(stream, bitorder="little").tobytes()
+
+
+def unpack_bits(blob, off: int, count: int, bits: int):
+    if bits == 0 or count == 0:
+        return np.empty(0, dtype=np.uint8), off + ((count * bits + 7) // 8 if bits else 0)
+    nbytes = (count * bits + 7) // 8
+    if off + nbytes > len(blob):
+        raise ValueError("truncated bit stream")
+    packed = np.frombuffer(blob, dtype=np.uint8, count=nbytes, offset=off)
+    stream = np.unpackbits(packed, bitorder="little")[: count * bits].reshape(count, bits)
+    weights = (1 << np.arange(bits, dtype=np.uint32))
+    out = (stream.astype(np.uint32) * weights).sum(axis=1)
+    return out.astype(np.uint8 if bits <= 8 else np.uint16), off + nbytes
+
+
+def _f16_round(x):
+    return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
+# ---------------------------------------------------------------------------
+# NINT  (mfq/formats/nint.py, mfq/quantize/nint_quant.py, mfq/formats/io.py:191-248)
+# ---------------------------------------------------------------------------
+@dataclass
+class NintTensor:
+    bits: int
+    groupsize: int
+    sub_bits: int
+    shape: tuple
+    axis: int
+    neuron_len: int
+    q: np.ndarray             # (out, ng, gs) uint8
+    neuron_scale: np.ndarray  # (out,) f32 (f16-representable)
+    neuron_min: np.ndarray    # (out,) f32
+    sub_scale: np.ndarray     # (out, ng) uint8
+    sub_min: np.ndarray       # (out, ng) uint8
+
+    @property
+    def out(self):
+        return self.q.shape[0]
+
+    @property
+    def ng(self):
+        return self.q.shape[1]
+
+
+_NINT_HDR = struct.Struct("<BBiii")
+
+
+def nint_payload_nbytes(out, neuron_len, bits, gs, sub_bits):
+    """Compact payload bytes without the blob header (mfq/formats/io.py:191-203)."""
+    ng = -(-neuron_len // gs)
+    return 4 * out + 2 * ((out * ng * sub_bits + 7) // 8) + (out * ng * gs * bits + 7) // 8
+
+
+def pack_nint(t: NintTensor) -> bytes:
+    """mfq/formats/io.py:191-203."""
+    out, ng, _ = t.q.shape
+    parts = [_NINT_HDR.pack(t.bits, t.sub_bits, t.groupsize, t.axis, t.neuron_len),
+             struct.pack("<I", len(t.shape)), struct.pack(f"<{len(t.shape)}q", *t.shape),
+             struct.pack("<II", out, ng),
+             np.ascontiguousarray(t.neuron_scale, dtype=np.float16).tobytes(),
+             np.ascontiguousarray(t.neuron_min, dtype=np.float16).tobytes(),
+             pack_bits(t.sub_scale, t.sub_bits), pack_bits(t.sub_min, t.sub_bits),
+             pack_bits(t.q, t.bits)]
+    return b"".join(parts)
+
+
+def unpack_nint(blob) -> NintTensor:
+    """mfq/formats/io.py:206-248 (bit-stream tail and the legacy one-byte-per-value tail)."""
+    blob = bytes(blob)
+    bits, sub_bits, gs, axis, neuron_len = _NINT_HDR.unpack_from(blob, 0)
+    off = _NINT_HDR.size
+    ndim = struct.unpack_from("<I", blob, off)[0]
+    off += 4
+    shape = struct.unpack_from(f"<{ndim}q", blob, off)
+    off += 8 * ndim
+    out, ng = struct.unpack_from("<II", blob, off)
+    off += 8
+    ns = np.frombuffer(blob, dtype=np.float16, count=out, offset=off).astype(np.float32)
+    off += 2 * out
+    nm = np.frombuffer(blob, dtype=np.float16, count=out, offset=off).astype(np.float32)
+    off += 2 * out
+    sub_count, q_count = out * ng, out * ng * gs
+    packed_tail = ((sub_count * sub_bits + 7) // 8) * 2 + (q_count * bits + 7) // 8
+    old_tail = sub_count * 2 + q_count
+    remaining = len(blob) - off
+    if remaining == old_tail and bits <= 8 and sub_bits <= 8:
+        ss = np.frombuffer(blob, dtype=np.uint8, count=sub_count, offset=off).copy()
+        off += sub_count
+        sm = np.frombuffer(blob, dtype=np.uint8, count=sub_count, offset=off).copy()
+        off += sub_count
+        q = np.frombuffer(blob, dtype=np.uint8, count=q_count, offset=off).copy()
+    else:
+        if remaining != packed_tail:
+            raise ValueError(f"invalid NINT blob tail: remaining={remaining}, packed={packed_tail}, old={old_tail}")
+        ss, off = unpack_bits(blob, off, sub_count, sub_bits)
+        sm, off = unpack_bits(blob, off, sub_count, sub_bits)
+        q, off = unpack_bits(blob, off, q_count, bits)
+    return NintTensor(bits, gs, sub_bits, tuple(shape), axis, neuron_len,
+                      q.reshape(out, ng, gs), ns, nm, ss.reshape(out, ng), sm.reshape(out, ng))
+
+
+def dequantize_nint(t: NintTensor) -> np.ndarray:
+    """mfq/quantize/nint_quant.py:896-908: four separate fp32 roundings, no FMA."""
+    out, ng, gs = t.q.shape
+    q = t.q.astype(np.float32)
+    d_eff = t.neuron_scale.astype(np.float32)[:, None] * t.sub_scale.astype(np.float32)
+    m_eff = t.neuron_min.astype(np.float32)[:, None] * t.sub_min.astype(np.float32)
+    recon = d_eff[..., None] * q - m_eff[..., None]
+    return np.ascontiguousarray(recon.reshape(out, ng * gs)[:, : t.neuron_len])
+
+
+def make_qkx2(x, w, nmax=15):
+    """mfq/formats/nint.py:119-174 (weighted LS search of (scale, zp) per group)."""
+    nmax = int(nmax)
+    rmin, rdelta, nstep = (-1.0, 0.1, 20) if nmax <= 15 else (-0.5, 0.1, 15)
+    mn = np.minimum(x.min(-1), 0.0)
+    mx = x.max(-1)
+    sum_w = w.sum(-1)
+    sum_x = (w * x).sum(-1)
+    degen = (mx == mn) | (sum_w <= 0)
+    rng = np.where(degen, 1.0, mx - mn)
+    iscale0 = nmax / rng
+    scale0 = 1.0 / iscale0
+    L0 = np.clip(np.rint(iscale0[..., None] * (x - mn[..., None])), 0, nmax).astype(np.int32)
+    diff = scale0[..., None] * L0 + mn[..., None] - x
+    best_err = (w * diff * diff).sum(-1)
+    best_scale = scale0.copy()
+    best_min = mn.copy()
+    for is_ in range(nstep + 1):
+        iscale = (rmin + rdelta * is_ + nmax) / rng
+        Laux = np.clip(np.rint(iscale[..., None] * (x - mn[..., None])), 0, nmax).astype(np.int32)
+        Laf = Laux.astype(np.float32)
+        sl = (w * Laf).sum(-1)
+        sl2 = (w * Laf * Laf).sum(-1)
+        sxl = (w * Laf * x).sum(-1)
+        D = sum_w * sl2 - sl * sl
+        valid = D > 0
+        Ds = np.where(valid, D, 1.0)
+        ts = (sum_w * sxl - sum_x * sl) / Ds
+        tm = (sl2 * sum_x - sl * sxl) / Ds
+        pos = tm > 0
+        sl2s = np.where(sl2 > 0, sl2, 1.0)
+        ts = np.where(pos, sxl / sl2s, ts)
+        tm = np.where(pos, 0.0, tm)
+        cd = ts[..., None] * Laux + tm[..., None] - x
+        ce = (w * cd * cd).sum(-1)
+        better = valid & (ce < best_err)
+        best_err = np.where(better, ce, best_err)
+        best_scale = np.where(better, ts, best_scale)
+        best_min = np.where(better, tm, best_min)
+    best_scale = np.where(degen, 0.0, best_scale)
+    best_min = np.where(degen, np.minimum(mn, 0.0), best_min)
+    return best_scale.astype(np.float32), best_min.astype(np.float32)
+
+
+def quantize_nint(weight, bits=4, gs=24, sub_bits=6) -> NintTensor:
+    """mfq/quantize/nint_quant.py:745-823, 883-893 (weight-only branch, axis=0, rank 2)."""
+    bits, gs, sub_bits = int(bits), int(gs), int(sub_bits)   # numpy ints would promote to fp64
+    W = np.asarray(weight, dtype=np.float32)
+    out, neuron_len = W.shape
+    nmax = (1 << bits) - 1
+    K = (1 << sub_bits) - 1
+    W2 = W.copy()
+    pad = (-neuron_len) % gs
+    if pad:
+        W2 = np.concatenate([W2, np.zeros((out, pad), dtype=np.float32)], axis=1)
+    ng = W2.shape[1] // gs
+    grps = W2.reshape(out, ng, gs)
+    sx2 = (grps * grps).sum(-1)
+    av = np.sqrt(sx2 / gs)
+    w = av[..., None] + np.abs(grps)
+    if pad:
+        w[:, -1, gs - pad:] = 0.0
+    scale, zp = make_qkx2(grps, w, nmax=nmax)
+    the_min = -zp
+    neu_s = scale.max(-1)
+    neu_m = the_min.max(-1)
+    neu_d = np.where(neu_s > 0, (neu_s / K).astype(np.float16).astype(np.float32), np.float32(0.0))
+    neu_dm = np.where(neu_m > 0, (neu_m / K).astype(np.float16).astype(np.float32), np.float32(0.0))
+    nss = np.where(neu_s > 0, neu_s, 1.0)
+    nmm = np.where(neu_m > 0, neu_m, 1.0)
+    sub_scale = np.clip(np.rint(K * scale / nss[..., None]), 0, K)
+    sub_min = np.clip(np.rint(K * the_min / nmm[..., None]), 0, K)
+    d_eff = neu_d[:, None] * sub_scale.astype(np.float32)
+    m_eff = neu_dm[:, None] * sub_min.astype(np.float32)
+    de = np.where(d_eff > 0, d_eff, 1.0)
+    q = np.clip(np.rint((grps + m_eff[..., None]) / de[..., None]), 0, nmax)
+    return NintTensor(bits, gs, sub_bits, (out, neuron_len), 0, neuron_len, q.astype(np.uint8),
+                      neu_d.astype(np.float32), neu_dm.astype(np.float32),
+                      sub_scale.astype(np.uint8), sub_min.astype(np.uint8))
+
+
+# ---------------------------------------------------------------------------
+# NVQ  (mfq/formats/nvq.py)
+# ---------------------------------------------------------------------------
+_NVQ_HDR = struct.Struct("<4sBBHiiI")
+_NVQ_CODEBOOK_ID = {"e8_256": 1, "d4_256": 2, "d4_512": 3, "e8_1024": 4, "e8_4096": 5, "d4_1024": 6}
+_NVQ_ID_CODEBOOK = {v: k for k, v in _NVQ_CODEBOOK_ID.items()}
+_NVQ_INDEX_BITS = {"e8_256": 8, "e8_1024": 10, "e8_4096": 12, "d4_256": 8, "d4_512": 9, "d4_1024": 10}
+
+
+def nvq_vector_size(codebook: str) -> int:
+    return 8 if codebook.startswith("e8_") else 4
+
+
+def nvq_grid(name: str) -> np.ndarray:
+    """Built-in magnitude grids, decoded as 2*digit+1 (mfq/formats/nvq.py:102-129)."""
+    raw = np.frombuffer((_DATA / f"{name}.bin").read_bytes(), dtype="<u2")
+    dims, digit_bits = (8, 2) if name.startswith("e8_") else (4, 3)
+    shifts = digit_bits * np.arange(dims, dtype=np.uint16)
+    digits = (raw[:, None] >> shifts[None, :]) & ((1 << digit_bits) - 1)
+    return np.ascontiguousarray(2 * digits + 1, dtype=np.int8)
+
+
+def nvq_payload_nbytes(codebook, out, neuron_len, gs=24, sub_bits=4):
+    """mfq/formats/nvq.py:197-207 (streams + anchors, excluding tables and header)."""
+    ng = math.ceil(neuron_len / gs)
+    nvec = math.ceil(neuron_len / nvq_vector_size(codebook))
+    nsign = math.ceil(neuron_len / 8)
+    return (out * 2 + (out * ng * sub_bits + 7) // 8
+            + (out * nvec * _NVQ_INDEX_BITS[codebook] + 7) // 8 + (out * nsign * 7 + 7) // 8)
+
+
+@dataclass
+class NvqJscTensor:
+    codebook: str
+    shape: tuple
+    neuron_len: int
+    neuron_scale: np.ndarray   # (out,) f32
+    scale_lut: np.ndarray      # (16,) f32
+    bank_for_state: np.ndarray # (16,) u8
+    state: np.ndarray          # (out, ng) u8
+    indices: np.ndarray        # (out, nvec) u16
+    signs: np.ndarray          # (out, nsign) u8
+    codebooks: np.ndarray      # (banks, entries, dim) i8, values 0..127
+    axis: int = 0
+    groupsize: int = 24
+    sub_bits: int = 4
+
+
+@dataclass
+class NvqTensor:
+    codebook: str
+    shape: tuple
+    neuron_len: int
+    neuron_scale: np.ndarray
+    sub_scale: np.ndarray      # (out, ng) u8 integer relative scale
+    indices: np.ndarray
+    signs: np.ndarray
+    axis: int = 0
+    groupsize: int = 24
+    sub_bits: int = 4
+    sign_mode: str = "even"
+    custom_codebook: np.ndarray | None = None
+
+
+def pack_jsc_tables(scale_lut, bank_for_state, codebooks) -> bytes:
+    """mfq/formats/nvq.py:446-483 (64-byte header + raw int8 banks)."""
+    codebooks = np.ascontiguousarray(codebooks, dtype=np.int8)
+    banks = codebooks.shape[0]
+    lut = np.asarray(scale_lut, dtype=np.float32).reshape(16)
+    bfs = np.ascontiguousarray(bank_for_state, dtype=np.uint8).reshape(16)
+    header = bytearray(64)
+    header[0], header[1], header[2] = 1, banks, 16
+    st = np.arange(16, dtype=np.uint8)
+    a_bank = st % banks
+    if banks == 1:
+        a_scale = st.astype(np.float32)
+    elif codebooks.shape[2] == 4:
+        a_scale = (st // banks).astype(np.float32) + 1.0
+    else:
+        a_scale = 15.0 * ((st // banks).astype(np.float32) + 1.0) / (16 // banks)
+    if np.array_equal(lut, a_scale) and np.array_equal(bfs, a_bank):
+        header[3] = 1
+    header[4:36] = lut.astype("<f2").tobytes()
+    header[36:52] = bfs.tobytes()
+    return bytes(header) + codebooks.tobytes()
+
+
+def pack_nvq_jsc(t: NvqJscTensor) -> bytes:
+    """mfq/formats/nvq.py:644-716."""
+    out = int(t.neuron_scale.size)
+    return b"".join([
+        _NVQ_HDR.pack(b"NVQ1", _NVQ_CODEBOOK_ID[t.codebook] | 0x20, 4, 24, t.axis, t.neuron_len, len(t.shape)),
+        struct.pack(f"<{len(t.shape)}q", *t.shape), struct.pack("<I", out),
+        pack_jsc_tables(t.scale_lut, t.bank_for_state, t.codebooks),
+        np.ascontiguousarray(t.neuron_scale, dtype=np.float16).tobytes(),
+        pack_bits(t.state, 4), pack_bits(t.indices, _NVQ_INDEX_BITS[t.codebook]), pack_bits(t.signs, 7)])
+
+
+def pack_nvq_plain(t: NvqTensor) -> bytes:
+    """mfq/formats/nvq.py:603-641 (non-JSC NVQ2/NVQ3 with the built-in grid)."""
+    out = int(t.neuron_scale.size)
+    cid = _NVQ_CODEBOOK_ID[t.codebook] | (0x80 if t.sign_mode == "index_parity" else 0)
+    return b"".join([
+        _NVQ_HDR.pack(b"NVQ1", cid, t.sub_bits, t.groupsize, t.axis, t.neuron_len, len(t.shape)),
+        struct.pack(f"<{len(t.shape)}q", *t.shape), struct.pack("<I", out),
+        np.ascontiguousarray(t.neuron_scale, dtype=np.float16).tobytes(),
+        pack_bits(t.sub_scale, t.sub_bits), pack_bits(t.indices, _NVQ_INDEX_BITS[t.codebook]),
+        pack_bits(t.signs, 7)])
+
+
+def unpack_nvq(blob):
+    """mfq/formats/nvq.py:719-820."""
+    blob = bytes(blob)
+    magic, enc_id, sub_bits, gs, axis, neuron_len, ndim = _NVQ_HDR.unpack_from(blob)
+    if magic not in (b"NVQ1", b"NIQ1"):
+        raise ValueError(f"invalid NVQ magic: {magic!r}")
+    sign_mode = "index_parity" if enc_id & 0x80 else "even"
+    custom, is_jsc = bool(enc_id & 0x40), bool(enc_id & 0x20)
+    cid = enc_id & ~0xE0
+    if cid not in _NVQ_ID_CODEBOOK:
+        raise ValueError(f"unknown NVQ codebook id: {cid}")
+    codebook = _NVQ_ID_CODEBOOK[cid]
+    off = _NVQ_HDR.size
+    shape = struct.unpack_from(f"<{ndim}q", blob, off)
+    off += 8 * ndim
+    out = struct.unpack_from("<I", blob, off)[0]
+    off += 4
+    vs, ib = nvq_vector_size(codebook), _NVQ_INDEX_BITS[codebook]
+    ng, nvec, nsign = math.ceil(neuron_len / gs), math.ceil(neuron_len / vs), math.ceil(neuron_len / 8)
+    if is_jsc:
+        if custom or sign_mode != "even" or gs != 24 or sub_bits != 4:
+            raise ValueError("invalid NVQ-JSC profile flags")
+        if len(blob) < off + 64:
+            raise ValueError("truncated NVQ-JSC metadata header")
+        hdr = blob[off:off + 64]
+        version, banks, states, mode = hdr[0], hdr[1], hdr[2], hdr[3]
+        if version != 1 or banks not in (1, 2, 4) or states != 16 or mode not in (0, 1) or any(hdr[52:64]):
+            raise ValueError("invalid NVQ-JSC metadata")
+        lut = np.frombuffer(hdr[4:36], dtype="<f2").astype(np.float32)
+        bfs = np.frombuffer(hdr[36:52], dtype=np.uint8).copy()
+        entries = 1 << ib
+        cb_bytes = banks * entries * vs
+        off += 64
+        if len(blob) < off + cb_bytes:
+            raise ValueError("truncated NVQ-JSC codebook banks")
+        cbs = np.frombuffer(blob, dtype=np.int8, count=cb_bytes, offset=off).copy().reshape(banks, entries, vs)
+        off += cb_bytes
+        if np.any(cbs < 0) or np.any(bfs >= banks) or not np.isfinite(lut).all() or np.any(lut < 0):
+            raise ValueError("invalid NVQ-JSC tables")
+        if off + 2 * out > len(blob):
+            raise ValueError("truncated NVQ-JSC neuron anchors")
+        ns = np.frombuffer(blob, dtype=np.float16, count=out, offset=off).astype(np.float32)
+        off += 2 * out
+        state, off = unpack_bits(blob, off, out * ng, 4)
+        idx, off = unpack_bits(blob, off, out * nvec, ib)
+        sg, off = unpack_bits(blob, off, out * nsign, 7)
+        if off != len(blob):
+            raise ValueError(f"invalid NVQ-JSC blob tail: consumed={off}, size={len(blob)}")
+        return NvqJscTensor(codebook, tuple(shape), neuron_len, ns, lut, bfs, state.reshape(out, ng),
+                            idx.reshape(out, nvec).astype(np.uint16), sg.reshape(out, nsign), cbs, axis)
+    cbk = None
+    if custom:
+        n = (1 << ib) * 2
+        raw = np.frombuffer(blob, dtype="<u2", count=n // 2, offset=off)
+        digit_bits = 2 if vs == 8 else 3
+        shifts = (digit_bits * np.arange(vs, dtype=np.uint16))[None, :]
+        cbk = (2 * ((raw[:, None] >> shifts) & ((1 << digit_bits) - 1)) + 1).astype(np.int8)
+        off += n
+    ns = np.frombuffer(blob, dtype=np.float16, count=out, offset=off).astype(np.float32)
+    off += 2 * out
+    ss, off = unpack_bits(blob, off, out * ng, sub_bits)
+    idx, off = unpack_bits(blob, off, out * nvec, ib)
+    sg, off = unpack_bits(blob, off, out * nsign, 7)
+    if off != len(blob):
+        raise ValueError(f"invalid NVQ blob tail: consumed={off}, size={len(blob)}")
+    return NvqTensor(codebook, tuple(shape), neuron_len, ns, ss.reshape(out, ng),
+                     idx.reshape(out, nvec).astype(np.uint16), sg.reshape(out, nsign), axis, gs, sub_bits,
+                     sign_mode, cbk)
+
+
+def _nvq_signs(masks, neuron_len, index_parity_bank=None):
+    """Bits 0..6 from the mask, bit 7 = parity of the seven (mfq/quantize/nvq_jsc.py:1066-1071)."""
+    masks = np.asarray(masks, dtype=np.uint8)
+    lower = ((masks[..., None] >> np.arange(7, dtype=np.uint8)) & 1).astype(np.uint8)
+    last = (lower.sum(axis=-1, keepdims=True) & 1).astype(np.uint8)
+    if index_parity_bank is not None:
+        last = last ^ index_parity_bank[..., None]
+    negative = np.concatenate([lower, last], axis=-1)
+    sign = np.where(negative != 0, -1.0, 1.0).astype(np.float32)
+    return sign.reshape(masks.shape[0], -1)[:, :neuron_len]
+
+
+def dequantize_nvq_jsc(t: NvqJscTensor) -> np.ndarray:
+    """mfq/quantize/nvq_jsc.py:1053-1079: f32(mag) * sign * fl(anchor * lut[state])."""
+    out, neuron_len = t.shape
+    gs, vs = 24, nvq_vector_size(t.codebook)
+    ng = math.ceil(neuron_len / gs)
+    vpg = gs // vs
+    idx = np.zeros((out, ng * vpg), dtype=np.uint16)
+    idx[:, : t.indices.shape[1]] = t.indices
+    group_bank = t.bank_for_state[t.state]
+    vector_bank = np.repeat(group_bank, vpg, axis=1)
+    magnitude = t.codebooks[vector_bank, idx].reshape(out, -1)[:, :neuron_len]
+    sign = _nvq_signs(t.signs, neuron_len)
+    group_scale = t.neuron_scale.astype(np.float32)[:, None] * t.scale_lut[t.state].astype(np.float32)
+    scale = np.repeat(group_scale, gs, axis=1)[:, :neuron_len]
+    return magnitude.astype(np.float32) * sign * scale
+
+
+def dequantize_nvq(t: NvqTensor) -> np.ndarray:
+    """mfq/quantize/nvq_quant.py:608-626: (table[idx] * sign) * (anchor * sub_scale)."""
+    out = t.neuron_scale.size
+    table = (t.custom_codebook if t.custom_codebook is not None else nvq_grid(t.codebook)).astype(np.float32)
+    magnitude = table[t.indices].reshape(out, -1)[:, : t.neuron_len]
+    bank = None
+    if t.sign_mode == "index_parity":
+        bank = ((np.asarray(t.indices, dtype=np.uint16) >> 7) & 1).astype(np.uint8)
+    sign = _nvq_signs(t.signs, t.neuron_len, bank)
+    group_scale = t.neuron_scale.astype(np.float32)[:, None] * t.sub_scale.astype(np.float32)
+    scale = np.repeat(group_scale, t.groupsize, axis=1)[:, : t.neuron_len]
+    return magnitude * sign * scale
+
+
+# ---------------------------------------------------------------------------
+# NEPQ  (mfq/formats/nepq.py; NEPQ1-S / NEPQ1-L only)
+# ---------------------------------------------------------------------------
+_NEPQ_HDR = struct.Struct("<4sBBBBIIIIIQ")
+#              label: (profile_id, state_bits, index_bits, aux_bits, table_bytes)
+NEPQ_SPECS = {"NEPQ0-S": (0, 2, 6, 0, None), "NEPQ0-L": (1, 3, 7, 0, None),
+              "NEPQ1-S": (2, 4, 9, 1, 2048), "NEPQ1-L": (3, 3, 11, 1, 4096)}
+_NEPQ_BY_ID = {v[0]: k for k, v in NEPQ_SPECS.items()}
+
+
+@dataclass
+class NepqTensor:
+    label: str
+    shape: tuple              # (experts, out, K)
+    neuron_scale: np.ndarray  # (E, out) f32
+    state: np.ndarray         # (E, out, ng)
+    indices: np.ndarray       # (E, out, nvec) u16
+    aux: np.ndarray           # (E, out, ng)
+    bank_ids: np.ndarray      # (E, out, nsuper) u8
+    table_payloads: np.ndarray  # (banks, table_bytes) u8
+    rotation_block: int = 0
+    rotation_seed: int = 0
+
+
+def nepq_payload_nbytes(label, n_experts, out, K, bank_count):
+    """mfq/formats/nepq.py:53-75."""
+    _, sb, ib, ab, tb = NEPQ_SPECS[label]
+    rows = n_experts * out
+    ng, nvec = math.ceil(K / 24), K // 8
+    nsuper = math.ceil(ng / 4)
+    pk = lambda c, b: (c * b + 7) // 8 if b else 0
+    return bank_count * tb + 2 * rows + pk(rows * ng, sb) + pk(rows * nvec, ib) + pk(rows * ng, ab) + rows * nsuper
+
+
+def unpack_ternary_table(payload: bytes) -> np.ndarray:
+    """2 bits per digit, digit = code + 1, 8 digits per u16 (mfq/formats/nvq1_l.py:121-130)."""
+    enc = np.frombuffer(payload, dtype="<u2")
+    digits = (enc[:, None] >> (2 * np.arange(8, dtype=np.uint16))[None, :]) & 3
+    if np.any(digits > 2):
+        raise ValueError("non-ternary digit in packed table")
+    return digits.astype(np.int8) - 1
+
+
+def pack_ternary_table(codes: np.ndarray) -> bytes:
+    d = (np.asarray(codes, dtype=np.int16) + 1).astype(np.uint16)
+    return np.bitwise_or.reduce(d << (2 * np.arange(8, dtype=np.uint16))[None, :], axis=1).astype("<u2").tobytes()
+
+
+def pack_nepq(t: NepqTensor) -> bytes:
+    """mfq/formats/nepq.py:368-399."""
+    pid, sb, ib, ab, tb = NEPQ_SPECS[t.label]
+    E, out, K = t.shape
+    return b"".join([
+        _NEPQ_HDR.pack(b"NEP1", 1, pid, 4, 1 if t.rotation_block else 0, E, out, K,
+                       int(t.table_payloads.shape[0]), int(t.rotation_block), int(t.rotation_seed)),
+        np.ascontiguousarray(t.table_payloads, dtype=np.uint8).tobytes(),
+        np.ascontiguousarray(t.neuron_scale, dtype="<f2").tobytes(),
+        pack_bits(t.state, sb), pack_bits(t.indices, ib), pack_bits(t.aux, ab) if ab else b"",
+        np.ascontiguousarray(t.bank_ids, dtype=np.uint8).tobytes()])
+
+
+def unpack_nepq(blob) -> NepqTensor:
+    """mfq/formats/nepq.py:402-474."""
+    blob = bytes(blob)
+    if len(blob) < _NEPQ_HDR.size:
+        raise ValueError("truncated NEPQ header")
+    magic, ver, pid, gps, flags, E, out, K, banks, rblock, rseed = _NEPQ_HDR.unpack_from(blob)
+    if magic != b"NEP1" or ver != 1 or pid not in _NEPQ_BY_ID or gps != 4:
+        raise ValueError("invalid or unsupported NEPQ header")
+    if flags & ~1 or bool(flags & 1) != bool(rblock):
+        raise ValueError("inconsistent NEPQ flags")
+    if E <= 0 or out <= 0 or K <= 0 or K % 8 or not 1 <= banks <= 256:
+        raise ValueError("invalid NEPQ dimensions")
+    label = _NEPQ_BY_ID[pid]
+    _, sb, ib, ab, tb = NEPQ_SPECS[label]
+    if tb is None:
+        raise NotImplementedError(f"{label} tables are outside the oracle's scope")
+    rows = E * out
+    ng, nvec = math.ceil(K / 24), K // 8
+    nsuper = math.ceil(ng / 4)
+    off = _NEPQ_HDR.size
+    if off + banks * tb > len(blob):
+        raise ValueError("truncated NEPQ table pool")
+    tables = np.frombuffer(blob, dtype=np.uint8, count=banks * tb, offset=off).copy().reshape(banks, tb)
+    off += banks * tb
+    if off + 2 * rows > len(blob):
+        raise ValueError("truncated NEPQ neuron anchors")
+    ns = np.frombuffer(blob, dtype="<f2", count=rows, offset=off).astype(np.float32).reshape(E, out)
+    off += 2 * rows
+    state, off = unpack_bits(blob, off, rows * ng, sb)
+    idx, off = unpack_bits(blob, off, rows * nvec, ib)
+    aux, off = unpack_bits(blob, off, rows * ng, ab)
+    if off + rows * nsuper > len(blob):
+        raise ValueError("truncated NEPQ bank selectors")
+    bank_ids = np.frombuffer(blob, dtype=np.uint8, count=rows * nsuper, offset=off).copy().reshape(E, out, nsuper)
+    off += rows * nsuper
+    if off != len(blob):
+        raise ValueError(f"invalid NEPQ tail: consumed={off}, size={len(blob)}")
+    if np.any(bank_ids >= banks):
+        raise ValueError("NEPQ bank ID exceeds the table pool")
+    for tbl in tables:   # ternary validity (mfq/formats/nepq.py:270-290)
+        unpack_ternary_table(tbl.tobytes())
+    return NepqTensor(label, (E, out, K), ns, state.reshape(E, out, ng), idx.reshape(E, out, nvec).astype(np.uint16),
+                      aux.reshape(E, out, ng), bank_ids, tables, rblock, rseed)
+
+
+def dequantize_nepq(t: NepqTensor) -> np.ndarray:
+    """mfq/formats/nepq.py:492-544: fl(anchor*state) * (code + (-/+)delta), code+delta exact."""
+    E, out, K = t.shape
+    rows = E * out
+    ng, nvec = math.ceil(K / 24), K // 8
+    state = t.state.reshape(rows, ng).astype(np.uint8)
+    idx = t.indices.reshape(rows, nvec).astype(np.int64)
+    anchors = t.neuron_scale.reshape(rows).astype(np.float32)
+    bank_ids = t.bank_ids.reshape(rows, -1)
+    group_bank = np.repeat(bank_ids, 4, axis=1)[:, :ng]
+    vector_bank = np.repeat(group_bank, 3, axis=1)[:, :nvec].astype(np.int64)
+    aux = t.aux.reshape(rows, ng).astype(np.uint8)
+    if t.label == "NEPQ1-S":
+        tables = np.stack([np.stack([unpack_ternary_table(p.tobytes()[:1024]),
+                                     unpack_ternary_table(p.tobytes()[1024:])]) for p in t.table_payloads])
+        vector_aux = np.repeat(aux, 3, axis=1)[:, :nvec].astype(np.int64)
+        code = tables[vector_bank, vector_aux, idx]
+        delta = np.where(aux != 0, -0.15625, 0.15625).astype(np.float32)
+    elif t.label == "NEPQ1-L":
+        tables = np.stack([unpack_ternary_table(p.tobytes()) for p in t.table_payloads])
+        code = tables[vector_bank, idx]
+        delta = np.where(aux != 0, -0.125, 0.125).astype(np.float32)
+    else:
+        raise NotImplementedError(t.label)
+    group_scale = anchors[:, None] * state.astype(np.float32)
+    scale = np.repeat(group_scale, 24, axis=1)[:, :K]
+    bias = np.repeat(delta, 24, axis=1)[:, :K]
+    result = scale * (code.reshape(rows, K).astype(np.float32) + bias)
+    return result.reshape(t.shape)
+
+
+# ---------------------------------------------------------------------------
+# NINTM container  (mfq/formats/io.py:251-446, mfq/formats/moe.py:83-155)
+# ---------------------------------------------------------------------------
+@dataclass
+class MoePool:
+    expert_ids: np.ndarray
+    dtype: str
+    tensor: object
+
+
+@dataclass
+class NintMoeTensor:
+    shape: tuple               # (experts, out_per_expert, K)
+    pools: list = field(default_factory=list)
+
+
+def tensor_dtype(t) -> str:
+    """Public dtype label (mfq/formats/io.py:576-640)."""
+    if isinstance(t, NintTensor):
+        return f"NINT{t.bits}"
+    if isinstance(t, NvqJscTensor):
+        return {"e8_256": "NVQ2J", "e8_1024": "NVQ2J-L", "e8_4096": "NVQ2J-XL", "d4_256": "NVQ3J",
+                "d4_512": "NVQ3J-512", "d4_1024": "NVQ3J-L"}[t.codebook]
+    if isinstance(t, NvqTensor):
+        return {"e8_256": "NVQ2", "d4_256": "NVQ3"}[t.codebook]
+    if isinstance(t, NepqTensor):
+        return t.label
+    if isinstance(t, NintMoeTensor):
+        return "NINTM"
+    raise TypeError(type(t))
+
+
+def pack_tensor(t) -> tuple[str, bytes]:
+    dt = tensor_dtype(t)
+    if isinstance(t, NintTensor):
+        return dt, pack_nint(t)
+    if isinstance(t, NvqJscTensor):
+        return dt, pack_nvq_jsc(t)
+    if isinstance(t, NvqTensor):
+        return dt, pack_nvq_plain(t)
+    if isinstance(t, NepqTensor):
+        return dt, pack_nepq(t)
+    return dt, pack_nint_moe(t)
+
+
+def unpack_tensor(dtype: str, blob):
+    """dtype-string dispatch (mfq/formats/io.py:488-576)."""
+    dtype = {"NIQ2": "NVQ2", "NIQ2J": "NVQ2J", "NIQ3": "NVQ3"}.get(dtype, dtype)
+    if dtype == "NINTM":
+        return unpack_nint_moe(blob)
+    if dtype in NEPQ_SPECS:
+        t = unpack_nepq(blob)
+        if t.label != dtype:
+            raise ValueError(f"MFQ dtype/blob mismatch: {dtype} contains {t.label}")
+        return t
+    if dtype.startswith("NINT"):
+        return unpack_nint(blob)
+    if dtype.startswith("NVQ"):
+        t = unpack_nvq(blob)
+        if tensor_dtype(t) != dtype:
+            raise ValueError(f"MFQ dtype/blob mismatch: {dtype} contains {tensor_dtype(t)}")
+        return t
+    raise ValueError(f"unsupported dtype {dtype}")
+
+
+_NIM_HDR = struct.Struct("<4sIIII")
+_NIM_POOL = struct.Struct("<IIQQ")
+
+
+def pack_nint_moe(t: NintMoeTensor) -> bytes:
+    """mfq/formats/io.py:304-336 (NIM2)."""
+    E, out, K = t.shape
+    parts = [_NIM_HDR.pack(b"NIM2", E, out, K, len(t.pools))]
+    for p in t.pools:
+        ids = np.ascontiguousarray(p.expert_ids, dtype=np.int32).reshape(-1)
+        dtype, payload = pack_tensor(p.tensor)
+        db = dtype.encode("ascii")
+        parts += [_NIM_POOL.pack(ids.size, len(db), len(payload), 0), ids.tobytes(), db, b"", payload]
+    return b"".join(parts)
+
+
+def unpack_nint_moe(blob) -> NintMoeTensor:
+    """mfq/formats/io.py:382-446 + invariants of mfq/formats/moe.py:98-134."""
+    blob = bytes(blob)
+    if len(blob) < _NIM_HDR.size:
+        raise ValueError("truncated NINTM header")
+    magic, E, out, K, npools = _NIM_HDR.unpack_from(blob, 0)
+    if magic != b"NIM2":
+        raise ValueError(f"invalid NINTM magic: {magic!r}")
+    if npools == 0 or npools > E:
+        raise ValueError("invalid NINTM pool count")
+    off = _NIM_HDR.size
+    pools, owners = [], np.full(E, -1, dtype=np.int32)
+    for pi in range(npools):
+        if off + _NIM_POOL.size > len(blob):
+            raise ValueError("truncated NINTM v2 pool header")
+        n_ids, dlen, plen, rlen = _NIM_POOL.unpack_from(blob, off)
+        off += _NIM_POOL.size
+        if n_ids == 0 or dlen == 0 or dlen > 32:
+            raise ValueError("invalid NINTM v2 pool metadata")
+        end = off + 4 * n_ids + dlen + rlen + plen
+        if end > len(blob):
+            raise ValueError("truncated NINTM v2 pool payload")
+        ids = np.frombuffer(blob, dtype=np.int32, count=n_ids, offset=off).copy()
+        off += 4 * n_ids
+        dtype = blob[off:off + dlen].decode("ascii")
+        off += dlen + rlen
+        tensor = unpack_tensor(dtype, blob[off:end])
+        off = end
+        if np.any(ids < 0) or np.any(ids >= E) or np.unique(ids).size != ids.size or np.any(owners[ids] >= 0):
+            raise ValueError("invalid NINTM expert ids")
+        owners[ids] = pi
+        expect = (n_ids, out, K) if isinstance(tensor, NepqTensor) else (n_ids * out, K)
+        if tuple(tensor.shape) != expect:
+            raise ValueError(f"NINTM pool {pi} tensor shape {tensor.shape} must be {expect}")
+        pools.append(MoePool(ids, dtype, tensor))
+    if off != len(blob):
+        raise ValueError(f"invalid NINTM tail: {len(blob) - off} extra bytes")
+    if np.any(owners < 0):
+        raise ValueError("NINTM pools do not cover all experts")
+    return NintMoeTensor((E, out, K), pools)
+
+
+def dequantize_tensor(t) -> np.ndarray:
+    if isinstance(t, NintTensor):
+        return dequantize_nint(t)
+    if isinstance(t, NvqJscTensor):
+        return dequantize_nvq_jsc(t)
+    if isinstance(t, NvqTensor):
+        return dequantize_nvq(t)
+    if isinstance(t, NepqTensor):
+        return dequantize_nepq(t)
+    raise TypeError(type(t))
+
+
+def dequantize_expertwise(t: NintMoeTensor) -> np.ndarray:
+    """mfq/quantize/expert_nint.py:605-615."""
+    E, out, K = t.shape
+    result = np.empty(t.shape, dtype=np.float32)
+    for p in t.pools:
+        result[p.expert_ids] = dequantize_tensor(p.tensor).reshape(len(p.expert_ids), out, K)
+    return result
+
+
+# ---------------------------------------------------------------------------
+# MFQ1 container  (mfq/formats/io.py:646-685, mfq/formats/header.py:14)
+# ---------------------------------------------------------------------------
+def mfq_file_write(path, tensors: dict, model_arch="synthetic", version=1):
+    packed = {n: (pack_tensor(t) if not isinstance(t, tuple) else t) for n, t in tensors.items()}
+    with open(path, "wb") as f:
+        f.write(b"MFQ1" + struct.pack("<I", version))
+        a = model_arch.encode()
+        f.write(struct.pack("<I", len(a)) + a)
+        if version >= 2:
+            f.write(struct.pack("<I", 0))
+        f.write(struct.pack("<I", len(packed)))
+        for n, (dt, blob) in packed.items():
+            nb, db = n.encode(), dt.encode()
+            f.write(struct.pack("<I", len(nb)) + nb + struct.pack("<I", len(db)) + db + struct.pack("<Q", len(blob)))
+        for n, (dt, blob) in packed.items():
+            f.write(blob)
+
+
+def mfq_file_read(path) -> dict:
+    data = Path(path).read_bytes()
+    if data[:4] != b"MFQ1":
+        raise ValueError("bad MFQ magic")
+    version, = struct.unpack_from("<I", data, 4)
+    off = 8
+    n, = struct.unpack_from("<I", data, off)
+    off += 4 + n
+    if version >= 2:
+        ne, = struct.unpack_from("<I", data, off)
+        off += 4
+        for _ in range(2 * ne):
+            n, = struct.unpack_from("<I", data, off)
+            off += 4 + n
+    nt, = struct.unpack_from("<I", data, off)
+    off += 4
+    recs = []
+    for _ in range(nt):
+        n, = struct.unpack_from("<I", data, off)
+        name = data[off + 4: off + 4 + n].decode()
+        off += 4 + n
+        n, = struct.unpack_from("<I", data, off)
+        dt = data[off + 4: off + 4 + n].decode()
+        off += 4 + n
+        ln, = struct.unpack_from("<Q", data, off)
+        off += 8
+        recs.append((name, dt, ln))
+    out = {}
+    for name, dt, ln in recs:
+        out[name] = (dt, data[off: off + ln])
+        off += ln
+    return out
+
+
+# ---------------------------------------------------------------------------
+# the CPU matmul path  (mfq/runtime/linear.py:37-42)
+# ---------------------------------------------------------------------------
+def bf16_round(x) -> np.ndarray:
+    """Round fp32 to the nearest bf16 (ties to even), returned as fp32."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    return r.astype(np.uint32).view(np.float32)
+
+
+def bf16_bits(x) -> np.ndarray:
+    return (bf16_round(x).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def linear_forward(W: np.ndarray, x: np.ndarray) -> np.ndarray:
+    """y = f32(x) @ dequant(W).T, numpy fp32 (mfq/runtime/linear.py:37-42)."""
+    return np.asarray(x, dtype=np.float32) @ np.asarray(W, dtype=np.float32).T
+
+
+def linear_forward_f64(W, x) -> np.ndarray:
+    """The same product accumulated in fp64: the tolerance yardstick for GPU outputs."""
+    return np.asarray(x, dtype=np.float64) @ np.asarray(W, dtype=np.float64).T
+
+
+# ---------------------------------------------------------------------------
+# MoE routing + grouped matmul  (mfq/kernels/cuda/moe.cu, tests/test_moe_kernels_cuda.py)
+# ---------------------------------------------------------------------------
+def moe_topk(logits, top_k, use_sigmoid=False, use_sqrt_softplus=False, normalize=False,
+             delayed_softmax=False, bias=None, norm_floor=1e-20, scale=1.0):
+    """mfq/kernels/cuda/moe.cu:124-263: iterative arg-max, tie -> lower expert id, NaN -> -FLT_MAX,
+    bias added to the selection score only."""
+    x = np.asarray(logits, dtype=np.float32)
+    x = np.where(np.isnan(x), -np.finfo(np.float32).max, x).astype(np.float32)
+    T, E = x.shape
+    if delayed_softmax:
+        w = x
+    elif use_sigmoid:
+        w = (1.0 / (1.0 + np.exp(-x.astype(np.float64)))).astype(np.float32)
+    elif use_sqrt_softplus:
+        xd = x.astype(np.float64)
+        w = np.sqrt(np.where(xd > 20.0, xd, np.log1p(np.exp(np.minimum(xd, 20.0))))).astype(np.float32)
+    else:
+        xd = x.astype(np.float64)
+        e = np.exp(xd - xd.max(-1, keepdims=True))
+        w = (e / e.sum(-1, keepdims=True)).astype(np.float32)
+    score = w if bias is None else (w + np.asarray(bias, dtype=np.float32)[None, :]).astype(np.float32)
+    # stable sort on -score keeps the lower expert id first among equal scores
+    order = np.argsort(-score, axis=-1, kind="stable")[:, :top_k]
+    ids = order.astype(np.int32)
+    sel = np.take_along_axis(w, order, axis=-1).astype(np.float32)
+    if delayed_softmax:
+        sd = sel.astype(np.float64)
+        e = np.exp(sd - sd.max(-1, keepdims=True))
+        sel = (e / e.sum(-1, keepdims=True)).astype(np.float32)
+    elif normalize:
+        sel = (sel / np.maximum(sel.sum(-1, keepdims=True), np.float32(norm_floor))).astype(np.float32)
+    return ids, (sel * np.float32(scale)).astype(np.float32)
+
+
+def build_expert_map(ids, n_experts, tile_m=8):
+    """mfq/kernels/cuda/moe.cu:472-542: counts, exclusive bounds, tile bounds, tile->expert, and a
+    grouping permutation of the (token, route) pairs (stable order inside an expert)."""
+    flat = np.asarray(ids, dtype=np.int32).reshape(-1)
+    valid = (flat >= 0) & (flat < n_experts)
+    counts = np.bincount(flat[valid], minlength=n_experts).astype(np.int32)
+    expert_bounds = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    tiles = (counts + tile_m - 1) // tile_m
+    tile_bounds = np.concatenate([[0], np.cumsum(tiles)]).astype(np.int32)
+    tile_experts = np.repeat(np.arange(n_experts, dtype=np.int32), tiles)
+    pairs = np.flatnonzero(valid)
+    ids_dst = pairs[np.argsort(flat[valid], kind="stable")].astype(np.int32)
+    return ids_dst, expert_bounds, tile_bounds, tile_experts, counts
+
+
+def moe_grouped_matmul(dense, x, ids):
+    """tests/test_moe_kernels_cuda.py:58-68: out[t, r] = x[t(,r)] @ dense[ids[t, r]].T in fp32.
+    A route with an out-of-range expert id yields zeros."""
+    dense = np.asarray(dense, dtype=np.float32)
+    x = np.asarray(x, dtype=np.float32)
+    T, R = ids.shape
+    out = np.zeros((T, R, dense.shape[1]), dtype=np.float32)
+    for t in range(T):
+        for r in range(R):
+            e = int(ids[t, r])
+            if 0 <= e < dense.shape[0]:
+                src = x[t, r] if x.ndim == 3 else x[t]
+                out[t, r] = src @ dense[e].T
+    return out
+
+
+def moe_swiglu(gate_up):
+    """silu(gate) * up over [..., 2W] -> [..., W], gate = first half (mfq/kernels/cuda/moe.cu:2980-2996)."""
+    g = np.asarray(gate_up, dtype=np.float32)
+    W = g.shape[-1] // 2
+    gate, up = g[..., :W].astype(np.float64), g[..., W:].astype(np.float64)
+    return ((gate / (1.0 + np.exp(-gate))) * up).astype(np.float32)
+
+
+def moe_weighted_reduce(pair, weights):
+    """out[t] = sum_r w[t, r] * pair[t, r] in fp32, r ascending (mfq/kernels/cuda/moe.cu:2957-2978)."""
+    pair = np.asarray(pair, dtype=np.float32)
+    w = np.asarray(weights, dtype=np.float32)
+    out = np.zeros((pair.shape[0], pair.shape[2]), dtype=np.float32)
+    for r in range(pair.shape[1]):
+        out += w[:, r:r + 1] * pair[:, r]
+    return out
+
+
+def moe_ffn(gate_up_dense, down_dense, x, router_logits, top_k, shared=None, **topk_kw):
+    """cpp_runtime/mfq_decode.cpp:3394-3416 (+ ungated shared expert add, :11077-11080).
+    `shared` = (gate_up_dense [2W, H], down_dense [H, W]) of the shared expert, or None."""
+    ids, w = moe_topk(router_logits, top_k, **topk_kw)
+    gu = moe_grouped_matmul(gate_up_dense, x, ids)
+    hidden = moe_swiglu(gu)
+    dn = moe_grouped_matmul(down_dense, hidden, ids)
+    out = moe_weighted_reduce(dn, w)
+    if shared is not None:
+        sgu, sdn = shared
+        h = moe_swiglu(linear_forward(sgu, x))
+        out = out + linear_forward(sdn, h)
+    return out, ids, w

@@ -1,0 +1,112 @@
+"""GPU parity of the NINT path against the oracle (through the C ABI)."""
+import numpy as np
+import pytest
+
+from conftest import ABS_TOL, REL_TOL, rel_l2
+from oracle import mfq_oracle as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+# (bits, gs, sub_bits): the production profiles plus odd ones that take the generic unit
+SPECS = [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (6, 24, 6), (8, 24, 8), (4, 16, 6), (4, 48, 6),
+         (6, 26, 6), (2, 32, 5), (5, 16, 5)]
+
+
+def _rand_tensor(rng, out, K, bits, gs, sb):
+    """Packed-domain random tensor (every code / sub-scale value occurs)."""
+    ng = -(-K // gs)
+    return O.NintTensor(bits, gs, sb, (out, K), 0, K,
+                        rng.integers(0, 1 << bits, (out, ng, gs), dtype=np.uint8),
+                        O._f16_round(rng.uniform(1e-4, 2e-3, out)), O._f16_round(rng.uniform(1e-3, 2e-2, out)),
+                        rng.integers(0, 1 << sb, (out, ng), dtype=np.uint8),
+                        rng.integers(0, 1 << sb, (out, ng), dtype=np.uint8))
+
+
+def _load(t):
+    from tyloquant_amd import runtime as R
+    return R.load_quant_linear(f"NINT{t.bits}", O.pack_nint(t))
+
+
+def _x(rng, M, K, dtype=None):
+    dtype = dtype or torch.bfloat16
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype)
+    return x.cuda(), x.float().numpy()
+
+
+@pytest.mark.parametrize("bits,gs,sb", SPECS)
+@pytest.mark.parametrize("out,K", [(48, 88), (37, 96), (64, 200), (257, 224), (73, 1537)])
+def test_dequant_bit_exact(bits, gs, sb, out, K):
+    rng = np.random.default_rng(1000 + bits * 100 + gs + out)
+    t = _rand_tensor(rng, out, K, bits, gs, sb)
+    lin = _load(t)
+    got = lin.dequantize().cpu().numpy()
+    want = O.dequantize_nint(t)
+    assert got.shape == want.shape
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("bits,gs,sb", SPECS)
+@pytest.mark.parametrize("M", [1, 2, 3, 8])
+def test_gemv_matches_oracle(bits, gs, sb, M):
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(70 + bits + M)
+    out, K = 48, 88
+    t = O.quantize_nint((rng.standard_normal((out, K)) * 0.02).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    for dtype in (torch.bfloat16, torch.float16):
+        x, xf = _x(rng, M, K, dtype)
+        y = R.nint_matmul(lin.weight, x, force="gemv").cpu().numpy()
+        ref = O.linear_forward(O.dequantize_nint(t), xf)
+        assert rel_l2(y, ref) < REL_TOL, (dtype, rel_l2(y, ref))
+        assert np.abs(y - ref).max() < ABS_TOL
+
+
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (4, 24, 6)])
+@pytest.mark.parametrize("out,K,M", [(128, 280, 16), (257, 224, 23), (73, 1537, 65), (512, 1024, 257)])
+def test_gemm_matches_oracle(bits, gs, sb, out, K, M):
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(170 + bits + M)
+    t = O.quantize_nint((rng.standard_normal((out, K)) * 0.02).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    x, xf = _x(rng, M, K)
+    y = lin(x).cpu().numpy()
+    ref = O.linear_forward_f64(O.dequantize_nint(t), xf)
+    assert rel_l2(y, ref) < REL_TOL, rel_l2(y, ref)
+    assert np.abs(y - ref).max() < ABS_TOL
+
+
+def test_config1_shape_nint3():
+    """BASELINE config 1: 4096x4096 N(0, 0.02) NINT3 (3,24,5), bf16 x at batch 1."""
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(1)
+    out = K = 4096
+    W = (rng.standard_normal((out, K)) * 0.02).astype(np.float32)
+    t = O.quantize_nint(W, 3, 24, 5)
+    blob = O.pack_nint(t)
+    assert len(blob) - 0 >= O.nint_payload_nbytes(out, K, 3, 24, 5) == 7195648
+    lin = R.load_quant_linear("NINT3", blob)
+    deq = O.dequantize_nint(t)
+    assert np.array_equal(lin.dequantize().cpu().numpy().view(np.uint32), deq.view(np.uint32))
+    x, xf = _x(rng, 1, K)
+    y = lin(x).cpu().numpy()
+    ref = O.linear_forward(deq, xf)
+    assert rel_l2(y, ref) < REL_TOL
+    assert np.abs(y - ref).max() < ABS_TOL
+
+
+def test_legacy_byte_tail_and_errors():
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(5)
+    t = _rand_tensor(rng, 8, 96, 4, 24, 6)
+    blob = O.pack_nint(t)
+    hdr = blob[: len(blob) - (O.nint_payload_nbytes(8, 96, 4, 24, 6) - 32)]
+    legacy = hdr + t.sub_scale.tobytes() + t.sub_min.tobytes() + t.q.tobytes()
+    lin = R.load_quant_linear("NINT4", legacy)
+    assert np.array_equal(lin.dequantize().cpu().numpy(), O.dequantize_nint(t))
+    with pytest.raises(ValueError, match="invalid NINT blob tail"):
+        R.load_quant_linear("NINT4", blob[:-1])
+    with pytest.raises(ValueError, match="dtype/blob mismatch"):
+        R.load_quant_linear("NINT5", blob)
+    with pytest.raises(ValueError):
+        R.load_quant_linear("NOPE", blob)

@@ -1,0 +1,113 @@
+"""ctypes binding of libmfq_hip.so (the C ABI declared in include/mfq_hip.h).
+
+The library is built in-tree by `make -C tyloquant_amd/csrc` (see __graft_entry__.build).
+Loading fails loudly when it is missing: there is no CPU fallback for any kernel.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from pathlib import Path
+
+_HERE = Path(__file__).resolve().parent
+LIB_PATH = _HERE / "lib" / "libmfq_hip.so"
+
+X_BF16, X_F16 = 0, 1
+TOPK_SOFTMAX, TOPK_SIGMOID, TOPK_SQRT_SOFTPLUS, TOPK_DELAYED_SOFTMAX = 0, 1, 2, 3
+
+i32, i64, vp, sz = C.c_int32, C.c_int64, C.c_void_p, C.c_size_t
+
+
+class NintDesc(C.Structure):
+    _fields_ = [(n, i32) for n in ("bits", "sub_bits", "gs", "out", "neuron_len", "ng", "kind", "dwords",
+                                   "tail_bytes", "ngp", "nsteps", "n_rowblocks")] + \
+               [(n, i64) for n in ("step_bytes", "rowblock_bytes", "anchors_off", "total_bytes", "payload_bytes")]
+
+
+class NvqDesc(C.Structure):
+    _fields_ = [(n, i32) for n in ("index_bits", "entries", "banks", "out", "neuron_len", "ng", "nvec", "nsign",
+                                   "ngp", "nsteps", "n_rowblocks")] + \
+               [(n, i64) for n in ("step_bytes", "rowblock_bytes", "tables_off", "anchors_off", "total_bytes",
+                                   "payload_bytes")]
+
+
+class NepqDesc(C.Structure):
+    _fields_ = [(n, i32) for n in ("profile", "state_bits", "index_bits", "banks", "rows", "neuron_len", "ng", "nvec",
+                                   "nsuper", "ngp", "nsteps", "n_rowblocks", "table_entries")] + \
+               [(n, i64) for n in ("step_bytes", "rowblock_bytes", "tables_off", "anchors_off", "total_bytes",
+                                   "payload_bytes")]
+
+
+class MoePool(C.Structure):
+    _fields_ = [("desc", NintDesc), ("weight", vp)]
+
+
+class MfqError(RuntimeError):
+    pass
+
+
+_SIGS = {
+    "mfq_hip_version": (C.c_int, []),
+    "mfq_hip_nint_plan": (C.c_int, [C.c_int] * 5 + [C.POINTER(NintDesc)]),
+    "mfq_hip_nint_repack": (C.c_int, [C.POINTER(NintDesc), vp, i64, C.c_int, vp, vp]),
+    "mfq_hip_nint_dequant_f32": (C.c_int, [C.POINTER(NintDesc), vp, vp, i64, vp]),
+    "mfq_hip_nint_gemv": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
+    "mfq_hip_nint_gemm_workspace_bytes": (sz, [C.POINTER(NintDesc), C.c_int]),
+    "mfq_hip_nint_gemm": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
+    "mfq_hip_nvq_plan": (C.c_int, [C.c_int] * 4 + [C.POINTER(NvqDesc)]),
+    "mfq_hip_nvq_repack": (C.c_int, [C.POINTER(NvqDesc), vp, i64, vp, vp]),
+    "mfq_hip_nvq_repack_plain": (C.c_int, [C.POINTER(NvqDesc), vp, i64, vp, vp, vp]),
+    "mfq_hip_nvq_dequant_f32": (C.c_int, [C.POINTER(NvqDesc), vp, vp, i64, vp]),
+    "mfq_hip_nvq_gemv": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
+    "mfq_hip_nvq_gemm_workspace_bytes": (sz, [C.POINTER(NvqDesc), C.c_int]),
+    "mfq_hip_nvq_gemm": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
+    "mfq_hip_nepq_plan": (C.c_int, [C.c_int] * 4 + [C.POINTER(NepqDesc)]),
+    "mfq_hip_nepq_repack": (C.c_int, [C.POINTER(NepqDesc), vp, i64, vp, vp]),
+    "mfq_hip_nepq_dequant_f32": (C.c_int, [C.POINTER(NepqDesc), vp, vp, i64, vp]),
+    "mfq_hip_nepq_gemv": (C.c_int, [C.POINTER(NepqDesc), vp, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
+    "mfq_hip_nepq_gemm_workspace_bytes": (sz, [C.POINTER(NepqDesc), C.c_int, C.c_int]),
+    "mfq_hip_nepq_gemm": (C.c_int, [C.POINTER(NepqDesc), vp, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp, i64,
+                                    vp, sz, vp]),
+    "mfq_hip_nepq_hadamard": (C.c_int, [vp, C.c_int, i64, C.c_int, C.c_int, C.c_int, vp, vp, i64, vp]),
+    "mfq_hip_moe_topk": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp,
+                                   vp]),
+    "mfq_hip_moe_route_map": (C.c_int, [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, C.c_int, vp, vp]),
+    "mfq_hip_moe_grouped_workspace_bytes": (sz, [C.c_int, C.c_int, C.c_int]),
+    "mfq_hip_moe_grouped_matmul": (C.c_int, [C.POINTER(MoePool), C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, vp,
+                                             C.c_int, i64, C.c_int, vp, C.c_int, C.c_int, vp, vp, vp, i64, vp, sz,
+                                             vp]),
+    "mfq_hip_moe_swiglu": (C.c_int, [vp, i64, C.c_int, C.c_int, vp, C.c_int, i64, vp]),
+    "mfq_hip_moe_weighted_reduce": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]),
+    "mfq_hip_gemm_f16_nt": (C.c_int, [vp, i64, vp, i64, C.c_int, C.c_int, C.c_int, vp, i64, vp]),
+}
+
+_lib = None
+
+
+def exported_symbols() -> list[str]:
+    """Every entry point include/mfq_hip.h declares (kept in step with the header by a test)."""
+    return sorted(list(_SIGS) + ["mfq_hip_last_error"])
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise MfqError(f"{LIB_PATH} is missing: build it with `make -C tyloquant_amd/csrc` "
+                           "(or python -c 'import __graft_entry__ as g; g.build()'); there is no CPU fallback")
+        _lib = C.CDLL(str(LIB_PATH))
+        _lib.mfq_hip_last_error.restype = C.c_char_p
+        _lib.mfq_hip_last_error.argtypes = []
+        for name, (res, args) in _SIGS.items():
+            fn = getattr(_lib, name, None)
+            if fn is None:
+                if os.environ.get("MFQ_ALLOW_MISSING_SYMBOLS") == "1":  # partial builds during kernel bring-up
+                    continue
+                raise MfqError(f"{LIB_PATH} does not export {name}: rebuild it (make -C tyloquant_amd/csrc)")
+            fn.restype, fn.argtypes = res, args
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise MfqError(f"mfq_hip status {rc}: {lib().mfq_hip_last_error().decode(errors='replace')}")

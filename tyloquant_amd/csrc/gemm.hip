@@ -1,0 +1,214 @@
+// Prefill / large-M path: activations are rescaled per row by an exact power of two into fp16,
+// weights are dequantized into fp16 (scaled per neuron by an exact power of two), and an
+// fp16 x fp16 -> fp32 MFMA GEMM (v_mfma_f32_32x32x16_f16) produces y; the epilogue multiplies
+// the two power-of-two scales back.  fp16 (11 significant bits) keeps the weight rounding error
+// near 1e-4 relative, which bf16 tiles (8 bits) cannot.
+#include "common.hpp"
+
+namespace mfq {
+
+// ---- core: thread-local error text ---------------------------------------------------
+char *error_buffer() {
+    static thread_local char buf[512] = {0};
+    return buf;
+}
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(error_buffer(), 512, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+// ---- activation prep: x16[m, k] = fp16(x[m, k] * 2^-f_m), xscale[m] = 2^f_m ---------------
+template <int XF16>
+__global__ __launch_bounds__(256) void x_prep_kernel(const uint16_t *__restrict__ x, int64_t ldx, int K, int Kp,
+                                                     uint16_t *__restrict__ x16, float *__restrict__ xscale) {
+    __shared__ float red[4];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const uint16_t *xr = x + static_cast<int64_t>(m) * ldx;
+    float amax = 0.f;
+    for (int k = tid; k < K; k += 256) {
+        const float v = fabsf(x_to_f32<XF16>(xr[k]));
+        if (v == v && v <= 3.0e38f) amax = fmaxf(amax, v);
+    }
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    int e = 0;
+    if (amax > 0.f) frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
+    const float inv = ldexpf(1.f, 9 - e);  // row maximum lands in [256, 512)
+    if (tid == 0) xscale[m] = ldexpf(1.f, e - 9);
+    uint16_t *o16 = x16 + static_cast<int64_t>(m) * Kp;
+    for (int k = tid; k < Kp; k += 256) o16[k] = k < K ? f32_to_f16_rne(x_to_f32<XF16>(xr[k]) * inv) : uint16_t(0);
+}
+
+// ---- fp16 NT GEMM: y[m, n] = sa[m] * sb[n] * sum_k a[m, k] * b[n, k] ----------------------
+// 128 x 128 x 32 block tile, 256 threads = 4 waves of 64 x 64 (2 x 2 MFMA 32x32x16 tiles).
+constexpr int GBM = 128, GBN = 128, GBK = 32, GLD = GBK + 8;  // LDS row stride in halves (80 bytes)
+
+__global__ __launch_bounds__(256) void gemm_f16_nt_kernel(const uint16_t *__restrict__ a, int64_t lda,
+                                                          const uint16_t *__restrict__ b, int64_t ldb, int M, int N,
+                                                          int K, const float *__restrict__ sa,
+                                                          const float *__restrict__ sb, float *__restrict__ y,
+                                                          int64_t ldy) {
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][GBM * GLD];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][GBN * GLD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bm = blockIdx.y * GBM, bn = blockIdx.x * GBN;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    // global -> LDS: each thread moves 16 halves of A and of B per K step (row = tid/2, half-row = tid&1)
+    const int lr = tid >> 1, lc = (tid & 1) * 16;
+    const bool a_ok = bm + lr < M, b_ok = bn + lr < N;
+    const uint16_t *ap = a + static_cast<int64_t>(bm + lr) * lda + lc;
+    const uint16_t *bp = b + static_cast<int64_t>(bn + lr) * ldb + lc;
+    float16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int t = 0; t < 16; ++t) acc[i][j][t] = 0.f;
+
+    const int nk = K / GBK;  // K is a multiple of 32 (callers pad)
+    u32x4_t ra[2], rbv[2];
+    auto gload = [&](int kt) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            ra[h] = a_ok ? *reinterpret_cast<const u32x4_t *>(ap + kt * GBK + 8 * h) : u32x4_t{0, 0, 0, 0};
+            rbv[h] = b_ok ? *reinterpret_cast<const u32x4_t *>(bp + kt * GBK + 8 * h) : u32x4_t{0, 0, 0, 0};
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            *reinterpret_cast<u32x4_t *>(&As[buf][lr * GLD + lc + 8 * h]) = ra[h];
+            *reinterpret_cast<u32x4_t *>(&Bs[buf][lr * GLD + lc + 8 * h]) = rbv[h];
+        }
+    };
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    const int fr = lane & 31, fk = (lane >> 5) * 8;
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) gload(kt + 1);
+#pragma unroll
+        for (int kk = 0; kk < GBK; kk += 16) {
+            half8_t fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fa[i] = *reinterpret_cast<const half8_t *>(&As[buf][(wm + 32 * i + fr) * GLD + kk + fk]);
+                fb[i] = *reinterpret_cast<const half8_t *>(&Bs[buf][(wn + 32 * i + fr) * GLD + kk + fk]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) lstore(buf ^ 1);
+        __syncthreads();
+    }
+    // D[row = m, col = n]: lane holds col = lane & 31, rows 8 * (t / 4) + 4 * (lane / 32) + t % 4
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = bn + wn + 32 * j + (lane & 31);
+            if (n >= N) continue;
+            const float sn = sb ? sb[n] : 1.f;
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const int m = bm + wm + 32 * i + 8 * (t >> 2) + 4 * (lane >> 5) + (t & 3);
+                if (m < M) y[static_cast<int64_t>(m) * ldy + n] = acc[i][j][t] * sn * (sa ? sa[m] : 1.f);
+            }
+        }
+    }
+}
+
+int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, const float *sa,
+                const float *sb, float *y, int64_t ldy, hipStream_t st) {
+    MFQ_REQUIRE(K % GBK == 0 && lda % 8 == 0 && ldb % 8 == 0, MFQ_ERR_INVALID,
+                "gemm_f16_nt: K=%d, lda=%lld, ldb=%lld must be multiples of 32 / 8 / 8", K, (long long)lda, (long long)ldb);
+    const dim3 grid(static_cast<unsigned>(ceil_div(N, GBN)), static_cast<unsigned>(ceil_div(M, GBM)));
+    hipLaunchKernelGGL(gemm_f16_nt_kernel, grid, dim3(256), 0, st, static_cast<const uint16_t *>(a), lda,
+                       static_cast<const uint16_t *>(b), ldb, M, N, K, sa, sb, y, ldy);
+    return check_launch("gemm_f16_nt");
+}
+
+int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, hipStream_t st) {
+    if (x_dtype == MFQ_X_F16)
+        hipLaunchKernelGGL((x_prep_kernel<1>), dim3(M), dim3(256), 0, st, static_cast<const uint16_t *>(x), ldx, K, Kp,
+                           static_cast<uint16_t *>(x16), xscale);
+    else
+        hipLaunchKernelGGL((x_prep_kernel<0>), dim3(M), dim3(256), 0, st, static_cast<const uint16_t *>(x), ldx, K, Kp,
+                           static_cast<uint16_t *>(x16), xscale);
+    return check_launch("x_prep");
+}
+
+// Workspace carve-up of the dequant + GEMM path: x16 [M, Kp] | xscale [M] | w16 [N, Kp] | wscale [N]
+static size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+size_t dequant_gemm_workspace(int N, int K, int M) {
+    const size_t Kp = static_cast<size_t>(ceil_div(K, GBK)) * GBK;
+    return align256(static_cast<size_t>(M) * Kp * 2) + align256(static_cast<size_t>(M) * 4) +
+           align256(static_cast<size_t>(N) * Kp * 2) + align256(static_cast<size_t>(N) * 4);
+}
+void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&xscale, uint16_t *&w16, float *&wscale,
+                        int &Kp) {
+    Kp = static_cast<int>(ceil_div(K, GBK)) * GBK;
+    uint8_t *p = static_cast<uint8_t *>(ws);
+    x16 = reinterpret_cast<uint16_t *>(p); p += align256(static_cast<size_t>(M) * Kp * 2);
+    xscale = reinterpret_cast<float *>(p); p += align256(static_cast<size_t>(M) * 4);
+    w16 = reinterpret_cast<uint16_t *>(p); p += align256(static_cast<size_t>(N) * Kp * 2);
+    wscale = reinterpret_cast<float *>(p);
+}
+
+int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M, float *y,
+                  int64_t ldy, hipStream_t st);
+int nint_dequant_f16(const mfq_nint_desc *d, const void *weight, void *w16, int64_t ld, float *rowscale, hipStream_t st);
+
+}  // namespace mfq
+
+using namespace mfq;
+
+extern "C" const char *mfq_hip_last_error(void) { return error_buffer(); }
+extern "C" int mfq_hip_version(void) { return 1; }
+
+extern "C" int mfq_hip_gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, float *y,
+                                   int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(a && b && y, MFQ_ERR_INVALID, "gemm_f16_nt: null argument");
+    return gemm_f16_nt(a, lda, b, ldb, M, N, K, nullptr, nullptr, y, ldy, as_stream(stream));
+}
+
+// Below this many activation rows the weight stream dominates and the GEMV kernels win.
+static constexpr int kGemvMaxM = 8;
+
+extern "C" size_t mfq_hip_nint_gemm_workspace_bytes(const mfq_nint_desc *d, int M) {
+    if (!d || M <= kGemvMaxM) return 0;
+    return dequant_gemm_workspace(d->out, d->neuron_len, M);
+}
+
+extern "C" int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                                 int M, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                                 mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nint_gemm: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nint_gemm: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint_gemm: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nint_gemm: ldx/ldy smaller than the tensor");
+    hipStream_t st = as_stream(stream);
+    if (M <= kGemvMaxM) return nint_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, st);
+    const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
+    MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nint_gemm: workspace %zu < %zu bytes",
+                workspace_bytes, need);
+    uint16_t *x16, *w16;
+    float *xscale, *wscale;
+    int Kp;
+    dequant_gemm_carve(workspace, d->out, d->neuron_len, M, x16, xscale, w16, wscale, Kp);
+    int rc = x_prep(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, st);
+    if (rc) return rc;
+    rc = nint_dequant_f16(d, weight, w16, Kp, wscale, st);
+    if (rc) return rc;
+    return gemm_f16_nt(x16, Kp, w16, Kp, M, d->out, Kp, xscale, wscale, y, ldy, st);
+}

@@ -1,0 +1,476 @@
+// NINT: device layout plan, load-time repack, bit-exact dequantizer and the decode GEMV.
+//
+// Layout (one allocation per tensor):
+//   row-block rb (16 neurons) -> step s (16 groups per neuron) -> three lane-interleaved regions
+//     Q: [j=0..3][lane=0..63][dwords]   codes of group 16s + 4j + (lane>>4) of neuron 16rb + (lane&15)
+//     T: [lane][4 bytes]                one tail byte per j (3-bit units only)
+//     S: [lane][8 bytes]                (sub_scale, sub_min) per j
+//   then float ns[16*n_rowblocks], float nm[16*n_rowblocks].
+// A wave therefore streams a contiguous span of HBM per step and every load instruction of the
+// wave covers whole 128-byte lines.
+//
+// "Paired" units keep two code fields 16 bits apart in each dword (even weight in the low half,
+// odd weight in the high half) so that one AND/OR turns a dword into two exact bf16 (or fp16)
+// integers biased by 128 (1024), ready for a packed dot product against the natural (x[2i], x[2i+1])
+// activation pairs.  The bias is removed per group with the group sum of x.
+#include "common.hpp"
+#include "gemv_common.hpp"
+
+namespace mfq {
+
+struct NintK {  // what kernels need of mfq_nint_desc, passed by value
+    int bits, sub_bits, gs, out, neuron_len, ng, kind, dwords, tail, nsteps, n_rowblocks;
+    int64_t step_bytes, rowblock_bytes, anchors_off;
+};
+
+static NintK to_k(const mfq_nint_desc *d) {
+    NintK k;
+    k.bits = d->bits; k.sub_bits = d->sub_bits; k.gs = d->gs; k.out = d->out; k.neuron_len = d->neuron_len;
+    k.ng = d->ng; k.kind = d->kind; k.dwords = d->dwords; k.tail = d->tail_bytes; k.nsteps = d->nsteps;
+    k.n_rowblocks = d->n_rowblocks; k.step_bytes = d->step_bytes; k.rowblock_bytes = d->rowblock_bytes;
+    k.anchors_off = d->anchors_off;
+    return k;
+}
+
+static bool paired_profile(int bits, int gs) {
+    if (bits == 4) return gs == 16 || gs == 24 || gs == 32 || gs == 48;
+    if (bits == 2) return gs == 16 || gs == 32;
+    if (bits == 3) return gs == 24;
+    return false;
+}
+
+// ---- field placement shared by repack and dequant ----------------------------------------
+// Position of weight i inside a paired unit: word index (dwords == tail word) and bit offset;
+// 3-bit weights 22 and 23 are split over spare bits and are handled by the callers.
+__device__ __forceinline__ void paired_pos(int bits, int i, int &word, int &bit) {
+    const int per_half = (bits == 3) ? 5 : 16 / bits;
+    const int per_word = 2 * per_half;
+    word = i / per_word;
+    const int r = i - word * per_word;
+    bit = (r >> 1) * bits + ((r & 1) << 4);
+}
+
+__device__ __forceinline__ uint32_t unit_code(const NintK &k, const uint32_t *q, uint32_t tail, int i) {
+    if (k.kind == 0) {
+        const int bit = i * k.bits;
+        const int w = bit >> 5, sh = bit & 31;
+        uint64_t v = q[w];
+        if (w + 1 < k.dwords) v |= static_cast<uint64_t>(q[w + 1]) << 32;
+        return static_cast<uint32_t>(v >> sh) & ((1u << k.bits) - 1u);
+    }
+    if (k.bits == 3 && i >= 20) {
+        if (i == 20) return tail & 7u;
+        if (i == 21) return (tail >> 3) & 7u;
+        const int h = (i == 23) ? 16 : 0;
+        return ((q[1] >> (15 + h)) & 1u) | (((tail >> (i == 23 ? 7 : 6)) & 1u) << 1) | (((q[0] >> (15 + h)) & 1u) << 2);
+    }
+    int w, b;
+    paired_pos(k.bits, i, w, b);
+    return (q[w] >> b) & ((1u << k.bits) - 1u);
+}
+
+// ---- repack ----------------------------------------------------------------------------
+__global__ void nint_repack_kernel(NintK k, const uint8_t *__restrict__ payload, int64_t payload_bytes, int legacy,
+                                   uint8_t *__restrict__ dst) {
+    const int lane = threadIdx.x;
+    const int rb = blockIdx.x, s = blockIdx.y;
+    const int r = lane & 15, kb = lane >> 4;
+    const int row = rb * 16 + r;
+    const int64_t out = k.out, ng = k.ng, gs = k.gs;
+    const int64_t sub_count = out * ng, q_count = out * ng * gs;
+    const int sb = legacy ? 8 : k.sub_bits, qb = legacy ? 8 : k.bits;
+    const int64_t ss_bytes = (sub_count * sb + 7) / 8, q_bytes = (q_count * qb + 7) / 8;
+    const uint8_t *ss_s = payload + 4 * out;
+    const uint8_t *sm_s = ss_s + ss_bytes;
+    const uint8_t *q_s = sm_s + ss_bytes;
+    uint8_t *sp = dst + rb * k.rowblock_bytes + s * k.step_bytes;
+    uint32_t *qreg = reinterpret_cast<uint32_t *>(sp);
+    uint8_t *treg = sp + 4 * 64 * k.dwords * 4;
+    uint8_t *sreg = treg + (k.tail ? 256 : 0);
+    for (int j = 0; j < 4; ++j) {
+        const int g = 16 * s + 4 * j + kb;
+        const bool live = row < k.out && g < k.ng;
+        uint32_t q[16];
+        for (int w = 0; w < k.dwords; ++w) q[w] = 0;
+        uint32_t tail = 0, ssv = 0, smv = 0;
+        if (live) {
+            const int64_t u = static_cast<int64_t>(row) * ng + g;
+            ssv = read_bits(ss_s, u, sb, ss_bytes);
+            smv = read_bits(sm_s, u, sb, ss_bytes);
+            for (int i = 0; i < k.gs; ++i) {
+                const uint32_t c = read_bits(q_s, u * gs + i, qb, q_bytes) & ((1u << k.bits) - 1u);
+                if (k.kind == 0) {
+                    const int bit = i * k.bits;
+                    const int w = bit >> 5, sh = bit & 31;
+                    q[w] |= c << sh;
+                    if (sh + k.bits > 32) q[w + 1] |= c >> (32 - sh);
+                } else if (k.bits == 3 && i >= 20) {
+                    if (i == 20) tail |= c;
+                    else if (i == 21) tail |= c << 3;
+                    else {
+                        const int h = (i == 23) ? 16 : 0;
+                        q[1] |= (c & 1u) << (15 + h);
+                        tail |= ((c >> 1) & 1u) << (i == 23 ? 7 : 6);
+                        q[0] |= ((c >> 2) & 1u) << (15 + h);
+                    }
+                } else {
+                    int w, b;
+                    paired_pos(k.bits, i, w, b);
+                    q[w] |= c << b;
+                }
+            }
+        }
+        for (int w = 0; w < k.dwords; ++w) qreg[(j * 64 + lane) * k.dwords + w] = q[w];
+        if (k.tail) treg[lane * 4 + j] = static_cast<uint8_t>(tail);
+        sreg[lane * 8 + 2 * j] = static_cast<uint8_t>(ssv);
+        sreg[lane * 8 + 2 * j + 1] = static_cast<uint8_t>(smv);
+    }
+    if (s == 0 && kb == 0) {
+        float *anchors = reinterpret_cast<float *>(dst + k.anchors_off);
+        const uint16_t *ns16 = reinterpret_cast<const uint16_t *>(payload);
+        const uint16_t *nm16 = ns16 + out;
+        const int out_pad = 16 * k.n_rowblocks;
+        anchors[row] = row < k.out ? f16_to_f32(ns16[row]) : 0.f;
+        anchors[out_pad + row] = row < k.out ? f16_to_f32(nm16[row]) : 0.f;
+    }
+}
+
+// ---- dequant (bit-exact: four separate fp32 roundings) -----------------------------------
+template <typename OutT>
+__global__ void nint_dequant_kernel(NintK k, const uint8_t *__restrict__ w, OutT *__restrict__ outp, int64_t ld,
+                                    float *__restrict__ rowscale, int kpad) {
+    const int lane = threadIdx.x;
+    const int rb = blockIdx.x, s = blockIdx.y;
+    const int r = lane & 15, kb = lane >> 4;
+    const int row = rb * 16 + r;
+    const uint8_t *sp = w + rb * k.rowblock_bytes + s * k.step_bytes;
+    const uint32_t *qreg = reinterpret_cast<const uint32_t *>(sp);
+    const uint8_t *treg = sp + 4 * 64 * k.dwords * 4;
+    const uint8_t *sreg = treg + (k.tail ? 256 : 0);
+    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
+    const int out_pad = 16 * k.n_rowblocks;
+    if (row >= k.out) return;
+    const float ns = anchors[row], nm = anchors[out_pad + row];
+    float inv = 1.f;
+    if constexpr (sizeof(OutT) == 2) {
+        // fp16 output is scaled per neuron by an exact power of two so the largest representable
+        // weight of the neuron lands near 2^12; the GEMM epilogue multiplies it back.
+        const float bound = ns * static_cast<float>(((1 << k.sub_bits) - 1) * ((1 << k.bits) - 1)) +
+                            nm * static_cast<float>((1 << k.sub_bits) - 1);
+        int e = 0;
+        if (bound > 0.f) { frexpf(bound, &e); }
+        inv = ldexpf(1.f, 12 - e);
+        if (s == 0 && kb == 0) {
+            rowscale[row] = ldexpf(1.f, e - 12);
+            for (int col = k.neuron_len; col < kpad; ++col) outp[row * ld + col] = 0;  // K padding of the GEMM
+        }
+    }
+    for (int j = 0; j < 4; ++j) {
+        const int g = 16 * s + 4 * j + kb;
+        if (g >= k.ng) continue;
+        uint32_t q[16];
+        for (int t = 0; t < k.dwords; ++t) q[t] = qreg[(j * 64 + lane) * k.dwords + t];
+        const uint32_t tail = k.tail ? treg[lane * 4 + j] : 0u;
+        const float ss = static_cast<float>(sreg[lane * 8 + 2 * j]);
+        const float sm = static_cast<float>(sreg[lane * 8 + 2 * j + 1]);
+        const float d_eff = __fmul_rn(ns, ss);
+        const float m_eff = __fmul_rn(nm, sm);
+        for (int i = 0; i < k.gs; ++i) {
+            const int col = g * k.gs + i;
+            if (col >= k.neuron_len) break;
+            const float qf = static_cast<float>(unit_code(k, q, tail, i));
+            const float v = __fsub_rn(__fmul_rn(d_eff, qf), m_eff);
+            if constexpr (sizeof(OutT) == 2) outp[row * ld + col] = f32_to_f16_rne(v * inv);
+            else outp[row * ld + col] = v;
+        }
+    }
+}
+
+// ---- GEMV ------------------------------------------------------------------------------
+template <int BITS, int GS, int XF16>
+struct PairedUnit {
+    static constexpr int D = (BITS == 3) ? 2 : GS * BITS / 32;
+    static constexpr bool TAIL = (BITS == 3);
+    static constexpr uint32_t MAGIC = XF16 ? 0x64006400u : 0x43004300u;
+    static constexpr float BIAS = XF16 ? 1024.f : 128.f;
+    static constexpr uint32_t FMASK = ((1u << BITS) - 1u) * 0x00010001u;
+    // sum_i (BIAS + code_i) * x_i over the group, xs = GS/2 activation pairs in LDS
+    __device__ static __forceinline__ float dot(const uint32_t (&q)[D], uint32_t tail, const uint32_t *xs) {
+        float acc = 0.f;
+        if constexpr (BITS == 3) {
+#pragma unroll
+            for (int d = 0; d < 2; ++d) {
+#pragma unroll
+                for (int p = 0; p < 5; ++p) {
+                    const uint32_t v = ((q[d] >> (3 * p)) & FMASK) | MAGIC;
+                    acc = dot2<XF16>(v, xs[5 * d + p], acc);
+                }
+            }
+            const uint32_t a = ((tail & 7u) | MAGIC) | ((tail & 0x38u) << 13);
+            acc = dot2<XF16>(a, xs[10], acc);
+            uint32_t b = ((q[1] >> 15) & 0x00010001u) | MAGIC;
+            b |= (q[0] >> 13) & 0x00040004u;
+            b |= ((tail >> 6) & 1u) << 1;
+            b |= ((tail >> 7) & 1u) << 17;
+            acc = dot2<XF16>(b, xs[11], acc);
+        } else {
+            constexpr int PER = 16 / BITS;
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+#pragma unroll
+                for (int p = 0; p < PER; ++p) {
+                    const uint32_t v = ((q[d] >> (BITS * p)) & FMASK) | MAGIC;
+                    acc = dot2<XF16>(v, xs[PER * d + p], acc);
+                }
+            }
+        }
+        return acc;
+    }
+};
+
+template <int BITS, int GS, int XF16, int MB>
+__global__ __launch_bounds__(1024) void nint_gemv_paired_kernel(NintK k, const uint8_t *__restrict__ w,
+                                                                const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                                float *__restrict__ y, int64_t ldy, int spw) {
+    using U = PairedUnit<BITS, GS, XF16>;
+    constexpr int D = U::D;
+    extern __shared__ uint32_t lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int rb = blockIdx.x, m0 = blockIdx.y * MB;
+    const int s0 = wave * spw;
+    const int s1 = min(k.nsteps, s0 + spw);
+    const int ngl = spw * 16, npairs = ngl * (GS / 2);
+    uint32_t *xs = lds + wave * (MB * (npairs + ngl));
+    float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
+    stage_x<XF16, MB>(x, ldx, M, m0, k.neuron_len, s0 * 16 * GS, npairs, GS, ngl, xs, xsum, lane);
+
+    const int r = lane & 15, kb = lane >> 4;
+    const uint8_t *base = w + rb * k.rowblock_bytes;
+    float accS[MB], accM[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) accS[m] = accM[m] = 0.f;
+    for (int s = s0; s < s1; ++s) {
+        const uint8_t *sp = base + s * k.step_bytes;
+        uint32_t q[4][D];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load_unit<D>(reinterpret_cast<const uint32_t *>(sp) + (j * 64 + lane) * D, q[j]);
+        uint32_t tails = 0;
+        if constexpr (U::TAIL) tails = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sp + 1024 * D) + lane);
+        const u32x2_t sc = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp + 1024 * D + (U::TAIL ? 256 : 0)) + lane);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int lg = (s - s0) * 16 + 4 * j + kb;
+            const uint32_t scw = (j < 2) ? sc.x : sc.y;
+            const float ss = ubyte_f32(scw, 2 * (j & 1));
+            const float sm = ubyte_f32(scw, 2 * (j & 1) + 1);
+            const uint32_t tail = (tails >> (8 * j)) & 0xffu;
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                const float raw = U::dot(q[j], tail, xs + m * npairs + lg * (GS / 2));
+                const float xg = xsum[m * ngl + lg];
+                accS[m] = fmaf(ss, fmaf(-U::BIAS, xg, raw), accS[m]);
+                accM[m] = fmaf(sm, xg, accM[m]);
+            }
+        }
+    }
+    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
+    const float ns = anchors[rb * 16 + r], nm = anchors[16 * k.n_rowblocks + rb * 16 + r];
+    float v[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) v[m] = ns * accS[m] - nm * accM[m];
+    finish_rows<MB>(v, reinterpret_cast<float *>(lds), wave, nwaves, lane, rb, k.out, M, m0, y, ldy);
+}
+
+// Any (bits, gs): natural-order units, one code at a time in fp32.
+template <int XF16, int MB>
+__global__ __launch_bounds__(1024) void nint_gemv_generic_kernel(NintK k, const uint8_t *__restrict__ w,
+                                                                 const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                                 float *__restrict__ y, int64_t ldy, int spw) {
+    extern __shared__ uint32_t lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int rb = blockIdx.x, m0 = blockIdx.y * MB;
+    const int s0 = wave * spw;
+    const int s1 = min(k.nsteps, s0 + spw);
+    const int gs = k.gs, ngl = spw * 16, npairs = ngl * gs / 2;
+    uint32_t *xs = lds + wave * (MB * (npairs + ngl));
+    float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
+    stage_x<XF16, MB>(x, ldx, M, m0, k.neuron_len, s0 * 16 * gs, npairs, gs, ngl, xs, xsum, lane);
+    const uint16_t *xh = reinterpret_cast<const uint16_t *>(xs);
+
+    const int r = lane & 15, kb = lane >> 4;
+    const uint8_t *base = w + rb * k.rowblock_bytes;
+    const uint32_t cmask = (1u << k.bits) - 1u;
+    float accS[MB], accM[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) accS[m] = accM[m] = 0.f;
+    for (int s = s0; s < s1; ++s) {
+        const uint8_t *sp = base + s * k.step_bytes;
+        const uint8_t *sreg = sp + 1024 * k.dwords;
+        for (int j = 0; j < 4; ++j) {
+            const int lg = (s - s0) * 16 + 4 * j + kb;
+            const uint32_t *q = reinterpret_cast<const uint32_t *>(sp) + (j * 64 + lane) * k.dwords;
+            const float ss = static_cast<float>(sreg[lane * 8 + 2 * j]);
+            const float sm = static_cast<float>(sreg[lane * 8 + 2 * j + 1]);
+            float raw[MB];
+#pragma unroll
+            for (int m = 0; m < MB; ++m) raw[m] = 0.f;
+            for (int i = 0; i < gs; ++i) {
+                const int bit = i * k.bits;
+                const int wi = bit >> 5, sh = bit & 31;
+                uint64_t v = q[wi];
+                if (wi + 1 < k.dwords) v |= static_cast<uint64_t>(q[wi + 1]) << 32;
+                const float c = static_cast<float>(static_cast<uint32_t>(v >> sh) & cmask);
+#pragma unroll
+                for (int m = 0; m < MB; ++m) raw[m] = fmaf(c, x_to_f32<XF16>(xh[2 * (m * npairs) + lg * gs + i]), raw[m]);
+            }
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                accS[m] = fmaf(ss, raw[m], accS[m]);
+                accM[m] = fmaf(sm, xsum[m * ngl + lg], accM[m]);
+            }
+        }
+    }
+    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
+    const float ns = anchors[rb * 16 + r], nm = anchors[16 * k.n_rowblocks + rb * 16 + r];
+    float v[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) v[m] = ns * accS[m] - nm * accM[m];
+    finish_rows<MB>(v, reinterpret_cast<float *>(lds), wave, nwaves, lane, rb, k.out, M, m0, y, ldy);
+}
+
+// steps per wave / waves per block so that the grid has a few thousand waves and LDS fits
+static void gemv_shape(const NintK &k, int mb, int &spw, int &nwaves, size_t &lds_bytes) {
+    int want = static_cast<int>(ceil_div(6144, k.n_rowblocks));
+    if (want < 1) want = 1;
+    if (want > 16) want = 16;
+    if (want > k.nsteps) want = k.nsteps;
+    spw = static_cast<int>(ceil_div(k.nsteps, want));
+    nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
+    const size_t per_wave = static_cast<size_t>(mb) * spw * 16 * (k.gs / 2 + 1) * 4;
+    lds_bytes = per_wave * nwaves;
+    const size_t red = static_cast<size_t>(nwaves) * mb * 16 * 4;
+    if (lds_bytes < red) lds_bytes = red;
+}
+
+template <int XF16, int MB>
+static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                          hipStream_t st) {
+    int spw, nwaves;
+    size_t lds;
+    gemv_shape(k, MB, spw, nwaves, lds);
+    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nint_gemv: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
+    const dim3 grid(k.n_rowblocks, static_cast<unsigned>(ceil_div(M, MB)));
+    const dim3 block(64 * nwaves);
+#define MFQ_PAIRED(B, G)                                                                                     \
+    if (k.bits == B && k.gs == G) {                                                                          \
+        hipLaunchKernelGGL((nint_gemv_paired_kernel<B, G, XF16, MB>), grid, block, lds, st, k, w, x, ldx, M, y, \
+                           ldy, spw);                                                                        \
+        return check_launch("nint_gemv_paired");                                                             \
+    }
+    if (k.kind == 1) {
+        MFQ_PAIRED(4, 32) MFQ_PAIRED(4, 24) MFQ_PAIRED(4, 16) MFQ_PAIRED(4, 48) MFQ_PAIRED(3, 24) MFQ_PAIRED(2, 16)
+        MFQ_PAIRED(2, 32)
+        return fail(MFQ_ERR_UNSUPPORTED, "nint_gemv: no paired kernel for NINT%d-%d", k.bits, k.gs);
+    }
+#undef MFQ_PAIRED
+    hipLaunchKernelGGL((nint_gemv_generic_kernel<XF16, MB>), grid, block, lds, st, k, w, x, ldx, M, y, ldy, spw);
+    return check_launch("nint_gemv_generic");
+}
+
+int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M, float *y,
+                  int64_t ldy, hipStream_t st) {
+    const NintK k = to_k(d);
+    const uint8_t *w = static_cast<const uint8_t *>(weight);
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    // LDS per block grows with MB; large K falls back to narrower row batches.
+    int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
+    for (;;) {
+        int spw, nwaves;
+        size_t lds;
+        gemv_shape(k, mb, spw, nwaves, lds);
+        if (lds <= 65536 || mb == 1) break;
+        mb >>= 1;
+    }
+    if (x_dtype == MFQ_X_F16) {
+        if (mb == 4) return launch_gemv_mb<1, 4>(k, w, xp, ldx, M, y, ldy, st);
+        if (mb == 2) return launch_gemv_mb<1, 2>(k, w, xp, ldx, M, y, ldy, st);
+        return launch_gemv_mb<1, 1>(k, w, xp, ldx, M, y, ldy, st);
+    }
+    if (mb == 4) return launch_gemv_mb<0, 4>(k, w, xp, ldx, M, y, ldy, st);
+    if (mb == 2) return launch_gemv_mb<0, 2>(k, w, xp, ldx, M, y, ldy, st);
+    return launch_gemv_mb<0, 1>(k, w, xp, ldx, M, y, ldy, st);
+}
+
+int nint_dequant_f16(const mfq_nint_desc *d, const void *weight, void *w16, int64_t ld, float *rowscale, hipStream_t st) {
+    const NintK k = to_k(d);
+    hipLaunchKernelGGL((nint_dequant_kernel<uint16_t>), dim3(k.n_rowblocks, k.nsteps), dim3(64), 0, st, k,
+                       static_cast<const uint8_t *>(weight), static_cast<uint16_t *>(w16), ld, rowscale,
+                       static_cast<int>(ld));
+    return check_launch("nint_dequant_f16");
+}
+
+}  // namespace mfq
+
+using namespace mfq;
+
+extern "C" int mfq_hip_nint_plan(int bits, int sub_bits, int gs, int out, int neuron_len, mfq_nint_desc *d) {
+    MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nint_plan: null descriptor");
+    MFQ_REQUIRE(bits >= 1 && bits <= 8, MFQ_ERR_UNSUPPORTED, "nint_plan: bits=%d outside [1,8]", bits);
+    MFQ_REQUIRE(sub_bits >= 1 && sub_bits <= 8, MFQ_ERR_UNSUPPORTED, "nint_plan: sub_bits=%d outside [1,8]", sub_bits);
+    MFQ_REQUIRE(gs >= 2 && gs <= 64 && gs % 2 == 0, MFQ_ERR_UNSUPPORTED, "nint_plan: groupsize=%d must be even and in [2,64]", gs);
+    MFQ_REQUIRE(out > 0 && neuron_len > 0, MFQ_ERR_INVALID, "nint_plan: empty tensor %dx%d", out, neuron_len);
+    d->bits = bits; d->sub_bits = sub_bits; d->gs = gs; d->out = out; d->neuron_len = neuron_len;
+    d->ng = static_cast<int32_t>(ceil_div(neuron_len, gs));
+    d->kind = paired_profile(bits, gs) ? 1 : 0;
+    if (d->kind == 1) {
+        d->dwords = bits == 3 ? 2 : gs * bits / 32;
+        d->tail_bytes = bits == 3 ? 1 : 0;
+    } else {
+        d->dwords = static_cast<int32_t>(ceil_div(gs * bits, 32));
+        d->tail_bytes = 0;
+    }
+    d->ngp = static_cast<int32_t>(ceil_div(d->ng, 16) * 16);
+    d->nsteps = d->ngp / 16;
+    d->n_rowblocks = static_cast<int32_t>(ceil_div(out, 16));
+    d->step_bytes = 64ll * (16 * d->dwords + (d->tail_bytes ? 4 : 0) + 8);
+    d->rowblock_bytes = d->step_bytes * d->nsteps;
+    d->anchors_off = d->rowblock_bytes * d->n_rowblocks;
+    d->total_bytes = d->anchors_off + 2ll * 16 * d->n_rowblocks * 4;
+    const int64_t subs = static_cast<int64_t>(out) * d->ng;
+    d->payload_bytes = 4ll * out + 2 * ((subs * sub_bits + 7) / 8) + (subs * gs * bits + 7) / 8;
+    return MFQ_OK;
+}
+
+extern "C" int mfq_hip_nint_repack(const mfq_nint_desc *d, const void *payload, int64_t payload_bytes, int legacy_bytes,
+                                   void *weight, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && payload && weight, MFQ_ERR_INVALID, "nint_repack: null argument");
+    const int64_t subs = static_cast<int64_t>(d->out) * d->ng;
+    const int64_t expect = legacy_bytes ? 4ll * d->out + 2 * subs + subs * d->gs : d->payload_bytes;
+    MFQ_REQUIRE(payload_bytes == expect, MFQ_ERR_INVALID, "invalid NINT blob tail: remaining=%lld, expected=%lld",
+                static_cast<long long>(payload_bytes), static_cast<long long>(expect));
+    const NintK k = to_k(d);
+    hipLaunchKernelGGL(nint_repack_kernel, dim3(k.n_rowblocks, k.nsteps), dim3(64), 0, as_stream(stream), k,
+                       static_cast<const uint8_t *>(payload), payload_bytes, legacy_bytes,
+                       static_cast<uint8_t *>(weight));
+    return check_launch("nint_repack");
+}
+
+extern "C" int mfq_hip_nint_dequant_f32(const mfq_nint_desc *d, const void *weight, float *w_out, int64_t ld,
+                                        mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && w_out, MFQ_ERR_INVALID, "nint_dequant_f32: null argument");
+    MFQ_REQUIRE(ld >= d->neuron_len, MFQ_ERR_INVALID, "nint_dequant_f32: ld %lld < neuron_len %d",
+                static_cast<long long>(ld), d->neuron_len);
+    const NintK k = to_k(d);
+    hipLaunchKernelGGL((nint_dequant_kernel<float>), dim3(k.n_rowblocks, k.nsteps), dim3(64), 0, as_stream(stream), k,
+                       static_cast<const uint8_t *>(weight), w_out, ld, static_cast<float *>(nullptr), 0);
+    return check_launch("nint_dequant_f32");
+}
+
+extern "C" int mfq_hip_nint_gemv(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                                 int M, float *y, int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nint_gemv: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nint_gemv: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint_gemv: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nint_gemv: ldx/ldy smaller than the tensor");
+    return nint_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, as_stream(stream));
+}

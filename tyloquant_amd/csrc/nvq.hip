@@ -1,0 +1,419 @@
+// NVQ-JSC, D4 family (4-dim magnitude vectors, 8/9-bit indices, 7-bit parity sign masks per
+// 8 weights, 4-bit joint scale/codebook state per 24 weights).
+//
+// Device layout: same row-block / step / lane interleave as NINT.  One (neuron, group) unit is
+// 80 bits = two dwords plus one halfword:
+//   d0 = idx0 | idx1 << IB | idx2 << 2IB | (mask2 & 31) << 27
+//   d1 = idx3 | idx4 << IB | idx5 << 2IB | state << 27
+//   h  = mask0 | mask1 << 7 | (mask2 >> 5) << 14
+// Step = Q [j][lane][2 dwords] then H [lane][4 halfwords].  The tensor tail holds
+//   float lut[16]; uint32 bank_for_state[16]; int8 codebooks[banks][entries][4]; float anchor[].
+// In the GEMV the codebook banks (as ready-made activation-typed pairs), a 128-entry table that
+// expands a sign mask (with its parity bit) into XOR masks, and the scale LUT all stay in LDS.
+#include "common.hpp"
+#include "gemv_common.hpp"
+
+namespace mfq {
+
+struct NvqK {
+    int ib, entries, banks, out, neuron_len, ng, nvec, nsign, nsteps, n_rowblocks;
+    int64_t step_bytes, rowblock_bytes, tables_off, anchors_off;
+};
+
+static NvqK to_k(const mfq_nvq_desc *d) {
+    NvqK k;
+    k.ib = d->index_bits; k.entries = d->entries; k.banks = d->banks; k.out = d->out; k.neuron_len = d->neuron_len;
+    k.ng = d->ng; k.nvec = d->nvec; k.nsign = d->nsign; k.nsteps = d->nsteps; k.n_rowblocks = d->n_rowblocks;
+    k.step_bytes = d->step_bytes; k.rowblock_bytes = d->rowblock_bytes; k.tables_off = d->tables_off;
+    k.anchors_off = d->anchors_off;
+    return k;
+}
+
+__device__ __forceinline__ uint32_t parity8(uint32_t m7) { return m7 | ((__popc(m7) & 1u) << 7); }
+
+// ---- repack ----------------------------------------------------------------------------
+// `body` points at the anchors; `lut_src` is the fp16 LUT of the JSC header or null (plain NVQ:
+// lut[s] = s); `bank_src` the 16 state->bank bytes or null (all zero); `cb_src` the int8 banks.
+__global__ void nvq_repack_kernel(NvqK k, const uint8_t *__restrict__ body, int64_t body_bytes,
+                                  const uint16_t *__restrict__ lut_src, const uint8_t *__restrict__ bank_src,
+                                  const int8_t *__restrict__ cb_src, uint8_t *__restrict__ dst) {
+    const int lane = threadIdx.x;
+    const int rb = blockIdx.x, s = blockIdx.y;
+    const int r = lane & 15, kb = lane >> 4;
+    const int row = rb * 16 + r;
+    const int64_t out = k.out;
+    const int64_t st_bytes = (out * k.ng * 4 + 7) / 8, ix_bytes = (out * k.nvec * k.ib + 7) / 8,
+                  sg_bytes = (out * k.nsign * 7 + 7) / 8;
+    const uint8_t *st_s = body + 2 * out;
+    const uint8_t *ix_s = st_s + st_bytes;
+    const uint8_t *sg_s = ix_s + ix_bytes;
+    uint8_t *sp = dst + rb * k.rowblock_bytes + s * k.step_bytes;
+    uint32_t *qreg = reinterpret_cast<uint32_t *>(sp);
+    uint16_t *hreg = reinterpret_cast<uint16_t *>(sp + 2048);
+    for (int j = 0; j < 4; ++j) {
+        const int g = 16 * s + 4 * j + kb;
+        uint32_t d0 = 0, d1 = 0, h = 0;
+        if (row < k.out && g < k.ng) {
+            uint32_t idx[6], m[3];
+            for (int t = 0; t < 6; ++t) {
+                const int v = 6 * g + t;
+                idx[t] = v < k.nvec ? read_bits(ix_s, static_cast<int64_t>(row) * k.nvec + v, k.ib, ix_bytes) : 0u;
+            }
+            for (int t = 0; t < 3; ++t) {
+                const int u = 3 * g + t;
+                m[t] = u < k.nsign ? read_bits(sg_s, static_cast<int64_t>(row) * k.nsign + u, 7, sg_bytes) : 0u;
+            }
+            const uint32_t state = read_bits(st_s, static_cast<int64_t>(row) * k.ng + g, 4, st_bytes);
+            d0 = idx[0] | (idx[1] << k.ib) | (idx[2] << (2 * k.ib)) | ((m[2] & 31u) << 27);
+            d1 = idx[3] | (idx[4] << k.ib) | (idx[5] << (2 * k.ib)) | (state << 27);
+            h = m[0] | (m[1] << 7) | ((m[2] >> 5) << 14);
+        }
+        qreg[(j * 64 + lane) * 2] = d0;
+        qreg[(j * 64 + lane) * 2 + 1] = d1;
+        hreg[lane * 4 + j] = static_cast<uint16_t>(h);
+    }
+    if (s == 0 && kb == 0) {
+        float *anchors = reinterpret_cast<float *>(dst + k.anchors_off);
+        anchors[row] = row < k.out ? f16_to_f32(reinterpret_cast<const uint16_t *>(body)[row]) : 0.f;
+    }
+    if (rb == 0 && s == 0) {
+        float *lut = reinterpret_cast<float *>(dst + k.tables_off);
+        uint32_t *bfs = reinterpret_cast<uint32_t *>(lut + 16);
+        int8_t *cb = reinterpret_cast<int8_t *>(bfs + 16);
+        if (lane < 16) {
+            lut[lane] = lut_src ? f16_to_f32(lut_src[lane]) : static_cast<float>(lane);
+            bfs[lane] = bank_src ? bank_src[lane] : 0u;
+        }
+        const int n = k.banks * k.entries * 4;
+        for (int i = lane; i < n; i += 64) cb[i] = cb_src[i];
+    }
+}
+
+struct NvqUnit {
+    uint32_t idx[6], mask[3], state;
+};
+__device__ __forceinline__ NvqUnit nvq_decode(int ib, uint32_t d0, uint32_t d1, uint32_t h) {
+    NvqUnit u;
+    const uint32_t im = (1u << ib) - 1u;
+    u.idx[0] = d0 & im; u.idx[1] = (d0 >> ib) & im; u.idx[2] = (d0 >> (2 * ib)) & im;
+    u.idx[3] = d1 & im; u.idx[4] = (d1 >> ib) & im; u.idx[5] = (d1 >> (2 * ib)) & im;
+    u.mask[0] = h & 127u; u.mask[1] = (h >> 7) & 127u; u.mask[2] = ((d0 >> 27) & 31u) | ((h >> 14) << 5);
+    u.state = (d1 >> 27) & 15u;
+    return u;
+}
+
+// ---- dequant: f32(mag * sign) * fl(anchor * lut[state]) ------------------------------------
+template <typename OutT>
+__global__ void nvq_dequant_kernel(NvqK k, const uint8_t *__restrict__ w, OutT *__restrict__ outp, int64_t ld,
+                                   float *__restrict__ rowscale, int kpad) {
+    const int lane = threadIdx.x;
+    const int rb = blockIdx.x, s = blockIdx.y;
+    const int r = lane & 15, kb = lane >> 4;
+    const int row = rb * 16 + r;
+    if (row >= k.out) return;
+    const uint8_t *sp = w + rb * k.rowblock_bytes + s * k.step_bytes;
+    const uint32_t *qreg = reinterpret_cast<const uint32_t *>(sp);
+    const uint16_t *hreg = reinterpret_cast<const uint16_t *>(sp + 2048);
+    const float *lut = reinterpret_cast<const float *>(w + k.tables_off);
+    const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+    const int8_t *cb = reinterpret_cast<const int8_t *>(bfs + 16);
+    const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[row];
+    float inv = 1.f;
+    if constexpr (sizeof(OutT) == 2) {
+        float lmax = 0.f;
+        for (int i = 0; i < 16; ++i) lmax = fmaxf(lmax, lut[i]);
+        const float bound = anchor * lmax * 127.f;
+        int e = 0;
+        if (bound > 0.f) frexpf(bound, &e);
+        inv = ldexpf(1.f, 12 - e);
+        if (s == 0 && kb == 0) {
+            rowscale[row] = ldexpf(1.f, e - 12);
+            for (int col = k.neuron_len; col < kpad; ++col) outp[row * ld + col] = 0;
+        }
+    }
+    for (int j = 0; j < 4; ++j) {
+        const int g = 16 * s + 4 * j + kb;
+        if (g >= k.ng) continue;
+        const NvqUnit u = nvq_decode(k.ib, qreg[(j * 64 + lane) * 2], qreg[(j * 64 + lane) * 2 + 1], hreg[lane * 4 + j]);
+        const float scale = __fmul_rn(anchor, lut[u.state]);
+        const int8_t *bank = cb + static_cast<int64_t>(bfs[u.state]) * k.entries * 4;
+        for (int i = 0; i < 24; ++i) {
+            const int col = g * 24 + i;
+            if (col >= k.neuron_len) break;
+            const int mag = bank[u.idx[i >> 2] * 4 + (i & 3)];
+            const uint32_t m8 = parity8(u.mask[i >> 3]);
+            const float sv = ((m8 >> (i & 7)) & 1u) ? -static_cast<float>(mag) : static_cast<float>(mag);
+            const float v = __fmul_rn(sv, scale);
+            if constexpr (sizeof(OutT) == 2) outp[row * ld + col] = f32_to_f16_rne(v * inv);
+            else outp[row * ld + col] = v;
+        }
+    }
+}
+
+// ---- GEMV ------------------------------------------------------------------------------
+// LDS map (dwords): [codebook pairs: banks*entries*2][sign xor table: 128*4][lut: 16][bank: 16][x staging ...]
+template <int XF16, int MB>
+__global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *__restrict__ w,
+                                                        const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                        float *__restrict__ y, int64_t ldy, int spw) {
+    extern __shared__ uint32_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int rb = blockIdx.x, m0 = blockIdx.y * MB;
+    const int ncb = k.banks * k.entries;
+    uint32_t *cbp = lds;                 // 2 dwords per entry: (m0, m1), (m2, m3) in the activation type
+    uint32_t *sgx = cbp + 2 * ncb;       // 4 dwords per 7-bit mask
+    float *lutf = reinterpret_cast<float *>(sgx + 512);
+    uint32_t *bankoff = reinterpret_cast<uint32_t *>(lutf + 16);
+    uint32_t *xbase = bankoff + 16;
+    {
+        const float *lut = reinterpret_cast<const float *>(w + k.tables_off);
+        const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+        const uint32_t *cb = bfs + 16;  // 4 int8 magnitudes per entry
+        for (int i = tid; i < ncb; i += blockDim.x) {
+            const uint32_t e = cb[i];
+            uint32_t h[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const float f = static_cast<float>((e >> (8 * t)) & 0xffu);
+                h[t] = XF16 ? f32_to_f16_rne(f) : f32_to_bf16_rne(f);
+            }
+            cbp[2 * i] = h[0] | (h[1] << 16);
+            cbp[2 * i + 1] = h[2] | (h[3] << 16);
+        }
+        for (int i = tid; i < 128; i += blockDim.x) {
+            const uint32_t m8 = parity8(i);
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+                sgx[4 * i + p] = (((m8 >> (2 * p)) & 1u) << 15) | (((m8 >> (2 * p + 1)) & 1u) << 31);
+        }
+        if (tid < 16) {
+            lutf[tid] = lut[tid];
+            bankoff[tid] = bfs[tid] * k.entries * 2;
+        }
+    }
+    const int s0 = wave * spw;
+    const int s1 = min(k.nsteps, s0 + spw);
+    const int ngl = spw * 16, npairs = ngl * 12;
+    uint32_t *xs = xbase + wave * (MB * (npairs + ngl));
+    float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
+    stage_x<XF16, MB>(x, ldx, M, m0, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane);
+
+    const int r = lane & 15, kb = lane >> 4;
+    const uint8_t *base = w + rb * k.rowblock_bytes;
+    const uint32_t im = (1u << k.ib) - 1u;
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = 0.f;
+    for (int s = s0; s < s1; ++s) {
+        const uint8_t *sp = base + s * k.step_bytes;
+        u32x2_t q[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) q[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp) + j * 64 + lane);
+        const u32x2_t hh = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp + 2048) + lane);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int lg = (s - s0) * 16 + 4 * j + kb;
+            const uint32_t d0 = q[j].x, d1 = q[j].y;
+            const uint32_t h = ((j < 2 ? hh.x : hh.y) >> (16 * (j & 1))) & 0xffffu;
+            const uint32_t state = (d1 >> 27) & 15u;
+            const uint32_t *bank = cbp + bankoff[state];
+            const float sc = lutf[state];
+            const uint32_t mk[3] = {h & 127u, (h >> 7) & 127u, ((d0 >> 27) & 31u) | ((h >> 14) << 5)};
+            const uint32_t ix[6] = {d0 & im, (d0 >> k.ib) & im, (d0 >> (2 * k.ib)) & im,
+                                    d1 & im, (d1 >> k.ib) & im, (d1 >> (2 * k.ib)) & im};
+            float raw[MB];
+#pragma unroll
+            for (int m = 0; m < MB; ++m) raw[m] = 0.f;
+#pragma unroll
+            for (int v = 0; v < 3; ++v) {
+                const u32x4_t sx = *reinterpret_cast<const u32x4_t *>(sgx + 4 * mk[v]);
+                const u32x2_t c0 = *reinterpret_cast<const u32x2_t *>(bank + 2 * ix[2 * v]);
+                const u32x2_t c1 = *reinterpret_cast<const u32x2_t *>(bank + 2 * ix[2 * v + 1]);
+                const uint32_t w0 = c0.x ^ sx.x, w1 = c0.y ^ sx.y, w2 = c1.x ^ sx.z, w3 = c1.y ^ sx.w;
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+                    const uint32_t *xp = xs + m * npairs + lg * 12 + 4 * v;
+                    raw[m] = dot2<XF16>(w0, xp[0], raw[m]);
+                    raw[m] = dot2<XF16>(w1, xp[1], raw[m]);
+                    raw[m] = dot2<XF16>(w2, xp[2], raw[m]);
+                    raw[m] = dot2<XF16>(w3, xp[3], raw[m]);
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < MB; ++m) acc[m] = fmaf(sc, raw[m], acc[m]);
+        }
+    }
+    const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[rb * 16 + r];
+    float v[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) v[m] = anchor * acc[m];
+    finish_rows<MB>(v, reinterpret_cast<float *>(xbase), wave, nwaves, lane, rb, k.out, M, m0, y, ldy);
+}
+
+static void nvq_gemv_shape(const NvqK &k, int mb, int &spw, int &nwaves, size_t &lds_bytes) {
+    int want = static_cast<int>(ceil_div(6144, k.n_rowblocks));
+    if (want < 1) want = 1;
+    if (want > 16) want = 16;
+    if (want > k.nsteps) want = k.nsteps;
+    spw = static_cast<int>(ceil_div(k.nsteps, want));
+    nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
+    size_t xb = static_cast<size_t>(mb) * spw * 16 * 13 * 4 * nwaves;
+    const size_t red = static_cast<size_t>(nwaves) * mb * 16 * 4;
+    if (xb < red) xb = red;
+    lds_bytes = (static_cast<size_t>(k.banks) * k.entries * 2 + 512 + 32) * 4 + xb;
+}
+
+template <int XF16, int MB>
+static int nvq_launch(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                      hipStream_t st) {
+    int spw, nwaves;
+    size_t lds;
+    nvq_gemv_shape(k, MB, spw, nwaves, lds);
+    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nvq_gemv: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
+    hipLaunchKernelGGL((nvq_gemv_kernel<XF16, MB>), dim3(k.n_rowblocks, static_cast<unsigned>(ceil_div(M, MB))),
+                       dim3(64 * nwaves), lds, st, k, w, x, ldx, M, y, ldy, spw);
+    return check_launch("nvq_gemv");
+}
+
+static int nvq_gemv_any(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
+                        float *y, int64_t ldy, hipStream_t st) {
+    const NvqK k = to_k(d);
+    const uint8_t *w = static_cast<const uint8_t *>(weight);
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
+    for (;;) {
+        int spw, nwaves;
+        size_t lds;
+        nvq_gemv_shape(k, mb, spw, nwaves, lds);
+        if (lds <= 65536 || mb == 1) break;
+        mb >>= 1;
+    }
+    if (x_dtype == MFQ_X_F16) {
+        if (mb == 4) return nvq_launch<1, 4>(k, w, xp, ldx, M, y, ldy, st);
+        if (mb == 2) return nvq_launch<1, 2>(k, w, xp, ldx, M, y, ldy, st);
+        return nvq_launch<1, 1>(k, w, xp, ldx, M, y, ldy, st);
+    }
+    if (mb == 4) return nvq_launch<0, 4>(k, w, xp, ldx, M, y, ldy, st);
+    if (mb == 2) return nvq_launch<0, 2>(k, w, xp, ldx, M, y, ldy, st);
+    return nvq_launch<0, 1>(k, w, xp, ldx, M, y, ldy, st);
+}
+
+int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, const float *sa,
+                const float *sb, float *y, int64_t ldy, hipStream_t st);
+int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, hipStream_t st);
+size_t dequant_gemm_workspace(int N, int K, int M);
+void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&xscale, uint16_t *&w16, float *&wscale,
+                        int &Kp);
+
+}  // namespace mfq
+
+using namespace mfq;
+
+extern "C" int mfq_hip_nvq_plan(int index_bits, int banks, int out, int neuron_len, mfq_nvq_desc *d) {
+    MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nvq_plan: null descriptor");
+    MFQ_REQUIRE(index_bits == 8 || index_bits == 9, MFQ_ERR_UNSUPPORTED,
+                "nvq_plan: only the D4 256/512-entry codebooks are on the accelerated path (index_bits=%d)", index_bits);
+    MFQ_REQUIRE(banks == 1 || banks == 2 || banks == 4, MFQ_ERR_INVALID, "nvq_plan: banks=%d", banks);
+    MFQ_REQUIRE(out > 0 && neuron_len > 0, MFQ_ERR_INVALID, "nvq_plan: empty tensor");
+    d->index_bits = index_bits; d->entries = 1 << index_bits; d->banks = banks; d->out = out; d->neuron_len = neuron_len;
+    d->ng = static_cast<int32_t>(ceil_div(neuron_len, 24));
+    d->nvec = static_cast<int32_t>(ceil_div(neuron_len, 4));
+    d->nsign = static_cast<int32_t>(ceil_div(neuron_len, 8));
+    d->ngp = static_cast<int32_t>(ceil_div(d->ng, 16) * 16);
+    d->nsteps = d->ngp / 16;
+    d->n_rowblocks = static_cast<int32_t>(ceil_div(out, 16));
+    d->step_bytes = 2048 + 512;
+    d->rowblock_bytes = d->step_bytes * d->nsteps;
+    d->tables_off = d->rowblock_bytes * d->n_rowblocks;
+    d->anchors_off = d->tables_off + 128 + static_cast<int64_t>(banks) * d->entries * 4;
+    d->total_bytes = d->anchors_off + 16ll * d->n_rowblocks * 4;
+    const int64_t o = out;
+    d->payload_bytes = 2 * o + (o * d->ng * 4 + 7) / 8 + (o * d->nvec * index_bits + 7) / 8 + (o * d->nsign * 7 + 7) / 8 +
+                       64 + static_cast<int64_t>(banks) * d->entries * 4;
+    return MFQ_OK;
+}
+
+static int64_t nvq_stream_bytes(const mfq_nvq_desc *d) {
+    const int64_t o = d->out;
+    return 2 * o + (o * d->ng * 4 + 7) / 8 + (o * d->nvec * d->index_bits + 7) / 8 + (o * d->nsign * 7 + 7) / 8;
+}
+
+extern "C" int mfq_hip_nvq_repack(const mfq_nvq_desc *d, const void *payload, int64_t payload_bytes, void *weight,
+                                  mfq_stream_t stream) {
+    MFQ_REQUIRE(d && payload && weight, MFQ_ERR_INVALID, "nvq_repack: null argument");
+    const int64_t cbb = static_cast<int64_t>(d->banks) * d->entries * 4;
+    const int64_t expect = 64 + cbb + nvq_stream_bytes(d);
+    MFQ_REQUIRE(payload_bytes == expect, MFQ_ERR_INVALID, "invalid NVQ-JSC blob tail: size=%lld, expected=%lld",
+                static_cast<long long>(payload_bytes), static_cast<long long>(expect));
+    const NvqK k = to_k(d);
+    const uint8_t *p = static_cast<const uint8_t *>(payload);
+    hipLaunchKernelGGL(nvq_repack_kernel, dim3(k.n_rowblocks, k.nsteps), dim3(64), 0, as_stream(stream), k, p + 64 + cbb,
+                       nvq_stream_bytes(d), reinterpret_cast<const uint16_t *>(p + 4), p + 36,
+                       reinterpret_cast<const int8_t *>(p + 64), static_cast<uint8_t *>(weight));
+    return check_launch("nvq_repack");
+}
+
+extern "C" int mfq_hip_nvq_repack_plain(const mfq_nvq_desc *d, const void *payload, int64_t payload_bytes,
+                                        const void *grid, void *weight, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && payload && weight && grid, MFQ_ERR_INVALID, "nvq_repack_plain: null argument");
+    MFQ_REQUIRE(d->banks == 1, MFQ_ERR_INVALID, "nvq_repack_plain: plain NVQ has one codebook bank");
+    MFQ_REQUIRE(payload_bytes == nvq_stream_bytes(d), MFQ_ERR_INVALID, "invalid NVQ blob tail: size=%lld, expected=%lld",
+                static_cast<long long>(payload_bytes), static_cast<long long>(nvq_stream_bytes(d)));
+    const NvqK k = to_k(d);
+    hipLaunchKernelGGL(nvq_repack_kernel, dim3(k.n_rowblocks, k.nsteps), dim3(64), 0, as_stream(stream), k,
+                       static_cast<const uint8_t *>(payload), payload_bytes, static_cast<const uint16_t *>(nullptr),
+                       static_cast<const uint8_t *>(nullptr), static_cast<const int8_t *>(grid),
+                       static_cast<uint8_t *>(weight));
+    return check_launch("nvq_repack_plain");
+}
+
+extern "C" int mfq_hip_nvq_dequant_f32(const mfq_nvq_desc *d, const void *weight, float *w_out, int64_t ld,
+                                       mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && w_out, MFQ_ERR_INVALID, "nvq_dequant_f32: null argument");
+    MFQ_REQUIRE(ld >= d->neuron_len, MFQ_ERR_INVALID, "nvq_dequant_f32: ld smaller than neuron_len");
+    const NvqK k = to_k(d);
+    hipLaunchKernelGGL((nvq_dequant_kernel<float>), dim3(k.n_rowblocks, k.nsteps), dim3(64), 0, as_stream(stream), k,
+                       static_cast<const uint8_t *>(weight), w_out, ld, static_cast<float *>(nullptr), 0);
+    return check_launch("nvq_dequant_f32");
+}
+
+extern "C" int mfq_hip_nvq_gemv(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
+                                float *y, int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nvq_gemv: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nvq_gemv: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvq_gemv: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nvq_gemv: ldx/ldy smaller than the tensor");
+    return nvq_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, as_stream(stream));
+}
+
+static constexpr int kNvqGemvMaxM = 13;  // the reference keeps the D4 family on its GEMV up to M = 13
+
+extern "C" size_t mfq_hip_nvq_gemm_workspace_bytes(const mfq_nvq_desc *d, int M) {
+    if (!d || M <= kNvqGemvMaxM) return 0;
+    return dequant_gemm_workspace(d->out, d->neuron_len, M);
+}
+
+extern "C" int mfq_hip_nvq_gemm(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
+                                float *y, int64_t ldy, void *workspace, size_t workspace_bytes, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nvq_gemm: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nvq_gemm: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvq_gemm: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nvq_gemm: ldx/ldy smaller than the tensor");
+    hipStream_t st = as_stream(stream);
+    if (M <= kNvqGemvMaxM) return nvq_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, st);
+    const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
+    MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nvq_gemm: workspace %zu < %zu bytes",
+                workspace_bytes, need);
+    uint16_t *x16, *w16;
+    float *xscale, *wscale;
+    int Kp;
+    dequant_gemm_carve(workspace, d->out, d->neuron_len, M, x16, xscale, w16, wscale, Kp);
+    int rc = x_prep(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, st);
+    if (rc) return rc;
+    const NvqK k = to_k(d);
+    hipLaunchKernelGGL((nvq_dequant_kernel<uint16_t>), dim3(k.n_rowblocks, k.nsteps), dim3(64), 0, st, k,
+                       static_cast<const uint8_t *>(weight), w16, static_cast<int64_t>(Kp), wscale, Kp);
+    rc = check_launch("nvq_dequant_f16");
+    if (rc) return rc;
+    return gemm_f16_nt(x16, Kp, w16, Kp, M, d->out, Kp, xscale, wscale, y, ldy, st);
+}

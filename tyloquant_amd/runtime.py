@@ -1,0 +1,200 @@
+"""Python twin of the host dispatch layer: weight objects, the dtype-string registry and the
+matmul entry points, over the C ABI of libmfq_hip.so.
+
+Mirrors the reference's operator surface for this path (names, argument meaning, errors):
+  load_quant_linear / is_nint_linear_dtype / is_nvq_linear_dtype  cpp_runtime/mfq_decode.cpp:9409-9420, 9489-9771
+  NintWeight / nint_matmul                                         cpp_runtime/mfq_decode.cpp:2101-2165, 8130-8315
+  NvqWeight / nvq_matmul                                           cpp_runtime/mfq_decode.cpp:4019-4150, 7884-7931
+  NepqWeight / nepq_matmul                                         mfq/kernels/cuda/nepq_matmul.py:215-280
+  NintMoeWeight / MoeRoutePlan / build_moe_route_plan / nint_moe_ffn_forward
+                                                                   cpp_runtime/mfq_decode.cpp:2579-2592, 2681-2708, 2908-3071, 3394-3416
+torch is used only to own device memory and to name the current stream; every computation is a
+HIP kernel behind the C ABI, and nothing here falls back to the CPU.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import _lib as L
+from . import formats as F
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _x_dtype(x: torch.Tensor) -> int:
+    if x.dtype == torch.bfloat16:
+        return L.X_BF16
+    if x.dtype == torch.float16:
+        return L.X_F16
+    raise TypeError(f"activations must be bfloat16 or float16, got {x.dtype}")
+
+
+def _as_2d(x: torch.Tensor, K: int) -> torch.Tensor:
+    if x.shape[-1] != K:
+        raise ValueError(f"activation width {x.shape[-1]} != neuron length {K}")
+    x2 = x.reshape(-1, K)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    return x2
+
+
+def _upload(blob, off: int, nbytes: int, device) -> torch.Tensor:
+    arr = np.frombuffer(blob, dtype=np.uint8, count=nbytes, offset=off)
+    return torch.from_numpy(arr.copy()).to(device, non_blocking=False)
+
+
+class _Workspace:
+    """Grow-only device scratch, cached per weight like the reference's per-M workspaces
+    (cpp_runtime/mfq_decode.cpp:2120-2132)."""
+
+    def __init__(self):
+        self.buf = None
+
+    def get(self, nbytes: int, device) -> torch.Tensor | None:
+        if nbytes == 0:
+            return None
+        if self.buf is None or self.buf.numel() < nbytes or self.buf.device != device:
+            self.buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        return self.buf
+
+
+# ---------------------------------------------------------------------------------------
+# NINT
+# ---------------------------------------------------------------------------------------
+class NintWeight:
+    def __init__(self, desc: L.NintDesc, data: torch.Tensor, shape):
+        self.desc, self.data, self.shape = desc, data, tuple(shape)
+        self.out, self.neuron_len = desc.out, desc.neuron_len
+        self.bits, self.gs, self.ng = desc.bits, desc.gs, desc.ng
+        self._ws = _Workspace()
+
+    @property
+    def payload_bytes(self) -> int:
+        return int(self.desc.payload_bytes)
+
+    @staticmethod
+    def from_blob(blob, device="cuda") -> "NintWeight":
+        h = F.parse_nint(blob)
+        if h.axis != 0:
+            raise ValueError("NINT linear weights must be quantized along axis 0")
+        desc = L.NintDesc()
+        L.check(L.lib().mfq_hip_nint_plan(h.bits, h.sub_bits, h.gs, h.out, h.neuron_len, C.byref(desc)))
+        device = torch.device(device)
+        payload = _upload(blob, h.body_off, h.body_bytes, device)
+        data = torch.empty(int(desc.total_bytes), dtype=torch.uint8, device=device)
+        L.check(L.lib().mfq_hip_nint_repack(C.byref(desc), _ptr(payload), h.body_bytes, int(h.legacy), _ptr(data),
+                                            _stream()))
+        torch.cuda.current_stream().synchronize()  # payload may be freed after this
+        return NintWeight(desc, data, h.shape)
+
+    def dequantize(self) -> torch.Tensor:
+        w = torch.empty((self.out, self.neuron_len), dtype=torch.float32, device=self.data.device)
+        L.check(L.lib().mfq_hip_nint_dequant_f32(C.byref(self.desc), _ptr(self.data), _ptr(w), self.neuron_len,
+                                                 _stream()))
+        return w
+
+
+def nint_matmul(w: NintWeight, x: torch.Tensor, *, force: str | None = None) -> torch.Tensor:
+    """y[..., out] = x[..., K] @ W^T in fp32 (cpp_runtime/mfq_decode.cpp:8130).  `force` = "gemv"
+    or "gemm" pins the kernel family (the reference's MFQ_* path overrides)."""
+    x2 = _as_2d(x, w.neuron_len)
+    M = x2.shape[0]
+    y = torch.empty((M, w.out), dtype=torch.float32, device=x.device)
+    lib = L.lib()
+    if force == "gemv":
+        L.check(lib.mfq_hip_nint_gemv(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
+                                      w.out, _stream()))
+    else:
+        Mq = max(M, 9) if force == "gemm" else M
+        need = lib.mfq_hip_nint_gemm_workspace_bytes(C.byref(w.desc), Mq)
+        ws = w._ws.get(need, x.device)
+        if force == "gemm" and M < 9:
+            raise ValueError("force='gemm' needs at least 9 activation rows")
+        L.check(lib.mfq_hip_nint_gemm(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
+                                      w.out, _ptr(ws), need, _stream()))
+    return y.reshape(*x.shape[:-1], w.out)
+
+
+# ---------------------------------------------------------------------------------------
+# dtype registry
+# ---------------------------------------------------------------------------------------
+def is_nint_linear_dtype(dtype: str) -> bool:
+    """NINT<bits> for any bit width (cpp_runtime/mfq_decode.cpp:9409-9412); NINT8-0 and NINTM are
+    separate families."""
+    return dtype.startswith("NINT") and dtype[4:].isdigit()
+
+
+def is_nvq_linear_dtype(dtype: str) -> bool:
+    return dtype in ("NVQ3", "NVQ3J", "NVQ3J-512", "NIQ3")
+
+
+def is_nepq_linear_dtype(dtype: str) -> bool:
+    return dtype in ("NEPQ1-S", "NEPQ1-L")
+
+
+@dataclass
+class QuantLinear:
+    kind: str
+    weight: object
+
+    @property
+    def out(self):
+        return self.weight.out
+
+    @property
+    def neuron_len(self):
+        return self.weight.neuron_len
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return _MATMUL[self.kind](self.weight, x)
+
+    __call__ = forward
+
+    def dequantize(self) -> torch.Tensor:
+        return self.weight.dequantize()
+
+
+def load_quant_linear(dtype: str, blob, device="cuda") -> QuantLinear:
+    """Switch on the MFQ dtype string and build the device weight (cpp_runtime/mfq_decode.cpp:9489-9771)."""
+    dtype = {"NIQ3": "NVQ3"}.get(dtype, dtype)
+    if is_nint_linear_dtype(dtype):
+        w = NintWeight.from_blob(blob, device)
+        if f"NINT{w.bits}" != dtype:
+            raise ValueError(f"MFQ dtype/blob mismatch: {dtype} contains NINT{w.bits}")
+        return QuantLinear("nint", w)
+    if is_nvq_linear_dtype(dtype):
+        from .runtime_vq import NvqWeight
+        w = NvqWeight.from_blob(blob, device)
+        if w.dtype != dtype:
+            raise ValueError(f"MFQ dtype/blob mismatch: {dtype} contains {w.dtype}")
+        return QuantLinear("nvq", w)
+    if is_nepq_linear_dtype(dtype):
+        from .runtime_vq import NepqWeight
+        w = NepqWeight.from_blob(blob, device)
+        if w.label != dtype:
+            raise ValueError(f"MFQ dtype/blob mismatch: {dtype} contains {w.label}")
+        return QuantLinear("nepq", w)
+    raise ValueError(f"unsupported quantized linear dtype: {dtype}")
+
+
+def _nvq_mm(w, x):
+    from .runtime_vq import nvq_matmul
+    return nvq_matmul(w, x)
+
+
+def _nepq_mm(w, x):
+    from .runtime_vq import nepq_matmul
+    return nepq_matmul(w, x)
+
+
+_MATMUL = {"nint": nint_matmul, "nvq": _nvq_mm, "nepq": _nepq_mm}
