@@ -137,7 +137,7 @@ typedef struct mfq_nepq_desc {
 } mfq_nepq_desc;
 
 int mfq_hip_nepq_plan(int profile, int banks, int rows, int neuron_len, mfq_nepq_desc *d);
-/* `payload` = device copy of the blob after the 40-byte header (mfq/formats/nepq.py:368-399):
+/* `payload` = device copy of the blob after the 36-byte header (mfq/formats/nepq.py:368-399):
  * tables u8[banks, table_bytes], anchors f16[rows], state / index / aux bit streams, bank ids. */
 int mfq_hip_nepq_repack(const mfq_nepq_desc *d, const void *payload, int64_t payload_bytes, void *weight,
                         mfq_stream_t stream);
@@ -187,14 +187,17 @@ typedef struct mfq_moe_pool {
  * routed_input != 0 (x is [T*R, K]) else pair / R (x is [T, K]).  Invalid expert ids give zero rows.
  * Replaces nint_moe_grouped_matmul_hetero_qx_cuda / _hetero_f16_cuda / _pool_ws_cuda
  * (cpp_runtime/mfq_decode.cpp:248-290; mfq/kernels/cuda/moe.cu:3971-4345). */
-size_t mfq_hip_moe_grouped_workspace_bytes(int n_pairs, int K, int out_per_expert);
+/* Routes of one expert are batched mfq_hip_moe_tile_m() at a time by the mapped path: build the
+ * route map with that tile_m.  Pass ids_dst == NULL (and NULL tables) to run every pair on its own
+ * (decode, T*R small). */
+int mfq_hip_moe_tile_m(void);
 int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools, const int32_t *expert_pool,
                                const int32_t *expert_local, int E, int out_per_expert, int K,
                                const void *x, int x_dtype, int64_t ldx, int routed_input,
                                const int32_t *ids, int T, int R,
-                               const int32_t *ids_dst, const int32_t *expert_bounds, /* NULL when T*R small */
-                               float *out, int64_t ldo, void *workspace, size_t workspace_bytes,
-                               mfq_stream_t stream);
+                               const int32_t *ids_dst, const int32_t *expert_bounds,
+                               const int32_t *tile_bounds, const int32_t *tile_experts,
+                               float *out, int64_t ldo, mfq_stream_t stream);
 
 /* hidden[r, c] = silu(gate_up[r, c]) * gate_up[r, W + c]  (moe_swiglu_split_cuda,
  * mfq/kernels/cuda/moe.cu:2980-2996); output fp16 (x_dtype MFQ_X_F16) or bf16. */

@@ -1,0 +1,128 @@
+"""Host-side product code without a GPU: payload writers/parsers against the oracle, loader errors,
+and the C ABI library's exported symbols."""
+import ctypes
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import synth
+from oracle import mfq_oracle as O
+from tyloquant_amd import formats as F
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def test_writers_are_byte_identical_to_the_oracle_packers():
+    rng = np.random.default_rng(0)
+    for spec in [(4, 32, 6), (3, 24, 5), (5, 28, 7), (2, 16, 5), (8, 24, 8), (6, 26, 6)]:
+        t = synth.nint_random(rng, 9, 131, *spec)
+        blob = F.nint_blob(t.bits, t.sub_bits, t.groupsize, t.neuron_len, t.neuron_scale, t.neuron_min, t.sub_scale,
+                           t.sub_min, t.q)
+        assert blob == O.pack_nint(t)
+        h = F.parse_nint(blob)
+        assert (h.bits, h.gs, h.sub_bits, h.out, h.ng, h.legacy) == (spec[0], spec[1], spec[2], 9, t.ng, False)
+        assert h.body_bytes == O.nint_payload_nbytes(9, 131, *spec)
+    j = synth.nvq_jsc_random(rng, 7, 100, "d4_512", 2)
+    jb = F.nvq_jsc_blob(j.codebook, j.neuron_len, j.neuron_scale, j.scale_lut, j.bank_for_state, j.codebooks, j.state,
+                        j.indices, j.signs)
+    assert jb == O.pack_nvq_jsc(j)
+    hj = F.parse_nvq(jb)
+    assert hj.dtype == "NVQ3J-512" and hj.banks == 2 and (hj.ng, hj.nvec, hj.nsign) == (5, 25, 13)
+    p = synth.nvq_plain_random(rng, 5, 96)
+    assert F.nvq_plain_blob(p.codebook, p.neuron_len, p.neuron_scale, p.sub_scale, p.indices, p.signs) == O.pack_nvq_plain(p)
+    for label in ("NEPQ1-S", "NEPQ1-L"):
+        n = synth.nepq_random(rng, label, 2, 16, 104, 3)
+        nb = F.nepq_blob(label, n.shape, n.table_payloads, n.neuron_scale, n.state, n.indices, n.aux, n.bank_ids)
+        assert nb == O.pack_nepq(n)
+        hn = F.parse_nepq(nb)
+        assert (hn.label, hn.banks, hn.ng, hn.nvec, hn.nsuper) == (label, 3, 5, 13, 2)
+    m = synth.moe_random(rng, 5, 16, 48, [4, 3, 4, 2, 3])
+    mb = F.nintm_blob(5, 16, 48, [(p.expert_ids, p.dtype, O.pack_nint(p.tensor)) for p in m.pools])
+    assert mb == O.pack_nint_moe(m)
+    hm = F.parse_nintm(mb)
+    assert [p.dtype for p in hm.pools] == ["NINT2", "NINT3", "NINT4"]
+    assert bytes(mb[hm.pools[1].payload_off: hm.pools[1].payload_off + hm.pools[1].payload_bytes]) == O.pack_nint(m.pools[1].tensor)
+
+
+def test_parsers_reject_what_the_reference_loaders_reject():
+    rng = np.random.default_rng(1)
+    t = synth.nint_random(rng, 8, 96, 4, 24, 6)
+    blob = O.pack_nint(t)
+    with pytest.raises(ValueError, match="invalid NINT blob tail"):
+        F.parse_nint(blob[:-1])
+    with pytest.raises(ValueError, match="truncated NINT header"):
+        F.parse_nint(blob[:10])
+    j = O.pack_nvq_jsc(synth.nvq_jsc_random(rng, 4, 48))
+    with pytest.raises(ValueError, match="invalid NVQ magic"):
+        F.parse_nvq(b"NOPE" + j[4:])
+    bad = bytearray(j)
+    bad[40 + 36] = 9                                      # state -> bank 9 of 2
+    with pytest.raises(ValueError, match="state-to-bank"):
+        F.parse_nvq(bytes(bad))
+    bad = bytearray(j)
+    bad[40 + 60] = 1                                      # reserved byte
+    with pytest.raises(ValueError, match="invalid NVQ-JSC metadata"):
+        F.parse_nvq(bytes(bad))
+    n = O.pack_nepq(synth.nepq_random(rng, "NEPQ1-S", 1, 16, 96, 2))
+    with pytest.raises(ValueError, match="truncated NEPQ header"):
+        F.parse_nepq(n[:20])
+    with pytest.raises(ValueError, match="invalid NEPQ tail"):
+        F.parse_nepq(n[:-1])
+    with pytest.raises(ValueError, match="K divisible by 8"):
+        F.parse_nepq(n[:16] + (100).to_bytes(4, "little") + n[20:])
+    m = O.pack_nint_moe(synth.moe_random(rng, 4, 16, 48, [4, 4, 3, 3]))
+    with pytest.raises(ValueError, match="invalid NINTM magic"):
+        F.parse_nintm(b"NIM1" + m[4:])
+    with pytest.raises(ValueError, match="truncated NINTM"):
+        F.parse_nintm(m[: len(m) // 2])
+
+
+def test_mfq_container_round_trip(tmp_path):
+    rng = np.random.default_rng(2)
+    a = O.pack_tensor(synth.nint_random(rng, 8, 96, 3, 24, 5))
+    b = O.pack_tensor(synth.nvq_jsc_random(rng, 4, 48))
+    path = tmp_path / "x.mfq"
+    F.write_mfq(path, {"layers.0.q": a, "layers.0.k": b}, version=2)
+    data = path.read_bytes()
+    d = F.read_mfq_directory(data)
+    assert list(d) == ["layers.0.q", "layers.0.k"]
+    assert d["layers.0.q"][0] == "NINT3" and data[d["layers.0.k"][1]: d["layers.0.k"][1] + d["layers.0.k"][2]] == b[1]
+    assert O.mfq_file_read(path)["layers.0.q"] == a       # the oracle reads what the product wrote
+
+
+def test_library_exports_every_symbol_the_header_declares():
+    from tyloquant_amd import _lib as L
+    header = (ROOT / "include" / "mfq_hip.h").read_text()
+    declared = sorted(set(re.findall(r"\b(mfq_hip_\w+)\s*\(", header)))
+    assert declared == L.exported_symbols()
+    if not L.LIB_PATH.exists():
+        pytest.skip("libmfq_hip.so is not built (run __graft_entry__.build())")
+    lib = ctypes.CDLL(str(L.LIB_PATH))
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert L.lib().mfq_hip_version() >= 1
+
+
+def test_plan_calls_need_no_gpu():
+    """Layout planning is pure host arithmetic: sizes, padding and the payload accounting."""
+    from tyloquant_amd import _lib as L
+    if not L.LIB_PATH.exists():
+        pytest.skip("libmfq_hip.so is not built")
+    lib = L.lib()
+    d = L.NintDesc()
+    L.check(lib.mfq_hip_nint_plan(3, 5, 24, 4096, 4096, ctypes.byref(d)))
+    assert (d.kind, d.dwords, d.tail_bytes, d.ng, d.ngp, d.nsteps, d.n_rowblocks) == (1, 2, 1, 171, 176, 11, 256)
+    assert d.payload_bytes == 7195648 and d.step_bytes == 64 * (32 + 4 + 8)
+    L.check(lib.mfq_hip_nint_plan(4, 6, 32, 12288, 4096, ctypes.byref(d)))
+    assert d.payload_bytes == 27574272 and d.kind == 1 and d.dwords == 4
+    L.check(lib.mfq_hip_nint_plan(5, 7, 28, 64, 112, ctypes.byref(d)))
+    assert d.kind == 0 and d.dwords == 5
+    with pytest.raises(L.MfqError, match="bits"):
+        L.check(lib.mfq_hip_nint_plan(9, 5, 24, 8, 8, ctypes.byref(d)))
+    q = L.NepqDesc()
+    L.check(lib.mfq_hip_nepq_plan(2, 1, 12288, 4096, ctypes.byref(q)))
+    assert q.payload_bytes - 2048 == 8944128
+    with pytest.raises(L.MfqError, match="divisible by 8"):
+        L.check(lib.mfq_hip_nepq_plan(2, 1, 16, 100, ctypes.byref(q)))

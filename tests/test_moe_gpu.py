@@ -1,0 +1,139 @@
+"""GPU parity of the MoE path (top-k, expert map, grouped matmul, FFN) against the oracle."""
+import numpy as np
+import pytest
+
+import synth
+from conftest import ABS_TOL, REL_TOL, rel_l2
+from oracle import mfq_oracle as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+def _topk(logits, k, **kw):
+    from tyloquant_amd.runtime_moe import moe_topk
+    ids, w = moe_topk(torch.from_numpy(logits).cuda(), k, **kw)
+    return ids.cpu().numpy(), w.cpu().numpy()
+
+
+@pytest.mark.parametrize("T,E,k", [(9, 64, 6), (1, 256, 8), (5, 128, 8), (33, 300, 16), (3, 8, 8)])
+def test_topk_modes_match_oracle(T, E, k):
+    rng = np.random.default_rng(71 + T)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    bias = (rng.standard_normal(E) * 0.1).astype(np.float32)
+    for kw in ({}, {"delayed_softmax": True}, {"normalize": True}, {"use_sigmoid": True, "normalize": True},
+               {"use_sqrt_softplus": True, "normalize": True, "scale": 2.5}):
+        ids, w = _topk(logits, k, **kw)
+        rids, rw = O.moe_topk(logits, k, **kw)
+        assert np.array_equal(ids, rids), kw
+        np.testing.assert_allclose(w, rw, rtol=2e-6, atol=2e-7)
+    from tyloquant_amd.runtime_moe import moe_topk
+    ids, w = moe_topk(torch.from_numpy(logits).cuda(), k, use_sigmoid=True, bias=torch.from_numpy(bias).cuda())
+    rids, rw = O.moe_topk(logits, k, use_sigmoid=True, bias=bias)
+    assert np.array_equal(ids.cpu().numpy(), rids)
+    np.testing.assert_allclose(w.cpu().numpy(), rw, rtol=2e-6, atol=2e-7)
+
+
+def test_topk_ties_and_nan():
+    logits = np.zeros((2, 16), dtype=np.float32)
+    logits[1, 3] = np.nan
+    logits[1, 7] = 1.0
+    ids, w = _topk(logits, 4, delayed_softmax=True)
+    assert ids[0].tolist() == [0, 1, 2, 3]            # ties -> lower expert id
+    assert ids[1].tolist() == [7, 0, 1, 2]            # NaN sinks to -FLT_MAX
+    rids, rw = O.moe_topk(logits, 4, delayed_softmax=True)
+    assert np.array_equal(ids, rids)
+    np.testing.assert_allclose(w, rw, rtol=2e-6, atol=2e-7)
+
+
+@pytest.mark.parametrize("T,R,E,tile_m", [(17, 2, 5, 8), (64, 8, 256, 4), (300, 3, 40, 4), (9, 1, 2000, 8)])
+def test_expert_map_invariants(T, R, E, tile_m):
+    from tyloquant_amd.runtime_moe import build_expert_map
+    rng = np.random.default_rng(991 + T)
+    ids = rng.integers(0, E, (T, R)).astype(np.int32)
+    ids[0, 0] = E + 5 if T > 9 else ids[0, 0]         # one out-of-range id is dropped
+    dst, eb, tb, te, counts = [a.cpu().numpy() for a in build_expert_map(torch.from_numpy(ids).cuda(), E, tile_m)]
+    rdst, reb, rtb, rte, rcounts = O.build_expert_map(ids, E, tile_m)
+    assert np.array_equal(counts, rcounts) and np.array_equal(eb, reb) and np.array_equal(tb, rtb)
+    assert np.array_equal(te[: rtb[-1]], rte)
+    assert np.array_equal(dst[: reb[-1]], rdst)       # deterministic: ascending pair index inside an expert
+
+
+def _moe(rng, E, out, K, bits, quantize=True):
+    from tyloquant_amd.runtime_moe import NintMoeWeight
+    t = synth.moe_random(rng, E, out, K, bits, quantize)
+    blob = O.pack_nint_moe(t)
+    return O.unpack_nint_moe(blob), NintMoeWeight.from_blob(blob)
+
+
+@pytest.mark.parametrize("tokens", [1, 4, 13, 70])
+def test_grouped_matmul_matches_reference_loop(tokens):
+    from tyloquant_amd.runtime_moe import build_moe_route_plan
+    rng = np.random.default_rng(10 + tokens)
+    E, out, K, R = 10, 48, 88, 3
+    bits = [(2, 4, 6, 8, 5, 3)[i % 6] for i in range(E)]
+    t, w = _moe(rng, E, out, K, bits)
+    dense = O.dequantize_expertwise(t)
+    assert np.array_equal(w.dequantize().cpu().numpy().view(np.uint32), dense.view(np.uint32))
+    scores = rng.standard_normal((tokens, E))
+    ids = np.argsort(-scores, axis=1)[:, :R].astype(np.int32)
+    x = torch.from_numpy((rng.standard_normal((tokens, K)) * 0.1).astype(np.float32)).to(torch.bfloat16)
+    route = build_moe_route_plan(torch.from_numpy(ids).cuda(), E)
+    got = w(x.cuda(), route).cpu().numpy()
+    ref = O.moe_grouped_matmul(dense, x.float().numpy(), ids)
+    assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL
+
+
+def test_grouped_matmul_routed_input_and_invalid_expert():
+    from tyloquant_amd.runtime_moe import build_moe_route_plan
+    rng = np.random.default_rng(44)
+    E, out, K, T, R = 6, 16, 64, 17, 2
+    t, w = _moe(rng, E, out, K, [4, 3, 4, 2, 3, 5])
+    dense = O.dequantize_expertwise(t)
+    ids = rng.integers(0, E, (T, R)).astype(np.int32)
+    ids[3, 1] = 99                                     # invalid id -> zero row, not garbage
+    x = torch.from_numpy((rng.standard_normal((T, R, K)) * 0.1).astype(np.float32)).to(torch.float16)
+    for sub in (slice(0, T), slice(0, 4)):             # mapped (T > 8) and unmapped paths
+        route = build_moe_route_plan(torch.from_numpy(ids[sub]).cuda(), E)
+        got = w(x[sub].cuda(), route).cpu().numpy()
+        ref = O.moe_grouped_matmul(dense, x[sub].float().numpy(), ids[sub])
+        assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL
+        assert np.all(got[3, 1] == 0)
+
+
+@pytest.mark.parametrize("T", [1, 5, 64])
+def test_moe_ffn_forward_matches_oracle(T):
+    """Scaled-down BASELINE config 4: mixed 2/3/4/5-bit experts, top-8 delayed softmax, ungated shared expert."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_moe import nint_moe_ffn_forward
+    rng = np.random.default_rng(400 + T)
+    E, H, W, k = 32, 256, 128, 8
+    bits = rng.choice([2, 3, 4, 5], size=E, p=[0.1, 0.4, 0.4, 0.1])
+    tg, gu = _moe(rng, E, 2 * W, H, bits)
+    td, dn = _moe(rng, E, H, W, bits)
+    sg = O.quantize_nint((rng.standard_normal((2 * W, H)) * 0.02).astype(np.float32), 4, 24, 6)
+    sd = O.quantize_nint((rng.standard_normal((H, W)) * 0.02).astype(np.float32), 4, 24, 6)
+    shared = (R.load_quant_linear("NINT4", O.pack_nint(sg)).weight, R.load_quant_linear("NINT4", O.pack_nint(sd)).weight)
+    x = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).to(torch.bfloat16)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    out, ids, wts = nint_moe_ffn_forward(gu, dn, x.cuda(), torch.from_numpy(logits).cuda(), k, delayed_softmax=True,
+                                         shared=shared)
+    ref, rids, rw = O.moe_ffn(O.dequantize_expertwise(tg), O.dequantize_expertwise(td), x.float().numpy(), logits, k,
+                              shared=(O.dequantize_nint(sg), O.dequantize_nint(sd)), delayed_softmax=True)
+    assert np.array_equal(ids.cpu().numpy(), rids)
+    got = out.cpu().numpy()
+    assert rel_l2(got, ref) < REL_TOL, rel_l2(got, ref)
+    assert np.abs(got - ref).max() < ABS_TOL
+
+
+def test_moe_errors():
+    from tyloquant_amd.runtime_moe import NintMoeWeight, build_moe_route_plan
+    rng = np.random.default_rng(2)
+    t = synth.moe_random(rng, 4, 16, 48, [4, 4, 3, 3])
+    blob = O.pack_nint_moe(t)
+    with pytest.raises(ValueError, match="invalid NINTM magic"):
+        NintMoeWeight.from_blob(b"NIM9" + blob[4:])
+    with pytest.raises(ValueError, match="invalid NINTM tail"):
+        NintMoeWeight.from_blob(blob + b"\0")
+    with pytest.raises(RuntimeError, match="int32"):
+        build_moe_route_plan(torch.zeros((2, 2), dtype=torch.int64).cuda(), 4)

@@ -2,6 +2,7 @@
 import numpy as np
 import pytest
 
+import synth
 from conftest import ABS_TOL, REL_TOL, rel_l2
 from oracle import mfq_oracle as O
 
@@ -13,14 +14,7 @@ SPECS = [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (6, 24, 6),
          (6, 26, 6), (2, 32, 5), (5, 16, 5)]
 
 
-def _rand_tensor(rng, out, K, bits, gs, sb):
-    """Packed-domain random tensor (every code / sub-scale value occurs)."""
-    ng = -(-K // gs)
-    return O.NintTensor(bits, gs, sb, (out, K), 0, K,
-                        rng.integers(0, 1 << bits, (out, ng, gs), dtype=np.uint8),
-                        O._f16_round(rng.uniform(1e-4, 2e-3, out)), O._f16_round(rng.uniform(1e-3, 2e-2, out)),
-                        rng.integers(0, 1 << sb, (out, ng), dtype=np.uint8),
-                        rng.integers(0, 1 << sb, (out, ng), dtype=np.uint8))
+_rand_tensor = synth.nint_random
 
 
 def _load(t):

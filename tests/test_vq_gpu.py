@@ -1,0 +1,117 @@
+"""GPU parity of the NVQ (D4 family) and NEPQ1 paths against the oracle (through the C ABI)."""
+import numpy as np
+import pytest
+
+import synth
+from conftest import check_close, rel_l2
+from oracle import mfq_oracle as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+def _x(rng, M, K, dtype=None):
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dtype or torch.bfloat16)
+    return x.cuda(), x.float().numpy()
+
+
+_check = check_close
+
+
+@pytest.mark.parametrize("codebook,banks", [("d4_512", 2), ("d4_512", 4), ("d4_512", 1), ("d4_256", 2)])
+@pytest.mark.parametrize("out,K", [(37, 96), (24, 80), (64, 200), (73, 1537), (33, 100)])
+def test_nvq_jsc_dequant_bit_exact_and_gemv(codebook, banks, out, K):
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import nvq_matmul
+    rng = np.random.default_rng(7 + out + K + banks)
+    t = synth.nvq_jsc_random(rng, out, K, codebook, banks)
+    dtype, blob = O.pack_tensor(t)
+    lin = R.load_quant_linear(dtype, blob)
+    want = O.dequantize_nvq_jsc(O.unpack_nvq(blob))
+    got = lin.dequantize().cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    for M in (1, 4, 8):
+        for xd in (torch.bfloat16, torch.float16):
+            x, xf = _x(rng, M, K, xd)
+            _check(nvq_matmul(lin.weight, x, force="gemv").cpu().numpy(), O.linear_forward(want, xf))
+    x, xf = _x(rng, 65, K)
+    _check(lin(x).cpu().numpy(), O.linear_forward_f64(want, xf))
+
+
+def test_nvq_payload_sizes_match_reference_identities():
+    """tests/test_formats/test_nvq.py:44-50 and tests/test_nvq_kernels_cuda.py:410-449 (host side)."""
+    from tyloquant_amd import _lib as L
+    import ctypes as C
+    d = L.NvqDesc()
+    L.check(L.lib().mfq_hip_nvq_plan(9, 2, 4096, 5120, C.byref(d)))
+    streams = d.payload_bytes - 64 - 2 * 512 * 4
+    assert 8.0 * streams / (4096 * 5120) == 3.2953125
+    L.check(L.lib().mfq_hip_nvq_plan(9, 2, 17408, 5120, C.byref(d)))
+    assert d.payload_bytes - 64 - 4096 == 36713472
+
+
+def test_nvq_plain_d4_256():
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(11)
+    t = synth.nvq_plain_random(rng, 40, 104)
+    dtype, blob = O.pack_tensor(t)
+    assert dtype == "NVQ3"
+    lin = R.load_quant_linear("NIQ3", blob)   # legacy alias
+    want = O.dequantize_nvq(O.unpack_nvq(blob))
+    assert np.array_equal(lin.dequantize().cpu().numpy().view(np.uint32), want.view(np.uint32))
+    x, xf = _x(rng, 3, 104)
+    _check(lin(x).cpu().numpy(), O.linear_forward(want, xf))
+
+
+@pytest.mark.parametrize("label", ["NEPQ1-S", "NEPQ1-L"])
+@pytest.mark.parametrize("E,out,K,banks", [(1, 48, 96, 3), (3, 32, 200, 5), (2, 16, 1544, 40), (1, 33, 88, 1)])
+def test_nepq_dequant_bit_exact_and_matmul(label, E, out, K, banks):
+    from tyloquant_amd.runtime_vq import NepqWeight, nepq_matmul
+    rng = np.random.default_rng(23 + E + out + K)
+    t = synth.nepq_random(rng, label, E, out, K, banks)
+    blob = O.pack_nepq(t)
+    w = NepqWeight.from_blob(blob)
+    want = O.dequantize_nepq(O.unpack_nepq(blob))
+    got = w.dequantize().cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    for e in range(E):
+        for M in (1, 5, 16):
+            x, xf = _x(rng, M, K)
+            _check(nepq_matmul(w, x, e).cpu().numpy(), O.linear_forward(want[e], xf))
+        x, xf = _x(rng, 40, K)
+        _check(nepq_matmul(w, x, e).cpu().numpy(), O.linear_forward_f64(want[e], xf))
+
+
+def test_nepq_hadamard_matches_fwht():
+    from tyloquant_amd.runtime_vq import nepq_hadamard
+    rng = np.random.default_rng(3)
+    K, block = 512, 128
+    x = rng.standard_normal((5, K)).astype(np.float32)
+    xb = torch.from_numpy(x).to(torch.bfloat16)
+    signs = np.where(rng.integers(0, 2, K), 1, -1).astype(np.int8)
+    got = nepq_hadamard(xb.cuda(), torch.from_numpy(signs).cuda(), block).float().cpu().numpy()
+    v = (xb.float().numpy() * signs).reshape(5, K // block, block)
+    H = np.array([[1.0]])
+    while H.shape[0] < block:
+        H = np.block([[H, H], [H, -H]])
+    ref = (v @ H.T / np.sqrt(block)).reshape(5, K)
+    assert np.abs(got - ref).max() < 0.05 and rel_l2(got, ref) < 4e-3   # output is rounded to bf16
+
+
+def test_vq_loader_errors():
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(9)
+    t = synth.nvq_jsc_random(rng, 8, 96)
+    dtype, blob = O.pack_tensor(t)
+    with pytest.raises(ValueError, match="invalid NVQ"):
+        R.load_quant_linear(dtype, blob[:-3])
+    with pytest.raises(ValueError, match="invalid NVQ magic"):
+        R.load_quant_linear(dtype, b"XXXX" + blob[4:])
+    with pytest.raises(ValueError, match="dtype/blob mismatch"):
+        R.load_quant_linear("NVQ3J", blob)
+    n = synth.nepq_random(rng, "NEPQ1-S", 1, 16, 96, 2)
+    nb = O.pack_nepq(n)
+    with pytest.raises(ValueError, match="invalid NEPQ tail"):
+        R.load_quant_linear("NEPQ1-S", nb + b"\0")
+    with pytest.raises(ValueError, match="dtype/blob mismatch"):
+        R.load_quant_linear("NEPQ1-L", nb)

@@ -72,9 +72,9 @@ _SIGS = {
     "mfq_hip_moe_topk": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp,
                                    vp]),
     "mfq_hip_moe_route_map": (C.c_int, [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, C.c_int, vp, vp]),
-    "mfq_hip_moe_grouped_workspace_bytes": (sz, [C.c_int, C.c_int, C.c_int]),
+    "mfq_hip_moe_tile_m": (C.c_int, []),
     "mfq_hip_moe_grouped_matmul": (C.c_int, [C.POINTER(MoePool), C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, vp,
-                                             C.c_int, i64, C.c_int, vp, C.c_int, C.c_int, vp, vp, vp, i64, vp, sz,
+                                             C.c_int, i64, C.c_int, vp, C.c_int, C.c_int, vp, vp, vp, vp, vp, i64,
                                              vp]),
     "mfq_hip_moe_swiglu": (C.c_int, [vp, i64, C.c_int, C.c_int, vp, C.c_int, i64, vp]),
     "mfq_hip_moe_weighted_reduce": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]),

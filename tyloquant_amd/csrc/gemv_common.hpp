@@ -25,20 +25,19 @@ __device__ __forceinline__ void load_unit(const uint32_t *__restrict__ p, uint32
     }
 }
 
-// Stage the wave's K-slice of x (MB rows) into its private LDS region as (x[2i], x[2i+1]) pairs,
-// zero beyond K, and the per-group sums next to it.
+// Stage the wave's K-slice of the MB activation rows xr[m] (null = absent row) into its private
+// LDS region as (x[2i], x[2i+1]) pairs, zero beyond K, with the per-group sums next to it.
 template <int XF16, int MB>
-__device__ __forceinline__ void stage_x(const uint16_t *__restrict__ x, int64_t ldx, int M, int m0, int K, int k0,
-                                        int npairs, int gs, int ngl, uint32_t *xs, float *xsum, int lane) {
+__device__ __forceinline__ void stage_x(const uint16_t *const (&xr)[MB], int K, int k0, int npairs, int gs, int ngl,
+                                        uint32_t *xs, float *xsum, int lane) {
 #pragma unroll
     for (int m = 0; m < MB; ++m) {
-        const bool mv = (m0 + m) < M;
-        const uint16_t *xr = x + static_cast<int64_t>(m0 + m) * ldx;
+        const uint16_t *p = xr[m];
         for (int i = lane; i < npairs; i += 64) {
             const int kk = k0 + 2 * i;
             uint32_t lo = 0, hi = 0;
-            if (mv && kk < K) lo = xr[kk];
-            if (mv && kk + 1 < K) hi = xr[kk + 1];
+            if (p && kk < K) lo = p[kk];
+            if (p && kk + 1 < K) hi = p[kk + 1];
             xs[m * npairs + i] = lo | (hi << 16);
         }
     }
@@ -55,9 +54,11 @@ __device__ __forceinline__ void stage_x(const uint16_t *__restrict__ x, int64_t 
     __syncthreads();
 }
 
+// Reduce the K-split (4 lanes inside the wave, then the waves of the block through LDS, in a fixed
+// order) and store neuron `rb*16 + r - row_base` of each output row yr[m] (null = absent row).
 template <int MB>
 __device__ __forceinline__ void finish_rows(float (&v)[MB], float *red, int wave, int nwaves, int lane, int rb,
-                                            int out, int M, int m0, float *__restrict__ y, int64_t ldy) {
+                                            int row_base, int out_rows, float *const (&yr)[MB]) {
 #pragma unroll
     for (int m = 0; m < MB; ++m) v[m] = reduce_kb4(v[m]);
     __syncthreads();  // everyone is done with the staged x: the region is reused for the cross-wave sums
@@ -66,14 +67,30 @@ __device__ __forceinline__ void finish_rows(float (&v)[MB], float *red, int wave
         for (int m = 0; m < MB; ++m) red[(wave * MB + m) * 16 + lane] = v[m];
     }
     __syncthreads();
-    if (wave == 0 && lane < 16 * MB) {
-        const int m = lane >> 4, r = lane & 15;
-        float s = 0.f;
-        for (int wv = 0; wv < nwaves; ++wv) s += red[(wv * MB + m) * 16 + r];
-        const int row = rb * 16 + r;
-        if (row < out && m0 + m < M) y[static_cast<int64_t>(m0 + m) * ldy + row] = s;
+    if (wave == 0) {
+        const int r = lane & 15;
+        const int row = rb * 16 + r - row_base;
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            if ((lane >> 4) == (m & 3)) {
+                float s = 0.f;
+                for (int wv = 0; wv < nwaves; ++wv) s += red[(wv * MB + m) * 16 + r];
+                if (yr[m] && row >= 0 && row < out_rows) yr[m][row] = s;
+            }
+        }
     }
 }
 
+// Dense activations: rows m0 .. m0+MB-1 of x[M, ldx] / y[M, ldy].
+template <int MB>
+__device__ __forceinline__ void dense_rows(const uint16_t *x, int64_t ldx, float *y, int64_t ldy, int M, int m0,
+                                           const uint16_t *(&xr)[MB], float *(&yr)[MB]) {
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        const bool ok = m0 + m < M;
+        xr[m] = ok ? x + static_cast<int64_t>(m0 + m) * ldx : nullptr;
+        yr[m] = ok ? y + static_cast<int64_t>(m0 + m) * ldy : nullptr;
+    }
+}
 
 }  // namespace mfq

@@ -1,0 +1,434 @@
+// NEPQ1-S / NEPQ1-L: 8-dim ternary code vectors from a cross-expert table pool, one bank id per
+// 96 weights, per-group integer state (scale), one delta-sign bit per group.
+//
+// Device layout (rows = experts * out_per_expert neurons, same row-block / step / lane interleave):
+//   NEPQ1-S unit = one dword   idx0 | idx1 << 9 | idx2 << 18 | state << 27 | aux << 31
+//   NEPQ1-L unit = dword + byte  idx0 | idx1 << 11 | (idx2 & 1023) << 22 ;  (idx2 >> 10) | state << 1 | aux << 4
+//   step = Q [j][lane] dwords, T [lane][4 bytes] (L only), B [16 neurons][4 bank ids (one per j)]
+// tail: uint16 table[banks][entries] (S: aux * 512 + idx, L: idx; 8 two-bit digits = code + 1 each),
+//       float anchor[].
+// value = fl(anchor * state) * (code + bias), bias = +-5/32 (S) or +-1/8 (L), minus when aux is set.
+#include "common.hpp"
+#include "gemv_common.hpp"
+
+namespace mfq {
+
+struct NepqK {
+    int profile, sb, ib, banks, rows, neuron_len, ng, nvec, nsuper, nsteps, n_rowblocks, entries, tail;
+    int64_t step_bytes, rowblock_bytes, tables_off, anchors_off;
+};
+
+static NepqK to_k(const mfq_nepq_desc *d) {
+    NepqK k;
+    k.profile = d->profile; k.sb = d->state_bits; k.ib = d->index_bits; k.banks = d->banks; k.rows = d->rows;
+    k.neuron_len = d->neuron_len; k.ng = d->ng; k.nvec = d->nvec; k.nsuper = d->nsuper; k.nsteps = d->nsteps;
+    k.n_rowblocks = d->n_rowblocks; k.entries = d->table_entries; k.tail = d->profile == 3 ? 1 : 0;
+    k.step_bytes = d->step_bytes; k.rowblock_bytes = d->rowblock_bytes; k.tables_off = d->tables_off;
+    k.anchors_off = d->anchors_off;
+    return k;
+}
+
+struct NepqUnit {
+    uint32_t idx[3], state, aux;
+};
+__device__ __forceinline__ NepqUnit nepq_decode(int profile, uint32_t d, uint32_t t) {
+    NepqUnit u;
+    if (profile == 2) {
+        u.idx[0] = d & 511u; u.idx[1] = (d >> 9) & 511u; u.idx[2] = (d >> 18) & 511u;
+        u.state = (d >> 27) & 15u; u.aux = d >> 31;
+        // the S table is indexed by aux * 512 + idx
+        u.idx[0] += u.aux << 9; u.idx[1] += u.aux << 9; u.idx[2] += u.aux << 9;
+    } else {
+        u.idx[0] = d & 2047u; u.idx[1] = (d >> 11) & 2047u; u.idx[2] = (d >> 22) | ((t & 1u) << 10);
+        u.state = (t >> 1) & 7u; u.aux = (t >> 4) & 1u;
+    }
+    return u;
+}
+
+__global__ void nepq_repack_kernel(NepqK k, const uint8_t *__restrict__ payload, uint8_t *__restrict__ dst) {
+    const int lane = threadIdx.x;
+    const int rb = blockIdx.x, s = blockIdx.y;
+    const int r = lane & 15, kb = lane >> 4;
+    const int row = rb * 16 + r;
+    const int64_t rows = k.rows;
+    const int64_t tb = static_cast<int64_t>(k.banks) * k.entries * 2;
+    const int64_t st_bytes = (rows * k.ng * k.sb + 7) / 8, ix_bytes = (rows * k.nvec * k.ib + 7) / 8,
+                  ax_bytes = (rows * k.ng + 7) / 8;
+    const uint8_t *an_s = payload + tb;
+    const uint8_t *st_s = an_s + 2 * rows;
+    const uint8_t *ix_s = st_s + st_bytes;
+    const uint8_t *ax_s = ix_s + ix_bytes;
+    const uint8_t *bk_s = ax_s + ax_bytes;
+    uint8_t *sp = dst + rb * k.rowblock_bytes + s * k.step_bytes;
+    uint32_t *qreg = reinterpret_cast<uint32_t *>(sp);
+    uint8_t *treg = sp + 1024;
+    uint8_t *breg = treg + (k.tail ? 256 : 0);
+    for (int j = 0; j < 4; ++j) {
+        const int g = 16 * s + 4 * j + kb;
+        uint32_t d = 0, t = 0;
+        if (row < k.rows && g < k.ng) {
+            uint32_t idx[3];
+            for (int v = 0; v < 3; ++v) {
+                const int vi = 3 * g + v;
+                idx[v] = vi < k.nvec ? read_bits(ix_s, static_cast<int64_t>(row) * k.nvec + vi, k.ib, ix_bytes) : 0u;
+            }
+            const uint32_t state = read_bits(st_s, static_cast<int64_t>(row) * k.ng + g, k.sb, st_bytes);
+            const uint32_t aux = read_bits(ax_s, static_cast<int64_t>(row) * k.ng + g, 1, ax_bytes);
+            if (k.profile == 2) {
+                d = idx[0] | (idx[1] << 9) | (idx[2] << 18) | (state << 27) | (aux << 31);
+            } else {
+                d = idx[0] | (idx[1] << 11) | ((idx[2] & 1023u) << 22);
+                t = (idx[2] >> 10) | (state << 1) | (aux << 4);
+            }
+        }
+        qreg[j * 64 + lane] = d;
+        if (k.tail) treg[lane * 4 + j] = static_cast<uint8_t>(t);
+        if (kb == 0) {
+            const int sg = 4 * s + j;
+            breg[r * 4 + j] = (row < k.rows && sg < k.nsuper) ? bk_s[static_cast<int64_t>(row) * k.nsuper + sg] : 0;
+        }
+    }
+    if (s == 0 && kb == 0) {
+        float *anchors = reinterpret_cast<float *>(dst + k.anchors_off);
+        anchors[row] = row < k.rows ? f16_to_f32(reinterpret_cast<const uint16_t *>(an_s)[row]) : 0.f;
+    }
+    if (rb == 0 && s == 0) {
+        uint16_t *tab = reinterpret_cast<uint16_t *>(dst + k.tables_off);
+        const uint16_t *src = reinterpret_cast<const uint16_t *>(payload);
+        for (int i = lane; i < k.banks * k.entries; i += 64) tab[i] = src[i];
+    }
+}
+
+template <typename OutT>
+__global__ void nepq_dequant_kernel(NepqK k, const uint8_t *__restrict__ w, int rb0, int row0, int nrows,
+                                    OutT *__restrict__ outp, int64_t ld, float *__restrict__ rowscale, int kpad) {
+    const int lane = threadIdx.x;
+    const int rb = rb0 + blockIdx.x, s = blockIdx.y;
+    const int r = lane & 15, kb = lane >> 4;
+    const int row = rb * 16 + r;
+    const int orow = row - row0;
+    if (orow < 0 || orow >= nrows) return;
+    const uint8_t *sp = w + rb * k.rowblock_bytes + s * k.step_bytes;
+    const uint32_t *qreg = reinterpret_cast<const uint32_t *>(sp);
+    const uint8_t *treg = sp + 1024;
+    const uint8_t *breg = treg + (k.tail ? 256 : 0);
+    const uint16_t *tab = reinterpret_cast<const uint16_t *>(w + k.tables_off);
+    const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[row];
+    const float delta = k.profile == 2 ? 0.15625f : 0.125f;
+    float inv = 1.f;
+    if constexpr (sizeof(OutT) == 2) {
+        const float bound = anchor * static_cast<float>((1 << k.sb) - 1) * 1.25f;
+        int e = 0;
+        if (bound > 0.f) frexpf(bound, &e);
+        inv = ldexpf(1.f, 12 - e);
+        if (s == 0 && kb == 0) {
+            rowscale[orow] = ldexpf(1.f, e - 12);
+            for (int col = k.neuron_len; col < kpad; ++col) outp[orow * ld + col] = 0;
+        }
+    }
+    for (int j = 0; j < 4; ++j) {
+        const int g = 16 * s + 4 * j + kb;
+        if (g >= k.ng) continue;
+        const NepqUnit u = nepq_decode(k.profile, qreg[j * 64 + lane], k.tail ? treg[lane * 4 + j] : 0u);
+        const uint16_t *bank = tab + static_cast<int64_t>(breg[r * 4 + j]) * k.entries;
+        const float scale = __fmul_rn(anchor, static_cast<float>(u.state));
+        const float bias = u.aux ? -delta : delta;
+        for (int i = 0; i < 24; ++i) {
+            const int col = g * 24 + i;
+            if (col >= k.neuron_len) break;
+            const uint32_t e = bank[u.idx[i >> 3]];
+            const float code = static_cast<float>(static_cast<int>((e >> (2 * (i & 7))) & 3u) - 1);
+            const float v = __fmul_rn(scale, __fadd_rn(code, bias));
+            if constexpr (sizeof(OutT) == 2) outp[orow * ld + col] = f32_to_f16_rne(v * inv);
+            else outp[orow * ld + col] = v;
+        }
+    }
+}
+
+// GEMV: sum_i (code_i + bias) x_i = sum_i digit_i x_i + (bias - 1) * xsum, digit = code + 1 in {0,1,2};
+// a table entry e (8 two-bit digits) becomes four biased pairs from t = e | e << 14.
+template <int XF16, int MB, int TAB_LDS>
+__global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t *__restrict__ w, int rb0, int row0,
+                                                         int nrows, const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                         float *__restrict__ y, int64_t ldy, int spw) {
+    extern __shared__ uint32_t lds[];
+    constexpr uint32_t MAGIC = XF16 ? 0x64006400u : 0x43004300u;
+    constexpr float BIAS = XF16 ? 1024.f : 128.f;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int rb = rb0 + blockIdx.x;
+    const uint16_t *xr[MB];
+    float *yr[MB];
+    dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
+    const uint16_t *gtab = reinterpret_cast<const uint16_t *>(w + k.tables_off);
+    const int ntab = k.banks * k.entries;  // u16 entries
+    uint16_t *ltab = reinterpret_cast<uint16_t *>(lds);
+    uint32_t *xbase = lds;
+    if constexpr (TAB_LDS) {
+        for (int i = tid; i < ntab / 2; i += blockDim.x) lds[i] = reinterpret_cast<const uint32_t *>(gtab)[i];
+        xbase = lds + ntab / 2;
+    }
+    const uint16_t *tab = TAB_LDS ? ltab : gtab;
+    const int s0 = wave * spw;
+    const int s1 = min(k.nsteps, s0 + spw);
+    const int ngl = spw * 16, npairs = ngl * 12;
+    uint32_t *xs = xbase + wave * (MB * (npairs + ngl));
+    float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
+    stage_x<XF16, MB>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane);
+
+    const int r = lane & 15, kb = lane >> 4;
+    const uint8_t *base = w + static_cast<int64_t>(rb) * k.rowblock_bytes;
+    const float delta = k.profile == 2 ? 0.15625f : 0.125f;
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = 0.f;
+    for (int s = s0; s < s1; ++s) {
+        const uint8_t *sp = base + s * k.step_bytes;
+        uint32_t q[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) q[j] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sp) + j * 64 + lane);
+        uint32_t tails = 0;
+        if (k.tail) tails = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sp + 1024) + lane);
+        const uint32_t banks4 = *(reinterpret_cast<const uint32_t *>(sp + 1024 + (k.tail ? 256 : 0)) + r);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int lg = (s - s0) * 16 + 4 * j + kb;
+            const NepqUnit u = nepq_decode(k.profile, q[j], (tails >> (8 * j)) & 0xffu);
+            const uint16_t *bank = tab + ((banks4 >> (8 * j)) & 0xffu) * k.entries;
+            const float st = static_cast<float>(u.state);
+            const float off = (u.aux ? -delta : delta) - 1.f - BIAS;
+            float raw[MB];
+#pragma unroll
+            for (int m = 0; m < MB; ++m) raw[m] = 0.f;
+#pragma unroll
+            for (int v = 0; v < 3; ++v) {
+                const uint32_t e = bank[u.idx[v]];
+                const uint32_t t = e | (e << 14);
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    const uint32_t pr = ((t >> (4 * p)) & 0x00030003u) | MAGIC;
+#pragma unroll
+                    for (int m = 0; m < MB; ++m) raw[m] = dot2<XF16>(pr, xs[m * npairs + lg * 12 + 4 * v + p], raw[m]);
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < MB; ++m) acc[m] = fmaf(st, fmaf(off, xsum[m * ngl + lg], raw[m]), acc[m]);
+        }
+    }
+    const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[rb * 16 + r];
+    float v[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) v[m] = anchor * acc[m];
+    finish_rows<MB>(v, reinterpret_cast<float *>(xbase), wave, nwaves, lane, rb, row0, nrows, yr);
+}
+
+static void nepq_gemv_shape(const NepqK &k, int nrb, int mb, int &spw, int &nwaves, size_t &lds_bytes, bool &tab_lds) {
+    int want = static_cast<int>(ceil_div(6144, nrb));
+    if (want < 1) want = 1;
+    if (want > 16) want = 16;
+    if (want > k.nsteps) want = k.nsteps;
+    spw = static_cast<int>(ceil_div(k.nsteps, want));
+    nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
+    size_t xb = static_cast<size_t>(mb) * spw * 16 * 13 * 4 * nwaves;
+    const size_t red = static_cast<size_t>(nwaves) * mb * 16 * 4;
+    if (xb < red) xb = red;
+    const size_t tabb = static_cast<size_t>(k.banks) * k.entries * 2;
+    tab_lds = tabb + xb <= 65536;
+    lds_bytes = xb + (tab_lds ? tabb : 0);
+}
+
+template <int XF16, int MB>
+static int nepq_launch(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
+                       float *y, int64_t ldy, hipStream_t st) {
+    const int rb0 = row0 / 16, nrb = static_cast<int>(ceil_div(nrows, 16));
+    int spw, nwaves;
+    size_t lds;
+    bool tab_lds;
+    nepq_gemv_shape(k, nrb, MB, spw, nwaves, lds, tab_lds);
+    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nepq_gemv: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
+    const dim3 grid(nrb, static_cast<unsigned>(ceil_div(M, MB))), block(64 * nwaves);
+    if (tab_lds)
+        hipLaunchKernelGGL((nepq_gemv_kernel<XF16, MB, 1>), grid, block, lds, st, k, w, rb0, row0, nrows, x, ldx, M, y, ldy, spw);
+    else
+        hipLaunchKernelGGL((nepq_gemv_kernel<XF16, MB, 0>), grid, block, lds, st, k, w, rb0, row0, nrows, x, ldx, M, y, ldy, spw);
+    return check_launch("nepq_gemv");
+}
+
+static int nepq_gemv_any(const mfq_nepq_desc *d, const void *weight, int row0, int nrows, const void *x, int x_dtype,
+                         int64_t ldx, int M, float *y, int64_t ldy, hipStream_t st) {
+    const NepqK k = to_k(d);
+    const uint8_t *w = static_cast<const uint8_t *>(weight);
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    const int nrb = static_cast<int>(ceil_div(nrows, 16));
+    int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
+    for (;;) {
+        int spw, nwaves;
+        size_t lds;
+        bool tl;
+        nepq_gemv_shape(k, nrb, mb, spw, nwaves, lds, tl);
+        if (lds <= 65536 || mb == 1) break;
+        mb >>= 1;
+    }
+    if (x_dtype == MFQ_X_F16) {
+        if (mb == 4) return nepq_launch<1, 4>(k, w, row0, nrows, xp, ldx, M, y, ldy, st);
+        if (mb == 2) return nepq_launch<1, 2>(k, w, row0, nrows, xp, ldx, M, y, ldy, st);
+        return nepq_launch<1, 1>(k, w, row0, nrows, xp, ldx, M, y, ldy, st);
+    }
+    if (mb == 4) return nepq_launch<0, 4>(k, w, row0, nrows, xp, ldx, M, y, ldy, st);
+    if (mb == 2) return nepq_launch<0, 2>(k, w, row0, nrows, xp, ldx, M, y, ldy, st);
+    return nepq_launch<0, 1>(k, w, row0, nrows, xp, ldx, M, y, ldy, st);
+}
+
+// ---- signed block-Hadamard input transform ------------------------------------------------
+template <int XF16>
+__global__ __launch_bounds__(256) void hadamard_kernel(const uint16_t *__restrict__ x, int64_t ldx, int K, int block,
+                                                       const int8_t *__restrict__ signs, uint16_t *__restrict__ out,
+                                                       int64_t ldo) {
+    extern __shared__ float hbuf[];
+    const int b = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
+    const uint16_t *xr = x + row * ldx + static_cast<int64_t>(b) * block;
+    for (int i = tid; i < block; i += 256) hbuf[i] = x_to_f32<XF16>(xr[i]) * static_cast<float>(signs[b * block + i]);
+    __syncthreads();
+    for (int h = 1; h < block; h <<= 1) {
+        for (int i = tid; i < block / 2; i += 256) {
+            const int lo = ((i / h) * 2 * h) + (i % h);
+            const float a = hbuf[lo], c = hbuf[lo + h];
+            hbuf[lo] = a + c;
+            hbuf[lo + h] = a - c;
+        }
+        __syncthreads();
+    }
+    const float norm = rsqrtf(static_cast<float>(block));
+    uint16_t *o = out + row * ldo + static_cast<int64_t>(b) * block;
+    for (int i = tid; i < block; i += 256) {
+        const float v = hbuf[i] * norm;
+        o[i] = XF16 ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
+    }
+}
+
+int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, const float *sa,
+                const float *sb, float *y, int64_t ldy, hipStream_t st);
+int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, hipStream_t st);
+size_t dequant_gemm_workspace(int N, int K, int M);
+void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&xscale, uint16_t *&w16, float *&wscale,
+                        int &Kp);
+
+}  // namespace mfq
+
+using namespace mfq;
+
+extern "C" int mfq_hip_nepq_plan(int profile, int banks, int rows, int neuron_len, mfq_nepq_desc *d) {
+    MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nepq_plan: null descriptor");
+    MFQ_REQUIRE(profile == 2 || profile == 3, MFQ_ERR_UNSUPPORTED,
+                "nepq_plan: only NEPQ1-S (2) and NEPQ1-L (3) are on the accelerated path (profile=%d)", profile);
+    MFQ_REQUIRE(banks >= 1 && banks <= 256, MFQ_ERR_INVALID, "NEPQ bank count must be in [1,256]");
+    MFQ_REQUIRE(rows > 0 && neuron_len > 0 && neuron_len % 8 == 0, MFQ_ERR_INVALID, "NEPQ K must be divisible by 8");
+    d->profile = profile;
+    d->state_bits = profile == 2 ? 4 : 3;
+    d->index_bits = profile == 2 ? 9 : 11;
+    d->banks = banks; d->rows = rows; d->neuron_len = neuron_len;
+    d->ng = static_cast<int32_t>(ceil_div(neuron_len, 24));
+    d->nvec = neuron_len / 8;
+    d->nsuper = static_cast<int32_t>(ceil_div(d->ng, 4));
+    d->ngp = static_cast<int32_t>(ceil_div(d->ng, 16) * 16);
+    d->nsteps = d->ngp / 16;
+    d->n_rowblocks = static_cast<int32_t>(ceil_div(rows, 16));
+    d->table_entries = profile == 2 ? 1024 : 2048;
+    d->step_bytes = 1024 + (profile == 3 ? 256 : 0) + 64;
+    d->rowblock_bytes = d->step_bytes * d->nsteps;
+    d->tables_off = d->rowblock_bytes * d->n_rowblocks;
+    d->anchors_off = d->tables_off + static_cast<int64_t>(banks) * d->table_entries * 2;
+    d->total_bytes = d->anchors_off + 16ll * d->n_rowblocks * 4;
+    const int64_t r = rows;
+    d->payload_bytes = static_cast<int64_t>(banks) * d->table_entries * 2 + 2 * r + (r * d->ng * d->state_bits + 7) / 8 +
+                       (r * d->nvec * d->index_bits + 7) / 8 + (r * d->ng + 7) / 8 + r * d->nsuper;
+    return MFQ_OK;
+}
+
+extern "C" int mfq_hip_nepq_repack(const mfq_nepq_desc *d, const void *payload, int64_t payload_bytes, void *weight,
+                                   mfq_stream_t stream) {
+    MFQ_REQUIRE(d && payload && weight, MFQ_ERR_INVALID, "nepq_repack: null argument");
+    MFQ_REQUIRE(payload_bytes == d->payload_bytes, MFQ_ERR_INVALID, "invalid NEPQ tail: size=%lld, expected=%lld",
+                static_cast<long long>(payload_bytes), static_cast<long long>(d->payload_bytes));
+    const NepqK k = to_k(d);
+    hipLaunchKernelGGL(nepq_repack_kernel, dim3(k.n_rowblocks, k.nsteps), dim3(64), 0, as_stream(stream), k,
+                       static_cast<const uint8_t *>(payload), static_cast<uint8_t *>(weight));
+    return check_launch("nepq_repack");
+}
+
+extern "C" int mfq_hip_nepq_dequant_f32(const mfq_nepq_desc *d, const void *weight, float *w_out, int64_t ld,
+                                        mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && w_out, MFQ_ERR_INVALID, "nepq_dequant_f32: null argument");
+    MFQ_REQUIRE(ld >= d->neuron_len, MFQ_ERR_INVALID, "nepq_dequant_f32: ld smaller than neuron_len");
+    const NepqK k = to_k(d);
+    hipLaunchKernelGGL((nepq_dequant_kernel<float>), dim3(k.n_rowblocks, k.nsteps), dim3(64), 0, as_stream(stream), k,
+                       static_cast<const uint8_t *>(weight), 0, 0, k.rows, w_out, ld, static_cast<float *>(nullptr), 0);
+    return check_launch("nepq_dequant_f32");
+}
+
+static int nepq_check_rows(const mfq_nepq_desc *d, int row0, int nrows) {
+    MFQ_REQUIRE(row0 >= 0 && nrows > 0 && row0 + nrows <= d->rows, MFQ_ERR_INVALID, "nepq: rows [%d, %d) outside [0, %d)",
+                row0, row0 + nrows, d->rows);
+    MFQ_REQUIRE(row0 % 16 == 0, MFQ_ERR_UNSUPPORTED, "nepq: expert row offset %d must be a multiple of 16", row0);
+    return MFQ_OK;
+}
+
+extern "C" int mfq_hip_nepq_gemv(const mfq_nepq_desc *d, const void *weight, int row0, int nrows, const void *x,
+                                 int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nepq_gemv: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nepq_gemv: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nepq_gemv: x_dtype=%d", x_dtype);
+    if (int rc = nepq_check_rows(d, row0, nrows)) return rc;
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= nrows, MFQ_ERR_INVALID, "nepq_gemv: ldx/ldy smaller than the tensor");
+    return nepq_gemv_any(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, as_stream(stream));
+}
+
+static constexpr int kNepqGemvMaxM = 16;  // the reference's Python policy: M <= 16 stays on the GEMV
+
+extern "C" size_t mfq_hip_nepq_gemm_workspace_bytes(const mfq_nepq_desc *d, int nrows, int M) {
+    if (!d || M <= kNepqGemvMaxM) return 0;
+    return dequant_gemm_workspace(nrows, d->neuron_len, M);
+}
+
+extern "C" int mfq_hip_nepq_gemm(const mfq_nepq_desc *d, const void *weight, int row0, int nrows, const void *x,
+                                 int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, void *workspace,
+                                 size_t workspace_bytes, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nepq_gemm: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nepq_gemm: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nepq_gemm: x_dtype=%d", x_dtype);
+    if (int rc = nepq_check_rows(d, row0, nrows)) return rc;
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= nrows, MFQ_ERR_INVALID, "nepq_gemm: ldx/ldy smaller than the tensor");
+    hipStream_t st = as_stream(stream);
+    if (M <= kNepqGemvMaxM) return nepq_gemv_any(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, st);
+    const size_t need = dequant_gemm_workspace(nrows, d->neuron_len, M);
+    MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nepq_gemm: workspace %zu < %zu bytes",
+                workspace_bytes, need);
+    uint16_t *x16, *w16;
+    float *xscale, *wscale;
+    int Kp;
+    dequant_gemm_carve(workspace, nrows, d->neuron_len, M, x16, xscale, w16, wscale, Kp);
+    int rc = x_prep(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, st);
+    if (rc) return rc;
+    const NepqK k = to_k(d);
+    hipLaunchKernelGGL((nepq_dequant_kernel<uint16_t>), dim3(static_cast<unsigned>(ceil_div(nrows, 16)), k.nsteps), dim3(64),
+                       0, st, k, static_cast<const uint8_t *>(weight), row0 / 16, row0, nrows, w16,
+                       static_cast<int64_t>(Kp), wscale, Kp);
+    rc = check_launch("nepq_dequant_f16");
+    if (rc) return rc;
+    return gemm_f16_nt(x16, Kp, w16, Kp, M, nrows, Kp, xscale, wscale, y, ldy, st);
+}
+
+extern "C" int mfq_hip_nepq_hadamard(const void *x, int x_dtype, int64_t ldx, int rows, int K, int block,
+                                     const int8_t *signs, void *x_out, int64_t ldo, mfq_stream_t stream) {
+    MFQ_REQUIRE(x && signs && x_out, MFQ_ERR_INVALID, "nepq_hadamard: null argument");
+    MFQ_REQUIRE(block >= 2 && block <= 8192 && (block & (block - 1)) == 0 && K % block == 0, MFQ_ERR_INVALID,
+                "NEPQ rotation block must be a power of two dividing K (block=%d, K=%d)", block, K);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nepq_hadamard: x_dtype=%d", x_dtype);
+    const dim3 grid(K / block, rows);
+    if (x_dtype == MFQ_X_F16)
+        hipLaunchKernelGGL((hadamard_kernel<1>), grid, dim3(256), block * 4, as_stream(stream),
+                           static_cast<const uint16_t *>(x), ldx, K, block, signs, static_cast<uint16_t *>(x_out), ldo);
+    else
+        hipLaunchKernelGGL((hadamard_kernel<0>), grid, dim3(256), block * 4, as_stream(stream),
+                           static_cast<const uint16_t *>(x), ldx, K, block, signs, static_cast<uint16_t *>(x_out), ldo);
+    return check_launch("nepq_hadamard");
+}

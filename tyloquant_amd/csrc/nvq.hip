@@ -158,7 +158,10 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
                                                         float *__restrict__ y, int64_t ldy, int spw) {
     extern __shared__ uint32_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
-    const int rb = blockIdx.x, m0 = blockIdx.y * MB;
+    const int rb = blockIdx.x;
+    const uint16_t *xr[MB];
+    float *yr[MB];
+    dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
     const int ncb = k.banks * k.entries;
     uint32_t *cbp = lds;                 // 2 dwords per entry: (m0, m1), (m2, m3) in the activation type
     uint32_t *sgx = cbp + 2 * ncb;       // 4 dwords per 7-bit mask
@@ -196,7 +199,7 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
     const int ngl = spw * 16, npairs = ngl * 12;
     uint32_t *xs = xbase + wave * (MB * (npairs + ngl));
     float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
-    stage_x<XF16, MB>(x, ldx, M, m0, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane);
+    stage_x<XF16, MB>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane);
 
     const int r = lane & 15, kb = lane >> 4;
     const uint8_t *base = w + rb * k.rowblock_bytes;
@@ -247,7 +250,7 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
     float v[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) v[m] = anchor * acc[m];
-    finish_rows<MB>(v, reinterpret_cast<float *>(xbase), wave, nwaves, lane, rb, k.out, M, m0, y, ldy);
+    finish_rows<MB>(v, reinterpret_cast<float *>(xbase), wave, nwaves, lane, rb, 0, k.out, yr);
 }
 
 static void nvq_gemv_shape(const NvqK &k, int mb, int &spw, int &nwaves, size_t &lds_bytes) {

@@ -1,0 +1,209 @@
+"""Expert-wise mixed-bit MoE: NINTM weights, the route plan and the FFN forward (see runtime.py)."""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import _lib as L
+from . import formats as F
+from .runtime import NintWeight, _ptr, _stream, _x_dtype, nint_matmul
+
+_MODE = {"softmax": L.TOPK_SOFTMAX, "sigmoid": L.TOPK_SIGMOID, "sqrt_softplus": L.TOPK_SQRT_SOFTPLUS,
+         "delayed_softmax": L.TOPK_DELAYED_SOFTMAX}
+
+
+def moe_topk(logits: torch.Tensor, top_k: int, use_sigmoid=False, use_sqrt_softplus=False, normalize=False,
+             delayed_softmax=False, bias: torch.Tensor | None = None, norm_floor=1e-20, scale=1.0):
+    """moe_topk_cuda (mfq/kernels/cuda/moe.cu:3552-3637): returns (ids int32 [T,k], weights f32 [T,k])."""
+    if logits.dim() != 2 or not logits.is_cuda:
+        raise ValueError("logits must be contiguous CUDA [tokens, experts]")
+    if normalize and delayed_softmax:
+        raise ValueError("selected-weight normalization and delayed softmax are mutually exclusive")
+    if sum((use_sigmoid, use_sqrt_softplus, delayed_softmax)) > 1:
+        raise ValueError("sigmoid, sqrt-softplus and delayed-softmax routing are mutually exclusive")
+    logits = logits.float().contiguous()
+    T, E = logits.shape
+    if not 1 <= top_k <= min(16, E):
+        raise ValueError("top_k must be in [1, min(16, experts)]")
+    mode = L.TOPK_DELAYED_SOFTMAX if delayed_softmax else L.TOPK_SIGMOID if use_sigmoid else \
+        L.TOPK_SQRT_SOFTPLUS if use_sqrt_softplus else L.TOPK_SOFTMAX
+    if bias is not None:
+        bias = bias.float().contiguous()
+        if bias.numel() != E:
+            raise ValueError("bias must be contiguous CUDA float32 [experts]")
+    ids = torch.empty((T, top_k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((T, top_k), dtype=torch.float32, device=logits.device)
+    L.check(L.lib().mfq_hip_moe_topk(_ptr(logits), _ptr(bias), T, E, top_k, mode, int(normalize), norm_floor, scale,
+                                     _ptr(ids), _ptr(w), _stream()))
+    return ids, w
+
+
+@dataclass
+class MoeRoutePlan:
+    """cpp_runtime/mfq_decode.cpp:2579-2592."""
+    ids: torch.Tensor
+    n_experts: int
+    ids_dst: torch.Tensor | None = None
+    expert_bounds: torch.Tensor | None = None
+    tile_bounds: torch.Tensor | None = None
+    tile_experts: torch.Tensor | None = None
+    counts: torch.Tensor | None = None
+    map_ready: bool = False
+
+    @property
+    def tokens(self):
+        return self.ids.shape[0]
+
+    @property
+    def routes(self):
+        return self.ids.shape[1]
+
+
+def build_expert_map(ids: torch.Tensor, n_experts: int, tile_m: int):
+    """moe_build_expert_map_cuda (mfq/kernels/cuda/moe.cu:3082-3130)."""
+    n_pairs = ids.numel()
+    dev = ids.device
+    max_tiles = -(-n_pairs // tile_m) + n_experts
+    counts = torch.empty(n_experts, dtype=torch.int32, device=dev)
+    eb = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+    tb = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+    te = torch.zeros(max_tiles, dtype=torch.int32, device=dev)
+    dst = torch.zeros(n_pairs, dtype=torch.int32, device=dev)
+    L.check(L.lib().mfq_hip_moe_route_map(_ptr(ids), n_pairs, n_experts, tile_m, _ptr(counts), _ptr(eb), _ptr(tb),
+                                          _ptr(te), max_tiles, _ptr(dst), _stream()))
+    return dst, eb, tb, te, counts
+
+
+def build_moe_route_plan(ids: torch.Tensor, n_experts: int) -> MoeRoutePlan:
+    """cpp_runtime/mfq_decode.cpp:2681-2708: the expert map is built only above 8 tokens."""
+    if not ids.is_cuda or ids.dtype != torch.int32 or ids.dim() != 2:
+        raise RuntimeError("MoE ids must be CUDA int32 [tokens, routes]")
+    plan = MoeRoutePlan(ids.contiguous(), n_experts)
+    if plan.tokens > 8:
+        plan.ids_dst, plan.expert_bounds, plan.tile_bounds, plan.tile_experts, plan.counts = build_expert_map(
+            plan.ids, n_experts, L.lib().mfq_hip_moe_tile_m())
+    plan.map_ready = True
+    return plan
+
+
+class NintMoeWeight:
+    """One logical [experts, out_per_expert, K] tensor made of NINT cohorts (NINTM / NIM2)."""
+
+    def __init__(self, n_experts, out_per_expert, neuron_len, pools, expert_ids, device):
+        self.n_experts, self.out_per_expert, self.neuron_len = n_experts, out_per_expert, neuron_len
+        self.pools: list[NintWeight] = pools
+        self.pool_expert_ids = expert_ids
+        ep = np.full(n_experts, -1, dtype=np.int32)
+        el = np.full(n_experts, -1, dtype=np.int32)
+        for pi, ids in enumerate(expert_ids):
+            ep[ids] = pi
+            el[ids] = np.arange(len(ids), dtype=np.int32)
+        # device dispatch tables (initialize_nint_moe_dispatch, cpp_runtime/mfq_decode.cpp:3249-3343)
+        self.expert_pool = torch.from_numpy(ep).to(device)
+        self.expert_local = torch.from_numpy(el).to(device)
+        self._pool_array = (L.MoePool * len(pools))()
+        for i, p in enumerate(pools):
+            self._pool_array[i].desc = p.desc
+            self._pool_array[i].weight = p.data.data_ptr()
+        self.expert_bits = np.zeros(n_experts, dtype=np.int32)
+        for pi, ids in enumerate(expert_ids):
+            self.expert_bits[ids] = pools[pi].bits
+
+    @property
+    def payload_bytes(self) -> int:
+        return sum(p.payload_bytes for p in self.pools)
+
+    def expert_payload_bytes(self, e: int) -> float:
+        pi = int(self.expert_pool[e].item())
+        return self.pools[pi].payload_bytes / len(self.pool_expert_ids[pi])
+
+    @staticmethod
+    def from_blob(blob, device="cuda") -> "NintMoeWeight":
+        h = F.parse_nintm(blob)
+        device = torch.device(device)
+        pools, ids = [], []
+        for p in h.pools:
+            if not (p.dtype.startswith("NINT") and p.dtype[4:].isdigit()):
+                raise NotImplementedError(f"NINTM cohort family {p.dtype} is not on the accelerated path")
+            if p.runtime_bytes:
+                raise ValueError("unexpected NINTM cohort runtime metadata")
+            w = NintWeight.from_blob(bytes(blob[p.payload_off: p.payload_off + p.payload_bytes]), device)
+            if w.out != len(p.expert_ids) * h.out_per_expert or w.neuron_len != h.neuron_len:
+                raise ValueError(f"NINTM pool tensor shape {(w.out, w.neuron_len)} must be "
+                                 f"{(len(p.expert_ids) * h.out_per_expert, h.neuron_len)}")
+            pools.append(w)
+            ids.append(p.expert_ids)
+        return NintMoeWeight(h.n_experts, h.out_per_expert, h.neuron_len, pools, ids, device)
+
+    def dequantize(self) -> torch.Tensor:
+        out = torch.empty((self.n_experts, self.out_per_expert, self.neuron_len), dtype=torch.float32,
+                          device=self.expert_pool.device)
+        for p, ids in zip(self.pools, self.pool_expert_ids):
+            out[torch.from_numpy(ids.astype(np.int64)).to(out.device)] = p.dequantize().reshape(
+                len(ids), self.out_per_expert, self.neuron_len)
+        return out
+
+    def forward(self, x: torch.Tensor, route: MoeRoutePlan) -> torch.Tensor:
+        """NintMoeWeight::forward (cpp_runtime/mfq_decode.cpp:2908-3071): x is [T, K] (shared by the
+        routes of a token) or [T, R, K] (routed input); returns fp32 [T, R, out_per_expert]."""
+        T, R = route.tokens, route.routes
+        routed = x.dim() == 3
+        if x.shape[-1] != self.neuron_len or x.shape[0] != T or (routed and x.shape[1] != R):
+            raise ValueError("MoE activations must be [tokens, K] or [tokens, routes, K]")
+        x2 = x.reshape(-1, self.neuron_len)
+        if x2.stride(-1) != 1:
+            x2 = x2.contiguous()
+        out = torch.empty((T, R, self.out_per_expert), dtype=torch.float32, device=x.device)
+        mapped = route.ids_dst is not None
+        L.check(L.lib().mfq_hip_moe_grouped_matmul(
+            self._pool_array, len(self.pools), _ptr(self.expert_pool), _ptr(self.expert_local), self.n_experts,
+            self.out_per_expert, self.neuron_len, _ptr(x2), _x_dtype(x2), x2.stride(0), int(routed), _ptr(route.ids),
+            T, R, _ptr(route.ids_dst) if mapped else None, _ptr(route.expert_bounds) if mapped else None,
+            _ptr(route.tile_bounds) if mapped else None, _ptr(route.tile_experts) if mapped else None,
+            _ptr(out), self.out_per_expert, _stream()))
+        return out
+
+    __call__ = forward
+
+
+def moe_swiglu(gate_up: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """silu(gate) * up, gate = first half of the last axis (moe_swiglu_split_cuda)."""
+    W = gate_up.shape[-1] // 2
+    g2 = gate_up.reshape(-1, 2 * W)
+    hidden = torch.empty((g2.shape[0], W), dtype=out_dtype, device=gate_up.device)
+    L.check(L.lib().mfq_hip_moe_swiglu(_ptr(g2), g2.stride(0), g2.shape[0], W, _ptr(hidden),
+                                       L.X_F16 if out_dtype == torch.float16 else L.X_BF16, W, _stream()))
+    return hidden.reshape(*gate_up.shape[:-1], W)
+
+
+def moe_weighted_reduce(pair: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None = None,
+                        gate_logits: torch.Tensor | None = None) -> torch.Tensor:
+    T, R, H = pair.shape
+    out = torch.empty((T, H), dtype=torch.float32, device=pair.device)
+    L.check(L.lib().mfq_hip_moe_weighted_reduce(_ptr(pair.contiguous()), _ptr(weights.contiguous()), T, R, H,
+                                                _ptr(shared), _ptr(gate_logits), _ptr(out), _stream()))
+    return out
+
+
+def nint_moe_ffn_forward(gate_up: NintMoeWeight, down: NintMoeWeight, x: torch.Tensor, router_logits: torch.Tensor,
+                         top_k: int, use_sigmoid=False, use_sqrt_softplus=False, normalize=False,
+                         delayed_softmax=False, router_bias=None, router_scale=1.0, shared=None):
+    """cpp_runtime/mfq_decode.cpp:3394-3416.  `shared` = (gate_up NintWeight [2W, H], down NintWeight [H, W]) of the
+    shared expert, added ungated (cpp_runtime/mfq_decode.cpp:11077-11080).  Returns (out, ids, weights)."""
+    if gate_up.n_experts != down.n_experts or gate_up.out_per_expert != 2 * down.neuron_len or \
+            down.out_per_expert != gate_up.neuron_len:
+        raise RuntimeError("incompatible fused gate_up/down NINTM tensors")
+    ids, w = moe_topk(router_logits, top_k, use_sigmoid, use_sqrt_softplus, normalize, delayed_softmax, router_bias,
+                      1e-20, router_scale)
+    route = build_moe_route_plan(ids, gate_up.n_experts)
+    gu = gate_up.forward(x, route)
+    hidden = moe_swiglu(gu)
+    dn = down.forward(hidden, route)
+    sh = None
+    if shared is not None:
+        sgu, sdn = shared
+        sh = nint_matmul(sdn, moe_swiglu(nint_matmul(sgu, x)))
+    return moe_weighted_reduce(dn, w, sh), ids, w

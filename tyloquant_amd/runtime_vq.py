@@ -1,0 +1,152 @@
+"""NVQ (D4 family) and NEPQ1 weights and their matmul entry points (see runtime.py)."""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+import numpy as np
+import torch
+
+from . import _lib as L
+from . import formats as F
+from .runtime import _Workspace, _as_2d, _ptr, _stream, _upload, _x_dtype
+
+_DATA = Path(__file__).resolve().parent / "data"
+
+
+def builtin_grid(name: str) -> np.ndarray:
+    """The magnitude grids of the non-JSC formats, decoded as 2*digit+1 from the raw tables
+    (mfq/formats/nvq.py:102-129)."""
+    raw = np.frombuffer((_DATA / f"{name}.bin").read_bytes(), dtype="<u2")
+    dims, digit_bits = (8, 2) if name.startswith("e8_") else (4, 3)
+    digits = (raw[:, None] >> (digit_bits * np.arange(dims, dtype=np.uint16))[None, :]) & ((1 << digit_bits) - 1)
+    return np.ascontiguousarray(2 * digits + 1, dtype=np.int8)
+
+
+class NvqWeight:
+    def __init__(self, desc, data, dtype):
+        self.desc, self.data, self.dtype = desc, data, dtype
+        self.out, self.neuron_len = desc.out, desc.neuron_len
+        self._ws = _Workspace()
+
+    @property
+    def payload_bytes(self) -> int:
+        return int(self.desc.payload_bytes)
+
+    @staticmethod
+    def from_blob(blob, device="cuda") -> "NvqWeight":
+        h = F.parse_nvq(blob)
+        if h.vector_size != 4 or h.index_bits > 9:
+            raise NotImplementedError(f"{h.dtype}: only the D4 256/512-entry NVQ formats are on the accelerated path")
+        device = torch.device(device)
+        desc = L.NvqDesc()
+        lib = L.lib()
+        L.check(lib.mfq_hip_nvq_plan(h.index_bits, h.banks if h.jsc else 1, h.out, h.neuron_len, C.byref(desc)))
+        payload = _upload(blob, h.body_off, h.body_bytes, device)
+        data = torch.empty(int(desc.total_bytes), dtype=torch.uint8, device=device)
+        if h.jsc:
+            L.check(lib.mfq_hip_nvq_repack(C.byref(desc), _ptr(payload), h.body_bytes, _ptr(data), _stream()))
+        else:
+            if h.gs != 24 or h.sub_bits != 4 or h.sign_mode != "even":
+                raise NotImplementedError("plain NVQ3 runs only with gs24, 4-bit sub-scales and parity signs")
+            grid = torch.from_numpy(builtin_grid(h.codebook)).to(device)
+            L.check(lib.mfq_hip_nvq_repack_plain(C.byref(desc), _ptr(payload), h.body_bytes, _ptr(grid), _ptr(data),
+                                                 _stream()))
+        torch.cuda.current_stream().synchronize()
+        return NvqWeight(desc, data, h.dtype)
+
+    def dequantize(self) -> torch.Tensor:
+        w = torch.empty((self.out, self.neuron_len), dtype=torch.float32, device=self.data.device)
+        L.check(L.lib().mfq_hip_nvq_dequant_f32(C.byref(self.desc), _ptr(self.data), _ptr(w), self.neuron_len, _stream()))
+        return w
+
+
+def nvq_matmul(w: NvqWeight, x: torch.Tensor, *, force: str | None = None) -> torch.Tensor:
+    """cpp_runtime/mfq_decode.cpp:7884: GEMV up to M = 13 for the D4 family, MFMA path above."""
+    x2 = _as_2d(x, w.neuron_len)
+    M = x2.shape[0]
+    y = torch.empty((M, w.out), dtype=torch.float32, device=x.device)
+    lib = L.lib()
+    if force == "gemv":
+        L.check(lib.mfq_hip_nvq_gemv(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
+                                     w.out, _stream()))
+    else:
+        need = lib.mfq_hip_nvq_gemm_workspace_bytes(C.byref(w.desc), M)
+        ws = w._ws.get(need, x.device)
+        L.check(lib.mfq_hip_nvq_gemm(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
+                                     w.out, _ptr(ws), need, _stream()))
+    return y.reshape(*x.shape[:-1], w.out)
+
+
+class NepqWeight:
+    """[experts, out_per_expert, K]; a dense linear is the experts == 1 case."""
+
+    def __init__(self, desc, data, header: F.NepqHeader, signs):
+        self.desc, self.data, self.label = desc, data, header.label
+        self.n_experts, self.out_per_expert, self.neuron_len = header.n_experts, header.out_per_expert, header.neuron_len
+        self.out = header.out_per_expert
+        self.rotation_block, self.rotation_seed, self.signs = header.rotation_block, header.rotation_seed, signs
+        self._ws = _Workspace()
+
+    @property
+    def payload_bytes(self) -> int:
+        return int(self.desc.payload_bytes)
+
+    @staticmethod
+    def from_blob(blob, device="cuda", rotation_signs=None) -> "NepqWeight":
+        h = F.parse_nepq(blob)
+        device = torch.device(device)
+        desc = L.NepqDesc()
+        lib = L.lib()
+        L.check(lib.mfq_hip_nepq_plan(h.profile, h.banks, h.n_experts * h.out_per_expert, h.neuron_len, C.byref(desc)))
+        payload = _upload(blob, h.body_off, h.body_bytes, device)
+        data = torch.empty(int(desc.total_bytes), dtype=torch.uint8, device=device)
+        L.check(lib.mfq_hip_nepq_repack(C.byref(desc), _ptr(payload), h.body_bytes, _ptr(data), _stream()))
+        torch.cuda.current_stream().synchronize()
+        signs = None
+        if h.rotation_block:
+            if rotation_signs is None:
+                raise ValueError("rotated NEPQ cohort lacks its runtime sign vector")
+            sv = np.ascontiguousarray(rotation_signs, dtype=np.int8).reshape(-1)
+            if sv.size != h.neuron_len or not np.all(np.abs(sv) == 1):
+                raise ValueError("NEPQ rotation sign vector is corrupt")
+            signs = torch.from_numpy(sv).to(device)
+        return NepqWeight(desc, data, h, signs)
+
+    def dequantize(self) -> torch.Tensor:
+        rows = self.n_experts * self.out_per_expert
+        w = torch.empty((rows, self.neuron_len), dtype=torch.float32, device=self.data.device)
+        L.check(L.lib().mfq_hip_nepq_dequant_f32(C.byref(self.desc), _ptr(self.data), _ptr(w), self.neuron_len, _stream()))
+        return w.reshape(self.n_experts, self.out_per_expert, self.neuron_len)
+
+
+def nepq_hadamard(x: torch.Tensor, signs: torch.Tensor, block: int) -> torch.Tensor:
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    out = torch.empty_like(x2)
+    L.check(L.lib().mfq_hip_nepq_hadamard(_ptr(x2), _x_dtype(x2), x2.stride(0), x2.shape[0], x2.shape[1], block,
+                                          _ptr(signs), _ptr(out), out.stride(0), _stream()))
+    return out.reshape(x.shape)
+
+
+def nepq_matmul(w: NepqWeight, x: torch.Tensor, expert: int = 0, *, force: str | None = None) -> torch.Tensor:
+    """mfq/kernels/cuda/nepq_matmul.py:215-280: rotate the input when the tensor is rotated, then
+    GEMV (M <= 16) or the MFMA path."""
+    if not 0 <= expert < w.n_experts:
+        raise ValueError(f"expert {expert} outside [0, {w.n_experts})")
+    if w.rotation_block:
+        x = nepq_hadamard(x, w.signs, w.rotation_block)
+    x2 = _as_2d(x, w.neuron_len)
+    M = x2.shape[0]
+    n = w.out_per_expert
+    y = torch.empty((M, n), dtype=torch.float32, device=x.device)
+    lib = L.lib()
+    row0 = expert * n
+    if force == "gemv":
+        L.check(lib.mfq_hip_nepq_gemv(C.byref(w.desc), _ptr(w.data), row0, n, _ptr(x2), _x_dtype(x2), x2.stride(0), M,
+                                      _ptr(y), n, _stream()))
+    else:
+        need = lib.mfq_hip_nepq_gemm_workspace_bytes(C.byref(w.desc), n, M)
+        ws = w._ws.get(need, x.device)
+        L.check(lib.mfq_hip_nepq_gemm(C.byref(w.desc), _ptr(w.data), row0, n, _ptr(x2), _x_dtype(x2), x2.stride(0), M,
+                                      _ptr(y), n, _ptr(ws), need, _stream()))
+    return y.reshape(*x.shape[:-1], n)
