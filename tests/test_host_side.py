@@ -126,3 +126,14 @@ def test_plan_calls_need_no_gpu():
     assert q.payload_bytes - 2048 == 8944128
     with pytest.raises(L.MfqError, match="divisible by 8"):
         L.check(lib.mfq_hip_nepq_plan(2, 1, 16, 100, ctypes.byref(q)))
+
+
+def test_product_quantizer_matches_the_reference_golden_vectors():
+    from tyloquant_amd.quantize import nint_quantize
+    g = np.load(Path(__file__).parent / "golden" / "nint_quant_vectors.npz")
+    for k in sorted({n.split("_")[0] for n in g.files}):
+        _, rows, K, bits, gs, sb = (int(v) for v in g[k + "_meta"])
+        r = nint_quantize(g[k + "_W"], bits, gs, sb, row_chunk=5)
+        assert np.array_equal(r["q"], g[k + "_q"]) and np.array_equal(r["ss"], g[k + "_ss"]), k
+        assert np.array_equal(r["sm"], g[k + "_sm"]) and np.array_equal(r["ns"], g[k + "_ns"]), k
+        assert np.array_equal(r["nm"], g[k + "_nm"]), k

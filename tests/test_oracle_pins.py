@@ -329,3 +329,25 @@ def test_bf16_rounding_is_nearest_even():
     torch = pytest.importorskip("torch")
     x = np.random.default_rng(10).standard_normal(4096).astype(np.float32) * 3
     assert np.array_equal(O.bf16_round(x), torch.from_numpy(x).to(torch.bfloat16).float().numpy())
+
+
+def test_c_restatement_matches_the_numpy_oracle_bit_for_bit():
+    """oracle/mfq_oracle_c.c (timed as the CPU baseline) against oracle/mfq_oracle.py and the golden vectors."""
+    from oracle import c_oracle
+    if not c_oracle.LIB.exists():
+        pytest.skip("oracle/libmfq_oracle.so is not built (make -C oracle)")
+    rng = np.random.default_rng(12)
+    for spec in [(3, 24, 5), (4, 32, 6), (5, 28, 7), (8, 24, 8), (2, 16, 5)]:
+        t = synth.nint_random(rng, 19, 203, *spec)
+        blob = O.pack_nint(t)
+        body = blob[14 + 4 + 16 + 8:]
+        W = c_oracle.nint_dequant(body, spec[0], spec[2], spec[1], 19, 203)
+        assert np.array_equal(W.view(np.uint32), O.dequantize_nint(t).view(np.uint32))
+    g = np.load(GOLD / "nint_quant_vectors.npz")
+    t = O.quantize_nint(g["c7_W"], 3, 24, 5)
+    W = c_oracle.nint_dequant(O.pack_nint(t)[42:], 3, 5, 24, 16, 4096)
+    assert np.array_equal(W, g["c7_deq"])
+    x = rng.standard_normal((3, 4096)).astype(np.float32)
+    y = c_oracle.matmul_nt(x, W)
+    ref = O.linear_forward_f64(W, x)
+    assert np.abs(y - ref).max() < 1e-4 * np.abs(ref).max()
