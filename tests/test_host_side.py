@@ -137,3 +137,15 @@ def test_product_quantizer_matches_the_reference_golden_vectors():
         assert np.array_equal(r["q"], g[k + "_q"]) and np.array_equal(r["ss"], g[k + "_ss"]), k
         assert np.array_equal(r["sm"], g[k + "_sm"]) and np.array_equal(r["ns"], g[k + "_ns"]), k
         assert np.array_equal(r["nm"], g[k + "_nm"]), k
+
+
+def test_grouped_projection_blob_is_the_row_concatenation():
+    rng = np.random.default_rng(5)
+    a, b = synth.nint_random(rng, 16, 100, 3, 24, 5), synth.nint_random(rng, 9, 100, 3, 24, 5)
+    cat = O.unpack_nint(F.nint_concat_rows([O.pack_nint(a), O.pack_nint(b)]))
+    assert np.array_equal(O.dequantize_nint(cat), np.concatenate([O.dequantize_nint(a), O.dequantize_nint(b)]))
+    for bits in (1, 3, 5, 7, 8, 9, 11):
+        v = rng.integers(0, 1 << bits, 77)
+        assert np.array_equal(F.unpack_bitstream(O.pack_bits(v, bits), 0, 77, bits), v)
+    with pytest.raises(ValueError, match="must share"):
+        F.nint_concat_rows([O.pack_nint(a), O.pack_nint(synth.nint_random(rng, 4, 100, 4, 24, 6))])

@@ -359,11 +359,9 @@ extern "C" int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools
         k.step_bytes = d.step_bytes; k.rowblock_bytes = d.rowblock_bytes; k.anchors_off = d.anchors_off;
         P.w[i] = static_cast<const uint8_t *>(pools[i].weight);
         P.spw[i] = static_cast<int>(ceil_div(d.nsteps, nwaves));
-        const size_t need = static_cast<size_t>(mb) * P.spw[i] * 16 * (d.gs / 2 + 1) * 4 * nwaves;
+        const size_t need = gemv_lds_bytes(mb, P.spw[i], d.gs, nwaves);
         if (need > lds) lds = need;
     }
-    const size_t red = static_cast<size_t>(nwaves) * mb * 16 * 4;
-    if (lds < red) lds = red;
     MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "moe_grouped_matmul: K=%d needs %zu bytes of LDS", K, lds);
     hipStream_t st = as_stream(stream);
     const dim3 grid(static_cast<unsigned>(tiles), rbe), block(64 * nwaves);

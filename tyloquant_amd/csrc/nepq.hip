@@ -152,8 +152,8 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
                                                          int nrows, const uint16_t *__restrict__ x, int64_t ldx, int M,
                                                          float *__restrict__ y, int64_t ldy, int spw) {
     extern __shared__ uint32_t lds[];
-    constexpr uint32_t MAGIC = XF16 ? 0x64006400u : 0x43004300u;
-    constexpr float BIAS = XF16 ? 1024.f : 128.f;
+    constexpr uint32_t MAGIC = 0x64006400u;  // fp16 (1024, 1024): digit d becomes 1024 + d
+    constexpr float BIAS = 1024.f;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const int rb = rb0 + blockIdx.x;
     const uint16_t *xr[MB];
@@ -171,9 +171,11 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
     const int s0 = wave * spw;
     const int s1 = min(k.nsteps, s0 + spw);
     const int ngl = spw * 16, npairs = ngl * 12;
-    uint32_t *xs = xbase + wave * (MB * (npairs + ngl));
+    uint32_t *xs = xbase + wave * (MB * (npairs + 2 * ngl));
     float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
-    stage_x<XF16, MB>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane);
+    float *red = reinterpret_cast<float *>(xbase + nwaves * (MB * (npairs + 2 * ngl)));
+    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane);
+    if constexpr (TAB_LDS) __syncthreads();  // the LDS table copy was made by the whole block
 
     const int r = lane & 15, kb = lane >> 4;
     const uint8_t *base = w + static_cast<int64_t>(rb) * k.rowblock_bytes;
@@ -207,30 +209,28 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
                 for (int p = 0; p < 4; ++p) {
                     const uint32_t pr = ((t >> (4 * p)) & 0x00030003u) | MAGIC;
 #pragma unroll
-                    for (int m = 0; m < MB; ++m) raw[m] = dot2<XF16>(pr, xs[m * npairs + lg * 12 + 4 * v + p], raw[m]);
+                    for (int m = 0; m < MB; ++m) raw[m] = dot2h(pr, xs[m * npairs + lg * 12 + 4 * v + p], raw[m]);
                 }
             }
 #pragma unroll
-            for (int m = 0; m < MB; ++m) acc[m] = fmaf(st, fmaf(off, xsum[m * ngl + lg], raw[m]), acc[m]);
+            for (int m = 0; m < MB; ++m) acc[m] = fmaf(st, fmaf(off, xsum[(m * ngl + lg) * 2], raw[m]), acc[m]);
         }
     }
     const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[rb * 16 + r];
     float v[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) v[m] = anchor * acc[m];
-    finish_rows<MB>(v, reinterpret_cast<float *>(xbase), wave, nwaves, lane, rb, row0, nrows, yr);
+    finish_rows<MB>(v, red, wave, nwaves, lane, rb, row0, nrows, yr);
 }
 
 static void nepq_gemv_shape(const NepqK &k, int nrb, int mb, int &spw, int &nwaves, size_t &lds_bytes, bool &tab_lds) {
-    int want = static_cast<int>(ceil_div(6144, nrb));
+    int want = static_cast<int>(ceil_div(gemv_target_waves(), nrb));
     if (want < 1) want = 1;
     if (want > 16) want = 16;
     if (want > k.nsteps) want = k.nsteps;
     spw = static_cast<int>(ceil_div(k.nsteps, want));
     nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
-    size_t xb = static_cast<size_t>(mb) * spw * 16 * 13 * 4 * nwaves;
-    const size_t red = static_cast<size_t>(nwaves) * mb * 16 * 4;
-    if (xb < red) xb = red;
+    const size_t xb = gemv_lds_bytes(mb, spw, 24, nwaves);
     const size_t tabb = static_cast<size_t>(k.banks) * k.entries * 2;
     tab_lds = tabb + xb <= 65536;
     lds_bytes = xb + (tab_lds ? tabb : 0);

@@ -185,16 +185,13 @@ __global__ void nint_dequant_kernel(NintK k, const uint8_t *__restrict__ w, OutT
 // ---- GEMV ------------------------------------------------------------------------------
 // steps per wave / waves per block so that the grid has a few thousand waves and LDS fits
 static void gemv_shape(const NintK &k, int mb, int &spw, int &nwaves, size_t &lds_bytes) {
-    int want = static_cast<int>(ceil_div(6144, k.n_rowblocks));
+    int want = static_cast<int>(ceil_div(gemv_target_waves(), k.n_rowblocks));
     if (want < 1) want = 1;
     if (want > 16) want = 16;
     if (want > k.nsteps) want = k.nsteps;
     spw = static_cast<int>(ceil_div(k.nsteps, want));
     nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
-    const size_t per_wave = static_cast<size_t>(mb) * spw * 16 * (k.gs / 2 + 1) * 4;
-    lds_bytes = per_wave * nwaves;
-    const size_t red = static_cast<size_t>(nwaves) * mb * 16 * 4;
-    if (lds_bytes < red) lds_bytes = red;
+    lds_bytes = gemv_lds_bytes(mb, spw, k.gs, nwaves);
 }
 
 template <int XF16, int MB>

@@ -163,7 +163,7 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
     float *yr[MB];
     dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
     const int ncb = k.banks * k.entries;
-    uint32_t *cbp = lds;                 // 2 dwords per entry: (m0, m1), (m2, m3) in the activation type
+    uint32_t *cbp = lds;                 // 2 dwords per entry: (m0, m1), (m2, m3) as fp16 pairs
     uint32_t *sgx = cbp + 2 * ncb;       // 4 dwords per 7-bit mask
     float *lutf = reinterpret_cast<float *>(sgx + 512);
     uint32_t *bankoff = reinterpret_cast<uint32_t *>(lutf + 16);
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const float f = static_cast<float>((e >> (8 * t)) & 0xffu);
-                h[t] = XF16 ? f32_to_f16_rne(f) : f32_to_bf16_rne(f);
+                h[t] = f32_to_f16_rne(f);
             }
             cbp[2 * i] = h[0] | (h[1] << 16);
             cbp[2 * i + 1] = h[2] | (h[3] << 16);
@@ -197,22 +197,33 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
     const int s0 = wave * spw;
     const int s1 = min(k.nsteps, s0 + spw);
     const int ngl = spw * 16, npairs = ngl * 12;
-    uint32_t *xs = xbase + wave * (MB * (npairs + ngl));
+    uint32_t *xs = xbase + wave * (MB * (npairs + 2 * ngl));
     float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
-    stage_x<XF16, MB>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane);
+    float *red = reinterpret_cast<float *>(xbase + nwaves * (MB * (npairs + 2 * ngl)));
+    const uint8_t *base = w + static_cast<int64_t>(rb) * k.rowblock_bytes;
+    struct Step {
+        u32x2_t q[4], hh;
+    };
+    auto load_step = [&](int s, Step &st) {
+        const uint8_t *sp = base + s * k.step_bytes;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) st.q[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp) + j * 64 + lane);
+        st.hh = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp + 2048) + lane);
+    };
+    Step cur, nxt;
+    if (s0 < s1) load_step(s0, cur);
+    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane);
+    __syncthreads();  // the LDS tables were filled by the whole block
 
     const int r = lane & 15, kb = lane >> 4;
-    const uint8_t *base = w + rb * k.rowblock_bytes;
     const uint32_t im = (1u << k.ib) - 1u;
     float acc[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) acc[m] = 0.f;
     for (int s = s0; s < s1; ++s) {
-        const uint8_t *sp = base + s * k.step_bytes;
-        u32x2_t q[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) q[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp) + j * 64 + lane);
-        const u32x2_t hh = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp + 2048) + lane);
+        if (s + 1 < s1) load_step(s + 1, nxt);
+        const u32x2_t *q = cur.q;
+        const u32x2_t hh = cur.hh;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int lg = (s - s0) * 16 + 4 * j + kb;
@@ -236,34 +247,32 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
 #pragma unroll
                 for (int m = 0; m < MB; ++m) {
                     const uint32_t *xp = xs + m * npairs + lg * 12 + 4 * v;
-                    raw[m] = dot2<XF16>(w0, xp[0], raw[m]);
-                    raw[m] = dot2<XF16>(w1, xp[1], raw[m]);
-                    raw[m] = dot2<XF16>(w2, xp[2], raw[m]);
-                    raw[m] = dot2<XF16>(w3, xp[3], raw[m]);
+                    raw[m] = dot2h(w0, xp[0], raw[m]);
+                    raw[m] = dot2h(w1, xp[1], raw[m]);
+                    raw[m] = dot2h(w2, xp[2], raw[m]);
+                    raw[m] = dot2h(w3, xp[3], raw[m]);
                 }
             }
 #pragma unroll
             for (int m = 0; m < MB; ++m) acc[m] = fmaf(sc, raw[m], acc[m]);
         }
+        if (s + 1 < s1) cur = nxt;
     }
     const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[rb * 16 + r];
     float v[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) v[m] = anchor * acc[m];
-    finish_rows<MB>(v, reinterpret_cast<float *>(xbase), wave, nwaves, lane, rb, 0, k.out, yr);
+    finish_rows<MB>(v, red, wave, nwaves, lane, rb, 0, k.out, yr);
 }
 
 static void nvq_gemv_shape(const NvqK &k, int mb, int &spw, int &nwaves, size_t &lds_bytes) {
-    int want = static_cast<int>(ceil_div(6144, k.n_rowblocks));
+    int want = static_cast<int>(ceil_div(gemv_target_waves(), k.n_rowblocks));
     if (want < 1) want = 1;
     if (want > 16) want = 16;
     if (want > k.nsteps) want = k.nsteps;
     spw = static_cast<int>(ceil_div(k.nsteps, want));
     nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
-    size_t xb = static_cast<size_t>(mb) * spw * 16 * 13 * 4 * nwaves;
-    const size_t red = static_cast<size_t>(nwaves) * mb * 16 * 4;
-    if (xb < red) xb = red;
-    lds_bytes = (static_cast<size_t>(k.banks) * k.entries * 2 + 512 + 32) * 4 + xb;
+    lds_bytes = (static_cast<size_t>(k.banks) * k.entries * 2 + 512 + 32) * 4 + gemv_lds_bytes(mb, spw, 24, nwaves);
 }
 
 template <int XF16, int MB>

@@ -40,6 +40,24 @@ def pack_bitstream(values, bits: int) -> bytes:
     return b"".join(parts)
 
 
+def unpack_bitstream(blob, off: int, count: int, bits: int) -> np.ndarray:
+    """Inverse of pack_bitstream (mfq/formats/io.py:165-188); returns uint8 (bits <= 8) or uint16 values."""
+    if bits == 0 or count == 0:
+        return np.empty(0, dtype=np.uint8)
+    nbytes = (count * bits + 7) // 8
+    if off + nbytes > len(blob):
+        raise ValueError("truncated bit stream")
+    packed = np.frombuffer(blob, dtype=np.uint8, count=nbytes, offset=off)
+    if bits == 8:
+        return packed.copy()
+    rows = np.unpackbits(packed, bitorder="little")[: count * bits].reshape(count, bits)
+    if bits <= 8:
+        return np.packbits(rows, axis=1, bitorder="little").reshape(-1)
+    lo = np.packbits(rows[:, :8], axis=1, bitorder="little").reshape(-1).astype(np.uint16)
+    hi = np.packbits(rows[:, 8:], axis=1, bitorder="little").reshape(-1).astype(np.uint16)
+    return lo | (hi << 8)
+
+
 # ---------------------------------------------------------------------------------------
 # NINT (mfq/formats/io.py:191-248)
 # ---------------------------------------------------------------------------------------
@@ -103,6 +121,37 @@ def parse_nint(blob) -> NintHeader:
         raise ValueError(f"invalid NINT blob tail: remaining={remaining - 4 * out}, "
                          f"packed={packed - 4 * out}, old={old - 4 * out}")
     return NintHeader(bits, sub_bits, gs, axis, neuron_len, tuple(shape), out, ng, off, remaining, legacy)
+
+
+def nint_arrays(blob) -> dict:
+    """Packed-domain arrays of a NINT blob (the unpack half of mfq/formats/io.py:206-248)."""
+    h = parse_nint(blob)
+    out, ng, gs = h.out, h.ng, h.gs
+    off = h.body_off
+    ns = np.frombuffer(blob, dtype=np.float16, count=out, offset=off).astype(np.float32)
+    nm = np.frombuffer(blob, dtype=np.float16, count=out, offset=off + 2 * out).astype(np.float32)
+    off += 4 * out
+    sb, qb = (8, 8) if h.legacy else (h.sub_bits, h.bits)
+    ss = unpack_bitstream(blob, off, out * ng, sb).reshape(out, ng)
+    off += (out * ng * sb + 7) // 8
+    sm = unpack_bitstream(blob, off, out * ng, sb).reshape(out, ng)
+    off += (out * ng * sb + 7) // 8
+    q = unpack_bitstream(blob, off, out * ng * gs, qb).reshape(out, ng, gs)
+    return {"bits": h.bits, "sub_bits": h.sub_bits, "gs": gs, "neuron_len": h.neuron_len, "ns": ns, "nm": nm,
+            "ss": ss, "sm": sm, "q": q}
+
+
+def nint_concat_rows(blobs) -> bytes:
+    """One NINT blob holding the neurons of several tensors of the same spec one after the other: the
+    concatenated weight of a projection group (NintLinearGroup, cpp_runtime/mfq_decode.cpp:8618-8660)."""
+    parts = [nint_arrays(b) for b in blobs]
+    a = parts[0]
+    for p in parts[1:]:
+        if (p["bits"], p["sub_bits"], p["gs"], p["neuron_len"]) != (a["bits"], a["sub_bits"], a["gs"], a["neuron_len"]):
+            raise ValueError("grouped NINT projections must share bits, sub_bits, groupsize and neuron length")
+    cat = {k: np.concatenate([p[k] for p in parts], axis=0) for k in ("ns", "nm", "ss", "sm", "q")}
+    return nint_blob(a["bits"], a["sub_bits"], a["gs"], a["neuron_len"], cat["ns"], cat["nm"], cat["ss"], cat["sm"],
+                     cat["q"])
 
 
 # ---------------------------------------------------------------------------------------

@@ -125,6 +125,24 @@ def nint_matmul(w: NintWeight, x: torch.Tensor, *, force: str | None = None) -> 
     return y.reshape(*x.shape[:-1], w.out)
 
 
+class NintLinearGroup:
+    """Projections that share their input (gate/up, Q/K/V) kept as one concatenated NintWeight and run as
+    one matmul whose output is split afterwards (cpp_runtime/mfq_decode.cpp:8618-8660)."""
+
+    def __init__(self, weight: NintWeight, outs):
+        self.w, self.outs = weight, [int(o) for o in outs]
+
+    @staticmethod
+    def from_blobs(blobs, device="cuda") -> "NintLinearGroup":
+        outs = [F.parse_nint(b).out for b in blobs]
+        return NintLinearGroup(NintWeight.from_blob(F.nint_concat_rows(blobs), device), outs)
+
+    def forward(self, x: torch.Tensor):
+        return list(nint_matmul(self.w, x).split(self.outs, dim=-1))
+
+    __call__ = forward
+
+
 # ---------------------------------------------------------------------------------------
 # dtype registry
 # ---------------------------------------------------------------------------------------
