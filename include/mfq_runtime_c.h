@@ -1,0 +1,40 @@
+/*
+ * mfq_runtime_c.h -- flat C view of the C++ host runtime (libmfq_runtime.so), for language bindings
+ * and tests.  The C++ API itself is tyloquant_amd/cpp_runtime/mfq_runtime.h; the kernel-level
+ * drop-in boundary is mfq_hip.h.  Every call returns 0 on success; mfq_rt_last_error() holds the
+ * message of the last failure on the calling thread.  Pointers named x / y / out are device pointers.
+ */
+#ifndef MFQ_RUNTIME_C_H
+#define MFQ_RUNTIME_C_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char *mfq_rt_last_error(void);
+
+/* load_quant_linear (cpp_runtime/mfq_decode.cpp:9489-9771): host blob + MFQ dtype string -> device weight. */
+int mfq_rt_load_quant_linear(const char *dtype, const void *blob, size_t n, void **handle);
+void mfq_rt_free_quant_linear(void *handle);
+int64_t mfq_rt_linear_out(void *handle);
+int64_t mfq_rt_linear_neuron_len(void *handle);
+/* QuantLinear::forward (cpp_runtime/mfq_decode.cpp:9209-9226): y[M, out] fp32 = x[M, K] . W^T. */
+int mfq_rt_linear_forward(void *handle, const void *x, int x_dtype, int64_t ldx, int M, float *y, void *stream);
+int mfq_rt_linear_dequantize(void *handle, float *out, void *stream);
+/* run_linear_check (cpp_runtime/mfq_decode.cpp:16510-16638): out6 = production_ms, production_weight_gbps,
+ * payload_gbps, production_rel, production_mean_abs, production_max_abs. */
+int mfq_rt_linear_check(void *handle, int M, int reps, double *out6);
+
+/* NINTM expert-wise tensors and nint_moe_ffn_forward (cpp_runtime/mfq_decode.cpp:3394-3416). */
+int mfq_rt_load_nint_moe(const void *blob, size_t n, void **handle);
+void mfq_rt_free_nint_moe(void *handle);
+int mfq_rt_moe_ffn_forward(void *gate_up, void *down, const void *x, int x_dtype, int64_t ldx, int T,
+                           const float *router_logits, int top_k, int topk_mode, int normalize,
+                           void *shared_gate_up, void *shared_down, float *out, int32_t *ids_out,
+                           float *weights_out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

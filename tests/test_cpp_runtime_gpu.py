@@ -1,0 +1,121 @@
+"""The C++ host runtime (libmfq_runtime.so) and the mfq-check-linear tool on the GPU, in the style of the
+reference's C++-runtime subprocess tests (tests/test_nvq3j512_cpp_runtime.py:111-143): write a tiny .mfq
+with Python, run the tool, parse its key=value report."""
+import ctypes as C
+import re
+import subprocess
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import synth
+from conftest import check_close
+from oracle import mfq_oracle as O
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+LIBDIR = Path(__file__).resolve().parents[1] / "tyloquant_amd" / "lib"
+
+
+@pytest.fixture(scope="module")
+def rt():
+    lib = C.CDLL(str(LIBDIR / "libmfq_runtime.so"))
+    lib.mfq_rt_last_error.restype = C.c_char_p
+    lib.mfq_rt_linear_out.restype = C.c_int64
+    lib.mfq_rt_linear_neuron_len.restype = C.c_int64
+    lib.mfq_rt_linear_out.argtypes = lib.mfq_rt_linear_neuron_len.argtypes = [C.c_void_p]
+    lib.mfq_rt_load_quant_linear.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_void_p)]
+    lib.mfq_rt_free_quant_linear.argtypes = [C.c_void_p]
+    lib.mfq_rt_linear_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]
+    lib.mfq_rt_linear_dequantize.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.mfq_rt_load_nint_moe.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(C.c_void_p)]
+    lib.mfq_rt_free_nint_moe.argtypes = [C.c_void_p]
+    lib.mfq_rt_moe_ffn_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p,
+                                           C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                           C.c_void_p, C.c_void_p]
+    return lib
+
+
+def _load(rt, dtype, blob):
+    h = C.c_void_p()
+    rc = rt.mfq_rt_load_quant_linear(dtype.encode(), blob, len(blob), C.byref(h))
+    if rc:
+        raise RuntimeError(rt.mfq_rt_last_error().decode())
+    return h
+
+
+def test_check_linear_tool_reports_small_error(tmp_path):
+    rng = np.random.default_rng(3)
+    tensors = {
+        "blk.0.q.nint3": synth.nint_random(rng, 37, 96, 3, 24, 5),
+        "blk.0.ffn.nint4": O.quantize_nint((rng.standard_normal((64, 200)) * 0.02).astype(np.float32), 4, 32, 6),
+        "blk.0.k.nvq3j512": synth.nvq_jsc_random(rng, 37, 96),
+        "blk.0.v.nepq1s": synth.nepq_random(rng, "NEPQ1-S", 1, 48, 96, 3),
+    }
+    path = tmp_path / "tiny.mfq"
+    O.mfq_file_write(path, tensors, version=2)
+    for name in tensors:
+        for M in (1, 16, 65):
+            r = subprocess.run([str(LIBDIR / "mfq-check-linear"), str(path), name, str(M), "20"], capture_output=True,
+                               text=True, timeout=120)
+            assert r.returncode == 0, r.stderr
+            rel = float(re.search(r"production_rel=([0-9.eE+-]+)", r.stdout).group(1))
+            assert rel < 1e-3, (name, M, r.stdout)
+            assert "production_weight_gbps=" in r.stdout and "payload_gbps=" in r.stdout
+    r = subprocess.run([str(LIBDIR / "mfq-check-linear"), str(path), "missing"], capture_output=True, text=True)
+    assert r.returncode == 1 and "tensor not found" in r.stderr
+
+
+def test_cpp_load_quant_linear_and_forward(rt):
+    rng = np.random.default_rng(4)
+    t = O.quantize_nint((rng.standard_normal((48, 88)) * 0.02).astype(np.float32), 3, 24, 5)
+    h = _load(rt, "NINT3", O.pack_nint(t))
+    assert rt.mfq_rt_linear_out(h) == 48 and rt.mfq_rt_linear_neuron_len(h) == 88
+    W = torch.empty((48, 88), dtype=torch.float32, device="cuda")
+    assert rt.mfq_rt_linear_dequantize(h, W.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    deq = O.dequantize_nint(t)
+    assert np.array_equal(W.cpu().numpy().view(np.uint32), deq.view(np.uint32))
+    for M in (1, 9, 40):
+        x = torch.from_numpy(rng.standard_normal((M, 88)).astype(np.float32)).to(torch.bfloat16).cuda()
+        y = torch.empty((M, 48), dtype=torch.float32, device="cuda")
+        assert rt.mfq_rt_linear_forward(h, x.data_ptr(), 0, 88, M, y.data_ptr(), None) == 0
+        torch.cuda.synchronize()
+        check_close(y.cpu().numpy(), O.linear_forward_f64(deq, x.float().cpu().numpy()))
+    rt.mfq_rt_free_quant_linear(h)
+    with pytest.raises(RuntimeError, match="invalid NINT blob tail"):
+        _load(rt, "NINT3", O.pack_nint(t)[:-1])
+    with pytest.raises(RuntimeError, match="dtype/blob mismatch"):
+        _load(rt, "NINT4", O.pack_nint(t))
+    with pytest.raises(RuntimeError, match="unsupported quantized linear dtype"):
+        _load(rt, "MXFP4", b"\0" * 64)
+
+
+@pytest.mark.parametrize("T", [1, 20])
+def test_cpp_moe_ffn_forward(rt, T):
+    rng = np.random.default_rng(40 + T)
+    E, H, W, k = 16, 128, 64, 4
+    bits = rng.choice([2, 3, 4, 5], size=E, p=[0.1, 0.4, 0.4, 0.1])
+    tg, td = synth.moe_random(rng, E, 2 * W, H, bits, True), synth.moe_random(rng, E, H, W, bits, True)
+    bg, bd = O.pack_nint_moe(tg), O.pack_nint_moe(td)
+    hg, hd = C.c_void_p(), C.c_void_p()
+    assert rt.mfq_rt_load_nint_moe(bg, len(bg), C.byref(hg)) == 0, rt.mfq_rt_last_error()
+    assert rt.mfq_rt_load_nint_moe(bd, len(bd), C.byref(hd)) == 0, rt.mfq_rt_last_error()
+    x = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).to(torch.bfloat16).cuda()
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    lg = torch.from_numpy(logits).cuda()
+    out = torch.empty((T, H), dtype=torch.float32, device="cuda")
+    ids = torch.empty((T, k), dtype=torch.int32, device="cuda")
+    wts = torch.empty((T, k), dtype=torch.float32, device="cuda")
+    rc = rt.mfq_rt_moe_ffn_forward(hg, hd, x.data_ptr(), 0, H, T, lg.data_ptr(), k, 3, 0, None, None, out.data_ptr(),
+                                   ids.data_ptr(), wts.data_ptr(), None)
+    assert rc == 0, rt.mfq_rt_last_error()
+    torch.cuda.synchronize()
+    ref, rids, rw = O.moe_ffn(O.dequantize_expertwise(tg), O.dequantize_expertwise(td), x.float().cpu().numpy(), logits, k,
+                              delayed_softmax=True)
+    assert np.array_equal(ids.cpu().numpy(), rids)
+    check_close(out.cpu().numpy(), ref)
+    rt.mfq_rt_free_nint_moe(hg)
+    rt.mfq_rt_free_nint_moe(hd)

@@ -149,3 +149,15 @@ def test_grouped_projection_blob_is_the_row_concatenation():
         assert np.array_equal(F.unpack_bitstream(O.pack_bits(v, bits), 0, 77, bits), v)
     with pytest.raises(ValueError, match="must share"):
         F.nint_concat_rows([O.pack_nint(a), O.pack_nint(synth.nint_random(rng, 4, 100, 4, 24, 6))])
+
+
+def test_runtime_library_exports_its_c_view():
+    header = (ROOT / "include" / "mfq_runtime_c.h").read_text()
+    declared = sorted(set(re.findall(r"\b(mfq_rt_\w+)\s*\(", header)))
+    path = ROOT / "tyloquant_amd" / "lib" / "libmfq_runtime.so"
+    if not path.exists():
+        pytest.skip("libmfq_runtime.so is not built")
+    lib = ctypes.CDLL(str(path))
+    assert len(declared) >= 10
+    for name in declared:
+        assert hasattr(lib, name), name

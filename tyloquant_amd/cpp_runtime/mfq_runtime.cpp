@@ -1,0 +1,617 @@
+// C++ host runtime over the C ABI of libmfq_hip.so (see mfq_runtime.h for the map to the reference).
+#include "mfq_runtime.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <stdexcept>
+
+namespace mfq_rt {
+
+namespace {
+
+[[noreturn]] void fail(const std::string &msg) { throw std::runtime_error(msg); }
+
+void hip_check(hipError_t e, const char *what) {
+    if (e != hipSuccess) fail(std::string(what) + ": " + hipGetErrorString(e));
+}
+void abi_check(int rc) {
+    if (rc != MFQ_OK) fail(std::string("mfq_hip: ") + mfq_hip_last_error());
+}
+hipStream_t hs(mfq_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+template <typename T>
+T rd(const uint8_t *p, size_t off) {
+    T v;
+    std::memcpy(&v, p + off, sizeof(T));
+    return v;
+}
+int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace
+
+// ---- DeviceBuffer ---------------------------------------------------------------------------------
+DeviceBuffer::DeviceBuffer(size_t bytes) : bytes_(bytes) {
+    if (bytes) hip_check(hipMalloc(&ptr_, bytes), "hipMalloc");
+}
+DeviceBuffer::~DeviceBuffer() {
+    if (ptr_) (void)hipFree(ptr_);
+}
+DeviceBuffer::DeviceBuffer(DeviceBuffer &&o) noexcept : ptr_(o.ptr_), bytes_(o.bytes_) { o.ptr_ = nullptr; o.bytes_ = 0; }
+DeviceBuffer &DeviceBuffer::operator=(DeviceBuffer &&o) noexcept {
+    if (this != &o) {
+        if (ptr_) (void)hipFree(ptr_);
+        ptr_ = o.ptr_; bytes_ = o.bytes_;
+        o.ptr_ = nullptr; o.bytes_ = 0;
+    }
+    return *this;
+}
+void DeviceBuffer::ensure(size_t bytes) {
+    if (bytes <= bytes_) return;
+    if (ptr_) hip_check(hipFree(ptr_), "hipFree");
+    ptr_ = nullptr; bytes_ = 0;
+    hip_check(hipMalloc(&ptr_, bytes), "hipMalloc");
+    bytes_ = bytes;
+}
+DeviceBuffer DeviceBuffer::from_host(const void *src, size_t bytes) {
+    DeviceBuffer b(bytes);
+    if (bytes) hip_check(hipMemcpy(b.get(), src, bytes, hipMemcpyHostToDevice), "hipMemcpy");
+    return b;
+}
+
+// ---- header parsers ---------------------------------------------------------------------------------
+NintHeader parse_nint(const uint8_t *b, size_t n) {
+    if (n < 18) fail("truncated NINT header");
+    NintHeader h;
+    h.bits = b[0]; h.sub_bits = b[1];
+    h.gs = rd<int32_t>(b, 2); h.axis = rd<int32_t>(b, 6); h.neuron_len = rd<int32_t>(b, 10);
+    const uint32_t ndim = rd<uint32_t>(b, 14);
+    size_t off = 18;
+    if (ndim > 8 || n < off + 8 * ndim + 8) fail("truncated NINT header");
+    for (uint32_t i = 0; i < ndim; ++i) h.shape.push_back(rd<int64_t>(b, off + 8 * i));
+    off += 8 * ndim;
+    h.out = static_cast<int>(rd<uint32_t>(b, off)); h.ng = static_cast<int>(rd<uint32_t>(b, off + 4));
+    off += 8;
+    if (h.bits < 1 || h.bits > 8 || h.sub_bits < 1 || h.sub_bits > 8 || h.gs <= 0 || h.neuron_len <= 0 || h.out <= 0)
+        fail("unsupported NINT spec");
+    if (h.ng != cdiv(h.neuron_len, h.gs)) fail("NINT header group count does not match neuron_len");
+    const int64_t subs = static_cast<int64_t>(h.out) * h.ng, qn = subs * h.gs;
+    const int64_t packed = 4ll * h.out + 2 * ((subs * h.sub_bits + 7) / 8) + (qn * h.bits + 7) / 8;
+    const int64_t old = 4ll * h.out + 2 * subs + qn;
+    const int64_t remaining = static_cast<int64_t>(n) - static_cast<int64_t>(off);
+    if (remaining == packed) h.legacy = false;
+    else if (remaining == old) h.legacy = true;
+    else fail("invalid NINT blob tail: remaining=" + std::to_string(remaining - 4ll * h.out) + ", packed=" +
+              std::to_string(packed - 4ll * h.out) + ", old=" + std::to_string(old - 4ll * h.out));
+    h.body_off = off; h.body_bytes = static_cast<size_t>(remaining);
+    return h;
+}
+
+NvqHeader parse_nvq(const uint8_t *b, size_t n) {
+    if (n < 20) fail("truncated NVQ header");
+    if (std::memcmp(b, "NVQ1", 4) != 0 && std::memcmp(b, "NIQ1", 4) != 0) fail("invalid NVQ magic");
+    NvqHeader h;
+    const uint8_t enc = b[4];
+    h.sub_bits = b[5]; h.gs = rd<uint16_t>(b, 6);
+    h.neuron_len = rd<int32_t>(b, 12);
+    const uint32_t ndim = rd<uint32_t>(b, 16);
+    static const char *names[] = {"", "e8_256", "d4_256", "d4_512", "e8_1024", "e8_4096", "d4_1024"};
+    static const int ibits[] = {0, 8, 8, 9, 10, 12, 10};
+    const int cid = enc & 0x1f;
+    if (cid < 1 || cid > 6) fail("unknown NVQ codebook id: " + std::to_string(cid));
+    h.codebook = names[cid]; h.index_bits = ibits[cid];
+    h.vector_size = h.codebook[0] == 'e' ? 8 : 4;
+    h.jsc = enc & 0x20; h.index_parity = enc & 0x80;
+    const bool custom = enc & 0x40;
+    size_t off = 20 + 8 * static_cast<size_t>(ndim);
+    if (n < off + 4) fail("truncated NVQ header");
+    h.out = static_cast<int>(rd<uint32_t>(b, off));
+    off += 4;
+    const int64_t o = h.out, ng = cdiv(h.neuron_len, h.gs), nvec = cdiv(h.neuron_len, h.vector_size),
+                  nsign = cdiv(h.neuron_len, 8);
+    const int64_t streams = 2 * o + (o * ng * h.sub_bits + 7) / 8 + (o * nvec * h.index_bits + 7) / 8 + (o * nsign * 7 + 7) / 8;
+    int64_t expect = streams;
+    h.banks = 0;
+    if (h.jsc) {
+        if (custom || h.index_parity || h.gs != 24 || h.sub_bits != 4) fail("invalid NVQ-JSC profile flags");
+        if (n < off + 64) fail("truncated NVQ-JSC metadata header");
+        const uint8_t *m = b + off;
+        h.banks = m[1];
+        bool reserved = false;
+        for (int i = 52; i < 64; ++i) reserved |= m[i] != 0;
+        if (m[0] != 1 || (h.banks != 1 && h.banks != 2 && h.banks != 4) || m[2] != 16 || m[3] > 1 || reserved)
+            fail("invalid NVQ-JSC metadata");
+        for (int i = 36; i < 52; ++i)
+            if (m[i] >= h.banks) fail("invalid NVQ-JSC state-to-bank map");
+        expect += 64 + static_cast<int64_t>(h.banks) * (1ll << h.index_bits) * h.vector_size;
+        static const std::unordered_map<std::string, std::string> dt = {
+            {"e8_256", "NVQ2J"}, {"e8_1024", "NVQ2J-L"}, {"e8_4096", "NVQ2J-XL"},
+            {"d4_256", "NVQ3J"}, {"d4_512", "NVQ3J-512"}, {"d4_1024", "NVQ3J-L"}};
+        h.dtype = dt.at(h.codebook);
+    } else {
+        if (custom) fail("custom-codebook NVQ blobs are outside this runtime's scope");
+        h.dtype = h.codebook == "e8_256" ? "NVQ2" : h.codebook == "d4_256" ? "NVQ3" : "";
+        if (h.dtype.empty()) fail(h.codebook + " requires an NVQ-JSC file profile");
+    }
+    if (static_cast<int64_t>(n) - static_cast<int64_t>(off) != expect)
+        fail("invalid NVQ blob tail: consumed=" + std::to_string(off + expect) + ", size=" + std::to_string(n));
+    h.body_off = off; h.body_bytes = static_cast<size_t>(expect);
+    return h;
+}
+
+NepqHeader parse_nepq(const uint8_t *b, size_t n) {
+    if (n < 36) fail("truncated NEPQ header");
+    if (std::memcmp(b, "NEP1", 4) != 0 || b[4] != 1) fail("invalid or unsupported NEPQ header");
+    NepqHeader h;
+    h.profile = b[5];
+    const int gps = b[6], flags = b[7];
+    h.n_experts = static_cast<int>(rd<uint32_t>(b, 8)); h.out_per_expert = static_cast<int>(rd<uint32_t>(b, 12));
+    h.neuron_len = static_cast<int>(rd<uint32_t>(b, 16)); h.banks = static_cast<int>(rd<uint32_t>(b, 20));
+    h.rotation_block = static_cast<int>(rd<uint32_t>(b, 24)); h.rotation_seed = rd<uint64_t>(b, 28);
+    static const char *labels[] = {"NEPQ0-S", "NEPQ0-L", "NEPQ1-S", "NEPQ1-L"};
+    if (h.profile > 3 || gps != 4) fail("unsupported NEPQ super-group profile");
+    h.label = labels[h.profile];
+    if ((flags & ~1) || ((flags & 1) != 0) != (h.rotation_block != 0)) fail("inconsistent NEPQ rotation flag");
+    if (h.n_experts <= 0 || h.out_per_expert <= 0 || h.neuron_len <= 0 || h.neuron_len % 8 || h.banks < 1 || h.banks > 256)
+        fail("NEPQ shape dimensions must be positive, K divisible by 8, banks in [1,256]");
+    if (h.profile < 2) fail(h.label + " is not on the accelerated path");
+    const int sb = h.profile == 2 ? 4 : 3, ib = h.profile == 2 ? 9 : 11, tb = h.profile == 2 ? 2048 : 4096;
+    const int64_t rows = static_cast<int64_t>(h.n_experts) * h.out_per_expert, ng = cdiv(h.neuron_len, 24),
+                  nvec = h.neuron_len / 8, nsuper = cdiv(ng, 4);
+    const int64_t expect = static_cast<int64_t>(h.banks) * tb + 2 * rows + (rows * ng * sb + 7) / 8 +
+                           (rows * nvec * ib + 7) / 8 + (rows * ng + 7) / 8 + rows * nsuper;
+    if (static_cast<int64_t>(n) - 36 != expect)
+        fail("invalid NEPQ tail: consumed=" + std::to_string(36 + expect) + ", size=" + std::to_string(n));
+    h.body_off = 36; h.body_bytes = static_cast<size_t>(expect);
+    return h;
+}
+
+NintmHeader parse_nintm(const uint8_t *b, size_t n) {
+    if (n < 20) fail("truncated NINTM header");
+    if (std::memcmp(b, "NIM2", 4) != 0) fail("invalid NINTM magic");
+    NintmHeader h;
+    h.n_experts = static_cast<int>(rd<uint32_t>(b, 4)); h.out_per_expert = static_cast<int>(rd<uint32_t>(b, 8));
+    h.neuron_len = static_cast<int>(rd<uint32_t>(b, 12));
+    const uint32_t npools = rd<uint32_t>(b, 16);
+    if (npools == 0 || static_cast<int>(npools) > h.n_experts) fail("invalid NINTM pool count");
+    std::vector<int> owner(h.n_experts, -1);
+    size_t off = 20;
+    for (uint32_t pi = 0; pi < npools; ++pi) {
+        if (off + 24 > n) fail("truncated NINTM v2 pool header");
+        const uint32_t n_ids = rd<uint32_t>(b, off), dlen = rd<uint32_t>(b, off + 4);
+        const uint64_t plen = rd<uint64_t>(b, off + 8), rlen = rd<uint64_t>(b, off + 16);
+        off += 24;
+        if (n_ids == 0 || dlen == 0 || dlen > 32) fail("invalid NINTM v2 pool metadata");
+        const size_t end = off + 4ull * n_ids + dlen + rlen + plen;
+        if (end > n) fail("truncated NINTM v2 pool payload");
+        NintmPool p;
+        for (uint32_t i = 0; i < n_ids; ++i) {
+            const int32_t e = rd<int32_t>(b, off + 4ull * i);
+            if (e < 0 || e >= h.n_experts) fail("NINTM pool " + std::to_string(pi) + " contains an invalid expert id");
+            if (owner[e] == static_cast<int>(pi)) fail("NINTM pool " + std::to_string(pi) + " repeats an expert id");
+            if (owner[e] >= 0) fail("an expert belongs to multiple NINTM pools");
+            owner[e] = static_cast<int>(pi);
+            p.expert_ids.push_back(e);
+        }
+        off += 4ull * n_ids;
+        p.dtype.assign(reinterpret_cast<const char *>(b + off), dlen);
+        off += dlen;
+        p.runtime_off = off; p.runtime_bytes = rlen;
+        p.payload_off = off + rlen; p.payload_bytes = plen;
+        off = end;
+        h.pools.push_back(std::move(p));
+    }
+    if (off != n) fail("invalid NINTM tail: " + std::to_string(n - off) + " extra bytes");
+    for (int e = 0; e < h.n_experts; ++e)
+        if (owner[e] < 0) fail("NINTM pools do not cover expert " + std::to_string(e));
+    return h;
+}
+
+// ---- weights -------------------------------------------------------------------------------------------
+NintWeight NintWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream) {
+    const NintHeader h = parse_nint(blob, n);
+    if (h.axis != 0) fail("NINT linear weights must be quantized along axis 0");
+    NintWeight w;
+    abi_check(mfq_hip_nint_plan(h.bits, h.sub_bits, h.gs, h.out, h.neuron_len, &w.desc));
+    w.shape = h.shape;
+    DeviceBuffer payload = DeviceBuffer::from_host(blob + h.body_off, h.body_bytes);
+    w.data = DeviceBuffer(static_cast<size_t>(w.desc.total_bytes));
+    abi_check(mfq_hip_nint_repack(&w.desc, payload.get(), static_cast<int64_t>(h.body_bytes), h.legacy ? 1 : 0,
+                                  w.data.get(), stream));
+    hip_check(hipStreamSynchronize(hs(stream)), "nint repack");  // the staged payload is freed on return
+    return w;
+}
+
+NvqWeight NvqWeight::from_blob(const uint8_t *blob, size_t n, const int8_t *grid256, mfq_stream_t stream) {
+    const NvqHeader h = parse_nvq(blob, n);
+    if (h.vector_size != 4 || h.index_bits > 9)
+        fail(h.dtype + ": only the D4 256/512-entry NVQ formats are on the accelerated path");
+    NvqWeight w;
+    w.dtype = h.dtype;
+    abi_check(mfq_hip_nvq_plan(h.index_bits, h.jsc ? h.banks : 1, h.out, h.neuron_len, &w.desc));
+    DeviceBuffer payload = DeviceBuffer::from_host(blob + h.body_off, h.body_bytes);
+    w.data = DeviceBuffer(static_cast<size_t>(w.desc.total_bytes));
+    if (h.jsc) {
+        abi_check(mfq_hip_nvq_repack(&w.desc, payload.get(), static_cast<int64_t>(h.body_bytes), w.data.get(), stream));
+    } else {
+        if (h.gs != 24 || h.sub_bits != 4 || h.index_parity)
+            fail("plain NVQ3 runs only with gs24, 4-bit sub-scales and parity signs");
+        if (!grid256) fail("plain NVQ3 needs the 256-entry D4 magnitude grid");
+        DeviceBuffer grid = DeviceBuffer::from_host(grid256, 1024);
+        abi_check(mfq_hip_nvq_repack_plain(&w.desc, payload.get(), static_cast<int64_t>(h.body_bytes), grid.get(),
+                                           w.data.get(), stream));
+        hip_check(hipStreamSynchronize(hs(stream)), "nvq repack");
+    }
+    hip_check(hipStreamSynchronize(hs(stream)), "nvq repack");
+    return w;
+}
+
+NepqWeight NepqWeight::from_blob(const uint8_t *blob, size_t n, const int8_t *rotation_signs, mfq_stream_t stream) {
+    const NepqHeader h = parse_nepq(blob, n);
+    NepqWeight w;
+    w.label = h.label; w.n_experts = h.n_experts; w.out_per_expert = h.out_per_expert; w.rotation_block = h.rotation_block;
+    abi_check(mfq_hip_nepq_plan(h.profile, h.banks, h.n_experts * h.out_per_expert, h.neuron_len, &w.desc));
+    DeviceBuffer payload = DeviceBuffer::from_host(blob + h.body_off, h.body_bytes);
+    w.data = DeviceBuffer(static_cast<size_t>(w.desc.total_bytes));
+    abi_check(mfq_hip_nepq_repack(&w.desc, payload.get(), static_cast<int64_t>(h.body_bytes), w.data.get(), stream));
+    hip_check(hipStreamSynchronize(hs(stream)), "nepq repack");
+    if (h.rotation_block) {
+        if (!rotation_signs) fail("rotated NEPQ cohort lacks its runtime sign vector");
+        for (int i = 0; i < h.neuron_len; ++i)
+            if (rotation_signs[i] != 1 && rotation_signs[i] != -1) fail("NEPQ rotation sign vector is corrupt");
+        w.signs = DeviceBuffer::from_host(rotation_signs, static_cast<size_t>(h.neuron_len));
+    }
+    return w;
+}
+
+void nint_matmul(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) {
+    const size_t need = mfq_hip_nint_gemm_workspace_bytes(&w.desc, M);
+    w.workspace.ensure(need);
+    abi_check(mfq_hip_nint_gemm(&w.desc, w.data.get(), x, x_dtype, ldx, M, y, w.desc.out, w.workspace.get(), need, stream));
+}
+void nvq_matmul(const NvqWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) {
+    const size_t need = mfq_hip_nvq_gemm_workspace_bytes(&w.desc, M);
+    w.workspace.ensure(need);
+    abi_check(mfq_hip_nvq_gemm(&w.desc, w.data.get(), x, x_dtype, ldx, M, y, w.desc.out, w.workspace.get(), need, stream));
+}
+void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y,
+                 mfq_stream_t stream) {
+    if (expert < 0 || expert >= w.n_experts) fail("expert outside the NEPQ tensor");
+    const int K = w.desc.neuron_len;
+    if (w.rotation_block) {
+        w.rotated.ensure(static_cast<size_t>(M) * K * 2);
+        abi_check(mfq_hip_nepq_hadamard(x, x_dtype, ldx, M, K, w.rotation_block, static_cast<const int8_t *>(w.signs.get()),
+                                        w.rotated.get(), K, stream));
+        x = w.rotated.get();
+        ldx = K;
+    }
+    const size_t need = mfq_hip_nepq_gemm_workspace_bytes(&w.desc, w.out_per_expert, M);
+    w.workspace.ensure(need);
+    abi_check(mfq_hip_nepq_gemm(&w.desc, w.data.get(), expert * w.out_per_expert, w.out_per_expert, x, x_dtype, ldx, M, y,
+                                w.out_per_expert, w.workspace.get(), need, stream));
+}
+void nint_dequantize(const NintWeight &w, float *out, mfq_stream_t stream) {
+    abi_check(mfq_hip_nint_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
+}
+void nvq_dequantize(const NvqWeight &w, float *out, mfq_stream_t stream) {
+    abi_check(mfq_hip_nvq_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
+}
+void nepq_dequantize(const NepqWeight &w, float *out, mfq_stream_t stream) {
+    abi_check(mfq_hip_nepq_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
+}
+
+// ---- registry -------------------------------------------------------------------------------------------
+bool is_nint_linear_dtype(const std::string &d) {
+    if (d.size() <= 4 || d.compare(0, 4, "NINT") != 0) return false;
+    return std::all_of(d.begin() + 4, d.end(), [](char c) { return c >= '0' && c <= '9'; });
+}
+bool is_nvq_linear_dtype(const std::string &d) { return d == "NVQ3" || d == "NVQ3J" || d == "NVQ3J-512" || d == "NIQ3"; }
+bool is_nepq_linear_dtype(const std::string &d) { return d == "NEPQ1-S" || d == "NEPQ1-L"; }
+
+int64_t QuantLinear::out() const { return kind == QuantLinearKind::Nint ? nint->out() : kind == QuantLinearKind::Nvq ? nvq->out() : nepq->out(); }
+int64_t QuantLinear::neuron_len() const {
+    return kind == QuantLinearKind::Nint ? nint->neuron_len() : kind == QuantLinearKind::Nvq ? nvq->neuron_len() : nepq->neuron_len();
+}
+int64_t QuantLinear::payload_bytes() const {
+    return kind == QuantLinearKind::Nint ? nint->desc.payload_bytes : kind == QuantLinearKind::Nvq ? nvq->desc.payload_bytes
+                                                                                                   : nepq->desc.payload_bytes;
+}
+void QuantLinear::forward(const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const {
+    if (kind == QuantLinearKind::Nint) nint_matmul(*nint, x, x_dtype, ldx, M, y, stream);
+    else if (kind == QuantLinearKind::Nvq) nvq_matmul(*nvq, x, x_dtype, ldx, M, y, stream);
+    else nepq_matmul(*nepq, 0, x, x_dtype, ldx, M, y, stream);
+}
+void QuantLinear::dequantize(float *out, mfq_stream_t stream) const {
+    if (kind == QuantLinearKind::Nint) nint_dequantize(*nint, out, stream);
+    else if (kind == QuantLinearKind::Nvq) nvq_dequantize(*nvq, out, stream);
+    else nepq_dequantize(*nepq, out, stream);
+}
+
+QuantLinear load_quant_linear(const std::string &dtype_in, const uint8_t *blob, size_t n, mfq_stream_t stream) {
+    const std::string dtype = dtype_in == "NIQ3" ? "NVQ3" : dtype_in;
+    QuantLinear q;
+    if (is_nint_linear_dtype(dtype)) {
+        q.kind = QuantLinearKind::Nint;
+        q.nint = std::make_shared<NintWeight>(NintWeight::from_blob(blob, n, stream));
+        if ("NINT" + std::to_string(q.nint->desc.bits) != dtype)
+            fail("MFQ dtype/blob mismatch: " + dtype + " contains NINT" + std::to_string(q.nint->desc.bits));
+        return q;
+    }
+    if (is_nvq_linear_dtype(dtype)) {
+        q.kind = QuantLinearKind::Nvq;
+        q.nvq = std::make_shared<NvqWeight>(NvqWeight::from_blob(blob, n, nullptr, stream));
+        if (q.nvq->dtype != dtype) fail("MFQ dtype/blob mismatch: " + dtype + " contains " + q.nvq->dtype);
+        return q;
+    }
+    if (is_nepq_linear_dtype(dtype)) {
+        q.kind = QuantLinearKind::Nepq;
+        q.nepq = std::make_shared<NepqWeight>(NepqWeight::from_blob(blob, n, nullptr, stream));
+        if (q.nepq->label != dtype) fail("MFQ dtype/blob mismatch: " + dtype + " contains " + q.nepq->label);
+        return q;
+    }
+    fail("unsupported quantized linear dtype: " + dtype);
+}
+
+// ---- MoE ---------------------------------------------------------------------------------------------------
+MoeRoutePlan build_moe_route_plan(const int32_t *ids, int tokens, int routes, int n_experts, mfq_stream_t stream) {
+    if (!ids || tokens <= 0 || routes <= 0) fail("MoE ids must be device int32 [tokens, routes]");
+    MoeRoutePlan p;
+    p.ids = ids; p.tokens = tokens; p.routes = routes; p.n_experts = n_experts;
+    if (tokens > 8) {
+        const int n_pairs = tokens * routes, tile_m = mfq_hip_moe_tile_m();
+        const int max_tiles = static_cast<int>(cdiv(n_pairs, tile_m)) + n_experts;
+        p.counts = DeviceBuffer(4ull * n_experts);
+        p.expert_bounds = DeviceBuffer(4ull * (n_experts + 1));
+        p.tile_bounds = DeviceBuffer(4ull * (n_experts + 1));
+        p.tile_experts = DeviceBuffer(4ull * max_tiles);
+        p.ids_dst = DeviceBuffer(4ull * n_pairs);
+        abi_check(mfq_hip_moe_route_map(ids, n_pairs, n_experts, tile_m, static_cast<int32_t *>(p.counts.get()),
+                                        static_cast<int32_t *>(p.expert_bounds.get()),
+                                        static_cast<int32_t *>(p.tile_bounds.get()),
+                                        static_cast<int32_t *>(p.tile_experts.get()), max_tiles,
+                                        static_cast<int32_t *>(p.ids_dst.get()), stream));
+    }
+    p.map_ready = true;
+    return p;
+}
+
+NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream) {
+    const NintmHeader h = parse_nintm(blob, n);
+    NintMoeWeight w;
+    w.n_experts = h.n_experts; w.out_per_expert = h.out_per_expert; w.neuron_len = h.neuron_len;
+    std::vector<int32_t> ep(h.n_experts, -1), el(h.n_experts, -1);
+    for (size_t pi = 0; pi < h.pools.size(); ++pi) {
+        const NintmPool &p = h.pools[pi];
+        if (!is_nint_linear_dtype(p.dtype)) fail("NINTM cohort family " + p.dtype + " is not on the accelerated path");
+        if (p.runtime_bytes) fail("unexpected NINTM cohort runtime metadata");
+        auto pw = std::make_shared<NintWeight>(NintWeight::from_blob(blob + p.payload_off, p.payload_bytes, stream));
+        if (pw->out() != static_cast<int64_t>(p.expert_ids.size()) * h.out_per_expert || pw->neuron_len() != h.neuron_len)
+            fail("NINTM pool " + std::to_string(pi) + " tensor shape does not match its expert count");
+        for (size_t i = 0; i < p.expert_ids.size(); ++i) {
+            ep[p.expert_ids[i]] = static_cast<int32_t>(pi);
+            el[p.expert_ids[i]] = static_cast<int32_t>(i);
+        }
+        w.pool_table.push_back(mfq_moe_pool{pw->desc, pw->data.get()});
+        w.pools.push_back(std::move(pw));
+        w.pool_expert_ids.push_back(p.expert_ids);
+    }
+    w.expert_pool = DeviceBuffer::from_host(ep.data(), 4ull * ep.size());
+    w.expert_local = DeviceBuffer::from_host(el.data(), 4ull * el.size());
+    return w;
+}
+
+void NintMoeWeight::forward(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &r, float *out,
+                            mfq_stream_t stream) const {
+    const bool mapped = r.mapped();
+    abi_check(mfq_hip_moe_grouped_matmul(
+        pool_table.data(), static_cast<int>(pool_table.size()), static_cast<const int32_t *>(expert_pool.get()),
+        static_cast<const int32_t *>(expert_local.get()), n_experts, out_per_expert, neuron_len, x, x_dtype, ldx,
+        routed_input ? 1 : 0, r.ids, r.tokens, r.routes, mapped ? static_cast<const int32_t *>(r.ids_dst.get()) : nullptr,
+        mapped ? static_cast<const int32_t *>(r.expert_bounds.get()) : nullptr,
+        mapped ? static_cast<const int32_t *>(r.tile_bounds.get()) : nullptr,
+        mapped ? static_cast<const int32_t *>(r.tile_experts.get()) : nullptr, out, out_per_expert, stream));
+}
+
+void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &down, const void *x, int x_dtype, int64_t ldx,
+                          int T, const float *router_logits, int top_k, int topk_mode, bool normalize,
+                          const float *router_bias, float router_scale, const NintWeight *shared_gate_up,
+                          const NintWeight *shared_down, MoeFfnScratch &s, float *out, mfq_stream_t stream) {
+    if (gate_up.n_experts != down.n_experts || gate_up.out_per_expert != 2 * down.neuron_len ||
+        down.out_per_expert != gate_up.neuron_len)
+        fail("incompatible fused gate_up/down NINTM tensors");
+    const int E = gate_up.n_experts, W = down.neuron_len, H = down.out_per_expert;
+    const size_t pairs = static_cast<size_t>(T) * top_k;
+    s.ids.ensure(4 * pairs); s.weights.ensure(4 * pairs);
+    s.gate_up.ensure(4 * pairs * 2 * W); s.hidden.ensure(2 * pairs * W); s.down.ensure(4 * pairs * H);
+    int32_t *ids = static_cast<int32_t *>(s.ids.get());
+    float *wts = static_cast<float *>(s.weights.get());
+    abi_check(mfq_hip_moe_topk(router_logits, router_bias, T, E, top_k, topk_mode, normalize ? 1 : 0, 1e-20f, router_scale, ids,
+                               wts, stream));
+    MoeRoutePlan route = build_moe_route_plan(ids, T, top_k, E, stream);
+    float *gu = static_cast<float *>(s.gate_up.get());
+    gate_up.forward(x, x_dtype, ldx, false, route, gu, stream);
+    abi_check(mfq_hip_moe_swiglu(gu, 2 * W, static_cast<int>(pairs), W, s.hidden.get(), MFQ_X_F16, W, stream));
+    float *dn = static_cast<float *>(s.down.get());
+    down.forward(s.hidden.get(), MFQ_X_F16, W, true, route, dn, stream);
+    const float *shared = nullptr;
+    if (shared_gate_up && shared_down) {
+        s.shared_gu.ensure(4ull * T * 2 * W); s.shared_h.ensure(2ull * T * W); s.shared_out.ensure(4ull * T * H);
+        nint_matmul(*shared_gate_up, x, x_dtype, ldx, T, static_cast<float *>(s.shared_gu.get()), stream);
+        abi_check(mfq_hip_moe_swiglu(static_cast<float *>(s.shared_gu.get()), 2 * W, T, W, s.shared_h.get(), MFQ_X_F16, W, stream));
+        nint_matmul(*shared_down, s.shared_h.get(), MFQ_X_F16, W, T, static_cast<float *>(s.shared_out.get()), stream);
+        shared = static_cast<const float *>(s.shared_out.get());
+    }
+    abi_check(mfq_hip_moe_weighted_reduce(dn, wts, T, top_k, H, shared, nullptr, out, stream));
+    // the route plan's device tables are freed on return: wait for the kernels that read them
+    hip_check(hipStreamSynchronize(hs(stream)), "nint_moe_ffn_forward");
+}
+
+// ---- MFQ1 container ---------------------------------------------------------------------------------------
+MfqFile::MfqFile(const std::string &path) {
+    std::ifstream f(path, std::ios::binary);
+    if (!f) fail("cannot open " + path);
+    bytes.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+    const uint8_t *b = bytes.data();
+    const size_t n = bytes.size();
+    if (n < 12 || std::memcmp(b, "MFQ1", 4) != 0) fail("invalid MFQ magic");
+    const uint32_t version = rd<uint32_t>(b, 4);
+    size_t off = 8;
+    auto str = [&](std::string &s) {
+        if (off + 4 > n) fail("truncated MFQ header");
+        const uint32_t len = rd<uint32_t>(b, off);
+        off += 4;
+        if (off + len > n) fail("truncated MFQ header");
+        s.assign(reinterpret_cast<const char *>(b + off), len);
+        off += len;
+    };
+    str(model_arch);
+    if (version >= 2) {
+        if (off + 4 > n) fail("truncated MFQ header");
+        const uint32_t extra = rd<uint32_t>(b, off);
+        off += 4;
+        std::string tmp;
+        for (uint32_t i = 0; i < 2 * extra; ++i) str(tmp);
+    }
+    if (off + 4 > n) fail("truncated MFQ header");
+    const uint32_t count = rd<uint32_t>(b, off);
+    off += 4;
+    for (uint32_t i = 0; i < count; ++i) {
+        MfqRecord r;
+        str(r.name);
+        str(r.dtype);
+        if (off + 8 > n) fail("truncated MFQ directory");
+        r.nbytes = rd<uint64_t>(b, off);
+        off += 8;
+        records.push_back(std::move(r));
+    }
+    for (auto &r : records) {
+        if (off + r.nbytes > n) fail("truncated MFQ blob for " + r.name);
+        r.offset = off;
+        off += r.nbytes;
+    }
+}
+const MfqRecord &MfqFile::find(const std::string &name) const {
+    for (const auto &r : records)
+        if (r.name == name) return r;
+    fail("tensor not found: " + name);
+}
+
+// ---- --check-linear -------------------------------------------------------------------------------------------
+LinearCheckResult run_linear_check(const QuantLinear &lin, int M, int reps) {
+    const int64_t N = lin.out(), K = lin.neuron_len();
+    std::vector<uint16_t> x(static_cast<size_t>(M) * K);
+    std::vector<float> xf(x.size());
+    for (size_t i = 0; i < x.size(); ++i) {
+        const float v = (static_cast<float>(static_cast<int>(i % 97) - 48)) / 512.f;  // exact in bf16
+        uint32_t u;
+        std::memcpy(&u, &v, 4);
+        x[i] = static_cast<uint16_t>(u >> 16);
+        xf[i] = v;
+    }
+    DeviceBuffer dx = DeviceBuffer::from_host(x.data(), x.size() * 2);
+    DeviceBuffer dy(static_cast<size_t>(M) * N * 4), dw(static_cast<size_t>(N) * K * 4);
+    hipStream_t st;
+    hip_check(hipStreamCreate(&st), "hipStreamCreate");
+    for (int i = 0; i < std::min(30, reps); ++i) lin.forward(dx.get(), MFQ_X_BF16, K, M, static_cast<float *>(dy.get()), st);
+    hipEvent_t e0, e1;
+    hip_check(hipEventCreate(&e0), "hipEventCreate");
+    hip_check(hipEventCreate(&e1), "hipEventCreate");
+    hip_check(hipEventRecord(e0, st), "hipEventRecord");
+    for (int i = 0; i < reps; ++i) lin.forward(dx.get(), MFQ_X_BF16, K, M, static_cast<float *>(dy.get()), st);
+    hip_check(hipEventRecord(e1, st), "hipEventRecord");
+    hip_check(hipEventSynchronize(e1), "hipEventSynchronize");
+    float ms = 0.f;
+    hip_check(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+    lin.dequantize(static_cast<float *>(dw.get()), st);
+    hip_check(hipStreamSynchronize(st), "sync");
+    std::vector<float> y(static_cast<size_t>(M) * N), W(static_cast<size_t>(N) * K);
+    hip_check(hipMemcpy(y.data(), dy.get(), y.size() * 4, hipMemcpyDeviceToHost), "copy y");
+    hip_check(hipMemcpy(W.data(), dw.get(), W.size() * 4, hipMemcpyDeviceToHost), "copy W");
+    double num = 0, den = 0, sum_abs = 0, max_abs = 0;
+    for (int m = 0; m < M; ++m)
+        for (int64_t r = 0; r < N; ++r) {
+            double acc = 0;
+            for (int64_t k = 0; k < K; ++k) acc += static_cast<double>(xf[m * K + k]) * W[r * K + k];
+            const double d = y[m * N + r] - acc;
+            num += d * d; den += acc * acc; sum_abs += std::fabs(d); max_abs = std::max(max_abs, std::fabs(d));
+        }
+    LinearCheckResult res;
+    res.production_ms = ms / reps;
+    res.payload_bytes = lin.payload_bytes();
+    res.weight_bytes = lin.kind == QuantLinearKind::Nint ? lin.nint->desc.total_bytes
+                     : lin.kind == QuantLinearKind::Nvq ? lin.nvq->desc.total_bytes : lin.nepq->desc.total_bytes;
+    res.production_weight_gbps = res.weight_bytes / (res.production_ms * 1e6);
+    res.payload_gbps = res.payload_bytes / (res.production_ms * 1e6);
+    res.production_rel = den > 0 ? std::sqrt(num / den) : std::sqrt(num);
+    res.production_mean_abs = sum_abs / (static_cast<double>(M) * N);
+    res.production_max_abs = max_abs;
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); (void)hipStreamDestroy(st);
+    return res;
+}
+
+}  // namespace mfq_rt
+
+// ---- flat C wrappers, for bindings and tests ----------------------------------------------------------------------
+using namespace mfq_rt;
+namespace {
+thread_local std::string g_err;
+template <typename F>
+int guard(F &&f) {
+    try {
+        f();
+        return 0;
+    } catch (const std::exception &e) {
+        g_err = e.what();
+        return 1;
+    }
+}
+}  // namespace
+
+extern "C" {
+const char *mfq_rt_last_error(void) { return g_err.c_str(); }
+
+int mfq_rt_load_quant_linear(const char *dtype, const void *blob, size_t n, void **handle) {
+    return guard([&] { *handle = new QuantLinear(load_quant_linear(dtype, static_cast<const uint8_t *>(blob), n)); });
+}
+void mfq_rt_free_quant_linear(void *handle) { delete static_cast<QuantLinear *>(handle); }
+int64_t mfq_rt_linear_out(void *h) { return static_cast<QuantLinear *>(h)->out(); }
+int64_t mfq_rt_linear_neuron_len(void *h) { return static_cast<QuantLinear *>(h)->neuron_len(); }
+int mfq_rt_linear_forward(void *h, const void *x, int x_dtype, int64_t ldx, int M, float *y, void *stream) {
+    return guard([&] { static_cast<QuantLinear *>(h)->forward(x, x_dtype, ldx, M, y, stream); });
+}
+int mfq_rt_linear_dequantize(void *h, float *out, void *stream) {
+    return guard([&] { static_cast<QuantLinear *>(h)->dequantize(out, stream); });
+}
+int mfq_rt_linear_check(void *h, int M, int reps, double *out6) {
+    return guard([&] {
+        const LinearCheckResult r = run_linear_check(*static_cast<QuantLinear *>(h), M, reps);
+        out6[0] = r.production_ms; out6[1] = r.production_weight_gbps; out6[2] = r.payload_gbps;
+        out6[3] = r.production_rel; out6[4] = r.production_mean_abs; out6[5] = r.production_max_abs;
+    });
+}
+
+int mfq_rt_load_nint_moe(const void *blob, size_t n, void **handle) {
+    return guard([&] { *handle = new NintMoeWeight(NintMoeWeight::from_blob(static_cast<const uint8_t *>(blob), n)); });
+}
+void mfq_rt_free_nint_moe(void *handle) { delete static_cast<NintMoeWeight *>(handle); }
+int mfq_rt_moe_ffn_forward(void *gate_up, void *down, const void *x, int x_dtype, int64_t ldx, int T,
+                           const float *router_logits, int top_k, int topk_mode, int normalize, void *shared_gate_up,
+                           void *shared_down, float *out, int32_t *ids_out, float *weights_out, void *stream) {
+    return guard([&] {
+        MoeFfnScratch s;
+        const NintWeight *sg = shared_gate_up ? static_cast<QuantLinear *>(shared_gate_up)->nint.get() : nullptr;
+        const NintWeight *sd = shared_down ? static_cast<QuantLinear *>(shared_down)->nint.get() : nullptr;
+        nint_moe_ffn_forward(*static_cast<NintMoeWeight *>(gate_up), *static_cast<NintMoeWeight *>(down), x, x_dtype, ldx, T,
+                             router_logits, top_k, topk_mode, normalize != 0, nullptr, 1.f, sg, sd, s, out, stream);
+        const size_t pairs = static_cast<size_t>(T) * top_k;
+        if (ids_out && hipMemcpy(ids_out, s.ids.get(), 4 * pairs, hipMemcpyDeviceToDevice) != hipSuccess)
+            throw std::runtime_error("copy ids");
+        if (weights_out && hipMemcpy(weights_out, s.weights.get(), 4 * pairs, hipMemcpyDeviceToDevice) != hipSuccess)
+            throw std::runtime_error("copy weights");
+    });
+}
+}

@@ -1,0 +1,205 @@
+// C++ host runtime of the MFQ packed-weight matmul path on MI355X.
+//
+// Keeps the operator surface of the reference's cpp_runtime for this path -- the dtype-string
+// registry and loaders, the weight structs, nint_matmul / nvq_matmul / nepq_matmul,
+// build_moe_route_plan, NintMoeWeight::forward and nint_moe_ffn_forward, and the --check-linear
+// harness -- over the C ABI of libmfq_hip.so (include/mfq_hip.h).  Activations and outputs are
+// plain device pointers (bf16 or fp16 in, fp32 out) instead of torch tensors; errors are
+// std::runtime_error, as in the reference's loaders.
+//
+//   reference (cpp_runtime/mfq_decode.cpp)            here
+//   NintCpu / unpack_nint            :1529-1589       parse_nint + NintWeight::from_blob (device repack)
+//   NintWeight / to_device_nint      :2101-2165,2268  NintWeight
+//   nint_matmul                      :8130-8315       nint_matmul
+//   NvqCpu / unpack_nvq / NvqWeight  :3418-4150       parse_nvq + NvqWeight
+//   nvq_matmul                       :7884-7931       nvq_matmul
+//   NepqCpu / unpack_nepq            :4166-4463       parse_nepq + NepqWeight, nepq_matmul
+//   unpack_nint_moe_impl / NintMoeWeight :2367-2478, 2908-3071   parse_nintm + NintMoeWeight
+//   MoeRoutePlan / build_moe_route_plan  :2579-2592, 2681-2708   MoeRoutePlan / build_moe_route_plan
+//   nint_moe_ffn_forward             :3394-3416       nint_moe_ffn_forward
+//   is_nint_linear_dtype / load_quant_linear :9409-9420, 9489-9771   same names
+//   MfqFile                          :1294-1527       MfqFile (directory + blobs, single file)
+//   run_linear_check                 :16510-16638     run_linear_check
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/mfq_hip.h"
+
+namespace mfq_rt {
+
+// ---- device memory ---------------------------------------------------------------------------
+class DeviceBuffer {
+public:
+    DeviceBuffer() = default;
+    explicit DeviceBuffer(size_t bytes);
+    ~DeviceBuffer();
+    DeviceBuffer(DeviceBuffer &&o) noexcept;
+    DeviceBuffer &operator=(DeviceBuffer &&o) noexcept;
+    DeviceBuffer(const DeviceBuffer &) = delete;
+    DeviceBuffer &operator=(const DeviceBuffer &) = delete;
+    void *get() const { return ptr_; }
+    size_t size() const { return bytes_; }
+    void ensure(size_t bytes);  // grow-only
+    static DeviceBuffer from_host(const void *src, size_t bytes);
+
+private:
+    void *ptr_ = nullptr;
+    size_t bytes_ = 0;
+};
+
+// ---- payload headers (host side; the bit streams themselves are read on the GPU) ----------------
+struct NintHeader {
+    int bits, sub_bits, gs, axis, neuron_len, out, ng;
+    std::vector<int64_t> shape;
+    size_t body_off, body_bytes;
+    bool legacy;
+};
+struct NvqHeader {
+    std::string codebook, dtype;
+    int index_bits, vector_size, banks, out, neuron_len, gs, sub_bits;
+    bool jsc, index_parity;
+    size_t body_off, body_bytes;
+};
+struct NepqHeader {
+    std::string label;
+    int profile, n_experts, out_per_expert, neuron_len, banks, rotation_block;
+    uint64_t rotation_seed;
+    size_t body_off, body_bytes;
+};
+struct NintmPool {
+    std::vector<int32_t> expert_ids;
+    std::string dtype;
+    size_t payload_off, payload_bytes, runtime_off, runtime_bytes;
+};
+struct NintmHeader {
+    int n_experts, out_per_expert, neuron_len;
+    std::vector<NintmPool> pools;
+};
+NintHeader parse_nint(const uint8_t *blob, size_t n);
+NvqHeader parse_nvq(const uint8_t *blob, size_t n);
+NepqHeader parse_nepq(const uint8_t *blob, size_t n);
+NintmHeader parse_nintm(const uint8_t *blob, size_t n);
+
+// ---- weights ------------------------------------------------------------------------------------
+struct NintWeight {
+    mfq_nint_desc desc{};
+    DeviceBuffer data;
+    std::vector<int64_t> shape;
+    mutable DeviceBuffer workspace;  // grows with M, like the reference's per-weight workspaces
+    int64_t out() const { return desc.out; }
+    int64_t neuron_len() const { return desc.neuron_len; }
+    static NintWeight from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream = nullptr);
+};
+struct NvqWeight {
+    mfq_nvq_desc desc{};
+    DeviceBuffer data;
+    std::string dtype;
+    mutable DeviceBuffer workspace;
+    int64_t out() const { return desc.out; }
+    int64_t neuron_len() const { return desc.neuron_len; }
+    // `grid256` = the 256-entry int8 D4 magnitude grid [256,4], needed only by plain (non-JSC) NVQ3
+    static NvqWeight from_blob(const uint8_t *blob, size_t n, const int8_t *grid256 = nullptr,
+                               mfq_stream_t stream = nullptr);
+};
+struct NepqWeight {
+    mfq_nepq_desc desc{};
+    DeviceBuffer data;
+    std::string label;
+    int n_experts = 0, out_per_expert = 0, rotation_block = 0;
+    DeviceBuffer signs;  // int8 [K] when rotated
+    mutable DeviceBuffer workspace, rotated;
+    int64_t out() const { return out_per_expert; }
+    int64_t neuron_len() const { return desc.neuron_len; }
+    static NepqWeight from_blob(const uint8_t *blob, size_t n, const int8_t *rotation_signs = nullptr,
+                                mfq_stream_t stream = nullptr);
+};
+
+// y[M, out] (fp32, row stride out) = x[M, K] (x_dtype MFQ_X_BF16 / MFQ_X_F16, row stride ldx) . W^T
+void nint_matmul(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y,
+                 mfq_stream_t stream = nullptr);
+void nvq_matmul(const NvqWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y,
+                mfq_stream_t stream = nullptr);
+void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y,
+                 mfq_stream_t stream = nullptr);
+void nint_dequantize(const NintWeight &w, float *out, mfq_stream_t stream = nullptr);
+void nvq_dequantize(const NvqWeight &w, float *out, mfq_stream_t stream = nullptr);
+void nepq_dequantize(const NepqWeight &w, float *out, mfq_stream_t stream = nullptr);
+
+// ---- dtype registry -------------------------------------------------------------------------------
+bool is_nint_linear_dtype(const std::string &dtype);
+bool is_nvq_linear_dtype(const std::string &dtype);
+bool is_nepq_linear_dtype(const std::string &dtype);
+enum class QuantLinearKind { Nint, Nvq, Nepq };
+struct QuantLinear {
+    QuantLinearKind kind;
+    std::shared_ptr<NintWeight> nint;
+    std::shared_ptr<NvqWeight> nvq;
+    std::shared_ptr<NepqWeight> nepq;
+    int64_t out() const;
+    int64_t neuron_len() const;
+    int64_t payload_bytes() const;
+    void forward(const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream = nullptr) const;
+    void dequantize(float *out, mfq_stream_t stream = nullptr) const;
+};
+QuantLinear load_quant_linear(const std::string &dtype, const uint8_t *blob, size_t n, mfq_stream_t stream = nullptr);
+
+// ---- MoE ----------------------------------------------------------------------------------------
+struct MoeRoutePlan {
+    const int32_t *ids = nullptr;  // device int32 [tokens, routes]
+    int tokens = 0, routes = 0, n_experts = 0;
+    DeviceBuffer ids_dst, expert_bounds, tile_bounds, tile_experts, counts;
+    bool map_ready = false;
+    bool mapped() const { return ids_dst.get() != nullptr; }
+};
+// Builds the expert map only above 8 tokens, like the reference.
+MoeRoutePlan build_moe_route_plan(const int32_t *ids, int tokens, int routes, int n_experts,
+                                  mfq_stream_t stream = nullptr);
+
+struct NintMoeWeight {
+    int n_experts = 0, out_per_expert = 0, neuron_len = 0;
+    std::vector<std::shared_ptr<NintWeight>> pools;
+    std::vector<std::vector<int32_t>> pool_expert_ids;
+    DeviceBuffer expert_pool, expert_local;  // int32 [E] dispatch tables
+    std::vector<mfq_moe_pool> pool_table;
+    static NintMoeWeight from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream = nullptr);
+    // x: [T, K] (routed_input = false) or [T*R, K]; out: fp32 [T*R, out_per_expert]
+    void forward(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &route, float *out,
+                 mfq_stream_t stream = nullptr) const;
+};
+
+struct MoeFfnScratch {  // caller-owned intermediates of nint_moe_ffn_forward, grown on demand
+    DeviceBuffer ids, weights, gate_up, hidden, down, shared_gu, shared_h, shared_out;
+};
+// out fp32 [T, hidden]; top-k ids / weights stay in `scratch`.  `shared_gate_up` / `shared_down` may be null.
+void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &down, const void *x, int x_dtype,
+                          int64_t ldx, int T, const float *router_logits, int top_k, int topk_mode, bool normalize,
+                          const float *router_bias, float router_scale, const NintWeight *shared_gate_up,
+                          const NintWeight *shared_down, MoeFfnScratch &scratch, float *out,
+                          mfq_stream_t stream = nullptr);
+
+// ---- MFQ1 container + the --check-linear harness ----------------------------------------------------
+struct MfqRecord {
+    std::string name, dtype;
+    size_t offset, nbytes;
+};
+struct MfqFile {
+    std::vector<uint8_t> bytes;
+    std::string model_arch;
+    std::vector<MfqRecord> records;
+    explicit MfqFile(const std::string &path);
+    const MfqRecord &find(const std::string &name) const;
+};
+struct LinearCheckResult {
+    double production_ms, production_weight_gbps, payload_gbps, production_rel, production_mean_abs, production_max_abs;
+    int64_t weight_bytes, payload_bytes;
+};
+// Deterministic input x[i] = ((i mod 97) - 48) / 512, warm-ups, `reps` timed launches between two HIP
+// events, reference = device full dequant (fp32) times x on the host in fp64.
+LinearCheckResult run_linear_check(const QuantLinear &lin, int M, int reps = 200);
+
+}  // namespace mfq_rt
