@@ -186,7 +186,7 @@ typedef struct mfq_moe_pool {
 /* out[pair, :] = x[src(pair), :] . W[ids[pair]]^T for every (token, route) pair; src = pair when
  * routed_input != 0 (x is [T*R, K]) else pair / R (x is [T, K]).  Invalid expert ids give zero rows.
  * Replaces nint_moe_grouped_matmul_hetero_qx_cuda / _hetero_f16_cuda / _pool_ws_cuda
- * (cpp_runtime/mfq_decode.cpp:248-290; mfq/kernels/cuda/moe.cu:3971-4345). */
+ * (cpp_runtime/mfq_decode.cpp:236-280; mfq/kernels/cuda/moe.cu:3971-4345). */
 /* Routes of one expert are batched mfq_hip_moe_tile_m() at a time by the mapped path: build the
  * route map with that tile_m.  Pass ids_dst == NULL (and NULL tables) to run every pair on its own
  * (decode, T*R small). */
