@@ -27,6 +27,39 @@ __device__ __forceinline__ void load_unit(const uint32_t *__restrict__ p, uint32
     }
 }
 
+// Range-checked window over the bytes one wave streams.  Loads through it are unconditional
+// instructions: an offset at or beyond `bytes` returns zeros and moves no data, so the prefetch of a
+// step that does not exist needs no branch and the compiler can count outstanding loads exactly.
+// `base` and `bytes` must be the same in every lane of the wave.
+constexpr uint32_t kNoStep = 0x80000000u;  // an offset outside every window
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_window(const uint8_t *base, uint32_t bytes) {
+    const uint64_t a = reinterpret_cast<uint64_t>(base);
+    const uint64_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(a)));
+    const uint64_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(a >> 32)));
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>((hi << 32) | lo), 0,
+                                             __builtin_amdgcn_readfirstlane(static_cast<int>(bytes)), 0x00020000);
+}
+
+template <int D>
+__device__ __forceinline__ void load_unit_win(__amdgpu_buffer_rsrc_t win, uint32_t off, uint32_t (&q)[D]) {
+    if constexpr (D % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < D / 4; ++i) {
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(win, off + 16 * i, 0, 2);
+            q[4 * i] = v.x; q[4 * i + 1] = v.y; q[4 * i + 2] = v.z; q[4 * i + 3] = v.w;
+        }
+    } else if constexpr (D % 2 == 0) {
+#pragma unroll
+        for (int i = 0; i < D / 2; ++i) {
+            const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(win, off + 8 * i, 0, 2);
+            q[2 * i] = v.x; q[2 * i + 1] = v.y;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < D; ++i) q[i] = __builtin_amdgcn_raw_buffer_load_b32(win, off + 4 * i, 0, 2);
+    }
+}
+
 // Order LDS traffic between the lanes of one wave (the staged activations are wave-private, so no
 // block barrier is needed).
 __device__ __forceinline__ void wave_sync() {
@@ -64,39 +97,110 @@ __device__ __forceinline__ float quad_sum(float v) {
     return v;
 }
 
-struct PlainBias {  // formats whose unpack needs no per-pair bias weights
+// Staging policy.  xscale(pos, t): power of two by which pair pos + t of a group is multiplied
+// while it is staged (pos = first pair of a 4-pair chunk); inv_xscale(i) its reciprocal for pair i;
+// bw(i): weight of the staged pair sum in T_g.
+struct PlainBias {  // formats whose unpack needs neither
+    static constexpr bool SCALED = false;
     __device__ static __forceinline__ float bw(int) { return 0.f; }
+    __device__ static __forceinline__ float xscale(int, int) { return 1.f; }
+    __device__ static __forceinline__ float inv_xscale(int) { return 1.f; }
 };
 
+// staged fp16 pair times a power of two
+__device__ __forceinline__ uint32_t scale_h2(uint32_t pair, float s) {
+    const _Float16 h = static_cast<_Float16>(s);
+    const half2_t v = __builtin_bit_cast(half2_t, pair) * half2_t{h, h};
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+// Activation chunks a lane may hold in registers while the first weight loads are in flight.
+constexpr int kXChunks = 4;
+template <int MB>
+struct XRegs {
+    u32x4_t v[MB][kXChunks];
+    bool on;
+};
+
+// First half of the staging: request the wave's K-slice of the activation rows into registers.  Issued
+// before the weight loads so that (loads retiring in order) the staging never waits for weights.  Only the
+// common case is prefetched -- aligned rows, slice wholly inside K, at most 256 * kXChunks pairs, MB <= 2;
+// anything else is fetched by stage_x itself.
+template <int MB>
+__device__ __forceinline__ void stage_x_issue(const uint16_t *const (&xr)[MB], int K, int k0, int npairs, int lane,
+                                              XRegs<MB> &xg) {
+    bool ok = MB <= 2 && npairs <= 256 * kXChunks && k0 + 2 * npairs <= K;
+#pragma unroll
+    for (int m = 0; m < MB; ++m) ok = ok && (reinterpret_cast<uintptr_t>(xr[m]) & 15) == 0;
+    xg.on = ok;
+    if (ok) {
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+#pragma unroll
+            for (int c = 0; c < kXChunks; ++c) {
+                const int i = lane * 4 + c * 256;
+                const int ii = i < npairs ? i : 0;
+                u32x4_t v = {0u, 0u, 0u, 0u};
+                if (xr[m]) v = *reinterpret_cast<const u32x4_t *>(xr[m] + k0 + 2 * ii);
+                xg.v[m][c] = v;
+            }
+        }
+    }
+}
+
 // Stage the wave's K-slice of the MB activation rows xr[m] (null = absent row) into its private
-// LDS region as fp16 (x[2i], x[2i+1]) pairs, zero beyond K.  Next to it, per group g, two floats:
-// X_g = sum of x over the group and T_g = sum over its pairs i of (x[2i] + x[2i+1]) * BW::bw(i)
-// (the bias the unpack trick adds to the dot product).  npairs is a multiple of 8; xs is 16-byte
-// aligned.
+// LDS region as fp16 (x[2i], x[2i+1]) pairs times BW::xscale, zero beyond K.  Next to it, per group
+// g, two floats: X_g = sum of x over the group and -T_g, T_g = sum over its pairs i of the staged
+// pair sum times BW::bw(i) (the bias the unpack trick adds to the dot product).  npairs is a multiple
+// of 8; xs is 16-byte aligned.  `xg` = what stage_x_issue requested.
 template <int XF16, int MB, class BW>
 __device__ __forceinline__ void stage_x(const uint16_t *const (&xr)[MB], int K, int k0, int npairs, int gs, int ngl,
-                                        uint32_t *xs, float *xsum, int lane) {
+                                        uint32_t *xs, float *xsum, int lane, const XRegs<MB> &xg) {
+    if (xg.on) {
 #pragma unroll
-    for (int m = 0; m < MB; ++m) {
-        const uint16_t *p = xr[m];
-        const bool vec = p && (reinterpret_cast<uintptr_t>(p) & 15) == 0;
-        for (int i = lane * 4; i < npairs; i += 256) {
-            const int kk = k0 + 2 * i;
-            u32x4_t v = {0u, 0u, 0u, 0u};
-            if (vec && kk + 8 <= K) {
-                v = *reinterpret_cast<const u32x4_t *>(p + kk);
-            } else if (p) {
+        for (int m = 0; m < MB; ++m) {
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    uint32_t lo = 0, hi = 0;
-                    if (kk + 2 * t < K) lo = p[kk + 2 * t];
-                    if (kk + 2 * t + 1 < K) hi = p[kk + 2 * t + 1];
-                    v[t] = lo | (hi << 16);
+            for (int c = 0; c < kXChunks; ++c) {
+                const int i = lane * 4 + c * 256;
+                u32x4_t v = xg.v[m][c];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) v[t] = to_h2<XF16>(v[t]);
+                if constexpr (BW::SCALED) {
+                    const int pos = i % (gs / 2);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) v[t] = scale_h2(v[t], BW::xscale(pos, t));
                 }
+                if (i < npairs) *reinterpret_cast<u32x4_t *>(xs + m * npairs + i) = v;
             }
+        }
+    } else {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) v[t] = to_h2<XF16>(v[t]);
-            *reinterpret_cast<u32x4_t *>(xs + m * npairs + i) = v;
+        for (int m = 0; m < MB; ++m) {
+            const uint16_t *p = xr[m];
+            const bool vec = p && (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+            for (int i = lane * 4; i < npairs; i += 256) {
+                const int kk = k0 + 2 * i;
+                u32x4_t v = {0u, 0u, 0u, 0u};
+                if (vec && kk + 8 <= K) {
+                    v = *reinterpret_cast<const u32x4_t *>(p + kk);
+                } else if (p) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        uint32_t lo = 0, hi = 0;
+                        if (kk + 2 * t < K) lo = p[kk + 2 * t];
+                        if (kk + 2 * t + 1 < K) hi = p[kk + 2 * t + 1];
+                        v[t] = lo | (hi << 16);
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) v[t] = to_h2<XF16>(v[t]);
+                if constexpr (BW::SCALED) {
+                    const int pos = i % (gs / 2);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) v[t] = scale_h2(v[t], BW::xscale(pos, t));
+                }
+                *reinterpret_cast<u32x4_t *>(xs + m * npairs + i) = v;
+            }
         }
     }
     wave_sync();
@@ -109,62 +213,74 @@ __device__ __forceinline__ void stage_x(const uint16_t *const (&xr)[MB], int K, 
             const int i1 = min(hp, (part + 1) * quarter);
             for (int i = part * quarter; i < i1; ++i) {
                 const float ps = dot2h(xs[m * npairs + g * hp + i], 0x3c003c00u, 0.f);
-                sx += ps;
+                sx = fmaf(ps, BW::inv_xscale(i), sx);
                 st = fmaf(ps, BW::bw(i), st);
             }
             sx = quad_sum(sx);
             st = quad_sum(st);
             if (part == 0) {
                 xsum[(m * ngl + g) * 2] = sx;
-                xsum[(m * ngl + g) * 2 + 1] = st;
+                xsum[(m * ngl + g) * 2 + 1] = -st;
             }
         }
     }
     wave_sync();
 }
 
-// Reduce the K-split (4 lanes inside the wave, then the waves of the block through `red`, a region
-// of nwaves * MB * 16 floats that nothing else uses, in a fixed order) and store neuron
-// `rb*16 + r - row_base` of each output row yr[m] (null = absent row).
+// Output reduction.  park_rows: reduce the K-split of the 4 lanes of a neuron and leave the wave's
+// partial sums of one 16-neuron row-block in `red` slot (rbi * nwaves + wave).  flush_rows: after a
+// block barrier, add the waves' partials in a fixed order and store neuron (rb0 + rbi) * 16 + r -
+// row_base of each output row yr[m] (null = absent row).  `red` holds rbw * nwaves * MB * 16 floats
+// that nothing else uses.
 template <int MB>
-__device__ __forceinline__ void finish_rows(float (&v)[MB], float *red, int wave, int nwaves, int lane, int rb,
-                                            int row_base, int out_rows, float *const (&yr)[MB]) {
+__device__ __forceinline__ void park_rows(float (&v)[MB], float *red, int slot, int lane) {
 #pragma unroll
     for (int m = 0; m < MB; ++m) v[m] = reduce_kb4(v[m]);
     if (lane < 16) {
 #pragma unroll
-        for (int m = 0; m < MB; ++m) red[(wave * MB + m) * 16 + lane] = v[m];
-    }
-    __syncthreads();
-    if (wave == 0) {
-        const int r = lane & 15;
-        const int row = rb * 16 + r - row_base;
-#pragma unroll
-        for (int m = 0; m < MB; ++m) {
-            if ((lane >> 4) == (m & 3)) {
-                float s = 0.f;
-                for (int wv = 0; wv < nwaves; ++wv) s += red[(wv * MB + m) * 16 + r];
-                if (yr[m] && row >= 0 && row < out_rows) yr[m][row] = s;
-            }
-        }
+        for (int m = 0; m < MB; ++m) red[(slot * MB + m) * 16 + lane] = v[m];
     }
 }
 
-// Waves a decode GEMV launch aims for (the K-split per row-block follows from it); MFQ_GEMV_WAVES
-// overrides the default for tuning.
+template <int MB>
+__device__ __forceinline__ void flush_rows(const float *red, int nwaves, int rbw, int rb0, int row_base, int out_rows,
+                                           float *const (&yr)[MB]) {
+    __syncthreads();
+    for (int o = threadIdx.x; o < rbw * MB * 16; o += blockDim.x) {
+        const int r = o & 15, m = (o >> 4) % MB, rbi = (o >> 4) / MB;
+        float s = 0.f;
+        for (int wv = 0; wv < nwaves; ++wv) s += red[((rbi * nwaves + wv) * MB + m) * 16 + r];
+        const int row = (rb0 + rbi) * 16 + r - row_base;
+        float *dst = nullptr;
+#pragma unroll
+        for (int mm = 0; mm < MB; ++mm)
+            if (mm == m) dst = yr[mm];
+        if (dst && row >= 0 && row < out_rows) dst[row] = s;
+    }
+}
+
+template <int MB>
+__device__ __forceinline__ void finish_rows(float (&v)[MB], float *red, int wave, int nwaves, int lane, int rb,
+                                            int row_base, int out_rows, float *const (&yr)[MB]) {
+    park_rows<MB>(v, red, wave, lane);
+    flush_rows<MB>(red, nwaves, 1, rb, row_base, out_rows, yr);
+}
+
+// Fewest waves a decode GEMV launch aims for before a wave is given more than one step;
+// MFQ_GEMV_WAVES overrides the default for tuning.
 inline int gemv_target_waves() {
     static const int v = [] {
         const char *e = getenv("MFQ_GEMV_WAVES");
         const int n = e ? atoi(e) : 0;
-        return n > 0 ? n : 6144;
+        return n > 0 ? n : 2048;
     }();
     return v;
 }
 
 // LDS bytes of a GEMV block: per wave MB * steps_per_wave * 16 groups * (gs/2 pairs + 2 sums) dwords,
-// plus the cross-wave reduction area.
-inline size_t gemv_lds_bytes(int mb, int spw, int gs, int nwaves) {
-    return (static_cast<size_t>(mb) * spw * 16 * (gs / 2 + 2) * nwaves + static_cast<size_t>(nwaves) * mb * 16) * 4;
+// plus the cross-wave reduction area of rbw row-blocks.
+inline size_t gemv_lds_bytes(int mb, int spw, int gs, int nwaves, int rbw = 1) {
+    return (static_cast<size_t>(mb) * spw * 16 * (gs / 2 + 2) * nwaves + static_cast<size_t>(rbw) * nwaves * mb * 16) * 4;
 }
 
 // Dense activations: rows m0 .. m0+MB-1 of x[M, ldx] / y[M, ldy].

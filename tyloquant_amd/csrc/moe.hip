@@ -228,7 +228,7 @@ __global__ __launch_bounds__(1024) void moe_grouped_kernel(MoePools P, const int
     const int spw = P.spw[pool];
 #define MFQ_MOE_CASE(B, G)                                                                                    \
     if (k.bits == B && k.gs == G) {                                                                           \
-        nint_paired_body<B, G, XF16, MB>(k, w, rb, row_base, out_per_expert, xr, yr, spw, lds);               \
+        nint_paired_body<B, G, XF16, MB>(k, w, rb, 1, row_base, out_per_expert, xr, yr, spw, lds);            \
         return;                                                                                               \
     }
     if (k.kind == 1) {

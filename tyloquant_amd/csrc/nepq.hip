@@ -174,7 +174,9 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
     uint32_t *xs = xbase + wave * (MB * (npairs + 2 * ngl));
     float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
     float *red = reinterpret_cast<float *>(xbase + nwaves * (MB * (npairs + 2 * ngl)));
-    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane);
+    XRegs<MB> xg;
+    stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * 24, npairs, lane, xg);
+    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane, xg);
     if constexpr (TAB_LDS) __syncthreads();  // the LDS table copy was made by the whole block
 
     const int r = lane & 15, kb = lane >> 4;
@@ -224,7 +226,7 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
 }
 
 static void nepq_gemv_shape(const NepqK &k, int nrb, int mb, int &spw, int &nwaves, size_t &lds_bytes, bool &tab_lds) {
-    int want = static_cast<int>(ceil_div(gemv_target_waves(), nrb));
+    int want = static_cast<int>(ceil_div(3 * gemv_target_waves(), nrb));
     if (want < 1) want = 1;
     if (want > 16) want = 16;
     if (want > k.nsteps) want = k.nsteps;

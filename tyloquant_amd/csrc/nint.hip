@@ -183,30 +183,50 @@ __global__ void nint_dequant_kernel(NintK k, const uint8_t *__restrict__ w, OutT
 }
 
 // ---- GEMV ------------------------------------------------------------------------------
-// steps per wave / waves per block so that the grid has a few thousand waves and LDS fits
-static void gemv_shape(const NintK &k, int mb, int &spw, int &nwaves, size_t &lds_bytes) {
-    int want = static_cast<int>(ceil_div(gemv_target_waves(), k.n_rowblocks));
-    if (want < 1) want = 1;
-    if (want > 16) want = 16;
-    if (want > k.nsteps) want = k.nsteps;
-    spw = static_cast<int>(ceil_div(k.nsteps, want));
+// Block shape: the waves of a block split the K steps (spw steps each, at most 16 waves) and walk
+// through rbw row-blocks.  A wave takes up to three (row-block, step) items -- what the kernel variant
+// without a prefetch ring holds in registers -- as long as the grid keeps about gemv_target_waves()
+// waves; long neurons spend the items on K (fewer waves to reduce), short ones on row-blocks (the
+// staged activations are reused).  MFQ_GEMV_SPW / MFQ_GEMV_RBW override the choice for tuning.
+static void gemv_shape(const NintK &k, int mb, int &spw, int &nwaves, int &rbw, size_t &lds_bytes) {
+    static const int env_spw = [] { const char *e = getenv("MFQ_GEMV_SPW"); return e ? atoi(e) : 0; }();
+    static const int env_rbw = [] { const char *e = getenv("MFQ_GEMV_RBW"); return e ? atoi(e) : 0; }();
+    const int64_t items = static_cast<int64_t>(k.n_rowblocks) * k.nsteps;
+    int per_wave = static_cast<int>(items / gemv_target_waves());
+    per_wave = per_wave < 1 ? 1 : (per_wave > 3 ? 3 : per_wave);
+    const int spw_min = static_cast<int>(ceil_div(k.nsteps, 16));
+    spw = k.nsteps >= 16 ? per_wave : 1;
+    if (spw < spw_min) spw = spw_min;
+    if (env_spw > 0) spw = env_spw < spw_min ? spw_min : env_spw;
+    if (spw > k.nsteps) spw = k.nsteps;
     nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
-    lds_bytes = gemv_lds_bytes(mb, spw, k.gs, nwaves);
+    rbw = k.kind == 1 ? per_wave / spw : 1;
+    if (env_rbw > 0 && k.kind == 1) rbw = env_rbw;
+    if (rbw < 1) rbw = 1;
+    if (rbw > kMaxRbw) rbw = kMaxRbw;
+    if (rbw > k.n_rowblocks) rbw = k.n_rowblocks;
+    while (rbw > 1 && static_cast<int64_t>(rbw) * k.rowblock_bytes >= (1ll << 31)) --rbw;
+    lds_bytes = gemv_lds_bytes(mb, spw, k.gs, nwaves, rbw);
 }
 
 template <int XF16, int MB>
 static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                           hipStream_t st) {
-    int spw, nwaves;
+    int spw, nwaves, rbw;
     size_t lds;
-    gemv_shape(k, MB, spw, nwaves, lds);
+    gemv_shape(k, MB, spw, nwaves, rbw, lds);
     MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nint_gemv: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
-    const dim3 grid(k.n_rowblocks, static_cast<unsigned>(ceil_div(M, MB)));
+    MFQ_REQUIRE(k.rowblock_bytes < (1ll << 31), MFQ_ERR_UNSUPPORTED, "nint_gemv: neuron_len %d is too long", k.neuron_len);
     const dim3 block(64 * nwaves);
 #define MFQ_PAIRED(B, G)                                                                                     \
     if (k.bits == B && k.gs == G) {                                                                          \
-        hipLaunchKernelGGL((nint_gemv_paired_kernel<B, G, XF16, MB>), grid, block, lds, st, k, w, x, ldx, M, y, \
-                           ldy, spw);                                                                        \
+        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, rbw)), static_cast<unsigned>(ceil_div(M, MB))); \
+        if (spw * rbw <= 3)                                                                                  \
+            hipLaunchKernelGGL((nint_gemv_paired_kernel<B, G, XF16, MB, false>), grid, block, lds, st, k, w, x, ldx, \
+                               M, y, ldy, spw, rbw);                                                         \
+        else                                                                                                 \
+            hipLaunchKernelGGL((nint_gemv_paired_kernel<B, G, XF16, MB, true>), grid, block, lds, st, k, w, x, ldx, \
+                               M, y, ldy, spw, rbw);                                                         \
         return check_launch("nint_gemv_paired");                                                             \
     }
     if (k.kind == 1) {
@@ -215,6 +235,7 @@ static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, i
         return fail(MFQ_ERR_UNSUPPORTED, "nint_gemv: no paired kernel for NINT%d-%d", k.bits, k.gs);
     }
 #undef MFQ_PAIRED
+    const dim3 grid(k.n_rowblocks, static_cast<unsigned>(ceil_div(M, MB)));
     hipLaunchKernelGGL((nint_gemv_generic_kernel<XF16, MB>), grid, block, lds, st, k, w, x, ldx, M, y, ldy, spw);
     return check_launch("nint_gemv_generic");
 }
@@ -227,9 +248,9 @@ int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int
     // LDS per block grows with MB; large K falls back to narrower row batches.
     int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
     for (;;) {
-        int spw, nwaves;
+        int spw, nwaves, rbw;
         size_t lds;
-        gemv_shape(k, mb, spw, nwaves, lds);
+        gemv_shape(k, mb, spw, nwaves, rbw, lds);
         if (lds <= 65536 || mb == 1) break;
         mb >>= 1;
     }

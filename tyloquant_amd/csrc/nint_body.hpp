@@ -4,10 +4,12 @@
 // and of the following odd weight in the high half, at the same offset.  OR-ing a field that sits
 // at mantissa offset o of each half into the fp16 constant 1024.0 gives the exact fp16 pair
 // (1024 + 2^o * c_even, 1024 + 2^o * c_odd) without shifting it down, and one packed dot product
-// (v_dot2_f32_f16) multiplies the pair with the matching activations.  Fields at different offsets
-// go to different accumulators ("classes") that are rescaled by 2^-o once per group; the 1024 bias
-// leaves through T_g, the bias-weighted activation sum that the staging step precomputes:
-//     sum_i c_i x_i = sum_classes acc_class * 2^-o  -  T_g,   T_g = sum_pairs (x_2i + x_2i+1) * 1024 * 2^-o(i)
+// (v_dot2_f32_f16) multiplies the pair with the matching activations.  The activations of a pair
+// whose field sits at offset o are staged multiplied by 2^-o (exact in fp16), so every product is
+// 1024 * x' + c * x and one accumulator per group suffices; the 1024 bias leaves through T_g, the
+// 1024-weighted sum of the staged activations that the staging step precomputes and the
+// accumulator starts from:
+//     sum_i c_i x_i = sum_pairs (1024 + 2^o c) . x'  -  T_g,   T_g = 1024 * sum_pairs (x'_2i + x'_2i+1)
 // Ten mantissa bits hold two 4-bit fields, three 3-bit fields or two 2-bit fields (more with one
 // shift), so a dword of codes costs one shift plus one AND-OR and one dot2 per pair.
 #pragma once
@@ -22,30 +24,36 @@ struct NintK {  // what kernels need of mfq_nint_desc, passed by value
 };
 
 constexpr uint32_t kMagicH2 = 0x64006400u;  // (1024.0, 1024.0) in fp16
+constexpr int kMaxRbw = 4;                  // row-blocks one wave may walk through
 
 template <int BITS, int GS>
 struct PairedUnit {
     static constexpr int D = (BITS == 3) ? 2 : GS * BITS / 32;
     static constexpr bool TAIL = (BITS == 3);
-    static constexpr int NCLS = (BITS == 3) ? 3 : 2;
-    // reciprocal field scale of class c
-    __device__ static __forceinline__ constexpr float inv_scale(int c) {
-        return BITS == 4 ? (c ? 1.f / 16.f : 1.f) : BITS == 2 ? (c ? 0.25f : 1.f) : (c == 0 ? 1.f : c == 1 ? 0.125f : 1.f / 64.f);
-    }
-    // class of pair i of a group (pair i = weights 2i, 2i+1)
+    // mantissa offset class of pair i of a group (pair i = weights 2i, 2i+1): 4- and 2-bit fields
+    // alternate between offset 0 and BITS; 3-bit pairs sit at offsets 0,3,6,0,3 | 0,3,6,0,3 | 0,0
     __device__ static __forceinline__ int cls(int i) {
-        if constexpr (BITS == 3) return i < 10 ? static_cast<int>((0x10210u >> (4 * (i % 5))) & 3u) : 0;  // offsets 0,3,6,0,3
+        if constexpr (BITS == 3) return static_cast<int>((0x49124u >> (2 * i)) & 3u);
         else return i & 1;
     }
     struct Bias {
-        __device__ static __forceinline__ float bw(int i) { return 1024.f * inv_scale(cls(i)); }
+        static constexpr bool SCALED = true;
+        __device__ static __forceinline__ float bw(int) { return 1024.f; }
+        // 2^(-BITS * class): built in the exponent field
+        __device__ static __forceinline__ float xscale(int pos, int t) {
+            return __uint_as_float(0x3f800000u - (static_cast<uint32_t>(BITS * cls(BITS == 3 ? pos + t : t)) << 23));
+        }
+        __device__ static __forceinline__ float inv_xscale(int i) {
+            return __uint_as_float(0x3f800000u + (static_cast<uint32_t>(BITS * cls(i)) << 23));
+        }
     };
 
-    // acc[m][c] += sum over the pairs of class c of (1024 + scale_c * code) . x_m; xs = the group's GS/2 fp16
-    // pairs of activation row 0 in LDS, row m sits mstride dwords further.  Each pair is unpacked once for all rows.
+    // acc[m] += sum over the pairs of the group of (1024 + 2^o * code) . x'_m; xs = the group's GS/2 staged
+    // fp16 pairs of activation row 0 in LDS, row m sits mstride dwords further.  Each pair is unpacked
+    // once for all rows.
     template <int MB>
     __device__ static __forceinline__ void dot(const uint32_t (&q)[D], uint32_t tail, const uint32_t *xs, int mstride,
-                                               float (&acc)[MB][NCLS]) {
+                                               float (&acc)[MB]) {
         const uint32_t magic = kMagicH2;
         if constexpr (BITS == 4) {
 #pragma unroll
@@ -56,10 +64,10 @@ struct PairedUnit {
 #pragma unroll
                 for (int m = 0; m < MB; ++m) {
                     const u32x4_t x = *reinterpret_cast<const u32x4_t *>(xs + m * mstride + 4 * d);
-                    acc[m][0] = dot2h(v0, x.x, acc[m][0]);
-                    acc[m][1] = dot2h(v1, x.y, acc[m][1]);
-                    acc[m][0] = dot2h(v2, x.z, acc[m][0]);
-                    acc[m][1] = dot2h(v3, x.w, acc[m][1]);
+                    acc[m] = dot2h(v0, x.x, acc[m]);
+                    acc[m] = dot2h(v1, x.y, acc[m]);
+                    acc[m] = dot2h(v2, x.z, acc[m]);
+                    acc[m] = dot2h(v3, x.w, acc[m]);
                 }
             }
         } else if constexpr (BITS == 2) {
@@ -73,10 +81,10 @@ struct PairedUnit {
 #pragma unroll
                     for (int m = 0; m < MB; ++m) {
                         const u32x4_t x = *reinterpret_cast<const u32x4_t *>(xs + m * mstride + 8 * d + 4 * h);
-                        acc[m][0] = dot2h(v0, x.x, acc[m][0]);
-                        acc[m][1] = dot2h(v1, x.y, acc[m][1]);
-                        acc[m][0] = dot2h(v2, x.z, acc[m][0]);
-                        acc[m][1] = dot2h(v3, x.w, acc[m][1]);
+                        acc[m] = dot2h(v0, x.x, acc[m]);
+                        acc[m] = dot2h(v1, x.y, acc[m]);
+                        acc[m] = dot2h(v2, x.z, acc[m]);
+                        acc[m] = dot2h(v3, x.w, acc[m]);
                     }
                 }
             }
@@ -106,24 +114,22 @@ struct PairedUnit {
                 const u32x4_t x2 = *reinterpret_cast<const u32x4_t *>(xp + 8);
                 const uint32_t xv[12] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w, x2.x, x2.y, x2.z, x2.w};
 #pragma unroll
-                for (int i = 0; i < 12; ++i) {
-                    const int p5 = i % 5;
-                    const int c = i < 10 ? (p5 == 2 ? 2 : ((p5 == 1 || p5 == 4) ? 1 : 0)) : 0;   // offsets 0,3,6,0,3 | 0,0
-                    acc[m][c] = dot2h(v[i], xv[i], acc[m][c]);
-                }
+                for (int i = 0; i < 12; ++i) acc[m] = dot2h(v[i], xv[i], acc[m]);
             }
         }
     }
 };
 
+// Requests one step (16 groups of the row-block's 16 neurons) at window offset `off`; lane_q / lane_t /
+// lane_s are the lane's byte offsets inside the step's code, tail and scale regions.
 template <int D, bool TAIL>
-__device__ __forceinline__ void nint_load_step(const uint8_t *__restrict__ sp, int lane, uint32_t (&q)[4][D],
-                                               uint32_t &tails, u32x2_t &sc) {
+__device__ __forceinline__ void nint_load_step(__amdgpu_buffer_rsrc_t win, uint32_t off, int lane,
+                                               uint32_t (&q)[4][D], uint32_t &tails, u32x2_t &sc) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) load_unit<D>(reinterpret_cast<const uint32_t *>(sp) + (j * 64 + lane) * D, q[j]);
+    for (int j = 0; j < 4; ++j) load_unit_win<D>(win, off + (j * 64 + lane) * (D * 4), q[j]);
     tails = 0;
-    if constexpr (TAIL) tails = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sp + 1024 * D) + lane);
-    sc = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp + 1024 * D + (TAIL ? 256 : 0)) + lane);
+    if constexpr (TAIL) tails = __builtin_amdgcn_raw_buffer_load_b32(win, off + 1024 * D + lane * 4, 0, 2);
+    sc = __builtin_amdgcn_raw_buffer_load_b64(win, off + 1024 * D + (TAIL ? 256 : 0) + lane * 8, 0, 2);
 }
 
 template <int BITS, int GS, int MB>
@@ -138,77 +144,127 @@ __device__ __forceinline__ void nint_compute_step(const uint32_t (&q)[4][PairedU
         const float ss = ubyte_f32(scw, 2 * (j & 1));
         const float sm = ubyte_f32(scw, 2 * (j & 1) + 1);
         const uint32_t tail = (tails >> (8 * j)) & 0xffu;
-        float a[MB][U::NCLS];
-#pragma unroll
-        for (int m = 0; m < MB; ++m)
-#pragma unroll
-            for (int c = 0; c < U::NCLS; ++c) a[m][c] = 0.f;
-        U::template dot<MB>(q[j], tail, xs + lg * (GS / 2), npairs, a);
+        float a[MB], xg[MB];
 #pragma unroll
         for (int m = 0; m < MB; ++m) {
             const float2 xt = *reinterpret_cast<const float2 *>(xsum + (m * ngl + lg) * 2);
-            float raw = a[m][0] - xt.y;
+            xg[m] = xt.x;
+            a[m] = xt.y;  // -T_g
+        }
+        U::template dot<MB>(q[j], tail, xs + lg * (GS / 2), npairs, a);
 #pragma unroll
-            for (int c = 1; c < U::NCLS; ++c) raw = fmaf(a[m][c], U::inv_scale(c), raw);
-            accS[m] = fmaf(ss, raw, accS[m]);
-            accM[m] = fmaf(sm, xt.x, accM[m]);
+        for (int m = 0; m < MB; ++m) {
+            accS[m] = fmaf(ss, a[m], accS[m]);
+            accM[m] = fmaf(sm, xg[m], accM[m]);
         }
     }
 }
 
-// One block = one 16-neuron row-block `rb` of the tensor at `w`; its waves split the steps, `spw`
-// steps per wave.  xr / yr name the MB activation and output rows (see finish_rows for row_base).
-// The anchors and the first steps' weights are requested before the activations are staged, and
-// each later step is requested three steps ahead into a ring of register buffers, so HBM latency
-// overlaps the LDS staging and the unpack arithmetic.
-template <int BITS, int GS, int XF16, int MB>
-__device__ __forceinline__ void nint_paired_body(const NintK &k, const uint8_t *__restrict__ w, int rb, int row_base,
-                                                 int out_rows, const uint16_t *const (&xr)[MB], float *const (&yr)[MB],
-                                                 int spw, uint32_t *lds) {
+// One block = `rbw` consecutive 16-neuron row-blocks starting at `rb0` of the tensor at `w`; its waves
+// split the K steps, `spw` steps per wave, and every wave walks through its K-slice of each row-block
+// in turn, so the slice of the activations is staged once for all of them.  xr / yr name the MB
+// activation and output rows (see flush_rows for row_base).
+// The activations are requested first, then the anchors and the first three steps, and each later
+// step three steps ahead into a ring of register buffers: loads retire in order and every weight load
+// is an unconditional window load, so the staging waits for the activations only and the unpack of a
+// step only for that step.  RING = false is the variant for waves with at most three steps in all, which
+// never requests more.
+template <int BITS, int GS, int XF16, int MB, bool RING = true>
+__device__ __forceinline__ void nint_paired_body(const NintK &k, const uint8_t *__restrict__ w, int rb0, int rbw,
+                                                 int row_base, int out_rows, const uint16_t *const (&xr)[MB],
+                                                 float *const (&yr)[MB], int spw, uint32_t *lds) {
     using U = PairedUnit<BITS, GS>;
     constexpr int D = U::D;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
     const int r = lane & 15, kb = lane >> 4;
     const int s0 = wave * spw;
-    const int s1 = min(k.nsteps, s0 + spw);
+    const int n = min(k.nsteps, s0 + spw) - s0;         // steps of this wave in each row-block
+    const int nrb = min(rbw, k.n_rowblocks - rb0);      // row-blocks of this block
     const int ngl = spw * 16, npairs = ngl * (GS / 2);
     uint32_t *xs = lds + wave * (MB * (npairs + 2 * ngl));
     float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
     float *red = reinterpret_cast<float *>(lds + nwaves * (MB * (npairs + 2 * ngl)));
-    const int sb = static_cast<int>(k.step_bytes);
-    const uint8_t *base = w + static_cast<int64_t>(rb) * k.rowblock_bytes + static_cast<int64_t>(s0) * sb;
-    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
-    const float ns = anchors[rb * 16 + r], nm = anchors[16 * k.n_rowblocks + rb * 16 + r];
+    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
 
-    // four register buffers in a ring: three steps are in flight while one is being unpacked
-    uint32_t q0[4][D], q1[4][D], q2[4][D], q3[4][D], t0 = 0, t1 = 0, t2 = 0, t3 = 0;
-    u32x2_t c0 = {0u, 0u}, c1 = c0, c2 = c0, c3 = c0;
-    const int n = s1 - s0;
-    if (n > 0) nint_load_step<D, U::TAIL>(base, lane, q0, t0, c0);
-    if (n > 1) nint_load_step<D, U::TAIL>(base + sb, lane, q1, t1, c1);
-    if (n > 2) nint_load_step<D, U::TAIL>(base + 2 * sb, lane, q2, t2, c2);
-    stage_x<XF16, MB, typename U::Bias>(xr, k.neuron_len, s0 * 16 * GS, npairs, GS, ngl, xs, xsum, lane);
+    XRegs<MB> xg;
+    stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * GS, npairs, lane, xg);
+    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
+    float ns[kMaxRbw], nm[kMaxRbw];
+#pragma unroll
+    for (int i = 0; i < kMaxRbw; ++i) {
+        const int rb = min(rb0 + i, k.n_rowblocks - 1);
+        ns[i] = anchors[rb * 16 + r];
+        nm[i] = anchors[16 * k.n_rowblocks + rb * 16 + r];
+    }
+    const __amdgpu_buffer_rsrc_t win =
+        wave_window(w + static_cast<int64_t>(rb0) * k.rowblock_bytes + static_cast<int64_t>(s0) * sb,
+                    n > 0 ? (nrb - 1) * rbb + n * sb : 0u);
+
+    // issue cursor (row-block, step) three items ahead of the compute cursor; both are wave-uniform
+    int irb = 0, is = 0;
+#define MFQ_ISSUE(Q, T, C)                                                        \
+    {                                                                             \
+        const uint32_t off = (irb < nrb && n > 0) ? irb * rbb + is * sb : kNoStep; \
+        nint_load_step<D, U::TAIL>(win, off, lane, Q, T, C);                      \
+        if (++is >= n) { is = 0; ++irb; }                                         \
+    }
+    uint32_t q0[4][D], q1[4][D], q2[4][D], t0, t1, t2;
+    u32x2_t c0, c1, c2;
+    MFQ_ISSUE(q0, t0, c0)
+    MFQ_ISSUE(q1, t1, c1)
+    MFQ_ISSUE(q2, t2, c2)
+    stage_x<XF16, MB, typename U::Bias>(xr, k.neuron_len, s0 * 16 * GS, npairs, GS, ngl, xs, xsum, lane, xg);
 
     float accS[MB], accM[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) accS[m] = accM[m] = 0.f;
-    for (int i = 0; i < n; i += 4) {
-        if (i + 3 < n) nint_load_step<D, U::TAIL>(base + (i + 3) * sb, lane, q3, t3, c3);
-        nint_compute_step<BITS, GS, MB>(q0, t0, c0, i * 16 + kb, xs, xsum, npairs, ngl, accS, accM);
-        if (i + 1 >= n) break;
-        if (i + 4 < n) nint_load_step<D, U::TAIL>(base + (i + 4) * sb, lane, q0, t0, c0);
-        nint_compute_step<BITS, GS, MB>(q1, t1, c1, (i + 1) * 16 + kb, xs, xsum, npairs, ngl, accS, accM);
-        if (i + 2 >= n) break;
-        if (i + 5 < n) nint_load_step<D, U::TAIL>(base + (i + 5) * sb, lane, q1, t1, c1);
-        nint_compute_step<BITS, GS, MB>(q2, t2, c2, (i + 2) * 16 + kb, xs, xsum, npairs, ngl, accS, accM);
-        if (i + 3 >= n) break;
-        if (i + 6 < n) nint_load_step<D, U::TAIL>(base + (i + 6) * sb, lane, q2, t2, c2);
-        nint_compute_step<BITS, GS, MB>(q3, t3, c3, (i + 3) * 16 + kb, xs, xsum, npairs, ngl, accS, accM);
+    int crb = 0, cs = 0;
+#define MFQ_COMPUTE(Q, T, C)                                                                              \
+    {                                                                                                     \
+        nint_compute_step<BITS, GS, MB>(Q, T, C, cs * 16 + kb, xs, xsum, npairs, ngl, accS, accM);         \
+        if (++cs >= n) {                                                                                  \
+            float a_s = ns[0], a_m = nm[0];                                                               \
+            _Pragma("unroll") for (int i = 1; i < kMaxRbw; ++i) if (crb == i) { a_s = ns[i]; a_m = nm[i]; } \
+            float v[MB];                                                                                  \
+            _Pragma("unroll") for (int m = 0; m < MB; ++m) {                                              \
+                v[m] = a_s * accS[m] - a_m * accM[m];                                                     \
+                accS[m] = accM[m] = 0.f;                                                                  \
+            }                                                                                             \
+            park_rows<MB>(v, red, crb * nwaves + wave, lane);                                             \
+            cs = 0;                                                                                       \
+            ++crb;                                                                                        \
+        }                                                                                                 \
     }
-    float v[MB];
+    const int items = nrb * n;
+    if (n <= 0) {  // a wave beyond the last step still owes its (zero) partial sums
+        float z[MB];
+        for (int i = 0; i < nrb; ++i) {
 #pragma unroll
-    for (int m = 0; m < MB; ++m) v[m] = ns * accS[m] - nm * accM[m];
-    finish_rows<MB>(v, red, wave, nwaves, lane, rb, row_base, out_rows, yr);
+            for (int m = 0; m < MB; ++m) z[m] = 0.f;
+            park_rows<MB>(z, red, i * nwaves + wave, lane);
+        }
+    } else if constexpr (!RING) {  // at most 3 items: everything is already requested
+        MFQ_COMPUTE(q0, t0, c0)
+        if (items > 1) MFQ_COMPUTE(q1, t1, c1)
+        if (items > 2) MFQ_COMPUTE(q2, t2, c2)
+    } else {
+        uint32_t q3[4][D], t3;
+        u32x2_t c3;
+        for (int t = 0; t < items; t += 4) {
+            MFQ_ISSUE(q3, t3, c3)
+            MFQ_COMPUTE(q0, t0, c0)
+            MFQ_ISSUE(q0, t0, c0)
+            if (t + 1 < items) MFQ_COMPUTE(q1, t1, c1)
+            MFQ_ISSUE(q1, t1, c1)
+            if (t + 2 < items) MFQ_COMPUTE(q2, t2, c2)
+            MFQ_ISSUE(q2, t2, c2)
+            if (t + 3 < items) MFQ_COMPUTE(q3, t3, c3)
+        }
+    }
+#undef MFQ_ISSUE
+#undef MFQ_COMPUTE
+    flush_rows<MB>(red, nwaves, nrb, rb0, row_base, out_rows, yr);
 }
 
 // Any (bits, gs): natural-order units, one code at a time in fp32.
@@ -223,7 +279,9 @@ __device__ __forceinline__ void nint_generic_body(const NintK &k, const uint8_t 
     uint32_t *xs = lds + wave * (MB * (npairs + 2 * ngl));
     float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
     float *red = reinterpret_cast<float *>(lds + nwaves * (MB * (npairs + 2 * ngl)));
-    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * gs, npairs, gs, ngl, xs, xsum, lane);
+    XRegs<MB> xg;
+    stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * gs, npairs, lane, xg);
+    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * gs, npairs, gs, ngl, xs, xsum, lane, xg);
     const uint16_t *xh = reinterpret_cast<const uint16_t *>(xs);
 
     const int r = lane & 15, kb = lane >> 4;
@@ -268,15 +326,15 @@ __device__ __forceinline__ void nint_generic_body(const NintK &k, const uint8_t 
 }
 
 // Dense wrappers: block (rb, m-chunk).
-template <int BITS, int GS, int XF16, int MB>
+template <int BITS, int GS, int XF16, int MB, bool RING>
 __global__ __launch_bounds__(1024) void nint_gemv_paired_kernel(NintK k, const uint8_t *__restrict__ w,
                                                                 const uint16_t *__restrict__ x, int64_t ldx, int M,
-                                                                float *__restrict__ y, int64_t ldy, int spw) {
+                                                                float *__restrict__ y, int64_t ldy, int spw, int rbw) {
     extern __shared__ uint32_t lds[];
     const uint16_t *xr[MB];
     float *yr[MB];
     dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
-    nint_paired_body<BITS, GS, XF16, MB>(k, w, blockIdx.x, 0, k.out, xr, yr, spw, lds);
+    nint_paired_body<BITS, GS, XF16, MB, RING>(k, w, blockIdx.x * rbw, rbw, 0, k.out, xr, yr, spw, lds);
 }
 
 template <int XF16, int MB>

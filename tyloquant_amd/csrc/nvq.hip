@@ -211,8 +211,10 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
         st.hh = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp + 2048) + lane);
     };
     Step cur, nxt;
+    XRegs<MB> xg;
+    stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * 24, npairs, lane, xg);
     if (s0 < s1) load_step(s0, cur);
-    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane);
+    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane, xg);
     __syncthreads();  // the LDS tables were filled by the whole block
 
     const int r = lane & 15, kb = lane >> 4;
@@ -266,7 +268,7 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
 }
 
 static void nvq_gemv_shape(const NvqK &k, int mb, int &spw, int &nwaves, size_t &lds_bytes) {
-    int want = static_cast<int>(ceil_div(gemv_target_waves(), k.n_rowblocks));
+    int want = static_cast<int>(ceil_div(3 * gemv_target_waves(), k.n_rowblocks));
     if (want < 1) want = 1;
     if (want > 16) want = 16;
     if (want > k.nsteps) want = k.nsteps;
