@@ -159,18 +159,157 @@ def main() -> int:
         torch.cuda.synchronize()
         return a.elapsed_time(b) / reps
 
+    def graph_ms(fn, reps, warm=2):
+        """ms per call of fn() when it is replayed from a HIP graph (decode runs under graphs)."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        for _ in range(warm):
+            g.replay()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps
+
+    def clone_w(w):
+        import copy
+        c = copy.copy(w)
+        c.data = w.data.clone()
+        if hasattr(w, "_ws"):
+            c._ws = type(w._ws)()
+        return c
+
+    def bf16(a):
+        return torch.from_numpy(a).to(torch.bfloat16).to(dev)
+
     if not args.no_extras:
+        from tyloquant_amd import runtime_moe as RM
+        from tyloquant_amd import runtime_vq as RV
         # hot (one weight set, cache-resident between launches)
         hot_ms = time_fn(lambda: launch(sets[0], stream_ptr()), 100)
         extras["decode_hot_gbps"] = step_bytes / (hot_ms * 1e-3) / 1e9
-        # prefill qGEMM on the gate shape
+        # ---- config 2: batch sweep on the gate shape (GEMV up to 8 rows, MFMA path above) -------------
         wg = sets[0]["gate"]
         for M in (16, 512, 2048):
-            xm = torch.from_numpy(synth.activations(rng, M, H, outlier_frac=0.001)).to(torch.bfloat16).to(dev)
+            xm = bf16(synth.activations(rng, M, H, outlier_frac=0.001))
             ms = time_fn(lambda: R.nint_matmul(wg, xm), 10, warm=3)
             extras[f"prefill_M{M}_tflops"] = 2.0 * M * FF * H / (ms * 1e-3) / 1e12
             extras[f"prefill_M{M}_ms"] = ms
-        log(f"[bench] extras: {extras}")
+            extras[f"prefill_M{M}_frac_of_f16_mfma_peak"] = extras[f"prefill_M{M}_tflops"] / MFMA_F16_PEAK_TFLOPS
+        log(f"[bench] config 2 extras: {extras}")
+        del sets[1:]
+        torch.cuda.empty_cache()
+
+        # ---- config 1: NINT3 (3,24,5) 4096x4096 at batch 1, rotating over 40 copies (310 MB) --------
+        w1 = R.load_quant_linear("NINT3", synth.nint_linear_blob(7, 4096, 4096, 3, 24, 5, slab_rows=1024)[1]).weight
+        c1 = [w1] + [clone_w(w1) for _ in range(39)]
+        x1 = bf16(synth.activations(rng, 1, 4096))
+        ms = graph_ms(lambda: [R.nint_matmul(w, x1, force="gemv") for w in c1], 20) / len(c1)
+        b1 = w1.payload_bytes + 2 * 4096 + 4 * 4096
+        extras["config1_nint3_us"] = ms * 1e3
+        extras["config1_nint3_gbps"] = b1 / (ms * 1e-3) / 1e9
+        log(f"[bench] config 1 NINT3 4096x4096 M=1: {ms * 1e3:.2f} us, {extras['config1_nint3_gbps']:.0f} GB/s")
+        del c1
+
+        # ---- config 3: NVQ3J-512 17408x5120 and its transpose, batch {1,4,8}, 8 rotating copies -----
+        for name, (n3, k3) in {"up": (17408, 5120), "down": (5120, 17408)}.items():
+            w3 = synth.tile_rows(RV.NvqWeight.from_blob(synth.nvq3j512_blob(11, 1024, k3)[1]), n3)
+            c3 = [w3] + [clone_w(w3) for _ in range(7)]
+            for M in (1, 4, 8):
+                x3 = bf16(synth.activations(rng, M, k3))
+                ms = graph_ms(lambda: [RV.nvq_matmul(w, x3) for w in c3], 10) / len(c3)
+                b3 = w3.payload_bytes + 2 * M * k3 + 4 * M * n3
+                extras[f"config3_nvq_{name}_M{M}_us"] = ms * 1e3
+                extras[f"config3_nvq_{name}_M{M}_gbps"] = b3 / (ms * 1e-3) / 1e9
+            log(f"[bench] config 3 NVQ3J-512 {n3}x{k3}: " + ", ".join(
+                f"M={M} {extras[f'config3_nvq_{name}_M{M}_gbps']:.0f} GB/s" for M in (1, 4, 8)))
+            del c3, w3
+        torch.cuda.empty_cache()
+
+        # ---- config 4: 256 mixed-bit experts + 1 shared, hidden 4096, intermediate 2048, top-8 ------
+        E, HID, INTER, TOPK = 256, 4096, 2048, 8
+        ebits = np.random.default_rng(4).choice([2, 3, 4, 5], size=E, p=[0.1, 0.4, 0.4, 0.1])
+        gu = synth.random_nint_moe(40, E, 2 * INTER, HID, ebits)
+        dn = synth.random_nint_moe(41, E, HID, INTER, ebits)
+        shared = (synth.random_nint_weight(42, 2 * INTER, HID, 4, 24, 6), synth.random_nint_weight(43, HID, INTER, 4, 24, 6))
+        shared_bytes = shared[0].payload_bytes + shared[1].payload_bytes
+        per_expert = np.array([gu.expert_payload_bytes(e) + dn.expert_payload_bytes(e) for e in range(E)])
+        for T, nb in ((1, 8), (64, 2), (2048, 1)):
+            xs4 = [bf16(synth.activations(rng, T, HID)) for _ in range(nb)]
+            lg4 = [torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).to(dev) for _ in range(nb)]
+
+            def moe_all():
+                return [RM.nint_moe_ffn_forward(gu, dn, xs4[i], lg4[i], TOPK, delayed_softmax=True, shared=shared)
+                        for i in range(nb)]
+            eager = moe_all()
+            torch.cuda.synchronize()
+            hit_bytes = 0.0
+            for (_, ids, _w) in eager:
+                hit_bytes += per_expert[np.unique(ids.cpu().numpy())].sum() + shared_bytes
+            try:
+                ms = graph_ms(moe_all, 5 if T < 2048 else 2) / nb
+                how = "hip graph"
+            except Exception as exc:  # capture refused by an op: time eager launches instead
+                log(f"[bench] MoE T={T}: graph capture failed ({exc}); timing eager")
+                torch.cuda.synchronize()
+                ms = time_fn(moe_all, 3, warm=1) / nb
+                how = "eager"
+            extras[f"config4_moe_T{T}_ms"] = ms
+            extras[f"config4_moe_T{T}_tokens_per_s"] = T / (ms * 1e-3)
+            extras[f"config4_moe_T{T}_weight_gbps"] = hit_bytes / nb / (ms * 1e-3) / 1e9
+            extras[f"config4_moe_T{T}_tflops"] = (2.0 * T * TOPK * 3 * HID * INTER + 2.0 * T * 3 * HID * INTER) / (ms * 1e-3) / 1e12
+            log(f"[bench] config 4 MoE T={T}: {ms:.3f} ms ({how}), {T / (ms * 1e-3):.0f} tokens/s, "
+                f"{extras[f'config4_moe_T{T}_weight_gbps']:.0f} GB/s of expert payload")
+            del eager
+        del gu, dn, shared
+        torch.cuda.empty_cache()
+
+        # ---- config 5: 36-layer linear stack, mixed formats by seed, batch {1,16} -------------------
+        shapes5 = {"qkv": (6144, 4096), "o": (4096, 4096), "gate": (12288, 4096), "up": (12288, 4096), "down": (4096, 12288)}
+        fmts = ["NEPQ1-S", "NINT3", "NVQ3J-512", "NINT5"]
+        pick = np.random.default_rng(5).choice(4, size=(36, 5), p=[0.2, 0.4, 0.25, 0.15])
+        proto = {}
+
+        def proto_weight(fmt, n, k):
+            key = (fmt, n, k)
+            if key not in proto:
+                if fmt == "NINT3":
+                    proto[key] = ("nint", synth.random_nint_weight(50, n, k, 3, 24, 5))
+                elif fmt == "NINT5":
+                    proto[key] = ("nint", synth.random_nint_weight(51, n, k, 5, 28, 7))
+                elif fmt == "NVQ3J-512":
+                    proto[key] = ("nvq", synth.tile_rows(RV.NvqWeight.from_blob(synth.nvq3j512_blob(52, 512, k)[1]), n))
+                else:
+                    proto[key] = ("nepq", synth.tile_rows(RV.NepqWeight.from_blob(synth.nepq1_blob(53, fmt, 512, k)[1]), n))
+            return proto[key]
+        stack, bytes5 = [], 0
+        for layer in range(36):
+            for ti, (tname, (n, k)) in enumerate(shapes5.items()):
+                kind, w = proto_weight(fmts[pick[layer, ti]], n, k)
+                stack.append((kind, clone_w(w), n, k))
+                bytes5 += w.payload_bytes
+        extras["config5_payload_gb"] = bytes5 / 1e9
+        mm = {"nint": R.nint_matmul, "nvq": RV.nvq_matmul, "nepq": RV.nepq_matmul}
+        for M in (1, 16):
+            xk = {k: bf16(synth.activations(rng, M, k)) for k in (4096, 12288)}
+            ms = graph_ms(lambda: [mm[kind](w, xk[k]) for kind, w, n, k in stack], 3, warm=1)
+            tot = bytes5 + sum(2 * M * k + 4 * M * n for _, _, n, k in stack)
+            extras[f"config5_stack_M{M}_ms"] = ms
+            extras[f"config5_stack_M{M}_gbps"] = tot / (ms * 1e-3) / 1e9
+            log(f"[bench] config 5 stack (180 matmuls, {bytes5 / 1e9:.2f} GB) M={M}: {ms:.3f} ms, "
+                f"{extras[f'config5_stack_M{M}_gbps']:.0f} GB/s")
+        del stack, proto
+        torch.cuda.empty_cache()
 
     cpu = None
     if not args.no_cpu:

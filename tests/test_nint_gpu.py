@@ -56,6 +56,26 @@ def test_gemv_matches_oracle(bits, gs, sb, M):
         assert np.abs(y - ref).max() < ABS_TOL
 
 
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (4, 16, 6), (4, 48, 6),
+                                        (2, 32, 5), (4, 32, 8)])
+@pytest.mark.parametrize("out,K,M", [(128, 1024, 2), (200, 2056, 16), (80, 4096, 5), (96, 1544, 17), (64, 12288, 40)])
+def test_small_batch_matrix_core_path(bits, gs, sb, out, K, M):
+    """Batches of 2..64 rows stream the packed weights once per 16 rows through the MFMA kernel (K % 8 == 0,
+    16-byte aligned rows); ragged K, a row stride above K and more rows than one 16-row tile."""
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(900 + bits * 10 + gs + M)
+    t = O.quantize_nint((rng.standard_normal((out, K)) * 0.02).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    deq = O.dequantize_nint(t)
+    for dtype in (torch.bfloat16, torch.float16):
+        xw = torch.from_numpy(rng.standard_normal((M, K + 8)).astype(np.float32)).to(dtype).cuda()
+        x = xw[:, :K]                       # row stride K + 8
+        y = R.nint_matmul(lin.weight, x, force="gemv").cpu().numpy()
+        ref = O.linear_forward_f64(deq, x.float().cpu().numpy())
+        assert rel_l2(y, ref) < REL_TOL, (dtype, rel_l2(y, ref))
+        assert np.abs(y - ref).max() < ABS_TOL
+
+
 @pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (4, 24, 6)])
 @pytest.mark.parametrize("out,K,M", [(128, 280, 16), (257, 224, 23), (73, 1537, 65), (512, 1024, 257)])
 def test_gemm_matches_oracle(bits, gs, sb, out, K, M):

@@ -6,7 +6,6 @@ Loading fails loudly when it is missing: there is no CPU fallback for any kernel
 from __future__ import annotations
 
 import ctypes as C
-import os
 from pathlib import Path
 
 _HERE = Path(__file__).resolve().parent
@@ -101,8 +100,6 @@ def lib() -> C.CDLL:
         for name, (res, args) in _SIGS.items():
             fn = getattr(_lib, name, None)
             if fn is None:
-                if os.environ.get("MFQ_ALLOW_MISSING_SYMBOLS") == "1":  # partial builds during kernel bring-up
-                    continue
                 raise MfqError(f"{LIB_PATH} does not export {name}: rebuild it (make -C tyloquant_amd/csrc)")
             fn.restype, fn.argtypes = res, args
     return _lib

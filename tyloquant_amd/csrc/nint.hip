@@ -16,6 +16,7 @@
 #include "common.hpp"
 #include "gemv_common.hpp"
 #include "nint_body.hpp"
+#include "nint_mfma.hpp"
 
 namespace mfq {
 
@@ -240,11 +241,58 @@ static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, i
     return check_launch("nint_gemv_generic");
 }
 
+// ---- small batches on the matrix cores ----------------------------------------------------
+// natural-order profiles with a matrix-core kernel (the paired ones all have one)
+static bool mfma_generic_profile(const NintK &k) { return k.kind == 0 && k.bits == 5 && k.gs == 28; }
+
+static bool mfma_eligible(const NintK &k, const void *x, int64_t ldx) {
+    return (k.kind == 1 || mfma_generic_profile(k)) && k.neuron_len >= 8 && k.neuron_len % 8 == 0 && ldx % 8 == 0 &&
+           (reinterpret_cast<uintptr_t>(x) & 15) == 0 && 4 * k.rowblock_bytes < (1ll << 31);
+}
+
+template <int XF16, int NB>
+static int launch_mfma_nb(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                          hipStream_t st) {
+    const int64_t groups = ceil_div(k.n_rowblocks, NB);
+    int spw = static_cast<int>(ceil_div(k.nsteps, 8));
+    while (spw < k.nsteps && groups * ceil_div(k.nsteps, spw) > 8192) ++spw;
+    const int nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
+    const size_t lds = static_cast<size_t>(nwaves) * NB * 1024;
+    const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(ceil_div(M, 16))), block(64 * nwaves);
+#define MFQ_MFMA(UNIT, B, G)                                                                                   \
+    if (k.bits == B && k.gs == G) {                                                                             \
+        hipLaunchKernelGGL((nint_mfma_kernel<UNIT<B, G>, XF16, NB>), grid, block, lds, st, k, w, x, ldx, M, y, ldy, \
+                           spw);                                                                                \
+        return check_launch("nint_mfma");                                                                       \
+    }
+    if (k.kind == 1) {
+        MFQ_MFMA(PairedUnit, 4, 32) MFQ_MFMA(PairedUnit, 4, 24) MFQ_MFMA(PairedUnit, 4, 16) MFQ_MFMA(PairedUnit, 4, 48)
+        MFQ_MFMA(PairedUnit, 3, 24) MFQ_MFMA(PairedUnit, 2, 16) MFQ_MFMA(PairedUnit, 2, 32)
+    } else {
+        MFQ_MFMA(GenericUnit, 5, 28)
+    }
+#undef MFQ_MFMA
+    return fail(MFQ_ERR_UNSUPPORTED, "nint_mfma: no kernel for NINT%d-%d", k.bits, k.gs);
+}
+
+template <int XF16>
+static int launch_mfma(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                       hipStream_t st) {
+    // row-blocks per wave: as many as still leave about 1500 waves
+    const int64_t items = static_cast<int64_t>(k.n_rowblocks) * k.nsteps;
+    if (items >= 4 * 1536) return launch_mfma_nb<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
+    if (items >= 2 * 1536) return launch_mfma_nb<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
+    return launch_mfma_nb<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
+}
+
 int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                   int64_t ldy, hipStream_t st) {
     const NintK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
+    if ((M >= 2 || k.kind == 0) && mfma_eligible(k, x, ldx))
+        return x_dtype == MFQ_X_F16 ? launch_mfma<1>(k, w, xp, ldx, M, y, ldy, st)
+                                    : launch_mfma<0>(k, w, xp, ldx, M, y, ldy, st);
     // LDS per block grows with MB; large K falls back to narrower row batches.
     int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
     for (;;) {

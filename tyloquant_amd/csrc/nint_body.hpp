@@ -30,9 +30,10 @@ template <int BITS, int GS>
 struct PairedUnit {
     static constexpr int D = (BITS == 3) ? 2 : GS * BITS / 32;
     static constexpr bool TAIL = (BITS == 3);
+    static constexpr int GROUP = GS, NPAIR = GS / 2, CBITS = BITS;
     // mantissa offset class of pair i of a group (pair i = weights 2i, 2i+1): 4- and 2-bit fields
     // alternate between offset 0 and BITS; 3-bit pairs sit at offsets 0,3,6,0,3 | 0,3,6,0,3 | 0,0
-    __device__ static __forceinline__ int cls(int i) {
+    __device__ static __forceinline__ constexpr int cls(int i) {
         if constexpr (BITS == 3) return static_cast<int>((0x49124u >> (2 * i)) & 3u);
         else return i & 1;
     }
@@ -48,27 +49,17 @@ struct PairedUnit {
         }
     };
 
-    // acc[m] += sum over the pairs of the group of (1024 + 2^o * code) . x'_m; xs = the group's GS/2 staged
-    // fp16 pairs of activation row 0 in LDS, row m sits mstride dwords further.  Each pair is unpacked
-    // once for all rows.
-    template <int MB>
-    __device__ static __forceinline__ void dot(const uint32_t (&q)[D], uint32_t tail, const uint32_t *xs, int mstride,
-                                               float (&acc)[MB]) {
+    // v[i] = fp16 pair (1024 + 2^o * code_2i, 1024 + 2^o * code_2i+1) of pair i of the group, o = BITS * cls(i)
+    __device__ static __forceinline__ void unpack(const uint32_t (&q)[D], uint32_t tail, uint32_t (&v)[GS / 2]) {
         const uint32_t magic = kMagicH2;
         if constexpr (BITS == 4) {
 #pragma unroll
             for (int d = 0; d < D; ++d) {
                 const uint32_t hi = q[d] >> 8;
-                const uint32_t v0 = and_or(q[d], 0x000F000Fu, magic), v1 = and_or(q[d], 0x00F000F0u, magic);
-                const uint32_t v2 = and_or(hi, 0x000F000Fu, magic), v3 = and_or(hi, 0x00F000F0u, magic);
-#pragma unroll
-                for (int m = 0; m < MB; ++m) {
-                    const u32x4_t x = *reinterpret_cast<const u32x4_t *>(xs + m * mstride + 4 * d);
-                    acc[m] = dot2h(v0, x.x, acc[m]);
-                    acc[m] = dot2h(v1, x.y, acc[m]);
-                    acc[m] = dot2h(v2, x.z, acc[m]);
-                    acc[m] = dot2h(v3, x.w, acc[m]);
-                }
+                v[4 * d] = and_or(q[d], 0x000F000Fu, magic);
+                v[4 * d + 1] = and_or(q[d], 0x00F000F0u, magic);
+                v[4 * d + 2] = and_or(hi, 0x000F000Fu, magic);
+                v[4 * d + 3] = and_or(hi, 0x00F000F0u, magic);
             }
         } else if constexpr (BITS == 2) {
 #pragma unroll
@@ -76,20 +67,13 @@ struct PairedUnit {
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     const uint32_t a = q[d] >> (8 * h), b = q[d] >> (8 * h + 4);
-                    const uint32_t v0 = and_or(a, 0x00030003u, magic), v1 = and_or(a, 0x000C000Cu, magic);
-                    const uint32_t v2 = and_or(b, 0x00030003u, magic), v3 = and_or(b, 0x000C000Cu, magic);
-#pragma unroll
-                    for (int m = 0; m < MB; ++m) {
-                        const u32x4_t x = *reinterpret_cast<const u32x4_t *>(xs + m * mstride + 8 * d + 4 * h);
-                        acc[m] = dot2h(v0, x.x, acc[m]);
-                        acc[m] = dot2h(v1, x.y, acc[m]);
-                        acc[m] = dot2h(v2, x.z, acc[m]);
-                        acc[m] = dot2h(v3, x.w, acc[m]);
-                    }
+                    v[8 * d + 4 * h] = and_or(a, 0x00030003u, magic);
+                    v[8 * d + 4 * h + 1] = and_or(a, 0x000C000Cu, magic);
+                    v[8 * d + 4 * h + 2] = and_or(b, 0x00030003u, magic);
+                    v[8 * d + 4 * h + 3] = and_or(b, 0x000C000Cu, magic);
                 }
             }
         } else {
-            uint32_t v[12];
 #pragma unroll
             for (int d = 0; d < 2; ++d) {
                 const uint32_t hi = q[d] >> 9;
@@ -106,16 +90,53 @@ struct PairedUnit {
             b |= ((tail >> 6) & 1u) << 1;
             b |= ((tail >> 7) & 1u) << 17;
             v[11] = b;
+        }
+    }
+
+    // acc[m] += sum over the pairs of the group of (1024 + 2^o * code) . x'_m; xs = the group's GS/2 staged
+    // fp16 pairs of activation row 0 in LDS, row m sits mstride dwords further.  Each pair is unpacked
+    // once for all rows.
+    template <int MB>
+    __device__ static __forceinline__ void dot(const uint32_t (&q)[D], uint32_t tail, const uint32_t *xs, int mstride,
+                                               float (&acc)[MB]) {
+        uint32_t v[GS / 2];
+        unpack(q, tail, v);
 #pragma unroll
-            for (int m = 0; m < MB; ++m) {
-                const uint32_t *xp = xs + m * mstride;
-                const u32x4_t x0 = *reinterpret_cast<const u32x4_t *>(xp);
-                const u32x4_t x1 = *reinterpret_cast<const u32x4_t *>(xp + 4);
-                const u32x4_t x2 = *reinterpret_cast<const u32x4_t *>(xp + 8);
-                const uint32_t xv[12] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w, x2.x, x2.y, x2.z, x2.w};
+        for (int m = 0; m < MB; ++m) {
 #pragma unroll
-                for (int i = 0; i < 12; ++i) acc[m] = dot2h(v[i], xv[i], acc[m]);
+            for (int c = 0; c < GS / 8; ++c) {
+                const u32x4_t x = *reinterpret_cast<const u32x4_t *>(xs + m * mstride + 4 * c);
+                acc[m] = dot2h(v[4 * c], x.x, acc[m]);
+                acc[m] = dot2h(v[4 * c + 1], x.y, acc[m]);
+                acc[m] = dot2h(v[4 * c + 2], x.z, acc[m]);
+                acc[m] = dot2h(v[4 * c + 3], x.w, acc[m]);
             }
+        }
+    }
+};
+
+// Natural-order unit of any (bits <= 8, even groupsize): ceil(GS * BITS / 32) dwords, code i at bit i * BITS.
+// unpack() yields the same (1024 + code) fp16 pairs as the paired units (offset class 0 throughout), padded
+// with zero codes up to a multiple of 8 weights.
+template <int BITS, int GS>
+struct GenericUnit {
+    static constexpr int D = (GS * BITS + 31) / 32;
+    static constexpr bool TAIL = false;
+    static constexpr int GROUP = GS, NPAIR = ((GS + 7) / 8) * 4, CBITS = 0;
+    __device__ static __forceinline__ constexpr int cls(int) { return 0; }
+    __device__ static __forceinline__ uint32_t code(const uint32_t (&q)[D], int i) {
+        const int bit = i * BITS, wi = bit >> 5, sh = bit & 31;
+        uint32_t c = q[wi] >> sh;
+        if (sh + BITS > 32) c |= q[wi + 1] << (32 - sh);
+        return c & ((1u << BITS) - 1u);
+    }
+    __device__ static __forceinline__ void unpack(const uint32_t (&q)[D], uint32_t, uint32_t (&v)[NPAIR]) {
+#pragma unroll
+        for (int p = 0; p < NPAIR; ++p) {
+            uint32_t pr = kMagicH2;
+            if (2 * p < GS) pr |= code(q, 2 * p);
+            if (2 * p + 1 < GS) pr |= code(q, 2 * p + 1) << 16;
+            v[p] = pr;
         }
     }
 };

@@ -84,3 +84,79 @@ def nepq1_blob(seed, label, out, K, banks=16, experts=1):
                        rng.integers(0, 2, (experts, out, ng), dtype=np.uint8),
                        rng.integers(0, banks, (experts, out, nsuper), dtype=np.uint8))
     return label, blob
+
+
+# ---- timing-only weights -------------------------------------------------------------------------
+# Tensors too large to push through the CPU quantizer for a benchmark (hundreds of experts, whole
+# linear stacks) are drawn directly in the device layout: uniformly random code / sub-scale bytes and
+# constant anchors.  Every byte pattern is a valid payload, the kernels do the same work as on real
+# weights, and byte counts are those of the format; the values mean nothing, so these are for
+# throughput runs only -- parity is tested on quantized and packed-domain fixtures.
+def random_nint_weight(seed, out, K, bits, gs, sub_bits, device="cuda", anchor=1e-6):
+    import ctypes as C
+
+    import torch
+
+    from . import _lib as L
+    from .runtime import NintWeight
+
+    desc = L.NintDesc()
+    L.check(L.lib().mfq_hip_nint_plan(bits, sub_bits, gs, out, K, C.byref(desc)))
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    total = int(desc.total_bytes)
+    data = torch.empty(total, dtype=torch.uint8, device=device)
+    body = int(desc.anchors_off)
+    # int32 draws fill four bytes at a time (the body is a whole number of dwords)
+    data[:body].view(torch.int32).random_(-2 ** 31, 2 ** 31 - 1, generator=g)
+    data[body:].view(torch.float32).fill_(anchor)
+    return NintWeight(desc, data, (out, K))
+
+
+def random_nint_moe(seed, n_experts, out_per_expert, K, expert_bits, device="cuda"):
+    """NintMoeWeight whose expert e has bit width expert_bits[e] (cohorts by MOE_PROFILES)."""
+    from .runtime_moe import NintMoeWeight
+
+    expert_bits = np.asarray(expert_bits)
+    pools, ids = [], []
+    for b in sorted(set(int(v) for v in expert_bits)):
+        members = np.nonzero(expert_bits == b)[0].astype(np.int32)
+        bits, gs, sb = MOE_PROFILES[b]
+        pools.append(random_nint_weight(seed * 16 + b, len(members) * out_per_expert, K, bits, gs, sb, device))
+        ids.append(members)
+    return NintMoeWeight(n_experts, out_per_expert, K, pools, ids, device)
+
+
+def tile_rows(w, out):
+    """Timing-only: an [out, K] NVQ / dense NEPQ weight whose rows repeat those of the smaller weight `w`
+    (built from a real packed payload).  Device layout = row-block bodies | tables | fp32 anchors."""
+    import copy
+    import ctypes as C
+
+    import torch
+
+    from . import _lib as L
+
+    small = w.desc
+    rows = small.out if hasattr(small, "out") else small.rows
+    if rows % 16 or out % rows:
+        raise ValueError("tile_rows needs a source of a multiple of 16 rows that divides the target")
+    if isinstance(small, L.NvqDesc):
+        big = L.NvqDesc()
+        L.check(L.lib().mfq_hip_nvq_plan(small.index_bits, small.banks, out, small.neuron_len, C.byref(big)))
+    else:
+        big = L.NepqDesc()
+        L.check(L.lib().mfq_hip_nepq_plan(small.profile, small.banks, out, small.neuron_len, C.byref(big)))
+    reps = out // rows
+    data = torch.empty(int(big.total_bytes), dtype=torch.uint8, device=w.data.device)
+    data[: big.tables_off] = w.data[: small.tables_off].repeat(reps)
+    ntab = small.anchors_off - small.tables_off
+    data[big.tables_off: big.tables_off + ntab] = w.data[small.tables_off: small.anchors_off]
+    data[big.anchors_off:] = w.data[small.anchors_off:].repeat(reps)
+    t = copy.copy(w)
+    t.desc, t.data = big, data
+    t.out = out
+    if hasattr(t, "out_per_expert"):
+        t.out_per_expert = out
+    t._ws = type(w._ws)()
+    return t
