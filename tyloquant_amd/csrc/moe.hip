@@ -5,6 +5,7 @@
 #include "common.hpp"
 #include "gemv_common.hpp"
 #include "nint_body.hpp"
+#include "nint_mfma.hpp"
 
 namespace mfq {
 
@@ -175,8 +176,28 @@ struct MoePools {
     int n;
 };
 
-// A tile is up to MB (token, route) pairs of one expert.  Without a route map every pair is its
-// own tile (MB = 1, decode); with one, tile t of the map holds pairs ids_dst[lo .. lo+MB).
+constexpr int kMoeTileM = 16;  // (token, route) pairs of one expert per tile of the route map
+
+// One cohort dispatch of the vector-ALU path: MB pairs of one expert, one 16-neuron row-block.
+template <int XF16, int MB>
+__device__ __forceinline__ void moe_valu_chunk(const NintK &k, const uint8_t *w, int rb, int row_base, int out_per_expert,
+                                               const uint16_t *const (&xr)[MB], float *const (&yr)[MB], int spw,
+                                               uint32_t *lds) {
+#define MFQ_MOE_CASE(B, G)                                                                                    \
+    if (k.bits == B && k.gs == G) {                                                                           \
+        nint_paired_body<B, G, XF16, MB>(k, w, rb, 1, row_base, out_per_expert, xr, yr, spw, lds);            \
+        return;                                                                                               \
+    }
+    if (k.kind == 1) {
+        MFQ_MOE_CASE(4, 24) MFQ_MOE_CASE(3, 24) MFQ_MOE_CASE(2, 16) MFQ_MOE_CASE(4, 32) MFQ_MOE_CASE(4, 16)
+        MFQ_MOE_CASE(4, 48) MFQ_MOE_CASE(2, 32)
+    }
+#undef MFQ_MOE_CASE
+    nint_generic_body<XF16, MB>(k, w, rb, row_base, out_per_expert, xr, yr, spw, lds);
+}
+
+// Vector-ALU path (any NINT profile, any K).  Without a route map every pair is its own tile (MB = 1,
+// decode); with one, tile t holds pairs ids_dst[lo .. lo + kMoeTileM), taken MB at a time.
 template <int XF16, int MB>
 __global__ __launch_bounds__(1024) void moe_grouped_kernel(MoePools P, const int32_t *__restrict__ expert_pool,
                                                            const int32_t *__restrict__ expert_local, int E,
@@ -189,54 +210,114 @@ __global__ __launch_bounds__(1024) void moe_grouped_kernel(MoePools P, const int
                                                            float *__restrict__ out, int64_t ldo) {
     extern __shared__ uint32_t lds[];
     const int tile = blockIdx.x;
-    int e;
-    int pairs[MB];
+    int e, lo = 0, hi = 0;
     if (ids_dst == nullptr) {
         e = ids[tile];
-        pairs[0] = tile;
-#pragma unroll
-        for (int m = 1; m < MB; ++m) pairs[m] = -1;
     } else {
         if (tile >= tile_bounds[E]) return;
         e = tile_experts[tile];
-        const int lo = expert_bounds[e] + (tile - tile_bounds[e]) * MB, hi = expert_bounds[e + 1];
-#pragma unroll
-        for (int m = 0; m < MB; ++m) pairs[m] = lo + m < hi ? ids_dst[lo + m] : -1;
-    }
-    const uint16_t *xr[MB];
-    float *yr[MB];
-#pragma unroll
-    for (int m = 0; m < MB; ++m) {
-        const int p = pairs[m];
-        xr[m] = p >= 0 ? x + static_cast<int64_t>(routed_input ? p : p / R) * ldx : nullptr;
-        yr[m] = p >= 0 ? out + static_cast<int64_t>(p) * ldo : nullptr;
+        lo = expert_bounds[e] + (tile - tile_bounds[e]) * kMoeTileM;
+        hi = min(expert_bounds[e + 1], lo + kMoeTileM);
     }
     const int rbl = blockIdx.y;  // row-block inside the expert
-    if (e < 0 || e >= E || expert_pool[e] < 0) {  // invalid expert id: defined as a zero row
-        const int row = rbl * 16 + (threadIdx.x & 15);
-        if (threadIdx.x < 16 && row < out_per_expert)
+    const bool valid = e >= 0 && e < E && expert_pool[e] >= 0;
+    for (int c = 0; c == 0 || lo + c < hi; c += MB) {
+        int pairs[MB];
 #pragma unroll
-            for (int m = 0; m < MB; ++m)
-                if (yr[m]) yr[m][row] = 0.f;
+        for (int m = 0; m < MB; ++m) pairs[m] = ids_dst ? (lo + c + m < hi ? ids_dst[lo + c + m] : -1) : (m == 0 ? tile : -1);
+        const uint16_t *xr[MB];
+        float *yr[MB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            const int p = pairs[m];
+            xr[m] = p >= 0 ? x + static_cast<int64_t>(routed_input ? p : p / R) * ldx : nullptr;
+            yr[m] = p >= 0 ? out + static_cast<int64_t>(p) * ldo : nullptr;
+        }
+        if (!valid) {  // invalid expert id: defined as a zero row
+            const int row = rbl * 16 + (threadIdx.x & 15);
+            if (threadIdx.x < 16 && row < out_per_expert)
+#pragma unroll
+                for (int m = 0; m < MB; ++m)
+                    if (yr[m]) yr[m][row] = 0.f;
+            return;
+        }
+        const int pool = expert_pool[e];
+        const int row_base = expert_local[e] * out_per_expert;
+        moe_valu_chunk<XF16, MB>(P.k[pool], P.w[pool], row_base / 16 + rbl, row_base, out_per_expert, xr, yr, P.spw[pool],
+                                 lds);
+        __syncthreads();  // the next chunk reuses the reduction area
+    }
+}
+
+// Matrix-core path: a tile of up to 16 pairs of one expert against NB row-blocks, weights streamed once
+// per tile (nint_mfma_body).  Needs K % 8 == 0, 16-byte aligned activation rows and cohorts with an MFMA
+// unit; P.spw holds the steps per wave of each cohort.
+template <int XF16, int NB>
+__global__ __launch_bounds__(512) void moe_mfma_kernel(MoePools P, const int32_t *__restrict__ expert_pool,
+                                                       const int32_t *__restrict__ expert_local, int E,
+                                                       int out_per_expert, const uint16_t *__restrict__ x, int64_t ldx,
+                                                       int routed_input, const int32_t *__restrict__ ids, int n_pairs,
+                                                       int R, const int32_t *__restrict__ ids_dst,
+                                                       const int32_t *__restrict__ expert_bounds,
+                                                       const int32_t *__restrict__ tile_bounds,
+                                                       const int32_t *__restrict__ tile_experts,
+                                                       float *__restrict__ out, int64_t ldo) {
+    extern __shared__ uint32_t lds[];
+    float *red = reinterpret_cast<float *>(lds);
+    const int tile = blockIdx.x;
+    int e, lo = 0, hi = 0;
+    if (ids_dst == nullptr) {
+        e = ids[tile];
+    } else {
+        if (tile >= tile_bounds[E]) return;
+        e = tile_experts[tile];
+        lo = expert_bounds[e] + (tile - tile_bounds[e]) * kMoeTileM;
+        hi = min(expert_bounds[e + 1], lo + kMoeTileM);
+    }
+    const int rbe = out_per_expert / 16, rbl0 = blockIdx.y * NB;
+    auto pair_of = [&](int slot) -> int {  // -1 = empty slot
+        if (ids_dst == nullptr) return slot == 0 ? tile : -1;
+        return lo + slot < hi ? ids_dst[lo + slot] : -1;
+    };
+    if (e < 0 || e >= E || expert_pool[e] < 0) {  // invalid expert id: defined as a zero row (unmapped tiles only)
+        const int p = pair_of(0);
+        for (int c = threadIdx.x; c < min(NB, rbe - rbl0) * 16; c += blockDim.x)
+            if (p >= 0) out[static_cast<int64_t>(p) * ldo + rbl0 * 16 + c] = 0.f;
         return;
     }
     const int pool = expert_pool[e];
-    const int row_base = expert_local[e] * out_per_expert;
-    const int rb = row_base / 16 + rbl;
+    const int rb_first = expert_local[e] * rbe;
+    int p = pair_of(threadIdx.x & 15);
+    if (p < 0) p = pair_of(0);
+    const uint16_t *xrow = x + static_cast<int64_t>(routed_input ? p : p / R) * ldx;
     const NintK &k = P.k[pool];
     const uint8_t *w = P.w[pool];
     const int spw = P.spw[pool];
-#define MFQ_MOE_CASE(B, G)                                                                                    \
-    if (k.bits == B && k.gs == G) {                                                                           \
-        nint_paired_body<B, G, XF16, MB>(k, w, rb, 1, row_base, out_per_expert, xr, yr, spw, lds);            \
-        return;                                                                                               \
-    }
+#define MFQ_MOE_MFMA(UNIT, B, G) \
+    if (k.bits == B && k.gs == G) nint_mfma_body<UNIT<B, G>, XF16, NB>(k, w, rb_first + rbl0, rb_first + rbe, xrow, spw, red);
     if (k.kind == 1) {
-        MFQ_MOE_CASE(4, 24) MFQ_MOE_CASE(3, 24) MFQ_MOE_CASE(2, 16) MFQ_MOE_CASE(4, 32) MFQ_MOE_CASE(4, 16)
-        MFQ_MOE_CASE(4, 48) MFQ_MOE_CASE(2, 32)
+        MFQ_MOE_MFMA(PairedUnit, 4, 24)
+        else MFQ_MOE_MFMA(PairedUnit, 3, 24)
+        else MFQ_MOE_MFMA(PairedUnit, 2, 16)
+        else MFQ_MOE_MFMA(PairedUnit, 4, 32)
+        else MFQ_MOE_MFMA(PairedUnit, 4, 16)
+        else MFQ_MOE_MFMA(PairedUnit, 4, 48)
+        else MFQ_MOE_MFMA(PairedUnit, 2, 32)
+    } else {
+        MFQ_MOE_MFMA(GenericUnit, 5, 28)
     }
-#undef MFQ_MOE_CASE
-    nint_generic_body<XF16, MB>(k, w, rb, row_base, out_per_expert, xr, yr, spw, lds);
+#undef MFQ_MOE_MFMA
+    __syncthreads();
+    const int nwaves = blockDim.x >> 6;
+    for (int o = threadIdx.x; o < NB * 256; o += blockDim.x) {
+        const int rr = o & 15, t = (o >> 4) & 15, nb = o >> 8;
+        const int pt = pair_of(t);
+        if (pt < 0 || rbl0 + nb >= rbe) continue;
+        const int slot = (nb * 4 + (t & 3)) * 64 + rr + 16 * (t >> 2);
+        float s = 0.f;
+        for (int wv = 0; wv < nwaves; ++wv) s += red[wv * NB * 256 + slot];
+        out[static_cast<int64_t>(pt) * ldo + (rbl0 + nb) * 16 + rr] = s;
+    }
 }
 
 // rows of pairs whose expert id is out of range are not in any tile of the map: clear them
@@ -313,7 +394,6 @@ extern "C" int mfq_hip_moe_route_map(const int32_t *ids, int n_pairs, int E, int
 }
 
 // the grouped kernel batches this many routes of one expert per block
-static constexpr int kMoeTileM = 4;
 
 extern "C" int mfq_hip_moe_tile_m(void) { return kMoeTileM; }
 
@@ -333,18 +413,55 @@ extern "C" int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools
     MFQ_REQUIRE(ldx >= K && ldo >= out_per_expert, MFQ_ERR_INVALID, "moe_grouped_matmul: ldx/ldo smaller than the tensor");
     const int n_pairs = T * R;
     const bool mapped = ids_dst != nullptr;
-    const int mb = mapped ? kMoeTileM : 1;
+    if (mapped)
+        MFQ_REQUIRE(expert_bounds && tile_bounds && tile_experts, MFQ_ERR_INVALID,
+                    "moe_grouped_matmul: route map without its bounds / tile tables");
     MoePools P;
     P.n = n_pools;
-    // one block shape for every cohort: waves = min(16, fewest steps that keeps every wave busy)
     int max_steps = 1;
+    bool mfma = K >= 8 && K % 8 == 0 && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
     for (int i = 0; i < n_pools; ++i) {
-        MFQ_REQUIRE(pools[i].desc.neuron_len == K && pools[i].weight, MFQ_ERR_INVALID,
-                    "moe_grouped_matmul: cohort %d has neuron_len %d, expected %d", i, pools[i].desc.neuron_len, K);
-        if (pools[i].desc.nsteps > max_steps) max_steps = pools[i].desc.nsteps;
+        const mfq_nint_desc &d = pools[i].desc;
+        MFQ_REQUIRE(d.neuron_len == K && pools[i].weight, MFQ_ERR_INVALID,
+                    "moe_grouped_matmul: cohort %d has neuron_len %d, expected %d", i, d.neuron_len, K);
+        if (d.nsteps > max_steps) max_steps = d.nsteps;
+        NintK &k = P.k[i];
+        k.bits = d.bits; k.sub_bits = d.sub_bits; k.gs = d.gs; k.out = d.out; k.neuron_len = d.neuron_len; k.ng = d.ng;
+        k.kind = d.kind; k.dwords = d.dwords; k.tail = d.tail_bytes; k.nsteps = d.nsteps; k.n_rowblocks = d.n_rowblocks;
+        k.step_bytes = d.step_bytes; k.rowblock_bytes = d.rowblock_bytes; k.anchors_off = d.anchors_off;
+        P.w[i] = static_cast<const uint8_t *>(pools[i].weight);
+        mfma = mfma && (d.kind == 1 || (d.bits == 5 && d.gs == 28)) && 4 * d.rowblock_bytes < (1ll << 31);
     }
     const int rbe = out_per_expert / 16;
-    const int64_t tiles = mapped ? ceil_div(n_pairs, mb) + E : n_pairs;
+    const int64_t tiles = mapped ? ceil_div(n_pairs, kMoeTileM) + E : n_pairs;
+    hipStream_t st = as_stream(stream);
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    if (mapped)
+        hipLaunchKernelGGL(moe_zero_invalid_kernel, dim3(n_pairs), dim3(256), 0, st, ids, n_pairs, E, expert_pool,
+                           out_per_expert, out, ldo);
+#define MFQ_MOE_LAUNCH(KERNEL, GRID, BLOCK, LDS)                                                                      \
+    hipLaunchKernelGGL(KERNEL, GRID, BLOCK, LDS, st, P, expert_pool, expert_local, E, out_per_expert, xp, ldx,      \
+                       routed_input, ids, n_pairs, R, ids_dst, expert_bounds, tile_bounds, tile_experts, out, ldo)
+    if (mfma) {
+        // row-blocks per wave: 4 while the grid still has a few thousand waves, else 1
+        const int64_t live_tiles = mapped ? ceil_div(n_pairs, kMoeTileM) : n_pairs;
+        const bool nb4 = live_tiles * rbe * max_steps >= 4 * 2048 && rbe >= 4;
+        const int nb = nb4 ? 4 : 1;
+        int nwaves = max_steps < 8 ? max_steps : 8;
+        for (int i = 0; i < n_pools; ++i) P.spw[i] = static_cast<int>(ceil_div(P.k[i].nsteps, nwaves));
+        const size_t lds = static_cast<size_t>(nwaves) * nb * 1024;
+        const dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(ceil_div(rbe, nb))), block(64 * nwaves);
+        if (x_dtype == MFQ_X_F16) {
+            if (nb4) MFQ_MOE_LAUNCH((moe_mfma_kernel<1, 4>), grid, block, lds);
+            else MFQ_MOE_LAUNCH((moe_mfma_kernel<1, 1>), grid, block, lds);
+        } else {
+            if (nb4) MFQ_MOE_LAUNCH((moe_mfma_kernel<0, 4>), grid, block, lds);
+            else MFQ_MOE_LAUNCH((moe_mfma_kernel<0, 1>), grid, block, lds);
+        }
+        return check_launch("moe_grouped_matmul");
+    }
+    // vector-ALU path: one block shape for every cohort, waves = min(16, fewest steps that keeps every wave busy)
+    const int mb = mapped ? 4 : 1;
     int want = static_cast<int>(ceil_div(8192, static_cast<int64_t>(rbe) * (mapped ? ceil_div(n_pairs, mb) : n_pairs)));
     if (want < 1) want = 1;
     if (want > 16) want = 16;
@@ -352,42 +469,20 @@ extern "C" int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools
     const int nwaves = want;
     size_t lds = 0;
     for (int i = 0; i < n_pools; ++i) {
-        const mfq_nint_desc &d = pools[i].desc;
-        NintK &k = P.k[i];
-        k.bits = d.bits; k.sub_bits = d.sub_bits; k.gs = d.gs; k.out = d.out; k.neuron_len = d.neuron_len; k.ng = d.ng;
-        k.kind = d.kind; k.dwords = d.dwords; k.tail = d.tail_bytes; k.nsteps = d.nsteps; k.n_rowblocks = d.n_rowblocks;
-        k.step_bytes = d.step_bytes; k.rowblock_bytes = d.rowblock_bytes; k.anchors_off = d.anchors_off;
-        P.w[i] = static_cast<const uint8_t *>(pools[i].weight);
-        P.spw[i] = static_cast<int>(ceil_div(d.nsteps, nwaves));
-        const size_t need = gemv_lds_bytes(mb, P.spw[i], d.gs, nwaves);
+        P.spw[i] = static_cast<int>(ceil_div(P.k[i].nsteps, nwaves));
+        const size_t need = gemv_lds_bytes(mb, P.spw[i], P.k[i].gs, nwaves);
         if (need > lds) lds = need;
     }
     MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "moe_grouped_matmul: K=%d needs %zu bytes of LDS", K, lds);
-    hipStream_t st = as_stream(stream);
     const dim3 grid(static_cast<unsigned>(tiles), rbe), block(64 * nwaves);
-    const uint16_t *xp = static_cast<const uint16_t *>(x);
     if (mapped) {
-        MFQ_REQUIRE(expert_bounds && tile_bounds && tile_experts, MFQ_ERR_INVALID,
-                    "moe_grouped_matmul: route map without its bounds / tile tables");
-        hipLaunchKernelGGL(moe_zero_invalid_kernel, dim3(n_pairs), dim3(256), 0, st, ids, n_pairs, E, expert_pool,
-                           out_per_expert, out, ldo);
-        if (x_dtype == MFQ_X_F16)
-            hipLaunchKernelGGL((moe_grouped_kernel<1, kMoeTileM>), grid, block, lds, st, P, expert_pool, expert_local, E,
-                               out_per_expert, xp, ldx, routed_input, ids, n_pairs, R, ids_dst, expert_bounds, tile_bounds,
-                               tile_experts, out, ldo);
-        else
-            hipLaunchKernelGGL((moe_grouped_kernel<0, kMoeTileM>), grid, block, lds, st, P, expert_pool, expert_local, E,
-                               out_per_expert, xp, ldx, routed_input, ids, n_pairs, R, ids_dst, expert_bounds, tile_bounds,
-                               tile_experts, out, ldo);
+        if (x_dtype == MFQ_X_F16) MFQ_MOE_LAUNCH((moe_grouped_kernel<1, 4>), grid, block, lds);
+        else MFQ_MOE_LAUNCH((moe_grouped_kernel<0, 4>), grid, block, lds);
     } else {
-        const int32_t *np = nullptr;
-        if (x_dtype == MFQ_X_F16)
-            hipLaunchKernelGGL((moe_grouped_kernel<1, 1>), grid, block, lds, st, P, expert_pool, expert_local, E,
-                               out_per_expert, xp, ldx, routed_input, ids, n_pairs, R, np, np, np, np, out, ldo);
-        else
-            hipLaunchKernelGGL((moe_grouped_kernel<0, 1>), grid, block, lds, st, P, expert_pool, expert_local, E,
-                               out_per_expert, xp, ldx, routed_input, ids, n_pairs, R, np, np, np, np, out, ldo);
+        if (x_dtype == MFQ_X_F16) MFQ_MOE_LAUNCH((moe_grouped_kernel<1, 1>), grid, block, lds);
+        else MFQ_MOE_LAUNCH((moe_grouped_kernel<0, 1>), grid, block, lds);
     }
+#undef MFQ_MOE_LAUNCH
     return check_launch("moe_grouped_matmul");
 }
 
