@@ -168,6 +168,7 @@ void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&x
 int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                   int64_t ldy, hipStream_t st);
 int nint_dequant_f16(const mfq_nint_desc *d, const void *weight, void *w16, int64_t ld, float *rowscale, hipStream_t st);
+bool nint_stream_capable(const mfq_nint_desc *d);
 
 }  // namespace mfq
 
@@ -182,11 +183,16 @@ extern "C" int mfq_hip_gemm_f16_nt(const void *a, int64_t lda, const void *b, in
     return gemm_f16_nt(a, lda, b, ldb, M, N, K, nullptr, nullptr, y, ldy, as_stream(stream));
 }
 
-// Below this many activation rows the weight stream dominates and the GEMV kernels win.
-static constexpr int kGemvMaxM = 8;
+// Up to kGemvMaxM activation rows the weight stream dominates and the GEMV kernels win; tensors with a
+// matrix-core streaming kernel (16 rows per pass over the packed weights) stay on it up to kStreamMaxM rows,
+// where re-streaming the weights is still cheaper than dequantizing them to fp16 once.
+static constexpr int kGemvMaxM = 8, kStreamMaxM = 256;
+static bool nint_streams(const mfq_nint_desc *d, int M) {
+    return M <= kGemvMaxM || (M <= kStreamMaxM && nint_stream_capable(d));
+}
 
 extern "C" size_t mfq_hip_nint_gemm_workspace_bytes(const mfq_nint_desc *d, int M) {
-    if (!d || M <= kGemvMaxM) return 0;
+    if (!d || nint_streams(d, M)) return 0;
     return dequant_gemm_workspace(d->out, d->neuron_len, M);
 }
 
@@ -198,7 +204,7 @@ extern "C" int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, con
     MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint_gemm: x_dtype=%d", x_dtype);
     MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nint_gemm: ldx/ldy smaller than the tensor");
     hipStream_t st = as_stream(stream);
-    if (M <= kGemvMaxM) return nint_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, st);
+    if (nint_streams(d, M)) return nint_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, st);
     const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
     MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nint_gemm: workspace %zu < %zu bytes",
                 workspace_bytes, need);

@@ -250,6 +250,12 @@ static bool mfma_eligible(const NintK &k, const void *x, int64_t ldx) {
            (reinterpret_cast<uintptr_t>(x) & 15) == 0 && 4 * k.rowblock_bytes < (1ll << 31);
 }
 
+bool nint_stream_capable(const mfq_nint_desc *d) {
+    const NintK k = to_k(d);
+    return (k.kind == 1 || mfma_generic_profile(k)) && k.neuron_len >= 8 && k.neuron_len % 8 == 0 &&
+           4 * k.rowblock_bytes < (1ll << 31);
+}
+
 template <int XF16, int NB>
 static int launch_mfma_nb(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                           hipStream_t st) {
