@@ -38,6 +38,22 @@ def test_nvq_jsc_dequant_bit_exact_and_gemv(codebook, banks, out, K):
     _check(lin(x).cpu().numpy(), O.linear_forward_f64(want, xf))
 
 
+@pytest.mark.parametrize("out,K,M", [(48, 2048, 1), (40, 4104, 16), (130, 1024, 33), (64, 5120, 8)])
+def test_nvq_matrix_core_path_multi_step(out, K, M):
+    """K % 8 == 0 rows take the MFMA streaming kernel: several steps per neuron, K split over waves, ragged last
+    group, more rows than one 16-row tile, a row stride above K."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import nvq_matmul
+    rng = np.random.default_rng(70 + out + M)
+    t = synth.nvq_jsc_random(rng, out, K, "d4_512", 2)
+    dtype, blob = O.pack_tensor(t)
+    lin = R.load_quant_linear(dtype, blob)
+    want = O.dequantize_nvq_jsc(O.unpack_nvq(blob))
+    xw = torch.from_numpy(rng.standard_normal((M, K + 16)).astype(np.float32)).to(torch.bfloat16).cuda()
+    x = xw[:, :K]
+    _check(nvq_matmul(lin.weight, x, force="gemv").cpu().numpy(), O.linear_forward_f64(want, x.float().cpu().numpy()))
+
+
 def test_nvq_payload_sizes_match_reference_identities():
     """tests/test_formats/test_nvq.py:44-50 and tests/test_nvq_kernels_cuda.py:410-449 (host side)."""
     from tyloquant_amd import _lib as L

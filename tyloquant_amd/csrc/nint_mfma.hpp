@@ -48,6 +48,23 @@ __device__ __forceinline__ float4_t mfma16(u32x4_t a, u32x4_t b, float4_t c) {
                                                   0);
 }
 
+// Adds the waves' partial tiles left in `red` (layout of nint_mfma_body) after a block barrier and stores
+// y[m0 + token][rb0 * 16 + neuron] for the tokens below M and the neurons below out_rows.
+template <int NB>
+__device__ __forceinline__ void mfma_store_dense(const float *red, int rb0, int m0, int M, int out_rows,
+                                                 float *__restrict__ y, int64_t ldy) {
+    __syncthreads();
+    const int nwaves = blockDim.x >> 6;
+    for (int o = threadIdx.x; o < NB * 256; o += blockDim.x) {
+        const int rr = o & 15, t = (o >> 4) & 15, nb = o >> 8;
+        const int slot = (nb * 4 + (t & 3)) * 64 + rr + 16 * (t >> 2);
+        float s = 0.f;
+        for (int wv = 0; wv < nwaves; ++wv) s += red[wv * NB * 256 + slot];
+        const int row = (rb0 + nb) * 16 + rr;
+        if (m0 + t < M && row < out_rows) y[static_cast<int64_t>(m0 + t) * ldy + row] = s;
+    }
+}
+
 // Block = the row-blocks [rb0, min(rb0 + NB, rb_end)); its waves split the K steps (spw each).  xrow: the
 // activation row of token (lane & 15) of this 16-token tile (any valid row for an absent token).
 // Leaves, in `red`, the wave's partial results: red[((wave * NB + nb) * 4 + v) * 64 + lane] =
@@ -157,19 +174,10 @@ __global__ __launch_bounds__(512) void nint_mfma_kernel(NintK k, const uint8_t *
                                                          float *__restrict__ y, int64_t ldy, int spw) {
     extern __shared__ uint32_t lds[];
     float *red = reinterpret_cast<float *>(lds);
-    const int nwaves = blockDim.x >> 6;
     const int rb0 = blockIdx.x * NB, m0 = blockIdx.y * 16;
     const int tok = min(m0 + static_cast<int>(threadIdx.x & 15), M - 1);
     nint_mfma_body<U, XF16, NB>(k, w, rb0, k.n_rowblocks, x + static_cast<int64_t>(tok) * ldx, spw, red);
-    __syncthreads();
-    for (int o = threadIdx.x; o < NB * 256; o += blockDim.x) {
-        const int rr = o & 15, t = (o >> 4) & 15, nb = o >> 8;
-        const int slot = (nb * 4 + (t & 3)) * 64 + rr + 16 * (t >> 2);
-        float s = 0.f;
-        for (int wv = 0; wv < nwaves; ++wv) s += red[wv * NB * 256 + slot];
-        const int row = (rb0 + nb) * 16 + rr;
-        if (m0 + t < M && row < k.out) y[static_cast<int64_t>(m0 + t) * ldy + row] = s;
-    }
+    mfma_store_dense<NB>(red, rb0, m0, M, k.out, y, ldy);
 }
 
 }  // namespace mfq

@@ -12,6 +12,7 @@
 // expands a sign mask (with its parity bit) into XOR masks, and the scale LUT all stay in LDS.
 #include "common.hpp"
 #include "gemv_common.hpp"
+#include "nint_mfma.hpp"
 
 namespace mfq {
 
@@ -267,6 +268,145 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
     finish_rows<MB>(v, red, wave, nwaves, lane, rb, 0, k.out, yr);
 }
 
+// ---- matrix-core path: up to 16 activation rows per streamed pass ----------------------------------
+// Same scheme as the NINT kernel (nint_mfma.hpp): lane (r, kb) holds the unit of group 4j + kb of neuron r,
+// fragment m of a unit is its weights 8m .. 8m+7 = two codebook vectors and one sign mask.  The magnitudes
+// come from LDS as fp16 pairs, get their sign bits XOR-ed in and are multiplied by the group's scale-LUT
+// entry in fp16 (one rounding of mag * lut, relative error below 2^-12); the neuron anchor is applied to
+// the fp32 accumulator.  Codes of padding groups are zero (not zero weights), so the activation fragments
+// read as zero at and beyond K.
+// LDS map (dwords): [codebook pairs: banks*entries*2][sign xor table: 512][lut pairs: 16][bank offset: 16][red]
+template <int XF16, int NB>
+__global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__restrict__ w,
+                                                       const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                       float *__restrict__ y, int64_t ldy, int spw) {
+    extern __shared__ uint32_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ncb = k.banks * k.entries;
+    uint32_t *cbp = lds;
+    uint32_t *sgx = cbp + 2 * ncb;
+    uint32_t *luth = sgx + 512;
+    uint32_t *bankoff = luth + 16;
+    float *red = reinterpret_cast<float *>(bankoff + 16);
+    {
+        const float *lut = reinterpret_cast<const float *>(w + k.tables_off);
+        const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+        const uint32_t *cb = bfs + 16;  // 4 int8 magnitudes per entry
+        for (int i = tid; i < ncb; i += blockDim.x) {
+            const uint32_t e = cb[i];
+            uint32_t h[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) h[t] = f32_to_f16_rne(static_cast<float>((e >> (8 * t)) & 0xffu));
+            cbp[2 * i] = h[0] | (h[1] << 16);
+            cbp[2 * i + 1] = h[2] | (h[3] << 16);
+        }
+        for (int i = tid; i < 128; i += blockDim.x) {
+            const uint32_t m8 = parity8(i);
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+                sgx[4 * i + p] = (((m8 >> (2 * p)) & 1u) << 15) | (((m8 >> (2 * p + 1)) & 1u) << 31);
+        }
+        if (tid < 16) {
+            const uint32_t h = f32_to_f16_rne(lut[tid]);  // the LUT is fp16 in the payload: exact
+            luth[tid] = h | (h << 16);
+            bankoff[tid] = bfs[tid] * k.entries * 2;
+        }
+    }
+    const int rb0 = blockIdx.x * NB, m0 = blockIdx.y * 16;
+    const int tok = min(m0 + (lane & 15), M - 1);
+    const uint16_t *xrow = x + static_cast<int64_t>(tok) * ldx;
+    const int r = lane & 15, kb = lane >> 4;
+    const int s0 = wave * spw;
+    const int n = min(k.nsteps, s0 + spw) - s0;
+    const int nrb = min(NB, k.n_rowblocks - rb0);
+    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
+    float anchor[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+        anchor[i] = reinterpret_cast<const float *>(w + k.anchors_off)[min(rb0 + i, k.n_rowblocks - 1) * 16 + r];
+    const __amdgpu_buffer_rsrc_t win =
+        wave_window(w + static_cast<int64_t>(rb0) * k.rowblock_bytes + static_cast<int64_t>(s0) * sb,
+                    n > 0 ? (nrb - 1) * rbb + n * sb : 0u);
+    float4_t acc[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();  // tables
+
+    const uint32_t ib = static_cast<uint32_t>(k.ib), im = (1u << ib) - 1u;
+    for (int s = 0; s < n; ++s) {
+        u32x2_t q[NB][4], hh[NB];
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            const uint32_t off = i < nrb ? i * rbb + s * sb : kNoStep;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) q[i][j] = __builtin_amdgcn_raw_buffer_load_b64(win, off + (j * 64 + lane) * 8, 0, 2);
+            hh[i] = __builtin_amdgcn_raw_buffer_load_b64(win, off + 2048 + lane * 8, 0, 2);
+        }
+        const int kbase = (s0 + s) * 16 * 24 + kb * 24;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            u32x4_t a[3];
+#pragma unroll
+            for (int m = 0; m < 3; ++m) a[m] = load_xfrag<XF16, true>(xrow, kbase + 4 * j * 24 + 8 * m, k.neuron_len);
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const uint32_t d0 = q[i][j].x, d1 = q[i][j].y;
+                const uint32_t h = ((j < 2 ? hh[i].x : hh[i].y) >> (16 * (j & 1))) & 0xffffu;
+                const uint32_t state = (d1 >> 27) & 15u;
+                const uint32_t *bank = cbp + bankoff[state];
+                const half2_t sc = __builtin_bit_cast(half2_t, luth[state]);
+                const uint32_t mk[3] = {h & 127u, (h >> 7) & 127u, ((d0 >> 27) & 31u) | ((h >> 14) << 5)};
+                const uint32_t ix[6] = {d0 & im, (d0 >> ib) & im, (d0 >> (2 * ib)) & im,
+                                        d1 & im, (d1 >> ib) & im, (d1 >> (2 * ib)) & im};
+#pragma unroll
+                for (int m = 0; m < 3; ++m) {
+                    const u32x4_t sx = *reinterpret_cast<const u32x4_t *>(sgx + 4 * mk[m]);
+                    const u32x2_t c0 = *reinterpret_cast<const u32x2_t *>(bank + 2 * ix[2 * m]);
+                    const u32x2_t c1 = *reinterpret_cast<const u32x2_t *>(bank + 2 * ix[2 * m + 1]);
+                    const uint32_t wv[4] = {c0.x ^ sx.x, c0.y ^ sx.y, c1.x ^ sx.z, c1.y ^ sx.w};
+                    u32x4_t b;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) b[t] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, wv[t]) * sc);
+                    acc[i] = mfma16(a[m], b, acc[i]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[((wave * NB + i) * 4 + v) * 64 + lane] = anchor[i] * acc[i][v];
+    mfma_store_dense<NB>(red, rb0, m0, M, k.out, y, ldy);
+}
+
+static bool nvq_stream_capable(const NvqK &k) {
+    return k.neuron_len >= 8 && k.neuron_len % 8 == 0 && 4 * k.rowblock_bytes < (1ll << 31);
+}
+
+template <int XF16, int NB>
+static int nvq_launch_mfma(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                           hipStream_t st) {
+    const int64_t groups = ceil_div(k.n_rowblocks, NB);
+    int spw = static_cast<int>(ceil_div(k.nsteps, 8));
+    while (spw < k.nsteps && groups * ceil_div(k.nsteps, spw) > 8192) ++spw;
+    const int nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
+    const size_t lds = (static_cast<size_t>(k.banks) * k.entries * 2 + 512 + 32) * 4 + static_cast<size_t>(nwaves) * NB * 1024;
+    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nvq_mfma: %zu bytes of LDS", lds);
+    hipLaunchKernelGGL((nvq_mfma_kernel<XF16, NB>), dim3(static_cast<unsigned>(groups), static_cast<unsigned>(ceil_div(M, 16))),
+                       dim3(64 * nwaves), lds, st, k, w, x, ldx, M, y, ldy, spw);
+    return check_launch("nvq_mfma");
+}
+
+template <int XF16>
+static int nvq_mfma_any(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                        hipStream_t st) {
+    const int64_t items = static_cast<int64_t>(k.n_rowblocks) * k.nsteps;
+    if (items >= 4 * 1536) return nvq_launch_mfma<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
+    if (items >= 2 * 1536) return nvq_launch_mfma<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
+    return nvq_launch_mfma<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
+}
+
 static void nvq_gemv_shape(const NvqK &k, int mb, int &spw, int &nwaves, size_t &lds_bytes) {
     int want = static_cast<int>(ceil_div(3 * gemv_target_waves(), k.n_rowblocks));
     if (want < 1) want = 1;
@@ -294,6 +434,8 @@ static int nvq_gemv_any(const mfq_nvq_desc *d, const void *weight, const void *x
     const NvqK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
+    if (nvq_stream_capable(k) && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
+        return x_dtype == MFQ_X_F16 ? nvq_mfma_any<1>(k, w, xp, ldx, M, y, ldy, st) : nvq_mfma_any<0>(k, w, xp, ldx, M, y, ldy, st);
     int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
     for (;;) {
         int spw, nwaves;
@@ -400,10 +542,15 @@ extern "C" int mfq_hip_nvq_gemv(const mfq_nvq_desc *d, const void *weight, const
     return nvq_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, as_stream(stream));
 }
 
-static constexpr int kNvqGemvMaxM = 13;  // the reference keeps the D4 family on its GEMV up to M = 13
+// The reference keeps the D4 family on its GEMV up to M = 13; tensors the matrix-core streaming kernel
+// takes stay on it up to kNvqStreamMaxM rows.
+static constexpr int kNvqGemvMaxM = 13, kNvqStreamMaxM = 256;
+static bool nvq_streams(const mfq_nvq_desc *d, int M) {
+    return M <= kNvqGemvMaxM || (M <= kNvqStreamMaxM && nvq_stream_capable(to_k(d)));
+}
 
 extern "C" size_t mfq_hip_nvq_gemm_workspace_bytes(const mfq_nvq_desc *d, int M) {
-    if (!d || M <= kNvqGemvMaxM) return 0;
+    if (!d || nvq_streams(d, M)) return 0;
     return dequant_gemm_workspace(d->out, d->neuron_len, M);
 }
 
@@ -414,7 +561,7 @@ extern "C" int mfq_hip_nvq_gemm(const mfq_nvq_desc *d, const void *weight, const
     MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvq_gemm: x_dtype=%d", x_dtype);
     MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nvq_gemm: ldx/ldy smaller than the tensor");
     hipStream_t st = as_stream(stream);
-    if (M <= kNvqGemvMaxM) return nvq_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, st);
+    if (nvq_streams(d, M)) return nvq_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, st);
     const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
     MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nvq_gemm: workspace %zu < %zu bytes",
                 workspace_bytes, need);
