@@ -169,6 +169,10 @@ int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int
                   int64_t ldy, hipStream_t st);
 int nint_dequant_f16(const mfq_nint_desc *d, const void *weight, void *w16, int64_t ld, float *rowscale, hipStream_t st);
 bool nint_stream_capable(const mfq_nint_desc *d);
+bool nint_prefill_capable(const mfq_nint_desc *d);
+size_t nint_prefill_xg_bytes(const mfq_nint_desc *d, int M);
+int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16, int Kp, const float *xscale, uint32_t *xg,
+                 int M, float *y, int64_t ldy, hipStream_t st);
 
 }  // namespace mfq
 
@@ -191,8 +195,15 @@ static bool nint_streams(const mfq_nint_desc *d, int M) {
     return M <= kGemvMaxM || (M <= kStreamMaxM && nint_stream_capable(d));
 }
 
+// prefill workspace: x16 [M, Kp] | xscale [M] | group sums
+static size_t prefill_workspace(const mfq_nint_desc *d, int M) {
+    const size_t Kp = static_cast<size_t>(ceil_div(d->neuron_len, GBK)) * GBK;
+    return align256(static_cast<size_t>(M) * Kp * 2) + align256(static_cast<size_t>(M) * 4) + nint_prefill_xg_bytes(d, M);
+}
+
 extern "C" size_t mfq_hip_nint_gemm_workspace_bytes(const mfq_nint_desc *d, int M) {
     if (!d || nint_streams(d, M)) return 0;
+    if (nint_prefill_capable(d)) return prefill_workspace(d, M);
     return dequant_gemm_workspace(d->out, d->neuron_len, M);
 }
 
@@ -205,6 +216,20 @@ extern "C" int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, con
     MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nint_gemm: ldx/ldy smaller than the tensor");
     hipStream_t st = as_stream(stream);
     if (nint_streams(d, M)) return nint_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, st);
+    if (nint_prefill_capable(d)) {
+        const size_t need = prefill_workspace(d, M);
+        MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nint_gemm: workspace %zu < %zu bytes",
+                    workspace_bytes, need);
+        const int Kp = static_cast<int>(ceil_div(d->neuron_len, GBK)) * GBK;
+        uint8_t *p = static_cast<uint8_t *>(workspace);
+        uint16_t *x16 = reinterpret_cast<uint16_t *>(p);
+        p += align256(static_cast<size_t>(M) * Kp * 2);
+        float *xscale = reinterpret_cast<float *>(p);
+        p += align256(static_cast<size_t>(M) * 4);
+        int rc = x_prep(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, st);
+        if (rc) return rc;
+        return nint_prefill(d, weight, x16, Kp, xscale, reinterpret_cast<uint32_t *>(p), M, y, ldy, st);
+    }
     const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
     MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nint_gemm: workspace %zu < %zu bytes",
                 workspace_bytes, need);

@@ -17,6 +17,7 @@
 #include "gemv_common.hpp"
 #include "nint_body.hpp"
 #include "nint_mfma.hpp"
+#include "nint_prefill.hpp"
 
 namespace mfq {
 
@@ -289,6 +290,35 @@ static int launch_mfma(const NintK &k, const uint8_t *w, const uint16_t *x, int6
     if (items >= 4 * 1536) return launch_mfma_nb<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
     if (items >= 2 * 1536) return launch_mfma_nb<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
     return launch_mfma_nb<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
+}
+
+// ---- prefill: block-tiled MFMA GEMM with in-register dequantization ---------------------------
+bool nint_prefill_capable(const mfq_nint_desc *d) {
+    return d->kind == 1 && d->neuron_len >= 8 && 4 * d->rowblock_bytes < (1ll << 31);
+}
+size_t nint_prefill_xg_bytes(const mfq_nint_desc *d, int M) { return static_cast<size_t>(M) * d->nsteps * 64; }
+
+// x16 [M, Kp] fp16 (rows scaled by 1 / xscale[m], zero beyond K), xg = workspace of nint_prefill_xg_bytes
+int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16, int Kp, const float *xscale,
+                 uint32_t *xg, int M, float *y, int64_t ldy, hipStream_t st) {
+    const NintK k = to_k(d);
+    const uint8_t *w = static_cast<const uint8_t *>(weight);
+    const int64_t nthreads = static_cast<int64_t>(M) * k.nsteps * 4;
+    hipLaunchKernelGGL(x_group_sums_kernel, dim3(static_cast<unsigned>(ceil_div(nthreads, 256))), dim3(256), 0, st, x16, Kp, M,
+                       k.gs, k.nsteps, xg);
+    constexpr int MT = 4, NB = 4;
+    const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, 2 * NB)), static_cast<unsigned>(ceil_div(M, 2 * MT * 16)));
+#define MFQ_PREFILL(B, G)                                                                                      \
+    if (k.bits == B && k.gs == G) {                                                                            \
+        const size_t lds = static_cast<size_t>(2 * MT * 16) * (4 * G + 8) * 2;                                 \
+        hipLaunchKernelGGL((nint_prefill_kernel<PairedUnit<B, G>, MT, NB>), grid, dim3(256), lds, st, k, w, x16, Kp, \
+                           xscale, xg, M, y, ldy);                                                             \
+        return check_launch("nint_prefill");                                                                   \
+    }
+    MFQ_PREFILL(4, 32) MFQ_PREFILL(4, 24) MFQ_PREFILL(4, 16) MFQ_PREFILL(4, 48) MFQ_PREFILL(3, 24) MFQ_PREFILL(2, 16)
+    MFQ_PREFILL(2, 32)
+#undef MFQ_PREFILL
+    return fail(MFQ_ERR_UNSUPPORTED, "nint_prefill: no kernel for NINT%d-%d", k.bits, k.gs);
 }
 
 int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M, float *y,
