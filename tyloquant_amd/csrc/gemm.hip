@@ -21,10 +21,15 @@ int fail(int code, const char *fmt, ...) {
 }
 
 // ---- activation prep: x16[m, k] = fp16(x[m, k] * 2^-f_m), xscale[m] = 2^f_m ---------------
+// With xg != null the block also leaves the row's group sums for the NINT prefill kernel:
+// xg[((m * nsteps + s) * 4 + kb) * 4 + {0,1,2,3}] = fp16 pairs (Xhi_j0, Xhi_j1), (Xhi_j2, Xhi_j3), (Xlo_j0, Xlo_j1),
+// (Xlo_j2, Xlo_j3), X_j = sum of x16[m] over group 16 s + 4 j + kb (gs values), split into two fp16 halves.
 template <int XF16>
 __global__ __launch_bounds__(256) void x_prep_kernel(const uint16_t *__restrict__ x, int64_t ldx, int K, int Kp,
-                                                     uint16_t *__restrict__ x16, float *__restrict__ xscale) {
+                                                     uint16_t *__restrict__ x16, float *__restrict__ xscale, int gs,
+                                                     int nsteps, uint32_t *__restrict__ xg) {
     __shared__ float red[4];
+    __shared__ float gsum[256];
     const int m = blockIdx.x, tid = threadIdx.x;
     const uint16_t *xr = x + static_cast<int64_t>(m) * ldx;
     float amax = 0.f;
@@ -42,6 +47,36 @@ __global__ __launch_bounds__(256) void x_prep_kernel(const uint16_t *__restrict_
     if (tid == 0) xscale[m] = ldexpf(1.f, e - 9);
     uint16_t *o16 = x16 + static_cast<int64_t>(m) * Kp;
     for (int k = tid; k < Kp; k += 256) o16[k] = k < K ? f32_to_f16_rne(x_to_f32<XF16>(xr[k]) * inv) : uint16_t(0);
+    if (xg == nullptr) return;
+    // group sums of the fp16 values just written (recomputed from x: the same roundings), 256 groups at a time
+    for (int g0 = 0; g0 < nsteps * 16; g0 += 256) {
+        const int g = g0 + tid;
+        float acc = 0.f;
+        if (g < nsteps * 16)
+            for (int i = 0; i < gs; ++i) {
+                const int k = g * gs + i;
+                if (k < K) acc += f16_to_f32(f32_to_f16_rne(x_to_f32<XF16>(xr[k]) * inv));
+            }
+        __syncthreads();
+        gsum[tid] = acc;
+        __syncthreads();
+        // thread (s_local, kb) of this chunk: groups 16 s + 4 j + kb
+        if (tid < 64 && g0 / 16 + (tid >> 2) < nsteps) {
+            const int sl = tid >> 2, kb = tid & 3;
+            float X[4];
+            for (int j = 0; j < 4; ++j) X[j] = gsum[sl * 16 + 4 * j + kb];
+            uint32_t out[4];
+            for (int p = 0; p < 2; ++p) {
+                const _Float16 h0 = static_cast<_Float16>(X[2 * p]), h1 = static_cast<_Float16>(X[2 * p + 1]);
+                const _Float16 l0 = static_cast<_Float16>(X[2 * p] - static_cast<float>(h0));
+                const _Float16 l1 = static_cast<_Float16>(X[2 * p + 1] - static_cast<float>(h1));
+                out[p] = __builtin_bit_cast(uint16_t, h0) | (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, h1)) << 16);
+                out[2 + p] = __builtin_bit_cast(uint16_t, l0) | (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, l1)) << 16);
+            }
+            uint32_t *o = xg + ((static_cast<int64_t>(m) * nsteps + g0 / 16 + sl) * 4 + kb) * 4;
+            for (int t = 0; t < 4; ++t) o[t] = out[t];
+        }
+    }
 }
 
 // ---- fp16 NT GEMM: y[m, n] = sa[m] * sb[n] * sum_k a[m, k] * b[n, k] ----------------------
@@ -138,14 +173,18 @@ int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, i
     return check_launch("gemm_f16_nt");
 }
 
-int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, hipStream_t st) {
+int x_prep_groups(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, int gs,
+                  int nsteps, uint32_t *xg, hipStream_t st) {
     if (x_dtype == MFQ_X_F16)
         hipLaunchKernelGGL((x_prep_kernel<1>), dim3(M), dim3(256), 0, st, static_cast<const uint16_t *>(x), ldx, K, Kp,
-                           static_cast<uint16_t *>(x16), xscale);
+                           static_cast<uint16_t *>(x16), xscale, gs, nsteps, xg);
     else
         hipLaunchKernelGGL((x_prep_kernel<0>), dim3(M), dim3(256), 0, st, static_cast<const uint16_t *>(x), ldx, K, Kp,
-                           static_cast<uint16_t *>(x16), xscale);
+                           static_cast<uint16_t *>(x16), xscale, gs, nsteps, xg);
     return check_launch("x_prep");
+}
+int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, hipStream_t st) {
+    return x_prep_groups(x, x_dtype, ldx, M, K, Kp, x16, xscale, 0, 0, nullptr, st);
 }
 
 // Workspace carve-up of the dequant + GEMM path: x16 [M, Kp] | xscale [M] | w16 [N, Kp] | wscale [N]
@@ -226,9 +265,10 @@ extern "C" int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, con
         p += align256(static_cast<size_t>(M) * Kp * 2);
         float *xscale = reinterpret_cast<float *>(p);
         p += align256(static_cast<size_t>(M) * 4);
-        int rc = x_prep(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, st);
+        uint32_t *xg = reinterpret_cast<uint32_t *>(p);
+        int rc = x_prep_groups(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, d->gs, d->nsteps, xg, st);
         if (rc) return rc;
-        return nint_prefill(d, weight, x16, Kp, xscale, reinterpret_cast<uint32_t *>(p), M, y, ldy, st);
+        return nint_prefill(d, weight, x16, Kp, xscale, xg, M, y, ldy, st);
     }
     const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
     MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nint_gemm: workspace %zu < %zu bytes",

@@ -40,23 +40,24 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t wave_window(const uint8_t *bas
                                              __builtin_amdgcn_readfirstlane(static_cast<int>(bytes)), 0x00020000);
 }
 
-template <int D>
+// POLICY = 2: non-temporal (weights streamed once, decode); 0: cached (weights re-read by other blocks, prefill)
+template <int D, int POLICY = 2>
 __device__ __forceinline__ void load_unit_win(__amdgpu_buffer_rsrc_t win, uint32_t off, uint32_t (&q)[D]) {
     if constexpr (D % 4 == 0) {
 #pragma unroll
         for (int i = 0; i < D / 4; ++i) {
-            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(win, off + 16 * i, 0, 2);
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(win, off + 16 * i, 0, POLICY);
             q[4 * i] = v.x; q[4 * i + 1] = v.y; q[4 * i + 2] = v.z; q[4 * i + 3] = v.w;
         }
     } else if constexpr (D % 2 == 0) {
 #pragma unroll
         for (int i = 0; i < D / 2; ++i) {
-            const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(win, off + 8 * i, 0, 2);
+            const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(win, off + 8 * i, 0, POLICY);
             q[2 * i] = v.x; q[2 * i + 1] = v.y;
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < D; ++i) q[i] = __builtin_amdgcn_raw_buffer_load_b32(win, off + 4 * i, 0, 2);
+        for (int i = 0; i < D; ++i) q[i] = __builtin_amdgcn_raw_buffer_load_b32(win, off + 4 * i, 0, POLICY);
     }
 }
 

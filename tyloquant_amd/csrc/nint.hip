@@ -298,26 +298,37 @@ bool nint_prefill_capable(const mfq_nint_desc *d) {
 }
 size_t nint_prefill_xg_bytes(const mfq_nint_desc *d, int M) { return static_cast<size_t>(M) * d->nsteps * 64; }
 
-// x16 [M, Kp] fp16 (rows scaled by 1 / xscale[m], zero beyond K), xg = workspace of nint_prefill_xg_bytes
+// x16 [M, Kp] fp16 (rows scaled by 1 / xscale[m], zero beyond K), xg = the rows' group sums (x_prep_groups)
 int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16, int Kp, const float *xscale,
                  uint32_t *xg, int M, float *y, int64_t ldy, hipStream_t st) {
     const NintK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
-    const int64_t nthreads = static_cast<int64_t>(M) * k.nsteps * 4;
-    hipLaunchKernelGGL(x_group_sums_kernel, dim3(static_cast<unsigned>(ceil_div(nthreads, 256))), dim3(256), 0, st, x16, Kp, M,
-                       k.gs, k.nsteps, xg);
-    constexpr int MT = 4, NB = 4;
-    const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, 2 * NB)), static_cast<unsigned>(ceil_div(M, 2 * MT * 16)));
-#define MFQ_PREFILL(B, G)                                                                                      \
-    if (k.bits == B && k.gs == G) {                                                                            \
-        const size_t lds = static_cast<size_t>(2 * MT * 16) * (4 * G + 8) * 2;                                 \
-        hipLaunchKernelGGL((nint_prefill_kernel<PairedUnit<B, G>, MT, NB>), grid, dim3(256), lds, st, k, w, x16, Kp, \
-                           xscale, xg, M, y, ldy);                                                             \
+#define MFQ_PREFILL_CFG(B, G, MT, NB, WM, NW)                                                                  \
+    {                                                                                                          \
+        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, (NW / WM) * NB)),                        \
+                        static_cast<unsigned>(ceil_div(M, WM * MT * 16)));                                     \
+        const size_t lds = static_cast<size_t>(2 * WM * MT * 16) * (4 * G + 8) * 2;                            \
+        auto kern = nint_prefill_kernel<PairedUnit<B, G>, MT, NB, WM, NW>;                                     \
+        if (lds > 65536) {                                                                                     \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                           \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+            MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nint_prefill: %s", hipGetErrorString(e));            \
+        }                                                                                                      \
+        hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, st, k, w, x16, Kp, xscale, xg, M, y, ldy);          \
         return check_launch("nint_prefill");                                                                   \
+    }
+    // wave tile MT*16 tokens x NB*16 neurons, NW waves side by side on the neurons
+    // 512 neurons per block; 256 when that leaves CUs without a block
+    const bool narrow = ceil_div(k.n_rowblocks, 32) * ceil_div(M, 64) < 256;
+#define MFQ_PREFILL(B, G)                              \
+    if (k.bits == B && k.gs == G) {                    \
+        if (narrow) MFQ_PREFILL_CFG(B, G, 4, 2, 1, 8)  \
+        MFQ_PREFILL_CFG(B, G, 4, 4, 1, 8)              \
     }
     MFQ_PREFILL(4, 32) MFQ_PREFILL(4, 24) MFQ_PREFILL(4, 16) MFQ_PREFILL(4, 48) MFQ_PREFILL(3, 24) MFQ_PREFILL(2, 16)
     MFQ_PREFILL(2, 32)
 #undef MFQ_PREFILL
+#undef MFQ_PREFILL_CFG
     return fail(MFQ_ERR_UNSUPPORTED, "nint_prefill: no kernel for NINT%d-%d", k.bits, k.gs);
 }
 
