@@ -98,6 +98,22 @@ def test_nepq_dequant_bit_exact_and_matmul(label, E, out, K, banks):
         _check(nepq_matmul(w, x, e).cpu().numpy(), O.linear_forward_f64(want[e], xf))
 
 
+@pytest.mark.parametrize("label,out,K,M,banks", [("NEPQ1-S", 64, 2048, 1, 16), ("NEPQ1-L", 48, 4104, 16, 16),
+                                                  ("NEPQ1-S", 130 - 2, 1024, 33, 4), ("NEPQ1-L", 32, 6144, 7, 3)])
+def test_nepq_matrix_core_path_multi_step(label, out, K, M, banks):
+    """K % 8 == 0 rows take the MFMA streaming kernel: several steps, K split over waves, ragged last group,
+    tables in LDS (S) or read from global memory (L, 16 banks), a second expert, a row stride above K."""
+    from tyloquant_amd.runtime_vq import NepqWeight, nepq_matmul
+    rng = np.random.default_rng(300 + out + M)
+    t = synth.nepq_random(rng, label, 2, out, K, banks)
+    w = NepqWeight.from_blob(O.pack_nepq(t))
+    want = O.dequantize_nepq(t)
+    xw = torch.from_numpy(rng.standard_normal((M, K + 8)).astype(np.float32)).to(torch.bfloat16).cuda()
+    x = xw[:, :K]
+    for e in (0, 1):
+        _check(nepq_matmul(w, x, e, force="gemv").cpu().numpy(), O.linear_forward_f64(want[e], x.float().cpu().numpy()))
+
+
 def test_nepq_hadamard_matches_fwht():
     from tyloquant_amd.runtime_vq import nepq_hadamard
     rng = np.random.default_rng(3)

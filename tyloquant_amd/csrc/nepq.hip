@@ -10,6 +10,7 @@
 // value = fl(anchor * state) * (code + bias), bias = +-5/32 (S) or +-1/8 (L), minus when aux is set.
 #include "common.hpp"
 #include "gemv_common.hpp"
+#include "nint_mfma.hpp"
 
 namespace mfq {
 
@@ -225,6 +226,159 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
     finish_rows<MB>(v, red, wave, nwaves, lane, rb, row0, nrows, yr);
 }
 
+// ---- matrix-core path: up to 16 activation rows per streamed pass ----------------------------------
+// Same scheme as the NINT kernel (nint_mfma.hpp).  Fragment m of a unit is one table entry: 8 two-bit digits
+// (code + 1) that become four (1024 + digit) fp16 pairs and, with one packed FMA each, state * digit (exact).
+// The remaining part of the value, state * (bias - 1) * X_g, is one more MFMA per step against the group sums
+// X_g (two fp16 halves), exactly as the NINT minimum term.  Padding groups have state 0.
+template <int XF16, int NB, int TAB_LDS>
+__global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *__restrict__ w, int rb_first, int row0,
+                                                        int nrows, const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                        float *__restrict__ y, int64_t ldy, int spw) {
+    extern __shared__ uint32_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint16_t *gtab = reinterpret_cast<const uint16_t *>(w + k.tables_off);
+    const int ntab = k.banks * k.entries;  // u16 entries
+    float *red = reinterpret_cast<float *>(lds);
+    if constexpr (TAB_LDS) {
+        for (int i = tid; i < ntab / 2; i += blockDim.x) lds[i] = reinterpret_cast<const uint32_t *>(gtab)[i];
+        red = reinterpret_cast<float *>(lds + ntab / 2);
+    }
+    const uint16_t *tab = TAB_LDS ? reinterpret_cast<const uint16_t *>(lds) : gtab;
+    const int rbl0 = blockIdx.x * NB, m0 = blockIdx.y * 16;  // row-blocks relative to rb_first
+    const int rb0 = rb_first + rbl0, rb_end = rb_first + (nrows + 15) / 16;
+    const int tok = min(m0 + (lane & 15), M - 1);
+    const uint16_t *xrow = x + static_cast<int64_t>(tok) * ldx;
+    const int r = lane & 15, kb = lane >> 4;
+    const int s0 = wave * spw;
+    const int n = min(k.nsteps, s0 + spw) - s0;
+    const int nrb = min(NB, rb_end - rb0);
+    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
+    float anchor[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+        anchor[i] = reinterpret_cast<const float *>(w + k.anchors_off)[min(rb0 + i, k.n_rowblocks - 1) * 16 + r];
+    const __amdgpu_buffer_rsrc_t win =
+        wave_window(w + static_cast<int64_t>(rb0) * k.rowblock_bytes + static_cast<int64_t>(s0) * sb,
+                    n > 0 ? (nrb - 1) * rbb + n * sb : 0u);
+    float4_t acc[NB], accB[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) acc[i] = accB[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    if constexpr (TAB_LDS) __syncthreads();
+
+    const float delta = k.profile == 2 ? 0.15625f : 0.125f;
+    const uint32_t toff = 1024u, boff = 1024u + (k.tail ? 256u : 0u);
+    for (int s = 0; s < n; ++s) {
+        uint32_t q[NB][4], tails[NB], banks4[NB];
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            const uint32_t off = i < nrb ? i * rbb + s * sb : kNoStep;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) q[i][j] = __builtin_amdgcn_raw_buffer_load_b32(win, off + (j * 64 + lane) * 4, 0, 2);
+            tails[i] = k.tail ? __builtin_amdgcn_raw_buffer_load_b32(win, off + toff + lane * 4, 0, 2) : 0u;
+            banks4[i] = __builtin_amdgcn_raw_buffer_load_b32(win, off + boff + r * 4, 0, 2);
+        }
+        const int kbase = (s0 + s) * 16 * 24 + kb * 24;
+        float xsum[4];
+        uint32_t stw[NB][4];  // per unit: state * (bias - 1) as an fp16
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            u32x4_t a[3];
+#pragma unroll
+            for (int m = 0; m < 3; ++m) a[m] = load_xfrag<XF16, true>(xrow, kbase + 4 * j * 24 + 8 * m, k.neuron_len);
+            float xs = 0.f;
+#pragma unroll
+            for (int m = 0; m < 3; ++m)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) xs = dot2h(a[m][t], 0x3c003c00u, xs);
+            xsum[j] = xs;
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const NepqUnit u = nepq_decode(k.profile, q[i][j], (tails[i] >> (8 * j)) & 0xffu);
+                const uint16_t *bank = tab + ((banks4[i] >> (8 * j)) & 0xffu) * k.entries;
+                const float st = static_cast<float>(u.state);
+                const half2_t S = pk_h2(st, st), C = pk_h2(-1024.f * st, -1024.f * st);
+                stw[i][j] = f32_to_f16_rne(st * ((u.aux ? -delta : delta) - 1.f));
+#pragma unroll
+                for (int m = 0; m < 3; ++m) {
+                    const uint32_t e = bank[u.idx[m]];
+                    const uint32_t t2 = e | (e << 14);
+                    u32x4_t b;
+#pragma unroll
+                    for (int p = 0; p < 4; ++p)
+                        b[p] = __builtin_bit_cast(uint32_t, h2_fma(((t2 >> (4 * p)) & 0x00030003u) | kMagicH2, S, C));
+                    acc[i] = mfma16(a[m], b, acc[i]);
+                }
+            }
+        }
+        u32x4_t ax;
+        {
+            half2_t hi[2], lo[2];
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                hi[p] = pk_h2(xsum[2 * p], xsum[2 * p + 1]);
+                lo[p] = pk_h2(xsum[2 * p] - static_cast<float>(hi[p].x), xsum[2 * p + 1] - static_cast<float>(hi[p].y));
+            }
+            ax = u32x4_t{__builtin_bit_cast(uint32_t, hi[0]), __builtin_bit_cast(uint32_t, hi[1]),
+                         __builtin_bit_cast(uint32_t, lo[0]), __builtin_bit_cast(uint32_t, lo[1])};
+        }
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            const uint32_t b01 = stw[i][0] | (stw[i][1] << 16), b23 = stw[i][2] | (stw[i][3] << 16);
+            accB[i] = mfma16(ax, u32x4_t{b01, b23, b01, b23}, accB[i]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[((wave * NB + i) * 4 + v) * 64 + lane] = anchor[i] * (acc[i][v] + accB[i][v]);
+    // rows are relative to row0 in y
+    __syncthreads();
+    const int nwaves = blockDim.x >> 6;
+    for (int o = threadIdx.x; o < NB * 256; o += blockDim.x) {
+        const int rr = o & 15, t = (o >> 4) & 15, nb = o >> 8;
+        const int slot = (nb * 4 + (t & 3)) * 64 + rr + 16 * (t >> 2);
+        float sacc = 0.f;
+        for (int wv = 0; wv < nwaves; ++wv) sacc += red[wv * NB * 256 + slot];
+        const int row = (rb0 + nb) * 16 + rr - row0;
+        if (m0 + t < M && row >= 0 && row < nrows) y[static_cast<int64_t>(m0 + t) * ldy + row] = sacc;
+    }
+}
+
+static bool nepq_stream_capable(const NepqK &k) {
+    return k.neuron_len >= 8 && k.neuron_len % 8 == 0 && 4 * k.rowblock_bytes < (1ll << 31);
+}
+
+template <int XF16, int NB>
+static int nepq_launch_mfma(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
+                            float *y, int64_t ldy, hipStream_t st) {
+    const int nrb = static_cast<int>(ceil_div(nrows, 16));
+    const int64_t groups = ceil_div(nrb, NB);
+    int spw = static_cast<int>(ceil_div(k.nsteps, 8));
+    while (spw < k.nsteps && groups * ceil_div(k.nsteps, spw) > 8192) ++spw;
+    const int nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
+    const size_t redb = static_cast<size_t>(nwaves) * NB * 1024, tabb = static_cast<size_t>(k.banks) * k.entries * 2;
+    const bool tab_lds = redb + tabb <= 65536;
+    const size_t lds = redb + (tab_lds ? tabb : 0);
+    const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(ceil_div(M, 16))), block(64 * nwaves);
+    if (tab_lds)
+        hipLaunchKernelGGL((nepq_mfma_kernel<XF16, NB, 1>), grid, block, lds, st, k, w, row0 / 16, row0, nrows, x, ldx, M, y,
+                           ldy, spw);
+    else
+        hipLaunchKernelGGL((nepq_mfma_kernel<XF16, NB, 0>), grid, block, lds, st, k, w, row0 / 16, row0, nrows, x, ldx, M, y,
+                           ldy, spw);
+    return check_launch("nepq_mfma");
+}
+
+template <int XF16>
+static int nepq_mfma_any(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
+                         float *y, int64_t ldy, hipStream_t st) {
+    const int64_t items = ceil_div(nrows, 16) * k.nsteps;
+    if (items >= 4 * 1536) return nepq_launch_mfma<XF16, 4>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
+    return nepq_launch_mfma<XF16, 1>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
+}
+
 static void nepq_gemv_shape(const NepqK &k, int nrb, int mb, int &spw, int &nwaves, size_t &lds_bytes, bool &tab_lds) {
     int want = static_cast<int>(ceil_div(3 * gemv_target_waves(), nrb));
     if (want < 1) want = 1;
@@ -261,6 +415,10 @@ static int nepq_gemv_any(const mfq_nepq_desc *d, const void *weight, int row0, i
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
     const int nrb = static_cast<int>(ceil_div(nrows, 16));
+    // a single row is still cheaper on the vector-ALU kernel
+    if (M >= 2 && nepq_stream_capable(k) && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
+        return x_dtype == MFQ_X_F16 ? nepq_mfma_any<1>(k, w, row0, nrows, xp, ldx, M, y, ldy, st)
+                                    : nepq_mfma_any<0>(k, w, row0, nrows, xp, ldx, M, y, ldy, st);
     int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
     for (;;) {
         int spw, nwaves;
@@ -384,10 +542,15 @@ extern "C" int mfq_hip_nepq_gemv(const mfq_nepq_desc *d, const void *weight, int
     return nepq_gemv_any(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, as_stream(stream));
 }
 
-static constexpr int kNepqGemvMaxM = 16;  // the reference's Python policy: M <= 16 stays on the GEMV
+// The reference's Python policy keeps M <= 16 on the GEMV; tensors the matrix-core streaming kernel takes stay
+// on it up to kNepqStreamMaxM rows.
+static constexpr int kNepqGemvMaxM = 16, kNepqStreamMaxM = 256;
+static bool nepq_streams(const mfq_nepq_desc *d, int M) {
+    return M <= kNepqGemvMaxM || (M <= kNepqStreamMaxM && nepq_stream_capable(to_k(d)));
+}
 
 extern "C" size_t mfq_hip_nepq_gemm_workspace_bytes(const mfq_nepq_desc *d, int nrows, int M) {
-    if (!d || M <= kNepqGemvMaxM) return 0;
+    if (!d || nepq_streams(d, M)) return 0;
     return dequant_gemm_workspace(nrows, d->neuron_len, M);
 }
 
@@ -400,7 +563,7 @@ extern "C" int mfq_hip_nepq_gemm(const mfq_nepq_desc *d, const void *weight, int
     if (int rc = nepq_check_rows(d, row0, nrows)) return rc;
     MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= nrows, MFQ_ERR_INVALID, "nepq_gemm: ldx/ldy smaller than the tensor");
     hipStream_t st = as_stream(stream);
-    if (M <= kNepqGemvMaxM) return nepq_gemv_any(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, st);
+    if (nepq_streams(d, M)) return nepq_gemv_any(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, st);
     const size_t need = dequant_gemm_workspace(nrows, d->neuron_len, M);
     MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nepq_gemm: workspace %zu < %zu bytes",
                 workspace_bytes, need);
