@@ -40,6 +40,9 @@ def main() -> int:
     ap.add_argument("--copies", type=int, default=8)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run a plain 256 MiB device copy 20 times (the reference kernel the HBM counters of a "
+                         "rocprofv3 --pmc run are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
@@ -146,6 +149,13 @@ def main() -> int:
     assert lin_err < 1e-5, f"GEMV is not linear in x / copies differ: {lin_err}"
 
     extras = {"linearity_rel_err": lin_err, "gpu_ms_total": gpu_ms}
+    if args.calibrate:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(20):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     def time_fn(fn, reps, warm=5):
         for _ in range(warm):
@@ -350,8 +360,11 @@ def main() -> int:
                                f"({args.copies * step_bytes / 1e6:.0f} MB)",
                    "step_bytes": step_bytes, "launches_per_step": n_per_step, "hip_graph": True},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "nint_gemv_paired_kernel<4,32,0,1>", "avg_launch_us": avg_launch_us,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, each scaled by what the counter
+                     # reads for a plain 256 MiB copy (2.000 and 1.000): profiles/nint_gemv_paired_4_32_config2_decode.md
+                     "traffic": 43.0e6,
+                     "kernel": "nint_gemv_paired_kernel<4,32,0,1,false>", "avg_launch_us": avg_launch_us,
                      "bytes_per_launch": bytes_per_launch},
         "cpu_baseline": cpu,
         "extras": extras,

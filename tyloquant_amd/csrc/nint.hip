@@ -285,10 +285,10 @@ static int launch_mfma_nb(const NintK &k, const uint8_t *w, const uint16_t *x, i
 template <int XF16>
 static int launch_mfma(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                        hipStream_t st) {
-    // row-blocks per wave: as many as still leave about 1500 waves
-    const int64_t items = static_cast<int64_t>(k.n_rowblocks) * k.nsteps;
-    if (items >= 4 * 1536) return launch_mfma_nb<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
-    if (items >= 2 * 1536) return launch_mfma_nb<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
+    // row-blocks per wave: as many as still leave about 1500 waves (a block has at most 8)
+    const int64_t wpb = k.nsteps < 8 ? k.nsteps : 8;
+    if (ceil_div(k.n_rowblocks, 4) * wpb >= 1536) return launch_mfma_nb<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
+    if (ceil_div(k.n_rowblocks, 2) * wpb >= 1536) return launch_mfma_nb<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
     return launch_mfma_nb<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
 }
 

@@ -401,9 +401,9 @@ static int nvq_launch_mfma(const NvqK &k, const uint8_t *w, const uint16_t *x, i
 template <int XF16>
 static int nvq_mfma_any(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                         hipStream_t st) {
-    const int64_t items = static_cast<int64_t>(k.n_rowblocks) * k.nsteps;
-    if (items >= 4 * 1536) return nvq_launch_mfma<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
-    if (items >= 2 * 1536) return nvq_launch_mfma<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
+    const int64_t wpb = k.nsteps < 8 ? k.nsteps : 8;  // waves of a block
+    if (ceil_div(k.n_rowblocks, 4) * wpb >= 1536) return nvq_launch_mfma<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
+    if (ceil_div(k.n_rowblocks, 2) * wpb >= 1536) return nvq_launch_mfma<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
     return nvq_launch_mfma<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
 }
 
