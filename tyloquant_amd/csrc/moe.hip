@@ -51,31 +51,64 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float *__restrict__
         for (int e = lane; e < E; e += 64) ssum += expf(raw_at(e) - smax);
         ssum = wave_sum(ssum);
     }
-    int selected[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) selected[i] = -1;
+    auto weight_of = [&](float raw) {
+        if (mode == MFQ_TOPK_DELAYED_SOFTMAX) return raw;
+        if (mode == MFQ_TOPK_SIGMOID) return 1.f / (1.f + expf(-raw));
+        if (mode == MFQ_TOPK_SQRT_SOFTPLUS) return sqrtf(raw > 20.f ? raw : log1pf(expf(raw)));
+        return expf(raw - smax) / ssum;
+    };
     float mine = 0.f;  // lane r keeps the weight of rank r
-    for (int rank = 0; rank < k; ++rank) {
-        float bs = -INFINITY, bw = -INFINITY;
-        int bi = INT_MAX;
-        for (int e = lane; e < E; e += 64) {
-            bool taken = false;
+    constexpr int PER = 8;  // experts a lane keeps in registers: rows up to 512 experts are read once
+    if (E <= 64 * PER) {
+        float sc[PER], wv[PER];
 #pragma unroll
-            for (int p = 0; p < 16; ++p) taken |= (p < rank && selected[p] == e);
-            if (taken) continue;
-            const float raw = raw_at(e);
-            float wv;
-            if (mode == MFQ_TOPK_DELAYED_SOFTMAX) wv = raw;
-            else if (mode == MFQ_TOPK_SIGMOID) wv = 1.f / (1.f + expf(-raw));
-            else if (mode == MFQ_TOPK_SQRT_SOFTPLUS) wv = sqrtf(raw > 20.f ? raw : log1pf(expf(raw)));
-            else wv = expf(raw - smax) / ssum;
-            const float sc = wv + (bias ? bias[e] : 0.f);
-            if (sc > bs || (sc == bs && e < bi)) { bs = sc; bw = wv; bi = e; }
+        for (int i = 0; i < PER; ++i) {
+            const int e = lane + 64 * i;
+            sc[i] = -INFINITY;
+            wv[i] = -INFINITY;
+            if (e < E) {
+                wv[i] = weight_of(raw_at(e));
+                sc[i] = wv[i] + (bias ? bias[e] : 0.f);
+            }
         }
-        wave_argmax(bs, bw, bi);
-        selected[rank] = bi;
-        if (lane == rank) mine = bw;
-        if (lane == 0) ids[static_cast<int64_t>(t) * k + rank] = bi;
+        bool taken[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) taken[i] = lane + 64 * i >= E;
+        for (int rank = 0; rank < k; ++rank) {
+            float bs = -INFINITY, bw = -INFINITY;
+            int bi = INT_MAX;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                const int e = lane + 64 * i;
+                if (!taken[i] && (sc[i] > bs || (sc[i] == bs && e < bi))) { bs = sc[i]; bw = wv[i]; bi = e; }
+            }
+            wave_argmax(bs, bw, bi);
+#pragma unroll
+            for (int i = 0; i < PER; ++i) taken[i] = taken[i] || (lane + 64 * i == bi);
+            if (lane == rank) mine = bw;
+            if (lane == 0) ids[static_cast<int64_t>(t) * k + rank] = bi;
+        }
+    } else {
+        int selected[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) selected[i] = -1;
+        for (int rank = 0; rank < k; ++rank) {
+            float bs = -INFINITY, bw = -INFINITY;
+            int bi = INT_MAX;
+            for (int e = lane; e < E; e += 64) {
+                bool taken = false;
+#pragma unroll
+                for (int p = 0; p < 16; ++p) taken |= (p < rank && selected[p] == e);
+                if (taken) continue;
+                const float wv = weight_of(raw_at(e));
+                const float sc = wv + (bias ? bias[e] : 0.f);
+                if (sc > bs || (sc == bs && e < bi)) { bs = sc; bw = wv; bi = e; }
+            }
+            wave_argmax(bs, bw, bi);
+            selected[rank] = bi;
+            if (lane == rank) mine = bw;
+            if (lane == 0) ids[static_cast<int64_t>(t) * k + rank] = bi;
+        }
     }
     float v = lane < k ? mine : 0.f;
     if (mode == MFQ_TOPK_DELAYED_SOFTMAX) {
