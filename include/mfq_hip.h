@@ -67,13 +67,18 @@ int mfq_hip_nint_repack(const mfq_nint_desc *d, const void *payload, int64_t pay
 int mfq_hip_nint_dequant_f32(const mfq_nint_desc *d, const void *weight, float *w_out, int64_t ld,
                              mfq_stream_t stream);
 
-/* y[M, out] = x[M, neuron_len] . W^T, fp32 accumulate, for small M (decode).  Replaces
+/* y[M, out] = x[M, neuron_len] . W^T, fp32 accumulate, streaming the packed weights: once for M = 1,
+ * once per 16 rows on the matrix cores for larger M (needs neuron_len % 8 == 0, ldx % 8 == 0 and a
+ * 16-byte aligned x; otherwise once per 4 rows on the vector ALUs).  Any M >= 1 is valid.  Replaces
  * nint_gemv_packed_ws_cuda / nint_gemv_packed_bits_ws_cuda (cpp_runtime/mfq_decode.cpp:421-435). */
 int mfq_hip_nint_gemv(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
                       int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream);
 
-/* Prefill / large-M path (MFMA).  Replaces nint_mmq_f16_packed_cuda / nint_mmq_f32_packed_cuda
- * and the dequant + cuBLAS fallback (cpp_runtime/mfq_decode.cpp:480-520, 8309-8314). */
+/* Any-M entry: the streaming kernels of mfq_hip_nint_gemv up to 256 rows, above that a block-tiled MFMA
+ * GEMM with in-register dequantization (paired profiles) or dequantize-to-fp16 + MFMA GEMM.  The workspace
+ * (size from the query, 0 when none is needed) holds fp16 activations and, for the second case, fp16
+ * weights.  Replaces nint_mmq_f16_packed_cuda / nint_mmq_f32_packed_cuda and the dequant + cuBLAS fallback
+ * (cpp_runtime/mfq_decode.cpp:480-520, 8309-8314). */
 size_t mfq_hip_nint_gemm_workspace_bytes(const mfq_nint_desc *d, int M);
 int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
                       int64_t ldx, int M, float *y, int64_t ldy, void *workspace,
