@@ -204,6 +204,22 @@ int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools, const int
                                const int32_t *tile_bounds, const int32_t *tile_experts,
                                float *out, int64_t ldo, mfq_stream_t stream);
 
+/* The same with a workspace, which unlocks the prefill kernel when a mapped call carries many pairs per
+ * expert (64 pairs of an expert against 512 neurons per block; activations pre-scaled to fp16 in the
+ * workspace).  x_rows = T * R with routed_input, else T.  The size query returns 0 when the cohorts have no
+ * prefill kernel; a NULL or short workspace simply keeps the streaming kernels.  No counterpart in the
+ * reference, whose hetero kernels allocate their workspace through torch
+ * (cpp_runtime/mfq_decode.cpp:3008-3016). */
+size_t mfq_hip_moe_grouped_workspace_bytes(const mfq_moe_pool *pools, int n_pools, int K, int x_rows);
+int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_pools, const int32_t *expert_pool,
+                                  const int32_t *expert_local, int E, int out_per_expert, int K,
+                                  const void *x, int x_dtype, int64_t ldx, int routed_input,
+                                  const int32_t *ids, int T, int R,
+                                  const int32_t *ids_dst, const int32_t *expert_bounds,
+                                  const int32_t *tile_bounds, const int32_t *tile_experts,
+                                  float *out, int64_t ldo, void *workspace, size_t workspace_bytes,
+                                  mfq_stream_t stream);
+
 /* hidden[r, c] = silu(gate_up[r, c]) * gate_up[r, W + c]  (moe_swiglu_split_cuda,
  * mfq/kernels/cuda/moe.cu:2980-2996); output fp16 (x_dtype MFQ_X_F16) or bf16. */
 int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,

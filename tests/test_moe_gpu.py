@@ -84,6 +84,27 @@ def test_grouped_matmul_matches_reference_loop(tokens):
     assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL
 
 
+@pytest.mark.parametrize("routed", [False, True])
+def test_grouped_matmul_prefill_path_many_pairs_per_expert(routed):
+    """At 24+ pairs per expert the paired cohorts run the prefill kernel (64 pairs of an expert per block), the
+    NINT5-28 cohort stays on the streaming kernel; experts with 0, 1 and > 64 pairs, an invalid id, ragged K."""
+    from tyloquant_amd.runtime_moe import build_moe_route_plan
+    rng = np.random.default_rng(77)
+    E, out, K, T, R = 6, 80, 776, 150, 2
+    t, w = _moe(rng, E, out, K, [4, 3, 2, 5, 4, 3])
+    dense = O.dequantize_expertwise(t)
+    ids = rng.choice(5, size=(T, R), p=[0.5, 0.2, 0.15, 0.1, 0.05]).astype(np.int32)   # expert 5 unused
+    ids[0, 0] = 5
+    ids[7, 1] = 99
+    shape = (T, R, K) if routed else (T, K)
+    x = torch.from_numpy((rng.standard_normal(shape) * 0.1).astype(np.float32)).to(torch.bfloat16)
+    route = build_moe_route_plan(torch.from_numpy(ids).cuda(), E)
+    got = w(x.cuda(), route).cpu().numpy()
+    ref = O.moe_grouped_matmul(dense, x.float().numpy(), ids)
+    assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL
+    assert np.all(got[7, 1] == 0)
+
+
 def test_grouped_matmul_routed_input_and_invalid_expert():
     from tyloquant_amd.runtime_moe import build_moe_route_plan
     rng = np.random.default_rng(44)

@@ -407,13 +407,20 @@ NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream
 void NintMoeWeight::forward(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &r, float *out,
                             mfq_stream_t stream) const {
     const bool mapped = r.mapped();
-    abi_check(mfq_hip_moe_grouped_matmul(
+    // a workspace unlocks the prefill kernel for mapped calls with many pairs per expert
+    const int x_rows = routed_input ? r.tokens * r.routes : r.tokens;
+    size_t need = 0;
+    if (mapped && static_cast<int64_t>(r.tokens) * r.routes >= 24ll * n_experts)
+        need = mfq_hip_moe_grouped_workspace_bytes(pool_table.data(), static_cast<int>(pool_table.size()), neuron_len, x_rows);
+    if (need) workspace.ensure(need);
+    abi_check(mfq_hip_moe_grouped_matmul_ws(
         pool_table.data(), static_cast<int>(pool_table.size()), static_cast<const int32_t *>(expert_pool.get()),
         static_cast<const int32_t *>(expert_local.get()), n_experts, out_per_expert, neuron_len, x, x_dtype, ldx,
         routed_input ? 1 : 0, r.ids, r.tokens, r.routes, mapped ? static_cast<const int32_t *>(r.ids_dst.get()) : nullptr,
         mapped ? static_cast<const int32_t *>(r.expert_bounds.get()) : nullptr,
         mapped ? static_cast<const int32_t *>(r.tile_bounds.get()) : nullptr,
-        mapped ? static_cast<const int32_t *>(r.tile_experts.get()) : nullptr, out, out_per_expert, stream));
+        mapped ? static_cast<const int32_t *>(r.tile_experts.get()) : nullptr, out, out_per_expert,
+        need ? workspace.get() : nullptr, need, stream));
 }
 
 void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &down, const void *x, int x_dtype, int64_t ldx,

@@ -166,6 +166,7 @@ struct NintMoeWeight {
     std::vector<std::vector<int32_t>> pool_expert_ids;
     DeviceBuffer expert_pool, expert_local;  // int32 [E] dispatch tables
     std::vector<mfq_moe_pool> pool_table;
+    mutable DeviceBuffer workspace;  // prefill path, grown on demand (do not grow it under graph capture)
     static NintMoeWeight from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream = nullptr);
     // x: [T, K] (routed_input = false) or [T*R, K]; out: fp32 [T*R, out_per_expert]
     void forward(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &route, float *out,

@@ -6,6 +6,7 @@
 #include "gemv_common.hpp"
 #include "nint_body.hpp"
 #include "nint_mfma.hpp"
+#include "nint_prefill.hpp"
 
 namespace mfq {
 
@@ -205,8 +206,10 @@ constexpr int kMaxPools = 8;
 struct MoePools {
     NintK k[kMaxPools];
     const uint8_t *w[kMaxPools];
+    const uint32_t *xg[kMaxPools];  // prefill path: group sums of the activations for this cohort's groupsize
     int spw[kMaxPools];
     int n;
+    int prefill[kMaxPools];  // cohort runs on the prefill kernel in this call (the streaming kernel skips it)
 };
 
 constexpr int kMoeTileM = 16;  // (token, route) pairs of one expert per tile of the route map
@@ -324,6 +327,7 @@ __global__ __launch_bounds__(512) void moe_mfma_kernel(MoePools P, const int32_t
     if (p < 0) p = pair_of(0);
     const uint16_t *xrow = x + static_cast<int64_t>(routed_input ? p : p / R) * ldx;
     const NintK &k = P.k[pool];
+    if (P.prefill[pool]) return;
     const uint8_t *w = P.w[pool];
     const int spw = P.spw[pool];
 #define MFQ_MOE_MFMA(UNIT, B, G) \
@@ -351,6 +355,57 @@ __global__ __launch_bounds__(512) void moe_mfma_kernel(MoePools P, const int32_t
         for (int wv = 0; wv < nwaves; ++wv) s += red[wv * NB * 256 + slot];
         out[static_cast<int64_t>(pt) * ldo + (rbl0 + nb) * 16 + rr] = s;
     }
+}
+
+// Prefill path for many pairs per expert: a block takes four consecutive tiles (64 pairs) of one expert and 512 of
+// its neurons through nint_prefill_body.  Blocks of the other tiles exit at once.  x16 / xscale / P.xg are indexed by the source row of a pair.
+__global__ __launch_bounds__(512) void moe_prefill_kernel(MoePools P, const int32_t *__restrict__ expert_pool,
+                                                          const int32_t *__restrict__ expert_local, int E,
+                                                          int out_per_expert, const uint16_t *__restrict__ x16, int Kp,
+                                                          const float *__restrict__ xscale, int routed_input, int R,
+                                                          const int32_t *__restrict__ ids_dst,
+                                                          const int32_t *__restrict__ expert_bounds,
+                                                          const int32_t *__restrict__ tile_bounds,
+                                                          const int32_t *__restrict__ tile_experts,
+                                                          float *__restrict__ out, int64_t ldo) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t plds[];
+    const int tile = blockIdx.x;
+    if (tile >= tile_bounds[E]) return;
+    const int e = tile_experts[tile];
+    const int ti = tile - tile_bounds[e];
+    if (ti & 3) return;
+    const int pool = expert_pool[e];
+    if (pool < 0 || !P.prefill[pool]) return;
+    const int lo = expert_bounds[e] + ti * kMoeTileM, hi = min(expert_bounds[e + 1], lo + 4 * kMoeTileM);
+    int *srcv = reinterpret_cast<int *>(plds), *dstv = srcv + 64;
+    uint16_t *xt = reinterpret_cast<uint16_t *>(plds + 128);
+    if (threadIdx.x < 64) {
+        const int p = lo + static_cast<int>(threadIdx.x) < hi ? ids_dst[lo + threadIdx.x] : -1;
+        const int pp = p >= 0 ? p : ids_dst[lo];
+        dstv[threadIdx.x] = p;
+        srcv[threadIdx.x] = routed_input ? pp : pp / R;
+    }
+    __syncthreads();
+    const int rbe = out_per_expert / 16, rb_first = expert_local[e] * rbe;
+    const int rb_base = rb_first + static_cast<int>(blockIdx.y) * 32;
+    const NintK &k = P.k[pool];
+    const MappedRows rows{srcv, dstv};
+#define MFQ_MOE_PREFILL(UNIT, B, G)                                                                                  \
+    if (k.bits == B && k.gs == G)                                                                                    \
+        nint_prefill_body<UNIT<B, G>, 4, 4, 1, 8>(k, P.w[pool], rb_base, rb_first + rbe, rb_first, out_per_expert, x16, Kp, \
+                                                  xscale, P.xg[pool], rows, out, ldo, xt);
+    if (k.kind == 1) {
+        MFQ_MOE_PREFILL(PairedUnit, 4, 24)
+        else MFQ_MOE_PREFILL(PairedUnit, 3, 24)
+        else MFQ_MOE_PREFILL(PairedUnit, 2, 16)
+        else MFQ_MOE_PREFILL(PairedUnit, 4, 32)
+        else MFQ_MOE_PREFILL(PairedUnit, 4, 16)
+        else MFQ_MOE_PREFILL(PairedUnit, 4, 48)
+        else MFQ_MOE_PREFILL(PairedUnit, 2, 32)
+    } else {
+        MFQ_MOE_PREFILL(GenericUnit, 5, 28)
+    }
+#undef MFQ_MOE_PREFILL
 }
 
 // rows of pairs whose expert id is out of range are not in any tile of the map: clear them
@@ -430,12 +485,49 @@ extern "C" int mfq_hip_moe_route_map(const int32_t *ids, int n_pairs, int E, int
 
 extern "C" int mfq_hip_moe_tile_m(void) { return kMoeTileM; }
 
+namespace mfq {
+int x_prep_groups(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, int gs,
+                  int nsteps, uint32_t *xg, hipStream_t st);
+}
+
+// prefill workspace: x16 [rows, Kp] | xscale [rows] | one group-sum table per distinct groupsize of the paired cohorts
+static size_t moe_align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+static int moe_kp(int K) { return static_cast<int>(ceil_div(K, 32)) * 32; }
+static bool moe_prefill_unit(const mfq_nint_desc &d) { return d.kind == 1 || (d.bits == 5 && d.gs == 28); }
+static bool moe_prefill_pools(const mfq_moe_pool *pools, int n_pools) {  // every cohort has a prefill unit
+    for (int i = 0; i < n_pools; ++i)
+        if (!moe_prefill_unit(pools[i].desc) || 4 * pools[i].desc.rowblock_bytes >= (1ll << 31)) return false;
+    return true;
+}
+
+extern "C" size_t mfq_hip_moe_grouped_workspace_bytes(const mfq_moe_pool *pools, int n_pools, int K, int x_rows) {
+    if (!pools || n_pools < 1 || n_pools > kMaxPools || x_rows < 1 || !moe_prefill_pools(pools, n_pools)) return 0;
+    size_t total = moe_align256(static_cast<size_t>(x_rows) * moe_kp(K) * 2) + moe_align256(static_cast<size_t>(x_rows) * 4);
+    for (int i = 0; i < n_pools; ++i) {
+        bool seen = false;
+        for (int j = 0; j < i; ++j) seen = seen || pools[j].desc.gs == pools[i].desc.gs;
+        if (!seen) total += moe_align256(static_cast<size_t>(x_rows) * pools[i].desc.nsteps * 64);
+    }
+    return total;
+}
+
 extern "C" int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools, const int32_t *expert_pool,
                                           const int32_t *expert_local, int E, int out_per_expert, int K, const void *x,
                                           int x_dtype, int64_t ldx, int routed_input, const int32_t *ids, int T, int R,
                                           const int32_t *ids_dst, const int32_t *expert_bounds,
                                           const int32_t *tile_bounds, const int32_t *tile_experts, float *out,
                                           int64_t ldo, mfq_stream_t stream) {
+    return mfq_hip_moe_grouped_matmul_ws(pools, n_pools, expert_pool, expert_local, E, out_per_expert, K, x, x_dtype, ldx,
+                                         routed_input, ids, T, R, ids_dst, expert_bounds, tile_bounds, tile_experts, out, ldo,
+                                         nullptr, 0, stream);
+}
+
+extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_pools, const int32_t *expert_pool,
+                                             const int32_t *expert_local, int E, int out_per_expert, int K, const void *x,
+                                             int x_dtype, int64_t ldx, int routed_input, const int32_t *ids, int T, int R,
+                                             const int32_t *ids_dst, const int32_t *expert_bounds,
+                                             const int32_t *tile_bounds, const int32_t *tile_experts, float *out,
+                                             int64_t ldo, void *workspace, size_t workspace_bytes, mfq_stream_t stream) {
     MFQ_REQUIRE(pools && expert_pool && expert_local && x && ids && out, MFQ_ERR_INVALID, "moe_grouped_matmul: null argument");
     MFQ_REQUIRE(n_pools >= 1 && n_pools <= kMaxPools, MFQ_ERR_UNSUPPORTED, "moe_grouped_matmul: %d cohorts (max %d)", n_pools,
                 kMaxPools);
@@ -463,6 +555,8 @@ extern "C" int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools
         k.kind = d.kind; k.dwords = d.dwords; k.tail = d.tail_bytes; k.nsteps = d.nsteps; k.n_rowblocks = d.n_rowblocks;
         k.step_bytes = d.step_bytes; k.rowblock_bytes = d.rowblock_bytes; k.anchors_off = d.anchors_off;
         P.w[i] = static_cast<const uint8_t *>(pools[i].weight);
+        P.xg[i] = nullptr;
+        P.prefill[i] = 0;
         mfma = mfma && (d.kind == 1 || (d.bits == 5 && d.gs == 28)) && 4 * d.rowblock_bytes < (1ll << 31);
     }
     const int rbe = out_per_expert / 16;
@@ -475,6 +569,36 @@ extern "C" int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools
 #define MFQ_MOE_LAUNCH(KERNEL, GRID, BLOCK, LDS)                                                                      \
     hipLaunchKernelGGL(KERNEL, GRID, BLOCK, LDS, st, P, expert_pool, expert_local, E, out_per_expert, xp, ldx,      \
                        routed_input, ids, n_pairs, R, ids_dst, expert_bounds, tile_bounds, tile_experts, out, ldo)
+    // many pairs per expert: the paired cohorts go through the prefill kernel, 64 pairs of an expert per block
+    const int x_rows = routed_input ? n_pairs : T;
+    if (mfma && mapped && workspace && n_pairs >= 24ll * E && moe_prefill_pools(pools, n_pools) &&
+        workspace_bytes >= mfq_hip_moe_grouped_workspace_bytes(pools, n_pools, K, x_rows)) {
+        const int Kp = moe_kp(K);
+        uint8_t *p = static_cast<uint8_t *>(workspace);
+        uint16_t *x16 = reinterpret_cast<uint16_t *>(p);
+        p += moe_align256(static_cast<size_t>(x_rows) * Kp * 2);
+        float *xscale = reinterpret_cast<float *>(p);
+        p += moe_align256(static_cast<size_t>(x_rows) * 4);
+        int max_gs = 16;
+        for (int i = 0; i < n_pools; ++i) {
+            P.prefill[i] = 1;
+            for (int j = 0; j < i; ++j)
+                if (P.k[j].gs == P.k[i].gs) P.xg[i] = P.xg[j];
+            if (!P.xg[i]) {
+                uint32_t *xg = reinterpret_cast<uint32_t *>(p);
+                p += moe_align256(static_cast<size_t>(x_rows) * P.k[i].nsteps * 64);
+                const int rc = x_prep_groups(x, x_dtype, ldx, x_rows, K, Kp, x16, xscale, P.k[i].gs, P.k[i].nsteps, xg, st);
+                if (rc) return rc;
+                P.xg[i] = xg;
+            }
+            if (P.k[i].gs > max_gs) max_gs = P.k[i].gs;
+        }
+        const size_t plds = 512 + static_cast<size_t>(2 * 64) * (4 * ((max_gs + 7) / 8 * 8) + 8) * 2;
+        const dim3 pgrid(static_cast<unsigned>(tiles), static_cast<unsigned>(ceil_div(rbe, 32)));
+        hipLaunchKernelGGL(moe_prefill_kernel, pgrid, dim3(512), plds, st, P, expert_pool, expert_local, E, out_per_expert, x16,
+                           Kp, xscale, routed_input, R, ids_dst, expert_bounds, tile_bounds, tile_experts, out, ldo);
+        return check_launch("moe_prefill");
+    }
     if (mfma) {
         // row-blocks per wave: 4 while the grid still has a few thousand waves, else 1
         const int64_t live_tiles = mapped ? ceil_div(n_pairs, kMoeTileM) : n_pairs;

@@ -294,7 +294,7 @@ static int launch_mfma(const NintK &k, const uint8_t *w, const uint16_t *x, int6
 
 // ---- prefill: block-tiled MFMA GEMM with in-register dequantization ---------------------------
 bool nint_prefill_capable(const mfq_nint_desc *d) {
-    return d->kind == 1 && d->neuron_len >= 8 && 4 * d->rowblock_bytes < (1ll << 31);
+    return (d->kind == 1 || (d->bits == 5 && d->gs == 28)) && d->neuron_len >= 8 && 4 * d->rowblock_bytes < (1ll << 31);
 }
 size_t nint_prefill_xg_bytes(const mfq_nint_desc *d, int M) { return static_cast<size_t>(M) * d->nsteps * 64; }
 
@@ -303,12 +303,12 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
                  uint32_t *xg, int M, float *y, int64_t ldy, hipStream_t st) {
     const NintK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
-#define MFQ_PREFILL_CFG(B, G, MT, NB, WM, NW)                                                                  \
+#define MFQ_PREFILL_CFG(UNIT, B, G, MT, NB, WM, NW)                                                                 \
     {                                                                                                          \
         const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, (NW / WM) * NB)),                        \
                         static_cast<unsigned>(ceil_div(M, WM * MT * 16)));                                     \
-        const size_t lds = static_cast<size_t>(2 * WM * MT * 16) * (4 * G + 8) * 2;                            \
-        auto kern = nint_prefill_kernel<PairedUnit<B, G>, MT, NB, WM, NW>;                                     \
+        const size_t lds = static_cast<size_t>(2 * WM * MT * 16) * (4 * ((G + 7) / 8 * 8) + 8) * 2;            \
+        auto kern = nint_prefill_kernel<UNIT<B, G>, MT, NB, WM, NW>;                                           \
         if (lds > 65536) {                                                                                     \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                           \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
@@ -320,13 +320,18 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
     // wave tile MT*16 tokens x NB*16 neurons, NW waves side by side on the neurons
     // 512 neurons per block; 256 when that leaves CUs without a block
     const bool narrow = ceil_div(k.n_rowblocks, 32) * ceil_div(M, 64) < 256;
-#define MFQ_PREFILL(B, G)                              \
-    if (k.bits == B && k.gs == G) {                    \
-        if (narrow) MFQ_PREFILL_CFG(B, G, 4, 2, 1, 8)  \
-        MFQ_PREFILL_CFG(B, G, 4, 4, 1, 8)              \
+#define MFQ_PREFILL(UNIT, B, G)                              \
+    if (k.bits == B && k.gs == G) {                          \
+        if (narrow) MFQ_PREFILL_CFG(UNIT, B, G, 4, 2, 1, 8)  \
+        MFQ_PREFILL_CFG(UNIT, B, G, 4, 4, 1, 8)              \
     }
-    MFQ_PREFILL(4, 32) MFQ_PREFILL(4, 24) MFQ_PREFILL(4, 16) MFQ_PREFILL(4, 48) MFQ_PREFILL(3, 24) MFQ_PREFILL(2, 16)
-    MFQ_PREFILL(2, 32)
+    if (k.kind == 1) {
+        MFQ_PREFILL(PairedUnit, 4, 32) MFQ_PREFILL(PairedUnit, 4, 24) MFQ_PREFILL(PairedUnit, 4, 16)
+        MFQ_PREFILL(PairedUnit, 4, 48) MFQ_PREFILL(PairedUnit, 3, 24) MFQ_PREFILL(PairedUnit, 2, 16)
+        MFQ_PREFILL(PairedUnit, 2, 32)
+    } else {
+        MFQ_PREFILL(GenericUnit, 5, 28)
+    }
 #undef MFQ_PREFILL
 #undef MFQ_PREFILL_CFG
     return fail(MFQ_ERR_UNSUPPORTED, "nint_prefill: no kernel for NINT%d-%d", k.bits, k.gs);

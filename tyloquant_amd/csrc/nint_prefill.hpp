@@ -13,30 +13,47 @@
 
 namespace mfq {
 
-// xg: the group sums x_prep leaves, [token][step][kb] x 16 bytes (see gemm.hip).
-template <class U, int MT, int NB, int WM, int NW>
-__global__ __launch_bounds__(64 * NW) void nint_prefill_kernel(NintK k, const uint8_t *__restrict__ w,
-                                                           const uint16_t *__restrict__ x16, int Kp,
-                                                           const float *__restrict__ xscale,
-                                                           const uint32_t *__restrict__ xg, int M,
-                                                           float *__restrict__ y, int64_t ldy) {
+// Rows of a block tile: src(i) = row of x16 / xscale / xg that tile row i reads (always valid), dst(i) = row of y it
+// writes or -1.
+struct DenseRows {
+    int tok0, M;
+    __device__ __forceinline__ int src(int i) const { return min(tok0 + i, M - 1); }
+    __device__ __forceinline__ int dst(int i) const { return tok0 + i < M ? tok0 + i : -1; }
+};
+struct MappedRows {  // both tables live in LDS
+    const int *srcv, *dstv;
+    __device__ __forceinline__ int src(int i) const { return srcv[i]; }
+    __device__ __forceinline__ int dst(int i) const { return dstv[i]; }
+};
+
+// One block: tile rows `rows`, neurons of the row-blocks [rb_base, rb_base + WN * NB) below rb_end; y column of a
+// neuron = (row-block - rb_col0) * 16 + r, stored when below ncols.  xg: the group sums x_prep leaves,
+// [row][step][kb] x 16 bytes (see gemm.hip).  xt: LDS, two buffers of [BM][4 * GS + 8] halves.
+template <class U, int MT, int NB, int WM, int NW, class Rows>
+__device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t *__restrict__ w, int rb_base, int rb_end,
+                                                  int rb_col0, int ncols, const uint16_t *__restrict__ x16, int Kp,
+                                                  const float *__restrict__ xscale, const uint32_t *__restrict__ xg,
+                                                  const Rows &rows, float *__restrict__ y, int64_t ldy, uint16_t *xt) {
     constexpr int D = U::D, GS = U::GROUP, NM = U::NPAIR / 4, BITS = U::CBITS;
     constexpr int NCLS = BITS == 0 ? 1 : (BITS == 3 ? 3 : 2);
     constexpr int WN = NW / WM;                // waves along the neurons
     constexpr int NT = 64 * NW;                // threads
     constexpr int BM = WM * MT * 16;           // tokens per block
-    constexpr int ROW = 4 * GS + 8;            // LDS row stride in halves (16 bytes of padding)
-    constexpr int CHUNKS = 4 * GS / 8;         // 16-byte chunks per tile row
+    constexpr int EL = GS % 8 == 0 ? 8 : 4;    // halves per copy chunk (16 or 8 bytes)
+    constexpr int GSP = (GS + 7) / 8 * 8;      // group width in LDS: fragments stay 16-byte aligned
+    constexpr int ROW = 4 * GSP + 8;           // LDS row stride in halves (16 bytes of padding)
+    constexpr int CPG = GS / EL;               // chunks per group
+    constexpr int CHUNKS = 4 * CPG;            // chunks per tile row
     constexpr int PER_THREAD = (BM * CHUNKS + NT - 1) / NT;
-    extern __shared__ __attribute__((aligned(16))) uint16_t xt[];  // two buffers of [BM][ROW]
+    static_assert(GS % EL == 0, "groupsize must be a multiple of 4");
+    typedef uint32_t chunk_t __attribute__((ext_vector_type(EL / 2)));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WM, wn = wave / WM;
     const int r = lane & 15, kb = lane >> 4;
-    const int tok0 = blockIdx.y * BM;
-    const int rb0 = (blockIdx.x * WN + wn) * NB;
-    const int nrb = max(0, min(NB, k.n_rowblocks - rb0));
+    const int rb0 = rb_base + wn * NB;
+    const int nrb = max(0, min(NB, rb_end - rb0));
     const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
     const __amdgpu_buffer_rsrc_t win =
         wave_window(w + static_cast<int64_t>(min(rb0, k.n_rowblocks - 1)) * k.rowblock_bytes, nrb * rbb);
@@ -48,18 +65,18 @@ __global__ __launch_bounds__(64 * NW) void nint_prefill_kernel(NintK k, const ui
         for (int b = 0; b < NB; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // global -> register copy of the activation tile of sub-step `it` (chunk c of a row = 8 halves at k0 + 8 c)
-    u32x4_t xr[PER_THREAD];
+    chunk_t xr[PER_THREAD];
     auto xload = [&](int it) {
         const int k0 = it * 4 * GS;
 #pragma unroll
         for (int p = 0; p < PER_THREAD; ++p) {
             const int c = min(tid + NT * p, BM * CHUNKS - 1);
             const int row = c / CHUNKS, ch = c - row * CHUNKS;
-            const int m = min(tok0 + row, M - 1);
-            const int kk = k0 + 8 * ch;
-            const int kc = min(kk, Kp - 8);
-            u32x4_t v = *reinterpret_cast<const u32x4_t *>(x16 + static_cast<int64_t>(m) * Kp + kc);
-            if (kk >= Kp) v = u32x4_t{0u, 0u, 0u, 0u};
+            const int m = rows.src(row);
+            const int kk = k0 + EL * ch;  // groups are contiguous in k: chunk ch of the row starts here
+            const int kc = min(kk, Kp - EL);
+            chunk_t v = *reinterpret_cast<const chunk_t *>(x16 + static_cast<int64_t>(m) * Kp + kc);
+            if (kk >= Kp) v = chunk_t(0u);
             xr[p] = v;
         }
     };
@@ -68,9 +85,15 @@ __global__ __launch_bounds__(64 * NW) void nint_prefill_kernel(NintK k, const ui
         for (int p = 0; p < PER_THREAD; ++p) {
             const int c = tid + NT * p;
             const int row = c / CHUNKS, ch = c - row * CHUNKS;
-            if (c < BM * CHUNKS) *reinterpret_cast<u32x4_t *>(xt + buf * (BM * ROW) + row * ROW + 8 * ch) = xr[p];
+            const int g = ch / CPG, ci = ch - g * CPG;
+            if (c < BM * CHUNKS)
+                *reinterpret_cast<chunk_t *>(xt + buf * (BM * ROW) + row * ROW + g * GSP + EL * ci) = xr[p];
         }
     };
+    if constexpr (GSP != GS) {  // the padding halves of a group are multiplied by zero weights: keep them finite
+        for (int i = tid; i < 2 * BM * ROW / 2; i += NT) reinterpret_cast<uint32_t *>(xt)[i] = 0u;
+        __syncthreads();
+    }
 
     uint32_t q[NB][D], qn[NB][D], tails[NB], tailsn[NB];
     u32x2_t sc[NB], scn[NB];
@@ -126,7 +149,7 @@ __global__ __launch_bounds__(64 * NW) void nint_prefill_kernel(NintK k, const ui
             u32x4_t af[MT];
 #pragma unroll
             for (int a = 0; a < MT; ++a)
-                af[a] = *reinterpret_cast<const u32x4_t *>(xt + (j & 1) * (BM * ROW) + ((wm * MT + a) * 16 + r) * ROW + kb * GS + 8 * m);
+                af[a] = *reinterpret_cast<const u32x4_t *>(xt + (j & 1) * (BM * ROW) + ((wm * MT + a) * 16 + r) * ROW + kb * GSP + 8 * m);
             // all weight fragments of this k-slice first, then the MFMAs back to back: while one wave's MFMAs run,
             // the other wave of the SIMD unpacks
             u32x4_t bf[NB];
@@ -173,7 +196,7 @@ __global__ __launch_bounds__(64 * NW) void nint_prefill_kernel(NintK k, const ui
     int64_t xgrow[MT];
 #pragma unroll
     for (int a = 0; a < MT; ++a)
-        xgrow[a] = static_cast<int64_t>(min(tok0 + (wm * MT + a) * 16 + r, M - 1)) * k.nsteps * 16 + kb * 4;
+        xgrow[a] = static_cast<int64_t>(rows.src((wm * MT + a) * 16 + r)) * k.nsteps * 16 + kb * 4;
     u32x4_t ax[MT], axn[MT];
     auto gload = [&](int s, u32x4_t (&dst)[MT]) {
         const int sc_ = min(s, k.nsteps - 1);
@@ -203,16 +226,31 @@ __global__ __launch_bounds__(64 * NW) void nint_prefill_kernel(NintK k, const ui
     for (int a = 0; a < MT; ++a) {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            const int m = tok0 + (wm * MT + a) * 16 + 4 * kb + v;
-            if (m >= M) continue;
-            const float xs = xscale[m];
+            const int ti = (wm * MT + a) * 16 + 4 * kb + v;
+            const int m = rows.dst(ti);
+            if (m < 0) continue;
+            const float xs = xscale[rows.src(ti)];
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
-                const int row = (rb0 + b) * 16 + r;
-                if (row < k.out) y[static_cast<int64_t>(m) * ldy + row] = xs * (ns[b] * acc[a][b][v] - nm[b] * accM[a][b][v]);
+                const int col = (rb0 + b - rb_col0) * 16 + r;
+                if (rb0 + b < rb_end && col < ncols)
+                    y[static_cast<int64_t>(m) * ldy + col] = xs * (ns[b] * acc[a][b][v] - nm[b] * accM[a][b][v]);
             }
         }
     }
+}
+
+// Dense wrapper: block (neuron tile, token tile).
+template <class U, int MT, int NB, int WM, int NW>
+__global__ __launch_bounds__(64 * NW) void nint_prefill_kernel(NintK k, const uint8_t *__restrict__ w,
+                                                               const uint16_t *__restrict__ x16, int Kp,
+                                                               const float *__restrict__ xscale,
+                                                               const uint32_t *__restrict__ xg, int M,
+                                                               float *__restrict__ y, int64_t ldy) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t xt[];
+    const DenseRows rows{static_cast<int>(blockIdx.y) * WM * MT * 16, M};
+    nint_prefill_body<U, MT, NB, WM, NW>(k, w, static_cast<int>(blockIdx.x) * (NW / WM) * NB, k.n_rowblocks, 0, k.out, x16, Kp,
+                                         xscale, xg, rows, y, ldy, xt);
 }
 
 }  // namespace mfq

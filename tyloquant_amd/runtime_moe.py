@@ -9,7 +9,7 @@ import torch
 
 from . import _lib as L
 from . import formats as F
-from .runtime import NintWeight, _ptr, _stream, _x_dtype, nint_matmul
+from .runtime import NintWeight, _Workspace, _ptr, _stream, _x_dtype, nint_matmul
 
 _MODE = {"softmax": L.TOPK_SOFTMAX, "sigmoid": L.TOPK_SIGMOID, "sqrt_softplus": L.TOPK_SQRT_SOFTPLUS,
          "delayed_softmax": L.TOPK_DELAYED_SOFTMAX}
@@ -108,6 +108,7 @@ class NintMoeWeight:
         for i, p in enumerate(pools):
             self._pool_array[i].desc = p.desc
             self._pool_array[i].weight = p.data.data_ptr()
+        self._ws = _Workspace()
         self.expert_bits = np.zeros(n_experts, dtype=np.int32)
         for pi, ids in enumerate(expert_ids):
             self.expert_bits[ids] = pools[pi].bits
@@ -158,12 +159,17 @@ class NintMoeWeight:
             x2 = x2.contiguous()
         out = torch.empty((T, R, self.out_per_expert), dtype=torch.float32, device=x.device)
         mapped = route.ids_dst is not None
-        L.check(L.lib().mfq_hip_moe_grouped_matmul(
+        lib = L.lib()
+        # a workspace unlocks the prefill kernel for mapped calls with many pairs per expert
+        need = lib.mfq_hip_moe_grouped_workspace_bytes(self._pool_array, len(self.pools), self.neuron_len,
+                                                       x2.shape[0]) if mapped and T * R >= 24 * self.n_experts else 0
+        ws = self._ws.get(need, x.device)
+        L.check(lib.mfq_hip_moe_grouped_matmul_ws(
             self._pool_array, len(self.pools), _ptr(self.expert_pool), _ptr(self.expert_local), self.n_experts,
             self.out_per_expert, self.neuron_len, _ptr(x2), _x_dtype(x2), x2.stride(0), int(routed), _ptr(route.ids),
             T, R, _ptr(route.ids_dst) if mapped else None, _ptr(route.expert_bounds) if mapped else None,
             _ptr(route.tile_bounds) if mapped else None, _ptr(route.tile_experts) if mapped else None,
-            _ptr(out), self.out_per_expert, _stream()))
+            _ptr(out), self.out_per_expert, _ptr(ws), need, _stream()))
         return out
 
     __call__ = forward
