@@ -204,9 +204,8 @@ int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools, const int
                                const int32_t *tile_bounds, const int32_t *tile_experts,
                                float *out, int64_t ldo, mfq_stream_t stream);
 
-/* The same with a workspace, which unlocks the prefill kernel when a mapped call carries many pairs per
- * expert (64 pairs of an expert against 512 neurons per block; activations pre-scaled to fp16 in the
- * workspace).  x_rows = T * R with routed_input, else T.  The size query returns 0 when the cohorts have no
+/* The same with a workspace, which lets mapped calls run the prefill kernel (64 pairs of an expert against
+ * 512 neurons per block; activations pre-scaled to fp16 in the workspace).  x_rows = T * R with routed_input, else T.  The size query returns 0 when the cohorts have no
  * prefill kernel; a NULL or short workspace simply keeps the streaming kernels.  No counterpart in the
  * reference, whose hetero kernels allocate their workspace through torch
  * (cpp_runtime/mfq_decode.cpp:3008-3016). */

@@ -105,6 +105,29 @@ def test_grouped_matmul_prefill_path_many_pairs_per_expert(routed):
     assert np.all(got[7, 1] == 0)
 
 
+def test_grouped_matmul_without_workspace_keeps_the_streaming_kernels():
+    """The plain entry point (no workspace) runs mapped calls on the streaming kernels; same result as the prefill path."""
+    import ctypes as C
+    from tyloquant_amd import _lib as L
+    from tyloquant_amd.runtime_moe import build_moe_route_plan
+    rng = np.random.default_rng(78)
+    E, out, K, T, R = 6, 48, 512, 40, 2
+    t, w = _moe(rng, E, out, K, [4, 3, 2, 5, 4, 3])
+    ids = rng.integers(0, E, (T, R)).astype(np.int32)
+    x = torch.from_numpy((rng.standard_normal((T, K)) * 0.1).astype(np.float32)).to(torch.bfloat16).cuda()
+    route = build_moe_route_plan(torch.from_numpy(ids).cuda(), E)
+    with_ws = w(x, route)
+    plain = torch.empty_like(with_ws)
+    p = lambda t_: C.c_void_p(t_.data_ptr())
+    L.check(L.lib().mfq_hip_moe_grouped_matmul(
+        w._pool_array, len(w.pools), p(w.expert_pool), p(w.expert_local), E, out, K, p(x), L.X_BF16, K, 0, p(route.ids), T, R,
+        p(route.ids_dst), p(route.expert_bounds), p(route.tile_bounds), p(route.tile_experts), p(plain), out, None))
+    torch.cuda.synchronize()
+    ref = O.moe_grouped_matmul(O.dequantize_expertwise(t), x.float().cpu().numpy(), ids)
+    for got in (with_ws.cpu().numpy(), plain.cpu().numpy()):
+        assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL
+
+
 def test_grouped_matmul_routed_input_and_invalid_expert():
     from tyloquant_amd.runtime_moe import build_moe_route_plan
     rng = np.random.default_rng(44)

@@ -407,10 +407,10 @@ NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream
 void NintMoeWeight::forward(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &r, float *out,
                             mfq_stream_t stream) const {
     const bool mapped = r.mapped();
-    // a workspace unlocks the prefill kernel for mapped calls with many pairs per expert
+    // a workspace lets the library take the prefill kernel when a mapped call has many pairs per expert
     const int x_rows = routed_input ? r.tokens * r.routes : r.tokens;
     size_t need = 0;
-    if (mapped && static_cast<int64_t>(r.tokens) * r.routes >= 24ll * n_experts)
+    if (mapped)
         need = mfq_hip_moe_grouped_workspace_bytes(pool_table.data(), static_cast<int>(pool_table.size()), neuron_len, x_rows);
     if (need) workspace.ensure(need);
     abi_check(mfq_hip_moe_grouped_matmul_ws(

@@ -569,9 +569,11 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
 #define MFQ_MOE_LAUNCH(KERNEL, GRID, BLOCK, LDS)                                                                      \
     hipLaunchKernelGGL(KERNEL, GRID, BLOCK, LDS, st, P, expert_pool, expert_local, E, out_per_expert, xp, ldx,      \
                        routed_input, ids, n_pairs, R, ids_dst, expert_bounds, tile_bounds, tile_experts, out, ldo)
-    // many pairs per expert: the paired cohorts go through the prefill kernel, 64 pairs of an expert per block
+    // mapped calls with a workspace go through the prefill kernel, 64 pairs of an expert per block (faster than the
+    // streaming kernel from about one pair per expert on; MFQ_MOE_PREFILL_PAIRS raises the threshold for tuning)
     const int x_rows = routed_input ? n_pairs : T;
-    if (mfma && mapped && workspace && n_pairs >= 24ll * E && moe_prefill_pools(pools, n_pools) &&
+    static const int min_pairs = [] { const char *e = getenv("MFQ_MOE_PREFILL_PAIRS"); return e ? atoi(e) : 0; }();
+    if (mfma && mapped && workspace && n_pairs >= static_cast<int64_t>(min_pairs) * E && moe_prefill_pools(pools, n_pools) &&
         workspace_bytes >= mfq_hip_moe_grouped_workspace_bytes(pools, n_pools, K, x_rows)) {
         const int Kp = moe_kp(K);
         uint8_t *p = static_cast<uint8_t *>(workspace);

@@ -160,9 +160,9 @@ class NintMoeWeight:
         out = torch.empty((T, R, self.out_per_expert), dtype=torch.float32, device=x.device)
         mapped = route.ids_dst is not None
         lib = L.lib()
-        # a workspace unlocks the prefill kernel for mapped calls with many pairs per expert
+        # a workspace lets the library take the prefill kernel when a mapped call has many pairs per expert
         need = lib.mfq_hip_moe_grouped_workspace_bytes(self._pool_array, len(self.pools), self.neuron_len,
-                                                       x2.shape[0]) if mapped and T * R >= 24 * self.n_experts else 0
+                                                       x2.shape[0]) if mapped else 0
         ws = self._ws.get(need, x.device)
         L.check(lib.mfq_hip_moe_grouped_matmul_ws(
             self._pool_array, len(self.pools), _ptr(self.expert_pool), _ptr(self.expert_local), self.n_experts,
