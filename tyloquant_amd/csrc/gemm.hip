@@ -3,6 +3,8 @@
 // fp16 x fp16 -> fp32 MFMA GEMM (v_mfma_f32_32x32x16_f16) produces y; the epilogue multiplies
 // the two power-of-two scales back.  fp16 (11 significant bits) keeps the weight rounding error
 // near 1e-4 relative, which bf16 tiles (8 bits) cannot.
+#include <stdlib.h>
+
 #include "common.hpp"
 
 namespace mfq {
@@ -228,10 +230,15 @@ extern "C" int mfq_hip_gemm_f16_nt(const void *a, int64_t lda, const void *b, in
 
 // Up to kGemvMaxM activation rows the weight stream dominates and the GEMV kernels win; tensors with a
 // matrix-core streaming kernel (16 rows per pass over the packed weights) stay on it up to kStreamMaxM rows,
-// where re-streaming the weights is still cheaper than dequantizing them to fp16 once.
+// where re-streaming the weights is still cheaper than dequantizing them to fp16 once, or up to the measured
+// crossover with the prefill kernel.
 static constexpr int kGemvMaxM = 8, kStreamMaxM = 256;
 static bool nint_streams(const mfq_nint_desc *d, int M) {
-    return M <= kGemvMaxM || (M <= kStreamMaxM && nint_stream_capable(d));
+    static const int env_max = [] { const char *e = getenv("MFQ_STREAM_MAX_M"); return e ? atoi(e) : 0; }();
+    // the prefill kernel takes over earlier when it has enough neurons to fill the chip with 512-neuron blocks
+    int stream_max = nint_prefill_capable(d) ? (d->out >= 8192 ? 128 : 192) : kStreamMaxM;
+    if (env_max > 0) stream_max = env_max;
+    return M <= kGemvMaxM || (M <= stream_max && nint_stream_capable(d));
 }
 
 // prefill workspace: x16 [M, Kp] | xscale [M] | group sums
