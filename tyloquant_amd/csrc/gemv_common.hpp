@@ -125,12 +125,12 @@ struct XRegs {
 
 // First half of the staging: request the wave's K-slice of the activation rows into registers.  Issued
 // before the weight loads so that (loads retiring in order) the staging never waits for weights.  Only the
-// common case is prefetched -- aligned rows, slice wholly inside K, at most 256 * kXChunks pairs, MB <= 2;
-// anything else is fetched by stage_x itself.
+// common case is prefetched -- aligned rows, K % 8 == 0, at most 256 * kXChunks pairs, MB <= 2; anything
+// else is fetched by stage_x itself.
 template <int MB>
 __device__ __forceinline__ void stage_x_issue(const uint16_t *const (&xr)[MB], int K, int k0, int npairs, int lane,
                                               XRegs<MB> &xg) {
-    bool ok = MB <= 2 && npairs <= 256 * kXChunks && k0 + 2 * npairs <= K;
+    bool ok = MB <= 2 && npairs <= 256 * kXChunks && K % 8 == 0;  // K % 8: no 8-element chunk straddles the end
 #pragma unroll
     for (int m = 0; m < MB; ++m) ok = ok && (reinterpret_cast<uintptr_t>(xr[m]) & 15) == 0;
     xg.on = ok;
@@ -140,10 +140,10 @@ __device__ __forceinline__ void stage_x_issue(const uint16_t *const (&xr)[MB], i
 #pragma unroll
             for (int c = 0; c < kXChunks; ++c) {
                 const int i = lane * 4 + c * 256;
-                const int ii = i < npairs ? i : 0;
+                const bool in = i < npairs && k0 + 2 * i + 8 <= K;  // else: a zero chunk, read from a safe place
                 u32x4_t v = {0u, 0u, 0u, 0u};
-                if (xr[m]) v = *reinterpret_cast<const u32x4_t *>(xr[m] + k0 + 2 * ii);
-                xg.v[m][c] = v;
+                if (xr[m]) v = *reinterpret_cast<const u32x4_t *>(xr[m] + (in ? k0 + 2 * i : 0));
+                xg.v[m][c] = in ? v : u32x4_t{0u, 0u, 0u, 0u};
             }
         }
     }

@@ -209,19 +209,20 @@ struct MoePools {
     const uint32_t *xg[kMaxPools];  // prefill path: group sums of the activations for this cohort's groupsize
     int spw[kMaxPools];
     int n;
-    int prefill[kMaxPools];  // cohort runs on the prefill kernel in this call (the streaming kernel skips it)
+    int prefill[kMaxPools];  // cohort is taken by another kernel of this call (the streaming kernel skips it)
 };
 
 constexpr int kMoeTileM = 16;  // (token, route) pairs of one expert per tile of the route map
 
-// One cohort dispatch of the vector-ALU path: MB pairs of one expert, one 16-neuron row-block.
-template <int XF16, int MB>
+// One cohort dispatch of the vector-ALU path: MB pairs of one expert, one 16-neuron row-block.  RING = false
+// when no wave has more than three steps.
+template <int XF16, int MB, bool RING>
 __device__ __forceinline__ void moe_valu_chunk(const NintK &k, const uint8_t *w, int rb, int row_base, int out_per_expert,
                                                const uint16_t *const (&xr)[MB], float *const (&yr)[MB], int spw,
                                                uint32_t *lds) {
 #define MFQ_MOE_CASE(B, G)                                                                                    \
     if (k.bits == B && k.gs == G) {                                                                           \
-        nint_paired_body<B, G, XF16, MB>(k, w, rb, 1, row_base, out_per_expert, xr, yr, spw, lds);            \
+        nint_paired_body<B, G, XF16, MB, RING>(k, w, rb, 1, row_base, out_per_expert, xr, yr, spw, lds);            \
         return;                                                                                               \
     }
     if (k.kind == 1) {
@@ -234,8 +235,8 @@ __device__ __forceinline__ void moe_valu_chunk(const NintK &k, const uint8_t *w,
 
 // Vector-ALU path (any NINT profile, any K).  Without a route map every pair is its own tile (MB = 1,
 // decode); with one, tile t holds pairs ids_dst[lo .. lo + kMoeTileM), taken MB at a time.
-template <int XF16, int MB>
-__global__ __launch_bounds__(1024) void moe_grouped_kernel(MoePools P, const int32_t *__restrict__ expert_pool,
+template <int XF16, int MB, bool RING>
+__global__ __launch_bounds__(512) void moe_grouped_kernel(MoePools P, const int32_t *__restrict__ expert_pool,
                                                            const int32_t *__restrict__ expert_local, int E,
                                                            int out_per_expert, const uint16_t *__restrict__ x,
                                                            int64_t ldx, int routed_input, const int32_t *__restrict__ ids,
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(1024) void moe_grouped_kernel(MoePools P, const int
                                                            const int32_t *__restrict__ tile_experts,
                                                            float *__restrict__ out, int64_t ldo) {
     extern __shared__ uint32_t lds[];
-    const int tile = blockIdx.x;
+    const int tile = blockIdx.y;  // row-blocks run fastest, so that the blocks of one tile spread over the XCDs
     int e, lo = 0, hi = 0;
     if (ids_dst == nullptr) {
         e = ids[tile];
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(1024) void moe_grouped_kernel(MoePools P, const int
         lo = expert_bounds[e] + (tile - tile_bounds[e]) * kMoeTileM;
         hi = min(expert_bounds[e + 1], lo + kMoeTileM);
     }
-    const int rbl = blockIdx.y;  // row-block inside the expert
+    const int rbl = blockIdx.x;  // row-block inside the expert
     const bool valid = e >= 0 && e < E && expert_pool[e] >= 0;
     for (int c = 0; c == 0 || lo + c < hi; c += MB) {
         int pairs[MB];
@@ -279,10 +280,51 @@ __global__ __launch_bounds__(1024) void moe_grouped_kernel(MoePools P, const int
         }
         const int pool = expert_pool[e];
         const int row_base = expert_local[e] * out_per_expert;
-        moe_valu_chunk<XF16, MB>(P.k[pool], P.w[pool], row_base / 16 + rbl, row_base, out_per_expert, xr, yr, P.spw[pool],
+        moe_valu_chunk<XF16, MB, RING>(P.k[pool], P.w[pool], row_base / 16 + rbl, row_base, out_per_expert, xr, yr, P.spw[pool],
                                  lds);
         __syncthreads();  // the next chunk reuses the reduction area
     }
+}
+
+// Batch-1 path (no route map): block (group of rbw row-blocks, pair), the body of the dense GEMV with the unit
+// of the pair's cohort.  P.spw: steps per wave of each cohort; RING = false when no wave has more than three
+// (row-block, step) items.
+template <int XF16, bool RING>
+__global__ __launch_bounds__(1024) void moe_decode_kernel(MoePools P, int rbw, const int32_t *__restrict__ expert_pool,
+                                                          const int32_t *__restrict__ expert_local, int E,
+                                                          int out_per_expert, const uint16_t *__restrict__ x, int64_t ldx,
+                                                          int routed_input, const int32_t *__restrict__ ids, int R,
+                                                          float *__restrict__ out, int64_t ldo) {
+    extern __shared__ uint32_t lds[];
+    const int pair = blockIdx.y;
+    const int e = ids[pair];
+    const int rbl0 = blockIdx.x * rbw;
+    float *yrow = out + static_cast<int64_t>(pair) * ldo;
+    if (e < 0 || e >= E || expert_pool[e] < 0) {  // invalid expert id: defined as a zero row
+        for (int c = threadIdx.x; c < rbw * 16; c += blockDim.x) yrow[rbl0 * 16 + c] = 0.f;
+        return;
+    }
+    const int pool = expert_pool[e];
+    const NintK &k = P.k[pool];
+    const uint8_t *w = P.w[pool];
+    const int spw = P.spw[pool];
+    const int row_base = expert_local[e] * out_per_expert;
+    const uint16_t *xrow = x + static_cast<int64_t>(routed_input ? pair : pair / R) * ldx;
+    const uint16_t *xr[1] = {xrow};
+    float *yr[1] = {yrow};
+    if (k.kind == 1) {
+#define MFQ_MOE_CASE(B, G)                                                                                             \
+    if (k.bits == B && k.gs == G) {                                                                                    \
+        nint_paired_body<B, G, XF16, 1, RING>(k, w, row_base / 16 + rbl0, rbw, row_base, out_per_expert, xr, yr, spw, lds); \
+        return;                                                                                                        \
+    }
+        MFQ_MOE_CASE(4, 24) MFQ_MOE_CASE(3, 24) MFQ_MOE_CASE(2, 16) MFQ_MOE_CASE(4, 32) MFQ_MOE_CASE(4, 16)
+        MFQ_MOE_CASE(4, 48) MFQ_MOE_CASE(2, 32)
+#undef MFQ_MOE_CASE
+        return;
+    }
+    nint_unit_body<GenericUnit<5, 28>, XF16, 1, RING>(k, w, row_base / 16 + rbl0, rbw, row_base, out_per_expert, xr, yr, spw,
+                                                      lds);
 }
 
 // Matrix-core path: a tile of up to 16 pairs of one expert against NB row-blocks, weights streamed once
@@ -300,7 +342,7 @@ __global__ __launch_bounds__(512) void moe_mfma_kernel(MoePools P, const int32_t
                                                        float *__restrict__ out, int64_t ldo) {
     extern __shared__ uint32_t lds[];
     float *red = reinterpret_cast<float *>(lds);
-    const int tile = blockIdx.x;
+    const int tile = blockIdx.y;  // row-blocks run fastest, so that the blocks of one tile spread over the XCDs
     int e, lo = 0, hi = 0;
     if (ids_dst == nullptr) {
         e = ids[tile];
@@ -310,7 +352,7 @@ __global__ __launch_bounds__(512) void moe_mfma_kernel(MoePools P, const int32_t
         lo = expert_bounds[e] + (tile - tile_bounds[e]) * kMoeTileM;
         hi = min(expert_bounds[e + 1], lo + kMoeTileM);
     }
-    const int rbe = out_per_expert / 16, rbl0 = blockIdx.y * NB;
+    const int rbe = out_per_expert / 16, rbl0 = blockIdx.x * NB;
     auto pair_of = [&](int slot) -> int {  // -1 = empty slot
         if (ids_dst == nullptr) return slot == 0 ? tile : -1;
         return lo + slot < hi ? ids_dst[lo + slot] : -1;
@@ -544,6 +586,7 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
     MoePools P;
     P.n = n_pools;
     int max_steps = 1;
+    bool units = true;  // every cohort has a unit with GEMV, streaming and prefill bodies
     bool mfma = K >= 8 && K % 8 == 0 && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
     for (int i = 0; i < n_pools; ++i) {
         const mfq_nint_desc &d = pools[i].desc;
@@ -557,10 +600,13 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
         P.w[i] = static_cast<const uint8_t *>(pools[i].weight);
         P.xg[i] = nullptr;
         P.prefill[i] = 0;
-        mfma = mfma && (d.kind == 1 || (d.bits == 5 && d.gs == 28)) && 4 * d.rowblock_bytes < (1ll << 31);
+        units = units && moe_prefill_unit(d) && 4 * d.rowblock_bytes < (1ll << 31);
+        mfma = mfma && units;
     }
     const int rbe = out_per_expert / 16;
     const int64_t tiles = mapped ? ceil_div(n_pairs, kMoeTileM) + E : n_pairs;
+    MFQ_REQUIRE(tiles <= 65535, MFQ_ERR_UNSUPPORTED, "moe_grouped_matmul: %lld tiles in one call (max 65535)",
+                static_cast<long long>(tiles));
     hipStream_t st = as_stream(stream);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
     if (mapped)
@@ -601,15 +647,90 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
                            Kp, xscale, routed_input, R, ids_dst, expert_bounds, tile_bounds, tile_experts, out, ldo);
         return check_launch("moe_prefill");
     }
+    // vector-ALU path: one block shape for every cohort, waves = min(16, fewest steps that keeps every wave busy)
+    auto launch_valu = [&]() -> int {
+        const int mb = mapped ? 4 : 1;
+        int want = static_cast<int>(ceil_div(8192, static_cast<int64_t>(rbe) * (mapped ? ceil_div(n_pairs, mb) : n_pairs)));
+        if (want < 1) want = 1;
+        if (want > 8) want = 8;
+        if (want > max_steps) want = max_steps;
+        // with at most three steps per wave every load is in flight before the first use and the body needs no ring
+        if (!mapped && want * 3 < max_steps && max_steps <= 24) want = static_cast<int>(ceil_div(max_steps, 3));
+        const int nwaves = want;
+        const bool ring = mapped || ceil_div(max_steps, nwaves) > 3;
+        size_t lds = 0;
+        for (int i = 0; i < n_pools; ++i) {
+            P.spw[i] = static_cast<int>(ceil_div(P.k[i].nsteps, nwaves));
+            const size_t need = gemv_lds_bytes(mb, P.spw[i], P.k[i].gs, nwaves);
+            if (need > lds) lds = need;
+        }
+        MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "moe_grouped_matmul: K=%d needs %zu bytes of LDS", K, lds);
+        const dim3 grid(rbe, static_cast<unsigned>(tiles)), block(64 * nwaves);
+        if (mapped) {
+            if (x_dtype == MFQ_X_F16) MFQ_MOE_LAUNCH((moe_grouped_kernel<1, 4, true>), grid, block, lds);
+            else MFQ_MOE_LAUNCH((moe_grouped_kernel<0, 4, true>), grid, block, lds);
+        } else if (ring) {
+            if (x_dtype == MFQ_X_F16) MFQ_MOE_LAUNCH((moe_grouped_kernel<1, 1, true>), grid, block, lds);
+            else MFQ_MOE_LAUNCH((moe_grouped_kernel<0, 1, true>), grid, block, lds);
+        } else {
+            if (x_dtype == MFQ_X_F16) MFQ_MOE_LAUNCH((moe_grouped_kernel<1, 1, false>), grid, block, lds);
+            else MFQ_MOE_LAUNCH((moe_grouped_kernel<0, 1, false>), grid, block, lds);
+        }
+        return check_launch("moe_grouped_matmul");
+    };
+    static const int split = [] { const char *e = getenv("MFQ_MOE_SPLIT"); return e ? atoi(e) : 1; }();
+    if (!mapped && units && split) {
+        // One pair per tile (no route map): one launch of the batch-1 GEMV bodies for every cohort.  Waves split
+        // the K steps; a wave takes more (row-block, step) items while the grid keeps about gemv_target_waves() waves.
+        static const int env_w = [] { const char *e = getenv("MFQ_MOE_DEC_WAVES"); return e ? atoi(e) : 16; }();
+        static const int env_rbw = [] { const char *e = getenv("MFQ_MOE_DEC_RBW"); return e ? atoi(e) : 0; }();
+        const int nwaves = max_steps < env_w ? max_steps : env_w;
+        const int spw_max = static_cast<int>(ceil_div(max_steps, nwaves));
+        int64_t items = 0;
+        for (int i = 0; i < n_pools; ++i) items += P.k[i].nsteps;
+        items = items / n_pools * rbe * n_pairs;
+        int per_wave = static_cast<int>(items / gemv_target_waves());
+        per_wave = per_wave < 1 ? 1 : (per_wave > 3 ? 3 : per_wave);
+        {
+            int rbw = per_wave / spw_max < 1 ? 1 : per_wave / spw_max;
+            if (env_rbw) rbw = env_rbw;
+            while (rbe % rbw) --rbw;
+            size_t lds = 0;
+            bool ring = false;
+            for (int i = 0; i < n_pools; ++i) {
+                P.spw[i] = static_cast<int>(ceil_div(P.k[i].nsteps, nwaves));
+                const size_t need = gemv_lds_bytes(1, P.spw[i], P.k[i].gs, nwaves, rbw);
+                if (need > lds) lds = need;
+                if (P.spw[i] * rbw > 3) ring = true;
+            }
+            if (lds <= 65536) {
+                const dim3 grid(static_cast<unsigned>(rbe / rbw), static_cast<unsigned>(n_pairs)), block(64 * nwaves);
+#define MFQ_MOE_DECODE(XF, RG)                                                                                     \
+hipLaunchKernelGGL((moe_decode_kernel<XF, RG>), grid, block, lds, st, P, rbw, expert_pool, expert_local, E,     \
+                   out_per_expert, xp, ldx, routed_input, ids, R, out, ldo)
+                if (x_dtype == MFQ_X_F16) {
+                    if (ring) MFQ_MOE_DECODE(1, true);
+                    else MFQ_MOE_DECODE(1, false);
+                } else {
+                    if (ring) MFQ_MOE_DECODE(0, true);
+                    else MFQ_MOE_DECODE(0, false);
+                }
+#undef MFQ_MOE_DECODE
+                return check_launch("moe_decode");
+            }
+        }
+    }
     if (mfma) {
         // row-blocks per wave: 4 while the grid still has a few thousand waves, else 1
         const int64_t live_tiles = mapped ? ceil_div(n_pairs, kMoeTileM) : n_pairs;
-        const bool nb4 = live_tiles * rbe * max_steps >= 4 * 2048 && rbe >= 4;
+        static const int env_nb = [] { const char *e = getenv("MFQ_MOE_NB"); return e ? atoi(e) : 0; }();
+        const bool nb4 = env_nb ? env_nb == 4 : (live_tiles * rbe * max_steps >= 4 * 2048 && rbe >= 4);
         const int nb = nb4 ? 4 : 1;
         int nwaves = max_steps < 8 ? max_steps : 8;
-        for (int i = 0; i < n_pools; ++i) P.spw[i] = static_cast<int>(ceil_div(P.k[i].nsteps, nwaves));
+        for (int i = 0; i < n_pools; ++i)
+            if (!P.prefill[i]) P.spw[i] = static_cast<int>(ceil_div(P.k[i].nsteps, nwaves));
         const size_t lds = static_cast<size_t>(nwaves) * nb * 1024;
-        const dim3 grid(static_cast<unsigned>(tiles), static_cast<unsigned>(ceil_div(rbe, nb))), block(64 * nwaves);
+        const dim3 grid(static_cast<unsigned>(ceil_div(rbe, nb)), static_cast<unsigned>(tiles)), block(64 * nwaves);
         if (x_dtype == MFQ_X_F16) {
             if (nb4) MFQ_MOE_LAUNCH((moe_mfma_kernel<1, 4>), grid, block, lds);
             else MFQ_MOE_LAUNCH((moe_mfma_kernel<1, 1>), grid, block, lds);
@@ -619,30 +740,8 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
         }
         return check_launch("moe_grouped_matmul");
     }
-    // vector-ALU path: one block shape for every cohort, waves = min(16, fewest steps that keeps every wave busy)
-    const int mb = mapped ? 4 : 1;
-    int want = static_cast<int>(ceil_div(8192, static_cast<int64_t>(rbe) * (mapped ? ceil_div(n_pairs, mb) : n_pairs)));
-    if (want < 1) want = 1;
-    if (want > 16) want = 16;
-    if (want > max_steps) want = max_steps;
-    const int nwaves = want;
-    size_t lds = 0;
-    for (int i = 0; i < n_pools; ++i) {
-        P.spw[i] = static_cast<int>(ceil_div(P.k[i].nsteps, nwaves));
-        const size_t need = gemv_lds_bytes(mb, P.spw[i], P.k[i].gs, nwaves);
-        if (need > lds) lds = need;
-    }
-    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "moe_grouped_matmul: K=%d needs %zu bytes of LDS", K, lds);
-    const dim3 grid(static_cast<unsigned>(tiles), rbe), block(64 * nwaves);
-    if (mapped) {
-        if (x_dtype == MFQ_X_F16) MFQ_MOE_LAUNCH((moe_grouped_kernel<1, 4>), grid, block, lds);
-        else MFQ_MOE_LAUNCH((moe_grouped_kernel<0, 4>), grid, block, lds);
-    } else {
-        if (x_dtype == MFQ_X_F16) MFQ_MOE_LAUNCH((moe_grouped_kernel<1, 1>), grid, block, lds);
-        else MFQ_MOE_LAUNCH((moe_grouped_kernel<0, 1>), grid, block, lds);
-    }
+    return launch_valu();
 #undef MFQ_MOE_LAUNCH
-    return check_launch("moe_grouped_matmul");
 }
 
 extern "C" int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,

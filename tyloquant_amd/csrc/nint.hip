@@ -190,6 +190,9 @@ __global__ void nint_dequant_kernel(NintK k, const uint8_t *__restrict__ w, OutT
 // without a prefetch ring holds in registers -- as long as the grid keeps about gemv_target_waves()
 // waves; long neurons spend the items on K (fewer waves to reduce), short ones on row-blocks (the
 // staged activations are reused).  MFQ_GEMV_SPW / MFQ_GEMV_RBW override the choice for tuning.
+// natural-order profiles with a unit of their own (GEMV, streaming and prefill kernels)
+static bool mfma_generic_profile(const NintK &k) { return k.kind == 0 && k.bits == 5 && k.gs == 28; }
+
 static void gemv_shape(const NintK &k, int mb, int &spw, int &nwaves, int &rbw, size_t &lds_bytes) {
     static const int env_spw = [] { const char *e = getenv("MFQ_GEMV_SPW"); return e ? atoi(e) : 0; }();
     static const int env_rbw = [] { const char *e = getenv("MFQ_GEMV_RBW"); return e ? atoi(e) : 0; }();
@@ -202,8 +205,9 @@ static void gemv_shape(const NintK &k, int mb, int &spw, int &nwaves, int &rbw, 
     if (env_spw > 0) spw = env_spw < spw_min ? spw_min : env_spw;
     if (spw > k.nsteps) spw = k.nsteps;
     nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
-    rbw = k.kind == 1 ? per_wave / spw : 1;
-    if (env_rbw > 0 && k.kind == 1) rbw = env_rbw;
+    const bool unit = k.kind == 1 || mfma_generic_profile(k);
+    rbw = unit ? per_wave / spw : 1;
+    if (env_rbw > 0 && unit) rbw = env_rbw;
     if (rbw < 1) rbw = 1;
     if (rbw > kMaxRbw) rbw = kMaxRbw;
     if (rbw > k.n_rowblocks) rbw = k.n_rowblocks;
@@ -237,15 +241,22 @@ static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, i
         return fail(MFQ_ERR_UNSUPPORTED, "nint_gemv: no paired kernel for NINT%d-%d", k.bits, k.gs);
     }
 #undef MFQ_PAIRED
+    if (mfma_generic_profile(k)) {
+        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, rbw)), static_cast<unsigned>(ceil_div(M, MB)));
+        if (spw * rbw <= 3)
+            hipLaunchKernelGGL((nint_gemv_natural_kernel<5, 28, XF16, MB, false>), grid, block, lds, st, k, w, x, ldx, M, y,
+                               ldy, spw, rbw);
+        else
+            hipLaunchKernelGGL((nint_gemv_natural_kernel<5, 28, XF16, MB, true>), grid, block, lds, st, k, w, x, ldx, M, y,
+                               ldy, spw, rbw);
+        return check_launch("nint_gemv_natural");
+    }
     const dim3 grid(k.n_rowblocks, static_cast<unsigned>(ceil_div(M, MB)));
     hipLaunchKernelGGL((nint_gemv_generic_kernel<XF16, MB>), grid, block, lds, st, k, w, x, ldx, M, y, ldy, spw);
     return check_launch("nint_gemv_generic");
 }
 
 // ---- small batches on the matrix cores ----------------------------------------------------
-// natural-order profiles with a matrix-core kernel (the paired ones all have one)
-static bool mfma_generic_profile(const NintK &k) { return k.kind == 0 && k.bits == 5 && k.gs == 28; }
-
 static bool mfma_eligible(const NintK &k, const void *x, int64_t ldx) {
     return (k.kind == 1 || mfma_generic_profile(k)) && k.neuron_len >= 8 && k.neuron_len % 8 == 0 && ldx % 8 == 0 &&
            (reinterpret_cast<uintptr_t>(x) & 15) == 0 && 4 * k.rowblock_bytes < (1ll << 31);
@@ -342,7 +353,7 @@ int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int
     const NintK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
-    if ((M >= 2 || k.kind == 0) && mfma_eligible(k, x, ldx))
+    if (M >= 2 && mfma_eligible(k, x, ldx))
         return x_dtype == MFQ_X_F16 ? launch_mfma<1>(k, w, xp, ldx, M, y, ldy, st)
                                     : launch_mfma<0>(k, w, xp, ldx, M, y, ldy, st);
     // LDS per block grows with MB; large K falls back to narrower row batches.

@@ -123,20 +123,53 @@ struct GenericUnit {
     static constexpr int D = (GS * BITS + 31) / 32;
     static constexpr bool TAIL = false;
     static constexpr int GROUP = GS, NPAIR = ((GS + 7) / 8) * 4, CBITS = 0;
+    static_assert(BITS <= 8 && GS % 2 == 0, "natural-order units hold an even number of codes of at most 8 bits");
     __device__ static __forceinline__ constexpr int cls(int) { return 0; }
+    struct Bias {  // every pair is (1024 + code): unscaled activations, T_g = 1024 * X_g
+        static constexpr bool SCALED = false;
+        __device__ static __forceinline__ float bw(int) { return 1024.f; }
+        __device__ static __forceinline__ float xscale(int, int) { return 1.f; }
+        __device__ static __forceinline__ float inv_xscale(int) { return 1.f; }
+    };
     __device__ static __forceinline__ uint32_t code(const uint32_t (&q)[D], int i) {
         const int bit = i * BITS, wi = bit >> 5, sh = bit & 31;
         uint32_t c = q[wi] >> sh;
         if (sh + BITS > 32) c |= q[wi + 1] << (32 - sh);
         return c & ((1u << BITS) - 1u);
     }
+    // Pair p = the 2 * BITS bits from bit 2 * p * BITS: extracted (through a funnel shift when they straddle two
+    // dwords), a shift-or copies the second code to bit 16, one AND-OR drops the rest and adds the magic exponent.
     __device__ static __forceinline__ void unpack(const uint32_t (&q)[D], uint32_t, uint32_t (&v)[NPAIR]) {
+        constexpr uint32_t M = (1u << BITS) - 1u;
 #pragma unroll
         for (int p = 0; p < NPAIR; ++p) {
-            uint32_t pr = kMagicH2;
-            if (2 * p < GS) pr |= code(q, 2 * p);
-            if (2 * p + 1 < GS) pr |= code(q, 2 * p + 1) << 16;
-            v[p] = pr;
+            if (2 * p >= GS) {
+                v[p] = kMagicH2;
+                continue;
+            }
+            const int bit = 2 * p * BITS, wi = bit >> 5, sh = bit & 31;
+            uint32_t win = q[wi] >> sh;
+            if (sh + 2 * BITS > 32) win = __builtin_amdgcn_alignbit(q[wi + 1], q[wi], sh);
+            win &= (1u << (2 * BITS)) - 1u;  // with the shift: one bit-field extract
+            v[p] = and_or((win << (16 - BITS)) | win, M | (M << 16), kMagicH2);
+        }
+    }
+    // acc[m] += sum over the pairs of the group of (1024 + code) . x_m; xs = the group's GS/2 staged fp16 pairs
+    // of activation row 0 in LDS (8-byte aligned when GS/2 is even), row m sits mstride dwords further.
+    template <int MB>
+    __device__ static __forceinline__ void dot(const uint32_t (&q)[D], uint32_t, const uint32_t *xs, int mstride,
+                                               float (&acc)[MB]) {
+        static_assert(GS % 4 == 0, "the staged pairs of a group are read two at a time");
+        uint32_t v[NPAIR];
+        unpack(q, 0u, v);
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+#pragma unroll
+            for (int c = 0; c < GS / 4; ++c) {
+                const u32x2_t x = *reinterpret_cast<const u32x2_t *>(xs + m * mstride + 2 * c);
+                acc[m] = dot2h(v[2 * c], x.x, acc[m]);
+                acc[m] = dot2h(v[2 * c + 1], x.y, acc[m]);
+            }
         }
     }
 };
@@ -153,11 +186,11 @@ __device__ __forceinline__ void nint_load_step(__amdgpu_buffer_rsrc_t win, uint3
     sc = __builtin_amdgcn_raw_buffer_load_b64(win, off + 1024 * D + (TAIL ? 256 : 0) + lane * 8, 0, 2);
 }
 
-template <int BITS, int GS, int MB>
-__device__ __forceinline__ void nint_compute_step(const uint32_t (&q)[4][PairedUnit<BITS, GS>::D], uint32_t tails,
-                                                  u32x2_t sc, int lg0, const uint32_t *xs, const float *xsum,
-                                                  int npairs, int ngl, float (&accS)[MB], float (&accM)[MB]) {
-    using U = PairedUnit<BITS, GS>;
+template <class U, int MB>
+__device__ __forceinline__ void nint_compute_step(const uint32_t (&q)[4][U::D], uint32_t tails, u32x2_t sc, int lg0,
+                                                  const uint32_t *xs, const float *xsum, int npairs, int ngl,
+                                                  float (&accS)[MB], float (&accM)[MB]) {
+    constexpr int GS = U::GROUP;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int lg = lg0 + 4 * j;
@@ -190,12 +223,11 @@ __device__ __forceinline__ void nint_compute_step(const uint32_t (&q)[4][PairedU
 // is an unconditional window load, so the staging waits for the activations only and the unpack of a
 // step only for that step.  RING = false is the variant for waves with at most three steps in all, which
 // never requests more.
-template <int BITS, int GS, int XF16, int MB, bool RING = true>
-__device__ __forceinline__ void nint_paired_body(const NintK &k, const uint8_t *__restrict__ w, int rb0, int rbw,
-                                                 int row_base, int out_rows, const uint16_t *const (&xr)[MB],
-                                                 float *const (&yr)[MB], int spw, uint32_t *lds) {
-    using U = PairedUnit<BITS, GS>;
-    constexpr int D = U::D;
+template <class U, int XF16, int MB, bool RING = true>
+__device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__restrict__ w, int rb0, int rbw,
+                                               int row_base, int out_rows, const uint16_t *const (&xr)[MB],
+                                               float *const (&yr)[MB], int spw, uint32_t *lds) {
+    constexpr int D = U::D, GS = U::GROUP;
     const int lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
     const int r = lane & 15, kb = lane >> 4;
@@ -243,7 +275,7 @@ __device__ __forceinline__ void nint_paired_body(const NintK &k, const uint8_t *
     int crb = 0, cs = 0;
 #define MFQ_COMPUTE(Q, T, C)                                                                              \
     {                                                                                                     \
-        nint_compute_step<BITS, GS, MB>(Q, T, C, cs * 16 + kb, xs, xsum, npairs, ngl, accS, accM);         \
+        nint_compute_step<U, MB>(Q, T, C, cs * 16 + kb, xs, xsum, npairs, ngl, accS, accM);                 \
         if (++cs >= n) {                                                                                  \
             float a_s = ns[0], a_m = nm[0];                                                               \
             _Pragma("unroll") for (int i = 1; i < kMaxRbw; ++i) if (crb == i) { a_s = ns[i]; a_m = nm[i]; } \
@@ -286,6 +318,13 @@ __device__ __forceinline__ void nint_paired_body(const NintK &k, const uint8_t *
 #undef MFQ_ISSUE
 #undef MFQ_COMPUTE
     flush_rows<MB>(red, nwaves, nrb, rb0, row_base, out_rows, yr);
+}
+
+template <int BITS, int GS, int XF16, int MB, bool RING = true>
+__device__ __forceinline__ void nint_paired_body(const NintK &k, const uint8_t *__restrict__ w, int rb0, int rbw,
+                                                 int row_base, int out_rows, const uint16_t *const (&xr)[MB],
+                                                 float *const (&yr)[MB], int spw, uint32_t *lds) {
+    nint_unit_body<PairedUnit<BITS, GS>, XF16, MB, RING>(k, w, rb0, rbw, row_base, out_rows, xr, yr, spw, lds);
 }
 
 // Any (bits, gs): natural-order units, one code at a time in fp32.
@@ -356,6 +395,18 @@ __global__ __launch_bounds__(1024) void nint_gemv_paired_kernel(NintK k, const u
     float *yr[MB];
     dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
     nint_paired_body<BITS, GS, XF16, MB, RING>(k, w, blockIdx.x * rbw, rbw, 0, k.out, xr, yr, spw, lds);
+}
+
+// natural-order profiles with a unit of their own
+template <int BITS, int GS, int XF16, int MB, bool RING>
+__global__ __launch_bounds__(1024) void nint_gemv_natural_kernel(NintK k, const uint8_t *__restrict__ w,
+                                                                 const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                                 float *__restrict__ y, int64_t ldy, int spw, int rbw) {
+    extern __shared__ uint32_t lds[];
+    const uint16_t *xr[MB];
+    float *yr[MB];
+    dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
+    nint_unit_body<GenericUnit<BITS, GS>, XF16, MB, RING>(k, w, blockIdx.x * rbw, rbw, 0, k.out, xr, yr, spw, lds);
 }
 
 template <int XF16, int MB>
