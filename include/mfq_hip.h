@@ -219,6 +219,23 @@ int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_pools, const 
                                   float *out, int64_t ldo, void *workspace, size_t workspace_bytes,
                                   mfq_stream_t stream);
 
+/* Decode form of the grouped matmul (no route map; a handful of tokens): one launch of the batch-1 GEMV over
+ * rows p = t * R + r (pair p against expert ids[p]) and, when a shared tensor [out_per_expert, K] is given, rows
+ * T * R + t (the shared tensor against token t).  x row of a pair: p with routed_input, else t; of a shared row:
+ * T * R + t with routed_input, else t.  swiglu = 0: out is float [rows, ldo].  swiglu != 0: out_per_expert =
+ * 2 W, gate rows first, and out is bf16 / fp16 (out_dtype, MFQ_X_*) [rows, ldo] = silu(gate) * up, the fusion
+ * of NintMoeWeight::forward_swiglu (cpp_runtime/mfq_decode.cpp:3203-3205) and nint_gemv_packed_swiglu_ws_cuda
+ * (cpp_runtime/mfq_decode.cpp:393-396) moved to the producer.  Same values as mfq_hip_moe_grouped_matmul +
+ * mfq_hip_moe_swiglu and mfq_hip_nint_gemv on the shared rows, up to the order of the fp32 sums over K.
+ * MFQ_ERR_UNSUPPORTED when a cohort has no batch-1 unit, the shared tensor's rows differ from out_per_expert, or
+ * K is too long for one block. */
+int mfq_hip_moe_decode_matmul(const mfq_moe_pool *pools, int n_pools, const int32_t *expert_pool,
+                              const int32_t *expert_local, int E, int out_per_expert, int K,
+                              const void *x, int x_dtype, int64_t ldx, int routed_input,
+                              const int32_t *ids, int T, int R,
+                              const mfq_nint_desc *shared_desc, const void *shared_weight, int swiglu,
+                              void *out, int out_dtype, int64_t ldo, mfq_stream_t stream);
+
 /* hidden[r, c] = silu(gate_up[r, c]) * gate_up[r, W + c]  (moe_swiglu_split_cuda,
  * mfq/kernels/cuda/moe.cu:2980-2996); output fp16 (x_dtype MFQ_X_F16) or bf16. */
 int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,

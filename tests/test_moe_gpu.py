@@ -16,7 +16,8 @@ def _topk(logits, k, **kw):
     return ids.cpu().numpy(), w.cpu().numpy()
 
 
-@pytest.mark.parametrize("T,E,k", [(9, 64, 6), (1, 256, 8), (5, 128, 8), (33, 300, 16), (3, 8, 8)])
+@pytest.mark.parametrize("T,E,k", [(9, 64, 6), (1, 256, 8), (5, 128, 8), (33, 300, 16), (3, 8, 8), (4, 701, 9), (2, 1024, 8),
+                                   (3, 1500, 8)])
 def test_topk_modes_match_oracle(T, E, k):
     rng = np.random.default_rng(71 + T)
     logits = rng.standard_normal((T, E)).astype(np.float32)
@@ -168,6 +169,45 @@ def test_moe_ffn_forward_matches_oracle(T):
     got = out.cpu().numpy()
     assert rel_l2(got, ref) < REL_TOL, rel_l2(got, ref)
     assert np.abs(got - ref).max() < ABS_TOL
+
+
+@pytest.mark.parametrize("T,H,W", [(1, 256, 128), (3, 256, 128), (2, 8192, 64)])
+def test_decode_matmul_matches_the_separate_calls(T, H, W):
+    """The one-launch decode form (routes + shared tensor, fused SwiGLU) against grouped matmul + swiglu + dense matmul:
+    the same values up to the order of the fp32 sums over K.  H = 8192 gives the 2-bit cohort 32 steps: more than
+    three items per wave, the variant with a prefetch ring."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_moe import build_moe_route_plan, moe_swiglu
+    rng = np.random.default_rng(900 + T + H)
+    E, k = 12, 4
+    bits = [(2, 3, 4, 5)[i % 4] for i in range(E)]
+    _, gu = _moe(rng, E, 2 * W, H, bits)
+    _, dn = _moe(rng, E, H, W, bits)
+    sg = O.quantize_nint((rng.standard_normal((2 * W, H)) * 0.02).astype(np.float32), 4, 24, 6)
+    sd = O.quantize_nint((rng.standard_normal((H, W)) * 0.02).astype(np.float32), 5, 28, 6)
+    sgu = R.load_quant_linear("NINT4", O.pack_nint(sg)).weight
+    sdn = R.load_quant_linear("NINT5", O.pack_nint(sd)).weight
+    ids = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    ids[0, 1] = E + 3                                  # invalid id -> zero row
+    ids_d = torch.from_numpy(ids).cuda()
+    route = build_moe_route_plan(ids_d, E)
+
+    def close(got, want, tol):
+        got, want = got.float().cpu().numpy(), want.float().cpu().numpy()
+        assert rel_l2(got, want) < tol, rel_l2(got, want)
+
+    for dtype in (torch.bfloat16, torch.float16):
+        x = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).to(dtype).cuda()
+        assert gu.decode_capable(sgu) and dn.decode_capable(sdn)
+        hid = gu.forward_decode(x, ids_d, sgu, swiglu=True)
+        want = torch.cat([moe_swiglu(gu(x, route)).reshape(T * k, W), moe_swiglu(R.nint_matmul(sgu, x))])
+        close(hid, want, 1e-3)                         # fp16 outputs: half an ulp is 5e-4
+        assert torch.all(hid[1] == 0)
+        out = dn.forward_decode(hid, ids_d, sdn, routed=True)
+        want = torch.cat([dn(hid[: T * k].reshape(T, k, W), route).reshape(T * k, H), R.nint_matmul(sdn, hid[T * k:])])
+        close(out, want, 1e-5)
+        plain = gu.forward_decode(x, ids_d)            # no shared tensor, no SwiGLU: the grouped matmul itself
+        assert torch.equal(plain.view(torch.int32), gu(x, route).reshape(T * k, 2 * W).view(torch.int32))
 
 
 def test_moe_errors():

@@ -79,6 +79,8 @@ _SIGS = {
     "mfq_hip_moe_grouped_matmul_ws": (C.c_int, [C.POINTER(MoePool), C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, vp,
                                                 C.c_int, i64, C.c_int, vp, C.c_int, C.c_int, vp, vp, vp, vp, vp, i64,
                                                 vp, sz, vp]),
+    "mfq_hip_moe_decode_matmul": (C.c_int, [C.POINTER(MoePool), C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, vp, C.c_int,
+                                            i64, C.c_int, vp, C.c_int, C.c_int, vp, vp, C.c_int, vp, C.c_int, i64, vp]),
     "mfq_hip_moe_swiglu": (C.c_int, [vp, i64, C.c_int, C.c_int, vp, C.c_int, i64, vp]),
     "mfq_hip_moe_weighted_reduce": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]),
     "mfq_hip_gemm_f16_nt": (C.c_int, [vp, i64, vp, i64, C.c_int, C.c_int, C.c_int, vp, i64, vp]),

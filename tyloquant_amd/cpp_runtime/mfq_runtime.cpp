@@ -423,6 +423,26 @@ void NintMoeWeight::forward(const void *x, int x_dtype, int64_t ldx, bool routed
         need ? workspace.get() : nullptr, need, stream));
 }
 
+static bool nint_decode_unit(const mfq_nint_desc &d) { return d.kind == 1 || (d.bits == 5 && d.gs == 28); }
+
+bool NintMoeWeight::decode_capable(const NintWeight *shared) const {
+    if (pools.size() + (shared ? 1 : 0) > 8) return false;
+    for (const auto &p : pools)
+        if (!nint_decode_unit(p->desc)) return false;
+    return !shared || (nint_decode_unit(shared->desc) && shared->desc.out == out_per_expert &&
+                       shared->desc.neuron_len == neuron_len);
+}
+
+void NintMoeWeight::forward_decode(const void *x, int x_dtype, int64_t ldx, bool routed_input, const int32_t *ids, int T,
+                                   int R, const NintWeight *shared, bool swiglu, void *out, mfq_stream_t stream) const {
+    abi_check(mfq_hip_moe_decode_matmul(pool_table.data(), static_cast<int>(pool_table.size()),
+                                        static_cast<const int32_t *>(expert_pool.get()),
+                                        static_cast<const int32_t *>(expert_local.get()), n_experts, out_per_expert,
+                                        neuron_len, x, x_dtype, ldx, routed_input ? 1 : 0, ids, T, R,
+                                        shared ? &shared->desc : nullptr, shared ? shared->data.get() : nullptr,
+                                        swiglu ? 1 : 0, out, MFQ_X_F16, swiglu ? out_per_expert / 2 : out_per_expert, stream));
+}
+
 void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &down, const void *x, int x_dtype, int64_t ldx,
                           int T, const float *router_logits, int top_k, int topk_mode, bool normalize,
                           const float *router_bias, float router_scale, const NintWeight *shared_gate_up,
@@ -433,12 +453,27 @@ void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &dow
     const int E = gate_up.n_experts, W = down.neuron_len, H = down.out_per_expert;
     const size_t pairs = static_cast<size_t>(T) * top_k;
     s.ids.ensure(4 * pairs); s.weights.ensure(4 * pairs);
-    s.gate_up.ensure(4 * pairs * 2 * W); s.hidden.ensure(2 * pairs * W); s.down.ensure(4 * pairs * H);
     int32_t *ids = static_cast<int32_t *>(s.ids.get());
     float *wts = static_cast<float *>(s.weights.get());
     abi_check(mfq_hip_moe_topk(router_logits, router_bias, T, E, top_k, topk_mode, normalize ? 1 : 0, 1e-20f, router_scale, ids,
                                wts, stream));
+    const bool with_shared = shared_gate_up && shared_down;
+    if (T <= 8 && gate_up.decode_capable(with_shared ? shared_gate_up : nullptr) &&
+        down.decode_capable(with_shared ? shared_down : nullptr)) {
+        // decode step: gate/up + SwiGLU of the routes and the shared expert in one launch, the down projections in a
+        // second one; rows pairs .. pairs + T - 1 of both buffers belong to the shared expert
+        const size_t rows = pairs + (with_shared ? T : 0);
+        s.hidden.ensure(2 * rows * W); s.down.ensure(4 * rows * H);
+        gate_up.forward_decode(x, x_dtype, ldx, false, ids, T, top_k, with_shared ? shared_gate_up : nullptr, true,
+                               s.hidden.get(), stream);
+        float *dn = static_cast<float *>(s.down.get());
+        down.forward_decode(s.hidden.get(), MFQ_X_F16, W, true, ids, T, top_k, with_shared ? shared_down : nullptr, false, dn,
+                            stream);
+        abi_check(mfq_hip_moe_weighted_reduce(dn, wts, T, top_k, H, with_shared ? dn + pairs * H : nullptr, nullptr, out, stream));
+        return;
+    }
     MoeRoutePlan route = build_moe_route_plan(ids, T, top_k, E, stream);
+    s.gate_up.ensure(4 * pairs * 2 * W); s.hidden.ensure(2 * pairs * W); s.down.ensure(4 * pairs * H);
     float *gu = static_cast<float *>(s.gate_up.get());
     gate_up.forward(x, x_dtype, ldx, false, route, gu, stream);
     abi_check(mfq_hip_moe_swiglu(gu, 2 * W, static_cast<int>(pairs), W, s.hidden.get(), MFQ_X_F16, W, stream));

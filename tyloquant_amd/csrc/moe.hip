@@ -124,6 +124,101 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float *__restrict__
     if (lane < k) weights[static_cast<int64_t>(t) * k + lane] = v * scale;
 }
 
+// Rank-by-counting variant for up to 256 * PER experts: one block per token, thread e counts the experts that beat
+// expert e (higher score, or the same score and a lower id); the k experts with rank < k are the selection, in
+// rank order.  No serial chain of k wave-wide arg-max reductions: a decode step's single token takes about a
+// microsecond.  Same results as moe_topk_kernel.
+template <int PER>
+__global__ __launch_bounds__(256) void moe_topk_rank_kernel(const float *__restrict__ logits, const float *__restrict__ bias,
+                                                            int E, int k, int mode, int normalize, float norm_floor,
+                                                            float scale, int32_t *__restrict__ ids,
+                                                            float *__restrict__ weights) {
+    __shared__ __attribute__((aligned(16))) int s_key[256 * PER];
+    __shared__ float s_red[8];
+    __shared__ float s_w[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int t = blockIdx.x;
+    const float *row = logits + static_cast<int64_t>(t) * E;
+    float raw[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = tid + 256 * i;
+        const float v = e < E ? row[e] : -INFINITY;
+        raw[i] = v != v ? -FLT_MAX : v;
+    }
+    float smax = 0.f, ssum = 1.f;
+    if (mode == MFQ_TOPK_SOFTMAX) {
+        float m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) m = fmaxf(m, raw[i]);
+        m = wave_max(m);
+        if (lane == 0) s_red[wave] = m;
+        __syncthreads();
+        smax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+        float a = 0.f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            if (tid + 256 * i < E) a += expf(raw[i] - smax);
+        a = wave_sum(a);
+        if (lane == 0) s_red[4 + wave] = a;
+        __syncthreads();
+        ssum = (s_red[4] + s_red[5]) + (s_red[6] + s_red[7]);
+    }
+    float wv[PER];
+    int key[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = tid + 256 * i;
+        float w = raw[i];
+        if (mode == MFQ_TOPK_SIGMOID) w = 1.f / (1.f + expf(-raw[i]));
+        else if (mode == MFQ_TOPK_SQRT_SOFTPLUS) w = sqrtf(raw[i] > 20.f ? raw[i] : log1pf(expf(raw[i])));
+        else if (mode == MFQ_TOPK_SOFTMAX) w = expf(raw[i] - smax) / ssum;
+        wv[i] = w;
+        const float sc = e < E ? w + (bias ? bias[e] : 0.f) : -INFINITY;
+        // order-preserving map of the float to a signed int (-0 and +0 compare equal, as they do as floats)
+        const int b = __float_as_int(sc + 0.f);
+        key[i] = b ^ ((b >> 31) & 0x7fffffff);
+        if (key[i] == INT_MIN) key[i] = INT_MIN + 1;  // unreachable from a float; keeps key - 1 from wrapping
+        s_key[e] = e < E ? key[i] : INT_MIN;
+    }
+    __syncthreads();
+    int rank[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) rank[i] = 0;
+    const int n4 = (E + 3) >> 2;
+    for (int j4 = 0; j4 < n4; ++j4) {
+        const int4 o = reinterpret_cast<const int4 *>(s_key)[j4];
+        const int ov[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int j = 4 * j4 + c;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) rank[i] += ov[c] > key[i] - (j < tid + 256 * i);  // >= for the lower ids
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = tid + 256 * i;
+        if (e < E && rank[i] < k) {
+            ids[static_cast<int64_t>(t) * k + rank[i]] = e;
+            s_w[rank[i]] = wv[i];
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float v = lane < k ? s_w[lane] : 0.f;
+    if (mode == MFQ_TOPK_DELAYED_SOFTMAX) {
+        const float mx = wave_max(lane < k ? v : -INFINITY);
+        v = lane < k ? expf(v - mx) : 0.f;
+        const float den = wave_sum(v);
+        v /= den;
+    } else if (normalize) {
+        const float den = fmaxf(wave_sum(v), norm_floor);
+        v /= den;
+    }
+    if (lane < k) weights[static_cast<int64_t>(t) * k + lane] = v * scale;
+}
+
 // ---- expert map ------------------------------------------------------------------------------
 // counts: one block per expert counts its pairs (no atomics, nothing to pre-clear).
 __global__ __launch_bounds__(256) void moe_count_kernel(const int32_t *__restrict__ ids, int n_pairs,
@@ -286,45 +381,76 @@ __global__ __launch_bounds__(512) void moe_grouped_kernel(MoePools P, const int3
     }
 }
 
-// Batch-1 path (no route map): block (group of rbw row-blocks, pair), the body of the dense GEMV with the unit
-// of the pair's cohort.  P.spw: steps per wave of each cohort; RING = false when no wave has more than three
-// (row-block, step) items.
-template <int XF16, bool RING>
+// Batch-1 path (no route map): block (group of rbw row-blocks, row), the body of the dense GEMV with the unit of
+// the row's cohort.  Rows below n_pairs are (token, route) pairs; row n_pairs + t applies the shared tensor
+// (cohort slot P.n) to token t.  P.spw: steps per wave of each cohort; RING = false when no wave has more than
+// three (row-block, step) items.  SWIGLU: the block takes row-block blockIdx.x of the gate half and of the up half
+// of the expert and stores silu(gate) * up as 16-bit values, out_f16 selecting fp16 over bf16.
+template <int XF16, bool RING, bool SWIGLU>
 __global__ __launch_bounds__(1024) void moe_decode_kernel(MoePools P, int rbw, const int32_t *__restrict__ expert_pool,
                                                           const int32_t *__restrict__ expert_local, int E,
                                                           int out_per_expert, const uint16_t *__restrict__ x, int64_t ldx,
-                                                          int routed_input, const int32_t *__restrict__ ids, int R,
-                                                          float *__restrict__ out, int64_t ldo) {
+                                                          int routed_input, const int32_t *__restrict__ ids, int n_pairs,
+                                                          int R, void *__restrict__ out, int out_f16, int64_t ldo) {
     extern __shared__ uint32_t lds[];
-    const int pair = blockIdx.y;
-    const int e = ids[pair];
-    const int rbl0 = blockIdx.x * rbw;
-    float *yrow = out + static_cast<int64_t>(pair) * ldo;
-    if (e < 0 || e >= E || expert_pool[e] < 0) {  // invalid expert id: defined as a zero row
-        for (int c = threadIdx.x; c < rbw * 16; c += blockDim.x) yrow[rbl0 * 16 + c] = 0.f;
-        return;
+    const int row = blockIdx.y;
+    const int half_rb = out_per_expert / 32;  // SWIGLU: row-blocks of the gate half
+    const int rbl0 = SWIGLU ? blockIdx.x : blockIdx.x * rbw;
+    int pool, row_base, xi;
+    if (row < n_pairs) {
+        const int e = ids[row];
+        if (e < 0 || e >= E || expert_pool[e] < 0) {  // invalid expert id: defined as a zero row
+            if constexpr (SWIGLU) {
+                if (threadIdx.x < 16) static_cast<uint16_t *>(out)[row * ldo + rbl0 * 16 + threadIdx.x] = 0;
+            } else {
+                for (int c = threadIdx.x; c < rbw * 16; c += blockDim.x)
+                    static_cast<float *>(out)[row * ldo + rbl0 * 16 + c] = 0.f;
+            }
+            return;
+        }
+        pool = expert_pool[e];
+        row_base = expert_local[e] * out_per_expert;
+        xi = routed_input ? row : row / R;
+    } else {
+        pool = P.n;
+        row_base = 0;
+        xi = routed_input ? row : row - n_pairs;
     }
-    const int pool = expert_pool[e];
     const NintK &k = P.k[pool];
     const uint8_t *w = P.w[pool];
     const int spw = P.spw[pool];
-    const int row_base = expert_local[e] * out_per_expert;
-    const uint16_t *xrow = x + static_cast<int64_t>(routed_input ? pair : pair / R) * ldx;
-    const uint16_t *xr[1] = {xrow};
-    float *yr[1] = {yrow};
+    const uint16_t *xr[1] = {x + static_cast<int64_t>(xi) * ldx};
+    float *yr[1] = {SWIGLU ? nullptr : static_cast<float *>(out) + static_cast<int64_t>(row) * ldo};
+    const int rb0 = row_base / 16 + rbl0, nrb = SWIGLU ? 2 : rbw, step = SWIGLU ? half_rb : 1;
+#define MFQ_MOE_CASE(UNIT, B, G)                                                                                        \
+    if (k.bits == B && k.gs == G)                                                                                      \
+        nint_unit_body<UNIT<B, G>, XF16, 1, RING, !SWIGLU>(k, w, rb0, nrb, row_base, out_per_expert, xr, yr, spw, lds, step);
     if (k.kind == 1) {
-#define MFQ_MOE_CASE(B, G)                                                                                             \
-    if (k.bits == B && k.gs == G) {                                                                                    \
-        nint_paired_body<B, G, XF16, 1, RING>(k, w, row_base / 16 + rbl0, rbw, row_base, out_per_expert, xr, yr, spw, lds); \
-        return;                                                                                                        \
+        MFQ_MOE_CASE(PairedUnit, 4, 24)
+        else MFQ_MOE_CASE(PairedUnit, 3, 24)
+        else MFQ_MOE_CASE(PairedUnit, 2, 16)
+        else MFQ_MOE_CASE(PairedUnit, 4, 32)
+        else MFQ_MOE_CASE(PairedUnit, 4, 16)
+        else MFQ_MOE_CASE(PairedUnit, 4, 48)
+        else MFQ_MOE_CASE(PairedUnit, 2, 32)
+    } else {
+        MFQ_MOE_CASE(GenericUnit, 5, 28)
     }
-        MFQ_MOE_CASE(4, 24) MFQ_MOE_CASE(3, 24) MFQ_MOE_CASE(2, 16) MFQ_MOE_CASE(4, 32) MFQ_MOE_CASE(4, 16)
-        MFQ_MOE_CASE(4, 48) MFQ_MOE_CASE(2, 32)
 #undef MFQ_MOE_CASE
-        return;
+    if constexpr (SWIGLU) {
+        __syncthreads();
+        if (threadIdx.x < 16) {
+            const int nwaves = blockDim.x >> 6;
+            const float *red = reinterpret_cast<const float *>(lds + gemv_red_offset(nwaves, 1, spw, k.gs));
+            float g = 0.f, u = 0.f;
+            for (int wv = 0; wv < nwaves; ++wv) {
+                g += red[wv * 16 + threadIdx.x];
+                u += red[(nwaves + wv) * 16 + threadIdx.x];
+            }
+            const float v = g / (1.f + expf(-g)) * u;
+            static_cast<uint16_t *>(out)[row * ldo + rbl0 * 16 + threadIdx.x] = out_f16 ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
+        }
     }
-    nint_unit_body<GenericUnit<5, 28>, XF16, 1, RING>(k, w, row_base / 16 + rbl0, rbw, row_base, out_per_expert, xr, yr, spw,
-                                                      lds);
 }
 
 // Matrix-core path: a tile of up to 16 pairs of one expert against NB row-blocks, weights streamed once
@@ -502,8 +628,16 @@ extern "C" int mfq_hip_moe_topk(const float *logits, const float *bias, int T, i
     MFQ_REQUIRE(mode >= 0 && mode <= 3, MFQ_ERR_INVALID, "moe_topk: unknown mode %d", mode);
     MFQ_REQUIRE(!(normalize && mode == MFQ_TOPK_DELAYED_SOFTMAX), MFQ_ERR_INVALID,
                 "selected-weight normalization and delayed softmax are mutually exclusive");
-    hipLaunchKernelGGL(moe_topk_kernel, dim3(static_cast<unsigned>(ceil_div(T, 4))), dim3(256), 0, as_stream(stream), logits,
-                       bias, T, E, k, mode, normalize, norm_floor, scale, ids, weights);
+#define MFQ_TOPK_RANK(PER)                                                                                        \
+    hipLaunchKernelGGL(moe_topk_rank_kernel<PER>, dim3(static_cast<unsigned>(T)), dim3(256), 0, as_stream(stream), \
+                       logits, bias, E, k, mode, normalize, norm_floor, scale, ids, weights)
+    if (E <= 256) MFQ_TOPK_RANK(1);
+    else if (E <= 512) MFQ_TOPK_RANK(2);
+    else if (E <= 1024) MFQ_TOPK_RANK(4);
+#undef MFQ_TOPK_RANK
+    else
+        hipLaunchKernelGGL(moe_topk_kernel, dim3(static_cast<unsigned>(ceil_div(T, 4))), dim3(256), 0, as_stream(stream),
+                           logits, bias, T, E, k, mode, normalize, norm_floor, scale, ids, weights);
     return check_launch("moe_topk");
 }
 
@@ -553,6 +687,69 @@ extern "C" size_t mfq_hip_moe_grouped_workspace_bytes(const mfq_moe_pool *pools,
     return total;
 }
 
+static void moe_fill_k(NintK &k, const mfq_nint_desc &d) {
+    k.bits = d.bits; k.sub_bits = d.sub_bits; k.gs = d.gs; k.out = d.out; k.neuron_len = d.neuron_len; k.ng = d.ng;
+    k.kind = d.kind; k.dwords = d.dwords; k.tail = d.tail_bytes; k.nsteps = d.nsteps; k.n_rowblocks = d.n_rowblocks;
+    k.step_bytes = d.step_bytes; k.rowblock_bytes = d.rowblock_bytes; k.anchors_off = d.anchors_off;
+}
+
+// Batch-1 launch (moe_decode_kernel) over n_rows rows: the n_pairs routed pairs, then one row per token for the
+// shared tensor in cohort slot P.n, if any.  Every cohort slot has a GEMV unit.  Returns -1 when the shape does
+// not fit the kernel (the caller takes another path), else a status.
+static int moe_decode_launch(MoePools &P, int n_slots, int max_steps, const int32_t *expert_pool,
+                             const int32_t *expert_local, int E, int out_per_expert, const uint16_t *xp, int x_dtype,
+                             int64_t ldx, int routed_input, const int32_t *ids, int n_pairs, int n_rows, int R, int swiglu,
+                             void *out, int out_f16, int64_t ldo, hipStream_t st) {
+    static const int env_off = [] { const char *e = getenv("MFQ_MOE_SPLIT"); return e ? atoi(e) == 0 : 0; }();
+    static const int env_w = [] { const char *e = getenv("MFQ_MOE_DEC_WAVES"); return e ? atoi(e) : 16; }();
+    static const int env_rbw = [] { const char *e = getenv("MFQ_MOE_DEC_RBW"); return e ? atoi(e) : 0; }();
+    if (env_off || n_rows > 65535) return -1;
+    const int rbe = out_per_expert / 16;
+    // Waves split the K steps; a wave takes more (row-block, step) items while the grid keeps about
+    // gemv_target_waves() waves.  With the fused SwiGLU a block always takes two row-blocks: gate and up.
+    const int nwaves = max_steps < env_w ? max_steps : env_w;
+    const int spw_max = static_cast<int>(ceil_div(max_steps, nwaves));
+    int64_t items = 0;
+    for (int i = 0; i < n_slots; ++i) items += P.k[i].nsteps;
+    items = items / n_slots * rbe * n_rows;
+    int per_wave = static_cast<int>(items / gemv_target_waves());
+    per_wave = per_wave < 1 ? 1 : (per_wave > 3 ? 3 : per_wave);
+    int rbw = per_wave / spw_max < 1 ? 1 : per_wave / spw_max;
+    if (env_rbw) rbw = env_rbw;
+    if (rbw > kMaxRbw) rbw = kMaxRbw;
+    while (rbe % rbw) --rbw;
+    if (swiglu) {
+        if (out_per_expert % 32) return -1;
+        rbw = 2;
+    }
+    size_t lds = 0;
+    bool ring = false;
+    for (int i = 0; i < n_slots; ++i) {
+        P.spw[i] = static_cast<int>(ceil_div(P.k[i].nsteps, nwaves));
+        const size_t need = gemv_lds_bytes(1, P.spw[i], P.k[i].gs, nwaves, rbw);
+        if (need > lds) lds = need;
+        if (P.spw[i] * rbw > 3) ring = true;
+        if (swiglu && static_cast<int64_t>(rbe / 2) * P.k[i].rowblock_bytes >= (1ll << 31)) return -1;
+    }
+    if (lds > 65536) return -1;
+    const dim3 grid(static_cast<unsigned>(swiglu ? rbe / 2 : rbe / rbw), static_cast<unsigned>(n_rows)), block(64 * nwaves);
+#define MFQ_MOE_DECODE(XF, RG, SW)                                                                                   \
+    hipLaunchKernelGGL((moe_decode_kernel<XF, RG, SW>), grid, block, lds, st, P, rbw, expert_pool, expert_local, E,   \
+                       out_per_expert, xp, ldx, routed_input, ids, n_pairs, R, out, out_f16, ldo)
+#define MFQ_MOE_DECODE_X(XF)                        \
+    if (swiglu) {                                   \
+        if (ring) MFQ_MOE_DECODE(XF, true, true);   \
+        else MFQ_MOE_DECODE(XF, false, true);       \
+    } else {                                        \
+        if (ring) MFQ_MOE_DECODE(XF, true, false);  \
+        else MFQ_MOE_DECODE(XF, false, false);      \
+    }
+    if (x_dtype == MFQ_X_F16) MFQ_MOE_DECODE_X(1) else MFQ_MOE_DECODE_X(0)
+#undef MFQ_MOE_DECODE_X
+#undef MFQ_MOE_DECODE
+    return check_launch("moe_decode");
+}
+
 extern "C" int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools, const int32_t *expert_pool,
                                           const int32_t *expert_local, int E, int out_per_expert, int K, const void *x,
                                           int x_dtype, int64_t ldx, int routed_input, const int32_t *ids, int T, int R,
@@ -593,10 +790,7 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
         MFQ_REQUIRE(d.neuron_len == K && pools[i].weight, MFQ_ERR_INVALID,
                     "moe_grouped_matmul: cohort %d has neuron_len %d, expected %d", i, d.neuron_len, K);
         if (d.nsteps > max_steps) max_steps = d.nsteps;
-        NintK &k = P.k[i];
-        k.bits = d.bits; k.sub_bits = d.sub_bits; k.gs = d.gs; k.out = d.out; k.neuron_len = d.neuron_len; k.ng = d.ng;
-        k.kind = d.kind; k.dwords = d.dwords; k.tail = d.tail_bytes; k.nsteps = d.nsteps; k.n_rowblocks = d.n_rowblocks;
-        k.step_bytes = d.step_bytes; k.rowblock_bytes = d.rowblock_bytes; k.anchors_off = d.anchors_off;
+        moe_fill_k(P.k[i], d);
         P.w[i] = static_cast<const uint8_t *>(pools[i].weight);
         P.xg[i] = nullptr;
         P.prefill[i] = 0;
@@ -678,47 +872,10 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
         }
         return check_launch("moe_grouped_matmul");
     };
-    static const int split = [] { const char *e = getenv("MFQ_MOE_SPLIT"); return e ? atoi(e) : 1; }();
-    if (!mapped && units && split) {
-        // One pair per tile (no route map): one launch of the batch-1 GEMV bodies for every cohort.  Waves split
-        // the K steps; a wave takes more (row-block, step) items while the grid keeps about gemv_target_waves() waves.
-        static const int env_w = [] { const char *e = getenv("MFQ_MOE_DEC_WAVES"); return e ? atoi(e) : 16; }();
-        static const int env_rbw = [] { const char *e = getenv("MFQ_MOE_DEC_RBW"); return e ? atoi(e) : 0; }();
-        const int nwaves = max_steps < env_w ? max_steps : env_w;
-        const int spw_max = static_cast<int>(ceil_div(max_steps, nwaves));
-        int64_t items = 0;
-        for (int i = 0; i < n_pools; ++i) items += P.k[i].nsteps;
-        items = items / n_pools * rbe * n_pairs;
-        int per_wave = static_cast<int>(items / gemv_target_waves());
-        per_wave = per_wave < 1 ? 1 : (per_wave > 3 ? 3 : per_wave);
-        {
-            int rbw = per_wave / spw_max < 1 ? 1 : per_wave / spw_max;
-            if (env_rbw) rbw = env_rbw;
-            while (rbe % rbw) --rbw;
-            size_t lds = 0;
-            bool ring = false;
-            for (int i = 0; i < n_pools; ++i) {
-                P.spw[i] = static_cast<int>(ceil_div(P.k[i].nsteps, nwaves));
-                const size_t need = gemv_lds_bytes(1, P.spw[i], P.k[i].gs, nwaves, rbw);
-                if (need > lds) lds = need;
-                if (P.spw[i] * rbw > 3) ring = true;
-            }
-            if (lds <= 65536) {
-                const dim3 grid(static_cast<unsigned>(rbe / rbw), static_cast<unsigned>(n_pairs)), block(64 * nwaves);
-#define MFQ_MOE_DECODE(XF, RG)                                                                                     \
-hipLaunchKernelGGL((moe_decode_kernel<XF, RG>), grid, block, lds, st, P, rbw, expert_pool, expert_local, E,     \
-                   out_per_expert, xp, ldx, routed_input, ids, R, out, ldo)
-                if (x_dtype == MFQ_X_F16) {
-                    if (ring) MFQ_MOE_DECODE(1, true);
-                    else MFQ_MOE_DECODE(1, false);
-                } else {
-                    if (ring) MFQ_MOE_DECODE(0, true);
-                    else MFQ_MOE_DECODE(0, false);
-                }
-#undef MFQ_MOE_DECODE
-                return check_launch("moe_decode");
-            }
-        }
+    if (!mapped && units) {
+        const int rc = moe_decode_launch(P, n_pools, max_steps, expert_pool, expert_local, E, out_per_expert, xp, x_dtype, ldx,
+                                         routed_input, ids, n_pairs, n_pairs, R, 0, out, 0, ldo, st);
+        if (rc >= 0) return rc;
     }
     if (mfma) {
         // row-blocks per wave: 4 while the grid still has a few thousand waves, else 1
@@ -742,6 +899,52 @@ hipLaunchKernelGGL((moe_decode_kernel<XF, RG>), grid, block, lds, st, P, rbw, ex
     }
     return launch_valu();
 #undef MFQ_MOE_LAUNCH
+}
+
+extern "C" int mfq_hip_moe_decode_matmul(const mfq_moe_pool *pools, int n_pools, const int32_t *expert_pool,
+                                         const int32_t *expert_local, int E, int out_per_expert, int K, const void *x,
+                                         int x_dtype, int64_t ldx, int routed_input, const int32_t *ids, int T, int R,
+                                         const mfq_nint_desc *shared_desc, const void *shared_weight, int swiglu,
+                                         void *out, int out_dtype, int64_t ldo, mfq_stream_t stream) {
+    MFQ_REQUIRE(pools && expert_pool && expert_local && x && ids && out, MFQ_ERR_INVALID, "moe_decode_matmul: null argument");
+    MFQ_REQUIRE(T > 0 && R > 0 && E > 0, MFQ_ERR_INVALID, "MoE ids must be int32 [tokens, routes]");
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "moe_decode_matmul: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(!swiglu || out_dtype == MFQ_X_BF16 || out_dtype == MFQ_X_F16, MFQ_ERR_INVALID,
+                "moe_decode_matmul: the fused SwiGLU stores bf16 or fp16, out_dtype=%d", out_dtype);
+    MFQ_REQUIRE((shared_desc == nullptr) == (shared_weight == nullptr), MFQ_ERR_INVALID,
+                "moe_decode_matmul: shared tensor without its descriptor (or the reverse)");
+    const int n_slots = n_pools + (shared_desc ? 1 : 0);
+    MFQ_REQUIRE(n_pools >= 1 && n_slots <= kMaxPools, MFQ_ERR_UNSUPPORTED, "moe_decode_matmul: %d cohorts (max %d)", n_slots,
+                kMaxPools);
+    MFQ_REQUIRE(out_per_expert % 16 == 0, MFQ_ERR_UNSUPPORTED, "moe_decode_matmul: out_per_expert %d must be a multiple of 16",
+                out_per_expert);
+    MFQ_REQUIRE(ldx >= K && ldo >= (swiglu ? out_per_expert / 2 : out_per_expert), MFQ_ERR_INVALID,
+                "moe_decode_matmul: ldx/ldo smaller than the tensor");
+    MoePools P;
+    P.n = n_pools;
+    int max_steps = 1;
+    for (int i = 0; i < n_slots; ++i) {
+        const mfq_nint_desc &d = i < n_pools ? pools[i].desc : *shared_desc;
+        const void *wt = i < n_pools ? pools[i].weight : shared_weight;
+        MFQ_REQUIRE(d.neuron_len == K && wt, MFQ_ERR_INVALID, "moe_decode_matmul: cohort %d has neuron_len %d, expected %d", i,
+                    d.neuron_len, K);
+        MFQ_REQUIRE(moe_prefill_unit(d) && 4 * d.rowblock_bytes < (1ll << 31), MFQ_ERR_UNSUPPORTED,
+                    "moe_decode_matmul: no batch-1 kernel for NINT%d-%d", d.bits, d.gs);
+        if (d.nsteps > max_steps) max_steps = d.nsteps;
+        moe_fill_k(P.k[i], d);
+        P.w[i] = static_cast<const uint8_t *>(wt);
+        P.xg[i] = nullptr;
+        P.prefill[i] = 0;
+    }
+    MFQ_REQUIRE(!shared_desc || shared_desc->out == out_per_expert, MFQ_ERR_UNSUPPORTED,
+                "moe_decode_matmul: shared tensor has %d rows, the experts %d", shared_desc ? shared_desc->out : 0,
+                out_per_expert);
+    const int n_pairs = T * R, n_rows = n_pairs + (shared_desc ? T : 0);
+    const int rc = moe_decode_launch(P, n_slots, max_steps, expert_pool, expert_local, E, out_per_expert,
+                                     static_cast<const uint16_t *>(x), x_dtype, ldx, routed_input, ids, n_pairs, n_rows, R,
+                                     swiglu, out, out_dtype == MFQ_X_F16, ldo, as_stream(stream));
+    if (rc < 0) return fail(MFQ_ERR_UNSUPPORTED, "moe_decode_matmul: shape outside the batch-1 kernel (rows %d, K %d)", n_rows, K);
+    return rc;
 }
 
 extern "C" int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,

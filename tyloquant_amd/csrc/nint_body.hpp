@@ -223,22 +223,29 @@ __device__ __forceinline__ void nint_compute_step(const uint32_t (&q)[4][U::D], 
 // is an unconditional window load, so the staging waits for the activations only and the unpack of a
 // step only for that step.  RING = false is the variant for waves with at most three steps in all, which
 // never requests more.
-template <class U, int XF16, int MB, bool RING = true>
+// rb_step: distance, in row-blocks, between the block's row-blocks (1 = consecutive).  FLUSH = false leaves the
+// partial sums parked (see park_rows; the reduction area starts at gemv_red_offset dwords) for the caller to
+// combine after a block barrier.
+__device__ __forceinline__ int gemv_red_offset(int nwaves, int mb, int spw, int gs) {
+    return nwaves * (mb * (spw * 16 * (gs / 2) + 2 * spw * 16));
+}
+
+template <class U, int XF16, int MB, bool RING = true, bool FLUSH = true>
 __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__restrict__ w, int rb0, int rbw,
                                                int row_base, int out_rows, const uint16_t *const (&xr)[MB],
-                                               float *const (&yr)[MB], int spw, uint32_t *lds) {
+                                               float *const (&yr)[MB], int spw, uint32_t *lds, int rb_step = 1) {
     constexpr int D = U::D, GS = U::GROUP;
     const int lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
     const int r = lane & 15, kb = lane >> 4;
     const int s0 = wave * spw;
     const int n = min(k.nsteps, s0 + spw) - s0;         // steps of this wave in each row-block
-    const int nrb = min(rbw, k.n_rowblocks - rb0);      // row-blocks of this block
+    const int nrb = min(rbw, (k.n_rowblocks - 1 - rb0) / rb_step + 1);  // row-blocks of this block
     const int ngl = spw * 16, npairs = ngl * (GS / 2);
     uint32_t *xs = lds + wave * (MB * (npairs + 2 * ngl));
     float *xsum = reinterpret_cast<float *>(xs + MB * npairs);
     float *red = reinterpret_cast<float *>(lds + nwaves * (MB * (npairs + 2 * ngl)));
-    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
+    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes) * rb_step;
 
     XRegs<MB> xg;
     stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * GS, npairs, lane, xg);
@@ -246,7 +253,7 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     float ns[kMaxRbw], nm[kMaxRbw];
 #pragma unroll
     for (int i = 0; i < kMaxRbw; ++i) {
-        const int rb = min(rb0 + i, k.n_rowblocks - 1);
+        const int rb = min(rb0 + i * rb_step, k.n_rowblocks - 1);
         ns[i] = anchors[rb * 16 + r];
         nm[i] = anchors[16 * k.n_rowblocks + rb * 16 + r];
     }
@@ -317,7 +324,7 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     }
 #undef MFQ_ISSUE
 #undef MFQ_COMPUTE
-    flush_rows<MB>(red, nwaves, nrb, rb0, row_base, out_rows, yr);
+    if constexpr (FLUSH) flush_rows<MB>(red, nwaves, nrb, rb0, row_base, out_rows, yr);
 }
 
 template <int BITS, int GS, int XF16, int MB, bool RING = true>

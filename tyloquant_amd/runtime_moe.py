@@ -174,6 +174,35 @@ class NintMoeWeight:
 
     __call__ = forward
 
+    def decode_capable(self, shared: NintWeight | None = None) -> bool:
+        """Whether forward_decode takes these cohorts (every one has a batch-1 unit) and this shared tensor."""
+        def unit(d):
+            return d.kind == 1 or (d.bits == 5 and d.gs == 28)
+        if not all(unit(p.desc) for p in self.pools) or len(self.pools) + (shared is not None) > 8:
+            return False
+        return shared is None or (unit(shared.desc) and shared.out == self.out_per_expert and
+                                  shared.neuron_len == self.neuron_len)
+
+    def forward_decode(self, x: torch.Tensor, ids: torch.Tensor, shared: NintWeight | None = None, swiglu=False,
+                       routed=False, out_dtype=torch.float16) -> torch.Tensor:
+        """One launch for a decode step: rows t * R + r are the routed pairs, rows T * R + t the shared tensor on
+        token t.  x is [T, K], or with `routed` [T * R (+ T), K] with one row per output row.  Returns fp32
+        [rows, out_per_expert], or with `swiglu` 16-bit [rows, out_per_expert / 2] = silu(gate) * up."""
+        T, R = ids.shape
+        rows = T * R + (T if shared is not None else 0)
+        if x.dim() != 2 or x.shape[1] != self.neuron_len or x.shape[0] != (rows if routed else T):
+            raise ValueError("decode activations must be [tokens, K] or one row per output row")
+        if x.stride(-1) != 1:
+            x = x.contiguous()
+        cols = self.out_per_expert // 2 if swiglu else self.out_per_expert
+        out = torch.empty((rows, cols), dtype=out_dtype if swiglu else torch.float32, device=x.device)
+        L.check(L.lib().mfq_hip_moe_decode_matmul(
+            self._pool_array, len(self.pools), _ptr(self.expert_pool), _ptr(self.expert_local), self.n_experts,
+            self.out_per_expert, self.neuron_len, _ptr(x), _x_dtype(x), x.stride(0), int(routed), _ptr(ids), T, R,
+            C.byref(shared.desc) if shared is not None else None, _ptr(shared.data) if shared is not None else None,
+            int(swiglu), _ptr(out), L.X_F16 if out.dtype == torch.float16 else L.X_BF16, cols, _stream()))
+        return out
+
 
 def moe_swiglu(gate_up: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
     """silu(gate) * up, gate = first half of the last axis (moe_swiglu_split_cuda)."""
@@ -205,6 +234,15 @@ def nint_moe_ffn_forward(gate_up: NintMoeWeight, down: NintMoeWeight, x: torch.T
     ids, w = moe_topk(router_logits, top_k, use_sigmoid, use_sqrt_softplus, normalize, delayed_softmax, router_bias,
                       1e-20, router_scale)
     route = build_moe_route_plan(ids, gate_up.n_experts)
+    sgu, sdn = shared if shared is not None else (None, None)
+    if route.ids_dst is None and gate_up.decode_capable(sgu) and down.decode_capable(sdn):
+        # decode step: gate/up + SwiGLU of the routes and of the shared expert in one launch, the down projections in
+        # a second one, then the weighted sum
+        T, R = ids.shape
+        hidden = gate_up.forward_decode(x, ids, sgu, swiglu=True)
+        dn = down.forward_decode(hidden, ids, sdn, routed=True)
+        pair = dn[: T * R].reshape(T, R, -1)
+        return moe_weighted_reduce(pair, w, dn[T * R:] if shared is not None else None), ids, w
     gu = gate_up.forward(x, route)
     hidden = moe_swiglu(gu)
     dn = down.forward(hidden, route)
