@@ -81,6 +81,99 @@ __global__ __launch_bounds__(256) void x_prep_kernel(const uint16_t *__restrict_
     }
 }
 
+// The same for 16-byte aligned rows with K % 8 == 0 and Kp * 2 bytes of LDS: 8 values per load and store, the row
+// read once (twice beyond 8192 values), the group sums taken from the fp16 row kept in LDS.  Bit-identical results.
+template <int XF16>
+__global__ __launch_bounds__(256) void x_prep_vec_kernel(const uint16_t *__restrict__ x, int64_t ldx, int K, int Kp,
+                                                         uint16_t *__restrict__ x16, float *__restrict__ xscale, int gs,
+                                                         int nsteps, uint32_t *__restrict__ xg) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t rowh[];  // [Kp] halves
+    __shared__ float red[4];
+    __shared__ float gsum[256];
+    constexpr int KEEP = 4;  // chunks of 8 values a thread keeps in registers between the two passes
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const u32x4_t *xr = reinterpret_cast<const u32x4_t *>(x + static_cast<int64_t>(m) * ldx);
+    const int nchunks = K >> 3;
+    u32x4_t keep[KEEP];
+    float amax = 0.f;
+    auto chunk_amax = [&](u32x4_t v) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float a = fabsf(x_to_f32<XF16>(static_cast<uint16_t>(v[t] & 0xffffu)));
+            const float b = fabsf(x_to_f32<XF16>(static_cast<uint16_t>(v[t] >> 16)));
+            if (a == a && a <= 3.0e38f) amax = fmaxf(amax, a);
+            if (b == b && b <= 3.0e38f) amax = fmaxf(amax, b);
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+        const int c = tid + 256 * i;
+        keep[i] = u32x4_t{0u, 0u, 0u, 0u};
+        if (c < nchunks) {
+            keep[i] = xr[c];
+            chunk_amax(keep[i]);
+        }
+    }
+    for (int c = tid + 256 * KEEP; c < nchunks; c += 256) chunk_amax(xr[c]);
+    for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    int e = 0;
+    if (amax > 0.f) frexpf(amax, &e);
+    const float inv = ldexpf(1.f, 9 - e);
+    if (tid == 0) xscale[m] = ldexpf(1.f, e - 9);
+    u32x4_t *o16 = reinterpret_cast<u32x4_t *>(x16 + static_cast<int64_t>(m) * Kp);
+    u32x4_t *rowv = reinterpret_cast<u32x4_t *>(rowh);
+    auto emit = [&](int c, u32x4_t v) {
+        u32x4_t h;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t lo = f32_to_f16_rne(x_to_f32<XF16>(static_cast<uint16_t>(v[t] & 0xffffu)) * inv);
+            const uint32_t hi = f32_to_f16_rne(x_to_f32<XF16>(static_cast<uint16_t>(v[t] >> 16)) * inv);
+            h[t] = lo | (hi << 16);
+        }
+        o16[c] = h;
+        rowv[c] = h;
+    };
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i)
+        if (tid + 256 * i < nchunks) emit(tid + 256 * i, keep[i]);
+    for (int c = tid + 256 * KEEP; c < nchunks; c += 256) emit(c, xr[c]);
+    for (int c = nchunks + tid; c < (Kp >> 3); c += 256) {
+        o16[c] = u32x4_t{0u, 0u, 0u, 0u};
+        rowv[c] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    if (xg == nullptr) return;
+    __syncthreads();
+    for (int g0 = 0; g0 < nsteps * 16; g0 += 256) {
+        const int g = g0 + tid;
+        float acc = 0.f;
+        if (g < nsteps * 16)
+            for (int i = 0; i < gs; ++i) {
+                const int k = g * gs + i;
+                if (k < K) acc += f16_to_f32(rowh[k]);
+            }
+        __syncthreads();
+        gsum[tid] = acc;
+        __syncthreads();
+        if (tid < 64 && g0 / 16 + (tid >> 2) < nsteps) {
+            const int sl = tid >> 2, kb = tid & 3;
+            float X[4];
+            for (int j = 0; j < 4; ++j) X[j] = gsum[sl * 16 + 4 * j + kb];
+            u32x4_t out;
+            for (int p = 0; p < 2; ++p) {
+                const _Float16 h0 = static_cast<_Float16>(X[2 * p]), h1 = static_cast<_Float16>(X[2 * p + 1]);
+                const _Float16 l0 = static_cast<_Float16>(X[2 * p] - static_cast<float>(h0));
+                const _Float16 l1 = static_cast<_Float16>(X[2 * p + 1] - static_cast<float>(h1));
+                out[p] = __builtin_bit_cast(uint16_t, h0) | (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, h1)) << 16);
+                out[2 + p] = __builtin_bit_cast(uint16_t, l0) | (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, l1)) << 16);
+            }
+            *reinterpret_cast<u32x4_t *>(xg + ((static_cast<int64_t>(m) * nsteps + g0 / 16 + sl) * 4 + kb) * 4) = out;
+        }
+    }
+}
+
 // ---- fp16 NT GEMM: y[m, n] = sa[m] * sb[n] * sum_k a[m, k] * b[n, k] ----------------------
 // 128 x 128 x 32 block tile, 256 threads = 4 waves of 64 x 64 (2 x 2 MFMA 32x32x16 tiles).
 constexpr int GBM = 128, GBN = 128, GBK = 32, GLD = GBK + 8;  // LDS row stride in halves (80 bytes)
@@ -177,6 +270,18 @@ int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, i
 
 int x_prep_groups(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, int gs,
                   int nsteps, uint32_t *xg, hipStream_t st) {
+    const bool vec = K % 8 == 0 && ldx % 8 == 0 && Kp % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(x16) & 15) == 0 && Kp <= 28 * 1024;
+    if (vec) {
+        const size_t lds = static_cast<size_t>(Kp) * 2;
+        if (x_dtype == MFQ_X_F16)
+            hipLaunchKernelGGL((x_prep_vec_kernel<1>), dim3(M), dim3(256), lds, st, static_cast<const uint16_t *>(x), ldx, K,
+                               Kp, static_cast<uint16_t *>(x16), xscale, gs, nsteps, xg);
+        else
+            hipLaunchKernelGGL((x_prep_vec_kernel<0>), dim3(M), dim3(256), lds, st, static_cast<const uint16_t *>(x), ldx, K,
+                               Kp, static_cast<uint16_t *>(x16), xscale, gs, nsteps, xg);
+        return check_launch("x_prep");
+    }
     if (x_dtype == MFQ_X_F16)
         hipLaunchKernelGGL((x_prep_kernel<1>), dim3(M), dim3(256), 0, st, static_cast<const uint16_t *>(x), ldx, K, Kp,
                            static_cast<uint16_t *>(x16), xscale, gs, nsteps, xg);

@@ -835,7 +835,7 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
             }
             if (P.k[i].gs > max_gs) max_gs = P.k[i].gs;
         }
-        const size_t plds = 512 + static_cast<size_t>(2 * 64) * (4 * ((max_gs + 7) / 8 * 8) + 8) * 2;
+        const size_t plds = 512 + prefill_lds_bytes(64, max_gs);
         const dim3 pgrid(static_cast<unsigned>(tiles), static_cast<unsigned>(ceil_div(rbe, 32)));
         hipLaunchKernelGGL(moe_prefill_kernel, pgrid, dim3(512), plds, st, P, expert_pool, expert_local, E, out_per_expert, x16,
                            Kp, xscale, routed_input, R, ids_dst, expert_bounds, tile_bounds, tile_experts, out, ldo);

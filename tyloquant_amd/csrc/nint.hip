@@ -318,7 +318,7 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
     {                                                                                                          \
         const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, (NW / WM) * NB)),                        \
                         static_cast<unsigned>(ceil_div(M, WM * MT * 16)));                                     \
-        const size_t lds = static_cast<size_t>(2 * WM * MT * 16) * (4 * ((G + 7) / 8 * 8) + 8) * 2;            \
+        const size_t lds = prefill_lds_bytes(WM * MT * 16, G);                                                 \
         auto kern = nint_prefill_kernel<UNIT<B, G>, MT, NB, WM, NW>;                                           \
         if (lds > 65536) {                                                                                     \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                           \

@@ -13,6 +13,16 @@
 
 namespace mfq {
 
+constexpr int kMinSteps = 8;  // steps whose minimum-term operands a block stages at once
+
+// LDS bytes of a block of BM tile rows: two activation buffers of [BM][4 * GS' + 8] halves (GS' = groupsize padded to 8),
+// reused for the group sums of kMinSteps steps ([BM][kMinSteps * 16 + 4] dwords).
+inline size_t prefill_lds_bytes(int bm, int gs) {
+    const size_t xt = static_cast<size_t>(2 * bm) * (4 * ((gs + 7) / 8 * 8) + 8) * 2;
+    const size_t mn = static_cast<size_t>(bm) * (kMinSteps * 16 + 4) * 4;
+    return xt > mn ? xt : mn;
+}
+
 // Rows of a block tile: src(i) = row of x16 / xscale / xg that tile row i reads (always valid), dst(i) = row of y it
 // writes or -1.
 struct DenseRows {
@@ -28,7 +38,7 @@ struct MappedRows {  // both tables live in LDS
 
 // One block: tile rows `rows`, neurons of the row-blocks [rb_base, rb_base + WN * NB) below rb_end; y column of a
 // neuron = (row-block - rb_col0) * 16 + r, stored when below ncols.  xg: the group sums x_prep leaves,
-// [row][step][kb] x 16 bytes (see gemm.hip).  xt: LDS, two buffers of [BM][4 * GS + 8] halves.
+// [row][step][kb] x 16 bytes (see gemm.hip).  xt: LDS, prefill_lds_bytes(BM, GS) bytes.
 template <class U, int MT, int NB, int WM, int NW, class Rows>
 __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t *__restrict__ w, int rb_base, int rb_end,
                                                   int rb_col0, int ncols, const uint16_t *__restrict__ x16, int Kp,
@@ -187,40 +197,60 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
         ns[b] = anchors[rb * 16 + r] * 64.f;
         nm[b] = anchors[16 * k.n_rowblocks + rb * 16 + r];
     }
-    // sum_g sub_min_g X_g: one MFMA per step and tile, operands of step s + 1 requested while step s multiplies
+    // sum_g sub_min_g X_g: one MFMA per step and tile.  The operands of kMinSteps steps are requested at once --
+    // the tile rows' group sums through LDS (the activation buffers are free now), the sub_min bytes straight
+    // into registers -- so a chunk costs one round trip to memory instead of one per step.
     float4_t accM[MT][NB];
 #pragma unroll
     for (int a = 0; a < MT; ++a)
 #pragma unroll
         for (int b = 0; b < NB; ++b) accM[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
-    int64_t xgrow[MT];
+    constexpr int SC = kMinSteps, XGROW = SC * 16 + 4;  // dwords per tile row in LDS, padded against bank conflicts
+    constexpr int XG_PER_THREAD = (BM * SC * 4 + NT - 1) / NT;
+    uint32_t *xgl = reinterpret_cast<uint32_t *>(xt);
+    for (int c0 = 0; c0 < k.nsteps; c0 += SC) {
+        __syncthreads();  // the last reads of the activation tile / of the previous chunk are done
+        u32x4_t gx[XG_PER_THREAD];
 #pragma unroll
-    for (int a = 0; a < MT; ++a)
-        xgrow[a] = static_cast<int64_t>(rows.src((wm * MT + a) * 16 + r)) * k.nsteps * 16 + kb * 4;
-    u32x4_t ax[MT], axn[MT];
-    auto gload = [&](int s, u32x4_t (&dst)[MT]) {
-        const int sc_ = min(s, k.nsteps - 1);
-#pragma unroll
-        for (int a = 0; a < MT; ++a) dst[a] = *reinterpret_cast<const u32x4_t *>(xg + xgrow[a] + sc_ * 16);
-    };
-    sload(0, tails, sc);
-    gload(0, ax);
-    for (int s = 0; s < k.nsteps; ++s) {
-        sload(s + 1, tailsn, scn);
-        gload(s + 1, axn);
-#pragma unroll
-        for (int b = 0; b < NB; ++b) {
-            const half2_t m01 = pk_h2(ubyte_f32(sc[b].x, 1), ubyte_f32(sc[b].x, 3));
-            const half2_t m23 = pk_h2(ubyte_f32(sc[b].y, 1), ubyte_f32(sc[b].y, 3));
-            const uint32_t b01 = __builtin_bit_cast(uint32_t, m01), b23 = __builtin_bit_cast(uint32_t, m23);
-            const u32x4_t bfm = u32x4_t{b01, b23, b01, b23};
-#pragma unroll
-            for (int a = 0; a < MT; ++a) accM[a][b] = mfma16(ax[a], bfm, accM[a][b]);
+        for (int p = 0; p < XG_PER_THREAD; ++p) {
+            const int i = min(tid + NT * p, BM * SC * 4 - 1);
+            const int row = i / (SC * 4), rem = i - row * (SC * 4);
+            const int sc_ = min(c0 + (rem >> 2), k.nsteps - 1);
+            gx[p] = *reinterpret_cast<const u32x4_t *>(xg + (static_cast<int64_t>(rows.src(row)) * k.nsteps + sc_) * 16 + (rem & 3) * 4);
         }
+        u32x2_t scs[SC][NB];
 #pragma unroll
-        for (int b = 0; b < NB; ++b) sc[b] = scn[b];
+        for (int t = 0; t < SC; ++t)
 #pragma unroll
-        for (int a = 0; a < MT; ++a) ax[a] = axn[a];
+            for (int b = 0; b < NB; ++b) {
+                const int s = c0 + t;
+                const uint32_t off = b < nrb && s < k.nsteps ? b * rbb + s * sb + 1024 * D + (U::TAIL ? 256 : 0) : kNoStep;
+                scs[t][b] = __builtin_amdgcn_raw_buffer_load_b64(win, off + lane * 8, 0, 0);
+            }
+#pragma unroll
+        for (int p = 0; p < XG_PER_THREAD; ++p) {
+            const int i = tid + NT * p;
+            const int row = i / (SC * 4), rem = i - row * (SC * 4);
+            if (i < BM * SC * 4) *reinterpret_cast<u32x4_t *>(xgl + row * XGROW + rem * 4) = gx[p];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < SC; ++t) {
+            if (c0 + t >= k.nsteps) break;
+            u32x4_t ax[MT];
+#pragma unroll
+            for (int a = 0; a < MT; ++a)
+                ax[a] = *reinterpret_cast<const u32x4_t *>(xgl + ((wm * MT + a) * 16 + r) * XGROW + t * 16 + kb * 4);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const half2_t m01 = pk_h2(ubyte_f32(scs[t][b].x, 1), ubyte_f32(scs[t][b].x, 3));
+                const half2_t m23 = pk_h2(ubyte_f32(scs[t][b].y, 1), ubyte_f32(scs[t][b].y, 3));
+                const uint32_t b01 = __builtin_bit_cast(uint32_t, m01), b23 = __builtin_bit_cast(uint32_t, m23);
+                const u32x4_t bfm = u32x4_t{b01, b23, b01, b23};
+#pragma unroll
+                for (int a = 0; a < MT; ++a) accM[a][b] = mfma16(ax[a], bfm, accM[a][b]);
+            }
+        }
     }
 #pragma unroll
     for (int a = 0; a < MT; ++a) {
