@@ -340,8 +340,11 @@ extern "C" int mfq_hip_gemm_f16_nt(const void *a, int64_t lda, const void *b, in
 static constexpr int kGemvMaxM = 8, kStreamMaxM = 256;
 static bool nint_streams(const mfq_nint_desc *d, int M) {
     static const int env_max = [] { const char *e = getenv("MFQ_STREAM_MAX_M"); return e ? atoi(e) : 0; }();
-    // the prefill kernel takes over earlier when it has enough neurons to fill the chip with 512-neuron blocks
-    int stream_max = nint_prefill_capable(d) ? (d->out >= 8192 ? 128 : 192) : kStreamMaxM;
+    // measured crossovers with the prefill kernel, whose time is flat up to a few hundred rows: it takes over earlier
+    // when it has enough neurons to fill the chip with 512-neuron blocks, and for the natural-order unit, whose
+    // unpack costs the streaming kernel more per 16-row pass
+    int stream_max = kStreamMaxM;
+    if (nint_prefill_capable(d)) stream_max = d->kind != 1 ? 64 : (d->out >= 8192 ? 112 : 160);
     if (env_max > 0) stream_max = env_max;
     return M <= kGemvMaxM || (M <= stream_max && nint_stream_capable(d));
 }
