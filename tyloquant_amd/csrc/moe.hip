@@ -558,10 +558,23 @@ __global__ __launch_bounds__(512) void moe_prefill_kernel(MoePools P, const int3
     const int rb_base = rb_first + static_cast<int>(blockIdx.y) * 32;
     const NintK &k = P.k[pool];
     const MappedRows rows{srcv, dstv};
+    // up to 16 / 32 pairs: a 16- / 32-row tile with a whole step of weights and activations in flight (the weight stream
+    // sets the pace); else the 64-row tile of the dense prefill kernel
+    const int npair = hi - lo;
 #define MFQ_MOE_PREFILL(UNIT, B, G)                                                                                  \
-    if (k.bits == B && k.gs == G)                                                                                    \
-        nint_prefill_body<UNIT<B, G>, 4, 4, 1, 8>(k, P.w[pool], rb_base, rb_first + rbe, rb_first, out_per_expert, x16, Kp, \
-                                                  xscale, P.xg[pool], rows, out, ldo, xt);
+    if (k.bits == B && k.gs == G) {                                                                                  \
+        if (npair <= kMoeTileM)                                                                                      \
+            nint_prefill_body<UNIT<B, G>, 1, 4, 1, 8, MappedRows, 4>(k, P.w[pool], rb_base, rb_first + rbe, rb_first,  \
+                                                                     out_per_expert, x16, Kp, xscale, P.xg[pool], rows, \
+                                                                     out, ldo, xt);                                  \
+        else if (npair <= 2 * kMoeTileM)                                                                             \
+            nint_prefill_body<UNIT<B, G>, 2, 4, 1, 8, MappedRows, 4>(k, P.w[pool], rb_base, rb_first + rbe, rb_first,  \
+                                                                     out_per_expert, x16, Kp, xscale, P.xg[pool], rows, \
+                                                                     out, ldo, xt);                                  \
+        else                                                                                                         \
+            nint_prefill_body<UNIT<B, G>, 4, 4, 1, 8>(k, P.w[pool], rb_base, rb_first + rbe, rb_first, out_per_expert, \
+                                                      x16, Kp, xscale, P.xg[pool], rows, out, ldo, xt);              \
+    }
     if (k.kind == 1) {
         MFQ_MOE_PREFILL(PairedUnit, 4, 24)
         else MFQ_MOE_PREFILL(PairedUnit, 3, 24)

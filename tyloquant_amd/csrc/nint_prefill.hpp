@@ -39,7 +39,10 @@ struct MappedRows {  // both tables live in LDS
 // One block: tile rows `rows`, neurons of the row-blocks [rb_base, rb_base + WN * NB) below rb_end; y column of a
 // neuron = (row-block - rb_col0) * 16 + r, stored when below ncols.  xg: the group sums x_prep leaves,
 // [row][step][kb] x 16 bytes (see gemm.hip).  xt: LDS, prefill_lds_bytes(BM, GS) bytes.
-template <class U, int MT, int NB, int WM, int NW, class Rows>
+// PF: register buffers of weight units per row-block; the unit of sub-step it + PF - 1 is requested while sub-step it
+// multiplies (2 = ping-pong; 4 keeps a whole step in flight for tiles with few rows, where the weight stream and
+// not the matrix cores sets the pace).
+template <class U, int MT, int NB, int WM, int NW, class Rows, int PF = 2>
 __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t *__restrict__ w, int rb_base, int rb_end,
                                                   int rb_col0, int ncols, const uint16_t *__restrict__ x16, int Kp,
                                                   const float *__restrict__ xscale, const uint32_t *__restrict__ xg,
@@ -75,8 +78,9 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
         for (int b = 0; b < NB; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // global -> register copy of the activation tile of sub-step `it` (chunk c of a row = 8 halves at k0 + 8 c)
-    chunk_t xr[PER_THREAD];
-    auto xload = [&](int it) {
+    constexpr int XD = PF == 4 ? 4 : 1;  // activation tiles in flight in registers
+    chunk_t xr[XD][PER_THREAD];
+    auto xload = [&](int it, chunk_t (&xq)[PER_THREAD]) {
         const int k0 = it * 4 * GS;
 #pragma unroll
         for (int p = 0; p < PER_THREAD; ++p) {
@@ -87,17 +91,17 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
             const int kc = min(kk, Kp - EL);
             chunk_t v = *reinterpret_cast<const chunk_t *>(x16 + static_cast<int64_t>(m) * Kp + kc);
             if (kk >= Kp) v = chunk_t(0u);
-            xr[p] = v;
+            xq[p] = v;
         }
     };
-    auto xstore = [&](int buf) {
+    auto xstore = [&](int buf, const chunk_t (&xq)[PER_THREAD]) {
 #pragma unroll
         for (int p = 0; p < PER_THREAD; ++p) {
             const int c = tid + NT * p;
             const int row = c / CHUNKS, ch = c - row * CHUNKS;
             const int g = ch / CPG, ci = ch - g * CPG;
             if (c < BM * CHUNKS)
-                *reinterpret_cast<chunk_t *>(xt + buf * (BM * ROW) + row * ROW + g * GSP + EL * ci) = xr[p];
+                *reinterpret_cast<chunk_t *>(xt + buf * (BM * ROW) + row * ROW + g * GSP + EL * ci) = xq[p];
         }
     };
     if constexpr (GSP != GS) {  // the padding halves of a group are multiplied by zero weights: keep them finite
@@ -105,7 +109,8 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
         __syncthreads();
     }
 
-    uint32_t q[NB][D], qn[NB][D], tails[NB], tailsn[NB];
+    static_assert(PF == 2 || PF == 4, "the sub-step loop is unrolled four times");
+    uint32_t qr[PF][NB][D], tails[NB], tailsn[NB];
     u32x2_t sc[NB], scn[NB];
     auto wload = [&](int it, uint32_t (&qq)[NB][D]) {
         const int s = it >> 2, j = it & 3;
@@ -123,19 +128,21 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
         }
     };
 
-    xload(0);
-    wload(0, q);
+    xload(0, xr[0]);
+#pragma unroll
+    for (int i = 0; i < PF - 1; ++i) wload(i, qr[i]);
     sload(0, tails, sc);
-    xstore(0);
+    xstore(0, xr[0]);
+#pragma unroll
+    for (int i = 1; i < XD; ++i) xload(i, xr[i]);
     __syncthreads();
     for (int s = 0; s < k.nsteps; ++s) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int it = 4 * s + j;
-        xload(it + 1);  // past the end: clamped addresses, zeros
-        if (j & 1) wload(it + 1, q);
-        else wload(it + 1, qn);
-        if (j == 3) sload(s + 1, tailsn, scn);
+        xload(it + XD, xr[j % XD]);  // past the end: clamped addresses, zeros
+        wload(it + PF - 1, qr[(j + PF - 1) % PF]);
+        if (j == (PF == 4 ? 0 : 3)) sload(s + 1, tailsn, scn);
 
         // fragment scale S = sub_scale / 64 / 2^o and bias C = -1024 S, both from the fp16 pair 1024 + sub_scale
         // (the byte dropped into the mantissa of 1024.0) with one exact packed FMA each
@@ -166,7 +173,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 uint32_t v[U::NPAIR];
-                U::unpack((j & 1) ? qn[b] : q[b], (tails[b] >> (8 * j)) & 0xffu, v);
+                U::unpack(qr[j % PF][b], (tails[b] >> (8 * j)) & 0xffu, v);
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                     bf[b][t] = __builtin_bit_cast(uint32_t, h2_fma(v[4 * m + t], S[b][U::cls(4 * m + t)], C[b][U::cls(4 * m + t)]));
@@ -176,7 +183,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
 #pragma unroll
                 for (int a = 0; a < MT; ++a) acc[a][b] = mfma16(af[a], bf[b], acc[a][b]);
         }
-        xstore((j + 1) & 1);  // the other buffer: nobody reads it during this sub-step
+        xstore((j + 1) & 1, xr[(j + 1) % XD]);  // the other buffer: nobody reads it during this sub-step
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             if (j == 3) {
