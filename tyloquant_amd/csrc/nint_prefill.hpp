@@ -36,7 +36,7 @@ struct MappedRows {  // both tables live in LDS
     __device__ __forceinline__ int dst(int i) const { return dstv[i]; }
 };
 
-// One block: tile rows `rows`, neurons of the row-blocks [rb_base, rb_base + WN * NB) below rb_end; y column of a
+// One block: tile rows `rows`, neurons of the row-blocks [rb_base, rb_base + (NW / WM) * NB) below rb_end; y column of a
 // neuron = (row-block - rb_col0) * 16 + r, stored when below ncols.  xg: the group sums x_prep leaves,
 // [row][step][kb] x 16 bytes (see gemm.hip).  xt: LDS, prefill_lds_bytes(BM, GS) bytes.
 // PF: register buffers of weight units per row-block; the unit of sub-step it + PF - 1 is requested while sub-step it
@@ -49,7 +49,6 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
                                                   const Rows &rows, float *__restrict__ y, int64_t ldy, uint16_t *xt) {
     constexpr int D = U::D, GS = U::GROUP, NM = U::NPAIR / 4, BITS = U::CBITS;
     constexpr int NCLS = BITS == 0 ? 1 : (BITS == 3 ? 3 : 2);
-    constexpr int WN = NW / WM;                // waves along the neurons
     constexpr int NT = 64 * NW;                // threads
     constexpr int BM = WM * MT * 16;           // tokens per block
     constexpr int EL = GS % 8 == 0 ? 8 : 4;    // halves per copy chunk (16 or 8 bytes)
@@ -80,16 +79,23 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
     // global -> register copy of the activation tile of sub-step `it` (chunk c of a row = 8 halves at k0 + 8 c)
     constexpr int XD = PF == 4 ? 4 : 1;  // activation tiles in flight in registers
     chunk_t xr[XD][PER_THREAD];
+    // the thread's chunks of a tile: source row (looked up once: a mapped tile keeps its row table in LDS) and k offset
+    const uint16_t *xsrc[PER_THREAD];
+    int xk[PER_THREAD];
+#pragma unroll
+    for (int p = 0; p < PER_THREAD; ++p) {
+        const int c = min(tid + NT * p, BM * CHUNKS - 1);
+        const int row = c / CHUNKS;
+        xsrc[p] = x16 + static_cast<int64_t>(rows.src(row)) * Kp;
+        xk[p] = EL * (c - row * CHUNKS);  // groups are contiguous in k: chunk ch of the row starts EL * ch further
+    }
     auto xload = [&](int it, chunk_t (&xq)[PER_THREAD]) {
         const int k0 = it * 4 * GS;
 #pragma unroll
         for (int p = 0; p < PER_THREAD; ++p) {
-            const int c = min(tid + NT * p, BM * CHUNKS - 1);
-            const int row = c / CHUNKS, ch = c - row * CHUNKS;
-            const int m = rows.src(row);
-            const int kk = k0 + EL * ch;  // groups are contiguous in k: chunk ch of the row starts here
+            const int kk = k0 + xk[p];
             const int kc = min(kk, Kp - EL);
-            chunk_t v = *reinterpret_cast<const chunk_t *>(x16 + static_cast<int64_t>(m) * Kp + kc);
+            chunk_t v = *reinterpret_cast<const chunk_t *>(xsrc[p] + kc);
             if (kk >= Kp) v = chunk_t(0u);
             xq[p] = v;
         }
