@@ -335,16 +335,22 @@ extern "C" int mfq_hip_gemm_f16_nt(const void *a, int64_t lda, const void *b, in
 
 // Up to kGemvMaxM activation rows the weight stream dominates and the GEMV kernels win; tensors with a
 // matrix-core streaming kernel (16 rows per pass over the packed weights) stay on it up to kStreamMaxM rows,
-// where re-streaming the weights is still cheaper than dequantizing them to fp16 once, or up to the measured
-// crossover with the prefill kernel.
+// where re-streaming the weights is still cheaper than dequantizing them to fp16 once, or up to the crossover
+// with the prefill kernel.  That crossover comes from a two-line model fitted to measurements on 4096..12288-wide
+// tensors: 64 rows of streaming cost about 8 us + 0.85 us per MB of payload (twice that for the natural-order
+// unit), the prefill kernel a flat 10 us + 12.6 us per 1024 of K up to a few hundred rows (its blocks walk all of
+// K; a quarter more for the natural-order unit).
 static constexpr int kGemvMaxM = 8, kStreamMaxM = 256;
 static bool nint_streams(const mfq_nint_desc *d, int M) {
     static const int env_max = [] { const char *e = getenv("MFQ_STREAM_MAX_M"); return e ? atoi(e) : 0; }();
-    // measured crossovers with the prefill kernel, whose time is flat up to a few hundred rows: it takes over earlier
-    // when it has enough neurons to fill the chip with 512-neuron blocks, and for the natural-order unit, whose
-    // unpack costs the streaming kernel more per 16-row pass
     int stream_max = kStreamMaxM;
-    if (nint_prefill_capable(d)) stream_max = d->kind != 1 ? 64 : (d->out >= 8192 ? 112 : 160);
+    if (nint_prefill_capable(d)) {
+        const bool natural = d->kind != 1;
+        const double t64 = (8.0 + 0.85e-6 * static_cast<double>(d->payload_bytes)) * (natural ? 2.0 : 1.0);
+        const double tp = (10.0 + 12.6 * d->neuron_len / 1024.0) * (natural ? 1.25 : 1.0);
+        const int m = static_cast<int>(64.0 * tp / t64) / 16 * 16;
+        stream_max = m < 64 ? 64 : (m > 512 ? 512 : m);
+    }
     if (env_max > 0) stream_max = env_max;
     return M <= kGemvMaxM || (M <= stream_max && nint_stream_capable(d));
 }

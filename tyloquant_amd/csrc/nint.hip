@@ -296,8 +296,13 @@ static int launch_mfma_nb(const NintK &k, const uint8_t *w, const uint16_t *x, i
 template <int XF16>
 static int launch_mfma(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                        hipStream_t st) {
-    // row-blocks per wave: as many as still leave about 1500 waves (a block has at most 8)
-    const int64_t wpb = k.nsteps < 8 ? k.nsteps : 8;
+    // row-blocks per wave: as many as still leave about 1500 waves over all 16-row tiles (a block has at most 8 waves);
+    // more row-blocks share the activation fragments, and the tiles of one row-block group re-read its weights from L2
+    const int64_t wpb = (k.nsteps < 8 ? k.nsteps : 8) * ceil_div(M, 16);
+    static const int env_nb = [] { const char *e = getenv("MFQ_MFMA_NB"); return e ? atoi(e) : 0; }();
+    if (env_nb == 4) return launch_mfma_nb<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
+    if (env_nb == 2) return launch_mfma_nb<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
+    if (env_nb == 1) return launch_mfma_nb<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
     if (ceil_div(k.n_rowblocks, 4) * wpb >= 1536) return launch_mfma_nb<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
     if (ceil_div(k.n_rowblocks, 2) * wpb >= 1536) return launch_mfma_nb<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
     return launch_mfma_nb<XF16, 1>(k, w, x, ldx, M, y, ldy, st);

@@ -34,6 +34,24 @@ __device__ __forceinline__ u32x4_t load_xfrag(const uint16_t *__restrict__ xrow,
     if (kpos >= K) v = u32x4_t{0u, 0u, 0u, 0u};
     return v;
 }
+// The same in two halves for a software pipeline: the request (clamped address, 16 raw bytes) and, when the value is
+// needed, the conversion to fp16 and the zeroing at and beyond K.
+template <bool ALIGN8>
+__device__ __forceinline__ u32x4_t load_xfrag_raw(const uint16_t *__restrict__ xrow, int kpos, int K) {
+    const int kc = max(0, min(kpos, K - 8));
+    if constexpr (ALIGN8) return *reinterpret_cast<const u32x4_t *>(xrow + kc);
+    else return *reinterpret_cast<const u32x4_a4_t *>(xrow + kc);
+}
+template <int XF16, bool ALIGN8>
+__device__ __forceinline__ u32x4_t xfrag_finish(u32x4_t v, int kpos, int K) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) v[t] = to_h2<XF16>(v[t]);
+    if constexpr (!ALIGN8) {
+        if (kpos + 4 == K) v = u32x4_t{v.z, v.w, 0u, 0u};
+    }
+    if (kpos >= K) v = u32x4_t{0u, 0u, 0u, 0u};
+    return v;
+}
 
 __device__ __forceinline__ half2_t pk_h2(float lo, float hi) {
     return __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
@@ -98,19 +116,51 @@ __device__ __forceinline__ void nint_mfma_body(const NintK &k, const uint8_t *__
 #pragma unroll
     for (int i = 0; i < NB; ++i) accS[i] = accM[i] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int s = 0; s < n; ++s) {
-        uint32_t q[NB][4][D], tails[NB];
-        u32x2_t sc[NB];
+    // One step of register buffers per row-block, refilled unit by unit: as soon as unit j of step s is unpacked, unit j
+    // of step s + 1 is requested into the same registers, so the weight stream runs most of a step ahead of the unpack
+    // without a second set of buffers.  Requests past the wave's last step are out-of-range offsets that move no data.
+    uint32_t q[NB][4][D], tails[NB], tailsn[NB];
+    u32x2_t sc[NB], scn[NB];
+    auto unit_off = [&](int i, int s, int j) -> uint32_t {
+        return i < nrb && s < n ? i * rbb + s * sb + (j * 64 + lane) * (D * 4) : kNoStep;
+    };
+    auto scale_load = [&](int s, uint32_t (&tt)[NB], u32x2_t (&ss)[NB]) {
 #pragma unroll
-        for (int i = 0; i < NB; ++i)
-            nint_load_step<D, U::TAIL>(win, i < nrb ? i * rbb + s * sb : kNoStep, lane, q[i], tails[i], sc[i]);
-        const int kbase = (s0 + s) * 16 * GS + kb * GS;
+        for (int i = 0; i < NB; ++i) {
+            const uint32_t off = i < nrb && s < n ? i * rbb + s * sb + 1024 * D : kNoStep;
+            tt[i] = 0;
+            if constexpr (U::TAIL) tt[i] = __builtin_amdgcn_raw_buffer_load_b32(win, off + lane * 4, 0, 2);
+            ss[i] = __builtin_amdgcn_raw_buffer_load_b64(win, off + (U::TAIL ? 256 : 0) + lane * 8, 0, 2);
+        }
+    };
+    scale_load(0, tails, sc);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < NB; ++i) load_unit_win<D>(win, unit_off(i, 0, j), q[i][j]);
+    // Activation fragments run two units ahead of their use and are requested before the weight refill of the unit:
+    // loads retire in order, so a fragment waits for the refills issued before it -- three units old by then -- and
+    // never for the one just issued.
+    auto xfrags = [&](int it, u32x4_t (&dst)[NM]) {  // fragments of unit it (= 4 * step + j) of the wave's K-slice
+        const int kpos = (s0 + (it >> 2)) * 16 * GS + kb * GS + 4 * (it & 3) * GS;
+#pragma unroll
+        for (int m = 0; m < NM; ++m) dst[m] = load_xfrag_raw<ALIGN8>(xrow, kpos + 8 * m, k.neuron_len);
+    };
+    u32x4_t a1[NM], a2[NM];
+    xfrags(0, a1);
+    xfrags(1, a2);
+    for (int s = 0; s < n; ++s) {
+        scale_load(s + 1, tailsn, scn);
         float xsum[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             u32x4_t a[NM];
 #pragma unroll
-            for (int m = 0; m < NM; ++m) a[m] = load_xfrag<XF16, ALIGN8>(xrow, kbase + 4 * j * GS + 8 * m, k.neuron_len);
+            for (int m = 0; m < NM; ++m) {
+                a[m] = xfrag_finish<XF16, ALIGN8>(a1[m], (s0 + s) * 16 * GS + kb * GS + 4 * j * GS + 8 * m, k.neuron_len);
+                a1[m] = a2[m];
+            }
+            xfrags(4 * s + j + 2, a2);
             float xs = 0.f;
 #pragma unroll
             for (int m = 0; m < NM; ++m)
@@ -131,6 +181,7 @@ __device__ __forceinline__ void nint_mfma_body(const NintK &k, const uint8_t *__
                 }
                 uint32_t v[U::NPAIR];
                 U::unpack(q[i][j], (tails[i] >> (8 * j)) & 0xffu, v);
+                load_unit_win<D>(win, unit_off(i, s + 1, j), q[i][j]);
 #pragma unroll
                 for (int m = 0; m < NM; ++m) {
                     u32x4_t b;
@@ -159,6 +210,11 @@ __device__ __forceinline__ void nint_mfma_body(const NintK &k, const uint8_t *__
             const half2_t m23 = pk_h2(ubyte_f32(sc[i].y, 1), ubyte_f32(sc[i].y, 3));
             const uint32_t b01 = __builtin_bit_cast(uint32_t, m01), b23 = __builtin_bit_cast(uint32_t, m23);
             accM[i] = mfma16(ax, u32x4_t{b01, b23, b01, b23}, accM[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            tails[i] = tailsn[i];
+            sc[i] = scn[i];
         }
     }
 #pragma unroll
