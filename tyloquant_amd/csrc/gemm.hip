@@ -338,7 +338,7 @@ extern "C" int mfq_hip_gemm_f16_nt(const void *a, int64_t lda, const void *b, in
 // where re-streaming the weights is still cheaper than dequantizing them to fp16 once, or up to the crossover
 // with the prefill kernel.  That crossover comes from a two-line model fitted to measurements on 4096..12288-wide
 // tensors: 64 rows of streaming cost about 8 us + 0.85 us per MB of payload (twice that for the natural-order
-// unit), the prefill kernel a flat 10 us + 12.6 us per 1024 of K up to a few hundred rows (its blocks walk all of
+// unit), the prefill kernel a flat 17 us + 8.2 us per 1024 of K up to a few hundred rows (its blocks walk all of
 // K; a quarter more for the natural-order unit).
 static constexpr int kGemvMaxM = 8, kStreamMaxM = 256;
 static bool nint_streams(const mfq_nint_desc *d, int M) {
@@ -347,7 +347,7 @@ static bool nint_streams(const mfq_nint_desc *d, int M) {
     if (nint_prefill_capable(d)) {
         const bool natural = d->kind != 1;
         const double t64 = (8.0 + 0.85e-6 * static_cast<double>(d->payload_bytes)) * (natural ? 2.0 : 1.0);
-        const double tp = (10.0 + 12.6 * d->neuron_len / 1024.0) * (natural ? 1.25 : 1.0);
+        const double tp = (17.0 + 8.2 * d->neuron_len / 1024.0) * (natural ? 1.25 : 1.0);
         const int m = static_cast<int>(64.0 * tp / t64) / 16 * 16;
         stream_max = m < 64 ? 64 : (m > 512 ? 512 : m);
     }

@@ -319,27 +319,29 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
                  uint32_t *xg, int M, float *y, int64_t ldy, hipStream_t st) {
     const NintK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
-#define MFQ_PREFILL_CFG(UNIT, B, G, MT, NB, WM, NW)                                                                 \
+#define MFQ_PREFILL_CFG(UNIT, B, G, MT, NB, PF, XD)                                                                 \
     {                                                                                                          \
-        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, (NW / WM) * NB)),                        \
-                        static_cast<unsigned>(ceil_div(M, WM * MT * 16)));                                     \
-        const size_t lds = prefill_lds_bytes(WM * MT * 16, G);                                                 \
-        auto kern = nint_prefill_kernel<UNIT<B, G>, MT, NB, WM, NW>;                                           \
+        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, 8 * NB)),                                \
+                        static_cast<unsigned>(ceil_div(M, MT * 16)));                                          \
+        const size_t lds = prefill_lds_bytes(MT * 16, G);                                                      \
+        auto kern = nint_prefill_kernel<UNIT<B, G>, MT, NB, 1, 8, PF, XD>;                                     \
         if (lds > 65536) {                                                                                     \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                           \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
             MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nint_prefill: %s", hipGetErrorString(e));            \
         }                                                                                                      \
-        hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, st, k, w, x16, Kp, xscale, xg, M, y, ldy);          \
+        hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, k, w, x16, Kp, xscale, xg, M, y, ldy);              \
         return check_launch("nint_prefill");                                                                   \
     }
-    // wave tile MT*16 tokens x NB*16 neurons, NW waves side by side on the neurons
-    // 512 neurons per block; 256 when that leaves CUs without a block
-    const bool narrow = ceil_div(k.n_rowblocks, 32) * ceil_div(M, 64) < 256;
+    // Block = 8 waves side by side on 256 neurons (two row-blocks per wave), each with four unit buffers per row-block
+    // (three sub-steps of weights in flight).  While 64-token tiles give at most one block per CU, they are used with
+    // four activation tiles in flight: the time is then that of one block's walk through K, and short tiles walk
+    // fastest.  Beyond that, 128-token tiles: every dequantized fragment feeds eight MFMAs instead of four.
+    const bool small = ceil_div(k.n_rowblocks, 16) * ceil_div(M, 64) <= 256;
 #define MFQ_PREFILL(UNIT, B, G)                              \
     if (k.bits == B && k.gs == G) {                          \
-        if (narrow) MFQ_PREFILL_CFG(UNIT, B, G, 4, 2, 1, 8)  \
-        MFQ_PREFILL_CFG(UNIT, B, G, 4, 4, 1, 8)              \
+        if (small) MFQ_PREFILL_CFG(UNIT, B, G, 4, 2, 4, 4)   \
+        MFQ_PREFILL_CFG(UNIT, B, G, 8, 2, 4, (UNIT<B, G>::D >= 5 ? 1 : 2)) /* wide units: registers for one tile */ \
     }
     if (k.kind == 1) {
         MFQ_PREFILL(PairedUnit, 4, 32) MFQ_PREFILL(PairedUnit, 4, 24) MFQ_PREFILL(PairedUnit, 4, 16)

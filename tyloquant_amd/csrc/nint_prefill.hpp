@@ -42,7 +42,7 @@ struct MappedRows {  // both tables live in LDS
 // PF: register buffers of weight units per row-block; the unit of sub-step it + PF - 1 is requested while sub-step it
 // multiplies (2 = ping-pong; 4 keeps a whole step in flight for tiles with few rows, where the weight stream and
 // not the matrix cores sets the pace).
-template <class U, int MT, int NB, int WM, int NW, class Rows, int PF = 2>
+template <class U, int MT, int NB, int WM, int NW, class Rows, int PF = 2, int XD = (PF == 4 ? 4 : 1)>
 __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t *__restrict__ w, int rb_base, int rb_end,
                                                   int rb_col0, int ncols, const uint16_t *__restrict__ x16, int Kp,
                                                   const float *__restrict__ xscale, const uint32_t *__restrict__ xg,
@@ -77,7 +77,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
         for (int b = 0; b < NB; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // global -> register copy of the activation tile of sub-step `it` (chunk c of a row = 8 halves at k0 + 8 c)
-    constexpr int XD = PF == 4 ? 4 : 1;  // activation tiles in flight in registers
+    static_assert(XD == 1 || XD == 2 || XD == 4, "activation tiles in flight in registers");
     chunk_t xr[XD][PER_THREAD];
     // the thread's chunks of a tile: source row (looked up once: a mapped tile keeps its row table in LDS) and k offset
     const uint16_t *xsrc[PER_THREAD];
@@ -284,7 +284,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
 }
 
 // Dense wrapper: block (neuron tile, token tile).
-template <class U, int MT, int NB, int WM, int NW>
+template <class U, int MT, int NB, int WM, int NW, int PF = 2, int XD = (PF == 4 ? 4 : 1)>
 __global__ __launch_bounds__(64 * NW) void nint_prefill_kernel(NintK k, const uint8_t *__restrict__ w,
                                                                const uint16_t *__restrict__ x16, int Kp,
                                                                const float *__restrict__ xscale,
@@ -292,8 +292,8 @@ __global__ __launch_bounds__(64 * NW) void nint_prefill_kernel(NintK k, const ui
                                                                float *__restrict__ y, int64_t ldy) {
     extern __shared__ __attribute__((aligned(16))) uint16_t xt[];
     const DenseRows rows{static_cast<int>(blockIdx.y) * WM * MT * 16, M};
-    nint_prefill_body<U, MT, NB, WM, NW>(k, w, static_cast<int>(blockIdx.x) * (NW / WM) * NB, k.n_rowblocks, 0, k.out, x16, Kp,
-                                         xscale, xg, rows, y, ldy, xt);
+    nint_prefill_body<U, MT, NB, WM, NW, DenseRows, PF, XD>(k, w, static_cast<int>(blockIdx.x) * (NW / WM) * NB, k.n_rowblocks, 0,
+                                                        k.out, x16, Kp, xscale, xg, rows, y, ldy, xt);
 }
 
 }  // namespace mfq
