@@ -90,6 +90,21 @@ def test_gemm_matches_oracle(bits, gs, sb, out, K, M):
     assert np.abs(y - ref).max() < ABS_TOL
 
 
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (4, 48, 6)])
+def test_gemm_many_rows_takes_the_128_token_tiles(bits, gs, sb):
+    """More than one block per CU (5 neuron blocks x 53 token tiles of 64): the prefill kernel switches to its 128-token
+    tile.  Ragged everywhere: 65 row-blocks, K not a multiple of the groupsize, one token past 26 full tiles."""
+    rng = np.random.default_rng(270 + bits)
+    out, K, M = 1040, 280, 3329
+    t = O.quantize_nint((rng.standard_normal((out, K)) * 0.02).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    x, xf = _x(rng, M, K)
+    y = lin(x).cpu().numpy()
+    ref = O.linear_forward_f64(O.dequantize_nint(t), xf)
+    assert rel_l2(y, ref) < REL_TOL, rel_l2(y, ref)
+    assert np.abs(y - ref).max() < ABS_TOL
+
+
 def test_config1_shape_nint3():
     """BASELINE config 1: 4096x4096 N(0, 0.02) NINT3 (3,24,5), bf16 x at batch 1."""
     from tyloquant_amd import runtime as R
