@@ -105,6 +105,22 @@ def test_gemm_many_rows_takes_the_128_token_tiles(bits, gs, sb):
     assert np.abs(y - ref).max() < ABS_TOL
 
 
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (5, 28, 7)])
+def test_gemm_long_k_few_neurons_is_split_over_k(bits, gs, sb):
+    """A grid of nine 64-token tiles on 256 neurons leaves most CUs idle: the prefill launch is cut along K (four
+    splits of five steps, the last one shorter and ragged) and the partial results are added afterwards."""
+    rng = np.random.default_rng(370 + bits)
+    out, K, M = 256, 8200, 520
+    t = O.quantize_nint((rng.standard_normal((out, K)) * 0.02).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    x, xf = _x(rng, M, K)
+    y = lin(x).cpu().numpy()
+    ref = O.linear_forward_f64(O.dequantize_nint(t), xf)
+    assert rel_l2(y, ref) < REL_TOL, rel_l2(y, ref)
+    assert np.abs(y - ref).max() < ABS_TOL
+    assert np.array_equal(y, lin(x).cpu().numpy())   # partial sums are added in a fixed order
+
+
 def test_config1_shape_nint3():
     """BASELINE config 1: 4096x4096 N(0, 0.02) NINT3 (3,24,5), bf16 x at batch 1."""
     from tyloquant_amd import runtime as R

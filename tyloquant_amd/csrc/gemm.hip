@@ -317,8 +317,9 @@ int nint_dequant_f16(const mfq_nint_desc *d, const void *weight, void *w16, int6
 bool nint_stream_capable(const mfq_nint_desc *d);
 bool nint_prefill_capable(const mfq_nint_desc *d);
 size_t nint_prefill_xg_bytes(const mfq_nint_desc *d, int M);
+size_t nint_prefill_split_bytes(const mfq_nint_desc *d, int M);
 int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16, int Kp, const float *xscale, uint32_t *xg,
-                 int M, float *y, int64_t ldy, hipStream_t st);
+                 int M, float *y, int64_t ldy, float *part, hipStream_t st);
 
 }  // namespace mfq
 
@@ -338,8 +339,8 @@ extern "C" int mfq_hip_gemm_f16_nt(const void *a, int64_t lda, const void *b, in
 // where re-streaming the weights is still cheaper than dequantizing them to fp16 once, or up to the crossover
 // with the prefill kernel.  That crossover comes from a two-line model fitted to measurements on 4096..12288-wide
 // tensors: 64 rows of streaming cost about 8 us + 0.85 us per MB of payload (twice that for the natural-order
-// unit), the prefill kernel a flat 17 us + 8.2 us per 1024 of K up to a few hundred rows (its blocks walk all of
-// K; a quarter more for the natural-order unit).
+// unit), the prefill kernel a flat 30 us + 1.9 us per 1024 of K up to a few hundred rows (small grids are split
+// over K; a quarter more for the natural-order unit).
 static constexpr int kGemvMaxM = 8, kStreamMaxM = 256;
 static bool nint_streams(const mfq_nint_desc *d, int M) {
     static const int env_max = [] { const char *e = getenv("MFQ_STREAM_MAX_M"); return e ? atoi(e) : 0; }();
@@ -347,7 +348,7 @@ static bool nint_streams(const mfq_nint_desc *d, int M) {
     if (nint_prefill_capable(d)) {
         const bool natural = d->kind != 1;
         const double t64 = (8.0 + 0.85e-6 * static_cast<double>(d->payload_bytes)) * (natural ? 2.0 : 1.0);
-        const double tp = (17.0 + 8.2 * d->neuron_len / 1024.0) * (natural ? 1.25 : 1.0);
+        const double tp = (30.0 + 1.9 * d->neuron_len / 1024.0) * (natural ? 1.25 : 1.0);
         const int m = static_cast<int>(64.0 * tp / t64) / 16 * 16;
         stream_max = m < 64 ? 64 : (m > 512 ? 512 : m);
     }
@@ -358,7 +359,8 @@ static bool nint_streams(const mfq_nint_desc *d, int M) {
 // prefill workspace: x16 [M, Kp] | xscale [M] | group sums
 static size_t prefill_workspace(const mfq_nint_desc *d, int M) {
     const size_t Kp = static_cast<size_t>(ceil_div(d->neuron_len, GBK)) * GBK;
-    return align256(static_cast<size_t>(M) * Kp * 2) + align256(static_cast<size_t>(M) * 4) + nint_prefill_xg_bytes(d, M);
+    return align256(static_cast<size_t>(M) * Kp * 2) + align256(static_cast<size_t>(M) * 4) +
+           align256(nint_prefill_xg_bytes(d, M)) + nint_prefill_split_bytes(d, M);
 }
 
 extern "C" size_t mfq_hip_nint_gemm_workspace_bytes(const mfq_nint_desc *d, int M) {
@@ -387,9 +389,11 @@ extern "C" int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, con
         float *xscale = reinterpret_cast<float *>(p);
         p += align256(static_cast<size_t>(M) * 4);
         uint32_t *xg = reinterpret_cast<uint32_t *>(p);
+        p += align256(nint_prefill_xg_bytes(d, M));
+        float *part = nint_prefill_split_bytes(d, M) ? reinterpret_cast<float *>(p) : nullptr;
         int rc = x_prep_groups(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, d->gs, d->nsteps, xg, st);
         if (rc) return rc;
-        return nint_prefill(d, weight, x16, Kp, xscale, xg, M, y, ldy, st);
+        return nint_prefill(d, weight, x16, Kp, xscale, xg, M, y, ldy, part, st);
     }
     const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
     MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nint_gemm: workspace %zu < %zu bytes",

@@ -315,14 +315,55 @@ bool nint_prefill_capable(const mfq_nint_desc *d) {
 size_t nint_prefill_xg_bytes(const mfq_nint_desc *d, int M) { return static_cast<size_t>(M) * d->nsteps * 64; }
 
 // x16 [M, Kp] fp16 (rows scaled by 1 / xscale[m], zero beyond K), xg = the rows' group sums (x_prep_groups)
+// y[m][n] = sum over the splits of part[z][m][n], in split order
+__global__ __launch_bounds__(256) void prefill_sum_splits_kernel(const float *__restrict__ part, int64_t ystride, int splits,
+                                                                 int M, int N, float *__restrict__ y, int64_t ldy) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;  // float4 index
+    const int n4 = N >> 2;
+    if (i >= static_cast<int64_t>(M) * n4) return;
+    const int m = static_cast<int>(i / n4), c = static_cast<int>(i - static_cast<int64_t>(m) * n4) * 4;
+    float4_t acc = *reinterpret_cast<const float4_t *>(part + static_cast<int64_t>(m) * N + c);
+    for (int z = 1; z < splits; ++z) acc += *reinterpret_cast<const float4_t *>(part + z * ystride + static_cast<int64_t>(m) * N + c);
+    if ((ldy & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0) {
+        *reinterpret_cast<float4_t *>(y + static_cast<int64_t>(m) * ldy + c) = acc;
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) y[static_cast<int64_t>(m) * ldy + c + t] = acc[t];
+    }
+}
+
+// Splits over K of a prefill launch: grids of 64-token tiles that leave CUs idle are cut along K as long as every
+// split keeps at least four steps and the neuron count allows 16-byte partial rows; the partial results go to a
+// workspace and are added in split order (deterministic).  1 = no split.
+int nint_prefill_splits(const mfq_nint_desc *d, int M) {
+    static const int env = [] { const char *e = getenv("MFQ_PREFILL_SPLITS"); return e ? atoi(e) : 0; }();
+    const int64_t blocks = ceil_div(d->n_rowblocks, 16) * ceil_div(M, 64);
+    if (blocks > 128 || d->out % 4) return 1;
+    int splits = static_cast<int>(256 / blocks);
+    if (splits > 4) splits = 4;
+    if (splits > d->nsteps / 4) splits = d->nsteps / 4;
+    if (env > 0) splits = env;
+    return splits < 1 ? 1 : splits;
+}
+size_t nint_prefill_split_bytes(const mfq_nint_desc *d, int M) {
+    const int splits = nint_prefill_splits(d, M);
+    return splits > 1 ? static_cast<size_t>(splits) * M * d->out * 4 : 0;
+}
+
+// part: nint_prefill_split_bytes(d, M) bytes when nint_prefill_splits(d, M) > 1
 int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16, int Kp, const float *xscale,
-                 uint32_t *xg, int M, float *y, int64_t ldy, hipStream_t st) {
+                 uint32_t *xg, int M, float *y, int64_t ldy, float *part, hipStream_t st) {
     const NintK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
+    const int splits = part ? nint_prefill_splits(d, M) : 1;
+    const int spz = static_cast<int>(ceil_div(k.nsteps, splits));
+    const int64_t ystride = static_cast<int64_t>(M) * k.out;
+    float *yk = splits > 1 ? part : y;
+    const int64_t ldk = splits > 1 ? k.out : ldy;
 #define MFQ_PREFILL_CFG(UNIT, B, G, MT, NB, PF, XD)                                                                 \
     {                                                                                                          \
         const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, 8 * NB)),                                \
-                        static_cast<unsigned>(ceil_div(M, MT * 16)));                                          \
+                        static_cast<unsigned>(ceil_div(M, MT * 16)), static_cast<unsigned>(splits));           \
         const size_t lds = prefill_lds_bytes(MT * 16, G);                                                      \
         auto kern = nint_prefill_kernel<UNIT<B, G>, MT, NB, 1, 8, PF, XD>;                                     \
         if (lds > 65536) {                                                                                     \
@@ -330,7 +371,12 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
                                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
             MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nint_prefill: %s", hipGetErrorString(e));            \
         }                                                                                                      \
-        hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, k, w, x16, Kp, xscale, xg, M, y, ldy);              \
+        hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, k, w, x16, Kp, xscale, xg, M, yk, ldk, spz, ystride); \
+        if (splits > 1) {                                                                                      \
+            const int64_t n4 = static_cast<int64_t>(M) * (k.out / 4);                                          \
+            hipLaunchKernelGGL(prefill_sum_splits_kernel, dim3(static_cast<unsigned>(ceil_div(n4, 256))), dim3(256), 0, st, \
+                               part, ystride, splits, M, k.out, y, ldy);                                       \
+        }                                                                                                      \
         return check_launch("nint_prefill");                                                                   \
     }
     // Block = 8 waves side by side on 256 neurons (two row-blocks per wave), each with four unit buffers per row-block

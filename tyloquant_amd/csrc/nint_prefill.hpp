@@ -46,7 +46,9 @@ template <class U, int MT, int NB, int WM, int NW, class Rows, int PF = 2, int X
 __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t *__restrict__ w, int rb_base, int rb_end,
                                                   int rb_col0, int ncols, const uint16_t *__restrict__ x16, int Kp,
                                                   const float *__restrict__ xscale, const uint32_t *__restrict__ xg,
-                                                  const Rows &rows, float *__restrict__ y, int64_t ldy, uint16_t *xt) {
+                                                  const Rows &rows, float *__restrict__ y, int64_t ldy, uint16_t *xt,
+                                                  int s_begin = 0, int s_end = -1) {
+    if (s_end < 0) s_end = k.nsteps;  // steps [s_begin, s_end) of K: a block of a split over K leaves a partial sum
     constexpr int D = U::D, GS = U::GROUP, NM = U::NPAIR / 4, BITS = U::CBITS;
     constexpr int NCLS = BITS == 0 ? 1 : (BITS == 3 ? 3 : 2);
     constexpr int NT = 64 * NW;                // threads
@@ -122,27 +124,27 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
         const int s = it >> 2, j = it & 3;
 #pragma unroll
         for (int b = 0; b < NB; ++b)
-            load_unit_win<D, 0>(win, b < nrb && s < k.nsteps ? b * rbb + s * sb + (j * 64 + lane) * (D * 4) : kNoStep, qq[b]);
+            load_unit_win<D, 0>(win, b < nrb && s < s_end ? b * rbb + s * sb + (j * 64 + lane) * (D * 4) : kNoStep, qq[b]);
     };
     auto sload = [&](int s, uint32_t (&tt)[NB], u32x2_t (&ss)[NB]) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            const uint32_t off = b < nrb && s < k.nsteps ? b * rbb + s * sb + 1024 * D : kNoStep;
+            const uint32_t off = b < nrb && s < s_end ? b * rbb + s * sb + 1024 * D : kNoStep;
             tt[b] = 0;
             if constexpr (U::TAIL) tt[b] = __builtin_amdgcn_raw_buffer_load_b32(win, off + lane * 4, 0, 0);
             ss[b] = __builtin_amdgcn_raw_buffer_load_b64(win, off + (U::TAIL ? 256 : 0) + lane * 8, 0, 0);
         }
     };
 
-    xload(0, xr[0]);
+    xload(4 * s_begin, xr[0]);
 #pragma unroll
-    for (int i = 0; i < PF - 1; ++i) wload(i, qr[i]);
-    sload(0, tails, sc);
+    for (int i = 0; i < PF - 1; ++i) wload(4 * s_begin + i, qr[i]);
+    sload(s_begin, tails, sc);
     xstore(0, xr[0]);
 #pragma unroll
-    for (int i = 1; i < XD; ++i) xload(i, xr[i]);
+    for (int i = 1; i < XD; ++i) xload(4 * s_begin + i, xr[i]);
     __syncthreads();
-    for (int s = 0; s < k.nsteps; ++s) {
+    for (int s = s_begin; s < s_end; ++s) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int it = 4 * s + j;
@@ -221,7 +223,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
     constexpr int SC = kMinSteps, XGROW = SC * 16 + 4;  // dwords per tile row in LDS, padded against bank conflicts
     constexpr int XG_PER_THREAD = (BM * SC * 4 + NT - 1) / NT;
     uint32_t *xgl = reinterpret_cast<uint32_t *>(xt);
-    for (int c0 = 0; c0 < k.nsteps; c0 += SC) {
+    for (int c0 = s_begin; c0 < s_end; c0 += SC) {
         __syncthreads();  // the last reads of the activation tile / of the previous chunk are done
         u32x4_t gx[XG_PER_THREAD];
 #pragma unroll
@@ -237,7 +239,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const int s = c0 + t;
-                const uint32_t off = b < nrb && s < k.nsteps ? b * rbb + s * sb + 1024 * D + (U::TAIL ? 256 : 0) : kNoStep;
+                const uint32_t off = b < nrb && s < s_end ? b * rbb + s * sb + 1024 * D + (U::TAIL ? 256 : 0) : kNoStep;
                 scs[t][b] = __builtin_amdgcn_raw_buffer_load_b64(win, off + lane * 8, 0, 0);
             }
 #pragma unroll
@@ -249,7 +251,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
         __syncthreads();
 #pragma unroll
         for (int t = 0; t < SC; ++t) {
-            if (c0 + t >= k.nsteps) break;
+            if (c0 + t >= s_end) break;
             u32x4_t ax[MT];
 #pragma unroll
             for (int a = 0; a < MT; ++a)
@@ -283,17 +285,21 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
     }
 }
 
-// Dense wrapper: block (neuron tile, token tile).
+// Dense wrapper: block (neuron tile, token tile, K split).  Split z handles the steps [z * spz, (z + 1) * spz) and
+// writes its partial result to y + z * ystride (one split: y itself).
 template <class U, int MT, int NB, int WM, int NW, int PF = 2, int XD = (PF == 4 ? 4 : 1)>
 __global__ __launch_bounds__(64 * NW) void nint_prefill_kernel(NintK k, const uint8_t *__restrict__ w,
                                                                const uint16_t *__restrict__ x16, int Kp,
                                                                const float *__restrict__ xscale,
                                                                const uint32_t *__restrict__ xg, int M,
-                                                               float *__restrict__ y, int64_t ldy) {
+                                                               float *__restrict__ y, int64_t ldy, int spz,
+                                                               int64_t ystride) {
     extern __shared__ __attribute__((aligned(16))) uint16_t xt[];
     const DenseRows rows{static_cast<int>(blockIdx.y) * WM * MT * 16, M};
+    const int z = blockIdx.z;
     nint_prefill_body<U, MT, NB, WM, NW, DenseRows, PF, XD>(k, w, static_cast<int>(blockIdx.x) * (NW / WM) * NB, k.n_rowblocks, 0,
-                                                        k.out, x16, Kp, xscale, xg, rows, y, ldy, xt);
+                                                            k.out, x16, Kp, xscale, xg, rows, y + z * ystride, ldy, xt,
+                                                            z * spz, min(k.nsteps, (z + 1) * spz));
 }
 
 }  // namespace mfq
