@@ -572,7 +572,7 @@ __global__ __launch_bounds__(512) void moe_prefill_kernel(MoePools P, const int3
                                                                      out_per_expert, x16, Kp, xscale, P.xg[pool], rows, \
                                                                      out, ldo, xt);                                  \
         else                                                                                                         \
-            nint_prefill_body<UNIT<B, G>, 4, 4, 1, 8>(k, P.w[pool], rb_base, rb_first + rbe, rb_first, out_per_expert, \
+            nint_prefill_body<UNIT<B, G>, 4, 4, 1, 8, MappedRows, 2, 2>(k, P.w[pool], rb_base, rb_first + rbe, rb_first, out_per_expert, \
                                                       x16, Kp, xscale, P.xg[pool], rows, out, ldo, xt);              \
     }
     if (k.kind == 1) {
