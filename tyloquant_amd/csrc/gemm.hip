@@ -22,14 +22,21 @@ int fail(int code, const char *fmt, ...) {
     return code;
 }
 
+// group-sum tables one activation prep launch leaves: one per distinct groupsize of the tensors that will read x16
+struct XGroups {
+    int n;
+    int gs[4], nsteps[4];
+    uint32_t *xg[4];
+};
+
 // ---- activation prep: x16[m, k] = fp16(x[m, k] * 2^-f_m), xscale[m] = 2^f_m ---------------
 // With xg != null the block also leaves the row's group sums for the NINT prefill kernel:
 // xg[((m * nsteps + s) * 4 + kb) * 4 + {0,1,2,3}] = fp16 pairs (Xhi_j0, Xhi_j1), (Xhi_j2, Xhi_j3), (Xlo_j0, Xlo_j1),
 // (Xlo_j2, Xlo_j3), X_j = sum of x16[m] over group 16 s + 4 j + kb (gs values), split into two fp16 halves.
 template <int XF16>
 __global__ __launch_bounds__(256) void x_prep_kernel(const uint16_t *__restrict__ x, int64_t ldx, int K, int Kp,
-                                                     uint16_t *__restrict__ x16, float *__restrict__ xscale, int gs,
-                                                     int nsteps, uint32_t *__restrict__ xg) {
+                                                     uint16_t *__restrict__ x16, float *__restrict__ xscale,
+                                                     XGroups grp) {
     __shared__ float red[4];
     __shared__ float gsum[256];
     const int m = blockIdx.x, tid = threadIdx.x;
@@ -49,8 +56,10 @@ __global__ __launch_bounds__(256) void x_prep_kernel(const uint16_t *__restrict_
     if (tid == 0) xscale[m] = ldexpf(1.f, e - 9);
     uint16_t *o16 = x16 + static_cast<int64_t>(m) * Kp;
     for (int k = tid; k < Kp; k += 256) o16[k] = k < K ? f32_to_f16_rne(x_to_f32<XF16>(xr[k]) * inv) : uint16_t(0);
-    if (xg == nullptr) return;
     // group sums of the fp16 values just written (recomputed from x: the same roundings), 256 groups at a time
+    for (int gi = 0; gi < grp.n; ++gi) {
+    const int gs = grp.gs[gi], nsteps = grp.nsteps[gi];
+    uint32_t *xg = grp.xg[gi];
     for (int g0 = 0; g0 < nsteps * 16; g0 += 256) {
         const int g = g0 + tid;
         float acc = 0.f;
@@ -79,14 +88,15 @@ __global__ __launch_bounds__(256) void x_prep_kernel(const uint16_t *__restrict_
             for (int t = 0; t < 4; ++t) o[t] = out[t];
         }
     }
+    }
 }
 
 // The same for 16-byte aligned rows with K % 8 == 0 and Kp * 2 bytes of LDS: 8 values per load and store, the row
 // read once (twice beyond 8192 values), the group sums taken from the fp16 row kept in LDS.  Bit-identical results.
 template <int XF16>
 __global__ __launch_bounds__(256) void x_prep_vec_kernel(const uint16_t *__restrict__ x, int64_t ldx, int K, int Kp,
-                                                         uint16_t *__restrict__ x16, float *__restrict__ xscale, int gs,
-                                                         int nsteps, uint32_t *__restrict__ xg) {
+                                                         uint16_t *__restrict__ x16, float *__restrict__ xscale,
+                                                         XGroups grp) {
     extern __shared__ __attribute__((aligned(16))) uint16_t rowh[];  // [Kp] halves
     __shared__ float red[4];
     __shared__ float gsum[256];
@@ -144,8 +154,11 @@ __global__ __launch_bounds__(256) void x_prep_vec_kernel(const uint16_t *__restr
         o16[c] = u32x4_t{0u, 0u, 0u, 0u};
         rowv[c] = u32x4_t{0u, 0u, 0u, 0u};
     }
-    if (xg == nullptr) return;
+    if (grp.n == 0) return;
     __syncthreads();
+    for (int gi = 0; gi < grp.n; ++gi) {
+    const int gs = grp.gs[gi], nsteps = grp.nsteps[gi];
+    uint32_t *xg = grp.xg[gi];
     for (int g0 = 0; g0 < nsteps * 16; g0 += 256) {
         const int g = g0 + tid;
         float acc = 0.f;
@@ -171,6 +184,7 @@ __global__ __launch_bounds__(256) void x_prep_vec_kernel(const uint16_t *__restr
             }
             *reinterpret_cast<u32x4_t *>(xg + ((static_cast<int64_t>(m) * nsteps + g0 / 16 + sl) * 4 + kb) * 4) = out;
         }
+    }
     }
 }
 
@@ -268,27 +282,39 @@ int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, i
     return check_launch("gemm_f16_nt");
 }
 
-int x_prep_groups(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, int gs,
-                  int nsteps, uint32_t *xg, hipStream_t st) {
+int x_prep_multi(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, int n_groups,
+                 const int *gs, const int *nsteps, uint32_t *const *xg, hipStream_t st) {
+    MFQ_REQUIRE(n_groups >= 0 && n_groups <= 4, MFQ_ERR_UNSUPPORTED, "x_prep: %d group-sum tables (max 4)", n_groups);
+    XGroups grp;
+    grp.n = n_groups;
+    for (int i = 0; i < 4; ++i) {
+        grp.gs[i] = i < n_groups ? gs[i] : 0;
+        grp.nsteps[i] = i < n_groups ? nsteps[i] : 0;
+        grp.xg[i] = i < n_groups ? xg[i] : nullptr;
+    }
     const bool vec = K % 8 == 0 && ldx % 8 == 0 && Kp % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
                      (reinterpret_cast<uintptr_t>(x16) & 15) == 0 && Kp <= 28 * 1024;
     if (vec) {
         const size_t lds = static_cast<size_t>(Kp) * 2;
         if (x_dtype == MFQ_X_F16)
             hipLaunchKernelGGL((x_prep_vec_kernel<1>), dim3(M), dim3(256), lds, st, static_cast<const uint16_t *>(x), ldx, K,
-                               Kp, static_cast<uint16_t *>(x16), xscale, gs, nsteps, xg);
+                               Kp, static_cast<uint16_t *>(x16), xscale, grp);
         else
             hipLaunchKernelGGL((x_prep_vec_kernel<0>), dim3(M), dim3(256), lds, st, static_cast<const uint16_t *>(x), ldx, K,
-                               Kp, static_cast<uint16_t *>(x16), xscale, gs, nsteps, xg);
+                               Kp, static_cast<uint16_t *>(x16), xscale, grp);
         return check_launch("x_prep");
     }
     if (x_dtype == MFQ_X_F16)
         hipLaunchKernelGGL((x_prep_kernel<1>), dim3(M), dim3(256), 0, st, static_cast<const uint16_t *>(x), ldx, K, Kp,
-                           static_cast<uint16_t *>(x16), xscale, gs, nsteps, xg);
+                           static_cast<uint16_t *>(x16), xscale, grp);
     else
         hipLaunchKernelGGL((x_prep_kernel<0>), dim3(M), dim3(256), 0, st, static_cast<const uint16_t *>(x), ldx, K, Kp,
-                           static_cast<uint16_t *>(x16), xscale, gs, nsteps, xg);
+                           static_cast<uint16_t *>(x16), xscale, grp);
     return check_launch("x_prep");
+}
+int x_prep_groups(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, int gs,
+                  int nsteps, uint32_t *xg, hipStream_t st) {
+    return x_prep_multi(x, x_dtype, ldx, M, K, Kp, x16, xscale, xg ? 1 : 0, &gs, &nsteps, &xg, st);
 }
 int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, hipStream_t st) {
     return x_prep_groups(x, x_dtype, ldx, M, K, Kp, x16, xscale, 0, 0, nullptr, st);

@@ -675,8 +675,8 @@ extern "C" int mfq_hip_moe_route_map(const int32_t *ids, int n_pairs, int E, int
 extern "C" int mfq_hip_moe_tile_m(void) { return kMoeTileM; }
 
 namespace mfq {
-int x_prep_groups(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, int gs,
-                  int nsteps, uint32_t *xg, hipStream_t st);
+int x_prep_multi(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, int n_groups,
+                 const int *gs, const int *nsteps, uint32_t *const *xg, hipStream_t st);
 }
 
 // prefill workspace: x16 [rows, Kp] | xscale [rows] | one group-sum table per distinct groupsize of the paired cohorts
@@ -834,7 +834,9 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
         p += moe_align256(static_cast<size_t>(x_rows) * Kp * 2);
         float *xscale = reinterpret_cast<float *>(p);
         p += moe_align256(static_cast<size_t>(x_rows) * 4);
-        int max_gs = 16;
+        // one activation prep launch leaves a group-sum table per distinct groupsize (at most four per launch)
+        int max_gs = 16, ng = 0, g_gs[4], g_steps[4];
+        uint32_t *g_xg[4];
         for (int i = 0; i < n_pools; ++i) {
             P.prefill[i] = 1;
             for (int j = 0; j < i; ++j)
@@ -842,11 +844,19 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
             if (!P.xg[i]) {
                 uint32_t *xg = reinterpret_cast<uint32_t *>(p);
                 p += moe_align256(static_cast<size_t>(x_rows) * P.k[i].nsteps * 64);
-                const int rc = x_prep_groups(x, x_dtype, ldx, x_rows, K, Kp, x16, xscale, P.k[i].gs, P.k[i].nsteps, xg, st);
-                if (rc) return rc;
+                g_gs[ng] = P.k[i].gs; g_steps[ng] = P.k[i].nsteps; g_xg[ng] = xg;
+                if (++ng == 4) {
+                    const int rc = x_prep_multi(x, x_dtype, ldx, x_rows, K, Kp, x16, xscale, ng, g_gs, g_steps, g_xg, st);
+                    if (rc) return rc;
+                    ng = 0;
+                }
                 P.xg[i] = xg;
             }
             if (P.k[i].gs > max_gs) max_gs = P.k[i].gs;
+        }
+        if (ng) {
+            const int rc = x_prep_multi(x, x_dtype, ldx, x_rows, K, Kp, x16, xscale, ng, g_gs, g_steps, g_xg, st);
+            if (rc) return rc;
         }
         const size_t plds = 512 + prefill_lds_bytes(64, max_gs);
         const dim3 pgrid(static_cast<unsigned>(tiles), static_cast<unsigned>(ceil_div(rbe, 32)));
