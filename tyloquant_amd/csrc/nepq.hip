@@ -374,7 +374,7 @@ static int nepq_launch_mfma(const NepqK &k, const uint8_t *w, int row0, int nrow
 template <int XF16>
 static int nepq_mfma_any(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
                          float *y, int64_t ldy, hipStream_t st) {
-    const int64_t wpb = k.nsteps < 8 ? k.nsteps : 8;  // waves of a block
+    const int64_t wpb = (k.nsteps < 8 ? k.nsteps : 8) * ceil_div(M, 16);  // waves of a block x 16-row tiles
     if (ceil_div(ceil_div(nrows, 16), 4) * wpb >= 1536) return nepq_launch_mfma<XF16, 4>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
     return nepq_launch_mfma<XF16, 1>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
 }

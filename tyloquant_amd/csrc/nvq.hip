@@ -12,7 +12,7 @@
 // expands a sign mask (with its parity bit) into XOR masks, and the scale LUT all stay in LDS.
 #include "common.hpp"
 #include "gemv_common.hpp"
-#include "nint_mfma.hpp"
+#include "nint_prefill.hpp"
 
 namespace mfq {
 
@@ -380,6 +380,219 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
     mfma_store_dense<NB>(red, rb0, m0, M, k.out, y, ldy);
 }
 
+// ---- prefill: block-tiled MFMA GEMM, weight fragments built from the codebooks in LDS ----------------------
+// Block = 8 waves side by side on 8 * NB row-blocks, wave tile MT * 16 tokens x NB * 16 neurons.  Activations as in
+// the NINT prefill kernel: fp16 rows scaled per token (x_prep), the 96 k-values of a sub-step (unit j of a step) staged
+// in LDS, two buffers, XD tiles in flight in registers.  Weights: PF unit buffers per row-block (PF - 1 sub-steps in
+// flight), each fragment built as in nvq_mfma_kernel -- two codebook vectors, sign bits XOR-ed in, one packed fp16
+// multiply by the state's scale -- and shared by the MT token tiles of the wave.
+// LDS map (dwords): [codebook pairs: banks*entries*2][sign xor table: 512][lut pairs: 16][bank offset: 16][x tiles]
+template <int MT, int NB, int PF, int XD>
+__global__ __launch_bounds__(512) void nvq_prefill_kernel(NvqK k, const uint8_t *__restrict__ w,
+                                                          const uint16_t *__restrict__ x16, int Kp,
+                                                          const float *__restrict__ xscale, int M,
+                                                          float *__restrict__ y, int64_t ldy) {
+    static_assert((PF == 2 || PF == 4) && (XD == 1 || XD == 2 || XD == 4), "the sub-step loop is unrolled four times");
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    constexpr int GS = 24, NM = 3, NT = 512, BM = MT * 16, EL = 8;
+    constexpr int ROW = 4 * GS + 8;  // LDS row stride in halves
+    constexpr int CPG = GS / EL, CHUNKS = 4 * CPG;
+    constexpr int PER_THREAD = (BM * CHUNKS + NT - 1) / NT;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, kb = lane >> 4;
+    const int ncb = k.banks * k.entries;
+    uint32_t *cbp = lds;
+    uint32_t *sgx = cbp + 2 * ncb;
+    uint32_t *luth = sgx + 512;
+    uint32_t *bankoff = luth + 16;
+    uint16_t *xt = reinterpret_cast<uint16_t *>(bankoff + 16);
+    {
+        const float *lut = reinterpret_cast<const float *>(w + k.tables_off);
+        const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+        const uint32_t *cb = bfs + 16;  // 4 int8 magnitudes per entry
+        for (int i = tid; i < ncb; i += NT) {
+            const uint32_t e = cb[i];
+            uint32_t h[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) h[t] = f32_to_f16_rne(static_cast<float>((e >> (8 * t)) & 0xffu));
+            cbp[2 * i] = h[0] | (h[1] << 16);
+            cbp[2 * i + 1] = h[2] | (h[3] << 16);
+        }
+        for (int i = tid; i < 128; i += NT) {
+            const uint32_t m8 = parity8(i);
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+                sgx[4 * i + p] = (((m8 >> (2 * p)) & 1u) << 15) | (((m8 >> (2 * p + 1)) & 1u) << 31);
+        }
+        if (tid < 16) {
+            const uint32_t h = f32_to_f16_rne(lut[tid]);
+            luth[tid] = h | (h << 16);
+            bankoff[tid] = bfs[tid] * k.entries * 2;
+        }
+    }
+    const DenseRows rows{static_cast<int>(blockIdx.y) * BM, M};
+    const int rb0 = (static_cast<int>(blockIdx.x) * 8 + wave) * NB;
+    const int nrb = max(0, min(NB, k.n_rowblocks - rb0));
+    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
+    const __amdgpu_buffer_rsrc_t win =
+        wave_window(w + static_cast<int64_t>(min(rb0, k.n_rowblocks - 1)) * k.rowblock_bytes, nrb * rbb);
+    float4_t acc[MT][NB];
+#pragma unroll
+    for (int a = 0; a < MT; ++a)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const uint16_t *xsrc[PER_THREAD];
+    int xk[PER_THREAD];
+#pragma unroll
+    for (int p = 0; p < PER_THREAD; ++p) {
+        const int c = min(tid + NT * p, BM * CHUNKS - 1);
+        const int row = c / CHUNKS;
+        xsrc[p] = x16 + static_cast<int64_t>(rows.src(row)) * Kp;
+        xk[p] = EL * (c - row * CHUNKS);
+    }
+    u32x4_t xr[XD][PER_THREAD];
+    auto xload = [&](int it, u32x4_t (&xq)[PER_THREAD]) {
+        const int k0 = it * 4 * GS;
+#pragma unroll
+        for (int p = 0; p < PER_THREAD; ++p) {
+            const int kk = k0 + xk[p];
+            u32x4_t v = *reinterpret_cast<const u32x4_t *>(xsrc[p] + min(kk, Kp - EL));
+            if (kk >= Kp) v = u32x4_t{0u, 0u, 0u, 0u};
+            xq[p] = v;
+        }
+    };
+    auto xstore = [&](int buf, const u32x4_t (&xq)[PER_THREAD]) {
+#pragma unroll
+        for (int p = 0; p < PER_THREAD; ++p) {
+            const int c = tid + NT * p;
+            const int row = c / CHUNKS, ch = c - row * CHUNKS;
+            if (c < BM * CHUNKS) *reinterpret_cast<u32x4_t *>(xt + buf * (BM * ROW) + row * ROW + EL * ch) = xq[p];
+        }
+    };
+    u32x2_t qr[PF][NB], hh[NB], hhn[NB];
+    auto wload = [&](int it, u32x2_t (&qq)[NB]) {
+        const int s = it >> 2, j = it & 3;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            qq[b] = __builtin_amdgcn_raw_buffer_load_b64(
+                win, b < nrb && s < k.nsteps ? b * rbb + s * sb + (j * 64 + lane) * 8 : kNoStep, 0, 0);
+    };
+    auto hload = [&](int s, u32x2_t (&h)[NB]) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            h[b] = __builtin_amdgcn_raw_buffer_load_b64(win, b < nrb && s < k.nsteps ? b * rbb + s * sb + 2048 + lane * 8 : kNoStep,
+                                                        0, 0);
+    };
+    xload(0, xr[0]);
+#pragma unroll
+    for (int i = 0; i < PF - 1; ++i) wload(i, qr[i]);
+    hload(0, hh);
+    xstore(0, xr[0]);
+#pragma unroll
+    for (int i = 1; i < XD; ++i) xload(i, xr[i]);
+    __syncthreads();  // tables and the first tile
+
+    const uint32_t ib = static_cast<uint32_t>(k.ib), im = (1u << ib) - 1u;
+    for (int s = 0; s < k.nsteps; ++s) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int it = 4 * s + j;
+            xload(it + XD, xr[j % XD]);
+            wload(it + PF - 1, qr[(j + PF - 1) % PF]);
+            if (j == 0) hload(s + 1, hhn);
+            const uint32_t *bank[NB];
+            half2_t sc[NB];
+            uint32_t mk[NB][3], ix[NB][6];
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const uint32_t d0 = qr[j % PF][b].x, d1 = qr[j % PF][b].y;
+                const uint32_t h = ((j < 2 ? hh[b].x : hh[b].y) >> (16 * (j & 1))) & 0xffffu;
+                const uint32_t state = (d1 >> 27) & 15u;
+                bank[b] = cbp + bankoff[state];
+                sc[b] = __builtin_bit_cast(half2_t, luth[state]);
+                mk[b][0] = h & 127u; mk[b][1] = (h >> 7) & 127u; mk[b][2] = ((d0 >> 27) & 31u) | ((h >> 14) << 5);
+                ix[b][0] = d0 & im; ix[b][1] = (d0 >> ib) & im; ix[b][2] = (d0 >> (2 * ib)) & im;
+                ix[b][3] = d1 & im; ix[b][4] = (d1 >> ib) & im; ix[b][5] = (d1 >> (2 * ib)) & im;
+            }
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                u32x4_t af[MT];
+#pragma unroll
+                for (int a = 0; a < MT; ++a)
+                    af[a] = *reinterpret_cast<const u32x4_t *>(xt + (j & 1) * (BM * ROW) + (a * 16 + r) * ROW + kb * GS + 8 * m);
+                u32x4_t bf[NB];
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    const u32x4_t sx = *reinterpret_cast<const u32x4_t *>(sgx + 4 * mk[b][m]);
+                    const u32x2_t c0 = *reinterpret_cast<const u32x2_t *>(bank[b] + 2 * ix[b][2 * m]);
+                    const u32x2_t c1 = *reinterpret_cast<const u32x2_t *>(bank[b] + 2 * ix[b][2 * m + 1]);
+                    const uint32_t wv[4] = {c0.x ^ sx.x, c0.y ^ sx.y, c1.x ^ sx.z, c1.y ^ sx.w};
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        bf[b][t] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, wv[t]) * sc[b]);
+                }
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+#pragma unroll
+                    for (int a = 0; a < MT; ++a) acc[a][b] = mfma16(af[a], bf[b], acc[a][b]);
+            }
+            xstore((j + 1) & 1, xr[(j + 1) % XD]);
+            if (j == 3) {
+#pragma unroll
+                for (int b = 0; b < NB; ++b) hh[b] = hhn[b];
+            }
+            __syncthreads();
+        }
+    }
+    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
+    float an[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) an[b] = anchors[min(rb0 + b, k.n_rowblocks - 1) * 16 + r];
+#pragma unroll
+    for (int a = 0; a < MT; ++a) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int ti = a * 16 + 4 * kb + v;
+            const int m = rows.dst(ti);
+            if (m < 0) continue;
+            const float xs = xscale[m];
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const int col = (rb0 + b) * 16 + r;
+                if (rb0 + b < k.n_rowblocks && col < k.out) y[static_cast<int64_t>(m) * ldy + col] = xs * (an[b] * acc[a][b][v]);
+            }
+        }
+    }
+}
+
+static size_t nvq_prefill_lds(const NvqK &k, int bm) {
+    return (static_cast<size_t>(k.banks) * k.entries * 2 + 512 + 32) * 4 + static_cast<size_t>(2 * bm) * (4 * 24 + 8) * 2;
+}
+
+// x16 [M, Kp] fp16 rows scaled by 1 / xscale[m], zero beyond K (x_prep)
+static int nvq_prefill(const NvqK &k, const uint8_t *w, const uint16_t *x16, int Kp, const float *xscale, int M, float *y,
+                       int64_t ldy, hipStream_t st) {
+#define MFQ_NVQ_PREFILL(MT, XD)                                                                                       \
+    {                                                                                                                  \
+        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, 16)), static_cast<unsigned>(ceil_div(M, MT * 16))); \
+        const size_t lds = nvq_prefill_lds(k, MT * 16);                                                                \
+        auto kern = nvq_prefill_kernel<MT, 2, 4, XD>;                                                                  \
+        if (lds > 65536) {                                                                                             \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                   \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));     \
+            MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nvq_prefill: %s", hipGetErrorString(e));                     \
+        }                                                                                                              \
+        hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, k, w, x16, Kp, xscale, M, y, ldy);                          \
+        return check_launch("nvq_prefill");                                                                            \
+    }
+    // 64-token tiles while they give at most one block per CU (four activation tiles in flight), 128-token tiles beyond
+    if (ceil_div(k.n_rowblocks, 16) * ceil_div(M, 64) <= 256) MFQ_NVQ_PREFILL(4, 4)
+    MFQ_NVQ_PREFILL(8, 2)
+#undef MFQ_NVQ_PREFILL
+}
+
 static bool nvq_stream_capable(const NvqK &k) {
     return k.neuron_len >= 8 && k.neuron_len % 8 == 0 && 4 * k.rowblock_bytes < (1ll << 31);
 }
@@ -401,7 +614,7 @@ static int nvq_launch_mfma(const NvqK &k, const uint8_t *w, const uint16_t *x, i
 template <int XF16>
 static int nvq_mfma_any(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                         hipStream_t st) {
-    const int64_t wpb = k.nsteps < 8 ? k.nsteps : 8;  // waves of a block
+    const int64_t wpb = (k.nsteps < 8 ? k.nsteps : 8) * ceil_div(M, 16);  // waves of a block x 16-row tiles
     if (ceil_div(k.n_rowblocks, 4) * wpb >= 1536) return nvq_launch_mfma<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
     if (ceil_div(k.n_rowblocks, 2) * wpb >= 1536) return nvq_launch_mfma<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
     return nvq_launch_mfma<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
@@ -545,12 +758,33 @@ extern "C" int mfq_hip_nvq_gemv(const mfq_nvq_desc *d, const void *weight, const
 // The reference keeps the D4 family on its GEMV up to M = 13; tensors the matrix-core streaming kernel
 // takes stay on it up to kNvqStreamMaxM rows.
 static constexpr int kNvqGemvMaxM = 13, kNvqStreamMaxM = 256;
-static bool nvq_streams(const mfq_nvq_desc *d, int M) {
-    return M <= kNvqGemvMaxM || (M <= kNvqStreamMaxM && nvq_stream_capable(to_k(d)));
+static bool nvq_prefill_capable(const NvqK &k) {
+    return nvq_stream_capable(k) && (static_cast<size_t>(k.banks) * k.entries * 2 + 544) * 4 <= 16384 &&
+           (static_cast<size_t>(k.banks) * k.entries) % 2 == 0 && 2 * k.rowblock_bytes < (1ll << 31);
 }
+// Rows up to which re-streaming the weights (16 rows per pass) beats the prefill kernel, from a two-term model fitted
+// to measurements (17408x5120 and 5120x17408): 64 rows of streaming cost about 6 us + 1.7 us per MB of payload, the
+// prefill kernel a flat 20 us + 13.2 us per 1024 of K up to a few hundred rows (a block walks all of K).
+static int nvq_stream_max(const mfq_nvq_desc *d, const NvqK &k) {
+    static const int env = [] { const char *e = getenv("MFQ_NVQ_STREAM_MAX_M"); return e ? atoi(e) : 0; }();
+    if (env > 0) return env;
+    if (!nvq_prefill_capable(k)) return kNvqStreamMaxM;
+    const double t64 = 6.0 + 1.7e-6 * static_cast<double>(d->payload_bytes);
+    const double tp = 20.0 + 13.2 * k.neuron_len / 1024.0;
+    const int m = static_cast<int>(64.0 * tp / t64) / 16 * 16;
+    return m < 32 ? 32 : (m > 512 ? 512 : m);
+}
+static bool nvq_streams(const mfq_nvq_desc *d, int M) {
+    const NvqK k = to_k(d);
+    return M <= kNvqGemvMaxM || (M <= nvq_stream_max(d, k) && nvq_stream_capable(k));
+}
+static size_t nvq_align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+static int nvq_kp(int K) { return static_cast<int>(ceil_div(K, 32)) * 32; }
 
 extern "C" size_t mfq_hip_nvq_gemm_workspace_bytes(const mfq_nvq_desc *d, int M) {
     if (!d || nvq_streams(d, M)) return 0;
+    if (nvq_prefill_capable(to_k(d)))  // x16 [M, Kp] | xscale [M]
+        return nvq_align256(static_cast<size_t>(M) * nvq_kp(d->neuron_len) * 2) + nvq_align256(static_cast<size_t>(M) * 4);
     return dequant_gemm_workspace(d->out, d->neuron_len, M);
 }
 
@@ -562,6 +796,18 @@ extern "C" int mfq_hip_nvq_gemm(const mfq_nvq_desc *d, const void *weight, const
     MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nvq_gemm: ldx/ldy smaller than the tensor");
     hipStream_t st = as_stream(stream);
     if (nvq_streams(d, M)) return nvq_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, st);
+    if (nvq_prefill_capable(to_k(d))) {
+        const NvqK k = to_k(d);
+        const int Kp = nvq_kp(k.neuron_len);
+        const size_t need = mfq_hip_nvq_gemm_workspace_bytes(d, M);
+        MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nvq_gemm: workspace %zu < %zu bytes",
+                    workspace_bytes, need);
+        uint16_t *x16 = static_cast<uint16_t *>(workspace);
+        float *xscale = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + nvq_align256(static_cast<size_t>(M) * Kp * 2));
+        const int rc = x_prep(x, x_dtype, ldx, M, k.neuron_len, Kp, x16, xscale, st);
+        if (rc) return rc;
+        return nvq_prefill(k, static_cast<const uint8_t *>(weight), x16, Kp, xscale, M, y, ldy, st);
+    }
     const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
     MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nvq_gemm: workspace %zu < %zu bytes",
                 workspace_bytes, need);
