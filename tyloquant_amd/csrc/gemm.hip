@@ -376,7 +376,7 @@ static bool nint_streams(const mfq_nint_desc *d, int M) {
         const double t64 = (8.0 + 0.85e-6 * static_cast<double>(d->payload_bytes)) * (natural ? 2.0 : 1.0);
         const double tp = (30.0 + 1.9 * d->neuron_len / 1024.0) * (natural ? 1.25 : 1.0);
         const int m = static_cast<int>(64.0 * tp / t64) / 16 * 16;
-        stream_max = m < 64 ? 64 : (m > 512 ? 512 : m);
+        stream_max = m < 32 ? 32 : (m > 512 ? 512 : m);
     }
     if (env_max > 0) stream_max = env_max;
     return M <= kGemvMaxM || (M <= stream_max && nint_stream_capable(d));

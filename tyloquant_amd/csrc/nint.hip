@@ -332,18 +332,20 @@ __global__ __launch_bounds__(256) void prefill_sum_splits_kernel(const float *__
     }
 }
 
-// Splits over K of a prefill launch: grids of 64-token tiles that leave CUs idle are cut along K as long as every
-// split keeps at least four steps and the neuron count allows 16-byte partial rows; the partial results go to a
+// Splits over K of a prefill launch: grids of 64-token tiles that leave CUs idle are cut along K (up to eight
+// splits) as long as every split keeps at least two steps and the neuron count allows 16-byte partial rows; the partial results go to a
 // workspace and are added in split order (deterministic).  1 = no split.
 int nint_prefill_splits(const mfq_nint_desc *d, int M) {
     static const int env = [] { const char *e = getenv("MFQ_PREFILL_SPLITS"); return e ? atoi(e) : 0; }();
     const int64_t blocks = ceil_div(d->n_rowblocks, 16) * ceil_div(M, 64);
     if (blocks > 128 || d->out % 4) return 1;
     int splits = static_cast<int>(256 / blocks);
-    if (splits > 4) splits = 4;
-    if (splits > d->nsteps / 4) splits = d->nsteps / 4;
+    if (splits > 8) splits = 8;
+    if (splits > d->nsteps / 2) splits = d->nsteps / 2;
     if (env > 0) splits = env;
-    return splits < 1 ? 1 : splits;
+    if (splits <= 1) return 1;
+    const int spz = static_cast<int>(ceil_div(d->nsteps, splits));
+    return static_cast<int>(ceil_div(d->nsteps, spz));  // no empty split
 }
 size_t nint_prefill_split_bytes(const mfq_nint_desc *d, int M) {
     const int splits = nint_prefill_splits(d, M);
