@@ -332,6 +332,13 @@ __global__ __launch_bounds__(256) void prefill_sum_splits_kernel(const float *__
     }
 }
 
+int prefill_sum_splits(const float *part, int64_t ystride, int splits, int M, int N, float *y, int64_t ldy, hipStream_t st) {
+    const int64_t n4 = static_cast<int64_t>(M) * (N / 4);
+    hipLaunchKernelGGL(prefill_sum_splits_kernel, dim3(static_cast<unsigned>(ceil_div(n4, 256))), dim3(256), 0, st, part,
+                       ystride, splits, M, N, y, ldy);
+    return check_launch("prefill_sum_splits");
+}
+
 // Splits over K of a prefill launch: grids of 64-token tiles that leave CUs idle are cut along K (up to eight
 // splits) as long as every split keeps at least two steps and the neuron count allows 16-byte partial rows; the partial results go to a
 // workspace and are added in split order (deterministic).  1 = no split.

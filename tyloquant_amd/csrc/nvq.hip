@@ -391,8 +391,11 @@ template <int MT, int NB, int PF, int XD>
 __global__ __launch_bounds__(512) void nvq_prefill_kernel(NvqK k, const uint8_t *__restrict__ w,
                                                           const uint16_t *__restrict__ x16, int Kp,
                                                           const float *__restrict__ xscale, int M,
-                                                          float *__restrict__ y, int64_t ldy) {
+                                                          float *__restrict__ y, int64_t ldy, int spz, int64_t ystride) {
     static_assert((PF == 2 || PF == 4) && (XD == 1 || XD == 2 || XD == 4), "the sub-step loop is unrolled four times");
+    // split blockIdx.z over K: steps [s_begin, s_end), partial result at y + z * ystride
+    const int s_begin = static_cast<int>(blockIdx.z) * spz, s_end = min(k.nsteps, s_begin + spz);
+    y += static_cast<int64_t>(blockIdx.z) * ystride;
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     constexpr int GS = 24, NM = 3, NT = 512, BM = MT * 16, EL = 8;
     constexpr int ROW = 4 * GS + 8;  // LDS row stride in halves
@@ -477,25 +480,25 @@ __global__ __launch_bounds__(512) void nvq_prefill_kernel(NvqK k, const uint8_t 
 #pragma unroll
         for (int b = 0; b < NB; ++b)
             qq[b] = __builtin_amdgcn_raw_buffer_load_b64(
-                win, b < nrb && s < k.nsteps ? b * rbb + s * sb + (j * 64 + lane) * 8 : kNoStep, 0, 0);
+                win, b < nrb && s < s_end ? b * rbb + s * sb + (j * 64 + lane) * 8 : kNoStep, 0, 0);
     };
     auto hload = [&](int s, u32x2_t (&h)[NB]) {
 #pragma unroll
         for (int b = 0; b < NB; ++b)
-            h[b] = __builtin_amdgcn_raw_buffer_load_b64(win, b < nrb && s < k.nsteps ? b * rbb + s * sb + 2048 + lane * 8 : kNoStep,
+            h[b] = __builtin_amdgcn_raw_buffer_load_b64(win, b < nrb && s < s_end ? b * rbb + s * sb + 2048 + lane * 8 : kNoStep,
                                                         0, 0);
     };
-    xload(0, xr[0]);
+    xload(4 * s_begin, xr[0]);
 #pragma unroll
-    for (int i = 0; i < PF - 1; ++i) wload(i, qr[i]);
-    hload(0, hh);
+    for (int i = 0; i < PF - 1; ++i) wload(4 * s_begin + i, qr[i]);
+    hload(s_begin, hh);
     xstore(0, xr[0]);
 #pragma unroll
-    for (int i = 1; i < XD; ++i) xload(i, xr[i]);
+    for (int i = 1; i < XD; ++i) xload(4 * s_begin + i, xr[i]);
     __syncthreads();  // tables and the first tile
 
     const uint32_t ib = static_cast<uint32_t>(k.ib), im = (1u << ib) - 1u;
-    for (int s = 0; s < k.nsteps; ++s) {
+    for (int s = s_begin; s < s_end; ++s) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int it = 4 * s + j;
@@ -571,12 +574,33 @@ static size_t nvq_prefill_lds(const NvqK &k, int bm) {
     return (static_cast<size_t>(k.banks) * k.entries * 2 + 512 + 32) * 4 + static_cast<size_t>(2 * bm) * (4 * 24 + 8) * 2;
 }
 
-// x16 [M, Kp] fp16 rows scaled by 1 / xscale[m], zero beyond K (x_prep)
+int prefill_sum_splits(const float *part, int64_t ystride, int splits, int M, int N, float *y, int64_t ldy, hipStream_t st);
+
+// Splits over K: grids of 64-token tiles that leave CUs idle are cut along K (up to eight splits of at least two
+// steps); the partial results go to the workspace and are added in split order.  1 = no split.
+static int nvq_prefill_splits(const NvqK &k, int M) {
+    const int64_t blocks = ceil_div(k.n_rowblocks, 16) * ceil_div(M, 64);
+    if (blocks > 128 || k.out % 4) return 1;
+    int splits = static_cast<int>(256 / blocks);
+    if (splits > 8) splits = 8;
+    if (splits > k.nsteps / 2) splits = k.nsteps / 2;
+    if (splits <= 1) return 1;
+    const int spz = static_cast<int>(ceil_div(k.nsteps, splits));
+    return static_cast<int>(ceil_div(k.nsteps, spz));  // no empty split
+}
+
+// x16 [M, Kp] fp16 rows scaled by 1 / xscale[m], zero beyond K (x_prep); part: splits * M * out floats when split
 static int nvq_prefill(const NvqK &k, const uint8_t *w, const uint16_t *x16, int Kp, const float *xscale, int M, float *y,
-                       int64_t ldy, hipStream_t st) {
+                       int64_t ldy, float *part, hipStream_t st) {
+    const int splits = part ? nvq_prefill_splits(k, M) : 1;
+    const int spz = static_cast<int>(ceil_div(k.nsteps, splits));
+    const int64_t ystride = static_cast<int64_t>(M) * k.out;
+    float *yk = splits > 1 ? part : y;
+    const int64_t ldk = splits > 1 ? k.out : ldy;
 #define MFQ_NVQ_PREFILL(MT, XD)                                                                                       \
     {                                                                                                                  \
-        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, 16)), static_cast<unsigned>(ceil_div(M, MT * 16))); \
+        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, 16)), static_cast<unsigned>(ceil_div(M, MT * 16)), \
+                        static_cast<unsigned>(splits));                                                                \
         const size_t lds = nvq_prefill_lds(k, MT * 16);                                                                \
         auto kern = nvq_prefill_kernel<MT, 2, 4, XD>;                                                                  \
         if (lds > 65536) {                                                                                             \
@@ -584,7 +608,8 @@ static int nvq_prefill(const NvqK &k, const uint8_t *w, const uint16_t *x16, int
                                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));     \
             MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nvq_prefill: %s", hipGetErrorString(e));                     \
         }                                                                                                              \
-        hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, k, w, x16, Kp, xscale, M, y, ldy);                          \
+        hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, k, w, x16, Kp, xscale, M, yk, ldk, spz, ystride);           \
+        if (splits > 1) return prefill_sum_splits(part, ystride, splits, M, k.out, y, ldy, st);                        \
         return check_launch("nvq_prefill");                                                                            \
     }
     // 64-token tiles while they give at most one block per CU (four activation tiles in flight), 128-token tiles beyond
@@ -764,13 +789,13 @@ static bool nvq_prefill_capable(const NvqK &k) {
 }
 // Rows up to which re-streaming the weights (16 rows per pass) beats the prefill kernel, from a two-term model fitted
 // to measurements (17408x5120 and 5120x17408): 64 rows of streaming cost about 6 us + 1.7 us per MB of payload, the
-// prefill kernel a flat 20 us + 13.2 us per 1024 of K up to a few hundred rows (a block walks all of K).
+// prefill kernel a flat 38 us + 1 us per 1024 of K up to about a hundred rows (small grids are split over K).
 static int nvq_stream_max(const mfq_nvq_desc *d, const NvqK &k) {
     static const int env = [] { const char *e = getenv("MFQ_NVQ_STREAM_MAX_M"); return e ? atoi(e) : 0; }();
     if (env > 0) return env;
     if (!nvq_prefill_capable(k)) return kNvqStreamMaxM;
     const double t64 = 6.0 + 1.7e-6 * static_cast<double>(d->payload_bytes);
-    const double tp = 20.0 + 13.2 * k.neuron_len / 1024.0;
+    const double tp = 38.0 + 1.0 * k.neuron_len / 1024.0;
     const int m = static_cast<int>(64.0 * tp / t64) / 16 * 16;
     return m < 32 ? 32 : (m > 512 ? 512 : m);
 }
@@ -783,8 +808,11 @@ static int nvq_kp(int K) { return static_cast<int>(ceil_div(K, 32)) * 32; }
 
 extern "C" size_t mfq_hip_nvq_gemm_workspace_bytes(const mfq_nvq_desc *d, int M) {
     if (!d || nvq_streams(d, M)) return 0;
-    if (nvq_prefill_capable(to_k(d)))  // x16 [M, Kp] | xscale [M]
-        return nvq_align256(static_cast<size_t>(M) * nvq_kp(d->neuron_len) * 2) + nvq_align256(static_cast<size_t>(M) * 4);
+    if (nvq_prefill_capable(to_k(d))) {  // x16 [M, Kp] | xscale [M] | partial results of a split over K
+        const int splits = nvq_prefill_splits(to_k(d), M);
+        return nvq_align256(static_cast<size_t>(M) * nvq_kp(d->neuron_len) * 2) + nvq_align256(static_cast<size_t>(M) * 4) +
+               (splits > 1 ? static_cast<size_t>(splits) * M * d->out * 4 : 0);
+    }
     return dequant_gemm_workspace(d->out, d->neuron_len, M);
 }
 
@@ -803,10 +831,13 @@ extern "C" int mfq_hip_nvq_gemm(const mfq_nvq_desc *d, const void *weight, const
         MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nvq_gemm: workspace %zu < %zu bytes",
                     workspace_bytes, need);
         uint16_t *x16 = static_cast<uint16_t *>(workspace);
-        float *xscale = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + nvq_align256(static_cast<size_t>(M) * Kp * 2));
+        uint8_t *p = static_cast<uint8_t *>(workspace) + nvq_align256(static_cast<size_t>(M) * Kp * 2);
+        float *xscale = reinterpret_cast<float *>(p);
+        p += nvq_align256(static_cast<size_t>(M) * 4);
+        float *part = nvq_prefill_splits(k, M) > 1 ? reinterpret_cast<float *>(p) : nullptr;
         const int rc = x_prep(x, x_dtype, ldx, M, k.neuron_len, Kp, x16, xscale, st);
         if (rc) return rc;
-        return nvq_prefill(k, static_cast<const uint8_t *>(weight), x16, Kp, xscale, M, y, ldy, st);
+        return nvq_prefill(k, static_cast<const uint8_t *>(weight), x16, Kp, xscale, M, y, ldy, part, st);
     }
     const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
     MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nvq_gemm: workspace %zu < %zu bytes",
