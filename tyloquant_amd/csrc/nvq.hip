@@ -334,41 +334,106 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
     __syncthreads();  // tables
 
     const uint32_t ib = static_cast<uint32_t>(k.ib), im = (1u << ib) - 1u;
-    for (int s = 0; s < n; ++s) {
-        u32x2_t q[NB][4], hh[NB];
+    if constexpr (NB <= 2) {
+        // Software pipeline as in nint_mfma_body: a row-block's four unit buffers are refilled unit by unit for the next
+        // step, and the activation fragments run two units ahead and are requested before that refill.
+        u32x2_t q[NB][4], hh[NB], hhn[NB];
+        auto unit_off = [&](int i, int s, int j) -> uint32_t {
+            return i < nrb && s < n ? i * rbb + s * sb + (j * 64 + lane) * 8 : kNoStep;
+        };
+        auto hload = [&](int s, u32x2_t (&h)[NB]) {
 #pragma unroll
-        for (int i = 0; i < NB; ++i) {
-            const uint32_t off = i < nrb ? i * rbb + s * sb : kNoStep;
+            for (int i = 0; i < NB; ++i)
+                h[i] = __builtin_amdgcn_raw_buffer_load_b64(win, i < nrb && s < n ? i * rbb + s * sb + 2048 + lane * 8 : kNoStep, 0, 2);
+        };
+        auto xfrags = [&](int it, u32x4_t (&dst)[3]) {
+            const int kpos = (s0 + (it >> 2)) * 16 * 24 + kb * 24 + 4 * (it & 3) * 24;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) q[i][j] = __builtin_amdgcn_raw_buffer_load_b64(win, off + (j * 64 + lane) * 8, 0, 2);
-            hh[i] = __builtin_amdgcn_raw_buffer_load_b64(win, off + 2048 + lane * 8, 0, 2);
-        }
-        const int kbase = (s0 + s) * 16 * 24 + kb * 24;
+            for (int m = 0; m < 3; ++m) dst[m] = load_xfrag_raw<true>(xrow, kpos + 8 * m, k.neuron_len);
+        };
+        hload(0, hh);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            u32x4_t a[3];
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int m = 0; m < 3; ++m) a[m] = load_xfrag<XF16, true>(xrow, kbase + 4 * j * 24 + 8 * m, k.neuron_len);
+            for (int i = 0; i < NB; ++i) q[i][j] = __builtin_amdgcn_raw_buffer_load_b64(win, unit_off(i, 0, j), 0, 2);
+        u32x4_t a1[3], a2[3];
+        xfrags(0, a1);
+        xfrags(1, a2);
+        for (int s = 0; s < n; ++s) {
+            hload(s + 1, hhn);
 #pragma unroll
-            for (int i = 0; i < NB; ++i) {
-                const uint32_t d0 = q[i][j].x, d1 = q[i][j].y;
-                const uint32_t h = ((j < 2 ? hh[i].x : hh[i].y) >> (16 * (j & 1))) & 0xffffu;
-                const uint32_t state = (d1 >> 27) & 15u;
-                const uint32_t *bank = cbp + bankoff[state];
-                const half2_t sc = __builtin_bit_cast(half2_t, luth[state]);
-                const uint32_t mk[3] = {h & 127u, (h >> 7) & 127u, ((d0 >> 27) & 31u) | ((h >> 14) << 5)};
-                const uint32_t ix[6] = {d0 & im, (d0 >> ib) & im, (d0 >> (2 * ib)) & im,
-                                        d1 & im, (d1 >> ib) & im, (d1 >> (2 * ib)) & im};
+            for (int j = 0; j < 4; ++j) {
+                u32x4_t a[3];
 #pragma unroll
                 for (int m = 0; m < 3; ++m) {
-                    const u32x4_t sx = *reinterpret_cast<const u32x4_t *>(sgx + 4 * mk[m]);
-                    const u32x2_t c0 = *reinterpret_cast<const u32x2_t *>(bank + 2 * ix[2 * m]);
-                    const u32x2_t c1 = *reinterpret_cast<const u32x2_t *>(bank + 2 * ix[2 * m + 1]);
-                    const uint32_t wv[4] = {c0.x ^ sx.x, c0.y ^ sx.y, c1.x ^ sx.z, c1.y ^ sx.w};
-                    u32x4_t b;
+                    a[m] = xfrag_finish<XF16, true>(a1[m], (s0 + s) * 16 * 24 + kb * 24 + 4 * j * 24 + 8 * m, k.neuron_len);
+                    a1[m] = a2[m];
+                }
+                xfrags(4 * s + j + 2, a2);
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) b[t] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, wv[t]) * sc);
-                    acc[i] = mfma16(a[m], b, acc[i]);
+                for (int i = 0; i < NB; ++i) {
+                    const uint32_t d0 = q[i][j].x, d1 = q[i][j].y;
+                    q[i][j] = __builtin_amdgcn_raw_buffer_load_b64(win, unit_off(i, s + 1, j), 0, 2);
+                    const uint32_t h = ((j < 2 ? hh[i].x : hh[i].y) >> (16 * (j & 1))) & 0xffffu;
+                    const uint32_t state = (d1 >> 27) & 15u;
+                    const uint32_t *bank = cbp + bankoff[state];
+                    const half2_t sc = __builtin_bit_cast(half2_t, luth[state]);
+                    const uint32_t mk[3] = {h & 127u, (h >> 7) & 127u, ((d0 >> 27) & 31u) | ((h >> 14) << 5)};
+                    const uint32_t ix[6] = {d0 & im, (d0 >> ib) & im, (d0 >> (2 * ib)) & im,
+                                            d1 & im, (d1 >> ib) & im, (d1 >> (2 * ib)) & im};
+#pragma unroll
+                    for (int m = 0; m < 3; ++m) {
+                        const u32x4_t sx = *reinterpret_cast<const u32x4_t *>(sgx + 4 * mk[m]);
+                        const u32x2_t c0 = *reinterpret_cast<const u32x2_t *>(bank + 2 * ix[2 * m]);
+                        const u32x2_t c1 = *reinterpret_cast<const u32x2_t *>(bank + 2 * ix[2 * m + 1]);
+                        const uint32_t wv[4] = {c0.x ^ sx.x, c0.y ^ sx.y, c1.x ^ sx.z, c1.y ^ sx.w};
+                        u32x4_t b;
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) b[t] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, wv[t]) * sc);
+                        acc[i] = mfma16(a[m], b, acc[i]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < NB; ++i) hh[i] = hhn[i];
+        }
+    } else {  // four row-blocks per wave: the plain loop is faster (measured on 17408x5120)
+        for (int s = 0; s < n; ++s) {
+            u32x2_t q[NB][4], hh[NB];
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const uint32_t off = i < nrb ? i * rbb + s * sb : kNoStep;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) q[i][j] = __builtin_amdgcn_raw_buffer_load_b64(win, off + (j * 64 + lane) * 8, 0, 2);
+                hh[i] = __builtin_amdgcn_raw_buffer_load_b64(win, off + 2048 + lane * 8, 0, 2);
+            }
+            const int kbase = (s0 + s) * 16 * 24 + kb * 24;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                u32x4_t a[3];
+#pragma unroll
+                for (int m = 0; m < 3; ++m) a[m] = load_xfrag<XF16, true>(xrow, kbase + 4 * j * 24 + 8 * m, k.neuron_len);
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    const uint32_t d0 = q[i][j].x, d1 = q[i][j].y;
+                    const uint32_t h = ((j < 2 ? hh[i].x : hh[i].y) >> (16 * (j & 1))) & 0xffffu;
+                    const uint32_t state = (d1 >> 27) & 15u;
+                    const uint32_t *bank = cbp + bankoff[state];
+                    const half2_t sc = __builtin_bit_cast(half2_t, luth[state]);
+                    const uint32_t mk[3] = {h & 127u, (h >> 7) & 127u, ((d0 >> 27) & 31u) | ((h >> 14) << 5)};
+                    const uint32_t ix[6] = {d0 & im, (d0 >> ib) & im, (d0 >> (2 * ib)) & im,
+                                            d1 & im, (d1 >> ib) & im, (d1 >> (2 * ib)) & im};
+#pragma unroll
+                    for (int m = 0; m < 3; ++m) {
+                        const u32x4_t sx = *reinterpret_cast<const u32x4_t *>(sgx + 4 * mk[m]);
+                        const u32x2_t c0 = *reinterpret_cast<const u32x2_t *>(bank + 2 * ix[2 * m]);
+                        const u32x2_t c1 = *reinterpret_cast<const u32x2_t *>(bank + 2 * ix[2 * m + 1]);
+                        const uint32_t wv[4] = {c0.x ^ sx.x, c0.y ^ sx.y, c1.x ^ sx.z, c1.y ^ sx.w};
+                        u32x4_t b;
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) b[t] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, wv[t]) * sc);
+                        acc[i] = mfma16(a[m], b, acc[i]);
+                    }
                 }
             }
         }
