@@ -704,9 +704,13 @@ static int nvq_launch_mfma(const NvqK &k, const uint8_t *w, const uint16_t *x, i
 template <int XF16>
 static int nvq_mfma_any(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                         hipStream_t st) {
+    // two row-blocks per wave (they share the activation fragments) while that leaves about 1000 waves over all 16-row
+    // tiles; four were slower on both config 3 shapes (1.2 vs 1.4 TB/s).  MFQ_NVQ_NB overrides for tuning.
     const int64_t wpb = (k.nsteps < 8 ? k.nsteps : 8) * ceil_div(M, 16);  // waves of a block x 16-row tiles
-    if (ceil_div(k.n_rowblocks, 4) * wpb >= 1536) return nvq_launch_mfma<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
-    if (ceil_div(k.n_rowblocks, 2) * wpb >= 1536) return nvq_launch_mfma<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
+    static const int env_nb = [] { const char *e = getenv("MFQ_NVQ_NB"); return e ? atoi(e) : 0; }();
+    if (env_nb == 4) return nvq_launch_mfma<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
+    if (env_nb == 1) return nvq_launch_mfma<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
+    if (env_nb == 2 || ceil_div(k.n_rowblocks, 2) * wpb >= 1024) return nvq_launch_mfma<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
     return nvq_launch_mfma<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
 }
 
