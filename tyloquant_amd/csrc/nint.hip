@@ -415,7 +415,10 @@ int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int
     const NintK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
-    if (M >= 2 && mfma_eligible(k, x, ldx))
+    static const int valu_max = [] { const char *e = getenv("MFQ_GEMV_VALU_MAX_M"); return e ? atoi(e) : 2; }();
+    // two rows: the vector-ALU GEMV unpacks once and takes two dot products (10.6 vs 12.9 us on 12288x4096);
+    // from three rows on the matrix-core kernel wins
+    if (M > valu_max && mfma_eligible(k, x, ldx))
         return x_dtype == MFQ_X_F16 ? launch_mfma<1>(k, w, xp, ldx, M, y, ldy, st)
                                     : launch_mfma<0>(k, w, xp, ldx, M, y, ldy, st);
     // LDS per block grows with MB; large K falls back to narrower row batches.

@@ -170,14 +170,19 @@ __device__ __forceinline__ void nint_mfma_body(const NintK &k, const uint8_t *__
             xsum[j] = xs;
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
+                // fragment scale S = sub_scale / 64 / 2^o and bias C = -1024 S, both from the fp16 pair 1024 + sub_scale
+                // (the byte dropped into the mantissa of 1024.0) with one exact packed FMA each
                 const uint32_t scw = (j < 2) ? sc[i].x : sc[i].y;
-                const float ss = ubyte_f32(scw, 2 * (j & 1)) * (1.f / 64.f);
+                const uint32_t sel = 0x03000100u | ((4u + 2u * (j & 1)) << 16) | (4u + 2u * (j & 1));
+                const half2_t X = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(scw, kMagicH2, sel));
                 half2_t S[NCLS], C[NCLS];
 #pragma unroll
                 for (int c = 0; c < NCLS; ++c) {
-                    const float f = ss * __uint_as_float(0x3f800000u - (static_cast<uint32_t>(BITS * c) << 23));
-                    S[c] = pk_h2(f, f);
-                    C[c] = pk_h2(-1024.f * f, -1024.f * f);
+                    const _Float16 f = static_cast<_Float16>(1.f / static_cast<float>(64 << (BITS * c)));
+                    const _Float16 g = static_cast<_Float16>(1024.f / static_cast<float>(64 << (BITS * c)));
+                    const _Float16 h = static_cast<_Float16>(1024.f * 1024.f / static_cast<float>(64 << (BITS * c)));
+                    S[c] = __builtin_elementwise_fma(X, half2_t{f, f}, half2_t{-g, -g});
+                    C[c] = __builtin_elementwise_fma(X, half2_t{-g, -g}, half2_t{h, h});
                 }
                 uint32_t v[U::NPAIR];
                 U::unpack(q[i][j], (tails[i] >> (8 * j)) & 0xffu, v);
