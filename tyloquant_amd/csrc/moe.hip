@@ -714,12 +714,14 @@ static int moe_decode_launch(MoePools &P, int n_slots, int max_steps, const int3
                              int64_t ldx, int routed_input, const int32_t *ids, int n_pairs, int n_rows, int R, int swiglu,
                              void *out, int out_f16, int64_t ldo, hipStream_t st) {
     static const int env_off = [] { const char *e = getenv("MFQ_MOE_SPLIT"); return e ? atoi(e) == 0 : 0; }();
-    static const int env_w = [] { const char *e = getenv("MFQ_MOE_DEC_WAVES"); return e ? atoi(e) : 16; }();
+    static const int env_w = [] { const char *e = getenv("MFQ_MOE_DEC_WAVES"); return e ? atoi(e) : 8; }();
     static const int env_rbw = [] { const char *e = getenv("MFQ_MOE_DEC_RBW"); return e ? atoi(e) : 0; }();
     if (env_off || n_rows > 65535) return -1;
     const int rbe = out_per_expert / 16;
-    // Waves split the K steps; a wave takes more (row-block, step) items while the grid keeps about
-    // gemv_target_waves() waves.  With the fused SwiGLU a block always takes two row-blocks: gate and up.
+    // At most eight waves split the K steps (two blocks fit a CU at the kernel's 128 registers; measured best at
+    // T = 1: 54 us per layer against 60-62 us with 11..16 waves); a wave takes more (row-block, step) items while
+    // the grid keeps about gemv_target_waves() waves.  With the fused SwiGLU a block always takes two row-blocks:
+    // gate and up.
     const int nwaves = max_steps < env_w ? max_steps : env_w;
     const int spw_max = static_cast<int>(ceil_div(max_steps, nwaves));
     int64_t items = 0;
