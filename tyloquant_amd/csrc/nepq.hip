@@ -269,24 +269,46 @@ __global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *
 
     const float delta = k.profile == 2 ? 0.15625f : 0.125f;
     const uint32_t toff = 1024u, boff = 1024u + (k.tail ? 256u : 0u);
-    for (int s = 0; s < n; ++s) {
-        uint32_t q[NB][4], tails[NB], banks4[NB];
+    // Software pipeline as in nint_mfma_body: the four unit dwords of a row-block are refilled unit by unit for the
+    // next step, tails and bank bytes one step ahead, activation fragments two units ahead and before the refill.
+    uint32_t q[NB][4], tails[NB], banks4[NB], tailsn[NB], banks4n[NB];
+    auto unit_off = [&](int i, int s, int j) -> uint32_t {
+        return i < nrb && s < n ? i * rbb + s * sb + (j * 64 + lane) * 4 : kNoStep;
+    };
+    auto side_load = [&](int s, uint32_t (&tt)[NB], uint32_t (&bb)[NB]) {
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
-            const uint32_t off = i < nrb ? i * rbb + s * sb : kNoStep;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) q[i][j] = __builtin_amdgcn_raw_buffer_load_b32(win, off + (j * 64 + lane) * 4, 0, 2);
-            tails[i] = k.tail ? __builtin_amdgcn_raw_buffer_load_b32(win, off + toff + lane * 4, 0, 2) : 0u;
-            banks4[i] = __builtin_amdgcn_raw_buffer_load_b32(win, off + boff + r * 4, 0, 2);
+            const uint32_t off = i < nrb && s < n ? i * rbb + s * sb : kNoStep;
+            tt[i] = k.tail ? __builtin_amdgcn_raw_buffer_load_b32(win, off + toff + lane * 4, 0, 2) : 0u;
+            bb[i] = __builtin_amdgcn_raw_buffer_load_b32(win, off + boff + r * 4, 0, 2);
         }
-        const int kbase = (s0 + s) * 16 * 24 + kb * 24;
+    };
+    auto xfrags = [&](int it, u32x4_t (&dst)[3]) {
+        const int kpos = (s0 + (it >> 2)) * 16 * 24 + kb * 24 + 4 * (it & 3) * 24;
+#pragma unroll
+        for (int m = 0; m < 3; ++m) dst[m] = load_xfrag_raw<true>(xrow, kpos + 8 * m, k.neuron_len);
+    };
+    side_load(0, tails, banks4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < NB; ++i) q[i][j] = __builtin_amdgcn_raw_buffer_load_b32(win, unit_off(i, 0, j), 0, 2);
+    u32x4_t a1[3], a2[3];
+    xfrags(0, a1);
+    xfrags(1, a2);
+    for (int s = 0; s < n; ++s) {
+        side_load(s + 1, tailsn, banks4n);
         float xsum[4];
         uint32_t stw[NB][4];  // per unit: state * (bias - 1) as an fp16
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             u32x4_t a[3];
 #pragma unroll
-            for (int m = 0; m < 3; ++m) a[m] = load_xfrag<XF16, true>(xrow, kbase + 4 * j * 24 + 8 * m, k.neuron_len);
+            for (int m = 0; m < 3; ++m) {
+                a[m] = xfrag_finish<XF16, true>(a1[m], (s0 + s) * 16 * 24 + kb * 24 + 4 * j * 24 + 8 * m, k.neuron_len);
+                a1[m] = a2[m];
+            }
+            xfrags(4 * s + j + 2, a2);
             float xs = 0.f;
 #pragma unroll
             for (int m = 0; m < 3; ++m)
@@ -296,6 +318,7 @@ __global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
                 const NepqUnit u = nepq_decode(k.profile, q[i][j], (tails[i] >> (8 * j)) & 0xffu);
+                q[i][j] = __builtin_amdgcn_raw_buffer_load_b32(win, unit_off(i, s + 1, j), 0, 2);
                 const uint16_t *bank = tab + ((banks4[i] >> (8 * j)) & 0xffu) * k.entries;
                 const float st = static_cast<float>(u.state);
                 const half2_t S = pk_h2(st, st), C = pk_h2(-1024.f * st, -1024.f * st);
@@ -327,6 +350,11 @@ __global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *
         for (int i = 0; i < NB; ++i) {
             const uint32_t b01 = stw[i][0] | (stw[i][1] << 16), b23 = stw[i][2] | (stw[i][3] << 16);
             accB[i] = mfma16(ax, u32x4_t{b01, b23, b01, b23}, accB[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < NB; ++i) {
+            tails[i] = tailsn[i];
+            banks4[i] = banks4n[i];
         }
     }
 #pragma unroll
@@ -375,6 +403,10 @@ template <int XF16>
 static int nepq_mfma_any(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
                          float *y, int64_t ldy, hipStream_t st) {
     const int64_t wpb = (k.nsteps < 8 ? k.nsteps : 8) * ceil_div(M, 16);  // waves of a block x 16-row tiles
+    static const int env_nb = [] { const char *e = getenv("MFQ_NEPQ_NB"); return e ? atoi(e) : 0; }();
+    if (env_nb == 4) return nepq_launch_mfma<XF16, 4>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
+    if (env_nb == 2) return nepq_launch_mfma<XF16, 2>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
+    if (env_nb == 1) return nepq_launch_mfma<XF16, 1>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
     if (ceil_div(ceil_div(nrows, 16), 4) * wpb >= 1536) return nepq_launch_mfma<XF16, 4>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
     return nepq_launch_mfma<XF16, 1>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
 }
