@@ -91,11 +91,14 @@ def test_gemm_matches_oracle(bits, gs, sb, out, K, M):
 
 
 @pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (4, 48, 6)])
-def test_gemm_many_rows_takes_the_128_token_tiles(bits, gs, sb):
-    """More than one block per CU (5 neuron blocks x 53 token tiles of 64): the prefill kernel switches to its 128-token
-    tile.  Ragged everywhere: 65 row-blocks, K not a multiple of the groupsize, one token past 26 full tiles."""
-    rng = np.random.default_rng(270 + bits)
-    out, K, M = 1040, 280, 3329
+@pytest.mark.parametrize("out,M", [(1040, 3329), (256, 16500)])
+def test_gemm_many_rows_takes_the_large_tiles(bits, gs, sb, out, M):
+    """More than one block per CU with 64 x 256 tiles: the prefill kernel switches to 64 x 384 tiles (65 row-blocks x
+    53 token tiles: one round of 159 blocks instead of 135 larger ones; the profiles with wide units keep 128 x 256) or
+    to 128 x 256 tiles (16 row-blocks x 16500 tokens: 129 blocks instead of 258).  Ragged everywhere: row-blocks, K not
+    a multiple of the groupsize, a last token tile with one or 116 rows."""
+    rng = np.random.default_rng(270 + bits + out)
+    K = 280
     t = O.quantize_nint((rng.standard_normal((out, K)) * 0.02).astype(np.float32), bits, gs, sb)
     lin = _load(t)
     x, xf = _x(rng, M, K)

@@ -388,15 +388,22 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
         }                                                                                                      \
         return check_launch("nint_prefill");                                                                   \
     }
-    // Block = 8 waves side by side on 256 neurons (two row-blocks per wave), each with four unit buffers per row-block
-    // (three sub-steps of weights in flight).  While 64-token tiles give at most one block per CU, they are used with
-    // four activation tiles in flight: the time is then that of one block's walk through K, and short tiles walk
-    // fastest.  Beyond that, 128-token tiles: every dequantized fragment feeds eight MFMAs instead of four.
+    // Block = 8 waves side by side on the neurons, each with four unit buffers per row-block (three sub-steps of
+    // weights in flight).  While 64-token x 256-neuron tiles give at most one block per CU, they are used with four
+    // activation tiles in flight: the time is then that of one block's walk through K, and short tiles walk fastest.
+    // Beyond that, the cheaper of 128 x 256 (every dequantized fragment feeds eight MFMAs) and 64 x 384 (three
+    // row-blocks per wave) by rounds of 256 blocks x tile area; the second runs at 0.97 of the first's rate per area.
     const bool small = ceil_div(k.n_rowblocks, 16) * ceil_div(M, 64) <= 256;
-#define MFQ_PREFILL(UNIT, B, G)                              \
-    if (k.bits == B && k.gs == G) {                          \
-        if (small) MFQ_PREFILL_CFG(UNIT, B, G, 4, 2, 4, 4)   \
-        MFQ_PREFILL_CFG(UNIT, B, G, 8, 2, 4, (UNIT<B, G>::D >= 5 ? 1 : 2)) /* wide units: registers for one tile */ \
+    const double cost_a = static_cast<double>(ceil_div(ceil_div(k.n_rowblocks, 16) * ceil_div(M, 128), 256)) * (128 * 256);
+    const double cost_b = static_cast<double>(ceil_div(ceil_div(k.n_rowblocks, 24) * ceil_div(M, 64), 256)) * (64 * 384) / 0.97;
+    const bool wide3 = cost_b < cost_a;
+#define MFQ_PREFILL(UNIT, B, G)                                                                                       \
+    if (k.bits == B && k.gs == G) {                                                                                   \
+        if (small) MFQ_PREFILL_CFG(UNIT, B, G, 4, 2, 4, 4)                                                            \
+        if constexpr (UNIT<B, G>::D <= 4) {                                                                           \
+            if (wide3) MFQ_PREFILL_CFG(UNIT, B, G, 4, 3, 4, 2)                                                        \
+        }                                                                                                             \
+        MFQ_PREFILL_CFG(UNIT, B, G, 8, 2, 4, (UNIT<B, G>::D >= 5 ? 1 : 2)) /* wide units: registers for one tile */   \
     }
     if (k.kind == 1) {
         MFQ_PREFILL(PairedUnit, 4, 32) MFQ_PREFILL(PairedUnit, 4, 24) MFQ_PREFILL(PairedUnit, 4, 16)
