@@ -54,11 +54,13 @@ def test_nvq_matrix_core_path_multi_step(out, K, M):
     _check(nvq_matmul(lin.weight, x, force="gemv").cpu().numpy(), O.linear_forward_f64(want, x.float().cpu().numpy()))
 
 
-@pytest.mark.parametrize("out,K,M,banks", [(130, 1024, 520, 2), (96, 4104, 600, 4), (272, 1024, 8300, 2)])
+@pytest.mark.parametrize("out,K,M,banks", [(130, 1024, 520, 2), (96, 4104, 600, 4), (272, 1024, 8300, 2),
+                                          (1040, 1024, 3329, 2)])
 def test_nvq_prefill_kernel(out, K, M, banks):
     """Above the streaming range (at most 512 rows) the block-tiled kernel takes over: 64-token tiles, and 128-token
-    tiles once the grid exceeds one block per CU (130 token tiles x 2 neuron blocks); ragged row-blocks, K not a
-    multiple of 96, a last token tile with one row."""
+    tiles once the grid exceeds one block per CU (130 token tiles x 2 neuron blocks) or 64 x 384 tiles where they take
+    fewer rounds (65 row-blocks x 53 token tiles); ragged row-blocks, K not a multiple of 96, a last token tile with one
+    row."""
     from tyloquant_amd import runtime as R
     rng = np.random.default_rng(170 + out + M)
     t = synth.nvq_jsc_random(rng, out, K, "d4_512", banks)

@@ -662,12 +662,12 @@ static int nvq_prefill(const NvqK &k, const uint8_t *w, const uint16_t *x16, int
     const int64_t ystride = static_cast<int64_t>(M) * k.out;
     float *yk = splits > 1 ? part : y;
     const int64_t ldk = splits > 1 ? k.out : ldy;
-#define MFQ_NVQ_PREFILL(MT, XD)                                                                                       \
+#define MFQ_NVQ_PREFILL(MT, NB, XD)                                                                                   \
     {                                                                                                                  \
-        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, 16)), static_cast<unsigned>(ceil_div(M, MT * 16)), \
+        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, 8 * NB)), static_cast<unsigned>(ceil_div(M, MT * 16)), \
                         static_cast<unsigned>(splits));                                                                \
         const size_t lds = nvq_prefill_lds(k, MT * 16);                                                                \
-        auto kern = nvq_prefill_kernel<MT, 2, 4, XD>;                                                                  \
+        auto kern = nvq_prefill_kernel<MT, NB, 4, XD>;                                                                 \
         if (lds > 65536) {                                                                                             \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                   \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));     \
@@ -677,9 +677,14 @@ static int nvq_prefill(const NvqK &k, const uint8_t *w, const uint16_t *x16, int
         if (splits > 1) return prefill_sum_splits(part, ystride, splits, M, k.out, y, ldy, st);                        \
         return check_launch("nvq_prefill");                                                                            \
     }
-    // 64-token tiles while they give at most one block per CU (four activation tiles in flight), 128-token tiles beyond
-    if (ceil_div(k.n_rowblocks, 16) * ceil_div(M, 64) <= 256) MFQ_NVQ_PREFILL(4, 4)
-    MFQ_NVQ_PREFILL(8, 2)
+    // 64 x 256 tiles while they give at most one block per CU (four activation tiles in flight); beyond, the cheaper
+    // of 128 x 256 and 64 x 384 by rounds of 256 blocks x tile area (see nint_prefill; here the second runs at 0.85 of
+    // the first's rate per area: building a fragment costs more, so sharing it among eight token tiles counts for more)
+    if (ceil_div(k.n_rowblocks, 16) * ceil_div(M, 64) <= 256) MFQ_NVQ_PREFILL(4, 2, 4)
+    const double cost_a = static_cast<double>(ceil_div(ceil_div(k.n_rowblocks, 16) * ceil_div(M, 128), 256)) * (128 * 256);
+    const double cost_b = static_cast<double>(ceil_div(ceil_div(k.n_rowblocks, 24) * ceil_div(M, 64), 256)) * (64 * 384) / 0.85;
+    if (cost_b < cost_a) MFQ_NVQ_PREFILL(4, 3, 2)
+    MFQ_NVQ_PREFILL(8, 2, 2)
 #undef MFQ_NVQ_PREFILL
 }
 
