@@ -210,6 +210,32 @@ def test_decode_matmul_matches_the_separate_calls(T, H, W):
         assert torch.equal(plain.view(torch.int32), gu(x, route).reshape(T * k, 2 * W).view(torch.int32))
 
 
+def test_decode_matmul_rejects_what_it_cannot_run():
+    """Cohorts without a batch-1 unit (6-bit experts) and a shared tensor of another height are refused with a message,
+    and the FFN forward then takes the separate calls."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_moe import nint_moe_ffn_forward
+    rng = np.random.default_rng(77)
+    E, H, W, k = 6, 96, 48, 2
+    _, gu = _moe(rng, E, 2 * W, H, [4, 6, 3, 4, 6, 2])
+    _, dn = _moe(rng, E, H, W, [4, 6, 3, 4, 6, 2])
+    ids = torch.from_numpy(np.array([[0, 2]], dtype=np.int32)).cuda()
+    x = torch.from_numpy(rng.standard_normal((1, H)).astype(np.float32)).to(torch.bfloat16).cuda()
+    assert not gu.decode_capable()
+    with pytest.raises(RuntimeError, match="no batch-1 kernel"):
+        gu.forward_decode(x, ids)
+    tg, gu4 = _moe(rng, E, 2 * W, H, [4, 3, 3, 4, 2, 2])
+    td, dn4 = _moe(rng, E, H, W, [4, 3, 3, 4, 2, 2])
+    other = R.load_quant_linear("NINT4", O.pack_nint(O.quantize_nint(
+        (rng.standard_normal((W, H)) * 0.02).astype(np.float32), 4, 24, 6))).weight
+    assert not gu4.decode_capable(other)
+    with pytest.raises(RuntimeError, match="shared tensor has"):
+        gu4.forward_decode(x, ids, other)
+    logits = rng.standard_normal((1, E)).astype(np.float32)
+    out, _, _ = nint_moe_ffn_forward(gu, dn, x, torch.from_numpy(logits).cuda(), k, delayed_softmax=True)
+    assert out.shape == (1, H) and bool(torch.isfinite(out).all())
+
+
 def test_moe_errors():
     from tyloquant_amd.runtime_moe import NintMoeWeight, build_moe_route_plan
     rng = np.random.default_rng(2)
