@@ -132,6 +132,23 @@ def test_nepq_matrix_core_path_multi_step(label, out, K, M, banks):
         _check(nepq_matmul(w, x, e, force="gemv").cpu().numpy(), O.linear_forward_f64(want[e], x.float().cpu().numpy()))
 
 
+@pytest.mark.parametrize("label,out,K,M,banks", [("NEPQ1-S", 130 - 2, 1024, 70, 4), ("NEPQ1-L", 48, 4104, 300, 16),
+                                                  ("NEPQ1-L", 272, 1544, 100, 40), ("NEPQ1-S", 272, 1024, 8300, 3),
+                                                  ("NEPQ1-S", 1040, 1024, 3329, 5)])
+def test_nepq_prefill_kernel(label, out, K, M, banks):
+    """From 64 rows on the block-tiled kernel takes over: 64 x 256 tiles (split over K for the long-K case), 128 x 256
+    and 64 x 384 tiles for the large grids, tables in LDS or read from global memory (40 banks of the L profile), a
+    second expert's row slice, ragged row-blocks, K not a multiple of 96, a last token tile with one row."""
+    from tyloquant_amd.runtime_vq import NepqWeight, nepq_matmul
+    rng = np.random.default_rng(500 + out + M)
+    t = synth.nepq_random(rng, label, 2, out, K, banks)
+    w = NepqWeight.from_blob(O.pack_nepq(t))
+    want = O.dequantize_nepq(t)
+    for e, xd in ((0, torch.bfloat16), (1, torch.float16)):
+        x, xf = _x(rng, M, K, xd)
+        _check(nepq_matmul(w, x, e).cpu().numpy(), O.linear_forward_f64(want[e], xf))
+
+
 def test_nepq_hadamard_matches_fwht():
     from tyloquant_amd.runtime_vq import nepq_hadamard
     rng = np.random.default_rng(3)

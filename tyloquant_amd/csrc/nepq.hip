@@ -10,7 +10,7 @@
 // value = fl(anchor * state) * (code + bias), bias = +-5/32 (S) or +-1/8 (L), minus when aux is set.
 #include "common.hpp"
 #include "gemv_common.hpp"
-#include "nint_mfma.hpp"
+#include "nint_prefill.hpp"
 
 namespace mfq {
 
@@ -374,6 +374,234 @@ __global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *
     }
 }
 
+// ---- prefill: block-tiled MFMA GEMM, weight fragments built from the ternary tables ------------------------
+// Same frame as the NVQ prefill kernel: block = 8 waves x NB row-blocks, wave tile MT * 16 tokens, activations as
+// scaled fp16 rows (x_prep) through two LDS buffers with XD tiles in flight, PF unit dwords per row-block in flight.
+// A fragment is one table entry: (1024 + digit) pairs -> state * digit with one exact packed FMA, plus
+// state * (bias - 1) with one packed add (exact for the 1/8 bias, one fp16 rounding for 5/32), so no separate bias
+// term is needed.  Rows [row0, row0 + nrows) of the tensor (an expert's slice) go to columns 0 .. nrows - 1 of y.
+// LDS: [table: banks * entries u16, when TAB_LDS][x tiles]
+template <int MT, int NB, int PF, int XD, int TAB_LDS>
+__global__ __launch_bounds__(512) void nepq_prefill_kernel(NepqK k, const uint8_t *__restrict__ w, int rb_first, int row0,
+                                                           int nrows, const uint16_t *__restrict__ x16, int Kp,
+                                                           const float *__restrict__ xscale, int M,
+                                                           float *__restrict__ y, int64_t ldy, int spz, int64_t ystride) {
+    static_assert((PF == 2 || PF == 4) && (XD == 1 || XD == 2 || XD == 4), "the sub-step loop is unrolled four times");
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    constexpr int GS = 24, NM = 3, NT = 512, BM = MT * 16, EL = 8;
+    constexpr int ROW = 4 * GS + 8;
+    constexpr int CPG = GS / EL, CHUNKS = 4 * CPG;
+    constexpr int PER_THREAD = (BM * CHUNKS + NT - 1) / NT;
+    const int s_begin = static_cast<int>(blockIdx.z) * spz, s_end = min(k.nsteps, s_begin + spz);
+    y += static_cast<int64_t>(blockIdx.z) * ystride;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, kb = lane >> 4;
+    const uint16_t *gtab = reinterpret_cast<const uint16_t *>(w + k.tables_off);
+    const int ntab = k.banks * k.entries;  // u16 entries, even
+    uint16_t *xt = reinterpret_cast<uint16_t *>(lds);
+    if constexpr (TAB_LDS) {
+        for (int i = tid; i < ntab / 2; i += NT) lds[i] = reinterpret_cast<const uint32_t *>(gtab)[i];
+        xt = reinterpret_cast<uint16_t *>(lds + (ntab / 2 + 3) / 4 * 4);
+    }
+    const uint16_t *tab = TAB_LDS ? reinterpret_cast<const uint16_t *>(lds) : gtab;
+    const DenseRows rows{static_cast<int>(blockIdx.y) * BM, M};
+    const int rb_end = rb_first + (nrows + 15) / 16;
+    const int rb0 = rb_first + (static_cast<int>(blockIdx.x) * 8 + wave) * NB;
+    const int nrb = max(0, min(NB, rb_end - rb0));
+    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
+    const __amdgpu_buffer_rsrc_t win =
+        wave_window(w + static_cast<int64_t>(min(rb0, k.n_rowblocks - 1)) * k.rowblock_bytes, nrb * rbb);
+    float4_t acc[MT][NB];
+#pragma unroll
+    for (int a = 0; a < MT; ++a)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const uint16_t *xsrc[PER_THREAD];
+    int xk[PER_THREAD];
+#pragma unroll
+    for (int p = 0; p < PER_THREAD; ++p) {
+        const int c = min(tid + NT * p, BM * CHUNKS - 1);
+        const int row = c / CHUNKS;
+        xsrc[p] = x16 + static_cast<int64_t>(rows.src(row)) * Kp;
+        xk[p] = EL * (c - row * CHUNKS);
+    }
+    u32x4_t xr[XD][PER_THREAD];
+    auto xload = [&](int it, u32x4_t (&xq)[PER_THREAD]) {
+        const int k0 = it * 4 * GS;
+#pragma unroll
+        for (int p = 0; p < PER_THREAD; ++p) {
+            const int kk = k0 + xk[p];
+            u32x4_t v = *reinterpret_cast<const u32x4_t *>(xsrc[p] + min(kk, Kp - EL));
+            if (kk >= Kp) v = u32x4_t{0u, 0u, 0u, 0u};
+            xq[p] = v;
+        }
+    };
+    auto xstore = [&](int buf, const u32x4_t (&xq)[PER_THREAD]) {
+#pragma unroll
+        for (int p = 0; p < PER_THREAD; ++p) {
+            const int c = tid + NT * p;
+            const int row = c / CHUNKS, ch = c - row * CHUNKS;
+            if (c < BM * CHUNKS) *reinterpret_cast<u32x4_t *>(xt + buf * (BM * ROW) + row * ROW + EL * ch) = xq[p];
+        }
+    };
+    const uint32_t toff = 1024u, boff = 1024u + (k.tail ? 256u : 0u);
+    uint32_t qr[PF][NB], tails[NB], banks4[NB], tailsn[NB], banks4n[NB];
+    auto wload = [&](int it, uint32_t (&qq)[NB]) {
+        const int s = it >> 2, j = it & 3;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            qq[b] = __builtin_amdgcn_raw_buffer_load_b32(win, b < nrb && s < s_end ? b * rbb + s * sb + (j * 64 + lane) * 4 : kNoStep,
+                                                         0, 0);
+    };
+    auto side_load = [&](int s, uint32_t (&tt)[NB], uint32_t (&bb)[NB]) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const uint32_t off = b < nrb && s < s_end ? b * rbb + s * sb : kNoStep;
+            tt[b] = k.tail ? __builtin_amdgcn_raw_buffer_load_b32(win, off + toff + lane * 4, 0, 0) : 0u;
+            bb[b] = __builtin_amdgcn_raw_buffer_load_b32(win, off + boff + r * 4, 0, 0);
+        }
+    };
+    xload(4 * s_begin, xr[0]);
+#pragma unroll
+    for (int i = 0; i < PF - 1; ++i) wload(4 * s_begin + i, qr[i]);
+    side_load(s_begin, tails, banks4);
+    xstore(0, xr[0]);
+#pragma unroll
+    for (int i = 1; i < XD; ++i) xload(4 * s_begin + i, xr[i]);
+    __syncthreads();  // table and the first tile
+
+    const float delta = k.profile == 2 ? 0.15625f : 0.125f;
+    for (int s = s_begin; s < s_end; ++s) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int it = 4 * s + j;
+            xload(it + XD, xr[j % XD]);
+            wload(it + PF - 1, qr[(j + PF - 1) % PF]);
+            if (j == 0) side_load(s + 1, tailsn, banks4n);
+            const uint16_t *bank[NB];
+            half2_t S[NB], C[NB], Bv[NB];
+            uint32_t ix[NB][3];
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const NepqUnit u = nepq_decode(k.profile, qr[j % PF][b], (tails[b] >> (8 * j)) & 0xffu);
+                bank[b] = tab + ((banks4[b] >> (8 * j)) & 0xffu) * k.entries;
+                const float st = static_cast<float>(u.state);
+                S[b] = pk_h2(st, st);
+                C[b] = pk_h2(-1024.f * st, -1024.f * st);
+                const float bs = st * ((u.aux ? -delta : delta) - 1.f);
+                Bv[b] = pk_h2(bs, bs);
+                ix[b][0] = u.idx[0]; ix[b][1] = u.idx[1]; ix[b][2] = u.idx[2];
+            }
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                u32x4_t af[MT];
+#pragma unroll
+                for (int a = 0; a < MT; ++a)
+                    af[a] = *reinterpret_cast<const u32x4_t *>(xt + (j & 1) * (BM * ROW) + (a * 16 + r) * ROW + kb * GS + 8 * m);
+                u32x4_t bf[NB];
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    const uint32_t e = bank[b][ix[b][m]];
+                    const uint32_t t2 = e | (e << 14);
+#pragma unroll
+                    for (int p = 0; p < 4; ++p)
+                        bf[b][p] = __builtin_bit_cast(uint32_t, h2_fma(((t2 >> (4 * p)) & 0x00030003u) | kMagicH2, S[b], C[b]) + Bv[b]);
+                }
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+#pragma unroll
+                    for (int a = 0; a < MT; ++a) acc[a][b] = mfma16(af[a], bf[b], acc[a][b]);
+            }
+            xstore((j + 1) & 1, xr[(j + 1) % XD]);
+            if (j == 3) {
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    tails[b] = tailsn[b];
+                    banks4[b] = banks4n[b];
+                }
+            }
+            __syncthreads();
+        }
+    }
+    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
+    float an[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) an[b] = anchors[min(rb0 + b, k.n_rowblocks - 1) * 16 + r];
+#pragma unroll
+    for (int a = 0; a < MT; ++a) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int ti = a * 16 + 4 * kb + v;
+            const int m = rows.dst(ti);
+            if (m < 0) continue;
+            const float xs = xscale[m];
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const int col = (rb0 + b) * 16 + r - row0;
+                if (rb0 + b < rb_end && col >= 0 && col < nrows) y[static_cast<int64_t>(m) * ldy + col] = xs * (an[b] * acc[a][b][v]);
+            }
+        }
+    }
+}
+
+int prefill_sum_splits(const float *part, int64_t ystride, int splits, int M, int N, float *y, int64_t ldy, hipStream_t st);
+
+static bool nepq_prefill_capable(const NepqK &k) {
+    return k.neuron_len >= 8 && (k.banks * k.entries) % 2 == 0 && 3 * k.rowblock_bytes < (1ll << 31);
+}
+static int nepq_prefill_splits(const NepqK &k, int nrows, int M) {
+    const int64_t blocks = ceil_div(ceil_div(nrows, 16), 16) * ceil_div(M, 64);
+    if (blocks > 128 || nrows % 4) return 1;
+    int splits = static_cast<int>(256 / blocks);
+    if (splits > 8) splits = 8;
+    if (splits > k.nsteps / 2) splits = k.nsteps / 2;
+    if (splits <= 1) return 1;
+    const int spz = static_cast<int>(ceil_div(k.nsteps, splits));
+    return static_cast<int>(ceil_div(k.nsteps, spz));
+}
+
+// x16 [M, Kp] fp16 rows scaled by 1 / xscale[m], zero beyond K (x_prep); part: splits * M * nrows floats when split
+static int nepq_prefill(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x16, int Kp,
+                        const float *xscale, int M, float *y, int64_t ldy, float *part, hipStream_t st) {
+    const int splits = part ? nepq_prefill_splits(k, nrows, M) : 1;
+    const int spz = static_cast<int>(ceil_div(k.nsteps, splits));
+    const int64_t ystride = static_cast<int64_t>(M) * nrows;
+    float *yk = splits > 1 ? part : y;
+    const int64_t ldk = splits > 1 ? nrows : ldy;
+    const int nrb = static_cast<int>(ceil_div(nrows, 16));
+    const size_t tabb = (static_cast<size_t>(k.banks) * k.entries * 2 + 15) / 16 * 16;
+    const bool tab_lds = tabb <= 48 * 1024;
+#define MFQ_NEPQ_PREFILL(MT, NB, XD)                                                                                   \
+    {                                                                                                                  \
+        const dim3 grid(static_cast<unsigned>(ceil_div(nrb, 8 * NB)), static_cast<unsigned>(ceil_div(M, MT * 16)),     \
+                        static_cast<unsigned>(splits));                                                                \
+        const size_t lds = (tab_lds ? tabb : 0) + static_cast<size_t>(2 * MT * 16) * (4 * 24 + 8) * 2;                 \
+        auto launch = [&](auto kern) -> int {                                                                          \
+            if (lds > 65536) {                                                                                         \
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                               \
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+                MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nepq_prefill: %s", hipGetErrorString(e));                \
+            }                                                                                                          \
+            hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, k, w, row0 / 16, row0, nrows, x16, Kp, xscale, M, yk, ldk, spz, \
+                               ystride);                                                                               \
+            return MFQ_OK;                                                                                             \
+        };                                                                                                             \
+        const int rc = tab_lds ? launch(nepq_prefill_kernel<MT, NB, 4, XD, 1>) : launch(nepq_prefill_kernel<MT, NB, 4, XD, 0>); \
+        if (rc) return rc;                                                                                             \
+        if (splits > 1) return prefill_sum_splits(part, ystride, splits, M, nrows, y, ldy, st);                        \
+        return check_launch("nepq_prefill");                                                                           \
+    }
+    // tiles as in nvq_prefill
+    if (ceil_div(nrb, 16) * ceil_div(M, 64) <= 256) MFQ_NEPQ_PREFILL(4, 2, 4)
+    const double cost_a = static_cast<double>(ceil_div(ceil_div(nrb, 16) * ceil_div(M, 128), 256)) * (128 * 256);
+    const double cost_b = static_cast<double>(ceil_div(ceil_div(nrb, 24) * ceil_div(M, 64), 256)) * (64 * 384) / 0.85;
+    if (cost_b < cost_a) MFQ_NEPQ_PREFILL(4, 3, 2)
+    MFQ_NEPQ_PREFILL(8, 2, 2)
+#undef MFQ_NEPQ_PREFILL
+}
+
 static bool nepq_stream_capable(const NepqK &k) {
     return k.neuron_len >= 8 && k.neuron_len % 8 == 0 && 4 * k.rowblock_bytes < (1ll << 31);
 }
@@ -574,15 +802,30 @@ extern "C" int mfq_hip_nepq_gemv(const mfq_nepq_desc *d, const void *weight, int
     return nepq_gemv_any(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, as_stream(stream));
 }
 
-// The reference's Python policy keeps M <= 16 on the GEMV; tensors the matrix-core streaming kernel takes stay
-// on it up to kNepqStreamMaxM rows.
-static constexpr int kNepqGemvMaxM = 16, kNepqStreamMaxM = 256;
-static bool nepq_streams(const mfq_nepq_desc *d, int M) {
-    return M <= kNepqGemvMaxM || (M <= kNepqStreamMaxM && nepq_stream_capable(to_k(d)));
+// The reference's Python policy keeps M <= 16 on the GEMV.  Two 16-row passes of the matrix-core streaming kernel cost
+// what the prefill kernel costs up to about a hundred rows (40 us on 12288x4096), so the prefill kernel takes over
+// from kNepqPrefillMinM rows; tensors it cannot take stay on the streaming kernel up to kNepqStreamMaxM rows.
+static constexpr int kNepqGemvMaxM = 16, kNepqStreamMaxM = 256, kNepqPrefillMinM = 33;
+static bool nepq_prefills(const NepqK &k, int M) {
+    static const int env = [] { const char *e = getenv("MFQ_NEPQ_PREFILL_MIN_M"); return e ? atoi(e) : 0; }();
+    return M >= (env > 0 ? env : kNepqPrefillMinM) && nepq_prefill_capable(k);
 }
+static bool nepq_streams(const mfq_nepq_desc *d, int M) {
+    const NepqK k = to_k(d);
+    if (M > kNepqGemvMaxM && nepq_prefills(k, M)) return false;
+    return M <= kNepqGemvMaxM || (M <= kNepqStreamMaxM && nepq_stream_capable(k));
+}
+static size_t nepq_align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+static int nepq_kp(int K) { return static_cast<int>(ceil_div(K, 32)) * 32; }
 
 extern "C" size_t mfq_hip_nepq_gemm_workspace_bytes(const mfq_nepq_desc *d, int nrows, int M) {
     if (!d || nepq_streams(d, M)) return 0;
+    const NepqK k = to_k(d);
+    if (nepq_prefills(k, M)) {  // x16 [M, Kp] | xscale [M] | partial results of a split over K
+        const int splits = nepq_prefill_splits(k, nrows, M);
+        return nepq_align256(static_cast<size_t>(M) * nepq_kp(k.neuron_len) * 2) + nepq_align256(static_cast<size_t>(M) * 4) +
+               (splits > 1 ? static_cast<size_t>(splits) * M * nrows * 4 : 0);
+    }
     return dequant_gemm_workspace(nrows, d->neuron_len, M);
 }
 
@@ -596,6 +839,21 @@ extern "C" int mfq_hip_nepq_gemm(const mfq_nepq_desc *d, const void *weight, int
     MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= nrows, MFQ_ERR_INVALID, "nepq_gemm: ldx/ldy smaller than the tensor");
     hipStream_t st = as_stream(stream);
     if (nepq_streams(d, M)) return nepq_gemv_any(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, st);
+    if (nepq_prefills(to_k(d), M)) {
+        const NepqK k = to_k(d);
+        const int Kp = nepq_kp(k.neuron_len);
+        const size_t need = mfq_hip_nepq_gemm_workspace_bytes(d, nrows, M);
+        MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nepq_gemm: workspace %zu < %zu bytes",
+                    workspace_bytes, need);
+        uint16_t *x16 = static_cast<uint16_t *>(workspace);
+        uint8_t *p = static_cast<uint8_t *>(workspace) + nepq_align256(static_cast<size_t>(M) * Kp * 2);
+        float *xscale = reinterpret_cast<float *>(p);
+        p += nepq_align256(static_cast<size_t>(M) * 4);
+        float *part = nepq_prefill_splits(k, nrows, M) > 1 ? reinterpret_cast<float *>(p) : nullptr;
+        const int rc = x_prep(x, x_dtype, ldx, M, k.neuron_len, Kp, x16, xscale, st);
+        if (rc) return rc;
+        return nepq_prefill(k, static_cast<const uint8_t *>(weight), row0, nrows, x16, Kp, xscale, M, y, ldy, part, st);
+    }
     const size_t need = dequant_gemm_workspace(nrows, d->neuron_len, M);
     MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nepq_gemm: workspace %zu < %zu bytes",
                 workspace_bytes, need);
