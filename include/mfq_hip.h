@@ -74,10 +74,18 @@ int mfq_hip_nint_dequant_f32(const mfq_nint_desc *d, const void *weight, float *
 int mfq_hip_nint_gemv(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
                       int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream);
 
-/* Any-M entry: the streaming kernels of mfq_hip_nint_gemv up to 256 rows, above that a block-tiled MFMA
- * GEMM with in-register dequantization (paired profiles) or dequantize-to-fp16 + MFMA GEMM.  The workspace
- * (size from the query, 0 when none is needed) holds fp16 activations and, for the second case, fp16
- * weights.  Replaces nint_mmq_f16_packed_cuda / nint_mmq_f32_packed_cuda and the dequant + cuBLAS fallback
+/* Decode gate/up projection with the SwiGLU fused: the tensor holds W gate neurons, then W up neurons (out = 2 W,
+ * W a multiple of 16); hidden[m, c] = silu(y[m, c]) * y[m, W + c] as bf16 / fp16 (out_dtype, MFQ_X_*), y as in
+ * mfq_hip_nint_gemv, M = 1 or 2.  Replaces nint_gemv_packed_swiglu_ws_cuda (cpp_runtime/mfq_decode.cpp:393-396).
+ * MFQ_ERR_UNSUPPORTED for M > 2 and for profiles without a unit: run mfq_hip_nint_gemm + mfq_hip_moe_swiglu then. */
+int mfq_hip_nint_gemv_swiglu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
+                             int64_t ldx, int M, void *hidden, int out_dtype, int64_t ldh, mfq_stream_t stream);
+
+/* Any-M entry: the streaming kernels of mfq_hip_nint_gemv up to a crossover that depends on the tensor (32 to
+ * 512 rows; 256 for profiles without a prefill kernel), above that a block-tiled MFMA GEMM with in-register
+ * dequantization (the paired profiles and NINT5-28) or dequantize-to-fp16 + MFMA GEMM.  The workspace (size
+ * from the query, 0 when none is needed) holds fp16 activations, group sums and the partial results of a split
+ * over K, or, for the second case, fp16 activations and weights.  Replaces nint_mmq_f16_packed_cuda / nint_mmq_f32_packed_cuda and the dequant + cuBLAS fallback
  * (cpp_runtime/mfq_decode.cpp:480-520, 8309-8314). */
 size_t mfq_hip_nint_gemm_workspace_bytes(const mfq_nint_desc *d, int M);
 int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,

@@ -124,6 +124,27 @@ def test_gemm_long_k_few_neurons_is_split_over_k(bits, gs, sb):
     assert np.array_equal(y, lin(x).cpu().numpy())   # partial sums are added in a fixed order
 
 
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (4, 24, 6)])
+@pytest.mark.parametrize("W,K", [(48, 280), (64, 9000)])
+def test_gate_up_gemv_with_fused_swiglu(bits, gs, sb, W, K):
+    """silu(gate) * up in the GEMV's epilogue for one and two rows (K = 9000: more than three steps per wave for the
+    16-wide groups, the variant with a prefetch ring); three rows fall back to matmul + SwiGLU."""
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(470 + bits + W)
+    t = O.quantize_nint((rng.standard_normal((2 * W, K)) * 0.02).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    deq = O.dequantize_nint(t)
+    for M in (1, 2, 3):
+        for dtype in (torch.bfloat16, torch.float16):
+            x, xf = _x(rng, M, K, dtype)
+            h = R.nint_matmul_swiglu(lin.weight, x).float().cpu().numpy()
+            y = O.linear_forward_f64(deq, xf)
+            g, u = y[:, :W], y[:, W:]
+            ref = g / (1.0 + np.exp(-g)) * u
+            assert h.shape == (M, W)
+            assert rel_l2(h, ref) < 2e-3, rel_l2(h, ref)   # fp16 output: half an ulp is 5e-4
+
+
 def test_config1_shape_nint3():
     """BASELINE config 1: 4096x4096 N(0, 0.02) NINT3 (3,24,5), bf16 x at batch 1."""
     from tyloquant_amd import runtime as R

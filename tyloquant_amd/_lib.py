@@ -51,6 +51,7 @@ _SIGS = {
     "mfq_hip_nint_repack": (C.c_int, [C.POINTER(NintDesc), vp, i64, C.c_int, vp, vp]),
     "mfq_hip_nint_dequant_f32": (C.c_int, [C.POINTER(NintDesc), vp, vp, i64, vp]),
     "mfq_hip_nint_gemv": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
+    "mfq_hip_nint_gemv_swiglu": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, C.c_int, i64, vp]),
     "mfq_hip_nint_gemm_workspace_bytes": (sz, [C.POINTER(NintDesc), C.c_int]),
     "mfq_hip_nint_gemm": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
     "mfq_hip_nvq_plan": (C.c_int, [C.c_int] * 4 + [C.POINTER(NvqDesc)]),

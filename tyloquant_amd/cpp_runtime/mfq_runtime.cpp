@@ -273,6 +273,18 @@ void nint_matmul(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, i
     w.workspace.ensure(need);
     abi_check(mfq_hip_nint_gemm(&w.desc, w.data.get(), x, x_dtype, ldx, M, y, w.desc.out, w.workspace.get(), need, stream));
 }
+void nint_matmul_swiglu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden, float *scratch,
+                        mfq_stream_t stream) {
+    const int W = w.desc.out / 2;
+    const bool unit = w.desc.kind == 1 || (w.desc.bits == 5 && w.desc.gs == 28);
+    if (M <= 2 && w.desc.out % 32 == 0 && unit) {
+        abi_check(mfq_hip_nint_gemv_swiglu(&w.desc, w.data.get(), x, x_dtype, ldx, M, hidden, MFQ_X_F16, W, stream));
+        return;
+    }
+    if (!scratch) fail("nint_matmul_swiglu: more than two rows need a [M, 2W] fp32 scratch buffer");
+    nint_matmul(w, x, x_dtype, ldx, M, scratch, stream);
+    abi_check(mfq_hip_moe_swiglu(scratch, 2 * W, M, W, hidden, MFQ_X_F16, W, stream));
+}
 void nvq_matmul(const NvqWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) {
     const size_t need = mfq_hip_nvq_gemm_workspace_bytes(&w.desc, M);
     w.workspace.ensure(need);

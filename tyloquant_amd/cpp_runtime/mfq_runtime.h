@@ -122,6 +122,10 @@ struct NepqWeight {
 // y[M, out] (fp32, row stride out) = x[M, K] (x_dtype MFQ_X_BF16 / MFQ_X_F16, row stride ldx) . W^T
 void nint_matmul(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                  mfq_stream_t stream = nullptr);
+// hidden fp16 [M, W] = silu(gate) * up of a [2W, K] gate/up tensor (gate rows first): one fused launch for one or two
+// rows (nint_gemv_packed_swiglu_ws_cuda :393-396), else nint_matmul into `scratch` (fp32 [M, 2W]) + the SwiGLU kernel
+void nint_matmul_swiglu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden,
+                        float *scratch = nullptr, mfq_stream_t stream = nullptr);
 void nvq_matmul(const NvqWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                 mfq_stream_t stream = nullptr);
 void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y,

@@ -512,6 +512,65 @@ extern "C" int mfq_hip_nint_dequant_f32(const mfq_nint_desc *d, const void *weig
     return check_launch("nint_dequant_f32");
 }
 
+template <int XF16, int MB>
+static int launch_gemv_swiglu(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, uint16_t *hidden,
+                              int out_f16, int64_t ldh, hipStream_t st) {
+    // a block takes a gate and an up row-block; its waves split the K steps, at most three (row-block, step) items each
+    // without the prefetch ring
+    const int nwaves = k.nsteps < 16 ? k.nsteps : 16;
+    const int spw = static_cast<int>(ceil_div(k.nsteps, nwaves));
+    const bool ring = 2 * spw > 3;
+    const size_t lds = gemv_lds_bytes(MB, spw, k.gs, nwaves, 2);
+    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nint_gemv_swiglu: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
+    const dim3 grid(static_cast<unsigned>(k.n_rowblocks / 2), static_cast<unsigned>(ceil_div(M, MB))), block(64 * nwaves);
+#define MFQ_SWIGLU(UNIT, B, G)                                                                                        \
+    if (k.bits == B && k.gs == G) {                                                                                   \
+        if (ring)                                                                                                     \
+            hipLaunchKernelGGL((nint_gemv_swiglu_kernel<UNIT<B, G>, XF16, MB, true>), grid, block, lds, st, k, w, x, ldx, M, \
+                               hidden, out_f16, ldh, spw);                                                            \
+        else                                                                                                          \
+            hipLaunchKernelGGL((nint_gemv_swiglu_kernel<UNIT<B, G>, XF16, MB, false>), grid, block, lds, st, k, w, x, ldx, M, \
+                               hidden, out_f16, ldh, spw);                                                            \
+        return check_launch("nint_gemv_swiglu");                                                                      \
+    }
+    if (k.kind == 1) {
+        MFQ_SWIGLU(PairedUnit, 4, 32) MFQ_SWIGLU(PairedUnit, 4, 24) MFQ_SWIGLU(PairedUnit, 4, 16) MFQ_SWIGLU(PairedUnit, 4, 48)
+        MFQ_SWIGLU(PairedUnit, 3, 24) MFQ_SWIGLU(PairedUnit, 2, 16) MFQ_SWIGLU(PairedUnit, 2, 32)
+    } else {
+        MFQ_SWIGLU(GenericUnit, 5, 28)
+    }
+#undef MFQ_SWIGLU
+    return fail(MFQ_ERR_UNSUPPORTED, "nint_gemv_swiglu: no fused kernel for NINT%d-%d", k.bits, k.gs);
+}
+
+extern "C" int mfq_hip_nint_gemv_swiglu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                                        int M, void *hidden, int out_dtype, int64_t ldh, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && hidden, MFQ_ERR_INVALID, "nint_gemv_swiglu: null argument");
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint_gemv_swiglu: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(out_dtype == MFQ_X_BF16 || out_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint_gemv_swiglu: out_dtype=%d", out_dtype);
+    MFQ_REQUIRE(M >= 1 && M <= 2, MFQ_ERR_UNSUPPORTED, "nint_gemv_swiglu: M=%d (the fused kernel takes one or two rows)", M);
+    MFQ_REQUIRE(d->out % 32 == 0, MFQ_ERR_UNSUPPORTED, "nint_gemv_swiglu: %d rows are not two halves of whole row-blocks", d->out);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldh >= d->out / 2, MFQ_ERR_INVALID, "nint_gemv_swiglu: ldx/ldh smaller than the tensor");
+    const NintK k = to_k(d);
+    MFQ_REQUIRE(k.kind == 1 || mfma_generic_profile(k), MFQ_ERR_UNSUPPORTED, "nint_gemv_swiglu: no fused kernel for NINT%d-%d",
+                k.bits, k.gs);
+    MFQ_REQUIRE(static_cast<int64_t>(k.n_rowblocks / 2) * k.rowblock_bytes < (1ll << 31), MFQ_ERR_UNSUPPORTED,
+                "nint_gemv_swiglu: tensor too large for one window");
+    const uint8_t *w = static_cast<const uint8_t *>(weight);
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    uint16_t *h = static_cast<uint16_t *>(hidden);
+    const int f16 = out_dtype == MFQ_X_F16;
+    hipStream_t st = as_stream(stream);
+    // two rows per block while their staged activations fit the LDS, else one row per block
+    const int nwaves = k.nsteps < 16 ? k.nsteps : 16;
+    const bool pair = M == 2 && gemv_lds_bytes(2, static_cast<int>(ceil_div(k.nsteps, nwaves)), k.gs, nwaves, 2) <= 65536;
+    if (x_dtype == MFQ_X_F16)
+        return pair ? launch_gemv_swiglu<1, 2>(k, w, xp, ldx, M, h, f16, ldh, st)
+                    : launch_gemv_swiglu<1, 1>(k, w, xp, ldx, M, h, f16, ldh, st);
+    return pair ? launch_gemv_swiglu<0, 2>(k, w, xp, ldx, M, h, f16, ldh, st)
+                : launch_gemv_swiglu<0, 1>(k, w, xp, ldx, M, h, f16, ldh, st);
+}
+
 extern "C" int mfq_hip_nint_gemv(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
                                  int M, float *y, int64_t ldy, mfq_stream_t stream) {
     MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nint_gemv: null argument");

@@ -416,6 +416,37 @@ __global__ __launch_bounds__(1024) void nint_gemv_natural_kernel(NintK k, const 
     nint_unit_body<GenericUnit<BITS, GS>, XF16, MB, RING>(k, w, blockIdx.x * rbw, rbw, 0, k.out, xr, yr, spw, lds);
 }
 
+// Gate/up GEMV with the SwiGLU fused: the tensor holds the W gate neurons, then the W up neurons.  Block
+// blockIdx.x takes row-block blockIdx.x of each half and stores hidden[m][16 * blockIdx.x + r] = silu(gate) * up
+// as fp16 (out_f16) or bf16.
+template <class U, int XF16, int MB, bool RING>
+__global__ __launch_bounds__(1024) void nint_gemv_swiglu_kernel(NintK k, const uint8_t *__restrict__ w,
+                                                                const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                                uint16_t *__restrict__ hidden, int out_f16, int64_t ldh,
+                                                                int spw) {
+    extern __shared__ uint32_t lds[];
+    const uint16_t *xr[MB];
+    float *yr[MB];
+    dense_rows<MB>(x, ldx, static_cast<float *>(nullptr), 0, M, blockIdx.y * MB, xr, yr);
+    const int half_rb = k.n_rowblocks / 2;
+    nint_unit_body<U, XF16, MB, RING, false>(k, w, blockIdx.x, 2, 0, k.out, xr, yr, spw, lds, half_rb);
+    __syncthreads();
+    const int nwaves = blockDim.x >> 6;
+    const float *red = reinterpret_cast<const float *>(lds + gemv_red_offset(nwaves, MB, spw, U::GROUP));
+    for (int o = threadIdx.x; o < MB * 16; o += blockDim.x) {
+        const int r = o & 15, m = o >> 4;
+        const int row = blockIdx.y * MB + m;
+        if (row >= M) continue;
+        float g = 0.f, u = 0.f;
+        for (int wv = 0; wv < nwaves; ++wv) {
+            g += red[(wv * MB + m) * 16 + r];
+            u += red[((nwaves + wv) * MB + m) * 16 + r];
+        }
+        const float v = g / (1.f + expf(-g)) * u;
+        hidden[static_cast<int64_t>(row) * ldh + blockIdx.x * 16 + r] = out_f16 ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
+    }
+}
+
 template <int XF16, int MB>
 __global__ __launch_bounds__(1024) void nint_gemv_generic_kernel(NintK k, const uint8_t *__restrict__ w,
                                                                  const uint16_t *__restrict__ x, int64_t ldx, int M,

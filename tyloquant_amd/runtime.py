@@ -125,6 +125,23 @@ def nint_matmul(w: NintWeight, x: torch.Tensor, *, force: str | None = None) -> 
     return y.reshape(*x.shape[:-1], w.out)
 
 
+def nint_matmul_swiglu(w: NintWeight, x: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """silu(gate) * up of a [2W, K] gate/up tensor (gate rows first) in one launch for one or two rows
+    (nint_gemv_packed_swiglu_ws_cuda, cpp_runtime/mfq_decode.cpp:393-396); matmul + SwiGLU kernel otherwise."""
+    x2 = _as_2d(x, w.neuron_len)
+    M, W = x2.shape[0], w.out // 2
+    d = w.desc
+    fused = M <= 2 and w.out % 32 == 0 and (d.kind == 1 or (d.bits == 5 and d.gs == 28))
+    if not fused:
+        from .runtime_moe import moe_swiglu
+        return moe_swiglu(nint_matmul(w, x), out_dtype)
+    hidden = torch.empty((M, W), dtype=out_dtype, device=x.device)
+    L.check(L.lib().mfq_hip_nint_gemv_swiglu(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M,
+                                             _ptr(hidden), L.X_F16 if out_dtype == torch.float16 else L.X_BF16, W,
+                                             _stream()))
+    return hidden.reshape(*x.shape[:-1], W)
+
+
 class NintLinearGroup:
     """Projections that share their input (gate/up, Q/K/V) kept as one concatenated NintWeight and run as
     one matmul whose output is split afterwards (cpp_runtime/mfq_decode.cpp:8618-8660)."""
