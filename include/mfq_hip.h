@@ -126,7 +126,10 @@ int mfq_hip_nvq_dequant_f32(const mfq_nvq_desc *d, const void *weight, float *w_
 /* Replaces nvq_gemv_ws_cuda (cpp_runtime/mfq_decode.cpp:555-559). */
 int mfq_hip_nvq_gemv(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
                      int M, float *y, int64_t ldy, mfq_stream_t stream);
-/* Replaces nvq_gemm_f16_cuda / dequant + cuBLAS (cpp_runtime/mfq_decode.cpp:561-575, 7928-7931). */
+/* Any-M entry: the streaming kernels of mfq_hip_nvq_gemv up to a crossover of 32 to 512 rows, above that a
+ * block-tiled MFMA GEMM that builds the weight fragments from the codebooks (neuron_len % 8 == 0), else
+ * dequantize-to-fp16 + MFMA GEMM.  Replaces nvq_mmq_* / nvq_gemm_f16_cuda / dequant + cuBLAS
+ * (cpp_runtime/mfq_decode.cpp:561-575, 7928-7931). */
 size_t mfq_hip_nvq_gemm_workspace_bytes(const mfq_nvq_desc *d, int M);
 int mfq_hip_nvq_gemm(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
                      int M, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
@@ -160,6 +163,9 @@ int mfq_hip_nepq_dequant_f32(const mfq_nepq_desc *d, const void *weight, float *
 /* `row0`, `nrows` select one expert's neurons; replaces nepq_gemv_ws_cuda. */
 int mfq_hip_nepq_gemv(const mfq_nepq_desc *d, const void *weight, int row0, int nrows, const void *x,
                       int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream);
+/* Any-M entry: mfq_hip_nepq_gemv's kernels up to 32 rows, from 33 rows a block-tiled MFMA GEMM that builds the
+ * weight fragments from the ternary tables; replaces nepq_mmq_ws_cuda / nepq_gemm_f16_cuda
+ * (mfq/kernels/cuda/mfq_cuda.cpp:331-350). */
 size_t mfq_hip_nepq_gemm_workspace_bytes(const mfq_nepq_desc *d, int nrows, int M);
 int mfq_hip_nepq_gemm(const mfq_nepq_desc *d, const void *weight, int row0, int nrows, const void *x,
                       int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, void *workspace,
