@@ -25,7 +25,7 @@ extern "C" {
 typedef void *mfq_stream_t; /* a hipStream_t; NULL = the default stream */
 
 enum { MFQ_OK = 0, MFQ_ERR_INVALID = 1, MFQ_ERR_UNSUPPORTED = 2, MFQ_ERR_LAUNCH = 3, MFQ_ERR_WORKSPACE = 4 };
-enum { MFQ_X_BF16 = 0, MFQ_X_F16 = 1 };
+enum { MFQ_X_BF16 = 0, MFQ_X_F16 = 1, MFQ_X_F32 = 2 /* outputs only, where an entry point says so */ };
 
 const char *mfq_hip_last_error(void);
 int mfq_hip_version(void);
@@ -80,6 +80,26 @@ int mfq_hip_nint_gemv(const mfq_nint_desc *d, const void *weight, const void *x,
  * MFQ_ERR_UNSUPPORTED for M > 2 and for profiles without a unit: run mfq_hip_nint_gemm + mfq_hip_moe_swiglu then. */
 int mfq_hip_nint_gemv_swiglu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
                              int64_t ldx, int M, void *hidden, int out_dtype, int64_t ldh, mfq_stream_t stream);
+
+/* Token-embedding rows from the packed table: out[n, 0:neuron_len] = row ids[n] of the dequantized tensor (the
+ * values of mfq_hip_nint_dequant_f32, rounded once more to out_dtype: MFQ_X_BF16, MFQ_X_F16 or MFQ_X_F32); ids
+ * outside [0, out) give a row of zeros.  ids are device int64.  Replaces
+ * nint_embedding_lookup_packed_compact_cuda / nint_embedding_lookup_packed_compact_bits_cuda
+ * (cpp_runtime/mfq_decode.cpp:358-365, called at :13929-13957; kernels mfq/kernels/cuda/embedding.cu:117-187). */
+int mfq_hip_nint_embedding(const mfq_nint_desc *d, const void *weight, const int64_t *ids, int n_ids,
+                           void *out, int out_dtype, int64_t ldo, mfq_stream_t stream);
+
+/* LM head for greedy decoding: token[m] = argmax_n y[m, n] with y as in mfq_hip_nint_gemv (equal logits go to the
+ * lower index, NaN never wins, -1 when every logit is NaN).  M = 1 on NINT4-32, NINT4-24, NINT3-24 and NINT5-28
+ * takes one GEMV launch whose blocks emit their winners, and a one-block final pass; other profiles and M > 1
+ * run the GEMV into the logits and reduce them in two passes.  logits (float [M, ldl]) may be null; when given
+ * it receives y.  token is device int64 [M].  The workspace holds the per-block winners (and the logits when
+ * none are passed).  Replaces nint_gemv_packed_bits_argmax_ws_cuda (cpp_runtime/mfq_decode.cpp:464-468, called
+ * at :14116-14129; reduction mfq/kernels/cuda/nint_matmul.cu:2300-2350). */
+size_t mfq_hip_nint_gemv_argmax_workspace_bytes(const mfq_nint_desc *d, int M);
+int mfq_hip_nint_gemv_argmax(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
+                             int64_t ldx, int M, float *logits, int64_t ldl, int64_t *token,
+                             void *workspace, size_t workspace_bytes, mfq_stream_t stream);
 
 /* Any-M entry: the streaming kernels of mfq_hip_nint_gemv up to a crossover that depends on the tensor (32 to
  * 512 rows; 256 for profiles without a prefill kernel), above that a block-tiled MFMA GEMM with in-register

@@ -22,6 +22,12 @@ int64_t mfq_rt_linear_neuron_len(void *handle);
 /* QuantLinear::forward (cpp_runtime/mfq_decode.cpp:9209-9226): y[M, out] fp32 = x[M, K] . W^T. */
 int mfq_rt_linear_forward(void *handle, const void *x, int x_dtype, int64_t ldx, int M, float *y, void *stream);
 int mfq_rt_linear_dequantize(void *handle, float *out, void *stream);
+/* embed_forward (cpp_runtime/mfq_decode.cpp:13929-13957) on a NINT table: out [n_ids, K] of out_dtype (MFQ_X_*),
+ * ids device int64; and next_token_from_hidden (:14107-14130): token[m] device int64, logits fp32 [M, out] or null.
+ * Both fail on a handle that does not hold a NINT tensor. */
+int mfq_rt_linear_embedding(void *handle, const int64_t *ids, int n_ids, void *out, int out_dtype, void *stream);
+int mfq_rt_linear_argmax(void *handle, const void *x, int x_dtype, int64_t ldx, int M, int64_t *token, float *logits,
+                         void *stream);
 /* run_linear_check (cpp_runtime/mfq_decode.cpp:16510-16638): out6 = production_ms, production_weight_gbps,
  * payload_gbps, production_rel, production_mean_abs, production_max_abs. */
 int mfq_rt_linear_check(void *handle, int M, int reps, double *out6);

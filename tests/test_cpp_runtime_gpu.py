@@ -30,6 +30,9 @@ def rt():
     lib.mfq_rt_free_quant_linear.argtypes = [C.c_void_p]
     lib.mfq_rt_linear_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]
     lib.mfq_rt_linear_dequantize.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.mfq_rt_linear_embedding.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
+    lib.mfq_rt_linear_argmax.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p,
+                                         C.c_void_p]
     lib.mfq_rt_load_nint_moe.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(C.c_void_p)]
     lib.mfq_rt_free_nint_moe.argtypes = [C.c_void_p]
     lib.mfq_rt_moe_ffn_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p,
@@ -91,6 +94,40 @@ def test_cpp_load_quant_linear_and_forward(rt):
         _load(rt, "NINT4", O.pack_nint(t))
     with pytest.raises(RuntimeError, match="unsupported quantized linear dtype"):
         _load(rt, "MXFP4", b"\0" * 64)
+
+
+def test_cpp_embedding_rows_and_argmax_head(rt):
+    """The host library's embed_forward / next_token_from_hidden twins on a NINT5-28 table: rows bit-exact against the
+    oracle's dequantizer, the token equal to the arg-max of the logits the call returns; other families refuse."""
+    rng = np.random.default_rng(14)
+    out, K = 700, 448
+    t = synth.nint_random(rng, out, K, 5, 28, 7)
+    h = _load(rt, "NINT5", O.pack_nint(t))
+    deq = O.dequantize_nint(t)
+    ids = np.array([3, 699, 0, 3, 700, -5], dtype=np.int64)
+    rows = torch.empty((len(ids), K), dtype=torch.float32, device="cuda")
+    assert rt.mfq_rt_linear_embedding(h, torch.from_numpy(ids).cuda().data_ptr(), len(ids), rows.data_ptr(), 2, None) == 0
+    torch.cuda.synchronize()
+    want = np.zeros((len(ids), K), np.float32)
+    want[:4] = deq[ids[:4]]
+    assert np.array_equal(rows.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    for M in (1, 4):
+        x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+        token = torch.empty((M,), dtype=torch.int64, device="cuda")
+        logits = torch.empty((M, out), dtype=torch.float32, device="cuda")
+        assert rt.mfq_rt_linear_argmax(h, x.data_ptr(), 0, K, M, token.data_ptr(), logits.data_ptr(), None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(token, logits.argmax(-1))
+        check_close(logits.cpu().numpy(), O.linear_forward_f64(deq, x.float().cpu().numpy()))
+        alone = torch.empty((M,), dtype=torch.int64, device="cuda")
+        assert rt.mfq_rt_linear_argmax(h, x.data_ptr(), 0, K, M, alone.data_ptr(), None, None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(alone, token)
+    rt.mfq_rt_free_quant_linear(h)
+    hv = _load(rt, "NVQ3J-512", O.pack_nvq_jsc(synth.nvq_jsc_random(rng, 32, 96)))
+    assert rt.mfq_rt_linear_embedding(hv, None, 0, None, 2, None) != 0
+    assert b"NINT" in rt.mfq_rt_last_error()
+    rt.mfq_rt_free_quant_linear(hv)
 
 
 @pytest.mark.parametrize("T", [1, 20])

@@ -11,7 +11,7 @@ from pathlib import Path
 _HERE = Path(__file__).resolve().parent
 LIB_PATH = _HERE / "lib" / "libmfq_hip.so"
 
-X_BF16, X_F16 = 0, 1
+X_BF16, X_F16, X_F32 = 0, 1, 2
 TOPK_SOFTMAX, TOPK_SIGMOID, TOPK_SQRT_SOFTPLUS, TOPK_DELAYED_SOFTMAX = 0, 1, 2, 3
 
 i32, i64, vp, sz = C.c_int32, C.c_int64, C.c_void_p, C.c_size_t
@@ -52,6 +52,9 @@ _SIGS = {
     "mfq_hip_nint_dequant_f32": (C.c_int, [C.POINTER(NintDesc), vp, vp, i64, vp]),
     "mfq_hip_nint_gemv": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
     "mfq_hip_nint_gemv_swiglu": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, C.c_int, i64, vp]),
+    "mfq_hip_nint_embedding": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, vp, C.c_int, i64, vp]),
+    "mfq_hip_nint_gemv_argmax_workspace_bytes": (sz, [C.POINTER(NintDesc), C.c_int]),
+    "mfq_hip_nint_gemv_argmax": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, vp, sz, vp]),
     "mfq_hip_nint_gemm_workspace_bytes": (sz, [C.POINTER(NintDesc), C.c_int]),
     "mfq_hip_nint_gemm": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
     "mfq_hip_nvq_plan": (C.c_int, [C.c_int] * 4 + [C.POINTER(NvqDesc)]),

@@ -285,6 +285,16 @@ void nint_matmul_swiglu(const NintWeight &w, const void *x, int x_dtype, int64_t
     nint_matmul(w, x, x_dtype, ldx, M, scratch, stream);
     abi_check(mfq_hip_moe_swiglu(scratch, 2 * W, M, W, hidden, MFQ_X_F16, W, stream));
 }
+void nint_embedding(const NintWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype, mfq_stream_t stream) {
+    abi_check(mfq_hip_nint_embedding(&w.desc, w.data.get(), ids, n_ids, out, out_dtype, w.desc.neuron_len, stream));
+}
+void nint_matmul_argmax(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, int64_t *token, float *logits,
+                        mfq_stream_t stream) {
+    const size_t need = mfq_hip_nint_gemv_argmax_workspace_bytes(&w.desc, M);
+    w.workspace.ensure(need);
+    abi_check(mfq_hip_nint_gemv_argmax(&w.desc, w.data.get(), x, x_dtype, ldx, M, logits, w.desc.out, token,
+                                       w.workspace.get(), need, stream));
+}
 void nvq_matmul(const NvqWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) {
     const size_t need = mfq_hip_nvq_gemm_workspace_bytes(&w.desc, M);
     w.workspace.ensure(need);
@@ -639,6 +649,20 @@ int mfq_rt_linear_forward(void *h, const void *x, int x_dtype, int64_t ldx, int 
 }
 int mfq_rt_linear_dequantize(void *h, float *out, void *stream) {
     return guard([&] { static_cast<QuantLinear *>(h)->dequantize(out, stream); });
+}
+int mfq_rt_linear_embedding(void *h, const int64_t *ids, int n_ids, void *out, int out_dtype, void *stream) {
+    return guard([&] {
+        const QuantLinear *q = static_cast<QuantLinear *>(h);
+        if (!q->nint) fail("embedding rows need a NINT table");
+        nint_embedding(*q->nint, ids, n_ids, out, out_dtype, stream);
+    });
+}
+int mfq_rt_linear_argmax(void *h, const void *x, int x_dtype, int64_t ldx, int M, int64_t *token, float *logits, void *stream) {
+    return guard([&] {
+        const QuantLinear *q = static_cast<QuantLinear *>(h);
+        if (!q->nint) fail("the arg-max LM head needs a NINT tensor");
+        nint_matmul_argmax(*q->nint, x, x_dtype, ldx, M, token, logits, stream);
+    });
 }
 int mfq_rt_linear_check(void *h, int M, int reps, double *out6) {
     return guard([&] {

@@ -126,6 +126,14 @@ void nint_matmul(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, i
 // rows (nint_gemv_packed_swiglu_ws_cuda :393-396), else nint_matmul into `scratch` (fp32 [M, 2W]) + the SwiGLU kernel
 void nint_matmul_swiglu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden,
                         float *scratch = nullptr, mfq_stream_t stream = nullptr);
+// out [n_ids, K] (out_dtype MFQ_X_BF16 / MFQ_X_F16 / MFQ_X_F32, row stride K) = rows ids[n] (device int64) of the
+// dequantized table, zeros for ids outside it (embed_forward :13929-13957)
+void nint_embedding(const NintWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype,
+                    mfq_stream_t stream = nullptr);
+// token[m] (device int64) = argmax over the neurons of x[m] . W^T, ties to the lower index; logits (fp32 [M, out],
+// may be null) receives the values the arg-max was taken from (next_token_from_hidden :14107-14130)
+void nint_matmul_argmax(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, int64_t *token,
+                        float *logits = nullptr, mfq_stream_t stream = nullptr);
 void nvq_matmul(const NvqWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                 mfq_stream_t stream = nullptr);
 void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y,

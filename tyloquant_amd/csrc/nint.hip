@@ -21,52 +21,6 @@
 
 namespace mfq {
 
-static NintK to_k(const mfq_nint_desc *d) {
-    NintK k;
-    k.bits = d->bits; k.sub_bits = d->sub_bits; k.gs = d->gs; k.out = d->out; k.neuron_len = d->neuron_len;
-    k.ng = d->ng; k.kind = d->kind; k.dwords = d->dwords; k.tail = d->tail_bytes; k.nsteps = d->nsteps;
-    k.n_rowblocks = d->n_rowblocks; k.step_bytes = d->step_bytes; k.rowblock_bytes = d->rowblock_bytes;
-    k.anchors_off = d->anchors_off;
-    return k;
-}
-
-static bool paired_profile(int bits, int gs) {
-    if (bits == 4) return gs == 16 || gs == 24 || gs == 32 || gs == 48;
-    if (bits == 2) return gs == 16 || gs == 32;
-    if (bits == 3) return gs == 24;
-    return false;
-}
-
-// ---- field placement shared by repack and dequant ----------------------------------------
-// Position of weight i inside a paired unit: word index (dwords == tail word) and bit offset;
-// 3-bit weights 22 and 23 are split over spare bits and are handled by the callers.
-__device__ __forceinline__ void paired_pos(int bits, int i, int &word, int &bit) {
-    const int per_half = (bits == 3) ? 5 : 16 / bits;
-    const int per_word = 2 * per_half;
-    word = i / per_word;
-    const int r = i - word * per_word;
-    bit = (r >> 1) * bits + ((r & 1) << 4);
-}
-
-__device__ __forceinline__ uint32_t unit_code(const NintK &k, const uint32_t *q, uint32_t tail, int i) {
-    if (k.kind == 0) {
-        const int bit = i * k.bits;
-        const int w = bit >> 5, sh = bit & 31;
-        uint64_t v = q[w];
-        if (w + 1 < k.dwords) v |= static_cast<uint64_t>(q[w + 1]) << 32;
-        return static_cast<uint32_t>(v >> sh) & ((1u << k.bits) - 1u);
-    }
-    if (k.bits == 3 && i >= 20) {
-        if (i == 20) return tail & 7u;
-        if (i == 21) return (tail >> 3) & 7u;
-        const int h = (i == 23) ? 16 : 0;
-        return ((q[1] >> (15 + h)) & 1u) | (((tail >> (i == 23 ? 7 : 6)) & 1u) << 1) | (((q[0] >> (15 + h)) & 1u) << 2);
-    }
-    int w, b;
-    paired_pos(k.bits, i, w, b);
-    return (q[w] >> b) & ((1u << k.bits) - 1u);
-}
-
 // ---- repack ----------------------------------------------------------------------------
 __global__ void nint_repack_kernel(NintK k, const uint8_t *__restrict__ payload, int64_t payload_bytes, int legacy,
                                    uint8_t *__restrict__ dst) {
@@ -190,10 +144,7 @@ __global__ void nint_dequant_kernel(NintK k, const uint8_t *__restrict__ w, OutT
 // without a prefetch ring holds in registers -- as long as the grid keeps about gemv_target_waves()
 // waves; long neurons spend the items on K (fewer waves to reduce), short ones on row-blocks (the
 // staged activations are reused).  MFQ_GEMV_SPW / MFQ_GEMV_RBW override the choice for tuning.
-// natural-order profiles with a unit of their own (GEMV, streaming and prefill kernels)
-static bool mfma_generic_profile(const NintK &k) { return k.kind == 0 && k.bits == 5 && k.gs == 28; }
-
-static void gemv_shape(const NintK &k, int mb, int &spw, int &nwaves, int &rbw, size_t &lds_bytes) {
+void gemv_shape(const NintK &k, int mb, int &spw, int &nwaves, int &rbw, size_t &lds_bytes) {
     static const int env_spw = [] { const char *e = getenv("MFQ_GEMV_SPW"); return e ? atoi(e) : 0; }();
     static const int env_rbw = [] { const char *e = getenv("MFQ_GEMV_RBW"); return e ? atoi(e) : 0; }();
     const int64_t items = static_cast<int64_t>(k.n_rowblocks) * k.nsteps;

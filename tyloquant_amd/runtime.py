@@ -142,6 +142,36 @@ def nint_matmul_swiglu(w: NintWeight, x: torch.Tensor, out_dtype=torch.float16) 
     return hidden.reshape(*x.shape[:-1], W)
 
 
+def nint_embedding(w: NintWeight, ids: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """Rows ids of the dequantized table as out_dtype, shape ids.shape + [neuron_len]; ids outside the table give
+    zeros (embed_forward, cpp_runtime/mfq_decode.cpp:13929-13957)."""
+    codes = {torch.bfloat16: L.X_BF16, torch.float16: L.X_F16, torch.float32: L.X_F32}
+    if out_dtype not in codes:
+        raise TypeError(f"embedding rows are bfloat16, float16 or float32, got {out_dtype}")
+    flat = ids.to(device=w.data.device, dtype=torch.int64).reshape(-1).contiguous()
+    out = torch.empty((flat.numel(), w.neuron_len), dtype=out_dtype, device=w.data.device)
+    L.check(L.lib().mfq_hip_nint_embedding(C.byref(w.desc), _ptr(w.data), _ptr(flat), flat.numel(), _ptr(out),
+                                           codes[out_dtype], w.neuron_len, _stream()))
+    return out.reshape(*ids.shape, w.neuron_len)
+
+
+def nint_matmul_argmax(w: NintWeight, x: torch.Tensor, return_logits: bool = False):
+    """Greedy next token of an LM head: argmax over the neurons of x . W^T per row of x, int64, ties to the lower
+    index (next_token_from_hidden, cpp_runtime/mfq_decode.cpp:14107-14130).  With return_logits also the fp32
+    logits the arg-max was taken from."""
+    x2 = _as_2d(x, w.neuron_len)
+    M = x2.shape[0]
+    lib = L.lib()
+    need = lib.mfq_hip_nint_gemv_argmax_workspace_bytes(C.byref(w.desc), M)
+    ws = w._ws.get(need, x.device)
+    token = torch.empty((M,), dtype=torch.int64, device=x.device)
+    logits = torch.empty((M, w.out), dtype=torch.float32, device=x.device) if return_logits else None
+    L.check(lib.mfq_hip_nint_gemv_argmax(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M,
+                                         _ptr(logits), w.out, _ptr(token), _ptr(ws), need, _stream()))
+    token = token.reshape(x.shape[:-1])
+    return (token, logits.reshape(*x.shape[:-1], w.out)) if return_logits else token
+
+
 class NintLinearGroup:
     """Projections that share their input (gate/up, Q/K/V) kept as one concatenated NintWeight and run as
     one matmul whose output is split afterwards (cpp_runtime/mfq_decode.cpp:8618-8660)."""
