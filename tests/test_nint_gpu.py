@@ -108,6 +108,26 @@ def test_gemm_many_rows_takes_the_large_tiles(bits, gs, sb, out, M):
     assert np.abs(y - ref).max() < ABS_TOL
 
 
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (4, 24, 6), (4, 16, 6), (4, 48, 6), (3, 24, 5), (2, 16, 5), (2, 32, 5)])
+@pytest.mark.parametrize("out,M", [(1040, 3329), (256, 16500), (512, 300)])
+def test_gemm_tiles_copied_straight_into_lds(bits, gs, sb, out, M):
+    """Profiles whose groups are whole 16-byte chunks copy the activation tiles from global memory straight into a ring
+    of LDS buffers, three sub-steps ahead of the multiply, on all three tile shapes (64 x 384, 128 x 256 -- not for
+    groups of 48, whose four buffers would not fit -- and 64 x 256).  K spans several steps and ends inside one; the
+    result is the same on every run."""
+    rng = np.random.default_rng(570 + bits + gs + out)
+    K = 2056
+    t = O.quantize_nint((rng.standard_normal((out, K)) * 0.02).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    x, xf = _x(rng, M, K)
+    y = lin(x).cpu().numpy()
+    ref = O.linear_forward_f64(O.dequantize_nint(t), xf)
+    assert rel_l2(y, ref) < REL_TOL, rel_l2(y, ref)
+    assert np.abs(y - ref).max() < ABS_TOL
+    for _ in range(3):
+        assert np.array_equal(y, lin(x).cpu().numpy())
+
+
 @pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (5, 28, 7)])
 def test_gemm_long_k_few_neurons_is_split_over_k(bits, gs, sb):
     """A grid of nine 64-token tiles on 256 neurons leaves most CUs idle: the prefill launch is cut along K (four

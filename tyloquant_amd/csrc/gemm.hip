@@ -382,9 +382,17 @@ static bool nint_streams(const mfq_nint_desc *d, int M) {
     return M <= kGemvMaxM || (M <= stream_max && nint_stream_capable(d));
 }
 
+// Row length of the fp16 activations of the prefill kernel: whole 16-group steps (tiles copied straight into LDS never
+// cross a row end), and a multiple of the GEMM's K block.
+static int prefill_kp(const mfq_nint_desc *d) {
+    const int64_t whole = static_cast<int64_t>(d->nsteps) * 16 * d->gs;
+    const int64_t k = whole > d->neuron_len ? whole : d->neuron_len;
+    return static_cast<int>(ceil_div(k, GBK) * GBK);
+}
+
 // prefill workspace: x16 [M, Kp] | xscale [M] | group sums
 static size_t prefill_workspace(const mfq_nint_desc *d, int M) {
-    const size_t Kp = static_cast<size_t>(ceil_div(d->neuron_len, GBK)) * GBK;
+    const size_t Kp = static_cast<size_t>(prefill_kp(d));
     return align256(static_cast<size_t>(M) * Kp * 2) + align256(static_cast<size_t>(M) * 4) +
            align256(nint_prefill_xg_bytes(d, M)) + nint_prefill_split_bytes(d, M);
 }
@@ -408,7 +416,7 @@ extern "C" int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, con
         const size_t need = prefill_workspace(d, M);
         MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nint_gemm: workspace %zu < %zu bytes",
                     workspace_bytes, need);
-        const int Kp = static_cast<int>(ceil_div(d->neuron_len, GBK)) * GBK;
+        const int Kp = prefill_kp(d);
         uint8_t *p = static_cast<uint8_t *>(workspace);
         uint16_t *x16 = reinterpret_cast<uint16_t *>(p);
         p += align256(static_cast<size_t>(M) * Kp * 2);

@@ -320,11 +320,11 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
     const int64_t ystride = static_cast<int64_t>(M) * k.out;
     float *yk = splits > 1 ? part : y;
     const int64_t ldk = splits > 1 ? k.out : ldy;
-#define MFQ_PREFILL_CFG(UNIT, B, G, MT, NB, PF, XD)                                                                 \
+#define MFQ_PREFILL_CFG(UNIT, B, G, MT, NB, PF, XD)                                                            \
     {                                                                                                          \
         const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, 8 * NB)),                                \
                         static_cast<unsigned>(ceil_div(M, MT * 16)), static_cast<unsigned>(splits));           \
-        const size_t lds = prefill_lds_bytes(MT * 16, G);                                                      \
+        const size_t lds = prefill_lds_bytes(MT * 16, G, (XD) == 0 ? 4 : 2);                                   \
         auto kern = nint_prefill_kernel<UNIT<B, G>, MT, NB, 1, 8, PF, XD>;                                     \
         if (lds > 65536) {                                                                                     \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                           \
@@ -350,11 +350,14 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
     const bool wide3 = cost_b < cost_a;
 #define MFQ_PREFILL(UNIT, B, G)                                                                                       \
     if (k.bits == B && k.gs == G) {                                                                                   \
-        if (small) MFQ_PREFILL_CFG(UNIT, B, G, 4, 2, 4, 4)                                                            \
+        /* XD = 0 (groups of whole 16-byte chunks): the activation tiles are copied straight into a ring of four LDS */ \
+        /* buffers, as long as those fit; else they pass through registers, as many tiles in flight as registers allow */ \
+        constexpr bool dma = G % 8 == 0, dma128 = dma && prefill_lds_bytes(128, G, 4) <= 160 * 1024;                  \
+        if (small) MFQ_PREFILL_CFG(UNIT, B, G, 4, 2, 4, (dma ? 0 : 4))                                                \
         if constexpr (UNIT<B, G>::D <= 4) {                                                                           \
-            if (wide3) MFQ_PREFILL_CFG(UNIT, B, G, 4, 3, 4, 2)                                                        \
+            if (wide3) MFQ_PREFILL_CFG(UNIT, B, G, 4, 3, 4, (dma ? 0 : 2))                                            \
         }                                                                                                             \
-        MFQ_PREFILL_CFG(UNIT, B, G, 8, 2, 4, (UNIT<B, G>::D >= 5 ? 1 : 2)) /* wide units: registers for one tile */   \
+        MFQ_PREFILL_CFG(UNIT, B, G, 8, 2, 4, (dma128 ? 0 : (UNIT<B, G>::D >= 5 ? 1 : 2)))                             \
     }
     if (k.kind == 1) {
         MFQ_PREFILL(PairedUnit, 4, 32) MFQ_PREFILL(PairedUnit, 4, 24) MFQ_PREFILL(PairedUnit, 4, 16)

@@ -4,8 +4,9 @@
 // small-batch kernel (nint_mfma.hpp), reads its weight units straight from HBM in the R16 layout, turns
 // each dword of codes into an fp16 fragment (sub_scale * code / 64) with one AND-OR and one packed FMA
 // per pair, and feeds v_mfma_f32_16x16x32_f16.  The activation tile (already fp16, see x_prep) of one
-// sub-step -- the 4 * GS k-values of units j of a step -- is staged in LDS (double-buffered) once per block and
-// shared by the waves; weights never touch LDS.  After the K loop the minimum term sum_g sub_min_g X_g runs as a
+// sub-step -- the 4 * GS k-values of units j of a step -- is staged in LDS once per block and shared by the waves
+// (two buffers filled through registers, or a ring of four filled by direct-to-LDS copies three sub-steps ahead);
+// weights never touch LDS.  After the K loop the minimum term sum_g sub_min_g X_g runs as a
 // short second loop (one MFMA per step and tile against precomputed group sums), then
 //     y = xscale[token] * (64 * neuron_scale * S1 - neuron_min * S2).
 #pragma once
@@ -15,10 +16,10 @@ namespace mfq {
 
 constexpr int kMinSteps = 8;  // steps whose minimum-term operands a block stages at once
 
-// LDS bytes of a block of BM tile rows: two activation buffers of [BM][4 * GS' + 8] halves (GS' = groupsize padded to 8),
+// LDS bytes of a block of BM tile rows: nbuf activation buffers of [BM][4 * GS' + 8] halves (GS' = groupsize padded to 8),
 // reused for the group sums of kMinSteps steps ([BM][kMinSteps * 16 + 4] dwords).
-inline size_t prefill_lds_bytes(int bm, int gs) {
-    const size_t xt = static_cast<size_t>(2 * bm) * (4 * ((gs + 7) / 8 * 8) + 8) * 2;
+constexpr size_t prefill_lds_bytes(int bm, int gs, int nbuf = 2) {
+    const size_t xt = static_cast<size_t>(nbuf * bm) * (4 * ((gs + 7) / 8 * 8) + 8) * 2;
     const size_t mn = static_cast<size_t>(bm) * (kMinSteps * 16 + 4) * 4;
     return xt > mn ? xt : mn;
 }
@@ -26,11 +27,13 @@ inline size_t prefill_lds_bytes(int bm, int gs) {
 // Rows of a block tile: src(i) = row of x16 / xscale / xg that tile row i reads (always valid), dst(i) = row of y it
 // writes or -1.
 struct DenseRows {
+    static constexpr bool kAscending = true;  // src(i) >= src(0)
     int tok0, M;
     __device__ __forceinline__ int src(int i) const { return min(tok0 + i, M - 1); }
     __device__ __forceinline__ int dst(int i) const { return tok0 + i < M ? tok0 + i : -1; }
 };
 struct MappedRows {  // both tables live in LDS
+    static constexpr bool kAscending = false;
     const int *srcv, *dstv;
     __device__ __forceinline__ int src(int i) const { return srcv[i]; }
     __device__ __forceinline__ int dst(int i) const { return dstv[i]; }
@@ -38,8 +41,9 @@ struct MappedRows {  // both tables live in LDS
 
 // One block: tile rows `rows`, neurons of the row-blocks [rb_base, rb_base + (NW / WM) * NB) below rb_end; y column of a
 // neuron = (row-block - rb_col0) * 16 + r, stored when below ncols.  xg: the group sums x_prep leaves,
-// [row][step][kb] x 16 bytes (see gemm.hip).  xt: LDS, prefill_lds_bytes(BM, GS) bytes.
-// PF: register buffers of weight units per row-block; the unit of sub-step it + PF - 1 is requested while sub-step it
+// [row][step][kb] x 16 bytes (see gemm.hip).  xt: LDS, prefill_lds_bytes(BM, GS, XD == 0 ? 4 : 2) bytes.
+// XD: activation tiles in flight in registers, or 0 for direct-to-LDS copies (rows of x16 then hold whole steps:
+// Kp >= 64 * GS * steps).  PF: register buffers of weight units per row-block; the unit of sub-step it + PF - 1 is requested while sub-step it
 // multiplies (2 = ping-pong; 4 keeps a whole step in flight for tiles with few rows, where the weight stream and
 // not the matrix cores sets the pace).
 template <class U, int MT, int NB, int WM, int NW, class Rows, int PF = 2, int XD = (PF == 4 ? 4 : 1)>
@@ -79,8 +83,14 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
         for (int b = 0; b < NB; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // global -> register copy of the activation tile of sub-step `it` (chunk c of a row = 8 halves at k0 + 8 c)
-    static_assert(XD == 1 || XD == 2 || XD == 4, "activation tiles in flight in registers");
-    chunk_t xr[XD][PER_THREAD];
+    // XD = 0: the tiles go from global memory straight into a ring of four LDS buffers (no registers in between),
+    // three sub-steps ahead.  Needs 16-byte chunks (GS % 8 == 0) and Kp >= 64 * GS * steps: every tile lies inside a row.
+    constexpr bool DMA = XD == 0;
+    static_assert(XD == 0 || XD == 1 || XD == 2 || XD == 4, "activation tiles in flight in registers");
+    static_assert(!DMA || (EL == 8 && GSP == GS), "direct-to-LDS tiles are made of 16-byte chunks");
+    static_assert(!DMA || Rows::kAscending, "the copies address the rows relative to the tile's first row");
+    constexpr int XR = DMA ? 1 : XD;
+    chunk_t xr[XR][PER_THREAD];
     // the thread's chunks of a tile: source row (looked up once: a mapped tile keeps its row table in LDS) and k offset
     const uint16_t *xsrc[PER_THREAD];
     int xk[PER_THREAD];
@@ -112,6 +122,47 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
                 *reinterpret_cast<chunk_t *>(xt + buf * (BM * ROW) + row * ROW + g * GSP + EL * ci) = xq[p];
         }
     };
+    // direct-to-LDS copies: chunk c of a tile (16 bytes; row c / CPR, the last chunk of a row is padding and takes a
+    // copy of the one before) lands at byte 16 c of its buffer -- lane l of a wave-wide copy writes 16 l bytes behind
+    // the wave's base, so a thread's chunks are tid, tid + NT, ...  The last round has work for LASTW waves only; the
+    // others repeat it (same bytes to the same place), so that every wave issues the same number of requests.
+    constexpr int CPR = ROW / 8, TILE_CH = BM * CPR, DPER = DMA ? (TILE_CH + NT - 1) / NT : 1;
+    constexpr int LASTW = (TILE_CH - NT * (DPER - 1)) / 64;
+    static_assert(!DMA || TILE_CH % 64 == 0, "whole waves of chunks");
+    uint32_t dsrc[DPER];  // byte offset of the thread's chunk p inside x16 at k = 0
+    int dbase[DPER];      // first chunk of the wave's copy p
+    // buffer-addressed copies (the flat-addressed form makes the compiler wait for all outstanding requests at every
+    // use of a loaded register); the tile rows of a block lie inside 4 GiB from xwin's base
+    __amdgpu_buffer_rsrc_t xwin;
+    if constexpr (DMA) {
+        const int row_lo = rows.src(0);
+        xwin = wave_window(reinterpret_cast<const uint8_t *>(x16 + static_cast<int64_t>(row_lo) * Kp),
+                           static_cast<uint32_t>(min(static_cast<int64_t>(BM) * Kp * 2, static_cast<int64_t>(0xffffffffu))));
+#pragma unroll
+        for (int p = 0; p < DPER; ++p) {
+            dbase[p] = NT * p + (p == DPER - 1 ? wave % LASTW : wave) * 64;
+            const int c = dbase[p] + lane;
+            const int row = c / CPR, cc = min(c - row * CPR, CPR - 2);
+            dsrc[p] = static_cast<uint32_t>((static_cast<int64_t>(rows.src(row) - row_lo) * Kp + 8 * cc) * 2);
+        }
+    }
+    const int it_last = 4 * k.nsteps - 1;  // tiles past the end of K re-read the last one (nobody multiplies them)
+    auto xdma = [&](int it, int buf) {
+        if constexpr (DMA) {
+            const int k0 = min(it, it_last) * 4 * GS;
+#pragma unroll
+            for (int p = 0; p < DPER; ++p) {
+                typedef __attribute__((address_space(3))) void *lds_ptr;
+                uint16_t *dst = xt + buf * (BM * ROW) + dbase[p] * 8;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(xwin, (lds_ptr)dst, 16, dsrc[p], k0 * 2, 0, 0);
+            }
+        }
+    };
+    // Requests of a thread in sub-step j: how many younger requests may
+    // be outstanding when the copies issued two sub-steps earlier must have landed.
+    constexpr int DMIN = DPER;
+    constexpr int WCNT = NB;                                   // weight units
+    constexpr int SCNT = NB * (U::TAIL ? 2 : 1);               // scale (and tail) loads, once per step
     if constexpr (GSP != GS) {  // the padding halves of a group are multiplied by zero weights: keep them finite
         for (int i = tid; i < 2 * BM * ROW / 2; i += NT) reinterpret_cast<uint32_t *>(xt)[i] = 0u;
         __syncthreads();
@@ -136,19 +187,29 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
         }
     };
 
-    xload(4 * s_begin, xr[0]);
+    if constexpr (DMA) {
+#pragma unroll
+        for (int i = 0; i < 3; ++i) xdma(4 * s_begin + i, i);
+    } else {
+        xload(4 * s_begin, xr[0]);
+    }
 #pragma unroll
     for (int i = 0; i < PF - 1; ++i) wload(4 * s_begin + i, qr[i]);
     sload(s_begin, tails, sc);
-    xstore(0, xr[0]);
+    if constexpr (DMA) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
+        xstore(0, xr[0]);
 #pragma unroll
-    for (int i = 1; i < XD; ++i) xload(4 * s_begin + i, xr[i]);
+        for (int i = 1; i < XD; ++i) xload(4 * s_begin + i, xr[i]);
+    }
     __syncthreads();
     for (int s = s_begin; s < s_end; ++s) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int it = 4 * s + j;
-        xload(it + XD, xr[j % XD]);  // past the end: clamped addresses, zeros
+        if constexpr (DMA) xdma(it + 3, (j + 3) & 3);  // the buffer the previous sub-step read
+        else xload(it + XD, xr[j % XR]);                // past the end: clamped addresses, zeros
         wload(it + PF - 1, qr[(j + PF - 1) % PF]);
         if (j == (PF == 4 ? 0 : 3)) sload(s + 1, tailsn, scn);
 
@@ -174,7 +235,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
             u32x4_t af[MT];
 #pragma unroll
             for (int a = 0; a < MT; ++a)
-                af[a] = *reinterpret_cast<const u32x4_t *>(xt + (j & 1) * (BM * ROW) + ((wm * MT + a) * 16 + r) * ROW + kb * GSP + 8 * m);
+                af[a] = *reinterpret_cast<const u32x4_t *>(xt + (DMA ? (j & 3) : (j & 1)) * (BM * ROW) + ((wm * MT + a) * 16 + r) * ROW + kb * GSP + 8 * m);
             // all weight fragments of this k-slice first, then the MFMAs back to back: while one wave's MFMAs run,
             // the other wave of the SIMD unpacks
             u32x4_t bf[NB];
@@ -191,7 +252,17 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
 #pragma unroll
                 for (int a = 0; a < MT; ++a) acc[a][b] = mfma16(af[a], bf[b], acc[a][b]);
         }
-        xstore((j + 1) & 1, xr[(j + 1) % XD]);  // the other buffer: nobody reads it during this sub-step
+        if constexpr (DMA) {
+            // tile it + 1 was requested two sub-steps ago; what this and the previous sub-step requested may still be
+            // in flight (the scale loads of a step belong to sub-step JS)
+            constexpr int JS = PF == 4 ? 0 : 3;
+            constexpr int N0 = 2 * (DMIN + WCNT), N1 = N0 + SCNT;
+            static_assert(N1 < 64, "vmcnt holds six bits");
+            if (j == JS || ((j + 3) & 3) == JS) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N1) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N0) : "memory");
+        } else {
+            xstore((j + 1) & 1, xr[(j + 1) % XR]);  // the other buffer: nobody reads it during this sub-step
+        }
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             if (j == 3) {
@@ -199,10 +270,20 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
                 sc[b] = scn[b];
             }
         }
-        __syncthreads();
+        if constexpr (DMA) {
+            // A bare barrier: the fences of __syncthreads would make every outstanding request land first (copies into
+            // LDS count as stores).  The wait above covers the tile the next sub-step reads; this sub-step's LDS reads
+            // have returned (the MFMAs above consumed them); nothing else in LDS is written in this loop.
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else {
+            __syncthreads();
+        }
       }
     }
 
+    if constexpr (DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // late copies must not land in reused LDS
     // minimum term and epilogue
     const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
     float ns[NB], nm[NB];
