@@ -359,6 +359,11 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
         }                                                                                                             \
         MFQ_PREFILL_CFG(UNIT, B, G, 8, 2, 4, (dma128 ? 0 : (UNIT<B, G>::D >= 5 ? 1 : 2)))                             \
     }
+    static const int env_big = [] { const char *e = getenv("MFQ_PREFILL_BIG"); return e ? atoi(e) : 0; }();
+    if (env_big && k.bits == 4 && k.gs == 32) {
+        if (env_big == 1) MFQ_PREFILL_CFG(PairedUnit, 4, 32, 8, 3, 4, 0)
+        if (env_big == 2) MFQ_PREFILL_CFG(PairedUnit, 4, 32, 8, 3, 2, 0)
+    }
     if (k.kind == 1) {
         MFQ_PREFILL(PairedUnit, 4, 32) MFQ_PREFILL(PairedUnit, 4, 24) MFQ_PREFILL(PairedUnit, 4, 16)
         MFQ_PREFILL(PairedUnit, 4, 48) MFQ_PREFILL(PairedUnit, 3, 24) MFQ_PREFILL(PairedUnit, 2, 16)
