@@ -54,6 +54,28 @@ def test_nvq_matrix_core_path_multi_step(out, K, M):
     _check(nvq_matmul(lin.weight, x, force="gemv").cpu().numpy(), O.linear_forward_f64(want, x.float().cpu().numpy()))
 
 
+@pytest.mark.parametrize("K", [1560, 6160])
+@pytest.mark.parametrize("rpb", [1, 2, 3, 4, 5, 6])
+def test_nvq_signed_table_kernel_row_blocks_per_block(monkeypatch, rpb, K):
+    """Up to 16 rows with the (entry, sign nibble) table in LDS: one block per CU owning rpb row-blocks.  With the CU
+    count the grid is sized for set to 8, 128 * rpb - 5 neurons give every rpb variant (ragged last row-block, last
+    block with fewer row-blocks); K = 1560 is one step per wave (5 waves), K = 6160 two steps per wave with a ragged
+    last group.  One- and two-bank 512-entry codebooks and the 256-entry one."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import nvq_matmul
+    monkeypatch.setenv("MFQ_CU_COUNT", "8")
+    out = 128 * rpb - 5
+    rng = np.random.default_rng(900 + rpb + K)
+    for codebook, banks in (("d4_512", 2), ("d4_512", 1), ("d4_256", 2)):
+        t = synth.nvq_jsc_random(rng, out, K, codebook, banks)
+        dtype, blob = O.pack_tensor(t)
+        lin = R.load_quant_linear(dtype, blob)
+        want = O.dequantize_nvq_jsc(O.unpack_nvq(blob))
+        for M, xd in ((1, torch.bfloat16), (7, torch.float16), (16, torch.bfloat16)):
+            x, xf = _x(rng, M, K, xd)
+            _check(nvq_matmul(lin.weight, x, force="gemv").cpu().numpy(), O.linear_forward_f64(want, xf))
+
+
 @pytest.mark.parametrize("out,K,M,banks", [(130, 1024, 520, 2), (96, 4104, 600, 4), (272, 1024, 8300, 2),
                                           (1040, 1024, 3329, 2)])
 def test_nvq_prefill_kernel(out, K, M, banks):

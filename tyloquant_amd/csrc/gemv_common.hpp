@@ -278,6 +278,14 @@ inline int gemv_target_waves() {
     return v;
 }
 
+// Compute units a one-block-per-CU grid is sized for (MI355X: 256).  MFQ_CU_COUNT overrides it and is read at every
+// call, so that a test can walk the row-blocks-per-block variants on small tensors.
+inline int gemv_cu_count() {
+    const char *e = getenv("MFQ_CU_COUNT");
+    const int n = e ? atoi(e) : 0;
+    return n > 0 ? n : 256;
+}
+
 // LDS bytes of a GEMV block: per wave MB * steps_per_wave * 16 groups * (gs/2 pairs + 2 sums) dwords,
 // plus the cross-wave reduction area of rbw row-blocks.
 inline size_t gemv_lds_bytes(int mb, int spw, int gs, int nwaves, int rbw = 1) {

@@ -1,15 +1,18 @@
 // NVQ-JSC, D4 family (4-dim magnitude vectors, 8/9-bit indices, 7-bit parity sign masks per
 // 8 weights, 4-bit joint scale/codebook state per 24 weights).
 //
-// Device layout: same row-block / step / lane interleave as NINT.  One (neuron, group) unit is
-// 80 bits = two dwords plus one halfword:
-//   d0 = idx0 | idx1 << IB | idx2 << 2IB | (mask2 & 31) << 27
-//   d1 = idx3 | idx4 << IB | idx5 << 2IB | state << 27
-//   h  = mask0 | mask1 << 7 | (mask2 >> 5) << 14
-// Step = Q [j][lane][2 dwords] then H [lane][4 halfwords].  The tensor tail holds
+// Device layout: same row-block / step / lane interleave as NINT.  One (neuron, group) unit is three
+// dwords made of six 16-bit fields F(t) = idx_t << 7 | nib_t << 3, one per 4-dim vector: nib_t is the vector's four
+// sign bits (the parity bit of the 7-bit mask is worked out at load time), so F(t) & 0xfff8 is the byte offset of
+// the vector in a table of (entry, sign nibble) -> four signed fp16 values:
+//   a = F(0) | F(1) << 16
+//   b = F(2) | F(3) << 16
+//   c = F(4) | state >> 3 | (F(5) >> 3) << 16 | (state & 7) << 29      (rotl(c, 6) & 0x78 = 8 * state)
+// Step = Q [j][lane][a, b] then C [lane][c of j = 0..3].  The tensor tail holds
 //   float lut[16]; uint32 bank_for_state[16]; int8 codebooks[banks][entries][4]; float anchor[].
 // In the GEMV the codebook banks (as ready-made activation-typed pairs), a 128-entry table that
-// expands a sign mask (with its parity bit) into XOR masks, and the scale LUT all stay in LDS.
+// expands a sign mask (with its parity bit) into XOR masks, and the scale LUT all stay in LDS; the small-batch
+// matrix-core kernel keeps the signed table (banks * entries * 16 vectors of 8 bytes) in LDS instead.
 #include "common.hpp"
 #include "gemv_common.hpp"
 #include "nint_prefill.hpp"
@@ -50,7 +53,7 @@ __global__ void nvq_repack_kernel(NvqK k, const uint8_t *__restrict__ body, int6
     const uint8_t *sg_s = ix_s + ix_bytes;
     uint8_t *sp = dst + rb * k.rowblock_bytes + s * k.step_bytes;
     uint32_t *qreg = reinterpret_cast<uint32_t *>(sp);
-    uint16_t *hreg = reinterpret_cast<uint16_t *>(sp + 2048);
+    uint32_t *creg = reinterpret_cast<uint32_t *>(sp + 2048);
     for (int j = 0; j < 4; ++j) {
         const int g = 16 * s + 4 * j + kb;
         uint32_t d0 = 0, d1 = 0, h = 0;
@@ -65,13 +68,19 @@ __global__ void nvq_repack_kernel(NvqK k, const uint8_t *__restrict__ body, int6
                 m[t] = u < k.nsign ? read_bits(sg_s, static_cast<int64_t>(row) * k.nsign + u, 7, sg_bytes) : 0u;
             }
             const uint32_t state = read_bits(st_s, static_cast<int64_t>(row) * k.ng + g, 4, st_bytes);
-            d0 = idx[0] | (idx[1] << k.ib) | (idx[2] << (2 * k.ib)) | ((m[2] & 31u) << 27);
-            d1 = idx[3] | (idx[4] << k.ib) | (idx[5] << (2 * k.ib)) | (state << 27);
-            h = m[0] | (m[1] << 7) | ((m[2] >> 5) << 14);
+            uint32_t f[6];
+            for (int t = 0; t < 3; ++t) {
+                const uint32_t m8 = parity8(m[t]);
+                f[2 * t] = (idx[2 * t] << 7) | ((m8 & 15u) << 3);
+                f[2 * t + 1] = (idx[2 * t + 1] << 7) | ((m8 >> 4) << 3);
+            }
+            d0 = f[0] | (f[1] << 16);
+            d1 = f[2] | (f[3] << 16);
+            h = f[4] | (state >> 3) | ((f[5] >> 3) << 16) | ((state & 7u) << 29);
         }
         qreg[(j * 64 + lane) * 2] = d0;
         qreg[(j * 64 + lane) * 2 + 1] = d1;
-        hreg[lane * 4 + j] = static_cast<uint16_t>(h);
+        creg[lane * 4 + j] = h;
     }
     if (s == 0 && kb == 0) {
         float *anchors = reinterpret_cast<float *>(dst + k.anchors_off);
@@ -93,13 +102,14 @@ __global__ void nvq_repack_kernel(NvqK k, const uint8_t *__restrict__ body, int6
 struct NvqUnit {
     uint32_t idx[6], mask[3], state;
 };
-__device__ __forceinline__ NvqUnit nvq_decode(int ib, uint32_t d0, uint32_t d1, uint32_t h) {
+__device__ __forceinline__ NvqUnit nvq_decode(uint32_t a, uint32_t b, uint32_t c) {
     NvqUnit u;
-    const uint32_t im = (1u << ib) - 1u;
-    u.idx[0] = d0 & im; u.idx[1] = (d0 >> ib) & im; u.idx[2] = (d0 >> (2 * ib)) & im;
-    u.idx[3] = d1 & im; u.idx[4] = (d1 >> ib) & im; u.idx[5] = (d1 >> (2 * ib)) & im;
-    u.mask[0] = h & 127u; u.mask[1] = (h >> 7) & 127u; u.mask[2] = ((d0 >> 27) & 31u) | ((h >> 14) << 5);
-    u.state = (d1 >> 27) & 15u;
+    const uint32_t f[6] = {a & 0xffffu, a >> 16, b & 0xffffu, b >> 16, c & 0xffffu, (c >> 13) & 0xfff8u};
+#pragma unroll
+    for (int t = 0; t < 6; ++t) u.idx[t] = f[t] >> 7;
+#pragma unroll
+    for (int m = 0; m < 3; ++m) u.mask[m] = (((f[2 * m] >> 3) & 15u) | (((f[2 * m + 1] >> 3) & 15u) << 4)) & 127u;
+    u.state = (__builtin_rotateleft32(c, 6) >> 3) & 15u;
     return u;
 }
 
@@ -114,7 +124,7 @@ __global__ void nvq_dequant_kernel(NvqK k, const uint8_t *__restrict__ w, OutT *
     if (row >= k.out) return;
     const uint8_t *sp = w + rb * k.rowblock_bytes + s * k.step_bytes;
     const uint32_t *qreg = reinterpret_cast<const uint32_t *>(sp);
-    const uint16_t *hreg = reinterpret_cast<const uint16_t *>(sp + 2048);
+    const uint32_t *creg = reinterpret_cast<const uint32_t *>(sp + 2048);
     const float *lut = reinterpret_cast<const float *>(w + k.tables_off);
     const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
     const int8_t *cb = reinterpret_cast<const int8_t *>(bfs + 16);
@@ -135,7 +145,7 @@ __global__ void nvq_dequant_kernel(NvqK k, const uint8_t *__restrict__ w, OutT *
     for (int j = 0; j < 4; ++j) {
         const int g = 16 * s + 4 * j + kb;
         if (g >= k.ng) continue;
-        const NvqUnit u = nvq_decode(k.ib, qreg[(j * 64 + lane) * 2], qreg[(j * 64 + lane) * 2 + 1], hreg[lane * 4 + j]);
+        const NvqUnit u = nvq_decode(qreg[(j * 64 + lane) * 2], qreg[(j * 64 + lane) * 2 + 1], creg[lane * 4 + j]);
         const float scale = __fmul_rn(anchor, lut[u.state]);
         const int8_t *bank = cb + static_cast<int64_t>(bfs[u.state]) * k.entries * 4;
         for (int i = 0; i < 24; ++i) {
@@ -203,13 +213,14 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
     float *red = reinterpret_cast<float *>(xbase + nwaves * (MB * (npairs + 2 * ngl)));
     const uint8_t *base = w + static_cast<int64_t>(rb) * k.rowblock_bytes;
     struct Step {
-        u32x2_t q[4], hh;
+        u32x2_t q[4];
+        u32x4_t cc;
     };
     auto load_step = [&](int s, Step &st) {
         const uint8_t *sp = base + s * k.step_bytes;
 #pragma unroll
         for (int j = 0; j < 4; ++j) st.q[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp) + j * 64 + lane);
-        st.hh = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(sp + 2048) + lane);
+        st.cc = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(sp + 2048) + lane);
     };
     Step cur, nxt;
     XRegs<MB> xg;
@@ -219,25 +230,22 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
     __syncthreads();  // the LDS tables were filled by the whole block
 
     const int r = lane & 15, kb = lane >> 4;
-    const uint32_t im = (1u << k.ib) - 1u;
     float acc[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) acc[m] = 0.f;
     for (int s = s0; s < s1; ++s) {
         if (s + 1 < s1) load_step(s + 1, nxt);
         const u32x2_t *q = cur.q;
-        const u32x2_t hh = cur.hh;
+        const u32x4_t cc = cur.cc;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int lg = (s - s0) * 16 + 4 * j + kb;
-            const uint32_t d0 = q[j].x, d1 = q[j].y;
-            const uint32_t h = ((j < 2 ? hh.x : hh.y) >> (16 * (j & 1))) & 0xffffu;
-            const uint32_t state = (d1 >> 27) & 15u;
+            const NvqUnit un = nvq_decode(q[j].x, q[j].y, cc[j]);
+            const uint32_t state = un.state;
             const uint32_t *bank = cbp + bankoff[state];
             const float sc = lutf[state];
-            const uint32_t mk[3] = {h & 127u, (h >> 7) & 127u, ((d0 >> 27) & 31u) | ((h >> 14) << 5)};
-            const uint32_t ix[6] = {d0 & im, (d0 >> k.ib) & im, (d0 >> (2 * k.ib)) & im,
-                                    d1 & im, (d1 >> k.ib) & im, (d1 >> (2 * k.ib)) & im};
+            const uint32_t(&mk)[3] = un.mask;
+            const uint32_t(&ix)[6] = un.idx;
             float raw[MB];
 #pragma unroll
             for (int m = 0; m < MB; ++m) raw[m] = 0.f;
@@ -333,18 +341,18 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
     for (int i = 0; i < NB; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
     __syncthreads();  // tables
 
-    const uint32_t ib = static_cast<uint32_t>(k.ib), im = (1u << ib) - 1u;
     if constexpr (NB <= 2) {
         // Software pipeline as in nint_mfma_body: a row-block's four unit buffers are refilled unit by unit for the next
         // step, and the activation fragments run two units ahead and are requested before that refill.
-        u32x2_t q[NB][4], hh[NB], hhn[NB];
+        u32x2_t q[NB][4];
+        u32x4_t hh[NB], hhn[NB];
         auto unit_off = [&](int i, int s, int j) -> uint32_t {
             return i < nrb && s < n ? i * rbb + s * sb + (j * 64 + lane) * 8 : kNoStep;
         };
-        auto hload = [&](int s, u32x2_t (&h)[NB]) {
+        auto hload = [&](int s, u32x4_t (&h)[NB]) {
 #pragma unroll
             for (int i = 0; i < NB; ++i)
-                h[i] = __builtin_amdgcn_raw_buffer_load_b64(win, i < nrb && s < n ? i * rbb + s * sb + 2048 + lane * 8 : kNoStep, 0, 2);
+                h[i] = __builtin_amdgcn_raw_buffer_load_b128(win, i < nrb && s < n ? i * rbb + s * sb + 2048 + lane * 16 : kNoStep, 0, 2);
         };
         auto xfrags = [&](int it, u32x4_t (&dst)[3]) {
             const int kpos = (s0 + (it >> 2)) * 16 * 24 + kb * 24 + 4 * (it & 3) * 24;
@@ -372,15 +380,13 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
                 xfrags(4 * s + j + 2, a2);
 #pragma unroll
                 for (int i = 0; i < NB; ++i) {
-                    const uint32_t d0 = q[i][j].x, d1 = q[i][j].y;
+                    const NvqUnit un = nvq_decode(q[i][j].x, q[i][j].y, hh[i][j]);
                     q[i][j] = __builtin_amdgcn_raw_buffer_load_b64(win, unit_off(i, s + 1, j), 0, 2);
-                    const uint32_t h = ((j < 2 ? hh[i].x : hh[i].y) >> (16 * (j & 1))) & 0xffffu;
-                    const uint32_t state = (d1 >> 27) & 15u;
+                    const uint32_t state = un.state;
                     const uint32_t *bank = cbp + bankoff[state];
                     const half2_t sc = __builtin_bit_cast(half2_t, luth[state]);
-                    const uint32_t mk[3] = {h & 127u, (h >> 7) & 127u, ((d0 >> 27) & 31u) | ((h >> 14) << 5)};
-                    const uint32_t ix[6] = {d0 & im, (d0 >> ib) & im, (d0 >> (2 * ib)) & im,
-                                            d1 & im, (d1 >> ib) & im, (d1 >> (2 * ib)) & im};
+                    const uint32_t(&mk)[3] = un.mask;
+                    const uint32_t(&ix)[6] = un.idx;
 #pragma unroll
                     for (int m = 0; m < 3; ++m) {
                         const u32x4_t sx = *reinterpret_cast<const u32x4_t *>(sgx + 4 * mk[m]);
@@ -399,13 +405,14 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
         }
     } else {  // four row-blocks per wave: the plain loop is faster (measured on 17408x5120)
         for (int s = 0; s < n; ++s) {
-            u32x2_t q[NB][4], hh[NB];
+            u32x2_t q[NB][4];
+            u32x4_t hh[NB];
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
                 const uint32_t off = i < nrb ? i * rbb + s * sb : kNoStep;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) q[i][j] = __builtin_amdgcn_raw_buffer_load_b64(win, off + (j * 64 + lane) * 8, 0, 2);
-                hh[i] = __builtin_amdgcn_raw_buffer_load_b64(win, off + 2048 + lane * 8, 0, 2);
+                hh[i] = __builtin_amdgcn_raw_buffer_load_b128(win, off + 2048 + lane * 16, 0, 2);
             }
             const int kbase = (s0 + s) * 16 * 24 + kb * 24;
 #pragma unroll
@@ -415,14 +422,12 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
                 for (int m = 0; m < 3; ++m) a[m] = load_xfrag<XF16, true>(xrow, kbase + 4 * j * 24 + 8 * m, k.neuron_len);
 #pragma unroll
                 for (int i = 0; i < NB; ++i) {
-                    const uint32_t d0 = q[i][j].x, d1 = q[i][j].y;
-                    const uint32_t h = ((j < 2 ? hh[i].x : hh[i].y) >> (16 * (j & 1))) & 0xffffu;
-                    const uint32_t state = (d1 >> 27) & 15u;
+                    const NvqUnit un = nvq_decode(q[i][j].x, q[i][j].y, hh[i][j]);
+                    const uint32_t state = un.state;
                     const uint32_t *bank = cbp + bankoff[state];
                     const half2_t sc = __builtin_bit_cast(half2_t, luth[state]);
-                    const uint32_t mk[3] = {h & 127u, (h >> 7) & 127u, ((d0 >> 27) & 31u) | ((h >> 14) << 5)};
-                    const uint32_t ix[6] = {d0 & im, (d0 >> ib) & im, (d0 >> (2 * ib)) & im,
-                                            d1 & im, (d1 >> ib) & im, (d1 >> (2 * ib)) & im};
+                    const uint32_t(&mk)[3] = un.mask;
+                    const uint32_t(&ix)[6] = un.idx;
 #pragma unroll
                     for (int m = 0; m < 3; ++m) {
                         const u32x4_t sx = *reinterpret_cast<const u32x4_t *>(sgx + 4 * mk[m]);
@@ -443,6 +448,185 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
 #pragma unroll
         for (int v = 0; v < 4; ++v) red[((wave * NB + i) * 4 + v) * 64 + lane] = anchor[i] * acc[i][v];
     mfma_store_dense<NB>(red, rb0, m0, M, k.out, y, ldy);
+}
+
+// ---- one 16-row tile with the signed table in LDS ------------------------------------------------
+// Up to 16 activation rows, one block per CU: a block owns up to RPB consecutive row-blocks, its waves split the K
+// steps.  The table maps (bank, entry, sign nibble) to the four signed fp16 magnitudes of a vector, so a fragment is
+// two 8-byte LDS reads at byte offsets that sit ready-made in the unit's fields, and one packed multiply per pair by
+// the state's scale; no sign table, no XOR, no index arithmetic.  A wave keeps the activation fragments of its current
+// step in registers (requested before any weights) and walks (step, row-block) items through a ring of RING unit
+// buffers: the only loads inside the walk are weights, each requested RING items before its use, so the waits are
+// for weights alone and the first request wave covers most of a block's share.
+// LDS map (bytes): [signed table: banks*entries*128][state table: 16 x {lut pair, bank base}][red: waves * 1024]
+// [raw codebook entries: banks*entries*4]
+typedef const __attribute__((address_space(3))) u32x2_t *lds_u32x2_ptr;
+template <int XF16, int RPB, int RING, bool ONE>
+__global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k, const uint8_t *__restrict__ w,
+                                                          const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                          float *__restrict__ y, int64_t ldy, int spw) {
+    // item (step ls, row-block i) lives in ring[i % RING]: the ring depth divides the row-blocks of a step
+    static_assert(ONE ? RING <= RPB : RPB % RING == 0, "ring slots are chosen at compile time");
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ncb = k.banks * k.entries;
+    uint32_t *stab = lds + ncb * 32;
+    float *red = reinterpret_cast<float *>(stab + 32);
+    // LDS byte address of the signed table (0 unless something else is placed first)
+    const uint32_t lds_base = static_cast<uint32_t>(
+        reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint32_t *)lds));
+
+    const int rb_first = blockIdx.x * RPB;
+    const int nrb = min(RPB, k.n_rowblocks - rb_first);  // row-blocks of this block
+    const int tok = min(static_cast<int>(lane & 15), M - 1);
+    const uint16_t *xrow = x + static_cast<int64_t>(tok) * ldx;
+    const int r = lane & 15, kb = lane >> 4;
+    const int s0 = wave * spw;
+    const int n = min(k.nsteps, s0 + spw) - s0;  // may be <= 0: the wave only takes part in the barriers
+    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
+    const __amdgpu_buffer_rsrc_t win =
+        wave_window(w + static_cast<int64_t>(rb_first) * k.rowblock_bytes + static_cast<int64_t>(s0) * sb,
+                    n > 0 ? (nrb - 1) * rbb + n * sb : 0u);
+
+    struct Item {
+        u32x2_t q[4];
+        u32x4_t c;
+    };
+    Item ring[RING];
+    auto wload = [&](int ls, int i, Item &it) {  // step s0 + ls of row-block rb_first + i; zeros when there is none
+        const uint32_t off = ls < n && i < nrb ? i * rbb + ls * sb : kNoStep;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) it.q[j] = __builtin_amdgcn_raw_buffer_load_b64(win, off + (j * 64 + lane) * 8, 0, 2);
+        it.c = __builtin_amdgcn_raw_buffer_load_b128(win, off + 2048 + lane * 16, 0, 2);
+    };
+    u32x4_t xf[4][3];
+    auto xload = [&](int ls) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int m = 0; m < 3; ++m)
+                xf[j][m] = load_xfrag_raw<true>(xrow, (s0 + ls) * 16 * 24 + kb * 24 + 4 * j * 24 + 8 * m, k.neuron_len);
+    };
+    auto xfinish = [&](int ls) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int m = 0; m < 3; ++m)
+                xf[j][m] = xfrag_finish<XF16, true>(xf[j][m], (s0 + ls) * 16 * 24 + kb * 24 + 4 * j * 24 + 8 * m, k.neuron_len);
+    };
+    // Everything a wave reads from global memory outside the walk is requested first, in the order of its use, so that
+    // no wait has to cover weight requests issued later (loads return in order): the raw codebook entries (at most
+    // four per thread: blocks have at least four waves), the state tables, the anchors, the activation fragments.
+    const float *lut = reinterpret_cast<const float *>(w + k.tables_off);
+    const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+    const uint32_t *cb = bfs + 16;  // 4 int8 magnitudes per entry
+    uint32_t craw[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) craw[t] = cb[min(tid + t * static_cast<int>(blockDim.x), ncb - 1)];
+    const float lutv = lut[tid & 15];
+    const uint32_t bankv = bfs[tid & 15];
+    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
+
+    // the first RING items: every wave requests its first item before any wave requests its second, so that the first
+    // items of all waves come back first (requests are served roughly in the order the CU issued them)
+    if (n > 0) xload(0);
+#pragma unroll
+    for (int t = 0; t < RING; ++t) {
+        if (n > 0) wload(t / RPB, t % RPB, ring[t]);
+        if (t + 1 < RING) __builtin_amdgcn_s_barrier();
+    }
+    uint32_t *rawcb = reinterpret_cast<uint32_t *>(red + (blockDim.x >> 6) * 256);  // ncb dwords behind the reduction area
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        if (tid + t * static_cast<int>(blockDim.x) < ncb) rawcb[tid + t * blockDim.x] = craw[t];
+    if (tid < 16) {
+        const uint32_t h = f32_to_f16_rne(lutv);  // the LUT is fp16 in the payload: exact
+        stab[2 * tid] = h | (h << 16);
+        stab[2 * tid + 1] = lds_base + bankv * k.entries * 128;
+    }
+    __syncthreads();  // raw entries
+    // chunk c = 16 bytes = the vectors of sign nibbles 2 * (c & 7) and 2 * (c & 7) + 1 of entry c >> 3
+    for (int c = tid; c < ncb * 8; c += blockDim.x) {
+        const uint32_t e = rawcb[c >> 3];
+        uint32_t h[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) h[t] = f32_to_f16_rne(static_cast<float>((e >> (8 * t)) & 0xffu));
+        const uint32_t p0 = h[0] | (h[1] << 16), p1 = h[2] | (h[3] << 16);
+        const uint32_t n0 = 2u * (c & 7), n1 = n0 + 1u;
+        u32x4_t v;
+        v.x = p0 ^ (((n0 & 1u) << 15) | ((n0 & 2u) << 30));
+        v.y = p1 ^ (((n0 & 4u) << 13) | ((n0 & 8u) << 28));
+        v.z = p0 ^ (((n1 & 1u) << 15) | ((n1 & 2u) << 30));
+        v.w = p1 ^ (((n1 & 4u) << 13) | ((n1 & 8u) << 28));
+        *reinterpret_cast<u32x4_t *>(lds + 4 * c) = v;
+    }
+    const uint32_t stab_base = lds_base + ncb * 128;
+    __syncthreads();  // tables
+
+    // one item = the four units of a (step, row-block); its registers are refilled unit by unit, as soon as each is
+    // read, from byte offset noff of the window (kNoStep: nothing left to request)
+    auto process = [&](Item &it, uint32_t noff, bool refill, float4_t &acc) {
+        const u32x4_t uc4 = it.c;
+        if (refill) it.c = __builtin_amdgcn_raw_buffer_load_b128(win, noff + 2048 + lane * 16, 0, 2);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t ua = it.q[j].x, ub = it.q[j].y, uc = uc4[j];
+            if (refill) it.q[j] = __builtin_amdgcn_raw_buffer_load_b64(win, noff + (j * 64 + lane) * 8, 0, 2);
+            const u32x2_t st = *reinterpret_cast<lds_u32x2_ptr>(stab_base + (__builtin_rotateleft32(uc, 6) & 0x78u));
+            const half2_t sc = __builtin_bit_cast(half2_t, st.x);
+            const uint32_t off[6] = {and_or(ua, 0xfff8u, st.y), and_or(ua >> 16, 0xfff8u, st.y),
+                                     and_or(ub, 0xfff8u, st.y), and_or(ub >> 16, 0xfff8u, st.y),
+                                     and_or(uc, 0xfff8u, st.y), and_or(uc >> 13, 0xfff8u, st.y)};
+#pragma unroll
+            for (int m = 0; m < 3; ++m) {
+                const u32x2_t c0 = *reinterpret_cast<lds_u32x2_ptr>(off[2 * m]);
+                const u32x2_t c1 = *reinterpret_cast<lds_u32x2_ptr>(off[2 * m + 1]);
+                const uint32_t wv[4] = {c0.x, c0.y, c1.x, c1.y};
+                u32x4_t b;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) b[t] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, wv[t]) * sc);
+                acc = mfma16(xf[j][m], b, acc);
+            }
+        }
+    };
+    auto store = [&](int i, const float4_t &acc) {  // adds the waves' partial sums of row-block i; block-uniform
+        const float av = anchors[(rb_first + i) * 16 + r];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[(wave * 4 + v) * 64 + lane] = av * acc[v];
+        mfma_store_dense<1>(red, rb_first + i, 0, M, k.out, y, ldy);
+        __syncthreads();
+    };
+    if constexpr (ONE) {  // one step per wave: the ring may have any depth up to RPB
+        float4_t acc[RPB];
+#pragma unroll
+        for (int i = 0; i < RPB; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+        if (n > 0) {
+            xfinish(0);
+#pragma unroll
+            for (int i = 0; i < RPB; ++i)
+                process(ring[i % RING], i + RING < nrb ? (i + RING) * rbb : kNoStep, i + RING < RPB, acc[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < RPB; ++i)
+            if (i < nrb) store(i, acc[i]);
+    } else {
+        float4_t acc[RPB];
+#pragma unroll
+        for (int i = 0; i < RPB; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int ls = 0; ls < n; ++ls) {
+            if (ls > 0) xload(ls);
+            xfinish(ls);
+#pragma unroll
+            for (int i = 0; i < RPB; ++i) {
+                const int nls = ls + (i + RING) / RPB, ni = (i + RING) % RPB;
+                process(ring[i % RING], nls < n && ni < nrb ? ni * rbb + nls * sb : kNoStep, true, acc[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < RPB; ++i)
+            if (i < nrb) store(i, acc[i]);
+    }
 }
 
 // ---- prefill: block-tiled MFMA GEMM, weight fragments built from the codebooks in LDS ----------------------
@@ -539,7 +723,8 @@ __global__ __launch_bounds__(512) void nvq_prefill_kernel(NvqK k, const uint8_t 
             if (c < BM * CHUNKS) *reinterpret_cast<u32x4_t *>(xt + buf * (BM * ROW) + row * ROW + EL * ch) = xq[p];
         }
     };
-    u32x2_t qr[PF][NB], hh[NB], hhn[NB];
+    u32x2_t qr[PF][NB];
+    u32x4_t hh[NB], hhn[NB];
     auto wload = [&](int it, u32x2_t (&qq)[NB]) {
         const int s = it >> 2, j = it & 3;
 #pragma unroll
@@ -547,11 +732,11 @@ __global__ __launch_bounds__(512) void nvq_prefill_kernel(NvqK k, const uint8_t 
             qq[b] = __builtin_amdgcn_raw_buffer_load_b64(
                 win, b < nrb && s < s_end ? b * rbb + s * sb + (j * 64 + lane) * 8 : kNoStep, 0, 0);
     };
-    auto hload = [&](int s, u32x2_t (&h)[NB]) {
+    auto hload = [&](int s, u32x4_t (&h)[NB]) {
 #pragma unroll
         for (int b = 0; b < NB; ++b)
-            h[b] = __builtin_amdgcn_raw_buffer_load_b64(win, b < nrb && s < s_end ? b * rbb + s * sb + 2048 + lane * 8 : kNoStep,
-                                                        0, 0);
+            h[b] = __builtin_amdgcn_raw_buffer_load_b128(win, b < nrb && s < s_end ? b * rbb + s * sb + 2048 + lane * 16 : kNoStep,
+                                                         0, 0);
     };
     xload(4 * s_begin, xr[0]);
 #pragma unroll
@@ -562,7 +747,6 @@ __global__ __launch_bounds__(512) void nvq_prefill_kernel(NvqK k, const uint8_t 
     for (int i = 1; i < XD; ++i) xload(4 * s_begin + i, xr[i]);
     __syncthreads();  // tables and the first tile
 
-    const uint32_t ib = static_cast<uint32_t>(k.ib), im = (1u << ib) - 1u;
     for (int s = s_begin; s < s_end; ++s) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -575,14 +759,14 @@ __global__ __launch_bounds__(512) void nvq_prefill_kernel(NvqK k, const uint8_t 
             uint32_t mk[NB][3], ix[NB][6];
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
-                const uint32_t d0 = qr[j % PF][b].x, d1 = qr[j % PF][b].y;
-                const uint32_t h = ((j < 2 ? hh[b].x : hh[b].y) >> (16 * (j & 1))) & 0xffffu;
-                const uint32_t state = (d1 >> 27) & 15u;
+                const NvqUnit un = nvq_decode(qr[j % PF][b].x, qr[j % PF][b].y, hh[b][j]);
+                const uint32_t state = un.state;
                 bank[b] = cbp + bankoff[state];
                 sc[b] = __builtin_bit_cast(half2_t, luth[state]);
-                mk[b][0] = h & 127u; mk[b][1] = (h >> 7) & 127u; mk[b][2] = ((d0 >> 27) & 31u) | ((h >> 14) << 5);
-                ix[b][0] = d0 & im; ix[b][1] = (d0 >> ib) & im; ix[b][2] = (d0 >> (2 * ib)) & im;
-                ix[b][3] = d1 & im; ix[b][4] = (d1 >> ib) & im; ix[b][5] = (d1 >> (2 * ib)) & im;
+#pragma unroll
+                for (int t = 0; t < 3; ++t) mk[b][t] = un.mask[t];
+#pragma unroll
+                for (int t = 0; t < 6; ++t) ix[b][t] = un.idx[t];
             }
 #pragma unroll
             for (int m = 0; m < NM; ++m) {
@@ -706,11 +890,61 @@ static int nvq_launch_mfma(const NvqK &k, const uint8_t *w, const uint16_t *x, i
     return check_launch("nvq_mfma");
 }
 
+// one 16-row tile through nvq_signed_kernel: at most one block per CU, each with up to six row-blocks
+static int nvq_signed_rpb(const NvqK &k) { return static_cast<int>(ceil_div(k.n_rowblocks, gemv_cu_count())); }
+static bool nvq_signed_capable(const NvqK &k, int M) {
+    static const int off = [] { const char *e = getenv("MFQ_NVQ_SIGNED_OFF"); return e ? atoi(e) : 0; }();
+    const int rpb = nvq_signed_rpb(k);
+    return !off && M <= 16 && static_cast<int64_t>(k.banks) * k.entries * 128 <= 131072 && rpb <= 6 && k.nsteps >= 4 &&
+           rpb * k.rowblock_bytes < (1ll << 31);
+}
+template <int XF16, int RPB, int RING, bool ONE>
+static int nvq_launch_signed_as(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y,
+                                int64_t ldy, hipStream_t st) {
+    const int spw = static_cast<int>(ceil_div(k.nsteps, 16));
+    const int nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
+    const size_t lds = static_cast<size_t>(k.banks) * k.entries * 132 + 128 + static_cast<size_t>(nwaves) * 1024;
+    auto kern = nvq_signed_kernel<XF16, RPB, RING, ONE>;
+    if (lds > 65536) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           static_cast<int>(lds));
+        MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nvq_signed: %s", hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(ceil_div(k.n_rowblocks, RPB))), dim3(64 * nwaves), lds, st, k, w, x,
+                       ldx, M, y, ldy, spw);
+    return check_launch("nvq_signed");
+}
+template <int XF16>
+static int nvq_launch_signed(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                             hipStream_t st) {
+    // ring depths: what fits in 128 registers beside the activation fragments (48) and the accumulators
+    const int rpb = nvq_signed_rpb(k);
+    if (k.nsteps <= 16) {  // one step per wave
+        switch (rpb) {
+        case 1: return nvq_launch_signed_as<XF16, 1, 1, true>(k, w, x, ldx, M, y, ldy, st);
+        case 2: return nvq_launch_signed_as<XF16, 2, 2, true>(k, w, x, ldx, M, y, ldy, st);
+        case 3: return nvq_launch_signed_as<XF16, 3, 3, true>(k, w, x, ldx, M, y, ldy, st);
+        case 4: return nvq_launch_signed_as<XF16, 4, 3, true>(k, w, x, ldx, M, y, ldy, st);
+        case 5: return nvq_launch_signed_as<XF16, 5, 3, true>(k, w, x, ldx, M, y, ldy, st);
+        default: return nvq_launch_signed_as<XF16, 6, 3, true>(k, w, x, ldx, M, y, ldy, st);
+        }
+    }
+    switch (rpb) {
+    case 1: return nvq_launch_signed_as<XF16, 1, 1, false>(k, w, x, ldx, M, y, ldy, st);
+    case 2: return nvq_launch_signed_as<XF16, 2, 2, false>(k, w, x, ldx, M, y, ldy, st);
+    case 3: return nvq_launch_signed_as<XF16, 3, 3, false>(k, w, x, ldx, M, y, ldy, st);
+    case 4: return nvq_launch_signed_as<XF16, 4, 2, false>(k, w, x, ldx, M, y, ldy, st);
+    case 5: return nvq_launch_signed_as<XF16, 5, 1, false>(k, w, x, ldx, M, y, ldy, st);
+    default: return nvq_launch_signed_as<XF16, 6, 1, false>(k, w, x, ldx, M, y, ldy, st);
+    }
+}
+
 template <int XF16>
 static int nvq_mfma_any(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                         hipStream_t st) {
     // two row-blocks per wave (they share the activation fragments) while that leaves about 1000 waves over all 16-row
     // tiles; four were slower on both config 3 shapes (1.2 vs 1.4 TB/s).  MFQ_NVQ_NB overrides for tuning.
+    if (nvq_signed_capable(k, M)) return nvq_launch_signed<XF16>(k, w, x, ldx, M, y, ldy, st);
     const int64_t wpb = (k.nsteps < 8 ? k.nsteps : 8) * ceil_div(M, 16);  // waves of a block x 16-row tiles
     static const int env_nb = [] { const char *e = getenv("MFQ_NVQ_NB"); return e ? atoi(e) : 0; }();
     if (env_nb == 4) return nvq_launch_mfma<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
@@ -790,7 +1024,7 @@ extern "C" int mfq_hip_nvq_plan(int index_bits, int banks, int out, int neuron_l
     d->ngp = static_cast<int32_t>(ceil_div(d->ng, 16) * 16);
     d->nsteps = d->ngp / 16;
     d->n_rowblocks = static_cast<int32_t>(ceil_div(out, 16));
-    d->step_bytes = 2048 + 512;
+    d->step_bytes = 2048 + 1024;
     d->rowblock_bytes = d->step_bytes * d->nsteps;
     d->tables_off = d->rowblock_bytes * d->n_rowblocks;
     d->anchors_off = d->tables_off + 128 + static_cast<int64_t>(banks) * d->entries * 4;
