@@ -26,6 +26,9 @@ typedef void *mfq_stream_t; /* a hipStream_t; NULL = the default stream */
 
 enum { MFQ_OK = 0, MFQ_ERR_INVALID = 1, MFQ_ERR_UNSUPPORTED = 2, MFQ_ERR_LAUNCH = 3, MFQ_ERR_WORKSPACE = 4 };
 enum { MFQ_X_BF16 = 0, MFQ_X_F16 = 1, MFQ_X_F32 = 2 /* outputs only, where an entry point says so */ };
+/* gate activation of a gated linear unit: act(gate) * up with SiLU (SwiGLU) or the tanh form of GELU (GEGLU); the
+ * numbering of mfq_glu_runtime (mfq/kernels/cuda/glu.cuh:18-20) */
+enum { MFQ_GLU_SILU = 0, MFQ_GLU_GELU = 1 };
 
 const char *mfq_hip_last_error(void);
 int mfq_hip_version(void);
@@ -80,6 +83,13 @@ int mfq_hip_nint_gemv(const mfq_nint_desc *d, const void *weight, const void *x,
  * MFQ_ERR_UNSUPPORTED for M > 2 and for profiles without a unit: run mfq_hip_nint_gemm + mfq_hip_moe_swiglu then. */
 int mfq_hip_nint_gemv_swiglu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
                              int64_t ldx, int M, void *hidden, int out_dtype, int64_t ldh, mfq_stream_t stream);
+/* The same with the gate activation chosen by `activation` (MFQ_GLU_*): MFQ_GLU_GELU gives
+ * hidden[m, c] = gelu_tanh(y[m, c]) * y[m, W + c] and replaces nint_gemv_packed_geglu_ws_cuda /
+ * nint_gemv_packed_bits_geglu_ws_cuda (cpp_runtime/mfq_decode.cpp:397-400, 448-451; called by nint_matmul_geglu
+ * :8462-8485).  mfq_hip_nint_gemv_swiglu is this call with MFQ_GLU_SILU. */
+int mfq_hip_nint_gemv_glu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
+                          int64_t ldx, int M, void *hidden, int out_dtype, int64_t ldh, int activation,
+                          mfq_stream_t stream);
 
 /* Token-embedding rows from the packed table: out[n, 0:neuron_len] = row ids[n] of the dequantized tensor (the
  * values of mfq_hip_nint_dequant_f32, rounded once more to out_dtype: MFQ_X_BF16, MFQ_X_F16 or MFQ_X_F32); ids
@@ -256,8 +266,9 @@ int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_pools, const 
 /* Decode form of the grouped matmul (no route map; a handful of tokens): one launch of the batch-1 GEMV over
  * rows p = t * R + r (pair p against expert ids[p]) and, when a shared tensor [out_per_expert, K] is given, rows
  * T * R + t (the shared tensor against token t).  x row of a pair: p with routed_input, else t; of a shared row:
- * T * R + t with routed_input, else t.  swiglu = 0: out is float [rows, ldo].  swiglu != 0: out_per_expert =
- * 2 W, gate rows first, and out is bf16 / fp16 (out_dtype, MFQ_X_*) [rows, ldo] = silu(gate) * up, the fusion
+ * T * R + t with routed_input, else t.  swiglu = 0: out is float [rows, ldo].  swiglu = 1 (SwiGLU) or 2 (GEGLU, the
+ * `gelu` flag of NintMoeWeight::forward_glu_output, cpp_runtime/mfq_decode.cpp:3074-3128): out_per_expert =
+ * 2 W, gate rows first, and out is bf16 / fp16 (out_dtype, MFQ_X_*) [rows, ldo] = act(gate) * up, the fusion
  * of NintMoeWeight::forward_swiglu (cpp_runtime/mfq_decode.cpp:3203-3205) and nint_gemv_packed_swiglu_ws_cuda
  * (cpp_runtime/mfq_decode.cpp:393-396) moved to the producer.  Same values as mfq_hip_moe_grouped_matmul +
  * mfq_hip_moe_swiglu and mfq_hip_nint_gemv on the shared rows, up to the order of the fp32 sums over K.
@@ -274,6 +285,10 @@ int mfq_hip_moe_decode_matmul(const mfq_moe_pool *pools, int n_pools, const int3
  * mfq/kernels/cuda/moe.cu:2980-2996); output fp16 (x_dtype MFQ_X_F16) or bf16. */
 int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,
                        int64_t ldh, mfq_stream_t stream);
+/* The same with the gate activation chosen by `activation` (MFQ_GLU_*); MFQ_GLU_GELU replaces moe_geglu_split_cuda
+ * (cpp_runtime/mfq_decode.cpp:320) and gelu_mul_cuda (mfq/kernels/cuda/activation.cu:69-104). */
+int mfq_hip_moe_glu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,
+                    int64_t ldh, int activation, mfq_stream_t stream);
 /* out[t, :] = sum_r w[t, r] * pair[t, r, :] (+ shared[t, :] when shared != NULL; ungated add,
  * cpp_runtime/mfq_decode.cpp:11077-11080; with gate_logits != NULL: + sigmoid(gate_logits[t]) * shared).
  * Replaces moe_weighted_reduce_cuda / moe_weighted_reduce_shared_gate_cuda. */

@@ -905,6 +905,16 @@ def moe_swiglu(gate_up):
     return ((gate / (1.0 + np.exp(-gate))) * up).astype(np.float32)
 
 
+def moe_geglu(gate_up):
+    """gelu_tanh(gate) * up over [..., 2W] -> [..., W], gate = first half: mfq_glu<true>
+    (mfq/kernels/cuda/glu.cuh:7-12), 0.5 g (1 + tanh(sqrt(2/pi) g (1 + 0.044715 g^2)))."""
+    g = np.asarray(gate_up, dtype=np.float32)
+    W = g.shape[-1] // 2
+    gate, up = g[..., :W].astype(np.float64), g[..., W:].astype(np.float64)
+    gelu = 0.5 * gate * (1.0 + np.tanh(0.79788456080286535587989211986876 * gate * (1.0 + 0.044715 * gate * gate)))
+    return (up * gelu).astype(np.float32)
+
+
 def moe_weighted_reduce(pair, weights):
     """out[t] = sum_r w[t, r] * pair[t, r] in fp32, r ascending (mfq/kernels/cuda/moe.cu:2957-2978)."""
     pair = np.asarray(pair, dtype=np.float32)

@@ -203,6 +203,12 @@ def test_decode_matmul_matches_the_separate_calls(T, H, W):
         want = torch.cat([moe_swiglu(gu(x, route)).reshape(T * k, W), moe_swiglu(R.nint_matmul(sgu, x))])
         close(hid, want, 1e-3)                         # fp16 outputs: half an ulp is 5e-4
         assert torch.all(hid[1] == 0)
+        from tyloquant_amd.runtime_moe import moe_geglu
+        hid_g = gu.forward_decode(x, ids_d, sgu, swiglu="gelu")   # the same launch with the GELU gate
+        want_g = torch.cat([moe_geglu(gu(x, route)).reshape(T * k, W), moe_geglu(R.nint_matmul(sgu, x))])
+        close(hid_g, want_g, 1e-3)
+        gu_np = gu(x, route).reshape(T * k, 2 * W).cpu().numpy()
+        assert rel_l2(moe_geglu(gu(x, route)).reshape(T * k, W).float().cpu().numpy(), O.moe_geglu(gu_np)) < 1e-3
         out = dn.forward_decode(hid, ids_d, sdn, routed=True)
         want = torch.cat([dn(hid[: T * k].reshape(T, k, W), route).reshape(T * k, H), R.nint_matmul(sdn, hid[T * k:])])
         close(out, want, 1e-5)

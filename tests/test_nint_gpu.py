@@ -165,6 +165,28 @@ def test_gate_up_gemv_with_fused_swiglu(bits, gs, sb, W, K):
             assert rel_l2(h, ref) < 2e-3, rel_l2(h, ref)   # fp16 output: half an ulp is 5e-4
 
 
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (5, 28, 7)])
+def test_gate_up_gemv_with_fused_geglu(bits, gs, sb):
+    """gelu_tanh(gate) * up in the same epilogue (one and two rows) and through matmul + the elementwise kernel (three
+    rows); the weights are scaled up so that the gate values cover the curved part of the GELU."""
+    from tyloquant_amd import runtime as R
+    W, K = 64, 1000
+    rng = np.random.default_rng(480 + bits)
+    t = O.quantize_nint((rng.standard_normal((2 * W, K)) * 0.06).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    deq = O.dequantize_nint(t)
+    for M in (1, 2, 3):
+        for dtype in (torch.bfloat16, torch.float16):
+            x, xf = _x(rng, M, K, dtype)
+            h = R.nint_matmul_geglu(lin.weight, x).float().cpu().numpy()
+            y = O.linear_forward_f64(deq, xf)
+            ref = O.moe_geglu(y)
+            assert h.shape == (M, W) and np.abs(y[:, :W]).max() > 2.0
+            assert rel_l2(h, ref) < 2e-3, rel_l2(h, ref)   # fp16 output: half an ulp is 5e-4
+            sw = R.nint_matmul_swiglu(lin.weight, x).float().cpu().numpy()
+            assert rel_l2(sw, O.moe_swiglu(y)) < 2e-3 and rel_l2(sw, h) > 1e-2   # the two activations differ
+
+
 def test_config1_shape_nint3():
     """BASELINE config 1: 4096x4096 N(0, 0.02) NINT3 (3,24,5), bf16 x at batch 1."""
     from tyloquant_amd import runtime as R

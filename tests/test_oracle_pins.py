@@ -321,6 +321,15 @@ def test_moe_reference_loop_and_ffn_pieces():
     gu = rng.standard_normal((3, 8)).astype(np.float32)
     g, u = gu[:, :4].astype(np.float64), gu[:, 4:].astype(np.float64)
     assert np.allclose(O.moe_swiglu(gu), g / (1 + np.exp(-g)) * u, atol=1e-6)
+    # GEGLU: the tanh form against the erf form it approximates (max difference of the two GELUs is below 5e-4 over
+    # the reals), exact zeros, and the large-|g| limits g and 0
+    from math import erf
+    gg = np.linspace(-6.0, 6.0, 241)
+    geglu = O.moe_geglu(np.concatenate([gg, np.ones_like(gg)]).astype(np.float32)[None, :])[0]
+    exact = np.array([0.5 * v * (1.0 + erf(v / np.sqrt(2.0))) for v in gg])
+    assert np.abs(geglu - exact).max() < 5e-4 and geglu[120] == 0.0
+    assert abs(geglu[-1] - 6.0) < 1e-6 and abs(geglu[0]) < 1e-6
+    assert np.allclose(O.moe_geglu(np.array([[1.0, 3.0]], np.float32)), 3.0 * 0.8411919906082768, atol=1e-6)
     w = rng.random((4, 2)).astype(np.float32)
     assert np.allclose(O.moe_weighted_reduce(out, w), (out * w[..., None]).sum(1), atol=1e-5)
 

@@ -13,6 +13,7 @@ LIB_PATH = _HERE / "lib" / "libmfq_hip.so"
 
 X_BF16, X_F16, X_F32 = 0, 1, 2
 TOPK_SOFTMAX, TOPK_SIGMOID, TOPK_SQRT_SOFTPLUS, TOPK_DELAYED_SOFTMAX = 0, 1, 2, 3
+GLU_SILU, GLU_GELU = 0, 1
 
 i32, i64, vp, sz = C.c_int32, C.c_int64, C.c_void_p, C.c_size_t
 
@@ -52,6 +53,7 @@ _SIGS = {
     "mfq_hip_nint_dequant_f32": (C.c_int, [C.POINTER(NintDesc), vp, vp, i64, vp]),
     "mfq_hip_nint_gemv": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
     "mfq_hip_nint_gemv_swiglu": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, C.c_int, i64, vp]),
+    "mfq_hip_nint_gemv_glu": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, C.c_int, i64, C.c_int, vp]),
     "mfq_hip_nint_embedding": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, vp, C.c_int, i64, vp]),
     "mfq_hip_nint_gemv_argmax_workspace_bytes": (sz, [C.POINTER(NintDesc), C.c_int]),
     "mfq_hip_nint_gemv_argmax": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, vp, sz, vp]),
@@ -86,6 +88,7 @@ _SIGS = {
     "mfq_hip_moe_decode_matmul": (C.c_int, [C.POINTER(MoePool), C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, vp, C.c_int,
                                             i64, C.c_int, vp, C.c_int, C.c_int, vp, vp, C.c_int, vp, C.c_int, i64, vp]),
     "mfq_hip_moe_swiglu": (C.c_int, [vp, i64, C.c_int, C.c_int, vp, C.c_int, i64, vp]),
+    "mfq_hip_moe_glu": (C.c_int, [vp, i64, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp]),
     "mfq_hip_moe_weighted_reduce": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]),
     "mfq_hip_gemm_f16_nt": (C.c_int, [vp, i64, vp, i64, C.c_int, C.c_int, C.c_int, vp, i64, vp]),
 }

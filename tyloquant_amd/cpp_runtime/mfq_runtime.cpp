@@ -273,17 +273,25 @@ void nint_matmul(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, i
     w.workspace.ensure(need);
     abi_check(mfq_hip_nint_gemm(&w.desc, w.data.get(), x, x_dtype, ldx, M, y, w.desc.out, w.workspace.get(), need, stream));
 }
-void nint_matmul_swiglu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden, float *scratch,
-                        mfq_stream_t stream) {
+static void nint_matmul_glu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden, float *scratch,
+                            int activation, const char *what, mfq_stream_t stream) {
     const int W = w.desc.out / 2;
     const bool unit = w.desc.kind == 1 || (w.desc.bits == 5 && w.desc.gs == 28);
     if (M <= 2 && w.desc.out % 32 == 0 && unit) {
-        abi_check(mfq_hip_nint_gemv_swiglu(&w.desc, w.data.get(), x, x_dtype, ldx, M, hidden, MFQ_X_F16, W, stream));
+        abi_check(mfq_hip_nint_gemv_glu(&w.desc, w.data.get(), x, x_dtype, ldx, M, hidden, MFQ_X_F16, W, activation, stream));
         return;
     }
-    if (!scratch) fail("nint_matmul_swiglu: more than two rows need a [M, 2W] fp32 scratch buffer");
+    if (!scratch) fail(std::string(what) + ": more than two rows need a [M, 2W] fp32 scratch buffer");
     nint_matmul(w, x, x_dtype, ldx, M, scratch, stream);
-    abi_check(mfq_hip_moe_swiglu(scratch, 2 * W, M, W, hidden, MFQ_X_F16, W, stream));
+    abi_check(mfq_hip_moe_glu(scratch, 2 * W, M, W, hidden, MFQ_X_F16, W, activation, stream));
+}
+void nint_matmul_swiglu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden, float *scratch,
+                        mfq_stream_t stream) {
+    nint_matmul_glu(w, x, x_dtype, ldx, M, hidden, scratch, MFQ_GLU_SILU, "nint_matmul_swiglu", stream);
+}
+void nint_matmul_geglu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden, float *scratch,
+                       mfq_stream_t stream) {
+    nint_matmul_glu(w, x, x_dtype, ldx, M, hidden, scratch, MFQ_GLU_GELU, "nint_matmul_geglu", stream);
 }
 void nint_embedding(const NintWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype, mfq_stream_t stream) {
     abi_check(mfq_hip_nint_embedding(&w.desc, w.data.get(), ids, n_ids, out, out_dtype, w.desc.neuron_len, stream));

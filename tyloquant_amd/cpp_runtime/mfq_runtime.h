@@ -126,6 +126,9 @@ void nint_matmul(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, i
 // rows (nint_gemv_packed_swiglu_ws_cuda :393-396), else nint_matmul into `scratch` (fp32 [M, 2W]) + the SwiGLU kernel
 void nint_matmul_swiglu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden,
                         float *scratch = nullptr, mfq_stream_t stream = nullptr);
+// the same with gelu_tanh(gate) * up (nint_matmul_geglu :8462-8485)
+void nint_matmul_geglu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden,
+                       float *scratch = nullptr, mfq_stream_t stream = nullptr);
 // out [n_ids, K] (out_dtype MFQ_X_BF16 / MFQ_X_F16 / MFQ_X_F32, row stride K) = rows ids[n] (device int64) of the
 // dequantized table, zeros for ids outside it (embed_forward :13929-13957)
 void nint_embedding(const NintWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype,

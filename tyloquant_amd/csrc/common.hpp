@@ -57,6 +57,17 @@ __device__ __forceinline__ float x_to_f32(uint16_t v) {
     if constexpr (XF16) return f16_to_f32(v);
     else return bf16_to_f32(v);
 }
+// Gated-linear-unit value act(gate) * up of the reference's mfq_glu (mfq/kernels/cuda/glu.cuh:5-16): SiLU, or the
+// tanh form of GELU when `gelu` is set.  Kernels carry the choice in bit 1 of their 16-bit output mode
+// (bit 0: fp16 rather than bf16).
+__device__ __forceinline__ float glu_value(float gate, float up, bool gelu) {
+    if (gelu) {
+        const float t = tanhf(0.79788456080286535587989211986876f * gate * (1.0f + 0.044715f * gate * gate));
+        return up * (0.5f * gate * (1.0f + t));
+    }
+    return gate / (1.f + expf(-gate)) * up;
+}
+
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
     uint32_t u = __float_as_uint(f);
     if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40);

@@ -385,7 +385,7 @@ __global__ __launch_bounds__(512) void moe_grouped_kernel(MoePools P, const int3
 // the row's cohort.  Rows below n_pairs are (token, route) pairs; row n_pairs + t applies the shared tensor
 // (cohort slot P.n) to token t.  P.spw: steps per wave of each cohort; RING = false when no wave has more than
 // three (row-block, step) items.  SWIGLU: the block takes row-block blockIdx.x of the gate half and of the up half
-// of the expert and stores silu(gate) * up as 16-bit values, out_f16 selecting fp16 over bf16.
+// of the expert and stores act(gate) * up as 16-bit values: bit 0 of out_f16 selects fp16 over bf16, bit 1 GELU over SiLU.
 template <int XF16, bool RING, bool SWIGLU>
 __global__ __launch_bounds__(1024) void moe_decode_kernel(MoePools P, int rbw, const int32_t *__restrict__ expert_pool,
                                                           const int32_t *__restrict__ expert_local, int E,
@@ -447,8 +447,8 @@ __global__ __launch_bounds__(1024) void moe_decode_kernel(MoePools P, int rbw, c
                 g += red[wv * 16 + threadIdx.x];
                 u += red[(nwaves + wv) * 16 + threadIdx.x];
             }
-            const float v = g / (1.f + expf(-g)) * u;
-            static_cast<uint16_t *>(out)[row * ldo + rbl0 * 16 + threadIdx.x] = out_f16 ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
+            const float v = glu_value(g, u, out_f16 & 2);
+            static_cast<uint16_t *>(out)[row * ldo + rbl0 * 16 + threadIdx.x] = (out_f16 & 1) ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
         }
     }
 }
@@ -601,12 +601,12 @@ __global__ void moe_zero_invalid_kernel(const int32_t *__restrict__ ids, int n_p
 
 template <int F16OUT>
 __global__ __launch_bounds__(256) void moe_swiglu_kernel(const float *__restrict__ gu, int64_t ld, int rows, int W,
-                                                         uint16_t *__restrict__ hidden, int64_t ldh) {
+                                                         uint16_t *__restrict__ hidden, int64_t ldh, int gelu) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= static_cast<int64_t>(rows) * W) return;
     const int row = static_cast<int>(idx / W), col = static_cast<int>(idx - static_cast<int64_t>(row) * W);
     const float g = gu[row * ld + col], u = gu[row * ld + W + col];
-    const float v = g / (1.f + expf(-g)) * u;
+    const float v = glu_value(g, u, gelu != 0);
     hidden[row * ldh + col] = F16OUT ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
 }
 
@@ -934,6 +934,7 @@ extern "C" int mfq_hip_moe_decode_matmul(const mfq_moe_pool *pools, int n_pools,
     MFQ_REQUIRE(pools && expert_pool && expert_local && x && ids && out, MFQ_ERR_INVALID, "moe_decode_matmul: null argument");
     MFQ_REQUIRE(T > 0 && R > 0 && E > 0, MFQ_ERR_INVALID, "MoE ids must be int32 [tokens, routes]");
     MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "moe_decode_matmul: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(swiglu >= 0 && swiglu <= 2, MFQ_ERR_INVALID, "moe_decode_matmul: swiglu=%d (0 none, 1 SwiGLU, 2 GEGLU)", swiglu);
     MFQ_REQUIRE(!swiglu || out_dtype == MFQ_X_BF16 || out_dtype == MFQ_X_F16, MFQ_ERR_INVALID,
                 "moe_decode_matmul: the fused SwiGLU stores bf16 or fp16, out_dtype=%d", out_dtype);
     MFQ_REQUIRE((shared_desc == nullptr) == (shared_weight == nullptr), MFQ_ERR_INVALID,
@@ -967,23 +968,29 @@ extern "C" int mfq_hip_moe_decode_matmul(const mfq_moe_pool *pools, int n_pools,
     const int n_pairs = T * R, n_rows = n_pairs + (shared_desc ? T : 0);
     const int rc = moe_decode_launch(P, n_slots, max_steps, expert_pool, expert_local, E, out_per_expert,
                                      static_cast<const uint16_t *>(x), x_dtype, ldx, routed_input, ids, n_pairs, n_rows, R,
-                                     swiglu, out, out_dtype == MFQ_X_F16, ldo, as_stream(stream));
+                                     swiglu, out, (out_dtype == MFQ_X_F16 ? 1 : 0) | (swiglu == 2 ? 2 : 0), ldo, as_stream(stream));
     if (rc < 0) return fail(MFQ_ERR_UNSUPPORTED, "moe_decode_matmul: shape outside the batch-1 kernel (rows %d, K %d)", n_rows, K);
     return rc;
 }
 
-extern "C" int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,
-                                  int64_t ldh, mfq_stream_t stream) {
-    MFQ_REQUIRE(gate_up && hidden, MFQ_ERR_INVALID, "moe_swiglu: null argument");
-    MFQ_REQUIRE(rows > 0 && W > 0 && ld >= 2 * W && ldh >= W, MFQ_ERR_INVALID, "moe_swiglu: bad shape");
+extern "C" int mfq_hip_moe_glu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype, int64_t ldh,
+                               int activation, mfq_stream_t stream) {
+    MFQ_REQUIRE(gate_up && hidden, MFQ_ERR_INVALID, "moe_glu: null argument");
+    MFQ_REQUIRE(rows > 0 && W > 0 && ld >= 2 * W && ldh >= W, MFQ_ERR_INVALID, "moe_glu: bad shape");
+    MFQ_REQUIRE(activation == MFQ_GLU_SILU || activation == MFQ_GLU_GELU, MFQ_ERR_INVALID, "moe_glu: activation=%d", activation);
     const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<int64_t>(rows) * W, 256));
     if (out_dtype == MFQ_X_F16)
         hipLaunchKernelGGL((moe_swiglu_kernel<1>), dim3(blocks), dim3(256), 0, as_stream(stream), gate_up, ld, rows, W,
-                           static_cast<uint16_t *>(hidden), ldh);
+                           static_cast<uint16_t *>(hidden), ldh, activation);
     else
         hipLaunchKernelGGL((moe_swiglu_kernel<0>), dim3(blocks), dim3(256), 0, as_stream(stream), gate_up, ld, rows, W,
-                           static_cast<uint16_t *>(hidden), ldh);
-    return check_launch("moe_swiglu");
+                           static_cast<uint16_t *>(hidden), ldh, activation);
+    return check_launch("moe_glu");
+}
+
+extern "C" int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,
+                                  int64_t ldh, mfq_stream_t stream) {
+    return mfq_hip_moe_glu(gate_up, ld, rows, W, hidden, out_dtype, ldh, MFQ_GLU_SILU, stream);
 }
 
 extern "C" int mfq_hip_moe_weighted_reduce(const float *pair, const float *weights, int T, int R, int H,

@@ -502,9 +502,10 @@ static int launch_gemv_swiglu(const NintK &k, const uint8_t *w, const uint16_t *
     return fail(MFQ_ERR_UNSUPPORTED, "nint_gemv_swiglu: no fused kernel for NINT%d-%d", k.bits, k.gs);
 }
 
-extern "C" int mfq_hip_nint_gemv_swiglu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
-                                        int M, void *hidden, int out_dtype, int64_t ldh, mfq_stream_t stream) {
+extern "C" int mfq_hip_nint_gemv_glu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                                     int M, void *hidden, int out_dtype, int64_t ldh, int activation, mfq_stream_t stream) {
     MFQ_REQUIRE(d && weight && x && hidden, MFQ_ERR_INVALID, "nint_gemv_swiglu: null argument");
+    MFQ_REQUIRE(activation == MFQ_GLU_SILU || activation == MFQ_GLU_GELU, MFQ_ERR_INVALID, "nint_gemv_glu: activation=%d", activation);
     MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint_gemv_swiglu: x_dtype=%d", x_dtype);
     MFQ_REQUIRE(out_dtype == MFQ_X_BF16 || out_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint_gemv_swiglu: out_dtype=%d", out_dtype);
     MFQ_REQUIRE(M >= 1 && M <= 2, MFQ_ERR_UNSUPPORTED, "nint_gemv_swiglu: M=%d (the fused kernel takes one or two rows)", M);
@@ -518,7 +519,7 @@ extern "C" int mfq_hip_nint_gemv_swiglu(const mfq_nint_desc *d, const void *weig
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
     uint16_t *h = static_cast<uint16_t *>(hidden);
-    const int f16 = out_dtype == MFQ_X_F16;
+    const int f16 = (out_dtype == MFQ_X_F16 ? 1 : 0) | (activation == MFQ_GLU_GELU ? 2 : 0);  // the kernel's output mode
     hipStream_t st = as_stream(stream);
     // two rows per block while their staged activations fit the LDS, else one row per block
     const int nwaves = k.nsteps < 16 ? k.nsteps : 16;
@@ -528,6 +529,11 @@ extern "C" int mfq_hip_nint_gemv_swiglu(const mfq_nint_desc *d, const void *weig
                     : launch_gemv_swiglu<1, 1>(k, w, xp, ldx, M, h, f16, ldh, st);
     return pair ? launch_gemv_swiglu<0, 2>(k, w, xp, ldx, M, h, f16, ldh, st)
                 : launch_gemv_swiglu<0, 1>(k, w, xp, ldx, M, h, f16, ldh, st);
+}
+
+extern "C" int mfq_hip_nint_gemv_swiglu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                                        int M, void *hidden, int out_dtype, int64_t ldh, mfq_stream_t stream) {
+    return mfq_hip_nint_gemv_glu(d, weight, x, x_dtype, ldx, M, hidden, out_dtype, ldh, MFQ_GLU_SILU, stream);
 }
 
 extern "C" int mfq_hip_nint_gemv(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,

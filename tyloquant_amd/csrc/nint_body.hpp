@@ -466,8 +466,8 @@ __global__ __launch_bounds__(1024) void nint_gemv_natural_kernel(NintK k, const 
 }
 
 // Gate/up GEMV with the SwiGLU fused: the tensor holds the W gate neurons, then the W up neurons.  Block
-// blockIdx.x takes row-block blockIdx.x of each half and stores hidden[m][16 * blockIdx.x + r] = silu(gate) * up
-// as fp16 (out_f16) or bf16.
+// blockIdx.x takes row-block blockIdx.x of each half and stores hidden[m][16 * blockIdx.x + r] = act(gate) * up
+// as fp16 (bit 0 of out_f16) or bf16, act = SiLU or (bit 1 of out_f16) GELU.
 template <class U, int XF16, int MB, bool RING>
 __global__ __launch_bounds__(1024) void nint_gemv_swiglu_kernel(NintK k, const uint8_t *__restrict__ w,
                                                                 const uint16_t *__restrict__ x, int64_t ldx, int M,
@@ -491,8 +491,8 @@ __global__ __launch_bounds__(1024) void nint_gemv_swiglu_kernel(NintK k, const u
             g += red[(wv * MB + m) * 16 + r];
             u += red[((nwaves + wv) * MB + m) * 16 + r];
         }
-        const float v = g / (1.f + expf(-g)) * u;
-        hidden[static_cast<int64_t>(row) * ldh + blockIdx.x * 16 + r] = out_f16 ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
+        const float v = glu_value(g, u, out_f16 & 2);
+        hidden[static_cast<int64_t>(row) * ldh + blockIdx.x * 16 + r] = (out_f16 & 1) ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
     }
 }
 

@@ -125,21 +125,31 @@ def nint_matmul(w: NintWeight, x: torch.Tensor, *, force: str | None = None) -> 
     return y.reshape(*x.shape[:-1], w.out)
 
 
-def nint_matmul_swiglu(w: NintWeight, x: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
-    """silu(gate) * up of a [2W, K] gate/up tensor (gate rows first) in one launch for one or two rows
-    (nint_gemv_packed_swiglu_ws_cuda, cpp_runtime/mfq_decode.cpp:393-396); matmul + SwiGLU kernel otherwise."""
+def _nint_matmul_glu(w: NintWeight, x: torch.Tensor, out_dtype, activation: int) -> torch.Tensor:
     x2 = _as_2d(x, w.neuron_len)
     M, W = x2.shape[0], w.out // 2
     d = w.desc
     fused = M <= 2 and w.out % 32 == 0 and (d.kind == 1 or (d.bits == 5 and d.gs == 28))
     if not fused:
-        from .runtime_moe import moe_swiglu
-        return moe_swiglu(nint_matmul(w, x), out_dtype)
+        from .runtime_moe import moe_glu
+        return moe_glu(nint_matmul(w, x), out_dtype, activation)
     hidden = torch.empty((M, W), dtype=out_dtype, device=x.device)
-    L.check(L.lib().mfq_hip_nint_gemv_swiglu(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M,
-                                             _ptr(hidden), L.X_F16 if out_dtype == torch.float16 else L.X_BF16, W,
-                                             _stream()))
+    L.check(L.lib().mfq_hip_nint_gemv_glu(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M,
+                                          _ptr(hidden), L.X_F16 if out_dtype == torch.float16 else L.X_BF16, W,
+                                          activation, _stream()))
     return hidden.reshape(*x.shape[:-1], W)
+
+
+def nint_matmul_swiglu(w: NintWeight, x: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """silu(gate) * up of a [2W, K] gate/up tensor (gate rows first) in one launch for one or two rows
+    (nint_gemv_packed_swiglu_ws_cuda, cpp_runtime/mfq_decode.cpp:393-396); matmul + SwiGLU kernel otherwise."""
+    return _nint_matmul_glu(w, x, out_dtype, L.GLU_SILU)
+
+
+def nint_matmul_geglu(w: NintWeight, x: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """gelu_tanh(gate) * up of a [2W, K] gate/up tensor, as nint_matmul_swiglu (nint_matmul_geglu,
+    cpp_runtime/mfq_decode.cpp:8462-8485; the reference fuses it for one row, here for one or two)."""
+    return _nint_matmul_glu(w, x, out_dtype, L.GLU_GELU)
 
 
 def nint_embedding(w: NintWeight, ids: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:

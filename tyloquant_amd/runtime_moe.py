@@ -187,7 +187,9 @@ class NintMoeWeight:
                        routed=False, out_dtype=torch.float16) -> torch.Tensor:
         """One launch for a decode step: rows t * R + r are the routed pairs, rows T * R + t the shared tensor on
         token t.  x is [T, K], or with `routed` [T * R (+ T), K] with one row per output row.  Returns fp32
-        [rows, out_per_expert], or with `swiglu` 16-bit [rows, out_per_expert / 2] = silu(gate) * up."""
+        [rows, out_per_expert], or with `swiglu` 16-bit [rows, out_per_expert / 2] = silu(gate) * up (swiglu = 2 or
+        "gelu": gelu_tanh(gate) * up, the `gelu` flag of forward_glu_output, cpp_runtime/mfq_decode.cpp:3074-3128)."""
+        swiglu = 2 if swiglu == "gelu" else int(swiglu)
         T, R = ids.shape
         rows = T * R + (T if shared is not None else 0)
         if x.dim() != 2 or x.shape[1] != self.neuron_len or x.shape[0] != (rows if routed else T):
@@ -204,14 +206,25 @@ class NintMoeWeight:
         return out
 
 
-def moe_swiglu(gate_up: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
-    """silu(gate) * up, gate = first half of the last axis (moe_swiglu_split_cuda)."""
+def moe_glu(gate_up: torch.Tensor, out_dtype=torch.float16, activation: int = L.GLU_SILU) -> torch.Tensor:
+    """act(gate) * up, gate = first half of the last axis; act = SiLU (moe_swiglu_split_cuda) or, with
+    activation = GLU_GELU, the tanh form of GELU (moe_geglu_split_cuda, cpp_runtime/mfq_decode.cpp:320)."""
     W = gate_up.shape[-1] // 2
     g2 = gate_up.reshape(-1, 2 * W)
     hidden = torch.empty((g2.shape[0], W), dtype=out_dtype, device=gate_up.device)
-    L.check(L.lib().mfq_hip_moe_swiglu(_ptr(g2), g2.stride(0), g2.shape[0], W, _ptr(hidden),
-                                       L.X_F16 if out_dtype == torch.float16 else L.X_BF16, W, _stream()))
+    L.check(L.lib().mfq_hip_moe_glu(_ptr(g2), g2.stride(0), g2.shape[0], W, _ptr(hidden),
+                                    L.X_F16 if out_dtype == torch.float16 else L.X_BF16, W, activation, _stream()))
     return hidden.reshape(*gate_up.shape[:-1], W)
+
+
+def moe_swiglu(gate_up: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """silu(gate) * up, gate = first half of the last axis (moe_swiglu_split_cuda)."""
+    return moe_glu(gate_up, out_dtype, L.GLU_SILU)
+
+
+def moe_geglu(gate_up: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """gelu_tanh(gate) * up (moe_geglu_split_cuda)."""
+    return moe_glu(gate_up, out_dtype, L.GLU_GELU)
 
 
 def moe_weighted_reduce(pair: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None = None,
