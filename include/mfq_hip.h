@@ -99,6 +99,15 @@ int mfq_hip_nint_gemv_glu(const mfq_nint_desc *d, const void *weight, const void
 int mfq_hip_nint_embedding(const mfq_nint_desc *d, const void *weight, const int64_t *ids, int n_ids,
                            void *out, int out_dtype, int64_t ldo, mfq_stream_t stream);
 
+/* Input gate of a projection: out[m, k] = x[m, k] * act(gate[m, k]) with act = SiLU (mode 0) or the logistic
+ * function (mode 1), the numbering of nint_matmul_input_mul (cpp_runtime/mfq_decode.cpp:8395-8417); x, gate and out
+ * are bf16 or fp16 (x_dtype) [M, K] with row strides ldx / ldg / ldo, the product is formed in fp32 and rounded once.
+ * Followed by mfq_hip_nint_gemv / mfq_hip_nint_gemm on `out` it replaces nint_gemv_packed_gate_ws_cuda /
+ * nint_gemv_packed_bits_gate_ws_cuda (:389-392, :488-491) and the reference's own unfused form
+ * nint_matmul(w, x * silu(gate)) (:8415-8416); the gate is not fused into the GEMV here. */
+int mfq_hip_input_gate(const void *x, const void *gate, int x_dtype, int64_t ldx, int64_t ldg, int M, int K,
+                       int mode, void *out, int64_t ldo, mfq_stream_t stream);
+
 /* LM head for greedy decoding: token[m] = argmax_n y[m, n] with y as in mfq_hip_nint_gemv (equal logits go to the
  * lower index, NaN never wins, -1 when every logit is NaN).  M = 1 on NINT4-32, NINT4-24, NINT3-24 and NINT5-28
  * takes one GEMV launch whose blocks emit their winners, and a one-block final pass; other profiles and M > 1

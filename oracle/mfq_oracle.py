@@ -905,6 +905,15 @@ def moe_swiglu(gate_up):
     return ((gate / (1.0 + np.exp(-gate))) * up).astype(np.float32)
 
 
+def input_mul(x, gate, mode=0):
+    """x * silu(gate) (mode 0) or x * sigmoid(gate) (mode 1) in float64: the input gate of nint_matmul_input_mul
+    (cpp_runtime/mfq_decode.cpp:8395-8417; unfused form :8415-8416)."""
+    x = np.asarray(x, dtype=np.float64)
+    g = np.asarray(gate, dtype=np.float64)
+    s = 1.0 / (1.0 + np.exp(-g))
+    return x * (s if mode == 1 else g * s)
+
+
 def moe_geglu(gate_up):
     """gelu_tanh(gate) * up over [..., 2W] -> [..., W], gate = first half: mfq_glu<true>
     (mfq/kernels/cuda/glu.cuh:7-12), 0.5 g (1 + tanh(sqrt(2/pi) g (1 + 0.044715 g^2)))."""

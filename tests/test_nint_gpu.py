@@ -187,6 +187,34 @@ def test_gate_up_gemv_with_fused_geglu(bits, gs, sb):
             assert rel_l2(sw, O.moe_swiglu(y)) < 2e-3 and rel_l2(sw, h) > 1e-2   # the two activations differ
 
 
+@pytest.mark.parametrize("K", [1000, 77])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_input_gate_then_matmul(mode, K):
+    """x * silu(gate) or x * sigmoid(gate) ahead of the projection: the gated rows against the float64 product (one
+    16-bit rounding), the matmul against the oracle on those rows; K = 77 takes the element-wise kernel."""
+    from tyloquant_amd import _lib as L
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(490 + mode + K)
+    t = O.quantize_nint((rng.standard_normal((48, K)) * 0.02).astype(np.float32), 4, 24, 6)
+    lin = _load(t)
+    deq = O.dequantize_nint(t)
+    for M in (1, 5):
+        for dtype in (torch.bfloat16, torch.float16):
+            x, xf = _x(rng, M, K, dtype)
+            g, gf = _x(rng, M, K, dtype)
+            gated = torch.empty_like(x)
+            L.check(L.lib().mfq_hip_input_gate(x.data_ptr(), g.data_ptr(), R._x_dtype(x), x.stride(0), g.stride(0), M, K,
+                                               mode, gated.data_ptr(), gated.stride(0), None))
+            want = O.input_mul(xf, gf, mode)
+            eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+            got = gated.float().cpu().numpy().astype(np.float64)
+            assert np.all(np.abs(got - want) <= eps * np.abs(want) + 1e-7)      # one rounding of the exact product
+            assert np.array_equal(got[want == 0], want[want == 0])
+            y = R.nint_matmul_input_mul(lin.weight, x, g, mode).cpu().numpy()
+            ref = O.linear_forward_f64(deq, got.astype(np.float32))
+            assert rel_l2(y, ref) < REL_TOL and np.abs(y - ref).max() < ABS_TOL
+
+
 def test_config1_shape_nint3():
     """BASELINE config 1: 4096x4096 N(0, 0.02) NINT3 (3,24,5), bf16 x at batch 1."""
     from tyloquant_amd import runtime as R

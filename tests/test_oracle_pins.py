@@ -321,6 +321,11 @@ def test_moe_reference_loop_and_ffn_pieces():
     gu = rng.standard_normal((3, 8)).astype(np.float32)
     g, u = gu[:, :4].astype(np.float64), gu[:, 4:].astype(np.float64)
     assert np.allclose(O.moe_swiglu(gu), g / (1 + np.exp(-g)) * u, atol=1e-6)
+    # input gate: silu(g) = g * sigmoid(g), sigmoid(0) = 1/2, sigmoid(-g) = 1 - sigmoid(g)
+    xs, gs_ = rng.standard_normal(9), rng.standard_normal(9)
+    assert np.allclose(O.input_mul(xs, gs_, 0), gs_ * O.input_mul(xs, gs_, 1), atol=1e-12)
+    assert np.allclose(O.input_mul(xs, np.zeros(9), 1), 0.5 * xs) and np.all(O.input_mul(xs, np.zeros(9), 0) == 0)
+    assert np.allclose(O.input_mul(xs, gs_, 1) + O.input_mul(xs, -gs_, 1), xs, atol=1e-12)
     # GEGLU: the tanh form against the erf form it approximates (max difference of the two GELUs is below 5e-4 over
     # the reals), exact zeros, and the large-|g| limits g and 0
     from math import erf

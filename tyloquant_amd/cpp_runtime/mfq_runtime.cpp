@@ -293,6 +293,13 @@ void nint_matmul_geglu(const NintWeight &w, const void *x, int x_dtype, int64_t 
                        mfq_stream_t stream) {
     nint_matmul_glu(w, x, x_dtype, ldx, M, hidden, scratch, MFQ_GLU_GELU, "nint_matmul_geglu", stream);
 }
+void nint_matmul_input_mul(const NintWeight &w, const void *x, const void *gate, int x_dtype, int64_t ldx, int64_t ldg, int M,
+                           int mode, void *gated, float *y, mfq_stream_t stream) {
+    if (!gated) fail("nint_matmul_input_mul: needs a [M, K] 16-bit buffer for the gated activations");
+    const int K = w.desc.neuron_len;
+    abi_check(mfq_hip_input_gate(x, gate, x_dtype, ldx, ldg, M, K, mode, gated, K, stream));
+    nint_matmul(w, gated, x_dtype, K, M, y, stream);
+}
 void nint_embedding(const NintWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype, mfq_stream_t stream) {
     abi_check(mfq_hip_nint_embedding(&w.desc, w.data.get(), ids, n_ids, out, out_dtype, w.desc.neuron_len, stream));
 }

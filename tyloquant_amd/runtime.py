@@ -152,6 +152,20 @@ def nint_matmul_geglu(w: NintWeight, x: torch.Tensor, out_dtype=torch.float16) -
     return _nint_matmul_glu(w, x, out_dtype, L.GLU_GELU)
 
 
+def nint_matmul_input_mul(w: NintWeight, x: torch.Tensor, gate: torch.Tensor, mode: int = 0) -> torch.Tensor:
+    """(x * silu(gate)) . W^T, or with mode 1 (x * sigmoid(gate)) . W^T (nint_matmul_input_mul,
+    cpp_runtime/mfq_decode.cpp:8395-8417): the gated activations are formed by one elementwise launch (fp32 product,
+    one rounding to the dtype of x) and go through nint_matmul."""
+    if gate.shape != x.shape:
+        raise ValueError("gate and activations must have the same shape")
+    x2 = _as_2d(x, w.neuron_len)
+    g2 = _as_2d(gate.to(x2.dtype), w.neuron_len)
+    out = torch.empty((x2.shape[0], w.neuron_len), dtype=x2.dtype, device=x2.device)
+    L.check(L.lib().mfq_hip_input_gate(_ptr(x2), _ptr(g2), _x_dtype(x2), x2.stride(0), g2.stride(0), x2.shape[0],
+                                       w.neuron_len, int(mode), _ptr(out), out.stride(0), _stream()))
+    return nint_matmul(w, out.reshape(x.shape))
+
+
 def nint_embedding(w: NintWeight, ids: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
     """Rows ids of the dequantized table as out_dtype, shape ids.shape + [neuron_len]; ids outside the table give
     zeros (embed_forward, cpp_runtime/mfq_decode.cpp:13929-13957)."""
