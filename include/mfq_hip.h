@@ -132,6 +132,43 @@ int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, const void *x,
                       size_t workspace_bytes, mfq_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
+ * NINT8-0: GGML Q8_0 blocks (fp16 scale + 32 signed 8-bit codes, weight = scale * code; mfq/formats/nint8_zero.py)
+ * under the dtype string "NINT8-0".  Replaces Nint8ZeroCpu + to_device_nint8_zero
+ * (cpp_runtime/mfq_decode.cpp:1591-1650, 2309-2330) and the q8_zero branch of nint_matmul (:8165-8185).
+ * ---------------------------------------------------------------------------------- */
+typedef struct mfq_nint8z_desc {
+    int32_t out, neuron_len, ng;   /* ng = neuron_len / 32 */
+    int32_t reserved;
+    int64_t scales_off;            /* fp16 [out][ng] */
+    int64_t codes_off;             /* int8 [out][neuron_len] */
+    int64_t total_bytes;
+    int64_t payload_bytes;         /* out * ng * 34: the blocks of the file */
+} mfq_nint8z_desc;
+
+/* MFQ_ERR_INVALID unless neuron_len is a positive multiple of 32 (the format's rule). */
+int mfq_hip_nint8z_plan(int out, int neuron_len, mfq_nint8z_desc *d);
+/* `blocks` = device copy of the out * ng 34-byte blocks that follow the blob header; splits them into the
+ * device layout.  Replaces the block loop of unpack_nint8_zero (cpp_runtime/mfq_decode.cpp:1640-1648). */
+int mfq_hip_nint8z_repack(const mfq_nint8z_desc *d, const void *blocks, int64_t block_bytes, void *weight,
+                          mfq_stream_t stream);
+/* w_out[out, ld] = f32(scale) * f32(code), bit-exact with dequantize_nint8_zero (mfq/formats/nint8_zero.py:208-218)
+ * and nint8_zero_dequant_cuda (cpp_runtime/mfq_decode.cpp:8180-8182). */
+int mfq_hip_nint8z_dequant_f32(const mfq_nint8z_desc *d, const void *weight, float *w_out, int64_t ld,
+                               mfq_stream_t stream);
+/* y[M, out] = x[M, neuron_len] . W^T streaming the codes once per pass of up to 8 rows (fewer when the fp16
+ * activations of a pass would not fit 64 KB of LDS; MFQ_ERR_UNSUPPORTED when one row does not).  Replaces
+ * nint8_zero_gemv_ws_cuda / nint8_zero_mmq_ws_cuda (cpp_runtime/mfq_decode.cpp:8167-8177). */
+int mfq_hip_nint8z_gemv(const mfq_nint8z_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                        int M, float *y, int64_t ldy, mfq_stream_t stream);
+/* Any M: the streaming kernel up to 32 rows, above that dequantize to fp16 (power-of-two row scales) + the dense
+ * fp16 MFMA GEMM in the workspace (size from the query; 0 when none is needed).  Replaces the
+ * nint8_zero_dequant_cuda + matmul fallback (cpp_runtime/mfq_decode.cpp:8179-8185). */
+size_t mfq_hip_nint8z_gemm_workspace_bytes(const mfq_nint8z_desc *d, int M);
+int mfq_hip_nint8z_gemm(const mfq_nint8z_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                        int M, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                        mfq_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
  * NVQ-JSC, D4 family (NVQ3J = d4_256, NVQ3J-512 = d4_512; plain NVQ3 maps onto the
  * analytic one-bank tables).  Replaces NvqWeight + to_device_nvq
  * (cpp_runtime/mfq_decode.cpp:4019-4150).

@@ -25,6 +25,9 @@ reference tree).  Parity status of each function:
     build_expert_map               mfq/kernels/cuda/moe.cu:472-542
     moe_grouped_matmul / moe_ffn   tests/test_moe_kernels_cuda.py:58-68, cpp_runtime/mfq_decode.cpp:3394-3416
     mfq_file_write / mfq_file_read mfq/formats/io.py:646-685
+    pack_nint8_zero / unpack_nint8_zero / dequantize_nint8_zero / quantize_nint8_zero
+                                   mfq/formats/nint8_zero.py:107-218 (the GGML Q8_0 rule: closed form)
+    moe_swiglu / moe_geglu / input_mul   mfq/kernels/cuda/glu.cuh:5-16, cpp_runtime/mfq_decode.cpp:8395-8417
 
   pinned by golden vectors written from the reference's own numpy quantizer
   (tests/golden/nint_quant_vectors.npz, made by tests/golden/make_nint_quant_vectors.py)
@@ -626,10 +629,103 @@ class NintMoeTensor:
     pools: list = field(default_factory=list)
 
 
+# ---------------------------------------------------------------------------
+# NINT8-0 = GGML Q8_0 blocks  (mfq/formats/nint8_zero.py)
+# ---------------------------------------------------------------------------
+@dataclass
+class Nint8ZeroTensor:
+    shape: tuple
+    axis: int
+    scale: np.ndarray   # (out, ng) float16
+    q: np.ndarray       # (out, ng, 32) int8
+    neuron_len: int
+
+    @property
+    def out(self):
+        return self.q.shape[0]
+
+    @property
+    def ng(self):
+        return self.q.shape[1]
+
+
+_N8Z_HDR = struct.Struct("<4siiI")
+
+
+def quantize_nint8_zero(weight, axis=0) -> Nint8ZeroTensor:
+    """The deterministic GGML Q8_0 rule per block of 32 (mfq/formats/nint8_zero.py:128-155): scale = max|x| / 127 in
+    fp32 (stored as fp16), codes = round-half-away(x * (1 / scale_f32)) clipped to +-127; an all-zero block gets
+    scale 0 and codes 0."""
+    values = np.asarray(weight, dtype=np.float32)
+    if not values.ndim or not 0 <= axis < values.ndim:
+        raise ValueError("NINT8-0 axis is outside the tensor rank")
+    moved = np.moveaxis(values, axis, 0)
+    out = moved.shape[0]
+    neuron_len = moved.size // out
+    if neuron_len <= 0 or neuron_len % 32:
+        raise ValueError("NINT8-0 neuron_len must be a positive multiple of 32")
+    blocks = np.ascontiguousarray(moved).reshape(out, neuron_len // 32, 32)
+    scale = np.max(np.abs(blocks), axis=-1, keepdims=True) / np.float32(127.0)
+    inv = np.zeros_like(scale, dtype=np.float32)
+    np.divide(np.float32(1.0), scale, out=inv, where=scale != 0)
+    norm = blocks * inv
+    q = np.clip(np.sign(norm) * np.floor(np.abs(norm) + np.float32(0.5)), -127, 127).astype(np.int8)
+    return Nint8ZeroTensor(tuple(int(v) for v in values.shape), axis, scale[..., 0].astype(np.float16), q, neuron_len)
+
+
+def pack_nint8_zero(t: Nint8ZeroTensor) -> bytes:
+    """"<4siiI" header ("NI80", axis, neuron_len, ndim) + shape i64[ndim] + out u32 + ng u32 + 34-byte blocks
+    (fp16 scale || 32 int8) in row order (mfq/formats/nint8_zero.py:84-124, 157-164)."""
+    head = _N8Z_HDR.pack(b"NI80", t.axis, t.neuron_len, len(t.shape)) + struct.pack(f"<{len(t.shape)}q", *t.shape)
+    head += struct.pack("<II", t.out, t.ng)
+    blocks = np.empty((t.out, t.ng, 34), dtype=np.uint8)
+    blocks[..., :2] = np.ascontiguousarray(t.scale.astype("<f2")).view(np.uint8).reshape(t.out, t.ng, 2)
+    blocks[..., 2:] = np.ascontiguousarray(t.q).view(np.uint8)
+    return head + blocks.tobytes()
+
+
+def unpack_nint8_zero(blob) -> Nint8ZeroTensor:
+    """mfq/formats/nint8_zero.py:166-205, with its error messages."""
+    if len(blob) < _N8Z_HDR.size:
+        raise ValueError("truncated NINT8-0 header")
+    magic, axis, neuron_len, ndim = _N8Z_HDR.unpack_from(blob, 0)
+    if magic != b"NI80":
+        raise ValueError(f"invalid NINT8-0 magic: {magic!r}")
+    if ndim == 0:
+        raise ValueError("NINT8-0 tensor rank cannot be zero")
+    off = _N8Z_HDR.size
+    if off + 8 * ndim + 8 > len(blob):
+        raise ValueError("truncated NINT8-0 shape")
+    shape = struct.unpack_from(f"<{ndim}q", blob, off)
+    off += 8 * ndim
+    out, ng = struct.unpack_from("<II", blob, off)
+    off += 8
+    expected = out * ng * 34
+    if len(blob) - off != expected:
+        raise ValueError(f"invalid NINT8-0 block bytes: got {len(blob) - off}, expected {expected}")
+    blocks = np.frombuffer(blob, dtype=np.uint8, count=expected, offset=off).reshape(out, ng, 34)
+    scale = np.ascontiguousarray(blocks[..., :2]).view("<f2").reshape(out, ng)
+    q = np.ascontiguousarray(blocks[..., 2:]).view(np.int8)
+    if not 0 <= axis < ndim:
+        raise ValueError("NINT8-0 axis is outside the tensor rank")
+    if neuron_len <= 0 or neuron_len % 32:
+        raise ValueError("NINT8-0 neuron_len must be a positive multiple of 32")
+    if shape[axis] != out or ng != neuron_len // 32 or math.prod(shape) != out * neuron_len:
+        raise ValueError("NINT8-0 dimensions disagree with the logical shape")
+    return Nint8ZeroTensor(tuple(int(v) for v in shape), int(axis), scale, q, int(neuron_len))
+
+
+def dequantize_nint8_zero(t: Nint8ZeroTensor) -> np.ndarray:
+    """float32 scale * float32 code, [out, neuron_len] (mfq/formats/nint8_zero.py:208-218)."""
+    return (t.scale.astype(np.float32)[..., None] * t.q.astype(np.float32)).reshape(t.out, t.neuron_len)
+
+
 def tensor_dtype(t) -> str:
     """Public dtype label (mfq/formats/io.py:576-640)."""
     if isinstance(t, NintTensor):
         return f"NINT{t.bits}"
+    if isinstance(t, Nint8ZeroTensor):
+        return "NINT8-0"
     if isinstance(t, NvqJscTensor):
         return {"e8_256": "NVQ2J", "e8_1024": "NVQ2J-L", "e8_4096": "NVQ2J-XL", "d4_256": "NVQ3J",
                 "d4_512": "NVQ3J-512", "d4_1024": "NVQ3J-L"}[t.codebook]
@@ -646,6 +742,8 @@ def pack_tensor(t) -> tuple[str, bytes]:
     dt = tensor_dtype(t)
     if isinstance(t, NintTensor):
         return dt, pack_nint(t)
+    if isinstance(t, Nint8ZeroTensor):
+        return dt, pack_nint8_zero(t)
     if isinstance(t, NvqJscTensor):
         return dt, pack_nvq_jsc(t)
     if isinstance(t, NvqTensor):
@@ -665,6 +763,8 @@ def unpack_tensor(dtype: str, blob):
         if t.label != dtype:
             raise ValueError(f"MFQ dtype/blob mismatch: {dtype} contains {t.label}")
         return t
+    if dtype == "NINT8-0":
+        return unpack_nint8_zero(blob)
     if dtype.startswith("NINT"):
         return unpack_nint(blob)
     if dtype.startswith("NVQ"):

@@ -215,6 +215,48 @@ def test_input_gate_then_matmul(mode, K):
             assert rel_l2(y, ref) < REL_TOL and np.abs(y - ref).max() < ABS_TOL
 
 
+@pytest.mark.parametrize("out,K", [(37, 96), (130, 1056), (64, 4096), (9000, 64)])
+def test_nint8_zero_dequant_bit_exact_and_matmul(out, K):
+    """NINT8-0 (GGML Q8_0 blocks): the device dequantizer against the oracle bit for bit; the streaming kernel for 1..33
+    rows (8 per pass, more than 8192 rows: several rows per wave) and the dequantize + fp16 GEMM path above it."""
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(600 + out + K)
+    w = (rng.standard_normal((out, K)) * 0.02).astype(np.float32)
+    w[0, :32] = 0.0                                   # an all-zero block: scale 0
+    t = O.quantize_nint8_zero(w)
+    dtype, blob = O.pack_tensor(t)
+    assert dtype == "NINT8-0"
+    lin = R.load_quant_linear(dtype, blob)
+    deq = O.dequantize_nint8_zero(O.unpack_nint8_zero(blob))
+    got = lin.dequantize().cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), deq.view(np.uint32))
+    for M in (1, 2, 3, 8, 11, 33, 300):
+        if out * K * M > 3e8:
+            continue
+        for xd in (torch.bfloat16, torch.float16):
+            x, xf = _x(rng, M, K, xd)
+            y = lin(x).cpu().numpy()
+            ref = O.linear_forward_f64(deq, xf)
+            assert rel_l2(y, ref) < REL_TOL, (M, rel_l2(y, ref))
+            assert np.abs(y - ref).max() < ABS_TOL
+    x, xf = _x(rng, 40, K)                            # the streaming kernel beyond its default range
+    y = R.nint8_zero_matmul(lin.weight, x, force="gemv").cpu().numpy()
+    assert rel_l2(y, O.linear_forward_f64(deq, xf)) < REL_TOL
+
+
+def test_nint8_zero_loader_errors():
+    from tyloquant_amd import runtime as R
+    t = O.quantize_nint8_zero(np.ones((4, 64), np.float32))
+    blob = O.pack_nint8_zero(t)
+    with pytest.raises(ValueError, match="invalid NINT8-0 block bytes"):
+        R.load_quant_linear("NINT8-0", blob[:-2])
+    with pytest.raises(ValueError, match="invalid NINT8-0 magic"):
+        R.load_quant_linear("NINT8-0", b"NI81" + blob[4:])
+    t1 = O.quantize_nint8_zero(np.ones((64, 4), np.float32), axis=1)
+    with pytest.raises(ValueError, match="axis 0"):
+        R.load_quant_linear("NINT8-0", O.pack_nint8_zero(t1))
+
+
 def test_config1_shape_nint3():
     """BASELINE config 1: 4096x4096 N(0, 0.02) NINT3 (3,24,5), bf16 x at batch 1."""
     from tyloquant_amd import runtime as R

@@ -365,3 +365,49 @@ def test_c_restatement_matches_the_numpy_oracle_bit_for_bit():
     y = c_oracle.matmul_nt(x, W)
     ref = O.linear_forward_f64(W, x)
     assert np.abs(y - ref).max() < 1e-4 * np.abs(ref).max()
+
+
+def test_nint8_zero_is_ggml_q8_0():
+    """NINT8-0 restates the textbook GGML Q8_0 block: fp16 scale = max|x| / 127, codes = round-half-away(x / scale),
+    34 bytes per 32 weights (8.5 bit/weight).  Known answers on hand-made blocks, the byte layout written out by hand,
+    round trips, and the reference's error messages (mfq/formats/nint8_zero.py)."""
+    import struct
+    blk = np.zeros((2, 64), np.float32)
+    blk[0, :32] = np.arange(32) - 10.0            # max |x| = 21 -> scale 21/127, x = -10 -> code round(-60.476) = -60
+    blk[0, 32:] = 0.0                             # all-zero block: scale 0, codes 0
+    blk[1, 0], blk[1, 1], blk[1, 2] = 127.0, 63.5, -0.5   # scale exactly 1: ties round away from zero
+    t = O.quantize_nint8_zero(blk)
+    assert t.q.shape == (2, 2, 32) and t.scale.dtype == np.float16
+    assert t.scale[0, 0] == np.float16(21.0 / 127.0) and t.scale[0, 1] == 0 and not t.q[0, 1].any()
+    assert t.q[0, 0, 0] == -60 and t.q[0, 0, 31] == 127 and t.q[0, 0, 10] == 0
+    assert t.scale[1, 0] == 1.0 and list(t.q[1, 0, :3]) == [127, 64, -1]
+    # codes use the fp32 scale, the file keeps its fp16 rounding: the reconstruction is scale_f16 * code
+    deq = O.dequantize_nint8_zero(t)
+    assert deq[0, 31] == np.float32(np.float16(21.0 / 127.0)) * np.float32(127.0) and deq.dtype == np.float32
+    blob = O.pack_nint8_zero(t)
+    assert blob[:4] == b"NI80" and struct.unpack_from("<iiI", blob, 4) == (0, 64, 2)
+    assert struct.unpack_from("<2q", blob, 16) == (2, 64) and struct.unpack_from("<II", blob, 32) == (2, 2)
+    assert len(blob) == 40 + 4 * 34                                   # 8.5 bits per weight behind a 40-byte header
+    first = blob[40:74]
+    assert first[:2] == np.float16(21.0 / 127.0).tobytes() and first[2] == (-60) & 0xff and first[33] == 127
+    back = O.unpack_nint8_zero(blob)
+    assert np.array_equal(back.q, t.q) and np.array_equal(back.scale, t.scale) and back.shape == (2, 64)
+    assert O.tensor_dtype(t) == "NINT8-0" and O.pack_tensor(t) == ("NINT8-0", blob)
+    rng = np.random.default_rng(5)
+    w = (rng.standard_normal((7, 96)) * 0.02).astype(np.float32)
+    tw = O.quantize_nint8_zero(w)
+    err = np.abs(O.dequantize_nint8_zero(tw) - w).reshape(7, 3, 32)
+    half_step = np.abs(w).reshape(7, 3, 32).max(-1) / 127.0 * 0.5
+    # half a step, plus the fp16 rounding of the scale (2^-11) carried by a code of up to 127: 0.062 of a step
+    assert np.all(err <= half_step[..., None] * (1.0 + 2 * 127 * 2.0 ** -11) + 1e-9)
+    for bad, msg in ((blob[:10], "truncated NINT8-0 header"), (b"XXXX" + blob[4:], "invalid NINT8-0 magic"),
+                     (blob[:-1], "invalid NINT8-0 block bytes"), (blob[:8] + struct.pack("<i", 48) + blob[12:], "multiple of 32")):
+        with pytest.raises(ValueError, match=msg):
+            O.unpack_nint8_zero(bad)
+    with pytest.raises(ValueError, match="multiple of 32"):
+        O.quantize_nint8_zero(np.zeros((3, 40), np.float32))
+    from tyloquant_amd import formats as F
+    h = F.parse_nint8_zero(blob)
+    assert (h.out, h.ng, h.neuron_len, h.body_off, h.body_bytes) == (2, 2, 64, 40, 136)
+    with pytest.raises(ValueError, match="invalid NINT8-0 block bytes"):
+        F.parse_nint8_zero(blob + b"\0")

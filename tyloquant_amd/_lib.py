@@ -38,6 +38,11 @@ class NepqDesc(C.Structure):
                                    "payload_bytes")]
 
 
+class Nint8zDesc(C.Structure):
+    _fields_ = [(n, i32) for n in ("out", "neuron_len", "ng", "reserved")] + \
+               [(n, i64) for n in ("scales_off", "codes_off", "total_bytes", "payload_bytes")]
+
+
 class MoePool(C.Structure):
     _fields_ = [("desc", NintDesc), ("weight", vp)]
 
@@ -60,6 +65,12 @@ _SIGS = {
     "mfq_hip_nint_gemv_argmax": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, vp, sz, vp]),
     "mfq_hip_nint_gemm_workspace_bytes": (sz, [C.POINTER(NintDesc), C.c_int]),
     "mfq_hip_nint_gemm": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
+    "mfq_hip_nint8z_plan": (C.c_int, [C.c_int, C.c_int, C.POINTER(Nint8zDesc)]),
+    "mfq_hip_nint8z_repack": (C.c_int, [C.POINTER(Nint8zDesc), vp, i64, vp, vp]),
+    "mfq_hip_nint8z_dequant_f32": (C.c_int, [C.POINTER(Nint8zDesc), vp, vp, i64, vp]),
+    "mfq_hip_nint8z_gemv": (C.c_int, [C.POINTER(Nint8zDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
+    "mfq_hip_nint8z_gemm_workspace_bytes": (sz, [C.POINTER(Nint8zDesc), C.c_int]),
+    "mfq_hip_nint8z_gemm": (C.c_int, [C.POINTER(Nint8zDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
     "mfq_hip_nvq_plan": (C.c_int, [C.c_int] * 4 + [C.POINTER(NvqDesc)]),
     "mfq_hip_nvq_repack": (C.c_int, [C.POINTER(NvqDesc), vp, i64, vp, vp]),
     "mfq_hip_nvq_repack_plain": (C.c_int, [C.POINTER(NvqDesc), vp, i64, vp, vp, vp]),

@@ -1,0 +1,276 @@
+// NINT8-0: the GGML Q8_0 block layout under an MFQ dtype label -- blocks of one fp16 scale and 32 signed 8-bit codes,
+// weight = scale * code (mfq/formats/nint8_zero.py:1-10).
+//
+// Device layout: the blocks of the file (34 bytes, which no aligned load can walk) are split at load time into
+//   scales: fp16 [out][ng]          (ng = neuron_len / 32; the format requires a multiple of 32)
+//   codes:  int8 [out][neuron_len]  (row-major: a wave reads 1 KB of one row per step, 16 codes per lane)
+// Small batches: a wave owns a row at a time; the activations of the pass (up to MB rows) sit in LDS as fp16 next to
+// their sums over 16-element chunks.  A code byte c becomes the fp16 value 1024 + (c ^ 0x80) = c + 1152 by dropping it
+// into the mantissa of 1024.0 (one byte permute per pair), so a lane's 16 codes cost 8 permutes and 8 dot2 per
+// activation row, and 1152 times the chunk sum comes off afterwards; the block scale multiplies the chunk's result.
+// Larger batches dequantize once to fp16 rows with a power-of-two row scale and run the dense fp16 GEMM.
+#include "common.hpp"
+
+namespace mfq {
+
+struct N8zK {
+    int out, neuron_len, ng;
+    int64_t scales_off, codes_off;
+};
+static N8zK to_k(const mfq_nint8z_desc *d) {
+    N8zK k;
+    k.out = d->out; k.neuron_len = d->neuron_len; k.ng = d->ng; k.scales_off = d->scales_off; k.codes_off = d->codes_off;
+    return k;
+}
+
+// one thread per 34-byte block of the payload
+__global__ __launch_bounds__(256) void nint8z_repack_kernel(N8zK k, const uint8_t *__restrict__ blocks, uint8_t *__restrict__ dst) {
+    const int64_t b = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (b >= static_cast<int64_t>(k.out) * k.ng) return;
+    const uint8_t *src = blocks + b * 34;
+    reinterpret_cast<uint16_t *>(dst + k.scales_off)[b] = static_cast<uint16_t>(src[0] | (src[1] << 8));
+    uint32_t *q = reinterpret_cast<uint32_t *>(dst + k.codes_off) + b * 8;
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+        q[t] = src[2 + 4 * t] | (src[3 + 4 * t] << 8) | (src[4 + 4 * t] << 16) | (static_cast<uint32_t>(src[5 + 4 * t]) << 24);
+}
+
+// fl(f32(scale) * f32(code)): the product of an 11-bit and an 8-bit significand is exact in fp32
+__global__ __launch_bounds__(256) void nint8z_dequant_f32_kernel(N8zK k, const uint8_t *__restrict__ w, float *__restrict__ outp,
+                                                                 int64_t ld) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= static_cast<int64_t>(k.out) * k.neuron_len) return;
+    const int row = static_cast<int>(i / k.neuron_len), col = static_cast<int>(i - static_cast<int64_t>(row) * k.neuron_len);
+    const float s = f16_to_f32(reinterpret_cast<const uint16_t *>(w + k.scales_off)[static_cast<int64_t>(row) * k.ng + (col >> 5)]);
+    const int c = reinterpret_cast<const int8_t *>(w + k.codes_off)[i];
+    outp[row * ld + col] = __fmul_rn(s, static_cast<float>(c));
+}
+
+// fp16 rows for the dense GEMM: block = one row; values times 2^(12 - e), e = exponent of the row's largest
+// |scale| * 127, so that they stay below 4096; rowscale[row] = 2^(e - 12); columns up to kpad are zero
+__global__ __launch_bounds__(256) void nint8z_dequant_f16_kernel(N8zK k, const uint8_t *__restrict__ w, uint16_t *__restrict__ outp,
+                                                                 int64_t ld, float *__restrict__ rowscale, int kpad) {
+    __shared__ float smax[256];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const uint16_t *sc = reinterpret_cast<const uint16_t *>(w + k.scales_off) + static_cast<int64_t>(row) * k.ng;
+    float m = 0.f;
+    for (int g = tid; g < k.ng; g += 256) {
+        const float s = fabsf(f16_to_f32(sc[g]));
+        if (s == s && s <= 65504.f) m = fmaxf(m, s);  // a NaN or infinite scale does not set the range
+    }
+    smax[tid] = m;
+    __syncthreads();
+    for (int st = 128; st > 0; st >>= 1) {
+        if (tid < st) smax[tid] = fmaxf(smax[tid], smax[tid + st]);
+        __syncthreads();
+    }
+    int e = 0;
+    const float bound = smax[0] * 127.f;
+    if (bound > 0.f) frexpf(bound, &e);
+    const float inv = ldexpf(1.f, 12 - e);
+    if (tid == 0) rowscale[row] = ldexpf(1.f, e - 12);
+    const int8_t *q = reinterpret_cast<const int8_t *>(w + k.codes_off) + static_cast<int64_t>(row) * k.neuron_len;
+    for (int col = tid; col < kpad; col += 256) {
+        float v = 0.f;
+        if (col < k.neuron_len) v = f16_to_f32(sc[col >> 5]) * static_cast<float>(q[col]) * inv;
+        outp[row * ld + col] = f32_to_f16_rne(v);
+    }
+}
+
+// ---- small batches -----------------------------------------------------------------------------------------------
+// Block = 4 waves, RW rows per wave in turn; activation rows m0 .. m0 + MB - 1 of the pass.  LDS: fp16 x [MB][K], then
+// float chunk sums [MB][K / 16].
+template <int XF16, int MB>
+__global__ __launch_bounds__(256) void nint8z_gemv_kernel(N8zK k, const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
+                                                          int64_t ldx, int M, float *__restrict__ y, int64_t ldy, int rw) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = k.neuron_len, m0 = blockIdx.y * MB;
+    uint16_t *xh = reinterpret_cast<uint16_t *>(lds);
+    float *xsum = reinterpret_cast<float *>(lds + MB * K / 2);
+    for (int i = tid; i < MB * K; i += 256) {
+        const int m = i / K, c = i - m * K;
+        const int row = min(m0 + m, M - 1);
+        const uint16_t v = x[row * ldx + c];
+        xh[i] = XF16 ? v : f32_to_f16_rne(bf16_to_f32(v));
+    }
+    __syncthreads();
+    for (int i = tid; i < MB * (K / 16); i += 256) {
+        const uint32_t *p = reinterpret_cast<const uint32_t *>(xh) + i * 8;
+        float s = 0.f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, p[t]), half2_t{1, 1}, s, false);
+        xsum[i] = s;
+    }
+    __syncthreads();
+    const uint16_t *scales = reinterpret_cast<const uint16_t *>(w + k.scales_off);
+    const uint8_t *codes = w + k.codes_off;
+    const int row_first = (blockIdx.x * 4 + wave) * rw;
+    for (int ri = 0; ri < rw; ++ri) {
+        const int row = row_first + ri;  // wave-uniform
+        if (row >= k.out) break;
+        float acc[MB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[m] = 0.f;
+        for (int c0 = 0; c0 < K; c0 += 1024) {
+            const int col = c0 + lane * 16;
+            if (col < K) {
+                const u32x4_t q = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(codes + static_cast<int64_t>(row) * K + col));
+                const float s = f16_to_f32(scales[static_cast<int64_t>(row) * k.ng + (col >> 5)]);
+                uint32_t pr[8];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const uint32_t u = q[t] ^ 0x80808080u;
+                    pr[2 * t] = __builtin_amdgcn_perm(u, 0x64006400u, 0x03050104u);
+                    pr[2 * t + 1] = __builtin_amdgcn_perm(u, 0x64006400u, 0x03070106u);
+                }
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+                    const u32x4_t xa = *reinterpret_cast<const u32x4_t *>(xh + m * K + col);
+                    const u32x4_t xb = *reinterpret_cast<const u32x4_t *>(xh + m * K + col + 8);
+                    // plain scalars: a bit cast of a vector element taken in place reads the vector's first element
+                    const uint32_t xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+                    float r = 0.f;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)
+                        r = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, pr[t]), __builtin_bit_cast(half2_t, xv[t]), r, false);
+                    acc[m] = fmaf(s, fmaf(-1152.f, xsum[m * (K / 16) + (col >> 4)], r), acc[m]);
+                }
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            float v = acc[m];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+            if (lane == 0 && m0 + m < M) y[static_cast<int64_t>(m0 + m) * ldy + row] = v;
+        }
+    }
+}
+
+int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, const float *sa,
+                const float *sb, float *y, int64_t ldy, hipStream_t st);
+int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, hipStream_t st);
+size_t dequant_gemm_workspace(int N, int K, int M);
+void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&xscale, uint16_t *&w16, float *&wscale,
+                        int &Kp);
+
+// activation rows per pass: the most of 8, 4, 2, 1 whose fp16 rows and chunk sums fit 64 KB of LDS; 0 = none does
+static int nint8z_rows_per_pass(int K, int M) {
+    for (int mb = 8; mb >= 1; mb >>= 1)
+        if (mb <= (M > 4 ? 8 : (M > 2 ? 4 : (M > 1 ? 2 : 1))) && static_cast<size_t>(mb) * K * 2 + static_cast<size_t>(mb) * (K / 16) * 4 <= 65536)
+            return mb;
+    return 0;
+}
+
+template <int XF16>
+static int nint8z_gemv_launch(const N8zK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                              hipStream_t st) {
+    const int mb = nint8z_rows_per_pass(k.neuron_len, M);
+    MFQ_REQUIRE(mb > 0, MFQ_ERR_UNSUPPORTED, "nint8z_gemv: neuron_len %d does not fit the LDS", k.neuron_len);
+    // rows per wave: one, or more once the grid would exceed about eight blocks per CU
+    int rw = static_cast<int>(ceil_div(k.out, 4 * 2048));
+    if (rw < 1) rw = 1;
+    const dim3 grid(static_cast<unsigned>(ceil_div(k.out, 4 * rw)), static_cast<unsigned>(ceil_div(M, mb)));
+    const size_t lds = static_cast<size_t>(mb) * k.neuron_len * 2 + static_cast<size_t>(mb) * (k.neuron_len / 16) * 4;
+#define MFQ_N8Z(MB)                                                                                                  \
+    if (mb == MB) hipLaunchKernelGGL((nint8z_gemv_kernel<XF16, MB>), grid, dim3(256), lds, st, k, w, x, ldx, M, y, ldy, rw);
+    MFQ_N8Z(8) MFQ_N8Z(4) MFQ_N8Z(2) MFQ_N8Z(1)
+#undef MFQ_N8Z
+    return check_launch("nint8z_gemv");
+}
+
+}  // namespace mfq
+
+using namespace mfq;
+
+extern "C" int mfq_hip_nint8z_plan(int out, int neuron_len, mfq_nint8z_desc *d) {
+    MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nint8z_plan: null descriptor");
+    MFQ_REQUIRE(out > 0, MFQ_ERR_INVALID, "nint8z_plan: empty tensor");
+    MFQ_REQUIRE(neuron_len > 0 && neuron_len % 32 == 0, MFQ_ERR_INVALID, "NINT8-0 neuron_len must be a positive multiple of 32");
+    d->out = out; d->neuron_len = neuron_len; d->ng = neuron_len / 32;
+    d->scales_off = 0;
+    const int64_t sb = static_cast<int64_t>(out) * d->ng * 2;
+    d->codes_off = (sb + 255) / 256 * 256;
+    d->total_bytes = d->codes_off + static_cast<int64_t>(out) * neuron_len;
+    d->payload_bytes = static_cast<int64_t>(out) * d->ng * 34;
+    return MFQ_OK;
+}
+
+extern "C" int mfq_hip_nint8z_repack(const mfq_nint8z_desc *d, const void *blocks, int64_t block_bytes, void *weight,
+                                     mfq_stream_t stream) {
+    MFQ_REQUIRE(d && blocks && weight, MFQ_ERR_INVALID, "nint8z_repack: null argument");
+    MFQ_REQUIRE(block_bytes == d->payload_bytes, MFQ_ERR_INVALID, "invalid NINT8-0 block bytes: got %lld, expected %lld",
+                static_cast<long long>(block_bytes), static_cast<long long>(d->payload_bytes));
+    const N8zK k = to_k(d);
+    const int64_t n = static_cast<int64_t>(k.out) * k.ng;
+    hipLaunchKernelGGL(nint8z_repack_kernel, dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, as_stream(stream), k,
+                       static_cast<const uint8_t *>(blocks), static_cast<uint8_t *>(weight));
+    return check_launch("nint8z_repack");
+}
+
+extern "C" int mfq_hip_nint8z_dequant_f32(const mfq_nint8z_desc *d, const void *weight, float *w_out, int64_t ld,
+                                          mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && w_out, MFQ_ERR_INVALID, "nint8z_dequant_f32: null argument");
+    MFQ_REQUIRE(ld >= d->neuron_len, MFQ_ERR_INVALID, "nint8z_dequant_f32: ld smaller than neuron_len");
+    const N8zK k = to_k(d);
+    const int64_t n = static_cast<int64_t>(k.out) * k.neuron_len;
+    hipLaunchKernelGGL(nint8z_dequant_f32_kernel, dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, as_stream(stream),
+                       k, static_cast<const uint8_t *>(weight), w_out, ld);
+    return check_launch("nint8z_dequant_f32");
+}
+
+static int nint8z_gemv_any(const mfq_nint8z_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
+                           float *y, int64_t ldy, hipStream_t st) {
+    const N8zK k = to_k(d);
+    const uint8_t *w = static_cast<const uint8_t *>(weight);
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    return x_dtype == MFQ_X_F16 ? nint8z_gemv_launch<1>(k, w, xp, ldx, M, y, ldy, st)
+                                : nint8z_gemv_launch<0>(k, w, xp, ldx, M, y, ldy, st);
+}
+
+extern "C" int mfq_hip_nint8z_gemv(const mfq_nint8z_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                                   int M, float *y, int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nint8z_gemv: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nint8z_gemv: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint8z_gemv: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nint8z_gemv: ldx/ldy smaller than the tensor");
+    return nint8z_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, as_stream(stream));
+}
+
+// rows up to which the weights are re-streamed (8 rows per pass) rather than dequantized for the dense GEMM
+static constexpr int kN8zStreamMaxM = 32;
+static bool nint8z_streams(const mfq_nint8z_desc *d, int M) {
+    return M <= kN8zStreamMaxM && nint8z_rows_per_pass(d->neuron_len, M) > 0;
+}
+
+extern "C" size_t mfq_hip_nint8z_gemm_workspace_bytes(const mfq_nint8z_desc *d, int M) {
+    if (!d || M < 1 || nint8z_streams(d, M)) return 0;
+    return dequant_gemm_workspace(d->out, d->neuron_len, M);
+}
+
+extern "C" int mfq_hip_nint8z_gemm(const mfq_nint8z_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                                   int M, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                                   mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nint8z_gemm: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nint8z_gemm: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint8z_gemm: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nint8z_gemm: ldx/ldy smaller than the tensor");
+    hipStream_t st = as_stream(stream);
+    if (nint8z_streams(d, M)) return nint8z_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, st);
+    const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
+    MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nint8z_gemm: workspace %zu < %zu bytes",
+                workspace_bytes, need);
+    uint16_t *x16, *w16;
+    float *xscale, *wscale;
+    int Kp;
+    dequant_gemm_carve(workspace, d->out, d->neuron_len, M, x16, xscale, w16, wscale, Kp);
+    int rc = x_prep(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, st);
+    if (rc) return rc;
+    const N8zK k = to_k(d);
+    hipLaunchKernelGGL(nint8z_dequant_f16_kernel, dim3(static_cast<unsigned>(k.out)), dim3(256), 0, st, k,
+                       static_cast<const uint8_t *>(weight), w16, static_cast<int64_t>(Kp), wscale, Kp);
+    rc = check_launch("nint8z_dequant_f16");
+    if (rc) return rc;
+    return gemm_f16_nt(x16, Kp, w16, Kp, M, d->out, Kp, xscale, wscale, y, ldy, st);
+}

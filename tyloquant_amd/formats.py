@@ -123,6 +123,48 @@ def parse_nint(blob) -> NintHeader:
     return NintHeader(bits, sub_bits, gs, axis, neuron_len, tuple(shape), out, ng, off, remaining, legacy)
 
 
+# NINT8-0 (GGML Q8_0 blocks): "<4siiI" ("NI80", axis, neuron_len, ndim) + shape i64[ndim] + out u32 + ng u32 + blocks
+# (mfq/formats/nint8_zero.py:20-23, 166-205; cpp_runtime/mfq_decode.cpp:1601-1650)
+_N8Z_HDR = struct.Struct("<4siiI")
+
+
+@dataclass
+class Nint8zHeader:
+    axis: int
+    neuron_len: int
+    shape: tuple
+    out: int
+    ng: int
+    body_off: int
+    body_bytes: int
+
+
+def parse_nint8_zero(blob) -> Nint8zHeader:
+    if len(blob) < _N8Z_HDR.size:
+        raise ValueError("truncated NINT8-0 header")
+    magic, axis, neuron_len, ndim = _N8Z_HDR.unpack_from(blob, 0)
+    if magic != b"NI80":
+        raise ValueError(f"invalid NINT8-0 magic: {magic!r}")
+    if ndim == 0:
+        raise ValueError("NINT8-0 tensor rank cannot be zero")
+    off = _N8Z_HDR.size
+    if ndim > 8 or off + 8 * ndim + 8 > len(blob):
+        raise ValueError("truncated NINT8-0 shape")
+    shape = struct.unpack_from(f"<{ndim}q", blob, off)
+    off += 8 * ndim
+    out, ng = struct.unpack_from("<II", blob, off)
+    off += 8
+    if not 0 <= axis < ndim:
+        raise ValueError("NINT8-0 axis is outside the tensor rank")
+    if neuron_len <= 0 or neuron_len % 32:
+        raise ValueError("NINT8-0 neuron_len must be a positive multiple of 32")
+    if len(blob) - off != out * ng * 34:
+        raise ValueError(f"invalid NINT8-0 block bytes: got {len(blob) - off}, expected {out * ng * 34}")
+    if out <= 0 or shape[axis] != out or ng != neuron_len // 32 or math.prod(shape) != out * neuron_len:
+        raise ValueError("NINT8-0 dimensions disagree with the logical shape")
+    return Nint8zHeader(axis, neuron_len, tuple(shape), out, ng, off, len(blob) - off)
+
+
 def nint_arrays(blob) -> dict:
     """Packed-domain arrays of a NINT blob (the unpack half of mfq/formats/io.py:206-248)."""
     h = parse_nint(blob)

@@ -104,6 +104,59 @@ class NintWeight:
         return w
 
 
+class Nint8ZeroWeight:
+    """NINT8-0 (GGML Q8_0 blocks) on the device: fp16 scales and row-major int8 codes (to_device_nint8_zero,
+    cpp_runtime/mfq_decode.cpp:2309-2330)."""
+
+    def __init__(self, desc: L.Nint8zDesc, data: torch.Tensor, shape):
+        self.desc, self.data, self.shape = desc, data, tuple(shape)
+        self.out, self.neuron_len, self.ng = desc.out, desc.neuron_len, desc.ng
+        self.bits, self.gs = 8, 32
+        self._ws = _Workspace()
+
+    @property
+    def payload_bytes(self) -> int:
+        return int(self.desc.payload_bytes)
+
+    @staticmethod
+    def from_blob(blob, device="cuda") -> "Nint8ZeroWeight":
+        h = F.parse_nint8_zero(blob)
+        if h.axis != 0:
+            raise ValueError("NINT8-0 linear weights must be quantized along axis 0")
+        desc = L.Nint8zDesc()
+        L.check(L.lib().mfq_hip_nint8z_plan(h.out, h.neuron_len, C.byref(desc)))
+        device = torch.device(device)
+        payload = _upload(blob, h.body_off, h.body_bytes, device)
+        data = torch.empty(int(desc.total_bytes), dtype=torch.uint8, device=device)
+        L.check(L.lib().mfq_hip_nint8z_repack(C.byref(desc), _ptr(payload), h.body_bytes, _ptr(data), _stream()))
+        torch.cuda.current_stream().synchronize()  # payload may be freed after this
+        return Nint8ZeroWeight(desc, data, h.shape)
+
+    def dequantize(self) -> torch.Tensor:
+        w = torch.empty((self.out, self.neuron_len), dtype=torch.float32, device=self.data.device)
+        L.check(L.lib().mfq_hip_nint8z_dequant_f32(C.byref(self.desc), _ptr(self.data), _ptr(w), self.neuron_len,
+                                                   _stream()))
+        return w
+
+
+def nint8_zero_matmul(w: Nint8ZeroWeight, x: torch.Tensor, *, force: str | None = None) -> torch.Tensor:
+    """y[..., out] = x[..., K] @ W^T in fp32 for a NINT8-0 tensor (the q8_zero branch of nint_matmul,
+    cpp_runtime/mfq_decode.cpp:8165-8185).  force = "gemv" pins the streaming kernel."""
+    x2 = _as_2d(x, w.neuron_len)
+    M = x2.shape[0]
+    y = torch.empty((M, w.out), dtype=torch.float32, device=x.device)
+    lib = L.lib()
+    if force == "gemv":
+        L.check(lib.mfq_hip_nint8z_gemv(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
+                                        w.out, _stream()))
+    else:
+        need = lib.mfq_hip_nint8z_gemm_workspace_bytes(C.byref(w.desc), M)
+        ws = w._ws.get(need, x.device)
+        L.check(lib.mfq_hip_nint8z_gemm(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
+                                        w.out, _ptr(ws), need, _stream()))
+    return y.reshape(*x.shape[:-1], w.out)
+
+
 def nint_matmul(w: NintWeight, x: torch.Tensor, *, force: str | None = None) -> torch.Tensor:
     """y[..., out] = x[..., K] @ W^T in fp32 (cpp_runtime/mfq_decode.cpp:8130).  `force` = "gemv"
     or "gemm" pins the kernel family (the reference's MFQ_* path overrides)."""
@@ -261,6 +314,8 @@ def load_quant_linear(dtype: str, blob, device="cuda") -> QuantLinear:
         if f"NINT{w.bits}" != dtype:
             raise ValueError(f"MFQ dtype/blob mismatch: {dtype} contains NINT{w.bits}")
         return QuantLinear("nint", w)
+    if dtype == "NINT8-0":
+        return QuantLinear("nint8z", Nint8ZeroWeight.from_blob(blob, device))
     if is_nvq_linear_dtype(dtype):
         from .runtime_vq import NvqWeight
         w = NvqWeight.from_blob(blob, device)
@@ -286,4 +341,4 @@ def _nepq_mm(w, x):
     return nepq_matmul(w, x)
 
 
-_MATMUL = {"nint": nint_matmul, "nvq": _nvq_mm, "nepq": _nepq_mm}
+_MATMUL = {"nint": nint_matmul, "nint8z": nint8_zero_matmul, "nvq": _nvq_mm, "nepq": _nepq_mm}
