@@ -836,6 +836,8 @@ def unpack_nint_moe(blob) -> NintMoeTensor:
 def dequantize_tensor(t) -> np.ndarray:
     if isinstance(t, NintTensor):
         return dequantize_nint(t)
+    if isinstance(t, Nint8ZeroTensor):
+        return dequantize_nint8_zero(t)
     if isinstance(t, NvqJscTensor):
         return dequantize_nvq_jsc(t)
     if isinstance(t, NvqTensor):

@@ -56,6 +56,7 @@ def test_check_linear_tool_reports_small_error(tmp_path):
         "blk.0.ffn.nint4": O.quantize_nint((rng.standard_normal((64, 200)) * 0.02).astype(np.float32), 4, 32, 6),
         "blk.0.k.nvq3j512": synth.nvq_jsc_random(rng, 37, 96),
         "blk.0.v.nepq1s": synth.nepq_random(rng, "NEPQ1-S", 1, 48, 96, 3),
+        "blk.0.o.nint8_0": O.quantize_nint8_zero((rng.standard_normal((40, 96)) * 0.02).astype(np.float32)),
     }
     path = tmp_path / "tiny.mfq"
     O.mfq_file_write(path, tensors, version=2)
@@ -94,6 +95,24 @@ def test_cpp_load_quant_linear_and_forward(rt):
         _load(rt, "NINT4", O.pack_nint(t))
     with pytest.raises(RuntimeError, match="unsupported quantized linear dtype"):
         _load(rt, "MXFP4", b"\0" * 64)
+    # NINT8-0 through the same registry
+    t8 = O.quantize_nint8_zero((rng.standard_normal((24, 64)) * 0.02).astype(np.float32))
+    h8 = _load(rt, "NINT8-0", O.pack_nint8_zero(t8))
+    assert rt.mfq_rt_linear_out(h8) == 24 and rt.mfq_rt_linear_neuron_len(h8) == 64
+    W8 = torch.empty((24, 64), dtype=torch.float32, device="cuda")
+    assert rt.mfq_rt_linear_dequantize(h8, W8.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    deq8 = O.dequantize_nint8_zero(t8)
+    assert np.array_equal(W8.cpu().numpy().view(np.uint32), deq8.view(np.uint32))
+    for M in (1, 9, 40):
+        x = torch.from_numpy(rng.standard_normal((M, 64)).astype(np.float32)).to(torch.bfloat16).cuda()
+        y = torch.empty((M, 24), dtype=torch.float32, device="cuda")
+        assert rt.mfq_rt_linear_forward(h8, x.data_ptr(), 0, 64, M, y.data_ptr(), None) == 0
+        torch.cuda.synchronize()
+        check_close(y.cpu().numpy(), O.linear_forward_f64(deq8, x.float().cpu().numpy()))
+    rt.mfq_rt_free_quant_linear(h8)
+    with pytest.raises(RuntimeError, match="invalid NINT8-0 block payload length"):
+        _load(rt, "NINT8-0", O.pack_nint8_zero(t8)[:-1])
 
 
 def test_cpp_embedding_rows_and_argmax_head(rt):

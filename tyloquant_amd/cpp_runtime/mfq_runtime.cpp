@@ -226,6 +226,38 @@ NintWeight NintWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream_t str
     return w;
 }
 
+// "<4siiI" ("NI80", axis, neuron_len, ndim) + shape i64[ndim] + out u32 + ng u32 + 34-byte blocks; the checks and
+// messages of unpack_nint8_zero (cpp_runtime/mfq_decode.cpp:1601-1650)
+Nint8ZeroWeight Nint8ZeroWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream) {
+    if (n < 24 || std::memcmp(blob, "NI80", 4) != 0) fail("invalid NINT8-0 header");
+    const int axis = rd<int32_t>(blob, 4), neuron_len = rd<int32_t>(blob, 8);
+    const uint32_t ndim = rd<uint32_t>(blob, 12);
+    if (ndim == 0 || ndim > 8 || axis < 0 || axis >= static_cast<int>(ndim) || neuron_len <= 0 || neuron_len % 32 != 0)
+        fail("invalid NINT8-0 dimensions");
+    size_t off = 16;
+    if (n < off + 8ull * ndim + 8) fail("invalid NINT8-0 header");
+    Nint8ZeroWeight w;
+    w.shape.resize(ndim);
+    for (uint32_t i = 0; i < ndim; ++i, off += 8) w.shape[i] = rd<int64_t>(blob, off);
+    const int64_t out = rd<uint32_t>(blob, off), ng = rd<uint32_t>(blob, off + 4);
+    off += 8;
+    if (out <= 0 || ng != neuron_len / 32 || w.shape[static_cast<size_t>(axis)] != out) fail("NINT8-0 shape/header mismatch");
+    int64_t elements = 1;
+    for (int64_t v : w.shape) {
+        if (v <= 0 || elements > INT64_MAX / v) fail("invalid NINT8-0 logical shape");
+        elements *= v;
+    }
+    if (elements != out * neuron_len) fail("NINT8-0 logical element count mismatch");
+    if (n - off != static_cast<size_t>(out * ng) * 34) fail("invalid NINT8-0 block payload length");
+    if (axis != 0) fail("NINT8-0 linear weights must be quantized along axis 0");
+    abi_check(mfq_hip_nint8z_plan(static_cast<int>(out), neuron_len, &w.desc));
+    DeviceBuffer payload = DeviceBuffer::from_host(blob + off, n - off);
+    w.data = DeviceBuffer(static_cast<size_t>(w.desc.total_bytes));
+    abi_check(mfq_hip_nint8z_repack(&w.desc, payload.get(), static_cast<int64_t>(n - off), w.data.get(), stream));
+    hip_check(hipStreamSynchronize(hs(stream)), "nint8-0 repack");
+    return w;
+}
+
 NvqWeight NvqWeight::from_blob(const uint8_t *blob, size_t n, const int8_t *grid256, mfq_stream_t stream) {
     const NvqHeader h = parse_nvq(blob, n);
     if (h.vector_size != 4 || h.index_bits > 9)
@@ -334,6 +366,14 @@ void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, in
 void nint_dequantize(const NintWeight &w, float *out, mfq_stream_t stream) {
     abi_check(mfq_hip_nint_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
 }
+void nint8_zero_matmul(const Nint8ZeroWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) {
+    const size_t need = mfq_hip_nint8z_gemm_workspace_bytes(&w.desc, M);
+    w.workspace.ensure(need);
+    abi_check(mfq_hip_nint8z_gemm(&w.desc, w.data.get(), x, x_dtype, ldx, M, y, w.desc.out, w.workspace.get(), need, stream));
+}
+void nint8_zero_dequantize(const Nint8ZeroWeight &w, float *out, mfq_stream_t stream) {
+    abi_check(mfq_hip_nint8z_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
+}
 void nvq_dequantize(const NvqWeight &w, float *out, mfq_stream_t stream) {
     abi_check(mfq_hip_nvq_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
 }
@@ -349,23 +389,29 @@ bool is_nint_linear_dtype(const std::string &d) {
 bool is_nvq_linear_dtype(const std::string &d) { return d == "NVQ3" || d == "NVQ3J" || d == "NVQ3J-512" || d == "NIQ3"; }
 bool is_nepq_linear_dtype(const std::string &d) { return d == "NEPQ1-S" || d == "NEPQ1-L"; }
 
-int64_t QuantLinear::out() const { return kind == QuantLinearKind::Nint ? nint->out() : kind == QuantLinearKind::Nvq ? nvq->out() : nepq->out(); }
+int64_t QuantLinear::out() const {
+    return kind == QuantLinearKind::Nint ? nint->out() : kind == QuantLinearKind::Nvq ? nvq->out()
+         : kind == QuantLinearKind::Nepq ? nepq->out() : nint8z->out();
+}
 int64_t QuantLinear::neuron_len() const {
-    return kind == QuantLinearKind::Nint ? nint->neuron_len() : kind == QuantLinearKind::Nvq ? nvq->neuron_len() : nepq->neuron_len();
+    return kind == QuantLinearKind::Nint ? nint->neuron_len() : kind == QuantLinearKind::Nvq ? nvq->neuron_len()
+         : kind == QuantLinearKind::Nepq ? nepq->neuron_len() : nint8z->neuron_len();
 }
 int64_t QuantLinear::payload_bytes() const {
     return kind == QuantLinearKind::Nint ? nint->desc.payload_bytes : kind == QuantLinearKind::Nvq ? nvq->desc.payload_bytes
-                                                                                                   : nepq->desc.payload_bytes;
+         : kind == QuantLinearKind::Nepq ? nepq->desc.payload_bytes : nint8z->desc.payload_bytes;
 }
 void QuantLinear::forward(const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const {
     if (kind == QuantLinearKind::Nint) nint_matmul(*nint, x, x_dtype, ldx, M, y, stream);
     else if (kind == QuantLinearKind::Nvq) nvq_matmul(*nvq, x, x_dtype, ldx, M, y, stream);
-    else nepq_matmul(*nepq, 0, x, x_dtype, ldx, M, y, stream);
+    else if (kind == QuantLinearKind::Nepq) nepq_matmul(*nepq, 0, x, x_dtype, ldx, M, y, stream);
+    else nint8_zero_matmul(*nint8z, x, x_dtype, ldx, M, y, stream);
 }
 void QuantLinear::dequantize(float *out, mfq_stream_t stream) const {
     if (kind == QuantLinearKind::Nint) nint_dequantize(*nint, out, stream);
     else if (kind == QuantLinearKind::Nvq) nvq_dequantize(*nvq, out, stream);
-    else nepq_dequantize(*nepq, out, stream);
+    else if (kind == QuantLinearKind::Nepq) nepq_dequantize(*nepq, out, stream);
+    else nint8_zero_dequantize(*nint8z, out, stream);
 }
 
 QuantLinear load_quant_linear(const std::string &dtype_in, const uint8_t *blob, size_t n, mfq_stream_t stream) {
@@ -376,6 +422,11 @@ QuantLinear load_quant_linear(const std::string &dtype_in, const uint8_t *blob, 
         q.nint = std::make_shared<NintWeight>(NintWeight::from_blob(blob, n, stream));
         if ("NINT" + std::to_string(q.nint->desc.bits) != dtype)
             fail("MFQ dtype/blob mismatch: " + dtype + " contains NINT" + std::to_string(q.nint->desc.bits));
+        return q;
+    }
+    if (dtype == "NINT8-0") {
+        q.kind = QuantLinearKind::Nint8Zero;
+        q.nint8z = std::make_shared<Nint8ZeroWeight>(Nint8ZeroWeight::from_blob(blob, n, stream));
         return q;
     }
     if (is_nvq_linear_dtype(dtype)) {
@@ -622,7 +673,8 @@ LinearCheckResult run_linear_check(const QuantLinear &lin, int M, int reps) {
     res.production_ms = ms / reps;
     res.payload_bytes = lin.payload_bytes();
     res.weight_bytes = lin.kind == QuantLinearKind::Nint ? lin.nint->desc.total_bytes
-                     : lin.kind == QuantLinearKind::Nvq ? lin.nvq->desc.total_bytes : lin.nepq->desc.total_bytes;
+                     : lin.kind == QuantLinearKind::Nvq ? lin.nvq->desc.total_bytes
+                     : lin.kind == QuantLinearKind::Nepq ? lin.nepq->desc.total_bytes : lin.nint8z->desc.total_bytes;
     res.production_weight_gbps = res.weight_bytes / (res.production_ms * 1e6);
     res.payload_gbps = res.payload_bytes / (res.production_ms * 1e6);
     res.production_rel = den > 0 ? std::sqrt(num / den) : std::sqrt(num);

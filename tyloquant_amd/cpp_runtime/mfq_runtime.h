@@ -95,6 +95,16 @@ struct NintWeight {
     int64_t neuron_len() const { return desc.neuron_len; }
     static NintWeight from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream = nullptr);
 };
+// NINT8-0: GGML Q8_0 blocks (Nint8ZeroCpu + to_device_nint8_zero :1591-1650, 2309-2330)
+struct Nint8ZeroWeight {
+    mfq_nint8z_desc desc{};
+    DeviceBuffer data;
+    std::vector<int64_t> shape;
+    mutable DeviceBuffer workspace;
+    int64_t out() const { return desc.out; }
+    int64_t neuron_len() const { return desc.neuron_len; }
+    static Nint8ZeroWeight from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream = nullptr);
+};
 struct NvqWeight {
     mfq_nvq_desc desc{};
     DeviceBuffer data;
@@ -147,16 +157,21 @@ void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, in
                  mfq_stream_t stream = nullptr);
 void nint_dequantize(const NintWeight &w, float *out, mfq_stream_t stream = nullptr);
 void nvq_dequantize(const NvqWeight &w, float *out, mfq_stream_t stream = nullptr);
+// the q8_zero branch of nint_matmul (:8165-8185) and nint8_zero_dequant_cuda
+void nint8_zero_matmul(const Nint8ZeroWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y,
+                       mfq_stream_t stream = nullptr);
+void nint8_zero_dequantize(const Nint8ZeroWeight &w, float *out, mfq_stream_t stream = nullptr);
 void nepq_dequantize(const NepqWeight &w, float *out, mfq_stream_t stream = nullptr);
 
 // ---- dtype registry -------------------------------------------------------------------------------
 bool is_nint_linear_dtype(const std::string &dtype);
 bool is_nvq_linear_dtype(const std::string &dtype);
 bool is_nepq_linear_dtype(const std::string &dtype);
-enum class QuantLinearKind { Nint, Nvq, Nepq };
+enum class QuantLinearKind { Nint, Nvq, Nepq, Nint8Zero };
 struct QuantLinear {
     QuantLinearKind kind;
     std::shared_ptr<NintWeight> nint;
+    std::shared_ptr<Nint8ZeroWeight> nint8z;
     std::shared_ptr<NvqWeight> nvq;
     std::shared_ptr<NepqWeight> nepq;
     int64_t out() const;

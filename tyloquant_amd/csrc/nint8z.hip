@@ -88,11 +88,28 @@ __global__ __launch_bounds__(256) void nint8z_gemv_kernel(N8zK k, const uint8_t 
     const int K = k.neuron_len, m0 = blockIdx.y * MB;
     uint16_t *xh = reinterpret_cast<uint16_t *>(lds);
     float *xsum = reinterpret_cast<float *>(lds + MB * K / 2);
-    for (int i = tid; i < MB * K; i += 256) {
-        const int m = i / K, c = i - m * K;
-        const int row = min(m0 + m, M - 1);
-        const uint16_t v = x[row * ldx + c];
-        xh[i] = XF16 ? v : f32_to_f16_rne(bf16_to_f32(v));
+    if (ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {  // 16-byte chunks (K is a multiple of 32)
+        const int cpr = K / 8;
+        for (int i = tid; i < MB * cpr; i += 256) {
+            const int m = i / cpr, c = i - m * cpr;
+            const int row = min(m0 + m, M - 1);
+            const u32x4_t v = *reinterpret_cast<const u32x4_t *>(x + row * ldx + 8 * c);
+            uint32_t h[4] = {v.x, v.y, v.z, v.w};
+            if constexpr (!XF16) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    h[t] = f32_to_f16_rne(__uint_as_float(h[t] << 16)) |
+                           (static_cast<uint32_t>(f32_to_f16_rne(__uint_as_float(h[t] & 0xffff0000u))) << 16);
+            }
+            *reinterpret_cast<u32x4_t *>(xh + m * K + 8 * c) = u32x4_t{h[0], h[1], h[2], h[3]};
+        }
+    } else {
+        for (int i = tid; i < MB * K; i += 256) {
+            const int m = i / K, c = i - m * K;
+            const int row = min(m0 + m, M - 1);
+            const uint16_t v = x[row * ldx + c];
+            xh[i] = XF16 ? v : f32_to_f16_rne(bf16_to_f32(v));
+        }
     }
     __syncthreads();
     for (int i = tid; i < MB * (K / 16); i += 256) {
@@ -168,8 +185,9 @@ static int nint8z_gemv_launch(const N8zK &k, const uint8_t *w, const uint16_t *x
                               hipStream_t st) {
     const int mb = nint8z_rows_per_pass(k.neuron_len, M);
     MFQ_REQUIRE(mb > 0, MFQ_ERR_UNSUPPORTED, "nint8z_gemv: neuron_len %d does not fit the LDS", k.neuron_len);
-    // rows per wave: one, or more once the grid would exceed about eight blocks per CU
-    int rw = static_cast<int>(ceil_div(k.out, 4 * 2048));
+    // rows per wave: as many as leave about four blocks per CU (one or two activation rows) or two (more: a block's
+    // staged activations then serve twice the weight rows)
+    int rw = k.out / (4 * (M <= 2 ? 1024 : 512));
     if (rw < 1) rw = 1;
     const dim3 grid(static_cast<unsigned>(ceil_div(k.out, 4 * rw)), static_cast<unsigned>(ceil_div(M, mb)));
     const size_t lds = static_cast<size_t>(mb) * k.neuron_len * 2 + static_cast<size_t>(mb) * (k.neuron_len / 16) * 4;
