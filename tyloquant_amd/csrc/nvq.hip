@@ -459,7 +459,7 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
 // buffers: the only loads inside the walk are weights, each requested RING items before its use, so the waits are
 // for weights alone and the first request wave covers most of a block's share.
 // LDS map (bytes): [signed table: banks*entries*128][state table: 16 x {lut pair, bank base}][red: waves * 1024]
-// [raw codebook entries: banks*entries*4]
+// [codebook entries as fp16 pairs: banks*entries*8]
 typedef const __attribute__((address_space(3))) u32x2_t *lds_u32x2_ptr;
 template <int XF16, int RPB, int RING, bool ONE>
 __global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k, const uint8_t *__restrict__ w,
@@ -536,10 +536,17 @@ __global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k, const uint8_t 
         if (n > 0) wload(t / RPB, t % RPB, ring[t]);
         if (t + 1 < RING) __builtin_amdgcn_s_barrier();
     }
-    uint32_t *rawcb = reinterpret_cast<uint32_t *>(red + (blockDim.x >> 6) * 256);  // ncb dwords behind the reduction area
+    // the entries as two fp16 pairs each, converted once (ncb x 8 bytes behind the reduction area)
+    u32x2_t *cbh = reinterpret_cast<u32x2_t *>(red + (blockDim.x >> 6) * 256);
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
-        if (tid + t * static_cast<int>(blockDim.x) < ncb) rawcb[tid + t * blockDim.x] = craw[t];
+    for (int t = 0; t < 4; ++t) {
+        if (tid + t * static_cast<int>(blockDim.x) < ncb) {
+            uint32_t h[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) h[b] = f32_to_f16_rne(static_cast<float>((craw[t] >> (8 * b)) & 0xffu));
+            cbh[tid + t * blockDim.x] = u32x2_t{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        }
+    }
     if (tid < 16) {
         const uint32_t h = f32_to_f16_rne(lutv);  // the LUT is fp16 in the payload: exact
         stab[2 * tid] = h | (h << 16);
@@ -548,11 +555,8 @@ __global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k, const uint8_t 
     __syncthreads();  // raw entries
     // chunk c = 16 bytes = the vectors of sign nibbles 2 * (c & 7) and 2 * (c & 7) + 1 of entry c >> 3
     for (int c = tid; c < ncb * 8; c += blockDim.x) {
-        const uint32_t e = rawcb[c >> 3];
-        uint32_t h[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) h[t] = f32_to_f16_rne(static_cast<float>((e >> (8 * t)) & 0xffu));
-        const uint32_t p0 = h[0] | (h[1] << 16), p1 = h[2] | (h[3] << 16);
+        const u32x2_t e = cbh[c >> 3];
+        const uint32_t p0 = e.x, p1 = e.y;
         const uint32_t n0 = 2u * (c & 7), n1 = n0 + 1u;
         u32x4_t v;
         v.x = p0 ^ (((n0 & 1u) << 15) | ((n0 & 2u) << 30));
@@ -903,7 +907,7 @@ static int nvq_launch_signed_as(const NvqK &k, const uint8_t *w, const uint16_t 
                                 int64_t ldy, hipStream_t st) {
     const int spw = static_cast<int>(ceil_div(k.nsteps, 16));
     const int nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
-    const size_t lds = static_cast<size_t>(k.banks) * k.entries * 132 + 128 + static_cast<size_t>(nwaves) * 1024;
+    const size_t lds = static_cast<size_t>(k.banks) * k.entries * 136 + 128 + static_cast<size_t>(nwaves) * 1024;
     auto kern = nvq_signed_kernel<XF16, RPB, RING, ONE>;
     if (lds > 65536) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
