@@ -573,11 +573,17 @@ __global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k, const uint8_t 
     auto process = [&](Item &it, uint32_t noff, bool refill, float4_t &acc) {
         const u32x4_t uc4 = it.c;
         if (refill) it.c = __builtin_amdgcn_raw_buffer_load_b128(win, noff + 2048 + lane * 16, 0, 2);
+        // the state entries of the four units first: one LDS round trip for the item instead of one per unit
+        const uint32_t ucv[4] = {uc4.x, uc4.y, uc4.z, uc4.w};
+        u32x2_t stv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            stv[j] = *reinterpret_cast<lds_u32x2_ptr>(stab_base + (__builtin_rotateleft32(ucv[j], 6) & 0x78u));
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const uint32_t ua = it.q[j].x, ub = it.q[j].y, uc = uc4[j];
+            const uint32_t ua = it.q[j].x, ub = it.q[j].y, uc = ucv[j];
             if (refill) it.q[j] = __builtin_amdgcn_raw_buffer_load_b64(win, noff + (j * 64 + lane) * 8, 0, 2);
-            const u32x2_t st = *reinterpret_cast<lds_u32x2_ptr>(stab_base + (__builtin_rotateleft32(uc, 6) & 0x78u));
+            const u32x2_t st = stv[j];
             const half2_t sc = __builtin_bit_cast(half2_t, st.x);
             const uint32_t off[6] = {and_or(ua, 0xfff8u, st.y), and_or(ua >> 16, 0xfff8u, st.y),
                                      and_or(ub, 0xfff8u, st.y), and_or(ub >> 16, 0xfff8u, st.y),
