@@ -57,7 +57,7 @@ def test_nvq_matrix_core_path_multi_step(out, K, M):
 @pytest.mark.parametrize("K", [1560, 6160])
 @pytest.mark.parametrize("rpb", [1, 2, 3, 4, 5, 6])
 def test_nvq_signed_table_kernel_row_blocks_per_block(monkeypatch, rpb, K):
-    """Up to 16 rows with the (entry, sign nibble) table in LDS: one block per CU owning rpb row-blocks.  With the CU
+    """Up to 32 rows (16 per tile) with the (entry, sign nibble) table in LDS: one block per CU and tile owning rpb row-blocks.  With the CU
     count the grid is sized for set to 8, 128 * rpb - 5 neurons give every rpb variant (ragged last row-block, last
     block with fewer row-blocks); K = 1560 is one step per wave (5 waves), K = 6160 two steps per wave with a ragged
     last group.  One- and two-bank 512-entry codebooks and the 256-entry one."""
@@ -71,7 +71,8 @@ def test_nvq_signed_table_kernel_row_blocks_per_block(monkeypatch, rpb, K):
         dtype, blob = O.pack_tensor(t)
         lin = R.load_quant_linear(dtype, blob)
         want = O.dequantize_nvq_jsc(O.unpack_nvq(blob))
-        for M, xd in ((1, torch.bfloat16), (7, torch.float16), (16, torch.bfloat16)):
+        for M, xd in ((1, torch.bfloat16), (7, torch.float16), (16, torch.bfloat16), (17, torch.bfloat16),
+                      (32, torch.float16)):                      # 17 and 32 rows: two 16-row tiles
             x, xf = _x(rng, M, K, xd)
             _check(nvq_matmul(lin.weight, x, force="gemv").cpu().numpy(), O.linear_forward_f64(want, xf))
 

@@ -450,8 +450,8 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
     mfma_store_dense<NB>(red, rb0, m0, M, k.out, y, ldy);
 }
 
-// ---- one 16-row tile with the signed table in LDS ------------------------------------------------
-// Up to 16 activation rows, one block per CU: a block owns up to RPB consecutive row-blocks, its waves split the K
+// ---- 16-row tiles with the signed table in LDS ---------------------------------------------------
+// Up to 16 activation rows per block (blockIdx.y = tile), one block per CU: a block owns up to RPB consecutive row-blocks, its waves split the K
 // steps.  The table maps (bank, entry, sign nibble) to the four signed fp16 magnitudes of a vector, so a fragment is
 // two 8-byte LDS reads at byte offsets that sit ready-made in the unit's fields, and one packed multiply per pair by
 // the state's scale; no sign table, no XOR, no index arithmetic.  A wave keeps the activation fragments of its current
@@ -479,7 +479,8 @@ __global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k, const uint8_t 
 
     const int rb_first = blockIdx.x * RPB;
     const int nrb = min(RPB, k.n_rowblocks - rb_first);  // row-blocks of this block
-    const int tok = min(static_cast<int>(lane & 15), M - 1);
+    const int m0 = static_cast<int>(blockIdx.y) * 16;  // the block's 16-row tile
+    const int tok = min(m0 + static_cast<int>(lane & 15), M - 1);
     const uint16_t *xrow = x + static_cast<int64_t>(tok) * ldx;
     const int r = lane & 15, kb = lane >> 4;
     const int s0 = wave * spw;
@@ -604,7 +605,7 @@ __global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k, const uint8_t 
         const float av = anchors[(rb_first + i) * 16 + r];
 #pragma unroll
         for (int v = 0; v < 4; ++v) red[(wave * 4 + v) * 64 + lane] = av * acc[v];
-        mfma_store_dense<1>(red, rb_first + i, 0, M, k.out, y, ldy);
+        mfma_store_dense<1>(red, rb_first + i, m0, M, k.out, y, ldy);
         __syncthreads();
     };
     if constexpr (ONE) {  // one step per wave: the ring may have any depth up to RPB
@@ -900,12 +901,15 @@ static int nvq_launch_mfma(const NvqK &k, const uint8_t *w, const uint16_t *x, i
     return check_launch("nvq_mfma");
 }
 
-// one 16-row tile through nvq_signed_kernel: at most one block per CU, each with up to six row-blocks
+// 16-row tiles through nvq_signed_kernel: at most one block per CU and tile, each with up to six row-blocks
 static int nvq_signed_rpb(const NvqK &k) { return static_cast<int>(ceil_div(k.n_rowblocks, gemv_cu_count())); }
 static bool nvq_signed_capable(const NvqK &k, int M) {
     static const int off = [] { const char *e = getenv("MFQ_NVQ_SIGNED_OFF"); return e ? atoi(e) : 0; }();
     const int rpb = nvq_signed_rpb(k);
-    return !off && M <= 16 && static_cast<int64_t>(k.banks) * k.entries * 128 <= 131072 && rpb <= 6 && k.nsteps >= 4 &&
+    // two 16-row tiles still beat the older streaming kernel and the prefill kernel on the config 3 tensors
+    // (17408 x 5120 at M = 32: 42 us against 54 and 46); MFQ_NVQ_SIGNED_MAX_M for tuning
+    static const int max_m = [] { const char *e = getenv("MFQ_NVQ_SIGNED_MAX_M"); return e ? atoi(e) : 32; }();
+    return !off && M <= max_m && static_cast<int64_t>(k.banks) * k.entries * 128 <= 131072 && rpb <= 6 && k.nsteps >= 4 &&
            rpb * k.rowblock_bytes < (1ll << 31);
 }
 template <int XF16, int RPB, int RING, bool ONE>
@@ -920,7 +924,8 @@ static int nvq_launch_signed_as(const NvqK &k, const uint8_t *w, const uint16_t 
                                            static_cast<int>(lds));
         MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nvq_signed: %s", hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(ceil_div(k.n_rowblocks, RPB))), dim3(64 * nwaves), lds, st, k, w, x,
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(ceil_div(k.n_rowblocks, RPB)), static_cast<unsigned>(ceil_div(M, 16))),
+                       dim3(64 * nwaves), lds, st, k, w, x,
                        ldx, M, y, ldy, spw);
     return check_launch("nvq_signed");
 }
