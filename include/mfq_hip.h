@@ -202,6 +202,13 @@ int mfq_hip_nvq_dequant_f32(const mfq_nvq_desc *d, const void *weight, float *w_
 /* Replaces nvq_gemv_ws_cuda (cpp_runtime/mfq_decode.cpp:555-559). */
 int mfq_hip_nvq_gemv(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
                      int M, float *y, int64_t ldy, mfq_stream_t stream);
+/* Two projections of the same activations in one launch: y[m, 0:out0] = x . W0^T, y[m, out0:out0+out1] = x . W1^T
+ * (both tensors with the same neuron_len).  Up to 32 rows on tensors the signed-table kernel takes it is one launch
+ * whose blocks are shared out over both tensors; otherwise the two mfq_hip_nvq_gemv calls.  Same values as those two
+ * calls.  Replaces nvq_gemv_multi2_ws_cuda (called by nvq_matmul_multi2, cpp_runtime/mfq_decode.cpp:7981-8003). */
+int mfq_hip_nvq_gemv_multi2(const mfq_nvq_desc *d0, const void *weight0, const mfq_nvq_desc *d1, const void *weight1,
+                            const void *x, int x_dtype, int64_t ldx, int M, float *y, int64_t ldy,
+                            mfq_stream_t stream);
 /* Any-M entry: the streaming kernels of mfq_hip_nvq_gemv up to a crossover of 32 to 512 rows, above that a
  * block-tiled MFMA GEMM that builds the weight fragments from the codebooks (neuron_len % 8 == 0), else
  * dequantize-to-fp16 + MFMA GEMM.  Replaces nvq_mmq_* / nvq_gemm_f16_cuda / dequant + cuBLAS

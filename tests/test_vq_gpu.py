@@ -77,6 +77,34 @@ def test_nvq_signed_table_kernel_row_blocks_per_block(monkeypatch, rpb, K):
             _check(nvq_matmul(lin.weight, x, force="gemv").cpu().numpy(), O.linear_forward_f64(want, xf))
 
 
+@pytest.mark.parametrize("cu", ["8", "256"])
+def test_nvq_two_projections_in_one_launch(monkeypatch, cu):
+    """Two tensors that share their input: the joint launch gives exactly what the two separate calls give (bit for
+    bit: same kernel, same order of sums), for one- and two-bank codebooks, different heights, 1 to 32 rows; with the
+    grid sized for 8 CUs the blocks hold several row-blocks.  A four-bank tensor takes the two-call path."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import nvq_matmul, nvq_matmul_multi2
+    monkeypatch.setenv("MFQ_CU_COUNT", cu)
+    rng = np.random.default_rng(950 + int(cu))
+    K = 1560
+    specs = [(("d4_512", 2), 250), (("d4_512", 1), 123), (("d4_256", 2), 64), (("d4_512", 4), 80)]
+    lins = []
+    for (cb, banks), out in specs:
+        dtype, blob = O.pack_tensor(synth.nvq_jsc_random(rng, out, K, cb, banks))
+        lins.append(R.load_quant_linear(dtype, blob))
+    for a, b in ((0, 1), (1, 2), (2, 0), (0, 3)):
+        for M, xd in ((1, torch.bfloat16), (8, torch.float16), (17, torch.bfloat16), (32, torch.bfloat16), (40, torch.bfloat16)):
+            x, xf = _x(rng, M, K, xd)
+            got = nvq_matmul_multi2(lins[a].weight, lins[b].weight, x)
+            force = "gemv" if M <= 32 else None
+            want = torch.cat([nvq_matmul(lins[a].weight, x, force=force), nvq_matmul(lins[b].weight, x, force=force)], dim=-1)
+            assert got.shape == (M, lins[a].out + lins[b].out)
+            assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    with pytest.raises(ValueError, match="compatible formats"):
+        other = R.load_quant_linear(*O.pack_tensor(synth.nvq_jsc_random(rng, 32, 96, "d4_512", 2)))
+        nvq_matmul_multi2(lins[0].weight, other.weight, torch.zeros((1, K), dtype=torch.bfloat16, device="cuda"))
+
+
 @pytest.mark.parametrize("out,K,M,banks", [(130, 1024, 520, 2), (96, 4104, 600, 4), (272, 1024, 8300, 2),
                                           (1040, 1024, 3329, 2)])
 def test_nvq_prefill_kernel(out, K, M, banks):

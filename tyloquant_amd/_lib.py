@@ -76,6 +76,7 @@ _SIGS = {
     "mfq_hip_nvq_repack_plain": (C.c_int, [C.POINTER(NvqDesc), vp, i64, vp, vp, vp]),
     "mfq_hip_nvq_dequant_f32": (C.c_int, [C.POINTER(NvqDesc), vp, vp, i64, vp]),
     "mfq_hip_nvq_gemv": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
+    "mfq_hip_nvq_gemv_multi2": (C.c_int, [C.POINTER(NvqDesc), vp, C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
     "mfq_hip_nvq_gemm_workspace_bytes": (sz, [C.POINTER(NvqDesc), C.c_int]),
     "mfq_hip_nvq_gemm": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
     "mfq_hip_nepq_plan": (C.c_int, [C.c_int] * 4 + [C.POINTER(NepqDesc)]),

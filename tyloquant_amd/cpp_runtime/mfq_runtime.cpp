@@ -347,6 +347,23 @@ void nvq_matmul(const NvqWeight &w, const void *x, int x_dtype, int64_t ldx, int
     w.workspace.ensure(need);
     abi_check(mfq_hip_nvq_gemm(&w.desc, w.data.get(), x, x_dtype, ldx, M, y, w.desc.out, w.workspace.get(), need, stream));
 }
+void nvq_matmul_multi2(const NvqWeight &first, const NvqWeight &second, const void *x, int x_dtype, int64_t ldx, int M,
+                       float *y, mfq_stream_t stream) {
+    if (first.desc.neuron_len != second.desc.neuron_len) fail("NVQ multi-projection requires compatible formats and input layouts");
+    const int64_t N = static_cast<int64_t>(first.desc.out) + second.desc.out;
+    if (M <= 32) {
+        abi_check(mfq_hip_nvq_gemv_multi2(&first.desc, first.data.get(), &second.desc, second.data.get(), x, x_dtype, ldx, M, y, N,
+                                          stream));
+        return;
+    }
+    // larger batches: the two matmuls, each into its columns
+    for (const NvqWeight *w : {&first, &second}) {
+        const size_t need = mfq_hip_nvq_gemm_workspace_bytes(&w->desc, M);
+        w->workspace.ensure(need);
+        abi_check(mfq_hip_nvq_gemm(&w->desc, w->data.get(), x, x_dtype, ldx, M, y + (w == &second ? first.desc.out : 0), N,
+                                   w->workspace.get(), need, stream));
+    }
+}
 void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                  mfq_stream_t stream) {
     if (expert < 0 || expert >= w.n_experts) fail("expert outside the NEPQ tensor");

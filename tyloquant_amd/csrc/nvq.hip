@@ -461,10 +461,22 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
 // LDS map (bytes): [signed table: banks*entries*128][state table: 16 x {lut pair, bank base}][red: waves * 1024]
 // [codebook entries as fp16 pairs: banks*entries*8]
 typedef const __attribute__((address_space(3))) u32x2_t *lds_u32x2_ptr;
+struct NvqSecond {  // the second tensor of a two-projection launch; blocks0 = grid.x when there is none
+    NvqK k;
+    const uint8_t *w;
+    int blocks0, col;
+};
 template <int XF16, int RPB, int RING, bool ONE>
-__global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k, const uint8_t *__restrict__ w,
+__global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k_first, const uint8_t *__restrict__ w_first,
                                                           const uint16_t *__restrict__ x, int64_t ldx, int M,
-                                                          float *__restrict__ y, int64_t ldy, int spw) {
+                                                          float *__restrict__ y_first, int64_t ldy, int spw, NvqSecond s2) {
+    // blocks from s2.blocks0 on belong to a second tensor of the same neuron length (same activations), whose
+    // outputs follow the first tensor's in each row of y
+    const bool second = static_cast<int>(blockIdx.x) >= s2.blocks0;
+    const NvqK &k = second ? s2.k : k_first;
+    const uint8_t *__restrict__ w = second ? s2.w : w_first;
+    float *__restrict__ y = y_first + (second ? s2.col : 0);
+    const int bx = static_cast<int>(blockIdx.x) - (second ? s2.blocks0 : 0);
     // item (step ls, row-block i) lives in ring[i % RING]: the ring depth divides the row-blocks of a step
     static_assert(ONE ? RING <= RPB : RPB % RING == 0, "ring slots are chosen at compile time");
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
@@ -477,7 +489,7 @@ __global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k, const uint8_t 
     const uint32_t lds_base = static_cast<uint32_t>(
         reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint32_t *)lds));
 
-    const int rb_first = blockIdx.x * RPB;
+    const int rb_first = bx * RPB;
     const int nrb = min(RPB, k.n_rowblocks - rb_first);  // row-blocks of this block
     const int m0 = static_cast<int>(blockIdx.y) * 16;  // the block's 16-row tile
     const int tok = min(m0 + static_cast<int>(lane & 15), M - 1);
@@ -902,10 +914,12 @@ static int nvq_launch_mfma(const NvqK &k, const uint8_t *w, const uint16_t *x, i
 }
 
 // 16-row tiles through nvq_signed_kernel: at most one block per CU and tile, each with up to six row-blocks
-static int nvq_signed_rpb(const NvqK &k) { return static_cast<int>(ceil_div(k.n_rowblocks, gemv_cu_count())); }
-static bool nvq_signed_capable(const NvqK &k, int M) {
+static int nvq_signed_rpb(const NvqK &k, int more_rowblocks = 0) {
+    return static_cast<int>(ceil_div(k.n_rowblocks + more_rowblocks, gemv_cu_count()));
+}
+static bool nvq_signed_capable(const NvqK &k, int M, int more_rowblocks = 0) {
     static const int off = [] { const char *e = getenv("MFQ_NVQ_SIGNED_OFF"); return e ? atoi(e) : 0; }();
-    const int rpb = nvq_signed_rpb(k);
+    const int rpb = nvq_signed_rpb(k, more_rowblocks);
     // two 16-row tiles still beat the older streaming kernel and the prefill kernel on the config 3 tensors
     // (17408 x 5120 at M = 32: 42 us against 54 and 46); MFQ_NVQ_SIGNED_MAX_M for tuning
     static const int max_m = [] { const char *e = getenv("MFQ_NVQ_SIGNED_MAX_M"); return e ? atoi(e) : 32; }();
@@ -914,50 +928,59 @@ static bool nvq_signed_capable(const NvqK &k, int M) {
 }
 template <int XF16, int RPB, int RING, bool ONE>
 static int nvq_launch_signed_as(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y,
-                                int64_t ldy, hipStream_t st) {
+                                int64_t ldy, hipStream_t st, const NvqSecond *second) {
     const int spw = static_cast<int>(ceil_div(k.nsteps, 16));
     const int nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
-    const size_t lds = static_cast<size_t>(k.banks) * k.entries * 136 + 128 + static_cast<size_t>(nwaves) * 1024;
+    const int blocks0 = static_cast<int>(ceil_div(k.n_rowblocks, RPB));
+    NvqSecond s2{k, w, blocks0, 0};
+    int blocks = blocks0;
+    size_t ncb = static_cast<size_t>(k.banks) * k.entries;
+    if (second) {
+        s2 = *second;
+        s2.blocks0 = blocks0;
+        blocks += static_cast<int>(ceil_div(s2.k.n_rowblocks, RPB));
+        if (static_cast<size_t>(s2.k.banks) * s2.k.entries > ncb) ncb = static_cast<size_t>(s2.k.banks) * s2.k.entries;
+    }
+    const size_t lds = ncb * 136 + 128 + static_cast<size_t>(nwaves) * 1024;
     auto kern = nvq_signed_kernel<XF16, RPB, RING, ONE>;
     if (lds > 65536) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            static_cast<int>(lds));
         MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nvq_signed: %s", hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(ceil_div(k.n_rowblocks, RPB)), static_cast<unsigned>(ceil_div(M, 16))),
-                       dim3(64 * nwaves), lds, st, k, w, x,
-                       ldx, M, y, ldy, spw);
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks), static_cast<unsigned>(ceil_div(M, 16))), dim3(64 * nwaves), lds,
+                       st, k, w, x, ldx, M, y, ldy, spw, s2);
     return check_launch("nvq_signed");
 }
 template <int XF16>
 static int nvq_launch_signed(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
-                             hipStream_t st) {
+                             hipStream_t st, const NvqSecond *s2 = nullptr) {
     // ring depths: what fits in 128 registers beside the activation fragments (48) and the accumulators
-    const int rpb = nvq_signed_rpb(k);
+    const int rpb = nvq_signed_rpb(k, s2 ? s2->k.n_rowblocks : 0);
     if (k.nsteps <= 16) {  // one step per wave
         switch (rpb) {
-        case 1: return nvq_launch_signed_as<XF16, 1, 1, true>(k, w, x, ldx, M, y, ldy, st);
-        case 2: return nvq_launch_signed_as<XF16, 2, 2, true>(k, w, x, ldx, M, y, ldy, st);
-        case 3: return nvq_launch_signed_as<XF16, 3, 3, true>(k, w, x, ldx, M, y, ldy, st);
-        case 4: return nvq_launch_signed_as<XF16, 4, 3, true>(k, w, x, ldx, M, y, ldy, st);
+        case 1: return nvq_launch_signed_as<XF16, 1, 1, true>(k, w, x, ldx, M, y, ldy, st, s2);
+        case 2: return nvq_launch_signed_as<XF16, 2, 2, true>(k, w, x, ldx, M, y, ldy, st, s2);
+        case 3: return nvq_launch_signed_as<XF16, 3, 3, true>(k, w, x, ldx, M, y, ldy, st, s2);
+        case 4: return nvq_launch_signed_as<XF16, 4, 3, true>(k, w, x, ldx, M, y, ldy, st, s2);
         case 5: {
             // ring depths 1 .. 4 run within 7 % of each other on 17408 x 5120 (two is the fastest): MFQ_NVQ_RING for tuning
             static const int ring = [] { const char *e = getenv("MFQ_NVQ_RING"); return e ? atoi(e) : 2; }();
-            if (ring == 1) return nvq_launch_signed_as<XF16, 5, 1, true>(k, w, x, ldx, M, y, ldy, st);
-            if (ring == 3) return nvq_launch_signed_as<XF16, 5, 3, true>(k, w, x, ldx, M, y, ldy, st);
-            if (ring == 4) return nvq_launch_signed_as<XF16, 5, 4, true>(k, w, x, ldx, M, y, ldy, st);
-            return nvq_launch_signed_as<XF16, 5, 2, true>(k, w, x, ldx, M, y, ldy, st);
+            if (ring == 1) return nvq_launch_signed_as<XF16, 5, 1, true>(k, w, x, ldx, M, y, ldy, st, s2);
+            if (ring == 3) return nvq_launch_signed_as<XF16, 5, 3, true>(k, w, x, ldx, M, y, ldy, st, s2);
+            if (ring == 4) return nvq_launch_signed_as<XF16, 5, 4, true>(k, w, x, ldx, M, y, ldy, st, s2);
+            return nvq_launch_signed_as<XF16, 5, 2, true>(k, w, x, ldx, M, y, ldy, st, s2);
         }
-        default: return nvq_launch_signed_as<XF16, 6, 3, true>(k, w, x, ldx, M, y, ldy, st);
+        default: return nvq_launch_signed_as<XF16, 6, 3, true>(k, w, x, ldx, M, y, ldy, st, s2);
         }
     }
     switch (rpb) {
-    case 1: return nvq_launch_signed_as<XF16, 1, 1, false>(k, w, x, ldx, M, y, ldy, st);
-    case 2: return nvq_launch_signed_as<XF16, 2, 2, false>(k, w, x, ldx, M, y, ldy, st);
-    case 3: return nvq_launch_signed_as<XF16, 3, 3, false>(k, w, x, ldx, M, y, ldy, st);
-    case 4: return nvq_launch_signed_as<XF16, 4, 2, false>(k, w, x, ldx, M, y, ldy, st);
-    case 5: return nvq_launch_signed_as<XF16, 5, 1, false>(k, w, x, ldx, M, y, ldy, st);
-    default: return nvq_launch_signed_as<XF16, 6, 1, false>(k, w, x, ldx, M, y, ldy, st);
+    case 1: return nvq_launch_signed_as<XF16, 1, 1, false>(k, w, x, ldx, M, y, ldy, st, s2);
+    case 2: return nvq_launch_signed_as<XF16, 2, 2, false>(k, w, x, ldx, M, y, ldy, st, s2);
+    case 3: return nvq_launch_signed_as<XF16, 3, 3, false>(k, w, x, ldx, M, y, ldy, st, s2);
+    case 4: return nvq_launch_signed_as<XF16, 4, 2, false>(k, w, x, ldx, M, y, ldy, st, s2);
+    case 5: return nvq_launch_signed_as<XF16, 5, 1, false>(k, w, x, ldx, M, y, ldy, st, s2);
+    default: return nvq_launch_signed_as<XF16, 6, 1, false>(k, w, x, ldx, M, y, ldy, st, s2);
     }
 }
 
@@ -1108,6 +1131,32 @@ extern "C" int mfq_hip_nvq_gemv(const mfq_nvq_desc *d, const void *weight, const
     MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvq_gemv: x_dtype=%d", x_dtype);
     MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nvq_gemv: ldx/ldy smaller than the tensor");
     return nvq_gemv_any(d, weight, x, x_dtype, ldx, M, y, ldy, as_stream(stream));
+}
+
+extern "C" int mfq_hip_nvq_gemv_multi2(const mfq_nvq_desc *d0, const void *weight0, const mfq_nvq_desc *d1, const void *weight1,
+                                       const void *x, int x_dtype, int64_t ldx, int M, float *y, int64_t ldy,
+                                       mfq_stream_t stream) {
+    MFQ_REQUIRE(d0 && d1 && weight0 && weight1 && x && y, MFQ_ERR_INVALID, "nvq_gemv_multi2: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nvq_gemv_multi2: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvq_gemv_multi2: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(d0->neuron_len == d1->neuron_len, MFQ_ERR_INVALID,
+                "NVQ multi-projection requires compatible formats and input layouts");
+    MFQ_REQUIRE(ldx >= d0->neuron_len && ldy >= static_cast<int64_t>(d0->out) + d1->out, MFQ_ERR_INVALID,
+                "nvq_gemv_multi2: ldx/ldy smaller than the tensors");
+    const NvqK k0 = to_k(d0), k1 = to_k(d1);
+    hipStream_t st = as_stream(stream);
+    const bool aligned = ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    if (aligned && nvq_stream_capable(k0) && nvq_stream_capable(k1) && nvq_signed_capable(k0, M, k1.n_rowblocks) &&
+        nvq_signed_capable(k1, M, k0.n_rowblocks)) {
+        const NvqSecond s2{k1, static_cast<const uint8_t *>(weight1), 0, d0->out};
+        const uint8_t *w0 = static_cast<const uint8_t *>(weight0);
+        const uint16_t *xp = static_cast<const uint16_t *>(x);
+        return x_dtype == MFQ_X_F16 ? nvq_launch_signed<1>(k0, w0, xp, ldx, M, y, ldy, st, &s2)
+                                    : nvq_launch_signed<0>(k0, w0, xp, ldx, M, y, ldy, st, &s2);
+    }
+    const int rc = nvq_gemv_any(d0, weight0, x, x_dtype, ldx, M, y, ldy, st);
+    if (rc) return rc;
+    return nvq_gemv_any(d1, weight1, x, x_dtype, ldx, M, y + d0->out, ldy, st);
 }
 
 // The reference keeps the D4 family on its GEMV up to M = 13; tensors the matrix-core streaming kernel

@@ -61,6 +61,21 @@ class NvqWeight:
         return w
 
 
+def nvq_matmul_multi2(first: NvqWeight, second: NvqWeight, x: torch.Tensor) -> torch.Tensor:
+    """cat(x @ W0^T, x @ W1^T) for two NVQ tensors that share their input, in one launch for small batches
+    (nvq_matmul_multi2, cpp_runtime/mfq_decode.cpp:7981-8003)."""
+    if first.neuron_len != second.neuron_len:
+        raise ValueError("NVQ multi-projection requires compatible formats and input layouts")
+    x2 = _as_2d(x, first.neuron_len)
+    M, N = x2.shape[0], first.out + second.out
+    if M > 32:
+        return torch.cat([nvq_matmul(first, x), nvq_matmul(second, x)], dim=-1)
+    y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    L.check(L.lib().mfq_hip_nvq_gemv_multi2(C.byref(first.desc), _ptr(first.data), C.byref(second.desc), _ptr(second.data),
+                                            _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y), N, _stream()))
+    return y.reshape(*x.shape[:-1], N)
+
+
 def nvq_matmul(w: NvqWeight, x: torch.Tensor, *, force: str | None = None) -> torch.Tensor:
     """cpp_runtime/mfq_decode.cpp:7884: GEMV up to M = 13 for the D4 family, MFMA path above."""
     x2 = _as_2d(x, w.neuron_len)
