@@ -100,6 +100,14 @@ def test_nvq_two_projections_in_one_launch(monkeypatch, cu):
             want = torch.cat([nvq_matmul(lins[a].weight, x, force=force), nvq_matmul(lins[b].weight, x, force=force)], dim=-1)
             assert got.shape == (M, lins[a].out + lins[b].out)
             assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    from tyloquant_amd.runtime_vq import nvq_matmul_swiglu
+    g, u = lins[0].weight, R.load_quant_linear(*O.pack_tensor(synth.nvq_jsc_random(rng, 250, K, "d4_512", 1))).weight
+    x, xf = _x(rng, 3, K)
+    h = nvq_matmul_swiglu(g, u, x).float().cpu().numpy()
+    yg, yu = nvq_matmul(g, x).cpu().numpy(), nvq_matmul(u, x).cpu().numpy()
+    assert rel_l2(h, O.moe_swiglu(np.concatenate([yg, yu], axis=-1))) < 1e-3      # fp16 output
+    with pytest.raises(ValueError, match="equal-width"):
+        nvq_matmul_swiglu(lins[0].weight, lins[1].weight, x)
     with pytest.raises(ValueError, match="compatible formats"):
         other = R.load_quant_linear(*O.pack_tensor(synth.nvq_jsc_random(rng, 32, 96, "d4_512", 2)))
         nvq_matmul_multi2(lins[0].weight, other.weight, torch.zeros((1, K), dtype=torch.bfloat16, device="cuda"))

@@ -364,6 +364,15 @@ void nvq_matmul_multi2(const NvqWeight &first, const NvqWeight &second, const vo
                                    w->workspace.get(), need, stream));
     }
 }
+void nvq_matmul_swiglu(const NvqWeight &gate, const NvqWeight &up, const void *x, int x_dtype, int64_t ldx, int M, void *hidden,
+                       float *scratch, mfq_stream_t stream) {
+    if (gate.desc.neuron_len != up.desc.neuron_len || gate.desc.out != up.desc.out)
+        fail("NVQ SwiGLU requires compatible equal-width gate/up weights");
+    if (!scratch) fail("nvq_matmul_swiglu: needs a [M, 2W] fp32 scratch buffer");
+    const int W = gate.desc.out;
+    nvq_matmul_multi2(gate, up, x, x_dtype, ldx, M, scratch, stream);
+    abi_check(mfq_hip_moe_swiglu(scratch, 2 * W, M, W, hidden, MFQ_X_F16, W, stream));
+}
 void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                  mfq_stream_t stream) {
     if (expert < 0 || expert >= w.n_experts) fail("expert outside the NEPQ tensor");

@@ -159,6 +159,10 @@ void nint_dequantize(const NintWeight &w, float *out, mfq_stream_t stream = null
 // y[M, out0 + out1] = cat(x . W0^T, x . W1^T) for two tensors that share their input (nvq_matmul_multi2 :7981-8003)
 void nvq_matmul_multi2(const NvqWeight &first, const NvqWeight &second, const void *x, int x_dtype, int64_t ldx, int M,
                        float *y, mfq_stream_t stream = nullptr);
+// hidden fp16 [M, W] = silu(x . Wg^T) * (x . Wu^T) for an equal-width gate/up pair (nvq_matmul_swiglu :8004-8029):
+// nvq_matmul_multi2 into `scratch` (fp32 [M, 2W]) + the SwiGLU kernel
+void nvq_matmul_swiglu(const NvqWeight &gate, const NvqWeight &up, const void *x, int x_dtype, int64_t ldx, int M,
+                       void *hidden, float *scratch, mfq_stream_t stream = nullptr);
 void nvq_dequantize(const NvqWeight &w, float *out, mfq_stream_t stream = nullptr);
 // the q8_zero branch of nint_matmul (:8165-8185) and nint8_zero_dequant_cuda
 void nint8_zero_matmul(const Nint8ZeroWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y,

@@ -76,6 +76,15 @@ def nvq_matmul_multi2(first: NvqWeight, second: NvqWeight, x: torch.Tensor) -> t
     return y.reshape(*x.shape[:-1], N)
 
 
+def nvq_matmul_swiglu(gate: NvqWeight, up: NvqWeight, x: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """silu(x @ Wg^T) * (x @ Wu^T) for an NVQ gate/up pair (nvq_matmul_swiglu, cpp_runtime/mfq_decode.cpp:8004-8029): the
+    joint two-projection launch followed by the elementwise SwiGLU kernel (the reference fuses the two for one row)."""
+    if gate.neuron_len != up.neuron_len or gate.out != up.out:
+        raise ValueError("NVQ SwiGLU requires compatible equal-width gate/up weights")
+    from .runtime_moe import moe_swiglu
+    return moe_swiglu(nvq_matmul_multi2(gate, up, x), out_dtype)
+
+
 def nvq_matmul(w: NvqWeight, x: torch.Tensor, *, force: str | None = None) -> torch.Tensor:
     """cpp_runtime/mfq_decode.cpp:7884: GEMV up to M = 13 for the D4 family, MFMA path above."""
     x2 = _as_2d(x, w.neuron_len)
