@@ -38,6 +38,8 @@ def rt():
     lib.mfq_rt_moe_ffn_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p,
                                            C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                            C.c_void_p, C.c_void_p]
+    lib.mfq_rt_nvq_ffn_swiglu_down.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int,
+                                               C.c_void_p, C.c_void_p]
     return lib
 
 
@@ -175,3 +177,28 @@ def test_cpp_moe_ffn_forward(rt, T):
     check_close(out.cpu().numpy(), ref)
     rt.mfq_rt_free_nint_moe(hg)
     rt.mfq_rt_free_nint_moe(hd)
+
+
+def test_cpp_nvq_ffn_swiglu_down(rt):
+    """nvq_ffn_swiglu_down of the C++ runtime (joint gate/up launch, SwiGLU kernel, down projection) against the
+    oracle's float64 evaluation of the dequantized weights; the hidden rows pass through fp16."""
+    from conftest import rel_l2
+    rng = np.random.default_rng(8071)
+    K, W, out = 1560, 240, 72
+    blobs = [O.pack_tensor(synth.nvq_jsc_random(rng, W, K, "d4_512", 2)),
+             O.pack_tensor(synth.nvq_jsc_random(rng, W, K, "d4_512", 1)),
+             O.pack_tensor(synth.nvq_jsc_random(rng, out, W, "d4_512", 2))]
+    hs = [_load(rt, d, b) for d, b in blobs]
+    wg, wu, wd = (O.dequantize_nvq_jsc(O.unpack_nvq(b)) for _, b in blobs)
+    for M in (1, 6, 40):
+        x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+        y = torch.empty((M, out), dtype=torch.float32, device="cuda")
+        assert rt.mfq_rt_nvq_ffn_swiglu_down(hs[0], hs[1], hs[2], x.data_ptr(), 0, K, M, y.data_ptr(), None) == 0
+        torch.cuda.synchronize()
+        xf = x.float().cpu().numpy()
+        g, u = O.linear_forward_f64(wg, xf), O.linear_forward_f64(wu, xf)
+        assert rel_l2(y.cpu().numpy(), O.linear_forward_f64(wd, g / (1.0 + np.exp(-g)) * u)) < 2e-3
+    assert rt.mfq_rt_nvq_ffn_swiglu_down(hs[0], hs[1], hs[0], x.data_ptr(), 0, K, 1, y.data_ptr(), None) == 1
+    assert "fused FFN weight layouts" in rt.mfq_rt_last_error().decode()
+    for h in hs:
+        rt.mfq_rt_free_quant_linear(h)

@@ -241,3 +241,27 @@ def test_vq_loader_errors():
         R.load_quant_linear("NEPQ1-S", nb + b"\0")
     with pytest.raises(ValueError, match="dtype/blob mismatch"):
         R.load_quant_linear("NEPQ1-L", nb)
+
+
+def test_nvq_ffn_swiglu_down():
+    """Feed-forward block of three NVQ tensors against the oracle's float64 evaluation of the dequantized weights
+    (the comparison the reference's tests/test_nvq_kernels_cuda.py:655-675 makes with its unfused path); the hidden
+    rows are rounded to fp16 between the two stages, hence the looser bound.  Mismatched widths raise."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import nvq_ffn_swiglu_down
+    rng = np.random.default_rng(8032)
+    K, W, out = 1560, 240, 72
+    blobs = [O.pack_tensor(synth.nvq_jsc_random(rng, W, K, "d4_512", 2)),
+             O.pack_tensor(synth.nvq_jsc_random(rng, W, K, "d4_512", 1)),
+             O.pack_tensor(synth.nvq_jsc_random(rng, out, W, "d4_512", 2))]
+    gate, up, down = (R.load_quant_linear(d, b).weight for d, b in blobs)
+    wg, wu, wd = (O.dequantize_nvq_jsc(O.unpack_nvq(b)) for _, b in blobs)
+    for M in (1, 5, 40):
+        x, xf = _x(rng, M, K)
+        got = nvq_ffn_swiglu_down(gate, up, down, x).cpu().numpy()
+        g, u = O.linear_forward_f64(wg, xf), O.linear_forward_f64(wu, xf)
+        want = O.linear_forward_f64(wd, g / (1.0 + np.exp(-g)) * u)
+        assert got.shape == (M, out)
+        assert rel_l2(got, want) < 2e-3
+    with pytest.raises(ValueError, match="fused FFN weight layouts"):
+        nvq_ffn_swiglu_down(gate, up, gate, x)

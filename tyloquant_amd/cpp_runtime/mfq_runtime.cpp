@@ -373,6 +373,14 @@ void nvq_matmul_swiglu(const NvqWeight &gate, const NvqWeight &up, const void *x
     nvq_matmul_multi2(gate, up, x, x_dtype, ldx, M, scratch, stream);
     abi_check(mfq_hip_moe_swiglu(scratch, 2 * W, M, W, hidden, MFQ_X_F16, W, stream));
 }
+void nvq_ffn_swiglu_down(const NvqWeight &gate, const NvqWeight &up, const NvqWeight &down, const void *x, int x_dtype,
+                         int64_t ldx, int M, float *y, void *hidden, float *scratch, mfq_stream_t stream) {
+    if (gate.desc.neuron_len != up.desc.neuron_len || gate.desc.out != up.desc.out || gate.desc.out != down.desc.neuron_len)
+        fail("NVQ fused FFN weight layouts are incompatible");
+    if (!hidden) fail("nvq_ffn_swiglu_down: needs a [M, W] fp16 buffer for the hidden rows");
+    nvq_matmul_swiglu(gate, up, x, x_dtype, ldx, M, hidden, scratch, stream);
+    nvq_matmul(down, hidden, MFQ_X_F16, gate.desc.out, M, y, stream);
+}
 void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                  mfq_stream_t stream) {
     if (expert < 0 || expert >= w.n_experts) fail("expert outside the NEPQ tensor");
@@ -762,6 +770,23 @@ int mfq_rt_linear_check(void *h, int M, int reps, double *out6) {
         const LinearCheckResult r = run_linear_check(*static_cast<QuantLinear *>(h), M, reps);
         out6[0] = r.production_ms; out6[1] = r.production_weight_gbps; out6[2] = r.payload_gbps;
         out6[3] = r.production_rel; out6[4] = r.production_mean_abs; out6[5] = r.production_max_abs;
+    });
+}
+
+// Feed-forward block of three NVQ linears (handles from mfq_rt_load_quant_linear); the hidden rows and the joint
+// gate/up output live in buffers of this call, so the stream is synchronised before they go.
+int mfq_rt_nvq_ffn_swiglu_down(void *gate, void *up, void *down, const void *x, int x_dtype, int64_t ldx, int M, float *y,
+                               void *stream) {
+    return guard([&] {
+        const QuantLinear *g = static_cast<QuantLinear *>(gate), *u = static_cast<QuantLinear *>(up),
+                          *d = static_cast<QuantLinear *>(down);
+        if (g->kind != QuantLinearKind::Nvq || u->kind != QuantLinearKind::Nvq || d->kind != QuantLinearKind::Nvq)
+            throw std::runtime_error("nvq_ffn_swiglu_down takes three NVQ linears");
+        const size_t W = static_cast<size_t>(g->out());
+        DeviceBuffer hidden(static_cast<size_t>(M) * W * 2), scratch(static_cast<size_t>(M) * W * 8);
+        nvq_ffn_swiglu_down(*g->nvq, *u->nvq, *d->nvq, x, x_dtype, ldx, M, y, hidden.get(),
+                            static_cast<float *>(scratch.get()), static_cast<mfq_stream_t>(stream));
+        hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "sync");
     });
 }
 

@@ -163,6 +163,10 @@ void nvq_matmul_multi2(const NvqWeight &first, const NvqWeight &second, const vo
 // nvq_matmul_multi2 into `scratch` (fp32 [M, 2W]) + the SwiGLU kernel
 void nvq_matmul_swiglu(const NvqWeight &gate, const NvqWeight &up, const void *x, int x_dtype, int64_t ldx, int M,
                        void *hidden, float *scratch, mfq_stream_t stream = nullptr);
+// y fp32 [M, down.out] = Wd . hidden with hidden = nvq_matmul_swiglu(gate, up, x) (nvq_ffn_swiglu_down :8032-8071);
+// `hidden` is a fp16 [M, W] buffer and `scratch` a fp32 [M, 2W] one, both the caller's
+void nvq_ffn_swiglu_down(const NvqWeight &gate, const NvqWeight &up, const NvqWeight &down, const void *x, int x_dtype,
+                         int64_t ldx, int M, float *y, void *hidden, float *scratch, mfq_stream_t stream = nullptr);
 void nvq_dequantize(const NvqWeight &w, float *out, mfq_stream_t stream = nullptr);
 // the q8_zero branch of nint_matmul (:8165-8185) and nint8_zero_dequant_cuda
 void nint8_zero_matmul(const Nint8ZeroWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y,

@@ -85,6 +85,15 @@ def nvq_matmul_swiglu(gate: NvqWeight, up: NvqWeight, x: torch.Tensor, out_dtype
     return moe_swiglu(nvq_matmul_multi2(gate, up, x), out_dtype)
 
 
+def nvq_ffn_swiglu_down(gate: NvqWeight, up: NvqWeight, down: NvqWeight, x: torch.Tensor) -> torch.Tensor:
+    """Wd · (silu(Wg·x) * (Wu·x)) for an NVQ feed-forward block (nvq_ffn_swiglu_down, cpp_runtime/mfq_decode.cpp:8032-8071):
+    the gate/up launch, the SwiGLU kernel and the down projection on its fp16 output -- three launches where the
+    reference quantizes the hidden row to int8 inside one kernel for a single row."""
+    if gate.neuron_len != up.neuron_len or gate.out != up.out or gate.out != down.neuron_len:
+        raise ValueError("NVQ fused FFN weight layouts are incompatible")
+    return nvq_matmul(down, nvq_matmul_swiglu(gate, up, x))
+
+
 def nvq_matmul(w: NvqWeight, x: torch.Tensor, *, force: str | None = None) -> torch.Tensor:
     """cpp_runtime/mfq_decode.cpp:7884: GEMV up to M = 13 for the D4 family, MFMA path above."""
     x2 = _as_2d(x, w.neuron_len)
