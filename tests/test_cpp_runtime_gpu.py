@@ -90,6 +90,8 @@ def test_cpp_load_quant_linear_and_forward(rt):
         assert rt.mfq_rt_linear_forward(h, x.data_ptr(), 0, 88, M, y.data_ptr(), None) == 0
         torch.cuda.synchronize()
         check_close(y.cpu().numpy(), O.linear_forward_f64(deq, x.float().cpu().numpy()))
+    assert rt.mfq_rt_linear_forward(h, None, 0, 88, 0, None, None) == 0       # an empty batch launches nothing
+    assert rt.mfq_rt_linear_forward(h, x.data_ptr(), 0, 88, -1, y.data_ptr(), None) == 1
     rt.mfq_rt_free_quant_linear(h)
     with pytest.raises(RuntimeError, match="invalid NINT blob tail"):
         _load(rt, "NINT3", O.pack_nint(t)[:-1])

@@ -265,3 +265,34 @@ def test_nvq_ffn_swiglu_down():
         assert rel_l2(got, want) < 2e-3
     with pytest.raises(ValueError, match="fused FFN weight layouts"):
         nvq_ffn_swiglu_down(gate, up, gate, x)
+
+
+def test_empty_batch_returns_empty_outputs():
+    """A batch with no rows gives an empty output of the right shape and dtype from every host matmul (nothing is
+    launched; the C entry points themselves reject M < 1)."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_moe import moe_swiglu
+    from tyloquant_amd.runtime_vq import NepqWeight, nepq_matmul, nvq_ffn_swiglu_down, nvq_matmul, nvq_matmul_multi2
+    rng = np.random.default_rng(0)
+    nint = R.load_quant_linear("NINT4", O.pack_nint(O.quantize_nint(
+        (rng.standard_normal((64, 96)) * 0.02).astype(np.float32), 4, 32, 6)))
+    q8 = R.load_quant_linear("NINT8-0", O.pack_nint8_zero(O.quantize_nint8_zero(
+        (rng.standard_normal((24, 64)) * 0.02).astype(np.float32))))
+    vq = [R.load_quant_linear(*O.pack_tensor(synth.nvq_jsc_random(rng, o, k, "d4_512", 2))).weight
+          for o, k in ((48, 96), (48, 96), (24, 48))]
+    e = lambda *s: torch.zeros(s, dtype=torch.bfloat16, device="cuda")
+    y = nint.forward(e(0, 96))
+    assert y.shape == (0, 64) and y.dtype == torch.float32
+    assert nint.forward(e(2, 0, 96)).shape == (2, 0, 64)
+    assert R.nint_matmul_swiglu(nint.weight, e(0, 96)).shape == (0, 32)
+    assert R.nint_matmul_input_mul(nint.weight, e(0, 96), e(0, 96)).shape == (0, 64)
+    assert q8.forward(e(0, 64)).shape == (0, 24)
+    assert nvq_matmul(vq[0], e(0, 96)).shape == (0, 48)
+    assert nvq_matmul_multi2(vq[0], vq[1], e(0, 96)).shape == (0, 96)
+    assert nvq_ffn_swiglu_down(vq[0], vq[1], vq[2], e(0, 96)).shape == (0, 24)
+    assert moe_swiglu(torch.zeros((0, 64), device="cuda")).shape == (0, 32)
+    t = synth.nepq_random(rng, "NEPQ1-S", 2, 32, 256, 1)
+    w = NepqWeight.from_blob(O.pack_nepq(t))
+    assert nepq_matmul(w, e(0, 256), 1).shape == (0, 32)
+    with pytest.raises(ValueError, match="activation width"):
+        nint.forward(e(0, 95))

@@ -436,6 +436,7 @@ int64_t QuantLinear::payload_bytes() const {
          : kind == QuantLinearKind::Nepq ? nepq->desc.payload_bytes : nint8z->desc.payload_bytes;
 }
 void QuantLinear::forward(const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const {
+    if (M == 0) return;  // an empty batch: no rows to write
     if (kind == QuantLinearKind::Nint) nint_matmul(*nint, x, x_dtype, ldx, M, y, stream);
     else if (kind == QuantLinearKind::Nvq) nvq_matmul(*nvq, x, x_dtype, ldx, M, y, stream);
     else if (kind == QuantLinearKind::Nepq) nepq_matmul(*nepq, 0, x, x_dtype, ldx, M, y, stream);

@@ -145,6 +145,8 @@ def nint8_zero_matmul(w: Nint8ZeroWeight, x: torch.Tensor, *, force: str | None 
     x2 = _as_2d(x, w.neuron_len)
     M = x2.shape[0]
     y = torch.empty((M, w.out), dtype=torch.float32, device=x.device)
+    if M == 0:                                   # an empty batch: nothing to launch
+        return y.reshape(*x.shape[:-1], w.out)
     lib = L.lib()
     if force == "gemv":
         L.check(lib.mfq_hip_nint8z_gemv(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
@@ -163,6 +165,8 @@ def nint_matmul(w: NintWeight, x: torch.Tensor, *, force: str | None = None) -> 
     x2 = _as_2d(x, w.neuron_len)
     M = x2.shape[0]
     y = torch.empty((M, w.out), dtype=torch.float32, device=x.device)
+    if M == 0:                                   # an empty batch: nothing to launch
+        return y.reshape(*x.shape[:-1], w.out)
     lib = L.lib()
     if force == "gemv":
         L.check(lib.mfq_hip_nint_gemv(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
@@ -182,6 +186,8 @@ def _nint_matmul_glu(w: NintWeight, x: torch.Tensor, out_dtype, activation: int)
     x2 = _as_2d(x, w.neuron_len)
     M, W = x2.shape[0], w.out // 2
     d = w.desc
+    if M == 0:
+        return torch.empty((*x.shape[:-1], W), dtype=out_dtype, device=x.device)
     fused = M <= 2 and w.out % 32 == 0 and (d.kind == 1 or (d.bits == 5 and d.gs == 28))
     if not fused:
         from .runtime_moe import moe_glu
@@ -214,6 +220,8 @@ def nint_matmul_input_mul(w: NintWeight, x: torch.Tensor, gate: torch.Tensor, mo
     x2 = _as_2d(x, w.neuron_len)
     g2 = _as_2d(gate.to(x2.dtype), w.neuron_len)
     out = torch.empty((x2.shape[0], w.neuron_len), dtype=x2.dtype, device=x2.device)
+    if x2.shape[0] == 0:
+        return nint_matmul(w, x)
     L.check(L.lib().mfq_hip_input_gate(_ptr(x2), _ptr(g2), _x_dtype(x2), x2.stride(0), g2.stride(0), x2.shape[0],
                                        w.neuron_len, int(mode), _ptr(out), out.stride(0), _stream()))
     return nint_matmul(w, out.reshape(x.shape))

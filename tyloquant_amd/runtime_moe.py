@@ -212,6 +212,8 @@ def moe_glu(gate_up: torch.Tensor, out_dtype=torch.float16, activation: int = L.
     W = gate_up.shape[-1] // 2
     g2 = gate_up.reshape(-1, 2 * W)
     hidden = torch.empty((g2.shape[0], W), dtype=out_dtype, device=gate_up.device)
+    if g2.shape[0] == 0:
+        return hidden.reshape(*gate_up.shape[:-1], W)
     L.check(L.lib().mfq_hip_moe_glu(_ptr(g2), g2.stride(0), g2.shape[0], W, _ptr(hidden),
                                     L.X_F16 if out_dtype == torch.float16 else L.X_BF16, W, activation, _stream()))
     return hidden.reshape(*gate_up.shape[:-1], W)

@@ -71,6 +71,8 @@ def nvq_matmul_multi2(first: NvqWeight, second: NvqWeight, x: torch.Tensor) -> t
     if M > 32:
         return torch.cat([nvq_matmul(first, x), nvq_matmul(second, x)], dim=-1)
     y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    if M == 0:
+        return y.reshape(*x.shape[:-1], N)
     L.check(L.lib().mfq_hip_nvq_gemv_multi2(C.byref(first.desc), _ptr(first.data), C.byref(second.desc), _ptr(second.data),
                                             _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y), N, _stream()))
     return y.reshape(*x.shape[:-1], N)
@@ -99,6 +101,8 @@ def nvq_matmul(w: NvqWeight, x: torch.Tensor, *, force: str | None = None) -> to
     x2 = _as_2d(x, w.neuron_len)
     M = x2.shape[0]
     y = torch.empty((M, w.out), dtype=torch.float32, device=x.device)
+    if M == 0:                                   # an empty batch: nothing to launch
+        return y.reshape(*x.shape[:-1], w.out)
     lib = L.lib()
     if force == "gemv":
         L.check(lib.mfq_hip_nvq_gemv(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
@@ -156,6 +160,8 @@ class NepqWeight:
 def nepq_hadamard(x: torch.Tensor, signs: torch.Tensor, block: int) -> torch.Tensor:
     x2 = x.reshape(-1, x.shape[-1]).contiguous()
     out = torch.empty_like(x2)
+    if x2.shape[0] == 0:
+        return out.reshape(x.shape)
     L.check(L.lib().mfq_hip_nepq_hadamard(_ptr(x2), _x_dtype(x2), x2.stride(0), x2.shape[0], x2.shape[1], block,
                                           _ptr(signs), _ptr(out), out.stride(0), _stream()))
     return out.reshape(x.shape)
@@ -172,6 +178,8 @@ def nepq_matmul(w: NepqWeight, x: torch.Tensor, expert: int = 0, *, force: str |
     M = x2.shape[0]
     n = w.out_per_expert
     y = torch.empty((M, n), dtype=torch.float32, device=x.device)
+    if M == 0:
+        return y.reshape(*x.shape[:-1], n)
     lib = L.lib()
     row0 = expert * n
     if force == "gemv":
