@@ -231,6 +231,17 @@ def main() -> int:
         log(f"[bench] config 1 NINT3 4096x4096 M=1: {ms * 1e3:.2f} us, {extras['config1_nint3_gbps']:.0f} GB/s")
         del c1
 
+        # ---- NINT8-0 (Q8_0 blocks) 12288x4096, batch {1, 8}, 8 rotating copies (428 MB) ---------------
+        w8 = R.load_quant_linear(*synth.nint8_zero_blob(8, FF, H)).weight
+        c8 = [w8] + [clone_w(w8) for _ in range(7)]
+        for M in (1, 8):
+            x8 = bf16(synth.activations(rng, M, H))
+            ms = graph_ms(lambda: [R.nint8_zero_matmul(w, x8) for w in c8], 10) / len(c8)
+            extras[f"nint8_zero_M{M}_us"] = ms * 1e3
+            extras[f"nint8_zero_M{M}_gbps"] = w8.payload_bytes / (ms * 1e-3) / 1e9
+            log(f"[bench] NINT8-0 {FF}x{H} M={M}: {ms * 1e3:.2f} us, {extras[f'nint8_zero_M{M}_gbps']:.0f} GB/s of payload")
+        del c8, w8
+
         # ---- config 3: NVQ3J-512 17408x5120 and its transpose, batch {1,4,8}, 8 rotating copies -----
         for name, (n3, k3) in {"up": (17408, 5120), "down": (5120, 17408)}.items():
             w3 = synth.tile_rows(RV.NvqWeight.from_blob(synth.nvq3j512_blob(11, 1024, k3)[1]), n3)

@@ -62,6 +62,19 @@ def nvq3j512_blob(seed, out, K, banks=2):
     return "NVQ3J-512", blob
 
 
+def nint8_zero_blob(seed, out, K):
+    """(dtype, blob) of an [out, K] NINT8-0 tensor drawn in the packed domain: 34-byte blocks of an fp16 scale
+    U(1, 3) * 1e-4 and 32 int8 codes in [-127, 127] (block layout of mfq/formats/nint8_zero.py:84-124)."""
+    rng = np.random.default_rng(seed)
+    ng = K // 32
+    blocks = np.zeros((out, ng), dtype=np.dtype([("d", "<f2"), ("q", "i1", (32,))]))
+    blocks["d"] = rng.uniform(1e-4, 3e-4, (out, ng)).astype(np.float16)
+    blocks["q"] = rng.integers(-127, 128, (out, ng, 32), dtype=np.int8)
+    import struct
+    head = F._N8Z_HDR.pack(b"NI80", 0, K, 2) + struct.pack("<2q", out, K) + struct.pack("<II", out, ng)
+    return "NINT8-0", head + blocks.tobytes()
+
+
 def nepq1_blob(seed, label, out, K, banks=16, experts=1):
     rng = np.random.default_rng(seed)
     pid = F.NEPQ_PROFILE[label]
