@@ -57,9 +57,21 @@ def pack_bits(values, bits: int) -> bytes:
         return b""
     if bits == 8:
         return v.astype(np.uint8).tobytes()
-    shifts = np.arange(bits, dtype=np.uint32)
-    stream = ((v[:, None] >> shifts[None, :]) & 1).astype(np.uint8).reshape(-1)
-    return np.packbits(stream, bitorder="little").tobytes()
+    # 8 values fill exactly `bits` bytes: value i of such a run is OR-ed in at bit i * bits (bits <= 16, so it
+    # touches at most the three bytes from byte (i * bits) // 8)
+    n = v.size
+    n8 = (n + 7) // 8
+    vv = np.zeros(n8 * 8, dtype=np.uint32)
+    vv[:n] = v & ((1 << bits) - 1)
+    vv = vv.reshape(n8, 8)
+    by = np.zeros((n8, bits + 2), dtype=np.uint32)
+    for i in range(8):
+        k, sh = (i * bits) // 8, (i * bits) % 8
+        w = vv[:, i] << sh
+        by[:, k] |= w & 0xFF
+        by[:, k + 1] |= (w >> 8) & 0xFF
+        by[:, k + 2] |= (w >> 16) & 0xFF
+    return by[:, :bits].astype(np.uint8).reshape(-1)[: (n * bits + 7) // 8].tobytes()
 
 
 def unpack_bits(blob, off: int, count: int, bits: int):
@@ -69,10 +81,19 @@ def unpack_bits(blob, off: int, count: int, bits: int):
     if off + nbytes > len(blob):
         raise ValueError("truncated bit stream")
     packed = np.frombuffer(blob, dtype=np.uint8, count=nbytes, offset=off)
-    stream = np.unpackbits(packed, bitorder="little")[: count * bits].reshape(count, bits)
-    weights = (1 << np.arange(bits, dtype=np.uint32))
-    out = (stream.astype(np.uint32) * weights).sum(axis=1)
-    return out.astype(np.uint8 if bits <= 8 else np.uint16), off + nbytes
+    # 8 values occupy exactly `bits` bytes; value i of such a run starts at bit i * bits, i.e. inside the three
+    # bytes from byte (i * bits) // 8 (bits <= 16).  Same stream definition as one bit at a time, a few bytes of
+    # scratch per value.
+    n8 = (count + 7) // 8
+    by = np.zeros((n8, bits + 2), dtype=np.uint32)
+    flat = np.zeros(n8 * bits, dtype=np.uint8)
+    flat[:nbytes] = packed
+    by[:, :bits] = flat.reshape(n8, bits)
+    out = np.empty((n8, 8), dtype=np.uint8 if bits <= 8 else np.uint16)
+    for i in range(8):
+        k, sh = (i * bits) // 8, (i * bits) % 8
+        out[:, i] = ((by[:, k] | (by[:, k + 1] << 8) | (by[:, k + 2] << 16)) >> sh) & ((1 << bits) - 1)
+    return out.reshape(-1)[:count], off + nbytes
 
 
 def _f16_round(x):

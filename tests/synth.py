@@ -72,3 +72,64 @@ def moe_random(rng, E, out, K, bits_per_expert, quantize=False):
             t = nint_random(rng, len(ids) * out, K, b, gs, sb)
         pools.append(O.MoePool(ids, f"NINT{bits}", t))
     return O.NintMoeTensor((E, out, K), pools)
+
+
+# ---- full-size payloads drawn in the packed domain ---------------------------------------------------
+# Every bit pattern of the three NINT streams is a valid payload, so a tensor too large for the numpy quantizer
+# is the blob header + fp16 anchors + random stream bytes; the anchors are chosen so that the dequantized weights
+# are roughly zero-mean with standard deviation `sigma` (min anchor = scale anchor * (2^bits - 1) / 2).
+def _random_bytes(rng, n):
+    return rng.integers(0, 1 << 64, (n + 7) // 8, dtype=np.uint64, endpoint=False).view(np.uint8)[:n]
+
+
+def nint_packed_blob(rng, out, K, bits, gs, sb, sigma=0.02):
+    import struct
+    ng = -(-K // gs)
+    ls, lq = (1 << sb) - 1, (1 << bits) - 1
+    var = lambda n: ((n + 1) ** 2 - 1) / 12.0          # variance of a uniform draw from 0..n
+    c = lq / 2.0
+    v_ssq = (var(ls) + (ls / 2) ** 2) * (var(lq) + c * c) - (ls / 2 * c) ** 2
+    unit = math.sqrt(v_ssq + c * c * var(ls))
+    ns = (rng.uniform(0.7, 1.3, out) * sigma / unit).astype(np.float16)
+    nm = (ns.astype(np.float32) * c).astype(np.float16)
+    sub = (out * ng * sb + 7) // 8
+    head = O._NINT_HDR.pack(bits, sb, gs, 0, K) + struct.pack("<I", 2) + struct.pack("<2q", out, K) + \
+        struct.pack("<II", out, ng)
+    streams = _random_bytes(rng, 2 * sub + (out * ng * gs * bits + 7) // 8)
+    return b"".join([head, ns.tobytes(), nm.tobytes(), streams.tobytes()])
+
+
+def nint_blob_rows(blob, row0, nrows):
+    """Rows [row0, row0 + nrows) of a NINT blob as an oracle tensor (row0 a multiple of 8, so that every stream is
+    byte-aligned there), decoded with the oracle's own bit-stream reader."""
+    import struct
+    assert row0 % 8 == 0
+    bits, sb, gs, axis, K = O._NINT_HDR.unpack_from(blob, 0)
+    off = O._NINT_HDR.size
+    ndim = struct.unpack_from("<I", blob, off)[0]
+    off += 4 + 8 * ndim
+    out, ng = struct.unpack_from("<II", blob, off)
+    off += 8
+    ns = np.frombuffer(blob, dtype=np.float16, count=nrows, offset=off + 2 * row0).astype(np.float32)
+    nm = np.frombuffer(blob, dtype=np.float16, count=nrows, offset=off + 2 * out + 2 * row0).astype(np.float32)
+    off += 4 * out
+    sub = (out * ng * sb + 7) // 8
+    ss, _ = O.unpack_bits(blob, off + row0 * ng * sb // 8, nrows * ng, sb)
+    sm, _ = O.unpack_bits(blob, off + sub + row0 * ng * sb // 8, nrows * ng, sb)
+    q, _ = O.unpack_bits(blob, off + 2 * sub + row0 * ng * gs * bits // 8, nrows * ng * gs, bits)
+    return O.NintTensor(bits, gs, sb, (nrows, K), axis, K, q.reshape(nrows, ng, gs), ns, nm, ss.reshape(nrows, ng),
+                        sm.reshape(nrows, ng))
+
+
+def nintm_packed_blob(rng, E, out, K, bits_per_expert, sigma=0.02):
+    """NIM2 container with one packed-domain cohort per distinct bit width; returns (blob, [(ids, pool_blob)])."""
+    parts = [O._NIM_HDR.pack(b"NIM2", E, out, K, len(set(int(b) for b in bits_per_expert)))]
+    pools = []
+    for bits in sorted(set(int(b) for b in bits_per_expert)):
+        ids = np.flatnonzero(np.asarray(bits_per_expert) == bits).astype(np.int32)
+        b, gs, sb = MOE_PROFILES[bits]
+        pb = nint_packed_blob(rng, len(ids) * out, K, b, gs, sb, sigma)
+        db = f"NINT{bits}".encode("ascii")
+        parts += [O._NIM_POOL.pack(ids.size, len(db), len(pb), 0), ids.tobytes(), db, pb]
+        pools.append((ids, pb))
+    return b"".join(parts), pools
