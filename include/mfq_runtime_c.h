@@ -32,6 +32,12 @@ int mfq_rt_linear_argmax(void *handle, const void *x, int x_dtype, int64_t ldx, 
  * payload_gbps, production_rel, production_mean_abs, production_max_abs. */
 int mfq_rt_linear_check(void *handle, int M, int reps, double *out6);
 
+/* nvq_ffn_swiglu_down (cpp_runtime/mfq_decode.cpp:8032-8071): y[M, out(down)] = down(silu(gate x) * up x) for three
+ * NVQ linears loaded with mfq_rt_load_quant_linear.  The hidden rows live in buffers of this call, so it
+ * allocates and synchronises the stream before returning (not capturable; the C++ API takes caller buffers). */
+int mfq_rt_nvq_ffn_swiglu_down(void *gate, void *up, void *down, const void *x, int x_dtype, int64_t ldx, int M, float *y,
+                               void *stream);
+
 /* NINTM expert-wise tensors and nint_moe_ffn_forward (cpp_runtime/mfq_decode.cpp:3394-3416). */
 int mfq_rt_load_nint_moe(const void *blob, size_t n, void **handle);
 void mfq_rt_free_nint_moe(void *handle);

@@ -102,7 +102,14 @@ def test_library_exports_every_symbol_the_header_declares():
     lib = ctypes.CDLL(str(L.LIB_PATH))
     for name in declared:
         assert hasattr(lib, name), name
+    assert _dynamic_symbols(L.LIB_PATH, "mfq_hip_") == declared      # and nothing is exported that the header omits
     assert L.lib().mfq_hip_version() >= 1
+
+
+def _dynamic_symbols(path, prefix):
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", str(path)], check=True, capture_output=True, text=True).stdout
+    return sorted({ln.split()[-1] for ln in out.splitlines() if ln.split() and ln.split()[-1].startswith(prefix)})
 
 
 def test_plan_calls_need_no_gpu():
@@ -161,3 +168,72 @@ def test_runtime_library_exports_its_c_view():
     assert len(declared) >= 10
     for name in declared:
         assert hasattr(lib, name), name
+    assert _dynamic_symbols(path, "mfq_rt_") == declared             # header and library agree both ways
+
+
+def _rt():
+    path = ROOT / "tyloquant_amd" / "lib" / "libmfq_runtime.so"
+    if not path.exists():
+        pytest.skip("libmfq_runtime.so is not built")
+    lib = ctypes.CDLL(str(path))
+    lib.mfq_rt_last_error.restype = ctypes.c_char_p
+    return lib
+
+
+def _rt_load_error(lib, fn, *args):
+    handle = ctypes.c_void_p()
+    rc = fn(*args, ctypes.byref(handle))
+    assert rc != 0 and not handle.value
+    return lib.mfq_rt_last_error().decode()
+
+
+def test_cpp_parsers_reject_malformed_headers_without_touching_the_gpu():
+    """Headers are validated before any division or device call: a zero groupsize, a negative
+    neuron length, lengths whose sum wraps 64 bits.  Each is an error message, not a signal or an out-of-bounds read."""
+    import struct
+    lib = _rt()
+    rng = np.random.default_rng(5)
+    blob = bytearray(O.pack_tensor(synth.nvq_jsc_random(rng, 4, 48))[1])
+    bad = bytearray(blob)
+    struct.pack_into("<H", bad, 6, 0)                                   # groupsize 0
+    msg = _rt_load_error(lib, lib.mfq_rt_load_quant_linear, b"NVQ3J-512", bytes(bad), ctypes.c_size_t(len(bad)))
+    assert "must be positive" in msg
+    bad = bytearray(blob)
+    struct.pack_into("<i", bad, 12, -48)                                # negative neuron_len
+    assert "must be positive" in _rt_load_error(lib, lib.mfq_rt_load_quant_linear, b"NVQ3J-512", bytes(bad),
+                                                ctypes.c_size_t(len(bad)))
+    # NINTM: payload_len + runtime_len wraps to a small number
+    t = synth.moe_random(rng, 4, 16, 48, [4, 4, 3, 3])
+    nim = bytearray(O.pack_nint_moe(t))
+    struct.pack_into("<QQ", nim, 20 + 8, 2 ** 64 - 64, 128)
+    msg = _rt_load_error(lib, lib.mfq_rt_load_nint_moe, bytes(nim), ctypes.c_size_t(len(nim)))
+    assert "truncated NINTM v2 pool payload" in msg
+
+
+def test_mfq_directory_checks_of_the_reference_reader(tmp_path):
+    """mfq/formats/io.py:818-828: duplicate names and a records-end != file-size are errors, in both readers."""
+    import subprocess
+    rng = np.random.default_rng(6)
+    a = O.pack_tensor(synth.nint_random(rng, 4, 48, 3, 24, 5))
+    path = tmp_path / "x.mfq"
+    F.write_mfq(path, {"w": a}, version=1)
+    data = path.read_bytes()
+    assert list(F.read_mfq_directory(data)) == ["w"]
+    with pytest.raises(ValueError, match="length mismatch"):
+        F.read_mfq_directory(data + b"\0")
+    with pytest.raises(ValueError, match="truncated MFQ blob"):
+        F.read_mfq_directory(data[:-1])
+    # two records with one name: the directory of a one-tensor file written twice
+    head_end = data.index(b"NINT3") + 5 + 8
+    rec = data[data.index(b"\x01\x00\x00\x00w"):head_end]               # u32 len + name, u32 len + dtype, u64 bytes
+    dup = data[:data.index(b"\x01\x00\x00\x00w") - 4] + (2).to_bytes(4, "little") + rec + rec + data[head_end:] * 2
+    with pytest.raises(ValueError, match="duplicate MFQ tensor record"):
+        F.read_mfq_directory(dup)
+    tool = ROOT / "tyloquant_amd" / "lib" / "mfq-check-linear"
+    if tool.exists():
+        for payload, want in ((dup, "duplicate MFQ tensor record"), (data + b"\0", "length mismatch"),
+                              (data[:-1], "truncated MFQ blob")):
+            bad = tmp_path / "bad.mfq"
+            bad.write_bytes(payload)
+            r = subprocess.run([str(tool), str(bad), "w"], capture_output=True, text=True)
+            assert r.returncode == 1 and want in r.stderr, r.stderr

@@ -296,3 +296,19 @@ def test_empty_batch_returns_empty_outputs():
     assert nepq_matmul(w, e(0, 256), 1).shape == (0, 32)
     with pytest.raises(ValueError, match="activation width"):
         nint.forward(e(0, 95))
+
+
+def test_multi_expert_nepq_blob_is_not_a_linear():
+    """The reference has no linear dtype for NEPQ tensors of several experts (they are NINTM cohorts): both
+    load_quant_linear implementations refuse one instead of sizing outputs for a single expert."""
+    import ctypes
+    from pathlib import Path
+    from tyloquant_amd import runtime as R
+    blob = O.pack_nepq(synth.nepq_random(np.random.default_rng(3), "NEPQ1-S", 2, 16, 96, 2))
+    with pytest.raises(ValueError, match="must hold one expert"):
+        R.load_quant_linear("NEPQ1-S", blob)
+    lib = ctypes.CDLL(str(Path(R.__file__).resolve().parent / "lib" / "libmfq_runtime.so"))
+    lib.mfq_rt_last_error.restype = ctypes.c_char_p
+    handle = ctypes.c_void_p()
+    assert lib.mfq_rt_load_quant_linear(b"NEPQ1-S", blob, ctypes.c_size_t(len(blob)), ctypes.byref(handle)) != 0
+    assert "must hold one expert" in lib.mfq_rt_last_error().decode()

@@ -107,10 +107,13 @@ NvqHeader parse_nvq(const uint8_t *b, size_t n) {
     h.vector_size = h.codebook[0] == 'e' ? 8 : 4;
     h.jsc = enc & 0x20; h.index_parity = enc & 0x80;
     const bool custom = enc & 0x40;
+    if (ndim > 8) fail("truncated NVQ header");
     size_t off = 20 + 8 * static_cast<size_t>(ndim);
     if (n < off + 4) fail("truncated NVQ header");
     h.out = static_cast<int>(rd<uint32_t>(b, off));
     off += 4;
+    if (h.gs <= 0 || h.neuron_len <= 0 || h.out <= 0 || h.sub_bits < 1 || h.sub_bits > 8)
+        fail("NVQ dimensions must be positive (groupsize, neuron_len, rows) and sub_bits in [1,8]");
     const int64_t o = h.out, ng = cdiv(h.neuron_len, h.gs), nvec = cdiv(h.neuron_len, h.vector_size),
                   nsign = cdiv(h.neuron_len, 8);
     const int64_t streams = 2 * o + (o * ng * h.sub_bits + 7) / 8 + (o * nvec * h.index_bits + 7) / 8 + (o * nsign * 7 + 7) / 8;
@@ -186,8 +189,16 @@ NintmHeader parse_nintm(const uint8_t *b, size_t n) {
         const uint64_t plen = rd<uint64_t>(b, off + 8), rlen = rd<uint64_t>(b, off + 16);
         off += 24;
         if (n_ids == 0 || dlen == 0 || dlen > 32) fail("invalid NINTM v2 pool metadata");
-        const size_t end = off + 4ull * n_ids + dlen + rlen + plen;
-        if (end > n) fail("truncated NINTM v2 pool payload");
+        // every length is compared with what is left, so that no sum of 64-bit header fields can wrap
+        size_t left = n - off;
+        if (4ull * n_ids > left) fail("truncated NINTM v2 pool payload");
+        left -= 4ull * n_ids;
+        if (dlen > left) fail("truncated NINTM v2 pool payload");
+        left -= dlen;
+        if (rlen > left) fail("truncated NINTM v2 pool payload");
+        left -= rlen;
+        if (plen > left) fail("truncated NINTM v2 pool payload");
+        const size_t end = off + 4ull * n_ids + dlen + static_cast<size_t>(rlen) + static_cast<size_t>(plen);
         NintmPool p;
         for (uint32_t i = 0; i < n_ids; ++i) {
             const int32_t e = rd<int32_t>(b, off + 4ull * i);
@@ -474,6 +485,9 @@ QuantLinear load_quant_linear(const std::string &dtype_in, const uint8_t *blob, 
         q.kind = QuantLinearKind::Nepq;
         q.nepq = std::make_shared<NepqWeight>(NepqWeight::from_blob(blob, n, nullptr, stream));
         if (q.nepq->label != dtype) fail("MFQ dtype/blob mismatch: " + dtype + " contains " + q.nepq->label);
+        if (q.nepq->n_experts != 1)
+            fail("a " + dtype + " linear must hold one expert, the blob holds " + std::to_string(q.nepq->n_experts) +
+                 " (multi-expert NEPQ tensors are NINTM cohorts)");
         return q;
     }
     fail("unsupported quantized linear dtype: " + dtype);
@@ -629,7 +643,7 @@ MfqFile::MfqFile(const std::string &path) {
         if (off + 4 > n) fail("truncated MFQ header");
         const uint32_t len = rd<uint32_t>(b, off);
         off += 4;
-        if (off + len > n) fail("truncated MFQ header");
+        if (len > n - off) fail("truncated MFQ header");
         s.assign(reinterpret_cast<const char *>(b + off), len);
         off += len;
     };
@@ -653,11 +667,15 @@ MfqFile::MfqFile(const std::string &path) {
         off += 8;
         records.push_back(std::move(r));
     }
-    for (auto &r : records) {
-        if (off + r.nbytes > n) fail("truncated MFQ blob for " + r.name);
+    for (size_t i = 0; i < records.size(); ++i) {
+        MfqRecord &r = records[i];
+        for (size_t j = 0; j < i; ++j)
+            if (records[j].name == r.name) fail("duplicate MFQ tensor record: " + r.name + ": " + path);
+        if (r.nbytes > n - off) fail("truncated MFQ blob for " + r.name);   // compared with what is left: cannot wrap
         r.offset = off;
-        off += r.nbytes;
+        off += static_cast<size_t>(r.nbytes);
     }
+    if (off != n) fail("MFQ file length mismatch: records end=" + std::to_string(off) + ", file size=" + std::to_string(n));
 }
 const MfqRecord &MfqFile::find(const std::string &name) const {
     for (const auto &r : records)

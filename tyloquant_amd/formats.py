@@ -508,8 +508,12 @@ def read_mfq_directory(data) -> dict:
         recs.append((name, dtype, ln))
     out = {}
     for name, dtype, ln in recs:
+        if name in out:
+            raise ValueError(f"duplicate MFQ tensor record: {name}")
         if off + ln > len(data):
             raise ValueError(f"truncated MFQ blob for {name}")
         out[name] = (dtype, off, ln)
         off += ln
+    if off != len(data):       # mfq/formats/io.py:826-827
+        raise ValueError(f"MFQ file length mismatch: records end={off}, file size={len(data)}")
     return out

@@ -335,6 +335,9 @@ def load_quant_linear(dtype: str, blob, device="cuda") -> QuantLinear:
         w = NepqWeight.from_blob(blob, device)
         if w.label != dtype:
             raise ValueError(f"MFQ dtype/blob mismatch: {dtype} contains {w.label}")
+        if w.n_experts != 1:
+            raise ValueError(f"a {dtype} linear must hold one expert, the blob holds {w.n_experts} "
+                             "(multi-expert NEPQ tensors are NINTM cohorts)")
         return QuantLinear("nepq", w)
     raise ValueError(f"unsupported quantized linear dtype: {dtype}")
 
