@@ -32,6 +32,14 @@ enum { MFQ_GLU_SILU = 0, MFQ_GLU_GELU = 1 };
 
 const char *mfq_hip_last_error(void);
 int mfq_hip_version(void);
+/* The effective launch configuration as text: "cu_count=256 MFQ_GEMV_WAVES=2048 ..." -- the device's compute-unit
+ * count and every tuning knob (environment variables, read once per process) consulted so far.  Benchmarks print it
+ * next to their numbers.  Thread-local buffer.  No counterpart in the reference, whose MFQ_* overrides are read where
+ * they are used (e.g. cpp_runtime/mfq_decode.cpp:8518-8523). */
+const char *mfq_hip_config(void);
+/* Test and tuning hook: size one-block-per-CU grids for n compute units instead of the device's own count
+ * (n <= 0 restores it).  Process-wide; not for production use. */
+void mfq_hip_set_cu_count(int n);
 
 /* ------------------------------------------------------------------------------------
  * NINT (neuron-anchored INT).  Device layout: row-blocks of 16 neurons; inside a block
@@ -333,6 +341,13 @@ int mfq_hip_moe_decode_matmul(const mfq_moe_pool *pools, int n_pools, const int3
                               const int32_t *ids, int T, int R,
                               const mfq_nint_desc *shared_desc, const void *shared_weight, int swiglu,
                               void *out, int out_dtype, int64_t ldo, mfq_stream_t stream);
+
+/* 1 when mfq_hip_moe_decode_matmul takes these cohorts (and shared tensor) at T x R pairs, else 0: the same checks
+ * the launch makes (a batch-1 unit for every cohort, the block's LDS need, the row count), so that a host can pick the
+ * mapped path up front, as the T <= 8 test of NintMoeWeight::forward_impl does (cpp_runtime/mfq_decode.cpp:2935-2960).
+ * Pure host arithmetic; the weight pointers of `pools` are not read. */
+int mfq_hip_moe_decode_capable(const mfq_moe_pool *pools, int n_pools, int out_per_expert, int K,
+                               const mfq_nint_desc *shared_desc, int T, int R, int swiglu);
 
 /* hidden[r, c] = silu(gate_up[r, c]) * gate_up[r, W + c]  (moe_swiglu_split_cuda,
  * mfq/kernels/cuda/moe.cu:2980-2996); output fp16 (x_dtype MFQ_X_F16) or bf16. */

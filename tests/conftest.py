@@ -12,6 +12,14 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+@pytest.fixture
+def cu_count():
+    """Setter that sizes one-block-per-CU grids for n compute units (the device's own count again after the test)."""
+    from tyloquant_amd import _lib as L
+    yield L.lib().mfq_hip_set_cu_count
+    L.lib().mfq_hip_set_cu_count(0)
+
+
 def rel_l2(a, b):
     import numpy as np
     a = np.asarray(a, dtype=np.float64)

@@ -291,3 +291,27 @@ def test_legacy_byte_tail_and_errors():
         R.load_quant_linear("NINT5", blob)
     with pytest.raises(ValueError):
         R.load_quant_linear("NOPE", blob)
+
+
+@pytest.mark.parametrize("K", [32768, 81920])
+def test_gemv_long_neurons(K):
+    """Neurons whose staged activation slice exceeds 64 KB of LDS: up to 160 KB the GEMV block opts in to the larger
+    LDS (K = 32768: 74 KB), beyond that the matrix-core streaming kernel takes over (K = 81920).  One and two rows,
+    and the fused gate/up SwiGLU on the first shape."""
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(K)
+    t = synth.nint_random(rng, 64, K, 4, 32, 6)
+    t.neuron_scale = O._f16_round(t.neuron_scale * 0.02)
+    t.neuron_min = O._f16_round(t.neuron_min * 0.02)
+    lin = _load(t)
+    deq = O.dequantize_nint(t)
+    for M in (1, 2):
+        x, xf = _x(rng, M, K)
+        y = R.nint_matmul(lin.weight, x, force="gemv").cpu().numpy()
+        ref = O.linear_forward_f64(deq, xf)
+        assert rel_l2(y, ref) < REL_TOL, (M, rel_l2(y, ref))
+    if K == 32768:
+        x, xf = _x(rng, 1, K)
+        h = R.nint_matmul_swiglu(lin.weight, x).float().cpu().numpy()
+        want = O.moe_swiglu(O.linear_forward_f64(deq, xf).astype(np.float32))
+        assert rel_l2(h, want) < 2e-3

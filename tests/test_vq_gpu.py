@@ -18,6 +18,7 @@ def _x(rng, M, K, dtype=None):
 _check = check_close
 
 
+
 @pytest.mark.parametrize("codebook,banks", [("d4_512", 2), ("d4_512", 4), ("d4_512", 1), ("d4_256", 2)])
 @pytest.mark.parametrize("out,K", [(37, 96), (24, 80), (64, 200), (73, 1537), (33, 100)])
 def test_nvq_jsc_dequant_bit_exact_and_gemv(codebook, banks, out, K):
@@ -56,14 +57,14 @@ def test_nvq_matrix_core_path_multi_step(out, K, M):
 
 @pytest.mark.parametrize("K", [1560, 6160])
 @pytest.mark.parametrize("rpb", [1, 2, 3, 4, 5, 6])
-def test_nvq_signed_table_kernel_row_blocks_per_block(monkeypatch, rpb, K):
+def test_nvq_signed_table_kernel_row_blocks_per_block(cu_count, rpb, K):
     """Up to 32 rows (16 per tile) with the (entry, sign nibble) table in LDS: one block per CU and tile owning rpb row-blocks.  With the CU
     count the grid is sized for set to 8, 128 * rpb - 5 neurons give every rpb variant (ragged last row-block, last
     block with fewer row-blocks); K = 1560 is one step per wave (5 waves), K = 6160 two steps per wave with a ragged
     last group.  One- and two-bank 512-entry codebooks and the 256-entry one."""
     from tyloquant_amd import runtime as R
     from tyloquant_amd.runtime_vq import nvq_matmul
-    monkeypatch.setenv("MFQ_CU_COUNT", "8")
+    cu_count(8)
     out = 128 * rpb - 5
     rng = np.random.default_rng(900 + rpb + K)
     for codebook, banks in (("d4_512", 2), ("d4_512", 1), ("d4_256", 2)):
@@ -78,13 +79,13 @@ def test_nvq_signed_table_kernel_row_blocks_per_block(monkeypatch, rpb, K):
 
 
 @pytest.mark.parametrize("cu", ["8", "256"])
-def test_nvq_two_projections_in_one_launch(monkeypatch, cu):
+def test_nvq_two_projections_in_one_launch(cu_count, cu):
     """Two tensors that share their input: the joint launch gives exactly what the two separate calls give (bit for
     bit: same kernel, same order of sums), for one- and two-bank codebooks, different heights, 1 to 32 rows; with the
     grid sized for 8 CUs the blocks hold several row-blocks.  A four-bank tensor takes the two-call path."""
     from tyloquant_amd import runtime as R
     from tyloquant_amd.runtime_vq import nvq_matmul, nvq_matmul_multi2
-    monkeypatch.setenv("MFQ_CU_COUNT", cu)
+    cu_count(int(cu))
     rng = np.random.default_rng(950 + int(cu))
     K = 1560
     specs = [(("d4_512", 2), 250), (("d4_512", 1), 123), (("d4_256", 2), 64), (("d4_512", 4), 80)]

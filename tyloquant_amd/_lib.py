@@ -53,6 +53,10 @@ class MfqError(RuntimeError):
 
 _SIGS = {
     "mfq_hip_version": (C.c_int, []),
+    "mfq_hip_config": (C.c_char_p, []),
+    "mfq_hip_set_cu_count": (None, [C.c_int]),
+    "mfq_hip_moe_decode_capable": (C.c_int, [C.POINTER(MoePool), C.c_int, C.c_int, C.c_int, C.POINTER(NintDesc), C.c_int,
+                                             C.c_int, C.c_int]),
     "mfq_hip_nint_plan": (C.c_int, [C.c_int] * 5 + [C.POINTER(NintDesc)]),
     "mfq_hip_nint_repack": (C.c_int, [C.POINTER(NintDesc), vp, i64, C.c_int, vp, vp]),
     "mfq_hip_nint_dequant_f32": (C.c_int, [C.POINTER(NintDesc), vp, vp, i64, vp]),

@@ -560,14 +560,10 @@ void NintMoeWeight::forward(const void *x, int x_dtype, int64_t ldx, bool routed
         need ? workspace.get() : nullptr, need, stream));
 }
 
-static bool nint_decode_unit(const mfq_nint_desc &d) { return d.kind == 1 || (d.bits == 5 && d.gs == 28); }
-
-bool NintMoeWeight::decode_capable(const NintWeight *shared) const {
-    if (pools.size() + (shared ? 1 : 0) > 8) return false;
-    for (const auto &p : pools)
-        if (!nint_decode_unit(p->desc)) return false;
-    return !shared || (nint_decode_unit(shared->desc) && shared->desc.out == out_per_expert &&
-                       shared->desc.neuron_len == neuron_len);
+bool NintMoeWeight::decode_capable(const NintWeight *shared, int tokens, int routes, bool swiglu) const {
+    if (shared && shared->desc.neuron_len != neuron_len) return false;
+    return mfq_hip_moe_decode_capable(pool_table.data(), static_cast<int>(pool_table.size()), out_per_expert, neuron_len,
+                                      shared ? &shared->desc : nullptr, tokens, routes, swiglu ? 1 : 0) != 0;
 }
 
 void NintMoeWeight::forward_decode(const void *x, int x_dtype, int64_t ldx, bool routed_input, const int32_t *ids, int T,
@@ -595,8 +591,8 @@ void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &dow
     abi_check(mfq_hip_moe_topk(router_logits, router_bias, T, E, top_k, topk_mode, normalize ? 1 : 0, 1e-20f, router_scale, ids,
                                wts, stream));
     const bool with_shared = shared_gate_up && shared_down;
-    if (T <= 8 && gate_up.decode_capable(with_shared ? shared_gate_up : nullptr) &&
-        down.decode_capable(with_shared ? shared_down : nullptr)) {
+    if (T <= 8 && gate_up.decode_capable(with_shared ? shared_gate_up : nullptr, T, top_k, true) &&
+        down.decode_capable(with_shared ? shared_down : nullptr, T, top_k, false)) {
         // decode step: gate/up + SwiGLU of the routes and the shared expert in one launch, the down projections in a
         // second one; rows pairs .. pairs + T - 1 of both buffers belong to the shared expert
         const size_t rows = pairs + (with_shared ? T : 0);

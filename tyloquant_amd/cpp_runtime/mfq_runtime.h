@@ -219,7 +219,7 @@ struct NintMoeWeight {
     // Decode step in one launch (mfq_hip_moe_decode_matmul): rows t * R + r are the routed pairs, rows T * R + t the
     // `shared` tensor (may be null) on token t.  swiglu: out is fp16 [rows, out_per_expert / 2], else fp32
     // [rows, out_per_expert].  decode_capable() tells whether the cohorts and the shared tensor fit that kernel.
-    bool decode_capable(const NintWeight *shared) const;
+    bool decode_capable(const NintWeight *shared, int tokens = 1, int routes = 1, bool swiglu = false) const;
     void forward_decode(const void *x, int x_dtype, int64_t ldx, bool routed_input, const int32_t *ids, int T, int R,
                         const NintWeight *shared, bool swiglu, void *out, mfq_stream_t stream = nullptr) const;
 };

@@ -6,6 +6,7 @@
 #include <stdlib.h>
 
 #include "common.hpp"
+#include "tune.hpp"
 
 namespace mfq {
 
@@ -369,7 +370,7 @@ extern "C" int mfq_hip_gemm_f16_nt(const void *a, int64_t lda, const void *b, in
 // over K; a quarter more for the natural-order unit).
 static constexpr int kGemvMaxM = 8, kStreamMaxM = 256;
 static bool nint_streams(const mfq_nint_desc *d, int M) {
-    static const int env_max = [] { const char *e = getenv("MFQ_STREAM_MAX_M"); return e ? atoi(e) : 0; }();
+    static const int env_max = tune_env("MFQ_STREAM_MAX_M", 0);
     int stream_max = kStreamMaxM;
     if (nint_prefill_capable(d)) {
         const bool natural = d->kind != 1;

@@ -4,6 +4,7 @@
 #include <stdlib.h>
 
 #include "common.hpp"
+#include "tune.hpp"
 
 namespace mfq {
 
@@ -271,20 +272,15 @@ __device__ __forceinline__ void finish_rows(float (&v)[MB], float *red, int wave
 // MFQ_GEMV_WAVES overrides the default for tuning.
 inline int gemv_target_waves() {
     static const int v = [] {
-        const char *e = getenv("MFQ_GEMV_WAVES");
-        const int n = e ? atoi(e) : 0;
+        const int n = tune_env("MFQ_GEMV_WAVES", 2048);
         return n > 0 ? n : 2048;
     }();
     return v;
 }
 
-// Compute units a one-block-per-CU grid is sized for (MI355X: 256).  MFQ_CU_COUNT overrides it and is read at every
-// call, so that a test can walk the row-blocks-per-block variants on small tensors.
-inline int gemv_cu_count() {
-    const char *e = getenv("MFQ_CU_COUNT");
-    const int n = e ? atoi(e) : 0;
-    return n > 0 ? n : 256;
-}
+// Compute units a one-block-per-CU grid is sized for: the device's own count (mfq_hip_set_cu_count overrides it, so
+// that a test can walk the row-blocks-per-block variants on small tensors).
+inline int gemv_cu_count() { return device_cu_count(); }
 
 // LDS bytes of a GEMV block: per wave MB * steps_per_wave * 16 groups * (gs/2 pairs + 2 sums) dwords,
 // plus the cross-wave reduction area of rbw row-blocks.

@@ -4,6 +4,7 @@
 
 #include "common.hpp"
 #include "gemv_common.hpp"
+#include "tune.hpp"
 #include "nint_body.hpp"
 #include "nint_mfma.hpp"
 #include "nint_prefill.hpp"
@@ -706,17 +707,18 @@ static void moe_fill_k(NintK &k, const mfq_nint_desc &d) {
     k.step_bytes = d.step_bytes; k.rowblock_bytes = d.rowblock_bytes; k.anchors_off = d.anchors_off;
 }
 
-// Batch-1 launch (moe_decode_kernel) over n_rows rows: the n_pairs routed pairs, then one row per token for the
-// shared tensor in cohort slot P.n, if any.  Every cohort slot has a GEMV unit.  Returns -1 when the shape does
-// not fit the kernel (the caller takes another path), else a status.
-static int moe_decode_launch(MoePools &P, int n_slots, int max_steps, const int32_t *expert_pool,
-                             const int32_t *expert_local, int E, int out_per_expert, const uint16_t *xp, int x_dtype,
-                             int64_t ldx, int routed_input, const int32_t *ids, int n_pairs, int n_rows, int R, int swiglu,
-                             void *out, int out_f16, int64_t ldo, hipStream_t st) {
-    static const int env_off = [] { const char *e = getenv("MFQ_MOE_SPLIT"); return e ? atoi(e) == 0 : 0; }();
-    static const int env_w = [] { const char *e = getenv("MFQ_MOE_DEC_WAVES"); return e ? atoi(e) : 8; }();
-    static const int env_rbw = [] { const char *e = getenv("MFQ_MOE_DEC_RBW"); return e ? atoi(e) : 0; }();
-    if (env_off || n_rows > 65535) return -1;
+// Block shape of the batch-1 launch: false when the shape does not fit the kernel.
+struct MoeDecodeShape {
+    int nwaves, rbw;
+    size_t lds;
+    bool ring;
+};
+static bool moe_decode_shape(MoePools &P, int n_slots, int max_steps, int out_per_expert, int n_rows, int swiglu,
+                             MoeDecodeShape &sh) {
+    static const int env_off = tune_env("MFQ_MOE_SPLIT", 1) == 0;
+    static const int env_w = tune_env("MFQ_MOE_DEC_WAVES", 8);
+    static const int env_rbw = tune_env("MFQ_MOE_DEC_RBW", 0);
+    if (env_off || n_rows > 65535) return false;
     const int rbe = out_per_expert / 16;
     // At most eight waves split the K steps (two blocks fit a CU at the kernel's 128 registers; measured best at
     // T = 1: 54 us per layer against 60-62 us with 11..16 waves); a wave takes more (row-block, step) items while
@@ -734,7 +736,7 @@ static int moe_decode_launch(MoePools &P, int n_slots, int max_steps, const int3
     if (rbw > kMaxRbw) rbw = kMaxRbw;
     while (rbe % rbw) --rbw;
     if (swiglu) {
-        if (out_per_expert % 32) return -1;
+        if (out_per_expert % 32) return false;
         rbw = 2;
     }
     size_t lds = 0;
@@ -744,13 +746,33 @@ static int moe_decode_launch(MoePools &P, int n_slots, int max_steps, const int3
         const size_t need = gemv_lds_bytes(1, P.spw[i], P.k[i].gs, nwaves, rbw);
         if (need > lds) lds = need;
         if (P.spw[i] * rbw > 3) ring = true;
-        if (swiglu && static_cast<int64_t>(rbe / 2) * P.k[i].rowblock_bytes >= (1ll << 31)) return -1;
+        if (swiglu && static_cast<int64_t>(rbe / 2) * P.k[i].rowblock_bytes >= (1ll << 31)) return false;
     }
-    if (lds > 65536) return -1;
+    if (lds > kMaxDynamicLds) return false;
+    sh.nwaves = nwaves; sh.rbw = rbw; sh.lds = lds; sh.ring = ring;
+    return true;
+}
+
+// Batch-1 launch (moe_decode_kernel) over n_rows rows: the n_pairs routed pairs, then one row per token for the
+// shared tensor in cohort slot P.n, if any.  Every cohort slot has a GEMV unit.  Returns -1 when the shape does
+// not fit the kernel (the caller takes another path), else a status.
+static int moe_decode_launch(MoePools &P, int n_slots, int max_steps, const int32_t *expert_pool,
+                             const int32_t *expert_local, int E, int out_per_expert, const uint16_t *xp, int x_dtype,
+                             int64_t ldx, int routed_input, const int32_t *ids, int n_pairs, int n_rows, int R, int swiglu,
+                             void *out, int out_f16, int64_t ldo, hipStream_t st) {
+    MoeDecodeShape sh;
+    if (!moe_decode_shape(P, n_slots, max_steps, out_per_expert, n_rows, swiglu, sh)) return -1;
+    const int rbe = out_per_expert / 16, rbw = sh.rbw, nwaves = sh.nwaves;
+    const size_t lds = sh.lds;
+    const bool ring = sh.ring;
     const dim3 grid(static_cast<unsigned>(swiglu ? rbe / 2 : rbe / rbw), static_cast<unsigned>(n_rows)), block(64 * nwaves);
 #define MFQ_MOE_DECODE(XF, RG, SW)                                                                                   \
-    hipLaunchKernelGGL((moe_decode_kernel<XF, RG, SW>), grid, block, lds, st, P, rbw, expert_pool, expert_local, E,   \
-                       out_per_expert, xp, ldx, routed_input, ids, n_pairs, R, out, out_f16, ldo)
+    do {                                                                                                             \
+        auto kern = moe_decode_kernel<XF, RG, SW>;                                                                   \
+        if (int rc_ = allow_dynamic_lds(reinterpret_cast<const void *>(kern), lds, "moe_decode")) return rc_;        \
+        hipLaunchKernelGGL(kern, grid, block, lds, st, P, rbw, expert_pool, expert_local, E, out_per_expert, xp, ldx, \
+                           routed_input, ids, n_pairs, R, out, out_f16, ldo);                                        \
+    } while (0)
 #define MFQ_MOE_DECODE_X(XF)                        \
     if (swiglu) {                                   \
         if (ring) MFQ_MOE_DECODE(XF, true, true);   \
@@ -827,7 +849,7 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
     // mapped calls with a workspace go through the prefill kernel, 64 pairs of an expert per block (faster than the
     // streaming kernel from about one pair per expert on; MFQ_MOE_PREFILL_PAIRS raises the threshold for tuning)
     const int x_rows = routed_input ? n_pairs : T;
-    static const int min_pairs = [] { const char *e = getenv("MFQ_MOE_PREFILL_PAIRS"); return e ? atoi(e) : 0; }();
+    static const int min_pairs = tune_env("MFQ_MOE_PREFILL_PAIRS", 0);
     if (mfma && mapped && workspace && n_pairs >= static_cast<int64_t>(min_pairs) * E && moe_prefill_pools(pools, n_pools) &&
         workspace_bytes >= mfq_hip_moe_grouped_workspace_bytes(pools, n_pools, K, x_rows)) {
         const int Kp = moe_kp(K);
@@ -905,7 +927,7 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
     if (mfma) {
         // row-blocks per wave: 4 while the grid still has a few thousand waves, else 1
         const int64_t live_tiles = mapped ? ceil_div(n_pairs, kMoeTileM) : n_pairs;
-        static const int env_nb = [] { const char *e = getenv("MFQ_MOE_NB"); return e ? atoi(e) : 0; }();
+        static const int env_nb = tune_env("MFQ_MOE_NB", 0);
         const bool nb4 = env_nb ? env_nb == 4 : (live_tiles * rbe * max_steps >= 4 * 2048 && rbe >= 4);
         const int nb = nb4 ? 4 : 1;
         int nwaves = max_steps < 8 ? max_steps : 8;
@@ -971,6 +993,25 @@ extern "C" int mfq_hip_moe_decode_matmul(const mfq_moe_pool *pools, int n_pools,
                                      swiglu, out, (out_dtype == MFQ_X_F16 ? 1 : 0) | (swiglu == 2 ? 2 : 0), ldo, as_stream(stream));
     if (rc < 0) return fail(MFQ_ERR_UNSUPPORTED, "moe_decode_matmul: shape outside the batch-1 kernel (rows %d, K %d)", n_rows, K);
     return rc;
+}
+
+extern "C" int mfq_hip_moe_decode_capable(const mfq_moe_pool *pools, int n_pools, int out_per_expert, int K,
+                                          const mfq_nint_desc *shared_desc, int T, int R, int swiglu) {
+    if (!pools || n_pools < 1 || T <= 0 || R <= 0 || out_per_expert % 16) return 0;
+    const int n_slots = n_pools + (shared_desc ? 1 : 0);
+    if (n_slots > kMaxPools) return 0;
+    if (shared_desc && shared_desc->out != out_per_expert) return 0;
+    MoePools P;
+    P.n = n_pools;
+    int max_steps = 1;
+    for (int i = 0; i < n_slots; ++i) {
+        const mfq_nint_desc &d = i < n_pools ? pools[i].desc : *shared_desc;
+        if (d.neuron_len != K || !moe_prefill_unit(d) || 4 * d.rowblock_bytes >= (1ll << 31)) return 0;
+        if (d.nsteps > max_steps) max_steps = d.nsteps;
+        moe_fill_k(P.k[i], d);
+    }
+    MoeDecodeShape sh;
+    return moe_decode_shape(P, n_slots, max_steps, out_per_expert, T * R + (shared_desc ? T : 0), swiglu, sh) ? 1 : 0;
 }
 
 extern "C" int mfq_hip_moe_glu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype, int64_t ldh,

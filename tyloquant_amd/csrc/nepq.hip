@@ -631,7 +631,7 @@ template <int XF16>
 static int nepq_mfma_any(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
                          float *y, int64_t ldy, hipStream_t st) {
     const int64_t wpb = (k.nsteps < 8 ? k.nsteps : 8) * ceil_div(M, 16);  // waves of a block x 16-row tiles
-    static const int env_nb = [] { const char *e = getenv("MFQ_NEPQ_NB"); return e ? atoi(e) : 0; }();
+    static const int env_nb = tune_env("MFQ_NEPQ_NB", 0);
     if (env_nb == 4) return nepq_launch_mfma<XF16, 4>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
     if (env_nb == 2) return nepq_launch_mfma<XF16, 2>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
     if (env_nb == 1) return nepq_launch_mfma<XF16, 1>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
@@ -807,7 +807,7 @@ extern "C" int mfq_hip_nepq_gemv(const mfq_nepq_desc *d, const void *weight, int
 // from kNepqPrefillMinM rows; tensors it cannot take stay on the streaming kernel up to kNepqStreamMaxM rows.
 static constexpr int kNepqGemvMaxM = 16, kNepqStreamMaxM = 256, kNepqPrefillMinM = 33;
 static bool nepq_prefills(const NepqK &k, int M) {
-    static const int env = [] { const char *e = getenv("MFQ_NEPQ_PREFILL_MIN_M"); return e ? atoi(e) : 0; }();
+    static const int env = tune_env("MFQ_NEPQ_PREFILL_MIN_M", 0);
     return M >= (env > 0 ? env : kNepqPrefillMinM) && nepq_prefill_capable(k);
 }
 static bool nepq_streams(const mfq_nepq_desc *d, int M) {

@@ -145,8 +145,8 @@ __global__ void nint_dequant_kernel(NintK k, const uint8_t *__restrict__ w, OutT
 // waves; long neurons spend the items on K (fewer waves to reduce), short ones on row-blocks (the
 // staged activations are reused).  MFQ_GEMV_SPW / MFQ_GEMV_RBW override the choice for tuning.
 void gemv_shape(const NintK &k, int mb, int &spw, int &nwaves, int &rbw, size_t &lds_bytes) {
-    static const int env_spw = [] { const char *e = getenv("MFQ_GEMV_SPW"); return e ? atoi(e) : 0; }();
-    static const int env_rbw = [] { const char *e = getenv("MFQ_GEMV_RBW"); return e ? atoi(e) : 0; }();
+    static const int env_spw = tune_env("MFQ_GEMV_SPW", 0);
+    static const int env_rbw = tune_env("MFQ_GEMV_RBW", 0);
     const int64_t items = static_cast<int64_t>(k.n_rowblocks) * k.nsteps;
     int per_wave = static_cast<int>(items / gemv_target_waves());
     per_wave = per_wave < 1 ? 1 : (per_wave > 3 ? 3 : per_wave);
@@ -172,18 +172,23 @@ static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, i
     int spw, nwaves, rbw;
     size_t lds;
     gemv_shape(k, MB, spw, nwaves, rbw, lds);
-    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nint_gemv: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
+    MFQ_REQUIRE(lds <= kMaxDynamicLds, MFQ_ERR_UNSUPPORTED, "nint_gemv: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
     MFQ_REQUIRE(k.rowblock_bytes < (1ll << 31), MFQ_ERR_UNSUPPORTED, "nint_gemv: neuron_len %d is too long", k.neuron_len);
     const dim3 block(64 * nwaves);
+    // blocks that stage more than 64 KB of activations (neurons longer than about 29k) opt in to the larger LDS
+#define MFQ_GEMV_LAUNCH(KERN, GRID, ...)                                                                     \
+    do {                                                                                                     \
+        auto kern_ = KERN;                                                                                   \
+        if (int rc_ = allow_dynamic_lds(reinterpret_cast<const void *>(kern_), lds, "nint_gemv")) return rc_; \
+        hipLaunchKernelGGL(kern_, GRID, block, lds, st, __VA_ARGS__);                                        \
+    } while (0)
 #define MFQ_PAIRED(B, G)                                                                                     \
     if (k.bits == B && k.gs == G) {                                                                          \
         const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, rbw)), static_cast<unsigned>(ceil_div(M, MB))); \
         if (spw * rbw <= 3)                                                                                  \
-            hipLaunchKernelGGL((nint_gemv_paired_kernel<B, G, XF16, MB, false>), grid, block, lds, st, k, w, x, ldx, \
-                               M, y, ldy, spw, rbw);                                                         \
+            MFQ_GEMV_LAUNCH((nint_gemv_paired_kernel<B, G, XF16, MB, false>), grid, k, w, x, ldx, M, y, ldy, spw, rbw); \
         else                                                                                                 \
-            hipLaunchKernelGGL((nint_gemv_paired_kernel<B, G, XF16, MB, true>), grid, block, lds, st, k, w, x, ldx, \
-                               M, y, ldy, spw, rbw);                                                         \
+            MFQ_GEMV_LAUNCH((nint_gemv_paired_kernel<B, G, XF16, MB, true>), grid, k, w, x, ldx, M, y, ldy, spw, rbw); \
         return check_launch("nint_gemv_paired");                                                             \
     }
     if (k.kind == 1) {
@@ -195,15 +200,14 @@ static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, i
     if (mfma_generic_profile(k)) {
         const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, rbw)), static_cast<unsigned>(ceil_div(M, MB)));
         if (spw * rbw <= 3)
-            hipLaunchKernelGGL((nint_gemv_natural_kernel<5, 28, XF16, MB, false>), grid, block, lds, st, k, w, x, ldx, M, y,
-                               ldy, spw, rbw);
+            MFQ_GEMV_LAUNCH((nint_gemv_natural_kernel<5, 28, XF16, MB, false>), grid, k, w, x, ldx, M, y, ldy, spw, rbw);
         else
-            hipLaunchKernelGGL((nint_gemv_natural_kernel<5, 28, XF16, MB, true>), grid, block, lds, st, k, w, x, ldx, M, y,
-                               ldy, spw, rbw);
+            MFQ_GEMV_LAUNCH((nint_gemv_natural_kernel<5, 28, XF16, MB, true>), grid, k, w, x, ldx, M, y, ldy, spw, rbw);
         return check_launch("nint_gemv_natural");
     }
     const dim3 grid(k.n_rowblocks, static_cast<unsigned>(ceil_div(M, MB)));
-    hipLaunchKernelGGL((nint_gemv_generic_kernel<XF16, MB>), grid, block, lds, st, k, w, x, ldx, M, y, ldy, spw);
+    MFQ_GEMV_LAUNCH((nint_gemv_generic_kernel<XF16, MB>), grid, k, w, x, ldx, M, y, ldy, spw);
+#undef MFQ_GEMV_LAUNCH
     return check_launch("nint_gemv_generic");
 }
 
@@ -250,7 +254,7 @@ static int launch_mfma(const NintK &k, const uint8_t *w, const uint16_t *x, int6
     // row-blocks per wave: as many as still leave about 1500 waves over all 16-row tiles (a block has at most 8 waves);
     // more row-blocks share the activation fragments, and the tiles of one row-block group re-read its weights from L2
     const int64_t wpb = (k.nsteps < 8 ? k.nsteps : 8) * ceil_div(M, 16);
-    static const int env_nb = [] { const char *e = getenv("MFQ_MFMA_NB"); return e ? atoi(e) : 0; }();
+    static const int env_nb = tune_env("MFQ_MFMA_NB", 0);
     if (env_nb == 4) return launch_mfma_nb<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
     if (env_nb == 2) return launch_mfma_nb<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
     if (env_nb == 1) return launch_mfma_nb<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
@@ -294,7 +298,7 @@ int prefill_sum_splits(const float *part, int64_t ystride, int splits, int M, in
 // splits) as long as every split keeps at least two steps and the neuron count allows 16-byte partial rows; the partial results go to a
 // workspace and are added in split order (deterministic).  1 = no split.
 int nint_prefill_splits(const mfq_nint_desc *d, int M) {
-    static const int env = [] { const char *e = getenv("MFQ_PREFILL_SPLITS"); return e ? atoi(e) : 0; }();
+    static const int env = tune_env("MFQ_PREFILL_SPLITS", 0);
     const int64_t blocks = ceil_div(d->n_rowblocks, 16) * ceil_div(M, 64);
     if (blocks > 128 || d->out % 4) return 1;
     int splits = static_cast<int>(256 / blocks);
@@ -359,7 +363,7 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
         }                                                                                                             \
         MFQ_PREFILL_CFG(UNIT, B, G, 8, 2, 4, (dma128 ? 0 : (UNIT<B, G>::D >= 5 ? 1 : 2)))                             \
     }
-    static const int env_big = [] { const char *e = getenv("MFQ_PREFILL_BIG"); return e ? atoi(e) : 0; }();
+    static const int env_big = tune_env("MFQ_PREFILL_BIG", 0);
     if (env_big && k.bits == 4 && k.gs == 32) {
         if (env_big == 1) MFQ_PREFILL_CFG(PairedUnit, 4, 32, 8, 3, 4, 0)
         if (env_big == 2) MFQ_PREFILL_CFG(PairedUnit, 4, 32, 8, 3, 2, 0)
@@ -381,19 +385,25 @@ int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int
     const NintK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
-    static const int valu_max = [] { const char *e = getenv("MFQ_GEMV_VALU_MAX_M"); return e ? atoi(e) : 2; }();
+    static const int valu_max = tune_env("MFQ_GEMV_VALU_MAX_M", 2);
     // two rows: the vector-ALU GEMV unpacks once and takes two dot products (10.6 vs 12.9 us on 12288x4096);
     // from three rows on the matrix-core kernel wins
     if (M > valu_max && mfma_eligible(k, x, ldx))
         return x_dtype == MFQ_X_F16 ? launch_mfma<1>(k, w, xp, ldx, M, y, ldy, st)
                                     : launch_mfma<0>(k, w, xp, ldx, M, y, ldy, st);
-    // LDS per block grows with MB; large K falls back to narrower row batches.
+    // LDS per block grows with MB; large K falls back to narrower row batches, and neurons whose one-row slice no
+    // block can stage (beyond about 70k elements) go to the matrix-core kernel, whose LDS use does not depend on K.
     int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
     for (;;) {
         int spw, nwaves, rbw;
         size_t lds;
         gemv_shape(k, mb, spw, nwaves, rbw, lds);
-        if (lds <= 65536 || mb == 1) break;
+        if (lds <= 65536 || mb == 1) {
+            if (lds > kMaxDynamicLds && mfma_eligible(k, x, ldx))
+                return x_dtype == MFQ_X_F16 ? launch_mfma<1>(k, w, xp, ldx, M, y, ldy, st)
+                                            : launch_mfma<0>(k, w, xp, ldx, M, y, ldy, st);
+            break;
+        }
         mb >>= 1;
     }
     if (x_dtype == MFQ_X_F16) {
@@ -480,16 +490,18 @@ static int launch_gemv_swiglu(const NintK &k, const uint8_t *w, const uint16_t *
     const int spw = static_cast<int>(ceil_div(k.nsteps, nwaves));
     const bool ring = 2 * spw > 3;
     const size_t lds = gemv_lds_bytes(MB, spw, k.gs, nwaves, 2);
-    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nint_gemv_swiglu: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
+    MFQ_REQUIRE(lds <= kMaxDynamicLds, MFQ_ERR_UNSUPPORTED, "nint_gemv_swiglu: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
     const dim3 grid(static_cast<unsigned>(k.n_rowblocks / 2), static_cast<unsigned>(ceil_div(M, MB))), block(64 * nwaves);
+#define MFQ_SWIGLU_LAUNCH(KERN)                                                                                       \
+    do {                                                                                                              \
+        auto kern_ = KERN;                                                                                            \
+        if (int rc_ = allow_dynamic_lds(reinterpret_cast<const void *>(kern_), lds, "nint_gemv_swiglu")) return rc_;  \
+        hipLaunchKernelGGL(kern_, grid, block, lds, st, k, w, x, ldx, M, hidden, out_f16, ldh, spw);                  \
+    } while (0)
 #define MFQ_SWIGLU(UNIT, B, G)                                                                                        \
     if (k.bits == B && k.gs == G) {                                                                                   \
-        if (ring)                                                                                                     \
-            hipLaunchKernelGGL((nint_gemv_swiglu_kernel<UNIT<B, G>, XF16, MB, true>), grid, block, lds, st, k, w, x, ldx, M, \
-                               hidden, out_f16, ldh, spw);                                                            \
-        else                                                                                                          \
-            hipLaunchKernelGGL((nint_gemv_swiglu_kernel<UNIT<B, G>, XF16, MB, false>), grid, block, lds, st, k, w, x, ldx, M, \
-                               hidden, out_f16, ldh, spw);                                                            \
+        if (ring) MFQ_SWIGLU_LAUNCH((nint_gemv_swiglu_kernel<UNIT<B, G>, XF16, MB, true>));                           \
+        else MFQ_SWIGLU_LAUNCH((nint_gemv_swiglu_kernel<UNIT<B, G>, XF16, MB, false>));                               \
         return check_launch("nint_gemv_swiglu");                                                                      \
     }
     if (k.kind == 1) {
@@ -499,6 +511,7 @@ static int launch_gemv_swiglu(const NintK &k, const uint8_t *w, const uint16_t *
         MFQ_SWIGLU(GenericUnit, 5, 28)
     }
 #undef MFQ_SWIGLU
+#undef MFQ_SWIGLU_LAUNCH
     return fail(MFQ_ERR_UNSUPPORTED, "nint_gemv_swiglu: no fused kernel for NINT%d-%d", k.bits, k.gs);
 }
 

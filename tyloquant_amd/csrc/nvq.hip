@@ -918,11 +918,11 @@ static int nvq_signed_rpb(const NvqK &k, int more_rowblocks = 0) {
     return static_cast<int>(ceil_div(k.n_rowblocks + more_rowblocks, gemv_cu_count()));
 }
 static bool nvq_signed_capable(const NvqK &k, int M, int more_rowblocks = 0) {
-    static const int off = [] { const char *e = getenv("MFQ_NVQ_SIGNED_OFF"); return e ? atoi(e) : 0; }();
+    static const int off = tune_env("MFQ_NVQ_SIGNED_OFF", 0);
     const int rpb = nvq_signed_rpb(k, more_rowblocks);
     // two 16-row tiles still beat the older streaming kernel and the prefill kernel on the config 3 tensors
     // (17408 x 5120 at M = 32: 42 us against 54 and 46); MFQ_NVQ_SIGNED_MAX_M for tuning
-    static const int max_m = [] { const char *e = getenv("MFQ_NVQ_SIGNED_MAX_M"); return e ? atoi(e) : 32; }();
+    static const int max_m = tune_env("MFQ_NVQ_SIGNED_MAX_M", 32);
     return !off && M <= max_m && static_cast<int64_t>(k.banks) * k.entries * 128 <= 131072 && rpb <= 6 && k.nsteps >= 4 &&
            rpb * k.rowblock_bytes < (1ll << 31);
 }
@@ -965,7 +965,7 @@ static int nvq_launch_signed(const NvqK &k, const uint8_t *w, const uint16_t *x,
         case 4: return nvq_launch_signed_as<XF16, 4, 3, true>(k, w, x, ldx, M, y, ldy, st, s2);
         case 5: {
             // ring depths 1 .. 4 run within 7 % of each other on 17408 x 5120 (two is the fastest): MFQ_NVQ_RING for tuning
-            static const int ring = [] { const char *e = getenv("MFQ_NVQ_RING"); return e ? atoi(e) : 2; }();
+            static const int ring = tune_env("MFQ_NVQ_RING", 2);
             if (ring == 1) return nvq_launch_signed_as<XF16, 5, 1, true>(k, w, x, ldx, M, y, ldy, st, s2);
             if (ring == 3) return nvq_launch_signed_as<XF16, 5, 3, true>(k, w, x, ldx, M, y, ldy, st, s2);
             if (ring == 4) return nvq_launch_signed_as<XF16, 5, 4, true>(k, w, x, ldx, M, y, ldy, st, s2);
@@ -991,7 +991,7 @@ static int nvq_mfma_any(const NvqK &k, const uint8_t *w, const uint16_t *x, int6
     // tiles; four were slower on both config 3 shapes (1.2 vs 1.4 TB/s).  MFQ_NVQ_NB overrides for tuning.
     if (nvq_signed_capable(k, M)) return nvq_launch_signed<XF16>(k, w, x, ldx, M, y, ldy, st);
     const int64_t wpb = (k.nsteps < 8 ? k.nsteps : 8) * ceil_div(M, 16);  // waves of a block x 16-row tiles
-    static const int env_nb = [] { const char *e = getenv("MFQ_NVQ_NB"); return e ? atoi(e) : 0; }();
+    static const int env_nb = tune_env("MFQ_NVQ_NB", 0);
     if (env_nb == 4) return nvq_launch_mfma<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
     if (env_nb == 1) return nvq_launch_mfma<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
     if (env_nb == 2 || ceil_div(k.n_rowblocks, 2) * wpb >= 1024) return nvq_launch_mfma<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
@@ -1170,7 +1170,7 @@ static bool nvq_prefill_capable(const NvqK &k) {
 // to measurements (17408x5120 and 5120x17408): 64 rows of streaming cost about 6 us + 1.7 us per MB of payload, the
 // prefill kernel a flat 38 us + 1 us per 1024 of K up to about a hundred rows (small grids are split over K).
 static int nvq_stream_max(const mfq_nvq_desc *d, const NvqK &k) {
-    static const int env = [] { const char *e = getenv("MFQ_NVQ_STREAM_MAX_M"); return e ? atoi(e) : 0; }();
+    static const int env = tune_env("MFQ_NVQ_STREAM_MAX_M", 0);
     if (env > 0) return env;
     if (!nvq_prefill_capable(k)) return kNvqStreamMaxM;
     const double t64 = 6.0 + 1.7e-6 * static_cast<double>(d->payload_bytes);

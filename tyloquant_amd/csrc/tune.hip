@@ -1,0 +1,96 @@
+// Tuning knobs (environment variables, read once), the device's CU count and the dynamic-LDS opt-in.
+#include <stdlib.h>
+#include <string.h>
+
+#include <atomic>
+#include <mutex>
+
+#include "common.hpp"
+#include "tune.hpp"
+
+namespace mfq {
+
+namespace {
+struct Knob {
+    const char *name;
+    const char *what;
+    int value;
+    bool read;
+};
+// 0 = "automatic" wherever the default is 0
+Knob g_knobs[] = {
+    {"MFQ_GEMV_WAVES", "waves a decode GEMV grid aims for before a wave takes more than one item", 0, false},
+    {"MFQ_GEMV_SPW", "K steps per wave of the NINT GEMV (0 = by shape)", 0, false},
+    {"MFQ_GEMV_RBW", "row-blocks per block of the NINT GEMV (0 = by shape)", 0, false},
+    {"MFQ_GEMV_VALU_MAX_M", "rows up to which the vector-ALU GEMV runs before the streaming MFMA kernel", 0, false},
+    {"MFQ_MFMA_NB", "row-blocks per wave of the NINT streaming MFMA kernel (0 = by shape)", 0, false},
+    {"MFQ_STREAM_MAX_M", "rows up to which NINT streams instead of the prefill kernel (0 = cost model)", 0, false},
+    {"MFQ_PREFILL_SPLITS", "splits over K of a NINT prefill launch (0 = by shape)", 0, false},
+    {"MFQ_PREFILL_BIG", "experimental 128 x 384 prefill tiles (0 = off)", 0, false},
+    {"MFQ_NVQ_NB", "row-blocks per wave of the NVQ streaming kernel (0 = by shape)", 0, false},
+    {"MFQ_NVQ_STREAM_MAX_M", "rows up to which NVQ streams instead of the prefill kernel (0 = cost model)", 0, false},
+    {"MFQ_NVQ_SIGNED_OFF", "1 = NVQ small batches on the older streaming kernel", 0, false},
+    {"MFQ_NVQ_SIGNED_MAX_M", "rows up to which the NVQ signed-table kernel runs", 0, false},
+    {"MFQ_NVQ_RING", "weight ring depth of the five-row-block NVQ kernel", 0, false},
+    {"MFQ_NEPQ_NB", "row-blocks per wave of the NEPQ streaming kernel (0 = by shape)", 0, false},
+    {"MFQ_NEPQ_PREFILL_MIN_M", "rows from which NEPQ takes the prefill kernel (0 = default)", 0, false},
+    {"MFQ_MOE_SPLIT", "0 = no one-launch MoE decode form", 0, false},
+    {"MFQ_MOE_DEC_WAVES", "waves per block of the MoE decode launch", 0, false},
+    {"MFQ_MOE_DEC_RBW", "row-blocks per block of the MoE decode launch (0 = by shape)", 0, false},
+    {"MFQ_MOE_PREFILL_PAIRS", "pairs per expert from which mapped MoE calls take the prefill kernel (0 = default)", 0, false},
+    {"MFQ_MOE_NB", "row-blocks per wave of the MoE streaming kernel (0 = by shape)", 0, false},
+};
+std::mutex g_mu;
+std::atomic<int> g_cu_override{0};
+std::atomic<int> g_cu_cached[64];
+}  // namespace
+
+int tune_env(const char *name, int dflt) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    for (Knob &k : g_knobs) {
+        if (strcmp(k.name, name) != 0) continue;
+        if (!k.read) {
+            const char *e = getenv(name);
+            k.value = e ? atoi(e) : dflt;
+            k.read = true;
+        }
+        return k.value;
+    }
+    return dflt;  // not in the table: still honoured, but not listed
+}
+
+int device_cu_count() {
+    const int forced = g_cu_override.load(std::memory_order_relaxed);
+    if (forced > 0) return forced;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = g_cu_cached[dev].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    g_cu_cached[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
+int allow_dynamic_lds(const void *kernel, size_t lds, const char *what) {
+    if (lds <= 65536) return MFQ_OK;
+    if (lds > kMaxDynamicLds) return fail(MFQ_ERR_UNSUPPORTED, "%s: %zu bytes of LDS exceed the %zu a block can have", what, lds, kMaxDynamicLds);
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return fail(MFQ_ERR_LAUNCH, "%s: %zu bytes of LDS: %s", what, lds, hipGetErrorString(e));
+    return MFQ_OK;
+}
+
+}  // namespace mfq
+
+using namespace mfq;
+
+extern "C" void mfq_hip_set_cu_count(int n) { g_cu_override.store(n > 0 ? n : 0, std::memory_order_relaxed); }
+
+extern "C" const char *mfq_hip_config(void) {
+    static thread_local char buf[2048];
+    size_t off = 0;
+    off += snprintf(buf + off, sizeof(buf) - off, "cu_count=%d", device_cu_count());
+    std::lock_guard<std::mutex> lock(g_mu);
+    for (const Knob &k : g_knobs)
+        if (k.read && off < sizeof(buf)) off += snprintf(buf + off, sizeof(buf) - off, " %s=%d", k.name, k.value);
+    return buf;
+}

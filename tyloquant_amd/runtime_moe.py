@@ -174,14 +174,14 @@ class NintMoeWeight:
 
     __call__ = forward
 
-    def decode_capable(self, shared: NintWeight | None = None) -> bool:
-        """Whether forward_decode takes these cohorts (every one has a batch-1 unit) and this shared tensor."""
-        def unit(d):
-            return d.kind == 1 or (d.bits == 5 and d.gs == 28)
-        if not all(unit(p.desc) for p in self.pools) or len(self.pools) + (shared is not None) > 8:
+    def decode_capable(self, shared: NintWeight | None = None, tokens: int = 1, routes: int = 1, swiglu=False) -> bool:
+        """Whether forward_decode takes these cohorts, this shared tensor and this many (token, route) pairs: the
+        library's own answer (unit per cohort, shared tensor's shape, the block's LDS need, the row count)."""
+        if shared is not None and shared.neuron_len != self.neuron_len:
             return False
-        return shared is None or (unit(shared.desc) and shared.out == self.out_per_expert and
-                                  shared.neuron_len == self.neuron_len)
+        return bool(L.lib().mfq_hip_moe_decode_capable(
+            self._pool_array, len(self.pools), self.out_per_expert, self.neuron_len,
+            C.byref(shared.desc) if shared is not None else None, int(tokens), int(routes), int(bool(swiglu))))
 
     def forward_decode(self, x: torch.Tensor, ids: torch.Tensor, shared: NintWeight | None = None, swiglu=False,
                        routed=False, out_dtype=torch.float16) -> torch.Tensor:
@@ -250,7 +250,8 @@ def nint_moe_ffn_forward(gate_up: NintMoeWeight, down: NintMoeWeight, x: torch.T
                       1e-20, router_scale)
     route = build_moe_route_plan(ids, gate_up.n_experts)
     sgu, sdn = shared if shared is not None else (None, None)
-    if route.ids_dst is None and gate_up.decode_capable(sgu) and down.decode_capable(sdn):
+    T_, R_ = ids.shape
+    if route.ids_dst is None and gate_up.decode_capable(sgu, T_, R_, True) and down.decode_capable(sdn, T_, R_):
         # decode step: gate/up + SwiGLU of the routes and of the shared expert in one launch, the down projections in
         # a second one, then the weighted sum
         T, R = ids.shape
