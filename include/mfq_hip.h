@@ -128,6 +128,17 @@ int mfq_hip_nint_gemv_argmax(const mfq_nint_desc *d, const void *weight, const v
                              int64_t ldx, int M, float *logits, int64_t ldl, int64_t *token,
                              void *workspace, size_t workspace_bytes, mfq_stream_t stream);
 
+/* mfq_hip_nint_gemv_argmax for callers that cannot allocate device memory or carry a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid allocation): the scratch is a 4 MiB device array built into the
+ * library (one copy per GPU, held until the process ends).  No counterpart in the reference.  Same arguments and
+ * results as mfq_hip_nint_gemv_argmax without the workspace pair; MFQ_ERR_WORKSPACE when
+ * mfq_hip_nint_gemv_argmax_workspace_bytes(d, M) exceeds 4 MiB (M = 1 fits any vocabulary up to about 900k; with
+ * logits passed in, far more).  Allocates nothing and frees nothing; the first call on a device looks the array's
+ * address up.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race. */
+int mfq_hip_nint_gemv_argmax_static(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
+                                    int64_t ldx, int M, float *logits, int64_t ldl, int64_t *token,
+                                    mfq_stream_t stream);
+
 /* Any-M entry: the streaming kernels of mfq_hip_nint_gemv up to a crossover that depends on the tensor (32 to
  * 512 rows; 256 for profiles without a prefill kernel), above that a block-tiled MFMA GEMM with in-register
  * dequantization (the paired profiles and NINT5-28) or dequantize-to-fp16 + MFMA GEMM.  The workspace (size

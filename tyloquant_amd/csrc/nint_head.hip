@@ -2,6 +2,8 @@
 // LM-head GEMV that also delivers the arg-max of the logits (greedy decoding never reads the logits back).
 #include <limits.h>
 
+#include <mutex>
+
 #include "common.hpp"
 #include "gemv_common.hpp"
 #include "nint_body.hpp"
@@ -269,6 +271,54 @@ extern "C" int mfq_hip_nint_gemv_argmax(const mfq_nint_desc *d, const void *weig
     }
     hipLaunchKernelGGL(argmax_final_kernel, dim3(static_cast<unsigned>(M)), dim3(1024), 0, st, vals, idxs, nb, slots, token);
     return check_launch("nint_argmax_final");
+}
+
+// ---- the same call for callers that cannot allocate ---------------------------------------------------------
+// The per-block winners (and the logits, when the caller passes none) live in a file-scope device array instead of a
+// caller workspace.  Each GPU holds its own copy of the array at its own address: the address is looked up once per
+// device, with that device current, and only that pointer is ever handed to a kernel.
+constexpr size_t kStaticScratchBytes = 4u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[64] = {nullptr};
+
+// Device address of `scratch` on the current device (0 on failure, with the error text set).
+void *static_scratch() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= 64) {
+        fail(MFQ_ERR_LAUNCH, "nint_gemv_argmax_static: hipGetDevice: %s", hipGetErrorString(e));
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            fail(MFQ_ERR_LAUNCH, "nint_gemv_argmax_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int mfq_hip_nint_gemv_argmax_static(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
+                                               int64_t ldx, int M, float *logits, int64_t ldl, int64_t *token,
+                                               mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && token, MFQ_ERR_INVALID, "nint_gemv_argmax_static: null argument");
+    MFQ_REQUIRE(M >= 1 && M <= 65535, MFQ_ERR_INVALID, "nint_gemv_argmax_static: M=%d outside [1, 65535]", M);
+    const size_t need = mfq_hip_nint_gemv_argmax_workspace_bytes(d, M);
+    MFQ_REQUIRE(need <= kStaticScratchBytes, MFQ_ERR_WORKSPACE,
+                "nint_gemv_argmax_static: %d rows of %d logits need %zu bytes of scratch, the built-in buffer holds %zu; use "
+                "mfq_hip_nint_gemv_argmax with a workspace", M, d->out, need, kStaticScratchBytes);
+    void *ptr = static_scratch();
+    if (!ptr) return MFQ_ERR_LAUNCH;
+    // nothing in the buffer has to start at zero: every slot the final pass reads is written by this call's first stage
+    return mfq_hip_nint_gemv_argmax(d, weight, x, x_dtype, ldx, M, logits, ldl, token, ptr, kStaticScratchBytes, stream);
 }
 
 extern "C" int mfq_hip_input_gate(const void *x, const void *gate, int x_dtype, int64_t ldx, int64_t ldg, int M, int K,
