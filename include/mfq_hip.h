@@ -99,6 +99,25 @@ int mfq_hip_nint_gemv_glu(const mfq_nint_desc *d, const void *weight, const void
                           int64_t ldx, int M, void *hidden, int out_dtype, int64_t ldh, int activation,
                           mfq_stream_t stream);
 
+/* Decode feed-forward block in ONE launch, one activation row: hidden = act(gate x) * (up x) as fp16, y = down hidden
+ * (fp32 [down.out]).  gate_up is the [2 W, H] gate/up tensor (gate rows first), down the [N, W] tensor of the same
+ * NINT profile; activation is MFQ_GLU_*.  One block per compute unit, all resident; the hidden vector crosses the
+ * chip behind a grid-wide barrier while the down weights are already streaming, so the second launch's ramp is gone.
+ * Replaces the batch-1 branch of FFN::forward_impl, gate_up.forward_swiglu(x) followed by down.forward(act)
+ * (cpp_runtime/mfq_decode.cpp:11199-11209), and its opt-in fused pair nint_ffn_gate_up_swiglu_quant_ws_cuda +
+ * nint_matmul_qx (:11176-11198).  Same values as mfq_hip_nint_gemv_glu (fp16 out) + mfq_hip_nint_gemv up to the order
+ * of the fp32 sums over K.  The workspace (size from the query; 0 = this pair of tensors is outside the kernel, as is
+ * MFQ_ERR_UNSUPPORTED from the call: run the two launches then) holds the barrier words and the hidden vector; its
+ * first 4096 bytes (one barrier flag per compute unit) must be zero before the first call
+ * (mfq_hip_nint_ffn_decode_workspace_init, or any memset) and belong to the library from then on: every call advances
+ * all flags by one.  Calls that share a workspace must not overlap, and a workspace stays with one device.  If another kernel keeps compute units
+ * busy so that the blocks cannot all run at once, the barrier gives up after a bounded number of polls and y is NaN. */
+size_t mfq_hip_nint_ffn_decode_workspace_bytes(const mfq_nint_desc *gate_up, const mfq_nint_desc *down);
+int mfq_hip_nint_ffn_decode_workspace_init(void *workspace, mfq_stream_t stream);
+int mfq_hip_nint_ffn_decode(const mfq_nint_desc *gate_up, const void *gate_up_weight, const mfq_nint_desc *down,
+                            const void *down_weight, const void *x, int x_dtype, int activation, float *y,
+                            void *workspace, size_t workspace_bytes, mfq_stream_t stream);
+
 /* Token-embedding rows from the packed table: out[n, 0:neuron_len] = row ids[n] of the dequantized tensor (the
  * values of mfq_hip_nint_dequant_f32, rounded once more to out_dtype: MFQ_X_BF16, MFQ_X_F16 or MFQ_X_F32); ids
  * outside [0, out) give a row of zeros.  ids are device int64.  Replaces

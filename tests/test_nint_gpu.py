@@ -315,3 +315,68 @@ def test_gemv_long_neurons(K):
         h = R.nint_matmul_swiglu(lin.weight, x).float().cpu().numpy()
         want = O.moe_swiglu(O.linear_forward_f64(deq, xf).astype(np.float32))
         assert rel_l2(h, want) < 2e-3
+
+
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5)])
+@pytest.mark.parametrize("H,W,N,cus", [(256, 384, 256, 8), (4096, 112, 128, 8), (520, 368, 48, 8), (512, 8448, 64, 0),
+                                       (1024, 160, 4096, 0)])
+def test_ffn_decode_one_launch(cu_count, bits, gs, sb, H, W, N, cus):
+    """The one-launch decode FFN (gate/up + GLU, grid barrier, down) against the oracle's fp64 FFN and the two-launch
+    path.  With the grid sized for 8 compute units the blocks own three row-block pairs and two down row-blocks;
+    W = 8448 gives the down phase two K steps per wave on the full grid; H = 520 ends inside a group; N = 4096 has
+    more down row-blocks than gate/up pairs.  Called twice per activation type: every block's barrier flag advances by one per call."""
+    from tyloquant_amd import _lib as L
+    from tyloquant_amd import runtime as R
+    if cus:
+        cu_count(cus)
+    if W == 8448 and gs == 16:
+        W = 8192                      # 32 steps: two per wave, as 8448 gives the wider groups
+    rng = np.random.default_rng(bits * 1000 + H + W)
+    tg = O.quantize_nint((rng.standard_normal((2 * W, H)) * 0.02).astype(np.float32), bits, gs, sb)
+    td = O.quantize_nint((rng.standard_normal((N, W)) * 0.02).astype(np.float32), bits, gs, sb)
+    gu, dn = _load(tg).weight, _load(td).weight
+    assert L.lib().mfq_hip_nint_ffn_decode_workspace_bytes(gu.desc, dn.desc) > 0
+    dg, dd = O.dequantize_nint(tg), O.dequantize_nint(td)
+    for dtype, act, glu in ((torch.bfloat16, L.GLU_SILU, O.moe_swiglu), (torch.float16, L.GLU_GELU, O.moe_geglu)):
+        x, xf = _x(rng, 1, H, dtype)
+        y1 = R.nint_ffn_decode(gu, dn, x, act, one_launch=True)
+        y2 = R.nint_ffn_decode(gu, dn, x, act, one_launch=True)
+        assert torch.equal(y1, y2) and bool(torch.isfinite(y1).all())
+        hidden = glu(O.linear_forward_f64(dg, xf).astype(np.float32)).astype(np.float64)
+        ref = hidden @ dd.astype(np.float64).T
+        y = y1.cpu().numpy()
+        assert rel_l2(y, ref) < REL_TOL, (dtype, rel_l2(y, ref))
+        assert np.abs(y - ref).max() < ABS_TOL
+        two = R.nint_matmul(dn, R._nint_matmul_glu(gu, x, torch.float16, act)).cpu().numpy()
+        assert rel_l2(y, two) < 1e-4                     # same hidden rounding, another order of the sums over K
+    G = cus or 256
+    words = gu._ffn_ws[:4096].view(torch.int32).cpu().numpy()
+    assert np.all(words[:G] == 4) and words[G] == 0       # every block crossed four barriers; the error word is clear
+
+
+def test_ffn_decode_shapes_outside_the_kernel_take_two_launches():
+    """Different profiles for gate/up and down, or more work per wave than the kernel keeps in registers: the
+    workspace query says 0, the C entry point refuses with a message, and the host path runs the two launches."""
+    import ctypes as C
+    from tyloquant_amd import _lib as L
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(3)
+    H, W, N = 256, 128, 64
+    tg = O.quantize_nint((rng.standard_normal((2 * W, H)) * 0.02).astype(np.float32), 4, 32, 6)
+    td = O.quantize_nint((rng.standard_normal((N, W)) * 0.02).astype(np.float32), 3, 24, 5)
+    gu, dn = _load(tg).weight, _load(td).weight
+    lib = L.lib()
+    assert lib.mfq_hip_nint_ffn_decode_workspace_bytes(gu.desc, dn.desc) == 0
+    x, xf = _x(rng, 1, H)
+    y = torch.empty((1, N), dtype=torch.float32, device="cuda")
+    ws = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    p = lambda t: C.c_void_p(t.data_ptr())
+    rc = lib.mfq_hip_nint_ffn_decode(C.byref(gu.desc), p(gu.data), C.byref(dn.desc), p(dn.data), p(x), L.X_BF16, L.GLU_SILU,
+                                     p(y), p(ws), 4096, None)
+    assert rc == 2 and b"outside the one-launch kernel" in lib.mfq_hip_last_error()
+    out = R.nint_ffn_decode(gu, dn, x, one_launch=True).cpu().numpy()
+    hidden = O.moe_swiglu(O.linear_forward_f64(O.dequantize_nint(tg), xf).astype(np.float32)).astype(np.float64)
+    assert rel_l2(out, hidden @ O.dequantize_nint(td).astype(np.float64).T) < REL_TOL
+    # three rows: the batch path
+    x3, x3f = _x(rng, 3, H)
+    assert R.nint_ffn_decode(gu, dn, x3).shape == (3, N)

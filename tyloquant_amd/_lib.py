@@ -64,6 +64,10 @@ _SIGS = {
     "mfq_hip_nint_gemv_swiglu": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, C.c_int, i64, vp]),
     "mfq_hip_input_gate": (C.c_int, [vp, vp, C.c_int, i64, i64, C.c_int, C.c_int, C.c_int, vp, i64, vp]),
     "mfq_hip_nint_gemv_glu": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, C.c_int, i64, C.c_int, vp]),
+    "mfq_hip_nint_ffn_decode_workspace_bytes": (sz, [C.POINTER(NintDesc), C.POINTER(NintDesc)]),
+    "mfq_hip_nint_ffn_decode_workspace_init": (C.c_int, [vp, vp]),
+    "mfq_hip_nint_ffn_decode": (C.c_int, [C.POINTER(NintDesc), vp, C.POINTER(NintDesc), vp, vp, C.c_int, C.c_int, vp, vp, sz,
+                                          vp]),
     "mfq_hip_nint_embedding": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, vp, C.c_int, i64, vp]),
     "mfq_hip_nint_gemv_argmax_workspace_bytes": (sz, [C.POINTER(NintDesc), C.c_int]),
     "mfq_hip_nint_gemv_argmax": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, vp, sz, vp]),

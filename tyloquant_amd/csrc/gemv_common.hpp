@@ -138,13 +138,16 @@ __device__ __forceinline__ void stage_x_issue(const uint16_t *const (&xr)[MB], i
     if (ok) {
 #pragma unroll
         for (int m = 0; m < MB; ++m) {
+            // range-checked window over the row (empty for an absent row): a chunk outside the slice or the row is an
+            // out-of-range offset that returns zeros, so nothing here depends on the loaded data and the weight requests
+            // that follow go out without waiting for the activations
+            const __amdgpu_buffer_rsrc_t wx =
+                wave_window(reinterpret_cast<const uint8_t *>(xr[m]), xr[m] ? static_cast<uint32_t>(K) * 2u : 0u);
 #pragma unroll
             for (int c = 0; c < kXChunks; ++c) {
                 const int i = lane * 4 + c * 256;
-                const bool in = i < npairs && k0 + 2 * i + 8 <= K;  // else: a zero chunk, read from a safe place
-                u32x4_t v = {0u, 0u, 0u, 0u};
-                if (xr[m]) v = *reinterpret_cast<const u32x4_t *>(xr[m] + (in ? k0 + 2 * i : 0));
-                xg.v[m][c] = in ? v : u32x4_t{0u, 0u, 0u, 0u};
+                const bool in = i < npairs && k0 + 2 * i + 8 <= K;
+                xg.v[m][c] = __builtin_amdgcn_raw_buffer_load_b128(wx, in ? static_cast<uint32_t>(k0 + 2 * i) * 2u : kNoStep, 0, 0);
             }
         }
     }

@@ -235,7 +235,9 @@ __device__ __forceinline__ void nint_load_step(__amdgpu_buffer_rsrc_t win, uint3
     sc = __builtin_amdgcn_raw_buffer_load_b64(win, off + 1024 * D + (TAIL ? 256 : 0) + lane * 8, 0, 2);
 }
 
-template <class U, int MB>
+// SERIAL: keep the four units of the step apart in the instruction schedule (one unit's unpacked pairs and staged
+// activations live at a time), for kernels that hold other buffers in flight next to the step.
+template <class U, int MB, bool SERIAL = false>
 __device__ __forceinline__ void nint_compute_step(const uint32_t (&q)[4][U::D], uint32_t tails, u32x2_t sc, int lg0,
                                                   const uint32_t *xs, const float *xsum, int npairs, int ngl,
                                                   float (&accS)[MB], float (&accM)[MB]) {
@@ -260,6 +262,7 @@ __device__ __forceinline__ void nint_compute_step(const uint32_t (&q)[4][U::D], 
             accS[m] = fmaf(ss, a[m], accS[m]);
             accM[m] = fmaf(sm, xg[m], accM[m]);
         }
+        if constexpr (SERIAL) __builtin_amdgcn_sched_barrier(0);
     }
 }
 

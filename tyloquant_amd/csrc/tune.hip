@@ -38,6 +38,8 @@ Knob g_knobs[] = {
     {"MFQ_MOE_DEC_WAVES", "waves per block of the MoE decode launch", 0, false},
     {"MFQ_MOE_DEC_RBW", "row-blocks per block of the MoE decode launch (0 = by shape)", 0, false},
     {"MFQ_MOE_PREFILL_PAIRS", "pairs per expert from which mapped MoE calls take the prefill kernel (0 = default)", 0, false},
+    {"MFQ_FFN_SPIN_LIMIT", "polls after which the one-launch FFN's grid barrier gives up", 0, false},
+    {"MFQ_FFN_TRACE", "1 = the one-launch FFN records per-block clocks behind its workspace", 0, false},
     {"MFQ_MOE_NB", "row-blocks per wave of the MoE streaming kernel (0 = by shape)", 0, false},
 };
 std::mutex g_mu;
