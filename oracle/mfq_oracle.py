@@ -29,6 +29,12 @@ reference tree).  Parity status of each function:
                                    mfq/formats/nint8_zero.py:107-218 (the GGML Q8_0 rule: closed form)
     moe_swiglu / moe_geglu / input_mul   mfq/kernels/cuda/glu.cuh:5-16, cpp_runtime/mfq_decode.cpp:8395-8417
 
+  additionally pinned by reference-written blobs and reference-dequantized values
+  (tests/golden/reference_blobs.npz, made by tests/golden/make_reference_blobs.py; tests/test_reference_blobs.py)
+    pack_nint / unpack_nint / dequantize_nint, pack_nvq_jsc / pack_nvq_plain / unpack_nvq / dequantize_nvq_jsc /
+    dequantize_nvq (incl. the index-parity sign rule on e8_256), pack_nepq / unpack_nepq / dequantize_nepq,
+    pack_nint_moe / unpack_nint_moe / dequantize_expertwise
+
   pinned by golden vectors written from the reference's own numpy quantizer
   (tests/golden/nint_quant_vectors.npz, made by tests/golden/make_nint_quant_vectors.py)
     make_qkx2 / quantize_nint      mfq/formats/nint.py:119-174, mfq/quantize/nint_quant.py:745-893
