@@ -380,3 +380,31 @@ def test_ffn_decode_shapes_outside_the_kernel_take_two_launches():
     # three rows: the batch path
     x3, x3f = _x(rng, 3, H)
     assert R.nint_ffn_decode(gu, dn, x3).shape == (3, N)
+
+
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (6, 24, 6)])
+@pytest.mark.parametrize("scale", [1e-6, 1e-4, 1e4, 3e6])
+def test_gemv_bf16_rows_of_any_magnitude(bits, gs, sb, scale):
+    """The stated range contract: a bf16 row far outside fp16's comfortable range (all of it scaled by 1e-6 ... 3e6,
+    i.e. beyond 65504 and deep inside fp16's subnormals) gives the accuracy of an ordinary row on the batch-1 / batch-2
+    NINT kernels and the fused GLU, and on the prefill kernel; config 2's outlier channels (x 20) on top."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd import synth as P
+    rng = np.random.default_rng(int(scale * 1e6) % 1000 + bits)
+    out, K = 64, 2048
+    t = O.quantize_nint((rng.standard_normal((out, K)) * 0.02).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    deq = O.dequantize_nint(t)
+    for M in (1, 2, 300):
+        x = torch.from_numpy(P.activations(rng, M, K, outlier_frac=0.001) * np.float32(scale)).to(torch.bfloat16)
+        ref = O.linear_forward_f64(deq, x.float().numpy())
+        y = (lin(x.cuda()) if M > 2 else R.nint_matmul(lin.weight, x.cuda(), force="gemv")).cpu().numpy()
+        assert np.isfinite(y).all()
+        assert rel_l2(y, ref) < REL_TOL, (M, scale, rel_l2(y, ref))
+    if bits != 6:
+        x = torch.from_numpy(P.activations(rng, 1, K) * np.float32(scale)).to(torch.bfloat16)
+        g = R.nint_matmul(lin.weight, x.cuda(), force="gemv").cpu().numpy()
+        want = O.moe_swiglu(O.linear_forward_f64(deq, x.float().numpy()).astype(np.float32))
+        if scale <= 1e4:                                   # beyond that silu(gate) * up leaves fp16's range by itself
+            h = R.nint_matmul_swiglu(lin.weight, x.cuda(), torch.bfloat16).float().cpu().numpy()
+            assert rel_l2(h, want) < 6e-3                  # bf16 output: half an ulp is 4e-3

@@ -153,23 +153,83 @@ __device__ __forceinline__ void stage_x_issue(const uint16_t *const (&xr)[MB], i
     }
 }
 
+// Largest bf16 magnitudes (bit patterns without the sign) seen so far in the low and the high halves, kept as a packed
+// pair of 16-bit maxima: one AND and one packed max per dword.
+typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t absmax_bf16(uint32_t m, uint32_t pair) {
+    const u16x2_t a = __builtin_bit_cast(u16x2_t, m), b = __builtin_bit_cast(u16x2_t, pair & 0x7fff7fffu);
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
+}
+
+// Power of two that brings the wave's slice of a bf16 row to a largest magnitude near 2^12, as an fp32 bit pattern
+// (`mx` = largest magnitude pattern over the slice, the same in every lane); 1.0 for an all-zero or non-finite slice.
+// The reciprocal is exact and comes back through `inv`.
+__device__ __forceinline__ float slice_scale(uint32_t mx, float &inv) {
+    const uint32_t e = mx >> 7;  // biased exponent of the largest magnitude
+    if (e == 0u || e == 255u) {
+        inv = 1.f;
+        return 1.f;
+    }
+    const uint32_t field = min(266u - e, 253u);  // 2^(139 - e), capped so that the reciprocal stays normal
+    inv = __uint_as_float((254u - field) << 23);
+    return __uint_as_float(field << 23);
+}
+
+// Largest 16-bit half over the whole wave of the packed pairs absmax_bf16 collects: four DPP steps spread the maximum
+// over each row of 16 lanes, the four rows meet in scalar registers -- no LDS round trips.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t packed) {
+    int v = static_cast<int>(max(packed & 0xffffu, packed >> 16));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true));  // row_half_mirror
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true));  // row_mirror
+    const int a = max(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16));
+    const int b = max(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48));
+    return static_cast<uint32_t>(max(a, b));
+}
+
+// bf16 pair times a power of two, as an fp16 pair
+__device__ __forceinline__ uint32_t to_h2_scaled(uint32_t pair, float s) {
+    const float lo = __uint_as_float(pair << 16) * s, hi = __uint_as_float(pair & 0xffff0000u) * s;
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+}
+
 // Stage the wave's K-slice of the MB activation rows xr[m] (null = absent row) into its private
 // LDS region as fp16 (x[2i], x[2i+1]) pairs times BW::xscale, zero beyond K.  Next to it, per group
 // g, two floats: X_g = sum of x over the group and -T_g, T_g = sum over its pairs i of the staged
 // pair sum times BW::bw(i) (the bias the unpack trick adds to the dot product).  npairs is a multiple
 // of 8; xs is 16-byte aligned.  `xg` = what stage_x_issue requested.
-template <int XF16, int MB, class BW>
+// SCALE (bf16 rows only): the slice of every row is first multiplied by the power of two that brings its largest
+// magnitude near 2^12, so that rows of any magnitude keep their bits inside fp16's range; xinv[m] receives the
+// reciprocal, which the caller multiplies into the sums it forms from this slice (1 without SCALE or for fp16 rows).
+template <int XF16, int MB, class BW, bool SCALE = false>
 __device__ __forceinline__ void stage_x(const uint16_t *const (&xr)[MB], int K, int k0, int npairs, int gs, int ngl,
-                                        uint32_t *xs, float *xsum, int lane, const XRegs<MB> &xg) {
+                                        uint32_t *xs, float *xsum, int lane, const XRegs<MB> &xg, float *xinv = nullptr) {
+    constexpr bool RESCALE = SCALE && !XF16;
+    float sc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) sc[m] = 1.f;
     if (xg.on) {
 #pragma unroll
         for (int m = 0; m < MB; ++m) {
+            if constexpr (RESCALE) {
+                uint32_t mx = 0;
+#pragma unroll
+                for (int c = 0; c < kXChunks; ++c)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) mx = absmax_bf16(mx, xg.v[m][c][t]);
+                float inv;
+                sc[m] = slice_scale(wave_max_u32(mx), inv);
+                if (xinv) xinv[m] = inv;
+            } else if (xinv) {
+                xinv[m] = 1.f;
+            }
 #pragma unroll
             for (int c = 0; c < kXChunks; ++c) {
                 const int i = lane * 4 + c * 256;
                 u32x4_t v = xg.v[m][c];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) v[t] = to_h2<XF16>(v[t]);
+                for (int t = 0; t < 4; ++t) v[t] = RESCALE ? to_h2_scaled(v[t], sc[m]) : to_h2<XF16>(v[t]);
                 if constexpr (BW::SCALED) {
                     const int pos = i % (gs / 2);
 #pragma unroll
@@ -183,7 +243,7 @@ __device__ __forceinline__ void stage_x(const uint16_t *const (&xr)[MB], int K, 
         for (int m = 0; m < MB; ++m) {
             const uint16_t *p = xr[m];
             const bool vec = p && (reinterpret_cast<uintptr_t>(p) & 15) == 0;
-            for (int i = lane * 4; i < npairs; i += 256) {
+            auto fetch = [&](int i) {
                 const int kk = k0 + 2 * i;
                 u32x4_t v = {0u, 0u, 0u, 0u};
                 if (vec && kk + 8 <= K) {
@@ -197,8 +257,25 @@ __device__ __forceinline__ void stage_x(const uint16_t *const (&xr)[MB], int K, 
                         v[t] = lo | (hi << 16);
                     }
                 }
+                return v;
+            };
+            if constexpr (RESCALE) {  // a first pass over the slice for its largest magnitude
+                uint32_t mx = 0;
+                for (int i = lane * 4; i < npairs; i += 256) {
+                    const u32x4_t v = fetch(i);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) v[t] = to_h2<XF16>(v[t]);
+                    for (int t = 0; t < 4; ++t) mx = absmax_bf16(mx, v[t]);
+                }
+                float inv;
+                sc[m] = slice_scale(wave_max_u32(mx), inv);
+                if (xinv) xinv[m] = inv;
+            } else if (xinv) {
+                xinv[m] = 1.f;
+            }
+            for (int i = lane * 4; i < npairs; i += 256) {
+                u32x4_t v = fetch(i);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) v[t] = RESCALE ? to_h2_scaled(v[t], sc[m]) : to_h2<XF16>(v[t]);
                 if constexpr (BW::SCALED) {
                     const int pos = i % (gs / 2);
 #pragma unroll

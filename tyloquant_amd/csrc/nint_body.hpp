@@ -326,7 +326,8 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     MFQ_ISSUE(q0, t0, c0)
     MFQ_ISSUE(q1, t1, c1)
     MFQ_ISSUE(q2, t2, c2)
-    stage_x<XF16, MB, typename U::Bias>(xr, k.neuron_len, s0 * 16 * GS, npairs, GS, ngl, xs, xsum, lane, xg);
+    float xinv[MB];  // bf16 rows are staged times a per-wave power of two; the sums are scaled back when they are parked
+    stage_x<XF16, MB, typename U::Bias, true>(xr, k.neuron_len, s0 * 16 * GS, npairs, GS, ngl, xs, xsum, lane, xg, xinv);
 
     float accS[MB], accM[MB];
 #pragma unroll
@@ -340,7 +341,7 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
             _Pragma("unroll") for (int i = 1; i < kMaxRbw; ++i) if (crb == i) { a_s = ns[i]; a_m = nm[i]; } \
             float v[MB];                                                                                  \
             _Pragma("unroll") for (int m = 0; m < MB; ++m) {                                              \
-                v[m] = a_s * accS[m] - a_m * accM[m];                                                     \
+                v[m] = (a_s * accS[m] - a_m * accM[m]) * xinv[m];                                         \
                 accS[m] = accM[m] = 0.f;                                                                  \
             }                                                                                             \
             park_rows<MB>(v, red, crb * nwaves + wave, lane);                                             \
@@ -400,7 +401,8 @@ __device__ __forceinline__ void nint_generic_body(const NintK &k, const uint8_t 
     float *red = reinterpret_cast<float *>(lds + nwaves * (MB * (npairs + 2 * ngl)));
     XRegs<MB> xg;
     stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * gs, npairs, lane, xg);
-    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * gs, npairs, gs, ngl, xs, xsum, lane, xg);
+    float xinv[MB];
+    stage_x<XF16, MB, PlainBias, true>(xr, k.neuron_len, s0 * 16 * gs, npairs, gs, ngl, xs, xsum, lane, xg, xinv);
     const uint16_t *xh = reinterpret_cast<const uint16_t *>(xs);
 
     const int r = lane & 15, kb = lane >> 4;
@@ -440,7 +442,7 @@ __device__ __forceinline__ void nint_generic_body(const NintK &k, const uint8_t 
     const float ns = anchors[rb * 16 + r], nm = anchors[16 * k.n_rowblocks + rb * 16 + r];
     float v[MB];
 #pragma unroll
-    for (int m = 0; m < MB; ++m) v[m] = ns * accS[m] - nm * accM[m];
+    for (int m = 0; m < MB; ++m) v[m] = (ns * accS[m] - nm * accM[m]) * xinv[m];
     finish_rows<MB>(v, red, wave, nwaves, lane, rb, row_base, out_rows, yr);
 }
 

@@ -128,7 +128,8 @@ __global__ __launch_bounds__(1024) void nint_ffn_decode_kernel(FfnK p) {
         nint_load_step<DA, UA::TAIL>(win_a, i < items_a ? irb * rbba + is * sba : kNoStep, lane, qa[i], ta[i], ca[i]);
     }
     float *xsum_a = reinterpret_cast<float *>(xs + npairs_a);
-    stage_x<XF16, 1, typename UA::Bias>(xr, p.a.neuron_len, sa0 * 16 * GSA, npairs_a, GSA, ngl_a, xs, xsum_a, lane, xg);
+    float xinv[1];
+    stage_x<XF16, 1, typename UA::Bias, true>(xr, p.a.neuron_len, sa0 * 16 * GSA, npairs_a, GSA, ngl_a, xs, xsum_a, lane, xg, xinv);
 
     if (kb == 0) {
 #pragma unroll
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(1024) void nint_ffn_decode_kernel(FfnK p) {
             ffn_item(i, na, irb, is);
             nint_compute_step<UA, 1>(qa[i], ta[i], ca[i], is * 16 + kb, xs, xsum_a, npairs_a, ngl_a, accS, accM);
             if (is == na - 1) {
-                float v[1] = {anc[(2 * irb) * 16 + r] * accS[0] - anc[(2 * irb + 1) * 16 + r] * accM[0]};
+                float v[1] = {(anc[(2 * irb) * 16 + r] * accS[0] - anc[(2 * irb + 1) * 16 + r] * accM[0]) * xinv[0]};
                 park_rows<1>(v, red, (team * kFfnItems + irb) * p.wpt + tw, lane);
                 accS[0] = accM[0] = 0.f;
             }
