@@ -162,6 +162,14 @@ struct PairedUnit {
             }
         }
     }
+    // the same against activations already in registers (x[i] = staged pair i of the group)
+    __device__ static __forceinline__ float dot_regs(const uint32_t (&q)[D], uint32_t tail, const uint32_t (&x)[GS / 2], float acc) {
+        uint32_t v[GS / 2];
+        unpack(q, tail, v);
+#pragma unroll
+        for (int i = 0; i < GS / 2; ++i) acc = dot2h(v[i], x[i], acc);
+        return acc;
+    }
 };
 
 // Natural-order unit of any (bits <= 8, even groupsize): ceil(GS * BITS / 32) dwords, code i at bit i * BITS.
@@ -242,6 +250,37 @@ __device__ __forceinline__ void nint_compute_step(const uint32_t (&q)[4][U::D], 
                                                   const uint32_t *xs, const float *xsum, int npairs, int ngl,
                                                   float (&accS)[MB], float (&accM)[MB]) {
     constexpr int GS = U::GROUP;
+    if constexpr (MB == 1 && U::CBITS != 0 && !SERIAL) {
+        // one row: the staged pairs of unit j + 1 are read from LDS while unit j is unpacked and multiplied, so that
+        // the read latency is paid once per step, not once per unit
+        uint32_t xa[GS / 2], xb[GS / 2];
+        float2 sa, sb2;
+        auto fetch = [&](int j, uint32_t (&xr_)[GS / 2], float2 &st) {
+            const int lg = lg0 + 4 * j;
+#pragma unroll
+            for (int c = 0; c < GS / 8; ++c) {
+                const u32x4_t x = *reinterpret_cast<const u32x4_t *>(xs + lg * (GS / 2) + 4 * c);
+                xr_[4 * c] = x.x; xr_[4 * c + 1] = x.y; xr_[4 * c + 2] = x.z; xr_[4 * c + 3] = x.w;
+            }
+            st = *reinterpret_cast<const float2 *>(xsum + lg * 2);
+        };
+        auto unit = [&](int j, const uint32_t (&xr_)[GS / 2], float2 st) {
+            const uint32_t scw = (j < 2) ? sc.x : sc.y;
+            const float ss = ubyte_f32(scw, 2 * (j & 1)), sm = ubyte_f32(scw, 2 * (j & 1) + 1);
+            const float a = U::dot_regs(q[j], (tails >> (8 * j)) & 0xffu, xr_, st.y);
+            accS[0] = fmaf(ss, a, accS[0]);
+            accM[0] = fmaf(sm, st.x, accM[0]);
+        };
+        fetch(0, xa, sa);
+        fetch(1, xb, sb2);
+        unit(0, xa, sa);
+        fetch(2, xa, sa);
+        unit(1, xb, sb2);
+        fetch(3, xb, sb2);
+        unit(2, xa, sa);
+        unit(3, xb, sb2);
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int lg = lg0 + 4 * j;
@@ -282,6 +321,25 @@ __device__ __forceinline__ int gemv_red_offset(int nwaves, int mb, int spw, int 
     return nwaves * (mb * (spw * 16 * (gs / 2) + 2 * spw * 16));
 }
 
+// Tuning builds (-DMFQ_GEMV_TRACE) record the 100 MHz clock per wave at start / activations staged / each item
+// computed / end into mfq_trace_ptr[wave_global * 8 + slot].
+#ifdef MFQ_GEMV_TRACE
+__device__ long long *mfq_trace_ptr;
+// the readings stay in registers until the wave is done, so that no store sits among the loads being timed
+#define MFQ_TRACE_DECL long long trace_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#define MFQ_TRACE(slot) trace_t[slot] = __builtin_readcyclecounter()
+#define MFQ_TRACE_FLUSH                                                                                             \
+    do {                                                                                                            \
+        if (mfq_trace_ptr && lane == 0)                                                                             \
+            for (int i_ = 0; i_ < 8; ++i_)                                                                          \
+                mfq_trace_ptr[(static_cast<size_t>(blockIdx.x) * (blockDim.x >> 6) + wave) * 8 + i_] = trace_t[i_]; \
+    } while (0)
+#else
+#define MFQ_TRACE_DECL
+#define MFQ_TRACE(slot) do { } while (0)
+#define MFQ_TRACE_FLUSH do { } while (0)
+#endif
+
 template <class U, int XF16, int MB, bool RING = true, bool FLUSH = true>
 __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__restrict__ w, int rb0, int rbw,
                                                int row_base, int out_rows, const uint16_t *const (&xr)[MB],
@@ -299,6 +357,8 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     float *red = reinterpret_cast<float *>(lds + nwaves * (MB * (npairs + 2 * ngl)));
     const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes) * rb_step;
 
+    MFQ_TRACE_DECL
+    MFQ_TRACE(0);
     XRegs<MB> xg;
     stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * GS, npairs, lane, xg);
     const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
@@ -329,6 +389,7 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     float xinv[MB];  // bf16 rows are staged times a per-wave power of two; the sums are scaled back when they are parked
     stage_x<XF16, MB, typename U::Bias, true>(xr, k.neuron_len, s0 * 16 * GS, npairs, GS, ngl, xs, xsum, lane, xg, xinv);
 
+    MFQ_TRACE(1);
     float accS[MB], accM[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) accS[m] = accM[m] = 0.f;
@@ -359,8 +420,11 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
         }
     } else if constexpr (!RING) {  // at most 3 items: everything is already requested
         MFQ_COMPUTE(q0, t0, c0)
+        MFQ_TRACE(2);
         if (items > 1) MFQ_COMPUTE(q1, t1, c1)
+        MFQ_TRACE(3);
         if (items > 2) MFQ_COMPUTE(q2, t2, c2)
+        MFQ_TRACE(4);
     } else {
         uint32_t q3[4][D], t3;
         u32x2_t c3;
@@ -378,6 +442,8 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
 #undef MFQ_ISSUE
 #undef MFQ_COMPUTE
     if constexpr (FLUSH) flush_rows<MB>(red, nwaves, nrb, rb0, row_base, out_rows, yr);
+    MFQ_TRACE(5);
+    MFQ_TRACE_FLUSH;
 }
 
 template <int BITS, int GS, int XF16, int MB, bool RING = true>
