@@ -404,6 +404,22 @@ int mfq_hip_moe_weighted_reduce(const float *pair, const float *weights, int T, 
                                 mfq_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
+ * Expert residency (experts kept in host memory, a GPU arena of slots for the ones in use).
+ * ---------------------------------------------------------------------------------- */
+/* One byte range to copy: destination = device address, source_offset = offset into the staging buffer.
+ * The layout of MoeCacheScatterDescriptor (cpp_runtime/moe_cache_transfer.h:9-17). */
+typedef struct mfq_scatter_desc {
+    uint64_t destination, source_offset, nbytes;
+} mfq_scatter_desc;
+/* Copies n_transfers ranges out of `staging` (a device buffer the host has just filled with one copy: expert bodies,
+ * anchors, dispatch-table words, and at descriptor_offset the table of mfq_scatter_desc) to their destinations in one
+ * launch; max_bytes = the largest nbytes (sizes the grid: big ranges are spread over up to 64 blocks).  Ranges whose
+ * addresses and length are multiples of 16 move as 16-byte words.  Replaces moe_cache_scatter_cuda
+ * (cpp_runtime/moe_cache_transfer.h:19-23, mfq/kernels/cuda/moe.cu:45-77, 3532-3550). */
+int mfq_hip_cache_scatter(const void *staging, int64_t descriptor_offset, int n_transfers, int64_t max_bytes,
+                          mfq_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
  * helpers shared by the GEMM paths
  * ---------------------------------------------------------------------------------- */
 /* Plain fp16 x fp16 -> fp32 MFMA GEMM: y[M, N] = a[M, K] . b[N, K]^T (used after a full dequant). */

@@ -253,3 +253,49 @@ def test_moe_errors():
         NintMoeWeight.from_blob(blob + b"\0")
     with pytest.raises(RuntimeError, match="int32"):
         build_moe_route_plan(torch.zeros((2, 2), dtype=torch.int64).cuda(), 4)
+
+
+def test_expert_cache_keeps_a_working_set_resident():
+    """Experts in pinned host memory, a GPU arena of a few slots per cohort: whatever the route, the cached tensor gives
+    bit for bit what the fully resident tensor gives (same kernels, same bytes), through decode-size and mapped calls;
+    slots are reused least-recently-used first, experts already resident cost nothing, and a route that needs more
+    experts of a cohort than its arena holds is refused."""
+    from tyloquant_amd.runtime_moe import MoeExpertCache, NintMoeWeight, build_moe_route_plan
+    rng = np.random.default_rng(2025)
+    E, out, K, R = 12, 32, 96, 2
+    bits = [4, 3, 4, 3, 4, 3, 4, 3, 4, 3, 4, 3]           # two cohorts of six experts
+    t = synth.moe_random(rng, E, out, K, bits, quantize=True)
+    blob = O.pack_nint_moe(t)
+    full = NintMoeWeight.from_blob(blob)
+    probe = MoeExpertCache(1 << 30)
+    per_slot = sum(c.slot_bytes for c in probe.register_source(blob).cohorts)
+    cache = MoeExpertCache(3 * per_slot + 64)              # three slots per cohort
+    src = cache.register_source(blob, minimum_slots=2)
+    with pytest.raises(RuntimeError, match="finalized before inference"):
+        cache.prepare(src, [0])
+    cache.finalize()
+    assert [len(c.free) for c in src.cohorts] == [3, 3] and cache.allocated_bytes <= 3 * per_slot + 2 * 4096
+    with pytest.raises(RuntimeError, match="after cache finalization"):
+        cache.register_source(blob)
+    for step, T in enumerate([1, 2, 20, 1, 3, 20, 2]):
+        # experts 2k are 4-bit, 2k+1 are 3-bit: draw at most three of each cohort per call
+        even = rng.choice(np.arange(0, E, 2), size=3, replace=False)
+        odd = rng.choice(np.arange(1, E, 2), size=3, replace=False)
+        ids = np.stack([np.array([rng.choice(even), rng.choice(odd)]) for _ in range(T)]).astype(np.int32)
+        x = torch.from_numpy((rng.standard_normal((T, K)) * 0.1).astype(np.float32)).to(torch.bfloat16).cuda()
+        route = build_moe_route_plan(torch.from_numpy(ids).cuda(), E)
+        got = cache.forward(src, x, route)
+        want = full(x, route)
+        assert torch.equal(got.view(torch.int32), want.view(torch.int32)), (step, T)
+    st = cache.stats
+    sizes = [c.slot_bytes for c in src.cohorts]
+    assert st["misses"] >= 6 and st["evictions"] > 0 and st["hits"] > 0
+    assert st["misses"] * min(sizes) <= st["bytes"] <= st["misses"] * max(sizes)     # only missing experts travel
+    resident = {int(src.cohorts[ci].expert_ids[l]) for ci in range(2) for l in src.cohorts[ci].slot_of}
+    table = src.weight.expert_local.cpu().numpy()
+    assert {e for e in range(E) if table[e] >= 0} == resident          # the device table says what is resident
+    before = dict(st)
+    cache.prepare(src, sorted(resident))                                # all hits: nothing moves
+    assert st["bytes"] == before["bytes"] and st["launches"] == before["launches"]
+    with pytest.raises(RuntimeError, match="its arena holds 3"):
+        cache.prepare(src, [0, 2, 4, 6])

@@ -112,6 +112,7 @@ _SIGS = {
     "mfq_hip_moe_swiglu": (C.c_int, [vp, i64, C.c_int, C.c_int, vp, C.c_int, i64, vp]),
     "mfq_hip_moe_glu": (C.c_int, [vp, i64, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp]),
     "mfq_hip_moe_weighted_reduce": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]),
+    "mfq_hip_cache_scatter": (C.c_int, [vp, i64, C.c_int, i64, vp]),
     "mfq_hip_gemm_f16_nt": (C.c_int, [vp, i64, vp, i64, C.c_int, C.c_int, C.c_int, vp, i64, vp]),
 }
 

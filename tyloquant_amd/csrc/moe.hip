@@ -630,9 +630,45 @@ __global__ __launch_bounds__(256) void moe_reduce_kernel(const float *__restrict
     out[idx] = v;
 }
 
+// Expert residency: copies `n` byte ranges out of one staging buffer (already on the device) to their destinations --
+// the body and anchors of every expert that has just been brought in, and the table words that now point at its
+// slot.  blockIdx.x = transfer, blockIdx.y = slice of it: a multi-megabyte expert body is spread over many blocks so
+// that one launch moves the whole batch at HBM speed.
+__global__ __launch_bounds__(256) void cache_scatter_kernel(const uint8_t *__restrict__ staging, int64_t descriptor_offset) {
+    const mfq_scatter_desc d = reinterpret_cast<const mfq_scatter_desc *>(staging + descriptor_offset)[blockIdx.x];
+    uint8_t *dst = reinterpret_cast<uint8_t *>(static_cast<uintptr_t>(d.destination));
+    const uint8_t *src = staging + d.source_offset;
+    const uint64_t n = d.nbytes;
+    if (((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | n) & 15u) == 0) {
+        const uint64_t n16 = n >> 4, per = (n16 + gridDim.y - 1) / gridDim.y;
+        const uint64_t lo = per * blockIdx.y, hi = lo + per < n16 ? lo + per : n16;
+        const u32x4_t *in = reinterpret_cast<const u32x4_t *>(src);
+        u32x4_t *out = reinterpret_cast<u32x4_t *>(dst);
+        for (uint64_t i = lo + threadIdx.x; i < hi; i += 256) out[i] = __builtin_nontemporal_load(in + i);
+        return;
+    }
+    const uint64_t per = (n + gridDim.y - 1) / gridDim.y;
+    const uint64_t lo = per * blockIdx.y, hi = lo + per < n ? lo + per : n;
+    for (uint64_t i = lo + threadIdx.x; i < hi; i += 256) dst[i] = src[i];
+}
+
 }  // namespace mfq
 
 using namespace mfq;
+
+extern "C" int mfq_hip_cache_scatter(const void *staging, int64_t descriptor_offset, int n_transfers, int64_t max_bytes,
+                                     mfq_stream_t stream) {
+    MFQ_REQUIRE(staging && descriptor_offset >= 0 && (descriptor_offset & 7) == 0, MFQ_ERR_INVALID,
+                "cache_scatter: null staging buffer or misaligned descriptor table");
+    MFQ_REQUIRE(n_transfers >= 0 && n_transfers <= 65535 * 32, MFQ_ERR_INVALID, "cache_scatter: %d transfers", n_transfers);
+    if (n_transfers == 0) return MFQ_OK;
+    // slices of about 64 KB of the largest transfer, at most 64 per transfer
+    int64_t slices = max_bytes > 0 ? ceil_div(max_bytes, 65536) : 1;
+    slices = slices < 1 ? 1 : (slices > 64 ? 64 : slices);
+    hipLaunchKernelGGL(cache_scatter_kernel, dim3(static_cast<unsigned>(n_transfers), static_cast<unsigned>(slices)), dim3(256), 0,
+                       as_stream(stream), static_cast<const uint8_t *>(staging), descriptor_offset);
+    return check_launch("cache_scatter");
+}
 
 extern "C" int mfq_hip_moe_topk(const float *logits, const float *bias, int T, int E, int k, int mode, int normalize,
                                 float norm_floor, float scale, int32_t *ids, float *weights, mfq_stream_t stream) {

@@ -267,3 +267,184 @@ def nint_moe_ffn_forward(gate_up: NintMoeWeight, down: NintMoeWeight, x: torch.T
         sgu, sdn = shared
         sh = nint_matmul(sdn, moe_swiglu(nint_matmul(sgu, x)))
     return moe_weighted_reduce(dn, w, sh), ids, w
+
+
+# ---------------------------------------------------------------------------------------
+# Expert residency: experts in pinned host memory, a GPU arena of slots for the ones in use
+# ---------------------------------------------------------------------------------------
+class _HostCohort:
+    """One cohort of a cached NINTM tensor: its experts' device-layout bytes in pinned host memory, and the arena
+    (a NintWeight of `slots` experts) its resident experts live in."""
+
+    def __init__(self, pool: NintWeight, expert_ids, out_per_expert):
+        self.src_desc, self.expert_ids, self.out = pool.desc, np.asarray(expert_ids, dtype=np.int32), out_per_expert
+        self.host = torch.empty(pool.data.numel(), dtype=torch.uint8, pin_memory=True)
+        self.host.copy_(pool.data)
+        rbe = out_per_expert // 16
+        self.body_bytes = rbe * int(pool.desc.rowblock_bytes)
+        self.slot_bytes = self.body_bytes + 2 * out_per_expert * 4
+        self.arena: NintWeight | None = None
+        self.slot_of: dict[int, int] = {}        # local expert index -> slot
+        self.lru: list[int] = []                  # local indices, least recently used first
+        self.free: list[int] = []
+
+    def segments(self, local: int, slot: int):
+        """(source offset in the host copy, destination offset in the arena, bytes) of an expert's body, scale
+        anchors and minimum anchors."""
+        s, a, out = self.src_desc, self.arena.desc, self.out
+        return [(local * self.body_bytes, slot * self.body_bytes, self.body_bytes),
+                (int(s.anchors_off) + local * out * 4, int(a.anchors_off) + slot * out * 4, out * 4),
+                (int(s.anchors_off) + 16 * s.n_rowblocks * 4 + local * out * 4,
+                 int(a.anchors_off) + 16 * a.n_rowblocks * 4 + slot * out * 4, out * 4)]
+
+
+class MoeCachedSource:
+    """A NINTM tensor whose experts live in host memory; `weight` is the NintMoeWeight view over the arenas, valid for
+    the experts made resident by the last MoeExpertCache.prepare (MoeCachedSource, cpp_runtime/mfq_decode.cpp:6440-6915)."""
+
+    def __init__(self, n_experts, out_per_expert, neuron_len, cohorts):
+        self.n_experts, self.out_per_expert, self.neuron_len, self.cohorts = n_experts, out_per_expert, neuron_len, cohorts
+        self.cohort_of = np.full(n_experts, -1, dtype=np.int32)
+        self.local_of = np.full(n_experts, -1, dtype=np.int32)
+        for ci, c in enumerate(cohorts):
+            self.cohort_of[c.expert_ids] = ci
+            self.local_of[c.expert_ids] = np.arange(len(c.expert_ids), dtype=np.int32)
+        self.weight: NintMoeWeight | None = None
+
+
+class MoeExpertCache:
+    """GPU residency of routed experts under a byte budget (MoeExpertCache, cpp_runtime/mfq_decode.cpp:5941-7500).
+
+    register_source() parses a NINTM blob, lets the GPU write each cohort's device layout once and keeps it in pinned
+    host memory; finalize() splits the budget into per-cohort arenas of expert slots; prepare(source, experts) makes
+    the given experts resident -- least recently used slots are reused, the bytes of all missing experts travel as one
+    host-to-device copy of a staging buffer and one scatter launch (mfq_hip_cache_scatter), which also rewrites the
+    dispatch-table words -- after which source.weight runs the ordinary grouped kernels."""
+
+    def __init__(self, budget_bytes: int, device="cuda"):
+        if budget_bytes <= 0:
+            raise ValueError("MoE GPU cache budget must be positive")
+        self.budget_bytes, self.device = int(budget_bytes), torch.device(device)
+        self.sources: list[MoeCachedSource] = []
+        self.finalized = False
+        self.allocated_bytes = 0
+        self.stats = {"hits": 0, "misses": 0, "evictions": 0, "bytes": 0, "launches": 0}
+        self._stage_host = self._stage_dev = None
+
+    def register_source(self, blob, minimum_slots: int = 1) -> MoeCachedSource:
+        if self.finalized:
+            raise RuntimeError("cannot register a MoE source after cache finalization")
+        full = NintMoeWeight.from_blob(blob, self.device)
+        cohorts = [_HostCohort(p, ids, full.out_per_expert) for p, ids in zip(full.pools, full.pool_expert_ids)]
+        for c in cohorts:
+            c.minimum_slots = min(int(minimum_slots), len(c.expert_ids))
+        src = MoeCachedSource(full.n_experts, full.out_per_expert, full.neuron_len, cohorts)
+        self.sources.append(src)
+        del full                                   # the device copies of the pools go away; the host copies stay
+        return src
+
+    def finalize(self):
+        """Slots per cohort: its minimum, plus a share of what the budget leaves in proportion to the cohort's bytes
+        (never more slots than it has experts)."""
+        if self.finalized:
+            return
+        cohorts = [c for s in self.sources for c in s.cohorts]
+        need = sum(c.minimum_slots * c.slot_bytes for c in cohorts)
+        if need > self.budget_bytes:
+            raise RuntimeError(f"MoE GPU cache budget {self.budget_bytes} is below the minimum working set {need}")
+        spare, total = self.budget_bytes - need, sum(len(c.expert_ids) * c.slot_bytes for c in cohorts)
+        for c in cohorts:
+            extra = int(spare * (len(c.expert_ids) * c.slot_bytes / total) // c.slot_bytes)
+            slots = min(len(c.expert_ids), c.minimum_slots + extra)
+            desc = L.NintDesc()
+            d = c.src_desc
+            L.check(L.lib().mfq_hip_nint_plan(d.bits, d.sub_bits, d.gs, slots * c.out, d.neuron_len, C.byref(desc)))
+            c.arena = NintWeight(desc, torch.zeros(int(desc.total_bytes), dtype=torch.uint8, device=self.device),
+                                 (slots * c.out, d.neuron_len))
+            c.free = list(range(slots))
+            self.allocated_bytes += int(desc.total_bytes)
+        for s in self.sources:
+            s.weight = NintMoeWeight(s.n_experts, s.out_per_expert, s.neuron_len, [c.arena for c in s.cohorts],
+                                     [np.zeros(0, dtype=np.int32) for _ in s.cohorts], self.device)
+            s.weight.expert_pool = torch.from_numpy(s.cohort_of.copy()).to(self.device)
+            s.weight.expert_local = torch.full((s.n_experts,), -1, dtype=torch.int32, device=self.device)
+        self.finalized = True
+
+    def prepare(self, source: MoeCachedSource, experts) -> None:
+        """Make `experts` (ids, any order, duplicates allowed) resident in `source`."""
+        if not self.finalized:
+            raise RuntimeError("MoE cache must be finalized before inference")
+        wanted = sorted({int(e) for e in np.asarray(experts).reshape(-1) if 0 <= int(e) < source.n_experts})
+        per_cohort: dict[int, list[int]] = {}
+        for e in wanted:
+            per_cohort.setdefault(int(source.cohort_of[e]), []).append(e)
+        for ci, es in per_cohort.items():
+            if len(es) > len(source.cohorts[ci].free) + len(source.cohorts[ci].slot_of):
+                raise RuntimeError(f"MoE route needs {len(es)} experts of one cohort, its arena holds "
+                                   f"{len(source.cohorts[ci].free) + len(source.cohorts[ci].slot_of)}")
+        copies, table = [], []                     # (host tensor, src off, dst address, bytes), (expert, slot)
+        for ci, es in per_cohort.items():
+            c = source.cohorts[ci]
+            keep = {int(source.local_of[e]) for e in es}
+            for e in es:
+                local = int(source.local_of[e])
+                if local in c.slot_of:
+                    self.stats["hits"] += 1
+                    c.lru.remove(local)
+                    c.lru.append(local)
+                    continue
+                self.stats["misses"] += 1
+                if c.free:
+                    slot = c.free.pop()
+                else:
+                    victim = next(v for v in c.lru if v not in keep)
+                    c.lru.remove(victim)
+                    slot = c.slot_of.pop(victim)
+                    table.append((int(c.expert_ids[victim]), -1))
+                    self.stats["evictions"] += 1
+                c.slot_of[local] = slot
+                c.lru.append(local)
+                base = c.arena.data.data_ptr()
+                for so, do, nb in c.segments(local, slot):
+                    copies.append((c.host, so, base + do, nb))
+                table.append((e, slot))
+        if not copies and not table:
+            return
+        # staging image: the byte ranges (16-byte aligned), the table words, then the descriptors
+        off, plan = 0, []
+        for host, so, dst, nb in copies:
+            plan.append((off, host, so, dst, nb))
+            off += (nb + 15) & ~15
+        words_off = off
+        off += (4 * len(table) + 15) & ~15
+        desc_off = off
+        n = len(copies) + len(table)
+        total = desc_off + 24 * n
+        if self._stage_host is None or self._stage_host.numel() < total:
+            self._stage_host = torch.empty(max(total, 1 << 20), dtype=torch.uint8, pin_memory=True)
+            self._stage_dev = torch.empty(self._stage_host.numel(), dtype=torch.uint8, device=self.device)
+        else:
+            torch.cuda.current_stream().synchronize()      # the previous batch has left the pinned buffer
+        img = self._stage_host.numpy()
+        descs = np.zeros((n, 3), dtype=np.uint64)
+        for i, (o, host, so, dst, nb) in enumerate(plan):
+            img[o:o + nb] = host.numpy()[so:so + nb]
+            descs[i] = (dst, o, nb)
+        words = np.array([slot for _, slot in table], dtype=np.int32)
+        img[words_off:words_off + 4 * len(table)] = words.view(np.uint8)
+        local_ptr = source.weight.expert_local.data_ptr()
+        for j, (e, _) in enumerate(table):
+            descs[len(copies) + j] = (local_ptr + 4 * e, words_off + 4 * j, 4)
+        img[desc_off:total] = descs.reshape(-1).view(np.uint8)
+        self._stage_dev[:total].copy_(self._stage_host[:total], non_blocking=True)
+        biggest = max([nb for *_, nb in copies] + [4])
+        L.check(L.lib().mfq_hip_cache_scatter(_ptr(self._stage_dev), desc_off, n, biggest, _stream()))
+        self.stats["bytes"] += sum(nb for *_, nb in copies)
+        self.stats["launches"] += 1
+
+    def forward(self, source: MoeCachedSource, x: torch.Tensor, route: MoeRoutePlan) -> torch.Tensor:
+        """Grouped matmul of a cached tensor: reads the route's expert ids back to the host, makes them resident and
+        runs NintMoeWeight.forward on the arenas (the readback of begin_route_experts / finish_route_experts,
+        cpp_runtime/mfq_decode.cpp:6066-6180)."""
+        self.prepare(source, route.ids.cpu().numpy())
+        return source.weight.forward(x, route)
