@@ -46,6 +46,19 @@ int mfq_rt_moe_ffn_forward(void *gate_up, void *down, const void *x, int x_dtype
                            void *shared_gate_up, void *shared_down, float *out, int32_t *ids_out,
                            float *weights_out, void *stream);
 
+/* Expert residency (MoeExpertCache, cpp_runtime/mfq_decode.cpp:5941-7500): experts of the registered NINTM tensors stay
+ * in pinned host memory, the GPU holds budget_bytes worth of expert slots; forward makes the route's experts resident
+ * (least recently used slots are reused, one staged copy + one scatter launch) and runs the grouped matmul.
+ * ids: device int32 [T, R]; out: device fp32 [T * R, out_per_expert]; stats: hits, misses, evictions, bytes, launches.
+ * Sources are owned by their cache. */
+int mfq_rt_moe_cache_create(int64_t budget_bytes, void **cache);
+void mfq_rt_moe_cache_free(void *cache);
+int mfq_rt_moe_cache_register(void *cache, const void *blob, size_t n, int minimum_slots, void **source);
+int mfq_rt_moe_cache_finalize(void *cache);
+int mfq_rt_moe_cache_forward(void *cache, void *source, const void *x, int x_dtype, int64_t ldx, int routed_input,
+                             const int32_t *ids, int T, int R, float *out, void *stream);
+int mfq_rt_moe_cache_stats(void *cache, int64_t *out5);
+
 #ifdef __cplusplus
 }
 #endif

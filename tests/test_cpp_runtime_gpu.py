@@ -204,3 +204,41 @@ def test_cpp_nvq_ffn_swiglu_down(rt):
     assert "fused FFN weight layouts" in rt.mfq_rt_last_error().decode()
     for h in hs:
         rt.mfq_rt_free_quant_linear(h)
+
+
+def test_cpp_expert_cache_matches_the_resident_tensor():
+    """The C++ MoeExpertCache through its C view: three slots per cohort, routes over twelve experts, outputs bit for
+    bit those of the fully resident NintMoeWeight (Python twin over the same C ABI), hits / misses / evictions counted."""
+    import ctypes as C
+    from pathlib import Path
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_moe import MoeExpertCache, NintMoeWeight, build_moe_route_plan
+    lib = C.CDLL(str(Path(R.__file__).resolve().parent / "lib" / "libmfq_runtime.so"))
+    lib.mfq_rt_last_error.restype = C.c_char_p
+    rng = np.random.default_rng(31)
+    E, out, K = 12, 32, 96
+    t = synth.moe_random(rng, E, out, K, [4, 3] * 6, quantize=True)
+    blob = O.pack_nint_moe(t)
+    full = NintMoeWeight.from_blob(blob)
+    per_slot = sum(c.slot_bytes for c in MoeExpertCache(1 << 30).register_source(blob).cohorts)
+    cache, src = C.c_void_p(), C.c_void_p()
+    assert lib.mfq_rt_moe_cache_create(C.c_int64(3 * per_slot + 64), C.byref(cache)) == 0
+    assert lib.mfq_rt_moe_cache_register(cache, blob, C.c_size_t(len(blob)), 2, C.byref(src)) == 0, lib.mfq_rt_last_error()
+    assert lib.mfq_rt_moe_cache_finalize(cache) == 0, lib.mfq_rt_last_error()
+    for T in (1, 20, 2, 20, 1):
+        even = rng.choice(np.arange(0, E, 2), size=3, replace=False)
+        odd = rng.choice(np.arange(1, E, 2), size=3, replace=False)
+        ids = np.stack([np.array([rng.choice(even), rng.choice(odd)]) for _ in range(T)]).astype(np.int32)
+        ids_d = torch.from_numpy(ids).cuda()
+        x = torch.from_numpy((rng.standard_normal((T, K)) * 0.1).astype(np.float32)).to(torch.bfloat16).cuda()
+        got = torch.empty((T, 2, out), dtype=torch.float32, device="cuda")
+        rc = lib.mfq_rt_moe_cache_forward(cache, src, C.c_void_p(x.data_ptr()), 0, C.c_int64(K), 0, C.c_void_p(ids_d.data_ptr()),
+                                          T, 2, C.c_void_p(got.data_ptr()), None)
+        assert rc == 0, lib.mfq_rt_last_error()
+        want = full(x, build_moe_route_plan(ids_d, E))
+        assert torch.equal(got.view(torch.int32), want.view(torch.int32)), T
+    stats = (C.c_int64 * 5)()
+    assert lib.mfq_rt_moe_cache_stats(cache, stats) == 0
+    hits, misses, evictions, nbytes, launches = list(stats)
+    assert misses >= 6 and evictions > 0 and hits > 0 and nbytes > 0 and launches <= 5
+    lib.mfq_rt_moe_cache_free(cache)

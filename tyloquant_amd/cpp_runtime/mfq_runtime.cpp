@@ -625,6 +625,189 @@ void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &dow
     hip_check(hipStreamSynchronize(hs(stream)), "nint_moe_ffn_forward");
 }
 
+// ---- expert residency -----------------------------------------------------------------------------------------
+MoeExpertCache::MoeExpertCache(int64_t budget_bytes) : budget_bytes_(budget_bytes) {
+    if (budget_bytes <= 0) fail("MoE GPU cache budget must be positive");
+}
+MoeExpertCache::~MoeExpertCache() {
+    for (auto &s : sources_)
+        for (auto &c : s->cohorts)
+            if (c.host) (void)hipHostFree(c.host);
+    if (stage_host_) (void)hipHostFree(stage_host_);
+}
+
+MoeCachedSource *MoeExpertCache::register_source(const uint8_t *blob, size_t n, int minimum_slots) {
+    if (finalized_) fail("cannot register a MoE source after cache finalization");
+    NintMoeWeight full = NintMoeWeight::from_blob(blob, n);
+    auto src = std::make_unique<MoeCachedSource>();
+    src->n_experts = full.n_experts; src->out_per_expert = full.out_per_expert; src->neuron_len = full.neuron_len;
+    src->cohort_of.assign(full.n_experts, -1);
+    src->local_of.assign(full.n_experts, -1);
+    for (size_t pi = 0; pi < full.pools.size(); ++pi) {
+        MoeCachedSource::Cohort c;
+        c.src = full.pools[pi]->desc;
+        c.expert_ids = full.pool_expert_ids[pi];
+        c.host_bytes = static_cast<size_t>(c.src.total_bytes);
+        hip_check(hipHostMalloc(&c.host, c.host_bytes, hipHostMallocDefault), "hipHostMalloc");
+        hip_check(hipMemcpy(c.host, full.pools[pi]->data.get(), c.host_bytes, hipMemcpyDeviceToHost), "expert cache: copy to host");
+        c.body_bytes = static_cast<int64_t>(full.out_per_expert / 16) * c.src.rowblock_bytes;
+        c.slot_bytes = c.body_bytes + 2ll * full.out_per_expert * 4;
+        c.minimum_slots = std::min<int>(minimum_slots, static_cast<int>(c.expert_ids.size()));
+        for (size_t l = 0; l < c.expert_ids.size(); ++l) {
+            src->cohort_of[c.expert_ids[l]] = static_cast<int32_t>(pi);
+            src->local_of[c.expert_ids[l]] = static_cast<int32_t>(l);
+        }
+        src->cohorts.push_back(std::move(c));
+    }
+    sources_.push_back(std::move(src));
+    return sources_.back().get();  // `full` (the device copies of the pools) goes away here; the host copies stay
+}
+
+void MoeExpertCache::finalize() {
+    if (finalized_) return;
+    int64_t need = 0;
+    double total = 0;
+    for (auto &s : sources_)
+        for (auto &c : s->cohorts) {
+            need += c.minimum_slots * c.slot_bytes;
+            total += static_cast<double>(c.expert_ids.size()) * c.slot_bytes;
+        }
+    if (need > budget_bytes_)
+        fail("MoE GPU cache budget " + std::to_string(budget_bytes_) + " is below the minimum working set " + std::to_string(need));
+    const int64_t spare = budget_bytes_ - need;
+    for (auto &s : sources_) {
+        NintMoeWeight &w = s->weight;
+        w.n_experts = s->n_experts; w.out_per_expert = s->out_per_expert; w.neuron_len = s->neuron_len;
+        for (auto &c : s->cohorts) {
+            const double share = static_cast<double>(c.expert_ids.size()) * c.slot_bytes / total;
+            const int extra = static_cast<int>(static_cast<int64_t>(spare * share) / c.slot_bytes);
+            const int slots = std::min<int>(static_cast<int>(c.expert_ids.size()), c.minimum_slots + extra);
+            c.arena = std::make_shared<NintWeight>();
+            abi_check(mfq_hip_nint_plan(c.src.bits, c.src.sub_bits, c.src.gs, slots * s->out_per_expert, c.src.neuron_len,
+                                        &c.arena->desc));
+            c.arena->data = DeviceBuffer(static_cast<size_t>(c.arena->desc.total_bytes));
+            hip_check(hipMemset(c.arena->data.get(), 0, static_cast<size_t>(c.arena->desc.total_bytes)), "hipMemset");
+            allocated_bytes_ += c.arena->desc.total_bytes;
+            for (int i = slots - 1; i >= 0; --i) c.free_slots.push_back(i);
+            w.pools.push_back(c.arena);
+            w.pool_expert_ids.emplace_back();
+            mfq_moe_pool entry;
+            entry.desc = c.arena->desc;
+            entry.weight = c.arena->data.get();
+            w.pool_table.push_back(entry);
+        }
+        std::vector<int32_t> none(static_cast<size_t>(s->n_experts), -1);
+        w.expert_pool = DeviceBuffer::from_host(s->cohort_of.data(), 4 * s->cohort_of.size());
+        w.expert_local = DeviceBuffer::from_host(none.data(), 4 * none.size());
+    }
+    finalized_ = true;
+}
+
+void MoeExpertCache::prepare(MoeCachedSource &source, const int32_t *experts, size_t count, mfq_stream_t stream) {
+    if (!finalized_) fail("MoE cache must be finalized before inference");
+    std::vector<std::vector<int>> wanted(source.cohorts.size());
+    {
+        std::vector<int32_t> uniq(experts, experts + count);
+        std::sort(uniq.begin(), uniq.end());
+        uniq.erase(std::unique(uniq.begin(), uniq.end()), uniq.end());
+        for (int32_t e : uniq)
+            if (e >= 0 && e < source.n_experts) wanted[source.cohort_of[e]].push_back(e);
+    }
+    struct Copy { const uint8_t *src; uint64_t dst; int64_t nbytes; };
+    std::vector<Copy> copies;
+    std::vector<std::pair<int32_t, int32_t>> table;  // (expert, slot or -1)
+    const int out = source.out_per_expert;
+    for (size_t ci = 0; ci < wanted.size(); ++ci) {
+        auto &c = source.cohorts[ci];
+        const size_t capacity = c.free_slots.size() + c.slot_of.size();
+        if (wanted[ci].size() > capacity)
+            fail("MoE route needs " + std::to_string(wanted[ci].size()) + " experts of one cohort, its arena holds " + std::to_string(capacity));
+        std::vector<bool> keep(c.expert_ids.size(), false);
+        for (int e : wanted[ci]) keep[source.local_of[e]] = true;
+        for (int e : wanted[ci]) {
+            const int local = source.local_of[e];
+            auto hit = c.slot_of.find(local);
+            if (hit != c.slot_of.end()) {
+                ++stats_.hits;
+                c.lru.erase(std::find(c.lru.begin(), c.lru.end(), local));
+                c.lru.push_back(local);
+                continue;
+            }
+            ++stats_.misses;
+            int slot;
+            if (!c.free_slots.empty()) {
+                slot = c.free_slots.back();
+                c.free_slots.pop_back();
+            } else {
+                auto victim = std::find_if(c.lru.begin(), c.lru.end(), [&](int v) { return !keep[v]; });
+                slot = c.slot_of[*victim];
+                table.emplace_back(c.expert_ids[*victim], -1);
+                c.slot_of.erase(*victim);
+                c.lru.erase(victim);
+                ++stats_.evictions;
+            }
+            c.slot_of[local] = slot;
+            c.lru.push_back(local);
+            const uint8_t *h = static_cast<const uint8_t *>(c.host);
+            const uint64_t base = reinterpret_cast<uint64_t>(c.arena->data.get());
+            const mfq_nint_desc &a = c.arena->desc;
+            copies.push_back({h + static_cast<int64_t>(local) * c.body_bytes, base + static_cast<uint64_t>(slot) * c.body_bytes, c.body_bytes});
+            copies.push_back({h + c.src.anchors_off + static_cast<int64_t>(local) * out * 4,
+                              base + a.anchors_off + static_cast<uint64_t>(slot) * out * 4, out * 4ll});
+            copies.push_back({h + c.src.anchors_off + 16ll * c.src.n_rowblocks * 4 + static_cast<int64_t>(local) * out * 4,
+                              base + a.anchors_off + 16ull * a.n_rowblocks * 4 + static_cast<uint64_t>(slot) * out * 4, out * 4ll});
+            table.emplace_back(e, slot);
+        }
+    }
+    if (copies.empty() && table.empty()) return;
+    // staging image: byte ranges (16-byte aligned), table words, descriptors
+    size_t off = 0;
+    std::vector<size_t> at(copies.size());
+    int64_t biggest = 4;
+    for (size_t i = 0; i < copies.size(); ++i) {
+        at[i] = off;
+        off += (static_cast<size_t>(copies[i].nbytes) + 15) & ~size_t(15);
+        biggest = std::max(biggest, copies[i].nbytes);
+    }
+    const size_t words_off = off;
+    off += (4 * table.size() + 15) & ~size_t(15);
+    const size_t desc_off = off, n = copies.size() + table.size(), total = desc_off + sizeof(mfq_scatter_desc) * n;
+    hipStream_t st = hs(stream);
+    if (total > stage_bytes_) {
+        hip_check(hipStreamSynchronize(st), "expert cache: sync");
+        if (stage_host_) hip_check(hipHostFree(stage_host_), "hipHostFree");
+        stage_bytes_ = std::max<size_t>(total, size_t(1) << 20);
+        hip_check(hipHostMalloc(&stage_host_, stage_bytes_, hipHostMallocDefault), "hipHostMalloc");
+        stage_dev_ = DeviceBuffer(stage_bytes_);
+    } else {
+        hip_check(hipStreamSynchronize(st), "expert cache: sync");  // the previous batch has left the pinned buffer
+    }
+    uint8_t *img = static_cast<uint8_t *>(stage_host_);
+    auto *descs = reinterpret_cast<mfq_scatter_desc *>(img + desc_off);
+    for (size_t i = 0; i < copies.size(); ++i) {
+        std::memcpy(img + at[i], copies[i].src, static_cast<size_t>(copies[i].nbytes));
+        descs[i] = {copies[i].dst, at[i], static_cast<uint64_t>(copies[i].nbytes)};
+        stats_.bytes += copies[i].nbytes;
+    }
+    const uint64_t local_ptr = reinterpret_cast<uint64_t>(source.weight.expert_local.get());
+    for (size_t j = 0; j < table.size(); ++j) {
+        std::memcpy(img + words_off + 4 * j, &table[j].second, 4);
+        descs[copies.size() + j] = {local_ptr + 4ull * table[j].first, words_off + 4 * j, 4};
+    }
+    hip_check(hipMemcpyAsync(stage_dev_.get(), stage_host_, total, hipMemcpyHostToDevice, st), "expert cache: staged copy");
+    abi_check(mfq_hip_cache_scatter(stage_dev_.get(), static_cast<int64_t>(desc_off), static_cast<int>(n), biggest, stream));
+    ++stats_.launches;
+}
+
+void MoeExpertCache::forward(MoeCachedSource &source, const void *x, int x_dtype, int64_t ldx, bool routed_input,
+                             const MoeRoutePlan &route, float *out, mfq_stream_t stream) {
+    std::vector<int32_t> ids(static_cast<size_t>(route.tokens) * route.routes);
+    hip_check(hipMemcpyAsync(ids.data(), route.ids, 4 * ids.size(), hipMemcpyDeviceToHost, hs(stream)), "route readback");
+    hip_check(hipStreamSynchronize(hs(stream)), "route readback");
+    prepare(source, ids.data(), ids.size(), stream);
+    source.weight.forward(x, x_dtype, ldx, routed_input, route, out, stream);
+}
+
 // ---- MFQ1 container ---------------------------------------------------------------------------------------
 MfqFile::MfqFile(const std::string &path) {
     std::ifstream f(path, std::ios::binary);
@@ -802,6 +985,36 @@ int mfq_rt_nvq_ffn_swiglu_down(void *gate, void *up, void *down, const void *x, 
         nvq_ffn_swiglu_down(*g->nvq, *u->nvq, *d->nvq, x, x_dtype, ldx, M, y, hidden.get(),
                             static_cast<float *>(scratch.get()), static_cast<mfq_stream_t>(stream));
         hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "sync");
+    });
+}
+
+// expert residency: cache handle, source handle (owned by the cache)
+int mfq_rt_moe_cache_create(int64_t budget_bytes, void **cache) {
+    return guard([&] { *cache = new MoeExpertCache(budget_bytes); });
+}
+void mfq_rt_moe_cache_free(void *cache) { delete static_cast<MoeExpertCache *>(cache); }
+int mfq_rt_moe_cache_register(void *cache, const void *blob, size_t n, int minimum_slots, void **source) {
+    return guard([&] {
+        *source = static_cast<MoeExpertCache *>(cache)->register_source(static_cast<const uint8_t *>(blob), n, minimum_slots);
+    });
+}
+int mfq_rt_moe_cache_finalize(void *cache) {
+    return guard([&] { static_cast<MoeExpertCache *>(cache)->finalize(); });
+}
+int mfq_rt_moe_cache_forward(void *cache, void *source, const void *x, int x_dtype, int64_t ldx, int routed_input,
+                             const int32_t *ids, int T, int R, float *out, void *stream) {
+    return guard([&] {
+        auto *src = static_cast<MoeCachedSource *>(source);
+        MoeRoutePlan route = build_moe_route_plan(ids, T, R, src->n_experts, static_cast<mfq_stream_t>(stream));
+        static_cast<MoeExpertCache *>(cache)->forward(*src, x, x_dtype, ldx, routed_input != 0, route, out,
+                                                      static_cast<mfq_stream_t>(stream));
+        hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "sync");  // the route plan's buffers go away
+    });
+}
+int mfq_rt_moe_cache_stats(void *cache, int64_t *out5) {
+    return guard([&] {
+        const MoeCacheStats &s = static_cast<MoeExpertCache *>(cache)->stats();
+        out5[0] = s.hits; out5[1] = s.misses; out5[2] = s.evictions; out5[3] = s.bytes; out5[4] = s.launches;
     });
 }
 

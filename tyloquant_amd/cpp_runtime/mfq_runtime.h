@@ -234,6 +234,61 @@ void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &dow
                           const NintWeight *shared_down, MoeFfnScratch &scratch, float *out,
                           mfq_stream_t stream = nullptr);
 
+// ---- expert residency (MoeExpertCache, cpp_runtime/mfq_decode.cpp:5941-7500) ----------------------------------
+// Experts live in pinned host memory in their device layout; a GPU arena per cohort holds `slots` of them.
+// prepare() makes a set of experts resident: least recently used slots are reused, all missing bytes travel as one
+// staged host-to-device copy and one mfq_hip_cache_scatter launch, which also rewrites the dispatch-table words.
+struct MoeCacheStats {
+    int64_t hits = 0, misses = 0, evictions = 0, bytes = 0, launches = 0;
+};
+class MoeExpertCache;
+class MoeCachedSource {
+public:
+    int n_experts = 0, out_per_expert = 0, neuron_len = 0;
+    NintMoeWeight weight;  // view over the arenas; valid for the experts of the last prepare()
+private:
+    friend class MoeExpertCache;
+    struct Cohort {
+        mfq_nint_desc src{};
+        std::vector<int32_t> expert_ids;
+        void *host = nullptr;  // pinned copy of the cohort's device layout
+        size_t host_bytes = 0;
+        int64_t body_bytes = 0, slot_bytes = 0;
+        int minimum_slots = 1;
+        std::shared_ptr<NintWeight> arena;
+        std::unordered_map<int, int> slot_of;  // local expert -> slot
+        std::vector<int> lru, free_slots;
+    };
+    std::vector<Cohort> cohorts;
+    std::vector<int32_t> cohort_of, local_of;
+};
+class MoeExpertCache {
+public:
+    explicit MoeExpertCache(int64_t budget_bytes);
+    ~MoeExpertCache();
+    MoeExpertCache(const MoeExpertCache &) = delete;
+    MoeExpertCache &operator=(const MoeExpertCache &) = delete;
+    MoeCachedSource *register_source(const uint8_t *blob, size_t n, int minimum_slots = 1);
+    void finalize();
+    // experts: host array of ids (any order, duplicates and out-of-range ids allowed)
+    void prepare(MoeCachedSource &source, const int32_t *experts, size_t count, mfq_stream_t stream = nullptr);
+    // reads the route's ids back to the host, prepares, and runs the grouped matmul on the arenas
+    void forward(MoeCachedSource &source, const void *x, int x_dtype, int64_t ldx, bool routed_input,
+                 const MoeRoutePlan &route, float *out, mfq_stream_t stream = nullptr);
+    const MoeCacheStats &stats() const { return stats_; }
+    int64_t allocated_bytes() const { return allocated_bytes_; }
+    bool finalized() const { return finalized_; }
+
+private:
+    int64_t budget_bytes_, allocated_bytes_ = 0;
+    bool finalized_ = false;
+    std::vector<std::unique_ptr<MoeCachedSource>> sources_;
+    MoeCacheStats stats_;
+    void *stage_host_ = nullptr;
+    size_t stage_bytes_ = 0;
+    DeviceBuffer stage_dev_;
+};
+
 // ---- MFQ1 container + the --check-linear harness ----------------------------------------------------
 struct MfqRecord {
     std::string name, dtype;
