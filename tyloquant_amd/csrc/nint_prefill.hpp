@@ -19,24 +19,32 @@ constexpr int kMinSteps = 8;  // steps whose minimum-term operands a block stage
 // LDS bytes of a block of BM tile rows: nbuf activation buffers of [BM][4 * GS' + 8] halves (GS' = groupsize padded to 8),
 // reused for the group sums of kMinSteps steps ([BM][kMinSteps * 16 + 4] dwords).
 constexpr size_t prefill_lds_bytes(int bm, int gs, int nbuf = 2) {
-    const size_t xt = static_cast<size_t>(nbuf * bm) * (4 * ((gs + 7) / 8 * 8) + 8) * 2;
+    // a buffer of the ring of four (direct-to-LDS copies) is a whole number of wave-wide copies of 16-byte chunks
+    const size_t row = 4 * ((gs + 7) / 8 * 8) + 8;
+    const size_t buf = nbuf == 4 ? (bm * (row / 8) + 63) / 64 * 64 * 16 : bm * row * 2;
+    const size_t xt = nbuf * buf;
     const size_t mn = static_cast<size_t>(bm) * (kMinSteps * 16 + 4) * 4;
     return xt > mn ? xt : mn;
 }
 
 // Rows of a block tile: src(i) = row of x16 / xscale / xg that tile row i reads (always valid), dst(i) = row of y it
 // writes or -1.
+// win_row0() / win_rows(bm): rows of x16 that the direct-to-LDS copies of a tile of bm rows address through one
+// buffer window (a window spans less than 4 GiB).
 struct DenseRows {
-    static constexpr bool kAscending = true;  // src(i) >= src(0)
     int tok0, M;
     __device__ __forceinline__ int src(int i) const { return min(tok0 + i, M - 1); }
     __device__ __forceinline__ int dst(int i) const { return tok0 + i < M ? tok0 + i : -1; }
+    __device__ __forceinline__ int win_row0() const { return min(tok0, M - 1); }
+    __device__ __forceinline__ int64_t win_rows(int bm) const { return bm; }
 };
-struct MappedRows {  // both tables live in LDS
-    static constexpr bool kAscending = false;
+struct MappedRows {  // both tables live in LDS; any row of x16 may be a source: the window spans all n_src of them
     const int *srcv, *dstv;
+    int n_src;
     __device__ __forceinline__ int src(int i) const { return srcv[i]; }
     __device__ __forceinline__ int dst(int i) const { return dstv[i]; }
+    __device__ __forceinline__ int win_row0() const { return 0; }
+    __device__ __forceinline__ int64_t win_rows(int) const { return n_src; }
 };
 
 // One block: tile rows `rows`, neurons of the row-blocks [rb_base, rb_base + (NW / WM) * NB) below rb_end; y column of a
@@ -88,7 +96,11 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
     constexpr bool DMA = XD == 0;
     static_assert(XD == 0 || XD == 1 || XD == 2 || XD == 4, "activation tiles in flight in registers");
     static_assert(!DMA || (EL == 8 && GSP == GS), "direct-to-LDS tiles are made of 16-byte chunks");
-    static_assert(!DMA || Rows::kAscending, "the copies address the rows relative to the tile's first row");
+    // A tile whose chunks do not fill the last wave-wide copy is followed by slack for the rest of that copy (which
+    // repeats the tile's last chunk): TILE_CH counts the slack, BUF is the distance between two buffers in halves.
+    constexpr int CPR = ROW / 8, TILE_CH = DMA ? (BM * CPR + 63) / 64 * 64 : BM * CPR, DPER = DMA ? (TILE_CH + NT - 1) / NT : 1;
+    constexpr int LASTW = (TILE_CH - NT * (DPER - 1)) / 64;
+    constexpr int BUF = DMA ? TILE_CH * 8 : BM * ROW;
     constexpr int XR = DMA ? 1 : XD;
     chunk_t xr[XR][PER_THREAD];
     // the thread's chunks of a tile: source row (looked up once: a mapped tile keeps its row table in LDS) and k offset
@@ -119,29 +131,26 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
             const int row = c / CHUNKS, ch = c - row * CHUNKS;
             const int g = ch / CPG, ci = ch - g * CPG;
             if (c < BM * CHUNKS)
-                *reinterpret_cast<chunk_t *>(xt + buf * (BM * ROW) + row * ROW + g * GSP + EL * ci) = xq[p];
+                *reinterpret_cast<chunk_t *>(xt + buf * BUF + row * ROW + g * GSP + EL * ci) = xq[p];
         }
     };
     // direct-to-LDS copies: chunk c of a tile (16 bytes; row c / CPR, the last chunk of a row is padding and takes a
     // copy of the one before) lands at byte 16 c of its buffer -- lane l of a wave-wide copy writes 16 l bytes behind
     // the wave's base, so a thread's chunks are tid, tid + NT, ...  The last round has work for LASTW waves only; the
     // others repeat it (same bytes to the same place), so that every wave issues the same number of requests.
-    constexpr int CPR = ROW / 8, TILE_CH = BM * CPR, DPER = DMA ? (TILE_CH + NT - 1) / NT : 1;
-    constexpr int LASTW = (TILE_CH - NT * (DPER - 1)) / 64;
-    static_assert(!DMA || TILE_CH % 64 == 0, "whole waves of chunks");
     uint32_t dsrc[DPER];  // byte offset of the thread's chunk p inside x16 at k = 0
     int dbase[DPER];      // first chunk of the wave's copy p
     // buffer-addressed copies (the flat-addressed form makes the compiler wait for all outstanding requests at every
     // use of a loaded register); the tile rows of a block lie inside 4 GiB from xwin's base
     __amdgpu_buffer_rsrc_t xwin;
     if constexpr (DMA) {
-        const int row_lo = rows.src(0);
+        const int row_lo = rows.win_row0();
         xwin = wave_window(reinterpret_cast<const uint8_t *>(x16 + static_cast<int64_t>(row_lo) * Kp),
-                           static_cast<uint32_t>(min(static_cast<int64_t>(BM) * Kp * 2, static_cast<int64_t>(0xffffffffu))));
+                           static_cast<uint32_t>(min(rows.win_rows(BM) * Kp * 2, static_cast<int64_t>(0xffffffffu))));
 #pragma unroll
         for (int p = 0; p < DPER; ++p) {
             dbase[p] = NT * p + (p == DPER - 1 ? wave % LASTW : wave) * 64;
-            const int c = dbase[p] + lane;
+            const int c = min(dbase[p] + lane, BM * CPR - 1);  // the slack behind the tile takes copies of its last chunk
             const int row = c / CPR, cc = min(c - row * CPR, CPR - 2);
             dsrc[p] = static_cast<uint32_t>((static_cast<int64_t>(rows.src(row) - row_lo) * Kp + 8 * cc) * 2);
         }
@@ -153,7 +162,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
 #pragma unroll
             for (int p = 0; p < DPER; ++p) {
                 typedef __attribute__((address_space(3))) void *lds_ptr;
-                uint16_t *dst = xt + buf * (BM * ROW) + dbase[p] * 8;
+                uint16_t *dst = xt + buf * BUF + dbase[p] * 8;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(xwin, (lds_ptr)dst, 16, dsrc[p], k0 * 2, 0, 0);
             }
         }
@@ -235,7 +244,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
             u32x4_t af[MT];
 #pragma unroll
             for (int a = 0; a < MT; ++a)
-                af[a] = *reinterpret_cast<const u32x4_t *>(xt + (DMA ? (j & 3) : (j & 1)) * (BM * ROW) + ((wm * MT + a) * 16 + r) * ROW + kb * GSP + 8 * m);
+                af[a] = *reinterpret_cast<const u32x4_t *>(xt + (DMA ? (j & 3) : (j & 1)) * BUF + ((wm * MT + a) * 16 + r) * ROW + kb * GSP + 8 * m);
             // all weight fragments of this k-slice first, then the MFMAs back to back: while one wave's MFMAs run,
             // the other wave of the SIMD unpacks
             u32x4_t bf[NB];
