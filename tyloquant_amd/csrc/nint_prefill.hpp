@@ -205,13 +205,16 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
 #pragma unroll
     for (int i = 0; i < PF - 1; ++i) wload(4 * s_begin + i, qr[i]);
     sload(s_begin, tails, sc);
-    if constexpr (DMA) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    } else {
+    if constexpr (!DMA) {
         xstore(0, xr[0]);
 #pragma unroll
         for (int i = 1; i < XD; ++i) xload(4 * s_begin + i, xr[i]);
     }
+    // Every request of the prologue lands before the loop, through a wait the compiler sees (not inline assembly): the
+    // waits it places inside the loop then count only the requests of earlier sub-steps.  Entering the loop with requests
+    // in flight makes it keep, for all iterations, the short distances of the first one -- a wait for a weight unit
+    // requested a few instructions earlier, once per step.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
     for (int s = s_begin; s < s_end; ++s) {
 #pragma unroll
