@@ -348,8 +348,8 @@ int mfq_hip_moe_grouped_matmul(const mfq_moe_pool *pools, int n_pools, const int
                                const int32_t *tile_bounds, const int32_t *tile_experts,
                                float *out, int64_t ldo, mfq_stream_t stream);
 
-/* The same with a workspace, which lets mapped calls run the prefill kernel (64 pairs of an expert against
- * 512 neurons per block; activations pre-scaled to fp16 in the workspace).  x_rows = T * R with routed_input, else T.  The size query returns 0 when the cohorts have no
+/* The same with a workspace, which lets mapped calls run the prefill kernels (the pairs of an expert in chunks of up to
+ * 128 against 256 or 512 of its neurons per block; activations pre-scaled to fp16 in the workspace).  x_rows = T * R with routed_input, else T.  The size query returns 0 when the cohorts have no
  * prefill kernel; a NULL or short workspace simply keeps the streaming kernels.  No counterpart in the
  * reference, whose hetero kernels allocate their workspace through torch
  * (cpp_runtime/mfq_decode.cpp:3008-3016). */
@@ -362,6 +362,22 @@ int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_pools, const 
                                   const int32_t *tile_bounds, const int32_t *tile_experts,
                                   float *out, int64_t ldo, void *workspace, size_t workspace_bytes,
                                   mfq_stream_t stream);
+
+/* Gate/up projection of a mapped call with the GLU in the matmul's epilogue: pools hold [2 W] neurons per expert, gate
+ * rows first; hidden [T * R, ldh] (16-bit, out_dtype) receives act(gate) * up, act = MFQ_GLU_SILU or MFQ_GLU_GELU --
+ * the values of mfq_hip_moe_grouped_matmul_ws followed by mfq_hip_moe_glu (the same fp32 sums through the same
+ * activation), without the fp32 [T * R, 2 W] round trip.  Needs the route map and a workspace of mfq_hip_moe_grouped_workspace_bytes; MFQ_ERR_UNSUPPORTED when the
+ * call cannot take the prefill kernels (a cohort without a prefill body, K % 8, an unaligned x, a short workspace): run
+ * the two calls then.  Replaces NintMoeWeight::forward_glu_output / nint_moe_grouped_matmul_hetero_glu_qx_cuda
+ * (cpp_runtime/mfq_decode.cpp:3073-3127), which the reference limits to 1-4 tokens; mfq_hip_moe_decode_matmul with
+ * swiglu covers those. */
+int mfq_hip_moe_grouped_glu_ws(const mfq_moe_pool *pools, int n_pools, const int32_t *expert_pool,
+                               const int32_t *expert_local, int E, int out_per_expert, int K,
+                               const void *x, int x_dtype, int64_t ldx, int routed_input,
+                               const int32_t *ids, int T, int R,
+                               const int32_t *ids_dst, const int32_t *expert_bounds, int activation,
+                               void *hidden, int out_dtype, int64_t ldh, void *workspace,
+                               size_t workspace_bytes, mfq_stream_t stream);
 
 /* Decode form of the grouped matmul (no route map; a handful of tokens): one launch of the batch-1 GEMV over
  * rows p = t * R + r (pair p against expert ids[p]) and, when a shared tensor [out_per_expert, K] is given, rows

@@ -299,3 +299,43 @@ def test_expert_cache_keeps_a_working_set_resident():
     assert st["bytes"] == before["bytes"] and st["launches"] == before["launches"]
     with pytest.raises(RuntimeError, match="its arena holds 3"):
         cache.prepare(src, [0, 2, 4, 6])
+
+
+@pytest.mark.parametrize("routed", [False, True])
+@pytest.mark.parametrize("activation,out_dtype", [(0, torch.float16), (1, torch.bfloat16)])
+def test_grouped_glu_epilogue_matches_the_two_calls(routed, activation, out_dtype):
+    """forward_glu (GLU in the epilogue of the mapped prefill kernels) against forward + moe_glu: the same 16-bit values
+    but for a last-place flip where the fp32 product sits on a rounding boundary (at most 1 in 1000 values, one unit);
+    experts with 0, 1, 15, 30, 45, 60, 70, 90 and 150 pairs (every tile count of the three kernel groups), an invalid id
+    (zero row), W = 80 neurons (a partial neuron tile) and ragged K; and against the oracle's loop."""
+    from tyloquant_amd.runtime_moe import build_moe_route_plan, moe_glu
+    rng = np.random.default_rng(91)
+    counts = [0, 1, 15, 30, 45, 60, 70, 90, 150, 33]
+    E, W, K, R = len(counts), 80, 776, 2
+    t, w = _moe(rng, E, 2 * W, K, [4, 3, 2, 5, 4, 3, 2, 5, 4, 3])
+    flat = np.concatenate([np.full(c, e, dtype=np.int32) for e, c in enumerate(counts)])
+    if len(flat) % R:
+        flat = np.concatenate([flat, np.array([9], dtype=np.int32)])
+    rng.shuffle(flat)
+    ids = flat.reshape(-1, R)
+    ids[3, 1] = 77                      # out of range: a zero row
+    T = ids.shape[0]
+    shape = (T, R, K) if routed else (T, K)
+    x = torch.from_numpy((rng.standard_normal(shape) * 0.1).astype(np.float32)).to(torch.bfloat16).cuda()
+    route = build_moe_route_plan(torch.from_numpy(ids).cuda(), E)
+    assert route.ids_dst is not None
+    fused = w.forward_glu(x, route, activation, out_dtype)
+    two = moe_glu(w(x, route), out_dtype, activation)
+    assert fused.shape == (T, R, W) and fused.dtype == out_dtype
+    ulp = (fused.view(torch.int16).int() - two.view(torch.int16).int()).abs()
+    assert int(ulp.max()) <= 1 and float((ulp != 0).float().mean()) < 1e-3
+    assert torch.all(fused[3, 1] == 0)
+    dense = O.dequantize_expertwise(t)
+    gu = O.moe_grouped_matmul(dense, x.float().cpu().numpy(), ids)
+    g, u = gu[..., :W], gu[..., W:]
+    if activation == 0:
+        ref = g / (1.0 + np.exp(-g)) * u
+    else:
+        ref = 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3))) * u
+    got = fused.float().cpu().numpy()
+    assert rel_l2(got, ref) < 5e-3 and np.abs(got - ref).max() < ABS_TOL

@@ -14,6 +14,7 @@ LIB_PATH = _HERE / "lib" / "libmfq_hip.so"
 X_BF16, X_F16, X_F32 = 0, 1, 2
 TOPK_SOFTMAX, TOPK_SIGMOID, TOPK_SQRT_SOFTPLUS, TOPK_DELAYED_SOFTMAX = 0, 1, 2, 3
 GLU_SILU, GLU_GELU = 0, 1
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_LAUNCH, ERR_WORKSPACE = 0, 1, 2, 3, 4
 
 i32, i64, vp, sz = C.c_int32, C.c_int64, C.c_void_p, C.c_size_t
 
@@ -104,6 +105,9 @@ _SIGS = {
                                              C.c_int, i64, C.c_int, vp, C.c_int, C.c_int, vp, vp, vp, vp, vp, i64,
                                              vp]),
     "mfq_hip_moe_grouped_workspace_bytes": (sz, [C.POINTER(MoePool), C.c_int, C.c_int, C.c_int]),
+    "mfq_hip_moe_grouped_glu_ws": (C.c_int, [C.POINTER(MoePool), C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, vp,
+                                             C.c_int, i64, C.c_int, vp, C.c_int, C.c_int, vp, vp, C.c_int, vp, C.c_int,
+                                             i64, vp, sz, vp]),
     "mfq_hip_moe_grouped_matmul_ws": (C.c_int, [C.POINTER(MoePool), C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, vp,
                                                 C.c_int, i64, C.c_int, vp, C.c_int, C.c_int, vp, vp, vp, vp, vp, i64,
                                                 vp, sz, vp]),

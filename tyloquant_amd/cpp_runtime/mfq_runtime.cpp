@@ -560,6 +560,30 @@ void NintMoeWeight::forward(const void *x, int x_dtype, int64_t ldx, bool routed
         need ? workspace.get() : nullptr, need, stream));
 }
 
+void NintMoeWeight::forward_glu(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &r, bool gelu,
+                                void *hidden, float *scratch, mfq_stream_t stream) const {
+    const int W = out_per_expert / 2, pairs = r.tokens * r.routes;
+    const int activation = gelu ? MFQ_GLU_GELU : MFQ_GLU_SILU;
+    if (r.mapped() && out_per_expert % 32 == 0) {
+        const int x_rows = routed_input ? pairs : r.tokens;
+        const size_t need =
+            mfq_hip_moe_grouped_workspace_bytes(pool_table.data(), static_cast<int>(pool_table.size()), neuron_len, x_rows);
+        if (need) {
+            workspace.ensure(need);
+            const int rc = mfq_hip_moe_grouped_glu_ws(
+                pool_table.data(), static_cast<int>(pool_table.size()), static_cast<const int32_t *>(expert_pool.get()),
+                static_cast<const int32_t *>(expert_local.get()), n_experts, out_per_expert, neuron_len, x, x_dtype, ldx,
+                routed_input ? 1 : 0, r.ids, r.tokens, r.routes, static_cast<const int32_t *>(r.ids_dst.get()),
+                static_cast<const int32_t *>(r.expert_bounds.get()), activation, hidden, MFQ_X_F16, W, workspace.get(), need,
+                stream);
+            if (rc == MFQ_OK) return;
+            if (rc != MFQ_ERR_UNSUPPORTED) abi_check(rc);
+        }
+    }
+    forward(x, x_dtype, ldx, routed_input, r, scratch, stream);
+    abi_check(mfq_hip_moe_glu(scratch, out_per_expert, pairs, W, hidden, MFQ_X_F16, W, activation, stream));
+}
+
 bool NintMoeWeight::decode_capable(const NintWeight *shared, int tokens, int routes, bool swiglu) const {
     if (shared && shared->desc.neuron_len != neuron_len) return false;
     return mfq_hip_moe_decode_capable(pool_table.data(), static_cast<int>(pool_table.size()), out_per_expert, neuron_len,
@@ -608,8 +632,7 @@ void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &dow
     MoeRoutePlan route = build_moe_route_plan(ids, T, top_k, E, stream);
     s.gate_up.ensure(4 * pairs * 2 * W); s.hidden.ensure(2 * pairs * W); s.down.ensure(4 * pairs * H);
     float *gu = static_cast<float *>(s.gate_up.get());
-    gate_up.forward(x, x_dtype, ldx, false, route, gu, stream);
-    abi_check(mfq_hip_moe_swiglu(gu, 2 * W, static_cast<int>(pairs), W, s.hidden.get(), MFQ_X_F16, W, stream));
+    gate_up.forward_glu(x, x_dtype, ldx, false, route, false, s.hidden.get(), gu, stream);
     float *dn = static_cast<float *>(s.down.get());
     down.forward(s.hidden.get(), MFQ_X_F16, W, true, route, dn, stream);
     const float *shared = nullptr;

@@ -216,6 +216,11 @@ struct NintMoeWeight {
     // x: [T, K] (routed_input = false) or [T*R, K]; out: fp32 [T*R, out_per_expert]
     void forward(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &route, float *out,
                  mfq_stream_t stream = nullptr) const;
+    // act(gate) * up of a gate/up tensor as fp16 [T*R, out_per_expert / 2] (NintMoeWeight::forward_glu_output,
+    // cpp_runtime/mfq_decode.cpp:3073-3127): the GLU runs in the epilogue of the mapped prefill kernels; where the library
+    // declines, forward() into `scratch` (fp32 [T*R, out_per_expert]) and mfq_hip_moe_glu.
+    void forward_glu(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &route, bool gelu,
+                     void *hidden, float *scratch, mfq_stream_t stream = nullptr) const;
     // Decode step in one launch (mfq_hip_moe_decode_matmul): rows t * R + r are the routed pairs, rows T * R + t the
     // `shared` tensor (may be null) on token t.  swiglu: out is fp16 [rows, out_per_expert / 2], else fp32
     // [rows, out_per_expert].  decode_capable() tells whether the cohorts and the shared tensor fit that kernel.

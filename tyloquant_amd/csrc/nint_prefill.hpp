@@ -54,12 +54,20 @@ struct MappedRows {  // both tables live in LDS; any row of x16 may be a source:
 // Kp >= 64 * GS * steps).  PF: register buffers of weight units per row-block; the unit of sub-step it + PF - 1 is requested while sub-step it
 // multiplies (2 = ping-pong; 4 keeps a whole step in flight for tiles with few rows, where the weight stream and
 // not the matrix cores sets the pace).
-template <class U, int MT, int NB, int WM, int NW, class Rows, int PF = 2, int XD = (PF == 4 ? 4 : 1)>
+// GLU: the wave's NB row-blocks are NB / 2 gate row-blocks from rb_base on and the NB / 2 row-blocks glu.rb_stride further
+// (up); rb_end bounds the gate row-blocks; instead of the two fp32 results the block stores act(gate) * up in 16 bits
+// (y is then uint16_t [rows, ldy], column = the gate neuron's).
+struct GluOut {
+    int rb_stride;  // row-blocks from a gate row-block to its up row-block
+    int gelu;       // 0: SiLU, 1: tanh form of GELU
+    int f16;        // output halves are fp16 (else bf16)
+};
+template <class U, int MT, int NB, int WM, int NW, class Rows, int PF = 2, int XD = (PF == 4 ? 4 : 1), bool GLU = false>
 __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t *__restrict__ w, int rb_base, int rb_end,
                                                   int rb_col0, int ncols, const uint16_t *__restrict__ x16, int Kp,
                                                   const float *__restrict__ xscale, const uint32_t *__restrict__ xg,
                                                   const Rows &rows, float *__restrict__ y, int64_t ldy, uint16_t *xt,
-                                                  int s_begin = 0, int s_end = -1) {
+                                                  int s_begin = 0, int s_end = -1, GluOut glu = GluOut{0, 0, 0}) {
     if (s_end < 0) s_end = k.nsteps;  // steps [s_begin, s_end) of K: a block of a split over K leaves a partial sum
     constexpr int D = U::D, GS = U::GROUP, NM = U::NPAIR / 4, BITS = U::CBITS;
     constexpr int NCLS = BITS == 0 ? 1 : (BITS == 3 ? 3 : 2);
@@ -78,11 +86,16 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WM, wn = wave / WM;
     const int r = lane & 15, kb = lane >> 4;
-    const int rb0 = rb_base + wn * NB;
-    const int nrb = max(0, min(NB, rb_end - rb0));
+    static_assert(!GLU || NB % 2 == 0, "gate and up row-blocks come in pairs");
+    constexpr int NBG = GLU ? NB / 2 : NB;  // row-blocks from rb0 on; with GLU the other half lies glu.rb_stride further
+    const int rb0 = rb_base + wn * NBG;
+    const int nrb = max(0, min(NBG, rb_end - rb0));
+    auto rbo = [&](int b) { return GLU ? (b % NBG) + (b / NBG) * glu.rb_stride : b; };  // row-block of b, relative to rb0
+    auto live = [&](int b) { return (b % NBG) < nrb; };
     const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
     const __amdgpu_buffer_rsrc_t win =
-        wave_window(w + static_cast<int64_t>(min(rb0, k.n_rowblocks - 1)) * k.rowblock_bytes, nrb * rbb);
+        wave_window(w + static_cast<int64_t>(min(rb0, k.n_rowblocks - 1)) * k.rowblock_bytes,
+                    nrb > 0 ? (rbo(NB - NBG) + nrb) * rbb : 0u);
 
     float4_t acc[MT][NB];
 #pragma unroll
@@ -184,12 +197,12 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
         const int s = it >> 2, j = it & 3;
 #pragma unroll
         for (int b = 0; b < NB; ++b)
-            load_unit_win<D, 0>(win, b < nrb && s < s_end ? b * rbb + s * sb + (j * 64 + lane) * (D * 4) : kNoStep, qq[b]);
+            load_unit_win<D, 0>(win, live(b) && s < s_end ? rbo(b) * rbb + s * sb + (j * 64 + lane) * (D * 4) : kNoStep, qq[b]);
     };
     auto sload = [&](int s, uint32_t (&tt)[NB], u32x2_t (&ss)[NB]) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            const uint32_t off = b < nrb && s < s_end ? b * rbb + s * sb + 1024 * D : kNoStep;
+            const uint32_t off = live(b) && s < s_end ? rbo(b) * rbb + s * sb + 1024 * D : kNoStep;
             tt[b] = 0;
             if constexpr (U::TAIL) tt[b] = __builtin_amdgcn_raw_buffer_load_b32(win, off + lane * 4, 0, 0);
             ss[b] = __builtin_amdgcn_raw_buffer_load_b64(win, off + (U::TAIL ? 256 : 0) + lane * 8, 0, 0);
@@ -301,7 +314,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
     float ns[NB], nm[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-        const int rb = min(rb0 + b, k.n_rowblocks - 1);
+        const int rb = min(rb0 + rbo(b), k.n_rowblocks - 1);
         ns[b] = anchors[rb * 16 + r] * 64.f;
         nm[b] = anchors[16 * k.n_rowblocks + rb * 16 + r];
     }
@@ -332,7 +345,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const int s = c0 + t;
-                const uint32_t off = b < nrb && s < s_end ? b * rbb + s * sb + 1024 * D + (U::TAIL ? 256 : 0) : kNoStep;
+                const uint32_t off = live(b) && s < s_end ? rbo(b) * rbb + s * sb + 1024 * D + (U::TAIL ? 256 : 0) : kNoStep;
                 scs[t][b] = __builtin_amdgcn_raw_buffer_load_b64(win, off + lane * 8, 0, 0);
             }
 #pragma unroll
@@ -368,11 +381,24 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
             const int m = rows.dst(ti);
             if (m < 0) continue;
             const float xs = xscale[rows.src(ti)];
+            if constexpr (GLU) {
+                uint16_t *h = reinterpret_cast<uint16_t *>(y);
 #pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                const int col = (rb0 + b - rb_col0) * 16 + r;
-                if (rb0 + b < rb_end && col < ncols)
-                    y[static_cast<int64_t>(m) * ldy + col] = xs * (ns[b] * acc[a][b][v] - nm[b] * accM[a][b][v]);
+                for (int b = 0; b < NBG; ++b) {
+                    const int col = (rb0 + b - rb_col0) * 16 + r;
+                    const float g = xs * (ns[b] * acc[a][b][v] - nm[b] * accM[a][b][v]);
+                    const float u = xs * (ns[b + NBG] * acc[a][b + NBG][v] - nm[b + NBG] * accM[a][b + NBG][v]);
+                    const float hv = glu_value(g, u, glu.gelu != 0);
+                    if (rb0 + b < rb_end && col < ncols)
+                        h[static_cast<int64_t>(m) * ldy + col] = glu.f16 ? f32_to_f16_rne(hv) : f32_to_bf16_rne(hv);
+                }
+            } else {
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    const int col = (rb0 + b - rb_col0) * 16 + r;
+                    if (rb0 + b < rb_end && col < ncols)
+                        y[static_cast<int64_t>(m) * ldy + col] = xs * (ns[b] * acc[a][b][v] - nm[b] * accM[a][b][v]);
+                }
             }
         }
     }

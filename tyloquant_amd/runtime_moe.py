@@ -174,6 +174,39 @@ class NintMoeWeight:
 
     __call__ = forward
 
+    def forward_glu(self, x: torch.Tensor, route: MoeRoutePlan, activation: int = L.GLU_SILU,
+                    out_dtype=torch.float16) -> torch.Tensor:
+        """act(gate) * up of the routed gate/up projection as 16-bit [T, R, out_per_expert / 2]
+        (NintMoeWeight::forward_glu_output, cpp_runtime/mfq_decode.cpp:3073-3127): one pass of the mapped prefill
+        kernels with the GLU in their epilogue; the two-call form (forward, then moe_glu) where the library
+        declines -- no route map, a cohort without a prefill body, unaligned activations."""
+        T, R = route.tokens, route.routes
+        routed = x.dim() == 3
+        if x.shape[-1] != self.neuron_len or x.shape[0] != T or (routed and x.shape[1] != R):
+            raise ValueError("MoE activations must be [tokens, K] or [tokens, routes, K]")
+        if self.out_per_expert % 2:
+            raise RuntimeError("fused gate/up GLU needs an even number of neurons per expert")
+        W = self.out_per_expert // 2
+        if route.ids_dst is not None and self.out_per_expert % 32 == 0:
+            x2 = x.reshape(-1, self.neuron_len)
+            if x2.stride(-1) != 1:
+                x2 = x2.contiguous()
+            lib = L.lib()
+            need = lib.mfq_hip_moe_grouped_workspace_bytes(self._pool_array, len(self.pools), self.neuron_len, x2.shape[0])
+            if need:
+                ws = self._ws.get(need, x.device)
+                hidden = torch.empty((T, R, W), dtype=out_dtype, device=x.device)
+                rc = lib.mfq_hip_moe_grouped_glu_ws(
+                    self._pool_array, len(self.pools), _ptr(self.expert_pool), _ptr(self.expert_local), self.n_experts,
+                    self.out_per_expert, self.neuron_len, _ptr(x2), _x_dtype(x2), x2.stride(0), int(routed),
+                    _ptr(route.ids), T, R, _ptr(route.ids_dst), _ptr(route.expert_bounds), int(activation), _ptr(hidden),
+                    L.X_F16 if out_dtype == torch.float16 else L.X_BF16, W, _ptr(ws), need, _stream())
+                if rc == 0:
+                    return hidden
+                if rc != L.ERR_UNSUPPORTED:
+                    L.check(rc)
+        return moe_glu(self.forward(x, route), out_dtype, activation)
+
     def decode_capable(self, shared: NintWeight | None = None, tokens: int = 1, routes: int = 1, swiglu=False) -> bool:
         """Whether forward_decode takes these cohorts, this shared tensor and this many (token, route) pairs: the
         library's own answer (unit per cohort, shared tensor's shape, the block's LDS need, the row count)."""
@@ -259,8 +292,7 @@ def nint_moe_ffn_forward(gate_up: NintMoeWeight, down: NintMoeWeight, x: torch.T
         dn = down.forward_decode(hidden, ids, sdn, routed=True)
         pair = dn[: T * R].reshape(T, R, -1)
         return moe_weighted_reduce(pair, w, dn[T * R:] if shared is not None else None), ids, w
-    gu = gate_up.forward(x, route)
-    hidden = moe_swiglu(gu)
+    hidden = gate_up.forward_glu(x, route)
     dn = down.forward(hidden, route)
     sh = None
     if shared is not None:
