@@ -139,10 +139,20 @@ int mfq_hip_nint_embedding(const mfq_nint_desc *d, const void *weight, const int
  * function (mode 1), the numbering of nint_matmul_input_mul (cpp_runtime/mfq_decode.cpp:8395-8417); x, gate and out
  * are bf16 or fp16 (x_dtype) [M, K] with row strides ldx / ldg / ldo, the product is formed in fp32 and rounded once.
  * Followed by mfq_hip_nint_gemv / mfq_hip_nint_gemm on `out` it replaces nint_gemv_packed_gate_ws_cuda /
- * nint_gemv_packed_bits_gate_ws_cuda (:389-392, :488-491) and the reference's own unfused form
- * nint_matmul(w, x * silu(gate)) (:8415-8416); the gate is not fused into the GEMV here. */
+ * nint_gemv_packed_bits_gate_ws_cuda (:389-392, :488-491) for the batches mfq_hip_nint_gemv_gate leaves out, and is
+ * the reference's own unfused form nint_matmul(w, x * silu(gate)) (:8415-8416). */
 int mfq_hip_input_gate(const void *x, const void *gate, int x_dtype, int64_t ldx, int64_t ldg, int M, int K,
                        int mode, void *out, int64_t ldo, mfq_stream_t stream);
+
+/* y[m, :] = (x[m, :] * act(gate[m, :])) . W^T in one launch for M = 1 or 2: the batch-1 GEMV whose waves fetch their
+ * slice of the gate row next to the activations and stage the product (fp32, rounded once to x_dtype as
+ * mfq_hip_input_gate rounds it).  mode as above.  MFQ_ERR_UNSUPPORTED for M > 2, rows that are not 16-byte aligned,
+ * neuron_len % 8 != 0 or neurons too long for one block: run mfq_hip_input_gate + mfq_hip_nint_gemm then.  Replaces
+ * nint_gemv_packed_gate_ws_cuda / nint_gemv_packed_bits_gate_ws_cuda (cpp_runtime/mfq_decode.cpp:389-392, 488-491,
+ * called at :8404-8413). */
+int mfq_hip_nint_gemv_gate(const mfq_nint_desc *d, const void *weight, const void *x, const void *gate,
+                           int x_dtype, int64_t ldx, int64_t ldg, int M, int mode, float *y, int64_t ldy,
+                           mfq_stream_t stream);
 
 /* LM head for greedy decoding: token[m] = argmax_n y[m, n] with y as in mfq_hip_nint_gemv (equal logits go to the
  * lower index, NaN never wins, -1 when every logit is NaN).  M = 1 on NINT4-32, NINT4-24, NINT3-24 and NINT5-28

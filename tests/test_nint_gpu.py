@@ -1,4 +1,6 @@
 """GPU parity of the NINT path against the oracle (through the C ABI)."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -213,6 +215,46 @@ def test_input_gate_then_matmul(mode, K):
             y = R.nint_matmul_input_mul(lin.weight, x, g, mode).cpu().numpy()
             ref = O.linear_forward_f64(deq, got.astype(np.float32))
             assert rel_l2(y, ref) < REL_TOL and np.abs(y - ref).max() < ABS_TOL
+
+
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (6, 20, 6)])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_input_gate_inside_the_gemv(bits, gs, sb, mode):
+    """One or two rows: the gate is applied by the GEMV's own activation staging (mfq_hip_nint_gemv_gate).  Against the
+    oracle on the once-rounded gated rows, and against the two-launch form (same rounding of the gated rows: the results
+    differ by fp32 summation order at most); three rows and misaligned rows take the two launches."""
+    from tyloquant_amd import _lib as L
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(4900 + 16 * bits + gs + mode)
+    for out, K in ((80, 2048), (48, 4096), (33, 840)):
+        t = O.quantize_nint((rng.standard_normal((out, K)) * 0.02).astype(np.float32), bits, gs, sb)
+        lin = _load(t)
+        deq = O.dequantize_nint(t)
+        for M in (1, 2):
+            for dtype in (torch.bfloat16, torch.float16):
+                x, xf = _x(rng, M, K, dtype)
+                g, gf = _x(rng, M, K, dtype)
+                y = torch.empty((M, out), dtype=torch.float32, device="cuda")
+                rc = L.lib().mfq_hip_nint_gemv_gate(C.byref(lin.weight.desc), lin.weight.data.data_ptr(), x.data_ptr(),
+                                                    g.data_ptr(), R._x_dtype(x), x.stride(0), g.stride(0), M, mode,
+                                                    y.data_ptr(), y.stride(0), None)
+                assert rc == 0, L.lib().mfq_hip_last_error()
+                two = R.nint_matmul_input_mul(lin.weight, x, g, mode, fused=False)
+                assert torch.allclose(y, two, rtol=1e-3, atol=1e-4)
+                one = R.nint_matmul_input_mul(lin.weight, x, g, mode)
+                assert torch.equal(one, y)
+                gated = torch.from_numpy(O.input_mul(xf, gf, mode).astype(np.float32)).to(dtype).float().numpy()
+                ref = O.linear_forward_f64(deq, gated)
+                yn = y.cpu().numpy()
+                assert rel_l2(yn, ref) < REL_TOL and np.abs(yn - ref).max() < ABS_TOL
+    # declined: three rows, a misaligned row
+    x, _ = _x(rng, 3, K, torch.bfloat16)
+    y = torch.empty((3, out), dtype=torch.float32, device="cuda")
+    args = (C.byref(lin.weight.desc), lin.weight.data.data_ptr())
+    assert L.lib().mfq_hip_nint_gemv_gate(*args, x.data_ptr(), x.data_ptr(), L.X_BF16, K, K, 3, 0, y.data_ptr(), out,
+                                          None) == L.ERR_UNSUPPORTED
+    assert L.lib().mfq_hip_nint_gemv_gate(*args, x.data_ptr() + 2, x.data_ptr(), L.X_BF16, K, K, 1, 0, y.data_ptr(), out,
+                                          None) == L.ERR_UNSUPPORTED
 
 
 @pytest.mark.parametrize("out,K", [(37, 96), (130, 1056), (64, 4096), (9000, 64)])

@@ -338,8 +338,13 @@ void nint_matmul_geglu(const NintWeight &w, const void *x, int x_dtype, int64_t 
 }
 void nint_matmul_input_mul(const NintWeight &w, const void *x, const void *gate, int x_dtype, int64_t ldx, int64_t ldg, int M,
                            int mode, void *gated, float *y, mfq_stream_t stream) {
-    if (!gated) fail("nint_matmul_input_mul: needs a [M, K] 16-bit buffer for the gated activations");
     const int K = w.desc.neuron_len;
+    if (M <= 2) {  // the GEMV gates its own activation slices
+        const int rc = mfq_hip_nint_gemv_gate(&w.desc, w.data.get(), x, gate, x_dtype, ldx, ldg, M, mode, y, w.desc.out, stream);
+        if (rc == MFQ_OK) return;
+        if (rc != MFQ_ERR_UNSUPPORTED) abi_check(rc);
+    }
+    if (!gated) fail("nint_matmul_input_mul: needs a [M, K] 16-bit buffer for the gated activations");
     abi_check(mfq_hip_input_gate(x, gate, x_dtype, ldx, ldg, M, K, mode, gated, K, stream));
     nint_matmul(w, gated, x_dtype, K, M, y, stream);
 }

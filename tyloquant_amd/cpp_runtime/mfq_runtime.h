@@ -136,8 +136,9 @@ void nint_matmul(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, i
 // rows (nint_gemv_packed_swiglu_ws_cuda :393-396), else nint_matmul into `scratch` (fp32 [M, 2W]) + the SwiGLU kernel
 void nint_matmul_swiglu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden,
                         float *scratch = nullptr, mfq_stream_t stream = nullptr);
-// y = (x * silu(gate)) . W^T (mode 0) or (x * sigmoid(gate)) . W^T (mode 1) (nint_matmul_input_mul :8395-8417): the gated
-// rows are formed in `gated` (device, 16-bit [M, K] of the type of x) by one elementwise launch, then nint_matmul
+// y = (x * silu(gate)) . W^T (mode 0) or (x * sigmoid(gate)) . W^T (mode 1) (nint_matmul_input_mul :8395-8417): one or
+// two rows in one GEMV launch that gates its activation slices; else the gated rows are formed in `gated` (device,
+// 16-bit [M, K] of the type of x; may be null for M <= 2 rows the fused launch takes) by one elementwise launch, then nint_matmul
 void nint_matmul_input_mul(const NintWeight &w, const void *x, const void *gate, int x_dtype, int64_t ldx, int64_t ldg, int M,
                            int mode, void *gated, float *y, mfq_stream_t stream = nullptr);
 // the same with gelu_tanh(gate) * up (nint_matmul_geglu :8462-8485)

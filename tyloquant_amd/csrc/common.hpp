@@ -103,4 +103,15 @@ __device__ __forceinline__ uint32_t read_bits(const uint8_t *s, int64_t idx, int
     return (v >> (bit & 7)) & ((1u << bits) - 1u);
 }
 
+// Input gate of a projection: x * act(gate), act = SiLU (mode 0) or the logistic function (mode 1), formed in fp32
+// and rounded once to the 16-bit type of x (F16: fp16, else bf16).
+template <int F16>
+__device__ __forceinline__ uint16_t input_gate_value(uint16_t xv, uint16_t gv, int mode) {
+    const float g = F16 ? f16_to_f32(gv) : __uint_as_float(static_cast<uint32_t>(gv) << 16);
+    const float x = F16 ? f16_to_f32(xv) : __uint_as_float(static_cast<uint32_t>(xv) << 16);
+    const float s = 1.f / (1.f + expf(-g));
+    const float v = x * (mode == 1 ? s : g * s);
+    return F16 ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
+}
+
 }  // namespace mfq

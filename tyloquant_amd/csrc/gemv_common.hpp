@@ -153,6 +153,52 @@ __device__ __forceinline__ void stage_x_issue(const uint16_t *const (&xr)[MB], i
     }
 }
 
+// Hook between the request of the activation slice and its staging: nothing (the plain GEMV) ...
+struct NoXPre {
+    template <int MB>
+    __device__ __forceinline__ void issue(int, int, int, int) {}
+    template <int XF16, int MB>
+    __device__ __forceinline__ void finish(XRegs<MB> &) {}
+};
+// ... or the input gate of a projection: the rows' gate slices are requested right after the activations (same
+// chunks, so the weight requests that follow still wait for nothing) and x * act(gate) replaces the activations in
+// their registers -- input_gate_value, the rounding of the separate elementwise launch -- before they are staged.
+// Needs the prefetched case of stage_x_issue (the launch checks it): MB <= 2, aligned rows, K % 8 == 0.
+template <int MB>
+struct InputGate {
+    const uint16_t *gr[MB];
+    int mode;
+    u32x4_t g[MB][kXChunks];
+    template <int MBX>
+    __device__ __forceinline__ void issue(int K, int k0, int npairs, int lane) {
+        static_assert(MBX == MB, "one gate row per activation row");
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            const __amdgpu_buffer_rsrc_t wg =
+                wave_window(reinterpret_cast<const uint8_t *>(gr[m]), gr[m] ? static_cast<uint32_t>(K) * 2u : 0u);
+#pragma unroll
+            for (int c = 0; c < kXChunks; ++c) {
+                const int i = lane * 4 + c * 256;
+                const bool in = i < npairs && k0 + 2 * i + 8 <= K;
+                g[m][c] = __builtin_amdgcn_raw_buffer_load_b128(wg, in ? static_cast<uint32_t>(k0 + 2 * i) * 2u : kNoStep, 0, 0);
+            }
+        }
+    }
+    template <int XF16, int MBX>
+    __device__ __forceinline__ void finish(XRegs<MB> &xg) {
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+#pragma unroll
+            for (int c = 0; c < kXChunks; ++c)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const uint32_t xv = xg.v[m][c][t], gv = g[m][c][t];
+                    xg.v[m][c][t] = input_gate_value<XF16>(xv & 0xffffu, gv & 0xffffu, mode) |
+                                    (static_cast<uint32_t>(input_gate_value<XF16>(xv >> 16, gv >> 16, mode)) << 16);
+                }
+    }
+};
+
 // Largest bf16 magnitudes (bit patterns without the sign) seen so far in the low and the high halves, kept as a packed
 // pair of 16-bit maxima: one AND and one packed max per dword.
 typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));

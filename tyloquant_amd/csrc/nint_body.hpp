@@ -340,10 +340,11 @@ __device__ long long *mfq_trace_ptr;
 #define MFQ_TRACE_FLUSH do { } while (0)
 #endif
 
-template <class U, int XF16, int MB, bool RING = true, bool FLUSH = true>
+template <class U, int XF16, int MB, bool RING = true, bool FLUSH = true, class XP = NoXPre>
 __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__restrict__ w, int rb0, int rbw,
                                                int row_base, int out_rows, const uint16_t *const (&xr)[MB],
-                                               float *const (&yr)[MB], int spw, uint32_t *lds, int rb_step = 1) {
+                                               float *const (&yr)[MB], int spw, uint32_t *lds, int rb_step = 1,
+                                               XP xp = XP()) {
     constexpr int D = U::D, GS = U::GROUP;
     const int lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
@@ -361,6 +362,7 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     MFQ_TRACE(0);
     XRegs<MB> xg;
     stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * GS, npairs, lane, xg);
+    xp.template issue<MB>(k.neuron_len, s0 * 16 * GS, npairs, lane);
     const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
     float ns[kMaxRbw], nm[kMaxRbw];
 #pragma unroll
@@ -387,6 +389,7 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     MFQ_ISSUE(q1, t1, c1)
     MFQ_ISSUE(q2, t2, c2)
     float xinv[MB];  // bf16 rows are staged times a per-wave power of two; the sums are scaled back when they are parked
+    xp.template finish<XF16, MB>(xg);
     stage_x<XF16, MB, typename U::Bias, true>(xr, k.neuron_len, s0 * 16 * GS, npairs, GS, ngl, xs, xsum, lane, xg, xinv);
 
     MFQ_TRACE(1);
@@ -454,10 +457,10 @@ __device__ __forceinline__ void nint_paired_body(const NintK &k, const uint8_t *
 }
 
 // Any (bits, gs): natural-order units, one code at a time in fp32.
-template <int XF16, int MB>
+template <int XF16, int MB, class XP = NoXPre>
 __device__ __forceinline__ void nint_generic_body(const NintK &k, const uint8_t *__restrict__ w, int rb, int row_base,
                                                   int out_rows, const uint16_t *const (&xr)[MB], float *const (&yr)[MB],
-                                                  int spw, uint32_t *lds) {
+                                                  int spw, uint32_t *lds, XP xp = XP()) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const int s0 = wave * spw;
     const int s1 = min(k.nsteps, s0 + spw);
@@ -467,7 +470,9 @@ __device__ __forceinline__ void nint_generic_body(const NintK &k, const uint8_t 
     float *red = reinterpret_cast<float *>(lds + nwaves * (MB * (npairs + 2 * ngl)));
     XRegs<MB> xg;
     stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * gs, npairs, lane, xg);
+    xp.template issue<MB>(k.neuron_len, s0 * 16 * gs, npairs, lane);
     float xinv[MB];
+    xp.template finish<XF16, MB>(xg);
     stage_x<XF16, MB, PlainBias, true>(xr, k.neuron_len, s0 * 16 * gs, npairs, gs, ngl, xs, xsum, lane, xg, xinv);
     const uint16_t *xh = reinterpret_cast<const uint16_t *>(xs);
 

@@ -180,13 +180,7 @@ __global__ __launch_bounds__(256) void input_gate_kernel(const uint16_t *__restr
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= static_cast<int64_t>(M) * per_row) return;
     const int m = static_cast<int>(idx / per_row), k0 = static_cast<int>(idx - static_cast<int64_t>(m) * per_row) * VEC;
-    auto to_f32 = [](uint16_t h) { return F16 ? f16_to_f32(h) : __uint_as_float(static_cast<uint32_t>(h) << 16); };
-    auto one = [&](uint16_t xv, uint16_t gv) -> uint16_t {
-        const float g = to_f32(gv);
-        const float s = 1.f / (1.f + expf(-g));
-        const float v = to_f32(xv) * (mode == 1 ? s : g * s);
-        return F16 ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
-    };
+    auto one = [&](uint16_t xv, uint16_t gv) -> uint16_t { return input_gate_value<F16>(xv, gv, mode); };
     if constexpr (VEC == 8) {
         const u32x4_t xv = *reinterpret_cast<const u32x4_t *>(x + m * ldx + k0);
         const u32x4_t gv = *reinterpret_cast<const u32x4_t *>(gate + m * ldg + k0);

@@ -235,17 +235,26 @@ def nint_ffn_decode(gate_up: NintWeight, down: NintWeight, x: torch.Tensor, acti
     return nint_matmul(down, _nint_matmul_glu(gate_up, x, torch.float16, activation))
 
 
-def nint_matmul_input_mul(w: NintWeight, x: torch.Tensor, gate: torch.Tensor, mode: int = 0) -> torch.Tensor:
+def nint_matmul_input_mul(w: NintWeight, x: torch.Tensor, gate: torch.Tensor, mode: int = 0, fused=True) -> torch.Tensor:
     """(x * silu(gate)) . W^T, or with mode 1 (x * sigmoid(gate)) . W^T (nint_matmul_input_mul,
-    cpp_runtime/mfq_decode.cpp:8395-8417): the gated activations are formed by one elementwise launch (fp32 product,
-    one rounding to the dtype of x) and go through nint_matmul."""
+    cpp_runtime/mfq_decode.cpp:8395-8417).  One or two rows: one GEMV launch whose waves gate their slice of the
+    activations as they stage it.  More rows (or rows the fused launch declines): the gated activations are formed by one
+    elementwise launch (fp32 product, one rounding to the dtype of x) and go through nint_matmul."""
     if gate.shape != x.shape:
         raise ValueError("gate and activations must have the same shape")
     x2 = _as_2d(x, w.neuron_len)
     g2 = _as_2d(gate.to(x2.dtype), w.neuron_len)
-    out = torch.empty((x2.shape[0], w.neuron_len), dtype=x2.dtype, device=x2.device)
     if x2.shape[0] == 0:
         return nint_matmul(w, x)
+    if x2.shape[0] <= 2 and fused:
+        y = torch.empty((x2.shape[0], w.out), dtype=torch.float32, device=x2.device)
+        rc = L.lib().mfq_hip_nint_gemv_gate(C.byref(w.desc), _ptr(w.data), _ptr(x2), _ptr(g2), _x_dtype(x2), x2.stride(0),
+                                            g2.stride(0), x2.shape[0], int(mode), _ptr(y), y.stride(0), _stream())
+        if rc == 0:
+            return y.reshape(*x.shape[:-1], w.out)
+        if rc != L.ERR_UNSUPPORTED:
+            L.check(rc)
+    out = torch.empty((x2.shape[0], w.neuron_len), dtype=x2.dtype, device=x2.device)
     L.check(L.lib().mfq_hip_input_gate(_ptr(x2), _ptr(g2), _x_dtype(x2), x2.stride(0), g2.stride(0), x2.shape[0],
                                        w.neuron_len, int(mode), _ptr(out), out.stride(0), _stream()))
     return nint_matmul(w, out.reshape(x.shape))
