@@ -32,6 +32,20 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+TRAFFIC_PROFILE = ROOT / "profiles" / "nint_gemv_paired_4_32_config2_decode.md"
+
+
+def profiled_traffic():
+    """HBM bytes per launch of the headline kernel as measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by a
+    plain copy): the line `TRAFFIC_BYTES_PER_LAUNCH = <bytes>` of the committed profile summary, or None."""
+    import re
+    try:
+        m = re.search(r"^TRAFFIC_BYTES_PER_LAUNCH\s*=\s*([0-9.eE+]+)", TRAFFIC_PROFILE.read_text(), re.M)
+    except OSError:
+        return None
+    return float(m.group(1)) if m else None
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -369,12 +383,14 @@ def main() -> int:
         "config": {"workload": "BASELINE config 2 decode: NINT4 (4,32,6) gate/up 12288x4096 + down 4096x12288 at M=1, "
                                f"gate+up as one grouped launch, {args.copies} rotating weight sets "
                                f"({args.copies * step_bytes / 1e6:.0f} MB)",
-                   "step_bytes": step_bytes, "launches_per_step": n_per_step, "hip_graph": True},
+                   "step_bytes": step_bytes, "launches_per_step": n_per_step, "hip_graph": True,
+                   # the library's effective tuning thresholds and CU count for this run
+                   "library": lib.mfq_hip_config().decode(errors="replace")},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, each scaled by what the counter
-                     # reads for a plain 256 MiB copy (2.000 and 1.000): profiles/nint_gemv_paired_4_32_config2_decode.md
-                     "traffic": 43.0e6,
+                     # reads for a plain 256 MiB copy: the figure the committed profile summary states
+                     "traffic": profiled_traffic(),
                      "kernel": "nint_gemv_paired_kernel<4,32,0,1,false>", "avg_launch_us": avg_launch_us,
                      "bytes_per_launch": bytes_per_launch},
         "cpu_baseline": cpu,

@@ -38,6 +38,24 @@ int mfq_rt_linear_check(void *handle, int M, int reps, double *out6);
 int mfq_rt_nvq_ffn_swiglu_down(void *gate, void *up, void *down, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                                void *stream);
 
+/* An MFQ1 file or shard set as one record table over read-only mappings (MfqFile, cpp_runtime/mfq_decode.cpp:1294-1527;
+ * open_mmap, mfq/formats/io.py:834-965).  `path` may name any shard of a set (<stem>-NNNNN-of-NNNNN.mfq).
+ * tensor_overlay / expert_overlay: NULL or "" take the environment variables MFQ_TENSOR_OVERLAY / MFQ_EXPERT_OVERLAY as
+ * the reference does, "-" takes none.  Records come in file order, shard after shard; `data` points into the mapping
+ * and stays valid until mfq_rt_file_close.  These calls need no GPU, except mfq_rt_file_load_quant_linear, which hands
+ * the mapped bytes to mfq_rt_load_quant_linear's loader. */
+int mfq_rt_file_open(const char *path, const char *tensor_overlay, const char *expert_overlay, void **handle);
+void mfq_rt_file_close(void *handle);
+int64_t mfq_rt_file_record_count(void *handle);
+int64_t mfq_rt_file_tensor_count(void *handle);
+int64_t mfq_rt_file_source_count(void *handle);
+const char *mfq_rt_file_arch(void *handle);
+const char *mfq_rt_file_extra(void *handle, const char *key); /* JSON text of a metadata value of the first shard, or NULL */
+int mfq_rt_file_record(void *handle, int64_t index, const char **name, const char **dtype, int *source,
+                       const void **data, size_t *nbytes);
+int mfq_rt_file_find(void *handle, const char *name, int64_t *index);
+int mfq_rt_file_load_quant_linear(void *handle, const char *name, void **linear);
+
 /* NINTM expert-wise tensors and nint_moe_ffn_forward (cpp_runtime/mfq_decode.cpp:3394-3416). */
 int mfq_rt_load_nint_moe(const void *blob, size_t n, void **handle);
 void mfq_rt_free_nint_moe(void *handle);

@@ -71,7 +71,7 @@ def test_check_linear_tool_reports_small_error(tmp_path):
             assert rel < 1e-3, (name, M, r.stdout)
             assert "production_weight_gbps=" in r.stdout and "payload_gbps=" in r.stdout
     r = subprocess.run([str(LIBDIR / "mfq-check-linear"), str(path), "missing"], capture_output=True, text=True)
-    assert r.returncode == 1 and "tensor not found" in r.stderr
+    assert r.returncode == 1 and "missing tensor" in r.stderr
 
 
 def test_cpp_load_quant_linear_and_forward(rt):
@@ -242,3 +242,49 @@ def test_cpp_expert_cache_matches_the_resident_tensor():
     hits, misses, evictions, nbytes, launches = list(stats)
     assert misses >= 6 and evictions > 0 and hits > 0 and nbytes > 0 and launches <= 5
     lib.mfq_rt_moe_cache_free(cache)
+
+
+def test_linears_load_from_a_mapped_shard_set(rt, tmp_path):
+    """A four-format model written as a shard set: both runtimes load every linear straight from the file mappings (any
+    shard names the set), dequantize bit-exactly, and mfq-check-linear takes a shard path; a tensor overlay swaps one
+    projection for another precision."""
+    from tyloquant_amd import formats as F
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(8)
+    tensors, want = {}, {}
+    for name, t in (("q", synth.nint_random(rng, 32, 96, 4, 24, 6)), ("k", synth.nint_random(rng, 16, 96, 3, 24, 5)),
+                    ("gate", synth.nvq_jsc_random(rng, 32, 96)), ("down", synth.nepq_random(rng, "NEPQ1-S", 1, 32, 192, 3))):
+        dtype, blob = O.pack_tensor(t)
+        tensors[name] = (dtype, blob)
+        want[name] = O.dequantize_tensor(t)
+    tensors[F.ASSET_PREFIX + "config.json"] = ("BLOB", b'{"hidden":96}')
+    paths = F.write_mfq_shards(tmp_path / "tiny.mfq", tensors, "tiny", extra={"general.name": "tiny"}, split_max_tensors=2)
+    assert len(paths) == 2
+    with F.MfqStore(paths[1], "", "") as st:
+        for name in want:
+            lin = R.load_quant_linear(st.record(name).dtype, st.blob(name))
+            got = lin.dequantize().cpu().numpy().reshape(want[name].shape)
+            assert np.array_equal(got.view(np.uint32), want[name].view(np.uint32)), name
+    rt.mfq_rt_file_open.argtypes = [C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(C.c_void_p)]
+    rt.mfq_rt_file_load_quant_linear.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]
+    rt.mfq_rt_file_close.argtypes = [C.c_void_p]
+    # an overlay that stores "k" at four bits instead of three
+    k4 = synth.nint_random(rng, 16, 96, 4, 24, 6)
+    over = tmp_path / "k4.mfq"
+    F.write_mfq(over, {"k": O.pack_tensor(k4)}, "tiny", 2)
+    for overlay, k_want in ((b"-", want["k"]), (str(over).encode(), O.dequantize_tensor(k4))):
+        f = C.c_void_p()
+        assert rt.mfq_rt_file_open(str(paths[0]).encode(), overlay, b"-", C.byref(f)) == 0, rt.mfq_rt_last_error()
+        for name in ("q", "k"):
+            h = C.c_void_p()
+            assert rt.mfq_rt_file_load_quant_linear(f, name.encode(), C.byref(h)) == 0, rt.mfq_rt_last_error()
+            ref = k_want if name == "k" else want[name]
+            out = torch.empty(ref.shape, dtype=torch.float32, device="cuda")
+            assert rt.mfq_rt_linear_dequantize(h, out.data_ptr(), None) == 0
+            torch.cuda.synchronize()
+            assert np.array_equal(out.cpu().numpy().view(np.uint32), ref.view(np.uint32)), name
+            rt.mfq_rt_free_quant_linear(h)
+        rt.mfq_rt_file_close(f)
+    r = subprocess.run([str(LIBDIR / "mfq-check-linear"), str(paths[1]), "q", "1", "20"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    assert float(re.search(r"production_rel=([0-9.e+-]+)", r.stdout).group(1)) < 1e-3

@@ -21,7 +21,7 @@ int main(int argc, char **argv) {
         mfq_rt::MfqFile file(argv[1]);
         const mfq_rt::MfqRecord &rec = file.find(argv[2]);
         const int M = argc > 3 ? std::atoi(argv[3]) : 1, reps = argc > 4 ? std::atoi(argv[4]) : 200;
-        mfq_rt::QuantLinear lin = mfq_rt::load_quant_linear(rec.dtype, file.bytes.data() + rec.offset, rec.nbytes);
+        mfq_rt::QuantLinear lin = mfq_rt::load_quant_linear(rec.dtype, file.data(rec), rec.nbytes);
         const mfq_rt::LinearCheckResult r = mfq_rt::run_linear_check(lin, M, reps);
         std::printf("check_linear tensor=%s dtype=%s out=%lld neuron_len=%lld m=%d reps=%d\n", rec.name.c_str(),
                     rec.dtype.c_str(), (long long)lin.out(), (long long)lin.neuron_len(), M, reps);

@@ -7,8 +7,16 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <cctype>
+#include <cstdlib>
 #include <fstream>
+#include <limits>
 #include <stdexcept>
+
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
 
 namespace mfq_rt {
 
@@ -837,57 +845,264 @@ void MoeExpertCache::forward(MoeCachedSource &source, const void *x, int x_dtype
 }
 
 // ---- MFQ1 container ---------------------------------------------------------------------------------------
-MfqFile::MfqFile(const std::string &path) {
-    std::ifstream f(path, std::ios::binary);
-    if (!f) fail("cannot open " + path);
-    bytes.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
-    const uint8_t *b = bytes.data();
-    const size_t n = bytes.size();
-    if (n < 12 || std::memcmp(b, "MFQ1", 4) != 0) fail("invalid MFQ magic");
-    const uint32_t version = rd<uint32_t>(b, 4);
-    size_t off = 8;
-    auto str = [&](std::string &s) {
-        if (off + 4 > n) fail("truncated MFQ header");
-        const uint32_t len = rd<uint32_t>(b, off);
+namespace {
+struct MfqHeaderInfo {
+    uint32_t version = 0, record_count = 0;
+    std::string architecture;
+    std::unordered_map<std::string, std::string> extra;
+};
+const uint64_t kNoCount = std::numeric_limits<uint64_t>::max();
+
+// integer metadata value (JSON text of a non-negative integer); `dflt` when the key is absent
+uint64_t json_uint(const std::unordered_map<std::string, std::string> &extra, const std::string &key, uint64_t dflt) {
+    auto it = extra.find(key);
+    if (it == extra.end()) return dflt;
+    const std::string &t = it->second;
+    size_t i = 0;
+    uint64_t v = 0;
+    bool digits = false;
+    for (; i < t.size() && t[i] >= '0' && t[i] <= '9'; ++i) {
+        if (v > (kNoCount - static_cast<uint64_t>(t[i] - '0')) / 10) fail("invalid MFQ integer metadata " + key + ": " + t);
+        v = v * 10 + static_cast<uint64_t>(t[i] - '0');
+        digits = true;
+    }
+    while (i < t.size() && std::isspace(static_cast<unsigned char>(t[i]))) ++i;
+    if (!digits || i != t.size()) fail("invalid MFQ integer metadata " + key + ": " + t);
+    return v;
+}
+
+// "<stem>-NNNNN-of-NNNNN.mfq": stem, 1-based index and count, or false
+bool parse_shard_name(const std::string &filename, std::string &stem, uint64_t &index, uint64_t &count) {
+    const size_t n = filename.size();  // tail: -ddddd-of-ddddd.mfq = 19 characters
+    if (n < 20 || filename.compare(n - 4, 4, ".mfq") != 0 || filename[n - 19] != '-' || filename.compare(n - 13, 4, "-of-") != 0)
+        return false;
+    index = count = 0;
+    for (size_t i = n - 18; i < n - 13; ++i) {
+        if (filename[i] < '0' || filename[i] > '9') return false;
+        index = index * 10 + static_cast<uint64_t>(filename[i] - '0');
+    }
+    for (size_t i = n - 9; i < n - 4; ++i) {
+        if (filename[i] < '0' || filename[i] > '9') return false;
+        count = count * 10 + static_cast<uint64_t>(filename[i] - '0');
+    }
+    stem = filename.substr(0, n - 19);
+    return !stem.empty();
+}
+
+std::vector<std::string> shard_paths(const std::string &path_value, uint64_t split_no, uint64_t split_count) {
+    const size_t slash = path_value.find_last_of('/');
+    const std::string dir = slash == std::string::npos ? "" : path_value.substr(0, slash + 1);
+    const std::string filename = slash == std::string::npos ? path_value : path_value.substr(slash + 1);
+    std::string stem;
+    uint64_t file_no = 0, file_count = 0;
+    if (!parse_shard_name(filename, stem, file_no, file_count))
+        fail("sharded MFQ path lacks -00001-of-00000 suffix: " + path_value);
+    if (file_no != split_no + 1 || file_count != split_count) fail("MFQ shard filename/metadata mismatch: " + path_value);
+    std::vector<std::string> result;
+    for (uint64_t i = 1; i <= split_count; ++i) {
+        char tail[32];
+        std::snprintf(tail, sizeof(tail), "-%05llu-of-%05llu.mfq", static_cast<unsigned long long>(i),
+                      static_cast<unsigned long long>(split_count));
+        const std::string shard = dir + stem + tail;
+        struct stat sb;
+        if (::stat(shard.c_str(), &sb) != 0 || !S_ISREG(sb.st_mode)) fail("missing MFQ shard: " + shard);
+        result.push_back(shard);
+    }
+    return result;
+}
+}  // namespace
+
+int MfqFile::map_file(const std::string &source) {
+    const int fd = ::open(source.c_str(), O_RDONLY);
+    if (fd < 0) fail("cannot open MFQ file: " + source);
+    struct stat sb;
+    if (::fstat(fd, &sb) != 0) {
+        ::close(fd);
+        fail("cannot stat MFQ file: " + source);
+    }
+    Mapping m;
+    m.size = static_cast<size_t>(sb.st_size);
+    if (m.size) {
+        void *p = ::mmap(nullptr, m.size, PROT_READ, MAP_PRIVATE, fd, 0);
+        if (p == MAP_FAILED) {
+            ::close(fd);
+            fail("cannot map MFQ file: " + source);
+        }
+        m.base = static_cast<const uint8_t *>(p);
+    }
+    ::close(fd);  // the mapping keeps the file
+    maps_.push_back(m);
+    source_paths.push_back(source);
+    return static_cast<int>(maps_.size()) - 1;
+}
+
+MfqFile::~MfqFile() {
+    for (const Mapping &m : maps_)
+        if (m.base) ::munmap(const_cast<uint8_t *>(m.base), m.size);
+}
+
+MfqFile::MfqFile(const std::string &path_in, const std::string &tensor_overlay, const std::string &expert_overlay)
+    : path(path_in) {
+    // header + record table of one file into `out` (its records appended in file order)
+    auto load_records = [this](const std::string &source, std::vector<MfqRecord> &out) {
+        const int src = map_file(source);
+        const uint8_t *b = maps_[static_cast<size_t>(src)].base;
+        const size_t n = maps_[static_cast<size_t>(src)].size;
+        if (n < 12 || std::memcmp(b, "MFQ1", 4) != 0) fail("invalid MFQ magic: " + source);
+        MfqHeaderInfo h;
+        h.version = rd<uint32_t>(b, 4);
+        size_t off = 8;
+        auto str = [&](std::string &s) {
+            if (off + 4 > n) fail("truncated MFQ header: " + source);
+            const uint32_t len = rd<uint32_t>(b, off);
+            off += 4;
+            if (len > n - off) fail("truncated MFQ header: " + source);
+            s.assign(reinterpret_cast<const char *>(b + off), len);
+            off += len;
+        };
+        str(h.architecture);
+        if (h.version >= 2) {
+            if (off + 4 > n) fail("truncated MFQ header: " + source);
+            const uint32_t n_extra = rd<uint32_t>(b, off);
+            off += 4;
+            for (uint32_t i = 0; i < n_extra; ++i) {
+                std::string key, value;
+                str(key);
+                str(value);
+                if (!h.extra.emplace(key, value).second) fail("duplicate MFQ metadata key: " + key + ": " + source);
+            }
+        }
+        if (off + 4 > n) fail("truncated MFQ header: " + source);
+        h.record_count = rd<uint32_t>(b, off);
         off += 4;
-        if (len > n - off) fail("truncated MFQ header");
-        s.assign(reinterpret_cast<const char *>(b + off), len);
-        off += len;
+        const size_t first = out.size();
+        for (uint32_t i = 0; i < h.record_count; ++i) {
+            MfqRecord r;
+            str(r.name);
+            str(r.dtype);
+            if (off + 8 > n) fail("truncated MFQ directory: " + source);
+            r.nbytes = static_cast<size_t>(rd<uint64_t>(b, off));
+            off += 8;
+            r.source = src;
+            out.push_back(std::move(r));
+        }
+        for (size_t i = first; i < out.size(); ++i) {
+            MfqRecord &r = out[i];
+            if (r.nbytes > n - off) fail("truncated MFQ blob for " + r.name + ": " + source);  // compared with what is left: cannot wrap
+            r.offset = off;
+            off += r.nbytes;
+        }
+        if (off != n)
+            fail("MFQ file length mismatch: records end=" + std::to_string(off) + ", file size=" + std::to_string(n) + ": " + source);
+        return h;
     };
-    str(model_arch);
-    if (version >= 2) {
-        if (off + 4 > n) fail("truncated MFQ header");
-        const uint32_t extra = rd<uint32_t>(b, off);
-        off += 4;
-        std::string tmp;
-        for (uint32_t i = 0; i < 2 * extra; ++i) str(tmp);
+    auto reject_duplicates = [](const std::vector<MfqRecord> &recs, const std::string &what) {
+        std::unordered_map<std::string, int> seen;
+        for (const MfqRecord &r : recs)
+            if (!seen.emplace(r.name, 1).second) fail("duplicate MFQ tensor record: " + r.name + ": " + what);
+    };
+
+    MfqHeaderInfo probe = load_records(path, records);
+    const uint64_t split_no = json_uint(probe.extra, "split.no", 0);
+    const uint64_t split_count = json_uint(probe.extra, "split.count", 1);
+    if (split_count < 1 || split_count > 99999 || split_no >= split_count) fail("invalid MFQ split metadata: " + path);
+    model_arch = probe.architecture;
+    version = probe.version;
+    extra = probe.extra;
+    if (split_count > 1) {
+        const std::vector<std::string> paths = shard_paths(path, split_no, split_count);
+        // start over in shard order
+        records.clear();
+        for (const Mapping &m : maps_)
+            if (m.base) ::munmap(const_cast<uint8_t *>(m.base), m.size);
+        maps_.clear();
+        source_paths.clear();
+        uint64_t expected_records = kNoCount, expected_tensors = kNoCount;
+        for (uint64_t i = 0; i < split_count; ++i) {
+            const std::string &shard = paths[static_cast<size_t>(i)];
+            const MfqHeaderInfo cur = load_records(shard, records);
+            if (json_uint(cur.extra, "split.no", split_count) != i || json_uint(cur.extra, "split.count", 0) != split_count)
+                fail("MFQ shard metadata mismatch: " + shard);
+            if (cur.version != probe.version || cur.architecture != probe.architecture)
+                fail("MFQ shard architecture/version mismatch: " + shard);
+            const uint64_t cr = json_uint(cur.extra, "split.records.count", kNoCount);
+            const uint64_t ct = json_uint(cur.extra, "split.tensors.count", kNoCount);
+            if (expected_records == kNoCount) expected_records = cr;
+            else if (cr != kNoCount && cr != expected_records) fail("MFQ shard record count mismatch: " + shard);
+            if (expected_tensors == kNoCount) expected_tensors = ct;
+            else if (ct != kNoCount && ct != expected_tensors) fail("MFQ shard tensor count mismatch: " + shard);
+            if (i == 0) extra = cur.extra;  // model metadata lives in the first shard
+        }
+        reject_duplicates(records, "across shards");
+        if (expected_records != kNoCount && records.size() != expected_records) fail("MFQ shard record total mismatch");
+        if (expected_tensors != kNoCount && tensor_count() != expected_tensors) fail("MFQ shard tensor total mismatch");
+        path = paths.front();
+    } else {
+        std::string stem;
+        uint64_t file_no = 0, file_count = 0;
+        const size_t slash = path.find_last_of('/');
+        if (parse_shard_name(slash == std::string::npos ? path : path.substr(slash + 1), stem, file_no, file_count) &&
+            file_count != 1)
+            fail("MFQ filename claims multiple shards but metadata does not: " + path);
+        reject_duplicates(records, path);
     }
-    if (off + 4 > n) fail("truncated MFQ header");
-    const uint32_t count = rd<uint32_t>(b, off);
-    off += 4;
-    for (uint32_t i = 0; i < count; ++i) {
-        MfqRecord r;
-        str(r.name);
-        str(r.dtype);
-        if (off + 8 > n) fail("truncated MFQ directory");
-        r.nbytes = rd<uint64_t>(b, off);
-        off += 8;
-        records.push_back(std::move(r));
+
+    auto overlay_path = [](const std::string &given, const char *env) -> std::string {
+        if (given == "-") return "";
+        if (!given.empty()) return given;
+        const char *v = std::getenv(env);
+        return v ? std::string(v) : std::string();
+    };
+    const std::string tensor_src = overlay_path(tensor_overlay, "MFQ_TENSOR_OVERLAY");
+    if (!tensor_src.empty()) {
+        std::vector<MfqRecord> over;
+        const MfqHeaderInfo oh = load_records(tensor_src, over);
+        if (json_uint(oh.extra, "split.count", 1) != 1) fail("sharded MFQ tensor overlays are not supported");
+        reject_duplicates(over, tensor_src);
+        for (MfqRecord &o : over) {
+            bool found = false;
+            for (MfqRecord &base : records)
+                if (base.name == o.name) {
+                    base = o;
+                    found = true;
+                }
+            if (!found) fail("tensor overlay replaces an unknown record: " + o.name);
+            tensor_overlays.emplace(o.name, o);
+        }
     }
-    for (size_t i = 0; i < records.size(); ++i) {
-        MfqRecord &r = records[i];
-        for (size_t j = 0; j < i; ++j)
-            if (records[j].name == r.name) fail("duplicate MFQ tensor record: " + r.name + ": " + path);
-        if (r.nbytes > n - off) fail("truncated MFQ blob for " + r.name);   // compared with what is left: cannot wrap
-        r.offset = off;
-        off += static_cast<size_t>(r.nbytes);
+    const std::string expert_src = overlay_path(expert_overlay, "MFQ_EXPERT_OVERLAY");
+    if (!expert_src.empty()) {
+        std::vector<MfqRecord> over;
+        const MfqHeaderInfo oh = load_records(expert_src, over);
+        if (json_uint(oh.extra, "split.count", 1) != 1) fail("sharded MFQ expert overlays are not supported");
+        reject_duplicates(over, expert_src);
+        for (MfqRecord &o : over) {
+            if (o.dtype != "NINTMD" || !has_record(o.name) || find(o.name).dtype != "NINTM")
+                fail("invalid expert overlay record: " + o.name);
+            expert_overlays.emplace(o.name, o);
+        }
     }
-    if (off != n) fail("MFQ file length mismatch: records end=" + std::to_string(off) + ", file size=" + std::to_string(n));
 }
 const MfqRecord &MfqFile::find(const std::string &name) const {
     for (const auto &r : records)
         if (r.name == name) return r;
-    fail("tensor not found: " + name);
+    fail("missing tensor: " + name);
+}
+bool MfqFile::has_record(const std::string &name) const {
+    for (const auto &r : records)
+        if (r.name == name) return true;
+    return false;
+}
+const uint8_t *MfqFile::data(const MfqRecord &r) const { return maps_.at(static_cast<size_t>(r.source)).base + r.offset; }
+size_t MfqFile::tensor_count() const {
+    size_t n = 0;
+    for (const auto &r : records) n += r.name.rfind("__mfq_asset__/", 0) != 0;
+    return n;
+}
+std::string MfqFile::read_asset_text(const std::string &name) const {
+    const MfqRecord &r = find(name);
+    if (r.dtype != "BLOB") fail("MFQ runtime asset has non-BLOB dtype: " + name);
+    return std::string(reinterpret_cast<const char *>(data(r)), r.nbytes);
 }
 
 // ---- --check-linear -------------------------------------------------------------------------------------------
@@ -1050,6 +1265,49 @@ int mfq_rt_load_nint_moe(const void *blob, size_t n, void **handle) {
     return guard([&] { *handle = new NintMoeWeight(NintMoeWeight::from_blob(static_cast<const uint8_t *>(blob), n)); });
 }
 void mfq_rt_free_nint_moe(void *handle) { delete static_cast<NintMoeWeight *>(handle); }
+int mfq_rt_file_open(const char *path, const char *tensor_overlay, const char *expert_overlay, void **handle) {
+    return guard([&] {
+        *handle = new MfqFile(path ? path : "", tensor_overlay ? tensor_overlay : "", expert_overlay ? expert_overlay : "");
+    });
+}
+void mfq_rt_file_close(void *handle) { delete static_cast<MfqFile *>(handle); }
+int64_t mfq_rt_file_record_count(void *handle) { return static_cast<int64_t>(static_cast<MfqFile *>(handle)->records.size()); }
+int64_t mfq_rt_file_tensor_count(void *handle) { return static_cast<int64_t>(static_cast<MfqFile *>(handle)->tensor_count()); }
+int64_t mfq_rt_file_source_count(void *handle) { return static_cast<int64_t>(static_cast<MfqFile *>(handle)->source_paths.size()); }
+const char *mfq_rt_file_arch(void *handle) { return static_cast<MfqFile *>(handle)->model_arch.c_str(); }
+const char *mfq_rt_file_extra(void *handle, const char *key) {
+    const MfqFile *f = static_cast<MfqFile *>(handle);
+    auto it = f->extra.find(key ? key : "");
+    return it == f->extra.end() ? nullptr : it->second.c_str();
+}
+int mfq_rt_file_record(void *handle, int64_t index, const char **name, const char **dtype, int *source, const void **data,
+                       size_t *nbytes) {
+    return guard([&] {
+        const MfqFile *f = static_cast<MfqFile *>(handle);
+        if (index < 0 || index >= static_cast<int64_t>(f->records.size())) fail("MFQ record index out of range");
+        const MfqRecord &r = f->records[static_cast<size_t>(index)];
+        if (name) *name = r.name.c_str();
+        if (dtype) *dtype = r.dtype.c_str();
+        if (source) *source = r.source;
+        if (data) *data = f->data(r);
+        if (nbytes) *nbytes = r.nbytes;
+    });
+}
+int mfq_rt_file_find(void *handle, const char *name, int64_t *index) {
+    return guard([&] {
+        const MfqFile *f = static_cast<MfqFile *>(handle);
+        const MfqRecord &r = f->find(name ? name : "");
+        *index = &r - f->records.data();
+    });
+}
+int mfq_rt_file_load_quant_linear(void *handle, const char *name, void **linear) {
+    return guard([&] {
+        const MfqFile *f = static_cast<MfqFile *>(handle);
+        const MfqRecord &r = f->find(name ? name : "");
+        *linear = new QuantLinear(load_quant_linear(r.dtype, f->data(r), r.nbytes));
+    });
+}
+
 int mfq_rt_moe_ffn_forward(void *gate_up, void *down, const void *x, int x_dtype, int64_t ldx, int T,
                            const float *router_logits, int top_k, int topk_mode, int normalize, void *shared_gate_up,
                            void *shared_down, float *out, int32_t *ids_out, float *weights_out, void *stream) {

@@ -18,7 +18,7 @@
 //   MoeRoutePlan / build_moe_route_plan  :2579-2592, 2681-2708   MoeRoutePlan / build_moe_route_plan
 //   nint_moe_ffn_forward             :3394-3416       nint_moe_ffn_forward
 //   is_nint_linear_dtype / load_quant_linear :9409-9420, 9489-9771   same names
-//   MfqFile                          :1294-1527       MfqFile (directory + blobs, single file)
+//   MfqFile                          :1294-1527       MfqFile (mapped files, shard sets, tensor / expert overlays)
 //   run_linear_check                 :16510-16638     run_linear_check
 #pragma once
 #include <cstddef>
@@ -296,16 +296,44 @@ private:
 };
 
 // ---- MFQ1 container + the --check-linear harness ----------------------------------------------------
+// One MFQ1 file or shard set as one record table over read-only mappings of the files (MfqFile,
+// cpp_runtime/mfq_decode.cpp:1294-1527; mfq/formats/io.py:834-965 open_mmap).  A file whose header carries
+// split.count > 1 must be named <stem>-NNNNN-of-NNNNN.mfq; any shard of the set may be given.  Checks and messages follow
+// the reference: split metadata against the file names, one architecture / version, the tensor and record totals,
+// no record twice, records ending at the file size.
 struct MfqRecord {
     std::string name, dtype;
-    size_t offset, nbytes;
+    size_t offset = 0, nbytes = 0;
+    int source = 0;  // index into MfqFile::source_paths
 };
 struct MfqFile {
-    std::vector<uint8_t> bytes;
+    std::string path;  // the first shard (or the file itself)
+    std::vector<std::string> source_paths;
     std::string model_arch;
-    std::vector<MfqRecord> records;
-    explicit MfqFile(const std::string &path);
+    uint32_t version = 0;
+    std::unordered_map<std::string, std::string> extra;  // metadata of the first shard: key -> JSON text
+    std::vector<MfqRecord> records;                     // file order, shard after shard
+    std::unordered_map<std::string, MfqRecord> tensor_overlays, expert_overlays;
+    // tensor_overlay: an unsharded MFQ1 file whose records replace records of the same name (each must exist);
+    // expert_overlay: NINTMD records over NINTM records of the same name, kept aside.  Empty: the environment variables
+    // MFQ_TENSOR_OVERLAY / MFQ_EXPERT_OVERLAY, as in the reference; "-" disables the lookup.
+    explicit MfqFile(const std::string &path, const std::string &tensor_overlay = "", const std::string &expert_overlay = "");
+    ~MfqFile();
+    MfqFile(const MfqFile &) = delete;
+    MfqFile &operator=(const MfqFile &) = delete;
     const MfqRecord &find(const std::string &name) const;
+    bool has_record(const std::string &name) const;
+    const uint8_t *data(const MfqRecord &r) const;  // the record's bytes inside the mapping of its file
+    size_t tensor_count() const;                    // records that are not runtime assets (__mfq_asset__/...)
+    std::string read_asset_text(const std::string &name) const;  // a BLOB record as text
+
+private:
+    struct Mapping {
+        const uint8_t *base = nullptr;
+        size_t size = 0;
+    };
+    std::vector<Mapping> maps_;
+    int map_file(const std::string &source);
 };
 struct LinearCheckResult {
     double production_ms, production_weight_gbps, payload_gbps, production_rel, production_mean_abs, production_max_abs;

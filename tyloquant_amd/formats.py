@@ -7,9 +7,13 @@ the bit streams in place.  No dequantization happens here: that is the GPU's job
 """
 from __future__ import annotations
 
+import json
 import math
+import os
+import re
 import struct
 from dataclasses import dataclass, field
+from pathlib import Path
 
 import numpy as np
 
@@ -462,50 +466,155 @@ def parse_nintm(blob) -> NintmHeader:
 
 
 # ---------------------------------------------------------------------------------------
-# MFQ1 container (mfq/formats/io.py:646-685): header, directory, blobs back to back
+# MFQ1 container (mfq/formats/io.py:646-965, mfq/formats/shards.py): header, directory, blobs back to back; one file or a
+# shard set <stem>-NNNNN-of-NNNNN.mfq whose headers carry split.* metadata
 # ---------------------------------------------------------------------------------------
-def write_mfq(path, tensors: dict, model_arch: str = "synthetic", version: int = 1) -> None:
-    """tensors: name -> (dtype string, blob bytes)."""
+ASSET_PREFIX = "__mfq_asset__/"        # runtime assets: container metadata, first shard only (mfq/formats/assets.py:17)
+SPLIT_NO, SPLIT_COUNT, SPLIT_TENSORS, SPLIT_RECORDS = "split.no", "split.count", "split.tensors.count", "split.records.count"
+_SHARD_RE = re.compile(r"^(?P<stem>.+)-(?P<index>[0-9]{5})-of-(?P<count>[0-9]{5})\.mfq$")
+
+
+def _mfq_head(records, model_arch: str, version: int, extra: dict | None) -> bytes:
+    """Header and record table: magic, version, architecture, (version >= 2) metadata as key / JSON text pairs, then
+    per record name, dtype string and byte length (mfq/formats/shards.py:205-236)."""
+    extra = dict(extra or {})
+    if extra and version < 2:
+        version = 2
+    a = model_arch.encode()
+    out = [b"MFQ1", struct.pack("<I", version), struct.pack("<I", len(a)), a]
+    if version >= 2:
+        out.append(struct.pack("<I", len(extra)))
+        for key, value in extra.items():
+            kb, vb = str(key).encode(), json.dumps(value).encode()
+            out += [struct.pack("<I", len(kb)), kb, struct.pack("<I", len(vb)), vb]
+    out.append(struct.pack("<I", len(records)))
+    for name, dtype, nbytes in records:
+        nb, db = name.encode(), dtype.encode()
+        out += [struct.pack("<I", len(nb)), nb, struct.pack("<I", len(db)), db, struct.pack("<Q", nbytes)]
+    return b"".join(out)
+
+
+def write_mfq(path, tensors: dict, model_arch: str = "synthetic", version: int = 1, extra: dict | None = None) -> None:
+    """tensors: name -> (dtype string, blob bytes); extra: metadata of a version 2 header (values are stored as JSON)."""
     with open(path, "wb") as f:
-        a = model_arch.encode()
-        f.write(b"MFQ1" + struct.pack("<I", version) + struct.pack("<I", len(a)) + a)
-        if version >= 2:
-            f.write(struct.pack("<I", 0))
-        f.write(struct.pack("<I", len(tensors)))
-        for name, (dtype, blob) in tensors.items():
-            nb, db = name.encode(), dtype.encode()
-            f.write(struct.pack("<I", len(nb)) + nb + struct.pack("<I", len(db)) + db + struct.pack("<Q", len(blob)))
+        f.write(_mfq_head([(n, d, len(b)) for n, (d, b) in tensors.items()], model_arch, version, extra))
         for _, (_, blob) in tensors.items():
             f.write(blob)
 
 
-def read_mfq_directory(data) -> dict:
-    """name -> (dtype, offset, nbytes) of an MFQ1 file image."""
-    if data[:4] != b"MFQ1":
+def format_shard_path(path, index: int, count: int) -> Path:
+    """<stem>-00001-of-00004.mfq, 1-based (format_shard_path, mfq/formats/shards.py:46-53)."""
+    source = Path(path)
+    if not 1 <= index <= count <= 99999:
+        raise ValueError(f"invalid MFQ shard index/count: {index}/{count}")
+    stem = source.name[:-4] if source.name.lower().endswith(".mfq") else source.name
+    return source.with_name(f"{stem}-{index:05d}-of-{count:05d}.mfq")
+
+
+def parse_shard_path(path):
+    """(base path, 1-based index, count) of a shard file name, or None (parse_shard_path, shards.py:56-68)."""
+    source = Path(path)
+    m = _SHARD_RE.fullmatch(source.name)
+    if m is None:
+        return None
+    count, index = int(m.group("count")), int(m.group("index"))
+    if count < 1 or index < 1 or index > count:
+        raise ValueError(f"invalid MFQ shard file name: {source}")
+    return source.with_name(f"{m.group('stem')}.mfq"), index, count
+
+
+def plan_shards(sizes, split_max_size: int = 0, split_max_tensors: int = 0):
+    """Records -> shards by the reference's rule (plan_record_shards, shards.py:133-173): `sizes` is [(name, nbytes)] in
+    file order; a tensor opens a new shard when adding it to a non-empty shard would pass split_max_size, or when the
+    shard already holds split_max_tensors tensors; runtime assets all go to the front of the first shard.  Returns the
+    list of shards, each a list of names."""
+    if split_max_size < 0 or split_max_tensors < 0:
+        raise ValueError("MFQ shard limits must be non-negative")
+    if split_max_size and split_max_tensors:
+        raise ValueError("--split-max-size and --split-max-tensors are mutually exclusive")
+    if not split_max_size and not split_max_tensors:
+        return [[n for n, _ in sizes]]
+    assets = [n for n, _ in sizes if n.startswith(ASSET_PREFIX)]
+    shards, payload, count = [[]], [0], [0]
+    for name, nbytes in sizes:
+        if name.startswith(ASSET_PREFIX):
+            continue
+        over_size = bool(split_max_size and count[-1] > 0 and payload[-1] + int(nbytes) > split_max_size)
+        over_count = bool(split_max_tensors and count[-1] >= split_max_tensors)
+        if over_size or over_count:
+            shards.append([]); payload.append(0); count.append(0)
+        shards[-1].append(name)
+        payload[-1] += int(nbytes)
+        count[-1] += 1
+    shards[0][0:0] = assets
+    return shards
+
+
+def write_mfq_shards(path, tensors: dict, model_arch: str = "synthetic", version: int = 2, extra: dict | None = None,
+                     split_max_size: int = 0, split_max_tensors: int = 0) -> list:
+    """The shard set of `tensors` next to `path` (write_blob_record_shards, shards.py:254-336): every shard is an MFQ1
+    file of version >= 2 whose metadata holds split.no / split.count and the totals of tensors and records; the model's
+    own metadata stays in the first shard only.  Without a limit: the single file `path`.  Returns the paths written."""
+    plan = plan_shards([(n, len(b)) for n, (_, b) in tensors.items()], split_max_size, split_max_tensors)
+    if not (split_max_size or split_max_tensors):
+        write_mfq(path, tensors, model_arch, version, extra)
+        return [Path(path)]
+    n_tensors = sum(not n.startswith(ASSET_PREFIX) for n in tensors)
+    paths = []
+    for no, names in enumerate(plan):
+        meta = {k: v for k, v in (extra or {}).items() if not k.startswith("split.")} if no == 0 else {}
+        meta.update({SPLIT_NO: no, SPLIT_COUNT: len(plan), SPLIT_TENSORS: n_tensors, SPLIT_RECORDS: len(tensors)})
+        dest = format_shard_path(path, no + 1, len(plan))
+        write_mfq(dest, {n: tensors[n] for n in names}, model_arch, max(2, version), meta)
+        paths.append(dest)
+    return paths
+
+
+def read_mfq_header(data):
+    """(version, architecture, metadata {key: decoded JSON value}, [(name, dtype, nbytes)], offset of the first blob)."""
+    if len(data) < 12 or bytes(data[:4]) != b"MFQ1":
         raise ValueError("invalid MFQ magic")
     version, = struct.unpack_from("<I", data, 4)
-    off = 8
-    n, = struct.unpack_from("<I", data, off)
-    off += 4 + n
+    pos = [8]
+
+    def text():
+        if pos[0] + 4 > len(data):
+            raise ValueError("truncated MFQ header")
+        n, = struct.unpack_from("<I", data, pos[0])
+        if n > len(data) - pos[0] - 4:
+            raise ValueError("truncated MFQ header")
+        v = bytes(data[pos[0] + 4: pos[0] + 4 + n]).decode()
+        pos[0] += 4 + n
+        return v
+
+    arch = text()
+    extra = {}
     if version >= 2:
-        ne, = struct.unpack_from("<I", data, off)
-        off += 4
-        for _ in range(2 * ne):
-            n, = struct.unpack_from("<I", data, off)
-            off += 4 + n
-    nt, = struct.unpack_from("<I", data, off)
-    off += 4
+        ne, = struct.unpack_from("<I", data, pos[0])
+        pos[0] += 4
+        for _ in range(ne):
+            key, value = text(), text()
+            if key in extra:
+                raise ValueError(f"duplicate MFQ metadata key: {key}")
+            extra[key] = json.loads(value)
+    if pos[0] + 4 > len(data):
+        raise ValueError("truncated MFQ header")
+    nt, = struct.unpack_from("<I", data, pos[0])
+    pos[0] += 4
     recs = []
     for _ in range(nt):
-        n, = struct.unpack_from("<I", data, off)
-        name = bytes(data[off + 4: off + 4 + n]).decode()
-        off += 4 + n
-        n, = struct.unpack_from("<I", data, off)
-        dtype = bytes(data[off + 4: off + 4 + n]).decode()
-        off += 4 + n
-        ln, = struct.unpack_from("<Q", data, off)
-        off += 8
+        name, dtype = text(), text()
+        if pos[0] + 8 > len(data):
+            raise ValueError("truncated MFQ directory")
+        ln, = struct.unpack_from("<Q", data, pos[0])
+        pos[0] += 8
         recs.append((name, dtype, ln))
+    return version, arch, extra, recs, pos[0]
+
+
+def read_mfq_directory(data) -> dict:
+    """name -> (dtype, offset, nbytes) of an MFQ1 file image."""
+    _, _, _, recs, off = read_mfq_header(data)
     out = {}
     for name, dtype, ln in recs:
         if name in out:
@@ -517,3 +626,178 @@ def read_mfq_directory(data) -> dict:
     if off != len(data):       # mfq/formats/io.py:826-827
         raise ValueError(f"MFQ file length mismatch: records end={off}, file size={len(data)}")
     return out
+
+
+def _split_values(extra: dict):
+    """(split.no, split.count, tensors total or None, records total or None) (split_values, shards.py:96-113)."""
+    no, count = int(extra.get(SPLIT_NO, 0)), int(extra.get(SPLIT_COUNT, 1))
+    if count < 1 or count > 99999:
+        raise ValueError(f"invalid {SPLIT_COUNT}: {count}")
+    if no < 0 or no >= count:
+        raise ValueError(f"invalid {SPLIT_NO}: {no}")
+    t, r = extra.get(SPLIT_TENSORS), extra.get(SPLIT_RECORDS)
+    return no, count, None if t is None else int(t), None if r is None else int(r)
+
+
+@dataclass
+class MfqRecord:
+    name: str
+    dtype: str
+    source: int      # index into MfqStore.paths
+    offset: int
+    nbytes: int
+
+
+class MfqStore:
+    """One MFQ1 file or shard set as one lazy record table over read-only memory maps (open_mmap,
+    mfq/formats/io.py:834-965; MfqFile, cpp_runtime/mfq_decode.cpp:1294-1527).  `path` may be any shard of a set.
+    blob(name) is a zero-copy view into the map.  tensor_overlay: an unsharded MFQ1 file whose records replace records
+    of the same name (each must exist); expert_overlay: NINTMD records over NINTM records, kept in expert_overlays.
+    None takes MFQ_TENSOR_OVERLAY / MFQ_EXPERT_OVERLAY from the environment, as the reference does; "" takes none."""
+
+    def __init__(self, path, tensor_overlay: str | None = None, expert_overlay: str | None = None):
+        self.paths, self._files, self._maps = [], [], []
+        self.records: dict[str, MfqRecord] = {}
+        self.tensor_overlays: dict[str, MfqRecord] = {}
+        self.expert_overlays: dict[str, MfqRecord] = {}
+        try:
+            self._open(Path(path), tensor_overlay, expert_overlay)
+        except Exception:
+            self.close()
+            raise
+
+    def _map(self, path: Path):
+        """Maps one file; returns (source index, version, architecture, metadata, {name: MfqRecord})."""
+        import mmap
+        if not path.is_file():
+            raise FileNotFoundError(f"cannot open MFQ file: {path}")
+        f = open(path, "rb")
+        self._files.append(f)
+        m = mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_READ)
+        self._maps.append(m)
+        self.paths.append(path)
+        src = len(self._maps) - 1
+        view = memoryview(m)
+        try:
+            version, arch, extra, recs, off = read_mfq_header(view)
+            out = {}
+            for name, dtype, ln in recs:
+                if name in out:
+                    raise ValueError(f"duplicate MFQ tensor record: {name}: {path}")
+                if ln > len(view) - off:
+                    raise ValueError(f"truncated MFQ blob for {name}: {path}")
+                out[name] = MfqRecord(name, dtype, src, off, ln)
+                off += ln
+            if off != len(view):
+                raise ValueError(f"MFQ file length mismatch: records end={off}, file size={len(view)}: {path}")
+        finally:
+            view.release()
+        return src, version, arch, extra, out
+
+    def _open(self, requested: Path, tensor_overlay, expert_overlay):
+        _, version, arch, extra, first = self._map(requested)
+        split_no, split_count, want_tensors, want_records = _split_values(extra)
+        parsed = parse_shard_path(requested)
+        self.version, self.model_arch, self.extra = version, arch, extra
+        if split_count == 1:
+            if parsed is not None and parsed[2] != 1:
+                raise ValueError(f"MFQ filename claims multiple shards but metadata does not: {requested}")
+            self.records = first
+        else:
+            if parsed is None:
+                raise ValueError(f"sharded MFQ path lacks -00001-of-00000 suffix: {requested}")
+            if parsed[1] - 1 != split_no or parsed[2] != split_count:
+                raise ValueError(f"MFQ shard filename/metadata mismatch: {requested}")
+            paths = [format_shard_path(parsed[0], i, split_count) for i in range(1, split_count + 1)]
+            for p in paths:
+                if not p.is_file():
+                    raise FileNotFoundError(f"missing MFQ shard: {p}")
+            self.close()                                    # start over in shard order
+            for i, p in enumerate(paths):
+                _, v, a, ex, recs = self._map(p)
+                no, count, t, r = _split_values(ex)
+                if no != i or count != split_count:
+                    raise ValueError(f"MFQ shard metadata mismatch: expected {i}/{split_count}, got {no}/{count}: {p}")
+                if v != version or a != arch:
+                    raise ValueError(f"MFQ shard architecture/version mismatch: {p}")
+                if want_tensors is None:
+                    want_tensors = t
+                elif t is not None and t != want_tensors:
+                    raise ValueError(f"MFQ shard tensor count mismatch: {p}")
+                if want_records is None:
+                    want_records = r
+                elif r is not None and r != want_records:
+                    raise ValueError(f"MFQ shard record count mismatch: {p}")
+                if i == 0:
+                    self.extra = ex                         # model metadata lives in the first shard
+                for name, rec in recs.items():
+                    if name in self.records:
+                        raise ValueError(f"duplicate MFQ tensor across shards: {name}")
+                    self.records[name] = rec
+            if want_records is not None and len(self.records) != want_records:
+                raise ValueError(f"MFQ shard record total mismatch: {len(self.records)} != {want_records}")
+            if want_tensors is not None and self.tensor_count() != want_tensors:
+                raise ValueError(f"MFQ shard tensor total mismatch: {self.tensor_count()} != {want_tensors}")
+        self.n_shards = len(self.paths)
+        if tensor_overlay is None:
+            tensor_overlay = os.environ.get("MFQ_TENSOR_OVERLAY", "")
+        if expert_overlay is None:
+            expert_overlay = os.environ.get("MFQ_EXPERT_OVERLAY", "")
+        if tensor_overlay:
+            _, _, _, ex, recs = self._map(Path(tensor_overlay))
+            if _split_values(ex)[1] != 1:
+                raise ValueError("sharded MFQ tensor overlays are not supported")
+            for name, rec in recs.items():
+                if name not in self.records:
+                    raise ValueError(f"tensor overlay replaces an unknown record: {name}")
+                self.records[name] = rec
+                self.tensor_overlays[name] = rec
+        if expert_overlay:
+            _, _, _, ex, recs = self._map(Path(expert_overlay))
+            if _split_values(ex)[1] != 1:
+                raise ValueError("sharded MFQ expert overlays are not supported")
+            for name, rec in recs.items():
+                if rec.dtype != "NINTMD" or name not in self.records or self.records[name].dtype != "NINTM":
+                    raise ValueError(f"invalid expert overlay record: {name}")
+                self.expert_overlays[name] = rec
+
+    def tensor_count(self) -> int:
+        return sum(not n.startswith(ASSET_PREFIX) for n in self.records)
+
+    def __contains__(self, name) -> bool:
+        return name in self.records
+
+    def names(self):
+        return list(self.records)
+
+    def record(self, name) -> MfqRecord:
+        if name not in self.records:
+            raise KeyError(f"missing tensor: {name}")
+        return self.records[name]
+
+    def blob(self, name) -> memoryview:
+        """The record's bytes as a read-only view into the file map (no copy); valid until close()."""
+        r = self.record(name)
+        return memoryview(self._maps[r.source])[r.offset: r.offset + r.nbytes]
+
+    def asset_text(self, name) -> str:
+        r = self.record(name)
+        if r.dtype != "BLOB":
+            raise ValueError(f"MFQ runtime asset has non-BLOB dtype: {name}")
+        return bytes(self.blob(name)).decode()
+
+    def close(self):
+        for m in self._maps:
+            try:
+                m.close()
+            except BufferError:          # a blob view is still alive: the map goes with its last view
+                pass
+        for f in self._files:
+            f.close()
+        self.paths, self._files, self._maps, self.records = [], [], [], {}
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
