@@ -276,6 +276,44 @@ int mfq_hip_nvq_gemm(const mfq_nvq_desc *d, const void *weight, const void *x, i
                      mfq_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
+ * NVQ payloads read in place from their bit streams: the E8 family -- NVQ2 (e8_256, plain, parity or index-parity
+ * signs), NVQ2J / NVQ2J-L / NVQ2J-XL (e8_256 / e8_1024 / e8_4096 with JSC state tables and up to four banks) -- and
+ * NVQ3J-L (d4_1024), whose 10-bit indices do not fit the lane-major D4 layout above.  Group size 24, 4-bit states.
+ * The device weight keeps the payload's three tensor-wide streams (4-bit state, index, 7-bit sign) as they are, with
+ * the tables widened in front (float lut[16], uint32 bank_for_state[16], int8 codebooks) and fp32 anchors; fields are
+ * fetched by bit offset, a wave per neuron.  Replaces the formats 2, 5, 13, 14 and 15 of unpack_nvq / NvqWeight
+ * (cpp_runtime/mfq_decode.cpp:3756-4013, 4019-4150) and their nvq_gemv_ws_cuda / nvq_mmq_* / nvq_dequant_cuda calls
+ * (:540-575, 7884-7931).
+ * ------------------------------------------------------------------------------------ */
+typedef struct mfq_nvqs_desc {
+    int32_t vector_size, index_bits, entries, banks, index_parity;
+    int32_t out, neuron_len, ng, nvec, nsign;
+    int64_t tables_off, anchors_off, state_off, index_off, sign_off;
+    int64_t total_bytes;
+    int64_t payload_bytes; /* anchors + the three streams */
+} mfq_nvqs_desc;
+
+int mfq_hip_nvqs_plan(int vector_size, int index_bits, int banks, int index_parity, int out, int neuron_len,
+                      mfq_nvqs_desc *d);
+/* `payload` = device copy of the blob from the 64-byte JSC header on (jsc != 0: header, int8 banks
+ * [banks, entries, vector_size], fp16 anchors, streams) or from the anchors on (jsc == 0; `grid` is then the device
+ * copy of the int8 magnitude grid [entries, vector_size], and the 4-bit state is the integer relative scale). */
+int mfq_hip_nvqs_repack(const mfq_nvqs_desc *d, const void *payload, int64_t payload_bytes, int jsc,
+                        const void *grid, void *weight, mfq_stream_t stream);
+/* Bit-exact twin of dequantize_nvq_jsc (mfq/quantize/nvq_jsc.py:1053-1079) and dequantize_nvq
+ * (mfq/quantize/nvq_quant.py:608-626), index-parity sign rule included. */
+int mfq_hip_nvqs_dequant_f32(const mfq_nvqs_desc *d, const void *weight, float *w_out, int64_t ld,
+                             mfq_stream_t stream);
+/* y = x . W^T: up to 16 rows re-read the streams once per eight rows (fp32 accumulation); above that the tensor is
+ * dequantized to fp16 in the workspace (size from the query, 0 up to 16 rows) and multiplied on the matrix cores. */
+int mfq_hip_nvqs_gemv(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                      int M, float *y, int64_t ldy, mfq_stream_t stream);
+size_t mfq_hip_nvqs_gemm_workspace_bytes(const mfq_nvqs_desc *d, int M);
+int mfq_hip_nvqs_gemm(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                      int M, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                      mfq_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
  * NEPQ1-S / NEPQ1-L (cross-expert table pool, bank id per 96 weights).  Rows are the
  * flattened [experts * out_per_expert] neurons.  Replaces NepqWeight
  * (cpp_runtime/mfq_decode.cpp:4166-4463) and the Python nepq_matmul

@@ -17,15 +17,29 @@ def nint_random(rng, out, K, bits, gs, sb):
 
 
 def nvq_jsc_random(rng, out, K, codebook="d4_512", banks=2):
-    grid = O.nvq_grid(codebook).astype(np.int16) * 8
+    """Random streams for a JSC tensor of any codebook: the built-in grids where the format has one, else random
+    magnitudes (the 1024- and 4096-entry codebooks travel in the payload anyway)."""
+    ib, vs = O._NVQ_INDEX_BITS[codebook], O.nvq_vector_size(codebook)
+    if codebook in ("e8_256", "d4_256", "d4_512"):
+        grid = O.nvq_grid(codebook).astype(np.int16) * 8
+    else:
+        grid = np.random.default_rng(ib * 100 + vs).integers(0, 128, (1 << ib, vs)).astype(np.int16)
     cbs = np.stack([np.roll(grid, b * 7, axis=0) for b in range(banks)]).astype(np.int8)
-    ib = O._NVQ_INDEX_BITS[codebook]
-    ng, nvec, nsign = math.ceil(K / 24), math.ceil(K / 4), math.ceil(K / 8)
+    ng, nvec, nsign = math.ceil(K / 24), math.ceil(K / vs), math.ceil(K / 8)
     return O.NvqJscTensor(codebook, (out, K), K, O._f16_round(rng.uniform(0.002, 0.02, out)),
                           O._f16_round(np.linspace(0.45, 1.55, 16)), (np.arange(16) % banks).astype(np.uint8),
                           rng.integers(0, 16, (out, ng), dtype=np.uint8),
                           rng.integers(0, 1 << ib, (out, nvec)).astype(np.uint16),
                           rng.integers(0, 128, (out, nsign), dtype=np.uint8), cbs)
+
+
+def nvq_plain_e8_random(rng, out, K, sign_mode="even"):
+    """Plain NVQ2: the built-in 256-entry E8 grid, integer relative scales, parity or index-parity signs."""
+    ng, nvec, nsign = math.ceil(K / 24), math.ceil(K / 8), math.ceil(K / 8)
+    return O.NvqTensor("e8_256", (out, K), K, O._f16_round(rng.uniform(0.0002, 0.002, out)),
+                       rng.integers(0, 16, (out, ng), dtype=np.uint8),
+                       rng.integers(0, 256, (out, nvec)).astype(np.uint16),
+                       rng.integers(0, 128, (out, nsign), dtype=np.uint8), sign_mode=sign_mode)
 
 
 def nvq_plain_random(rng, out, K):

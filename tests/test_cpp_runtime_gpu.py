@@ -57,6 +57,8 @@ def test_check_linear_tool_reports_small_error(tmp_path):
         "blk.0.q.nint3": synth.nint_random(rng, 37, 96, 3, 24, 5),
         "blk.0.ffn.nint4": O.quantize_nint((rng.standard_normal((64, 200)) * 0.02).astype(np.float32), 4, 32, 6),
         "blk.0.k.nvq3j512": synth.nvq_jsc_random(rng, 37, 96),
+        "blk.0.u.nvq2j": synth.nvq_jsc_random(rng, 37, 96, "e8_256", 2),           # E8: read from its bit streams in place
+        "blk.0.g.nvq3jl": synth.nvq_jsc_random(rng, 24, 104, "d4_1024", 4),
         "blk.0.v.nepq1s": synth.nepq_random(rng, "NEPQ1-S", 1, 48, 96, 3),
         "blk.0.o.nint8_0": O.quantize_nint8_zero((rng.standard_normal((40, 96)) * 0.02).astype(np.float32)),
     }

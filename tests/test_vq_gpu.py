@@ -313,3 +313,60 @@ def test_multi_expert_nepq_blob_is_not_a_linear():
     handle = ctypes.c_void_p()
     assert lib.mfq_rt_load_quant_linear(b"NEPQ1-S", blob, ctypes.c_size_t(len(blob)), ctypes.byref(handle)) != 0
     assert "must hold one expert" in lib.mfq_rt_last_error().decode()
+
+
+@pytest.mark.parametrize("codebook,banks,dtype", [("e8_256", 2, "NVQ2J"), ("e8_256", 4, "NVQ2J"), ("e8_1024", 2, "NVQ2J-L"),
+                                                  ("e8_4096", 1, "NVQ2J-XL"), ("e8_4096", 4, "NVQ2J-XL"),
+                                                  ("d4_1024", 2, "NVQ3J-L")])
+@pytest.mark.parametrize("out,K", [(37, 96), (24, 80), (70, 1544), (33, 100)])
+def test_nvq_stream_formats_dequant_bit_exact_and_matmul(codebook, banks, dtype, out, K):
+    """The E8 family and the 1024-entry D4 codebook, read in place from their bit streams (mfq_hip_nvqs_*): dequantized
+    weights bit for bit against the oracle (ragged K: partial last vector, sign block and group), the wave-per-neuron
+    kernel for 1 / 4 / 8 / 13 rows of both activation types, and the fp16 GEMM path above 16 rows."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import NvqsWeight, nvq_matmul
+    rng = np.random.default_rng(900 + out + K + banks)
+    t = synth.nvq_jsc_random(rng, out, K, codebook, banks)
+    got_dtype, blob = O.pack_tensor(t)
+    assert got_dtype == dtype
+    lin = R.load_quant_linear(dtype, blob)
+    assert isinstance(lin.weight, NvqsWeight) and lin.weight.payload_bytes == O.nvq_payload_nbytes(codebook, out, K)
+    want = O.dequantize_nvq_jsc(O.unpack_nvq(blob))
+    got = lin.dequantize().cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    for M in (1, 4, 8, 13):
+        for xd in (torch.bfloat16, torch.float16):
+            x, xf = _x(rng, M, K, xd)
+            _check(nvq_matmul(lin.weight, x).cpu().numpy(), O.linear_forward_f64(want, xf))
+    for M in (17, 70):
+        x, xf = _x(rng, M, K)
+        _check(lin(x).cpu().numpy(), O.linear_forward_f64(want, xf))
+    xs = torch.zeros((1, K + 3), dtype=torch.bfloat16, device="cuda")[:, 1:K + 1]       # a misaligned row
+    xs.copy_(torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)))
+    _check(nvq_matmul(lin.weight, xs).cpu().numpy(), O.linear_forward_f64(want, xs.float().cpu().numpy()))
+
+
+@pytest.mark.parametrize("sign_mode", ["even", "index_parity"])
+def test_nvq2_plain_e8_with_both_sign_rules(sign_mode):
+    """Plain NVQ2 (built-in E8 grid, the state is the integer relative scale): parity signs and the index-parity rule
+    (bit 7 of a block flips with bit 7 of its vector's index); and the reference-packed index-parity blob of the golden
+    fixture against the values the reference dequantized it to."""
+    from pathlib import Path
+
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(31)
+    t = synth.nvq_plain_e8_random(rng, 40, 200, sign_mode)
+    dtype, blob = O.pack_tensor(t)
+    assert dtype == "NVQ2"
+    lin = R.load_quant_linear("NIQ2", blob)           # the legacy alias
+    want = O.dequantize_nvq(O.unpack_nvq(blob))
+    assert np.array_equal(lin.dequantize().cpu().numpy().view(np.uint32), want.view(np.uint32))
+    for M in (1, 5, 40):
+        x, xf = _x(rng, M, 200)
+        _check(lin(x).cpu().numpy(), O.linear_forward_f64(want, xf))
+    gold = np.load(Path(__file__).resolve().parent / "golden" / "reference_blobs.npz")
+    ref_blob, ref_w = gold["nvq2ip_blob"].tobytes(), gold["nvq2ip_deq"]
+    lin = R.load_quant_linear("NVQ2", ref_blob)
+    assert np.array_equal(lin.dequantize().cpu().numpy().view(np.uint32), ref_w.astype(np.float32).view(np.uint32))
+    with pytest.raises(ValueError, match="dtype/blob mismatch"):
+        R.load_quant_linear("NVQ2J", ref_blob)

@@ -32,6 +32,13 @@ class NvqDesc(C.Structure):
                                    "payload_bytes")]
 
 
+class NvqsDesc(C.Structure):
+    _fields_ = [(n, i32) for n in ("vector_size", "index_bits", "entries", "banks", "index_parity", "out", "neuron_len",
+                                   "ng", "nvec", "nsign")] + \
+               [(n, i64) for n in ("tables_off", "anchors_off", "state_off", "index_off", "sign_off", "total_bytes",
+                                   "payload_bytes")]
+
+
 class NepqDesc(C.Structure):
     _fields_ = [(n, i32) for n in ("profile", "state_bits", "index_bits", "banks", "rows", "neuron_len", "ng", "nvec",
                                    "nsuper", "ngp", "nsteps", "n_rowblocks", "table_entries")] + \
@@ -91,6 +98,12 @@ _SIGS = {
     "mfq_hip_nvq_gemv_multi2": (C.c_int, [C.POINTER(NvqDesc), vp, C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
     "mfq_hip_nvq_gemm_workspace_bytes": (sz, [C.POINTER(NvqDesc), C.c_int]),
     "mfq_hip_nvq_gemm": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
+    "mfq_hip_nvqs_plan": (C.c_int, [C.c_int] * 6 + [C.POINTER(NvqsDesc)]),
+    "mfq_hip_nvqs_repack": (C.c_int, [C.POINTER(NvqsDesc), vp, i64, C.c_int, vp, vp, vp]),
+    "mfq_hip_nvqs_dequant_f32": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, i64, vp]),
+    "mfq_hip_nvqs_gemv": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
+    "mfq_hip_nvqs_gemm_workspace_bytes": (sz, [C.POINTER(NvqsDesc), C.c_int]),
+    "mfq_hip_nvqs_gemm": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
     "mfq_hip_nepq_plan": (C.c_int, [C.c_int] * 4 + [C.POINTER(NepqDesc)]),
     "mfq_hip_nepq_repack": (C.c_int, [C.POINTER(NepqDesc), vp, i64, vp, vp]),
     "mfq_hip_nepq_dequant_f32": (C.c_int, [C.POINTER(NepqDesc), vp, vp, i64, vp]),

@@ -279,10 +279,23 @@ Nint8ZeroWeight Nint8ZeroWeight::from_blob(const uint8_t *blob, size_t n, mfq_st
 
 NvqWeight NvqWeight::from_blob(const uint8_t *blob, size_t n, const int8_t *grid256, mfq_stream_t stream) {
     const NvqHeader h = parse_nvq(blob, n);
-    if (h.vector_size != 4 || h.index_bits > 9)
-        fail(h.dtype + ": only the D4 256/512-entry NVQ formats are on the accelerated path");
     NvqWeight w;
     w.dtype = h.dtype;
+    if (h.vector_size != 4 || h.index_bits > 9) {  // E8 family, d4_1024: the streams are read in place
+        if (h.gs != 24 || h.sub_bits != 4) fail(h.dtype + ": NVQ runs only with gs24 and 4-bit states");
+        if (!h.jsc && !grid256) fail("plain NVQ2 needs the 256-entry E8 magnitude grid");
+        w.streams = true;
+        abi_check(mfq_hip_nvqs_plan(h.vector_size, h.index_bits, h.jsc ? h.banks : 1, h.index_parity ? 1 : 0, h.out,
+                                    h.neuron_len, &w.sdesc));
+        DeviceBuffer payload = DeviceBuffer::from_host(blob + h.body_off, h.body_bytes);
+        DeviceBuffer grid;
+        if (!h.jsc) grid = DeviceBuffer::from_host(grid256, 256ull * h.vector_size);
+        w.data = DeviceBuffer(static_cast<size_t>(w.sdesc.total_bytes));
+        abi_check(mfq_hip_nvqs_repack(&w.sdesc, payload.get(), static_cast<int64_t>(h.body_bytes), h.jsc ? 1 : 0, grid.get(),
+                                      w.data.get(), stream));
+        hip_check(hipStreamSynchronize(hs(stream)), "nvq repack");
+        return w;
+    }
     abi_check(mfq_hip_nvq_plan(h.index_bits, h.jsc ? h.banks : 1, h.out, h.neuron_len, &w.desc));
     DeviceBuffer payload = DeviceBuffer::from_host(blob + h.body_off, h.body_bytes);
     w.data = DeviceBuffer(static_cast<size_t>(w.desc.total_bytes));
@@ -367,14 +380,31 @@ void nint_matmul_argmax(const NintWeight &w, const void *x, int x_dtype, int64_t
                                        w.workspace.get(), need, stream));
 }
 void nvq_matmul(const NvqWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) {
+    if (w.streams) {
+        const size_t need = mfq_hip_nvqs_gemm_workspace_bytes(&w.sdesc, M);
+        w.workspace.ensure(need);
+        abi_check(mfq_hip_nvqs_gemm(&w.sdesc, w.data.get(), x, x_dtype, ldx, M, y, w.sdesc.out, w.workspace.get(), need, stream));
+        return;
+    }
     const size_t need = mfq_hip_nvq_gemm_workspace_bytes(&w.desc, M);
     w.workspace.ensure(need);
     abi_check(mfq_hip_nvq_gemm(&w.desc, w.data.get(), x, x_dtype, ldx, M, y, w.desc.out, w.workspace.get(), need, stream));
 }
 void nvq_matmul_multi2(const NvqWeight &first, const NvqWeight &second, const void *x, int x_dtype, int64_t ldx, int M,
                        float *y, mfq_stream_t stream) {
-    if (first.desc.neuron_len != second.desc.neuron_len) fail("NVQ multi-projection requires compatible formats and input layouts");
-    const int64_t N = static_cast<int64_t>(first.desc.out) + second.desc.out;
+    if (first.neuron_len() != second.neuron_len()) fail("NVQ multi-projection requires compatible formats and input layouts");
+    const int64_t N = first.out() + second.out();
+    if (first.streams || second.streams) {  // no joint launch for tensors read from their streams: each into its columns
+        DeviceBuffer tmp(static_cast<size_t>(M) * static_cast<size_t>(std::max(first.out(), second.out())) * 4);
+        for (const NvqWeight *w : {&first, &second}) {
+            nvq_matmul(*w, x, x_dtype, ldx, M, static_cast<float *>(tmp.get()), stream);
+            hip_check(hipMemcpy2DAsync(y + (w == &second ? first.out() : 0), static_cast<size_t>(N) * 4, tmp.get(),
+                                       static_cast<size_t>(w->out()) * 4, static_cast<size_t>(w->out()) * 4, M,
+                                       hipMemcpyDeviceToDevice, hs(stream)), "nvq_matmul_multi2");
+        }
+        hip_check(hipStreamSynchronize(hs(stream)), "nvq_matmul_multi2");
+        return;
+    }
     if (M <= 32) {
         abi_check(mfq_hip_nvq_gemv_multi2(&first.desc, first.data.get(), &second.desc, second.data.get(), x, x_dtype, ldx, M, y, N,
                                           stream));
@@ -390,20 +420,20 @@ void nvq_matmul_multi2(const NvqWeight &first, const NvqWeight &second, const vo
 }
 void nvq_matmul_swiglu(const NvqWeight &gate, const NvqWeight &up, const void *x, int x_dtype, int64_t ldx, int M, void *hidden,
                        float *scratch, mfq_stream_t stream) {
-    if (gate.desc.neuron_len != up.desc.neuron_len || gate.desc.out != up.desc.out)
+    if (gate.neuron_len() != up.neuron_len() || gate.out() != up.out())
         fail("NVQ SwiGLU requires compatible equal-width gate/up weights");
     if (!scratch) fail("nvq_matmul_swiglu: needs a [M, 2W] fp32 scratch buffer");
-    const int W = gate.desc.out;
+    const int W = static_cast<int>(gate.out());
     nvq_matmul_multi2(gate, up, x, x_dtype, ldx, M, scratch, stream);
     abi_check(mfq_hip_moe_swiglu(scratch, 2 * W, M, W, hidden, MFQ_X_F16, W, stream));
 }
 void nvq_ffn_swiglu_down(const NvqWeight &gate, const NvqWeight &up, const NvqWeight &down, const void *x, int x_dtype,
                          int64_t ldx, int M, float *y, void *hidden, float *scratch, mfq_stream_t stream) {
-    if (gate.desc.neuron_len != up.desc.neuron_len || gate.desc.out != up.desc.out || gate.desc.out != down.desc.neuron_len)
+    if (gate.neuron_len() != up.neuron_len() || gate.out() != up.out() || gate.out() != down.neuron_len())
         fail("NVQ fused FFN weight layouts are incompatible");
     if (!hidden) fail("nvq_ffn_swiglu_down: needs a [M, W] fp16 buffer for the hidden rows");
     nvq_matmul_swiglu(gate, up, x, x_dtype, ldx, M, hidden, scratch, stream);
-    nvq_matmul(down, hidden, MFQ_X_F16, gate.desc.out, M, y, stream);
+    nvq_matmul(down, hidden, MFQ_X_F16, gate.out(), M, y, stream);
 }
 void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                  mfq_stream_t stream) {
@@ -433,6 +463,10 @@ void nint8_zero_dequantize(const Nint8ZeroWeight &w, float *out, mfq_stream_t st
     abi_check(mfq_hip_nint8z_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
 }
 void nvq_dequantize(const NvqWeight &w, float *out, mfq_stream_t stream) {
+    if (w.streams) {
+        abi_check(mfq_hip_nvqs_dequant_f32(&w.sdesc, w.data.get(), out, w.sdesc.neuron_len, stream));
+        return;
+    }
     abi_check(mfq_hip_nvq_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
 }
 void nepq_dequantize(const NepqWeight &w, float *out, mfq_stream_t stream) {
@@ -444,7 +478,10 @@ bool is_nint_linear_dtype(const std::string &d) {
     if (d.size() <= 4 || d.compare(0, 4, "NINT") != 0) return false;
     return std::all_of(d.begin() + 4, d.end(), [](char c) { return c >= '0' && c <= '9'; });
 }
-bool is_nvq_linear_dtype(const std::string &d) { return d == "NVQ3" || d == "NVQ3J" || d == "NVQ3J-512" || d == "NIQ3"; }
+bool is_nvq_linear_dtype(const std::string &d) {
+    return d == "NVQ3" || d == "NVQ3J" || d == "NVQ3J-512" || d == "NVQ3J-L" || d == "NVQ2" || d == "NVQ2J" || d == "NVQ2J-L" ||
+           d == "NVQ2J-XL" || d == "NIQ3" || d == "NIQ2" || d == "NIQ2J";
+}
 bool is_nepq_linear_dtype(const std::string &d) { return d == "NEPQ1-S" || d == "NEPQ1-L"; }
 
 int64_t QuantLinear::out() const {
@@ -456,7 +493,7 @@ int64_t QuantLinear::neuron_len() const {
          : kind == QuantLinearKind::Nepq ? nepq->neuron_len() : nint8z->neuron_len();
 }
 int64_t QuantLinear::payload_bytes() const {
-    return kind == QuantLinearKind::Nint ? nint->desc.payload_bytes : kind == QuantLinearKind::Nvq ? nvq->desc.payload_bytes
+    return kind == QuantLinearKind::Nint ? nint->desc.payload_bytes : kind == QuantLinearKind::Nvq ? nvq->payload_bytes()
          : kind == QuantLinearKind::Nepq ? nepq->desc.payload_bytes : nint8z->desc.payload_bytes;
 }
 void QuantLinear::forward(const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const {
@@ -474,7 +511,7 @@ void QuantLinear::dequantize(float *out, mfq_stream_t stream) const {
 }
 
 QuantLinear load_quant_linear(const std::string &dtype_in, const uint8_t *blob, size_t n, mfq_stream_t stream) {
-    const std::string dtype = dtype_in == "NIQ3" ? "NVQ3" : dtype_in;
+    const std::string dtype = dtype_in == "NIQ3" ? "NVQ3" : dtype_in == "NIQ2" ? "NVQ2" : dtype_in == "NIQ2J" ? "NVQ2J" : dtype_in;
     QuantLinear q;
     if (is_nint_linear_dtype(dtype)) {
         q.kind = QuantLinearKind::Nint;
@@ -1148,7 +1185,7 @@ LinearCheckResult run_linear_check(const QuantLinear &lin, int M, int reps) {
     res.production_ms = ms / reps;
     res.payload_bytes = lin.payload_bytes();
     res.weight_bytes = lin.kind == QuantLinearKind::Nint ? lin.nint->desc.total_bytes
-                     : lin.kind == QuantLinearKind::Nvq ? lin.nvq->desc.total_bytes
+                     : lin.kind == QuantLinearKind::Nvq ? lin.nvq->total_bytes()
                      : lin.kind == QuantLinearKind::Nepq ? lin.nepq->desc.total_bytes : lin.nint8z->desc.total_bytes;
     res.production_weight_gbps = res.weight_bytes / (res.production_ms * 1e6);
     res.payload_gbps = res.payload_bytes / (res.production_ms * 1e6);

@@ -106,13 +106,18 @@ struct Nint8ZeroWeight {
     static Nint8ZeroWeight from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream = nullptr);
 };
 struct NvqWeight {
-    mfq_nvq_desc desc{};
+    mfq_nvq_desc desc{};     // lane-major D4 layout (d4_256, d4_512)
+    mfq_nvqs_desc sdesc{};   // streams read in place (E8 family, d4_1024): `streams` set
+    bool streams = false;
     DeviceBuffer data;
     std::string dtype;
     mutable DeviceBuffer workspace;
-    int64_t out() const { return desc.out; }
-    int64_t neuron_len() const { return desc.neuron_len; }
-    // `grid256` = the 256-entry int8 D4 magnitude grid [256,4], needed only by plain (non-JSC) NVQ3
+    int64_t out() const { return streams ? sdesc.out : desc.out; }
+    int64_t neuron_len() const { return streams ? sdesc.neuron_len : desc.neuron_len; }
+    int64_t payload_bytes() const { return streams ? sdesc.payload_bytes : desc.payload_bytes; }
+    int64_t total_bytes() const { return streams ? sdesc.total_bytes : desc.total_bytes; }
+    // `grid256` = the built-in 256-entry int8 magnitude grid of a plain (non-JSC) tensor: [256,4] for NVQ3, [256,8] for
+    // NVQ2; JSC tensors carry their codebooks
     static NvqWeight from_blob(const uint8_t *blob, size_t n, const int8_t *grid256 = nullptr,
                                mfq_stream_t stream = nullptr);
 };

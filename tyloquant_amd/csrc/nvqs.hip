@@ -1,0 +1,343 @@
+// NVQ payloads read in place from their tensor-wide bit streams: the E8 family (8-dimensional vectors, 256 / 1024 /
+// 4096 entries, plain or JSC, parity or index-parity signs) and the 1024-entry D4 codebook, which the 16-bit fields
+// of the lane-major D4 layout (nvq.hip) cannot hold.  The device weight is the payload itself with its tables
+// widened: no re-layout, every field is fetched by bit offset.  A wave owns a neuron, its lanes the 8-weight sign
+// blocks of the row, so the three streams of a neuron are read as consecutive bytes.
+#include "common.hpp"
+#include "gemv_common.hpp"
+#include "tune.hpp"
+
+namespace mfq {
+
+struct NvqsK {
+    int vs, ib, entries, banks, index_parity;
+    int out, neuron_len, ng, nvec, nsign;
+    int64_t tables_off, anchors_off, state_off, index_off, sign_off;
+    int64_t state_bytes, index_bytes, sign_bytes;
+};
+
+static NvqsK to_k(const mfq_nvqs_desc *d) {
+    NvqsK k;
+    k.vs = d->vector_size; k.ib = d->index_bits; k.entries = d->entries; k.banks = d->banks; k.index_parity = d->index_parity;
+    k.out = d->out; k.neuron_len = d->neuron_len; k.ng = d->ng; k.nvec = d->nvec; k.nsign = d->nsign;
+    k.tables_off = d->tables_off; k.anchors_off = d->anchors_off; k.state_off = d->state_off; k.index_off = d->index_off;
+    k.sign_off = d->sign_off;
+    k.state_bytes = (static_cast<int64_t>(d->out) * d->ng * 4 + 7) / 8;
+    k.index_bytes = (static_cast<int64_t>(d->out) * d->nvec * d->index_bits + 7) / 8;
+    k.sign_bytes = (static_cast<int64_t>(d->out) * d->nsign * 7 + 7) / 8;
+    return k;
+}
+
+// tables: float lut[16] | uint32 bank_for_state[16] | int8 codebooks[banks * entries * vs]
+__device__ __forceinline__ const float *nvqs_lut(const NvqsK &k, const uint8_t *w) {
+    return reinterpret_cast<const float *>(w + k.tables_off);
+}
+
+// Field of `bits` (<= 12) bits at bit position `bit` of a stream that is followed by at least three readable bytes.
+__device__ __forceinline__ uint32_t stream_bits(const uint8_t *s, int64_t bit, int bits) {
+    const int64_t b = bit >> 3;
+    const uint32_t v = s[b] | (static_cast<uint32_t>(s[b + 1]) << 8) | (static_cast<uint32_t>(s[b + 2]) << 16);
+    return (v >> (bit & 7)) & ((1u << bits) - 1u);
+}
+
+// The eight weights of sign block sb of neuron n, as signed integer magnitudes, and the scale of their group:
+// w[i] = f32(mag[i]) * fl(anchor * lut[state])  (mfq/quantize/nvq_jsc.py:1053-1079; the plain formats are the case
+// lut[s] = s, one bank: mfq/quantize/nvq_quant.py:608-626).  Sign bit 7 of a block is the parity of its seven stored
+// bits, flipped by bit 7 of the vector's index in the index-parity mode (E8 only).
+struct NvqsBlock {
+    float mag[8];
+    float scale;
+};
+template <class CB>
+__device__ __forceinline__ NvqsBlock nvqs_block(const NvqsK &k, const uint8_t *w, const float *lut, const uint32_t *bfs,
+                                                CB cb, float anchor, int n, int sb) {
+    const uint8_t *st_s = w + k.state_off, *ix_s = w + k.index_off, *sg_s = w + k.sign_off;
+    const uint32_t mask = stream_bits(sg_s, (static_cast<int64_t>(n) * k.nsign + sb) * 7, 7);
+    const int g = sb / 3;  // groups of 24 weights = three sign blocks
+    const uint32_t state = stream_bits(st_s, (static_cast<int64_t>(n) * k.ng + g) * 4, 4);
+    const uint32_t bank = bfs[state];
+    NvqsBlock b;
+    b.scale = __fmul_rn(anchor, lut[state]);
+    uint32_t last = __popc(mask) & 1u;
+    if (k.vs == 8) {
+        const uint32_t idx = stream_bits(ix_s, (static_cast<int64_t>(n) * k.nvec + sb) * k.ib, k.ib);
+        if (k.index_parity) last ^= (idx >> 7) & 1u;
+        const int64_t e = (static_cast<int64_t>(bank) * k.entries + idx) * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) b.mag[i] = static_cast<float>(cb(e + i));
+    } else {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int v = 2 * sb + h;
+            const uint32_t idx = v < k.nvec ? stream_bits(ix_s, (static_cast<int64_t>(n) * k.nvec + v) * k.ib, k.ib) : 0u;
+            const int64_t e = (static_cast<int64_t>(bank) * k.entries + idx) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b.mag[4 * h + i] = static_cast<float>(cb(e + i));
+        }
+    }
+    const uint32_t neg = mask | (last << 7);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        if ((neg >> i) & 1u) b.mag[i] = -b.mag[i];
+    return b;
+}
+
+// ---- load: widen the tables, copy the streams ------------------------------------------------------------------
+// body: JSC = 64-byte header (fp16 lut at +4, u8 bank map at +36), int8 banks, then the plain layout; plain =
+// fp16 anchors, 4-bit state / sub-scale stream, index stream, 7-bit sign stream.
+__global__ __launch_bounds__(256) void nvqs_repack_kernel(NvqsK k, const uint8_t *__restrict__ body, int jsc,
+                                                          const int8_t *__restrict__ grid, uint8_t *__restrict__ dst) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x, nthreads = static_cast<int64_t>(gridDim.x) * 256;
+    float *lut = reinterpret_cast<float *>(dst + k.tables_off);
+    uint32_t *bfs = reinterpret_cast<uint32_t *>(lut + 16);
+    int8_t *cb = reinterpret_cast<int8_t *>(bfs + 16);
+    const int64_t ncb = static_cast<int64_t>(k.banks) * k.entries * k.vs;
+    const uint8_t *streams = body + (jsc ? 64 + ncb : 0);
+    if (tid < 16) {
+        if (jsc) {
+            lut[tid] = f16_to_f32(static_cast<uint16_t>(body[4 + 2 * tid] | (body[5 + 2 * tid] << 8)));
+            bfs[tid] = body[36 + tid];
+        } else {
+            lut[tid] = static_cast<float>(tid);  // the state is the integer relative scale
+            bfs[tid] = 0u;
+        }
+    }
+    for (int64_t i = tid; i < ncb; i += nthreads) cb[i] = jsc ? static_cast<int8_t>(body[64 + i]) : grid[i];
+    float *anchors = reinterpret_cast<float *>(dst + k.anchors_off);
+    for (int64_t i = tid; i < k.out; i += nthreads)
+        anchors[i] = f16_to_f32(static_cast<uint16_t>(streams[2 * i] | (streams[2 * i + 1] << 8)));
+    const uint8_t *st = streams + 2 * static_cast<int64_t>(k.out), *ix = st + k.state_bytes, *sg = ix + k.index_bytes;
+    for (int64_t i = tid; i < k.state_bytes + 4; i += nthreads) dst[k.state_off + i] = i < k.state_bytes ? st[i] : 0;
+    for (int64_t i = tid; i < k.index_bytes + 4; i += nthreads) dst[k.index_off + i] = i < k.index_bytes ? ix[i] : 0;
+    for (int64_t i = tid; i < k.sign_bytes + 4; i += nthreads) dst[k.sign_off + i] = i < k.sign_bytes ? sg[i] : 0;
+}
+
+// ---- dequant -------------------------------------------------------------------------------------------------------
+// One thread per (neuron, sign block).  OutT = float: the bit-exact dequantizer.  OutT = uint16_t: fp16 rows scaled by a
+// power of two per neuron (rowscale receives its reciprocal), zero-padded to kpad columns, for the fp16 GEMM.
+template <typename OutT>
+__global__ __launch_bounds__(256) void nvqs_dequant_kernel(NvqsK k, const uint8_t *__restrict__ w, OutT *__restrict__ outp,
+                                                           int64_t ld, float *__restrict__ rowscale, int kpad) {
+    const int n = blockIdx.y;
+    const float *lut = nvqs_lut(k, w);
+    const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+    const int8_t *cbp = reinterpret_cast<const int8_t *>(bfs + 16);
+    const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[n];
+    float inv = 1.f;
+    if constexpr (sizeof(OutT) == 2) {
+        float lmax = 0.f;
+        for (int i = 0; i < 16; ++i) lmax = fmaxf(lmax, lut[i]);
+        const float bound = anchor * lmax * 127.f;
+        int e = 0;
+        if (bound > 0.f) frexpf(bound, &e);
+        inv = ldexpf(1.f, 12 - e);
+        if (blockIdx.x == 0 && threadIdx.x == 0) rowscale[n] = ldexpf(1.f, e - 12);
+        for (int col = k.nsign * 8 + blockIdx.x * 256 + threadIdx.x; col < kpad; col += gridDim.x * 256) outp[n * ld + col] = 0;
+    }
+    const int sb = blockIdx.x * 256 + threadIdx.x;
+    if (sb >= k.nsign) return;
+    const NvqsBlock b = nvqs_block(k, w, lut, bfs, [&](int64_t i) { return cbp[i]; }, anchor, n, sb);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int col = sb * 8 + i;
+        const float v = __fmul_rn(b.mag[i], b.scale);
+        if constexpr (sizeof(OutT) == 2) {
+            if (col < kpad) outp[n * ld + col] = col < k.neuron_len ? f32_to_f16_rne(v * inv) : uint16_t(0);
+        } else {
+            if (col < k.neuron_len) outp[n * ld + col] = v;
+        }
+    }
+}
+
+// ---- GEMV: a wave per neuron, MB rows per pass --------------------------------------------------------------------
+// LDS (CB_LDS): the int8 codebooks.  The activation rows are read as 16-byte chunks straight from global memory (they
+// stay in L2: every wave of the grid reads the same rows).
+template <int XF16, int MB, bool CB_LDS>
+__global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *__restrict__ w,
+                                                        const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                        float *__restrict__ y, int64_t ldy) {
+    extern __shared__ __attribute__((aligned(16))) int8_t cbl[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float *lut = nvqs_lut(k, w);
+    const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+    const int8_t *cbp = reinterpret_cast<const int8_t *>(bfs + 16);
+    if constexpr (CB_LDS) {
+        const int ncb = k.banks * k.entries * k.vs;
+        for (int i = threadIdx.x * 4; i < ncb; i += blockDim.x * 4)
+            *reinterpret_cast<uint32_t *>(cbl + i) = *reinterpret_cast<const uint32_t *>(cbp + i);
+        __syncthreads();
+    }
+    const int n = blockIdx.x * (blockDim.x >> 6) + wave;
+    if (n >= k.out) return;
+    const int m0 = blockIdx.y * MB;
+    const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[n];
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = 0.f;
+    const bool vec = ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    for (int sb = lane; sb < k.nsign; sb += 64) {
+        NvqsBlock b;
+        if constexpr (CB_LDS) b = nvqs_block(k, w, lut, bfs, [&](int64_t i) { return cbl[i]; }, anchor, n, sb);
+        else b = nvqs_block(k, w, lut, bfs, [&](int64_t i) { return cbp[i]; }, anchor, n, sb);
+        float wv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) wv[i] = sb * 8 + i < k.neuron_len ? __fmul_rn(b.mag[i], b.scale) : 0.f;
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            if (m0 + m >= M) break;
+            const uint16_t *xr = x + static_cast<int64_t>(m0 + m) * ldx + sb * 8;
+            uint16_t xv[8];
+            if (vec && sb * 8 + 8 <= k.neuron_len) {
+                const u32x4_t q = *reinterpret_cast<const u32x4_t *>(xr);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    xv[2 * t] = static_cast<uint16_t>(q[t] & 0xffffu);
+                    xv[2 * t + 1] = static_cast<uint16_t>(q[t] >> 16);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xv[i] = sb * 8 + i < k.neuron_len ? xr[i] : uint16_t(0);
+            }
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s = fmaf(wv[i], x_to_f32<XF16>(xv[i]), s);
+            acc[m] += s;
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        float s = acc[m];
+        for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+        if (lane == 0 && m0 + m < M) y[static_cast<int64_t>(m0 + m) * ldy + n] = s;
+    }
+}
+
+int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, const float *sa,
+                const float *sb, float *y, int64_t ldy, hipStream_t st);
+int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, hipStream_t st);
+size_t dequant_gemm_workspace(int N, int K, int M);
+void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&xscale, uint16_t *&w16, float *&wscale,
+                        int &Kp);
+
+constexpr int kNvqsGemvMaxM = 16;  // rows up to which the weights are re-read per pass of eight rows
+
+template <int XF16, int MB>
+static int nvqs_launch_gemv(const NvqsK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                            hipStream_t st) {
+    const size_t ncb = static_cast<size_t>(k.banks) * k.entries * k.vs;
+    const dim3 grid(static_cast<unsigned>(ceil_div(k.out, 4)), static_cast<unsigned>(ceil_div(M, MB)));
+    if (ncb <= 49152 && ncb % 4 == 0)
+        hipLaunchKernelGGL((nvqs_gemv_kernel<XF16, MB, true>), grid, dim3(256), ncb, st, k, w, x, ldx, M, y, ldy);
+    else
+        hipLaunchKernelGGL((nvqs_gemv_kernel<XF16, MB, false>), grid, dim3(256), 0, st, k, w, x, ldx, M, y, ldy);
+    return check_launch("nvqs_gemv");
+}
+
+}  // namespace mfq
+
+using namespace mfq;
+
+static size_t nvqs_align(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+
+extern "C" int mfq_hip_nvqs_plan(int vector_size, int index_bits, int banks, int index_parity, int out, int neuron_len,
+                                 mfq_nvqs_desc *d) {
+    MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nvqs_plan: null descriptor");
+    MFQ_REQUIRE(vector_size == 4 || vector_size == 8, MFQ_ERR_INVALID, "nvqs_plan: vector_size=%d", vector_size);
+    MFQ_REQUIRE(index_bits >= 8 && index_bits <= 12, MFQ_ERR_UNSUPPORTED, "nvqs_plan: index_bits=%d", index_bits);
+    MFQ_REQUIRE(banks == 1 || banks == 2 || banks == 4, MFQ_ERR_INVALID, "nvqs_plan: banks=%d", banks);
+    MFQ_REQUIRE(!index_parity || (vector_size == 8 && index_bits == 8), MFQ_ERR_INVALID,
+                "nvqs_plan: index-parity signs need the 256-entry 8-dimensional codebook");
+    MFQ_REQUIRE(out > 0 && neuron_len > 0, MFQ_ERR_INVALID, "nvqs_plan: empty tensor");
+    d->vector_size = vector_size; d->index_bits = index_bits; d->entries = 1 << index_bits; d->banks = banks;
+    d->index_parity = index_parity ? 1 : 0; d->out = out; d->neuron_len = neuron_len;
+    d->ng = static_cast<int32_t>(ceil_div(neuron_len, 24));
+    d->nvec = static_cast<int32_t>(ceil_div(neuron_len, vector_size));
+    d->nsign = static_cast<int32_t>(ceil_div(neuron_len, 8));
+    const int64_t ncb = static_cast<int64_t>(banks) * d->entries * vector_size;
+    const int64_t st = (static_cast<int64_t>(out) * d->ng * 4 + 7) / 8, ix = (static_cast<int64_t>(out) * d->nvec * index_bits + 7) / 8,
+                  sg = (static_cast<int64_t>(out) * d->nsign * 7 + 7) / 8;
+    d->tables_off = 0;
+    d->anchors_off = static_cast<int64_t>(nvqs_align(128 + static_cast<size_t>(ncb)));
+    d->state_off = d->anchors_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(out) * 4));
+    d->index_off = d->state_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(st) + 4));
+    d->sign_off = d->index_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(ix) + 4));
+    d->total_bytes = d->sign_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(sg) + 4));
+    d->payload_bytes = 2ll * out + st + ix + sg;
+    return MFQ_OK;
+}
+
+extern "C" int mfq_hip_nvqs_repack(const mfq_nvqs_desc *d, const void *payload, int64_t payload_bytes, int jsc,
+                                   const void *grid, void *weight, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && payload && weight, MFQ_ERR_INVALID, "nvqs_repack: null argument");
+    MFQ_REQUIRE(jsc || grid, MFQ_ERR_INVALID, "nvqs_repack: a plain payload needs its magnitude grid");
+    MFQ_REQUIRE(jsc || d->banks == 1, MFQ_ERR_INVALID, "nvqs_repack: a plain payload has one bank");
+    const int64_t ncb = static_cast<int64_t>(d->banks) * d->entries * d->vector_size;
+    const int64_t expect = d->payload_bytes + (jsc ? 64 + ncb : 0);
+    MFQ_REQUIRE(payload_bytes == expect, MFQ_ERR_INVALID, "nvqs_repack: payload is %lld bytes, the tensor needs %lld",
+                static_cast<long long>(payload_bytes), static_cast<long long>(expect));
+    const NvqsK k = to_k(d);
+    hipLaunchKernelGGL(nvqs_repack_kernel, dim3(1024), dim3(256), 0, as_stream(stream), k, static_cast<const uint8_t *>(payload),
+                       jsc, static_cast<const int8_t *>(grid), static_cast<uint8_t *>(weight));
+    return check_launch("nvqs_repack");
+}
+
+extern "C" int mfq_hip_nvqs_dequant_f32(const mfq_nvqs_desc *d, const void *weight, float *w_out, int64_t ld,
+                                        mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && w_out, MFQ_ERR_INVALID, "nvqs_dequant_f32: null argument");
+    MFQ_REQUIRE(ld >= d->neuron_len, MFQ_ERR_INVALID, "nvqs_dequant_f32: ld smaller than neuron_len");
+    MFQ_REQUIRE(d->out <= 65535, MFQ_ERR_UNSUPPORTED, "nvqs_dequant_f32: %d neurons in one call (max 65535)", d->out);
+    const NvqsK k = to_k(d);
+    hipLaunchKernelGGL((nvqs_dequant_kernel<float>), dim3(static_cast<unsigned>(ceil_div(k.nsign, 256)), k.out), dim3(256), 0,
+                       as_stream(stream), k, static_cast<const uint8_t *>(weight), w_out, ld, static_cast<float *>(nullptr), 0);
+    return check_launch("nvqs_dequant_f32");
+}
+
+extern "C" int mfq_hip_nvqs_gemv(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
+                                 float *y, int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nvqs_gemv: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nvqs_gemv: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvqs_gemv: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nvqs_gemv: ldx/ldy smaller than the tensor");
+    const NvqsK k = to_k(d);
+    const uint8_t *w = static_cast<const uint8_t *>(weight);
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    hipStream_t st = as_stream(stream);
+    if (x_dtype == MFQ_X_F16) {
+        if (M == 1) return nvqs_launch_gemv<1, 1>(k, w, xp, ldx, M, y, ldy, st);
+        if (M <= 4) return nvqs_launch_gemv<1, 4>(k, w, xp, ldx, M, y, ldy, st);
+        return nvqs_launch_gemv<1, 8>(k, w, xp, ldx, M, y, ldy, st);
+    }
+    if (M == 1) return nvqs_launch_gemv<0, 1>(k, w, xp, ldx, M, y, ldy, st);
+    if (M <= 4) return nvqs_launch_gemv<0, 4>(k, w, xp, ldx, M, y, ldy, st);
+    return nvqs_launch_gemv<0, 8>(k, w, xp, ldx, M, y, ldy, st);
+}
+
+extern "C" size_t mfq_hip_nvqs_gemm_workspace_bytes(const mfq_nvqs_desc *d, int M) {
+    if (!d || M <= kNvqsGemvMaxM) return 0;
+    return dequant_gemm_workspace(d->out, d->neuron_len, M);
+}
+
+extern "C" int mfq_hip_nvqs_gemm(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
+                                 float *y, int64_t ldy, void *workspace, size_t workspace_bytes, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nvqs_gemm: null argument");
+    if (M <= kNvqsGemvMaxM) return mfq_hip_nvqs_gemv(d, weight, x, x_dtype, ldx, M, y, ldy, stream);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvqs_gemm: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nvqs_gemm: ldx/ldy smaller than the tensor");
+    MFQ_REQUIRE(d->out <= 65535, MFQ_ERR_UNSUPPORTED, "nvqs_gemm: %d neurons in one call (max 65535)", d->out);
+    const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
+    MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nvqs_gemm: workspace %zu < %zu bytes", workspace_bytes,
+                need);
+    hipStream_t st = as_stream(stream);
+    uint16_t *x16, *w16;
+    float *xscale, *wscale;
+    int Kp;
+    dequant_gemm_carve(workspace, d->out, d->neuron_len, M, x16, xscale, w16, wscale, Kp);
+    int rc = x_prep(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, st);
+    if (rc) return rc;
+    const NvqsK k = to_k(d);
+    hipLaunchKernelGGL((nvqs_dequant_kernel<uint16_t>), dim3(static_cast<unsigned>(ceil_div(Kp / 8 > k.nsign ? Kp / 8 : k.nsign, 256)), k.out),
+                       dim3(256), 0, st, k, static_cast<const uint8_t *>(weight), w16, static_cast<int64_t>(Kp), wscale, Kp);
+    rc = check_launch("nvqs_dequant_f16");
+    if (rc) return rc;
+    return gemm_f16_nt(x16, Kp, w16, Kp, M, d->out, Kp, xscale, wscale, y, ldy, st);
+}

@@ -318,7 +318,7 @@ def is_nint_linear_dtype(dtype: str) -> bool:
 
 
 def is_nvq_linear_dtype(dtype: str) -> bool:
-    return dtype in ("NVQ3", "NVQ3J", "NVQ3J-512", "NIQ3")
+    return dtype in ("NVQ3", "NVQ3J", "NVQ3J-512", "NVQ3J-L", "NVQ2", "NVQ2J", "NVQ2J-L", "NVQ2J-XL", "NIQ3", "NIQ2", "NIQ2J")
 
 
 def is_nepq_linear_dtype(dtype: str) -> bool:
@@ -349,7 +349,7 @@ class QuantLinear:
 
 def load_quant_linear(dtype: str, blob, device="cuda") -> QuantLinear:
     """Switch on the MFQ dtype string and build the device weight (cpp_runtime/mfq_decode.cpp:9489-9771)."""
-    dtype = {"NIQ3": "NVQ3"}.get(dtype, dtype)
+    dtype = {"NIQ3": "NVQ3", "NIQ2": "NVQ2", "NIQ2J": "NVQ2J"}.get(dtype, dtype)
     if is_nint_linear_dtype(dtype):
         w = NintWeight.from_blob(blob, device)
         if f"NINT{w.bits}" != dtype:

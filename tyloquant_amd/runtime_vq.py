@@ -1,4 +1,4 @@
-"""NVQ (D4 family) and NEPQ1 weights and their matmul entry points (see runtime.py)."""
+"""NVQ (D4 and E8 families) and NEPQ1 weights and their matmul entry points (see runtime.py)."""
 from __future__ import annotations
 
 import ctypes as C
@@ -37,7 +37,7 @@ class NvqWeight:
     def from_blob(blob, device="cuda") -> "NvqWeight":
         h = F.parse_nvq(blob)
         if h.vector_size != 4 or h.index_bits > 9:
-            raise NotImplementedError(f"{h.dtype}: only the D4 256/512-entry NVQ formats are on the accelerated path")
+            return NvqsWeight.from_header(h, blob, device)       # E8 family, d4_1024: read from the streams in place
         device = torch.device(device)
         desc = L.NvqDesc()
         lib = L.lib()
@@ -61,6 +61,45 @@ class NvqWeight:
         return w
 
 
+class NvqsWeight:
+    """NVQ tensors whose streams are read in place (mfq_hip_nvqs_*): NVQ2 (e8_256; parity or index-parity signs),
+    NVQ2J / NVQ2J-L / NVQ2J-XL (e8_256 / e8_1024 / e8_4096, JSC) and NVQ3J-L (d4_1024, JSC) -- formats 2, 5, 13, 14, 15
+    of the reference's unpack_nvq (cpp_runtime/mfq_decode.cpp:3756-3769)."""
+
+    def __init__(self, desc, data, dtype):
+        self.desc, self.data, self.dtype = desc, data, dtype
+        self.out, self.neuron_len = desc.out, desc.neuron_len
+        self._ws = _Workspace()
+
+    @property
+    def payload_bytes(self) -> int:
+        return int(self.desc.payload_bytes)
+
+    @staticmethod
+    def from_header(h: F.NvqHeader, blob, device="cuda") -> "NvqsWeight":
+        if h.gs != 24 or h.sub_bits != 4:
+            raise NotImplementedError(f"{h.dtype}: NVQ runs only with gs24 and 4-bit states")
+        if not h.jsc and h.codebook not in ("e8_256", "d4_256"):
+            raise NotImplementedError(f"plain NVQ with the {h.codebook} codebook has no dtype in the runtime")
+        device = torch.device(device)
+        desc = L.NvqsDesc()
+        lib = L.lib()
+        L.check(lib.mfq_hip_nvqs_plan(h.vector_size, h.index_bits, h.banks if h.jsc else 1,
+                                      int(h.sign_mode == "index_parity"), h.out, h.neuron_len, C.byref(desc)))
+        payload = _upload(blob, h.body_off, h.body_bytes, device)
+        data = torch.empty(int(desc.total_bytes), dtype=torch.uint8, device=device)
+        grid = None if h.jsc else torch.from_numpy(builtin_grid(h.codebook)).to(device)
+        L.check(lib.mfq_hip_nvqs_repack(C.byref(desc), _ptr(payload), h.body_bytes, int(h.jsc), _ptr(grid), _ptr(data),
+                                        _stream()))
+        torch.cuda.current_stream().synchronize()
+        return NvqsWeight(desc, data, h.dtype)
+
+    def dequantize(self) -> torch.Tensor:
+        w = torch.empty((self.out, self.neuron_len), dtype=torch.float32, device=self.data.device)
+        L.check(L.lib().mfq_hip_nvqs_dequant_f32(C.byref(self.desc), _ptr(self.data), _ptr(w), self.neuron_len, _stream()))
+        return w
+
+
 def nvq_matmul_multi2(first: NvqWeight, second: NvqWeight, x: torch.Tensor) -> torch.Tensor:
     """cat(x @ W0^T, x @ W1^T) for two NVQ tensors that share their input, in one launch for small batches
     (nvq_matmul_multi2, cpp_runtime/mfq_decode.cpp:7981-8003)."""
@@ -68,7 +107,7 @@ def nvq_matmul_multi2(first: NvqWeight, second: NvqWeight, x: torch.Tensor) -> t
         raise ValueError("NVQ multi-projection requires compatible formats and input layouts")
     x2 = _as_2d(x, first.neuron_len)
     M, N = x2.shape[0], first.out + second.out
-    if M > 32:
+    if M > 32 or isinstance(first, NvqsWeight) or isinstance(second, NvqsWeight):
         return torch.cat([nvq_matmul(first, x), nvq_matmul(second, x)], dim=-1)
     y = torch.empty((M, N), dtype=torch.float32, device=x.device)
     if M == 0:
@@ -104,6 +143,12 @@ def nvq_matmul(w: NvqWeight, x: torch.Tensor, *, force: str | None = None) -> to
     if M == 0:                                   # an empty batch: nothing to launch
         return y.reshape(*x.shape[:-1], w.out)
     lib = L.lib()
+    if isinstance(w, NvqsWeight):
+        need = lib.mfq_hip_nvqs_gemm_workspace_bytes(C.byref(w.desc), M)
+        ws = w._ws.get(need, x.device)
+        L.check(lib.mfq_hip_nvqs_gemm(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
+                                      w.out, _ptr(ws), need, _stream()))
+        return y.reshape(*x.shape[:-1], w.out)
     if force == "gemv":
         L.check(lib.mfq_hip_nvq_gemv(C.byref(w.desc), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, _ptr(y),
                                      w.out, _stream()))
