@@ -20,6 +20,9 @@ void mfq_rt_free_quant_linear(void *handle);
 int64_t mfq_rt_linear_out(void *handle);
 int64_t mfq_rt_linear_neuron_len(void *handle);
 /* QuantLinear::forward (cpp_runtime/mfq_decode.cpp:9209-9226): y[M, out] fp32 = x[M, K] . W^T. */
+/* Grows the weight's workspace for every batch of 1 .. max_M rows: after it, mfq_rt_linear_forward of such a batch neither
+ * frees nor allocates device memory (needed before capturing the call into a HIP graph). */
+int mfq_rt_linear_reserve(void *handle, int max_M);
 int mfq_rt_linear_forward(void *handle, const void *x, int x_dtype, int64_t ldx, int M, float *y, void *stream);
 int mfq_rt_linear_dequantize(void *handle, float *out, void *stream);
 /* embed_forward (cpp_runtime/mfq_decode.cpp:13929-13957) on a NINT table: out [n_ids, K] of out_dtype (MFQ_X_*),

@@ -450,3 +450,36 @@ def test_gemv_bf16_rows_of_any_magnitude(bits, gs, sb, scale):
         if scale <= 1e4:                                   # beyond that silu(gate) * up leaves fp16's range by itself
             h = R.nint_matmul_swiglu(lin.weight, x.cuda(), torch.bfloat16).float().cpu().numpy()
             assert rel_l2(h, want) < 6e-3                  # bf16 output: half an ulp is 4e-3
+
+
+def test_reserved_workspace_lets_forward_run_under_graph_capture():
+    """QuantLinear.reserve(max_rows) sizes the weight's workspace once; forward() of any smaller batch then allocates
+    nothing of its own and can be captured into a HIP graph (batch-1 GEMV, streaming kernel and prefill kernel with its
+    activation prep).  Every replay, with eager work in between, equals the eager result."""
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(77)
+    t = O.quantize_nint((rng.standard_normal((96, 1024)) * 0.02).astype(np.float32), 4, 32, 6)
+    lin = _load(t)
+    lin.reserve(300)
+    buf = lin.weight._ws.buf
+    for M in (1, 16, 300):
+        x, _ = _x(rng, M, 1024)
+        eager = lin(x).clone()
+        assert lin.weight._ws.buf is buf                     # no regrowth after reserve()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            lin(x)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            y = lin(x)
+        for rep in range(3):
+            y.fill_(float("nan"))
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, eager), (M, rep)
+            other, _ = _x(rng, 7, 1024)                      # eager work between the replays
+            lin(other)
+            torch.cuda.synchronize()

@@ -503,6 +503,30 @@ void QuantLinear::forward(const void *x, int x_dtype, int64_t ldx, int M, float 
     else if (kind == QuantLinearKind::Nepq) nepq_matmul(*nepq, 0, x, x_dtype, ldx, M, y, stream);
     else nint8_zero_matmul(*nint8z, x, x_dtype, ldx, M, y, stream);
 }
+void QuantLinear::reserve(int max_M) const {
+    // the need is not monotonic in M (the kernels change with the batch): take the largest over every batch size up to 512
+    // rows, every multiple of 64 beyond, and max_M itself
+    size_t need = 0, rot = 0;
+    auto one = [&](int M) {
+        size_t n = 0;
+        if (kind == QuantLinearKind::Nint) n = mfq_hip_nint_gemm_workspace_bytes(&nint->desc, M);
+        else if (kind == QuantLinearKind::Nvq)
+            n = nvq->streams ? mfq_hip_nvqs_gemm_workspace_bytes(&nvq->sdesc, M) : mfq_hip_nvq_gemm_workspace_bytes(&nvq->desc, M);
+        else if (kind == QuantLinearKind::Nepq) n = mfq_hip_nepq_gemm_workspace_bytes(&nepq->desc, nepq->out_per_expert, M);
+        else n = mfq_hip_nint8z_gemm_workspace_bytes(&nint8z->desc, M);
+        need = std::max(need, n);
+    };
+    for (int M = 1; M <= std::min(max_M, 512); ++M) one(M);
+    for (int M = 576; M < max_M; M += 64) one(M);
+    if (max_M > 0) one(max_M);
+    if (kind == QuantLinearKind::Nint) nint->workspace.ensure(need);
+    else if (kind == QuantLinearKind::Nvq) nvq->workspace.ensure(need);
+    else if (kind == QuantLinearKind::Nepq) {
+        nepq->workspace.ensure(need);
+        if (nepq->rotation_block) rot = static_cast<size_t>(std::max(max_M, 0)) * nepq->desc.neuron_len * 2;
+        nepq->rotated.ensure(rot);
+    } else nint8z->workspace.ensure(need);
+}
 void QuantLinear::dequantize(float *out, mfq_stream_t stream) const {
     if (kind == QuantLinearKind::Nint) nint_dequantize(*nint, out, stream);
     else if (kind == QuantLinearKind::Nvq) nvq_dequantize(*nvq, out, stream);
@@ -1223,6 +1247,9 @@ int mfq_rt_load_quant_linear(const char *dtype, const void *blob, size_t n, void
 void mfq_rt_free_quant_linear(void *handle) { delete static_cast<QuantLinear *>(handle); }
 int64_t mfq_rt_linear_out(void *h) { return static_cast<QuantLinear *>(h)->out(); }
 int64_t mfq_rt_linear_neuron_len(void *h) { return static_cast<QuantLinear *>(h)->neuron_len(); }
+int mfq_rt_linear_reserve(void *h, int max_M) {
+    return guard([&] { static_cast<QuantLinear *>(h)->reserve(max_M); });
+}
 int mfq_rt_linear_forward(void *h, const void *x, int x_dtype, int64_t ldx, int M, float *y, void *stream) {
     return guard([&] { static_cast<QuantLinear *>(h)->forward(x, x_dtype, ldx, M, y, stream); });
 }

@@ -196,6 +196,11 @@ struct QuantLinear {
     int64_t payload_bytes() const;
     void forward(const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream = nullptr) const;
     void dequantize(float *out, mfq_stream_t stream = nullptr) const;
+    // Grows the weight's workspace to the largest need of any batch of 1 .. max_M rows, so that forward() of such a batch
+    // neither frees nor allocates device memory: call it once before capturing forward() into a HIP graph, and before
+    // sharing the weight between threads or streams (the workspace itself is still one buffer per weight: concurrent
+    // forward() calls on one weight need a weight object each, or the C ABI with caller-owned workspaces).
+    void reserve(int max_M) const;
 };
 QuantLinear load_quant_linear(const std::string &dtype, const uint8_t *blob, size_t n, mfq_stream_t stream = nullptr);
 

@@ -343,6 +343,20 @@ class QuantLinear:
 
     __call__ = forward
 
+    def reserve(self, max_rows: int) -> None:
+        """Grow the weight's workspace to the largest need of any batch of 1 .. max_rows rows, so that forward() of such
+        a batch does not allocate: call once before capturing forward() into a HIP graph.  (The output tensor still comes
+        from torch's allocator, which is capture-aware.)"""
+        lib, w = L.lib(), self.weight
+        query = {"nint": lambda M: lib.mfq_hip_nint_gemm_workspace_bytes(C.byref(w.desc), M),
+                 "nint8z": lambda M: lib.mfq_hip_nint8z_gemm_workspace_bytes(C.byref(w.desc), M),
+                 "nvq": lambda M: (lib.mfq_hip_nvqs_gemm_workspace_bytes if type(w).__name__ == "NvqsWeight"
+                                   else lib.mfq_hip_nvq_gemm_workspace_bytes)(C.byref(w.desc), M),
+                 "nepq": lambda M: lib.mfq_hip_nepq_gemm_workspace_bytes(C.byref(w.desc), w.out_per_expert, M)}[self.kind]
+        sizes = set(range(1, min(max_rows, 512) + 1)) | set(range(576, max_rows, 64)) | {max_rows}
+        need = max((int(query(M)) for M in sizes if M > 0), default=0)
+        w._ws.get(need, w.data.device)
+
     def dequantize(self) -> torch.Tensor:
         return self.weight.dequantize()
 
