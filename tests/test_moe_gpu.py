@@ -339,3 +339,26 @@ def test_grouped_glu_epilogue_matches_the_two_calls(routed, activation, out_dtyp
         ref = 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3))) * u
     got = fused.float().cpu().numpy()
     assert rel_l2(got, ref) < 5e-3 and np.abs(got - ref).max() < ABS_TOL
+
+
+def test_mapped_path_with_hundreds_of_experts_and_skewed_routes():
+    """200 experts (the chunk lists are built 64 experts at a time), top-4 of 600 tokens with a skewed router: a few
+    experts receive several hundred pairs (several 128-pair chunks plus a remainder of every size class), most a
+    handful, some none.  Every pair against the oracle's loop."""
+    from tyloquant_amd.runtime_moe import build_moe_route_plan
+    rng = np.random.default_rng(1234)
+    E, out, K, T, R = 200, 48, 96, 600, 4
+    bits = [(4, 3, 2, 5)[i % 4] for i in range(E)]
+    t, w = _moe(rng, E, out, K, bits)
+    p = rng.dirichlet(np.full(E, 0.08))
+    ids = np.stack([rng.choice(E, size=R, replace=False, p=p) for _ in range(T)]).astype(np.int32)
+    counts = np.bincount(ids.reshape(-1), minlength=E)
+    assert counts.max() > 256 and (counts == 0).any() and ((counts > 0) & (counts <= 16)).any()
+    x = torch.from_numpy((rng.standard_normal((T, K)) * 0.1).astype(np.float32)).to(torch.bfloat16)
+    route = build_moe_route_plan(torch.from_numpy(ids).cuda(), E)
+    got = w(x.cuda(), route).cpu().numpy()
+    ref = O.moe_grouped_matmul(O.dequantize_expertwise(t), x.float().numpy(), ids)
+    assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL
+    fused = w.forward_glu(x.cuda(), route).float().cpu().numpy()
+    g, u = ref[..., : out // 2], ref[..., out // 2:]
+    assert rel_l2(fused, g / (1.0 + np.exp(-g)) * u) < 5e-3
