@@ -107,6 +107,16 @@ int mfq_hip_nint_gemv_swiglu(const mfq_nint_desc *d, const void *weight, const v
 int mfq_hip_nint_gemv_glu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
                           int64_t ldx, int M, void *hidden, int out_dtype, int64_t ldh, int activation,
                           mfq_stream_t stream);
+/* Prefill counterpart: the gate/up projection of M activation rows with the GLU in the matmul's epilogue, for the
+ * batches mfq_hip_nint_gemm runs on its block-tiled kernel in one pass over K.  hidden[m, c] = act(y[m, c]) * y[m, W + c]
+ * in 16 bits (out_dtype, MFQ_X_*), y as mfq_hip_nint_gemm gives it; the [M, 2 W] fp32 intermediate is never stored.
+ * Replaces nint_matmul followed by mfq_swiglu / the GeGLU kernel in FFN::forward_impl for M > 1
+ * (cpp_runtime/mfq_decode.cpp:11199-11209).  workspace: mfq_hip_nint_gemm_workspace_bytes(d, M) bytes.
+ * MFQ_ERR_UNSUPPORTED (nothing launched) for batches and profiles outside that kernel: run mfq_hip_nint_gemm +
+ * mfq_hip_moe_glu then.  Equal to those two calls up to the rounding of the fp32 product to 16 bits. */
+int mfq_hip_nint_gemm_glu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
+                          int activation, void *hidden, int out_dtype, int64_t ldh, void *workspace,
+                          size_t workspace_bytes, mfq_stream_t stream);
 
 /* Decode feed-forward block in ONE launch, one activation row: hidden = act(gate x) * (up x) as fp16, y = down hidden
  * (fp32 [down.out]).  gate_up is the [2 W, H] gate/up tensor (gate rows first), down the [N, W] tensor of the same

@@ -189,6 +189,75 @@ def test_gate_up_gemv_with_fused_geglu(bits, gs, sb):
             assert rel_l2(sw, O.moe_swiglu(y)) < 2e-3 and rel_l2(sw, h) > 1e-2   # the two activations differ
 
 
+@pytest.mark.parametrize("bits,gs,sb,W,K,M", [
+    (4, 32, 6, 1024, 200, 1100),   # 64-token tiles, ragged last tile, K short of a whole step
+    (4, 32, 6, 1040, 256, 2200),   # 128-token tiles; 65 gate row-blocks: the last block holds one
+    (3, 24, 5, 1024, 240, 1100),
+    (2, 16, 4, 1024, 256, 1100),
+    (5, 28, 7, 1024, 224, 1100),   # the natural-order unit
+    (4, 48, 6, 1024, 384, 2200),   # activation tiles through registers
+])
+def test_gate_up_prefill_with_fused_glu(bits, gs, sb, W, K, M):
+    """act(gate) * up in the epilogue of the block-tiled prefill kernel: the C entry point takes the call, its values
+    are those of matmul + the element-wise GLU kernel (same fp32 sums; the fused kernel contracts the last multiply,
+    so a product on a 16-bit rounding midpoint may land one unit apart) and match the float64 oracle."""
+    from tyloquant_amd import _lib as L
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_moe import moe_glu
+    rng = np.random.default_rng(4700 + bits + W + M)
+    t = O.quantize_nint((rng.standard_normal((2 * W, K)) * 0.08).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    w = lin.weight
+    deq = O.dequantize_nint(t)
+    lib = L.lib()
+    for dtype, act in ((torch.bfloat16, L.GLU_SILU), (torch.float16, L.GLU_GELU)):
+        x, xf = _x(rng, M, K, dtype)
+        need = lib.mfq_hip_nint_gemm_workspace_bytes(C.byref(w.desc), M)
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        h = torch.full((M, W + 8), 7.0, dtype=dtype, device="cuda")   # padded rows: the padding must stay untouched
+        rc = lib.mfq_hip_nint_gemm_glu(C.byref(w.desc), w.data.data_ptr(), x.data_ptr(), R._x_dtype(x), x.stride(0), M, act,
+                                       h.data_ptr(), R._x_dtype(h), h.stride(0), ws.data_ptr(), need, None)
+        assert rc == L.OK, L.lib().mfq_hip_last_error()
+        assert (h[:, W:] == 7.0).all()
+        two = moe_glu(R.nint_matmul(w, x), dtype, act)
+        def ordinal(v):                       # 16-bit patterns on a line: neighbours differ by 1, -0 and +0 coincide
+            i = v.contiguous().view(torch.int16).int()
+            return torch.where(i < 0, -(i & 0x7FFF), i)
+        diff = (ordinal(h[:, :W]) - ordinal(two)).abs()
+        assert diff.max().item() <= 1 and (diff != 0).float().mean().item() < 1e-3
+        y = O.linear_forward_f64(deq, xf)
+        ref = O.moe_swiglu(y) if act == L.GLU_SILU else O.moe_geglu(y)
+        assert np.abs(y[:, :W]).max() > 2.0
+        tol = 6e-3 if dtype == torch.bfloat16 else 2e-3                # one 16-bit rounding of the result
+        assert rel_l2(h[:, :W].float().cpu().numpy(), ref) < tol
+        host = (R.nint_matmul_swiglu if act == L.GLU_SILU else R.nint_matmul_geglu)(w, x, out_dtype=dtype)
+        assert torch.equal(host, h[:, :W])                             # the host wrapper takes the same path
+
+
+def test_gate_up_prefill_glu_declines_what_the_kernel_does_not_take():
+    """Few rows (the streaming kernels' range), grids that are split over K and an odd neuron count: nothing is launched,
+    the error names the reason, and the host wrapper runs matmul + GLU instead."""
+    from tyloquant_amd import _lib as L
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(4790)
+    t = O.quantize_nint((rng.standard_normal((2 * 64, 2048)) * 0.05).astype(np.float32), 4, 32, 6)
+    lin = _load(t)
+    w = lin.weight
+    lib = L.lib()
+    for M in (4, 700):
+        x, xf = _x(rng, M, 2048, torch.bfloat16)
+        need = lib.mfq_hip_nint_gemm_workspace_bytes(C.byref(w.desc), M)
+        ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+        h = torch.zeros((M, 64), dtype=torch.bfloat16, device="cuda")
+        rc = lib.mfq_hip_nint_gemm_glu(C.byref(w.desc), w.data.data_ptr(), x.data_ptr(), L.X_BF16, x.stride(0), M,
+                                       L.GLU_SILU, h.data_ptr(), L.X_BF16, 64, ws.data_ptr(), need, None)
+        assert rc == L.ERR_UNSUPPORTED and b"one-pass" in lib.mfq_hip_last_error()
+        assert not h.any()
+        got = R.nint_matmul_swiglu(w, x, out_dtype=torch.bfloat16).float().cpu().numpy()
+        ref = O.moe_swiglu(O.linear_forward_f64(O.dequantize_nint(t), xf))
+        assert rel_l2(got, ref) < 6e-3
+
+
 @pytest.mark.parametrize("K", [1000, 77])
 @pytest.mark.parametrize("mode", [0, 1])
 def test_input_gate_then_matmul(mode, K):

@@ -74,6 +74,8 @@ _SIGS = {
     "mfq_hip_nint_gemv_gate": (C.c_int, [C.POINTER(NintDesc), vp, vp, vp, C.c_int, i64, i64, C.c_int, C.c_int, vp, i64,
                                          vp]),
     "mfq_hip_nint_gemv_glu": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, C.c_int, i64, C.c_int, vp]),
+    "mfq_hip_nint_gemm_glu": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, C.c_int, vp, C.c_int, i64, vp,
+                                        sz, vp]),
     "mfq_hip_nint_ffn_decode_workspace_bytes": (sz, [C.POINTER(NintDesc), C.POINTER(NintDesc)]),
     "mfq_hip_nint_ffn_decode_workspace_init": (C.c_int, [vp, vp]),
     "mfq_hip_nint_ffn_decode": (C.c_int, [C.POINTER(NintDesc), vp, C.POINTER(NintDesc), vp, vp, C.c_int, C.c_int, vp, vp, sz,

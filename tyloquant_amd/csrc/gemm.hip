@@ -347,6 +347,10 @@ size_t nint_prefill_xg_bytes(const mfq_nint_desc *d, int M);
 size_t nint_prefill_split_bytes(const mfq_nint_desc *d, int M);
 int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16, int Kp, const float *xscale, uint32_t *xg,
                  int M, float *y, int64_t ldy, float *part, hipStream_t st);
+int nint_prefill_splits(const mfq_nint_desc *d, int M);
+bool nint_prefill_glu_capable(const mfq_nint_desc *d);
+int nint_prefill_glu(const mfq_nint_desc *d, const void *weight, const uint16_t *x16, int Kp, const float *xscale,
+                     const uint32_t *xg, int M, void *hidden, int64_t ldh, int f16, int gelu, hipStream_t st);
 
 }  // namespace mfq
 
@@ -442,4 +446,43 @@ extern "C" int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, con
     rc = nint_dequant_f16(d, weight, w16, Kp, wscale, st);
     if (rc) return rc;
     return gemm_f16_nt(x16, Kp, w16, Kp, M, d->out, Kp, xscale, wscale, y, ldy, st);
+}
+
+// The batch sizes at which mfq_hip_nint_gemm runs the block-tiled prefill kernel in one pass over K: only there does
+// the fused epilogue have both halves of a pair in one block.
+// Below about a thousand rows the two calls are as fast (measured on 24576 x 4096 and 34816 x 5120 NINT4-32: 152 against
+// 145 us at 512 rows, 458 against 494 us at 2048): the epilogue's narrow stores cost what the skipped intermediate saves.
+static bool nint_gemm_glu_fuses(const mfq_nint_desc *d, int M) {
+    static const int min_m = tune_env("MFQ_GLU_PREFILL_MIN_M", 1024);
+    return M >= min_m && !nint_streams(d, M) && nint_prefill_glu_capable(d) && nint_prefill_splits(d, M) == 1;
+}
+
+extern "C" int mfq_hip_nint_gemm_glu(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
+                                     int M, int activation, void *hidden, int out_dtype, int64_t ldh, void *workspace,
+                                     size_t workspace_bytes, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && x && hidden, MFQ_ERR_INVALID, "nint_gemm_glu: null argument");
+    MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nint_gemm_glu: M=%d", M);
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint_gemm_glu: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(out_dtype == MFQ_X_BF16 || out_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint_gemm_glu: out_dtype=%d", out_dtype);
+    MFQ_REQUIRE(activation == MFQ_GLU_SILU || activation == MFQ_GLU_GELU, MFQ_ERR_INVALID, "nint_gemm_glu: activation=%d",
+                activation);
+    MFQ_REQUIRE(d->out % 2 == 0 && ldx >= d->neuron_len && ldh >= d->out / 2, MFQ_ERR_INVALID,
+                "nint_gemm_glu: ldx/ldh smaller than the tensor");
+    if (!nint_gemm_glu_fuses(d, M))
+        return fail(MFQ_ERR_UNSUPPORTED, "nint_gemm_glu: %d rows of this tensor do not take the one-pass prefill kernel", M);
+    const size_t need = prefill_workspace(d, M);
+    MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nint_gemm_glu: workspace %zu < %zu bytes",
+                workspace_bytes, need);
+    hipStream_t st = as_stream(stream);
+    const int Kp = prefill_kp(d);
+    uint8_t *p = static_cast<uint8_t *>(workspace);
+    uint16_t *x16 = reinterpret_cast<uint16_t *>(p);
+    p += align256(static_cast<size_t>(M) * Kp * 2);
+    float *xscale = reinterpret_cast<float *>(p);
+    p += align256(static_cast<size_t>(M) * 4);
+    uint32_t *xg = reinterpret_cast<uint32_t *>(p);
+    int rc = x_prep_groups(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, d->gs, d->nsteps, xg, st);
+    if (rc) return rc;
+    return nint_prefill_glu(d, weight, x16, Kp, xscale, xg, M, hidden, ldh, out_dtype == MFQ_X_F16,
+                            activation == MFQ_GLU_GELU, st);
 }

@@ -373,6 +373,13 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
             }
         }
     }
+    // The rows' scales, all requested before the first store: a load issued between the stores would wait behind them
+    // (the output may alias anything, as far as the compiler knows), one round trip to memory per row.
+    float xsv[MT][4];
+#pragma unroll
+    for (int a = 0; a < MT; ++a)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) xsv[a][v] = xscale[rows.src((wm * MT + a) * 16 + 4 * kb + v)];
 #pragma unroll
     for (int a = 0; a < MT; ++a) {
 #pragma unroll
@@ -380,7 +387,7 @@ __device__ __forceinline__ void nint_prefill_body(const NintK &k, const uint8_t 
             const int ti = (wm * MT + a) * 16 + 4 * kb + v;
             const int m = rows.dst(ti);
             if (m < 0) continue;
-            const float xs = xscale[rows.src(ti)];
+            const float xs = xsv[a][v];
             if constexpr (GLU) {
                 uint16_t *h = reinterpret_cast<uint16_t *>(y);
 #pragma unroll

@@ -41,6 +41,8 @@ Knob g_knobs[] = {
     {"MFQ_FFN_SPIN_LIMIT", "polls after which the one-launch FFN's grid barrier gives up", 0, false},
     {"MFQ_FFN_TRACE", "1 = the one-launch FFN records per-block clocks behind its workspace", 0, false},
     {"MFQ_MOE_NB", "row-blocks per wave of the MoE streaming kernel (0 = by shape)", 0, false},
+    {"MFQ_MOE_GROUPS", "bit mask of the register groups the mapped MoE prefill path launches (7 = all)", 0, false},
+    {"MFQ_GLU_PREFILL_MIN_M", "rows from which the dense gate/up prefill fuses the GLU into its epilogue", 0, false},
 };
 std::mutex g_mu;
 std::atomic<int> g_cu_override{0};
@@ -58,7 +60,8 @@ int tune_env(const char *name, int dflt) {
         }
         return k.value;
     }
-    return dflt;  // not in the table: still honoured, but not listed
+    const char *e = getenv(name);  // not in the table: still honoured, but not listed
+    return e ? atoi(e) : dflt;
 }
 
 int device_cu_count() {

@@ -188,8 +188,21 @@ def _nint_matmul_glu(w: NintWeight, x: torch.Tensor, out_dtype, activation: int)
     d = w.desc
     if M == 0:
         return torch.empty((*x.shape[:-1], W), dtype=out_dtype, device=x.device)
-    fused = M <= 2 and w.out % 32 == 0 and (d.kind == 1 or (d.bits == 5 and d.gs == 28))
-    if not fused:
+    unit = w.out % 32 == 0 and (d.kind == 1 or (d.bits == 5 and d.gs == 28))
+    o16 = L.X_F16 if out_dtype == torch.float16 else L.X_BF16
+    if unit and M > 2:
+        # prefill batches: the GLU runs in the epilogue of the block-tiled matmul where that kernel takes the call
+        lib = L.lib()
+        need = lib.mfq_hip_nint_gemm_workspace_bytes(C.byref(d), M)
+        ws = w._ws.get(need, x.device)
+        hidden = torch.empty((M, W), dtype=out_dtype, device=x.device)
+        rc = lib.mfq_hip_nint_gemm_glu(C.byref(d), _ptr(w.data), _ptr(x2), _x_dtype(x2), x2.stride(0), M, activation,
+                                       _ptr(hidden), o16, W, _ptr(ws), need, _stream())
+        if rc == L.OK:
+            return hidden.reshape(*x.shape[:-1], W)
+        if rc != L.ERR_UNSUPPORTED:
+            L.check(rc)
+    if not unit or M > 2:
         from .runtime_moe import moe_glu
         return moe_glu(nint_matmul(w, x), out_dtype, activation)
     hidden = torch.empty((M, W), dtype=out_dtype, device=x.device)
