@@ -25,6 +25,12 @@ int64_t mfq_rt_linear_neuron_len(void *handle);
 int mfq_rt_linear_reserve(void *handle, int max_M);
 int mfq_rt_linear_forward(void *handle, const void *x, int x_dtype, int64_t ldx, int M, float *y, void *stream);
 int mfq_rt_linear_dequantize(void *handle, float *out, void *stream);
+/* QuantLinear::forward_swiglu / nint_matmul_geglu (cpp_runtime/mfq_decode.cpp:9228-9240, 8462-8485) on a NINT gate/up
+ * tensor [2 W, K]: hidden fp16 [M, W] = act(gate x) * (up x), act = SiLU or (gelu != 0) the tanh GELU.  One launch for one
+ * or two rows and for the prefill batches the block-tiled kernel takes; otherwise the matmul goes through `scratch`
+ * (fp32 [M, 2 W], may be null when the fused forms apply). */
+int mfq_rt_linear_forward_glu(void *handle, const void *x, int x_dtype, int64_t ldx, int M, int gelu, void *hidden,
+                              float *scratch, void *stream);
 /* embed_forward (cpp_runtime/mfq_decode.cpp:13929-13957) on a NINT table: out [n_ids, K] of out_dtype (MFQ_X_*),
  * ids device int64; and next_token_from_hidden (:14107-14130): token[m] device int64, logits fp32 [M, out] or null.
  * Both fail on a handle that does not hold a NINT tensor. */

@@ -30,6 +30,8 @@ def rt():
     lib.mfq_rt_free_quant_linear.argtypes = [C.c_void_p]
     lib.mfq_rt_linear_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p]
     lib.mfq_rt_linear_dequantize.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.mfq_rt_linear_forward_glu.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_int, C.c_void_p,
+                                              C.c_void_p, C.c_void_p]
     lib.mfq_rt_linear_embedding.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
     lib.mfq_rt_linear_argmax.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p, C.c_void_p,
                                          C.c_void_p]
@@ -119,6 +121,34 @@ def test_cpp_load_quant_linear_and_forward(rt):
     rt.mfq_rt_free_quant_linear(h8)
     with pytest.raises(RuntimeError, match="invalid NINT8-0 block payload length"):
         _load(rt, "NINT8-0", O.pack_nint8_zero(t8)[:-1])
+
+
+def test_cpp_gate_up_glu_across_batch_sizes(rt):
+    """nint_matmul_swiglu / nint_matmul_geglu of the C++ runtime: the fused GEMV (1, 2 rows), matmul + GLU kernel through
+    the scratch buffer (5 rows), the prefill kernel with the GLU in its epilogue (1100 rows, no scratch needed) --
+    against the oracle's float64 product; a batch that needs the scratch buffer without one is an error."""
+    rng = np.random.default_rng(41)
+    W, K = 1024, 256
+    t = O.quantize_nint((rng.standard_normal((2 * W, K)) * 0.08).astype(np.float32), 4, 32, 6)
+    h = _load(rt, "NINT4", O.pack_nint(t))
+    deq = O.dequantize_nint(t)
+    for M, with_scratch in ((1, False), (2, False), (5, True), (1100, False)):
+        x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+        scratch = torch.empty((M, 2 * W), dtype=torch.float32, device="cuda") if with_scratch else None
+        y = O.linear_forward_f64(deq, x.float().cpu().numpy())
+        for gelu, ref in ((0, O.moe_swiglu(y)), (1, O.moe_geglu(y))):
+            hid = torch.zeros((M, W), dtype=torch.float16, device="cuda")
+            rc = rt.mfq_rt_linear_forward_glu(h, x.data_ptr(), 0, K, M, gelu, hid.data_ptr(),
+                                              scratch.data_ptr() if with_scratch else None, None)
+            assert rc == 0, rt.mfq_rt_last_error()
+            torch.cuda.synchronize()
+            got = hid.float().cpu().numpy()
+            assert np.linalg.norm(got - ref) / np.linalg.norm(ref) < 2e-3
+    x = torch.zeros((5, K), dtype=torch.bfloat16, device="cuda")
+    hid = torch.zeros((5, W), dtype=torch.float16, device="cuda")
+    assert rt.mfq_rt_linear_forward_glu(h, x.data_ptr(), 0, K, 5, 0, hid.data_ptr(), None, None) == 1
+    assert b"scratch" in rt.mfq_rt_last_error()
+    rt.mfq_rt_free_quant_linear(h)
 
 
 def test_cpp_embedding_rows_and_argmax_head(rt):

@@ -345,7 +345,15 @@ static void nint_matmul_glu(const NintWeight &w, const void *x, int x_dtype, int
         abi_check(mfq_hip_nint_gemv_glu(&w.desc, w.data.get(), x, x_dtype, ldx, M, hidden, MFQ_X_F16, W, activation, stream));
         return;
     }
-    if (!scratch) fail(std::string(what) + ": more than two rows need a [M, 2W] fp32 scratch buffer");
+    if (w.desc.out % 32 == 0 && unit) {  // prefill batches: the block-tiled kernel with the GLU in its epilogue, where it runs
+        const size_t need = mfq_hip_nint_gemm_workspace_bytes(&w.desc, M);
+        w.workspace.ensure(need);
+        const int rc = mfq_hip_nint_gemm_glu(&w.desc, w.data.get(), x, x_dtype, ldx, M, activation, hidden, MFQ_X_F16, W,
+                                             w.workspace.get(), need, stream);
+        if (rc == MFQ_OK) return;
+        if (rc != MFQ_ERR_UNSUPPORTED) abi_check(rc);
+    }
+    if (!scratch) fail(std::string(what) + ": this batch needs a [M, 2W] fp32 scratch buffer");
     nint_matmul(w, x, x_dtype, ldx, M, scratch, stream);
     abi_check(mfq_hip_moe_glu(scratch, 2 * W, M, W, hidden, MFQ_X_F16, W, activation, stream));
 }
@@ -1252,6 +1260,15 @@ int mfq_rt_linear_reserve(void *h, int max_M) {
 }
 int mfq_rt_linear_forward(void *h, const void *x, int x_dtype, int64_t ldx, int M, float *y, void *stream) {
     return guard([&] { static_cast<QuantLinear *>(h)->forward(x, x_dtype, ldx, M, y, stream); });
+}
+int mfq_rt_linear_forward_glu(void *h, const void *x, int x_dtype, int64_t ldx, int M, int gelu, void *hidden, float *scratch,
+                              void *stream) {
+    return guard([&] {
+        const QuantLinear *q = static_cast<QuantLinear *>(h);
+        if (!q->nint) fail("the fused gate/up projection needs a NINT tensor");
+        if (gelu) nint_matmul_geglu(*q->nint, x, x_dtype, ldx, M, hidden, scratch, stream);
+        else nint_matmul_swiglu(*q->nint, x, x_dtype, ldx, M, hidden, scratch, stream);
+    });
 }
 int mfq_rt_linear_dequantize(void *h, float *out, void *stream) {
     return guard([&] { static_cast<QuantLinear *>(h)->dequantize(out, stream); });

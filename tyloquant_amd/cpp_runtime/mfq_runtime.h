@@ -138,7 +138,8 @@ struct NepqWeight {
 void nint_matmul(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                  mfq_stream_t stream = nullptr);
 // hidden fp16 [M, W] = silu(gate) * up of a [2W, K] gate/up tensor (gate rows first): one fused launch for one or two
-// rows (nint_gemv_packed_swiglu_ws_cuda :393-396), else nint_matmul into `scratch` (fp32 [M, 2W]) + the SwiGLU kernel
+// rows (nint_gemv_packed_swiglu_ws_cuda :393-396) and for prefill batches the block-tiled kernel takes
+// (mfq_hip_nint_gemm_glu), else nint_matmul into `scratch` (fp32 [M, 2W]) + the SwiGLU kernel
 void nint_matmul_swiglu(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, void *hidden,
                         float *scratch = nullptr, mfq_stream_t stream = nullptr);
 // y = (x * silu(gate)) . W^T (mode 0) or (x * sigmoid(gate)) . W^T (mode 1) (nint_matmul_input_mul :8395-8417): one or
