@@ -60,12 +60,15 @@ __device__ __forceinline__ float x_to_f32(uint16_t v) {
 // Gated-linear-unit value act(gate) * up of the reference's mfq_glu (mfq/kernels/cuda/glu.cuh:5-16): SiLU, or the
 // tanh form of GELU when `gelu` is set.  Kernels carry the choice in bit 1 of their 16-bit output mode
 // (bit 0: fp16 rather than bf16).
+// Both are gate * sigmoid(z) * up -- 0.5 (1 + tanh(u)) = sigmoid(2 u) -- with the sigmoid from the hardware's base-2
+// exponential and reciprocal (one unit in the last place each; the 16-bit result keeps 8 or 11 bits): a dozen
+// instructions per value where expf, tanhf and a division take several dozen, which the prefill epilogues notice.
+__device__ __forceinline__ float sigmoid_fast(float z) {
+    return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504088896340736f * z));
+}
 __device__ __forceinline__ float glu_value(float gate, float up, bool gelu) {
-    if (gelu) {
-        const float t = tanhf(0.79788456080286535587989211986876f * gate * (1.0f + 0.044715f * gate * gate));
-        return up * (0.5f * gate * (1.0f + t));
-    }
-    return gate / (1.f + expf(-gate)) * up;
+    const float z = gelu ? 1.59576912160573071176f * gate * (1.0f + 0.044715f * gate * gate) : gate;
+    return gate * sigmoid_fast(z) * up;
 }
 
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {

@@ -450,10 +450,10 @@ extern "C" int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, con
 
 // The batch sizes at which mfq_hip_nint_gemm runs the block-tiled prefill kernel in one pass over K: only there does
 // the fused epilogue have both halves of a pair in one block.
-// Below about a thousand rows the two calls are as fast (measured on 24576 x 4096 and 34816 x 5120 NINT4-32: 152 against
-// 145 us at 512 rows, 458 against 494 us at 2048): the epilogue's narrow stores cost what the skipped intermediate saves.
+// Below a few hundred rows the two calls are as fast (measured on 24576 x 4096 and 34816 x 5120 NINT4-32: 142 against
+// 143 us and 245 against 258 us at 512 rows, 441 against 481 us and 742 against 813 us at 2048).
 static bool nint_gemm_glu_fuses(const mfq_nint_desc *d, int M) {
-    static const int min_m = tune_env("MFQ_GLU_PREFILL_MIN_M", 1024);
+    static const int min_m = tune_env("MFQ_GLU_PREFILL_MIN_M", 512);
     return M >= min_m && !nint_streams(d, M) && nint_prefill_glu_capable(d) && nint_prefill_splits(d, M) == 1;
 }
 
