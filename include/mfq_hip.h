@@ -300,7 +300,10 @@ typedef struct mfq_nvqs_desc {
     int32_t out, neuron_len, ng, nvec, nsign;
     int64_t tables_off, anchors_off, state_off, index_off, sign_off;
     int64_t total_bytes;
-    int64_t payload_bytes; /* anchors + the three streams */
+    int64_t payload_bytes; /* anchors + the streams */
+    int32_t kind;          /* 0: the NVQ formats above; 1: NVQ1-L / NVQ1-S; 2: NPQ0-L / NPQ0-S (see below) */
+    int32_t state_bits, cb_bytes;
+    float delta;
 } mfq_nvqs_desc;
 
 int mfq_hip_nvqs_plan(int vector_size, int index_bits, int banks, int index_parity, int out, int neuron_len,
@@ -318,6 +321,27 @@ int mfq_hip_nvqs_dequant_f32(const mfq_nvqs_desc *d, const void *weight, float *
  * dequantized to fp16 in the workspace (size from the query, 0 up to 16 rows) and multiplied on the matrix cores. */
 int mfq_hip_nvqs_gemv(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
                       int M, float *y, int64_t ldy, mfq_stream_t stream);
+/* The 1-bit families on the same descriptor and the same dequant / gemv / gemm entry points: groups of 24 weights made of
+ * three 8-weight vectors, one fp16 anchor per neuron, tensor-wide streams read in place.
+ *   NVQ1-L (format 1 of unpack_nvq, cpp_runtime/mfq_decode.cpp:3759, 3805-3810; mfq/formats/nvq1_l.py): 11-bit indices
+ *     into a 2048-entry ternary grid (built in, or in the blob), 3- or 4-bit integer relative scale and a delta sign
+ *     per group: w = anchor * scale * (code -/+ 1/8).
+ *   NVQ1-S (format 8, :3769, 3811-3813; nvq1_s.py): 9-bit indices, two 512-entry ternary banks in the blob chosen by the
+ *     group's delta sign, 4-bit scale, delta 5/32.
+ *   NPQ0-L / NPQ0-S (formats 7 / 9, :3768-3770, 3845-3910; npq0_l.py, npq0_s.py): a vector is two 4-dimensional int8
+ *     sub-vectors, first[state][index & 7] and second[state][index >> 3] (7- / 6-bit indices, 8 / 4 states); the state
+ *     also selects the relative scale from an fp16 table: w = code * anchor * lut[state].
+ * `body` = device copy of the blob from behind its header, shape and neuron count on: the tables (NVQ1-L with a custom
+ * grid: 4096 bytes; NVQ1-S: 2048; NPQ0: 64-byte header + sub-codebooks), fp16 anchors, streams.  `grid` = device copy
+ * of the built-in grid as 2048 packed uint16 (needed only for an NVQ1-L body without a table).  The host validates the
+ * blob's header and table header before calling. */
+#define MFQ_NVQS_NVQ1_L 1
+#define MFQ_NVQS_NVQ1_S 2
+#define MFQ_NVQS_NPQ0_L 3
+#define MFQ_NVQS_NPQ0_S 4
+int mfq_hip_nvqs_plan_lowbit(int format, int state_bits, int out, int neuron_len, mfq_nvqs_desc *d);
+int mfq_hip_nvqs_repack_lowbit(const mfq_nvqs_desc *d, const void *body, int64_t body_bytes, const void *grid,
+                               void *weight, mfq_stream_t stream);
 size_t mfq_hip_nvqs_gemm_workspace_bytes(const mfq_nvqs_desc *d, int M);
 int mfq_hip_nvqs_gemm(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
                       int M, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,

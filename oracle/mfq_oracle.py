@@ -35,6 +35,13 @@ reference tree).  Parity status of each function:
     dequantize_nvq (incl. the index-parity sign rule on e8_256), pack_nepq / unpack_nepq / dequantize_nepq,
     pack_nint_moe / unpack_nint_moe / dequantize_expertwise
 
+  pinned by reference-written blobs and reference-dequantized values of the 1-bit families
+  (tests/golden/reference_lowbit.npz, made by tests/golden/make_reference_lowbit.py; tests/test_reference_lowbit.py)
+    pack_nvq1 / unpack_nvq1        mfq/formats/nvq1_l.py:234-345, nvq1_s.py:262-347
+    dequantize_nvq1                mfq/quantize/nvq1_l_quant.py:384-414, nvq1_s_quant.py:142-174
+    pack_npq0 / unpack_npq0        mfq/formats/npq0_l.py:112-185, 326-415, npq0_s.py:110-183, 320-406
+    dequantize_npq0                mfq/quantize/npq0_l.py:766-790, npq0_s.py:812-836
+
   pinned by golden vectors written from the reference's own numpy quantizer
   (tests/golden/nint_quant_vectors.npz, made by tests/golden/make_nint_quant_vectors.py)
     make_qkx2 / quantize_nint      mfq/formats/nint.py:119-174, mfq/quantize/nint_quant.py:745-893
@@ -747,6 +754,232 @@ def dequantize_nint8_zero(t: Nint8ZeroTensor) -> np.ndarray:
     return (t.scale.astype(np.float32)[..., None] * t.q.astype(np.float32)).reshape(t.out, t.neuron_len)
 
 
+# ---------------------------------------------------------------------------
+# The 1-bit families: NVQ1-L / NVQ1-S (8-dimensional ternary codebooks, an integer relative scale and a delta sign
+# per group of 24) and NPQ0-L / NPQ0-S (two 4-dimensional int8 sub-codebooks chosen by a per-group state that also
+# selects the relative scale).  One fp16 anchor per neuron; every stream is packed across the whole tensor.
+# (mfq/formats/nvq1_l.py:130-330, nvq1_s.py:168-347, npq0_l.py:20-415, npq0_s.py:18-406)
+# ---------------------------------------------------------------------------
+_LOWBIT_HDR = struct.Struct("<4sBBHiiI")      # magic, profile / version, state bits, groupsize, axis, neuron_len, ndim
+# label: magic, header byte, state bits, index bits, states, first / second sub-codebook entries, table version
+LOWBIT_SPECS = {
+    "NVQ1-L": dict(magic=b"NQ1L", index_bits=11, entries=2048, banks=1, delta=0.125),
+    "NVQ1-S": dict(magic=b"NQ1S", version=1, state_bits=4, index_bits=9, entries=512, banks=2, delta=0.15625),
+    "NPQ0-L": dict(magic=b"NPQL", version=1, state_bits=3, index_bits=7, states=8, second=16, table_version=1),
+    "NPQ0-S": dict(magic=b"NPQS", version=2, state_bits=2, index_bits=6, states=4, second=8, table_version=2),
+}
+
+
+@dataclass
+class Nvq1Tensor:
+    """NVQ1-L (codebook None: the built-in IQ1_S grid, else a custom [2048, 8] ternary table; state_bits 3 or 4) and
+    NVQ1-S (codebook [2, 512, 8]: the group's delta sign also selects the bank)."""
+    label: str
+    shape: tuple
+    axis: int
+    neuron_len: int
+    state_bits: int
+    neuron_scale: np.ndarray      # float32 [out], fp16-representable
+    sub_scale: np.ndarray         # [out, ng] integers below 2^state_bits
+    indices: np.ndarray           # [out, nvec]
+    delta_sign: np.ndarray        # [out, ng] 0 / 1
+    codebook: np.ndarray | None = None
+
+
+@dataclass
+class Npq0Tensor:
+    label: str
+    shape: tuple
+    axis: int
+    neuron_len: int
+    neuron_scale: np.ndarray      # float32 [out]
+    scale_lut: np.ndarray         # float32 [states], fp16-representable
+    state: np.ndarray             # [out, ng]
+    indices: np.ndarray           # [out, nvec]: first index in the low 3 bits, second above
+    first_codebooks: np.ndarray   # int8 [states, 8, 4]
+    second_codebooks: np.ndarray  # int8 [states, 8 or 16, 4]
+
+
+def iq1s_grid() -> np.ndarray:
+    """The 2048 x 8 ternary grid NVQ1-L uses when its blob carries none (mfq/formats/nvq1_l.py:78-94)."""
+    return unpack_ternary_table((_DATA / "iq1s_2048.bin").read_bytes())
+
+
+def nvq1s_default_banks() -> np.ndarray:
+    """The [2, 512, 8] table NVQ1-S writes when a tensor brings none (mfq/formats/nvq1_s.py:126-137)."""
+    raw = (_DATA / "nvq1s_banks.bin").read_bytes()
+    return np.stack([unpack_ternary_table(raw[:1024]), unpack_ternary_table(raw[1024:])])
+
+
+def _lowbit_counts(label, neuron_len):
+    ng = -(-neuron_len // 24)
+    nvec = -(-neuron_len // 8) if label == "NVQ1-L" else neuron_len // 8
+    return ng, nvec
+
+
+def pack_nvq1(t: Nvq1Tensor) -> bytes:
+    """mfq/formats/nvq1_l.py:234-284 (profile 1: built-in grid, 2: table in the blob) and nvq1_s.py:262-290."""
+    sp = LOWBIT_SPECS[t.label]
+    out = t.neuron_scale.size
+    if t.label == "NVQ1-L":
+        head = _LOWBIT_HDR.pack(sp["magic"], 2 if t.codebook is not None else 1, t.state_bits, 24, t.axis, t.neuron_len,
+                                len(t.shape))
+        table = pack_ternary_table(t.codebook) if t.codebook is not None else b""
+    else:
+        if t.neuron_len % 8:
+            raise ValueError("NVQ1-S neuron length must be divisible by 8")
+        head = _LOWBIT_HDR.pack(sp["magic"], sp["version"], 4, 24, t.axis, t.neuron_len, len(t.shape))
+        cb = nvq1s_default_banks() if t.codebook is None else np.asarray(t.codebook)
+        table = pack_ternary_table(cb[0]) + pack_ternary_table(cb[1])
+    return b"".join([head, struct.pack(f"<{len(t.shape)}q", *t.shape), struct.pack("<I", out), table,
+                     np.ascontiguousarray(t.neuron_scale, dtype="<f2").tobytes(), pack_bits(t.sub_scale, t.state_bits),
+                     pack_bits(t.indices, sp["index_bits"]), pack_bits(t.delta_sign, 1)])
+
+
+def _lowbit_head(blob, label):
+    sp = LOWBIT_SPECS[label]
+    if len(blob) < _LOWBIT_HDR.size:
+        raise ValueError(f"truncated {label} header")
+    magic, ver, sbits, gs, axis, neuron_len, ndim = _LOWBIT_HDR.unpack_from(blob)
+    if magic != sp["magic"]:
+        raise ValueError(f"invalid {label} magic: {magic!r}")
+    if ndim <= 0 or neuron_len <= 0 or gs != 24:
+        raise ValueError(f"invalid {label} dimensions")
+    off = _LOWBIT_HDR.size
+    if off + 8 * ndim + 4 > len(blob):
+        raise ValueError(f"truncated {label} shape")
+    shape = tuple(struct.unpack_from(f"<{ndim}q", blob, off))
+    off += 8 * ndim
+    out = struct.unpack_from("<I", blob, off)[0]
+    return ver, sbits, axis, neuron_len, shape, out, off + 4
+
+
+def unpack_nvq1(blob, label) -> Nvq1Tensor:
+    """mfq/formats/nvq1_l.py:287-345, nvq1_s.py:293-347."""
+    sp = LOWBIT_SPECS[label]
+    ver, sbits, axis, K, shape, out, off = _lowbit_head(blob, label)
+    codebook = None
+    if label == "NVQ1-L":
+        if ver not in (1, 2):
+            raise ValueError(f"unsupported NVQ1-L profile: {ver}")
+        if not 1 <= sbits <= 8:
+            raise ValueError("NVQ1-L sub_bits must be in [1, 8]")
+        if ver == 2:
+            if off + 4096 > len(blob):
+                raise ValueError("truncated NVQ1-L custom codebook")
+            codebook = unpack_ternary_table(bytes(blob[off:off + 4096]))
+            off += 4096
+    else:
+        if ver != sp["version"] or sbits != 4 or K % 8:
+            raise ValueError("unsupported NVQ1-S stream profile")
+        if off + 2048 > len(blob):
+            raise ValueError("truncated NVQ1-S codebook")
+        codebook = np.stack([unpack_ternary_table(bytes(blob[off:off + 1024])),
+                             unpack_ternary_table(bytes(blob[off + 1024:off + 2048]))])
+        off += 2048
+    ng, nvec = _lowbit_counts(label, K)
+    if off + 2 * out > len(blob):
+        raise ValueError(f"truncated {label} neuron anchors")
+    ns = np.frombuffer(blob, dtype="<f2", count=out, offset=off).astype(np.float32)
+    off += 2 * out
+    sub, off = unpack_bits(blob, off, out * ng, sbits)
+    idx, off = unpack_bits(blob, off, out * nvec, sp["index_bits"])
+    dsg, off = unpack_bits(blob, off, out * ng, 1)
+    if off != len(blob):
+        raise ValueError(f"invalid {label} blob tail: consumed={off}, size={len(blob)}")
+    return Nvq1Tensor(label, shape, axis, K, sbits, ns, sub.reshape(out, ng), idx.reshape(out, nvec).astype(np.uint16),
+                      dsg.reshape(out, ng), codebook)
+
+
+def dequantize_nvq1(t: Nvq1Tensor) -> np.ndarray:
+    """w = fl(fl(anchor * sub_scale) * (code + delta)), delta = -/+ 1/8 (L) or 5/32 (S) by the group's sign bit, which
+    for NVQ1-S also picks the bank of all three vectors of the group (mfq/quantize/nvq1_l_quant.py:384-414,
+    nvq1_s_quant.py:142-174).  code + delta is exact in fp32."""
+    sp = LOWBIT_SPECS[t.label]
+    out, K = t.neuron_scale.size, t.neuron_len
+    idx = np.asarray(t.indices, dtype=np.int64)
+    if t.label == "NVQ1-L":
+        table = iq1s_grid() if t.codebook is None else np.asarray(t.codebook, dtype=np.int8)
+        code = table[idx]
+    else:
+        table = nvq1s_default_banks() if t.codebook is None else np.asarray(t.codebook, dtype=np.int8)
+        bank = np.repeat(np.asarray(t.delta_sign, dtype=np.int64), 3, axis=1)[:, : idx.shape[1]]
+        code = table[bank, idx]
+    code = code.reshape(out, -1)[:, :K].astype(np.float32)
+    d = np.float32(sp["delta"])
+    delta = np.repeat(np.where(np.asarray(t.delta_sign) != 0, -d, d).astype(np.float32), 24, axis=1)[:, :K]
+    scale = np.repeat(t.neuron_scale.astype(np.float32)[:, None] * np.asarray(t.sub_scale).astype(np.float32), 24, axis=1)[:, :K]
+    return (scale * (code + delta)).astype(np.float32)
+
+
+def pack_npq0_tables(t: Npq0Tensor) -> bytes:
+    """64-byte header (version, states, first / second index bits, 24, 8; fp16 scale LUT at byte 8), then the int8
+    sub-codebooks (mfq/formats/npq0_l.py:112-133, npq0_s.py:110-131)."""
+    sp = LOWBIT_SPECS[t.label]
+    head = bytearray(64)
+    head[0:6] = bytes([sp["table_version"], sp["states"], 3, sp["index_bits"] - 3, 24, 8])
+    head[8:8 + 2 * sp["states"]] = np.ascontiguousarray(t.scale_lut, dtype="<f2").tobytes()
+    return bytes(head) + np.ascontiguousarray(t.first_codebooks, dtype=np.int8).tobytes() + \
+        np.ascontiguousarray(t.second_codebooks, dtype=np.int8).tobytes()
+
+
+def pack_npq0(t: Npq0Tensor) -> bytes:
+    """mfq/formats/npq0_l.py:326-351, npq0_s.py:320-345."""
+    sp = LOWBIT_SPECS[t.label]
+    if t.neuron_len % 8:
+        raise ValueError(f"{t.label} neuron length must be divisible by 8")
+    return b"".join([_LOWBIT_HDR.pack(sp["magic"], sp["version"], sp["state_bits"], 24, t.axis, t.neuron_len, len(t.shape)),
+                     struct.pack(f"<{len(t.shape)}q", *t.shape), struct.pack("<I", t.neuron_scale.size), pack_npq0_tables(t),
+                     np.ascontiguousarray(t.neuron_scale, dtype="<f2").tobytes(), pack_bits(t.state, sp["state_bits"]),
+                     pack_bits(t.indices, sp["index_bits"])])
+
+
+def unpack_npq0(blob, label) -> Npq0Tensor:
+    """mfq/formats/npq0_l.py:354-415 (tables :136-185), npq0_s.py:348-406 (tables :134-183)."""
+    sp = LOWBIT_SPECS[label]
+    ver, sbits, axis, K, shape, out, off = _lowbit_head(blob, label)
+    if ver != sp["version"] or sbits != sp["state_bits"] or K % 8:
+        raise ValueError(f"unsupported {label} stream profile")
+    S, E2 = sp["states"], sp["second"]
+    tb = 64 + S * 8 * 4 + S * E2 * 4
+    if off + tb > len(blob):
+        raise ValueError(f"truncated {label} product tables")
+    head = bytes(blob[off:off + 64])
+    if tuple(head[:6]) != (sp["table_version"], S, 3, sp["index_bits"] - 3, 24, 8):
+        raise ValueError(f"unsupported {label} table profile")
+    if any(head[6:8]) or any(head[8 + 2 * S:64]):
+        raise ValueError(f"{label} reserved table bytes must be zero")
+    lut = np.frombuffer(head, dtype="<f2", count=S, offset=8).astype(np.float32)
+    if not np.isfinite(lut).all() or np.any(lut < 0) or float(lut.max()) <= 0:
+        raise ValueError(f"{label} scale LUT must be finite, non-negative, and nonzero")
+    first = np.frombuffer(blob, dtype=np.int8, count=S * 32, offset=off + 64).reshape(S, 8, 4).copy()
+    second = np.frombuffer(blob, dtype=np.int8, count=S * E2 * 4, offset=off + 64 + S * 32).reshape(S, E2, 4).copy()
+    off += tb
+    ng, nvec = _lowbit_counts(label, K)
+    if off + 2 * out > len(blob):
+        raise ValueError(f"truncated {label} neuron anchors")
+    ns = np.frombuffer(blob, dtype="<f2", count=out, offset=off).astype(np.float32)
+    off += 2 * out
+    state, off = unpack_bits(blob, off, out * ng, sbits)
+    idx, off = unpack_bits(blob, off, out * nvec, sp["index_bits"])
+    if off != len(blob):
+        raise ValueError(f"invalid {label} blob tail: consumed={off}, size={len(blob)}")
+    return Npq0Tensor(label, shape, axis, K, ns, lut, state.reshape(out, ng), idx.reshape(out, nvec), first, second)
+
+
+def dequantize_npq0(t: Npq0Tensor) -> np.ndarray:
+    """w = int8 code * fl(anchor * scale_lut[state]); a vector's first four weights come from first[state][index & 7],
+    the last four from second[state][index >> 3] (mfq/quantize/npq0_l.py:766-790, npq0_s.py:812-836)."""
+    out, K = t.neuron_scale.size, t.neuron_len
+    idx = np.asarray(t.indices, dtype=np.int64)
+    vs = np.repeat(np.asarray(t.state, dtype=np.int64), 3, axis=1)[:, : idx.shape[1]]
+    code = np.concatenate((np.asarray(t.first_codebooks, dtype=np.int8)[vs, idx & 7],
+                           np.asarray(t.second_codebooks, dtype=np.int8)[vs, idx >> 3]), axis=-1)
+    scale = np.repeat(t.neuron_scale.astype(np.float32)[:, None] * np.asarray(t.scale_lut, dtype=np.float32)[np.asarray(t.state)],
+                      24, axis=1)[:, :K]
+    return (code.reshape(out, K).astype(np.float32) * scale).astype(np.float32)
+
+
 def tensor_dtype(t) -> str:
     """Public dtype label (mfq/formats/io.py:576-640)."""
     if isinstance(t, NintTensor):
@@ -762,6 +995,8 @@ def tensor_dtype(t) -> str:
         return t.label
     if isinstance(t, NintMoeTensor):
         return "NINTM"
+    if isinstance(t, (Nvq1Tensor, Npq0Tensor)):
+        return t.label
     raise TypeError(type(t))
 
 
@@ -777,6 +1012,10 @@ def pack_tensor(t) -> tuple[str, bytes]:
         return dt, pack_nvq_plain(t)
     if isinstance(t, NepqTensor):
         return dt, pack_nepq(t)
+    if isinstance(t, Nvq1Tensor):
+        return dt, pack_nvq1(t)
+    if isinstance(t, Npq0Tensor):
+        return dt, pack_npq0(t)
     return dt, pack_nint_moe(t)
 
 
@@ -792,6 +1031,10 @@ def unpack_tensor(dtype: str, blob):
         return t
     if dtype == "NINT8-0":
         return unpack_nint8_zero(blob)
+    if dtype in ("NVQ1-L", "NVQ1-S"):
+        return unpack_nvq1(blob, dtype)
+    if dtype in ("NPQ0-L", "NPQ0-S"):
+        return unpack_npq0(blob, dtype)
     if dtype.startswith("NINT"):
         return unpack_nint(blob)
     if dtype.startswith("NVQ"):
@@ -871,6 +1114,10 @@ def dequantize_tensor(t) -> np.ndarray:
         return dequantize_nvq(t)
     if isinstance(t, NepqTensor):
         return dequantize_nepq(t)
+    if isinstance(t, Nvq1Tensor):
+        return dequantize_nvq1(t)
+    if isinstance(t, Npq0Tensor):
+        return dequantize_npq0(t)
     raise TypeError(type(t))
 
 

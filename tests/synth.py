@@ -50,6 +50,31 @@ def nvq_plain_random(rng, out, K):
                        rng.integers(0, 128, (out, nsign), dtype=np.uint8))
 
 
+def nvq1_random(rng, label, out, K, state_bits=3, custom=False):
+    """NVQ1-L (state_bits 3 or 4; custom: a permuted grid travels in the blob, else the built-in one) / NVQ1-S."""
+    ng = math.ceil(K / 24)
+    if label == "NVQ1-L":
+        nvec, entries = math.ceil(K / 8), 2048
+        cb = rng.permutation(O.iq1s_grid()) if custom else None
+    else:
+        nvec, entries, state_bits = K // 8, 512, 4
+        cb = np.stack([rng.permutation(O.iq1s_grid())[:512], rng.permutation(O.iq1s_grid())[:512]]) if custom else None
+    return O.Nvq1Tensor(label, (out, K), 0, K, state_bits, O._f16_round(rng.uniform(0.002, 0.02, out)),
+                        rng.integers(0, 1 << state_bits, (out, ng), dtype=np.uint8),
+                        rng.integers(0, entries, (out, nvec)).astype(np.uint16),
+                        rng.integers(0, 2, (out, ng), dtype=np.uint8), cb)
+
+
+def npq0_random(rng, label, out, K):
+    sp = O.LOWBIT_SPECS[label]
+    S, E2 = sp["states"], sp["second"]
+    ng, nvec = math.ceil(K / 24), K // 8
+    return O.Npq0Tensor(label, (out, K), 0, K, O._f16_round(rng.uniform(0.0002, 0.002, out)),
+                        O._f16_round(rng.uniform(0.25, 2.0, S)), rng.integers(0, S, (out, ng), dtype=np.uint8),
+                        rng.integers(0, 1 << sp["index_bits"], (out, nvec), dtype=np.uint8),
+                        rng.integers(-127, 128, (S, 8, 4)).astype(np.int8), rng.integers(-127, 128, (S, E2, 4)).astype(np.int8))
+
+
 def nepq_random(rng, label, E, out, K, banks):
     _, sb, ib, ab, tb = O.NEPQ_SPECS[label]
     iq1s = np.frombuffer((O._DATA / "iq1s_2048.bin").read_bytes(), dtype="<u2")

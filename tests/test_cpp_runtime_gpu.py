@@ -63,6 +63,10 @@ def test_check_linear_tool_reports_small_error(tmp_path):
         "blk.0.g.nvq3jl": synth.nvq_jsc_random(rng, 24, 104, "d4_1024", 4),
         "blk.0.v.nepq1s": synth.nepq_random(rng, "NEPQ1-S", 1, 48, 96, 3),
         "blk.0.o.nint8_0": O.quantize_nint8_zero((rng.standard_normal((40, 96)) * 0.02).astype(np.float32)),
+        "blk.1.q.nvq1l": synth.nvq1_random(rng, "NVQ1-L", 37, 100, 3, custom=True),   # the 1-bit families
+        "blk.1.k.nvq1s": synth.nvq1_random(rng, "NVQ1-S", 24, 104),
+        "blk.1.v.npq0l": synth.npq0_random(rng, "NPQ0-L", 40, 96),
+        "blk.1.o.npq0s": synth.npq0_random(rng, "NPQ0-S", 33, 200),
     }
     path = tmp_path / "tiny.mfq"
     O.mfq_file_write(path, tensors, version=2)

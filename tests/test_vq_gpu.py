@@ -370,3 +370,63 @@ def test_nvq2_plain_e8_with_both_sign_rules(sign_mode):
     assert np.array_equal(lin.dequantize().cpu().numpy().view(np.uint32), ref_w.astype(np.float32).view(np.uint32))
     with pytest.raises(ValueError, match="dtype/blob mismatch"):
         R.load_quant_linear("NVQ2J", ref_blob)
+
+
+LOWBIT_CASES = [("NVQ1-L", dict(state_bits=3)), ("NVQ1-L", dict(state_bits=4, custom=True)), ("NVQ1-S", dict()),
+                ("NVQ1-S", dict(custom=True)), ("NPQ0-L", dict()), ("NPQ0-S", dict())]
+
+
+@pytest.mark.parametrize("dtype,kw", LOWBIT_CASES)
+@pytest.mark.parametrize("out,K", [(37, 96), (24, 80), (70, 1544), (33, 104)])
+def test_one_bit_families_dequant_bit_exact_and_matmul(dtype, kw, out, K):
+    """NVQ1-L / NVQ1-S / NPQ0-L / NPQ0-S through the in-place stream kernels: dequantized weights bit for bit against the
+    oracle, the wave-per-neuron kernel for 1 / 4 / 13 rows, the fp16 GEMM path above 16 rows.  K = 100 (NVQ1-L only:
+    the other three need whole vectors) leaves a partial last vector and group."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import NvqsWeight, nvq_matmul
+    if dtype == "NVQ1-L" and K == 104:
+        K = 100
+    rng = np.random.default_rng(950 + out + K)
+    t = synth.nvq1_random(rng, dtype, out, K, **kw) if dtype.startswith("NVQ1") else synth.npq0_random(rng, dtype, out, K)
+    got_dtype, blob = O.pack_tensor(t)
+    assert got_dtype == dtype
+    lin = R.load_quant_linear(dtype, blob)
+    assert isinstance(lin.weight, NvqsWeight)
+    want = O.dequantize_tensor(O.unpack_tensor(dtype, blob))
+    got = lin.dequantize().cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    for M in (1, 4, 13):
+        for xd in (torch.bfloat16, torch.float16):
+            x, xf = _x(rng, M, K, xd)
+            _check(nvq_matmul(lin.weight, x).cpu().numpy(), O.linear_forward_f64(want, xf))
+    for M in (17, 70):
+        x, xf = _x(rng, M, K)
+        _check(lin(x).cpu().numpy(), O.linear_forward_f64(want, xf))
+
+
+def test_one_bit_families_reference_blobs_and_loader_errors():
+    """The reference-packed blobs of the golden fixture dequantize on the device to the values the reference computed;
+    malformed blobs are refused with the reference's messages before anything is uploaded."""
+    from pathlib import Path
+
+    from tyloquant_amd import runtime as R
+    gold = np.load(Path(__file__).resolve().parent / "golden" / "reference_lowbit.npz")
+    keys = {"nvq1l_grid": "NVQ1-L", "nvq1l_custom": "NVQ1-L", "nvq1s_default": "NVQ1-S", "nvq1s_custom": "NVQ1-S",
+            "npq0l": "NPQ0-L", "npq0s": "NPQ0-S"}
+    for key, dtype in keys.items():
+        blob = bytes(gold[f"{key}_blob"])
+        lin = R.load_quant_linear(dtype, blob)
+        got = lin.dequantize().cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), gold[f"{key}_deq"].astype(np.float32).view(np.uint32)), key
+        with pytest.raises(ValueError, match="blob tail"):
+            R.load_quant_linear(dtype, blob + b"\0")
+        with pytest.raises(ValueError, match="magic"):
+            R.load_quant_linear(dtype, b"ZZZZ" + blob[4:])
+    bad = bytearray(gold["npq0s_blob"].tobytes())
+    bad[20 + 16 + 4 + 0] = 9                                   # the table header's version byte
+    with pytest.raises(ValueError, match="unsupported NPQ0-S table profile"):
+        R.load_quant_linear("NPQ0-S", bytes(bad))
+    bad = bytearray(gold["nvq1s_custom_blob"].tobytes())
+    bad[20 + 16 + 4] = 0xFF                                    # digit 3 in a ternary entry
+    with pytest.raises(ValueError, match="non-ternary"):
+        R.load_quant_linear("NVQ1-S", bytes(bad))

@@ -14,6 +14,7 @@ LIB_PATH = _HERE / "lib" / "libmfq_hip.so"
 X_BF16, X_F16, X_F32 = 0, 1, 2
 TOPK_SOFTMAX, TOPK_SIGMOID, TOPK_SQRT_SOFTPLUS, TOPK_DELAYED_SOFTMAX = 0, 1, 2, 3
 GLU_SILU, GLU_GELU = 0, 1
+NVQS_NVQ1_L, NVQS_NVQ1_S, NVQS_NPQ0_L, NVQS_NPQ0_S = 1, 2, 3, 4
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_LAUNCH, ERR_WORKSPACE = 0, 1, 2, 3, 4
 
 i32, i64, vp, sz = C.c_int32, C.c_int64, C.c_void_p, C.c_size_t
@@ -36,7 +37,8 @@ class NvqsDesc(C.Structure):
     _fields_ = [(n, i32) for n in ("vector_size", "index_bits", "entries", "banks", "index_parity", "out", "neuron_len",
                                    "ng", "nvec", "nsign")] + \
                [(n, i64) for n in ("tables_off", "anchors_off", "state_off", "index_off", "sign_off", "total_bytes",
-                                   "payload_bytes")]
+                                   "payload_bytes")] + \
+               [("kind", i32), ("state_bits", i32), ("cb_bytes", i32), ("delta", C.c_float)]
 
 
 class NepqDesc(C.Structure):
@@ -102,6 +104,8 @@ _SIGS = {
     "mfq_hip_nvq_gemm": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
     "mfq_hip_nvqs_plan": (C.c_int, [C.c_int] * 6 + [C.POINTER(NvqsDesc)]),
     "mfq_hip_nvqs_repack": (C.c_int, [C.POINTER(NvqsDesc), vp, i64, C.c_int, vp, vp, vp]),
+    "mfq_hip_nvqs_plan_lowbit": (C.c_int, [C.c_int] * 4 + [C.POINTER(NvqsDesc)]),
+    "mfq_hip_nvqs_repack_lowbit": (C.c_int, [C.POINTER(NvqsDesc), vp, i64, vp, vp, vp]),
     "mfq_hip_nvqs_dequant_f32": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, i64, vp]),
     "mfq_hip_nvqs_gemv": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
     "mfq_hip_nvqs_gemm_workspace_bytes": (sz, [C.POINTER(NvqsDesc), C.c_int]),

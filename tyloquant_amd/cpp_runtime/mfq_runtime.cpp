@@ -39,6 +39,27 @@ T rd(const uint8_t *p, size_t off) {
     return v;
 }
 int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+float half_to_float(uint16_t h) {  // IEEE binary16 -> binary32, subnormals and specials included
+    const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16, exp = (h >> 10) & 31u, man = h & 0x3ffu;
+    uint32_t u;
+    if (exp == 0) {
+        if (man == 0) {
+            u = sign;
+        } else {
+            int e = -1;
+            uint32_t m = man;
+            do { ++e; m <<= 1; } while (!(m & 0x400u));
+            u = sign | static_cast<uint32_t>(127 - 15 - e) << 23 | (m & 0x3ffu) << 13;
+        }
+    } else if (exp == 31) {
+        u = sign | 0x7f800000u | man << 13;
+    } else {
+        u = sign | (exp + 112u) << 23 | man << 13;
+    }
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
 
 }  // namespace
 
@@ -277,6 +298,89 @@ Nint8ZeroWeight Nint8ZeroWeight::from_blob(const uint8_t *blob, size_t n, mfq_st
     return w;
 }
 
+// Header, shape and table checks of the reference's loaders for the 1-bit families, with their messages
+// (mfq/formats/nvq1_l.py:287-345, nvq1_s.py:293-347, npq0_l.py:354-415, npq0_s.py:348-406; mfq_decode.cpp:3800-3910).
+NvqWeight NvqWeight::from_lowbit_blob(const std::string &dtype, const uint8_t *b, size_t n, const uint16_t *iq1s_grid,
+                                      mfq_stream_t stream) {
+    struct Fmt { const char *magic; int version, state_bits, index_bits, format, table_version, states, second; };
+    static const std::unordered_map<std::string, Fmt> fmts = {
+        {"NVQ1-L", {"NQ1L", 0, 0, 11, MFQ_NVQS_NVQ1_L, 0, 0, 0}}, {"NVQ1-S", {"NQ1S", 1, 4, 9, MFQ_NVQS_NVQ1_S, 0, 0, 0}},
+        {"NPQ0-L", {"NPQL", 1, 3, 7, MFQ_NVQS_NPQ0_L, 1, 8, 16}}, {"NPQ0-S", {"NPQS", 2, 2, 6, MFQ_NVQS_NPQ0_S, 2, 4, 8}}};
+    const auto it = fmts.find(dtype);
+    if (it == fmts.end()) fail("unsupported quantized linear dtype: " + dtype);
+    const Fmt &f = it->second;
+    if (n < 20) fail("truncated " + dtype + " header");
+    if (std::memcmp(b, f.magic, 4) != 0) fail("invalid " + dtype + " magic");
+    const int ver = b[4], sbits = b[5], gs = rd<uint16_t>(b, 6), neuron_len = rd<int32_t>(b, 12);
+    const uint32_t ndim = rd<uint32_t>(b, 16);
+    const bool nvq1l = dtype == "NVQ1-L", ternary = dtype[1] == 'V';
+    if (nvq1l) {
+        if (ver != 1 && ver != 2) fail("unsupported NVQ1-L profile: " + std::to_string(ver));
+        if (gs != 24 || (sbits != 3 && sbits != 4)) fail("unsupported NVQ1-L profile");
+    } else if (ver != f.version || sbits != f.state_bits || gs != 24) {
+        fail("unsupported " + dtype + " stream profile");
+    }
+    if (ndim == 0 || ndim > 8 || neuron_len <= 0 || (!nvq1l && neuron_len % 8)) fail("invalid " + dtype + " dimensions");
+    size_t off = 20 + 8 * static_cast<size_t>(ndim);
+    if (n < off + 4) fail("truncated " + dtype + " shape");
+    int64_t elements = 1;
+    for (uint32_t i = 0; i < ndim; ++i) {
+        const int64_t v = rd<int64_t>(b, 20 + 8 * static_cast<size_t>(i));
+        if (v <= 0 || elements > INT64_MAX / v) fail(dtype + " shape does not match neuron dimensions");
+        elements *= v;
+    }
+    const int64_t out = rd<uint32_t>(b, off);
+    off += 4;
+    if (out <= 0 || out > INT32_MAX || elements != out * neuron_len) fail(dtype + " shape does not match neuron dimensions");
+    size_t table = 0;
+    if (nvq1l) table = ver == 2 ? 4096 : 0;
+    else if (ternary) table = 2048;
+    else {
+        table = 64 + static_cast<size_t>(f.states) * 32 + static_cast<size_t>(f.states) * f.second * 4;
+        if (n < off + table) fail("truncated " + dtype + " product tables");
+        const uint8_t *t = b + off;
+        if (t[0] != f.table_version || t[1] != f.states || t[2] != 3 || t[3] != f.index_bits - 3 || t[4] != 24 || t[5] != 8)
+            fail("unsupported " + dtype + " table profile");
+        bool reserved = t[6] || t[7];
+        for (int i = 8 + 2 * f.states; i < 64; ++i) reserved = reserved || t[i];
+        if (reserved) fail("invalid " + dtype + " reserved table bytes");
+        float lmax = 0.f;
+        for (int i = 0; i < f.states; ++i) {
+            const float v = half_to_float(rd<uint16_t>(t, 8 + 2 * static_cast<size_t>(i)));
+            if (!(v >= 0.f) || std::isinf(v)) fail(dtype + " scale LUT must be finite and non-negative");
+            lmax = std::max(lmax, v);
+        }
+        if (lmax <= 0.f) fail(dtype + " scale LUT must be finite and non-negative");
+    }
+    if (ternary && table) {
+        if (n < off + table) fail("truncated " + dtype + " codebook");
+        for (size_t i = 0; i < table / 2; ++i) {
+            const uint16_t e = rd<uint16_t>(b, off + 2 * i);
+            if (e & (e >> 1) & 0x5555u) fail("packed " + dtype + " codebook contains a non-ternary digit");
+        }
+    }
+    const int64_t ng = cdiv(neuron_len, 24), nvec = nvq1l ? cdiv(neuron_len, 8) : neuron_len / 8;
+    const int64_t streams = 2 * out + (out * ng * sbits + 7) / 8 + (out * nvec * f.index_bits + 7) / 8 +
+                            (ternary ? (out * ng + 7) / 8 : 0);
+    const int64_t expect = static_cast<int64_t>(table) + streams;
+    if (static_cast<int64_t>(n) - static_cast<int64_t>(off) != expect)
+        fail("invalid " + dtype + " blob tail: remaining=" + std::to_string(n - off) + ", expected=" + std::to_string(expect));
+    NvqWeight w;
+    w.dtype = dtype;
+    w.streams = true;
+    abi_check(mfq_hip_nvqs_plan_lowbit(f.format, sbits, static_cast<int>(out), neuron_len, &w.sdesc));
+    DeviceBuffer body = DeviceBuffer::from_host(b + off, static_cast<size_t>(expect));
+    DeviceBuffer grid;
+    if (nvq1l && !table) {
+        if (!iq1s_grid) fail("an NVQ1-L blob without a table needs the built-in 2048-entry ternary grid");
+        grid = DeviceBuffer::from_host(iq1s_grid, 4096);
+    }
+    w.data = DeviceBuffer(static_cast<size_t>(w.sdesc.total_bytes));
+    abi_check(mfq_hip_nvqs_repack_lowbit(&w.sdesc, body.get(), expect, grid.get(), w.data.get(), stream));
+    hip_check(hipStreamSynchronize(hs(stream)), "1-bit family repack");
+    return w;
+}
+
 NvqWeight NvqWeight::from_blob(const uint8_t *blob, size_t n, const int8_t *grid256, mfq_stream_t stream) {
     const NvqHeader h = parse_nvq(blob, n);
     NvqWeight w;
@@ -491,6 +595,7 @@ bool is_nvq_linear_dtype(const std::string &d) {
            d == "NVQ2J-XL" || d == "NIQ3" || d == "NIQ2" || d == "NIQ2J";
 }
 bool is_nepq_linear_dtype(const std::string &d) { return d == "NEPQ1-S" || d == "NEPQ1-L"; }
+bool is_lowbit_linear_dtype(const std::string &d) { return d == "NVQ1-L" || d == "NVQ1-S" || d == "NPQ0-L" || d == "NPQ0-S"; }
 
 int64_t QuantLinear::out() const {
     return kind == QuantLinearKind::Nint ? nint->out() : kind == QuantLinearKind::Nvq ? nvq->out()
@@ -561,6 +666,11 @@ QuantLinear load_quant_linear(const std::string &dtype_in, const uint8_t *blob, 
         q.kind = QuantLinearKind::Nvq;
         q.nvq = std::make_shared<NvqWeight>(NvqWeight::from_blob(blob, n, nullptr, stream));
         if (q.nvq->dtype != dtype) fail("MFQ dtype/blob mismatch: " + dtype + " contains " + q.nvq->dtype);
+        return q;
+    }
+    if (is_lowbit_linear_dtype(dtype)) {
+        q.kind = QuantLinearKind::Nvq;
+        q.nvq = std::make_shared<NvqWeight>(NvqWeight::from_lowbit_blob(dtype, blob, n, nullptr, stream));
         return q;
     }
     if (is_nepq_linear_dtype(dtype)) {

@@ -120,7 +120,13 @@ struct NvqWeight {
     // NVQ2; JSC tensors carry their codebooks
     static NvqWeight from_blob(const uint8_t *blob, size_t n, const int8_t *grid256 = nullptr,
                                mfq_stream_t stream = nullptr);
+    // The 1-bit families NVQ1-L / NVQ1-S / NPQ0-L / NPQ0-S (formats 1, 8, 7, 9 of the reference's unpack_nvq,
+    // cpp_runtime/mfq_decode.cpp:3759-3770, 3800-3910), on the in-place stream kernels.  `iq1s_grid` = the built-in
+    // 2048-entry ternary grid as packed uint16 (2 bits per digit), needed only by an NVQ1-L blob that carries no table.
+    static NvqWeight from_lowbit_blob(const std::string &dtype, const uint8_t *blob, size_t n,
+                                      const uint16_t *iq1s_grid = nullptr, mfq_stream_t stream = nullptr);
 };
+bool is_lowbit_linear_dtype(const std::string &dtype);
 struct NepqWeight {
     mfq_nepq_desc desc{};
     DeviceBuffer data;

@@ -3,6 +3,9 @@
 // of the lane-major D4 layout (nvq.hip) cannot hold.  The device weight is the payload itself with its tables
 // widened: no re-layout, every field is fetched by bit offset.  A wave owns a neuron, its lanes the 8-weight sign
 // blocks of the row, so the three streams of a neuron are read as consecutive bytes.
+// The 1-bit families ride on the same machinery: NVQ1-L / NVQ1-S (kind 1: ternary 8-dimensional codebooks, an integer
+// relative scale and a delta sign per group, the sign also choosing NVQ1-S's bank) and NPQ0-L / NPQ0-S (kind 2: two
+// 4-dimensional int8 sub-codebooks and a relative scale chosen by the group's state).
 #include "common.hpp"
 #include "gemv_common.hpp"
 #include "tune.hpp"
@@ -14,6 +17,8 @@ struct NvqsK {
     int out, neuron_len, ng, nvec, nsign;
     int64_t tables_off, anchors_off, state_off, index_off, sign_off;
     int64_t state_bytes, index_bytes, sign_bytes;
+    int kind, sbits, cb_bytes;  // kind 0: sign-stream NVQ; 1: ternary + delta (sign_off = the delta-sign stream); 2: product
+    float delta, magmax;        // magmax: bound of |magnitude| for the fp16 row scaling
 };
 
 static NvqsK to_k(const mfq_nvqs_desc *d) {
@@ -22,9 +27,12 @@ static NvqsK to_k(const mfq_nvqs_desc *d) {
     k.out = d->out; k.neuron_len = d->neuron_len; k.ng = d->ng; k.nvec = d->nvec; k.nsign = d->nsign;
     k.tables_off = d->tables_off; k.anchors_off = d->anchors_off; k.state_off = d->state_off; k.index_off = d->index_off;
     k.sign_off = d->sign_off;
-    k.state_bytes = (static_cast<int64_t>(d->out) * d->ng * 4 + 7) / 8;
+    k.kind = d->kind; k.sbits = d->state_bits; k.cb_bytes = d->cb_bytes; k.delta = d->delta;
+    k.magmax = d->kind == 1 ? 2.f : 127.f;
+    k.state_bytes = (static_cast<int64_t>(d->out) * d->ng * d->state_bits + 7) / 8;
     k.index_bytes = (static_cast<int64_t>(d->out) * d->nvec * d->index_bits + 7) / 8;
-    k.sign_bytes = (static_cast<int64_t>(d->out) * d->nsign * 7 + 7) / 8;
+    k.sign_bytes = d->kind == 0 ? (static_cast<int64_t>(d->out) * d->nsign * 7 + 7) / 8
+                                : (d->kind == 1 ? (static_cast<int64_t>(d->out) * d->ng + 7) / 8 : 0);
     return k;
 }
 
@@ -52,12 +60,36 @@ template <class CB>
 __device__ __forceinline__ NvqsBlock nvqs_block(const NvqsK &k, const uint8_t *w, const float *lut, const uint32_t *bfs,
                                                 CB cb, float anchor, int n, int sb) {
     const uint8_t *st_s = w + k.state_off, *ix_s = w + k.index_off, *sg_s = w + k.sign_off;
-    const uint32_t mask = stream_bits(sg_s, (static_cast<int64_t>(n) * k.nsign + sb) * 7, 7);
-    const int g = sb / 3;  // groups of 24 weights = three sign blocks
-    const uint32_t state = stream_bits(st_s, (static_cast<int64_t>(n) * k.ng + g) * 4, 4);
-    const uint32_t bank = bfs[state];
+    const int g = sb / 3;  // groups of 24 weights = three 8-weight blocks
+    const uint32_t state = stream_bits(st_s, (static_cast<int64_t>(n) * k.ng + g) * k.sbits, k.sbits);
     NvqsBlock b;
     b.scale = __fmul_rn(anchor, lut[state]);
+    if (k.kind == 1) {
+        // w = fl(anchor * sub_scale) * (code + delta): delta = -d / +d by the group's sign bit, which with two banks also
+        // names the bank (mfq/quantize/nvq1_l_quant.py:384-414, nvq1_s_quant.py:142-174); code + delta is exact
+        const uint32_t neg = stream_bits(sg_s, static_cast<int64_t>(n) * k.ng + g, 1);
+        const uint32_t idx = sb < k.nvec ? stream_bits(ix_s, (static_cast<int64_t>(n) * k.nvec + sb) * k.ib, k.ib) : 0u;
+        const int64_t e = (static_cast<int64_t>(k.banks == 2 ? neg : 0u) * k.entries + idx) * 8;
+        const float dl = neg ? -k.delta : k.delta;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) b.mag[i] = static_cast<float>(cb(e + i)) + dl;
+        return b;
+    }
+    if (k.kind == 2) {
+        // a vector = first[state][index & 7] | second[state][index >> 3], four int8 weights each
+        // (mfq/quantize/npq0_l.py:766-790, npq0_s.py:812-836); banks = states, entries = second sub-codebook entries
+        const uint32_t idx = sb < k.nvec ? stream_bits(ix_s, (static_cast<int64_t>(n) * k.nvec + sb) * k.ib, k.ib) : 0u;
+        const int64_t e1 = (static_cast<int64_t>(state) * 8 + (idx & 7u)) * 4;
+        const int64_t e2 = static_cast<int64_t>(k.banks) * 32 + (static_cast<int64_t>(state) * k.entries + (idx >> 3)) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            b.mag[i] = static_cast<float>(cb(e1 + i));
+            b.mag[4 + i] = static_cast<float>(cb(e2 + i));
+        }
+        return b;
+    }
+    const uint32_t mask = stream_bits(sg_s, (static_cast<int64_t>(n) * k.nsign + sb) * 7, 7);
+    const uint32_t bank = bfs[state];
     uint32_t last = __popc(mask) & 1u;
     if (k.vs == 8) {
         const uint32_t idx = stream_bits(ix_s, (static_cast<int64_t>(n) * k.nvec + sb) * k.ib, k.ib);
@@ -112,6 +144,44 @@ __global__ __launch_bounds__(256) void nvqs_repack_kernel(NvqsK k, const uint8_t
     for (int64_t i = tid; i < k.sign_bytes + 4; i += nthreads) dst[k.sign_off + i] = i < k.sign_bytes ? sg[i] : 0;
 }
 
+// The 1-bit families.  body: [tables] | fp16 anchors | state stream | index stream | [delta-sign stream].  Tables:
+// kind 1 -- packed ternary entries (2 bits per digit, digit = code + 1, a uint16 per entry) from the body when
+// table_in_body, else from `grid` (the built-in 2048-entry grid); kind 2 -- a 64-byte header with the fp16 scale LUT at
+// byte 8, then the int8 sub-codebooks, copied as they are.
+__global__ __launch_bounds__(256) void nvqs_repack_lowbit_kernel(NvqsK k, const uint8_t *__restrict__ body, int table_in_body,
+                                                                 const uint16_t *__restrict__ grid, uint8_t *__restrict__ dst) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x, nthreads = static_cast<int64_t>(gridDim.x) * 256;
+    float *lut = reinterpret_cast<float *>(dst + k.tables_off);
+    uint32_t *bfs = reinterpret_cast<uint32_t *>(lut + 16);
+    int8_t *cb = reinterpret_cast<int8_t *>(bfs + 16);
+    int64_t table_bytes = 0;
+    if (k.kind == 1) {
+        const int64_t nent = static_cast<int64_t>(k.banks) * k.entries;
+        table_bytes = table_in_body ? 2 * nent : 0;
+        if (tid < 16) { lut[tid] = static_cast<float>(tid); bfs[tid] = 0u; }
+        for (int64_t i = tid; i < nent * 8; i += nthreads) {
+            const int64_t e = i >> 3;
+            const uint32_t enc = table_in_body ? (body[2 * e] | (static_cast<uint32_t>(body[2 * e + 1]) << 8)) : grid[e];
+            cb[i] = static_cast<int8_t>(static_cast<int>((enc >> (2 * (i & 7))) & 3u) - 1);
+        }
+    } else {
+        table_bytes = 64 + k.cb_bytes;
+        if (tid < 16) {
+            lut[tid] = tid < k.banks ? f16_to_f32(static_cast<uint16_t>(body[8 + 2 * tid] | (body[9 + 2 * tid] << 8))) : 0.f;
+            bfs[tid] = 0u;
+        }
+        for (int64_t i = tid; i < k.cb_bytes; i += nthreads) cb[i] = static_cast<int8_t>(body[64 + i]);
+    }
+    const uint8_t *streams = body + table_bytes;
+    float *anchors = reinterpret_cast<float *>(dst + k.anchors_off);
+    for (int64_t i = tid; i < k.out; i += nthreads)
+        anchors[i] = f16_to_f32(static_cast<uint16_t>(streams[2 * i] | (streams[2 * i + 1] << 8)));
+    const uint8_t *st = streams + 2 * static_cast<int64_t>(k.out), *ix = st + k.state_bytes, *sg = ix + k.index_bytes;
+    for (int64_t i = tid; i < k.state_bytes + 4; i += nthreads) dst[k.state_off + i] = i < k.state_bytes ? st[i] : 0;
+    for (int64_t i = tid; i < k.index_bytes + 4; i += nthreads) dst[k.index_off + i] = i < k.index_bytes ? ix[i] : 0;
+    for (int64_t i = tid; i < k.sign_bytes + 4; i += nthreads) dst[k.sign_off + i] = i < k.sign_bytes ? sg[i] : 0;
+}
+
 // ---- dequant -------------------------------------------------------------------------------------------------------
 // One thread per (neuron, sign block).  OutT = float: the bit-exact dequantizer.  OutT = uint16_t: fp16 rows scaled by a
 // power of two per neuron (rowscale receives its reciprocal), zero-padded to kpad columns, for the fp16 GEMM.
@@ -127,7 +197,7 @@ __global__ __launch_bounds__(256) void nvqs_dequant_kernel(NvqsK k, const uint8_
     if constexpr (sizeof(OutT) == 2) {
         float lmax = 0.f;
         for (int i = 0; i < 16; ++i) lmax = fmaxf(lmax, lut[i]);
-        const float bound = anchor * lmax * 127.f;
+        const float bound = anchor * lmax * k.magmax;
         int e = 0;
         if (bound > 0.f) frexpf(bound, &e);
         inv = ldexpf(1.f, 12 - e);
@@ -162,7 +232,7 @@ __global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *
     const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
     const int8_t *cbp = reinterpret_cast<const int8_t *>(bfs + 16);
     if constexpr (CB_LDS) {
-        const int ncb = k.banks * k.entries * k.vs;
+        const int ncb = k.cb_bytes;
         for (int i = threadIdx.x * 4; i < ncb; i += blockDim.x * 4)
             *reinterpret_cast<uint32_t *>(cbl + i) = *reinterpret_cast<const uint32_t *>(cbp + i);
         __syncthreads();
@@ -224,7 +294,7 @@ constexpr int kNvqsGemvMaxM = 16;  // rows up to which the weights are re-read p
 template <int XF16, int MB>
 static int nvqs_launch_gemv(const NvqsK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                             hipStream_t st) {
-    const size_t ncb = static_cast<size_t>(k.banks) * k.entries * k.vs;
+    const size_t ncb = static_cast<size_t>(k.cb_bytes);
     const dim3 grid(static_cast<unsigned>(ceil_div(k.out, 4)), static_cast<unsigned>(ceil_div(M, MB)));
     if (ncb <= 49152 && ncb % 4 == 0)
         hipLaunchKernelGGL((nvqs_gemv_kernel<XF16, MB, true>), grid, dim3(256), ncb, st, k, w, x, ldx, M, y, ldy);
@@ -263,7 +333,69 @@ extern "C" int mfq_hip_nvqs_plan(int vector_size, int index_bits, int banks, int
     d->sign_off = d->index_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(ix) + 4));
     d->total_bytes = d->sign_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(sg) + 4));
     d->payload_bytes = 2ll * out + st + ix + sg;
+    d->kind = 0; d->state_bits = 4; d->cb_bytes = static_cast<int32_t>(ncb); d->delta = 0.f;
     return MFQ_OK;
+}
+
+extern "C" int mfq_hip_nvqs_plan_lowbit(int format, int state_bits, int out, int neuron_len, mfq_nvqs_desc *d) {
+    MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nvqs_plan_lowbit: null descriptor");
+    MFQ_REQUIRE(out > 0 && neuron_len > 0, MFQ_ERR_INVALID, "nvqs_plan_lowbit: empty tensor");
+    d->vector_size = 8; d->index_parity = 0; d->out = out; d->neuron_len = neuron_len;
+    d->ng = static_cast<int32_t>(ceil_div(neuron_len, 24));
+    d->nsign = static_cast<int32_t>(ceil_div(neuron_len, 8));
+    d->nvec = d->nsign;
+    switch (format) {
+    case MFQ_NVQS_NVQ1_L:
+        MFQ_REQUIRE(state_bits == 3 || state_bits == 4, MFQ_ERR_UNSUPPORTED, "unsupported NVQ1-L profile: %d-bit scales", state_bits);
+        d->kind = 1; d->index_bits = 11; d->entries = 2048; d->banks = 1; d->state_bits = state_bits; d->delta = 0.125f;
+        d->cb_bytes = 2048 * 8;
+        break;
+    case MFQ_NVQS_NVQ1_S:
+        MFQ_REQUIRE(neuron_len % 8 == 0, MFQ_ERR_INVALID, "NVQ1-S neuron length must be divisible by 8");
+        d->kind = 1; d->index_bits = 9; d->entries = 512; d->banks = 2; d->state_bits = 4; d->delta = 0.15625f;
+        d->cb_bytes = 2 * 512 * 8;
+        break;
+    case MFQ_NVQS_NPQ0_L:
+        MFQ_REQUIRE(neuron_len % 8 == 0, MFQ_ERR_INVALID, "NPQ0-L neuron length must be divisible by 8");
+        d->kind = 2; d->index_bits = 7; d->entries = 16; d->banks = 8; d->state_bits = 3; d->delta = 0.f;
+        d->cb_bytes = 8 * 32 + 8 * 16 * 4;
+        break;
+    case MFQ_NVQS_NPQ0_S:
+        MFQ_REQUIRE(neuron_len % 8 == 0, MFQ_ERR_INVALID, "NPQ0-S neuron length must be divisible by 8");
+        d->kind = 2; d->index_bits = 6; d->entries = 8; d->banks = 4; d->state_bits = 2; d->delta = 0.f;
+        d->cb_bytes = 4 * 32 + 4 * 8 * 4;
+        break;
+    default:
+        return fail(MFQ_ERR_INVALID, "nvqs_plan_lowbit: format=%d", format);
+    }
+    const int64_t st = (static_cast<int64_t>(out) * d->ng * d->state_bits + 7) / 8;
+    const int64_t ix = (static_cast<int64_t>(out) * d->nvec * d->index_bits + 7) / 8;
+    const int64_t sg = d->kind == 1 ? (static_cast<int64_t>(out) * d->ng + 7) / 8 : 0;
+    d->tables_off = 0;
+    d->anchors_off = static_cast<int64_t>(nvqs_align(128 + static_cast<size_t>(d->cb_bytes)));
+    d->state_off = d->anchors_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(out) * 4));
+    d->index_off = d->state_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(st) + 4));
+    d->sign_off = d->index_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(ix) + 4));
+    d->total_bytes = d->sign_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(sg) + 4));
+    d->payload_bytes = 2ll * out + st + ix + sg;
+    return MFQ_OK;
+}
+
+extern "C" int mfq_hip_nvqs_repack_lowbit(const mfq_nvqs_desc *d, const void *body, int64_t body_bytes, const void *grid,
+                                          void *weight, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && body && weight, MFQ_ERR_INVALID, "nvqs_repack_lowbit: null argument");
+    MFQ_REQUIRE(d->kind == 1 || d->kind == 2, MFQ_ERR_INVALID, "nvqs_repack_lowbit: not a 1-bit family descriptor");
+    const int64_t table = d->kind == 1 ? 2ll * d->banks * d->entries : 64ll + d->cb_bytes;
+    const bool builtin = d->kind == 1 && d->banks == 1 && body_bytes == d->payload_bytes;  // NVQ1-L without a table
+    MFQ_REQUIRE(builtin || body_bytes == d->payload_bytes + table, MFQ_ERR_INVALID,
+                "nvqs_repack_lowbit: body is %lld bytes, the tensor needs %lld", static_cast<long long>(body_bytes),
+                static_cast<long long>(d->payload_bytes + table));
+    MFQ_REQUIRE(!builtin || grid, MFQ_ERR_INVALID, "nvqs_repack_lowbit: a blob without a table needs the built-in grid");
+    const NvqsK k = to_k(d);
+    hipLaunchKernelGGL(nvqs_repack_lowbit_kernel, dim3(1024), dim3(256), 0, as_stream(stream), k,
+                       static_cast<const uint8_t *>(body), builtin ? 0 : 1, static_cast<const uint16_t *>(grid),
+                       static_cast<uint8_t *>(weight));
+    return check_launch("nvqs_repack_lowbit");
 }
 
 extern "C" int mfq_hip_nvqs_repack(const mfq_nvqs_desc *d, const void *payload, int64_t payload_bytes, int jsc,

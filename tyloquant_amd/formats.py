@@ -277,6 +277,100 @@ def nvq_plain_blob(codebook, neuron_len, ns, sub_scale, indices, signs, gs=24, s
         pack_bitstream(signs, 7)])
 
 
+# ---------------------------------------------------------------------------
+# The 1-bit families: NVQ1-L / NVQ1-S / NPQ0-L / NPQ0-S (mfq/formats/nvq1_l.py, nvq1_s.py, npq0_l.py, npq0_s.py)
+# ---------------------------------------------------------------------------
+# dtype: magic, header byte (None: profile 1 or 2), state bits (None: in the header), index bits, table bytes in the blob
+LOWBIT_FORMATS = {
+    "NVQ1-L": (b"NQ1L", None, None, 11),
+    "NVQ1-S": (b"NQ1S", 1, 4, 9),
+    "NPQ0-L": (b"NPQL", 1, 3, 7),
+    "NPQ0-S": (b"NPQS", 2, 2, 6),
+}
+_NPQ0_TABLES = {"NPQ0-L": (1, 8, 16), "NPQ0-S": (2, 4, 8)}   # table version, states, second sub-codebook entries
+
+
+@dataclass
+class LowbitHeader:
+    dtype: str
+    state_bits: int
+    out: int
+    neuron_len: int
+    body_off: int      # tables (if the blob has them), fp16 anchors, streams
+    body_bytes: int
+    table_bytes: int
+
+
+def is_lowbit_dtype(dtype: str) -> bool:
+    return dtype in LOWBIT_FORMATS
+
+
+def lowbit_stream_bytes(dtype: str, out: int, neuron_len: int, state_bits: int) -> int:
+    """anchors + state / scale stream + index stream (+ delta-sign stream), every stream packed across the tensor
+    (mfq/formats/nvq1_l.py:157-169, nvq1_s.py:188-199, npq0_l.py:228-238, npq0_s.py:226-236)."""
+    ib = LOWBIT_FORMATS[dtype][3]
+    ng = -(-neuron_len // 24)
+    nvec = -(-neuron_len // 8) if dtype == "NVQ1-L" else neuron_len // 8
+    n = 2 * out + (out * ng * state_bits + 7) // 8 + (out * nvec * ib + 7) // 8
+    return n + ((out * ng + 7) // 8 if dtype.startswith("NVQ1") else 0)
+
+
+def parse_lowbit(dtype: str, blob) -> LowbitHeader:
+    """Header, shape and table checks of unpack_nvq1_l / unpack_nvq1_s / unpack_npq0_l / unpack_npq0_s (and of the C++
+    loader, cpp_runtime/mfq_decode.cpp:3800-3910), with their messages."""
+    magic, ver_want, sbits_want, _ = LOWBIT_FORMATS[dtype]
+    if len(blob) < _NVQ_HDR.size:
+        raise ValueError(f"truncated {dtype} header")
+    m, ver, sbits, gs, axis, neuron_len, ndim = _NVQ_HDR.unpack_from(blob, 0)
+    if m != magic:
+        raise ValueError(f"invalid {dtype} magic: {m!r}")
+    if dtype == "NVQ1-L":
+        if ver not in (1, 2):
+            raise ValueError(f"unsupported NVQ1-L profile: {ver}")
+        if gs != 24 or sbits not in (3, 4):
+            raise ValueError("unsupported NVQ1-L profile")
+    elif ver != ver_want or sbits != sbits_want or gs != 24:
+        raise ValueError(f"unsupported {dtype} stream profile")
+    if ndim <= 0 or neuron_len <= 0 or (dtype != "NVQ1-L" and neuron_len % 8):
+        raise ValueError(f"invalid {dtype} dimensions")
+    off = _NVQ_HDR.size
+    if off + 8 * ndim + 4 > len(blob):
+        raise ValueError(f"truncated {dtype} shape")
+    shape = struct.unpack_from(f"<{ndim}q", blob, off)
+    off += 8 * ndim
+    out = struct.unpack_from("<I", blob, off)[0]
+    off += 4
+    if out <= 0 or int(np.prod(shape)) != out * neuron_len:
+        raise ValueError(f"{dtype} shape does not match neuron dimensions")
+    if dtype == "NVQ1-L":
+        table = 4096 if ver == 2 else 0
+    elif dtype == "NVQ1-S":
+        table = 2048
+    else:
+        tv, states, second = _NPQ0_TABLES[dtype]
+        table = 64 + states * 32 + states * second * 4
+        if off + table > len(blob):
+            raise ValueError(f"truncated {dtype} product tables")
+        head = bytes(blob[off:off + 64])
+        if tuple(head[:6]) != (tv, states, 3, LOWBIT_FORMATS[dtype][3] - 3, 24, 8):
+            raise ValueError(f"unsupported {dtype} table profile")
+        if any(head[6:8]) or any(head[8 + 2 * states:64]):
+            raise ValueError(f"invalid {dtype} reserved table bytes")
+        lut = np.frombuffer(head, dtype="<f2", count=states, offset=8).astype(np.float32)
+        if not np.isfinite(lut).all() or np.any(lut < 0) or float(lut.max()) <= 0:
+            raise ValueError(f"{dtype} scale LUT must be finite and non-negative")
+    if table and dtype.startswith("NVQ1"):
+        if off + table > len(blob):
+            raise ValueError(f"truncated {dtype} codebook")
+        enc = np.frombuffer(blob, dtype="<u2", count=table // 2, offset=off)
+        if np.any(((enc[:, None] >> (2 * np.arange(8, dtype=np.uint16))[None, :]) & 3) > 2):
+            raise ValueError(f"packed {dtype} codebook contains a non-ternary digit")
+    expect = table + lowbit_stream_bytes(dtype, out, neuron_len, sbits)
+    if len(blob) - off != expect:
+        raise ValueError(f"invalid {dtype} blob tail: remaining={len(blob) - off}, expected={expect}")
+    return LowbitHeader(dtype, sbits, out, neuron_len, off, expect, table)
+
+
 def parse_nvq(blob) -> NvqHeader:
     if len(blob) < _NVQ_HDR.size:
         raise ValueError("truncated NVQ header")

@@ -390,6 +390,9 @@ def load_quant_linear(dtype: str, blob, device="cuda") -> QuantLinear:
         if w.dtype != dtype:
             raise ValueError(f"MFQ dtype/blob mismatch: {dtype} contains {w.dtype}")
         return QuantLinear("nvq", w)
+    if F.is_lowbit_dtype(dtype):
+        from .runtime_vq import NvqsWeight
+        return QuantLinear("nvq", NvqsWeight.from_lowbit_blob(dtype, blob, device))
     if is_nepq_linear_dtype(dtype):
         from .runtime_vq import NepqWeight
         w = NepqWeight.from_blob(blob, device)

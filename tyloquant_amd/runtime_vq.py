@@ -94,6 +94,26 @@ class NvqsWeight:
         torch.cuda.current_stream().synchronize()
         return NvqsWeight(desc, data, h.dtype)
 
+    @staticmethod
+    def from_lowbit_blob(dtype: str, blob, device="cuda") -> "NvqsWeight":
+        """NVQ1-L / NVQ1-S / NPQ0-L / NPQ0-S (formats 1, 8, 7, 9 of the reference's unpack_nvq,
+        cpp_runtime/mfq_decode.cpp:3759-3770): the same in-place streams, ternary or product codebooks."""
+        h = F.parse_lowbit(dtype, blob)
+        device = torch.device(device)
+        desc = L.NvqsDesc()
+        lib = L.lib()
+        fmt = {"NVQ1-L": L.NVQS_NVQ1_L, "NVQ1-S": L.NVQS_NVQ1_S, "NPQ0-L": L.NVQS_NPQ0_L, "NPQ0-S": L.NVQS_NPQ0_S}[dtype]
+        L.check(lib.mfq_hip_nvqs_plan_lowbit(fmt, h.state_bits, h.out, h.neuron_len, C.byref(desc)))
+        body = _upload(blob, h.body_off, h.body_bytes, device)
+        data = torch.empty(int(desc.total_bytes), dtype=torch.uint8, device=device)
+        grid = None
+        if dtype == "NVQ1-L" and h.table_bytes == 0:      # the built-in 2048-entry ternary grid, packed
+            raw = np.frombuffer((_DATA / "iq1s_2048.bin").read_bytes(), dtype=np.uint8)
+            grid = torch.from_numpy(raw.copy()).to(device)
+        L.check(lib.mfq_hip_nvqs_repack_lowbit(C.byref(desc), _ptr(body), h.body_bytes, _ptr(grid), _ptr(data), _stream()))
+        torch.cuda.current_stream().synchronize()
+        return NvqsWeight(desc, data, dtype)
+
     def dequantize(self) -> torch.Tensor:
         w = torch.empty((self.out, self.neuron_len), dtype=torch.float32, device=self.data.device)
         L.check(L.lib().mfq_hip_nvqs_dequant_f32(C.byref(self.desc), _ptr(self.data), _ptr(w), self.neuron_len, _stream()))
