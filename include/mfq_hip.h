@@ -486,6 +486,13 @@ int mfq_hip_moe_decode_matmul(const mfq_moe_pool *pools, int n_pools, const int3
 int mfq_hip_moe_decode_capable(const mfq_moe_pool *pools, int n_pools, int out_per_expert, int K,
                                const mfq_nint_desc *shared_desc, int T, int R, int swiglu);
 
+/* Row gather / scatter for hosts that walk a batch expert by expert (cohorts of families the grouped kernels do not
+ * hold): scatter == 0: dst row i = src row index[i]; scatter != 0: dst row index[i] = src row i, i < n.  Rows of
+ * row_bytes bytes (a multiple of 4), strides in bytes; index is a device array.  Stands in for the index_select /
+ * index_copy_ pair of the reference's per-expert walk over a mixed-family tensor (cpp_runtime/mfq_decode.cpp:17607-17629). */
+int mfq_hip_moe_move_rows(const void *src, int64_t src_stride, const int32_t *index, int n, int row_bytes, int scatter,
+                          void *dst, int64_t dst_stride, mfq_stream_t stream);
+
 /* hidden[r, c] = silu(gate_up[r, c]) * gate_up[r, W + c]  (moe_swiglu_split_cuda,
  * mfq/kernels/cuda/moe.cu:2980-2996); output fp16 (x_dtype MFQ_X_F16) or bf16. */
 int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,

@@ -217,6 +217,46 @@ def test_cpp_moe_ffn_forward(rt, T):
     rt.mfq_rt_free_nint_moe(hd)
 
 
+def _mixed_moe(rng, E_out, K):
+    """Eight experts in four cohorts of different families (NINT4, NVQ3J-512, NVQ1-S, NEPQ1-S)."""
+    def pool(ids, dtype, t):
+        return O.MoePool(np.asarray(ids, dtype=np.int32), dtype, t)
+    return O.NintMoeTensor((8, E_out, K), [
+        pool([0, 5, 7], "NINT4", synth.nint_random(rng, 3 * E_out, K, 4, 32, 6)),
+        pool([1, 4], "NVQ3J-512", synth.nvq_jsc_random(rng, 2 * E_out, K, "d4_512", 2)),
+        pool([2], "NVQ1-S", synth.nvq1_random(rng, "NVQ1-S", E_out, K)),
+        pool([6, 3], "NEPQ1-S", synth.nepq_random(rng, "NEPQ1-S", 2, E_out, K, 3))])
+
+
+@pytest.mark.parametrize("T", [3, 40])
+def test_cpp_moe_ffn_with_cohorts_of_other_families(rt, T):
+    """Gate/up and down tensors whose cohorts mix NINT with NVQ, a 1-bit family and NEPQ: the C++ runtime splits the
+    foreign cohorts into per-expert tensors and walks the routed experts on the host; the layer against the oracle."""
+    rng = np.random.default_rng(140 + T)
+    E, H, W, k = 8, 192, 96, 3
+    tg, td = _mixed_moe(rng, 2 * W, H), _mixed_moe(rng, H, W)
+    bg, bd = O.pack_nint_moe(tg), O.pack_nint_moe(td)
+    hg, hd = C.c_void_p(), C.c_void_p()
+    assert rt.mfq_rt_load_nint_moe(bg, len(bg), C.byref(hg)) == 0, rt.mfq_rt_last_error()
+    assert rt.mfq_rt_load_nint_moe(bd, len(bd), C.byref(hd)) == 0, rt.mfq_rt_last_error()
+    x = torch.from_numpy((rng.standard_normal((T, H)) * 3).astype(np.float32)).to(torch.bfloat16).cuda()
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    lg = torch.from_numpy(logits).cuda()
+    out = torch.empty((T, H), dtype=torch.float32, device="cuda")
+    ids = torch.empty((T, k), dtype=torch.int32, device="cuda")
+    wts = torch.empty((T, k), dtype=torch.float32, device="cuda")
+    rc = rt.mfq_rt_moe_ffn_forward(hg, hd, x.data_ptr(), 0, H, T, lg.data_ptr(), k, 3, 0, None, None, out.data_ptr(),
+                                   ids.data_ptr(), wts.data_ptr(), None)
+    assert rc == 0, rt.mfq_rt_last_error()
+    torch.cuda.synchronize()
+    ref, rids, rw = O.moe_ffn(O.dequantize_expertwise(tg), O.dequantize_expertwise(td), x.float().cpu().numpy(), logits, k,
+                              delayed_softmax=True)
+    assert np.array_equal(ids.cpu().numpy(), rids)
+    check_close(out.cpu().numpy(), ref)
+    rt.mfq_rt_free_nint_moe(hg)
+    rt.mfq_rt_free_nint_moe(hd)
+
+
 def test_cpp_nvq_ffn_swiglu_down(rt):
     """nvq_ffn_swiglu_down of the C++ runtime (joint gate/up launch, SwiGLU kernel, down projection) against the
     oracle's float64 evaluation of the dequantized weights; the hidden rows pass through fp16."""

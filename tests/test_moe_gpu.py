@@ -362,3 +362,59 @@ def test_mapped_path_with_hundreds_of_experts_and_skewed_routes():
     fused = w.forward_glu(x.cuda(), route).float().cpu().numpy()
     g, u = ref[..., : out // 2], ref[..., out // 2:]
     assert rel_l2(fused, g / (1.0 + np.exp(-g)) * u) < 5e-3
+
+
+def _mixed_family_moe(rng, out, K):
+    """Nine experts in five cohorts: NINT4 (3 experts), NVQ3J-512 (2), NVQ2J read from its streams (1), NPQ0-S (1),
+    NEPQ1-S (2)."""
+    def pool(ids, dtype, t):
+        return O.MoePool(np.asarray(ids, dtype=np.int32), dtype, t)
+    pools = [pool([0, 4, 8], "NINT4", synth.nint_random(rng, 3 * out, K, 4, 32, 6)),
+             pool([1, 6], "NVQ3J-512", synth.nvq_jsc_random(rng, 2 * out, K, "d4_512", 2)),
+             pool([2], "NVQ2J", synth.nvq_jsc_random(rng, out, K, "e8_256", 2)),
+             pool([5], "NPQ0-S", synth.npq0_random(rng, "NPQ0-S", out, K)),
+             pool([3, 7], "NEPQ1-S", synth.nepq_random(rng, "NEPQ1-S", 2, out, K, 3))]
+    return O.NintMoeTensor((9, out, K), pools)
+
+
+def test_mixed_family_cohorts_in_one_tensor():
+    """A NINTM tensor whose cohorts belong to different families: the NINT cohort on the grouped kernels, every other
+    expert on its family's kernels through the host's per-expert walk.  Dequantized experts bit for bit, the routed
+    product against the oracle's loop for a mapped batch, a decode-sized batch and routed (per-pair) inputs; a tensor
+    without any NINT cohort; the residency cache declines such a tensor."""
+    from tyloquant_amd.runtime_moe import MoeExpertCache, NintMoeWeight, build_moe_route_plan
+    rng = np.random.default_rng(77)
+    out, K, E, R = 32, 192, 9, 3
+    t = _mixed_family_moe(rng, out, K)
+    blob = O.pack_nint_moe(t)
+    w = NintMoeWeight.from_blob(blob)
+    assert len(w.pools) == 1 and [c.dtype for c in w.foreign] == ["NVQ3J-512", "NVQ2J", "NPQ0-S", "NEPQ1-S"]
+    dense = O.dequantize_expertwise(t)
+    assert np.array_equal(w.dequantize().cpu().numpy().view(np.uint32), dense.view(np.uint32))
+    assert not w.decode_capable(None, 1, R)
+    for T in (40, 2):
+        ids = np.stack([rng.choice(E, size=R, replace=False) for _ in range(T)]).astype(np.int32)
+        x = torch.from_numpy((rng.standard_normal((T, K)) * 0.1).astype(np.float32)).to(torch.bfloat16)
+        route = build_moe_route_plan(torch.from_numpy(ids).cuda(), E)
+        got = w(x.cuda(), route).cpu().numpy()
+        ref = O.moe_grouped_matmul(dense, x.float().numpy(), ids)
+        assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL
+        xr = torch.from_numpy((rng.standard_normal((T, R, K)) * 0.1).astype(np.float32)).to(torch.bfloat16)
+        got = w(xr.cuda(), route).cpu().numpy()
+        ref = np.stack([np.stack([dense[ids[t_, r]] @ xr[t_, r].float().numpy() for r in range(R)]) for t_ in range(T)])
+        assert rel_l2(got, ref) < REL_TOL
+        h = w.forward_glu(x.cuda(), route).float().cpu().numpy()
+        y = O.moe_grouped_matmul(dense, x.float().numpy(), ids)
+        assert rel_l2(h, O.moe_swiglu(y)) < 5e-3
+    only = O.NintMoeTensor((3, out, K), [O.MoePool(np.array([2, 0], dtype=np.int32), "NVQ3J-512",
+                                                   synth.nvq_jsc_random(rng, 2 * out, K, "d4_512", 2)),
+                                         O.MoePool(np.array([1], dtype=np.int32), "NVQ1-S",
+                                                   synth.nvq1_random(rng, "NVQ1-S", out, K))])
+    w2 = NintMoeWeight.from_blob(O.pack_nint_moe(only))
+    d2 = O.dequantize_expertwise(only)
+    ids = np.stack([rng.choice(3, size=2, replace=False) for _ in range(20)]).astype(np.int32)
+    x = torch.from_numpy((rng.standard_normal((20, K)) * 0.1).astype(np.float32)).to(torch.bfloat16)
+    got = w2(x.cuda(), build_moe_route_plan(torch.from_numpy(ids).cuda(), 3)).cpu().numpy()
+    assert rel_l2(got, O.moe_grouped_matmul(d2, x.float().numpy(), ids)) < REL_TOL
+    with pytest.raises(NotImplementedError, match="NINT cohorts only"):
+        MoeExpertCache(1 << 20).register_source(blob)

@@ -104,6 +104,7 @@ _SIGS = {
     "mfq_hip_nvq_gemm": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
     "mfq_hip_nvqs_plan": (C.c_int, [C.c_int] * 6 + [C.POINTER(NvqsDesc)]),
     "mfq_hip_nvqs_repack": (C.c_int, [C.POINTER(NvqsDesc), vp, i64, C.c_int, vp, vp, vp]),
+    "mfq_hip_moe_move_rows": (C.c_int, [vp, i64, vp, C.c_int, C.c_int, C.c_int, vp, i64, vp]),
     "mfq_hip_nvqs_plan_lowbit": (C.c_int, [C.c_int] * 4 + [C.POINTER(NvqsDesc)]),
     "mfq_hip_nvqs_repack_lowbit": (C.c_int, [C.POINTER(NvqsDesc), vp, i64, vp, vp, vp]),
     "mfq_hip_nvqs_dequant_f32": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, i64, vp]),

@@ -298,6 +298,79 @@ Nint8ZeroWeight Nint8ZeroWeight::from_blob(const uint8_t *blob, size_t n, mfq_st
     return w;
 }
 
+namespace {
+// bits [bit0, bit0 + nbits) of the little-endian bit stream at s (which has `avail` readable bytes), as a stream of its own
+std::vector<uint8_t> slice_bits(const uint8_t *s, size_t avail, int64_t bit0, int64_t nbits) {
+    std::vector<uint8_t> out(static_cast<size_t>((nbits + 7) / 8), 0);
+    const int sh = static_cast<int>(bit0 & 7);
+    for (size_t i = 0; i < out.size(); ++i) {
+        const size_t b = static_cast<size_t>(bit0 >> 3) + i;
+        const uint32_t lo = b < avail ? s[b] : 0u, hi = b + 1 < avail ? s[b + 1] : 0u;
+        out[i] = static_cast<uint8_t>(((lo | (hi << 8)) >> sh) & 0xffu);
+    }
+    if (nbits & 7) out.back() &= static_cast<uint8_t>((1u << (nbits & 7)) - 1u);
+    return out;
+}
+}  // namespace
+
+std::vector<std::vector<uint8_t>> split_rows(const std::string &dtype, const uint8_t *b, size_t n, int parts) {
+    size_t body_off, tables;
+    int64_t out, K;
+    std::vector<int64_t> per_row;
+    if (is_lowbit_linear_dtype(dtype)) {
+        if (n < 20) fail("truncated " + dtype + " header");
+        const int ver = b[4], sbits = b[5];
+        K = rd<int32_t>(b, 12);
+        const uint32_t ndim = rd<uint32_t>(b, 16);
+        if (ndim == 0 || ndim > 8 || K <= 0 || n < 24 + 8 * static_cast<size_t>(ndim)) fail("invalid " + dtype + " dimensions");
+        out = rd<uint32_t>(b, 20 + 8 * static_cast<size_t>(ndim));
+        body_off = 24 + 8 * static_cast<size_t>(ndim);
+        const bool nvq1l = dtype == "NVQ1-L", ternary = dtype[1] == 'V';
+        tables = nvq1l ? (ver == 2 ? 4096 : 0) : dtype == "NVQ1-S" ? 2048 : dtype == "NPQ0-L" ? 832 : 320;
+        const int ib = nvq1l ? 11 : dtype == "NVQ1-S" ? 9 : dtype == "NPQ0-L" ? 7 : 6;
+        const int64_t ng = cdiv(K, 24), nvec = nvq1l ? cdiv(K, 8) : K / 8;
+        per_row = {sbits * ng, ib * nvec};
+        if (ternary) per_row.push_back(ng);
+    } else {
+        const NvqHeader h = parse_nvq(b, n);
+        body_off = h.body_off; out = h.out; K = h.neuron_len;
+        tables = h.jsc ? 64 + static_cast<size_t>(h.banks) * (1ull << h.index_bits) * h.vector_size : 0;
+        per_row = {static_cast<int64_t>(h.sub_bits) * cdiv(K, h.gs), static_cast<int64_t>(h.index_bits) * cdiv(K, h.vector_size),
+                   7 * cdiv(K, 8)};
+    }
+    if (parts <= 0 || out <= 0 || out % parts) fail(dtype + ": " + std::to_string(out) + " neurons do not split into " +
+                                                     std::to_string(parts) + " equal parts");
+    const int64_t rows = out / parts;
+    const size_t anchors_off = body_off + tables;
+    std::vector<size_t> stream_off;
+    size_t off = anchors_off + 2 * static_cast<size_t>(out);
+    for (int64_t bits : per_row) {
+        stream_off.push_back(off);
+        off += static_cast<size_t>((out * bits + 7) / 8);
+    }
+    if (off != n) fail("invalid " + dtype + " blob tail: consumed=" + std::to_string(off) + ", size=" + std::to_string(n));
+    std::vector<std::vector<uint8_t>> res;
+    for (int i = 0; i < parts; ++i) {
+        std::vector<uint8_t> piece(b, b + 8);  // magic, flags / version, state bits, groupsize
+        auto put = [&](const void *p, size_t bytes) {
+            const uint8_t *q = static_cast<const uint8_t *>(p);
+            piece.insert(piece.end(), q, q + bytes);
+        };
+        const int32_t axis = 0, k32 = static_cast<int32_t>(K);
+        const uint32_t ndim = 2, o32 = static_cast<uint32_t>(rows);
+        const int64_t shape[2] = {rows, K};
+        put(&axis, 4); put(&k32, 4); put(&ndim, 4); put(shape, 16); put(&o32, 4);
+        put(b + body_off, tables);
+        put(b + anchors_off + 2 * static_cast<size_t>(i * rows), 2 * static_cast<size_t>(rows));
+        for (size_t si = 0; si < per_row.size(); ++si) {
+            const std::vector<uint8_t> bits = slice_bits(b + stream_off[si], n - stream_off[si], i * rows * per_row[si], rows * per_row[si]);
+            put(bits.data(), bits.size());
+        }
+        res.push_back(std::move(piece));
+    }
+    return res;
+}
+
 // Header, shape and table checks of the reference's loaders for the 1-bit families, with their messages
 // (mfq/formats/nvq1_l.py:287-345, nvq1_s.py:293-347, npq0_l.py:354-415, npq0_s.py:348-406; mfq_decode.cpp:3800-3910).
 NvqWeight NvqWeight::from_lowbit_blob(const std::string &dtype, const uint8_t *b, size_t n, const uint16_t *iq1s_grid,
@@ -715,13 +788,33 @@ NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream
     std::vector<int32_t> ep(h.n_experts, -1), el(h.n_experts, -1);
     for (size_t pi = 0; pi < h.pools.size(); ++pi) {
         const NintmPool &p = h.pools[pi];
-        if (!is_nint_linear_dtype(p.dtype)) fail("NINTM cohort family " + p.dtype + " is not on the accelerated path");
         if (p.runtime_bytes) fail("unexpected NINTM cohort runtime metadata");
+        const std::string shape_error = "NINTM pool " + std::to_string(pi) + " tensor shape does not match its expert count";
+        if (!is_nint_linear_dtype(p.dtype)) {
+            MoeForeignCohort c;
+            c.dtype = p.dtype; c.expert_ids = p.expert_ids;
+            const int parts = static_cast<int>(p.expert_ids.size());
+            if (is_nepq_linear_dtype(p.dtype)) {
+                c.nepq = std::make_shared<NepqWeight>(NepqWeight::from_blob(blob + p.payload_off, p.payload_bytes, nullptr, stream));
+                if (c.nepq->label != p.dtype) fail("MFQ dtype/blob mismatch: " + p.dtype + " contains " + c.nepq->label);
+                if (c.nepq->n_experts != parts || c.nepq->out_per_expert != h.out_per_expert || c.nepq->neuron_len() != h.neuron_len)
+                    fail(shape_error);
+            } else if (is_nvq_linear_dtype(p.dtype) || is_lowbit_linear_dtype(p.dtype)) {
+                for (const auto &piece : split_rows(p.dtype, blob + p.payload_off, p.payload_bytes, parts)) {
+                    c.linears.push_back(load_quant_linear(p.dtype, piece.data(), piece.size(), stream));
+                    if (c.linears.back().out() != h.out_per_expert || c.linears.back().neuron_len() != h.neuron_len) fail(shape_error);
+                }
+            } else {
+                fail("NINTM cohort family " + p.dtype + " is not supported");
+            }
+            w.foreign.push_back(std::move(c));
+            continue;
+        }
         auto pw = std::make_shared<NintWeight>(NintWeight::from_blob(blob + p.payload_off, p.payload_bytes, stream));
         if (pw->out() != static_cast<int64_t>(p.expert_ids.size()) * h.out_per_expert || pw->neuron_len() != h.neuron_len)
-            fail("NINTM pool " + std::to_string(pi) + " tensor shape does not match its expert count");
+            fail(shape_error);
         for (size_t i = 0; i < p.expert_ids.size(); ++i) {
-            ep[p.expert_ids[i]] = static_cast<int32_t>(pi);
+            ep[p.expert_ids[i]] = static_cast<int32_t>(w.pool_table.size());
             el[p.expert_ids[i]] = static_cast<int32_t>(i);
         }
         w.pool_table.push_back(mfq_moe_pool{pw->desc, pw->data.get()});
@@ -733,8 +826,72 @@ NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream
     return w;
 }
 
+int64_t MoeForeignCohort::payload_bytes() const {
+    if (nepq) return nepq->desc.payload_bytes;
+    int64_t n = 0;
+    for (const QuantLinear &q : linears) n += q.payload_bytes();
+    return n;
+}
+void MoeForeignCohort::matmul(int local, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const {
+    if (nepq) nepq_matmul(*nepq, local, x, x_dtype, ldx, M, y, stream);
+    else linears[static_cast<size_t>(local)].forward(x, x_dtype, ldx, M, y, stream);
+}
+void MoeForeignCohort::dequantize(int local, float *out, mfq_stream_t stream) const {
+    if (!nepq) { linears[static_cast<size_t>(local)].dequantize(out, stream); return; }
+    // the cohort dequantizes as a whole: take the expert's rows out of it
+    const size_t rows = static_cast<size_t>(nepq->out_per_expert), K = static_cast<size_t>(nepq->neuron_len());
+    DeviceBuffer all(static_cast<size_t>(nepq->n_experts) * rows * K * 4);
+    abi_check(mfq_hip_nepq_dequant_f32(&nepq->desc, nepq->data.get(), static_cast<float *>(all.get()), static_cast<int64_t>(K), stream));
+    hip_check(hipMemcpyAsync(out, static_cast<const float *>(all.get()) + static_cast<size_t>(local) * rows * K, rows * K * 4,
+                             hipMemcpyDeviceToDevice, hs(stream)), "foreign cohort dequantize");
+    hip_check(hipStreamSynchronize(hs(stream)), "foreign cohort dequantize");
+}
+
+void NintMoeWeight::add_foreign(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &r, float *out,
+                                mfq_stream_t stream) const {
+    if (foreign.empty()) return;
+    if (neuron_len % 2 || ldx % 2) fail("mixed NINTM cohorts need activation rows of whole 32-bit words");
+    const int T = r.tokens, R = r.routes;
+    std::vector<int32_t> ids(static_cast<size_t>(T) * R);
+    hip_check(hipStreamSynchronize(hs(stream)), "mixed NINTM: routing table");
+    hip_check(hipMemcpy(ids.data(), r.ids, 4 * ids.size(), hipMemcpyDeviceToHost), "mixed NINTM: routing table");
+    std::vector<int32_t> index;  // per expert: n pair rows, then n source rows
+    for (const MoeForeignCohort &c : foreign) {
+        for (size_t local = 0; local < c.expert_ids.size(); ++local) {
+            const int32_t e = c.expert_ids[local];
+            std::vector<int32_t> pair_rows, src_rows;
+            for (int t = 0; t < T; ++t)
+                for (int k = 0; k < R; ++k)
+                    if (ids[static_cast<size_t>(t) * R + k] == e) {
+                        pair_rows.push_back(t * R + k);
+                        src_rows.push_back(routed_input ? t * R + k : t);
+                    }
+            const int n = static_cast<int>(pair_rows.size());
+            if (!n) continue;
+            index = pair_rows;
+            index.insert(index.end(), src_rows.begin(), src_rows.end());
+            f_index.ensure(8ull * n);
+            f_x.ensure(2ull * n * neuron_len);
+            f_y.ensure(4ull * n * out_per_expert);
+            // the three buffers are reused by the next expert: the copy below waits for the previous expert's kernels
+            hip_check(hipStreamSynchronize(hs(stream)), "mixed NINTM: expert walk");
+            hip_check(hipMemcpy(f_index.get(), index.data(), 8ull * n, hipMemcpyHostToDevice), "mixed NINTM: row lists");
+            const int32_t *d_pairs = static_cast<const int32_t *>(f_index.get()), *d_src = d_pairs + n;
+            abi_check(mfq_hip_moe_move_rows(x, 2 * ldx, d_src, n, 2 * neuron_len, 0, f_x.get(), 2ll * neuron_len, stream));
+            c.matmul(static_cast<int>(local), f_x.get(), x_dtype, neuron_len, n, static_cast<float *>(f_y.get()), stream);
+            abi_check(mfq_hip_moe_move_rows(f_y.get(), 4ll * out_per_expert, d_pairs, n, 4 * out_per_expert, 1, out,
+                                            4ll * out_per_expert, stream));
+        }
+    }
+}
+
 void NintMoeWeight::forward(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &r, float *out,
                             mfq_stream_t stream) const {
+    if (pools.empty()) {  // no NINT cohort at all: every row comes from the host's walk
+        hip_check(hipMemsetAsync(out, 0, 4ull * r.tokens * r.routes * out_per_expert, hs(stream)), "mixed NINTM: clear");
+        add_foreign(x, x_dtype, ldx, routed_input, r, out, stream);
+        return;
+    }
     const bool mapped = r.mapped();
     // a workspace lets the library take the prefill kernel when a mapped call has many pairs per expert
     const int x_rows = routed_input ? r.tokens * r.routes : r.tokens;
@@ -750,13 +907,14 @@ void NintMoeWeight::forward(const void *x, int x_dtype, int64_t ldx, bool routed
         mapped ? static_cast<const int32_t *>(r.tile_bounds.get()) : nullptr,
         mapped ? static_cast<const int32_t *>(r.tile_experts.get()) : nullptr, out, out_per_expert,
         need ? workspace.get() : nullptr, need, stream));
+    add_foreign(x, x_dtype, ldx, routed_input, r, out, stream);
 }
 
 void NintMoeWeight::forward_glu(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &r, bool gelu,
                                 void *hidden, float *scratch, mfq_stream_t stream) const {
     const int W = out_per_expert / 2, pairs = r.tokens * r.routes;
     const int activation = gelu ? MFQ_GLU_GELU : MFQ_GLU_SILU;
-    if (r.mapped() && out_per_expert % 32 == 0) {
+    if (r.mapped() && out_per_expert % 32 == 0 && foreign.empty()) {
         const int x_rows = routed_input ? pairs : r.tokens;
         const size_t need =
             mfq_hip_moe_grouped_workspace_bytes(pool_table.data(), static_cast<int>(pool_table.size()), neuron_len, x_rows);
@@ -777,7 +935,7 @@ void NintMoeWeight::forward_glu(const void *x, int x_dtype, int64_t ldx, bool ro
 }
 
 bool NintMoeWeight::decode_capable(const NintWeight *shared, int tokens, int routes, bool swiglu) const {
-    if (shared && shared->desc.neuron_len != neuron_len) return false;
+    if (!foreign.empty() || (shared && shared->desc.neuron_len != neuron_len)) return false;
     return mfq_hip_moe_decode_capable(pool_table.data(), static_cast<int>(pool_table.size()), out_per_expert, neuron_len,
                                       shared ? &shared->desc : nullptr, tokens, routes, swiglu ? 1 : 0) != 0;
 }
@@ -854,6 +1012,8 @@ MoeExpertCache::~MoeExpertCache() {
 MoeCachedSource *MoeExpertCache::register_source(const uint8_t *blob, size_t n, int minimum_slots) {
     if (finalized_) fail("cannot register a MoE source after cache finalization");
     NintMoeWeight full = NintMoeWeight::from_blob(blob, n);
+    if (!full.foreign.empty())
+        fail("expert residency holds NINT cohorts only; this tensor has a " + full.foreign[0].dtype + " cohort");
     auto src = std::make_unique<MoeCachedSource>();
     src->n_experts = full.n_experts; src->out_per_expert = full.out_per_expert; src->neuron_len = full.neuron_len;
     src->cohort_of.assign(full.n_experts, -1);

@@ -223,10 +223,33 @@ struct MoeRoutePlan {
 MoeRoutePlan build_moe_route_plan(const int32_t *ids, int tokens, int routes, int n_experts,
                                   mfq_stream_t stream = nullptr);
 
+// Cuts an NVQ-family or 1-bit-family blob of parts * n neurons into `parts` blobs of n neurons each: same flags and
+// tables, the rows' anchors and their share of every tensor-wide bit stream re-packed from bit 0.
+std::vector<std::vector<uint8_t>> split_rows(const std::string &dtype, const uint8_t *blob, size_t n, int parts);
+
+// A NINTM cohort of another family (NVQ, the 1-bit families, NEPQ).  The reference runs them inside its grouped kernels
+// (cpp_runtime/mfq_decode.cpp:4800-5360); here every expert is a tensor of its own on that family's kernels and the host
+// walks the experts a batch routes to -- correct, one matmul per expert hit, not a fast path.
+struct MoeForeignCohort {
+    std::string dtype;
+    std::vector<int32_t> expert_ids;
+    std::vector<QuantLinear> linears;   // one per expert (NVQ, 1-bit families)
+    std::shared_ptr<NepqWeight> nepq;   // or the cohort as one expert-shaped tensor
+    int64_t payload_bytes() const;
+    void matmul(int local, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const;
+    void dequantize(int local, float *out, mfq_stream_t stream) const;  // [out_per_expert, K]
+};
+
 struct NintMoeWeight {
     int n_experts = 0, out_per_expert = 0, neuron_len = 0;
     std::vector<std::shared_ptr<NintWeight>> pools;
     std::vector<std::vector<int32_t>> pool_expert_ids;
+    std::vector<MoeForeignCohort> foreign;  // experts the grouped kernels skip (dispatch entry -1): added by add_foreign
+    mutable DeviceBuffer f_index, f_x, f_y;
+    // rows of the pairs routed to foreign experts: gather, multiply, scatter into out [T*R, out_per_expert]; reads the
+    // routing table on the host (synchronizes the stream)
+    void add_foreign(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &route, float *out,
+                     mfq_stream_t stream) const;
     DeviceBuffer expert_pool, expert_local;  // int32 [E] dispatch tables
     std::vector<mfq_moe_pool> pool_table;
     mutable DeviceBuffer workspace;  // prefill path, grown on demand (do not grow it under graph capture)

@@ -928,6 +928,31 @@ extern "C" int mfq_hip_moe_glu(const float *gate_up, int64_t ld, int rows, int W
     return check_launch("moe_glu");
 }
 
+namespace mfq {
+// dst row i = src row index[i] (gather), or dst row index[i] = src row i (scatter): rows of row_bytes bytes, a multiple
+// of 4, as 32-bit words
+__global__ __launch_bounds__(256) void moe_move_rows_kernel(const uint8_t *__restrict__ src, int64_t src_stride,
+                                                            const int32_t *__restrict__ index, int row_bytes, int scatter,
+                                                            uint8_t *__restrict__ dst, int64_t dst_stride) {
+    const int i = blockIdx.x, j = index[i];
+    const uint32_t *s = reinterpret_cast<const uint32_t *>(src + static_cast<int64_t>(scatter ? i : j) * src_stride);
+    uint32_t *d = reinterpret_cast<uint32_t *>(dst + static_cast<int64_t>(scatter ? j : i) * dst_stride);
+    for (int c = threadIdx.x; c < row_bytes / 4; c += blockDim.x) d[c] = s[c];
+}
+}  // namespace mfq
+
+extern "C" int mfq_hip_moe_move_rows(const void *src, int64_t src_stride, const int32_t *index, int n, int row_bytes,
+                                     int scatter, void *dst, int64_t dst_stride, mfq_stream_t stream) {
+    MFQ_REQUIRE(src && index && dst, MFQ_ERR_INVALID, "moe_move_rows: null argument");
+    MFQ_REQUIRE(n > 0 && row_bytes > 0 && row_bytes % 4 == 0 && src_stride % 4 == 0 && dst_stride % 4 == 0 &&
+                    (reinterpret_cast<uintptr_t>(src) & 3) == 0 && (reinterpret_cast<uintptr_t>(dst) & 3) == 0,
+                MFQ_ERR_INVALID, "moe_move_rows: rows must be made of whole aligned 32-bit words");
+    hipLaunchKernelGGL(moe_move_rows_kernel, dim3(static_cast<unsigned>(n)), dim3(256), 0, as_stream(stream),
+                       static_cast<const uint8_t *>(src), src_stride, index, row_bytes, scatter ? 1 : 0,
+                       static_cast<uint8_t *>(dst), dst_stride);
+    return check_launch("moe_move_rows");
+}
+
 extern "C" int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, int W, void *hidden, int out_dtype,
                                   int64_t ldh, mfq_stream_t stream) {
     return mfq_hip_moe_glu(gate_up, ld, rows, W, hidden, out_dtype, ldh, MFQ_GLU_SILU, stream);

@@ -371,6 +371,48 @@ def parse_lowbit(dtype: str, blob) -> LowbitHeader:
     return LowbitHeader(dtype, sbits, out, neuron_len, off, expect, table)
 
 
+def _slice_bits(buf, byte_off: int, bit0: int, nbits: int) -> bytes:
+    """Bits [bit0, bit0 + nbits) of the little-endian bit stream that starts at byte_off, as a stream of its own."""
+    b0, b1 = bit0 // 8, (bit0 + nbits + 7) // 8
+    bits = np.unpackbits(np.frombuffer(buf, dtype=np.uint8, count=b1 - b0, offset=byte_off + b0), bitorder="little")
+    return np.packbits(bits[bit0 - 8 * b0: bit0 - 8 * b0 + nbits], bitorder="little").tobytes()
+
+
+def split_rows(dtype: str, blob, parts: int) -> list[bytes]:
+    """Cut an NVQ-family or 1-bit-family tensor of parts * n neurons into `parts` blobs of n neurons each (the experts of a
+    NINTM cohort, cpp_runtime/mfq_decode.cpp:4800-5360): same header flags and tables, the anchors and the rows' share
+    of every tensor-wide bit stream re-packed from bit 0."""
+    blob = bytes(blob)
+    if is_lowbit_dtype(dtype):
+        h = parse_lowbit(dtype, blob)
+        ib = LOWBIT_FORMATS[dtype][3]
+        ng = -(-h.neuron_len // 24)
+        nvec = -(-h.neuron_len // 8) if dtype == "NVQ1-L" else h.neuron_len // 8
+        per_row = [h.state_bits * ng, ib * nvec] + ([ng] if dtype.startswith("NVQ1") else [])
+        tables, out, K = h.table_bytes, h.out, h.neuron_len
+    else:
+        h = parse_nvq(blob)
+        per_row = [h.sub_bits * h.ng, h.index_bits * h.nvec, 7 * h.nsign]
+        tables = 64 + h.banks * (1 << h.index_bits) * h.vector_size if h.jsc else 0
+        out, K = h.out, h.neuron_len
+    if parts <= 0 or out % parts:
+        raise ValueError(f"{dtype}: {out} neurons do not split into {parts} equal parts")
+    n = out // parts
+    head8 = blob[:8]                                         # magic, flags / version, state bits, groupsize
+    anchors_off = h.body_off + tables
+    stream_off, off = [], anchors_off + 2 * out
+    for bits in per_row:
+        stream_off.append(off)
+        off += (out * bits + 7) // 8
+    res = []
+    for i in range(parts):
+        piece = [head8, struct.pack("<iiI", 0, K, 2), struct.pack("<2q", n, K), struct.pack("<I", n),
+                 blob[h.body_off:h.body_off + tables], blob[anchors_off + 2 * i * n: anchors_off + 2 * (i + 1) * n]]
+        piece += [_slice_bits(blob, so, i * n * bits, n * bits) for so, bits in zip(stream_off, per_row)]
+        res.append(b"".join(piece))
+    return res
+
+
 def parse_nvq(blob) -> NvqHeader:
     if len(blob) < _NVQ_HDR.size:
         raise ValueError("truncated NVQ header")

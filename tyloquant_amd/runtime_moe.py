@@ -89,14 +89,56 @@ def build_moe_route_plan(ids: torch.Tensor, n_experts: int) -> MoeRoutePlan:
     return plan
 
 
-class NintMoeWeight:
-    """One logical [experts, out_per_expert, K] tensor made of NINT cohorts (NINTM / NIM2)."""
+class ForeignCohort:
+    """A NINTM cohort of another family (NVQ, the 1-bit families, NEPQ): the reference runs them inside its grouped
+    kernels (cpp_runtime/mfq_decode.cpp:4800-5360, mfq/kernels/cuda/nvq_matmul.cu:2588-3175); here every expert is a
+    tensor of its own on that family's kernels and the host walks the experts a batch routes to -- correct, one matmul
+    per expert hit, not a fast path."""
 
-    def __init__(self, n_experts, out_per_expert, neuron_len, pools, expert_ids, device):
+    def __init__(self, dtype, blob, expert_ids, out_per_expert, neuron_len, device):
+        from .runtime import is_nepq_linear_dtype, load_quant_linear
+        self.dtype, self.expert_ids = dtype, np.asarray(expert_ids, dtype=np.int32)
+        self.out, self.neuron_len = out_per_expert, neuron_len
+        n = len(self.expert_ids)
+        self.nepq, self.linears = None, []
+        if is_nepq_linear_dtype(dtype):
+            from .runtime_vq import NepqWeight
+            self.nepq = NepqWeight.from_blob(blob, device)
+            if self.nepq.label != dtype:
+                raise ValueError(f"MFQ dtype/blob mismatch: {dtype} contains {self.nepq.label}")
+            shape = (self.nepq.n_experts, self.nepq.out_per_expert, self.nepq.neuron_len)
+        else:
+            self.linears = [load_quant_linear(dtype, b, device) for b in F.split_rows(dtype, blob, n)]
+            shape = (n, self.linears[0].out, self.linears[0].neuron_len)
+        if shape != (n, out_per_expert, neuron_len):
+            raise ValueError(f"NINTM pool tensor shape {shape} must be {(n, out_per_expert, neuron_len)}")
+
+    @property
+    def payload_bytes(self) -> int:
+        return self.nepq.payload_bytes if self.nepq is not None else sum(q.weight.payload_bytes for q in self.linears)
+
+    def matmul(self, local: int, x: torch.Tensor) -> torch.Tensor:
+        if self.nepq is not None:
+            from .runtime_vq import nepq_matmul
+            return nepq_matmul(self.nepq, x, local)
+        return self.linears[local](x)
+
+    def dequantize(self) -> torch.Tensor:
+        if self.nepq is not None:
+            return self.nepq.dequantize().reshape(len(self.expert_ids), self.out, self.neuron_len)
+        return torch.stack([q.dequantize() for q in self.linears])
+
+
+class NintMoeWeight:
+    """One logical [experts, out_per_expert, K] tensor made of cohorts (NINTM / NIM2).  NINT cohorts run on the grouped
+    kernels; cohorts of other families (`foreign`) are added by the host, expert by expert."""
+
+    def __init__(self, n_experts, out_per_expert, neuron_len, pools, expert_ids, device, foreign=()):
         self.n_experts, self.out_per_expert, self.neuron_len = n_experts, out_per_expert, neuron_len
         self.pools: list[NintWeight] = pools
         self.pool_expert_ids = expert_ids
-        ep = np.full(n_experts, -1, dtype=np.int32)
+        self.foreign: list[ForeignCohort] = list(foreign)
+        ep = np.full(n_experts, -1, dtype=np.int32)       # -1: no NINT cohort -- the kernels leave a zero row
         el = np.full(n_experts, -1, dtype=np.int32)
         for pi, ids in enumerate(expert_ids):
             ep[ids] = pi
@@ -104,7 +146,7 @@ class NintMoeWeight:
         # device dispatch tables (initialize_nint_moe_dispatch, cpp_runtime/mfq_decode.cpp:3249-3343)
         self.expert_pool = torch.from_numpy(ep).to(device)
         self.expert_local = torch.from_numpy(el).to(device)
-        self._pool_array = (L.MoePool * len(pools))()
+        self._pool_array = (L.MoePool * max(len(pools), 1))()
         for i, p in enumerate(pools):
             self._pool_array[i].desc = p.desc
             self._pool_array[i].weight = p.data.data_ptr()
@@ -115,10 +157,13 @@ class NintMoeWeight:
 
     @property
     def payload_bytes(self) -> int:
-        return sum(p.payload_bytes for p in self.pools)
+        return sum(p.payload_bytes for p in self.pools) + sum(c.payload_bytes for c in self.foreign)
 
     def expert_payload_bytes(self, e: int) -> float:
         pi = int(self.expert_pool[e].item())
+        if pi < 0:
+            c = next(c for c in self.foreign if e in c.expert_ids)
+            return c.payload_bytes / len(c.expert_ids)
         return self.pools[pi].payload_bytes / len(self.pool_expert_ids[pi])
 
     @staticmethod
@@ -126,18 +171,24 @@ class NintMoeWeight:
         h = F.parse_nintm(blob)
         device = torch.device(device)
         pools, ids = [], []
+        foreign = []
         for p in h.pools:
-            if not (p.dtype.startswith("NINT") and p.dtype[4:].isdigit()):
-                raise NotImplementedError(f"NINTM cohort family {p.dtype} is not on the accelerated path")
             if p.runtime_bytes:
                 raise ValueError("unexpected NINTM cohort runtime metadata")
+            if not (p.dtype.startswith("NINT") and p.dtype[4:].isdigit()):
+                from .runtime import is_nepq_linear_dtype, is_nvq_linear_dtype
+                if not (is_nvq_linear_dtype(p.dtype) or is_nepq_linear_dtype(p.dtype) or F.is_lowbit_dtype(p.dtype)):
+                    raise NotImplementedError(f"NINTM cohort family {p.dtype} is not supported")
+                foreign.append(ForeignCohort(p.dtype, bytes(blob[p.payload_off: p.payload_off + p.payload_bytes]),
+                                             p.expert_ids, h.out_per_expert, h.neuron_len, device))
+                continue
             w = NintWeight.from_blob(bytes(blob[p.payload_off: p.payload_off + p.payload_bytes]), device)
             if w.out != len(p.expert_ids) * h.out_per_expert or w.neuron_len != h.neuron_len:
                 raise ValueError(f"NINTM pool tensor shape {(w.out, w.neuron_len)} must be "
                                  f"{(len(p.expert_ids) * h.out_per_expert, h.neuron_len)}")
             pools.append(w)
             ids.append(p.expert_ids)
-        return NintMoeWeight(h.n_experts, h.out_per_expert, h.neuron_len, pools, ids, device)
+        return NintMoeWeight(h.n_experts, h.out_per_expert, h.neuron_len, pools, ids, device, foreign)
 
     def dequantize(self) -> torch.Tensor:
         out = torch.empty((self.n_experts, self.out_per_expert, self.neuron_len), dtype=torch.float32,
@@ -145,7 +196,24 @@ class NintMoeWeight:
         for p, ids in zip(self.pools, self.pool_expert_ids):
             out[torch.from_numpy(ids.astype(np.int64)).to(out.device)] = p.dequantize().reshape(
                 len(ids), self.out_per_expert, self.neuron_len)
+        for c in self.foreign:
+            out[torch.from_numpy(c.expert_ids.astype(np.int64)).to(out.device)] = c.dequantize()
         return out
+
+    def _add_foreign(self, x2: torch.Tensor, routed: bool, route: MoeRoutePlan, out: torch.Tensor) -> None:
+        """The rows of the pairs routed to experts of other families: per expert, gather its activation rows, multiply
+        on that family's kernels, scatter into `out` [T, R, out_per_expert].  Reads the routing table on the host."""
+        T, R = route.tokens, route.routes
+        ids = route.ids.reshape(T, R).cpu().numpy()
+        flat = out.view(T * R, self.out_per_expert)
+        for c in self.foreign:
+            for local, e in enumerate(c.expert_ids):
+                t_idx, r_idx = np.nonzero(ids == e)
+                if t_idx.size == 0:
+                    continue
+                pairs = torch.from_numpy((t_idx * R + r_idx).astype(np.int64)).to(out.device)
+                src = pairs if routed else torch.from_numpy(t_idx.astype(np.int64)).to(out.device)
+                flat[pairs] = c.matmul(local, x2.index_select(0, src))
 
     def forward(self, x: torch.Tensor, route: MoeRoutePlan) -> torch.Tensor:
         """NintMoeWeight::forward (cpp_runtime/mfq_decode.cpp:2908-3071): x is [T, K] (shared by the
@@ -157,6 +225,10 @@ class NintMoeWeight:
         x2 = x.reshape(-1, self.neuron_len)
         if x2.stride(-1) != 1:
             x2 = x2.contiguous()
+        if not self.pools:                              # no NINT cohort at all: every row comes from the host loop
+            out = torch.zeros((T, R, self.out_per_expert), dtype=torch.float32, device=x.device)
+            self._add_foreign(x2, routed, route, out)
+            return out
         out = torch.empty((T, R, self.out_per_expert), dtype=torch.float32, device=x.device)
         mapped = route.ids_dst is not None
         lib = L.lib()
@@ -170,6 +242,8 @@ class NintMoeWeight:
             T, R, _ptr(route.ids_dst) if mapped else None, _ptr(route.expert_bounds) if mapped else None,
             _ptr(route.tile_bounds) if mapped else None, _ptr(route.tile_experts) if mapped else None,
             _ptr(out), self.out_per_expert, _ptr(ws), need, _stream()))
+        if self.foreign:
+            self._add_foreign(x2, routed, route, out)
         return out
 
     __call__ = forward
@@ -187,7 +261,7 @@ class NintMoeWeight:
         if self.out_per_expert % 2:
             raise RuntimeError("fused gate/up GLU needs an even number of neurons per expert")
         W = self.out_per_expert // 2
-        if route.ids_dst is not None and self.out_per_expert % 32 == 0:
+        if route.ids_dst is not None and self.out_per_expert % 32 == 0 and not self.foreign:
             x2 = x.reshape(-1, self.neuron_len)
             if x2.stride(-1) != 1:
                 x2 = x2.contiguous()
@@ -210,7 +284,7 @@ class NintMoeWeight:
     def decode_capable(self, shared: NintWeight | None = None, tokens: int = 1, routes: int = 1, swiglu=False) -> bool:
         """Whether forward_decode takes these cohorts, this shared tensor and this many (token, route) pairs: the
         library's own answer (unit per cohort, shared tensor's shape, the block's LDS need, the row count)."""
-        if shared is not None and shared.neuron_len != self.neuron_len:
+        if self.foreign or (shared is not None and shared.neuron_len != self.neuron_len):
             return False
         return bool(L.lib().mfq_hip_moe_decode_capable(
             self._pool_array, len(self.pools), self.out_per_expert, self.neuron_len,
@@ -367,6 +441,9 @@ class MoeExpertCache:
         if self.finalized:
             raise RuntimeError("cannot register a MoE source after cache finalization")
         full = NintMoeWeight.from_blob(blob, self.device)
+        if full.foreign:
+            raise NotImplementedError("expert residency holds NINT cohorts only; this tensor has a "
+                                      f"{full.foreign[0].dtype} cohort")
         cohorts = [_HostCohort(p, ids, full.out_per_expert) for p, ids in zip(full.pools, full.pool_expert_ids)]
         for c in cohorts:
             c.minimum_slots = min(int(minimum_slots), len(c.expert_ids))
