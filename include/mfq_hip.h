@@ -301,9 +301,10 @@ typedef struct mfq_nvqs_desc {
     int64_t tables_off, anchors_off, state_off, index_off, sign_off;
     int64_t total_bytes;
     int64_t payload_bytes; /* anchors + the streams */
-    int32_t kind;          /* 0: the NVQ formats above; 1: NVQ1-L / NVQ1-S; 2: NPQ0-L / NPQ0-S (see below) */
+    int32_t kind;          /* 0: the NVQ formats above; 1: NVQ1-L / NVQ1-S; 2: NPQ0-L / NPQ0-S; 3: NEPQ0-S / NEPQ0-L (see below) */
     int32_t state_bits, cb_bytes;
     float delta;
+    int32_t nbank, nsuper; /* kind 3 (NEPQ0): tables in the pool, bank ids per neuron (one per 96 weights) */
 } mfq_nvqs_desc;
 
 int mfq_hip_nvqs_plan(int vector_size, int index_bits, int banks, int index_parity, int out, int neuron_len,
@@ -342,6 +343,23 @@ int mfq_hip_nvqs_gemv(const mfq_nvqs_desc *d, const void *weight, const void *x,
 int mfq_hip_nvqs_plan_lowbit(int format, int state_bits, int out, int neuron_len, mfq_nvqs_desc *d);
 int mfq_hip_nvqs_repack_lowbit(const mfq_nvqs_desc *d, const void *body, int64_t body_bytes, const void *grid,
                                void *weight, mfq_stream_t stream);
+/* NEPQ0-S / NEPQ0-L (profiles 0 / 1 of the NEPQ container, mfq/formats/nepq.py:95-116; formats 9 / 7 with a table pool in
+ * the reference's loader, cpp_runtime/mfq_decode.cpp:4198-4260): the product form of NPQ0 on [experts * out_per_expert, K]
+ * neurons with a pool of `banks` tables; one bank id byte per neuron and 96 weights picks scale LUT and sub-codebooks
+ * (dequantize_nepq, nepq.py:492-521).  `body` = device copy of the blob behind its 36-byte header: tables, fp16 anchors,
+ * state and index streams, bank ids.  An expert is the row range [e * out_per_expert, (e + 1) * out_per_expert) of the
+ * row-range calls below, which exist for every descriptor kind: y / w_out hold nrows columns / rows. */
+int mfq_hip_nvqs_plan_nepq0(int profile, int banks, int rows, int neuron_len, mfq_nvqs_desc *d);
+int mfq_hip_nvqs_repack_nepq0(const mfq_nvqs_desc *d, const void *body, int64_t body_bytes, void *weight,
+                              mfq_stream_t stream);
+int mfq_hip_nvqs_dequant_rows_f32(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, float *w_out,
+                                  int64_t ld, mfq_stream_t stream);
+int mfq_hip_nvqs_gemv_rows(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, const void *x, int x_dtype,
+                           int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream);
+size_t mfq_hip_nvqs_gemm_rows_workspace_bytes(const mfq_nvqs_desc *d, int nrows, int M);
+int mfq_hip_nvqs_gemm_rows(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, const void *x, int x_dtype,
+                           int64_t ldx, int M, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
+                           mfq_stream_t stream);
 size_t mfq_hip_nvqs_gemm_workspace_bytes(const mfq_nvqs_desc *d, int M);
 int mfq_hip_nvqs_gemm(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
                       int M, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,

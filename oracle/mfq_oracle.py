@@ -41,6 +41,7 @@ reference tree).  Parity status of each function:
     dequantize_nvq1                mfq/quantize/nvq1_l_quant.py:384-414, nvq1_s_quant.py:142-174
     pack_npq0 / unpack_npq0        mfq/formats/npq0_l.py:112-185, 326-415, npq0_s.py:110-183, 320-406
     dequantize_npq0                mfq/quantize/npq0_l.py:766-790, npq0_s.py:812-836
+    pack_nepq / unpack_nepq / dequantize_nepq on NEPQ0-S / NEPQ0-L   mfq/formats/nepq.py:95-116, 368-474, 492-521
 
   pinned by golden vectors written from the reference's own numpy quantizer
   (tests/golden/nint_quant_vectors.npz, made by tests/golden/make_nint_quant_vectors.py)
@@ -511,11 +512,11 @@ def dequantize_nvq(t: NvqTensor) -> np.ndarray:
 
 
 # ---------------------------------------------------------------------------
-# NEPQ  (mfq/formats/nepq.py; NEPQ1-S / NEPQ1-L only)
+# NEPQ  (mfq/formats/nepq.py): NEPQ1-S / NEPQ1-L (ternary tables) and NEPQ0-S / NEPQ0-L (the product tables of NPQ0)
 # ---------------------------------------------------------------------------
 _NEPQ_HDR = struct.Struct("<4sBBBBIIIIIQ")
 #              label: (profile_id, state_bits, index_bits, aux_bits, table_bytes)
-NEPQ_SPECS = {"NEPQ0-S": (0, 2, 6, 0, None), "NEPQ0-L": (1, 3, 7, 0, None),
+NEPQ_SPECS = {"NEPQ0-S": (0, 2, 6, 0, 320), "NEPQ0-L": (1, 3, 7, 0, 832),
               "NEPQ1-S": (2, 4, 9, 1, 2048), "NEPQ1-L": (3, 3, 11, 1, 4096)}
 _NEPQ_BY_ID = {v[0]: k for k, v in NEPQ_SPECS.items()}
 
@@ -610,10 +611,13 @@ def unpack_nepq(blob) -> NepqTensor:
         raise ValueError(f"invalid NEPQ tail: consumed={off}, size={len(blob)}")
     if np.any(bank_ids >= banks):
         raise ValueError("NEPQ bank ID exceeds the table pool")
-    for tbl in tables:   # ternary validity (mfq/formats/nepq.py:270-290)
-        unpack_ternary_table(tbl.tobytes())
+    for tbl in tables:   # table validity (mfq/formats/nepq.py:270-290)
+        if label.startswith("NEPQ1"):
+            unpack_ternary_table(tbl.tobytes())
+        else:
+            _npq0_tables(tbl.tobytes(), "NPQ0" + label[5:])
     return NepqTensor(label, (E, out, K), ns, state.reshape(E, out, ng), idx.reshape(E, out, nvec).astype(np.uint16),
-                      aux.reshape(E, out, ng), bank_ids, tables, rblock, rseed)
+                      aux.reshape(E, out, ng) if ab else np.zeros(0, dtype=np.uint8), bank_ids, tables, rblock, rseed)
 
 
 def dequantize_nepq(t: NepqTensor) -> np.ndarray:
@@ -627,7 +631,7 @@ def dequantize_nepq(t: NepqTensor) -> np.ndarray:
     bank_ids = t.bank_ids.reshape(rows, -1)
     group_bank = np.repeat(bank_ids, 4, axis=1)[:, :ng]
     vector_bank = np.repeat(group_bank, 3, axis=1)[:, :nvec].astype(np.int64)
-    aux = t.aux.reshape(rows, ng).astype(np.uint8)
+    aux = t.aux.reshape(rows, ng).astype(np.uint8) if NEPQ_SPECS[t.label][3] else None   # NEPQ0 stores no aux stream
     if t.label == "NEPQ1-S":
         tables = np.stack([np.stack([unpack_ternary_table(p.tobytes()[:1024]),
                                      unpack_ternary_table(p.tobytes()[1024:])]) for p in t.table_payloads])
@@ -639,7 +643,15 @@ def dequantize_nepq(t: NepqTensor) -> np.ndarray:
         code = tables[vector_bank, idx]
         delta = np.where(aux != 0, -0.125, 0.125).astype(np.float32)
     else:
-        raise NotImplementedError(t.label)
+        # the product form: the bank id of a neuron's 96 weights picks scale LUT and sub-codebooks, the group state the
+        # entry of each (mfq/formats/nepq.py:509-521)
+        tabs = [_npq0_tables(p.tobytes(), "NPQ0" + t.label[5:]) for p in t.table_payloads]
+        lut = np.stack([x[0] for x in tabs]); first = np.stack([x[1] for x in tabs]); second = np.stack([x[2] for x in tabs])
+        vector_state = np.repeat(state, 3, axis=1)[:, :nvec].astype(np.int64)
+        code = np.concatenate((first[vector_bank, vector_state, idx & 7], second[vector_bank, vector_state, idx >> 3]), axis=-1)
+        group_scale = anchors[:, None] * lut[group_bank.astype(np.int64), state.astype(np.int64)]
+        scale = np.repeat(group_scale, 24, axis=1)[:, :K]
+        return (code.reshape(rows, K).astype(np.float32) * scale).astype(np.float32).reshape(t.shape)
     group_scale = anchors[:, None] * state.astype(np.float32)
     scale = np.repeat(group_scale, 24, axis=1)[:, :K]
     bias = np.repeat(delta, 24, axis=1)[:, :K]
@@ -910,6 +922,26 @@ def dequantize_nvq1(t: Nvq1Tensor) -> np.ndarray:
     delta = np.repeat(np.where(np.asarray(t.delta_sign) != 0, -d, d).astype(np.float32), 24, axis=1)[:, :K]
     scale = np.repeat(t.neuron_scale.astype(np.float32)[:, None] * np.asarray(t.sub_scale).astype(np.float32), 24, axis=1)[:, :K]
     return (scale * (code + delta)).astype(np.float32)
+
+
+def _npq0_tables(payload: bytes, label: str):
+    """One NPQ0 table: (scale LUT float32 [states], first int8 [states, 8, 4], second int8 [states, 8 or 16, 4]), with the
+    header checks of unpack_npq0_l_tables / unpack_npq0_s_tables (mfq/formats/npq0_l.py:136-185, npq0_s.py:134-183)."""
+    sp = LOWBIT_SPECS[label]
+    S, E2 = sp["states"], sp["second"]
+    if len(payload) < 64 + S * 32 + S * E2 * 4:
+        raise ValueError(f"truncated {label} product tables")
+    head = payload[:64]
+    if tuple(head[:6]) != (sp["table_version"], S, 3, sp["index_bits"] - 3, 24, 8):
+        raise ValueError(f"unsupported {label} table profile")
+    if any(head[6:8]) or any(head[8 + 2 * S:64]):
+        raise ValueError(f"{label} reserved table bytes must be zero")
+    lut = np.frombuffer(head, dtype="<f2", count=S, offset=8).astype(np.float32)
+    if not np.isfinite(lut).all() or np.any(lut < 0) or float(lut.max()) <= 0:
+        raise ValueError(f"{label} scale LUT must be finite, non-negative, and nonzero")
+    first = np.frombuffer(payload, dtype=np.int8, count=S * 32, offset=64).reshape(S, 8, 4).copy()
+    second = np.frombuffer(payload, dtype=np.int8, count=S * E2 * 4, offset=64 + S * 32).reshape(S, E2, 4).copy()
+    return lut, first, second
 
 
 def pack_npq0_tables(t: Npq0Tensor) -> bytes:

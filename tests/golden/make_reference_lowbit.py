@@ -1,7 +1,8 @@
-"""Write reference-made blobs and reference-dequantized values of the 1-bit families (NVQ1-L, NVQ1-S, NPQ0-L, NPQ0-S).
+"""Write reference-made blobs and reference-dequantized values of the 1-bit families (NVQ1-L, NVQ1-S, NPQ0-L, NPQ0-S and
+the expert forms NEPQ0-S, NEPQ0-L).
 
 As make_reference_blobs.py: the reference's own format modules are imported IN THE BUILD CONTAINER ONLY (from
-/root/reference: mfq.formats.{nvq1_l,nvq1_s,npq0_l,npq0_s} and the dequantizers of mfq.quantize.{nvq1_l_quant,
+/root/reference: mfq.formats.{nvq1_l,nvq1_s,npq0_l,npq0_s,nepq} and the dequantizers of mfq.quantize.{nvq1_l_quant,
 nvq1_s_quant,npq0_l,npq0_s}; numpy and CPU torch, nothing else), fed seeded random fields from tests/synth.py, and the
 fields, the packed bytes and the dequantized arrays are stored in tests/golden/reference_lowbit.npz.  The fixture is data;
 the reference never travels.
@@ -68,6 +69,17 @@ for key, label, fmod, qdeq, cls, (rows, K) in (("npq0l", "NPQ0-L", f_pl, q_pl.de
     pack = fmod.pack_npq0_l if label == "NPQ0-L" else fmod.pack_npq0_s
     put(key, meta=[rows, K], ns=t.neuron_scale, lut=t.scale_lut, state=t.state, idx=t.indices, first=t.first_codebooks,
         second=t.second_codebooks, blob=blob_array(pack(rt)), deq=qdeq(rt))
+
+# NEPQ0-S / NEPQ0-L: the NEPQ container with NPQ0 tables in its pool; two experts, three tables, K = 200 (three
+# super-groups of 96 weights, the last ragged)
+from mfq.formats import nepq as f_ne  # noqa: E402
+
+for key, label in {"nepq0s": "NEPQ0-S", "nepq0l": "NEPQ0-L"}.items():
+    t = synth.nepq_random(rng, label, 2, 8, 200, 3)
+    rt = f_ne.NepqTensor(spec=f_ne.nepq_spec(label), shape=t.shape, neuron_scale=t.neuron_scale, state=t.state,
+                         indices=t.indices, aux=t.aux, bank_ids=t.bank_ids, table_payloads=t.table_payloads)
+    put(key, meta=list(t.shape) + [3], anchors=t.neuron_scale, state=t.state, indices=t.indices, aux=t.aux,
+        bank_ids=t.bank_ids, tables=t.table_payloads, blob=blob_array(f_ne.pack_nepq(rt)), deq=f_ne.dequantize_nepq(rt))
 
 np.savez_compressed(HERE / "reference_lowbit.npz", **out)
 print("wrote", HERE / "reference_lowbit.npz", len(out), "arrays")

@@ -80,7 +80,14 @@ def nepq_random(rng, label, E, out, K, banks):
     iq1s = np.frombuffer((O._DATA / "iq1s_2048.bin").read_bytes(), dtype="<u2")
     tables = []
     for b in range(banks):
-        if label == "NEPQ1-L":
+        if label.startswith("NEPQ0"):       # an NPQ0 table: header with the fp16 scale LUT, then the int8 sub-codebooks
+            sp = O.LOWBIT_SPECS["NPQ0" + label[5:]]
+            S, E2 = sp["states"], sp["second"]
+            head = bytearray(64)
+            head[0:6] = bytes([sp["table_version"], S, 3, sp["index_bits"] - 3, 24, 8])
+            head[8:8 + 2 * S] = O._f16_round(rng.uniform(0.25, 2.0, S)).astype("<f2").tobytes()
+            tables.append(bytes(head) + rng.integers(-127, 128, S * 32 + S * E2 * 4).astype(np.int8).tobytes())
+        elif label == "NEPQ1-L":
             tables.append(rng.permutation(iq1s).astype("<u2").tobytes())
         else:
             tables.append(rng.permutation(iq1s)[:512].astype("<u2").tobytes()
@@ -91,7 +98,7 @@ def nepq_random(rng, label, E, out, K, banks):
     return O.NepqTensor(label, (E, out, K), O._f16_round(rng.uniform(0.0005, 0.005, (E, out))),
                         rng.integers(0, 1 << sb, (E, out, ng), dtype=np.uint8),
                         rng.integers(0, 1 << ib, (E, out, nvec)).astype(np.uint16),
-                        rng.integers(0, 2, (E, out, ng), dtype=np.uint8),
+                        rng.integers(0, 2, (E, out, ng), dtype=np.uint8) if ab else np.zeros(0, dtype=np.uint8),
                         rng.integers(0, banks, (E, out, nsuper), dtype=np.uint8), tables)
 
 

@@ -67,6 +67,8 @@ def test_check_linear_tool_reports_small_error(tmp_path):
         "blk.1.k.nvq1s": synth.nvq1_random(rng, "NVQ1-S", 24, 104),
         "blk.1.v.npq0l": synth.npq0_random(rng, "NPQ0-L", 40, 96),
         "blk.1.o.npq0s": synth.npq0_random(rng, "NPQ0-S", 33, 200),
+        "blk.2.q.nepq0s": synth.nepq_random(rng, "NEPQ0-S", 1, 48, 96, 3),            # NPQ0 tables in the NEPQ container
+        "blk.2.k.nepq0l": synth.nepq_random(rng, "NEPQ0-L", 1, 40, 200, 5),
     }
     path = tmp_path / "tiny.mfq"
     O.mfq_file_write(path, tensors, version=2)
@@ -218,14 +220,15 @@ def test_cpp_moe_ffn_forward(rt, T):
 
 
 def _mixed_moe(rng, E_out, K):
-    """Eight experts in four cohorts of different families (NINT4, NVQ3J-512, NVQ1-S, NEPQ1-S)."""
+    """Eight experts in five cohorts of different families (NINT4, NVQ3J-512, NVQ1-S, NEPQ1-S, NEPQ0-L)."""
     def pool(ids, dtype, t):
         return O.MoePool(np.asarray(ids, dtype=np.int32), dtype, t)
     return O.NintMoeTensor((8, E_out, K), [
         pool([0, 5, 7], "NINT4", synth.nint_random(rng, 3 * E_out, K, 4, 32, 6)),
         pool([1, 4], "NVQ3J-512", synth.nvq_jsc_random(rng, 2 * E_out, K, "d4_512", 2)),
         pool([2], "NVQ1-S", synth.nvq1_random(rng, "NVQ1-S", E_out, K)),
-        pool([6, 3], "NEPQ1-S", synth.nepq_random(rng, "NEPQ1-S", 2, E_out, K, 3))])
+        pool([6], "NEPQ1-S", synth.nepq_random(rng, "NEPQ1-S", 1, E_out, K, 3)),
+        pool([3], "NEPQ0-L", synth.nepq_random(rng, "NEPQ0-L", 1, E_out, K, 2))])
 
 
 @pytest.mark.parametrize("T", [3, 40])

@@ -365,15 +365,16 @@ def test_mapped_path_with_hundreds_of_experts_and_skewed_routes():
 
 
 def _mixed_family_moe(rng, out, K):
-    """Nine experts in five cohorts: NINT4 (3 experts), NVQ3J-512 (2), NVQ2J read from its streams (1), NPQ0-S (1),
-    NEPQ1-S (2)."""
+    """Nine experts in six cohorts: NINT4 (3 experts), NVQ3J-512 (2), NVQ2J read from its streams (1), NPQ0-S (1),
+    NEPQ1-S (1), NEPQ0-S (1)."""
     def pool(ids, dtype, t):
         return O.MoePool(np.asarray(ids, dtype=np.int32), dtype, t)
     pools = [pool([0, 4, 8], "NINT4", synth.nint_random(rng, 3 * out, K, 4, 32, 6)),
              pool([1, 6], "NVQ3J-512", synth.nvq_jsc_random(rng, 2 * out, K, "d4_512", 2)),
              pool([2], "NVQ2J", synth.nvq_jsc_random(rng, out, K, "e8_256", 2)),
              pool([5], "NPQ0-S", synth.npq0_random(rng, "NPQ0-S", out, K)),
-             pool([3, 7], "NEPQ1-S", synth.nepq_random(rng, "NEPQ1-S", 2, out, K, 3))]
+             pool([3], "NEPQ1-S", synth.nepq_random(rng, "NEPQ1-S", 1, out, K, 3)),
+             pool([7], "NEPQ0-S", synth.nepq_random(rng, "NEPQ0-S", 1, out, K, 4))]
     return O.NintMoeTensor((9, out, K), pools)
 
 
@@ -388,7 +389,7 @@ def test_mixed_family_cohorts_in_one_tensor():
     t = _mixed_family_moe(rng, out, K)
     blob = O.pack_nint_moe(t)
     w = NintMoeWeight.from_blob(blob)
-    assert len(w.pools) == 1 and [c.dtype for c in w.foreign] == ["NVQ3J-512", "NVQ2J", "NPQ0-S", "NEPQ1-S"]
+    assert len(w.pools) == 1 and [c.dtype for c in w.foreign] == ["NVQ3J-512", "NVQ2J", "NPQ0-S", "NEPQ1-S", "NEPQ0-S"]
     dense = O.dequantize_expertwise(t)
     assert np.array_equal(w.dequantize().cpu().numpy().view(np.uint32), dense.view(np.uint32))
     assert not w.decode_capable(None, 1, R)

@@ -67,6 +67,23 @@ def test_npq0_blob_and_values_match_the_reference(key):
         O.unpack_npq0(bytes(bad), t.label)
 
 
+@pytest.mark.parametrize("key,label", [("nepq0s", "NEPQ0-S"), ("nepq0l", "NEPQ0-L")])
+def test_nepq0_blob_and_values_match_the_reference(key, label):
+    """The expert form: NPQ0 tables in the NEPQ container's pool, one bank id per neuron and 96 weights."""
+    E, rows, K, banks = (int(v) for v in G[f"{key}_meta"])
+    t = O.NepqTensor(label, (E, rows, K), G[f"{key}_anchors"], G[f"{key}_state"], G[f"{key}_indices"], G[f"{key}_aux"],
+                     G[f"{key}_bank_ids"], G[f"{key}_tables"])
+    blob = bytes(G[f"{key}_blob"])
+    assert O.pack_nepq(t) == blob
+    back = O.unpack_nepq(blob)
+    assert back.label == label and np.array_equal(back.bank_ids, t.bank_ids) and np.array_equal(back.indices, t.indices)
+    assert _bits_equal(O.dequantize_nepq(back), G[f"{key}_deq"])
+    bad = bytearray(blob)
+    bad[O._NEPQ_HDR.size + 1] ^= 0xFF                       # the state count of the first table's header
+    with pytest.raises(ValueError, match="table profile"):
+        O.unpack_nepq(bytes(bad))
+
+
 def test_lowbit_mistakes_the_fixture_would_catch():
     """The checks above are not vacuous: swapping the delta's sign, taking the bank from the wrong bit, or splitting the
     product index the other way round changes the values."""

@@ -430,3 +430,44 @@ def test_one_bit_families_reference_blobs_and_loader_errors():
     bad[20 + 16 + 4] = 0xFF                                    # digit 3 in a ternary entry
     with pytest.raises(ValueError, match="non-ternary"):
         R.load_quant_linear("NVQ1-S", bytes(bad))
+
+
+@pytest.mark.parametrize("label", ["NEPQ0-S", "NEPQ0-L"])
+@pytest.mark.parametrize("E,out,K,banks", [(1, 48, 96, 3), (3, 32, 200, 5), (2, 16, 1544, 40), (1, 33, 88, 1)])
+def test_nepq0_dequant_bit_exact_and_matmul(label, E, out, K, banks):
+    """The expert form of the product codebooks (NPQ0 tables in the NEPQ container's pool): dequantized experts bit for
+    bit, every expert's matmul through the row-range calls for GEMV and GEMM batch sizes, the dense-linear registry for a
+    one-expert tensor, the reference-packed blobs of the golden fixture."""
+    from pathlib import Path
+
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import NepqWeight, nepq_matmul
+    rng = np.random.default_rng(123 + E + out + K)
+    t = synth.nepq_random(rng, label, E, out, K, banks)
+    blob = O.pack_nepq(t)
+    w = NepqWeight.from_blob(blob)
+    assert w.streams and w.label == label
+    want = O.dequantize_nepq(O.unpack_nepq(blob))
+    got = w.dequantize().cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    for e in range(E):
+        for M in (1, 5, 16):
+            x, xf = _x(rng, M, K)
+            _check(nepq_matmul(w, x, e).cpu().numpy(), O.linear_forward_f64(want[e], xf))
+        x, xf = _x(rng, 40, K)
+        _check(nepq_matmul(w, x, e).cpu().numpy(), O.linear_forward_f64(want[e], xf))
+    if E == 1:
+        lin = R.load_quant_linear(label, blob)
+        x, xf = _x(rng, 3, K)
+        _check(lin(x).cpu().numpy(), O.linear_forward_f64(want[0], xf))
+    else:
+        with pytest.raises(ValueError, match="must hold one expert"):
+            R.load_quant_linear(label, blob)
+    gold = np.load(Path(__file__).resolve().parent / "golden" / "reference_lowbit.npz")
+    key = "nepq0s" if label == "NEPQ0-S" else "nepq0l"
+    g = NepqWeight.from_blob(bytes(gold[f"{key}_blob"]))
+    assert np.array_equal(g.dequantize().cpu().numpy().view(np.uint32), gold[f"{key}_deq"].astype(np.float32).view(np.uint32))
+    bad = bytearray(blob)
+    bad[36 + 2] = 9                                    # first index width in the first table's header
+    with pytest.raises(ValueError, match="table profile"):
+        NepqWeight.from_blob(bytes(bad))

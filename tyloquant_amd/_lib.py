@@ -38,7 +38,7 @@ class NvqsDesc(C.Structure):
                                    "ng", "nvec", "nsign")] + \
                [(n, i64) for n in ("tables_off", "anchors_off", "state_off", "index_off", "sign_off", "total_bytes",
                                    "payload_bytes")] + \
-               [("kind", i32), ("state_bits", i32), ("cb_bytes", i32), ("delta", C.c_float)]
+               [("kind", i32), ("state_bits", i32), ("cb_bytes", i32), ("delta", C.c_float), ("nbank", i32), ("nsuper", i32)]
 
 
 class NepqDesc(C.Structure):
@@ -104,6 +104,13 @@ _SIGS = {
     "mfq_hip_nvq_gemm": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
     "mfq_hip_nvqs_plan": (C.c_int, [C.c_int] * 6 + [C.POINTER(NvqsDesc)]),
     "mfq_hip_nvqs_repack": (C.c_int, [C.POINTER(NvqsDesc), vp, i64, C.c_int, vp, vp, vp]),
+    "mfq_hip_nvqs_plan_nepq0": (C.c_int, [C.c_int] * 4 + [C.POINTER(NvqsDesc)]),
+    "mfq_hip_nvqs_repack_nepq0": (C.c_int, [C.POINTER(NvqsDesc), vp, i64, vp, vp]),
+    "mfq_hip_nvqs_dequant_rows_f32": (C.c_int, [C.POINTER(NvqsDesc), vp, C.c_int, C.c_int, vp, i64, vp]),
+    "mfq_hip_nvqs_gemv_rows": (C.c_int, [C.POINTER(NvqsDesc), vp, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
+    "mfq_hip_nvqs_gemm_rows_workspace_bytes": (sz, [C.POINTER(NvqsDesc), C.c_int, C.c_int]),
+    "mfq_hip_nvqs_gemm_rows": (C.c_int, [C.POINTER(NvqsDesc), vp, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz,
+                                         vp]),
     "mfq_hip_moe_move_rows": (C.c_int, [vp, i64, vp, C.c_int, C.c_int, C.c_int, vp, i64, vp]),
     "mfq_hip_nvqs_plan_lowbit": (C.c_int, [C.c_int] * 4 + [C.POINTER(NvqsDesc)]),
     "mfq_hip_nvqs_repack_lowbit": (C.c_int, [C.POINTER(NvqsDesc), vp, i64, vp, vp, vp]),

@@ -190,14 +190,32 @@ NepqHeader parse_nepq(const uint8_t *b, size_t n) {
     if ((flags & ~1) || ((flags & 1) != 0) != (h.rotation_block != 0)) fail("inconsistent NEPQ rotation flag");
     if (h.n_experts <= 0 || h.out_per_expert <= 0 || h.neuron_len <= 0 || h.neuron_len % 8 || h.banks < 1 || h.banks > 256)
         fail("NEPQ shape dimensions must be positive, K divisible by 8, banks in [1,256]");
-    if (h.profile < 2) fail(h.label + " is not on the accelerated path");
-    const int sb = h.profile == 2 ? 4 : 3, ib = h.profile == 2 ? 9 : 11, tb = h.profile == 2 ? 2048 : 4096;
+    static const int sbits[] = {2, 3, 4, 3}, ibits[] = {6, 7, 9, 11}, abits[] = {0, 0, 1, 1}, tbytes[] = {320, 832, 2048, 4096};
+    const int sb = sbits[h.profile], ib = ibits[h.profile], ab = abits[h.profile], tb = tbytes[h.profile];
     const int64_t rows = static_cast<int64_t>(h.n_experts) * h.out_per_expert, ng = cdiv(h.neuron_len, 24),
                   nvec = h.neuron_len / 8, nsuper = cdiv(ng, 4);
     const int64_t expect = static_cast<int64_t>(h.banks) * tb + 2 * rows + (rows * ng * sb + 7) / 8 +
-                           (rows * nvec * ib + 7) / 8 + (rows * ng + 7) / 8 + rows * nsuper;
+                           (rows * nvec * ib + 7) / 8 + (rows * ng * ab + 7) / 8 + rows * nsuper;
     if (static_cast<int64_t>(n) - 36 != expect)
         fail("invalid NEPQ tail: consumed=" + std::to_string(36 + expect) + ", size=" + std::to_string(n));
+    if (h.profile < 2) {  // NEPQ0: every table of the pool is an NPQ0 table (mfq/formats/nepq.py:270-290)
+        const int states = h.profile == 0 ? 4 : 8, version = h.profile == 0 ? 2 : 1;
+        for (int bank = 0; bank < h.banks; ++bank) {
+            const uint8_t *t = b + 36 + static_cast<size_t>(bank) * tb;
+            if (t[0] != version || t[1] != states || t[2] != 3 || t[3] != ib - 3 || t[4] != 24 || t[5] != 8)
+                fail("unsupported " + h.label + " table profile");
+            bool reserved = t[6] || t[7];
+            for (int i = 8 + 2 * states; i < 64; ++i) reserved = reserved || t[i];
+            if (reserved) fail("invalid " + h.label + " reserved table bytes");
+            float lmax = 0.f;
+            for (int i = 0; i < states; ++i) {
+                const float v = half_to_float(rd<uint16_t>(t, 8 + 2 * static_cast<size_t>(i)));
+                if (!(v >= 0.f) || std::isinf(v)) fail(h.label + " scale LUT must be finite and non-negative");
+                lmax = std::max(lmax, v);
+            }
+            if (lmax <= 0.f) fail(h.label + " scale LUT must be finite and non-negative");
+        }
+    }
     h.body_off = 36; h.body_bytes = static_cast<size_t>(expect);
     return h;
 }
@@ -495,10 +513,17 @@ NepqWeight NepqWeight::from_blob(const uint8_t *blob, size_t n, const int8_t *ro
     const NepqHeader h = parse_nepq(blob, n);
     NepqWeight w;
     w.label = h.label; w.n_experts = h.n_experts; w.out_per_expert = h.out_per_expert; w.rotation_block = h.rotation_block;
-    abi_check(mfq_hip_nepq_plan(h.profile, h.banks, h.n_experts * h.out_per_expert, h.neuron_len, &w.desc));
     DeviceBuffer payload = DeviceBuffer::from_host(blob + h.body_off, h.body_bytes);
-    w.data = DeviceBuffer(static_cast<size_t>(w.desc.total_bytes));
-    abi_check(mfq_hip_nepq_repack(&w.desc, payload.get(), static_cast<int64_t>(h.body_bytes), w.data.get(), stream));
+    if (h.profile < 2) {  // NEPQ0: read in place by the stream kernels
+        w.streams = true;
+        abi_check(mfq_hip_nvqs_plan_nepq0(h.profile, h.banks, h.n_experts * h.out_per_expert, h.neuron_len, &w.sdesc));
+        w.data = DeviceBuffer(static_cast<size_t>(w.sdesc.total_bytes));
+        abi_check(mfq_hip_nvqs_repack_nepq0(&w.sdesc, payload.get(), static_cast<int64_t>(h.body_bytes), w.data.get(), stream));
+    } else {
+        abi_check(mfq_hip_nepq_plan(h.profile, h.banks, h.n_experts * h.out_per_expert, h.neuron_len, &w.desc));
+        w.data = DeviceBuffer(static_cast<size_t>(w.desc.total_bytes));
+        abi_check(mfq_hip_nepq_repack(&w.desc, payload.get(), static_cast<int64_t>(h.body_bytes), w.data.get(), stream));
+    }
     hip_check(hipStreamSynchronize(hs(stream)), "nepq repack");
     if (h.rotation_block) {
         if (!rotation_signs) fail("rotated NEPQ cohort lacks its runtime sign vector");
@@ -623,13 +648,20 @@ void nvq_ffn_swiglu_down(const NvqWeight &gate, const NvqWeight &up, const NvqWe
 void nepq_matmul(const NepqWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y,
                  mfq_stream_t stream) {
     if (expert < 0 || expert >= w.n_experts) fail("expert outside the NEPQ tensor");
-    const int K = w.desc.neuron_len;
+    const int K = static_cast<int>(w.neuron_len());
     if (w.rotation_block) {
         w.rotated.ensure(static_cast<size_t>(M) * K * 2);
         abi_check(mfq_hip_nepq_hadamard(x, x_dtype, ldx, M, K, w.rotation_block, static_cast<const int8_t *>(w.signs.get()),
                                         w.rotated.get(), K, stream));
         x = w.rotated.get();
         ldx = K;
+    }
+    if (w.streams) {
+        const size_t need = mfq_hip_nvqs_gemm_rows_workspace_bytes(&w.sdesc, w.out_per_expert, M);
+        w.workspace.ensure(need);
+        abi_check(mfq_hip_nvqs_gemm_rows(&w.sdesc, w.data.get(), expert * w.out_per_expert, w.out_per_expert, x, x_dtype, ldx, M,
+                                         y, w.out_per_expert, w.workspace.get(), need, stream));
+        return;
     }
     const size_t need = mfq_hip_nepq_gemm_workspace_bytes(&w.desc, w.out_per_expert, M);
     w.workspace.ensure(need);
@@ -655,6 +687,10 @@ void nvq_dequantize(const NvqWeight &w, float *out, mfq_stream_t stream) {
     abi_check(mfq_hip_nvq_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
 }
 void nepq_dequantize(const NepqWeight &w, float *out, mfq_stream_t stream) {
+    if (w.streams) {
+        abi_check(mfq_hip_nvqs_dequant_rows_f32(&w.sdesc, w.data.get(), 0, w.sdesc.out, out, w.sdesc.neuron_len, stream));
+        return;
+    }
     abi_check(mfq_hip_nepq_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
 }
 
@@ -667,7 +703,7 @@ bool is_nvq_linear_dtype(const std::string &d) {
     return d == "NVQ3" || d == "NVQ3J" || d == "NVQ3J-512" || d == "NVQ3J-L" || d == "NVQ2" || d == "NVQ2J" || d == "NVQ2J-L" ||
            d == "NVQ2J-XL" || d == "NIQ3" || d == "NIQ2" || d == "NIQ2J";
 }
-bool is_nepq_linear_dtype(const std::string &d) { return d == "NEPQ1-S" || d == "NEPQ1-L"; }
+bool is_nepq_linear_dtype(const std::string &d) { return d == "NEPQ1-S" || d == "NEPQ1-L" || d == "NEPQ0-S" || d == "NEPQ0-L"; }
 bool is_lowbit_linear_dtype(const std::string &d) { return d == "NVQ1-L" || d == "NVQ1-S" || d == "NPQ0-L" || d == "NPQ0-S"; }
 
 int64_t QuantLinear::out() const {
@@ -680,7 +716,7 @@ int64_t QuantLinear::neuron_len() const {
 }
 int64_t QuantLinear::payload_bytes() const {
     return kind == QuantLinearKind::Nint ? nint->desc.payload_bytes : kind == QuantLinearKind::Nvq ? nvq->payload_bytes()
-         : kind == QuantLinearKind::Nepq ? nepq->desc.payload_bytes : nint8z->desc.payload_bytes;
+         : kind == QuantLinearKind::Nepq ? nepq->payload_bytes() : nint8z->desc.payload_bytes;
 }
 void QuantLinear::forward(const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const {
     if (M == 0) return;  // an empty batch: no rows to write
@@ -698,7 +734,9 @@ void QuantLinear::reserve(int max_M) const {
         if (kind == QuantLinearKind::Nint) n = mfq_hip_nint_gemm_workspace_bytes(&nint->desc, M);
         else if (kind == QuantLinearKind::Nvq)
             n = nvq->streams ? mfq_hip_nvqs_gemm_workspace_bytes(&nvq->sdesc, M) : mfq_hip_nvq_gemm_workspace_bytes(&nvq->desc, M);
-        else if (kind == QuantLinearKind::Nepq) n = mfq_hip_nepq_gemm_workspace_bytes(&nepq->desc, nepq->out_per_expert, M);
+        else if (kind == QuantLinearKind::Nepq)
+            n = nepq->streams ? mfq_hip_nvqs_gemm_rows_workspace_bytes(&nepq->sdesc, nepq->out_per_expert, M)
+                              : mfq_hip_nepq_gemm_workspace_bytes(&nepq->desc, nepq->out_per_expert, M);
         else n = mfq_hip_nint8z_gemm_workspace_bytes(&nint8z->desc, M);
         need = std::max(need, n);
     };
@@ -709,7 +747,7 @@ void QuantLinear::reserve(int max_M) const {
     else if (kind == QuantLinearKind::Nvq) nvq->workspace.ensure(need);
     else if (kind == QuantLinearKind::Nepq) {
         nepq->workspace.ensure(need);
-        if (nepq->rotation_block) rot = static_cast<size_t>(std::max(max_M, 0)) * nepq->desc.neuron_len * 2;
+        if (nepq->rotation_block) rot = static_cast<size_t>(std::max(max_M, 0)) * nepq->neuron_len() * 2;
         nepq->rotated.ensure(rot);
     } else nint8z->workspace.ensure(need);
 }
@@ -827,7 +865,7 @@ NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream
 }
 
 int64_t MoeForeignCohort::payload_bytes() const {
-    if (nepq) return nepq->desc.payload_bytes;
+    if (nepq) return nepq->payload_bytes();
     int64_t n = 0;
     for (const QuantLinear &q : linears) n += q.payload_bytes();
     return n;
@@ -841,7 +879,7 @@ void MoeForeignCohort::dequantize(int local, float *out, mfq_stream_t stream) co
     // the cohort dequantizes as a whole: take the expert's rows out of it
     const size_t rows = static_cast<size_t>(nepq->out_per_expert), K = static_cast<size_t>(nepq->neuron_len());
     DeviceBuffer all(static_cast<size_t>(nepq->n_experts) * rows * K * 4);
-    abi_check(mfq_hip_nepq_dequant_f32(&nepq->desc, nepq->data.get(), static_cast<float *>(all.get()), static_cast<int64_t>(K), stream));
+    nepq_dequantize(*nepq, static_cast<float *>(all.get()), stream);
     hip_check(hipMemcpyAsync(out, static_cast<const float *>(all.get()) + static_cast<size_t>(local) * rows * K, rows * K * 4,
                              hipMemcpyDeviceToDevice, hs(stream)), "foreign cohort dequantize");
     hip_check(hipStreamSynchronize(hs(stream)), "foreign cohort dequantize");
@@ -1488,7 +1526,7 @@ LinearCheckResult run_linear_check(const QuantLinear &lin, int M, int reps) {
     res.payload_bytes = lin.payload_bytes();
     res.weight_bytes = lin.kind == QuantLinearKind::Nint ? lin.nint->desc.total_bytes
                      : lin.kind == QuantLinearKind::Nvq ? lin.nvq->total_bytes()
-                     : lin.kind == QuantLinearKind::Nepq ? lin.nepq->desc.total_bytes : lin.nint8z->desc.total_bytes;
+                     : lin.kind == QuantLinearKind::Nepq ? lin.nepq->total_bytes() : lin.nint8z->desc.total_bytes;
     res.production_weight_gbps = res.weight_bytes / (res.production_ms * 1e6);
     res.payload_gbps = res.payload_bytes / (res.production_ms * 1e6);
     res.production_rel = den > 0 ? std::sqrt(num / den) : std::sqrt(num);

@@ -128,14 +128,18 @@ struct NvqWeight {
 };
 bool is_lowbit_linear_dtype(const std::string &dtype);
 struct NepqWeight {
-    mfq_nepq_desc desc{};
+    mfq_nepq_desc desc{};    // lane-major layout (NEPQ1-S, NEPQ1-L)
+    mfq_nvqs_desc sdesc{};   // streams read in place (NEPQ0-S, NEPQ0-L: the product tables of NPQ0): `streams` set
+    bool streams = false;
     DeviceBuffer data;
     std::string label;
     int n_experts = 0, out_per_expert = 0, rotation_block = 0;
     DeviceBuffer signs;  // int8 [K] when rotated
     mutable DeviceBuffer workspace, rotated;
     int64_t out() const { return out_per_expert; }
-    int64_t neuron_len() const { return desc.neuron_len; }
+    int64_t neuron_len() const { return streams ? sdesc.neuron_len : desc.neuron_len; }
+    int64_t payload_bytes() const { return streams ? sdesc.payload_bytes : desc.payload_bytes; }
+    int64_t total_bytes() const { return streams ? sdesc.total_bytes : desc.total_bytes; }
     static NepqWeight from_blob(const uint8_t *blob, size_t n, const int8_t *rotation_signs = nullptr,
                                 mfq_stream_t stream = nullptr);
 };

@@ -17,8 +17,11 @@ struct NvqsK {
     int out, neuron_len, ng, nvec, nsign;
     int64_t tables_off, anchors_off, state_off, index_off, sign_off;
     int64_t state_bytes, index_bytes, sign_bytes;
-    int kind, sbits, cb_bytes;  // kind 0: sign-stream NVQ; 1: ternary + delta (sign_off = the delta-sign stream); 2: product
+    int kind, sbits, cb_bytes;  // kind 0: sign-stream NVQ; 1: ternary + delta (sign_off = the delta-sign stream); 2: product;
+                                // 3: product with a table pool (sign_off = one bank id byte per neuron and 96 weights)
     float delta, magmax;        // magmax: bound of |magnitude| for the fp16 row scaling
+    int nbank, nsuper, bank_bytes;  // kind 3: tables of the pool, bank ids per neuron, codebook bytes of one table
+    int row0, nrows;            // the neurons a launch works on (an expert of an expert-shaped tensor)
 };
 
 static NvqsK to_k(const mfq_nvqs_desc *d) {
@@ -32,7 +35,10 @@ static NvqsK to_k(const mfq_nvqs_desc *d) {
     k.state_bytes = (static_cast<int64_t>(d->out) * d->ng * d->state_bits + 7) / 8;
     k.index_bytes = (static_cast<int64_t>(d->out) * d->nvec * d->index_bits + 7) / 8;
     k.sign_bytes = d->kind == 0 ? (static_cast<int64_t>(d->out) * d->nsign * 7 + 7) / 8
-                                : (d->kind == 1 ? (static_cast<int64_t>(d->out) * d->ng + 7) / 8 : 0);
+                 : d->kind == 1 ? (static_cast<int64_t>(d->out) * d->ng + 7) / 8
+                 : d->kind == 3 ? static_cast<int64_t>(d->out) * d->nsuper : 0;
+    k.nbank = d->nbank; k.nsuper = d->nsuper; k.bank_bytes = d->nbank > 0 ? (d->cb_bytes - 32 * d->nbank) / d->nbank : 0;
+    k.row0 = 0; k.nrows = d->out;
     return k;
 }
 
@@ -81,6 +87,24 @@ __device__ __forceinline__ NvqsBlock nvqs_block(const NvqsK &k, const uint8_t *w
         const uint32_t idx = sb < k.nvec ? stream_bits(ix_s, (static_cast<int64_t>(n) * k.nvec + sb) * k.ib, k.ib) : 0u;
         const int64_t e1 = (static_cast<int64_t>(state) * 8 + (idx & 7u)) * 4;
         const int64_t e2 = static_cast<int64_t>(k.banks) * 32 + (static_cast<int64_t>(state) * k.entries + (idx >> 3)) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            b.mag[i] = static_cast<float>(cb(e1 + i));
+            b.mag[4 + i] = static_cast<float>(cb(e2 + i));
+        }
+        return b;
+    }
+    if (k.kind == 3) {
+        // the product form with a pool of tables: the neuron's bank id for these 96 weights picks scale LUT and
+        // sub-codebooks (dequantize_nepq, mfq/formats/nepq.py:492-521); tables: per bank first | second, then the LUTs
+        const uint32_t pb = sg_s[static_cast<int64_t>(n) * k.nsuper + g / 4];
+        const float *lut3 = reinterpret_cast<const float *>(reinterpret_cast<const uint8_t *>(lut) + 128 +
+                                                            static_cast<int64_t>(k.nbank) * k.bank_bytes);
+        b.scale = __fmul_rn(anchor, lut3[pb * 8 + state]);
+        const uint32_t idx = sb < k.nvec ? stream_bits(ix_s, (static_cast<int64_t>(n) * k.nvec + sb) * k.ib, k.ib) : 0u;
+        const int64_t base = static_cast<int64_t>(pb) * k.bank_bytes;
+        const int64_t e1 = base + (static_cast<int64_t>(state) * 8 + (idx & 7u)) * 4;
+        const int64_t e2 = base + static_cast<int64_t>(k.banks) * 32 + (static_cast<int64_t>(state) * k.entries + (idx >> 3)) * 4;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             b.mag[i] = static_cast<float>(cb(e1 + i));
@@ -164,13 +188,32 @@ __global__ __launch_bounds__(256) void nvqs_repack_lowbit_kernel(NvqsK k, const 
             const uint32_t enc = table_in_body ? (body[2 * e] | (static_cast<uint32_t>(body[2 * e + 1]) << 8)) : grid[e];
             cb[i] = static_cast<int8_t>(static_cast<int>((enc >> (2 * (i & 7))) & 3u) - 1);
         }
-    } else {
+    } else if (k.kind == 2) {
         table_bytes = 64 + k.cb_bytes;
         if (tid < 16) {
             lut[tid] = tid < k.banks ? f16_to_f32(static_cast<uint16_t>(body[8 + 2 * tid] | (body[9 + 2 * tid] << 8))) : 0.f;
             bfs[tid] = 0u;
         }
         for (int64_t i = tid; i < k.cb_bytes; i += nthreads) cb[i] = static_cast<int8_t>(body[64 + i]);
+    } else {
+        // a pool of nbank tables of 64 + bank_bytes bytes each: the sub-codebooks of all banks, then eight LUT floats per
+        // bank; the 16-entry LUT in front holds the largest scale of any bank per state (the fp16 path's row bound)
+        const int64_t tb = 64 + k.bank_bytes;
+        table_bytes = k.nbank * tb;
+        float *lut3 = reinterpret_cast<float *>(cb + static_cast<int64_t>(k.nbank) * k.bank_bytes);
+        if (tid < 16) {
+            float m = 0.f;
+            for (int pb = 0; pb < k.nbank && tid < k.banks; ++pb)
+                m = fmaxf(m, f16_to_f32(static_cast<uint16_t>(body[pb * tb + 8 + 2 * tid] | (body[pb * tb + 9 + 2 * tid] << 8))));
+            lut[tid] = m;
+            bfs[tid] = 0u;
+        }
+        for (int64_t i = tid; i < static_cast<int64_t>(k.nbank) * 8; i += nthreads) {
+            const int64_t pb = i >> 3, st_ = i & 7;
+            lut3[i] = st_ < k.banks ? f16_to_f32(static_cast<uint16_t>(body[pb * tb + 8 + 2 * st_] | (body[pb * tb + 9 + 2 * st_] << 8))) : 0.f;
+        }
+        for (int64_t i = tid; i < static_cast<int64_t>(k.nbank) * k.bank_bytes; i += nthreads)
+            cb[i] = static_cast<int8_t>(body[(i / k.bank_bytes) * tb + 64 + i % k.bank_bytes]);
     }
     const uint8_t *streams = body + table_bytes;
     float *anchors = reinterpret_cast<float *>(dst + k.anchors_off);
@@ -188,7 +231,7 @@ __global__ __launch_bounds__(256) void nvqs_repack_lowbit_kernel(NvqsK k, const 
 template <typename OutT>
 __global__ __launch_bounds__(256) void nvqs_dequant_kernel(NvqsK k, const uint8_t *__restrict__ w, OutT *__restrict__ outp,
                                                            int64_t ld, float *__restrict__ rowscale, int kpad) {
-    const int n = blockIdx.y;
+    const int row = blockIdx.y, n = k.row0 + row;  // output row, neuron
     const float *lut = nvqs_lut(k, w);
     const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
     const int8_t *cbp = reinterpret_cast<const int8_t *>(bfs + 16);
@@ -201,8 +244,8 @@ __global__ __launch_bounds__(256) void nvqs_dequant_kernel(NvqsK k, const uint8_
         int e = 0;
         if (bound > 0.f) frexpf(bound, &e);
         inv = ldexpf(1.f, 12 - e);
-        if (blockIdx.x == 0 && threadIdx.x == 0) rowscale[n] = ldexpf(1.f, e - 12);
-        for (int col = k.nsign * 8 + blockIdx.x * 256 + threadIdx.x; col < kpad; col += gridDim.x * 256) outp[n * ld + col] = 0;
+        if (blockIdx.x == 0 && threadIdx.x == 0) rowscale[row] = ldexpf(1.f, e - 12);
+        for (int col = k.nsign * 8 + blockIdx.x * 256 + threadIdx.x; col < kpad; col += gridDim.x * 256) outp[row * ld + col] = 0;
     }
     const int sb = blockIdx.x * 256 + threadIdx.x;
     if (sb >= k.nsign) return;
@@ -212,9 +255,9 @@ __global__ __launch_bounds__(256) void nvqs_dequant_kernel(NvqsK k, const uint8_
         const int col = sb * 8 + i;
         const float v = __fmul_rn(b.mag[i], b.scale);
         if constexpr (sizeof(OutT) == 2) {
-            if (col < kpad) outp[n * ld + col] = col < k.neuron_len ? f32_to_f16_rne(v * inv) : uint16_t(0);
+            if (col < kpad) outp[row * ld + col] = col < k.neuron_len ? f32_to_f16_rne(v * inv) : uint16_t(0);
         } else {
-            if (col < k.neuron_len) outp[n * ld + col] = v;
+            if (col < k.neuron_len) outp[row * ld + col] = v;
         }
     }
 }
@@ -237,8 +280,9 @@ __global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *
             *reinterpret_cast<uint32_t *>(cbl + i) = *reinterpret_cast<const uint32_t *>(cbp + i);
         __syncthreads();
     }
-    const int n = blockIdx.x * (blockDim.x >> 6) + wave;
-    if (n >= k.out) return;
+    const int row = blockIdx.x * (blockDim.x >> 6) + wave;
+    if (row >= k.nrows) return;
+    const int n = k.row0 + row;
     const int m0 = blockIdx.y * MB;
     const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[n];
     float acc[MB];
@@ -278,7 +322,7 @@ __global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *
     for (int m = 0; m < MB; ++m) {
         float s = acc[m];
         for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-        if (lane == 0 && m0 + m < M) y[static_cast<int64_t>(m0 + m) * ldy + n] = s;
+        if (lane == 0 && m0 + m < M) y[static_cast<int64_t>(m0 + m) * ldy + row] = s;
     }
 }
 
@@ -295,7 +339,7 @@ template <int XF16, int MB>
 static int nvqs_launch_gemv(const NvqsK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                             hipStream_t st) {
     const size_t ncb = static_cast<size_t>(k.cb_bytes);
-    const dim3 grid(static_cast<unsigned>(ceil_div(k.out, 4)), static_cast<unsigned>(ceil_div(M, MB)));
+    const dim3 grid(static_cast<unsigned>(ceil_div(k.nrows, 4)), static_cast<unsigned>(ceil_div(M, MB)));
     if (ncb <= 49152 && ncb % 4 == 0)
         hipLaunchKernelGGL((nvqs_gemv_kernel<XF16, MB, true>), grid, dim3(256), ncb, st, k, w, x, ldx, M, y, ldy);
     else
@@ -334,6 +378,7 @@ extern "C" int mfq_hip_nvqs_plan(int vector_size, int index_bits, int banks, int
     d->total_bytes = d->sign_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(sg) + 4));
     d->payload_bytes = 2ll * out + st + ix + sg;
     d->kind = 0; d->state_bits = 4; d->cb_bytes = static_cast<int32_t>(ncb); d->delta = 0.f;
+    d->nbank = 0; d->nsuper = 0;
     return MFQ_OK;
 }
 
@@ -341,6 +386,7 @@ extern "C" int mfq_hip_nvqs_plan_lowbit(int format, int state_bits, int out, int
     MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nvqs_plan_lowbit: null descriptor");
     MFQ_REQUIRE(out > 0 && neuron_len > 0, MFQ_ERR_INVALID, "nvqs_plan_lowbit: empty tensor");
     d->vector_size = 8; d->index_parity = 0; d->out = out; d->neuron_len = neuron_len;
+    d->nbank = 0; d->nsuper = 0;
     d->ng = static_cast<int32_t>(ceil_div(neuron_len, 24));
     d->nsign = static_cast<int32_t>(ceil_div(neuron_len, 8));
     d->nvec = d->nsign;
@@ -413,24 +459,79 @@ extern "C" int mfq_hip_nvqs_repack(const mfq_nvqs_desc *d, const void *payload, 
     return check_launch("nvqs_repack");
 }
 
-extern "C" int mfq_hip_nvqs_dequant_f32(const mfq_nvqs_desc *d, const void *weight, float *w_out, int64_t ld,
-                                        mfq_stream_t stream) {
+extern "C" int mfq_hip_nvqs_plan_nepq0(int profile, int banks, int rows, int neuron_len, mfq_nvqs_desc *d) {
+    MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nvqs_plan_nepq0: null descriptor");
+    MFQ_REQUIRE(profile == 0 || profile == 1, MFQ_ERR_INVALID, "nvqs_plan_nepq0: profile=%d (0: NEPQ0-S, 1: NEPQ0-L)", profile);
+    MFQ_REQUIRE(banks >= 1 && banks <= 256, MFQ_ERR_INVALID, "nvqs_plan_nepq0: %d tables (1..256)", banks);
+    MFQ_REQUIRE(rows > 0 && neuron_len > 0 && neuron_len % 8 == 0, MFQ_ERR_INVALID,
+                "NEPQ shape dimensions must be positive, K divisible by 8");
+    int rc = mfq_hip_nvqs_plan_lowbit(profile ? MFQ_NVQS_NPQ0_L : MFQ_NVQS_NPQ0_S, 0, rows, neuron_len, d);
+    if (rc) return rc;
+    const int per_bank = d->cb_bytes;  // sub-codebooks of one table
+    d->kind = 3; d->nbank = banks; d->nsuper = static_cast<int32_t>(ceil_div(d->ng, 4));
+    d->cb_bytes = banks * (per_bank + 32);
+    const int64_t st = (static_cast<int64_t>(rows) * d->ng * d->state_bits + 7) / 8;
+    const int64_t ix = (static_cast<int64_t>(rows) * d->nvec * d->index_bits + 7) / 8;
+    const int64_t sel = static_cast<int64_t>(rows) * d->nsuper;
+    d->anchors_off = static_cast<int64_t>(nvqs_align(128 + static_cast<size_t>(d->cb_bytes)));
+    d->state_off = d->anchors_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(rows) * 4));
+    d->index_off = d->state_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(st) + 4));
+    d->sign_off = d->index_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(ix) + 4));
+    d->total_bytes = d->sign_off + static_cast<int64_t>(nvqs_align(static_cast<size_t>(sel) + 4));
+    d->payload_bytes = 2ll * rows + st + ix + sel;
+    return MFQ_OK;
+}
+
+extern "C" int mfq_hip_nvqs_repack_nepq0(const mfq_nvqs_desc *d, const void *body, int64_t body_bytes, void *weight,
+                                         mfq_stream_t stream) {
+    MFQ_REQUIRE(d && body && weight, MFQ_ERR_INVALID, "nvqs_repack_nepq0: null argument");
+    MFQ_REQUIRE(d->kind == 3, MFQ_ERR_INVALID, "nvqs_repack_nepq0: not a NEPQ0 descriptor");
+    const NvqsK k = to_k(d);
+    const int64_t expect = static_cast<int64_t>(k.nbank) * (64 + k.bank_bytes) + d->payload_bytes;
+    MFQ_REQUIRE(body_bytes == expect, MFQ_ERR_INVALID, "invalid NEPQ tail: remaining=%lld, expected=%lld",
+                static_cast<long long>(body_bytes), static_cast<long long>(expect));
+    hipLaunchKernelGGL(nvqs_repack_lowbit_kernel, dim3(1024), dim3(256), 0, as_stream(stream), k,
+                       static_cast<const uint8_t *>(body), 1, static_cast<const uint16_t *>(nullptr),
+                       static_cast<uint8_t *>(weight));
+    return check_launch("nvqs_repack_nepq0");
+}
+
+static bool nvqs_rows_ok(const mfq_nvqs_desc *d, int row0, int nrows) {
+    return row0 >= 0 && nrows > 0 && static_cast<int64_t>(row0) + nrows <= d->out;
+}
+
+extern "C" int mfq_hip_nvqs_dequant_rows_f32(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, float *w_out,
+                                             int64_t ld, mfq_stream_t stream) {
     MFQ_REQUIRE(d && weight && w_out, MFQ_ERR_INVALID, "nvqs_dequant_f32: null argument");
     MFQ_REQUIRE(ld >= d->neuron_len, MFQ_ERR_INVALID, "nvqs_dequant_f32: ld smaller than neuron_len");
-    MFQ_REQUIRE(d->out <= 65535, MFQ_ERR_UNSUPPORTED, "nvqs_dequant_f32: %d neurons in one call (max 65535)", d->out);
-    const NvqsK k = to_k(d);
-    hipLaunchKernelGGL((nvqs_dequant_kernel<float>), dim3(static_cast<unsigned>(ceil_div(k.nsign, 256)), k.out), dim3(256), 0,
-                       as_stream(stream), k, static_cast<const uint8_t *>(weight), w_out, ld, static_cast<float *>(nullptr), 0);
+    MFQ_REQUIRE(nvqs_rows_ok(d, row0, nrows), MFQ_ERR_INVALID, "nvqs_dequant_f32: rows [%d, %d) outside the tensor's %d", row0,
+                row0 + nrows, d->out);
+    NvqsK k = to_k(d);
+    for (int done = 0; done < nrows; done += 65535) {  // the grid's second dimension holds 65535 rows
+        k.row0 = row0 + done; k.nrows = nrows - done < 65535 ? nrows - done : 65535;
+        hipLaunchKernelGGL((nvqs_dequant_kernel<float>), dim3(static_cast<unsigned>(ceil_div(k.nsign, 256)), k.nrows), dim3(256),
+                           0, as_stream(stream), k, static_cast<const uint8_t *>(weight), w_out + static_cast<int64_t>(done) * ld,
+                           ld, static_cast<float *>(nullptr), 0);
+    }
     return check_launch("nvqs_dequant_f32");
 }
 
-extern "C" int mfq_hip_nvqs_gemv(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
-                                 float *y, int64_t ldy, mfq_stream_t stream) {
+extern "C" int mfq_hip_nvqs_dequant_f32(const mfq_nvqs_desc *d, const void *weight, float *w_out, int64_t ld,
+                                        mfq_stream_t stream) {
+    MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nvqs_dequant_f32: null argument");
+    return mfq_hip_nvqs_dequant_rows_f32(d, weight, 0, d->out, w_out, ld, stream);
+}
+
+extern "C" int mfq_hip_nvqs_gemv_rows(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, const void *x,
+                                      int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream) {
     MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nvqs_gemv: null argument");
     MFQ_REQUIRE(M >= 1, MFQ_ERR_INVALID, "nvqs_gemv: M=%d", M);
     MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvqs_gemv: x_dtype=%d", x_dtype);
-    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nvqs_gemv: ldx/ldy smaller than the tensor");
-    const NvqsK k = to_k(d);
+    MFQ_REQUIRE(nvqs_rows_ok(d, row0, nrows), MFQ_ERR_INVALID, "nvqs_gemv: rows [%d, %d) outside the tensor's %d", row0,
+                row0 + nrows, d->out);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= nrows, MFQ_ERR_INVALID, "nvqs_gemv: ldx/ldy smaller than the tensor");
+    NvqsK k = to_k(d);
+    k.row0 = row0; k.nrows = nrows;
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
     hipStream_t st = as_stream(stream);
@@ -444,32 +545,51 @@ extern "C" int mfq_hip_nvqs_gemv(const mfq_nvqs_desc *d, const void *weight, con
     return nvqs_launch_gemv<0, 8>(k, w, xp, ldx, M, y, ldy, st);
 }
 
-extern "C" size_t mfq_hip_nvqs_gemm_workspace_bytes(const mfq_nvqs_desc *d, int M) {
-    if (!d || M <= kNvqsGemvMaxM) return 0;
-    return dequant_gemm_workspace(d->out, d->neuron_len, M);
+extern "C" int mfq_hip_nvqs_gemv(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
+                                 float *y, int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nvqs_gemv: null argument");
+    return mfq_hip_nvqs_gemv_rows(d, weight, 0, d->out, x, x_dtype, ldx, M, y, ldy, stream);
 }
 
-extern "C" int mfq_hip_nvqs_gemm(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
-                                 float *y, int64_t ldy, void *workspace, size_t workspace_bytes, mfq_stream_t stream) {
+extern "C" size_t mfq_hip_nvqs_gemm_rows_workspace_bytes(const mfq_nvqs_desc *d, int nrows, int M) {
+    if (!d || M <= kNvqsGemvMaxM) return 0;
+    return dequant_gemm_workspace(nrows, d->neuron_len, M);
+}
+extern "C" size_t mfq_hip_nvqs_gemm_workspace_bytes(const mfq_nvqs_desc *d, int M) {
+    return d ? mfq_hip_nvqs_gemm_rows_workspace_bytes(d, d->out, M) : 0;
+}
+
+extern "C" int mfq_hip_nvqs_gemm_rows(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, const void *x,
+                                      int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, void *workspace,
+                                      size_t workspace_bytes, mfq_stream_t stream) {
     MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nvqs_gemm: null argument");
-    if (M <= kNvqsGemvMaxM) return mfq_hip_nvqs_gemv(d, weight, x, x_dtype, ldx, M, y, ldy, stream);
+    if (M <= kNvqsGemvMaxM) return mfq_hip_nvqs_gemv_rows(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, stream);
     MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvqs_gemm: x_dtype=%d", x_dtype);
-    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nvqs_gemm: ldx/ldy smaller than the tensor");
-    MFQ_REQUIRE(d->out <= 65535, MFQ_ERR_UNSUPPORTED, "nvqs_gemm: %d neurons in one call (max 65535)", d->out);
-    const size_t need = dequant_gemm_workspace(d->out, d->neuron_len, M);
+    MFQ_REQUIRE(nvqs_rows_ok(d, row0, nrows), MFQ_ERR_INVALID, "nvqs_gemm: rows [%d, %d) outside the tensor's %d", row0,
+                row0 + nrows, d->out);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= nrows, MFQ_ERR_INVALID, "nvqs_gemm: ldx/ldy smaller than the tensor");
+    MFQ_REQUIRE(nrows <= 65535, MFQ_ERR_UNSUPPORTED, "nvqs_gemm: %d neurons in one call (max 65535)", nrows);
+    const size_t need = dequant_gemm_workspace(nrows, d->neuron_len, M);
     MFQ_REQUIRE(workspace && workspace_bytes >= need, MFQ_ERR_WORKSPACE, "nvqs_gemm: workspace %zu < %zu bytes", workspace_bytes,
                 need);
     hipStream_t st = as_stream(stream);
     uint16_t *x16, *w16;
     float *xscale, *wscale;
     int Kp;
-    dequant_gemm_carve(workspace, d->out, d->neuron_len, M, x16, xscale, w16, wscale, Kp);
+    dequant_gemm_carve(workspace, nrows, d->neuron_len, M, x16, xscale, w16, wscale, Kp);
     int rc = x_prep(x, x_dtype, ldx, M, d->neuron_len, Kp, x16, xscale, st);
     if (rc) return rc;
-    const NvqsK k = to_k(d);
-    hipLaunchKernelGGL((nvqs_dequant_kernel<uint16_t>), dim3(static_cast<unsigned>(ceil_div(Kp / 8 > k.nsign ? Kp / 8 : k.nsign, 256)), k.out),
+    NvqsK k = to_k(d);
+    k.row0 = row0; k.nrows = nrows;
+    hipLaunchKernelGGL((nvqs_dequant_kernel<uint16_t>), dim3(static_cast<unsigned>(ceil_div(Kp / 8 > k.nsign ? Kp / 8 : k.nsign, 256)), nrows),
                        dim3(256), 0, st, k, static_cast<const uint8_t *>(weight), w16, static_cast<int64_t>(Kp), wscale, Kp);
     rc = check_launch("nvqs_dequant_f16");
     if (rc) return rc;
-    return gemm_f16_nt(x16, Kp, w16, Kp, M, d->out, Kp, xscale, wscale, y, ldy, st);
+    return gemm_f16_nt(x16, Kp, w16, Kp, M, nrows, Kp, xscale, wscale, y, ldy, st);
+}
+
+extern "C" int mfq_hip_nvqs_gemm(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
+                                 float *y, int64_t ldy, void *workspace, size_t workspace_bytes, mfq_stream_t stream) {
+    MFQ_REQUIRE(d != nullptr, MFQ_ERR_INVALID, "nvqs_gemm: null argument");
+    return mfq_hip_nvqs_gemm_rows(d, weight, 0, d->out, x, x_dtype, ldx, M, y, ldy, workspace, workspace_bytes, stream);
 }

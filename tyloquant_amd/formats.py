@@ -459,7 +459,7 @@ _NEPQ_HDR = struct.Struct("<4sBBBBIIIIIQ")
 NEPQ_PROFILE = {"NEPQ0-S": 0, "NEPQ0-L": 1, "NEPQ1-S": 2, "NEPQ1-L": 3}
 NEPQ_LABEL = {v: k for k, v in NEPQ_PROFILE.items()}
 #               profile: (state_bits, index_bits, aux_bits, table_bytes)
-NEPQ_BITS = {2: (4, 9, 1, 2048), 3: (3, 11, 1, 4096)}
+NEPQ_BITS = {0: (2, 6, 0, 320), 1: (3, 7, 0, 832), 2: (4, 9, 1, 2048), 3: (3, 11, 1, 4096)}
 
 
 @dataclass
@@ -515,6 +515,18 @@ def parse_nepq(blob) -> NepqHeader:
         (rows * ng * ab + 7) // 8 + rows * nsuper
     if len(blob) - _NEPQ_HDR.size != expect:
         raise ValueError(f"invalid NEPQ tail: consumed={_NEPQ_HDR.size + expect}, size={len(blob)}")
+    if pid < 2:     # NEPQ0: every table of the pool is an NPQ0 table (mfq/formats/nepq.py:270-290)
+        base = "NPQ0-S" if pid == 0 else "NPQ0-L"
+        tv, states, second = _NPQ0_TABLES[base]
+        for bnk in range(banks):
+            head = bytes(blob[_NEPQ_HDR.size + bnk * tb: _NEPQ_HDR.size + bnk * tb + 64])
+            if tuple(head[:6]) != (tv, states, 3, ib - 3, 24, 8):
+                raise ValueError(f"unsupported {NEPQ_LABEL[pid]} table profile")
+            if any(head[6:8]) or any(head[8 + 2 * states:64]):
+                raise ValueError(f"invalid {NEPQ_LABEL[pid]} reserved table bytes")
+            lut = np.frombuffer(head, dtype="<f2", count=states, offset=8).astype(np.float32)
+            if not np.isfinite(lut).all() or np.any(lut < 0) or float(lut.max()) <= 0:
+                raise ValueError(f"{NEPQ_LABEL[pid]} scale LUT must be finite and non-negative")
     return NepqHeader(NEPQ_LABEL[pid], pid, E, out, K, banks, rblock, rseed, ng, nvec, nsuper, _NEPQ_HDR.size, expect)
 
 

@@ -335,7 +335,7 @@ def is_nvq_linear_dtype(dtype: str) -> bool:
 
 
 def is_nepq_linear_dtype(dtype: str) -> bool:
-    return dtype in ("NEPQ1-S", "NEPQ1-L")
+    return dtype in ("NEPQ1-S", "NEPQ1-L", "NEPQ0-S", "NEPQ0-L")
 
 
 @dataclass

@@ -181,10 +181,12 @@ def nvq_matmul(w: NvqWeight, x: torch.Tensor, *, force: str | None = None) -> to
 
 
 class NepqWeight:
-    """[experts, out_per_expert, K]; a dense linear is the experts == 1 case."""
+    """[experts, out_per_expert, K]; a dense linear is the experts == 1 case.  NEPQ1-S / NEPQ1-L live in the lane-major
+    layout of mfq_hip_nepq_*; NEPQ0-S / NEPQ0-L (`streams`) keep their bit streams and run on mfq_hip_nvqs_*_rows."""
 
     def __init__(self, desc, data, header: F.NepqHeader, signs):
         self.desc, self.data, self.label = desc, data, header.label
+        self.streams = isinstance(desc, L.NvqsDesc)
         self.n_experts, self.out_per_expert, self.neuron_len = header.n_experts, header.out_per_expert, header.neuron_len
         self.out = header.out_per_expert
         self.rotation_block, self.rotation_seed, self.signs = header.rotation_block, header.rotation_seed, signs
@@ -198,12 +200,18 @@ class NepqWeight:
     def from_blob(blob, device="cuda", rotation_signs=None) -> "NepqWeight":
         h = F.parse_nepq(blob)
         device = torch.device(device)
-        desc = L.NepqDesc()
         lib = L.lib()
-        L.check(lib.mfq_hip_nepq_plan(h.profile, h.banks, h.n_experts * h.out_per_expert, h.neuron_len, C.byref(desc)))
         payload = _upload(blob, h.body_off, h.body_bytes, device)
-        data = torch.empty(int(desc.total_bytes), dtype=torch.uint8, device=device)
-        L.check(lib.mfq_hip_nepq_repack(C.byref(desc), _ptr(payload), h.body_bytes, _ptr(data), _stream()))
+        if h.profile < 2:       # NEPQ0: the product tables of NPQ0, read in place
+            desc = L.NvqsDesc()
+            L.check(lib.mfq_hip_nvqs_plan_nepq0(h.profile, h.banks, h.n_experts * h.out_per_expert, h.neuron_len, C.byref(desc)))
+            data = torch.empty(int(desc.total_bytes), dtype=torch.uint8, device=device)
+            L.check(lib.mfq_hip_nvqs_repack_nepq0(C.byref(desc), _ptr(payload), h.body_bytes, _ptr(data), _stream()))
+        else:
+            desc = L.NepqDesc()
+            L.check(lib.mfq_hip_nepq_plan(h.profile, h.banks, h.n_experts * h.out_per_expert, h.neuron_len, C.byref(desc)))
+            data = torch.empty(int(desc.total_bytes), dtype=torch.uint8, device=device)
+            L.check(lib.mfq_hip_nepq_repack(C.byref(desc), _ptr(payload), h.body_bytes, _ptr(data), _stream()))
         torch.cuda.current_stream().synchronize()
         signs = None
         if h.rotation_block:
@@ -218,7 +226,11 @@ class NepqWeight:
     def dequantize(self) -> torch.Tensor:
         rows = self.n_experts * self.out_per_expert
         w = torch.empty((rows, self.neuron_len), dtype=torch.float32, device=self.data.device)
-        L.check(L.lib().mfq_hip_nepq_dequant_f32(C.byref(self.desc), _ptr(self.data), _ptr(w), self.neuron_len, _stream()))
+        if self.streams:
+            L.check(L.lib().mfq_hip_nvqs_dequant_rows_f32(C.byref(self.desc), _ptr(self.data), 0, rows, _ptr(w),
+                                                          self.neuron_len, _stream()))
+        else:
+            L.check(L.lib().mfq_hip_nepq_dequant_f32(C.byref(self.desc), _ptr(self.data), _ptr(w), self.neuron_len, _stream()))
         return w.reshape(self.n_experts, self.out_per_expert, self.neuron_len)
 
 
@@ -247,6 +259,12 @@ def nepq_matmul(w: NepqWeight, x: torch.Tensor, expert: int = 0, *, force: str |
         return y.reshape(*x.shape[:-1], n)
     lib = L.lib()
     row0 = expert * n
+    if w.streams:
+        need = lib.mfq_hip_nvqs_gemm_rows_workspace_bytes(C.byref(w.desc), n, M)
+        ws = w._ws.get(need, x.device)
+        L.check(lib.mfq_hip_nvqs_gemm_rows(C.byref(w.desc), _ptr(w.data), row0, n, _ptr(x2), _x_dtype(x2), x2.stride(0), M,
+                                           _ptr(y), n, _ptr(ws), need, _stream()))
+        return y.reshape(*x.shape[:-1], n)
     if force == "gemv":
         L.check(lib.mfq_hip_nepq_gemv(C.byref(w.desc), _ptr(w.data), row0, n, _ptr(x2), _x_dtype(x2), x2.stride(0), M,
                                       _ptr(y), n, _stream()))
