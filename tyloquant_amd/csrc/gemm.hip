@@ -163,11 +163,24 @@ __global__ __launch_bounds__(256) void x_prep_vec_kernel(const uint16_t *__restr
     for (int g0 = 0; g0 < nsteps * 16; g0 += 256) {
         const int g = g0 + tid;
         float acc = 0.f;
-        if (g < nsteps * 16)
-            for (int i = 0; i < gs; ++i) {
-                const int k = g * gs + i;
-                if (k < K) acc += f16_to_f32(rowh[k]);
+        if (g < nsteps * 16) {
+            if (gs % 4 == 0 && (g + 1) * gs <= Kp) {
+                // four halves per LDS read, added in k order; the row is zero from K to Kp
+                const uint2 *q = reinterpret_cast<const uint2 *>(rowh + g * gs);
+                for (int i = 0; i < gs / 4; ++i) {
+                    const uint2 v = q[i];
+                    acc += f16_to_f32(static_cast<uint16_t>(v.x & 0xffffu));
+                    acc += f16_to_f32(static_cast<uint16_t>(v.x >> 16));
+                    acc += f16_to_f32(static_cast<uint16_t>(v.y & 0xffffu));
+                    acc += f16_to_f32(static_cast<uint16_t>(v.y >> 16));
+                }
+            } else {
+                for (int i = 0; i < gs; ++i) {
+                    const int k = g * gs + i;
+                    if (k < K) acc += f16_to_f32(rowh[k]);
+                }
             }
+        }
         __syncthreads();
         gsum[tid] = acc;
         __syncthreads();

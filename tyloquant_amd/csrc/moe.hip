@@ -228,7 +228,13 @@ __global__ __launch_bounds__(256) void moe_count_kernel(const int32_t *__restric
     __shared__ int red[4];
     const int e = blockIdx.x, tid = threadIdx.x;
     int c = 0;
-    for (int p = tid; p < n_pairs; p += 256) c += (ids[p] == e);
+    const bool vec = (reinterpret_cast<uintptr_t>(ids) & 15) == 0;  // four ids per load
+    const int n4 = vec ? n_pairs & ~3 : 0;
+    for (int p = tid * 4; p < n4; p += 1024) {
+        const int4 v = *reinterpret_cast<const int4 *>(ids + p);
+        c += (v.x == e) + (v.y == e) + (v.z == e) + (v.w == e);
+    }
+    for (int p = n4 + tid; p < n_pairs; p += 256) c += (ids[p] == e);
     for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
     if ((tid & 63) == 0) red[tid >> 6] = c;
     __syncthreads();
@@ -282,16 +288,31 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(const int32_t *__restr
     const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid == 0) base = expert_bounds[e];
     __syncthreads();
-    for (int p0 = 0; p0 < n_pairs; p0 += 256) {
-        const int p = p0 + tid;
-        const bool hit = p < n_pairs && ids[p] == e;
-        const unsigned long long ball = __ballot(hit);
-        const int before = __popcll(ball & ((1ull << lane) - 1ull));
-        if (lane == 0) wsum[wave] = __popcll(ball);
+    // windows of 1024 pairs, four consecutive ones per thread: the pairs of the expert keep their order
+    const bool vec = (reinterpret_cast<uintptr_t>(ids) & 15) == 0;
+    for (int p0 = 0; p0 < n_pairs; p0 += 1024) {
+        const int p = p0 + tid * 4;
+        int v[4];
+        if (vec && p + 3 < n_pairs) {
+            const int4 q = *reinterpret_cast<const int4 *>(ids + p);
+            v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) v[t] = p + t < n_pairs ? ids[p + t] : -1;
+        }
+        const int mine = (v[0] == e) + (v[1] == e) + (v[2] == e) + (v[3] == e);
+        int inc = mine;
+        for (int o = 1; o < 64; o <<= 1) {
+            const int u = __shfl_up(inc, o, 64);
+            if (lane >= o) inc += u;
+        }
+        if (lane == 63) wsum[wave] = inc;
         __syncthreads();
-        int off = 0;
+        int off = base + inc - mine;
         for (int wv = 0; wv < wave; ++wv) off += wsum[wv];
-        if (hit) ids_dst[base + off + before] = p;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (v[t] == e) ids_dst[off++] = p + t;
         __syncthreads();
         if (tid == 0) base += wsum[0] + wsum[1] + wsum[2] + wsum[3];
         __syncthreads();
