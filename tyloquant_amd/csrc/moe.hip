@@ -979,11 +979,47 @@ extern "C" int mfq_hip_moe_swiglu(const float *gate_up, int64_t ld, int rows, in
     return mfq_hip_moe_glu(gate_up, ld, rows, W, hidden, out_dtype, ldh, MFQ_GLU_SILU, stream);
 }
 
+namespace mfq {
+// The same sums, four neighbouring columns per thread (H % 4 == 0, 16-byte aligned rows): same order of the fused
+// multiply-adds per element, a quarter of the load instructions.
+__global__ __launch_bounds__(256) void moe_reduce4_kernel(const float *__restrict__ pair, const float *__restrict__ wts,
+                                                          int T, int R, int H, const float *__restrict__ shared,
+                                                          const float *__restrict__ gate_logits, float *__restrict__ out) {
+    const int h4 = H >> 2;
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= static_cast<int64_t>(T) * h4) return;
+    const int t = static_cast<int>(idx / h4), c = static_cast<int>(idx - static_cast<int64_t>(t) * h4) * 4;
+    float4_t v = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < R; ++r) {
+        const int64_t p = static_cast<int64_t>(t) * R + r;
+        const float w = wts[p];
+        const float4_t q = *reinterpret_cast<const float4_t *>(pair + p * H + c);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = fmaf(w, q[i], v[i]);
+    }
+    if (shared) {
+        const float g = gate_logits ? 1.f / (1.f + expf(-gate_logits[t])) : 1.f;
+        const float4_t q = *reinterpret_cast<const float4_t *>(shared + static_cast<int64_t>(t) * H + c);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = fmaf(g, q[i], v[i]);
+    }
+    *reinterpret_cast<float4_t *>(out + static_cast<int64_t>(t) * H + c) = v;
+}
+}  // namespace mfq
+
 extern "C" int mfq_hip_moe_weighted_reduce(const float *pair, const float *weights, int T, int R, int H,
                                            const float *shared, const float *gate_logits, float *out,
                                            mfq_stream_t stream) {
     MFQ_REQUIRE(pair && weights && out, MFQ_ERR_INVALID, "moe_weighted_reduce: null argument");
     MFQ_REQUIRE(T > 0 && R > 0 && H > 0, MFQ_ERR_INVALID, "moe_weighted_reduce: bad shape");
+    const bool vec = H % 4 == 0 && ((reinterpret_cast<uintptr_t>(pair) | reinterpret_cast<uintptr_t>(out) |
+                                     reinterpret_cast<uintptr_t>(shared)) & 15) == 0;
+    if (vec) {
+        const unsigned blocks4 = static_cast<unsigned>(ceil_div(static_cast<int64_t>(T) * (H / 4), 256));
+        hipLaunchKernelGGL(moe_reduce4_kernel, dim3(blocks4), dim3(256), 0, as_stream(stream), pair, weights, T, R, H, shared,
+                           gate_logits, out);
+        return check_launch("moe_weighted_reduce");
+    }
     const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<int64_t>(T) * H, 256));
     hipLaunchKernelGGL(moe_reduce_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), pair, weights, T, R, H, shared,
                        gate_logits, out);
