@@ -425,9 +425,13 @@ def parse_nvq(blob) -> NvqHeader:
     codebook = NVQ_ID_CODEBOOK[cid]
     jsc, custom = bool(enc & 0x20), bool(enc & 0x40)
     sign_mode = "index_parity" if enc & 0x80 else "even"
+    if ndim > 8 or len(blob) < _NVQ_HDR.size + 8 * ndim + 4:
+        raise ValueError("truncated NVQ header")
     off = _NVQ_HDR.size + 8 * ndim
     out, = struct.unpack_from("<I", blob, off)
     off += 4
+    if gs <= 0 or neuron_len <= 0 or out <= 0 or not 1 <= sub_bits <= 8:
+        raise ValueError("NVQ dimensions must be positive (groupsize, neuron_len, rows) and sub_bits in [1,8]")
     vs, ib = (8 if codebook.startswith("e8") else 4), NVQ_INDEX_BITS[codebook]
     ng, nvec, nsign = math.ceil(neuron_len / gs), math.ceil(neuron_len / vs), math.ceil(neuron_len / 8)
     streams = 2 * out + (out * ng * sub_bits + 7) // 8 + (out * nvec * ib + 7) // 8 + (out * nsign * 7 + 7) // 8
