@@ -192,6 +192,29 @@ def test_nepq_matrix_core_path_multi_step(label, out, K, M, banks):
         _check(nepq_matmul(w, x, e, force="gemv").cpu().numpy(), O.linear_forward_f64(want[e], x.float().cpu().numpy()))
 
 
+@pytest.mark.parametrize("label,banks", [("NEPQ1-S", 5), ("NEPQ1-L", 16)])
+@pytest.mark.parametrize("E,cus,out", [(2, 4, 128), (2, 2, 96), (2, 3, 208), (1, 2, 88), (1, 3, 200), (2, 2, 16)])
+def test_nepq_one_row_gemv_row_blocks_per_block(cu_count, label, banks, E, cus, out):
+    """One activation row: a block owns ceil(row-blocks / CUs) row-blocks, up to four (2, 3, 4, 3, 4 and 1 here), the
+    last block fewer than the others; a second expert at its own row offset; a ragged last row-block."""
+    from tyloquant_amd.runtime_vq import NepqWeight, nepq_matmul
+    rng = np.random.default_rng(910 + cus + out)
+    K = 1160
+    t = synth.nepq_random(rng, label, E, out, K, banks)
+    w = NepqWeight.from_blob(O.pack_nepq(t))
+    want = O.dequantize_nepq(t)
+    cu_count(cus)
+    for e in range(E):
+        x, xf = _x(rng, 1, K)
+        _check(nepq_matmul(w, x, e).cpu().numpy(), O.linear_forward(want[e], xf))
+    # 2 .. 32 rows: the 16-row tile kernel with the same ownership (up to three row-blocks per block; four fall back
+    # to the streaming kernel), one and two tiles
+    for M in (2, 16, 21):
+        x, xf = _x(rng, M, K)
+        for e in range(E):
+            _check(nepq_matmul(w, x, e, force="gemv").cpu().numpy(), O.linear_forward_f64(want[e], xf))
+
+
 @pytest.mark.parametrize("label,out,K,M,banks", [("NEPQ1-S", 130 - 2, 1024, 70, 4), ("NEPQ1-L", 48, 4104, 300, 16),
                                                   ("NEPQ1-L", 272, 1544, 100, 40), ("NEPQ1-S", 272, 1024, 8300, 3),
                                                   ("NEPQ1-S", 1040, 1024, 3329, 5)])

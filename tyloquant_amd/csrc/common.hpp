@@ -48,6 +48,27 @@ __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
     }
 }
 
+// Block-wide copy of n dwords (a lookup table) from global memory into LDS.  A thread requests four 16-byte pieces
+// before it stores the first: a plain dword loop waits one round trip to memory per piece, which for a 32 KB table
+// and a block of a thousand threads is eight round trips in a row at the head of the kernel.  dst: 16-byte aligned.
+__device__ __forceinline__ void table_to_lds(uint32_t *dst, const uint32_t *src, int n, int tid, int nt) {
+    if ((reinterpret_cast<uintptr_t>(src) & 15) == 0 && n % 4 == 0) {
+        const u32x4_t *s4 = reinterpret_cast<const u32x4_t *>(src);
+        u32x4_t *d4 = reinterpret_cast<u32x4_t *>(dst);
+        const int n4 = n / 4;
+        for (int i0 = tid; i0 < n4; i0 += 4 * nt) {
+            u32x4_t v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = s4[min(i0 + u * nt, n4 - 1)];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (i0 + u * nt < n4) d4[i0 + u * nt] = v[u];
+        }
+    } else {
+        for (int i = tid; i < n; i += nt) dst[i] = src[i];
+    }
+}
+
 __device__ __forceinline__ float bf16_to_f32(uint16_t v) { return __uint_as_float(static_cast<uint32_t>(v) << 16); }
 __device__ __forceinline__ float f16_to_f32(uint16_t v) {
     return static_cast<float>(__builtin_bit_cast(_Float16, v));

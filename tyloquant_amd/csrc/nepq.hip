@@ -148,15 +148,20 @@ __global__ void nepq_dequant_kernel(NepqK k, const uint8_t *__restrict__ w, int 
 
 // GEMV: sum_i (code_i + bias) x_i = sum_i digit_i x_i + (bias - 1) * xsum, digit = code + 1 in {0,1,2};
 // a table entry e (8 two-bit digits) becomes four biased pairs from t = e | e << 14.
-template <int XF16, int MB, int TAB_LDS>
+// A block owns RPB consecutive row-blocks: the lookup table and the activations are staged once for all of them, and a
+// wave requests the units of all its row-blocks of a step before it decodes the first.
+// PROF: the profile (2 = S, 3 = L) as a constant -- a decoder that branches on it at run time splits every unit into
+// basic blocks the scheduler cannot mix, and the kernel spills.
+template <int XF16, int MB, int TAB_LDS, int RPB, int PROF>
 __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t *__restrict__ w, int rb0, int row0,
                                                          int nrows, const uint16_t *__restrict__ x, int64_t ldx, int M,
                                                          float *__restrict__ y, int64_t ldy, int spw) {
-    extern __shared__ uint32_t lds[];
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     constexpr uint32_t MAGIC = 0x64006400u;  // fp16 (1024, 1024): digit d becomes 1024 + d
     constexpr float BIAS = 1024.f;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
-    const int rb = rb0 + blockIdx.x;
+    const int rb = rb0 + blockIdx.x * RPB;
+    const int rb_last = rb0 + (nrows + 15) / 16 - 1;  // row-blocks past it repeat it; their sums are dropped
     const uint16_t *xr[MB];
     float *yr[MB];
     dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
@@ -165,7 +170,7 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
     uint16_t *ltab = reinterpret_cast<uint16_t *>(lds);
     uint32_t *xbase = lds;
     if constexpr (TAB_LDS) {
-        for (int i = tid; i < ntab / 2; i += blockDim.x) lds[i] = reinterpret_cast<const uint32_t *>(gtab)[i];
+        table_to_lds(lds, reinterpret_cast<const uint32_t *>(gtab), ntab / 2, tid, blockDim.x);
         xbase = lds + ntab / 2;
     }
     const uint16_t *tab = TAB_LDS ? ltab : gtab;
@@ -181,49 +186,65 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
     if constexpr (TAB_LDS) __syncthreads();  // the LDS table copy was made by the whole block
 
     const int r = lane & 15, kb = lane >> 4;
-    const uint8_t *base = w + static_cast<int64_t>(rb) * k.rowblock_bytes;
-    const float delta = k.profile == 2 ? 0.15625f : 0.125f;
-    float acc[MB];
+    const float delta = PROF == 2 ? 0.15625f : 0.125f;
+    float acc[RPB][MB];
 #pragma unroll
-    for (int m = 0; m < MB; ++m) acc[m] = 0.f;
+    for (int i = 0; i < RPB; ++i)
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[i][m] = 0.f;
     for (int s = s0; s < s1; ++s) {
-        const uint8_t *sp = base + s * k.step_bytes;
-        uint32_t q[4];
+        uint32_t q[RPB][4], tails[RPB], banks4[RPB];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) q[j] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sp) + j * 64 + lane);
-        uint32_t tails = 0;
-        if (k.tail) tails = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sp + 1024) + lane);
-        const uint32_t banks4 = *(reinterpret_cast<const uint32_t *>(sp + 1024 + (k.tail ? 256 : 0)) + r);
+        for (int i = 0; i < RPB; ++i) {
+            const uint8_t *sp = w + static_cast<int64_t>(min(rb + i, rb_last)) * k.rowblock_bytes + s * k.step_bytes;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                q[i][j] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sp) + j * 64 + lane);
+            tails[i] = 0;
+            if ((PROF == 3)) tails[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(sp + 1024) + lane);
+            banks4[i] = *(reinterpret_cast<const uint32_t *>(sp + 1024 + ((PROF == 3) ? 256 : 0)) + r);
+        }
+        // unit column by unit column: the twelve activation pairs of a column are read once for all row-blocks
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int lg = (s - s0) * 16 + 4 * j + kb;
-            const NepqUnit u = nepq_decode(k.profile, q[j], (tails >> (8 * j)) & 0xffu);
-            const uint16_t *bank = tab + ((banks4 >> (8 * j)) & 0xffu) * k.entries;
-            const float st = static_cast<float>(u.state);
-            const float off = (u.aux ? -delta : delta) - 1.f - BIAS;
-            float raw[MB];
 #pragma unroll
-            for (int m = 0; m < MB; ++m) raw[m] = 0.f;
+            for (int i = 0; i < RPB; ++i) {
+                const int lg = (s - s0) * 16 + 4 * j + kb;
+                const NepqUnit u = nepq_decode(PROF, q[i][j], (tails[i] >> (8 * j)) & 0xffu);
+                const uint16_t *bank = tab + ((banks4[i] >> (8 * j)) & 0xffu) * k.entries;
+                const float st = static_cast<float>(u.state);
+                const float off = (u.aux ? -delta : delta) - 1.f - BIAS;
+                float raw[MB];
 #pragma unroll
-            for (int v = 0; v < 3; ++v) {
-                const uint32_t e = bank[u.idx[v]];
-                const uint32_t t = e | (e << 14);
+                for (int m = 0; m < MB; ++m) raw[m] = 0.f;
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    const uint32_t pr = ((t >> (4 * p)) & 0x00030003u) | MAGIC;
+                for (int v = 0; v < 3; ++v) {
+                    const uint32_t e = bank[u.idx[v]];
+                    const uint32_t t = e | (e << 14);
 #pragma unroll
-                    for (int m = 0; m < MB; ++m) raw[m] = dot2h(pr, xs[m * npairs + lg * 12 + 4 * v + p], raw[m]);
+                    for (int p = 0; p < 4; ++p) {
+                        const uint32_t pr = ((t >> (4 * p)) & 0x00030003u) | MAGIC;
+#pragma unroll
+                        for (int m = 0; m < MB; ++m) raw[m] = dot2h(pr, xs[m * npairs + lg * 12 + 4 * v + p], raw[m]);
+                    }
                 }
-            }
 #pragma unroll
-            for (int m = 0; m < MB; ++m) acc[m] = fmaf(st, fmaf(off, xsum[(m * ngl + lg) * 2], raw[m]), acc[m]);
+                for (int m = 0; m < MB; ++m) acc[i][m] = fmaf(st, fmaf(off, xsum[(m * ngl + lg) * 2], raw[m]), acc[i][m]);
+                // one unit at a time: left alone, the scheduler starts the table reads of all units at once and spills
+                if constexpr (RPB > 1 || MB > 2) __builtin_amdgcn_sched_barrier(0);
+            }
         }
     }
-    const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[rb * 16 + r];
-    float v[MB];
 #pragma unroll
-    for (int m = 0; m < MB; ++m) v[m] = anchor * acc[m];
-    finish_rows<MB>(v, red, wave, nwaves, lane, rb, row0, nrows, yr);
+    for (int i = 0; i < RPB; ++i) {
+        const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[min(rb + i, rb_last) * 16 + r];
+        float v[MB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) v[m] = anchor * acc[i][m];
+        park_rows<MB>(v, red, i * nwaves + wave, lane);
+    }
+    // a row-block past the tensor's last has rows beyond nrows: flush_rows drops them
+    flush_rows<MB>(red, nwaves, RPB, rb, row0, nrows, yr);
 }
 
 // ---- matrix-core path: up to 16 activation rows per streamed pass ----------------------------------
@@ -231,18 +252,18 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
 // (code + 1) that become four (1024 + digit) fp16 pairs and, with one packed FMA each, state * digit (exact).
 // The remaining part of the value, state * (bias - 1) * X_g, is one more MFMA per step against the group sums
 // X_g (two fp16 halves), exactly as the NINT minimum term.  Padding groups have state 0.
-template <int XF16, int NB, int TAB_LDS>
+template <int XF16, int NB, int TAB_LDS, int PROF>
 __global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *__restrict__ w, int rb_first, int row0,
                                                         int nrows, const uint16_t *__restrict__ x, int64_t ldx, int M,
                                                         float *__restrict__ y, int64_t ldy, int spw) {
-    extern __shared__ uint32_t lds[];
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint16_t *gtab = reinterpret_cast<const uint16_t *>(w + k.tables_off);
     const int ntab = k.banks * k.entries;  // u16 entries
     float *red = reinterpret_cast<float *>(lds);
     if constexpr (TAB_LDS) {
-        for (int i = tid; i < ntab / 2; i += blockDim.x) lds[i] = reinterpret_cast<const uint32_t *>(gtab)[i];
+        table_to_lds(lds, reinterpret_cast<const uint32_t *>(gtab), ntab / 2, tid, blockDim.x);
         red = reinterpret_cast<float *>(lds + ntab / 2);
     }
     const uint16_t *tab = TAB_LDS ? reinterpret_cast<const uint16_t *>(lds) : gtab;
@@ -267,8 +288,8 @@ __global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *
     for (int i = 0; i < NB; ++i) acc[i] = accB[i] = float4_t{0.f, 0.f, 0.f, 0.f};
     if constexpr (TAB_LDS) __syncthreads();
 
-    const float delta = k.profile == 2 ? 0.15625f : 0.125f;
-    const uint32_t toff = 1024u, boff = 1024u + (k.tail ? 256u : 0u);
+    const float delta = PROF == 2 ? 0.15625f : 0.125f;
+    const uint32_t toff = 1024u, boff = 1024u + ((PROF == 3) ? 256u : 0u);
     // Software pipeline as in nint_mfma_body: the four unit dwords of a row-block are refilled unit by unit for the
     // next step, tails and bank bytes one step ahead, activation fragments two units ahead and before the refill.
     uint32_t q[NB][4], tails[NB], banks4[NB], tailsn[NB], banks4n[NB];
@@ -279,7 +300,7 @@ __global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const uint32_t off = i < nrb && s < n ? i * rbb + s * sb : kNoStep;
-            tt[i] = k.tail ? __builtin_amdgcn_raw_buffer_load_b32(win, off + toff + lane * 4, 0, 2) : 0u;
+            tt[i] = (PROF == 3) ? __builtin_amdgcn_raw_buffer_load_b32(win, off + toff + lane * 4, 0, 2) : 0u;
             bb[i] = __builtin_amdgcn_raw_buffer_load_b32(win, off + boff + r * 4, 0, 2);
         }
     };
@@ -317,7 +338,7 @@ __global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *
             xsum[j] = xs;
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
-                const NepqUnit u = nepq_decode(k.profile, q[i][j], (tails[i] >> (8 * j)) & 0xffu);
+                const NepqUnit u = nepq_decode(PROF, q[i][j], (tails[i] >> (8 * j)) & 0xffu);
                 q[i][j] = __builtin_amdgcn_raw_buffer_load_b32(win, unit_off(i, s + 1, j), 0, 2);
                 const uint16_t *bank = tab + ((banks4[i] >> (8 * j)) & 0xffu) * k.entries;
                 const float st = static_cast<float>(u.state);
@@ -334,6 +355,10 @@ __global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *
                     acc[i] = mfma16(a[m], b, acc[i]);
                 }
             }
+            // Keeps the requests of this unit (activation fragments two units ahead, the refill of its registers) where
+            // they are written: the scheduler otherwise sinks every refill to the end of the step, and the next step
+            // begins with a wait for all of them.
+            __builtin_amdgcn_sched_barrier(0);
         }
         u32x4_t ax;
         {
@@ -374,6 +399,146 @@ __global__ __launch_bounds__(512) void nepq_mfma_kernel(NepqK k, const uint8_t *
     }
 }
 
+// ---- 16-row tiles, one block per compute unit --------------------------------------------------------------
+// The kernel above re-reads the 16 activation rows (and the lookup tables) once per block: 128 KB at K = 4096, which on a
+// 1.5-bit format is eight times the block's own weights when a wave owns one row-block.  Here a block owns RPB consecutive
+// row-blocks and its waves split the K steps: a wave requests the units of its first step for all its row-blocks and the
+// step's activation fragments (48 registers, converted once and shared by the row-blocks) before the table copy, then
+// walks the row-blocks unit by unit, refilling each unit's register for the next step as soon as it is decoded.  The
+// bias term goes into the same accumulator as the digits.
+// LDS: [table: banks * entries u16, when TAB_LDS][red: waves * RPB * 1 KB]
+template <int XF16, int RPB, int TAB_LDS, int PROF>
+__global__ __launch_bounds__(1024) void nepq_tile_kernel(NepqK k, const uint8_t *__restrict__ w, int rb_first, int row0,
+                                                         int nrows, const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                         float *__restrict__ y, int64_t ldy, int spw) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    constexpr bool TAIL = PROF == 3;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint16_t *gtab = reinterpret_cast<const uint16_t *>(w + k.tables_off);
+    const int ntab = k.banks * k.entries;  // u16 entries
+    float *red = reinterpret_cast<float *>(lds + (TAB_LDS ? ntab / 2 : 0));
+    const uint16_t *tab = TAB_LDS ? reinterpret_cast<const uint16_t *>(lds) : gtab;
+    const int rb0 = rb_first + static_cast<int>(blockIdx.x) * RPB, rb_end = rb_first + (nrows + 15) / 16;
+    const int m0 = static_cast<int>(blockIdx.y) * 16;
+    const int tok = min(m0 + (lane & 15), M - 1);
+    const uint16_t *xrow = x + static_cast<int64_t>(tok) * ldx;
+    const int r = lane & 15, kb = lane >> 4;
+    const int s0 = wave * spw;
+    const int n = min(k.nsteps, s0 + spw) - s0;  // may be <= 0: the wave only takes part in the barriers
+    const int nrb = min(RPB, rb_end - rb0);
+    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
+    const __amdgpu_buffer_rsrc_t win =
+        wave_window(w + static_cast<int64_t>(rb0) * k.rowblock_bytes + static_cast<int64_t>(s0) * sb,
+                    n > 0 ? (nrb - 1) * rbb + n * sb : 0u);
+    constexpr uint32_t toff = 1024u, boff = 1024u + (TAIL ? 256u : 0u);
+    uint32_t q[RPB][4], tails[RPB], banks4[RPB];
+    auto step_off = [&](int i, int ls) -> uint32_t { return i < nrb && ls < n ? i * rbb + ls * sb : kNoStep; };
+    auto side_load = [&](int i, int ls, uint32_t &tt, uint32_t &bb) {
+        const uint32_t off = step_off(i, ls);
+        tt = TAIL ? __builtin_amdgcn_raw_buffer_load_b32(win, off + toff + lane * 4, 0, 2) : 0u;
+        bb = __builtin_amdgcn_raw_buffer_load_b32(win, off + boff + r * 4, 0, 2);
+    };
+    u32x4_t xf[4][3];
+    auto xload = [&](int ls) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int m = 0; m < 3; ++m)
+                xf[j][m] = load_xfrag_raw<true>(xrow, (s0 + ls) * 16 * 24 + kb * 24 + 4 * j * 24 + 8 * m, k.neuron_len);
+    };
+    // everything the first step needs, before the table copy: the weights come from HBM, the rest from L2
+#pragma unroll
+    for (int i = 0; i < RPB; ++i) {
+        side_load(i, 0, tails[i], banks4[i]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) q[i][j] = __builtin_amdgcn_raw_buffer_load_b32(win, step_off(i, 0) + (j * 64 + lane) * 4, 0, 2);
+    }
+    if (n > 0) xload(0);
+    if constexpr (TAB_LDS) {
+        table_to_lds(lds, reinterpret_cast<const uint32_t *>(gtab), ntab / 2, tid, blockDim.x);
+        __syncthreads();
+    }
+
+    const float delta = PROF == 2 ? 0.15625f : 0.125f;
+    float4_t acc[RPB];
+#pragma unroll
+    for (int i = 0; i < RPB; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int ls = 0; ls < n; ++ls) {
+        // the step's activations as fp16 fragments and the group sums the bias term multiplies
+        u32x4_t ax;
+        {
+            float xsum[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float xs = 0.f;
+#pragma unroll
+                for (int m = 0; m < 3; ++m) {
+                    xf[j][m] = xfrag_finish<XF16, true>(xf[j][m], (s0 + ls) * 16 * 24 + kb * 24 + 4 * j * 24 + 8 * m, k.neuron_len);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) xs = dot2h(xf[j][m][t], 0x3c003c00u, xs);
+                }
+                xsum[j] = xs;
+            }
+            half2_t hi[2], lo[2];
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                hi[p] = pk_h2(xsum[2 * p], xsum[2 * p + 1]);
+                lo[p] = pk_h2(xsum[2 * p] - static_cast<float>(hi[p].x), xsum[2 * p + 1] - static_cast<float>(hi[p].y));
+            }
+            ax = u32x4_t{__builtin_bit_cast(uint32_t, hi[0]), __builtin_bit_cast(uint32_t, hi[1]),
+                         __builtin_bit_cast(uint32_t, lo[0]), __builtin_bit_cast(uint32_t, lo[1])};
+        }
+#pragma unroll
+        for (int i = 0; i < RPB; ++i) {
+            uint32_t tailsn, banksn;
+            side_load(i, ls + 1, tailsn, banksn);
+            uint32_t stw[4];  // per unit: state * (bias - 1) as an fp16
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const NepqUnit u = nepq_decode(PROF, q[i][j], (tails[i] >> (8 * j)) & 0xffu);
+                q[i][j] = __builtin_amdgcn_raw_buffer_load_b32(win, step_off(i, ls + 1) + (j * 64 + lane) * 4, 0, 2);
+                const uint16_t *bank = tab + ((banks4[i] >> (8 * j)) & 0xffu) * k.entries;
+                const float st = static_cast<float>(u.state);
+                const half2_t S = pk_h2(st, st), C = pk_h2(-1024.f * st, -1024.f * st);
+                stw[j] = f32_to_f16_rne(st * ((u.aux ? -delta : delta) - 1.f));
+#pragma unroll
+                for (int m = 0; m < 3; ++m) {
+                    const uint32_t e = bank[u.idx[m]];
+                    const uint32_t t2 = e | (e << 14);
+                    u32x4_t b;
+#pragma unroll
+                    for (int p = 0; p < 4; ++p)
+                        b[p] = __builtin_bit_cast(uint32_t, h2_fma(((t2 >> (4 * p)) & 0x00030003u) | kMagicH2, S, C));
+                    acc[i] = mfma16(xf[j][m], b, acc[i]);
+                }
+                __builtin_amdgcn_sched_barrier(0);  // the refill stays with its unit (the scheduler would sink it)
+            }
+            const uint32_t b01 = stw[0] | (stw[1] << 16), b23 = stw[2] | (stw[3] << 16);
+            acc[i] = mfma16(ax, u32x4_t{b01, b23, b01, b23}, acc[i]);
+            tails[i] = tailsn;
+            banks4[i] = banksn;
+        }
+        if (ls + 1 < n) xload(ls + 1);
+    }
+#pragma unroll
+    for (int i = 0; i < RPB; ++i) {
+        const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[min(rb0 + i, k.n_rowblocks - 1) * 16 + r];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[((wave * RPB + i) * 4 + v) * 64 + lane] = anchor * acc[i][v];
+    }
+    __syncthreads();
+    const int nwaves = blockDim.x >> 6;
+    for (int o = threadIdx.x; o < RPB * 256; o += blockDim.x) {
+        const int rr = o & 15, t = (o >> 4) & 15, nb = o >> 8;
+        const int slot = (nb * 4 + (t & 3)) * 64 + rr + 16 * (t >> 2);
+        float sacc = 0.f;
+        for (int wv = 0; wv < nwaves; ++wv) sacc += red[wv * RPB * 256 + slot];
+        const int row = (rb0 + nb) * 16 + rr - row0;  // rows are relative to row0 in y
+        if (m0 + t < M && nb < nrb && row >= 0 && row < nrows) y[static_cast<int64_t>(m0 + t) * ldy + row] = sacc;
+    }
+}
+
 // ---- prefill: block-tiled MFMA GEMM, weight fragments built from the ternary tables ------------------------
 // Same frame as the NVQ prefill kernel: block = 8 waves x NB row-blocks, wave tile MT * 16 tokens, activations as
 // scaled fp16 rows (x_prep) through two LDS buffers with XD tiles in flight, PF unit dwords per row-block in flight.
@@ -401,7 +566,7 @@ __global__ __launch_bounds__(512) void nepq_prefill_kernel(NepqK k, const uint8_
     const int ntab = k.banks * k.entries;  // u16 entries, even
     uint16_t *xt = reinterpret_cast<uint16_t *>(lds);
     if constexpr (TAB_LDS) {
-        for (int i = tid; i < ntab / 2; i += NT) lds[i] = reinterpret_cast<const uint32_t *>(gtab)[i];
+        table_to_lds(lds, reinterpret_cast<const uint32_t *>(gtab), ntab / 2, tid, NT);
         xt = reinterpret_cast<uint16_t *>(lds + (ntab / 2 + 3) / 4 * 4);
     }
     const uint16_t *tab = TAB_LDS ? reinterpret_cast<const uint16_t *>(lds) : gtab;
@@ -602,6 +767,18 @@ static int nepq_prefill(const NepqK &k, const uint8_t *w, int row0, int nrows, c
 #undef MFQ_NEPQ_PREFILL
 }
 
+// LDS a block may take when that lets the lookup tables live there (a 16-bank pool
+// of the L profile is 64 KB; up to 80 KB two blocks still fit a compute unit)
+constexpr size_t kNepqTableLds = 96 * 1024;
+template <class Kern>
+static int nepq_allow_lds(Kern kern, size_t lds) {
+    if (lds <= 65536) return MFQ_OK;
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             static_cast<int>(lds));
+    MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nepq: %s", hipGetErrorString(e));
+    return MFQ_OK;
+}
+
 static bool nepq_stream_capable(const NepqK &k) {
     return k.neuron_len >= 8 && k.neuron_len % 8 == 0 && 4 * k.rowblock_bytes < (1ll << 31);
 }
@@ -615,21 +792,73 @@ static int nepq_launch_mfma(const NepqK &k, const uint8_t *w, int row0, int nrow
     while (spw < k.nsteps && groups * ceil_div(k.nsteps, spw) > 8192) ++spw;
     const int nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
     const size_t redb = static_cast<size_t>(nwaves) * NB * 1024, tabb = static_cast<size_t>(k.banks) * k.entries * 2;
-    const bool tab_lds = redb + tabb <= 65536;
+    const bool tab_lds = redb + tabb <= kNepqTableLds;
     const size_t lds = redb + (tab_lds ? tabb : 0);
     const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(ceil_div(M, 16))), block(64 * nwaves);
-    if (tab_lds)
-        hipLaunchKernelGGL((nepq_mfma_kernel<XF16, NB, 1>), grid, block, lds, st, k, w, row0 / 16, row0, nrows, x, ldx, M, y,
-                           ldy, spw);
-    else
-        hipLaunchKernelGGL((nepq_mfma_kernel<XF16, NB, 0>), grid, block, lds, st, k, w, row0 / 16, row0, nrows, x, ldx, M, y,
-                           ldy, spw);
+#define MFQ_NEPQ_MFMA(T, P)                                                                                                      \
+    do {                                                                                                                         \
+        if (int rc = nepq_allow_lds(nepq_mfma_kernel<XF16, NB, T, P>, lds)) return rc;                                           \
+        hipLaunchKernelGGL((nepq_mfma_kernel<XF16, NB, T, P>), grid, block, lds, st, k, w, row0 / 16, row0, nrows, x, ldx, M, y, \
+                           ldy, spw);                                                                                            \
+    } while (0)
+    if (k.profile == 2) {
+        if (tab_lds) MFQ_NEPQ_MFMA(1, 2); else MFQ_NEPQ_MFMA(0, 2);
+    } else {
+        if (tab_lds) MFQ_NEPQ_MFMA(1, 3); else MFQ_NEPQ_MFMA(0, 3);
+    }
+#undef MFQ_NEPQ_MFMA
     return check_launch("nepq_mfma");
+}
+
+// One block per compute unit and 16-row tile: up to three row-blocks per block, up to 16 waves over the K steps.
+static bool nepq_tile_shape(const NepqK &k, int nrows, int &rpb, int &spw, int &nwaves, size_t &lds, bool &tab_lds) {
+    static const int off = tune_env("MFQ_NEPQ_TILE_OFF", 0);
+    const int nrb = static_cast<int>(ceil_div(nrows, 16));
+    rpb = static_cast<int>(ceil_div(nrb, gemv_cu_count()));
+    if (off || rpb > 3 || 3 * k.rowblock_bytes >= (1ll << 31)) return false;
+    spw = static_cast<int>(ceil_div(k.nsteps, 16));
+    nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
+    const size_t redb = static_cast<size_t>(nwaves) * rpb * 1024, tabb = static_cast<size_t>(k.banks) * k.entries * 2;
+    tab_lds = redb + tabb <= 128 * 1024;
+    lds = redb + (tab_lds ? tabb : 0);
+    // one row-block per block and two steps per wave (4096 x 12288): the streaming kernel's eight waves of four steps,
+    // with their fragments two units ahead, are faster (14.7 against 16 us) than a wait for the second step's fragments
+    if (rpb == 1 && spw > 1) return false;
+    return lds <= 128 * 1024;
+}
+template <int XF16, int RPB>
+static int nepq_launch_tile(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
+                            float *y, int64_t ldy, hipStream_t st, int spw, int nwaves, size_t lds, bool tab_lds) {
+    const dim3 grid(static_cast<unsigned>(ceil_div(ceil_div(nrows, 16), RPB)), static_cast<unsigned>(ceil_div(M, 16)));
+    const dim3 block(64 * nwaves);
+#define MFQ_NEPQ_TILE(T, P)                                                                                                       \
+    do {                                                                                                                          \
+        if (int rc = nepq_allow_lds(nepq_tile_kernel<XF16, RPB, T, P>, lds)) return rc;                                           \
+        hipLaunchKernelGGL((nepq_tile_kernel<XF16, RPB, T, P>), grid, block, lds, st, k, w, row0 / 16, row0, nrows, x, ldx, M, y, \
+                           ldy, spw);                                                                                             \
+    } while (0)
+    if (k.profile == 2) {
+        if (tab_lds) MFQ_NEPQ_TILE(1, 2); else MFQ_NEPQ_TILE(0, 2);
+    } else {
+        if (tab_lds) MFQ_NEPQ_TILE(1, 3); else MFQ_NEPQ_TILE(0, 3);
+    }
+#undef MFQ_NEPQ_TILE
+    return check_launch("nepq_tile");
 }
 
 template <int XF16>
 static int nepq_mfma_any(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
                          float *y, int64_t ldy, hipStream_t st) {
+    {
+        int rpb, spw, nwaves;
+        size_t lds;
+        bool tab_lds;
+        if (M <= 32 && nepq_tile_shape(k, nrows, rpb, spw, nwaves, lds, tab_lds)) {
+            if (rpb == 3) return nepq_launch_tile<XF16, 3>(k, w, row0, nrows, x, ldx, M, y, ldy, st, spw, nwaves, lds, tab_lds);
+            if (rpb == 2) return nepq_launch_tile<XF16, 2>(k, w, row0, nrows, x, ldx, M, y, ldy, st, spw, nwaves, lds, tab_lds);
+            return nepq_launch_tile<XF16, 1>(k, w, row0, nrows, x, ldx, M, y, ldy, st, spw, nwaves, lds, tab_lds);
+        }
+    }
     const int64_t wpb = (k.nsteps < 8 ? k.nsteps : 8) * ceil_div(M, 16);  // waves of a block x 16-row tiles
     static const int env_nb = tune_env("MFQ_NEPQ_NB", 0);
     if (env_nb == 4) return nepq_launch_mfma<XF16, 4>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
@@ -639,34 +868,64 @@ static int nepq_mfma_any(const NepqK &k, const uint8_t *w, int row0, int nrows, 
     return nepq_launch_mfma<XF16, 1>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
 }
 
-static void nepq_gemv_shape(const NepqK &k, int nrb, int mb, int &spw, int &nwaves, size_t &lds_bytes, bool &tab_lds) {
-    int want = static_cast<int>(ceil_div(3 * gemv_target_waves(), nrb));
+static void nepq_gemv_shape(const NepqK &k, int nrb, int mb, int rpb, int &spw, int &nwaves, size_t &lds_bytes, bool &tab_lds) {
+    int want = static_cast<int>(ceil_div(3 * gemv_target_waves(), ceil_div(nrb, rpb)));
     if (want < 1) want = 1;
     if (want > 16) want = 16;
     if (want > k.nsteps) want = k.nsteps;
     spw = static_cast<int>(ceil_div(k.nsteps, want));
     nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
-    const size_t xb = gemv_lds_bytes(mb, spw, 24, nwaves);
+    const size_t xb = gemv_lds_bytes(mb, spw, 24, nwaves, rpb);
     const size_t tabb = static_cast<size_t>(k.banks) * k.entries * 2;
-    tab_lds = tabb + xb <= 65536;
+    tab_lds = tabb + xb <= kNepqTableLds;
     lds_bytes = xb + (tab_lds ? tabb : 0);
 }
 
-template <int XF16, int MB>
-static int nepq_launch(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
-                       float *y, int64_t ldy, hipStream_t st) {
+template <int XF16, int MB, int RPB>
+static int nepq_launch_as(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
+                          float *y, int64_t ldy, hipStream_t st) {
     const int rb0 = row0 / 16, nrb = static_cast<int>(ceil_div(nrows, 16));
     int spw, nwaves;
     size_t lds;
     bool tab_lds;
-    nepq_gemv_shape(k, nrb, MB, spw, nwaves, lds, tab_lds);
-    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nepq_gemv: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
-    const dim3 grid(nrb, static_cast<unsigned>(ceil_div(M, MB))), block(64 * nwaves);
-    if (tab_lds)
-        hipLaunchKernelGGL((nepq_gemv_kernel<XF16, MB, 1>), grid, block, lds, st, k, w, rb0, row0, nrows, x, ldx, M, y, ldy, spw);
-    else
-        hipLaunchKernelGGL((nepq_gemv_kernel<XF16, MB, 0>), grid, block, lds, st, k, w, rb0, row0, nrows, x, ldx, M, y, ldy, spw);
+    nepq_gemv_shape(k, nrb, MB, RPB, spw, nwaves, lds, tab_lds);
+    MFQ_REQUIRE(lds <= kNepqTableLds, MFQ_ERR_UNSUPPORTED, "nepq_gemv: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
+    const dim3 grid(static_cast<unsigned>(ceil_div(nrb, RPB)), static_cast<unsigned>(ceil_div(M, MB))), block(64 * nwaves);
+#define MFQ_NEPQ_GEMV(T, P)                                                                                                     \
+    do {                                                                                                                        \
+        if (int rc = nepq_allow_lds(nepq_gemv_kernel<XF16, MB, T, RPB, P>, lds)) return rc;                                     \
+        hipLaunchKernelGGL((nepq_gemv_kernel<XF16, MB, T, RPB, P>), grid, block, lds, st, k, w, rb0, row0, nrows, x, ldx, M, y, \
+                           ldy, spw);                                                                                           \
+    } while (0)
+    if (k.profile == 2) {
+        if (tab_lds) MFQ_NEPQ_GEMV(1, 2); else MFQ_NEPQ_GEMV(0, 2);
+    } else {
+        if (tab_lds) MFQ_NEPQ_GEMV(1, 3); else MFQ_NEPQ_GEMV(0, 3);
+    }
+#undef MFQ_NEPQ_GEMV
     return check_launch("nepq_gemv");
+}
+template <int XF16, int MB>
+static int nepq_launch(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
+                       float *y, int64_t ldy, hipStream_t st) {
+    if constexpr (MB == 1) {
+        // One row: as many row-blocks per block as it takes to have one block per CU (up to four), so that the table is
+        // staged once per CU and every wave has several row-blocks' units in flight.  MFQ_NEPQ_RPB overrides for tuning.
+        static const int env = tune_env("MFQ_NEPQ_RPB", 0);
+        const int nrb = static_cast<int>(ceil_div(nrows, 16));
+        int rpb = env > 0 ? env : static_cast<int>(ceil_div(nrb, gemv_cu_count()));
+        int spw, nwaves;
+        size_t lds;
+        bool tl;
+        for (rpb = rpb > 4 ? 4 : rpb; rpb > 1; --rpb) {  // the reduction area grows with the row-blocks
+            nepq_gemv_shape(k, nrb, 1, rpb, spw, nwaves, lds, tl);
+            if (lds <= kNepqTableLds) break;
+        }
+        if (rpb >= 4) return nepq_launch_as<XF16, 1, 4>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
+        if (rpb == 3) return nepq_launch_as<XF16, 1, 3>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
+        if (rpb == 2) return nepq_launch_as<XF16, 1, 2>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
+    }
+    return nepq_launch_as<XF16, MB, 1>(k, w, row0, nrows, x, ldx, M, y, ldy, st);
 }
 
 static int nepq_gemv_any(const mfq_nepq_desc *d, const void *weight, int row0, int nrows, const void *x, int x_dtype,
@@ -676,7 +935,8 @@ static int nepq_gemv_any(const mfq_nepq_desc *d, const void *weight, int row0, i
     const uint16_t *xp = static_cast<const uint16_t *>(x);
     const int nrb = static_cast<int>(ceil_div(nrows, 16));
     // a single row is still cheaper on the vector-ALU kernel
-    if (M >= 2 && nepq_stream_capable(k) && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
+    static const int valu_max_m = tune_env("MFQ_NEPQ_VALU_MAX_M", 1);
+    if (M > valu_max_m && nepq_stream_capable(k) && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
         return x_dtype == MFQ_X_F16 ? nepq_mfma_any<1>(k, w, row0, nrows, xp, ldx, M, y, ldy, st)
                                     : nepq_mfma_any<0>(k, w, row0, nrows, xp, ldx, M, y, ldy, st);
     int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
@@ -684,8 +944,8 @@ static int nepq_gemv_any(const mfq_nepq_desc *d, const void *weight, int row0, i
         int spw, nwaves;
         size_t lds;
         bool tl;
-        nepq_gemv_shape(k, nrb, mb, spw, nwaves, lds, tl);
-        if (lds <= 65536 || mb == 1) break;
+        nepq_gemv_shape(k, nrb, mb, 1, spw, nwaves, lds, tl);
+        if (lds <= kNepqTableLds || mb == 1) break;
         mb >>= 1;
     }
     if (x_dtype == MFQ_X_F16) {

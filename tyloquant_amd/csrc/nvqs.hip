@@ -276,8 +276,7 @@ __global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *
     const int8_t *cbp = reinterpret_cast<const int8_t *>(bfs + 16);
     if constexpr (CB_LDS) {
         const int ncb = k.cb_bytes;
-        for (int i = threadIdx.x * 4; i < ncb; i += blockDim.x * 4)
-            *reinterpret_cast<uint32_t *>(cbl + i) = *reinterpret_cast<const uint32_t *>(cbp + i);
+        table_to_lds(reinterpret_cast<uint32_t *>(cbl), reinterpret_cast<const uint32_t *>(cbp), ncb / 4, threadIdx.x, blockDim.x);
         __syncthreads();
     }
     const int row = blockIdx.x * (blockDim.x >> 6) + wave;
