@@ -187,6 +187,10 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
 
     const int r = lane & 15, kb = lane >> 4;
     const float delta = PROF == 2 ? 0.15625f : 0.125f;
+    // requested here, ahead of the weights: at the end of the kernel each would cost a round trip to memory
+    float anchor[RPB];
+#pragma unroll
+    for (int i = 0; i < RPB; ++i) anchor[i] = reinterpret_cast<const float *>(w + k.anchors_off)[min(rb + i, rb_last) * 16 + r];
     float acc[RPB][MB];
 #pragma unroll
     for (int i = 0; i < RPB; ++i)
@@ -237,10 +241,9 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
     }
 #pragma unroll
     for (int i = 0; i < RPB; ++i) {
-        const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[min(rb + i, rb_last) * 16 + r];
         float v[MB];
 #pragma unroll
-        for (int m = 0; m < MB; ++m) v[m] = anchor * acc[i][m];
+        for (int m = 0; m < MB; ++m) v[m] = anchor[i] * acc[i][m];
         park_rows<MB>(v, red, i * nwaves + wave, lane);
     }
     // a row-block past the tensor's last has rows beyond nrows: flush_rows drops them
@@ -447,7 +450,12 @@ __global__ __launch_bounds__(1024) void nepq_tile_kernel(NepqK k, const uint8_t 
             for (int m = 0; m < 3; ++m)
                 xf[j][m] = load_xfrag_raw<true>(xrow, (s0 + ls) * 16 * 24 + kb * 24 + 4 * j * 24 + 8 * m, k.neuron_len);
     };
-    // everything the first step needs, before the table copy: the weights come from HBM, the rest from L2
+    // everything the first step needs, before the table copy: the weights come from HBM, the rest from L2; the anchors
+    // too (at the end of the kernel they would cost a round trip to memory of their own)
+    float anchor[RPB];
+#pragma unroll
+    for (int i = 0; i < RPB; ++i)
+        anchor[i] = reinterpret_cast<const float *>(w + k.anchors_off)[min(rb0 + i, k.n_rowblocks - 1) * 16 + r];
 #pragma unroll
     for (int i = 0; i < RPB; ++i) {
         side_load(i, 0, tails[i], banks4[i]);
@@ -523,9 +531,8 @@ __global__ __launch_bounds__(1024) void nepq_tile_kernel(NepqK k, const uint8_t 
     }
 #pragma unroll
     for (int i = 0; i < RPB; ++i) {
-        const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[min(rb0 + i, k.n_rowblocks - 1) * 16 + r];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) red[((wave * RPB + i) * 4 + v) * 64 + lane] = anchor * acc[i][v];
+        for (int v = 0; v < 4; ++v) red[((wave * RPB + i) * 4 + v) * 64 + lane] = anchor[i] * acc[i][v];
     }
     __syncthreads();
     const int nwaves = blockDim.x >> 6;
