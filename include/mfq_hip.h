@@ -366,6 +366,26 @@ int mfq_hip_nvqs_gemm(const mfq_nvqs_desc *d, const void *weight, const void *x,
                       mfq_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
+ * OCP MX weights of full-precision MFQ files (mfq/formats/mx.py:16-117): kind 4 = MXFP4 (E2M1 nibbles, low nibble =
+ * even column, one E8M0 scale per 32 columns of a row), kind 8 = MXFP8 (E4M3FN bytes, one E8M0 scale per 128 x 128
+ * block).  values / scales: device copies of the payload's two byte matrices as they lie behind its 56-byte header
+ * (values [rows, cols / 2] or [rows, cols]; scales [rows, cols / 32] or [ceil(rows / 128), cols / 128]); values
+ * 16-byte aligned.  Calls work on the rows [row0, row0 + nrows) -- a whole tensor, or one expert of a pool.
+ * mfq_hip_mx_dequant_rows: w_out[r - row0][c] = element * scale, one fp32 multiply (MFQ_X_F32; unpack_mxfp8 /
+ * dequant_mxfp4_cpu, cpp_runtime/mfq_decode.cpp:1832-1947, mxfp8_dequant_kernel, mfq/kernels/cuda/mx_matmul.cu:222-240),
+ * or that rounded once more to fp16 as the reference's device copy is (MFQ_X_F16); a scale byte 255 and the E4M3FN codes
+ * 0x7f / 0xff give NaN.
+ * mfq_hip_mx_gemm_rows: y[M, nrows] = x[M, cols] . W^T in fp32 (mxfp8_matmul_f32, mfq_decode.cpp:8784-8802): a wave
+ * per neuron up to 16 rows of x (mxfp8_small_m_f32_cuda serves 1..8), above that an fp16 copy of the rows, each
+ * relative to its largest scale, and the fp16 MFMA GEMM -- workspace of mfq_hip_mx_gemm_rows_workspace_bytes. */
+int mfq_hip_mx_dequant_rows(int kind, const void *values, const void *scales, int rows, int cols, int row0, int nrows,
+                            int out_dtype, void *w_out, int64_t ld, mfq_stream_t stream);
+size_t mfq_hip_mx_gemm_rows_workspace_bytes(int cols, int nrows, int M);
+int mfq_hip_mx_gemm_rows(int kind, const void *values, const void *scales, int rows, int cols, int row0, int nrows,
+                         const void *x, int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, void *workspace,
+                         size_t workspace_bytes, mfq_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
  * NEPQ1-S / NEPQ1-L (cross-expert table pool, bank id per 96 weights).  Rows are the
  * flattened [experts * out_per_expert] neurons.  Replaces NepqWeight
  * (cpp_runtime/mfq_decode.cpp:4166-4463) and the Python nepq_matmul

@@ -43,6 +43,12 @@ reference tree).  Parity status of each function:
     dequantize_npq0                mfq/quantize/npq0_l.py:766-790, npq0_s.py:812-836
     pack_nepq / unpack_nepq / dequantize_nepq on NEPQ0-S / NEPQ0-L   mfq/formats/nepq.py:95-116, 368-474, 492-521
 
+  pinned by a reference-written blob (tests/golden/reference_mx.npz, made by tests/golden/make_reference_mx.py), by
+  torch's own float8_e4m3fn conversion over all 256 codes, and by closed forms (tests/test_oracle_mx.py)
+    pack_mx / unpack_mx            mfq/formats/mx.py:65-182
+    dequantize_mx                  cpp_runtime/mfq_decode.cpp:1920-1947 (MXFP4), 8810-8840 and
+                                   mfq/kernels/cuda/mx_matmul.cu:17-47, 222-240 (MXFP8: E4M3FN x E8M0 per 128 x 128 block)
+
   pinned by golden vectors written from the reference's own numpy quantizer
   (tests/golden/nint_quant_vectors.npz, made by tests/golden/make_nint_quant_vectors.py)
     make_qkx2 / quantize_nint      mfq/formats/nint.py:119-174, mfq/quantize/nint_quant.py:745-893
@@ -1012,6 +1018,110 @@ def dequantize_npq0(t: Npq0Tensor) -> np.ndarray:
     return (code.reshape(out, K).astype(np.float32) * scale).astype(np.float32)
 
 
+# ---------------------------------------------------------------------------
+# OCP MX payloads: MXFP4 (E2M1 nibbles, one E8M0 scale per 32 columns of a row) and MXFP8 (E4M3FN bytes, one E8M0
+# scale per 128 x 128 block).  Container mfq/formats/mx.py:20-182.
+# ---------------------------------------------------------------------------
+MX_HEADER = struct.Struct("<4sBBHQQQQQQ")  # magic, version, kind, reserved, shape, storage shape, scale shape
+MX_KINDS = {"MXFP4": 4, "MXFP8": 8}
+FP4_E2M1 = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], dtype=np.float32)  # cpp_runtime/mfq_decode.cpp:1926-1928
+
+
+@dataclass
+class MxTensor:
+    dtype: str           # "MXFP4" | "MXFP8"
+    shape: tuple         # (rows, columns)
+    values: np.ndarray   # uint8: [rows, columns / 2] (low nibble = even column) or [rows, columns]
+    scales: np.ndarray   # uint8 E8M0: [rows, columns / 32] or [ceil(rows / 128), columns / 128]
+
+
+def mx_shapes(dtype: str, shape):
+    """(storage shape, scale shape) of a logical [rows, columns] matrix (validate_mx_shapes, mx.py:65-117)."""
+    if dtype not in MX_KINDS:
+        raise ValueError(f"unsupported MX dtype: {dtype}")
+    if len(shape) != 2:
+        raise ValueError("MFQ MX tensors must be rank-2 matrices")
+    rows, cols = int(shape[0]), int(shape[1])
+    if rows <= 0 or cols <= 0:
+        raise ValueError(f"invalid MX logical shape: {tuple(shape)}")
+    if dtype == "MXFP4":
+        if cols % 32:
+            raise ValueError("MXFP4 columns must be divisible by 32")
+        return (rows, cols // 2), (rows, cols // 32)
+    if cols % 128:
+        raise ValueError("MXFP8 columns must be divisible by 128")
+    return (rows, cols), ((rows + 127) // 128, cols // 128)
+
+
+def pack_mx(t: MxTensor) -> bytes:
+    """mx.py:120-151: header, value bytes, scale bytes."""
+    storage, scale = mx_shapes(t.dtype, t.shape)
+    values = np.ascontiguousarray(t.values, dtype=np.uint8)
+    scales = np.ascontiguousarray(t.scales, dtype=np.uint8)
+    if values.shape != storage:
+        raise ValueError(f"{t.dtype} storage shape {values.shape} != {storage}")
+    if scales.shape != scale:
+        raise ValueError(f"{t.dtype} scale shape {scales.shape} != {scale}")
+    head = MX_HEADER.pack(b"MXT1", 1, MX_KINDS[t.dtype], 0, *map(int, t.shape), *storage, *scale)
+    return head + values.tobytes() + scales.tobytes()
+
+
+def unpack_mx(dtype: str, blob) -> MxTensor:
+    """mx.py:154-182."""
+    blob = bytes(blob)
+    if len(blob) < MX_HEADER.size:
+        raise ValueError("truncated MFQ MX tensor header")
+    magic, version, kind, reserved, *dims = MX_HEADER.unpack_from(blob)
+    if magic != b"MXT1" or version != 1 or kind != MX_KINDS.get(dtype) or reserved:
+        raise ValueError(f"invalid {dtype} payload header: magic={magic!r}, version={version}, kind={kind}")
+    shape = (int(dims[0]), int(dims[1]))
+    storage, scale = mx_shapes(dtype, shape)
+    if (int(dims[2]), int(dims[3])) != storage:
+        raise ValueError(f"{dtype} storage shape {(int(dims[2]), int(dims[3]))} != {storage}")
+    if (int(dims[4]), int(dims[5])) != scale:
+        raise ValueError(f"{dtype} scale shape {(int(dims[4]), int(dims[5]))} != {scale}")
+    nv, ns = storage[0] * storage[1], scale[0] * scale[1]
+    if len(blob) != MX_HEADER.size + nv + ns:
+        raise ValueError(f"{dtype} payload size {len(blob)} != {MX_HEADER.size + nv + ns}")
+    values = np.frombuffer(blob, np.uint8, nv, MX_HEADER.size).reshape(storage).copy()
+    scales = np.frombuffer(blob, np.uint8, ns, MX_HEADER.size + nv).reshape(scale).copy()
+    return MxTensor(dtype, shape, values, scales)
+
+
+def decode_e8m0(raw) -> np.ndarray:
+    """2^(raw - 127) as fp32, NaN for 255 (mx_matmul.cu:17-28; raw 0 is the subnormal 2^-127)."""
+    raw = np.asarray(raw, dtype=np.uint8)
+    out = np.ldexp(np.float32(1.0), np.minimum(raw, 254).astype(np.int32) - 127).astype(np.float32)
+    return np.where(raw == 255, np.float32(np.nan), out)
+
+
+def decode_e4m3fn(raw) -> np.ndarray:
+    """mx_matmul.cu:30-47: no infinities, exponent 15 with mantissa 7 is NaN, subnormals are multiples of 2^-9."""
+    raw = np.asarray(raw, dtype=np.uint8)
+    e = ((raw >> 3) & 15).astype(np.int32)
+    m = (raw & 7).astype(np.float32)
+    mag = np.where(e == 0, m * np.float32(2.0 ** -9), np.ldexp(np.float32(1.0) + m / np.float32(8.0), e - 7)).astype(np.float32)
+    mag = np.where((e == 15) & ((raw & 7) == 7), np.float32(np.nan), mag)
+    return np.where(raw & 128, -mag, mag).astype(np.float32)
+
+
+def dequantize_mx(t: MxTensor) -> np.ndarray:
+    """fp32 [rows, columns] = element x block scale (one fp32 multiply: exact unless the product leaves fp32's range)."""
+    rows, cols = t.shape
+    if t.dtype == "MXFP4":
+        v = np.asarray(t.values, dtype=np.uint8)
+        codes = np.stack([v & 15, v >> 4], axis=-1).reshape(rows, cols)
+        mag = FP4_E2M1[codes & 7]
+        elem = np.where(codes & 8, -mag, mag).astype(np.float32)
+        scale = np.repeat(decode_e8m0(t.scales), 32, axis=1)
+    else:
+        elem = decode_e4m3fn(t.values)
+        scale = np.repeat(np.repeat(decode_e8m0(t.scales), 128, axis=0)[:rows], 128, axis=1)
+    with np.errstate(invalid="ignore", over="ignore", under="ignore"):
+        return (elem * scale).astype(np.float32)
+
+
+
 def tensor_dtype(t) -> str:
     """Public dtype label (mfq/formats/io.py:576-640)."""
     if isinstance(t, NintTensor):
@@ -1029,6 +1139,8 @@ def tensor_dtype(t) -> str:
         return "NINTM"
     if isinstance(t, (Nvq1Tensor, Npq0Tensor)):
         return t.label
+    if isinstance(t, MxTensor):
+        return t.dtype
     raise TypeError(type(t))
 
 
@@ -1048,6 +1160,8 @@ def pack_tensor(t) -> tuple[str, bytes]:
         return dt, pack_nvq1(t)
     if isinstance(t, Npq0Tensor):
         return dt, pack_npq0(t)
+    if isinstance(t, MxTensor):
+        return dt, pack_mx(t)
     return dt, pack_nint_moe(t)
 
 
@@ -1063,6 +1177,8 @@ def unpack_tensor(dtype: str, blob):
         return t
     if dtype == "NINT8-0":
         return unpack_nint8_zero(blob)
+    if dtype in MX_KINDS:
+        return unpack_mx(dtype, blob)
     if dtype in ("NVQ1-L", "NVQ1-S"):
         return unpack_nvq1(blob, dtype)
     if dtype in ("NPQ0-L", "NPQ0-S"):
@@ -1150,6 +1266,8 @@ def dequantize_tensor(t) -> np.ndarray:
         return dequantize_nvq1(t)
     if isinstance(t, Npq0Tensor):
         return dequantize_npq0(t)
+    if isinstance(t, MxTensor):
+        return dequantize_mx(t)
     raise TypeError(type(t))
 
 

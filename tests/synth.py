@@ -179,3 +179,14 @@ def nintm_packed_blob(rng, E, out, K, bits_per_expert, sigma=0.02):
         parts += [O._NIM_POOL.pack(ids.size, len(db), len(pb), 0), ids.tobytes(), db, pb]
         pools.append((ids, pb))
     return b"".join(parts), pools
+
+
+def mx_random(rng, dtype, rows, cols, lo=118, hi=132):
+    """An MXFP4 / MXFP8 tensor of random codes without NaNs (E4M3FN 0x7f / 0xff, scale byte 255), the block scales within
+    a few octaves of one."""
+    storage, scale = O.mx_shapes(dtype, (rows, cols))
+    values = rng.integers(0, 256, storage, dtype=np.uint8)
+    if dtype == "MXFP8":
+        values[(values & 0x7F) == 0x7F] = 0x38
+    return O.MxTensor(dtype, (rows, cols), values, rng.integers(lo, hi, scale, dtype=np.uint8))
+

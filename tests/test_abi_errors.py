@@ -109,3 +109,22 @@ def test_moe_helpers_check_their_arguments(lib):
     rc = lib.mfq_hip_moe_grouped_glu_ws(pools, 1, FAKE, FAKE, 8, 48, 256, FAKE, L.X_BF16, 256, 0, FAKE, 16, 2, FAKE, FAKE,
                                         L.GLU_SILU, FAKE, L.X_F16, 24, FAKE, 1 << 20, None)
     assert rc == L.ERR_UNSUPPORTED and "row-blocks" in _msg(lib)             # 48 is not two halves of whole row-blocks
+
+
+def test_mx_entry_points_check_geometry_rows_and_workspace(lib):
+    rc = lib.mfq_hip_mx_dequant_rows(5, FAKE, FAKE, 4, 96, 0, 4, L.X_F32, FAKE, 96, None)
+    assert rc == L.ERR_INVALID and "neither MXFP4 (4) nor MXFP8 (8)" in _msg(lib)
+    rc = lib.mfq_hip_mx_dequant_rows(4, FAKE, FAKE, 4, 48, 0, 4, L.X_F32, FAKE, 48, None)
+    assert rc == L.ERR_INVALID and "MXFP4 columns must be divisible by 32" in _msg(lib)
+    rc = lib.mfq_hip_mx_dequant_rows(8, FAKE, FAKE, 4, 96, 0, 4, L.X_F32, FAKE, 96, None)
+    assert rc == L.ERR_INVALID and "MXFP8 columns must be divisible by 128" in _msg(lib)
+    assert lib.mfq_hip_mx_dequant_rows(4, FAKE, FAKE, 4, 96, 0, 4, L.X_BF16, FAKE, 96, None) == L.ERR_INVALID   # fp32 / fp16 only
+    assert lib.mfq_hip_mx_dequant_rows(4, FAKE, None, 4, 96, 0, 4, L.X_F32, FAKE, 96, None) == L.ERR_INVALID
+    for row0, nrows in ((-1, 2), (3, 2), (0, 0), (4, 1)):
+        rc = lib.mfq_hip_mx_gemm_rows(4, FAKE, FAKE, 4, 96, row0, nrows, FAKE, L.X_BF16, 96, 1, FAKE, 4, None, 0, None)
+        assert rc == L.ERR_INVALID and "outside the tensor" in _msg(lib)
+    assert lib.mfq_hip_mx_gemm_rows(4, FAKE, FAKE, 4, 96, 0, 4, FAKE, L.X_F32, 96, 1, FAKE, 4, None, 0, None) == L.ERR_INVALID
+    assert lib.mfq_hip_mx_gemm_rows(4, FAKE, FAKE, 4, 96, 0, 4, FAKE, L.X_BF16, 64, 1, FAKE, 4, None, 0, None) == L.ERR_INVALID
+    assert lib.mfq_hip_mx_gemm_rows_workspace_bytes(96, 4, 16) == 0 and lib.mfq_hip_mx_gemm_rows_workspace_bytes(96, 4, 17) > 0
+    assert lib.mfq_hip_mx_gemm_rows(4, FAKE, FAKE, 4, 96, 0, 4, FAKE, L.X_BF16, 96, 17, FAKE, 4, None, 0, None) == L.ERR_WORKSPACE
+

@@ -69,6 +69,8 @@ def test_check_linear_tool_reports_small_error(tmp_path):
         "blk.1.o.npq0s": synth.npq0_random(rng, "NPQ0-S", 33, 200),
         "blk.2.q.nepq0s": synth.nepq_random(rng, "NEPQ0-S", 1, 48, 96, 3),            # NPQ0 tables in the NEPQ container
         "blk.2.k.nepq0l": synth.nepq_random(rng, "NEPQ0-L", 1, 40, 200, 5),
+        "blk.3.q.mxfp8": synth.mx_random(rng, "MXFP8", 130, 256),                     # OCP MX payloads
+        "blk.3.k.mxfp4": synth.mx_random(rng, "MXFP4", 37, 96),
     }
     path = tmp_path / "tiny.mfq"
     O.mfq_file_write(path, tensors, version=2)
@@ -108,7 +110,28 @@ def test_cpp_load_quant_linear_and_forward(rt):
     with pytest.raises(RuntimeError, match="dtype/blob mismatch"):
         _load(rt, "NINT4", O.pack_nint(t))
     with pytest.raises(RuntimeError, match="unsupported quantized linear dtype"):
+        _load(rt, "TPQ4", b"\0" * 64)
+    with pytest.raises(RuntimeError, match="invalid MXFP4 payload header"):
         _load(rt, "MXFP4", b"\0" * 64)
+    # MXFP8 / MXFP4 through the same registry: bit-exact dequantizer, GEMV and GEMM routes
+    for dtype, rows, cols in (("MXFP8", 130, 256), ("MXFP4", 70, 160)):
+        tm = synth.mx_random(rng, dtype, rows, cols)
+        hm = _load(rt, dtype, O.pack_mx(tm))
+        assert rt.mfq_rt_linear_out(hm) == rows and rt.mfq_rt_linear_neuron_len(hm) == cols
+        Wm = torch.empty((rows, cols), dtype=torch.float32, device="cuda")
+        assert rt.mfq_rt_linear_dequantize(hm, Wm.data_ptr(), None) == 0
+        torch.cuda.synchronize()
+        deqm = O.dequantize_mx(tm)
+        assert np.array_equal(Wm.cpu().numpy().view(np.uint32), deqm.view(np.uint32))
+        for M in (1, 9, 40):
+            x = torch.from_numpy(rng.standard_normal((M, cols)).astype(np.float32)).to(torch.bfloat16).cuda()
+            y = torch.empty((M, rows), dtype=torch.float32, device="cuda")
+            assert rt.mfq_rt_linear_forward(hm, x.data_ptr(), 0, cols, M, y.data_ptr(), None) == 0
+            torch.cuda.synchronize()
+            check_close(y.cpu().numpy(), O.linear_forward_f64(deqm, x.float().cpu().numpy()))
+        rt.mfq_rt_free_quant_linear(hm)
+        with pytest.raises(RuntimeError, match="payload size"):
+            _load(rt, dtype, O.pack_mx(tm)[:-1])
     # NINT8-0 through the same registry
     t8 = O.quantize_nint8_zero((rng.standard_normal((24, 64)) * 0.02).astype(np.float32))
     h8 = _load(rt, "NINT8-0", O.pack_nint8_zero(t8))
@@ -220,12 +243,14 @@ def test_cpp_moe_ffn_forward(rt, T):
 
 
 def _mixed_moe(rng, E_out, K):
-    """Eight experts in five cohorts of different families (NINT4, NVQ3J-512, NVQ1-S, NEPQ1-S, NEPQ0-L)."""
+    """Eight experts in seven cohorts of different families (NINT4, NINT8-0, NVQ3J-512, MXFP4, NVQ1-S, NEPQ1-S, NEPQ0-L)."""
     def pool(ids, dtype, t):
         return O.MoePool(np.asarray(ids, dtype=np.int32), dtype, t)
     return O.NintMoeTensor((8, E_out, K), [
-        pool([0, 5, 7], "NINT4", synth.nint_random(rng, 3 * E_out, K, 4, 32, 6)),
-        pool([1, 4], "NVQ3J-512", synth.nvq_jsc_random(rng, 2 * E_out, K, "d4_512", 2)),
+        pool([0, 7], "NINT4", synth.nint_random(rng, 2 * E_out, K, 4, 32, 6)),
+        pool([5], "NINT8-0", O.quantize_nint8_zero((rng.standard_normal((E_out, K)) * 0.02).astype(np.float32))),
+        pool([1], "NVQ3J-512", synth.nvq_jsc_random(rng, E_out, K, "d4_512", 2)),
+        pool([4], "MXFP4", synth.mx_random(rng, "MXFP4", E_out, K, 112, 116)),
         pool([2], "NVQ1-S", synth.nvq1_random(rng, "NVQ1-S", E_out, K)),
         pool([6], "NEPQ1-S", synth.nepq_random(rng, "NEPQ1-S", 1, E_out, K, 3)),
         pool([3], "NEPQ0-L", synth.nepq_random(rng, "NEPQ0-L", 1, E_out, K, 2))])
@@ -233,7 +258,7 @@ def _mixed_moe(rng, E_out, K):
 
 @pytest.mark.parametrize("T", [3, 40])
 def test_cpp_moe_ffn_with_cohorts_of_other_families(rt, T):
-    """Gate/up and down tensors whose cohorts mix NINT with NVQ, a 1-bit family and NEPQ: the C++ runtime splits the
+    """Gate/up and down tensors whose cohorts mix NINT with NVQ, MXFP4, a 1-bit family and NEPQ: the C++ runtime splits the
     foreign cohorts into per-expert tensors and walks the routed experts on the host; the layer against the oracle."""
     rng = np.random.default_rng(140 + T)
     E, H, W, k = 8, 192, 96, 3

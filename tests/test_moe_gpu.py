@@ -407,15 +407,26 @@ def test_mixed_family_cohorts_in_one_tensor():
         h = w.forward_glu(x.cuda(), route).float().cpu().numpy()
         y = O.moe_grouped_matmul(dense, x.float().numpy(), ids)
         assert rel_l2(h, O.moe_swiglu(y)) < 5e-3
-    only = O.NintMoeTensor((3, out, K), [O.MoePool(np.array([2, 0], dtype=np.int32), "NVQ3J-512",
+    # no NINT cohort at all; a NINT8-0 pool; a native MXFP4 pool (one [experts * out, K] tensor, its experts row ranges of it)
+    only = O.NintMoeTensor((6, out, K), [O.MoePool(np.array([5], dtype=np.int32), "NINT8-0", O.quantize_nint8_zero(
+                                             (rng.standard_normal((out, K)) * 0.02).astype(np.float32))),O.MoePool(np.array([2, 0], dtype=np.int32), "NVQ3J-512",
                                                    synth.nvq_jsc_random(rng, 2 * out, K, "d4_512", 2)),
                                          O.MoePool(np.array([1], dtype=np.int32), "NVQ1-S",
-                                                   synth.nvq1_random(rng, "NVQ1-S", out, K))])
+                                                   synth.nvq1_random(rng, "NVQ1-S", out, K)),
+                                         O.MoePool(np.array([4, 3], dtype=np.int32), "MXFP4",
+                                                   synth.mx_random(rng, "MXFP4", 2 * out, K, 120, 124))])
     w2 = NintMoeWeight.from_blob(O.pack_nint_moe(only))
+    assert [c.dtype for c in w2.foreign] == ["NINT8-0", "NVQ3J-512", "NVQ1-S", "MXFP4"]
     d2 = O.dequantize_expertwise(only)
-    ids = np.stack([rng.choice(3, size=2, replace=False) for _ in range(20)]).astype(np.int32)
-    x = torch.from_numpy((rng.standard_normal((20, K)) * 0.1).astype(np.float32)).to(torch.bfloat16)
-    got = w2(x.cuda(), build_moe_route_plan(torch.from_numpy(ids).cuda(), 3)).cpu().numpy()
-    assert rel_l2(got, O.moe_grouped_matmul(d2, x.float().numpy(), ids)) < REL_TOL
+    assert np.array_equal(w2.dequantize().cpu().numpy().view(np.uint32), d2.view(np.uint32))
+    for T in (20, 2):
+        ids = np.stack([rng.choice(6, size=2, replace=False) for _ in range(T)]).astype(np.int32)
+        x = torch.from_numpy((rng.standard_normal((T, K)) * 0.1).astype(np.float32)).to(torch.bfloat16)
+        got = w2(x.cuda(), build_moe_route_plan(torch.from_numpy(ids).cuda(), 6)).cpu().numpy()
+        ref = O.moe_grouped_matmul(d2, x.float().numpy(), ids)
+        assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL * max(1.0, float(np.sqrt(np.mean(ref * ref))))
+    bad = O.NintMoeTensor((1, 128, 128), [O.MoePool(np.array([0], dtype=np.int32), "MXFP8", synth.mx_random(rng, "MXFP8", 128, 128))])
+    with pytest.raises(ValueError, match="NINTM supports native MXFP4 expert pools, got MXFP8"):
+        NintMoeWeight.from_blob(O.pack_nint_moe(bad))
     with pytest.raises(NotImplementedError, match="NINT cohorts only"):
         MoeExpertCache(1 << 20).register_source(blob)

@@ -38,6 +38,8 @@ def _blobs():
         ("NEPQ0-L", O.pack_nepq(synth.nepq_random(rng, "NEPQ0-L", 1, 8, 200, 3))),
         ("NINTM", O.pack_nint_moe(moe)),
         ("NINTM", O.pack_nint_moe(mixed)),
+        ("MXFP4", O.pack_mx(synth.mx_random(rng, "MXFP4", 5, 96))),
+        ("MXFP8", O.pack_mx(synth.mx_random(rng, "MXFP8", 130, 128))),
     ]
 
 
@@ -70,6 +72,8 @@ def _py_parse(dtype, blob):
         return F.parse_nintm(blob)
     if dtype == "NINT8-0":
         return F.parse_nint8_zero(blob)
+    if F.is_mx_dtype(dtype):
+        return F.parse_mx(dtype, blob)
     if dtype.startswith("NINT"):
         return F.parse_nint(blob)
     if F.is_lowbit_dtype(dtype):
@@ -79,7 +83,7 @@ def _py_parse(dtype, blob):
     return F.parse_nvq(blob)
 
 
-@pytest.mark.parametrize("case", range(13))
+@pytest.mark.parametrize("case", range(15))
 def test_python_parsers_raise_on_malformed_blobs(case):
     dtype, blob = _blobs()[case]
     _py_parse(dtype, blob)                                   # the well-formed blob parses
@@ -105,7 +109,7 @@ def rt():
     return lib
 
 
-@pytest.mark.parametrize("case", range(13))
+@pytest.mark.parametrize("case", range(15))
 def test_cpp_loaders_return_errors_on_malformed_blobs(rt, case):
     dtype, blob = _blobs()[case]
     rng = np.random.default_rng(200 + case)

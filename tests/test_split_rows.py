@@ -1,4 +1,4 @@
-"""formats.split_rows: the per-expert blobs cut from a cohort tensor of the NVQ and 1-bit families parse on their own and
+"""formats.split_rows: the per-expert blobs cut from a cohort tensor of the NVQ, 1-bit and NINT8-0 families parse on their own and
 dequantize (oracle) to the expert's rows of the whole tensor, bit for bit -- for streams whose per-expert share does not
 start on a byte boundary."""
 import numpy as np
@@ -18,6 +18,7 @@ CASES = {
     "NVQ1-S": lambda rng: synth.nvq1_random(rng, "NVQ1-S", 45, 104, custom=True),
     "NPQ0-L": lambda rng: synth.npq0_random(rng, "NPQ0-L", 45, 104),
     "NPQ0-S": lambda rng: synth.npq0_random(rng, "NPQ0-S", 45, 104),
+    "NINT8-0": lambda rng: O.quantize_nint8_zero((rng.standard_normal((45, 96)) * 0.02).astype(np.float32)),
 }
 
 

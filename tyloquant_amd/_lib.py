@@ -118,6 +118,10 @@ _SIGS = {
     "mfq_hip_nvqs_gemv": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
     "mfq_hip_nvqs_gemm_workspace_bytes": (sz, [C.POINTER(NvqsDesc), C.c_int]),
     "mfq_hip_nvqs_gemm": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
+    "mfq_hip_mx_dequant_rows": (C.c_int, [C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, vp, i64, vp]),
+    "mfq_hip_mx_gemm_rows_workspace_bytes": (sz, [C.c_int, C.c_int, C.c_int]),
+    "mfq_hip_mx_gemm_rows": (C.c_int, [C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp, i64,
+                                       vp, sz, vp]),
     "mfq_hip_nepq_plan": (C.c_int, [C.c_int] * 4 + [C.POINTER(NepqDesc)]),
     "mfq_hip_nepq_repack": (C.c_int, [C.POINTER(NepqDesc), vp, i64, vp, vp]),
     "mfq_hip_nepq_dequant_f32": (C.c_int, [C.POINTER(NepqDesc), vp, vp, i64, vp]),

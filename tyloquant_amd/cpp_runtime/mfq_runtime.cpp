@@ -316,6 +316,42 @@ Nint8ZeroWeight Nint8ZeroWeight::from_blob(const uint8_t *blob, size_t n, mfq_st
     return w;
 }
 
+// parse_mx_layout / validate_mx_shapes (mfq/formats/mx.py:65-173; unpack_mxfp8 / unpack_mxfp4, cpp_runtime/mfq_decode.cpp:1832-1918)
+MxWeight MxWeight::from_blob(const std::string &dtype, const uint8_t *blob, size_t n, int64_t out_per_expert, mfq_stream_t stream) {
+    const int want_kind = dtype == "MXFP4" ? 4 : dtype == "MXFP8" ? 8 : 0;
+    if (!want_kind) fail("unsupported MX dtype: " + dtype);
+    if (n < 56) fail("truncated MFQ MX tensor header");
+    const int version = blob[4], kind = blob[5];
+    if (std::memcmp(blob, "MXT1", 4) != 0 || version != 1 || kind != want_kind || rd<uint16_t>(blob, 6) != 0)
+        fail("invalid " + dtype + " payload header");
+    uint64_t d[6];
+    for (int i = 0; i < 6; ++i) d[i] = rd<uint64_t>(blob, 8 + 8 * static_cast<size_t>(i));
+    const uint64_t rows = d[0], cols = d[1];
+    if (rows == 0 || cols == 0 || rows > INT32_MAX || cols > INT32_MAX) fail("invalid MX logical shape");
+    uint64_t sr, sc, qr, qc;
+    if (kind == 4) {
+        if (cols % 32) fail("MXFP4 columns must be divisible by 32");
+        sr = rows; sc = cols / 2; qr = rows; qc = cols / 32;
+    } else {
+        if (cols % 128) fail("MXFP8 columns must be divisible by 128");
+        sr = rows; sc = cols; qr = (rows + 127) / 128; qc = cols / 128;
+    }
+    if (d[2] != sr || d[3] != sc) fail(dtype + " storage shape does not match its logical shape");
+    if (d[4] != qr || d[5] != qc) fail(dtype + " scale shape does not match its logical shape");
+    const uint64_t nv = sr * sc, ns = qr * qc;
+    if (n != 56 + nv + ns) fail(dtype + " payload size " + std::to_string(n) + " != " + std::to_string(56 + nv + ns));
+    MxWeight w;
+    w.kind = kind; w.rows = static_cast<int64_t>(rows); w.cols = static_cast<int64_t>(cols); w.dtype = dtype;
+    w.out_per_expert = out_per_expert > 0 ? out_per_expert : w.rows;
+    if (w.rows % w.out_per_expert) fail(dtype + ": the rows are not a whole number of experts");
+    if (kind == 8 && w.out_per_expert != w.rows && w.out_per_expert % 128) fail("MXFP8 expert slices must preserve 128-row blocks");
+    w.values = DeviceBuffer::from_host(blob + 56, nv);
+    w.scales = DeviceBuffer::from_host(blob + 56 + nv, ns);
+    hip_check(hipStreamSynchronize(hs(stream)), "mx upload");
+    return w;
+}
+int64_t MxWeight::payload_bytes() const { return (kind == 4 ? rows * cols / 2 + rows * (cols / 32) : rows * cols + (rows + 127) / 128 * (cols / 128)); }
+
 namespace {
 // bits [bit0, bit0 + nbits) of the little-endian bit stream at s (which has `avail` readable bytes), as a stream of its own
 std::vector<uint8_t> slice_bits(const uint8_t *s, size_t avail, int64_t bit0, int64_t nbits) {
@@ -335,6 +371,28 @@ std::vector<std::vector<uint8_t>> split_rows(const std::string &dtype, const uin
     size_t body_off, tables;
     int64_t out, K;
     std::vector<int64_t> per_row;
+    if (dtype == "NINT8-0") {  // [rows, K] along axis 0: a row is its ng blocks of 34 bytes, back to back
+        if (n < 40 || std::memcmp(b, "NI80", 4) != 0) fail("invalid NINT8-0 header");
+        const int axis = rd<int32_t>(b, 4), neuron_len = rd<int32_t>(b, 8);
+        const uint32_t ndim = rd<uint32_t>(b, 12);
+        if (axis != 0 || ndim != 2 || neuron_len <= 0 || neuron_len % 32) fail("NINT8-0 cohorts are [rows, K] tensors quantized along axis 0");
+        const int64_t rows_all = rd<uint32_t>(b, 32), ng = rd<uint32_t>(b, 36);
+        if (rows_all <= 0 || ng != neuron_len / 32 || n - 40 != static_cast<size_t>(rows_all * ng) * 34) fail("invalid NINT8-0 block payload length");
+        if (parts <= 0 || rows_all % parts) fail(dtype + ": " + std::to_string(rows_all) + " neurons do not split into " + std::to_string(parts) + " equal parts");
+        const int64_t rows = rows_all / parts;
+        const size_t piece_bytes = static_cast<size_t>(rows * ng) * 34;
+        std::vector<std::vector<uint8_t>> res;
+        for (int i = 0; i < parts; ++i) {
+            std::vector<uint8_t> v(b, b + 16);  // magic, axis, neuron_len, ndim
+            auto put = [&](const void *p, size_t len) { const uint8_t *q = static_cast<const uint8_t *>(p); v.insert(v.end(), q, q + len); };
+            const int64_t shape[2] = {rows, neuron_len};
+            const uint32_t tail[2] = {static_cast<uint32_t>(rows), static_cast<uint32_t>(ng)};
+            put(shape, 16); put(tail, 8);
+            put(b + 40 + static_cast<size_t>(i) * piece_bytes, piece_bytes);
+            res.push_back(std::move(v));
+        }
+        return res;
+    }
     if (is_lowbit_linear_dtype(dtype)) {
         if (n < 20) fail("truncated " + dtype + " header");
         const int ver = b[4], sbits = b[5];
@@ -679,6 +737,20 @@ void nint8_zero_matmul(const Nint8ZeroWeight &w, const void *x, int x_dtype, int
 void nint8_zero_dequantize(const Nint8ZeroWeight &w, float *out, mfq_stream_t stream) {
     abi_check(mfq_hip_nint8z_dequant_f32(&w.desc, w.data.get(), out, w.desc.neuron_len, stream));
 }
+void mx_matmul(const MxWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) {
+    if (expert < 0 || expert >= w.n_experts()) fail(w.dtype + ": expert index out of range");
+    const int nrows = static_cast<int>(w.out_per_expert), row0 = expert * nrows;
+    const size_t need = mfq_hip_mx_gemm_rows_workspace_bytes(static_cast<int>(w.cols), nrows, M);
+    w.workspace.ensure(need);
+    abi_check(mfq_hip_mx_gemm_rows(w.kind, w.values.get(), w.scales.get(), static_cast<int>(w.rows), static_cast<int>(w.cols), row0,
+                                   nrows, x, x_dtype, ldx, M, y, nrows, w.workspace.get(), need, stream));
+}
+void mx_dequantize(const MxWeight &w, int expert, float *out, mfq_stream_t stream) {
+    if (expert < 0 || expert >= w.n_experts()) fail(w.dtype + ": expert index out of range");
+    const int nrows = static_cast<int>(w.out_per_expert), row0 = expert * nrows;
+    abi_check(mfq_hip_mx_dequant_rows(w.kind, w.values.get(), w.scales.get(), static_cast<int>(w.rows), static_cast<int>(w.cols),
+                                      row0, nrows, MFQ_X_F32, out, w.cols, stream));
+}
 void nvq_dequantize(const NvqWeight &w, float *out, mfq_stream_t stream) {
     if (w.streams) {
         abi_check(mfq_hip_nvqs_dequant_f32(&w.sdesc, w.data.get(), out, w.sdesc.neuron_len, stream));
@@ -705,24 +777,27 @@ bool is_nvq_linear_dtype(const std::string &d) {
 }
 bool is_nepq_linear_dtype(const std::string &d) { return d == "NEPQ1-S" || d == "NEPQ1-L" || d == "NEPQ0-S" || d == "NEPQ0-L"; }
 bool is_lowbit_linear_dtype(const std::string &d) { return d == "NVQ1-L" || d == "NVQ1-S" || d == "NPQ0-L" || d == "NPQ0-S"; }
+bool is_mx_linear_dtype(const std::string &d) { return d == "MXFP4" || d == "MXFP8"; }
 
 int64_t QuantLinear::out() const {
     return kind == QuantLinearKind::Nint ? nint->out() : kind == QuantLinearKind::Nvq ? nvq->out()
-         : kind == QuantLinearKind::Nepq ? nepq->out() : nint8z->out();
+         : kind == QuantLinearKind::Nepq ? nepq->out() : kind == QuantLinearKind::Mx ? mx->out() : nint8z->out();
 }
 int64_t QuantLinear::neuron_len() const {
     return kind == QuantLinearKind::Nint ? nint->neuron_len() : kind == QuantLinearKind::Nvq ? nvq->neuron_len()
-         : kind == QuantLinearKind::Nepq ? nepq->neuron_len() : nint8z->neuron_len();
+         : kind == QuantLinearKind::Nepq ? nepq->neuron_len() : kind == QuantLinearKind::Mx ? mx->neuron_len() : nint8z->neuron_len();
 }
 int64_t QuantLinear::payload_bytes() const {
     return kind == QuantLinearKind::Nint ? nint->desc.payload_bytes : kind == QuantLinearKind::Nvq ? nvq->payload_bytes()
-         : kind == QuantLinearKind::Nepq ? nepq->payload_bytes() : nint8z->desc.payload_bytes;
+         : kind == QuantLinearKind::Nepq ? nepq->payload_bytes() : kind == QuantLinearKind::Mx ? mx->payload_bytes()
+         : nint8z->desc.payload_bytes;
 }
 void QuantLinear::forward(const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const {
     if (M == 0) return;  // an empty batch: no rows to write
     if (kind == QuantLinearKind::Nint) nint_matmul(*nint, x, x_dtype, ldx, M, y, stream);
     else if (kind == QuantLinearKind::Nvq) nvq_matmul(*nvq, x, x_dtype, ldx, M, y, stream);
     else if (kind == QuantLinearKind::Nepq) nepq_matmul(*nepq, 0, x, x_dtype, ldx, M, y, stream);
+    else if (kind == QuantLinearKind::Mx) mx_matmul(*mx, 0, x, x_dtype, ldx, M, y, stream);
     else nint8_zero_matmul(*nint8z, x, x_dtype, ldx, M, y, stream);
 }
 void QuantLinear::reserve(int max_M) const {
@@ -737,6 +812,8 @@ void QuantLinear::reserve(int max_M) const {
         else if (kind == QuantLinearKind::Nepq)
             n = nepq->streams ? mfq_hip_nvqs_gemm_rows_workspace_bytes(&nepq->sdesc, nepq->out_per_expert, M)
                               : mfq_hip_nepq_gemm_workspace_bytes(&nepq->desc, nepq->out_per_expert, M);
+        else if (kind == QuantLinearKind::Mx)
+            n = mfq_hip_mx_gemm_rows_workspace_bytes(static_cast<int>(mx->cols), static_cast<int>(mx->out_per_expert), M);
         else n = mfq_hip_nint8z_gemm_workspace_bytes(&nint8z->desc, M);
         need = std::max(need, n);
     };
@@ -749,12 +826,14 @@ void QuantLinear::reserve(int max_M) const {
         nepq->workspace.ensure(need);
         if (nepq->rotation_block) rot = static_cast<size_t>(std::max(max_M, 0)) * nepq->neuron_len() * 2;
         nepq->rotated.ensure(rot);
-    } else nint8z->workspace.ensure(need);
+    } else if (kind == QuantLinearKind::Mx) mx->workspace.ensure(need);
+    else nint8z->workspace.ensure(need);
 }
 void QuantLinear::dequantize(float *out, mfq_stream_t stream) const {
     if (kind == QuantLinearKind::Nint) nint_dequantize(*nint, out, stream);
     else if (kind == QuantLinearKind::Nvq) nvq_dequantize(*nvq, out, stream);
     else if (kind == QuantLinearKind::Nepq) nepq_dequantize(*nepq, out, stream);
+    else if (kind == QuantLinearKind::Mx) mx_dequantize(*mx, 0, out, stream);
     else nint8_zero_dequantize(*nint8z, out, stream);
 }
 
@@ -791,6 +870,11 @@ QuantLinear load_quant_linear(const std::string &dtype_in, const uint8_t *blob, 
         if (q.nepq->n_experts != 1)
             fail("a " + dtype + " linear must hold one expert, the blob holds " + std::to_string(q.nepq->n_experts) +
                  " (multi-expert NEPQ tensors are NINTM cohorts)");
+        return q;
+    }
+    if (is_mx_linear_dtype(dtype)) {
+        q.kind = QuantLinearKind::Mx;
+        q.mx = std::make_shared<MxWeight>(MxWeight::from_blob(dtype, blob, n, 0, stream));
         return q;
     }
     fail("unsupported quantized linear dtype: " + dtype);
@@ -837,11 +921,16 @@ NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream
                 if (c.nepq->label != p.dtype) fail("MFQ dtype/blob mismatch: " + p.dtype + " contains " + c.nepq->label);
                 if (c.nepq->n_experts != parts || c.nepq->out_per_expert != h.out_per_expert || c.nepq->neuron_len() != h.neuron_len)
                     fail(shape_error);
-            } else if (is_nvq_linear_dtype(p.dtype) || is_lowbit_linear_dtype(p.dtype)) {
+            } else if (is_nvq_linear_dtype(p.dtype) || is_lowbit_linear_dtype(p.dtype) || p.dtype == "NINT8-0") {
                 for (const auto &piece : split_rows(p.dtype, blob + p.payload_off, p.payload_bytes, parts)) {
                     c.linears.push_back(load_quant_linear(p.dtype, piece.data(), piece.size(), stream));
                     if (c.linears.back().out() != h.out_per_expert || c.linears.back().neuron_len() != h.neuron_len) fail(shape_error);
                 }
+            } else if (p.dtype == "MXFP4") {  // mfq/formats/moe.py:122-124: one [experts * out, K] tensor
+                c.mx = std::make_shared<MxWeight>(MxWeight::from_blob(p.dtype, blob + p.payload_off, p.payload_bytes, h.out_per_expert, stream));
+                if (c.mx->rows != static_cast<int64_t>(parts) * h.out_per_expert || c.mx->cols != h.neuron_len) fail(shape_error);
+            } else if (p.dtype == "MXFP8") {  // expert_tensor_family, mfq/formats/moe.py:38-47
+                fail("NINTM supports native MXFP4 expert pools, got " + p.dtype);
             } else {
                 fail("NINTM cohort family " + p.dtype + " is not supported");
             }
@@ -865,16 +954,19 @@ NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream
 }
 
 int64_t MoeForeignCohort::payload_bytes() const {
+    if (mx) return mx->payload_bytes();
     if (nepq) return nepq->payload_bytes();
     int64_t n = 0;
     for (const QuantLinear &q : linears) n += q.payload_bytes();
     return n;
 }
 void MoeForeignCohort::matmul(int local, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const {
-    if (nepq) nepq_matmul(*nepq, local, x, x_dtype, ldx, M, y, stream);
+    if (mx) mx_matmul(*mx, local, x, x_dtype, ldx, M, y, stream);
+    else if (nepq) nepq_matmul(*nepq, local, x, x_dtype, ldx, M, y, stream);
     else linears[static_cast<size_t>(local)].forward(x, x_dtype, ldx, M, y, stream);
 }
 void MoeForeignCohort::dequantize(int local, float *out, mfq_stream_t stream) const {
+    if (mx) { mx_dequantize(*mx, local, out, stream); return; }
     if (!nepq) { linears[static_cast<size_t>(local)].dequantize(out, stream); return; }
     // the cohort dequantizes as a whole: take the expert's rows out of it
     const size_t rows = static_cast<size_t>(nepq->out_per_expert), K = static_cast<size_t>(nepq->neuron_len());
@@ -1526,7 +1618,8 @@ LinearCheckResult run_linear_check(const QuantLinear &lin, int M, int reps) {
     res.payload_bytes = lin.payload_bytes();
     res.weight_bytes = lin.kind == QuantLinearKind::Nint ? lin.nint->desc.total_bytes
                      : lin.kind == QuantLinearKind::Nvq ? lin.nvq->total_bytes()
-                     : lin.kind == QuantLinearKind::Nepq ? lin.nepq->total_bytes() : lin.nint8z->desc.total_bytes;
+                     : lin.kind == QuantLinearKind::Nepq ? lin.nepq->total_bytes()
+                     : lin.kind == QuantLinearKind::Mx ? lin.mx->payload_bytes() : lin.nint8z->desc.total_bytes;
     res.production_weight_gbps = res.weight_bytes / (res.production_ms * 1e6);
     res.payload_gbps = res.payload_bytes / (res.production_ms * 1e6);
     res.production_rel = den > 0 ? std::sqrt(num / den) : std::sqrt(num);

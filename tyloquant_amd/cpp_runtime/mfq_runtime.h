@@ -127,6 +127,26 @@ struct NvqWeight {
                                       const uint16_t *iq1s_grid = nullptr, mfq_stream_t stream = nullptr);
 };
 bool is_lowbit_linear_dtype(const std::string &dtype);
+// MXFP4 / MXFP8 (OCP MX payloads of full-precision MFQ files; Mxfp8Weight / Mxfp4Cpu of the reference,
+// cpp_runtime/mfq_decode.cpp:1807-1918, 2060-2100): the payload's value and scale bytes, used on the device as they lie
+// in the file.  A pool of experts is the same tensor with `out_per_expert` rows per expert (MXFP8: whole 128-row blocks).
+struct MxWeight {
+    int kind = 0;  // 4 = MXFP4, 8 = MXFP8
+    int64_t rows = 0, cols = 0, out_per_expert = 0;
+    std::string dtype;
+    DeviceBuffer values, scales;
+    mutable DeviceBuffer workspace;
+    int64_t out() const { return out_per_expert; }
+    int64_t neuron_len() const { return cols; }
+    int64_t n_experts() const { return rows / out_per_expert; }
+    int64_t payload_bytes() const;
+    static MxWeight from_blob(const std::string &dtype, const uint8_t *blob, size_t n, int64_t out_per_expert = 0,
+                              mfq_stream_t stream = nullptr);
+};
+bool is_mx_linear_dtype(const std::string &dtype);
+void mx_matmul(const MxWeight &w, int expert, const void *x, int x_dtype, int64_t ldx, int M, float *y,
+               mfq_stream_t stream = nullptr);
+void mx_dequantize(const MxWeight &w, int expert, float *out, mfq_stream_t stream = nullptr);
 struct NepqWeight {
     mfq_nepq_desc desc{};    // lane-major layout (NEPQ1-S, NEPQ1-L)
     mfq_nvqs_desc sdesc{};   // streams read in place (NEPQ0-S, NEPQ0-L: the product tables of NPQ0): `streams` set
@@ -195,13 +215,14 @@ void nepq_dequantize(const NepqWeight &w, float *out, mfq_stream_t stream = null
 bool is_nint_linear_dtype(const std::string &dtype);
 bool is_nvq_linear_dtype(const std::string &dtype);
 bool is_nepq_linear_dtype(const std::string &dtype);
-enum class QuantLinearKind { Nint, Nvq, Nepq, Nint8Zero };
+enum class QuantLinearKind { Nint, Nvq, Nepq, Nint8Zero, Mx };
 struct QuantLinear {
     QuantLinearKind kind;
     std::shared_ptr<NintWeight> nint;
     std::shared_ptr<Nint8ZeroWeight> nint8z;
     std::shared_ptr<NvqWeight> nvq;
     std::shared_ptr<NepqWeight> nepq;
+    std::shared_ptr<MxWeight> mx;
     int64_t out() const;
     int64_t neuron_len() const;
     int64_t payload_bytes() const;
@@ -231,7 +252,7 @@ MoeRoutePlan build_moe_route_plan(const int32_t *ids, int tokens, int routes, in
 // tables, the rows' anchors and their share of every tensor-wide bit stream re-packed from bit 0.
 std::vector<std::vector<uint8_t>> split_rows(const std::string &dtype, const uint8_t *blob, size_t n, int parts);
 
-// A NINTM cohort of another family (NVQ, the 1-bit families, NEPQ).  The reference runs them inside its grouped kernels
+// A NINTM cohort of another family (NVQ, the 1-bit families, NEPQ, MXFP4).  The reference runs them inside its grouped kernels
 // (cpp_runtime/mfq_decode.cpp:4800-5360); here every expert is a tensor of its own on that family's kernels and the host
 // walks the experts a batch routes to -- correct, one matmul per expert hit, not a fast path.
 struct MoeForeignCohort {
@@ -239,6 +260,7 @@ struct MoeForeignCohort {
     std::vector<int32_t> expert_ids;
     std::vector<QuantLinear> linears;   // one per expert (NVQ, 1-bit families)
     std::shared_ptr<NepqWeight> nepq;   // or the cohort as one expert-shaped tensor
+    std::shared_ptr<MxWeight> mx;       // or a native MXFP4 pool: one [experts * out, K] tensor, experts = row ranges
     int64_t payload_bytes() const;
     void matmul(int local, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const;
     void dequantize(int local, float *out, mfq_stream_t stream) const;  // [out_per_expert, K]

@@ -290,6 +290,75 @@ LOWBIT_FORMATS = {
 _NPQ0_TABLES = {"NPQ0-L": (1, 8, 16), "NPQ0-S": (2, 4, 8)}   # table version, states, second sub-codebook entries
 
 
+# OCP MX payloads (mfq/formats/mx.py:20-182): "MXT1", version, kind (4 | 8), reserved, logical / storage / scale shapes,
+# then the value bytes and the E8M0 scale bytes.
+MX_KINDS = {"MXFP4": 4, "MXFP8": 8}
+_MX_HEADER = struct.Struct("<4sBBHQQQQQQ")
+
+
+@dataclass
+class MxHeader:
+    dtype: str
+    kind: int
+    rows: int
+    cols: int
+    values_off: int
+    values_bytes: int
+    scales_off: int
+    scales_bytes: int
+
+
+def is_mx_dtype(dtype: str) -> bool:
+    return dtype in MX_KINDS
+
+
+def mx_shapes(dtype: str, rows: int, cols: int):
+    """(storage shape, scale shape) with the reference's geometry checks and messages (validate_mx_shapes,
+    mfq/formats/mx.py:65-117)."""
+    if dtype not in MX_KINDS:
+        raise ValueError(f"unsupported MX dtype: {dtype}")
+    if rows <= 0 or cols <= 0:
+        raise ValueError(f"invalid MX logical shape: {(rows, cols)}")
+    if dtype == "MXFP4":
+        if cols % 32:
+            raise ValueError("MXFP4 columns must be divisible by 32")
+        return (rows, cols // 2), (rows, cols // 32)
+    if cols % 128:
+        raise ValueError("MXFP8 columns must be divisible by 128")
+    return (rows, cols), ((rows + 127) // 128, cols // 128)
+
+
+def parse_mx(dtype: str, blob) -> MxHeader:
+    """parse_mx_layout (mfq/formats/mx.py:154-173; C++ unpack_mxfp8 / unpack_mxfp4, cpp_runtime/mfq_decode.cpp:1832-1918)."""
+    mv = memoryview(blob)
+    if len(mv) < _MX_HEADER.size:
+        raise ValueError("truncated MFQ MX tensor header")
+    magic, version, kind, reserved, *dims = _MX_HEADER.unpack_from(mv)
+    if magic != b"MXT1" or version != 1 or kind != MX_KINDS.get(dtype) or reserved:
+        raise ValueError(f"invalid {dtype} payload header: magic={magic!r}, version={version}, kind={kind}")
+    rows, cols = int(dims[0]), int(dims[1])
+    storage, scale = mx_shapes(dtype, rows, cols)
+    if (int(dims[2]), int(dims[3])) != storage:
+        raise ValueError(f"{dtype} storage shape {(int(dims[2]), int(dims[3]))} != {storage}")
+    if (int(dims[4]), int(dims[5])) != scale:
+        raise ValueError(f"{dtype} scale shape {(int(dims[4]), int(dims[5]))} != {scale}")
+    nv, ns = storage[0] * storage[1], scale[0] * scale[1]
+    if len(mv) != _MX_HEADER.size + nv + ns:
+        raise ValueError(f"{dtype} payload size {len(mv)} != {_MX_HEADER.size + nv + ns}")
+    return MxHeader(dtype, kind, rows, cols, _MX_HEADER.size, nv, _MX_HEADER.size + nv, ns)
+
+
+def write_mx(dtype: str, rows: int, cols: int, values, scales) -> bytes:
+    """pack_mx (mfq/formats/mx.py:120-151) from the two byte matrices."""
+    storage, scale = mx_shapes(dtype, rows, cols)
+    values, scales = np.ascontiguousarray(values, dtype=np.uint8), np.ascontiguousarray(scales, dtype=np.uint8)
+    if values.shape != storage:
+        raise ValueError(f"{dtype} storage shape {values.shape} != {storage}")
+    if scales.shape != scale:
+        raise ValueError(f"{dtype} scale shape {scales.shape} != {scale}")
+    return _MX_HEADER.pack(b"MXT1", 1, MX_KINDS[dtype], 0, rows, cols, *storage, *scale) + values.tobytes() + scales.tobytes()
+
+
 @dataclass
 class LowbitHeader:
     dtype: str
@@ -379,10 +448,19 @@ def _slice_bits(buf, byte_off: int, bit0: int, nbits: int) -> bytes:
 
 
 def split_rows(dtype: str, blob, parts: int) -> list[bytes]:
-    """Cut an NVQ-family or 1-bit-family tensor of parts * n neurons into `parts` blobs of n neurons each (the experts of a
+    """Cut an NVQ-family, 1-bit-family or NINT8-0 tensor of parts * n neurons into `parts` blobs of n neurons each (the experts of a
     NINTM cohort, cpp_runtime/mfq_decode.cpp:4800-5360): same header flags and tables, the anchors and the rows' share
     of every tensor-wide bit stream re-packed from bit 0."""
     blob = bytes(blob)
+    if dtype == "NINT8-0":                  # [rows, K] along axis 0: a row is its ng blocks of 34 bytes, back to back
+        h = parse_nint8_zero(blob)
+        if h.axis != 0 or len(h.shape) != 2:
+            raise ValueError("NINT8-0 cohorts are [rows, K] tensors quantized along axis 0")
+        if parts <= 0 or h.out % parts:
+            raise ValueError(f"{dtype}: {h.out} neurons do not split into {parts} equal parts")
+        n, row = h.out // parts, h.ng * 34
+        head = _N8Z_HDR.pack(b"NI80", 0, h.neuron_len, 2) + struct.pack("<2q", n, h.neuron_len) + struct.pack("<II", n, h.ng)
+        return [head + blob[h.body_off + i * n * row: h.body_off + (i + 1) * n * row] for i in range(parts)]
     if is_lowbit_dtype(dtype):
         h = parse_lowbit(dtype, blob)
         ib = LOWBIT_FORMATS[dtype][3]

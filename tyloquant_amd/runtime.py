@@ -365,7 +365,8 @@ class QuantLinear:
                  "nint8z": lambda M: lib.mfq_hip_nint8z_gemm_workspace_bytes(C.byref(w.desc), M),
                  "nvq": lambda M: (lib.mfq_hip_nvqs_gemm_workspace_bytes if type(w).__name__ == "NvqsWeight"
                                    else lib.mfq_hip_nvq_gemm_workspace_bytes)(C.byref(w.desc), M),
-                 "nepq": lambda M: lib.mfq_hip_nepq_gemm_workspace_bytes(C.byref(w.desc), w.out_per_expert, M)}[self.kind]
+                 "nepq": lambda M: lib.mfq_hip_nepq_gemm_workspace_bytes(C.byref(w.desc), w.out_per_expert, M),
+                 "mx": lambda M: lib.mfq_hip_mx_gemm_rows_workspace_bytes(w.neuron_len, w.out, M)}[self.kind]
         sizes = set(range(1, min(max_rows, 512) + 1)) | set(range(576, max_rows, 64)) | {max_rows}
         need = max((int(query(M)) for M in sizes if M > 0), default=0)
         w._ws.get(need, w.data.device)
@@ -402,7 +403,15 @@ def load_quant_linear(dtype: str, blob, device="cuda") -> QuantLinear:
             raise ValueError(f"a {dtype} linear must hold one expert, the blob holds {w.n_experts} "
                              "(multi-expert NEPQ tensors are NINTM cohorts)")
         return QuantLinear("nepq", w)
+    if F.is_mx_dtype(dtype):
+        from .runtime_mx import MxWeight
+        return QuantLinear("mx", MxWeight.from_blob(dtype, blob, device))
     raise ValueError(f"unsupported quantized linear dtype: {dtype}")
+
+
+def _mx_mm(w, x):
+    from .runtime_mx import mx_matmul
+    return mx_matmul(w, x)
 
 
 def _nvq_mm(w, x):
@@ -415,4 +424,4 @@ def _nepq_mm(w, x):
     return nepq_matmul(w, x)
 
 
-_MATMUL = {"nint": nint_matmul, "nint8z": nint8_zero_matmul, "nvq": _nvq_mm, "nepq": _nepq_mm}
+_MATMUL = {"nint": nint_matmul, "nint8z": nint8_zero_matmul, "nvq": _nvq_mm, "nepq": _nepq_mm, "mx": _mx_mm}

@@ -90,7 +90,7 @@ def build_moe_route_plan(ids: torch.Tensor, n_experts: int) -> MoeRoutePlan:
 
 
 class ForeignCohort:
-    """A NINTM cohort of another family (NVQ, the 1-bit families, NEPQ): the reference runs them inside its grouped
+    """A NINTM cohort of another family (NVQ, the 1-bit families, NEPQ, MXFP4): the reference runs them inside its grouped
     kernels (cpp_runtime/mfq_decode.cpp:4800-5360, mfq/kernels/cuda/nvq_matmul.cu:2588-3175); here every expert is a
     tensor of its own on that family's kernels and the host walks the experts a batch routes to -- correct, one matmul
     per expert hit, not a fast path."""
@@ -100,8 +100,15 @@ class ForeignCohort:
         self.dtype, self.expert_ids = dtype, np.asarray(expert_ids, dtype=np.int32)
         self.out, self.neuron_len = out_per_expert, neuron_len
         n = len(self.expert_ids)
-        self.nepq, self.linears = None, []
-        if is_nepq_linear_dtype(dtype):
+        self.nepq, self.mx, self.linears = None, None, []
+        if F.is_mx_dtype(dtype):               # a pool is one [experts * out, K] tensor (mfq/formats/moe.py:122-124)
+            from .runtime_mx import MxWeight
+            h = F.parse_mx(dtype, blob)
+            if (h.rows, h.cols) != (n * out_per_expert, neuron_len):
+                raise ValueError(f"NINTM pool tensor shape {(h.rows, h.cols)} must be {(n * out_per_expert, neuron_len)}")
+            self.mx = MxWeight.from_blob(dtype, blob, device, out=out_per_expert)
+            shape = (n, out_per_expert, neuron_len)
+        elif is_nepq_linear_dtype(dtype):
             from .runtime_vq import NepqWeight
             self.nepq = NepqWeight.from_blob(blob, device)
             if self.nepq.label != dtype:
@@ -115,15 +122,22 @@ class ForeignCohort:
 
     @property
     def payload_bytes(self) -> int:
+        if self.mx is not None:
+            return self.mx.payload_bytes
         return self.nepq.payload_bytes if self.nepq is not None else sum(q.weight.payload_bytes for q in self.linears)
 
     def matmul(self, local: int, x: torch.Tensor) -> torch.Tensor:
+        if self.mx is not None:
+            from .runtime_mx import mx_matmul
+            return mx_matmul(self.mx, x, local)
         if self.nepq is not None:
             from .runtime_vq import nepq_matmul
             return nepq_matmul(self.nepq, x, local)
         return self.linears[local](x)
 
     def dequantize(self) -> torch.Tensor:
+        if self.mx is not None:
+            return torch.stack([self.mx.dequantize(e) for e in range(self.mx.n_experts)])
         if self.nepq is not None:
             return self.nepq.dequantize().reshape(len(self.expert_ids), self.out, self.neuron_len)
         return torch.stack([q.dequantize() for q in self.linears])
@@ -177,7 +191,10 @@ class NintMoeWeight:
                 raise ValueError("unexpected NINTM cohort runtime metadata")
             if not (p.dtype.startswith("NINT") and p.dtype[4:].isdigit()):
                 from .runtime import is_nepq_linear_dtype, is_nvq_linear_dtype
-                if not (is_nvq_linear_dtype(p.dtype) or is_nepq_linear_dtype(p.dtype) or F.is_lowbit_dtype(p.dtype)):
+                if p.dtype == "MXFP8":      # expert_tensor_family, mfq/formats/moe.py:38-47
+                    raise ValueError(f"NINTM supports native MXFP4 expert pools, got {p.dtype}")
+                if not (is_nvq_linear_dtype(p.dtype) or is_nepq_linear_dtype(p.dtype) or F.is_lowbit_dtype(p.dtype)
+                        or p.dtype in ("MXFP4", "NINT8-0")):
                     raise NotImplementedError(f"NINTM cohort family {p.dtype} is not supported")
                 foreign.append(ForeignCohort(p.dtype, bytes(blob[p.payload_off: p.payload_off + p.payload_bytes]),
                                              p.expert_ids, h.out_per_expert, h.neuron_len, device))
