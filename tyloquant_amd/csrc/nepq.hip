@@ -553,7 +553,7 @@ __global__ __launch_bounds__(1024) void nepq_tile_kernel(NepqK k, const uint8_t 
 // state * (bias - 1) with one packed add (exact for the 1/8 bias, one fp16 rounding for 5/32), so no separate bias
 // term is needed.  Rows [row0, row0 + nrows) of the tensor (an expert's slice) go to columns 0 .. nrows - 1 of y.
 // LDS: [table: banks * entries u16, when TAB_LDS][x tiles]
-template <int MT, int NB, int PF, int XD, int TAB_LDS>
+template <int MT, int NB, int PF, int XD, int TAB_LDS, int PROF>
 __global__ __launch_bounds__(512) void nepq_prefill_kernel(NepqK k, const uint8_t *__restrict__ w, int rb_first, int row0,
                                                            int nrows, const uint16_t *__restrict__ x16, int Kp,
                                                            const float *__restrict__ xscale, int M,
@@ -618,7 +618,7 @@ __global__ __launch_bounds__(512) void nepq_prefill_kernel(NepqK k, const uint8_
             if (c < BM * CHUNKS) *reinterpret_cast<u32x4_t *>(xt + buf * (BM * ROW) + row * ROW + EL * ch) = xq[p];
         }
     };
-    const uint32_t toff = 1024u, boff = 1024u + (k.tail ? 256u : 0u);
+    const uint32_t toff = 1024u, boff = 1024u + ((PROF == 3) ? 256u : 0u);
     uint32_t qr[PF][NB], tails[NB], banks4[NB], tailsn[NB], banks4n[NB];
     auto wload = [&](int it, uint32_t (&qq)[NB]) {
         const int s = it >> 2, j = it & 3;
@@ -631,7 +631,7 @@ __global__ __launch_bounds__(512) void nepq_prefill_kernel(NepqK k, const uint8_
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const uint32_t off = b < nrb && s < s_end ? b * rbb + s * sb : kNoStep;
-            tt[b] = k.tail ? __builtin_amdgcn_raw_buffer_load_b32(win, off + toff + lane * 4, 0, 0) : 0u;
+            tt[b] = (PROF == 3) ? __builtin_amdgcn_raw_buffer_load_b32(win, off + toff + lane * 4, 0, 0) : 0u;
             bb[b] = __builtin_amdgcn_raw_buffer_load_b32(win, off + boff + r * 4, 0, 0);
         }
     };
@@ -644,7 +644,7 @@ __global__ __launch_bounds__(512) void nepq_prefill_kernel(NepqK k, const uint8_
     for (int i = 1; i < XD; ++i) xload(4 * s_begin + i, xr[i]);
     __syncthreads();  // table and the first tile
 
-    const float delta = k.profile == 2 ? 0.15625f : 0.125f;
+    const float delta = PROF == 2 ? 0.15625f : 0.125f;
     for (int s = s_begin; s < s_end; ++s) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -657,7 +657,7 @@ __global__ __launch_bounds__(512) void nepq_prefill_kernel(NepqK k, const uint8_
             uint32_t ix[NB][3];
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
-                const NepqUnit u = nepq_decode(k.profile, qr[j % PF][b], (tails[b] >> (8 * j)) & 0xffu);
+                const NepqUnit u = nepq_decode(PROF, qr[j % PF][b], (tails[b] >> (8 * j)) & 0xffu);
                 bank[b] = tab + ((banks4[b] >> (8 * j)) & 0xffu) * k.entries;
                 const float st = static_cast<float>(u.state);
                 S[b] = pk_h2(st, st);
@@ -744,7 +744,9 @@ static int nepq_prefill(const NepqK &k, const uint8_t *w, int row0, int nrows, c
     const int64_t ldk = splits > 1 ? nrows : ldy;
     const int nrb = static_cast<int>(ceil_div(nrows, 16));
     const size_t tabb = (static_cast<size_t>(k.banks) * k.entries * 2 + 15) / 16 * 16;
-    const bool tab_lds = tabb <= 48 * 1024;
+    // the tables live in LDS while they leave room for the activation tiles of the tallest block (53 KB): a 16-bank pool
+    // of the L profile (64 KB) does
+    const bool tab_lds = tabb <= 96 * 1024;
 #define MFQ_NEPQ_PREFILL(MT, NB, XD)                                                                                   \
     {                                                                                                                  \
         const dim3 grid(static_cast<unsigned>(ceil_div(nrb, 8 * NB)), static_cast<unsigned>(ceil_div(M, MT * 16)),     \
@@ -760,7 +762,8 @@ static int nepq_prefill(const NepqK &k, const uint8_t *w, int row0, int nrows, c
                                ystride);                                                                               \
             return MFQ_OK;                                                                                             \
         };                                                                                                             \
-        const int rc = tab_lds ? launch(nepq_prefill_kernel<MT, NB, 4, XD, 1>) : launch(nepq_prefill_kernel<MT, NB, 4, XD, 0>); \
+        const int rc = k.profile == 2 ? (tab_lds ? launch(nepq_prefill_kernel<MT, NB, 4, XD, 1, 2>) : launch(nepq_prefill_kernel<MT, NB, 4, XD, 0, 2>)) \
+                                      : (tab_lds ? launch(nepq_prefill_kernel<MT, NB, 4, XD, 1, 3>) : launch(nepq_prefill_kernel<MT, NB, 4, XD, 0, 3>)); \
         if (rc) return rc;                                                                                             \
         if (splits > 1) return prefill_sum_splits(part, ystride, splits, M, nrows, y, ldy, st);                        \
         return check_launch("nepq_prefill");                                                                           \
