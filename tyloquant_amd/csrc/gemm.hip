@@ -210,7 +210,9 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_kernel(const uint16_t *__rest
                                                           const uint16_t *__restrict__ b, int64_t ldb, int M, int N,
                                                           int K, const float *__restrict__ sa,
                                                           const float *__restrict__ sb, float *__restrict__ y,
-                                                          int64_t ldy) {
+                                                          int64_t ldy, int kps, int64_t ystride) {
+    // split blockIdx.z multiplies the K steps [z * kps, (z + 1) * kps) and writes its (scaled) partial tile to
+    // y + z * ystride; one split: the whole K, y itself
     __shared__ __attribute__((aligned(16))) uint16_t As[2][GBM * GLD];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[2][GBN * GLD];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -229,7 +231,8 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_kernel(const uint16_t *__rest
 #pragma unroll
             for (int t = 0; t < 16; ++t) acc[i][j][t] = 0.f;
 
-    const int nk = K / GBK;  // K is a multiple of 32 (callers pad)
+    const int k_begin = static_cast<int>(blockIdx.z) * kps, nk = min(K / GBK, k_begin + kps);  // K is a multiple of 32 (callers pad)
+    y += static_cast<int64_t>(blockIdx.z) * ystride;
     u32x4_t ra[2], rbv[2];
     auto gload = [&](int kt) {
 #pragma unroll
@@ -245,12 +248,12 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_kernel(const uint16_t *__rest
             *reinterpret_cast<u32x4_t *>(&Bs[buf][lr * GLD + lc + 8 * h]) = rbv[h];
         }
     };
-    gload(0);
+    gload(k_begin);
     lstore(0);
     __syncthreads();
     const int fr = lane & 31, fk = (lane >> 5) * 8;
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
+    for (int kt = k_begin; kt < nk; ++kt) {
+        const int buf = (kt - k_begin) & 1;
         if (kt + 1 < nk) gload(kt + 1);
 #pragma unroll
         for (int kk = 0; kk < GBK; kk += 16) {
@@ -286,15 +289,44 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_kernel(const uint16_t *__rest
     }
 }
 
+int prefill_sum_splits(const float *part, int64_t ystride, int splits, int M, int N, float *y, int64_t ldy, hipStream_t st);
+
+// Splits over K of the dequantize + GEMM path: a grid of 128 x 128 tiles that leaves compute units idle (64 rows against
+// 4096 neurons are 32 blocks) is cut along K, up to eight ways, while a split keeps at least four K steps of 32 and the
+// neuron count allows 16-byte partial rows; the partial tiles go to the end of the workspace and are added in split
+// order (deterministic).  1 = no split.
+static int gemm_splits(int M, int N, int K) {
+    const int64_t blocks = ceil_div(N, GBN) * ceil_div(M, GBM);
+    if (blocks > 128 || N % 4) return 1;
+    int64_t splits = 256 / blocks;
+    if (splits > 8) splits = 8;
+    if (splits > K / GBK / 4) splits = K / GBK / 4;
+    if (splits <= 1) return 1;
+    const int kps = static_cast<int>(ceil_div(K / GBK, splits));
+    return static_cast<int>(ceil_div(K / GBK, kps));
+}
+
+// part: splits * M * N floats when gemm_splits(M, N, K) > 1 (dequant_gemm_carve hands it out), else unused
 int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, const float *sa,
-                const float *sb, float *y, int64_t ldy, hipStream_t st) {
+                const float *sb, float *y, int64_t ldy, hipStream_t st, float *part = nullptr) {
     MFQ_REQUIRE(K % GBK == 0 && lda % 8 == 0 && ldb % 8 == 0, MFQ_ERR_INVALID,
                 "gemm_f16_nt: K=%d, lda=%lld, ldb=%lld must be multiples of 32 / 8 / 8", K, (long long)lda, (long long)ldb);
-    const dim3 grid(static_cast<unsigned>(ceil_div(N, GBN)), static_cast<unsigned>(ceil_div(M, GBM)));
+    const int splits = part ? gemm_splits(M, N, K) : 1;
+    const int kps = static_cast<int>(ceil_div(K / GBK, splits));
+    const dim3 grid(static_cast<unsigned>(ceil_div(N, GBN)), static_cast<unsigned>(ceil_div(M, GBM)), static_cast<unsigned>(splits));
+    if (splits == 1) {
+        hipLaunchKernelGGL(gemm_f16_nt_kernel, grid, dim3(256), 0, st, static_cast<const uint16_t *>(a), lda,
+                           static_cast<const uint16_t *>(b), ldb, M, N, K, sa, sb, y, ldy, kps, static_cast<int64_t>(0));
+        return check_launch("gemm_f16_nt");
+    }
+    const int64_t ystride = static_cast<int64_t>(M) * N;
     hipLaunchKernelGGL(gemm_f16_nt_kernel, grid, dim3(256), 0, st, static_cast<const uint16_t *>(a), lda,
-                       static_cast<const uint16_t *>(b), ldb, M, N, K, sa, sb, y, ldy);
-    return check_launch("gemm_f16_nt");
+                       static_cast<const uint16_t *>(b), ldb, M, N, K, sa, sb, part, static_cast<int64_t>(N), kps, ystride);
+    if (int rc = check_launch("gemm_f16_nt")) return rc;
+    return prefill_sum_splits(part, ystride, splits, M, N, y, ldy, st);
 }
+// The split buffer of the call that dequant_gemm_carve(ws, N, K, M, ...) prepared: behind the row scales of the weights.
+float *dequant_gemm_part(float *wscale, int N, int K, int M);
 
 int x_prep_multi(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, int n_groups,
                  const int *gs, const int *nsteps, uint32_t *const *xg, hipStream_t st) {
@@ -338,8 +370,15 @@ int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *
 static size_t align256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 size_t dequant_gemm_workspace(int N, int K, int M) {
     const size_t Kp = static_cast<size_t>(ceil_div(K, GBK)) * GBK;
+    const int splits = gemm_splits(M, N, static_cast<int>(Kp));
     return align256(static_cast<size_t>(M) * Kp * 2) + align256(static_cast<size_t>(M) * 4) +
-           align256(static_cast<size_t>(N) * Kp * 2) + align256(static_cast<size_t>(N) * 4);
+           align256(static_cast<size_t>(N) * Kp * 2) + align256(static_cast<size_t>(N) * 4) +
+           (splits > 1 ? align256(static_cast<size_t>(splits) * M * N * 4) : 0);   // partial tiles of a split over K
+}
+float *dequant_gemm_part(float *wscale, int N, int K, int M) {
+    const int Kp = static_cast<int>(ceil_div(K, GBK)) * GBK;
+    if (gemm_splits(M, N, Kp) <= 1) return nullptr;
+    return reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(wscale) + align256(static_cast<size_t>(N) * 4));
 }
 void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&xscale, uint16_t *&w16, float *&wscale,
                         int &Kp) {
@@ -458,7 +497,7 @@ extern "C" int mfq_hip_nint_gemm(const mfq_nint_desc *d, const void *weight, con
     if (rc) return rc;
     rc = nint_dequant_f16(d, weight, w16, Kp, wscale, st);
     if (rc) return rc;
-    return gemm_f16_nt(x16, Kp, w16, Kp, M, d->out, Kp, xscale, wscale, y, ldy, st);
+    return gemm_f16_nt(x16, Kp, w16, Kp, M, d->out, Kp, xscale, wscale, y, ldy, st, dequant_gemm_part(wscale, d->out, d->neuron_len, M));
 }
 
 // The batch sizes at which mfq_hip_nint_gemm runs the block-tiled prefill kernel in one pass over K: only there does

@@ -10,7 +10,8 @@
 namespace mfq {
 
 int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, const float *sa,
-                const float *sb, float *y, int64_t ldy, hipStream_t st);
+                const float *sb, float *y, int64_t ldy, hipStream_t st, float *part = nullptr);
+float *dequant_gemm_part(float *wscale, int N, int K, int M);
 int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, hipStream_t st);
 size_t dequant_gemm_workspace(int N, int K, int M);
 void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&xscale, uint16_t *&w16, float *&wscale,
@@ -236,5 +237,5 @@ extern "C" int mfq_hip_mx_gemm_rows(int kind, const void *values, const void *sc
     else hipLaunchKernelGGL((mx_stage_f16_kernel<8>), dim3(nrows), dim3(256), 0, st, k, w16, Kp, wscale);
     rc = check_launch("mx_stage_f16");
     if (rc) return rc;
-    return gemm_f16_nt(x16, Kp, w16, Kp, M, nrows, Kp, xscale, wscale, y, ldy, st);
+    return gemm_f16_nt(x16, Kp, w16, Kp, M, nrows, Kp, xscale, wscale, y, ldy, st, dequant_gemm_part(wscale, nrows, cols, M));
 }

@@ -326,7 +326,8 @@ __global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *
 }
 
 int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, const float *sa,
-                const float *sb, float *y, int64_t ldy, hipStream_t st);
+                const float *sb, float *y, int64_t ldy, hipStream_t st, float *part = nullptr);
+float *dequant_gemm_part(float *wscale, int N, int K, int M);
 int x_prep(const void *x, int x_dtype, int64_t ldx, int M, int K, int Kp, void *x16, float *xscale, hipStream_t st);
 size_t dequant_gemm_workspace(int N, int K, int M);
 void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&xscale, uint16_t *&w16, float *&wscale,
@@ -584,7 +585,7 @@ extern "C" int mfq_hip_nvqs_gemm_rows(const mfq_nvqs_desc *d, const void *weight
                        dim3(256), 0, st, k, static_cast<const uint8_t *>(weight), w16, static_cast<int64_t>(Kp), wscale, Kp);
     rc = check_launch("nvqs_dequant_f16");
     if (rc) return rc;
-    return gemm_f16_nt(x16, Kp, w16, Kp, M, nrows, Kp, xscale, wscale, y, ldy, st);
+    return gemm_f16_nt(x16, Kp, w16, Kp, M, nrows, Kp, xscale, wscale, y, ldy, st, dequant_gemm_part(wscale, nrows, d->neuron_len, M));
 }
 
 extern "C" int mfq_hip_nvqs_gemm(const mfq_nvqs_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
