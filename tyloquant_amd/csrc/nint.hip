@@ -231,13 +231,26 @@ template <int XF16, int NB>
 static int launch_mfma_nb(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                           hipStream_t st) {
     const int64_t groups = ceil_div(k.n_rowblocks, NB);
-    int spw = static_cast<int>(ceil_div(k.nsteps, 8));
+    // Up to 16 waves per block (128 registers each) where the grid is small and K has nine to sixteen steps: a wave then
+    // walks one step instead of two, and a compute unit holds twice the waves to hide each other's waits (6144 x 4096
+    // at 16 rows: NINT3-24 9.8 -> 8.5 us, NINT5-28 13.5 -> 11.4 us).  Three row-blocks per wave do not fit 128 registers
+    // (NINT5-28 spills and loses 18 %), longer K gains nothing.  MFQ_MFMA_WIDE = 0 keeps eight waves.
+    static const int env_wide = tune_env("MFQ_MFMA_WIDE", 1);
+    const bool wide = env_wide && NB <= 2 && k.nsteps > 8 && k.nsteps <= 16 && groups * ceil_div(M, 16) <= 2 * gemv_cu_count();
+    int spw = static_cast<int>(ceil_div(k.nsteps, wide ? 16 : 8));
     while (spw < k.nsteps && groups * ceil_div(k.nsteps, spw) > 8192) ++spw;
     const int nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
     const size_t lds = static_cast<size_t>(nwaves) * NB * 1024;
     const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(ceil_div(M, 16))), block(64 * nwaves);
 #define MFQ_MFMA(UNIT, B, G)                                                                                   \
     if (k.bits == B && k.gs == G) {                                                                             \
+        if constexpr (NB <= 2) {                                                                                \
+            if (wide) {                                                                                         \
+                hipLaunchKernelGGL((nint_mfma_kernel<UNIT<B, G>, XF16, NB, 16>), grid, block, lds, st, k, w, x, ldx, M, y, \
+                                   ldy, spw);                                                                   \
+                return check_launch("nint_mfma");                                                               \
+            }                                                                                                   \
+        }                                                                                                       \
         hipLaunchKernelGGL((nint_mfma_kernel<UNIT<B, G>, XF16, NB>), grid, block, lds, st, k, w, x, ldx, M, y, ldy, \
                            spw);                                                                                \
         return check_launch("nint_mfma");                                                                       \

@@ -229,8 +229,8 @@ __device__ __forceinline__ void nint_mfma_body(const NintK &k, const uint8_t *__
 }
 
 // Dense wrapper: block (row-block group, 16-token tile).
-template <class U, int XF16, int NB>
-__global__ __launch_bounds__(512) void nint_mfma_kernel(NintK k, const uint8_t *__restrict__ w,
+template <class U, int XF16, int NB, int MAXW = 8>
+__global__ __launch_bounds__(64 * MAXW) void nint_mfma_kernel(NintK k, const uint8_t *__restrict__ w,
                                                          const uint16_t *__restrict__ x, int64_t ldx, int M,
                                                          float *__restrict__ y, int64_t ldy, int spw) {
     extern __shared__ uint32_t lds[];
