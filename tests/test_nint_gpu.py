@@ -357,7 +357,7 @@ def test_nint8_zero_dequant_bit_exact_and_matmul(out, K):
 
 @pytest.mark.parametrize("cus,out,K", [(4, 200, 1056), (3, 96, 4096), (2, 40, 96), (64, 33, 2048)])
 def test_nint8_zero_tile_kernel_row_blocks_per_block(cu_count, cus, out, K):
-    """3 .. 32 rows on the matrix cores: a block owns ceil(row-blocks / CUs) row-blocks, up to four (4, 2, 2 and 1 here),
+    """2 .. 32 rows on the matrix cores: a block owns ceil(row-blocks / CUs) row-blocks, up to four (4, 2, 2 and 1 here),
     the last block fewer; one and two 16-row tiles; K with a partial last chunk of eight blocks (1056 = 33 blocks, 96 = 3);
     a row stride above K; rows that are not 16-byte aligned fall back to the vector-ALU kernel."""
     from tyloquant_amd import runtime as R
@@ -366,7 +366,7 @@ def test_nint8_zero_tile_kernel_row_blocks_per_block(cu_count, cus, out, K):
     lin = R.load_quant_linear("NINT8-0", O.pack_nint8_zero(t))
     deq = O.dequantize_nint8_zero(t)
     cu_count(cus)
-    for M in (3, 9, 16, 21, 32):
+    for M in (2, 9, 16, 21, 32):
         for xd in (torch.bfloat16, torch.float16):
             xw = torch.from_numpy(rng.standard_normal((M, K + 8)).astype(np.float32)).to(xd).cuda()
             x = xw[:, :K]

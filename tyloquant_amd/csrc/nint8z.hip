@@ -166,7 +166,7 @@ __global__ __launch_bounds__(256) void nint8z_gemv_kernel(N8zK k, const uint8_t 
     }
 }
 
-// ---- 3 .. 32 rows on the matrix cores ------------------------------------------------------------------------------
+// ---- 2 .. 32 rows on the matrix cores ------------------------------------------------------------------------------
 // One MFMA (16 tokens x 16 neurons x 32 k) covers exactly one Q8_0 block of each of its 16 neurons: the codes enter as
 // exact fp16 integers (byte -> mantissa of 1024, minus 1152), the product sum of the block comes out of an accumulator
 // that starts at zero, and the block's scale multiplies it in fp32 -- the arithmetic of the reference's
@@ -364,9 +364,10 @@ static int nint8z_gemv_any(const mfq_nint8z_desc *d, const void *weight, const v
     const N8zK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
-    // from three rows on: the matrix cores, where the activation rows allow 16-byte reads (two rows still run faster on
-    // the vector ALUs: 16.3 against 17.7 us on 12288 x 4096; MFQ_N8Z_TILE_MIN_M for tuning)
-    static const int tile_min = tune_env("MFQ_N8Z_TILE_MIN_M", 3);
+    // from two rows on: the matrix cores, where the activation rows allow 16-byte reads.  Two rows on the vector ALUs
+    // take 8.8 / 16.7 / 29.6 us on 4096 x 4096 / 12288 x 4096 / 4096 x 12288 against 7.6 / 17.7 / 17.8 us here
+    // (MFQ_N8Z_TILE_MIN_M for tuning)
+    static const int tile_min = tune_env("MFQ_N8Z_TILE_MIN_M", 2);
     if (M >= tile_min && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && k.neuron_len % 8 == 0)
         return x_dtype == MFQ_X_F16 ? nint8z_tile_launch<1>(k, w, xp, ldx, M, y, ldy, st)
                                     : nint8z_tile_launch<0>(k, w, xp, ldx, M, y, ldy, st);

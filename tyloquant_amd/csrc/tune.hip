@@ -34,7 +34,7 @@ Knob g_knobs[] = {
     {"MFQ_NVQ_SIGNED_MAX_M", "rows up to which the NVQ signed-table kernel runs", 0, false},
     {"MFQ_NVQ_RING", "weight ring depth of the five-row-block NVQ kernel", 0, false},
     {"MFQ_NEPQ_NB", "row-blocks per wave of the NEPQ streaming kernel (0 = by shape)", 0, false},
-    {"MFQ_N8Z_TILE_MIN_M", "rows from which NINT8-0 small batches run on the matrix cores (default 3)", 0, false},
+    {"MFQ_N8Z_TILE_MIN_M", "rows from which NINT8-0 small batches run on the matrix cores (default 2)", 0, false},
     {"MFQ_NEPQ_TILE_OFF", "1 = NEPQ small batches on the older streaming kernel", 0, false},
     {"MFQ_NEPQ_RPB", "row-blocks per block of the one-row NEPQ GEMV (0 = by shape)", 0, false},
     {"MFQ_NEPQ_VALU_MAX_M", "rows up to which NEPQ runs on the vector-ALU GEMV before the streaming MFMA kernel", 0, false},
