@@ -170,6 +170,7 @@ void gemv_shape(const NintK &k, int mb, int &spw, int &nwaves, int &rbw, size_t 
     lds_bytes = gemv_lds_bytes(mb, spw, k.gs, nwaves, rbw);
 }
 
+#define MFQ_SINGLE_ARG(...) __VA_ARGS__
 template <int XF16, int MB>
 static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                           hipStream_t st) {
@@ -186,8 +187,24 @@ static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, i
         if (int rc_ = allow_dynamic_lds(reinterpret_cast<const void *>(kern_), lds, "nint_gemv")) return rc_; \
         hipLaunchKernelGGL(kern_, GRID, block, lds, st, __VA_ARGS__);                                        \
     } while (0)
+    // Waves with at most three items keep the staged activations in registers when a group's pairs fit one row of
+    // lanes and the rows can be fetched pair by pair (4-byte aligned rows, even K): LDS then only holds the sums.
+    static const int env_xreg = tune_env("MFQ_GEMV_XREG", 1);
+    const bool xreg_rows = MB <= 2 && spw * rbw <= 3 && k.neuron_len % 2 == 0 && ldx % 2 == 0 &&
+                           (reinterpret_cast<uintptr_t>(x) & 3) == 0 && env_xreg != 0;
+    const size_t lds_xreg = static_cast<size_t>(rbw) * nwaves * MB * 16 * 4;
+#define MFQ_XREG(UNIT)                                                                                         \
+    if constexpr ((MB == 1 || (MB == 2 && UNIT::CBITS != 0)) && UNIT::NPAIR <= 16) { /* two rows of NINT5-28 spill */ \
+        if (xreg_rows) {                                                                                       \
+            const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, rbw)), static_cast<unsigned>(ceil_div(M, MB))); \
+            hipLaunchKernelGGL((nint_gemv_xreg_kernel<UNIT, XF16, MB>), grid, block, lds_xreg, st, k, w, x, ldx, M, y, ldy, \
+                               spw, rbw);                                                                      \
+            return check_launch("nint_gemv_xreg");                                                             \
+        }                                                                                                      \
+    }
 #define MFQ_PAIRED(B, G)                                                                                     \
     if (k.bits == B && k.gs == G) {                                                                          \
+        MFQ_XREG(MFQ_SINGLE_ARG(PairedUnit<B, G>))                                                           \
         const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, rbw)), static_cast<unsigned>(ceil_div(M, MB))); \
         if (spw * rbw <= 3)                                                                                  \
             MFQ_GEMV_LAUNCH((nint_gemv_paired_kernel<B, G, XF16, MB, false>), grid, k, w, x, ldx, M, y, ldy, spw, rbw); \
@@ -202,6 +219,7 @@ static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, i
     }
 #undef MFQ_PAIRED
     if (mfma_generic_profile(k)) {
+        MFQ_XREG(MFQ_SINGLE_ARG(GenericUnit<5, 28>))
         const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, rbw)), static_cast<unsigned>(ceil_div(M, MB)));
         if (spw * rbw <= 3)
             MFQ_GEMV_LAUNCH((nint_gemv_natural_kernel<5, 28, XF16, MB, false>), grid, k, w, x, ldx, M, y, ldy, spw, rbw);

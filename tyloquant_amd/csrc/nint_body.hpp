@@ -96,6 +96,10 @@ struct PairedUnit {
         __device__ static __forceinline__ float inv_xscale(int i) {
             return __uint_as_float(0x3f800000u + (static_cast<uint32_t>(BITS * cls(i)) << 23));
         }
+        // the scale of pair i of a group, whatever its position in a chunk
+        __device__ static __forceinline__ float pair_scale(int i) {
+            return __uint_as_float(0x3f800000u - (static_cast<uint32_t>(BITS * cls(i)) << 23));
+        }
     };
 
     // v[i] = fp16 pair (1024 + 2^o * code_2i, 1024 + 2^o * code_2i+1) of pair i of the group, o = BITS * cls(i)
@@ -187,6 +191,7 @@ struct GenericUnit {
         __device__ static __forceinline__ float bw(int) { return 1024.f; }
         __device__ static __forceinline__ float xscale(int, int) { return 1.f; }
         __device__ static __forceinline__ float inv_xscale(int) { return 1.f; }
+        __device__ static __forceinline__ float pair_scale(int) { return 1.f; }
     };
     __device__ static __forceinline__ uint32_t code(const uint32_t (&q)[D], int i) {
         const int bit = i * BITS, wi = bit >> 5, sh = bit & 31;
@@ -305,6 +310,111 @@ __device__ __forceinline__ void nint_compute_step(const uint32_t (&q)[4][U::D], 
     }
 }
 
+// ---- activations in registers ----------------------------------------------------------------------------------
+// For the batch-1 kernels without a ring the staged activations never touch LDS.  A unit is the group of lane (r, kb);
+// the 16 lanes of a DPP row (same kb) all need the same GS/2 activation pairs, so lane r of the row keeps pair r of the
+// row's group in one register and every dot product fetches its pair with a row broadcast
+// (v_dot2c_f32_f16_dpp ... row_newbcast:i).  Per item a lane holds, for each unit j, the pair register, X_g and -T_g.
+template <int MB>
+struct XItem {
+    uint32_t x[MB][4];   // staged fp16 pair r of group (step, j, kb), times the pair's class scale
+    float xg[MB][4];     // X_g of that group (every lane of the row holds the row's total)
+    float nt[MB][4];     // -T_g
+};
+
+// acc += dot(x pair I + t of the row, w[t]) for t = 0..3; one statement, so that nothing is scheduled between them.
+// On this target the result of a dot instruction may feed the accumulator of the same instruction at once, but any
+// other reader has to stay three issue slots behind it, and the compiler cannot see into the statement: LAST appends
+// those slots, and the caller sets it on the block whose result is read next.
+template <int I, bool LAST>
+__device__ __forceinline__ float dot2_bcast4(float acc, uint32_t x, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+    if constexpr (LAST)
+        asm("v_dot2c_f32_f16_dpp %0, %1, %2 row_newbcast:%6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_dot2c_f32_f16_dpp %0, %1, %3 row_newbcast:%7 row_mask:0xf bank_mask:0xf\n\t"
+            "v_dot2c_f32_f16_dpp %0, %1, %4 row_newbcast:%8 row_mask:0xf bank_mask:0xf\n\t"
+            "v_dot2c_f32_f16_dpp %0, %1, %5 row_newbcast:%9 row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 2"
+            : "+v"(acc)
+            : "v"(x), "v"(w0), "v"(w1), "v"(w2), "v"(w3), "n"(I), "n"(I + 1), "n"(I + 2), "n"(I + 3));
+    else
+        asm("v_dot2c_f32_f16_dpp %0, %1, %2 row_newbcast:%6 row_mask:0xf bank_mask:0xf\n\t"
+            "v_dot2c_f32_f16_dpp %0, %1, %3 row_newbcast:%7 row_mask:0xf bank_mask:0xf\n\t"
+            "v_dot2c_f32_f16_dpp %0, %1, %4 row_newbcast:%8 row_mask:0xf bank_mask:0xf\n\t"
+            "v_dot2c_f32_f16_dpp %0, %1, %5 row_newbcast:%9 row_mask:0xf bank_mask:0xf"
+            : "+v"(acc)
+            : "v"(x), "v"(w0), "v"(w1), "v"(w2), "v"(w3), "n"(I), "n"(I + 1), "n"(I + 2), "n"(I + 3));
+    return acc;
+}
+
+// sum over the 16 lanes of a DPP row, left in every lane of the row
+__device__ __forceinline__ float row_allsum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xF, 0xF, true));  // row_ror:8
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xF, 0xF, true));  // row_ror:4
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xF, 0xF, true));  // row_ror:2
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xF, 0xF, true));  // row_ror:1
+    return v;
+}
+
+template <class U, int MB>
+__device__ __forceinline__ void nint_compute_step_xreg(const uint32_t (&q)[4][U::D], uint32_t tails, u32x2_t sc,
+                                                       const XItem<MB> &xi, float (&accS)[MB], float (&accM)[MB]) {
+    constexpr int NP = U::NPAIR;
+    static_assert(NP % 4 == 0 && NP <= 16, "a row of 16 lanes holds the pairs of one group");
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t scw = (j < 2) ? sc.x : sc.y;
+        const float ss = ubyte_f32(scw, 2 * (j & 1)), sm = ubyte_f32(scw, 2 * (j & 1) + 1);
+        uint32_t v[NP];
+        U::unpack(q[j], (tails >> (8 * j)) & 0xffu, v);
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            float a = xi.nt[m][j];
+            a = dot2_bcast4<0, NP == 4>(a, xi.x[m][j], v[0], v[1], v[2], v[3]);
+            if constexpr (NP > 4) a = dot2_bcast4<4, NP == 8>(a, xi.x[m][j], v[4], v[5], v[6], v[7]);
+            if constexpr (NP > 8) a = dot2_bcast4<8, NP == 12>(a, xi.x[m][j], v[8], v[9], v[10], v[11]);
+            if constexpr (NP > 12) a = dot2_bcast4<12, true>(a, xi.x[m][j], v[12], v[13], v[14], v[15]);
+            accS[m] = fmaf(ss, a, accS[m]);
+            accM[m] = fmaf(sm, xi.xg[m][j], accM[m]);
+        }
+    }
+}
+
+// Requests the raw activation pairs of one item (K step `step`): lane (r, kb) asks for pair r of group 16 step + 4 j + kb
+// of every row through the row's range-checked window (lanes beyond the group's pairs and pairs beyond K read zeros).
+template <class U, int MB>
+__device__ __forceinline__ void xreg_issue(const __amdgpu_buffer_rsrc_t (&wx)[MB], int step, bool live, int lane,
+                                           uint32_t (&raw)[MB][4]) {
+    constexpr int P = U::GROUP / 2;
+    const int r = lane & 15, kb = lane >> 4;
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t off = (static_cast<uint32_t>((step * 16 + 4 * j + kb) * P + r)) * 4u;
+            raw[m][j] = __builtin_amdgcn_raw_buffer_load_b32(wx[m], (live && r < P) ? off : kNoStep, 0, 0);
+        }
+}
+
+// Converts what xreg_issue fetched: fp16 pairs times sc[m] (the wave's power of two for the row) and the pair's class
+// scale, and the two group sums, spread over each row of lanes.
+template <class U, int XF16, int MB>
+__device__ __forceinline__ void xreg_stage(const uint32_t (&raw)[MB][4], const float (&sc)[MB], int lane, XItem<MB> &xi) {
+    const int r = lane & 15;
+    const float cs = U::Bias::pair_scale(r), ci = U::Bias::inv_xscale(r);
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t h;
+            if constexpr (XF16) h = scale_h2(raw[m][j], cs);
+            else h = to_h2_scaled(raw[m][j], sc[m] * cs);
+            xi.x[m][j] = h;
+            const float ps = dot2h(h, 0x3c003c00u, 0.f);
+            xi.xg[m][j] = row_allsum(ps * ci);
+            xi.nt[m][j] = -row_allsum(ps * U::Bias::bw(r));
+        }
+}
+
 // One block = `rbw` consecutive 16-neuron row-blocks starting at `rb0` of the tensor at `w`; its waves
 // split the K steps, `spw` steps per wave, and every wave walks through its K-slice of each row-block
 // in turn, so the slice of the activations is staged once for all of them.  xr / yr name the MB
@@ -327,7 +437,10 @@ __device__ __forceinline__ int gemv_red_offset(int nwaves, int mb, int spw, int 
 __device__ long long *mfq_trace_ptr;
 // the readings stay in registers until the wave is done, so that no store sits among the loads being timed
 #define MFQ_TRACE_DECL long long trace_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#define MFQ_TRACE(slot) trace_t[slot] = __builtin_readcyclecounter()
+#ifndef MFQ_TRACE_CLOCK
+#define MFQ_TRACE_CLOCK() __builtin_readcyclecounter()
+#endif
+#define MFQ_TRACE(slot) trace_t[slot] = MFQ_TRACE_CLOCK()
 #define MFQ_TRACE_FLUSH                                                                                             \
     do {                                                                                                            \
         if (mfq_trace_ptr && lane == 0)                                                                             \
@@ -386,7 +499,13 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     uint32_t q0[4][D], q1[4][D], q2[4][D], t0, t1, t2;
     u32x2_t c0, c1, c2;
     MFQ_ISSUE(q0, t0, c0)
+#ifdef MFQ_GEMV_RR
+    if constexpr (!RING) { asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
+#endif
     MFQ_ISSUE(q1, t1, c1)
+#ifdef MFQ_GEMV_RR
+    if constexpr (!RING) { asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
+#endif
     MFQ_ISSUE(q2, t2, c2)
     float xinv[MB];  // bf16 rows are staged times a per-wave power of two; the sums are scaled back when they are parked
     xp.template finish<XF16, MB>(xg);
@@ -399,7 +518,7 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     int crb = 0, cs = 0;
 #define MFQ_COMPUTE(Q, T, C)                                                                              \
     {                                                                                                     \
-        nint_compute_step<U, MB>(Q, T, C, cs * 16 + kb, xs, xsum, npairs, ngl, accS, accM);                 \
+        MFQ_LAB_COMPUTE(Q, T, C)                                                                          \
         if (++cs >= n) {                                                                                  \
             float a_s = ns[0], a_m = nm[0];                                                               \
             _Pragma("unroll") for (int i = 1; i < kMaxRbw; ++i) if (crb == i) { a_s = ns[i]; a_m = nm[i]; } \
@@ -413,6 +532,16 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
             ++crb;                                                                                        \
         }                                                                                                 \
     }
+#ifdef MFQ_LAB_NOCOMPUTE
+#define MFQ_LAB_COMPUTE(Q, T, C)                                                                       \
+    {                                                                                                  \
+        uint32_t a_ = T ^ C.x ^ C.y;                                                                   \
+        _Pragma("unroll") for (int j_ = 0; j_ < 4; ++j_) _Pragma("unroll") for (int d_ = 0; d_ < D; ++d_) a_ ^= Q[j_][d_]; \
+        accS[0] += __uint_as_float(a_ & 0x3fffffffu);                                                  \
+    }
+#else
+#define MFQ_LAB_COMPUTE(Q, T, C) nint_compute_step<U, MB>(Q, T, C, cs * 16 + kb, xs, xsum, npairs, ngl, accS, accM);
+#endif
     const int items = nrb * n;
     if (n <= 0) {  // a wave beyond the last step still owes its (zero) partial sums
         float z[MB];
@@ -444,6 +573,114 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     }
 #undef MFQ_ISSUE
 #undef MFQ_COMPUTE
+    if constexpr (FLUSH) flush_rows<MB>(red, nwaves, nrb, rb0, row_base, out_rows, yr);
+    MFQ_TRACE(5);
+    MFQ_TRACE_FLUSH;
+}
+
+// The same block decomposition for waves with at most three items and activations in registers (see XItem): no LDS
+// in the walk, the only shared memory is the cross-wave reduction area at the start of `lds`.  Needs rows that are
+// 4-byte aligned and an even K (the caller checks); K need not be a multiple of the group size.
+template <class U, int XF16, int MB, bool FLUSH = true>
+__device__ __forceinline__ void nint_unit_body_xreg(const NintK &k, const uint8_t *__restrict__ w, int rb0, int rbw,
+                                                    int row_base, int out_rows, const uint16_t *const (&xr)[MB],
+                                                    float *const (&yr)[MB], int spw, uint32_t *lds, int rb_step = 1) {
+    constexpr int D = U::D;
+    const int lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+    const int r = lane & 15;
+    const int s0 = wave * spw;
+    const int n = min(k.nsteps, s0 + spw) - s0;                         // steps of this wave in each row-block
+    const int nrb = min(rbw, (k.n_rowblocks - 1 - rb0) / rb_step + 1);  // row-blocks of this block
+    float *red = reinterpret_cast<float *>(lds);
+    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes) * rb_step;
+    const int items = n > 0 ? nrb * n : 0;  // <= 3
+
+    MFQ_TRACE_DECL
+    MFQ_TRACE(0);
+    // item t = (row-block t / n, step t % n); requests in order of use: activations, anchors, weights
+    __amdgpu_buffer_rsrc_t wx[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+        wx[m] = wave_window(reinterpret_cast<const uint8_t *>(xr[m]), xr[m] ? static_cast<uint32_t>(k.neuron_len) * 2u : 0u);
+    int irb_[3], is_[3];
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+        irb_[t] = n > 0 ? t / n : 0;
+        is_[t] = t - irb_[t] * n;
+    }
+    // activations are requested and staged once per step: set u = step u of the wave (item t reads set t % n)
+    uint32_t raw[3][MB][4];
+#pragma unroll
+    for (int u = 0; u < 3; ++u) xreg_issue<U, MB>(wx, s0 + u, u < n, lane, raw[u]);
+    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
+    float ns[3], nm[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        const int rb = min(rb0 + i * rb_step, k.n_rowblocks - 1);
+        ns[i] = anchors[rb * 16 + r];
+        nm[i] = anchors[16 * k.n_rowblocks + rb * 16 + r];
+    }
+    const __amdgpu_buffer_rsrc_t win =
+        wave_window(w + static_cast<int64_t>(rb0) * k.rowblock_bytes + static_cast<int64_t>(s0) * sb,
+                    n > 0 ? (nrb - 1) * rbb + n * sb : 0u);
+    uint32_t q[3][4][D], tl[3];
+    u32x2_t sc[3];
+#pragma unroll
+    for (int t = 0; t < 3; ++t)
+        nint_load_step<D, U::TAIL>(win, t < items ? irb_[t] * rbb + is_[t] * sb : kNoStep, lane, q[t], tl[t], sc[t]);
+
+    // bf16 rows: one power of two per wave and row brings the slice near 2^12
+    float xs_[MB], xinv[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        xs_[m] = xinv[m] = 1.f;
+        if constexpr (!XF16) {
+            uint32_t mx = 0;
+#pragma unroll
+            for (int t = 0; t < 3; ++t)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) mx = absmax_bf16(mx, raw[t][m][j]);
+            xs_[m] = slice_scale(wave_max_u32(mx), xinv[m]);
+        }
+    }
+    MFQ_TRACE(1);
+    float accS[MB], accM[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) accS[m] = accM[m] = 0.f;
+    if (items <= 0) {  // a wave beyond the last step still owes its (zero) partial sums
+        float z[MB];
+        for (int i = 0; i < nrb; ++i) {
+#pragma unroll
+            for (int m = 0; m < MB; ++m) z[m] = 0.f;
+            park_rows<MB>(z, red, i * nwaves + wave, lane);
+        }
+    } else {
+        // a wave with one step walks row-blocks with the same staged set; with two or three steps item t is step t
+        XItem<MB> xi;
+        xreg_stage<U, XF16, MB>(raw[0], xs_, lane, xi);
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
+            if (t < items) {
+                if (t > 0 && n > 1) xreg_stage<U, XF16, MB>(raw[t], xs_, lane, xi);
+                nint_compute_step_xreg<U, MB>(q[t], tl[t], sc[t], xi, accS, accM);
+                if (is_[t] == n - 1) {
+                    float a_s = ns[0], a_m = nm[0];
+#pragma unroll
+                    for (int i = 1; i < 3; ++i)
+                        if (irb_[t] == i) { a_s = ns[i]; a_m = nm[i]; }
+                    float v[MB];
+#pragma unroll
+                    for (int m = 0; m < MB; ++m) {
+                        v[m] = (a_s * accS[m] - a_m * accM[m]) * xinv[m];
+                        accS[m] = accM[m] = 0.f;
+                    }
+                    park_rows<MB>(v, red, irb_[t] * nwaves + wave, lane);
+                }
+            }
+            MFQ_TRACE(2 + t);
+        }
+    }
     if constexpr (FLUSH) flush_rows<MB>(red, nwaves, nrb, rb0, row_base, out_rows, yr);
     MFQ_TRACE(5);
     MFQ_TRACE_FLUSH;
@@ -527,6 +764,18 @@ __global__ __launch_bounds__(1024) void nint_gemv_paired_kernel(NintK k, const u
     float *yr[MB];
     dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
     nint_paired_body<BITS, GS, XF16, MB, RING>(k, w, blockIdx.x * rbw, rbw, 0, k.out, xr, yr, spw, lds);
+}
+
+// the same for waves with at most three items: activations in registers, LDS only for the cross-wave sums
+template <class U, int XF16, int MB>
+__global__ __launch_bounds__(1024) void nint_gemv_xreg_kernel(NintK k, const uint8_t *__restrict__ w,
+                                                              const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                              float *__restrict__ y, int64_t ldy, int spw, int rbw) {
+    extern __shared__ uint32_t lds[];
+    const uint16_t *xr[MB];
+    float *yr[MB];
+    dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
+    nint_unit_body_xreg<U, XF16, MB>(k, w, blockIdx.x * rbw, rbw, 0, k.out, xr, yr, spw, lds);
 }
 
 // natural-order profiles with a unit of their own
