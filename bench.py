@@ -114,44 +114,64 @@ def main() -> int:
     def stream_ptr():
         return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
-    # one HIP graph = one pass over all weight sets (copies x 3 kernels): decode runs under graphs
+    # Decode runs under HIP graphs.  One graph = one pass over all weight sets; a second, shorter graph covers the
+    # steps left over when --steps is not a multiple of the number of sets, so that a timed window of exactly
+    # --steps steps is graph replays only.
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         launch(sets[0], stream_ptr())
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        for s in sets:
-            launch(s, stream_ptr())
     per_replay = len(sets)
+    full, rest = divmod(args.steps, per_replay)
+
+    def capture(nsets):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for s_ in sets[:nsets]:
+                launch(s_, stream_ptr())
+        return g
+    graph = capture(per_replay)
+    graph_rest = capture(rest) if rest else None
 
     def run_steps(nsteps):
-        full, rest = divmod(nsteps, per_replay)
-        for _ in range(full):
+        f, r = divmod(nsteps, per_replay)
+        for _ in range(f):
             graph.replay()
-        for i in range(rest):
-            launch(sets[i], stream_ptr())
+        if r == rest and graph_rest is not None:
+            graph_rest.replay()
+        else:
+            for i in range(r):
+                launch(sets[i], stream_ptr())
 
     run_steps(args.warmup)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t_start = time.perf_counter()
-    e0.record()
-    run_steps(args.steps)
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t_start
-    gpu_ms = e0.elapsed_time(e1)
+    # Timed region: `windows` windows of exactly --steps steps each, every window bracketed by a device synchronisation
+    # on both sides (wall clock) and by HIP events on the launch stream; the line reports the median window.
+    windows = max(5, -(-200 // max(1, args.steps * n_per_step)))
+    walls, gpus = [], []
+    for _ in range(windows):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t_start = time.perf_counter()
+        e0.record()
+        run_steps(args.steps)
+        e1.record()
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - t_start)
+        gpus.append(e0.elapsed_time(e1))
+    wall = float(np.median(walls))
+    gpu_ms = float(np.median(gpus))
     ms_per_step = wall * 1e3 / args.steps
     value = step_bytes * args.steps / wall / 1e9
     n_launch = n_per_step * args.steps
     avg_launch_us = gpu_ms * 1e3 / n_launch
     bytes_per_launch = step_bytes / float(n_per_step)
     achieved = bytes_per_launch / (avg_launch_us * 1e-6) / 1e9
-    log(f"[bench] decode C2 M=1: {value:.1f} GB/s whole-job, {avg_launch_us:.2f} us/launch by HIP events "
-        f"-> {achieved:.1f} GB/s per launch")
+    log(f"[bench] decode C2 M=1: {value:.1f} GB/s whole-job (median of {windows} windows of {args.steps} steps; "
+        f"min {step_bytes * args.steps / max(walls) / 1e9:.0f}, max {step_bytes * args.steps / min(walls) / 1e9:.0f}), "
+        f"{avg_launch_us:.2f} us/launch by HIP events -> {achieved:.1f} GB/s per launch")
 
     # parity guard on what was just timed (size-independent property: linearity in x)
     launch(sets[0], stream_ptr())
@@ -162,7 +182,55 @@ def main() -> int:
     lin_err = float(((yy - 2 * y1).norm() / (2 * y1).norm()).item())
     assert lin_err < 1e-5, f"GEMV is not linear in x / copies differ: {lin_err}"
 
-    extras = {"linearity_rel_err": lin_err, "gpu_ms_total": gpu_ms}
+    extras = {"linearity_rel_err": lin_err, "gpu_ms_median_window": gpu_ms, "windows": windows,
+              "value_min_gbps": step_bytes * args.steps / max(walls) / 1e9,
+              "value_max_gbps": step_bytes * args.steps / min(walls) / 1e9,
+              "launch_us_min_window": min(gpus) * 1e3 / n_launch, "launch_us_max_window": max(gpus) * 1e3 / n_launch}
+
+    # What the memory system gives a read-only launch, measured in this run: one kernel that only reads, (a) 1 GiB in
+    # one launch (the streaming ceiling), (b) buffers of the two GEMV launches' sizes, rotating over 8 copies in a graph
+    # exactly like the timed steps (start-up and drain of a launch of that size included).
+    def read_probe_gbps(nbytes, ncopies, reps):
+        bufs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(ncopies)]
+        sink = torch.zeros(16, dtype=torch.int32, device=dev)
+
+        def go():
+            for b in bufs:
+                rc = lib.mfq_hip_read_probe(b.data_ptr(), nbytes, sink.data_ptr(), stream_ptr())
+                if rc:
+                    L.check(rc)
+        s2 = torch.cuda.Stream()
+        s2.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s2):
+            go()
+        torch.cuda.current_stream().wait_stream(s2)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            go()
+        g.replay()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(5):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                g.replay()
+            b.record()
+            torch.cuda.synchronize()
+            ts.append(a.elapsed_time(b) / (reps * ncopies))
+        del bufs
+        return nbytes / (float(np.median(ts)) * 1e-3) / 1e9, float(np.median(ts)) * 1e3
+    extras["hbm_read_ceiling_gbps"], _ = read_probe_gbps(1 << 30, 2, 3)
+    for n in launches:
+        gb, us = read_probe_gbps(int(base[n][0].desc.total_bytes), 8, 10)
+        extras[f"read_only_{n}_gbps"], extras[f"read_only_{n}_us"] = gb, us
+    ro_us = 0.5 * (extras["read_only_gate_up_us"] + extras["read_only_down_us"])
+    extras["launch_us_vs_read_only_launch"] = avg_launch_us / ro_us
+    log(f"[bench] read-only kernel: 1 GiB {extras['hbm_read_ceiling_gbps']:.0f} GB/s; gate_up-sized "
+        f"{extras['read_only_gate_up_us']:.2f} us, down-sized {extras['read_only_down_us']:.2f} us per launch "
+        f"(GEMV launches take {extras['launch_us_vs_read_only_launch']:.2f}x that)")
+    torch.cuda.empty_cache()
     if args.calibrate:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)

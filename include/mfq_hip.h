@@ -46,6 +46,15 @@ int mfq_hip_version(void);
  * next to their numbers.  Thread-local buffer.  No counterpart in the reference, whose MFQ_* overrides are read where
  * they are used (e.g. cpp_runtime/mfq_decode.cpp:8518-8523). */
 const char *mfq_hip_config(void);
+/* Measurement aid: one launch that only reads `bytes` bytes at `data` (16-byte aligned; every wave requests a
+ * contiguous share with 16-byte loads, as the decode kernels do) and stores nothing but a 4-byte checksum word at
+ * `sink` when it happens to match a magic value.  Benchmarks time it next to the GEMVs: what it sustains is what the
+ * memory system gives a launch of that size, start-up and drain included.  No counterpart in the reference. */
+int mfq_hip_read_probe(const void *data, size_t bytes, void *sink, mfq_stream_t stream);
+/* Clears `bytes` bytes at `data` (4-byte aligned, a multiple of 4) with a kernel.  For hosts that must not record a
+ * memset node into a captured graph; stands in for the zero-initialised outputs of the reference's host code
+ * (torch::zeros, e.g. cpp_runtime/mfq_decode.cpp:2998). */
+int mfq_hip_fill_zero(void *data, size_t bytes, mfq_stream_t stream);
 /* Test and tuning hook: size one-block-per-CU grids for n compute units instead of the device's own count
  * (n <= 0 restores it).  Process-wide; not for production use. */
 void mfq_hip_set_cu_count(int n);

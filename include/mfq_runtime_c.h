@@ -72,6 +72,21 @@ int mfq_rt_moe_ffn_forward(void *gate_up, void *down, const void *x, int x_dtype
                            const float *router_logits, int top_k, int topk_mode, int normalize,
                            void *shared_gate_up, void *shared_down, float *out, int32_t *ids_out,
                            float *weights_out, void *stream);
+/* The same with the intermediates in a caller-owned scratch object (MoeFfnScratch): after mfq_rt_moe_scratch_reserve
+ * for the largest call, mfq_rt_moe_ffn_forward_scratch neither allocates nor waits for the device, so it may be recorded
+ * into a HIP graph (the reference's plan / forward allocate nothing under capture either,
+ * cpp_runtime/mfq_decode.cpp:2681-2708, 3008-3016).  The selected experts and their weights of the last call stay in
+ * the scratch: mfq_rt_moe_scratch_topk returns their device addresses (int32 / fp32 [T, top_k]).
+ * mfq_rt_moe_ffn_forward above is the convenience form: it builds and frees a scratch of its own per call and
+ * therefore waits for the stream before it returns. */
+int mfq_rt_moe_scratch_create(void **scratch);
+void mfq_rt_moe_scratch_free(void *scratch);
+int mfq_rt_moe_scratch_reserve(void *scratch, void *gate_up, void *down, int max_tokens, int top_k,
+                               void *shared_gate_up, void *shared_down);
+int mfq_rt_moe_scratch_topk(void *scratch, const int32_t **ids, const float **weights);
+int mfq_rt_moe_ffn_forward_scratch(void *scratch, void *gate_up, void *down, const void *x, int x_dtype, int64_t ldx,
+                                   int T, const float *router_logits, int top_k, int topk_mode, int normalize,
+                                   void *shared_gate_up, void *shared_down, float *out, void *stream);
 
 /* Expert residency (MoeExpertCache, cpp_runtime/mfq_decode.cpp:5941-7500): experts of the registered NINTM tensors stay
  * in pinned host memory, the GPU holds budget_bytes worth of expert slots; forward makes the route's experts resident

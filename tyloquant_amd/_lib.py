@@ -65,6 +65,8 @@ _SIGS = {
     "mfq_hip_version": (C.c_int, []),
     "mfq_hip_config": (C.c_char_p, []),
     "mfq_hip_set_cu_count": (None, [C.c_int]),
+    "mfq_hip_read_probe": (C.c_int, [vp, sz, vp, vp]),
+    "mfq_hip_fill_zero": (C.c_int, [vp, sz, vp]),
     "mfq_hip_moe_decode_capable": (C.c_int, [C.POINTER(MoePool), C.c_int, C.c_int, C.c_int, C.POINTER(NintDesc), C.c_int,
                                              C.c_int, C.c_int]),
     "mfq_hip_nint_plan": (C.c_int, [C.c_int] * 5 + [C.POINTER(NintDesc)]),

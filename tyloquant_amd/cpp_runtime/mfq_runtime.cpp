@@ -663,14 +663,15 @@ void nvq_matmul_multi2(const NvqWeight &first, const NvqWeight &second, const vo
     if (first.neuron_len() != second.neuron_len()) fail("NVQ multi-projection requires compatible formats and input layouts");
     const int64_t N = first.out() + second.out();
     if (first.streams || second.streams) {  // no joint launch for tensors read from their streams: each into its columns
-        DeviceBuffer tmp(static_cast<size_t>(M) * static_cast<size_t>(std::max(first.out(), second.out())) * 4);
+        // a grow-only buffer of the first tensor holds one projection at a time; the stream orders its two uses
+        DeviceBuffer &tmp = first.pair_tmp;
+        tmp.ensure(static_cast<size_t>(M) * static_cast<size_t>(std::max(first.out(), second.out())) * 4);
         for (const NvqWeight *w : {&first, &second}) {
             nvq_matmul(*w, x, x_dtype, ldx, M, static_cast<float *>(tmp.get()), stream);
             hip_check(hipMemcpy2DAsync(y + (w == &second ? first.out() : 0), static_cast<size_t>(N) * 4, tmp.get(),
                                        static_cast<size_t>(w->out()) * 4, static_cast<size_t>(w->out()) * 4, M,
                                        hipMemcpyDeviceToDevice, hs(stream)), "nvq_matmul_multi2");
         }
-        hip_check(hipStreamSynchronize(hs(stream)), "nvq_matmul_multi2");
         return;
     }
     if (M <= 32) {
@@ -881,18 +882,25 @@ QuantLinear load_quant_linear(const std::string &dtype_in, const uint8_t *blob, 
 }
 
 // ---- MoE ---------------------------------------------------------------------------------------------------
-MoeRoutePlan build_moe_route_plan(const int32_t *ids, int tokens, int routes, int n_experts, mfq_stream_t stream) {
+void MoeRoutePlan::reserve(int max_tokens, int routes_, int n_experts_) {
+    if (max_tokens <= 8 || routes_ <= 0 || n_experts_ <= 0) return;
+    const int n_pairs = max_tokens * routes_, tile_m = mfq_hip_moe_tile_m();
+    const int max_tiles = static_cast<int>(cdiv(n_pairs, tile_m)) + n_experts_;
+    counts.ensure(4ull * n_experts_);
+    expert_bounds.ensure(4ull * (n_experts_ + 1));
+    tile_bounds.ensure(4ull * (n_experts_ + 1));
+    tile_experts.ensure(4ull * max_tiles);
+    ids_dst.ensure(4ull * n_pairs);
+}
+
+void build_moe_route_plan(MoeRoutePlan &p, const int32_t *ids, int tokens, int routes, int n_experts, mfq_stream_t stream) {
     if (!ids || tokens <= 0 || routes <= 0) fail("MoE ids must be device int32 [tokens, routes]");
-    MoeRoutePlan p;
     p.ids = ids; p.tokens = tokens; p.routes = routes; p.n_experts = n_experts;
-    if (tokens > 8) {
+    p.has_map = tokens > 8;
+    if (p.has_map) {
         const int n_pairs = tokens * routes, tile_m = mfq_hip_moe_tile_m();
         const int max_tiles = static_cast<int>(cdiv(n_pairs, tile_m)) + n_experts;
-        p.counts = DeviceBuffer(4ull * n_experts);
-        p.expert_bounds = DeviceBuffer(4ull * (n_experts + 1));
-        p.tile_bounds = DeviceBuffer(4ull * (n_experts + 1));
-        p.tile_experts = DeviceBuffer(4ull * max_tiles);
-        p.ids_dst = DeviceBuffer(4ull * n_pairs);
+        p.reserve(tokens, routes, n_experts);
         abi_check(mfq_hip_moe_route_map(ids, n_pairs, n_experts, tile_m, static_cast<int32_t *>(p.counts.get()),
                                         static_cast<int32_t *>(p.expert_bounds.get()),
                                         static_cast<int32_t *>(p.tile_bounds.get()),
@@ -900,6 +908,11 @@ MoeRoutePlan build_moe_route_plan(const int32_t *ids, int tokens, int routes, in
                                         static_cast<int32_t *>(p.ids_dst.get()), stream));
     }
     p.map_ready = true;
+}
+
+MoeRoutePlan build_moe_route_plan(const int32_t *ids, int tokens, int routes, int n_experts, mfq_stream_t stream) {
+    MoeRoutePlan p;
+    build_moe_route_plan(p, ids, tokens, routes, n_experts, stream);
     return p;
 }
 
@@ -1018,7 +1031,7 @@ void NintMoeWeight::add_foreign(const void *x, int x_dtype, int64_t ldx, bool ro
 void NintMoeWeight::forward(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &r, float *out,
                             mfq_stream_t stream) const {
     if (pools.empty()) {  // no NINT cohort at all: every row comes from the host's walk
-        hip_check(hipMemsetAsync(out, 0, 4ull * r.tokens * r.routes * out_per_expert, hs(stream)), "mixed NINTM: clear");
+        abi_check(mfq_hip_fill_zero(out, 4ull * r.tokens * r.routes * out_per_expert, stream));
         add_foreign(x, x_dtype, ldx, routed_input, r, out, stream);
         return;
     }
@@ -1109,7 +1122,8 @@ void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &dow
         abi_check(mfq_hip_moe_weighted_reduce(dn, wts, T, top_k, H, with_shared ? dn + pairs * H : nullptr, nullptr, out, stream));
         return;
     }
-    MoeRoutePlan route = build_moe_route_plan(ids, T, top_k, E, stream);
+    MoeRoutePlan &route = s.route;  // lives in the scratch: nothing is freed on return, so nothing has to be waited for
+    build_moe_route_plan(route, ids, T, top_k, E, stream);
     s.gate_up.ensure(4 * pairs * 2 * W); s.hidden.ensure(2 * pairs * W); s.down.ensure(4 * pairs * H);
     float *gu = static_cast<float *>(s.gate_up.get());
     gate_up.forward_glu(x, x_dtype, ldx, false, route, false, s.hidden.get(), gu, stream);
@@ -1124,8 +1138,40 @@ void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &dow
         shared = static_cast<const float *>(s.shared_out.get());
     }
     abi_check(mfq_hip_moe_weighted_reduce(dn, wts, T, top_k, H, shared, nullptr, out, stream));
-    // the route plan's device tables are freed on return: wait for the kernels that read them
-    hip_check(hipStreamSynchronize(hs(stream)), "nint_moe_ffn_forward");
+}
+
+void MoeFfnScratch::reserve(const NintMoeWeight &wgu, const NintMoeWeight &wdn, int max_tokens, int top_k,
+                            const NintWeight *shared_gate_up, const NintWeight *shared_down) {
+    if (max_tokens <= 0 || top_k <= 0) return;
+    const size_t T = static_cast<size_t>(max_tokens), pairs = T * top_k;
+    const size_t W = static_cast<size_t>(wdn.neuron_len), H = static_cast<size_t>(wdn.out_per_expert);
+    const bool with_shared = shared_gate_up && shared_down;
+    const size_t rows = pairs + (with_shared ? T : 0);  // the decode form keeps the shared expert's rows behind the pairs
+    ids.ensure(4 * pairs); weights.ensure(4 * pairs);
+    hidden.ensure(2 * rows * W); down.ensure(4 * rows * H);
+    if (max_tokens > 8) {
+        gate_up.ensure(4 * pairs * 2 * W);
+        route.reserve(max_tokens, top_k, wgu.n_experts);
+        // the tensors' prefill workspaces: the need grows with the rows of the call
+        auto grouped = [](const NintMoeWeight &w, int x_rows) {
+            if (w.pool_table.empty()) return;
+            const size_t need = mfq_hip_moe_grouped_workspace_bytes(w.pool_table.data(), static_cast<int>(w.pool_table.size()),
+                                                                    w.neuron_len, x_rows);
+            w.workspace.ensure(need);
+        };
+        for (int t = 9; t <= max_tokens; t = t < 64 ? t + 1 : t + 64) { grouped(wgu, t); grouped(wdn, t * top_k); }
+        grouped(wgu, max_tokens); grouped(wdn, max_tokens * top_k);
+        if (with_shared) {
+            shared_gu.ensure(4 * T * 2 * W); shared_h.ensure(2 * T * W); shared_out.ensure(4 * T * H);
+            for (const NintWeight *w : {shared_gate_up, shared_down}) {
+                size_t need = 0;
+                for (int M = 1; M <= std::min(max_tokens, 512); ++M) need = std::max(need, mfq_hip_nint_gemm_workspace_bytes(&w->desc, M));
+                for (int M = 576; M < max_tokens; M += 64) need = std::max(need, mfq_hip_nint_gemm_workspace_bytes(&w->desc, M));
+                need = std::max(need, mfq_hip_nint_gemm_workspace_bytes(&w->desc, max_tokens));
+                w->workspace.ensure(need);
+            }
+        }
+    }
 }
 
 // ---- expert residency -----------------------------------------------------------------------------------------
@@ -1800,10 +1846,44 @@ int mfq_rt_moe_ffn_forward(void *gate_up, void *down, const void *x, int x_dtype
         nint_moe_ffn_forward(*static_cast<NintMoeWeight *>(gate_up), *static_cast<NintMoeWeight *>(down), x, x_dtype, ldx, T,
                              router_logits, top_k, topk_mode, normalize != 0, nullptr, 1.f, sg, sd, s, out, stream);
         const size_t pairs = static_cast<size_t>(T) * top_k;
+        // the scratch is freed on return: wait for the kernels that use it (the copies below are synchronous anyway)
+        if (hipStreamSynchronize(static_cast<hipStream_t>(stream)) != hipSuccess) throw std::runtime_error("nint_moe_ffn_forward");
         if (ids_out && hipMemcpy(ids_out, s.ids.get(), 4 * pairs, hipMemcpyDeviceToDevice) != hipSuccess)
             throw std::runtime_error("copy ids");
         if (weights_out && hipMemcpy(weights_out, s.weights.get(), 4 * pairs, hipMemcpyDeviceToDevice) != hipSuccess)
             throw std::runtime_error("copy weights");
+    });
+}
+
+int mfq_rt_moe_scratch_create(void **scratch) {
+    return guard([&] { *scratch = new MoeFfnScratch(); });
+}
+void mfq_rt_moe_scratch_free(void *scratch) { delete static_cast<MoeFfnScratch *>(scratch); }
+int mfq_rt_moe_scratch_reserve(void *scratch, void *gate_up, void *down, int max_tokens, int top_k, void *shared_gate_up,
+                               void *shared_down) {
+    return guard([&] {
+        const NintWeight *sg = shared_gate_up ? static_cast<QuantLinear *>(shared_gate_up)->nint.get() : nullptr;
+        const NintWeight *sd = shared_down ? static_cast<QuantLinear *>(shared_down)->nint.get() : nullptr;
+        static_cast<MoeFfnScratch *>(scratch)->reserve(*static_cast<NintMoeWeight *>(gate_up), *static_cast<NintMoeWeight *>(down),
+                                                       max_tokens, top_k, sg, sd);
+    });
+}
+int mfq_rt_moe_scratch_topk(void *scratch, const int32_t **ids, const float **weights) {
+    return guard([&] {
+        const MoeFfnScratch *s = static_cast<const MoeFfnScratch *>(scratch);
+        if (ids) *ids = static_cast<const int32_t *>(s->ids.get());
+        if (weights) *weights = static_cast<const float *>(s->weights.get());
+    });
+}
+int mfq_rt_moe_ffn_forward_scratch(void *scratch, void *gate_up, void *down, const void *x, int x_dtype, int64_t ldx, int T,
+                                   const float *router_logits, int top_k, int topk_mode, int normalize, void *shared_gate_up,
+                                   void *shared_down, float *out, void *stream) {
+    return guard([&] {
+        const NintWeight *sg = shared_gate_up ? static_cast<QuantLinear *>(shared_gate_up)->nint.get() : nullptr;
+        const NintWeight *sd = shared_down ? static_cast<QuantLinear *>(shared_down)->nint.get() : nullptr;
+        nint_moe_ffn_forward(*static_cast<NintMoeWeight *>(gate_up), *static_cast<NintMoeWeight *>(down), x, x_dtype, ldx, T,
+                             router_logits, top_k, topk_mode, normalize != 0, nullptr, 1.f, sg, sd,
+                             *static_cast<MoeFfnScratch *>(scratch), out, stream);
     });
 }
 }

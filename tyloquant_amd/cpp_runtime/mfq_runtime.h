@@ -112,6 +112,7 @@ struct NvqWeight {
     DeviceBuffer data;
     std::string dtype;
     mutable DeviceBuffer workspace;
+    mutable DeviceBuffer pair_tmp;  // nvq_matmul_multi2 on stream formats: one projection at a time, grow-only
     int64_t out() const { return streams ? sdesc.out : desc.out; }
     int64_t neuron_len() const { return streams ? sdesc.neuron_len : desc.neuron_len; }
     int64_t payload_bytes() const { return streams ? sdesc.payload_bytes : desc.payload_bytes; }
@@ -240,13 +241,20 @@ QuantLinear load_quant_linear(const std::string &dtype, const uint8_t *blob, siz
 struct MoeRoutePlan {
     const int32_t *ids = nullptr;  // device int32 [tokens, routes]
     int tokens = 0, routes = 0, n_experts = 0;
-    DeviceBuffer ids_dst, expert_bounds, tile_bounds, tile_experts, counts;
-    bool map_ready = false;
-    bool mapped() const { return ids_dst.get() != nullptr; }
+    DeviceBuffer ids_dst, expert_bounds, tile_bounds, tile_experts, counts;  // grow-only; valid when has_map
+    bool map_ready = false, has_map = false;
+    bool mapped() const { return has_map; }
+    // Sizes the tables for up to max_tokens x routes pairs over n_experts experts: building a plan of that size or
+    // smaller in place then allocates nothing (HIP graph capture, serving loops).
+    void reserve(int max_tokens, int routes, int n_experts);
 };
-// Builds the expert map only above 8 tokens, like the reference.
+// Builds the expert map only above 8 tokens, like the reference (cpp_runtime/mfq_decode.cpp:2681-2708).  The first form
+// returns a new plan; the second rebuilds `plan` in place, reusing its tables (no allocation once they are large
+// enough, no host synchronisation in either).
 MoeRoutePlan build_moe_route_plan(const int32_t *ids, int tokens, int routes, int n_experts,
                                   mfq_stream_t stream = nullptr);
+void build_moe_route_plan(MoeRoutePlan &plan, const int32_t *ids, int tokens, int routes, int n_experts,
+                          mfq_stream_t stream = nullptr);
 
 // Cuts an NVQ-family or 1-bit-family blob of parts * n neurons into `parts` blobs of n neurons each: same flags and
 // tables, the rows' anchors and their share of every tensor-wide bit stream re-packed from bit 0.
@@ -298,8 +306,16 @@ struct NintMoeWeight {
 
 struct MoeFfnScratch {  // caller-owned intermediates of nint_moe_ffn_forward, grown on demand
     DeviceBuffer ids, weights, gate_up, hidden, down, shared_gu, shared_h, shared_out;
+    MoeRoutePlan route;  // the expert map of the last call above 8 tokens
+    // Sizes every intermediate, the route tables and the tensors' own workspaces for calls of up to max_tokens tokens
+    // with top_k routes: nint_moe_ffn_forward then neither allocates nor waits for the device, so that a caller may
+    // capture it into a HIP graph (the reference's forward does neither under capture: cpp_runtime/mfq_decode.cpp:3008-3016).
+    // Tensors with cohorts of other families keep their host walk and cannot be captured.
+    void reserve(const NintMoeWeight &gate_up, const NintMoeWeight &down, int max_tokens, int top_k,
+                 const NintWeight *shared_gate_up = nullptr, const NintWeight *shared_down = nullptr);
 };
 // out fp32 [T, hidden]; top-k ids / weights stay in `scratch`.  `shared_gate_up` / `shared_down` may be null.
+// Never waits for the device; allocates only when `scratch` (see MoeFfnScratch::reserve) or a workspace must grow.
 void nint_moe_ffn_forward(const NintMoeWeight &gate_up, const NintMoeWeight &down, const void *x, int x_dtype,
                           int64_t ldx, int T, const float *router_logits, int top_k, int topk_mode, bool normalize,
                           const float *router_bias, float router_scale, const NintWeight *shared_gate_up,

@@ -397,7 +397,9 @@ __global__ __launch_bounds__(512) void moe_grouped_kernel(MoePools P, const int3
 // (cohort slot P.n) to token t.  P.spw: steps per wave of each cohort; RING = false when no wave has more than
 // three (row-block, step) items.  SWIGLU: the block takes row-block blockIdx.x of the gate half and of the up half
 // of the expert and stores act(gate) * up as 16-bit values: bit 0 of out_f16 selects fp16 over bf16, bit 1 GELU over SiLU.
-template <int XF16, bool RING, bool SWIGLU>
+// XR (only without a ring): cohorts whose groups fit a row of lanes keep the activations in registers
+// (nint_unit_body_xreg); the launch sets it when the rows are 4-byte aligned and K is even.
+template <int XF16, bool RING, bool SWIGLU, bool XR = false>
 __global__ __launch_bounds__(1024) void moe_decode_kernel(MoePools P, int rbw, const int32_t *__restrict__ expert_pool,
                                                           const int32_t *__restrict__ expert_local, int E,
                                                           int out_per_expert, const uint16_t *__restrict__ x, int64_t ldx,
@@ -433,9 +435,16 @@ __global__ __launch_bounds__(1024) void moe_decode_kernel(MoePools P, int rbw, c
     const uint16_t *xr[1] = {x + static_cast<int64_t>(xi) * ldx};
     float *yr[1] = {SWIGLU ? nullptr : static_cast<float *>(out) + static_cast<int64_t>(row) * ldo};
     const int rb0 = row_base / 16 + rbl0, nrb = SWIGLU ? 2 : rbw, step = SWIGLU ? half_rb : 1;
+    bool in_regs = false;  // this block's cohort ran the register body: its partial sums start at the head of the LDS
 #define MFQ_MOE_CASE(UNIT, B, G)                                                                                        \
-    if (k.bits == B && k.gs == G)                                                                                      \
-        nint_unit_body<UNIT<B, G>, XF16, 1, RING, !SWIGLU>(k, w, rb0, nrb, row_base, out_per_expert, xr, yr, spw, lds, step);
+    if (k.bits == B && k.gs == G) {                                                                                    \
+        if constexpr (XR && !RING && UNIT<B, G>::NPAIR <= 16) {                                                        \
+            in_regs = true;                                                                                            \
+            nint_unit_body_xreg<UNIT<B, G>, XF16, 1, !SWIGLU>(k, w, rb0, nrb, row_base, out_per_expert, xr, yr, spw, lds, step); \
+        } else {                                                                                                       \
+            nint_unit_body<UNIT<B, G>, XF16, 1, RING, !SWIGLU>(k, w, rb0, nrb, row_base, out_per_expert, xr, yr, spw, lds, step); \
+        }                                                                                                              \
+    }
     if (k.kind == 1) {
         MFQ_MOE_CASE(PairedUnit, 4, 24)
         else MFQ_MOE_CASE(PairedUnit, 3, 24)
@@ -452,7 +461,7 @@ __global__ __launch_bounds__(1024) void moe_decode_kernel(MoePools P, int rbw, c
         __syncthreads();
         if (threadIdx.x < 16) {
             const int nwaves = blockDim.x >> 6;
-            const float *red = reinterpret_cast<const float *>(lds + gemv_red_offset(nwaves, 1, spw, k.gs));
+            const float *red = reinterpret_cast<const float *>(lds + (in_regs ? 0 : gemv_red_offset(nwaves, 1, spw, k.gs)));
             float g = 0.f, u = 0.f;
             for (int wv = 0; wv < nwaves; ++wv) {
                 g += red[wv * 16 + threadIdx.x];
@@ -720,9 +729,12 @@ static int moe_decode_launch(MoePools &P, int n_slots, int max_steps, const int3
     const size_t lds = sh.lds;
     const bool ring = sh.ring;
     const dim3 grid(static_cast<unsigned>(swiglu ? rbe / 2 : rbe / rbw), static_cast<unsigned>(n_rows)), block(64 * nwaves);
+    static const int env_xreg = tune_env("MFQ_GEMV_XREG", 1);
+    const bool xreg = !ring && ldx % 2 == 0 && (reinterpret_cast<uintptr_t>(xp) & 3) == 0 && P.k[0].neuron_len % 2 == 0 &&
+                      env_xreg != 0;
 #define MFQ_MOE_DECODE(XF, RG, SW)                                                                                   \
     do {                                                                                                             \
-        auto kern = moe_decode_kernel<XF, RG, SW>;                                                                   \
+        auto kern = (!RG && xreg) ? moe_decode_kernel<XF, RG, SW, !RG> : moe_decode_kernel<XF, RG, SW, false>;       \
         if (int rc_ = allow_dynamic_lds(reinterpret_cast<const void *>(kern), lds, "moe_decode")) return rc_;        \
         hipLaunchKernelGGL(kern, grid, block, lds, st, P, rbw, expert_pool, expert_local, E, out_per_expert, xp, ldx, \
                            routed_input, ids, n_pairs, R, out, out_f16, ldo);                                        \

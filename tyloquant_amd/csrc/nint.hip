@@ -190,7 +190,7 @@ static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, i
     // Waves with at most three items keep the staged activations in registers when a group's pairs fit one row of
     // lanes and the rows can be fetched pair by pair (4-byte aligned rows, even K): LDS then only holds the sums.
     static const int env_xreg = tune_env("MFQ_GEMV_XREG", 1);
-    const bool xreg_rows = MB <= 2 && spw * rbw <= 3 && k.neuron_len % 2 == 0 && ldx % 2 == 0 &&
+    const bool xreg_rows = MB <= 2 && spw * rbw <= 3 && k.neuron_len % 2 == 0 && (M == 1 || ldx % 2 == 0) &&
                            (reinterpret_cast<uintptr_t>(x) & 3) == 0 && env_xreg != 0;
     const size_t lds_xreg = static_cast<size_t>(rbw) * nwaves * MB * 16 * 4;
 #define MFQ_XREG(UNIT)                                                                                         \
@@ -550,9 +550,12 @@ static int launch_gemv_swiglu(const NintK &k, const uint8_t *w, const uint16_t *
         if (int rc_ = allow_dynamic_lds(reinterpret_cast<const void *>(kern_), lds, "nint_gemv_swiglu")) return rc_;  \
         hipLaunchKernelGGL(kern_, grid, block, lds, st, k, w, x, ldx, M, hidden, out_f16, ldh, spw);                  \
     } while (0)
+    static const int env_xreg = tune_env("MFQ_GEMV_XREG", 1);
+    const bool xreg = env_xreg != 0 && k.neuron_len % 2 == 0 && ldx % 2 == 0 && (reinterpret_cast<uintptr_t>(x) & 3) == 0;
 #define MFQ_SWIGLU(UNIT, B, G)                                                                                        \
     if (k.bits == B && k.gs == G) {                                                                                   \
         if (ring) MFQ_SWIGLU_LAUNCH((nint_gemv_swiglu_kernel<UNIT<B, G>, XF16, MB, true>));                           \
+        else if (xreg) MFQ_SWIGLU_LAUNCH((nint_gemv_swiglu_kernel<UNIT<B, G>, XF16, MB, false, true>));               \
         else MFQ_SWIGLU_LAUNCH((nint_gemv_swiglu_kernel<UNIT<B, G>, XF16, MB, false>));                               \
         return check_launch("nint_gemv_swiglu");                                                                      \
     }

@@ -793,7 +793,7 @@ __global__ __launch_bounds__(1024) void nint_gemv_natural_kernel(NintK k, const 
 // Gate/up GEMV with the SwiGLU fused: the tensor holds the W gate neurons, then the W up neurons.  Block
 // blockIdx.x takes row-block blockIdx.x of each half and stores hidden[m][16 * blockIdx.x + r] = act(gate) * up
 // as fp16 (bit 0 of out_f16) or bf16, act = SiLU or (bit 1 of out_f16) GELU.
-template <class U, int XF16, int MB, bool RING>
+template <class U, int XF16, int MB, bool RING, bool XR = false>
 __global__ __launch_bounds__(1024) void nint_gemv_swiglu_kernel(NintK k, const uint8_t *__restrict__ w,
                                                                 const uint16_t *__restrict__ x, int64_t ldx, int M,
                                                                 uint16_t *__restrict__ hidden, int out_f16, int64_t ldh,
@@ -803,10 +803,12 @@ __global__ __launch_bounds__(1024) void nint_gemv_swiglu_kernel(NintK k, const u
     float *yr[MB];
     dense_rows<MB>(x, ldx, static_cast<float *>(nullptr), 0, M, blockIdx.y * MB, xr, yr);
     const int half_rb = k.n_rowblocks / 2;
-    nint_unit_body<U, XF16, MB, RING, false>(k, w, blockIdx.x, 2, 0, k.out, xr, yr, spw, lds, half_rb);
+    constexpr bool IN_REGS = XR && !RING && U::NPAIR <= 16 && (MB == 1 || U::CBITS != 0);  // see nint_unit_body_xreg
+    if constexpr (IN_REGS) nint_unit_body_xreg<U, XF16, MB, false>(k, w, blockIdx.x, 2, 0, k.out, xr, yr, spw, lds, half_rb);
+    else nint_unit_body<U, XF16, MB, RING, false>(k, w, blockIdx.x, 2, 0, k.out, xr, yr, spw, lds, half_rb);
     __syncthreads();
     const int nwaves = blockDim.x >> 6;
-    const float *red = reinterpret_cast<const float *>(lds + gemv_red_offset(nwaves, MB, spw, U::GROUP));
+    const float *red = reinterpret_cast<const float *>(lds + (IN_REGS ? 0 : gemv_red_offset(nwaves, MB, spw, U::GROUP)));
     for (int o = threadIdx.x; o < MB * 16; o += blockDim.x) {
         const int r = o & 15, m = o >> 4;
         const int row = blockIdx.y * MB + m;

@@ -61,7 +61,7 @@ __device__ __forceinline__ void argmax_wave(float &best, int &best_i) {
 
 // The batch-1 GEMV with the block's winner instead of (or besides) its 16 * rbw logits: partial sums are added in
 // the order of the plain kernel, so the logits are the same floats.
-template <class U, int XF16, bool RING>
+template <class U, int XF16, bool RING, bool XR = false>
 __global__ __launch_bounds__(1024) void nint_gemv_argmax_kernel(NintK k, const uint8_t *__restrict__ w,
                                                                 const uint16_t *__restrict__ x, float *__restrict__ logits,
                                                                 float *__restrict__ block_vals,
@@ -69,11 +69,13 @@ __global__ __launch_bounds__(1024) void nint_gemv_argmax_kernel(NintK k, const u
     extern __shared__ uint32_t lds[];
     const uint16_t *xr[1] = {x};
     float *yr[1] = {nullptr};
-    nint_unit_body<U, XF16, 1, RING, false>(k, w, blockIdx.x * rbw, rbw, 0, k.out, xr, yr, spw, lds);
+    constexpr bool IN_REGS = XR && !RING && U::NPAIR <= 16;  // the plain GEMV's choice, so that the sums are the same floats
+    if constexpr (IN_REGS) nint_unit_body_xreg<U, XF16, 1, false>(k, w, blockIdx.x * rbw, rbw, 0, k.out, xr, yr, spw, lds);
+    else nint_unit_body<U, XF16, 1, RING, false>(k, w, blockIdx.x * rbw, rbw, 0, k.out, xr, yr, spw, lds);
     __syncthreads();
     if (threadIdx.x >= 64) return;
     const int nwaves = blockDim.x >> 6;
-    const float *red = reinterpret_cast<const float *>(lds + gemv_red_offset(nwaves, 1, spw, U::GROUP));
+    const float *red = reinterpret_cast<const float *>(lds + (IN_REGS ? 0 : gemv_red_offset(nwaves, 1, spw, U::GROUP)));
     float best = -INFINITY;
     int best_i = INT_MAX;
     const int o = threadIdx.x;  // rbw <= 4 row-blocks: one lane per neuron
@@ -149,9 +151,15 @@ static int launch_gemv_argmax(const NintK &k, const uint8_t *w, const uint16_t *
     nb = -1;
     if (lds > 65536 || k.rowblock_bytes >= (1ll << 31)) return MFQ_OK;  // the caller takes the unfused form
     const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, rbw))), block(64 * nwaves);
+    // the plain GEMV's condition for activations in registers (launch_gemv_mb)
+    static const int env_xreg = tune_env("MFQ_GEMV_XREG", 1);
+    const bool xreg = env_xreg != 0 && k.neuron_len % 2 == 0 && (reinterpret_cast<uintptr_t>(x) & 3) == 0;
 #define MFQ_ARGMAX(UNIT, B, G)                                                                                        \
     if (k.bits == B && k.gs == G) {                                                                                   \
-        if (spw * rbw <= 3)                                                                                           \
+        if (spw * rbw <= 3 && xreg)                                                                                   \
+            hipLaunchKernelGGL((nint_gemv_argmax_kernel<UNIT<B, G>, XF16, false, true>), grid, block, lds, st, k, w, x, logits, \
+                               vals, idxs, spw, rbw);                                                                 \
+        else if (spw * rbw <= 3)                                                                                      \
             hipLaunchKernelGGL((nint_gemv_argmax_kernel<UNIT<B, G>, XF16, false>), grid, block, lds, st, k, w, x, logits, \
                                vals, idxs, spw, rbw);                                                                 \
         else                                                                                                          \

@@ -90,9 +90,49 @@ int allow_dynamic_lds(const void *kernel, size_t lds, const char *what) {
     return MFQ_OK;
 }
 
+// Read-only streaming probe: a wave owns 16 KB, requested up front.
+__global__ __launch_bounds__(512) void read_probe_kernel(const u32x4_t *__restrict__ p, size_t n16, uint32_t *sink) {
+    const size_t wave = static_cast<size_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const size_t base = wave * (16 * 64) + (threadIdx.x & 63);
+    u32x4_t v[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const size_t idx = base + static_cast<size_t>(i) * 64;
+        v[i] = idx < n16 ? __builtin_nontemporal_load(p + idx) : u32x4_t{0u, 0u, 0u, 0u};
+    }
+    uint32_t a = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    if (a == 0x12345678u) sink[0] = a;
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t *__restrict__ p, size_t n) {
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += static_cast<size_t>(gridDim.x) * 256) p[i] = 0u;
+}
+
 }  // namespace mfq
 
 using namespace mfq;
+
+extern "C" int mfq_hip_fill_zero(void *data, size_t bytes, mfq_stream_t stream) {
+    if (bytes == 0) return MFQ_OK;
+    MFQ_REQUIRE(data && (reinterpret_cast<uintptr_t>(data) & 3) == 0 && bytes % 4 == 0, MFQ_ERR_INVALID,
+                "fill_zero: null or unaligned buffer");
+    const size_t n = bytes / 4;
+    const size_t blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(static_cast<unsigned>(blocks < 4096 ? blocks : 4096)), dim3(256), 0, as_stream(stream),
+                       static_cast<uint32_t *>(data), n);
+    return check_launch("fill_zero");
+}
+
+extern "C" int mfq_hip_read_probe(const void *data, size_t bytes, void *sink, mfq_stream_t stream) {
+    MFQ_REQUIRE(data && sink && (reinterpret_cast<uintptr_t>(data) & 15) == 0, MFQ_ERR_INVALID, "read_probe: null or unaligned buffer");
+    const size_t n16 = bytes / 16, waves = ceil_div(static_cast<int64_t>(n16), 16 * 64);
+    MFQ_REQUIRE(n16 > 0 && waves / 8 + 1 < (1ull << 31), MFQ_ERR_INVALID, "read_probe: %zu bytes", bytes);
+    hipLaunchKernelGGL(read_probe_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(waves), 8))), dim3(512), 0,
+                       as_stream(stream), static_cast<const u32x4_t *>(data), n16, static_cast<uint32_t *>(sink));
+    return check_launch("read_probe");
+}
 
 extern "C" void mfq_hip_set_cu_count(int n) { g_cu_override.store(n > 0 ? n : 0, std::memory_order_relaxed); }
 
