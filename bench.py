@@ -285,7 +285,7 @@ def main() -> int:
         return torch.from_numpy(a).to(torch.bfloat16).to(dev)
 
     if not args.no_extras:
-        from tyloquant_amd import runtime_moe as RM
+        from tyloquant_amd import formats as F
         from tyloquant_amd import runtime_vq as RV
         # hot (one weight set, cache-resident between launches)
         hot_ms = time_fn(lambda: launch(sets[0], stream_ptr()), 100)
@@ -340,41 +340,80 @@ def main() -> int:
         torch.cuda.empty_cache()
 
         # ---- config 4: 256 mixed-bit experts + 1 shared, hidden 4096, intermediate 2048, top-8 ------
+        # N(0, 0.02) weights through the expert-wise NINT quantizer (a 1024-row slab per precision, tiled over its
+        # cohort), loaded and run by the C++ host runtime (libmfq_runtime.so): nint_moe_ffn_forward with a reserved
+        # scratch, recorded into a HIP graph.
+        rt = C.CDLL(str(ROOT / "tyloquant_amd" / "lib" / "libmfq_runtime.so"))
+        rt.mfq_rt_last_error.restype = C.c_char_p
+        rt.mfq_rt_load_nint_moe.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(C.c_void_p)]
+        rt.mfq_rt_free_nint_moe.argtypes = [C.c_void_p]
+        rt.mfq_rt_load_quant_linear.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_void_p)]
+        rt.mfq_rt_free_quant_linear.argtypes = [C.c_void_p]
+        rt.mfq_rt_moe_scratch_create.argtypes = [C.POINTER(C.c_void_p)]
+        rt.mfq_rt_moe_scratch_free.argtypes = [C.c_void_p]
+        rt.mfq_rt_moe_scratch_reserve.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        rt.mfq_rt_moe_ffn_forward_scratch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64,
+                                                      C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                                      C.c_void_p, C.c_void_p]
+
+        def rt_check(rc):
+            if rc:
+                raise RuntimeError(rt.mfq_rt_last_error().decode(errors="replace"))
         E, HID, INTER, TOPK = 256, 4096, 2048, 8
         ebits = np.random.default_rng(4).choice([2, 3, 4, 5], size=E, p=[0.1, 0.4, 0.4, 0.1])
-        gu = synth.random_nint_moe(40, E, 2 * INTER, HID, ebits)
-        dn = synth.random_nint_moe(41, E, HID, INTER, ebits)
-        shared = (synth.random_nint_weight(42, 2 * INTER, HID, 4, 24, 6), synth.random_nint_weight(43, HID, INTER, 4, 24, 6))
-        shared_bytes = shared[0].payload_bytes + shared[1].payload_bytes
-        per_expert = np.array([gu.expert_payload_bytes(e) + dn.expert_payload_bytes(e) for e in range(E)])
+        per_expert = np.zeros(E)
+        handles = []
+        for seed, (o_, k_) in ((40, (2 * INTER, HID)), (41, (HID, INTER))):
+            blob4, pools4 = synth.nintm_quantized_blob(seed, E, o_, k_, ebits)
+            for ids4, payload4 in pools4:
+                hdr = F.parse_nint(payload4)
+                per_expert[ids4] += hdr.body_bytes / len(ids4)
+            h4 = C.c_void_p()
+            rt_check(rt.mfq_rt_load_nint_moe(blob4, len(blob4), C.byref(h4)))
+            handles.append(h4)
+            del blob4, pools4
+        shared_bytes, shared_h = 0, []
+        for seed, (o_, k_) in ((42, (2 * INTER, HID)), (43, (HID, INTER))):
+            dt4, sb4 = synth.nint_linear_blob(seed, o_, k_, 4, 24, 6, slab_rows=1024)
+            shared_bytes += F.parse_nint(sb4).body_bytes
+            h4 = C.c_void_p()
+            rt_check(rt.mfq_rt_load_quant_linear(dt4.encode(), sb4, len(sb4), C.byref(h4)))
+            shared_h.append(h4)
+        scratch4 = C.c_void_p()
+        rt_check(rt.mfq_rt_moe_scratch_create(C.byref(scratch4)))
+        rt_check(rt.mfq_rt_moe_scratch_reserve(scratch4, handles[0], handles[1], 2048, TOPK, shared_h[0], shared_h[1]))
+        torch.cuda.synchronize()
+        log(f"[bench] config 4 tensors quantized and loaded by the C++ runtime ({time.time() - t0:.1f}s)")
         for T, nb in ((1, 8), (64, 2), (2048, 1)):
             xs4 = [bf16(synth.activations(rng, T, HID)) for _ in range(nb)]
             lg4 = [torch.from_numpy(rng.standard_normal((T, E)).astype(np.float32)).to(dev) for _ in range(nb)]
+            out4 = torch.empty((T, HID), dtype=torch.float32, device=dev)
 
             def moe_all():
-                return [RM.nint_moe_ffn_forward(gu, dn, xs4[i], lg4[i], TOPK, delayed_softmax=True, shared=shared)
-                        for i in range(nb)]
-            eager = moe_all()
+                for i in range(nb):
+                    rt_check(rt.mfq_rt_moe_ffn_forward_scratch(scratch4, handles[0], handles[1], xs4[i].data_ptr(), L.X_BF16,
+                                                               HID, T, lg4[i].data_ptr(), TOPK, L.TOPK_DELAYED_SOFTMAX, 0,
+                                                               shared_h[0], shared_h[1], out4.data_ptr(), stream_ptr()))
+            moe_all()
             torch.cuda.synchronize()
+            assert bool(torch.isfinite(out4).all()), "MoE layer produced non-finite outputs"
             hit_bytes = 0.0
-            for (_, ids, _w) in eager:
-                hit_bytes += per_expert[np.unique(ids.cpu().numpy())].sum() + shared_bytes
-            try:
-                ms = graph_ms(moe_all, 5 if T < 2048 else 2) / nb
-                how = "hip graph"
-            except Exception as exc:  # capture refused by an op: time eager launches instead
-                log(f"[bench] MoE T={T}: graph capture failed ({exc}); timing eager")
-                torch.cuda.synchronize()
-                ms = time_fn(moe_all, 3, warm=1) / nb
-                how = "eager"
+            for lgt in lg4:
+                hit = torch.unique(torch.topk(lgt, TOPK, dim=1).indices).cpu().numpy()
+                hit_bytes += per_expert[hit].sum() + shared_bytes
+            ms = graph_ms(moe_all, 5 if T < 2048 else 2) / nb
             extras[f"config4_moe_T{T}_ms"] = ms
             extras[f"config4_moe_T{T}_tokens_per_s"] = T / (ms * 1e-3)
             extras[f"config4_moe_T{T}_weight_gbps"] = hit_bytes / nb / (ms * 1e-3) / 1e9
             extras[f"config4_moe_T{T}_tflops"] = (2.0 * T * TOPK * 3 * HID * INTER + 2.0 * T * 3 * HID * INTER) / (ms * 1e-3) / 1e12
-            log(f"[bench] config 4 MoE T={T}: {ms:.3f} ms ({how}), {T / (ms * 1e-3):.0f} tokens/s, "
+            log(f"[bench] config 4 MoE T={T} (C++ host, HIP graph): {ms:.3f} ms, {T / (ms * 1e-3):.0f} tokens/s, "
                 f"{extras[f'config4_moe_T{T}_weight_gbps']:.0f} GB/s of expert payload")
-            del eager
-        del gu, dn, shared
+        extras["config4_host"] = "C++ runtime (libmfq_runtime.so), graph replay"
+        rt.mfq_rt_moe_scratch_free(scratch4)
+        for h4 in shared_h:
+            rt.mfq_rt_free_quant_linear(h4)
+        for h4 in handles:
+            rt.mfq_rt_free_nint_moe(h4)
         torch.cuda.empty_cache()
 
         # ---- config 5: 36-layer linear stack, mixed formats by seed, batch {1,16} -------------------

@@ -1271,6 +1271,29 @@ def dequantize_tensor(t) -> np.ndarray:
     raise TypeError(type(t))
 
 
+def quantize_expertwise(weight, profiles) -> NintMoeTensor:
+    """mfq/quantize/expert_nint.py:507-578, NINT cohorts only (`profiles[e]` = (bits, groupsize, sub_bits) of expert e):
+    cohorts in the order their precision first appears (:528-531, a dict keyed by precision), experts ascending inside a
+    cohort, the cohort's rows flattened to [n * out, K] (:559-561) and quantized weight-only like a dense tensor
+    (:340-351 with importance=None)."""
+    W = np.asarray(weight, dtype=np.float32)
+    if W.ndim != 3:
+        raise ValueError("expert-wise quantization expects [experts, out, in]")
+    E, out, K = W.shape
+    profiles = [tuple(int(v) for v in p) for p in profiles]
+    if len(profiles) != E:
+        raise ValueError(f"received {len(profiles)} precision descriptors for {E} experts")
+    cohorts = {}
+    for e, prof in enumerate(profiles):
+        cohorts.setdefault(prof, []).append(e)
+    pools = []
+    for (bits, gs, sub_bits), members in cohorts.items():
+        ids = np.asarray(members, dtype=np.int32)
+        rows = np.ascontiguousarray(W[ids]).reshape(ids.size * out, K)
+        pools.append(MoePool(ids, f"NINT{bits}", quantize_nint(rows, bits, gs, sub_bits)))
+    return NintMoeTensor((E, out, K), pools)
+
+
 def dequantize_expertwise(t: NintMoeTensor) -> np.ndarray:
     """mfq/quantize/expert_nint.py:605-615."""
     E, out, K = t.shape

@@ -40,6 +40,13 @@ def rt():
     lib.mfq_rt_moe_ffn_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p,
                                            C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                            C.c_void_p, C.c_void_p]
+    lib.mfq_rt_moe_scratch_create.argtypes = [C.POINTER(C.c_void_p)]
+    lib.mfq_rt_moe_scratch_free.argtypes = [C.c_void_p]
+    lib.mfq_rt_moe_scratch_reserve.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    lib.mfq_rt_moe_scratch_topk.argtypes = [C.c_void_p, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)]
+    lib.mfq_rt_moe_ffn_forward_scratch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int,
+                                                   C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                                   C.c_void_p]
     lib.mfq_rt_nvq_ffn_swiglu_down.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int,
                                                C.c_void_p, C.c_void_p]
     return lib
@@ -238,6 +245,81 @@ def test_cpp_moe_ffn_forward(rt, T):
                               delayed_softmax=True)
     assert np.array_equal(ids.cpu().numpy(), rids)
     check_close(out.cpu().numpy(), ref)
+    rt.mfq_rt_free_nint_moe(hg)
+    rt.mfq_rt_free_nint_moe(hd)
+
+
+@pytest.mark.parametrize("T", [1, 64])
+def test_cpp_moe_ffn_forward_replays_from_a_graph(rt, T):
+    """nint_moe_ffn_forward of the C++ runtime with a reserved scratch is recorded into a HIP graph (it must neither
+    allocate nor wait for the device: either would fail the capture) and replayed several times with new activations and
+    router logits in the same buffers and eager work in between; every replay equals the eager call bit for bit, and the
+    eager call matches the oracle.  T = 1 takes the decode form (no route map), T = 64 the mapped prefill kernels with a
+    shared expert next to the routed ones."""
+    rng = np.random.default_rng(400 + T)
+    E, H, W, k = 16, 256, 128, 4
+    bits = rng.choice([2, 3, 4, 5], size=E, p=[0.1, 0.4, 0.4, 0.1])
+    tg, td = synth.moe_random(rng, E, 2 * W, H, bits, True), synth.moe_random(rng, E, H, W, bits, True)
+    sg_t, sd_t = synth.nint_random(rng, 2 * W, H, 4, 24, 6), synth.nint_random(rng, H, W, 4, 24, 6)
+    bg, bd = O.pack_nint_moe(tg), O.pack_nint_moe(td)
+    hg, hd = C.c_void_p(), C.c_void_p()
+    assert rt.mfq_rt_load_nint_moe(bg, len(bg), C.byref(hg)) == 0, rt.mfq_rt_last_error()
+    assert rt.mfq_rt_load_nint_moe(bd, len(bd), C.byref(hd)) == 0, rt.mfq_rt_last_error()
+    sg, sd = _load(rt, "NINT4", O.pack_nint(sg_t)), _load(rt, "NINT4", O.pack_nint(sd_t))
+    scratch = C.c_void_p()
+    assert rt.mfq_rt_moe_scratch_create(C.byref(scratch)) == 0
+    assert rt.mfq_rt_moe_scratch_reserve(scratch, hg, hd, T, k, sg, sd) == 0, rt.mfq_rt_last_error()
+    x = torch.empty((T, H), dtype=torch.bfloat16, device="cuda")
+    lg = torch.empty((T, E), dtype=torch.float32, device="cuda")
+    out = torch.empty((T, H), dtype=torch.float32, device="cuda")
+
+    def fill(seed):
+        r = np.random.default_rng(seed)
+        xs = r.standard_normal((T, H)).astype(np.float32)
+        ls = r.standard_normal((T, E)).astype(np.float32)
+        x.copy_(torch.from_numpy(xs).to(torch.bfloat16))
+        lg.copy_(torch.from_numpy(ls))
+        return ls
+
+    def call(stream):
+        rc = rt.mfq_rt_moe_ffn_forward_scratch(scratch, hg, hd, x.data_ptr(), 0, H, T, lg.data_ptr(), k, 3, 0, sg, sd,
+                                               out.data_ptr(), stream)
+        assert rc == 0, rt.mfq_rt_last_error()
+
+    logits = fill(1)
+    call(None)  # eager: default stream
+    torch.cuda.synchronize()
+    eager1 = out.clone()
+    Wg, Wd = O.dequantize_expertwise(tg), O.dequantize_expertwise(td)
+    ref, rids, _ = O.moe_ffn(Wg, Wd, x.float().cpu().numpy(), logits, k, delayed_softmax=True,
+                             shared=(O.dequantize_nint(sg_t), O.dequantize_nint(sd_t)))
+    ids_p, w_p = C.c_void_p(), C.c_void_p()
+    assert rt.mfq_rt_moe_scratch_topk(scratch, C.byref(ids_p), C.byref(w_p)) == 0
+    check_close(eager1.cpu().numpy(), ref)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(C.c_void_p(side.cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        call(C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    for seed in (1, 2, 3, 1):
+        fill(seed)
+        call(None)
+        torch.cuda.synchronize()
+        want = out.clone()
+        out.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int32), want.view(torch.int32)), f"replay differs from the eager call (seed {seed})"
+    assert torch.equal(want.view(torch.int32), eager1.view(torch.int32))
+    rt.mfq_rt_moe_scratch_free(scratch)
+    for h in (sg, sd):
+        rt.mfq_rt_free_quant_linear(h)
     rt.mfq_rt_free_nint_moe(hg)
     rt.mfq_rt_free_nint_moe(hd)
 

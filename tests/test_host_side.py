@@ -237,3 +237,22 @@ def test_mfq_directory_checks_of_the_reference_reader(tmp_path):
             bad.write_bytes(payload)
             r = subprocess.run([str(tool), str(bad), "w"], capture_output=True, text=True)
             assert r.returncode == 1 and want in r.stderr, r.stderr
+
+
+def test_tiled_expertwise_blob_equals_quantizing_the_full_tensor():
+    """synth.nintm_quantized_blob quantizes one slab per precision and repeats the slab's streams over the cohort; the
+    NINT quantizer treats every neuron on its own, so the bytes must equal the oracle's expert-wise quantization of the
+    full tensor whose experts repeat the slabs -- cohort order, expert order and every stream included."""
+    from tyloquant_amd import synth as psynth
+    bits = [4, 3, 3, 5, 2, 4, 3, 3]
+    E, out, K, slab = len(bits), 32, 100, 16
+    blob, pools = psynth.nintm_quantized_blob(9, E, out, K, bits, slab_rows=slab)
+    order = list(dict.fromkeys(bits))
+    slabs = (np.random.default_rng(9).standard_normal((len(order), slab, K)) * 0.02).astype(np.float32)
+    W = np.stack([np.tile(slabs[order.index(b)], (out // slab, 1)) for b in bits])
+    t = O.quantize_expertwise(W, [psynth.MOE_PROFILES[b] for b in bits])
+    assert blob == O.pack_nint_moe(t)
+    assert [ids.tolist() for ids, _ in pools] == [p.expert_ids.tolist() for p in t.pools]
+    assert all(payload == O.pack_nint(p.tensor) for (_, payload), p in zip(pools, t.pools))
+    with pytest.raises(ValueError):
+        psynth.nintm_quantized_blob(9, E, 30, K, bits, slab_rows=16)

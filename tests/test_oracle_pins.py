@@ -411,3 +411,30 @@ def test_nint8_zero_is_ggml_q8_0():
     assert (h.out, h.ng, h.neuron_len, h.body_off, h.body_bytes) == (2, 2, 64, 40, 136)
     with pytest.raises(ValueError, match="invalid NINT8-0 block bytes"):
         F.parse_nint8_zero(blob + b"\0")
+
+
+@pytest.mark.parametrize("case", ["mixed", "single"])
+def test_expertwise_quantizer_matches_the_reference_fixture(case):
+    """quantize_expertwise on the fixture's weights and profiles: the oracle's and the product's NIM2 bytes equal the
+    bytes the reference packed (cohort order by first appearance of a precision, experts ascending inside a cohort, every
+    pool the flat-cohort NINT quantization), and the oracle dequantizes them to the reference's values bit for bit
+    (tests/golden/make_reference_expertwise.py wrote the fixture from mfq/quantize/expert_nint.py:507-578)."""
+    from tyloquant_amd.quantize import nint_quantize_expertwise
+    fx = np.load(Path(__file__).resolve().parent / "golden" / "reference_expertwise.npz")
+    W, profiles = fx[f"{case}_weight"], [tuple(p) for p in fx[f"{case}_profiles"].tolist()]
+    want = fx[f"{case}_blob"].tobytes()
+    t = O.quantize_expertwise(W, profiles)
+    assert O.pack_nint_moe(t) == want
+    assert np.concatenate([p.expert_ids for p in t.pools]).tolist() == fx[f"{case}_pool_ids"].tolist()
+    assert [len(p.expert_ids) for p in t.pools] == fx[f"{case}_pool_sizes"].tolist()
+    deq = O.dequantize_expertwise(t)
+    assert np.array_equal(deq.view(np.uint32), fx[f"{case}_deq"].view(np.uint32))
+    pools, blob = nint_quantize_expertwise(W, profiles)
+    assert blob == want
+    # the quantized tensor stays close to the weights it came from: a dropped cohort or a permuted expert would not
+    err = np.abs(deq - W).max(axis=(1, 2)) / np.abs(W).max(axis=(1, 2))
+    assert (err < 0.35).all(), err
+    with pytest.raises(ValueError):
+        O.quantize_expertwise(W, profiles[:-1])
+    with pytest.raises(ValueError):
+        nint_quantize_expertwise(W[0], profiles)

@@ -494,3 +494,32 @@ def test_nepq0_dequant_bit_exact_and_matmul(label, E, out, K, banks):
     bad[36 + 2] = 9                                    # first index width in the first table's header
     with pytest.raises(ValueError, match="table profile"):
         NepqWeight.from_blob(bytes(bad))
+
+
+@pytest.mark.parametrize("family", ["NVQ3J-512", "NEPQ0-L", "NEPQ1-S", "MXFP8"])
+def test_reserve_sizes_the_workspace_of_every_family(family):
+    """QuantLinear.reserve(max_rows) on an NVQ, an NEPQ0 (bit streams in place), an NEPQ1 and an MX linear: forward() of
+    any smaller batch afterwards leaves the workspace buffer as it is (no regrowth, so nothing to allocate under a HIP
+    graph) and still matches the oracle."""
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(515)
+    if family == "NVQ3J-512":
+        K = 192
+        dtype, blob = O.pack_tensor(synth.nvq_jsc_random(rng, 48, K, "d4_512", 2))
+        want = O.dequantize_nvq_jsc(O.unpack_nvq(blob))
+    elif family == "MXFP8":
+        K = 256
+        t = synth.mx_random(rng, "MXFP8", 128, K)
+        dtype, blob, want = "MXFP8", O.pack_mx(t), O.dequantize_mx(t)
+    else:
+        K = 192
+        t = synth.nepq_random(rng, family, 1, 48, K, 3)
+        dtype, blob = family, O.pack_nepq(t)
+        want = O.dequantize_nepq(O.unpack_nepq(blob))[0]
+    lin = R.load_quant_linear(dtype, blob)
+    lin.reserve(70)
+    buf = lin.weight._ws.buf
+    for M in (1, 5, 17, 40, 70):
+        x, xf = _x(rng, M, K)
+        _check(lin(x).cpu().numpy(), O.linear_forward_f64(want, xf))
+        assert lin.weight._ws.buf is buf, (family, M)

@@ -1,4 +1,4 @@
-"""NINT weight-only tensor quantizer (host side, numpy), processed in row chunks.
+"""NINT weight-only tensor quantizer and its expert-wise form (host side, numpy), processed in row chunks.
 
 Mirrors nint_quant.quantize with importance=None (mfq/quantize/nint_quant.py:745-823, 883-893) and
 its per-group affine search make_qkx2 (mfq/formats/nint.py:119-174): per neuron row, groups of `gs`
@@ -88,3 +88,32 @@ def nint_quantize(weight, bits: int = 4, gs: int = 24, sub_bits: int = 6, row_ch
         ns[sl], nm[sl], ss[sl], sm[sl], q[sl] = d, dm, sub_s, sub_m, codes
     return {"ns": ns, "nm": nm, "ss": ss, "sm": sm, "q": q, "bits": bits, "gs": gs, "sub_bits": sub_bits,
             "neuron_len": K}
+
+
+def nint_quantize_expertwise(weight, profiles, row_chunk: int = 512):
+    """weight [experts, out, K] fp32 and one (bits, groupsize, sub_bits) per expert -> (pools, blob).
+
+    Mirrors quantize_expertwise for NINT precisions (mfq/quantize/expert_nint.py:507-578): the experts of one precision
+    form a cohort -- cohorts in the order their precision first appears, experts ascending inside a cohort -- whose rows
+    are flattened to [n * out, K] and quantized like a dense tensor.  `pools` is a list of (expert_ids int32,
+    dtype string, dict as nint_quantize returns); `blob` the NIM2 payload holding them (mfq/formats/io.py:304-336).
+    """
+    from . import formats as F
+
+    W = np.asarray(weight, dtype=np.float32)
+    if W.ndim != 3:
+        raise ValueError("expert-wise quantization expects [experts, out, in]")
+    E, out, K = W.shape
+    profiles = [tuple(int(v) for v in p) for p in profiles]
+    if len(profiles) != E:
+        raise ValueError(f"received {len(profiles)} precision descriptors for {E} experts")
+    cohorts: dict = {}
+    for e, prof in enumerate(profiles):
+        cohorts.setdefault(prof, []).append(e)
+    pools, packed = [], []
+    for (bits, gs, sub_bits), members in cohorts.items():
+        ids = np.asarray(members, dtype=np.int32)
+        r = nint_quantize(W[ids].reshape(ids.size * out, K), bits, gs, sub_bits, row_chunk)
+        pools.append((ids, f"NINT{bits}", r))
+        packed.append((ids, f"NINT{bits}", F.nint_blob(bits, sub_bits, gs, K, r["ns"], r["nm"], r["ss"], r["sm"], r["q"])))
+    return pools, F.nintm_blob(E, out, K, packed)

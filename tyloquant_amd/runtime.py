@@ -365,7 +365,9 @@ class QuantLinear:
                  "nint8z": lambda M: lib.mfq_hip_nint8z_gemm_workspace_bytes(C.byref(w.desc), M),
                  "nvq": lambda M: (lib.mfq_hip_nvqs_gemm_workspace_bytes if type(w).__name__ == "NvqsWeight"
                                    else lib.mfq_hip_nvq_gemm_workspace_bytes)(C.byref(w.desc), M),
-                 "nepq": lambda M: lib.mfq_hip_nepq_gemm_workspace_bytes(C.byref(w.desc), w.out_per_expert, M),
+                 # NEPQ0-S / NEPQ0-L keep their bit streams (an NvqsDesc) and run on the stream kernels' row-range form
+                 "nepq": lambda M: (lib.mfq_hip_nvqs_gemm_rows_workspace_bytes if getattr(w, "streams", False)
+                                    else lib.mfq_hip_nepq_gemm_workspace_bytes)(C.byref(w.desc), w.out_per_expert, M),
                  "mx": lambda M: lib.mfq_hip_mx_gemm_rows_workspace_bytes(w.neuron_len, w.out, M)}[self.kind]
         sizes = set(range(1, min(max_rows, 512) + 1)) | set(range(576, max_rows, 64)) | {max_rows}
         need = max((int(query(M)) for M in sizes if M > 0), default=0)

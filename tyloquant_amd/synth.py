@@ -8,6 +8,7 @@ rows, which leaves the value distribution and every byte count unchanged.
 from __future__ import annotations
 
 import math
+import struct
 from pathlib import Path
 
 import numpy as np
@@ -41,6 +42,38 @@ def nint_linear_blob(seed, out, K, bits, gs, sub_bits, sigma=0.02, slab_rows=Non
         for k in ("ns", "nm", "ss", "sm", "q"):
             r[k] = np.concatenate([r[k]] * reps, axis=0)[:out]
     return f"NINT{bits}", F.nint_blob(bits, sub_bits, gs, K, r["ns"], r["nm"], r["ss"], r["sm"], r["q"])
+
+
+def nintm_quantized_blob(seed, n_experts, out_per_expert, K, expert_bits, sigma=0.02, slab_rows=1024):
+    """(blob, pools) of an expert-wise NINTM tensor of the BASELINE config-4 kind: expert e at MOE_PROFILES[expert_bits[e]].
+
+    One slab of N(0, sigma) weights per precision goes through the expert-wise quantizer (nint_quantize_expertwise on a
+    [precisions, slab_rows, K] tensor); each cohort of the result is then tiled over its experts -- every stream of a
+    NINT payload is the slab's stream repeated, because a slab ends on a byte boundary of every stream -- so that byte
+    counts, value distribution and cohort order are those of quantizing the full tensor, at the cost of repeated rows.
+    `pools` = [(expert_ids, NINT payload of the cohort)], in the container's order."""
+    from .quantize import nint_quantize_expertwise
+    expert_bits = [int(b) for b in expert_bits]
+    order = list(dict.fromkeys(expert_bits))           # precisions in order of first appearance, as the quantizer groups
+    rows = min(out_per_expert, slab_rows)
+    if out_per_expert % rows or rows % 8:
+        raise ValueError("the slab must divide the expert's rows and end on a byte boundary of every stream")
+    rng = np.random.default_rng(seed)
+    W = (rng.standard_normal((len(order), rows, K)) * sigma).astype(np.float32)
+    small, _ = nint_quantize_expertwise(W, [MOE_PROFILES[b] for b in order])
+    pools = []
+    for (_, dtype, r), b in zip(small, order):
+        ids = np.asarray([e for e, v in enumerate(expert_bits) if v == b], dtype=np.int32)
+        reps = len(ids) * (out_per_expert // rows)
+        out = reps * rows
+        bits, gs, sb = MOE_PROFILES[b]
+        ng = r["q"].shape[1]
+        head = F._NINT_HDR.pack(bits, sb, gs, 0, K) + struct.pack("<I", 2) + struct.pack("<2q", out, K) + \
+            struct.pack("<II", out, ng)
+        parts = [np.ascontiguousarray(r["ns"], dtype=np.float16).tobytes(), np.ascontiguousarray(r["nm"], dtype=np.float16).tobytes(),
+                 F.pack_bitstream(r["ss"], sb), F.pack_bitstream(r["sm"], sb), F.pack_bitstream(r["q"], bits)]
+        pools.append((ids, dtype, b"".join([head] + [p * reps for p in parts])))
+    return F.nintm_blob(n_experts, out_per_expert, K, pools), [(ids, payload) for ids, _, payload in pools]
 
 
 def d4_512_banks(banks=2) -> np.ndarray:
