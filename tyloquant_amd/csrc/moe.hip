@@ -679,13 +679,15 @@ struct MoeDecodeShape {
 static bool moe_decode_shape(MoePools &P, int n_slots, int max_steps, int out_per_expert, int n_rows, int swiglu,
                              MoeDecodeShape &sh) {
     static const int env_off = tune_env("MFQ_MOE_SPLIT", 1) == 0;
-    static const int env_w = tune_env("MFQ_MOE_DEC_WAVES", 8);
+    static const int env_w = tune_env("MFQ_MOE_DEC_WAVES", 3);
     static const int env_rbw = tune_env("MFQ_MOE_DEC_RBW", 0);
     if (env_off || n_rows > 65535) return false;
     const int rbe = out_per_expert / 16;
-    // At most eight waves split the K steps (two blocks fit a CU at the kernel's 128 registers; measured best at
-    // T = 1: 54 us per layer against 60-62 us with 11..16 waves); a wave takes more (row-block, step) items while
-    // the grid keeps about gemv_target_waves() waves.  With the fused SwiGLU a block always takes two row-blocks:
+    // Three waves split the K steps: a launch has one block per (row-block group, row), thousands of them, and small
+    // blocks let five or six sit on a compute unit at the kernel's 128 registers, so that the grid runs in fewer
+    // rounds (config-4 layer at T = 1 / 2 / 4: 50 / 72 / 118 us against 57 / 87 / 149 us with eight waves and
+    // 64 / 101 / 178 us with five).  A wave takes more (row-block, step) items while the grid keeps
+    // about gemv_target_waves() waves.  With the fused SwiGLU a block always takes two row-blocks:
     // gate and up.
     const int nwaves = max_steps < env_w ? max_steps : env_w;
     const int spw_max = static_cast<int>(ceil_div(max_steps, nwaves));

@@ -13,6 +13,8 @@
 // In the GEMV the codebook banks (as ready-made activation-typed pairs), a 128-entry table that
 // expands a sign mask (with its parity bit) into XOR masks, and the scale LUT all stay in LDS; the small-batch
 // matrix-core kernel keeps the signed table (banks * entries * 16 vectors of 8 bytes) in LDS instead.
+#include <type_traits>
+
 #include "common.hpp"
 #include "gemv_common.hpp"
 #include "nint_prefill.hpp"
@@ -652,6 +654,228 @@ __global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k_first, const ui
     }
 }
 
+// ---- one or two rows with the signed table in LDS and the activations in registers ------------------------------
+// The block frame of nvq_signed_kernel (one block per compute unit with RPB consecutive row-blocks, its waves split the
+// K steps, SPW steps per wave) for one or two activation rows, on the vector ALUs: a unit (24 weights of the neuron of
+// lane (r, kb)) is six 8-byte reads of signed fp16 vectors out of the LDS table and twelve packed dot products whose
+// activation pair comes out of another lane's register -- the 16 lanes of a DPP row share a group, lane r of the row
+// keeps pair r of it (12 pairs) and v_dot2c_f32_f16_dpp ... row_newbcast:i fetches pair i.  So the activations of a
+// step are four registers per row instead of 48 registers of matrix-core fragments, the unit's scale is one multiply
+// of its dot product, and the registers that frees hold a whole item's 24 gathers at once: an item costs two LDS round
+// trips (states, then all vectors) instead of eight.
+// Items are walked row-block by row-block (steps inside), item (row-block i, step ls) in ring slot ls (SPW >= 2) or
+// i % 2 (SPW = 1), each slot refilled with the same step of the next row-block (the row-block after next).
+// LDS map (bytes): [signed table: banks*entries*128][state table: 16 x {lut f32, bank base}][red: RPB * waves * MB * 16 f32]
+// [raw codebook entries as fp16 pairs: banks*entries*8]
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+template <int XF16, int MB, int SPW>
+__global__ __launch_bounds__(1024) void nvq_bcast_kernel(NvqK k_first, const uint8_t *__restrict__ w_first,
+                                                         const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                         float *__restrict__ y_first, int64_t ldy, int rpb, NvqSecond s2) {
+    constexpr int RING = SPW == 1 ? 2 : SPW;
+    const bool second = static_cast<int>(blockIdx.x) >= s2.blocks0;
+    const NvqK &k = second ? s2.k : k_first;
+    const uint8_t *__restrict__ w = second ? s2.w : w_first;
+    float *__restrict__ y = y_first + (second ? s2.col : 0);
+    const int bx = static_cast<int>(blockIdx.x) - (second ? s2.blocks0 : 0);
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, nwaves = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ncb = k.banks * k.entries;
+    uint32_t *stab = lds + ncb * 32;
+    float *red = reinterpret_cast<float *>(stab + 32);
+    const uint32_t lds_base = static_cast<uint32_t>(
+        reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint32_t *)lds));
+
+    const int rb_first = bx * rpb;
+    const int nrb = min(rpb, k.n_rowblocks - rb_first);
+    const int m0 = static_cast<int>(blockIdx.y) * MB;
+    const int r = lane & 15, kb = lane >> 4;
+    const int s0 = wave * SPW;
+    const int n = min(k.nsteps, s0 + SPW) - s0;  // steps of this wave, may be <= 0
+    const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes);
+    const __amdgpu_buffer_rsrc_t win =
+        wave_window(w + static_cast<int64_t>(rb_first) * k.rowblock_bytes + static_cast<int64_t>(s0) * sb,
+                    n > 0 ? (nrb - 1) * rbb + n * sb : 0u);
+    struct Item {
+        u32x2_t q[4];
+        u32x4_t c;
+    };
+    Item ring[RING];
+    auto wload = [&](int ls, int i, Item &it) {  // step s0 + ls of row-block rb_first + i; zeros when there is none
+        const uint32_t off = ls < n && i < nrb ? i * rbb + ls * sb : kNoStep;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) it.q[j] = __builtin_amdgcn_raw_buffer_load_b64(win, off + (j * 64 + lane) * 8, 0, 2);
+        it.c = __builtin_amdgcn_raw_buffer_load_b128(win, off + 2048 + lane * 16, 0, 2);
+    };
+    // requests in order of use: codebook entries, state tables, activations, anchors, the first items
+    const float *lut = reinterpret_cast<const float *>(w + k.tables_off);
+    const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+    const uint32_t *cb = bfs + 16;  // 4 int8 magnitudes per entry
+    uint32_t craw[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) craw[t] = cb[min(tid + t * static_cast<int>(blockDim.x), ncb - 1)];
+    const float lutv = lut[tid & 15];
+    const uint32_t bankv = bfs[tid & 15];
+    // activations: lane (r, kb) asks for pair r (of 12) of group 16 (s0 + ls) + 4 j + kb of every row
+    uint32_t xraw[MB][SPW][4];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        const bool row_ok = m0 + m < M;
+        const __amdgpu_buffer_rsrc_t wx = wave_window(reinterpret_cast<const uint8_t *>(x + static_cast<int64_t>(row_ok ? m0 + m : 0) * ldx),
+                                                      row_ok ? static_cast<uint32_t>(k.neuron_len) * 2u : 0u);
+#pragma unroll
+        for (int ls = 0; ls < SPW; ++ls)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t off = static_cast<uint32_t>(((s0 + ls) * 16 + 4 * j + kb) * 12 + r) * 4u;
+                xraw[m][ls][j] = __builtin_amdgcn_raw_buffer_load_b32(wx, (ls < n && r < 12) ? off : kNoStep, 0, 0);
+            }
+    }
+    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
+    if constexpr (SPW == 1) {
+        wload(0, 0, ring[0]);
+        wload(0, 1, ring[1]);
+    } else {
+#pragma unroll
+        for (int ls = 0; ls < SPW; ++ls) wload(ls, 0, ring[ls]);
+    }
+    // tables: the entries as two fp16 pairs each, then the signed table (see nvq_signed_kernel)
+    u32x2_t *cbh = reinterpret_cast<u32x2_t *>(red + rpb * nwaves * MB * 16);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        if (tid + t * static_cast<int>(blockDim.x) < ncb) {
+            uint32_t h[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) h[b] = f32_to_f16_rne(static_cast<float>((craw[t] >> (8 * b)) & 0xffu));
+            cbh[tid + t * blockDim.x] = u32x2_t{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        }
+    }
+    if (tid < 16) {
+        stab[2 * tid] = __float_as_uint(lutv);
+        stab[2 * tid + 1] = lds_base + bankv * k.entries * 128;
+    }
+    __syncthreads();  // raw entries
+    for (int c = tid; c < ncb * 8; c += blockDim.x) {
+        const u32x2_t e = cbh[c >> 3];
+        const uint32_t p0 = e.x, p1 = e.y;
+        const uint32_t n0 = 2u * (c & 7), n1 = n0 + 1u;
+        u32x4_t v;
+        v.x = p0 ^ (((n0 & 1u) << 15) | ((n0 & 2u) << 30));
+        v.y = p1 ^ (((n0 & 4u) << 13) | ((n0 & 8u) << 28));
+        v.z = p0 ^ (((n1 & 1u) << 15) | ((n1 & 2u) << 30));
+        v.w = p1 ^ (((n1 & 4u) << 13) | ((n1 & 8u) << 28));
+        *reinterpret_cast<u32x4_t *>(lds + 4 * c) = v;
+    }
+    const uint32_t stab_base = lds_base + ncb * 128;
+    // the activation pairs as fp16 (bf16 rows: times the wave's power of two that brings its slice near 2^12)
+    uint32_t xh[MB][SPW][4];
+    float xinv[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        float sc = 1.f;
+        xinv[m] = 1.f;
+        if constexpr (!XF16) {
+            uint32_t mx = 0;
+#pragma unroll
+            for (int ls = 0; ls < SPW; ++ls)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) mx = absmax_bf16(mx, xraw[m][ls][j]);
+            sc = slice_scale(wave_max_u32(mx), xinv[m]);
+        }
+#pragma unroll
+        for (int ls = 0; ls < SPW; ++ls)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xh[m][ls][j] = XF16 ? xraw[m][ls][j] : to_h2_scaled(xraw[m][ls][j], sc);
+    }
+    __syncthreads();  // tables
+
+    // one item: the states of its four units, then all 24 vectors at once, then the dot products
+    auto process = [&](Item &it, uint32_t noff, const uint32_t (&xs)[MB][SPW][4], auto LS, float (&acc)[MB]) {
+        constexpr int ls = decltype(LS)::value;  // compile time: the pair register goes into the dot products as it is
+        const u32x4_t uc4 = it.c;
+        it.c = __builtin_amdgcn_raw_buffer_load_b128(win, noff + 2048 + lane * 16, 0, 2);
+        const uint32_t ucv[4] = {uc4.x, uc4.y, uc4.z, uc4.w};
+        u32x2_t stv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            stv[j] = *reinterpret_cast<lds_u32x2_ptr>(stab_base + (__builtin_rotateleft32(ucv[j], 6) & 0x78u));
+        u32x2_t vec[4][6];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t ua = it.q[j].x, ub = it.q[j].y, uc = ucv[j];
+            it.q[j] = __builtin_amdgcn_raw_buffer_load_b64(win, noff + (j * 64 + lane) * 8, 0, 2);
+            const uint32_t base = stv[j].y;
+            const uint32_t off[6] = {and_or(ua, 0xfff8u, base), and_or(ua >> 16, 0xfff8u, base),
+                                     and_or(ub, 0xfff8u, base), and_or(ub >> 16, 0xfff8u, base),
+                                     and_or(uc, 0xfff8u, base), and_or(uc >> 13, 0xfff8u, base)};
+#pragma unroll
+            for (int t = 0; t < 6; ++t) vec[j][t] = *reinterpret_cast<lds_u32x2_ptr>(off[t]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float sc = __uint_as_float(stv[j].x);
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                float a = 0.f;
+                const uint32_t xv = xs[m][ls][j];
+                a = dot2_bcast4<0, false>(a, xv, vec[j][0].x, vec[j][0].y, vec[j][1].x, vec[j][1].y);
+                a = dot2_bcast4<4, false>(a, xv, vec[j][2].x, vec[j][2].y, vec[j][3].x, vec[j][3].y);
+                a = dot2_bcast4<8, true>(a, xv, vec[j][4].x, vec[j][4].y, vec[j][5].x, vec[j][5].y);
+                acc[m] = fmaf(sc, a, acc[m]);
+            }
+        }
+    };
+    // the waves' partial sums of row-block i: slot (i * nwaves + wave) * MB + m, 16 neurons each
+    auto park = [&](int i, float (&acc)[MB]) {
+        const float av = anchors[(rb_first + min(i, nrb - 1)) * 16 + r];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            const float v = reduce_kb4(acc[m]) * av * xinv[m];
+            if (lane < 16) red[((i * nwaves + wave) * MB + m) * 16 + lane] = v;
+            acc[m] = 0.f;
+        }
+    };
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = 0.f;
+    if constexpr (SPW == 1) {
+        for (int i = 0; i < rpb; i += 2) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int ii = i + u;
+                if (ii < rpb) {  // block-uniform
+                    if (n > 0 && ii < nrb)
+                        process(ring[u], ii + 2 < nrb ? (ii + 2) * rbb : kNoStep, xh, std::integral_constant<int, 0>{}, acc);
+                    park(ii, acc);
+                }
+            }
+        }
+    } else {
+        for (int i = 0; i < rpb; ++i) {
+            static_for<SPW>([&](auto LS) {
+                constexpr int ls = decltype(LS)::value;
+                if (ls < n && i < nrb) process(ring[ls], i + 1 < nrb ? (i + 1) * rbb + ls * sb : kNoStep, xh, LS, acc);
+            });
+            park(i, acc);
+        }
+    }
+    __syncthreads();
+    for (int o = tid; o < nrb * MB * 16; o += blockDim.x) {
+        const int rr = o & 15, m = (o >> 4) % MB, i = (o >> 4) / MB;
+        float sum = 0.f;
+        for (int wv = 0; wv < nwaves; ++wv) sum += red[((i * nwaves + wv) * MB + m) * 16 + rr];
+        const int row = (rb_first + i) * 16 + rr;
+        if (m0 + m < M && row < k.out) y[static_cast<int64_t>(m0 + m) * ldy + row] = sum;
+    }
+}
+
 // ---- prefill: block-tiled MFMA GEMM, weight fragments built from the codebooks in LDS ----------------------
 // Block = 8 waves side by side on 8 * NB row-blocks, wave tile MT * 16 tokens x NB * 16 neurons.  Activations as in
 // the NINT prefill kernel: fp16 rows scaled per token (x_prep), the 96 k-values of a sub-step (unit j of a step) staged
@@ -984,6 +1208,54 @@ static int nvq_launch_signed(const NvqK &k, const uint8_t *w, const uint16_t *x,
     }
 }
 
+// One or two rows on nvq_bcast_kernel: the signed table fits the LDS, the rows can be fetched pair by pair (4-byte
+// aligned, even K), at most three steps per wave (four would spill), and at least four waves (the table build spreads
+// over them).
+static bool nvq_bcast_capable(const NvqK &k, const void *x, int64_t ldx, int M, int more_rowblocks = 0) {
+    static const int off = tune_env("MFQ_NVQ_BCAST_OFF", 0);
+    const int rpb = nvq_signed_rpb(k, more_rowblocks);
+    const int spw = static_cast<int>(ceil_div(k.nsteps, 16));
+    return !off && M >= 1 && M <= 2 && static_cast<int64_t>(k.banks) * k.entries * 128 <= 131072 && rpb <= 8 && spw <= 3 &&
+           ceil_div(k.nsteps, spw) >= 4 && k.neuron_len % 2 == 0 && (M == 1 || ldx % 2 == 0) &&
+           (reinterpret_cast<uintptr_t>(x) & 3) == 0 && rpb * k.rowblock_bytes < (1ll << 31);
+}
+template <int XF16, int MB, int SPW>
+static int nvq_launch_bcast_as(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                               hipStream_t st, const NvqSecond *second) {
+    const int nwaves = static_cast<int>(ceil_div(k.nsteps, SPW));
+    const int rpb = nvq_signed_rpb(k, second ? second->k.n_rowblocks : 0);
+    const int blocks0 = static_cast<int>(ceil_div(k.n_rowblocks, rpb));
+    NvqSecond s2{k, w, blocks0, 0};
+    int blocks = blocks0;
+    size_t ncb = static_cast<size_t>(k.banks) * k.entries;
+    if (second) {
+        s2 = *second;
+        s2.blocks0 = blocks0;
+        blocks += static_cast<int>(ceil_div(s2.k.n_rowblocks, rpb));
+        if (static_cast<size_t>(s2.k.banks) * s2.k.entries > ncb) ncb = static_cast<size_t>(s2.k.banks) * s2.k.entries;
+    }
+    const size_t lds = ncb * 136 + 128 + static_cast<size_t>(rpb) * nwaves * MB * 64;
+    auto kern = nvq_bcast_kernel<XF16, MB, SPW>;
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), lds, "nvq_bcast")) return rc;
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks), static_cast<unsigned>(ceil_div(M, MB))), dim3(64 * nwaves), lds,
+                       st, k, w, x, ldx, M, y, ldy, rpb, s2);
+    return check_launch("nvq_bcast");
+}
+template <int XF16>
+static int nvq_launch_bcast(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                            hipStream_t st, const NvqSecond *s2 = nullptr) {
+    const int spw = static_cast<int>(ceil_div(k.nsteps, 16));
+#define MFQ_NVQ_BCAST(MB)                                                                                   \
+    switch (spw) {                                                                                          \
+    case 1: return nvq_launch_bcast_as<XF16, MB, 1>(k, w, x, ldx, M, y, ldy, st, s2);                       \
+    case 2: return nvq_launch_bcast_as<XF16, MB, 2>(k, w, x, ldx, M, y, ldy, st, s2);                       \
+    default: return nvq_launch_bcast_as<XF16, MB, 3>(k, w, x, ldx, M, y, ldy, st, s2);                      \
+    }
+    if (M == 1) { MFQ_NVQ_BCAST(1) }
+    MFQ_NVQ_BCAST(2)
+#undef MFQ_NVQ_BCAST
+}
+
 template <int XF16>
 static int nvq_mfma_any(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                         hipStream_t st) {
@@ -1025,6 +1297,9 @@ static int nvq_gemv_any(const mfq_nvq_desc *d, const void *weight, const void *x
     const NvqK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
+    if (nvq_bcast_capable(k, x, ldx, M))
+        return x_dtype == MFQ_X_F16 ? nvq_launch_bcast<1>(k, w, xp, ldx, M, y, ldy, st)
+                                    : nvq_launch_bcast<0>(k, w, xp, ldx, M, y, ldy, st);
     if (nvq_stream_capable(k) && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
         return x_dtype == MFQ_X_F16 ? nvq_mfma_any<1>(k, w, xp, ldx, M, y, ldy, st) : nvq_mfma_any<0>(k, w, xp, ldx, M, y, ldy, st);
     int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);
@@ -1146,6 +1421,14 @@ extern "C" int mfq_hip_nvq_gemv_multi2(const mfq_nvq_desc *d0, const void *weigh
                 "nvq_gemv_multi2: ldx/ldy smaller than the tensors");
     const NvqK k0 = to_k(d0), k1 = to_k(d1);
     hipStream_t st = as_stream(stream);
+    if (nvq_bcast_capable(k0, x, ldx, M, k1.n_rowblocks) && nvq_bcast_capable(k1, x, ldx, M, k0.n_rowblocks) &&
+        nvq_bcast_capable(k0, x, ldx, M) && nvq_bcast_capable(k1, x, ldx, M)) {  // what each tensor's own call would run
+        const NvqSecond s2{k1, static_cast<const uint8_t *>(weight1), 0, d0->out};
+        const uint8_t *w0 = static_cast<const uint8_t *>(weight0);
+        const uint16_t *xp = static_cast<const uint16_t *>(x);
+        return x_dtype == MFQ_X_F16 ? nvq_launch_bcast<1>(k0, w0, xp, ldx, M, y, ldy, st, &s2)
+                                    : nvq_launch_bcast<0>(k0, w0, xp, ldx, M, y, ldy, st, &s2);
+    }
     const bool aligned = ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
     if (aligned && nvq_stream_capable(k0) && nvq_stream_capable(k1) && nvq_signed_capable(k0, M, k1.n_rowblocks) &&
         nvq_signed_capable(k1, M, k0.n_rowblocks)) {

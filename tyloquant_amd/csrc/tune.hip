@@ -31,6 +31,7 @@ Knob g_knobs[] = {
     {"MFQ_PREFILL_BIG", "experimental 128 x 384 prefill tiles (0 = off)", 0, false},
     {"MFQ_NVQ_NB", "row-blocks per wave of the NVQ streaming kernel (0 = by shape)", 0, false},
     {"MFQ_NVQ_STREAM_MAX_M", "rows up to which NVQ streams instead of the prefill kernel (0 = cost model)", 0, false},
+    {"MFQ_NVQ_BCAST_OFF", "1 = one and two NVQ rows on the matrix-core signed-table kernel instead of the vector-ALU one", 0, false},
     {"MFQ_NVQ_SIGNED_OFF", "1 = NVQ small batches on the older streaming kernel", 0, false},
     {"MFQ_NVQ_SIGNED_MAX_M", "rows up to which the NVQ signed-table kernel runs", 0, false},
     {"MFQ_NVQ_RING", "weight ring depth of the five-row-block NVQ kernel", 0, false},
