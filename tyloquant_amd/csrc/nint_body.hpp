@@ -346,6 +346,14 @@ __device__ __forceinline__ float dot2_bcast4(float acc, uint32_t x, uint32_t w0,
     return acc;
 }
 
+// A register that a vector-ALU instruction has just written may be read through DPP only two issue slots later, and the
+// compiler, which cannot see the DPP reads inside dot2_bcast4, is free to sink the instruction that produces an
+// activation register right in front of them.  Every register that goes into dot2_bcast4 as x passes through here
+// once after it is computed: the statement counts as its last writer and carries the two slots.
+__device__ __forceinline__ void dpp_source_ready(uint32_t &a, uint32_t &b, uint32_t &c, uint32_t &d) {
+    asm volatile("s_nop 1" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+
 // sum over the 16 lanes of a DPP row, left in every lane of the row
 __device__ __forceinline__ float row_allsum(float v) {
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xF, 0xF, true));  // row_ror:8
@@ -413,6 +421,8 @@ __device__ __forceinline__ void xreg_stage(const uint32_t (&raw)[MB][4], const f
             xi.xg[m][j] = row_allsum(ps * ci);
             xi.nt[m][j] = -row_allsum(ps * U::Bias::bw(r));
         }
+#pragma unroll
+    for (int m = 0; m < MB; ++m) dpp_source_ready(xi.x[m][0], xi.x[m][1], xi.x[m][2], xi.x[m][3]);
 }
 
 // One block = `rbw` consecutive 16-neuron row-blocks starting at `rb0` of the tensor at `w`; its waves
@@ -499,13 +509,7 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     uint32_t q0[4][D], q1[4][D], q2[4][D], t0, t1, t2;
     u32x2_t c0, c1, c2;
     MFQ_ISSUE(q0, t0, c0)
-#ifdef MFQ_GEMV_RR
-    if constexpr (!RING) { asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
-#endif
     MFQ_ISSUE(q1, t1, c1)
-#ifdef MFQ_GEMV_RR
-    if constexpr (!RING) { asm volatile("" ::: "memory"); __builtin_amdgcn_s_barrier(); asm volatile("" ::: "memory"); }
-#endif
     MFQ_ISSUE(q2, t2, c2)
     float xinv[MB];  // bf16 rows are staged times a per-wave power of two; the sums are scaled back when they are parked
     xp.template finish<XF16, MB>(xg);
@@ -518,7 +522,7 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     int crb = 0, cs = 0;
 #define MFQ_COMPUTE(Q, T, C)                                                                              \
     {                                                                                                     \
-        MFQ_LAB_COMPUTE(Q, T, C)                                                                          \
+        nint_compute_step<U, MB>(Q, T, C, cs * 16 + kb, xs, xsum, npairs, ngl, accS, accM);               \
         if (++cs >= n) {                                                                                  \
             float a_s = ns[0], a_m = nm[0];                                                               \
             _Pragma("unroll") for (int i = 1; i < kMaxRbw; ++i) if (crb == i) { a_s = ns[i]; a_m = nm[i]; } \
@@ -532,16 +536,6 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
             ++crb;                                                                                        \
         }                                                                                                 \
     }
-#ifdef MFQ_LAB_NOCOMPUTE
-#define MFQ_LAB_COMPUTE(Q, T, C)                                                                       \
-    {                                                                                                  \
-        uint32_t a_ = T ^ C.x ^ C.y;                                                                   \
-        _Pragma("unroll") for (int j_ = 0; j_ < 4; ++j_) _Pragma("unroll") for (int d_ = 0; d_ < D; ++d_) a_ ^= Q[j_][d_]; \
-        accS[0] += __uint_as_float(a_ & 0x3fffffffu);                                                  \
-    }
-#else
-#define MFQ_LAB_COMPUTE(Q, T, C) nint_compute_step<U, MB>(Q, T, C, cs * 16 + kb, xs, xsum, npairs, ngl, accS, accM);
-#endif
     const int items = nrb * n;
     if (n <= 0) {  // a wave beyond the last step still owes its (zero) partial sums
         float z[MB];

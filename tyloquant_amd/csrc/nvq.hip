@@ -663,10 +663,17 @@ __global__ __launch_bounds__(1024) void nvq_signed_kernel(NvqK k_first, const ui
 // step are four registers per row instead of 48 registers of matrix-core fragments, the unit's scale is one multiply
 // of its dot product, and the registers that frees hold a whole item's 24 gathers at once: an item costs two LDS round
 // trips (states, then all vectors) instead of eight.
-// Items are walked row-block by row-block (steps inside), item (row-block i, step ls) in ring slot ls (SPW >= 2) or
-// i % 2 (SPW = 1), each slot refilled with the same step of the next row-block (the row-block after next).
+// Items are walked row-block by row-block (steps inside), item (row-block i, step ls) in ring slot (i % DEPTH) * SPW +
+// ls, each slot refilled -- after the last read of what it holds -- with the same step DEPTH row-blocks further on.
+// What bounds the kernel is the LDS: 128 KB of table writes (1.3 us at the 64 bytes a cycle a compute unit's LDS
+// takes) and 28 LDS instructions an item (24 of them 8-byte gathers at random addresses, about 7 cycles each against 4
+// without bank conflicts) -- on 17408 x 5120, 70 items a block, 6.5 us of LDS time after a table that stands at
+// 3.4 us, in a launch of 11.1 us.  A compute unit also keeps only about 64 memory requests in flight, whatever their
+// size, hands their data back in the order they were issued whichever wave they are for, and a wave whose request does
+// not fit waits at the request: asking for more than one item per wave before the tables stand only delays the waves
+// that have to build them (tables at 4.8 us with two items ahead, at 7.1 us with four).
 // LDS map (bytes): [signed table: banks*entries*128][state table: 16 x {lut f32, bank base}][red: RPB * waves * MB * 16 f32]
-// [raw codebook entries as fp16 pairs: banks*entries*8]
+// [anchors: RPB * 16 f32][raw codebook entries as fp16 pairs: banks*entries*8]
 template <int N, class F>
 __device__ __forceinline__ void static_for(F &&f) {
     if constexpr (N > 0) {
@@ -678,7 +685,10 @@ template <int XF16, int MB, int SPW>
 __global__ __launch_bounds__(1024) void nvq_bcast_kernel(NvqK k_first, const uint8_t *__restrict__ w_first,
                                                          const uint16_t *__restrict__ x, int64_t ldx, int M,
                                                          float *__restrict__ y_first, int64_t ldy, int rpb, NvqSecond s2) {
-    constexpr int RING = SPW == 1 ? 2 : SPW;
+    // DEPTH row-blocks of the wave's steps are in flight in the walk, PRE of them requested before the tables are built
+    // (17408 x 5120, DEPTH/PRE: 2/1 13.7 us, 2/2 14.3, 3/1 14.5, 4/2 15.5, 1/1 14.7)
+    constexpr int DEPTH = SPW <= 2 ? 2 : 1, RING = SPW * DEPTH;
+    constexpr int PRE = 1;
     const bool second = static_cast<int>(blockIdx.x) >= s2.blocks0;
     const NvqK &k = second ? s2.k : k_first;
     const uint8_t *__restrict__ w = second ? s2.w : w_first;
@@ -714,15 +724,23 @@ __global__ __launch_bounds__(1024) void nvq_bcast_kernel(NvqK k_first, const uin
         for (int j = 0; j < 4; ++j) it.q[j] = __builtin_amdgcn_raw_buffer_load_b64(win, off + (j * 64 + lane) * 8, 0, 2);
         it.c = __builtin_amdgcn_raw_buffer_load_b128(win, off + 2048 + lane * 16, 0, 2);
     };
-    // requests in order of use: codebook entries, state tables, activations, anchors, the first items
-    const float *lut = reinterpret_cast<const float *>(w + k.tables_off);
-    const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
-    const uint32_t *cb = bfs + 16;  // 4 int8 magnitudes per entry
-    uint32_t craw[4];
+    // A compute unit hands back what its waves asked for in the order they asked, whichever wave it is for.  The first
+    // wave of the block therefore asks for everything the tables are made of (codebook entries, state table, anchors)
+    // before any wave asks for weights: fetched by all waves, each wave's share would arrive behind the weights the
+    // waves launched before it have requested, and the tables -- which every wave waits for -- with the last of them.
+    const uint8_t *tb = w + k.tables_off;
+    u32x4_t craw[4] = {};   // wave 0: entries 4 * (t * 64 + lane) .. + 3, four int8 magnitudes each
+    uint32_t lutv = 0, bankv = 0;
+    u32x2_t anc_v = {0, 0};
+    if (wave == 0) {
+        const __amdgpu_buffer_rsrc_t wt = wave_window(tb, 128u + static_cast<uint32_t>(ncb) * 4u);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) craw[t] = cb[min(tid + t * static_cast<int>(blockDim.x), ncb - 1)];
-    const float lutv = lut[tid & 15];
-    const uint32_t bankv = bfs[tid & 15];
+        for (int t = 0; t < 4; ++t) craw[t] = __builtin_amdgcn_raw_buffer_load_b128(wt, 128u + static_cast<uint32_t>(t * 64 + lane) * 16u, 0, 0);
+        lutv = __builtin_amdgcn_raw_buffer_load_b32(wt, lane < 16 ? lane * 4u : kNoStep, 0, 0);
+        bankv = __builtin_amdgcn_raw_buffer_load_b32(wt, lane < 16 ? 64u + lane * 4u : kNoStep, 0, 0);
+        const __amdgpu_buffer_rsrc_t wa = wave_window(w + k.anchors_off + static_cast<int64_t>(rb_first) * 64, static_cast<uint32_t>(nrb) * 64u);
+        anc_v = __builtin_amdgcn_raw_buffer_load_b64(wa, lane * 8u, 0, 0);
+    }
     // activations: lane (r, kb) asks for pair r (of 12) of group 16 (s0 + ls) + 4 j + kb of every row
     uint32_t xraw[MB][SPW][4];
 #pragma unroll
@@ -738,28 +756,36 @@ __global__ __launch_bounds__(1024) void nvq_bcast_kernel(NvqK k_first, const uin
                 xraw[m][ls][j] = __builtin_amdgcn_raw_buffer_load_b32(wx, (ls < n && r < 12) ? off : kNoStep, 0, 0);
             }
     }
-    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
-    if constexpr (SPW == 1) {
-        wload(0, 0, ring[0]);
-        wload(0, 1, ring[1]);
-    } else {
+    // the first PRE row-blocks' items go out now, the rest of the ring once the tables stand
 #pragma unroll
-        for (int ls = 0; ls < SPW; ++ls) wload(ls, 0, ring[ls]);
-    }
-    // tables: the entries as two fp16 pairs each, then the signed table (see nvq_signed_kernel)
-    u32x2_t *cbh = reinterpret_cast<u32x2_t *>(red + rpb * nwaves * MB * 16);
+    for (int d = 0; d < PRE; ++d)
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        if (tid + t * static_cast<int>(blockDim.x) < ncb) {
-            uint32_t h[4];
+        for (int ls = 0; ls < SPW; ++ls) wload(ls, d, ring[d * SPW + ls]);
+    // tables: the entries as two fp16 pairs each, then the signed table (see nvq_signed_kernel); the anchors wait in LDS
+    // because a global load inside the walk would have to wait for every weight request before it
+    float *anc = red + rpb * nwaves * MB * 16;  // rpb * 16 anchors
+    u32x2_t *cbh = reinterpret_cast<u32x2_t *>(anc + rpb * 16);
+    if (wave == 0) {
 #pragma unroll
-            for (int b = 0; b < 4; ++b) h[b] = f32_to_f16_rne(static_cast<float>((craw[t] >> (8 * b)) & 0xffu));
-            cbh[tid + t * blockDim.x] = u32x2_t{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        for (int t = 0; t < 4; ++t) {
+            const int e0 = 4 * (t * 64 + lane);
+            if (e0 < ncb) {
+                const uint32_t cr[4] = {craw[t].x, craw[t].y, craw[t].z, craw[t].w};
+                uint32_t h[4][4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) h[e][b] = f32_to_f16_rne(static_cast<float>((cr[e] >> (8 * b)) & 0xffu));
+                u32x4_t *dst = reinterpret_cast<u32x4_t *>(cbh + e0);
+                dst[0] = u32x4_t{h[0][0] | (h[0][1] << 16), h[0][2] | (h[0][3] << 16), h[1][0] | (h[1][1] << 16), h[1][2] | (h[1][3] << 16)};
+                dst[1] = u32x4_t{h[2][0] | (h[2][1] << 16), h[2][2] | (h[2][3] << 16), h[3][0] | (h[3][1] << 16), h[3][2] | (h[3][3] << 16)};
+            }
         }
-    }
-    if (tid < 16) {
-        stab[2 * tid] = __float_as_uint(lutv);
-        stab[2 * tid + 1] = lds_base + bankv * k.entries * 128;
+        if (lane < 16) {
+            stab[2 * lane] = lutv;
+            stab[2 * lane + 1] = lds_base + bankv * k.entries * 128;
+        }
+        if (lane * 2 < nrb * 16) *reinterpret_cast<u32x2_t *>(anc + lane * 2) = anc_v;
     }
     __syncthreads();  // raw entries
     for (int c = tid; c < ncb * 8; c += blockDim.x) {
@@ -774,6 +800,11 @@ __global__ __launch_bounds__(1024) void nvq_bcast_kernel(NvqK k_first, const uin
         *reinterpret_cast<u32x4_t *>(lds + 4 * c) = v;
     }
     const uint32_t stab_base = lds_base + ncb * 128;
+    __syncthreads();  // tables
+#pragma unroll
+    for (int d = PRE; d < DEPTH; ++d)
+#pragma unroll
+        for (int ls = 0; ls < SPW; ++ls) wload(ls, d, ring[d * SPW + ls]);
     // the activation pairs as fp16 (bf16 rows: times the wave's power of two that brings its slice near 2^12)
     uint32_t xh[MB][SPW][4];
     float xinv[MB];
@@ -793,48 +824,61 @@ __global__ __launch_bounds__(1024) void nvq_bcast_kernel(NvqK k_first, const uin
         for (int ls = 0; ls < SPW; ++ls)
 #pragma unroll
             for (int j = 0; j < 4; ++j) xh[m][ls][j] = XF16 ? xraw[m][ls][j] : to_h2_scaled(xraw[m][ls][j], sc);
+#pragma unroll
+        for (int ls = 0; ls < SPW; ++ls) dpp_source_ready(xh[m][ls][0], xh[m][ls][1], xh[m][ls][2], xh[m][ls][3]);
     }
-    __syncthreads();  // tables
 
     // one item: the states of its four units, then all 24 vectors at once, then the dot products
     auto process = [&](Item &it, uint32_t noff, const uint32_t (&xs)[MB][SPW][4], auto LS, float (&acc)[MB]) {
         constexpr int ls = decltype(LS)::value;  // compile time: the pair register goes into the dot products as it is
-        const u32x4_t uc4 = it.c;
-        it.c = __builtin_amdgcn_raw_buffer_load_b128(win, noff + 2048 + lane * 16, 0, 2);
-        const uint32_t ucv[4] = {uc4.x, uc4.y, uc4.z, uc4.w};
+        // The slot is refilled only after the last use of what it holds: requested any earlier, the new values would need
+        // registers of their own and a copy into the slot, and that copy would wait for the request it came from.
+        const uint32_t ucv[4] = {it.c.x, it.c.y, it.c.z, it.c.w};
         u32x2_t stv[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             stv[j] = *reinterpret_cast<lds_u32x2_ptr>(stab_base + (__builtin_rotateleft32(ucv[j], 6) & 0x78u));
-        u32x2_t vec[4][6];
+        // GB units' vectors are gathered at once (all four where the registers allow it)
+        constexpr int GB = (SPW == 1) ? 4 : 2;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t ua = it.q[j].x, ub = it.q[j].y, uc = ucv[j];
-            it.q[j] = __builtin_amdgcn_raw_buffer_load_b64(win, noff + (j * 64 + lane) * 8, 0, 2);
-            const uint32_t base = stv[j].y;
-            const uint32_t off[6] = {and_or(ua, 0xfff8u, base), and_or(ua >> 16, 0xfff8u, base),
-                                     and_or(ub, 0xfff8u, base), and_or(ub >> 16, 0xfff8u, base),
-                                     and_or(uc, 0xfff8u, base), and_or(uc >> 13, 0xfff8u, base)};
+        for (int j0 = 0; j0 < 4; j0 += GB) {
+            u32x2_t vec[GB][6];
 #pragma unroll
-            for (int t = 0; t < 6; ++t) vec[j][t] = *reinterpret_cast<lds_u32x2_ptr>(off[t]);
-        }
+            for (int g = 0; g < GB; ++g) {
+                const int j = j0 + g;
+                const uint32_t ua = it.q[j].x, ub = it.q[j].y, uc = ucv[j];
+                const uint32_t base = stv[j].y;
+                const uint32_t off[6] = {and_or(ua, 0xfff8u, base), and_or(ua >> 16, 0xfff8u, base),
+                                         and_or(ub, 0xfff8u, base), and_or(ub >> 16, 0xfff8u, base),
+                                         and_or(uc, 0xfff8u, base), and_or(uc >> 13, 0xfff8u, base)};
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float sc = __uint_as_float(stv[j].x);
+                for (int t = 0; t < 6; ++t) vec[g][t] = *reinterpret_cast<lds_u32x2_ptr>(off[t]);
+            }
+            if (j0 + GB == 4) {  // every field of the slot has been read: refill it
+                asm volatile("" ::: "memory");
 #pragma unroll
-            for (int m = 0; m < MB; ++m) {
-                float a = 0.f;
-                const uint32_t xv = xs[m][ls][j];
-                a = dot2_bcast4<0, false>(a, xv, vec[j][0].x, vec[j][0].y, vec[j][1].x, vec[j][1].y);
-                a = dot2_bcast4<4, false>(a, xv, vec[j][2].x, vec[j][2].y, vec[j][3].x, vec[j][3].y);
-                a = dot2_bcast4<8, true>(a, xv, vec[j][4].x, vec[j][4].y, vec[j][5].x, vec[j][5].y);
-                acc[m] = fmaf(sc, a, acc[m]);
+                for (int j = 0; j < 4; ++j) it.q[j] = __builtin_amdgcn_raw_buffer_load_b64(win, noff + (j * 64 + lane) * 8, 0, 2);
+                it.c = __builtin_amdgcn_raw_buffer_load_b128(win, noff + 2048 + lane * 16, 0, 2);
+            }
+#pragma unroll
+            for (int g = 0; g < GB; ++g) {
+                const int j = j0 + g;
+                const float sc = __uint_as_float(stv[j].x);
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+                    float a = 0.f;
+                    const uint32_t xv = xs[m][ls][j];
+                    a = dot2_bcast4<0, false>(a, xv, vec[g][0].x, vec[g][0].y, vec[g][1].x, vec[g][1].y);
+                    a = dot2_bcast4<4, false>(a, xv, vec[g][2].x, vec[g][2].y, vec[g][3].x, vec[g][3].y);
+                    a = dot2_bcast4<8, true>(a, xv, vec[g][4].x, vec[g][4].y, vec[g][5].x, vec[g][5].y);
+                    acc[m] = fmaf(sc, a, acc[m]);
+                }
             }
         }
     };
     // the waves' partial sums of row-block i: slot (i * nwaves + wave) * MB + m, 16 neurons each
     auto park = [&](int i, float (&acc)[MB]) {
-        const float av = anchors[(rb_first + min(i, nrb - 1)) * 16 + r];
+        const float av = anc[i * 16 + r];
 #pragma unroll
         for (int m = 0; m < MB; ++m) {
             const float v = reduce_kb4(acc[m]) * av * xinv[m];
@@ -845,27 +889,21 @@ __global__ __launch_bounds__(1024) void nvq_bcast_kernel(NvqK k_first, const uin
     float acc[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) acc[m] = 0.f;
-    if constexpr (SPW == 1) {
-        for (int i = 0; i < rpb; i += 2) {
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int ii = i + u;
-                if (ii < rpb) {  // block-uniform
-                    if (n > 0 && ii < nrb)
-                        process(ring[u], ii + 2 < nrb ? (ii + 2) * rbb : kNoStep, xh, std::integral_constant<int, 0>{}, acc);
-                    park(ii, acc);
-                }
-            }
-        }
-    } else {
-        for (int i = 0; i < rpb; ++i) {
-            static_for<SPW>([&](auto LS) {
-                constexpr int ls = decltype(LS)::value;
-                if (ls < n && i < nrb) process(ring[ls], i + 1 < nrb ? (i + 1) * rbb + ls * sb : kNoStep, xh, LS, acc);
-            });
-            park(i, acc);
-        }
-    }
+    // The walk is straight-line code over up to eight row-blocks with one exit per row-block and nothing conditional in
+    // between (a wave without steps, or past the block's last row-block, walks zeros): with a loop, or a branch around an
+    // item, the compiler could not count the requests in flight and would wait for all of them -- the refill it has just
+    // issued included -- before every item.
+#define NVQ_RB(II)                                                                                                   \
+    if (II >= rpb) break;                                                                                            \
+    static_for<SPW>([&](auto LS) {                                                                                   \
+        constexpr int ls = decltype(LS)::value;                                                                      \
+        process(ring[(II % DEPTH) * SPW + ls], ls < n && II + DEPTH < nrb ? (II + DEPTH) * rbb + ls * sb : kNoStep, xh, LS, acc); \
+    });                                                                                                              \
+    park(II, acc);
+    do {
+        NVQ_RB(0) NVQ_RB(1) NVQ_RB(2) NVQ_RB(3) NVQ_RB(4) NVQ_RB(5) NVQ_RB(6) NVQ_RB(7)
+    } while (0);
+#undef NVQ_RB
     __syncthreads();
     for (int o = tid; o < nrb * MB * 16; o += blockDim.x) {
         const int rr = o & 15, m = (o >> 4) % MB, i = (o >> 4) / MB;
@@ -1211,30 +1249,42 @@ static int nvq_launch_signed(const NvqK &k, const uint8_t *w, const uint16_t *x,
 // One or two rows on nvq_bcast_kernel: the signed table fits the LDS, the rows can be fetched pair by pair (4-byte
 // aligned, even K), at most three steps per wave (four would spill), and at least four waves (the table build spreads
 // over them).
-static bool nvq_bcast_capable(const NvqK &k, const void *x, int64_t ldx, int M, int more_rowblocks = 0) {
+// Blocks of a launch over one tensor (nrb1 = 0) or two: every block gets the same number of consecutive row-blocks of
+// one tensor, the fewest that leave one block per compute unit.  (Dealing the row-blocks out evenly over as many blocks
+// as there are compute units measured slower on every shape tried, 17408 x 5120: 15.5 us against 15.0 -- the blocks
+// that finish early do not shorten the launch, and each block more builds another table.)
+static int nvq_bcast_split(int nrb0, int nrb1, int &b0, int &b1) {
+    const int rpb = static_cast<int>(ceil_div(nrb0 + nrb1, gemv_cu_count()));
+    b0 = static_cast<int>(ceil_div(nrb0, rpb));
+    b1 = static_cast<int>(ceil_div(nrb1, rpb));
+    return rpb;
+}
+static bool nvq_bcast_capable(const NvqK &k, const void *w, const void *x, int64_t ldx, int M, int more_rowblocks = 0) {
     static const int off = tune_env("MFQ_NVQ_BCAST_OFF", 0);
-    const int rpb = nvq_signed_rpb(k, more_rowblocks);
+    int b0, b1;
+    const int rpb = nvq_bcast_split(k.n_rowblocks, more_rowblocks, b0, b1);
     const int spw = static_cast<int>(ceil_div(k.nsteps, 16));
     return !off && M >= 1 && M <= 2 && static_cast<int64_t>(k.banks) * k.entries * 128 <= 131072 && rpb <= 8 && spw <= 3 &&
            ceil_div(k.nsteps, spw) >= 4 && k.neuron_len % 2 == 0 && (M == 1 || ldx % 2 == 0) &&
-           (reinterpret_cast<uintptr_t>(x) & 3) == 0 && rpb * k.rowblock_bytes < (1ll << 31);
+           (reinterpret_cast<uintptr_t>(x) & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 &&
+           rpb * k.rowblock_bytes < (1ll << 31);
 }
 template <int XF16, int MB, int SPW>
 static int nvq_launch_bcast_as(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                                hipStream_t st, const NvqSecond *second) {
     const int nwaves = static_cast<int>(ceil_div(k.nsteps, SPW));
-    const int rpb = nvq_signed_rpb(k, second ? second->k.n_rowblocks : 0);
-    const int blocks0 = static_cast<int>(ceil_div(k.n_rowblocks, rpb));
+    int blocks0, blocks1;
+    const int rpb = nvq_bcast_split(k.n_rowblocks, second ? second->k.n_rowblocks : 0, blocks0, blocks1);
     NvqSecond s2{k, w, blocks0, 0};
     int blocks = blocks0;
     size_t ncb = static_cast<size_t>(k.banks) * k.entries;
     if (second) {
         s2 = *second;
         s2.blocks0 = blocks0;
-        blocks += static_cast<int>(ceil_div(s2.k.n_rowblocks, rpb));
+        blocks += blocks1;
         if (static_cast<size_t>(s2.k.banks) * s2.k.entries > ncb) ncb = static_cast<size_t>(s2.k.banks) * s2.k.entries;
     }
-    const size_t lds = ncb * 136 + 128 + static_cast<size_t>(rpb) * nwaves * MB * 64;
+    const size_t lds = ncb * 136 + 128 + static_cast<size_t>(rpb) * nwaves * MB * 64 + static_cast<size_t>(rpb) * 64;
     auto kern = nvq_bcast_kernel<XF16, MB, SPW>;
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), lds, "nvq_bcast")) return rc;
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks), static_cast<unsigned>(ceil_div(M, MB))), dim3(64 * nwaves), lds,
@@ -1297,7 +1347,7 @@ static int nvq_gemv_any(const mfq_nvq_desc *d, const void *weight, const void *x
     const NvqK k = to_k(d);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
-    if (nvq_bcast_capable(k, x, ldx, M))
+    if (nvq_bcast_capable(k, w, x, ldx, M))
         return x_dtype == MFQ_X_F16 ? nvq_launch_bcast<1>(k, w, xp, ldx, M, y, ldy, st)
                                     : nvq_launch_bcast<0>(k, w, xp, ldx, M, y, ldy, st);
     if (nvq_stream_capable(k) && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
@@ -1421,8 +1471,8 @@ extern "C" int mfq_hip_nvq_gemv_multi2(const mfq_nvq_desc *d0, const void *weigh
                 "nvq_gemv_multi2: ldx/ldy smaller than the tensors");
     const NvqK k0 = to_k(d0), k1 = to_k(d1);
     hipStream_t st = as_stream(stream);
-    if (nvq_bcast_capable(k0, x, ldx, M, k1.n_rowblocks) && nvq_bcast_capable(k1, x, ldx, M, k0.n_rowblocks) &&
-        nvq_bcast_capable(k0, x, ldx, M) && nvq_bcast_capable(k1, x, ldx, M)) {  // what each tensor's own call would run
+    if (nvq_bcast_capable(k0, weight0, x, ldx, M, k1.n_rowblocks) && nvq_bcast_capable(k1, weight1, x, ldx, M, k0.n_rowblocks) &&
+        nvq_bcast_capable(k0, weight0, x, ldx, M) && nvq_bcast_capable(k1, weight1, x, ldx, M)) {  // what each tensor's own call would run
         const NvqSecond s2{k1, static_cast<const uint8_t *>(weight1), 0, d0->out};
         const uint8_t *w0 = static_cast<const uint8_t *>(weight0);
         const uint16_t *xp = static_cast<const uint16_t *>(x);
