@@ -284,6 +284,7 @@ def main() -> int:
     def bf16(a):
         return torch.from_numpy(a).to(torch.bfloat16).to(dev)
 
+    cpu4_rows = None
     if not args.no_extras:
         from tyloquant_amd import formats as F
         from tyloquant_amd import runtime_vq as RV
@@ -363,11 +364,22 @@ def main() -> int:
         ebits = np.random.default_rng(4).choice([2, 3, 4, 5], size=E, p=[0.1, 0.4, 0.4, 0.1])
         per_expert = np.zeros(E)
         handles = []
-        for seed, (o_, k_) in ((40, (2 * INTER, HID)), (41, (HID, INTER))):
+        # the CPU leg's sample of this config: one token, its eight routed experts (chosen here so that their rows can be
+        # cut out of the cohort payloads before those are dropped)
+        cpu4_logits = np.random.default_rng(44).standard_normal((1, E)).astype(np.float32)
+        cpu4_ids = np.argsort(-cpu4_logits, axis=-1, kind="stable")[:, :TOPK].astype(np.int32)
+        cpu4_rows = [{}, {}]      # per tensor: expert -> (packed body of its cohort, header, first row)
+        for ti4, (seed, (o_, k_)) in enumerate(((40, (2 * INTER, HID)), (41, (HID, INTER)))):
             blob4, pools4 = synth.nintm_quantized_blob(seed, E, o_, k_, ebits)
             for ids4, payload4 in pools4:
                 hdr = F.parse_nint(payload4)
                 per_expert[ids4] += hdr.body_bytes / len(ids4)
+                if not args.no_cpu:
+                    body4 = None
+                    for local4, e4 in enumerate(ids4):
+                        if int(e4) in cpu4_ids:
+                            body4 = bytes(payload4[hdr.body_off:]) if body4 is None else body4
+                            cpu4_rows[ti4][int(e4)] = (body4, hdr, local4 * o_, o_)
             h4 = C.c_void_p()
             rt_check(rt.mfq_rt_load_nint_moe(blob4, len(blob4), C.byref(h4)))
             handles.append(h4)
@@ -456,6 +468,59 @@ def main() -> int:
     cpu = None
     if not args.no_cpu:
         from oracle import c_oracle
+        from oracle import mfq_oracle as O
+
+        def best_of(fn, n=3):
+            best, res = 1e9, None
+            for _ in range(n):
+                t1 = time.perf_counter()
+                res = fn()
+                best = min(best, time.perf_counter() - t1)
+            return best, res
+        cpu_cfg = {}
+        # config 1: the whole NINT3 4096 x 4096 tensor, one row
+        blob1 = synth.nint_linear_blob(7, 4096, 4096, 3, 24, 5, slab_rows=1024)[1]
+        h1 = F.parse_nint(blob1)
+        body1 = bytes(blob1[h1.body_off:])
+        xc1 = synth.activations(np.random.default_rng(101), 1, 4096).astype(np.float32)
+        sec, _ = best_of(lambda: c_oracle.matmul_nt(xc1, c_oracle.nint_dequant(body1, 3, 5, 24, 4096, 4096)))
+        cpu_cfg["config1"] = {"value": (h1.body_bytes + 2 * 4096 + 4 * 4096) / sec / 1e9, "unit": "GB/s", "cores": c_oracle.threads(),
+                              "kind": "port", "sample": f"NINT3 (3,24,5) 4096x4096 at M=1, whole tensor: dequantize + x@W.T, best of 3 ({sec * 1e3:.0f} ms)"}
+        # config 3: a 1024-row slab of the NVQ3J-512 17408 x 5120 tensor, one row
+        blob3 = synth.nvq3j512_blob(11, 1024, 5120)[1]
+        t3 = O.unpack_nvq(blob3)
+        xc3 = synth.activations(np.random.default_rng(103), 1, 5120).astype(np.float32)
+        sec, _ = best_of(lambda: c_oracle.matmul_nt(xc3, c_oracle.nvq_jsc_dequant(t3)))
+        cpu_cfg["config3"] = {"value": O.nvq_payload_nbytes("d4_512", 1024, 5120) / sec / 1e9, "unit": "GB/s", "cores": c_oracle.threads(),
+                              "kind": "port", "sample": "NVQ3J-512 at M=1, a 1024-row slab of the 17408x5120 tensor (unpacked fields): "
+                                                        f"dequantize + x@W.T, best of 3 ({sec * 1e3:.0f} ms)"}
+        # config 4: one token through its eight routed experts (the shared expert's two GEMVs left out)
+        if cpu4_rows is not None and all(len(d) == cpu4_ids.size for d in cpu4_rows):
+            xc4 = synth.activations(np.random.default_rng(104), 1, HID).astype(np.float32)
+            sel4 = np.take_along_axis(cpu4_logits, cpu4_ids.astype(np.int64), axis=-1).astype(np.float64)
+            w4 = np.exp(sel4 - sel4.max(-1, keepdims=True))
+            w4 = (w4 / w4.sum(-1, keepdims=True)).astype(np.float32)
+
+            def moe_cpu():
+                dense = [{e: c_oracle.nint_dequant_rows(b, hd.bits, hd.sub_bits, hd.gs, hd.out, hd.neuron_len, r0, nr)
+                          for e, (b, hd, r0, nr) in rows.items()} for rows in cpu4_rows]
+                return c_oracle.moe_ffn(xc4, cpu4_ids, w4, dense[0], dense[1], E)
+            sec, _ = best_of(moe_cpu)
+            cpu_cfg["config4"] = {"value": 1.0 / sec, "unit": "tokens/s", "cores": c_oracle.threads(), "kind": "port",
+                                  "sample": "MoE layer at T=1: the token's 8 routed experts of 256 (mixed 2/3/4/5-bit), dequantize "
+                                            f"their rows + gate/up, SwiGLU, down, weighted sum; shared expert left out; best of 3 ({sec * 1e3:.0f} ms)"}
+            del cpu4_rows
+        # config 5: a 512-row slab of an NEPQ1-S 6144 x 4096 tensor (the other formats of the stack are configs 1 and 3)
+        blob5 = synth.nepq1_blob(53, "NEPQ1-S", 512, 4096)[1]
+        t5 = O.unpack_nepq(blob5)
+        tab5 = np.stack([np.stack([O.unpack_ternary_table(p.tobytes()[:1024]), O.unpack_ternary_table(p.tobytes()[1024:])])
+                         for p in t5.table_payloads])
+        xc5 = synth.activations(np.random.default_rng(105), 1, 4096).astype(np.float32)
+        sec, _ = best_of(lambda: c_oracle.matmul_nt(xc5, c_oracle.nepq1s_dequant(t5, tab5)[0]))
+        cpu_cfg["config5"] = {"value": O.nepq_payload_nbytes("NEPQ1-S", 1, 512, 4096, len(t5.table_payloads)) / sec / 1e9, "unit": "GB/s",
+                              "cores": c_oracle.threads(), "kind": "port",
+                              "sample": f"NEPQ1-S at M=1, a 512-row slab (unpacked fields): dequantize + x@W.T, best of 3 ({sec * 1e3:.0f} ms)"}
+        log(f"[bench] cpu baselines of configs 1, 3, 4, 5: {cpu_cfg}")
         blob = base["gate"][1]
         from tyloquant_amd import formats as F
         h = F.parse_nint(blob)
@@ -479,7 +544,7 @@ def main() -> int:
         cpu = {"value": gbytes / best_full, "unit": "GB/s", "cores": c_oracle.threads(), "kind": "port",
                "sample": "gate 12288x4096 NINT4-32 at M=1: dequantize to fp32 + x@W.T, best of 3 "
                          f"({best_full * 1e3:.0f} ms); matmul alone on pre-dequantized W {best_mm * 1e3:.1f} ms",
-               "matmul_only_value": gbytes / best_mm, "gpu_vs_cpu_rel_l2": cpu_rel}
+               "matmul_only_value": gbytes / best_mm, "gpu_vs_cpu_rel_l2": cpu_rel, "configs": cpu_cfg}
         log(f"[bench] cpu baseline: {cpu}")
 
     line = {
@@ -498,7 +563,7 @@ def main() -> int:
                      # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, each scaled by what the counter
                      # reads for a plain 256 MiB copy: the figure the committed profile summary states
                      "traffic": profiled_traffic(),
-                     "kernel": "nint_gemv_paired_kernel<4,32,0,1,false>", "avg_launch_us": avg_launch_us,
+                     "kernel": "nint_gemv_xreg_kernel<PairedUnit<4,32>,0,1>", "avg_launch_us": avg_launch_us,
                      "bytes_per_launch": bytes_per_launch},
         "cpu_baseline": cpu,
         "extras": extras,

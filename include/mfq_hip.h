@@ -138,10 +138,19 @@ int mfq_hip_nint_gemm_glu(const mfq_nint_desc *d, const void *weight, const void
  * MFQ_ERR_UNSUPPORTED from the call: run the two launches then) holds the barrier words and the hidden vector; its
  * first 4096 bytes (one barrier flag per compute unit) must be zero before the first call
  * (mfq_hip_nint_ffn_decode_workspace_init, or any memset) and belong to the library from then on: every call advances
- * all flags by one.  Calls that share a workspace must not overlap, and a workspace stays with one device.  If another kernel keeps compute units
- * busy so that the blocks cannot all run at once, the barrier gives up after a bounded number of polls and y is NaN. */
+ * all flags by one.  Calls that share a workspace must not overlap, and a workspace stays with one device.
+ * Contract of the barrier: (1) the launch needs the device to itself -- every block waits for all the others, so all
+ * of them have to be running at once; the call refuses a grid that the device's real compute units cannot hold
+ * (mfq_hip_set_cu_count above the device's count), but it cannot know of kernels on other streams or of other
+ * processes that keep compute units busy; (2) all flags of a workspace hold the same value between calls, so a
+ * workspace is used with one grid size: after mfq_hip_set_cu_count changes it, call ..._workspace_init again.
+ * When the blocks do not all run at once the barrier gives up after a bounded number of polls, y is NaN and the error
+ * word behind the flags is set; nothing hangs.  mfq_hip_nint_ffn_decode_status waits for the stream, returns MFQ_OK
+ * when no barrier of the calls since the last check gave up, else resets the workspace and returns MFQ_ERR_LAUNCH
+ * (run the two launches then).  No counterpart in the reference (it has no grid barrier). */
 size_t mfq_hip_nint_ffn_decode_workspace_bytes(const mfq_nint_desc *gate_up, const mfq_nint_desc *down);
 int mfq_hip_nint_ffn_decode_workspace_init(void *workspace, mfq_stream_t stream);
+int mfq_hip_nint_ffn_decode_status(void *workspace, mfq_stream_t stream);
 int mfq_hip_nint_ffn_decode(const mfq_nint_desc *gate_up, const void *gate_up_weight, const mfq_nint_desc *down,
                             const void *down_weight, const void *x, int x_dtype, int activation, float *y,
                             void *workspace, size_t workspace_bytes, mfq_stream_t stream);
@@ -190,8 +199,12 @@ int mfq_hip_nint_gemv_argmax(const mfq_nint_desc *d, const void *weight, const v
  * library (one copy per GPU, held until the process ends).  No counterpart in the reference.  Same arguments and
  * results as mfq_hip_nint_gemv_argmax without the workspace pair; MFQ_ERR_WORKSPACE when
  * mfq_hip_nint_gemv_argmax_workspace_bytes(d, M) exceeds 4 MiB (M = 1 fits any vocabulary up to about 900k; with
- * logits passed in, far more).  Allocates nothing and frees nothing; the first call on a device looks the array's
- * address up.  All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race. */
+ * logits passed in, far more).  Allocates nothing and frees nothing.  The first use on a device looks the array's
+ * address up (hipGetSymbolAddress, which may load the code object): that must not happen while a stream is being
+ * captured, so before capturing call mfq_hip_nint_gemv_argmax_static_init once per device with that device current
+ * (or make one eager call); it launches nothing and is cheap to repeat.  All calls on one GPU share the array: calls
+ * that overlap on one GPU (two streams, two threads) race, and so do overlapping replays of graphs that hold one. */
+int mfq_hip_nint_gemv_argmax_static_init(void);
 int mfq_hip_nint_gemv_argmax_static(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
                                     int64_t ldx, int M, float *logits, int64_t ldl, int64_t *token,
                                     mfq_stream_t stream);

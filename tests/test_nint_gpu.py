@@ -1,6 +1,8 @@
 """GPU parity of the NINT path against the oracle (through the C ABI)."""
 import ctypes as C
 
+import re
+
 import numpy as np
 import pytest
 
@@ -483,9 +485,35 @@ def test_ffn_decode_one_launch(cu_count, bits, gs, sb, H, W, N, cus):
         assert np.abs(y - ref).max() < ABS_TOL
         two = R.nint_matmul(dn, R._nint_matmul_glu(gu, x, torch.float16, act)).cpu().numpy()
         assert rel_l2(y, two) < 1e-4                     # same hidden rounding, another order of the sums over K
-    G = cus or 256
+    G = int(re.search(r"cu_count=(\d+)", L.lib().mfq_hip_config().decode()).group(1))   # the grid the library launched
+    assert G == cus or not cus
     words = gu._ffn_ws[:4096].view(torch.int32).cpu().numpy()
     assert np.all(words[:G] == 4) and words[G] == 0       # every block crossed four barriers; the error word is clear
+    assert L.lib().mfq_hip_nint_ffn_decode_status(gu._ffn_ws.data_ptr(), None) == 0
+
+
+def test_ffn_decode_refuses_a_grid_the_device_cannot_hold(cu_count):
+    """More blocks than the device has compute units could never all reach the grid barrier: the call refuses
+    (no launch), the workspace query still answers for the forced grid, and the host path runs the two launches."""
+    import ctypes as C
+    from tyloquant_amd import _lib as L
+    from tyloquant_amd import runtime as R
+    lib = L.lib()
+    real = int(re.search(r"cu_count=(\d+)", lib.mfq_hip_config().decode()).group(1))
+    rng = np.random.default_rng(9)
+    H, W, N = 256, 16 * (real + 8), 64
+    tg = O.quantize_nint((rng.standard_normal((2 * W, H)) * 0.02).astype(np.float32), 4, 32, 6)
+    td = O.quantize_nint((rng.standard_normal((N, W)) * 0.02).astype(np.float32), 4, 32, 6)
+    gu, dn = _load(tg).weight, _load(td).weight
+    x, xf = _x(rng, 1, H, torch.bfloat16)
+    cu_count(real + 8)
+    need = lib.mfq_hip_nint_ffn_decode_workspace_bytes(C.byref(gu.desc), C.byref(dn.desc))
+    if need:
+        ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+        y = torch.empty((1, N), dtype=torch.float32, device="cuda")
+        rc = lib.mfq_hip_nint_ffn_decode(C.byref(gu.desc), gu.data.data_ptr(), C.byref(dn.desc), dn.data.data_ptr(), x.data_ptr(),
+                                         L.X_BF16, L.GLU_SILU, y.data_ptr(), ws.data_ptr(), need, None)
+        assert rc == L.ERR_UNSUPPORTED and b"cannot all run at once" in lib.mfq_hip_last_error()
 
 
 def test_ffn_decode_shapes_outside_the_kernel_take_two_launches():

@@ -357,6 +357,8 @@ def test_c_restatement_matches_the_numpy_oracle_bit_for_bit():
         body = blob[14 + 4 + 16 + 8:]
         W = c_oracle.nint_dequant(body, spec[0], spec[2], spec[1], 19, 203)
         assert np.array_equal(W.view(np.uint32), O.dequantize_nint(t).view(np.uint32))
+        part = c_oracle.nint_dequant_rows(body, spec[0], spec[2], spec[1], 19, 203, 5, 9)
+        assert np.array_equal(part, W[5:14])
     g = np.load(GOLD / "nint_quant_vectors.npz")
     t = O.quantize_nint(g["c7_W"], 3, 24, 5)
     W = c_oracle.nint_dequant(O.pack_nint(t)[42:], 3, 5, 24, 16, 4096)
@@ -365,6 +367,35 @@ def test_c_restatement_matches_the_numpy_oracle_bit_for_bit():
     y = c_oracle.matmul_nt(x, W)
     ref = O.linear_forward_f64(W, x)
     assert np.abs(y - ref).max() < 1e-4 * np.abs(ref).max()
+
+
+def test_c_twins_of_the_nvq_and_nepq_dequantizers_and_the_moe_loop():
+    """The C restatements bench.py times for configs 3, 4 and 5 against the numpy oracle: dequantizers bit for bit
+    (ragged K, a second bank, indices that stop short of the last group), the MoE loop against the oracle's moe_ffn up to
+    the summation order of its matrix products."""
+    from oracle import c_oracle
+    if not c_oracle.LIB.exists():
+        pytest.skip("oracle/libmfq_oracle.so is not built (make -C oracle)")
+    rng = np.random.default_rng(13)
+    for out, K, cb, banks in ((7, 203, "d4_512", 2), (16, 384, "d4_512", 2), (5, 100, "d4_256", 1)):
+        t = synth.nvq_jsc_random(rng, out, K, cb, banks)
+        assert np.array_equal(c_oracle.nvq_jsc_dequant(t).view(np.uint32), O.dequantize_nvq_jsc(t).view(np.uint32))
+    for E, out, K, banks in ((1, 9, 192, 3), (2, 5, 360, 2)):
+        t = synth.nepq_random(rng, "NEPQ1-S", E, out, K, banks)
+        tables = np.stack([np.stack([O.unpack_ternary_table(p.tobytes()[:1024]), O.unpack_ternary_table(p.tobytes()[1024:])])
+                           for p in t.table_payloads])
+        assert np.array_equal(c_oracle.nepq1s_dequant(t, tables).view(np.uint32), O.dequantize_nepq(t).view(np.uint32))
+    E, H, W, T, k = 6, 96, 40, 5, 2
+    gu = (rng.standard_normal((E, 2 * W, H)) * 0.1).astype(np.float32)
+    dn = (rng.standard_normal((E, H, W)) * 0.1).astype(np.float32)
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    ref, ids, w = O.moe_ffn(gu, dn, x, logits, k)
+    ids[0, 1] = -1                                            # a dropped route contributes nothing
+    ref = O.moe_weighted_reduce(O.moe_grouped_matmul(dn, O.moe_swiglu(O.moe_grouped_matmul(gu, x, ids)), ids), w)
+    hit = sorted(set(int(e) for e in ids.reshape(-1) if e >= 0))
+    got = c_oracle.moe_ffn(x, ids, w, {e: gu[e] for e in hit}, {e: dn[e] for e in hit}, E)
+    assert np.abs(got - ref).max() < 1e-5 * np.abs(ref).max()
 
 
 def test_nint8_zero_is_ggml_q8_0():

@@ -164,3 +164,13 @@ def test_mfq_store_readers_reject_malformed_files(rt, tmp_path):
             rt.mfq_rt_file_close(h)
         elif len(mutated) < len(data):
             assert rt.mfq_rt_last_error()
+    # a refused file leaves no mapping behind: the failed opens above and 200 more of a truncated file
+    bad.write_bytes(data[: len(data) // 2])
+
+    def mappings():
+        return sum(1 for line in open("/proc/self/maps") if "bad.mfq" in line)
+
+    for _ in range(200):
+        h = C.c_void_p()
+        assert rt.mfq_rt_file_open(str(bad).encode(), b"-", b"-", C.byref(h)) == 1
+    assert mappings() == 0

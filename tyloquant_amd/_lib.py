@@ -82,11 +82,13 @@ _SIGS = {
                                         sz, vp]),
     "mfq_hip_nint_ffn_decode_workspace_bytes": (sz, [C.POINTER(NintDesc), C.POINTER(NintDesc)]),
     "mfq_hip_nint_ffn_decode_workspace_init": (C.c_int, [vp, vp]),
+    "mfq_hip_nint_ffn_decode_status": (C.c_int, [vp, vp]),
     "mfq_hip_nint_ffn_decode": (C.c_int, [C.POINTER(NintDesc), vp, C.POINTER(NintDesc), vp, vp, C.c_int, C.c_int, vp, vp, sz,
                                           vp]),
     "mfq_hip_nint_embedding": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, vp, C.c_int, i64, vp]),
     "mfq_hip_nint_gemv_argmax_workspace_bytes": (sz, [C.POINTER(NintDesc), C.c_int]),
     "mfq_hip_nint_gemv_argmax": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, vp, sz, vp]),
+    "mfq_hip_nint_gemv_argmax_static_init": (C.c_int, []),
     "mfq_hip_nint_gemv_argmax_static": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, vp]),
     "mfq_hip_nint_gemm_workspace_bytes": (sz, [C.POINTER(NintDesc), C.c_int]),
     "mfq_hip_nint_gemm": (C.c_int, [C.POINTER(NintDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),

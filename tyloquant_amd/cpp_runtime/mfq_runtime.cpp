@@ -1446,14 +1446,23 @@ int MfqFile::map_file(const std::string &source) {
         m.base = static_cast<const uint8_t *>(p);
     }
     ::close(fd);  // the mapping keeps the file
-    maps_.push_back(m);
+    maps_.push_back(std::move(m));
     source_paths.push_back(source);
     return static_cast<int>(maps_.size()) - 1;
 }
 
-MfqFile::~MfqFile() {
-    for (const Mapping &m : maps_)
-        if (m.base) ::munmap(const_cast<uint8_t *>(m.base), m.size);
+MfqFile::Mapping::~Mapping() {
+    if (base) ::munmap(const_cast<uint8_t *>(base), size);
+}
+MfqFile::Mapping &MfqFile::Mapping::operator=(Mapping &&o) noexcept {
+    if (this != &o) {
+        if (base) ::munmap(const_cast<uint8_t *>(base), size);
+        base = o.base;
+        size = o.size;
+        o.base = nullptr;
+        o.size = 0;
+    }
+    return *this;
 }
 
 MfqFile::MfqFile(const std::string &path_in, const std::string &tensor_overlay, const std::string &expert_overlay)
@@ -1528,8 +1537,6 @@ MfqFile::MfqFile(const std::string &path_in, const std::string &tensor_overlay, 
         const std::vector<std::string> paths = shard_paths(path, split_no, split_count);
         // start over in shard order
         records.clear();
-        for (const Mapping &m : maps_)
-            if (m.base) ::munmap(const_cast<uint8_t *>(m.base), m.size);
         maps_.clear();
         source_paths.clear();
         uint64_t expected_records = kNoCount, expected_tensors = kNoCount;

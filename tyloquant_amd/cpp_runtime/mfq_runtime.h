@@ -400,7 +400,7 @@ struct MfqFile {
     // expert_overlay: NINTMD records over NINTM records of the same name, kept aside.  Empty: the environment variables
     // MFQ_TENSOR_OVERLAY / MFQ_EXPERT_OVERLAY, as in the reference; "-" disables the lookup.
     explicit MfqFile(const std::string &path, const std::string &tensor_overlay = "", const std::string &expert_overlay = "");
-    ~MfqFile();
+    ~MfqFile() = default;
     MfqFile(const MfqFile &) = delete;
     MfqFile &operator=(const MfqFile &) = delete;
     const MfqRecord &find(const std::string &name) const;
@@ -410,9 +410,17 @@ struct MfqFile {
     std::string read_asset_text(const std::string &name) const;  // a BLOB record as text
 
 private:
+    // A read-only file mapping that unmaps itself: the constructor throws on any malformed file, and a member that
+    // cleans up after itself is released then, while ~MfqFile does not run for a half-built object.
     struct Mapping {
         const uint8_t *base = nullptr;
         size_t size = 0;
+        Mapping() = default;
+        Mapping(Mapping &&o) noexcept : base(o.base), size(o.size) { o.base = nullptr; o.size = 0; }
+        Mapping &operator=(Mapping &&o) noexcept;
+        Mapping(const Mapping &) = delete;
+        Mapping &operator=(const Mapping &) = delete;
+        ~Mapping();
     };
     std::vector<Mapping> maps_;
     int map_file(const std::string &source);

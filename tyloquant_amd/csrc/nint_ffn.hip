@@ -318,6 +318,23 @@ extern "C" int mfq_hip_nint_ffn_decode_workspace_init(void *workspace, mfq_strea
     return check_launch("nint_ffn_decode_workspace_init");
 }
 
+extern "C" int mfq_hip_nint_ffn_decode_status(void *workspace, mfq_stream_t stream) {
+    MFQ_REQUIRE(workspace, MFQ_ERR_INVALID, "nint_ffn_decode_status: null workspace");
+    const hipStream_t st = as_stream(stream);
+    // the error word follows the flags of however many blocks the launches used: any of the words behind the first
+    // device_cu_count() flags up to the end of the barrier area can only have been set by a timed-out barrier
+    int words[kFfnSyncBytes / 4];
+    hipError_t e = hipMemcpyAsync(words, workspace, kFfnSyncBytes, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    MFQ_REQUIRE(e == hipSuccess, MFQ_ERR_LAUNCH, "nint_ffn_decode_status: %s", hipGetErrorString(e));
+    const int G = device_cu_count();
+    if (words[G] == 0) return MFQ_OK;
+    hipLaunchKernelGGL(ffn_sync_clear_kernel, dim3(1), dim3(256), 0, st, static_cast<int *>(workspace));
+    if (int rc = check_launch("nint_ffn_decode_status")) return rc;
+    return fail(MFQ_ERR_LAUNCH, "nint_ffn_decode: a grid barrier gave up (the blocks did not all run at once); the outputs of the "
+                                "calls since the last check are NaN, the workspace has been reset");
+}
+
 extern "C" int mfq_hip_nint_ffn_decode(const mfq_nint_desc *gate_up, const void *gate_up_weight, const mfq_nint_desc *down,
                                        const void *down_weight, const void *x, int x_dtype, int activation, float *y,
                                        void *workspace, size_t workspace_bytes, mfq_stream_t stream) {
@@ -347,10 +364,11 @@ extern "C" int mfq_hip_nint_ffn_decode(const mfq_nint_desc *gate_up, const void 
     p.sync = static_cast<int *>(workspace);
     p.hidden = reinterpret_cast<uint16_t *>(static_cast<uint8_t *>(workspace) + kFfnSyncBytes);
     p.gelu = activation == MFQ_GLU_GELU ? 1 : 0;
-    p.spin_limit = tune_env("MFQ_FFN_SPIN_LIMIT", 1 << 18);
+    static const int spin_limit = tune_env("MFQ_FFN_SPIN_LIMIT", 1 << 18), want_trace = tune_env("MFQ_FFN_TRACE", 0);
+    p.spin_limit = spin_limit;
     // MFQ_FFN_TRACE=1: a workspace with 32 more bytes per compute unit behind the hidden vector receives each block's
     // clock (100 MHz) at its start, at its arrival at the barrier, after the barrier and at its end
-    p.trace = tune_env("MFQ_FFN_TRACE", 0) && workspace_bytes >= need + 32u * G
+    p.trace = want_trace && workspace_bytes >= need + 32u * G
                   ? reinterpret_cast<long long *>(static_cast<uint8_t *>(workspace) + ((need + 31) & ~size_t(31)))
                   : nullptr;
     const hipStream_t st = as_stream(stream);
@@ -361,13 +379,18 @@ extern "C" int mfq_hip_nint_ffn_decode(const mfq_nint_desc *gate_up, const void 
         if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), lds, "nint_ffn_decode")) return rc;       \
         /* all blocks must be resident at once: asked once per kernel and LDS size */                                  \
         static std::atomic<size_t> fits_lds{0};                                                                        \
+        static std::atomic<int> resident_blocks{1};                                                                    \
         if (fits_lds.load(std::memory_order_relaxed) < lds) {                                                          \
             int resident = 0;                                                                                          \
             const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, 64 * kFfnWaves, lds);   \
             MFQ_REQUIRE(e == hipSuccess && resident >= 1, MFQ_ERR_UNSUPPORTED,                                         \
                         "nint_ffn_decode: a block of %d waves with %zu bytes of LDS does not fit a compute unit", kFfnWaves, lds); \
             fits_lds.store(lds, std::memory_order_relaxed);                                                            \
+            resident_blocks.store(resident, std::memory_order_relaxed);                                                \
         }                                                                                                              \
+        MFQ_REQUIRE(G <= device_real_cu_count() * resident_blocks.load(std::memory_order_relaxed), MFQ_ERR_UNSUPPORTED, \
+                    "nint_ffn_decode: %d blocks cannot all run at once on %d compute units (%d block(s) each): the grid " \
+                    "barrier would never be crossed", G, device_real_cu_count(), resident_blocks.load(std::memory_order_relaxed)); \
         hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(G)), dim3(64 * kFfnWaves), lds, st, p);                    \
         return check_launch("nint_ffn_decode");                                                                        \
     }

@@ -308,6 +308,8 @@ void *static_scratch() {
 }
 }  // namespace
 
+extern "C" int mfq_hip_nint_gemv_argmax_static_init(void) { return static_scratch() ? MFQ_OK : MFQ_ERR_LAUNCH; }
+
 extern "C" int mfq_hip_nint_gemv_argmax_static(const mfq_nint_desc *d, const void *weight, const void *x, int x_dtype,
                                                int64_t ldx, int M, float *logits, int64_t ldl, int64_t *token,
                                                mfq_stream_t stream) {

@@ -74,6 +74,10 @@ int tune_env(const char *name, int dflt) {
 int device_cu_count() {
     const int forced = g_cu_override.load(std::memory_order_relaxed);
     if (forced > 0) return forced;
+    return device_real_cu_count();
+}
+
+int device_real_cu_count() {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
     int n = g_cu_cached[dev].load(std::memory_order_relaxed);

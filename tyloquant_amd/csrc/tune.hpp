@@ -14,6 +14,8 @@ int tune_env(const char *name, int dflt);
 // Compute units of the current device (hipDeviceAttributeMultiprocessorCount, queried once per device), or the
 // value given to mfq_hip_set_cu_count while that is non-zero.
 int device_cu_count();
+// the same without mfq_hip_set_cu_count's override: what the device really has
+int device_real_cu_count();
 
 // Largest dynamic LDS a block may ask for on gfx950 (160 KB per CU); above 64 KB the kernel has to opt in.
 constexpr size_t kMaxDynamicLds = 160 * 1024;

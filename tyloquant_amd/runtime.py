@@ -225,12 +225,14 @@ def nint_matmul_geglu(w: NintWeight, x: torch.Tensor, out_dtype=torch.float16) -
 
 
 def nint_ffn_decode(gate_up: NintWeight, down: NintWeight, x: torch.Tensor, activation: int = L.GLU_SILU,
-                    one_launch: bool = False) -> torch.Tensor:
+                    one_launch: bool = False, verify: bool = False) -> torch.Tensor:
     """y = down(act(gate x) * up x) in fp32 for a [2W, H] gate/up tensor and a [N, W] down tensor: the dense FFN of
     FFN::forward_impl (cpp_runtime/mfq_decode.cpp:11199-11209): the fused gate/up launch (or matmul + GLU kernel)
     followed by the down matmul.  one_launch=True runs one activation row on a pair of tensors the kernel takes as a
     single launch with a grid barrier (mfq_hip_nint_ffn_decode); it is not the default because crossing the barrier
-    costs what the launch boundary costs (measured: 23.7 us against 19.3 us on 12288 x 4096 NINT4-32)."""
+    costs what the launch boundary costs (measured: 23.7 us against 19.3 us on 12288 x 4096 NINT4-32).  The barrier
+    needs the device to itself; when it gives up the output is NaN.  verify=True waits for the launch, asks
+    mfq_hip_nint_ffn_decode_status and runs the two launches instead if a barrier gave up."""
     if gate_up.out != 2 * down.neuron_len:
         raise ValueError("gate/up rows must be twice the down tensor's neuron length")
     x2 = _as_2d(x, gate_up.neuron_len)
@@ -244,7 +246,8 @@ def nint_ffn_decode(gate_up: NintWeight, down: NintWeight, x: torch.Tensor, acti
             y = torch.empty((1, down.out), dtype=torch.float32, device=x.device)
             L.check(lib.mfq_hip_nint_ffn_decode(C.byref(gate_up.desc), _ptr(gate_up.data), C.byref(down.desc), _ptr(down.data),
                                                 _ptr(x2), _x_dtype(x2), activation, _ptr(y), _ptr(ws), need, _stream()))
-            return y.reshape(*x.shape[:-1], down.out)
+            if not verify or lib.mfq_hip_nint_ffn_decode_status(_ptr(ws), _stream()) == 0:
+                return y.reshape(*x.shape[:-1], down.out)
     return nint_matmul(down, _nint_matmul_glu(gate_up, x, torch.float16, activation))
 
 
