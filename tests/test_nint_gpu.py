@@ -572,6 +572,34 @@ def test_gemv_bf16_rows_of_any_magnitude(bits, gs, sb, scale):
             assert rel_l2(h, want) < 6e-3                  # bf16 output: half an ulp is 4e-3
 
 
+@pytest.mark.parametrize("bits,gs,sb,K", [(4, 32, 6, 2048), (4, 32, 6, 4040), (2, 16, 5, 1536), (2, 32, 5, 4096)])
+def test_small_batches_take_bf16_rows_of_any_magnitude(bits, gs, sb, K):
+    """3 to 16 rows on the kernel that keeps the activations in LDS (one K step per wave, groups of 32 or 16): every row
+    of the tile has its own magnitude, from 1e-6 to 3e6 times an ordinary row, in one batch -- each comes out with the
+    accuracy of an ordinary row, as on the one-row kernels.  K = 4040 ends inside a step (the rest of the step reads zeros)."""
+    from tyloquant_amd import synth as P
+    rng = np.random.default_rng(bits * 100 + gs + K)
+    out = 80
+    t = O.quantize_nint((rng.standard_normal((out, K)) * 0.02).astype(np.float32), bits, gs, sb)
+    lin = _load(t)
+    deq = O.dequantize_nint(t)
+    for M in (3, 5, 16):
+        scales = np.float32(10.0) ** rng.uniform(-6, 6.4, size=(M, 1)).astype(np.float32)
+        scales[0], scales[-1] = np.float32(1e-6), np.float32(3e6)
+        x = torch.from_numpy(P.activations(rng, M, K, outlier_frac=0.001) * scales).to(torch.bfloat16)
+        ref = O.linear_forward_f64(deq, x.float().numpy())
+        y = lin(x.cuda()).cpu().numpy()
+        assert np.isfinite(y).all()
+        for m in range(M):
+            assert rel_l2(y[m], ref[m]) < REL_TOL, (M, m, float(scales[m, 0]), rel_l2(y[m], ref[m]))
+    # groups whose 32 activations all sit at the row's largest magnitude, with one sign: the group sums of the minimum term
+    x = torch.full((4, K), 3.0, dtype=torch.bfloat16) * torch.tensor([[1.0], [-1.0], [1e-5], [2e5]], dtype=torch.bfloat16)
+    ref = O.linear_forward_f64(deq, x.float().numpy())
+    y = lin(x.cuda()).cpu().numpy()
+    for m in range(4):
+        assert rel_l2(y[m], ref[m]) < REL_TOL, (m, rel_l2(y[m], ref[m]))
+
+
 def test_reserved_workspace_lets_forward_run_under_graph_capture():
     """QuantLinear.reserve(max_rows) sizes the weight's workspace once; forward() of any smaller batch then allocates
     nothing of its own and can be captured into a HIP graph (batch-1 GEMV, streaming kernel and prefill kernel with its

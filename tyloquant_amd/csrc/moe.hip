@@ -511,15 +511,18 @@ __global__ __launch_bounds__(512) void moe_mfma_kernel(MoePools P, const int32_t
     }
     const int pool = expert_pool[e];
     const int rb_first = expert_local[e] * rbe;
-    int p = pair_of(threadIdx.x & 15);
-    if (p < 0) p = pair_of(0);
-    const uint16_t *xrow = x + static_cast<int64_t>(routed_input ? p : p / R) * ldx;
+    const int p = pair_of(threadIdx.x & 15);   // -1: an empty slot of the tile, whose lanes request no activations
     const NintK &k = P.k[pool];
     if (P.prefill[pool]) return;
+    // all activation rows through one window (the launcher checks that they span less than 4 GiB)
+    const int n_rows = routed_input ? n_pairs : (n_pairs + R - 1) / R;
+    const __amdgpu_buffer_rsrc_t xwin = wave_window(reinterpret_cast<const uint8_t *>(x),
+                                                    static_cast<uint32_t>((static_cast<int64_t>(n_rows - 1) * ldx + k.neuron_len) * 2));
+    const uint32_t xoff = p < 0 ? kNoStep : static_cast<uint32_t>(static_cast<int64_t>(routed_input ? p : p / R) * ldx * 2);
     const uint8_t *w = P.w[pool];
     const int spw = P.spw[pool];
 #define MFQ_MOE_MFMA(UNIT, B, G) \
-    if (k.bits == B && k.gs == G) nint_mfma_body<UNIT<B, G>, XF16, NB>(k, w, rb_first + rbl0, rb_first + rbe, xrow, spw, red);
+    if (k.bits == B && k.gs == G) nint_mfma_body<UNIT<B, G>, XF16, NB, mfma_x_ahead<UNIT<B, G>, NB, 8>()>(k, w, rb_first + rbl0, rb_first + rbe, xwin, xoff, spw, red);
     if (k.kind == 1) {
         MFQ_MOE_MFMA(PairedUnit, 4, 24)
         else MFQ_MOE_MFMA(PairedUnit, 3, 24)
@@ -789,7 +792,9 @@ extern "C" int mfq_hip_moe_grouped_matmul_ws(const mfq_moe_pool *pools, int n_po
     P.n = n_pools;
     int max_steps = 1;
     bool units = true;  // every cohort has a unit with GEMV, streaming and prefill bodies
-    bool mfma = K >= 8 && K % 8 == 0 && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    // (the matrix-core kernel addresses all activation rows through one buffer window: they span less than 4 GiB)
+    bool mfma = K >= 8 && K % 8 == 0 && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                (static_cast<int64_t>(n_pairs) * ldx + K) * 2 < (1ll << 32);
     for (int i = 0; i < n_pools; ++i) {
         const mfq_nint_desc &d = pools[i].desc;
         MFQ_REQUIRE(d.neuron_len == K && pools[i].weight, MFQ_ERR_INVALID,

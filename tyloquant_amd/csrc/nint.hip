@@ -236,7 +236,8 @@ static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, i
 // ---- small batches on the matrix cores ----------------------------------------------------
 static bool mfma_eligible(const NintK &k, const void *x, int64_t ldx) {
     return (k.kind == 1 || mfma_generic_profile(k)) && k.neuron_len >= 8 && k.neuron_len % 8 == 0 && ldx % 8 == 0 &&
-           (reinterpret_cast<uintptr_t>(x) & 15) == 0 && 4 * k.rowblock_bytes < (1ll << 31);
+           (reinterpret_cast<uintptr_t>(x) & 15) == 0 && 4 * k.rowblock_bytes < (1ll << 31) &&
+           (15 * ldx + k.neuron_len) * 2 < (1ll << 32);  // a tile's 16 rows through one buffer window
 }
 
 bool nint_stream_capable(const mfq_nint_desc *d) {
@@ -313,6 +314,55 @@ static int launch_mfma(const NintK &k, const uint8_t *w, const uint16_t *x, int6
     if (ceil_div(k.n_rowblocks, 4) * wpb >= 1536) return launch_mfma_nb<XF16, 4>(k, w, x, ldx, M, y, ldy, st);
     if (ceil_div(k.n_rowblocks, 2) * wpb >= 1536) return launch_mfma_nb<XF16, 2>(k, w, x, ldx, M, y, ldy, st);
     return launch_mfma_nb<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
+}
+
+// Up to 16 rows with the activations resident in LDS (nint_mfma_resident_kernel): one block per compute unit walks its
+// row-block groups.  NB as in launch_mfma: the fewest rounds of groups over the compute units, the larger NB on a tie.
+static bool mfma_resident_shape(const NintK &k, int M, int &nb, int &spw, int &nwaves, size_t &lds, int &red_slots) {
+    static const int on = tune_env("MFQ_MFMA_RESIDENT", 1);
+    if (!on || M > 16 || k.kind != 1 || (k.gs != 32 && k.gs != 16) || k.anchors_off >= (1ll << 31)) return false;
+    nwaves = k.nsteps < 8 ? k.nsteps : 8;
+    spw = static_cast<int>(ceil_div(k.nsteps, nwaves));
+    // one step per wave: with more (4096 x 12288 at 4 rows, three steps) the older kernel measured as fast (13.0 vs 13.9 us)
+    if (spw > 1 || spw * M * 2 * k.gs > 1024) return false;  // a wave stages at most 1024 16-byte chunks
+    const int64_t cus = gemv_cu_count();
+    int64_t best_cost = 0;
+    nb = 0;
+    for (int c = 1; c <= 3; ++c) {
+        const int64_t cost = ceil_div(ceil_div(k.n_rowblocks, c), cus) * c;
+        if (mfma_resident_lds(nwaves, c, spw, M, k.gs) > kMaxDynamicLds) break;
+        if (nb == 0 || cost <= best_cost) nb = c, best_cost = cost;
+    }
+    if (nb == 0) return false;
+    // as many reduction areas as the block has groups, where they fit (no barrier between groups then)
+    const int per_block = static_cast<int>(ceil_div(ceil_div(k.n_rowblocks, nb), cus));
+    red_slots = per_block <= 4 && mfma_resident_lds(nwaves, nb, spw, M, k.gs, per_block) <= kMaxDynamicLds ? per_block : 1;
+    lds = mfma_resident_lds(nwaves, nb, spw, M, k.gs, red_slots);
+    return true;
+}
+
+template <int XF16>
+static int launch_mfma_resident(const NintK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y,
+                                int64_t ldy, int nb, int spw, int nwaves, size_t lds, int red_slots, hipStream_t st) {
+    const int64_t groups = ceil_div(k.n_rowblocks, nb), cus = gemv_cu_count();
+    const dim3 grid(static_cast<unsigned>(groups < cus ? groups : cus), 1), block(64 * nwaves);
+#define MFQ_RES_NB(UNIT, B, G, NBV)                                                                                  \
+    {                                                                                                                \
+        auto kern = nint_mfma_resident_kernel<UNIT<B, G>, XF16, NBV>;                                                \
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), lds, "nint_mfma_resident")) return rc;  \
+        hipLaunchKernelGGL(kern, grid, block, lds, st, k, w, x, ldx, M, y, ldy, spw, red_slots);                     \
+        return check_launch("nint_mfma_resident");                                                                   \
+    }
+#define MFQ_RES(UNIT, B, G)                                                                                          \
+    if (k.bits == B && k.gs == G) {                                                                                  \
+        if (nb == 1) MFQ_RES_NB(UNIT, B, G, 1)                                                                       \
+        if (nb == 2) MFQ_RES_NB(UNIT, B, G, 2)                                                                       \
+        MFQ_RES_NB(UNIT, B, G, 3)                                                                                    \
+    }
+    MFQ_RES(PairedUnit, 4, 32) MFQ_RES(PairedUnit, 4, 16) MFQ_RES(PairedUnit, 2, 16) MFQ_RES(PairedUnit, 2, 32)
+#undef MFQ_RES
+#undef MFQ_RES_NB
+    return fail(MFQ_ERR_UNSUPPORTED, "nint_mfma_resident: no kernel for NINT%d-%d", k.bits, k.gs);
 }
 
 // ---- prefill: block-tiled MFMA GEMM with in-register dequantization ---------------------------
@@ -440,9 +490,15 @@ int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int
     static const int valu_max = tune_env("MFQ_GEMV_VALU_MAX_M", 2);
     // two rows: the vector-ALU GEMV unpacks once and takes two dot products (10.6 vs 12.9 us on 12288x4096);
     // from three rows on the matrix-core kernel wins
-    if (M > valu_max && mfma_eligible(k, x, ldx))
+    if (M > valu_max && mfma_eligible(k, x, ldx)) {
+        int nb, spw, nwaves, red_slots;
+        size_t lds;
+        if (mfma_resident_shape(k, M, nb, spw, nwaves, lds, red_slots))
+            return x_dtype == MFQ_X_F16 ? launch_mfma_resident<1>(k, w, xp, ldx, M, y, ldy, nb, spw, nwaves, lds, red_slots, st)
+                                        : launch_mfma_resident<0>(k, w, xp, ldx, M, y, ldy, nb, spw, nwaves, lds, red_slots, st);
         return x_dtype == MFQ_X_F16 ? launch_mfma<1>(k, w, xp, ldx, M, y, ldy, st)
                                     : launch_mfma<0>(k, w, xp, ldx, M, y, ldy, st);
+    }
     // LDS per block grows with MB; large K falls back to narrower row batches, and neurons whose one-row slice no
     // block can stage (beyond about 70k elements) go to the matrix-core kernel, whose LDS use does not depend on K.
     int mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1);

@@ -24,6 +24,7 @@ Knob g_knobs[] = {
     {"MFQ_GEMV_RBW", "row-blocks per block of the NINT GEMV (0 = by shape)", 0, false},
     {"MFQ_GEMV_XREG", "0 = the one- and two-row NINT GEMV stages its activations in LDS instead of registers", 0, false},
     {"MFQ_GEMV_VALU_MAX_M", "rows up to which the vector-ALU GEMV runs before the streaming MFMA kernel", 0, false},
+    {"MFQ_MFMA_RESIDENT", "0 = small batches never take the kernel that keeps the activations in LDS", 0, false},
     {"MFQ_MFMA_WIDE", "0 = the NINT streaming MFMA kernel keeps eight waves per block on small grids", 0, false},
     {"MFQ_MFMA_NB", "row-blocks per wave of the NINT streaming MFMA kernel (0 = by shape)", 0, false},
     {"MFQ_STREAM_MAX_M", "rows up to which NINT streams instead of the prefill kernel (0 = cost model)", 0, false},
