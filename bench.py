@@ -32,7 +32,7 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-TRAFFIC_PROFILE = ROOT / "profiles" / "nint_gemv_paired_4_32_config2_decode.md"
+TRAFFIC_PROFILE = ROOT / "profiles" / "nint_gemv_xreg_4_32_config2_decode.md"
 
 
 def profiled_traffic():
@@ -299,6 +299,16 @@ def main() -> int:
             extras[f"prefill_M{M}_tflops"] = 2.0 * M * FF * H / (ms * 1e-3) / 1e12
             extras[f"prefill_M{M}_ms"] = ms
             extras[f"prefill_M{M}_frac_of_f16_mfma_peak"] = extras[f"prefill_M{M}_tflops"] / MFMA_F16_PEAK_TFLOPS
+        # ---- config 2: small batches on the gate+up tensor, rotating over the weight sets (graph replay) ---------
+        one_us = None
+        for M in (1, 2, 4, 8, 16):
+            xm = bf16(synth.activations(rng, M, H, outlier_frac=0.001))
+            us = graph_ms(lambda: [R.nint_matmul(s_["gate_up"], xm) for s_ in sets], 10) / len(sets) * 1e3
+            one_us = one_us or us
+            extras[f"small_batch_gate_up_M{M}_us"] = us
+            extras[f"small_batch_gate_up_M{M}_vs_one_row"] = us / one_us
+        log("[bench] config 2 gate+up 24576x4096 at 1/2/4/8/16 rows: " + ", ".join(
+            f"{extras[f'small_batch_gate_up_M{M}_us']:.1f} us" for M in (1, 2, 4, 8, 16)))
         log(f"[bench] config 2 extras: {extras}")
         del sets[1:]
         torch.cuda.empty_cache()
