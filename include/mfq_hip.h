@@ -246,6 +246,12 @@ int mfq_hip_nint8z_repack(const mfq_nint8z_desc *d, const void *blocks, int64_t 
  * and nint8_zero_dequant_cuda (cpp_runtime/mfq_decode.cpp:8180-8182). */
 int mfq_hip_nint8z_dequant_f32(const mfq_nint8z_desc *d, const void *weight, float *w_out, int64_t ld,
                                mfq_stream_t stream);
+/* Token-embedding rows: out[n, 0:neuron_len] = row ids[n] of mfq_hip_nint8z_dequant_f32 rounded once to out_dtype
+ * (MFQ_X_BF16, MFQ_X_F16 or MFQ_X_F32); ids (device int64) outside [0, out) give a row of zeros.  Replaces
+ * nint8_zero_embedding_lookup_cuda (cpp_runtime/mfq_decode.cpp:366-370, called at :13943-13947; kernel
+ * mfq/kernels/cuda/embedding.cu:190-220). */
+int mfq_hip_nint8z_embedding(const mfq_nint8z_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,
+                             int out_dtype, int64_t ldo, mfq_stream_t stream);
 /* y[M, out] = x[M, neuron_len] . W^T streaming the codes once per pass of up to 8 rows (fewer when the fp16
  * activations of a pass would not fit 64 KB of LDS; MFQ_ERR_UNSUPPORTED when one row does not).  Replaces
  * nint8_zero_gemv_ws_cuda / nint8_zero_mmq_ws_cuda (cpp_runtime/mfq_decode.cpp:8167-8177). */
@@ -290,6 +296,13 @@ int mfq_hip_nvq_repack_plain(const mfq_nvq_desc *d, const void *payload, int64_t
  * nvq_dequant_cuda (cpp_runtime/mfq_decode.cpp:540-546). */
 int mfq_hip_nvq_dequant_f32(const mfq_nvq_desc *d, const void *weight, float *w_out, int64_t ld,
                             mfq_stream_t stream);
+/* Token-embedding rows: out[n, 0:neuron_len] = row ids[n] of mfq_hip_nvq_dequant_f32 rounded once to out_dtype
+ * (MFQ_X_BF16, MFQ_X_F16 or MFQ_X_F32; the reference stores fp16); ids (device int64) outside [0, out) give a row of
+ * zeros (the reference leaves such rows unwritten).  Replaces nvq_embedding_lookup_cuda
+ * (cpp_runtime/mfq_decode.cpp:608, called through nvq_embedding :8072-8079 at :13937-13939; kernel
+ * mfq/kernels/cuda/nvq_matmul.cu:1665-1719, launch :6026-6069). */
+int mfq_hip_nvq_embedding(const mfq_nvq_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,
+                          int out_dtype, int64_t ldo, mfq_stream_t stream);
 /* Replaces nvq_gemv_ws_cuda (cpp_runtime/mfq_decode.cpp:555-559). */
 int mfq_hip_nvq_gemv(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
                      int M, float *y, int64_t ldy, mfq_stream_t stream);
@@ -378,6 +391,11 @@ int mfq_hip_nvqs_repack_nepq0(const mfq_nvqs_desc *d, const void *body, int64_t 
                               mfq_stream_t stream);
 int mfq_hip_nvqs_dequant_rows_f32(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, float *w_out,
                                   int64_t ld, mfq_stream_t stream);
+/* Token-embedding rows of the families on this descriptor: the contract of mfq_hip_nvq_embedding over the rows of
+ * mfq_hip_nvqs_dequant_f32 (the same reference kernel, nvq_matmul.cu:1665-1719, instantiated per format by
+ * launch_by_format, :3344-3371). */
+int mfq_hip_nvqs_embedding(const mfq_nvqs_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,
+                           int out_dtype, int64_t ldo, mfq_stream_t stream);
 int mfq_hip_nvqs_gemv_rows(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, const void *x, int x_dtype,
                            int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream);
 size_t mfq_hip_nvqs_gemm_rows_workspace_bytes(const mfq_nvqs_desc *d, int nrows, int M);

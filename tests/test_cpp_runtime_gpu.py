@@ -189,7 +189,7 @@ def test_cpp_gate_up_glu_across_batch_sizes(rt):
 
 def test_cpp_embedding_rows_and_argmax_head(rt):
     """The host library's embed_forward / next_token_from_hidden twins on a NINT5-28 table: rows bit-exact against the
-    oracle's dequantizer, the token equal to the arg-max of the logits the call returns; other families refuse."""
+    oracle's dequantizer, the token equal to the arg-max of the logits the call returns; NVQ and NINT8-0 tables give their rows, NEPQ refuses."""
     rng = np.random.default_rng(14)
     out, K = 700, 448
     t = synth.nint_random(rng, out, K, 5, 28, 7)
@@ -215,10 +215,27 @@ def test_cpp_embedding_rows_and_argmax_head(rt):
         torch.cuda.synchronize()
         assert torch.equal(alone, token)
     rt.mfq_rt_free_quant_linear(h)
-    hv = _load(rt, "NVQ3J-512", O.pack_nvq_jsc(synth.nvq_jsc_random(rng, 32, 96)))
-    assert rt.mfq_rt_linear_embedding(hv, None, 0, None, 2, None) != 0
-    assert b"NINT" in rt.mfq_rt_last_error()
-    rt.mfq_rt_free_quant_linear(hv)
+    # the other table formats embed_forward takes: an NVQ table in the lane-major layout, one read from its streams, NINT8-0
+    tv = synth.nvq_jsc_random(rng, 32, 96)
+    te = synth.nvq_jsc_random(rng, 40, 104, "e8_256", 2)
+    t8 = O.quantize_nint8_zero((rng.standard_normal((24, 64)) * 0.02).astype(np.float32))
+    for dtype, blob, deq in (("NVQ3J-512", O.pack_nvq_jsc(tv), O.dequantize_nvq_jsc(tv)),
+                             (O.pack_tensor(te)[0], O.pack_tensor(te)[1], O.dequantize_nvq_jsc(te)),
+                             ("NINT8-0", O.pack_nint8_zero(t8), O.dequantize_nint8_zero(t8))):
+        hv = _load(rt, dtype, blob)
+        n, kk = deq.shape
+        ids = np.array([n - 1, 0, 5, n, -1], dtype=np.int64)
+        rows = torch.empty((len(ids), kk), dtype=torch.float16, device="cuda")
+        assert rt.mfq_rt_linear_embedding(hv, torch.from_numpy(ids).cuda().data_ptr(), len(ids), rows.data_ptr(), 1, None) == 0
+        torch.cuda.synchronize()
+        want = np.zeros((len(ids), kk), np.float32)
+        want[:3] = deq[ids[:3]]
+        assert np.array_equal(rows.cpu().numpy().view(np.uint16), want.astype(np.float16).view(np.uint16))
+        rt.mfq_rt_free_quant_linear(hv)
+    hp = _load(rt, "NEPQ1-S", O.pack_tensor(synth.nepq_random(rng, "NEPQ1-S", 1, 32, 96, 3))[1])
+    assert rt.mfq_rt_linear_embedding(hp, None, 0, None, 2, None) != 0
+    assert b"NINT, NINT8-0 or NVQ" in rt.mfq_rt_last_error()
+    rt.mfq_rt_free_quant_linear(hp)
 
 
 @pytest.mark.parametrize("T", [1, 20])

@@ -52,6 +52,61 @@ def test_embedding_rows_bit_exact(bits, gs, sb, out, K):
     assert torch.equal(gotb.view(torch.int16), torch.from_numpy(rows).to(torch.bfloat16).view(torch.int16))
 
 
+def _table(kind, rng, out, K):
+    """(dtype, blob, the oracle's dequantized rows) of an embedding table of the given format."""
+    if kind == "NINT8-0":
+        t = O.quantize_nint8_zero((rng.standard_normal((out, K)) * 0.02).astype(np.float32))
+        return "NINT8-0", O.pack_nint8_zero(t), O.dequantize_nint8_zero(t)
+    if isinstance(kind, str):
+        t = synth.nvq1_random(rng, kind, out, K) if kind.startswith("NVQ1") else synth.npq0_random(rng, kind, out, K)
+        dtype, blob = O.pack_tensor(t)
+        return dtype, blob, O.dequantize_tensor(O.unpack_tensor(dtype, blob))
+    codebook, banks = kind
+    dtype, blob = O.pack_tensor(synth.nvq_jsc_random(rng, out, K, codebook, banks))
+    return dtype, blob, O.dequantize_nvq_jsc(O.unpack_nvq(blob))
+
+
+@pytest.mark.parametrize("kind", ["NINT8-0", ("d4_512", 2), ("d4_512", 1), ("d4_256", 2), ("e8_256", 2), ("e8_4096", 4),
+                                  ("d4_1024", 2), "NVQ1-L", "NVQ1-S", "NPQ0-L", "NPQ0-S"], ids=str)
+@pytest.mark.parametrize("out,K", [(300, 96), (75, 1544), (33, 104)])
+def test_embedding_rows_of_the_other_table_formats(kind, out, K):
+    """embed_forward's other table formats (NINT8-0 and every NVQ family: the lane-major D4 layout and the families read
+    in place from their streams): rows picked by token id equal the oracle's dequantized rows bit for bit in fp32 and
+    rounded to nearest even in fp16 / bf16; ids outside the table give zeros; K = 104 and 1544 leave partial groups."""
+    from tyloquant_amd import runtime as R
+    if kind == "NINT8-0":
+        K = (K + 31) // 32 * 32                       # the format's rule: whole blocks of 32
+    rng = np.random.default_rng(1200 + out + K)
+    dtype, blob, want = _table(kind, rng, out, K)
+    lin = R.load_quant_linear(dtype, blob)
+    ids = rng.integers(0, out, (3, 7))
+    ids[0, 0], ids[1, 2], ids[2, 6], ids[0, 3], ids[0, 4] = -1, out, 2 ** 40, out - 1, 0
+    ids[1, 5] = ids[1, 4]
+    rows = np.zeros((3, 7, K), np.float32)
+    ok = (ids >= 0) & (ids < out)
+    rows[ok] = want[ids[ok]]
+    tid = torch.from_numpy(ids).cuda()
+    got = lin.embedding(tid, torch.float32).cpu().numpy()
+    assert got.shape == rows.shape
+    assert np.array_equal(got.view(np.uint32), rows.view(np.uint32))
+    got16 = R.embedding(lin.weight, tid, torch.float16).cpu().numpy()
+    assert np.array_equal(got16.view(np.uint16), rows.astype(np.float16).view(np.uint16))
+    gotb = R.embedding(lin, tid).to(torch.float32)   # default: fp16, the reference's output type
+    assert np.array_equal(gotb.cpu().numpy(), rows.astype(np.float16).astype(np.float32))
+    gotb = lin.embedding(tid, torch.bfloat16).cpu()
+    assert torch.equal(gotb.view(torch.int16), torch.from_numpy(rows).to(torch.bfloat16).view(torch.int16))
+    assert lin.embedding(tid[:0], torch.float16).shape == (0, 7, K)
+
+
+def test_embedding_refuses_tables_the_reference_refuses():
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(5)
+    dtype, blob = O.pack_tensor(synth.nepq_random(rng, "NEPQ1-S", 1, 32, 96, 3))
+    lin = R.load_quant_linear(dtype, blob)
+    with pytest.raises(TypeError):
+        lin.embedding(torch.zeros((2,), dtype=torch.int64, device="cuda"))
+
+
 def test_embedding_of_no_ids_and_bad_arguments():
     from tyloquant_amd import runtime as R
     rng = np.random.default_rng(3)

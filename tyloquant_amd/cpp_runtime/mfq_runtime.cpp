@@ -640,6 +640,14 @@ void nint_matmul_input_mul(const NintWeight &w, const void *x, const void *gate,
 void nint_embedding(const NintWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype, mfq_stream_t stream) {
     abi_check(mfq_hip_nint_embedding(&w.desc, w.data.get(), ids, n_ids, out, out_dtype, w.desc.neuron_len, stream));
 }
+void nint8_zero_embedding(const Nint8ZeroWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype,
+                          mfq_stream_t stream) {
+    abi_check(mfq_hip_nint8z_embedding(&w.desc, w.data.get(), ids, n_ids, out, out_dtype, w.desc.neuron_len, stream));
+}
+void nvq_embedding(const NvqWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype, mfq_stream_t stream) {
+    if (w.streams) abi_check(mfq_hip_nvqs_embedding(&w.sdesc, w.data.get(), ids, n_ids, out, out_dtype, w.sdesc.neuron_len, stream));
+    else abi_check(mfq_hip_nvq_embedding(&w.desc, w.data.get(), ids, n_ids, out, out_dtype, w.desc.neuron_len, stream));
+}
 void nint_matmul_argmax(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, int64_t *token, float *logits,
                         mfq_stream_t stream) {
     const size_t need = mfq_hip_nint_gemv_argmax_workspace_bytes(&w.desc, M);
@@ -836,6 +844,13 @@ void QuantLinear::dequantize(float *out, mfq_stream_t stream) const {
     else if (kind == QuantLinearKind::Nepq) nepq_dequantize(*nepq, out, stream);
     else if (kind == QuantLinearKind::Mx) mx_dequantize(*mx, 0, out, stream);
     else nint8_zero_dequantize(*nint8z, out, stream);
+}
+
+void QuantLinear::embedding(const int64_t *ids, int n_ids, void *out, int out_dtype, mfq_stream_t stream) const {
+    if (kind == QuantLinearKind::Nint) nint_embedding(*nint, ids, n_ids, out, out_dtype, stream);
+    else if (kind == QuantLinearKind::Nint8Zero) nint8_zero_embedding(*nint8z, ids, n_ids, out, out_dtype, stream);
+    else if (kind == QuantLinearKind::Nvq) nvq_embedding(*nvq, ids, n_ids, out, out_dtype, stream);
+    else fail("token embeddings need a NINT, NINT8-0 or NVQ table");
 }
 
 QuantLinear load_quant_linear(const std::string &dtype_in, const uint8_t *blob, size_t n, mfq_stream_t stream) {
@@ -1730,8 +1745,7 @@ int mfq_rt_linear_dequantize(void *h, float *out, void *stream) {
 int mfq_rt_linear_embedding(void *h, const int64_t *ids, int n_ids, void *out, int out_dtype, void *stream) {
     return guard([&] {
         const QuantLinear *q = static_cast<QuantLinear *>(h);
-        if (!q->nint) fail("embedding rows need a NINT table");
-        nint_embedding(*q->nint, ids, n_ids, out, out_dtype, stream);
+        q->embedding(ids, n_ids, out, out_dtype, stream);
     });
 }
 int mfq_rt_linear_argmax(void *h, const void *x, int x_dtype, int64_t ldx, int M, int64_t *token, float *logits, void *stream) {

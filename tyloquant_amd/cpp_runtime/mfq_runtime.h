@@ -185,6 +185,12 @@ void nint_matmul_geglu(const NintWeight &w, const void *x, int x_dtype, int64_t 
 // dequantized table, zeros for ids outside it (embed_forward :13929-13957)
 void nint_embedding(const NintWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype,
                     mfq_stream_t stream = nullptr);
+// the same for the other table formats embed_forward takes: NINT8-0 (:13943-13947) and every NVQ family
+// (nvq_embedding :8072-8079, called at :13937-13939)
+void nint8_zero_embedding(const Nint8ZeroWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype,
+                          mfq_stream_t stream = nullptr);
+void nvq_embedding(const NvqWeight &w, const int64_t *ids, int n_ids, void *out, int out_dtype,
+                   mfq_stream_t stream = nullptr);
 // token[m] (device int64) = argmax over the neurons of x[m] . W^T, ties to the lower index; logits (fp32 [M, out],
 // may be null) receives the values the arg-max was taken from (next_token_from_hidden :14107-14130)
 void nint_matmul_argmax(const NintWeight &w, const void *x, int x_dtype, int64_t ldx, int M, int64_t *token,
@@ -229,6 +235,9 @@ struct QuantLinear {
     int64_t payload_bytes() const;
     void forward(const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream = nullptr) const;
     void dequantize(float *out, mfq_stream_t stream = nullptr) const;
+    // The tensor as a token-embedding table (embed_forward :13929-13957): NINT, NINT8-0 and NVQ tables; NEPQ and MX
+    // tables are refused, as there.
+    void embedding(const int64_t *ids, int n_ids, void *out, int out_dtype, mfq_stream_t stream = nullptr) const;
     // Grows the weight's workspace to the largest need of any batch of 1 .. max_M rows, so that forward() of such a batch
     // neither frees nor allocates device memory: call it once before capturing forward() into a HIP graph, and before
     // sharing the weight between threads or streams (the workspace itself is still one buffer per weight: concurrent

@@ -102,6 +102,12 @@ __device__ __forceinline__ uint16_t f32_to_f16_rne(float f) {
     return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
 }
 
+// outp[at] = v rounded once to out_dtype (MFQ_X_F32: as is); outp is an array of that type.
+__device__ __forceinline__ void store_rounded(void *outp, int64_t at, float v, int out_dtype) {
+    if (out_dtype == MFQ_X_F32) static_cast<float *>(outp)[at] = v;
+    else static_cast<uint16_t *>(outp)[at] = out_dtype == MFQ_X_F16 ? f32_to_f16_rne(v) : f32_to_bf16_rne(v);
+}
+
 // A 1.0/1.0 pair in the activation type, for group sums through dot2.
 template <int XF16>
 __device__ __forceinline__ constexpr uint32_t ones_pair() { return XF16 ? 0x3c003c00u : 0x3f803f80u; }

@@ -47,6 +47,24 @@ __global__ __launch_bounds__(256) void nint8z_dequant_f32_kernel(N8zK k, const u
     outp[row * ld + col] = __fmul_rn(s, static_cast<float>(c));
 }
 
+// Embedding rows: out[n, col] = fl(scale * code) of neuron ids[n], rounded once more to the output type; ids outside
+// [0, out) give a row of zeros.
+__global__ __launch_bounds__(256) void nint8z_embedding_kernel(N8zK k, const uint8_t *__restrict__ w,
+                                                               const int64_t *__restrict__ ids, void *__restrict__ outp,
+                                                               int out_dtype, int64_t ldo) {
+    const int col = blockIdx.x * 256 + threadIdx.x;
+    if (col >= k.neuron_len) return;
+    const int n = blockIdx.y;
+    const int64_t tok = ids[n];
+    float v = 0.f;
+    if (tok >= 0 && tok < k.out) {
+        const float s = f16_to_f32(reinterpret_cast<const uint16_t *>(w + k.scales_off)[tok * k.ng + (col >> 5)]);
+        const int c = reinterpret_cast<const int8_t *>(w + k.codes_off)[(tok * k.ng + (col >> 5)) * 32 + (col & 31)];
+        v = __fmul_rn(s, static_cast<float>(c));
+    }
+    store_rounded(outp, static_cast<int64_t>(n) * ldo + col, v, out_dtype);
+}
+
 // fp16 rows for the dense GEMM: block = one row; values times 2^(12 - e), e = exponent of the row's largest
 // |scale| * 127, so that they stay below 4096; rowscale[row] = 2^(e - 12); columns up to kpad are zero
 __global__ __launch_bounds__(256) void nint8z_dequant_f16_kernel(N8zK k, const uint8_t *__restrict__ w, uint16_t *__restrict__ outp,
@@ -329,6 +347,27 @@ extern "C" int mfq_hip_nint8z_repack(const mfq_nint8z_desc *d, const void *block
     hipLaunchKernelGGL(nint8z_repack_kernel, dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, as_stream(stream), k,
                        static_cast<const uint8_t *>(blocks), static_cast<uint8_t *>(weight));
     return check_launch("nint8z_repack");
+}
+
+extern "C" int mfq_hip_nint8z_embedding(const mfq_nint8z_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,
+                                        int out_dtype, int64_t ldo, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight, MFQ_ERR_INVALID, "nint8z_embedding: null argument");
+    MFQ_REQUIRE(n_ids >= 0, MFQ_ERR_INVALID, "nint8z_embedding: n_ids=%d", n_ids);
+    MFQ_REQUIRE(out_dtype == MFQ_X_BF16 || out_dtype == MFQ_X_F16 || out_dtype == MFQ_X_F32, MFQ_ERR_INVALID,
+                "nint8z_embedding: out_dtype=%d", out_dtype);
+    MFQ_REQUIRE(ldo >= d->neuron_len, MFQ_ERR_INVALID, "nint8z_embedding: ldo %lld < neuron_len %d", static_cast<long long>(ldo),
+                d->neuron_len);
+    if (n_ids == 0) return MFQ_OK;
+    MFQ_REQUIRE(ids && out, MFQ_ERR_INVALID, "nint8z_embedding: null ids or output");
+    const N8zK k = to_k(d);
+    const size_t esize = out_dtype == MFQ_X_F32 ? 4 : 2;
+    for (int n0 = 0; n0 < n_ids; n0 += 65535) {  // the grid's second dimension holds 65535 rows
+        const int rows = n_ids - n0 < 65535 ? n_ids - n0 : 65535;
+        hipLaunchKernelGGL(nint8z_embedding_kernel, dim3(static_cast<unsigned>(ceil_div(k.neuron_len, 256)), static_cast<unsigned>(rows)),
+                           dim3(256), 0, as_stream(stream), k, static_cast<const uint8_t *>(weight), ids + n0,
+                           static_cast<void *>(static_cast<uint8_t *>(out) + static_cast<size_t>(n0) * ldo * esize), out_dtype, ldo);
+    }
+    return check_launch("nint8z_embedding");
 }
 
 extern "C" int mfq_hip_nint8z_dequant_f32(const mfq_nint8z_desc *d, const void *weight, float *w_out, int64_t ld,

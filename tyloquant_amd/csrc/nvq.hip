@@ -163,6 +163,44 @@ __global__ void nvq_dequant_kernel(NvqK k, const uint8_t *__restrict__ w, OutT *
     }
 }
 
+// ---- embedding rows: row ids[n] of the dequantized table, rounded once more to the output type -------------
+// One thread per group of 24 weights: a wave takes four steps of the neuron (16 groups each).  Group g of neuron
+// `tok` lives in row-block tok / 16, step g / 16, unit slot (g % 16) / 4 of lane (tok % 16) + 16 * (g % 4).  ids outside
+// [0, out) give a row of zeros.
+__global__ __launch_bounds__(64) void nvq_embedding_kernel(NvqK k, const uint8_t *__restrict__ w,
+                                                           const int64_t *__restrict__ ids, void *__restrict__ outp,
+                                                           int out_dtype, int64_t ldo) {
+    const int s = blockIdx.x * 4 + (threadIdx.x >> 4), slot = threadIdx.x & 15;
+    const int j = slot >> 2, kb = slot & 3;
+    const int g = 16 * s + 4 * j + kb;
+    if (s >= k.nsteps || g >= k.ng) return;
+    const int n = blockIdx.y;
+    const int64_t tok = ids[n];
+    const int64_t at = static_cast<int64_t>(n) * ldo + g * 24;
+    const int ncol = min(24, k.neuron_len - g * 24);
+    if (tok < 0 || tok >= k.out) {
+        for (int i = 0; i < ncol; ++i) store_rounded(outp, at + i, 0.f, out_dtype);
+        return;
+    }
+    const int rb = static_cast<int>(tok >> 4), lane = static_cast<int>(tok & 15) + 16 * kb;
+    const uint8_t *sp = w + rb * k.rowblock_bytes + s * k.step_bytes;
+    const uint32_t *qreg = reinterpret_cast<const uint32_t *>(sp);
+    const uint32_t *creg = reinterpret_cast<const uint32_t *>(sp + 2048);
+    const float *lut = reinterpret_cast<const float *>(w + k.tables_off);
+    const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+    const int8_t *cb = reinterpret_cast<const int8_t *>(bfs + 16);
+    const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[tok];
+    const NvqUnit u = nvq_decode(qreg[(j * 64 + lane) * 2], qreg[(j * 64 + lane) * 2 + 1], creg[lane * 4 + j]);
+    const float scale = __fmul_rn(anchor, lut[u.state]);
+    const int8_t *bank = cb + static_cast<int64_t>(bfs[u.state]) * k.entries * 4;
+    for (int i = 0; i < ncol; ++i) {
+        const int mag = bank[u.idx[i >> 2] * 4 + (i & 3)];
+        const uint32_t m8 = parity8(u.mask[i >> 3]);
+        const float sv = ((m8 >> (i & 7)) & 1u) ? -static_cast<float>(mag) : static_cast<float>(mag);
+        store_rounded(outp, at + i, __fmul_rn(sv, scale), out_dtype);
+    }
+}
+
 // ---- GEMV ------------------------------------------------------------------------------
 // LDS map (dwords): [codebook pairs: banks*entries*2][sign xor table: 128*4][lut: 16][bank: 16][x staging ...]
 template <int XF16, int MB>
@@ -1438,6 +1476,27 @@ extern "C" int mfq_hip_nvq_repack_plain(const mfq_nvq_desc *d, const void *paylo
                        static_cast<const uint8_t *>(nullptr), static_cast<const int8_t *>(grid),
                        static_cast<uint8_t *>(weight));
     return check_launch("nvq_repack_plain");
+}
+
+extern "C" int mfq_hip_nvq_embedding(const mfq_nvq_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,
+                                     int out_dtype, int64_t ldo, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight, MFQ_ERR_INVALID, "nvq_embedding: null argument");
+    MFQ_REQUIRE(n_ids >= 0, MFQ_ERR_INVALID, "nvq_embedding: n_ids=%d", n_ids);
+    MFQ_REQUIRE(out_dtype == MFQ_X_BF16 || out_dtype == MFQ_X_F16 || out_dtype == MFQ_X_F32, MFQ_ERR_INVALID,
+                "nvq_embedding: out_dtype=%d", out_dtype);
+    MFQ_REQUIRE(ldo >= d->neuron_len, MFQ_ERR_INVALID, "nvq_embedding: ldo %lld < neuron_len %d", static_cast<long long>(ldo),
+                d->neuron_len);
+    if (n_ids == 0) return MFQ_OK;
+    MFQ_REQUIRE(ids && out, MFQ_ERR_INVALID, "nvq_embedding: null ids or output");
+    const NvqK k = to_k(d);
+    const size_t esize = out_dtype == MFQ_X_F32 ? 4 : 2;
+    for (int n0 = 0; n0 < n_ids; n0 += 65535) {  // the grid's second dimension holds 65535 rows
+        const int rows = n_ids - n0 < 65535 ? n_ids - n0 : 65535;
+        hipLaunchKernelGGL(nvq_embedding_kernel, dim3(static_cast<unsigned>(ceil_div(k.nsteps, 4)), static_cast<unsigned>(rows)),
+                           dim3(64), 0, as_stream(stream), k, static_cast<const uint8_t *>(weight), ids + n0,
+                           static_cast<void *>(static_cast<uint8_t *>(out) + static_cast<size_t>(n0) * ldo * esize), out_dtype, ldo);
+    }
+    return check_launch("nvq_embedding");
 }
 
 extern "C" int mfq_hip_nvq_dequant_f32(const mfq_nvq_desc *d, const void *weight, float *w_out, int64_t ld,

@@ -262,6 +262,32 @@ __global__ __launch_bounds__(256) void nvqs_dequant_kernel(NvqsK k, const uint8_
     }
 }
 
+// Embedding rows: one thread per (id, sign block); row n of the output = neuron ids[n] of the bit-exact dequantizer,
+// rounded once more to the output type; ids outside [0, out) give a row of zeros.
+__global__ __launch_bounds__(256) void nvqs_embedding_kernel(NvqsK k, const uint8_t *__restrict__ w,
+                                                             const int64_t *__restrict__ ids, void *__restrict__ outp,
+                                                             int out_dtype, int64_t ldo) {
+    const int sb = blockIdx.x * 256 + threadIdx.x;
+    if (sb >= k.nsign) return;
+    const int row = blockIdx.y;
+    const int64_t tok = ids[row];
+    const int64_t at = static_cast<int64_t>(row) * ldo + sb * 8;
+    const int ncol = min(8, k.neuron_len - sb * 8);
+    if (tok < 0 || tok >= k.out) {
+        for (int i = 0; i < ncol; ++i) store_rounded(outp, at + i, 0.f, out_dtype);
+        return;
+    }
+    const int n = static_cast<int>(tok);
+    const float *lut = nvqs_lut(k, w);
+    const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+    const int8_t *cbp = reinterpret_cast<const int8_t *>(bfs + 16);
+    const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[n];
+    const NvqsBlock b = nvqs_block(k, w, lut, bfs, [&](int64_t i) { return cbp[i]; }, anchor, n, sb);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        if (i < ncol) store_rounded(outp, at + i, __fmul_rn(b.mag[i], b.scale), out_dtype);
+}
+
 // ---- GEMV: a wave per neuron, MB rows per pass --------------------------------------------------------------------
 // LDS (CB_LDS): the int8 codebooks.  The activation rows are read as 16-byte chunks straight from global memory (they
 // stay in L2: every wave of the grid reads the same rows).
@@ -514,6 +540,27 @@ extern "C" int mfq_hip_nvqs_dequant_rows_f32(const mfq_nvqs_desc *d, const void 
                            ld, static_cast<float *>(nullptr), 0);
     }
     return check_launch("nvqs_dequant_f32");
+}
+
+extern "C" int mfq_hip_nvqs_embedding(const mfq_nvqs_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,
+                                      int out_dtype, int64_t ldo, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight, MFQ_ERR_INVALID, "nvqs_embedding: null argument");
+    MFQ_REQUIRE(n_ids >= 0, MFQ_ERR_INVALID, "nvqs_embedding: n_ids=%d", n_ids);
+    MFQ_REQUIRE(out_dtype == MFQ_X_BF16 || out_dtype == MFQ_X_F16 || out_dtype == MFQ_X_F32, MFQ_ERR_INVALID,
+                "nvqs_embedding: out_dtype=%d", out_dtype);
+    MFQ_REQUIRE(ldo >= d->neuron_len, MFQ_ERR_INVALID, "nvqs_embedding: ldo %lld < neuron_len %d", static_cast<long long>(ldo),
+                d->neuron_len);
+    if (n_ids == 0) return MFQ_OK;
+    MFQ_REQUIRE(ids && out, MFQ_ERR_INVALID, "nvqs_embedding: null ids or output");
+    const NvqsK k = to_k(d);
+    const size_t esize = out_dtype == MFQ_X_F32 ? 4 : 2;
+    for (int n0 = 0; n0 < n_ids; n0 += 65535) {  // the grid's second dimension holds 65535 rows
+        const int rows = n_ids - n0 < 65535 ? n_ids - n0 : 65535;
+        hipLaunchKernelGGL(nvqs_embedding_kernel, dim3(static_cast<unsigned>(ceil_div(k.nsign, 256)), static_cast<unsigned>(rows)),
+                           dim3(256), 0, as_stream(stream), k, static_cast<const uint8_t *>(weight), ids + n0,
+                           static_cast<void *>(static_cast<uint8_t *>(out) + static_cast<size_t>(n0) * ldo * esize), out_dtype, ldo);
+    }
+    return check_launch("nvqs_embedding");
 }
 
 extern "C" int mfq_hip_nvqs_dequant_f32(const mfq_nvqs_desc *d, const void *weight, float *w_out, int64_t ld,

@@ -276,17 +276,40 @@ def nint_matmul_input_mul(w: NintWeight, x: torch.Tensor, gate: torch.Tensor, mo
     return nint_matmul(w, out.reshape(x.shape))
 
 
-def nint_embedding(w: NintWeight, ids: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
-    """Rows ids of the dequantized table as out_dtype, shape ids.shape + [neuron_len]; ids outside the table give
-    zeros (embed_forward, cpp_runtime/mfq_decode.cpp:13929-13957)."""
+def _embedding_rows(entry, w, ids: torch.Tensor, out_dtype) -> torch.Tensor:
     codes = {torch.bfloat16: L.X_BF16, torch.float16: L.X_F16, torch.float32: L.X_F32}
     if out_dtype not in codes:
         raise TypeError(f"embedding rows are bfloat16, float16 or float32, got {out_dtype}")
     flat = ids.to(device=w.data.device, dtype=torch.int64).reshape(-1).contiguous()
     out = torch.empty((flat.numel(), w.neuron_len), dtype=out_dtype, device=w.data.device)
-    L.check(L.lib().mfq_hip_nint_embedding(C.byref(w.desc), _ptr(w.data), _ptr(flat), flat.numel(), _ptr(out),
-                                           codes[out_dtype], w.neuron_len, _stream()))
+    L.check(entry(C.byref(w.desc), _ptr(w.data), _ptr(flat), flat.numel(), _ptr(out), codes[out_dtype], w.neuron_len,
+                  _stream()))
     return out.reshape(*ids.shape, w.neuron_len)
+
+
+def nint_embedding(w: NintWeight, ids: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """Rows ids of the dequantized table as out_dtype, shape ids.shape + [neuron_len]; ids outside the table give
+    zeros (embed_forward, cpp_runtime/mfq_decode.cpp:13929-13957)."""
+    return _embedding_rows(L.lib().mfq_hip_nint_embedding, w, ids, out_dtype)
+
+
+def embedding(w, ids: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+    """Token-embedding rows of any table format embed_forward takes (cpp_runtime/mfq_decode.cpp:13929-13957): NINT,
+    NINT8-0 and the NVQ families; shape ids.shape + [neuron_len], ids outside the table give zeros.  Like the
+    reference, MX and NEPQ tables are refused."""
+    from .runtime_vq import NvqsWeight, NvqWeight
+    lib = L.lib()
+    if isinstance(w, QuantLinear):
+        w = w.weight
+    if isinstance(w, NintWeight):
+        return _embedding_rows(lib.mfq_hip_nint_embedding, w, ids, out_dtype)
+    if isinstance(w, Nint8ZeroWeight):
+        return _embedding_rows(lib.mfq_hip_nint8z_embedding, w, ids, out_dtype)
+    if isinstance(w, NvqsWeight):
+        return _embedding_rows(lib.mfq_hip_nvqs_embedding, w, ids, out_dtype)
+    if isinstance(w, NvqWeight):
+        return _embedding_rows(lib.mfq_hip_nvq_embedding, w, ids, out_dtype)
+    raise TypeError(f"token embeddings are not supported for {type(w).__name__} tables")
 
 
 def nint_matmul_argmax(w: NintWeight, x: torch.Tensor, return_logits: bool = False):
@@ -378,6 +401,10 @@ class QuantLinear:
 
     def dequantize(self) -> torch.Tensor:
         return self.weight.dequantize()
+
+    def embedding(self, ids: torch.Tensor, out_dtype=torch.float16) -> torch.Tensor:
+        """The tensor as a token-embedding table: rows ids of its dequantized values (see embedding())."""
+        return embedding(self.weight, ids, out_dtype)
 
 
 def load_quant_linear(dtype: str, blob, device="cuda") -> QuantLinear:
