@@ -252,6 +252,11 @@ int mfq_hip_nint8z_dequant_f32(const mfq_nint8z_desc *d, const void *weight, flo
  * mfq/kernels/cuda/embedding.cu:190-220). */
 int mfq_hip_nint8z_embedding(const mfq_nint8z_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,
                              int out_dtype, int64_t ldo, mfq_stream_t stream);
+/* mfq_hip_nvq_gemv_pairs (below) for a cohort of NINT8-0 experts that are tensors of their own: the pairs of a MoE
+ * decode step in one launch, the routing table read on the device. */
+int mfq_hip_nint8z_gemv_pairs(const mfq_nint8z_desc *d, const void *const *expert_weights, const int32_t *expert_slot, int E,
+                              const void *x, int x_dtype, int64_t ldx, int routed_input, const int32_t *ids, int T, int R,
+                              float *y, int64_t ldy, mfq_stream_t stream);
 /* y[M, out] = x[M, neuron_len] . W^T streaming the codes once per pass of up to 8 rows (fewer when the fp16
  * activations of a pass would not fit 64 KB of LDS; MFQ_ERR_UNSUPPORTED when one row does not).  Replaces
  * nint8_zero_gemv_ws_cuda / nint8_zero_mmq_ws_cuda (cpp_runtime/mfq_decode.cpp:8167-8177). */
@@ -303,6 +308,15 @@ int mfq_hip_nvq_dequant_f32(const mfq_nvq_desc *d, const void *weight, float *w_
  * mfq/kernels/cuda/nvq_matmul.cu:1665-1719, launch :6026-6069). */
 int mfq_hip_nvq_embedding(const mfq_nvq_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,
                           int out_dtype, int64_t ldo, mfq_stream_t stream);
+/* A MoE decode step on a cohort of NVQ experts that are tensors of their own (one descriptor, one device pointer per
+ * expert in the device array expert_weights): y[p, 0:out] = W[ids[p]] . x[p (routed_input) or p / R] for every pair
+ * p < T * R whose expert belongs to the cohort -- expert_slot[e] (device, [E]) = index of expert e in expert_weights, -1
+ * for the experts of other cohorts and for ids outside [0, E), whose rows are left as they are.  One launch, nothing read
+ * back by the host.  Replaces the NVQ arm of the grouped decode kernels, nvq_moe_mmvq_kernel
+ * (mfq/kernels/cuda/nvq_matmul.cu:2588-3175; NintMoeWeight::forward's cohort loop, cpp_runtime/mfq_decode.cpp:4800-5360). */
+int mfq_hip_nvq_gemv_pairs(const mfq_nvq_desc *d, const void *const *expert_weights, const int32_t *expert_slot, int E,
+                           const void *x, int x_dtype, int64_t ldx, int routed_input, const int32_t *ids, int T, int R,
+                           float *y, int64_t ldy, mfq_stream_t stream);
 /* Replaces nvq_gemv_ws_cuda (cpp_runtime/mfq_decode.cpp:555-559). */
 int mfq_hip_nvq_gemv(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx,
                      int M, float *y, int64_t ldy, mfq_stream_t stream);
@@ -396,6 +410,12 @@ int mfq_hip_nvqs_dequant_rows_f32(const mfq_nvqs_desc *d, const void *weight, in
  * launch_by_format, :3344-3371). */
 int mfq_hip_nvqs_embedding(const mfq_nvqs_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,
                            int out_dtype, int64_t ldo, mfq_stream_t stream);
+/* mfq_hip_nvq_gemv_pairs for the families on this descriptor.  Either expert_weights (one tensor of out_per_expert rows
+ * per expert) or, with expert_weights null, `weight` = one tensor whose rows slot * out_per_expert ... are expert slot's
+ * (the NEPQ0 streams). */
+int mfq_hip_nvqs_gemv_pairs(const mfq_nvqs_desc *d, const void *const *expert_weights, const void *weight,
+                            int out_per_expert, const int32_t *expert_slot, int E, const void *x, int x_dtype, int64_t ldx,
+                            int routed_input, const int32_t *ids, int T, int R, float *y, int64_t ldy, mfq_stream_t stream);
 int mfq_hip_nvqs_gemv_rows(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, const void *x, int x_dtype,
                            int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream);
 size_t mfq_hip_nvqs_gemm_rows_workspace_bytes(const mfq_nvqs_desc *d, int nrows, int M);
@@ -426,6 +446,12 @@ size_t mfq_hip_mx_gemm_rows_workspace_bytes(int cols, int nrows, int M);
 int mfq_hip_mx_gemm_rows(int kind, const void *values, const void *scales, int rows, int cols, int row0, int nrows,
                          const void *x, int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, void *workspace,
                          size_t workspace_bytes, mfq_stream_t stream);
+/* mfq_hip_nvq_gemv_pairs for a native MXFP4 pool (one [experts * out_per_expert, cols] tensor, expert slot = rows
+ * slot * out_per_expert ...): the pairs of a MoE decode step in one launch (the MXFP4 arm of the grouped decode path,
+ * cpp_runtime/mfq_decode.cpp:4800-5360). */
+int mfq_hip_mx_gemv_pairs(int kind, const void *values, const void *scales, int rows, int cols, int out_per_expert,
+                          const int32_t *expert_slot, int E, const void *x, int x_dtype, int64_t ldx, int routed_input,
+                          const int32_t *ids, int T, int R, float *y, int64_t ldy, mfq_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
  * NEPQ1-S / NEPQ1-L (cross-expert table pool, bank id per 96 weights).  Rows are the
@@ -455,6 +481,11 @@ int mfq_hip_nepq_dequant_f32(const mfq_nepq_desc *d, const void *weight, float *
 /* `row0`, `nrows` select one expert's neurons; replaces nepq_gemv_ws_cuda. */
 int mfq_hip_nepq_gemv(const mfq_nepq_desc *d, const void *weight, int row0, int nrows, const void *x,
                       int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream);
+/* mfq_hip_nvq_gemv_pairs for an expert-shaped NEPQ1 tensor: expert slot owns rows slot * out_per_expert ... (a multiple of
+ * 16 rows per expert).  Replaces the NEPQ arm of the grouped decode kernels (nvq_matmul.cu:4210-4580). */
+int mfq_hip_nepq_gemv_pairs(const mfq_nepq_desc *d, const void *weight, int out_per_expert, const int32_t *expert_slot, int E,
+                            const void *x, int x_dtype, int64_t ldx, int routed_input, const int32_t *ids, int T, int R,
+                            float *y, int64_t ldy, mfq_stream_t stream);
 /* Any-M entry: mfq_hip_nepq_gemv's kernels up to 32 rows, from 33 rows a block-tiled MFMA GEMM that builds the
  * weight fragments from the ternary tables; replaces nepq_mmq_ws_cuda / nepq_gemm_f16_cuda
  * (mfq/kernels/cuda/mfq_cuda.cpp:331-350). */

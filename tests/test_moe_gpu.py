@@ -430,3 +430,80 @@ def test_mixed_family_cohorts_in_one_tensor():
         NintMoeWeight.from_blob(O.pack_nint_moe(bad))
     with pytest.raises(NotImplementedError, match="NINT cohorts only"):
         MoeExpertCache(1 << 20).register_source(blob)
+
+
+def test_mixed_family_decode_step_reads_the_routing_table_on_the_device():
+    """A decode-sized batch on a tensor with NVQ, stream-NVQ, 1-bit and NEPQ cohorts takes one launch per cohort over all
+    pairs (mfq_hip_*_gemv_pairs): the result agrees with the per-expert walk on the host; the whole call is captured
+    into a HIP graph and replayed with other routing tables and activations written into the same device buffers --
+    every replay equals the eager call, which only holds if nothing of the routing table is read by the host.  Ids
+    outside the table give zero rows."""
+    from tyloquant_amd.runtime_moe import ForeignCohort, MoeRoutePlan, NintMoeWeight, build_moe_route_plan
+    rng = np.random.default_rng(78)
+    out, K, E, R, T = 32, 192, 9, 3, 4
+    t = _mixed_family_moe(rng, out, K)
+    w = NintMoeWeight.from_blob(O.pack_nint_moe(t))
+    dense = O.dequantize_expertwise(t)
+    draws = []
+    for i in range(3):
+        ids = np.stack([rng.choice(E, size=R, replace=False) for _ in range(T)]).astype(np.int32)
+        if i == 2:
+            ids[0, 0], ids[1, 2] = -1, E + 5
+        draws.append((ids, torch.from_numpy((rng.standard_normal((T, K)) * 0.1).astype(np.float32)).to(torch.bfloat16)))
+    ids_d = torch.from_numpy(draws[0][0]).cuda()
+    x_d = draws[0][1].cuda()
+    route = build_moe_route_plan(ids_d, E)
+    assert route.ids_dst is None                         # a decode step: no route map
+    eager = w(x_d, route).clone()
+    saved, ForeignCohort.PAIRS_MAX = ForeignCohort.PAIRS_MAX, 0
+    try:
+        walked = w(x_d, route).clone()                   # the host's walk over the experts
+    finally:
+        ForeignCohort.PAIRS_MAX = saved
+    assert rel_l2(eager.cpu().numpy(), walked.cpu().numpy()) < REL_TOL    # other kernels, other fp16 roundings
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        y_g = w(x_d, route)
+    for ids, x in draws:
+        ids_d.copy_(torch.from_numpy(ids))
+        x_d.copy_(x)
+        want = w(x_d, route).clone()
+        torch.cuda.synchronize()
+        y_g.zero_()
+        (y_g.sum() + 1).item()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_g, want)
+        ok = (ids >= 0) & (ids < E)
+        ref = np.zeros((T, R, out), np.float32)
+        for t_ in range(T):
+            for r in range(R):
+                if ok[t_, r]:
+                    ref[t_, r] = dense[ids[t_, r]] @ x[t_].float().numpy()
+        got = want.cpu().numpy()
+        assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL
+        assert not got[~ok].any()
+    # a tensor without any NINT cohort, with a NINT8-0 cohort and a native MXFP4 pool: the same, captured and replayed
+    only = O.NintMoeTensor((6, out, K), [O.MoePool(np.array([5], dtype=np.int32), "NINT8-0", O.quantize_nint8_zero(
+                                             (rng.standard_normal((out, K)) * 0.02).astype(np.float32))),
+                                         O.MoePool(np.array([2, 0], dtype=np.int32), "NVQ3J-512",
+                                                   synth.nvq_jsc_random(rng, 2 * out, K, "d4_512", 2)),
+                                         O.MoePool(np.array([1], dtype=np.int32), "NVQ1-S", synth.nvq1_random(rng, "NVQ1-S", out, K)),
+                                         O.MoePool(np.array([4, 3], dtype=np.int32), "MXFP4",
+                                                   synth.mx_random(rng, "MXFP4", 2 * out, K, 120, 124))])
+    w2 = NintMoeWeight.from_blob(O.pack_nint_moe(only))
+    d2 = O.dequantize_expertwise(only)
+    ids2 = torch.from_numpy(np.stack([rng.choice(6, size=2, replace=False) for _ in range(T)]).astype(np.int32)).cuda()
+    route2 = build_moe_route_plan(ids2, 6)
+    w2(x_d, route2)                                      # builds the cohorts' device tables
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2):
+        y2 = w2(x_d, route2)
+    for _ in range(2):
+        idn = np.stack([rng.choice(6, size=2, replace=False) for _ in range(T)]).astype(np.int32)
+        ids2.copy_(torch.from_numpy(idn))
+        g2.replay()
+        torch.cuda.synchronize()
+        ref = O.moe_grouped_matmul(d2, x_d.float().cpu().numpy(), idn)
+        got = y2.cpu().numpy()
+        assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL * max(1.0, float(np.sqrt(np.mean(ref * ref))))

@@ -96,6 +96,8 @@ _SIGS = {
     "mfq_hip_nint8z_repack": (C.c_int, [C.POINTER(Nint8zDesc), vp, i64, vp, vp]),
     "mfq_hip_nint8z_dequant_f32": (C.c_int, [C.POINTER(Nint8zDesc), vp, vp, i64, vp]),
     "mfq_hip_nint8z_embedding": (C.c_int, [C.POINTER(Nint8zDesc), vp, vp, C.c_int, vp, C.c_int, i64, vp]),
+    "mfq_hip_nint8z_gemv_pairs": (C.c_int, [C.POINTER(Nint8zDesc), vp, vp, C.c_int, vp, C.c_int, i64, C.c_int, vp, C.c_int, C.c_int,
+                                  vp, i64, vp]),
     "mfq_hip_nint8z_gemv": (C.c_int, [C.POINTER(Nint8zDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
     "mfq_hip_nint8z_gemm_workspace_bytes": (sz, [C.POINTER(Nint8zDesc), C.c_int]),
     "mfq_hip_nint8z_gemm": (C.c_int, [C.POINTER(Nint8zDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
@@ -104,6 +106,8 @@ _SIGS = {
     "mfq_hip_nvq_repack_plain": (C.c_int, [C.POINTER(NvqDesc), vp, i64, vp, vp, vp]),
     "mfq_hip_nvq_dequant_f32": (C.c_int, [C.POINTER(NvqDesc), vp, vp, i64, vp]),
     "mfq_hip_nvq_embedding": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, vp, C.c_int, i64, vp]),
+    "mfq_hip_nvq_gemv_pairs": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, vp, C.c_int, i64, C.c_int, vp, C.c_int, C.c_int, vp,
+                               i64, vp]),
     "mfq_hip_nvq_gemv": (C.c_int, [C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
     "mfq_hip_nvq_gemv_multi2": (C.c_int, [C.POINTER(NvqDesc), vp, C.POINTER(NvqDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
     "mfq_hip_nvq_gemm_workspace_bytes": (sz, [C.POINTER(NvqDesc), C.c_int]),
@@ -114,6 +118,8 @@ _SIGS = {
     "mfq_hip_nvqs_repack_nepq0": (C.c_int, [C.POINTER(NvqsDesc), vp, i64, vp, vp]),
     "mfq_hip_nvqs_dequant_rows_f32": (C.c_int, [C.POINTER(NvqsDesc), vp, C.c_int, C.c_int, vp, i64, vp]),
     "mfq_hip_nvqs_embedding": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, C.c_int, vp, C.c_int, i64, vp]),
+    "mfq_hip_nvqs_gemv_pairs": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, C.c_int, vp, C.c_int, vp, C.c_int, i64, C.c_int, vp, C.c_int,
+                                C.c_int, vp, i64, vp]),
     "mfq_hip_nvqs_gemv_rows": (C.c_int, [C.POINTER(NvqsDesc), vp, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
     "mfq_hip_nvqs_gemm_rows_workspace_bytes": (sz, [C.POINTER(NvqsDesc), C.c_int, C.c_int]),
     "mfq_hip_nvqs_gemm_rows": (C.c_int, [C.POINTER(NvqsDesc), vp, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz,
@@ -127,12 +133,16 @@ _SIGS = {
     "mfq_hip_nvqs_gemm": (C.c_int, [C.POINTER(NvqsDesc), vp, vp, C.c_int, i64, C.c_int, vp, i64, vp, sz, vp]),
     "mfq_hip_mx_dequant_rows": (C.c_int, [C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, vp, i64, vp]),
     "mfq_hip_mx_gemm_rows_workspace_bytes": (sz, [C.c_int, C.c_int, C.c_int]),
+    "mfq_hip_mx_gemv_pairs": (C.c_int, [C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, vp, C.c_int, vp, C.c_int, i64, C.c_int, vp, C.c_int,
+                              C.c_int, vp, i64, vp]),
     "mfq_hip_mx_gemm_rows": (C.c_int, [C.c_int, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp, i64,
                                        vp, sz, vp]),
     "mfq_hip_nepq_plan": (C.c_int, [C.c_int] * 4 + [C.POINTER(NepqDesc)]),
     "mfq_hip_nepq_repack": (C.c_int, [C.POINTER(NepqDesc), vp, i64, vp, vp]),
     "mfq_hip_nepq_dequant_f32": (C.c_int, [C.POINTER(NepqDesc), vp, vp, i64, vp]),
     "mfq_hip_nepq_gemv": (C.c_int, [C.POINTER(NepqDesc), vp, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp, i64, vp]),
+    "mfq_hip_nepq_gemv_pairs": (C.c_int, [C.POINTER(NepqDesc), vp, C.c_int, vp, C.c_int, vp, C.c_int, i64, C.c_int, vp, C.c_int,
+                                C.c_int, vp, i64, vp]),
     "mfq_hip_nepq_gemm_workspace_bytes": (sz, [C.POINTER(NepqDesc), C.c_int, C.c_int]),
     "mfq_hip_nepq_gemm": (C.c_int, [C.POINTER(NepqDesc), vp, C.c_int, C.c_int, vp, C.c_int, i64, C.c_int, vp, i64,
                                     vp, sz, vp]),

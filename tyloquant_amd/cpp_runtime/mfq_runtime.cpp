@@ -962,6 +962,7 @@ NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream
             } else {
                 fail("NINTM cohort family " + p.dtype + " is not supported");
             }
+            c.prepare_pairs(h.n_experts, h.out_per_expert, stream);
             w.foreign.push_back(std::move(c));
             continue;
         }
@@ -1005,16 +1006,86 @@ void MoeForeignCohort::dequantize(int local, float *out, mfq_stream_t stream) co
     hip_check(hipStreamSynchronize(hs(stream)), "foreign cohort dequantize");
 }
 
+void MoeForeignCohort::prepare_pairs(int n_experts, int out_per_expert, mfq_stream_t stream) {
+    if (nepq && !nepq->streams && out_per_expert % 16) return;  // NEPQ1 experts must be whole row-blocks
+    std::vector<int32_t> slot(static_cast<size_t>(n_experts), -1);
+    for (size_t i = 0; i < expert_ids.size(); ++i) slot[static_cast<size_t>(expert_ids[i])] = static_cast<int32_t>(i);
+    pair_slot.ensure(slot.size() * 4);
+    hip_check(hipMemcpyAsync(pair_slot.get(), slot.data(), slot.size() * 4, hipMemcpyHostToDevice, hs(stream)), "NINTM cohort tables");
+    std::vector<const void *> ptrs;
+    if (!linears.empty()) {
+        for (const QuantLinear &q : linears) ptrs.push_back(q.kind == QuantLinearKind::Nint8Zero ? q.nint8z->data.get() : q.nvq->data.get());
+        pair_weights.ensure(ptrs.size() * sizeof(void *));
+        hip_check(hipMemcpyAsync(pair_weights.get(), ptrs.data(), ptrs.size() * sizeof(void *), hipMemcpyHostToDevice, hs(stream)),
+                  "NINTM cohort tables");
+    }
+    hip_check(hipStreamSynchronize(hs(stream)), "NINTM cohort tables");  // the host vectors go out of scope
+}
+
+bool MoeForeignCohort::matmul_pairs(int n_experts, int out_per_expert, const void *x, int x_dtype, int64_t ldx, bool routed_input,
+                                    const int32_t *ids, int T, int R, float *out, mfq_stream_t stream) const {
+    if (!pair_slot.get()) return false;
+    const int32_t *slot = static_cast<const int32_t *>(pair_slot.get());
+    if (mx) {
+        abi_check(mfq_hip_mx_gemv_pairs(mx->kind, mx->values.get(), mx->scales.get(), static_cast<int>(mx->rows),
+                                        static_cast<int>(mx->cols), out_per_expert, slot, n_experts, x, x_dtype, ldx,
+                                        routed_input ? 1 : 0, ids, T, R, out, out_per_expert, stream));
+        return true;
+    }
+    if (nepq) {
+        const NepqWeight &w = *nepq;
+        const int K = static_cast<int>(w.neuron_len());
+        if (w.rotation_block) {
+            const int rows = routed_input ? T * R : T;
+            w.rotated.ensure(static_cast<size_t>(rows) * K * 2);
+            abi_check(mfq_hip_nepq_hadamard(x, x_dtype, ldx, rows, K, w.rotation_block, static_cast<const int8_t *>(w.signs.get()),
+                                            w.rotated.get(), K, stream));
+            x = w.rotated.get();
+            ldx = K;
+        }
+        if (w.streams)
+            abi_check(mfq_hip_nvqs_gemv_pairs(&w.sdesc, nullptr, w.data.get(), out_per_expert, slot, n_experts, x, x_dtype, ldx,
+                                              routed_input ? 1 : 0, ids, T, R, out, out_per_expert, stream));
+        else
+            abi_check(mfq_hip_nepq_gemv_pairs(&w.desc, w.data.get(), out_per_expert, slot, n_experts, x, x_dtype, ldx,
+                                              routed_input ? 1 : 0, ids, T, R, out, out_per_expert, stream));
+        return true;
+    }
+    const void *const *ptrs = static_cast<const void *const *>(pair_weights.get());
+    if (linears[0].kind == QuantLinearKind::Nint8Zero) {
+        abi_check(mfq_hip_nint8z_gemv_pairs(&linears[0].nint8z->desc, ptrs, slot, n_experts, x, x_dtype, ldx, routed_input ? 1 : 0,
+                                            ids, T, R, out, out_per_expert, stream));
+        return true;
+    }
+    const NvqWeight &w0 = *linears[0].nvq;
+    if (w0.streams)
+        abi_check(mfq_hip_nvqs_gemv_pairs(&w0.sdesc, ptrs, nullptr, out_per_expert, slot, n_experts, x, x_dtype, ldx,
+                                          routed_input ? 1 : 0, ids, T, R, out, out_per_expert, stream));
+    else
+        abi_check(mfq_hip_nvq_gemv_pairs(&w0.desc, ptrs, slot, n_experts, x, x_dtype, ldx, routed_input ? 1 : 0, ids, T, R, out,
+                                         out_per_expert, stream));
+    return true;
+}
+
 void NintMoeWeight::add_foreign(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &r, float *out,
                                 mfq_stream_t stream) const {
     if (foreign.empty()) return;
     if (neuron_len % 2 || ldx % 2) fail("mixed NINTM cohorts need activation rows of whole 32-bit words");
     const int T = r.tokens, R = r.routes;
+    // a decode step: one launch per cohort over all pairs, nothing read back; the cohorts without such a launch (and
+    // every cohort of a larger batch) take the walk below
+    std::vector<const MoeForeignCohort *> walk;
+    for (const MoeForeignCohort &c : foreign)
+        if (T * R > MoeForeignCohort::kPairsMax ||
+            !c.matmul_pairs(n_experts, out_per_expert, x, x_dtype, ldx, routed_input, r.ids, T, R, out, stream))
+            walk.push_back(&c);
+    if (walk.empty()) return;
     std::vector<int32_t> ids(static_cast<size_t>(T) * R);
     hip_check(hipStreamSynchronize(hs(stream)), "mixed NINTM: routing table");
     hip_check(hipMemcpy(ids.data(), r.ids, 4 * ids.size(), hipMemcpyDeviceToHost), "mixed NINTM: routing table");
     std::vector<int32_t> index;  // per expert: n pair rows, then n source rows
-    for (const MoeForeignCohort &c : foreign) {
+    for (const MoeForeignCohort *cp : walk) {
+        const MoeForeignCohort &c = *cp;
         for (size_t local = 0; local < c.expert_ids.size(); ++local) {
             const int32_t e = c.expert_ids[local];
             std::vector<int32_t> pair_rows, src_rows;

@@ -281,6 +281,16 @@ struct MoeForeignCohort {
     int64_t payload_bytes() const;
     void matmul(int local, const void *x, int x_dtype, int64_t ldx, int M, float *y, mfq_stream_t stream) const;
     void dequantize(int local, float *out, mfq_stream_t stream) const;  // [out_per_expert, K]
+    // One launch over all (token, route) pairs of a decode step, the routing table read on the device
+    // (mfq_hip_{nvq,nvqs,nepq,nint8z,mx}_gemv_pairs): out[p] = W[ids[p]] . x[p or p / R] for the pairs routed to this
+    // cohort.  prepare_pairs builds the device tables at load; matmul_pairs returns false where they were not built
+    // (NEPQ1 experts that are not whole row-blocks).  Replaces the cohort arms of the reference's grouped decode
+    // kernels (mfq/kernels/cuda/nvq_matmul.cu:2588-3175, 4210-4580; cpp_runtime/mfq_decode.cpp:4800-5360).
+    static constexpr int kPairsMax = 64;  // pairs up to which add_foreign takes this form
+    DeviceBuffer pair_slot, pair_weights;
+    void prepare_pairs(int n_experts, int out_per_expert, mfq_stream_t stream);
+    bool matmul_pairs(int n_experts, int out_per_expert, const void *x, int x_dtype, int64_t ldx, bool routed_input,
+                      const int32_t *ids, int T, int R, float *out, mfq_stream_t stream) const;
 };
 
 struct NintMoeWeight {

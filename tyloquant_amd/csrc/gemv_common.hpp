@@ -414,6 +414,17 @@ inline size_t gemv_lds_bytes(int mb, int spw, int gs, int nwaves, int rbw = 1) {
     return (static_cast<size_t>(mb) * spw * 16 * (gs / 2 + 2) * nwaves + static_cast<size_t>(rbw) * nwaves * mb * 16) * 4;
 }
 
+// One launch over the (token, route) pairs of a MoE decode step on a cohort whose kernels know nothing of experts:
+// block row p = blockIdx.y multiplies the tensor of expert ids[p] with activation row p (routed input) or p / R into
+// output row p.  slot[e] = index of expert e among the cohort's experts, -1 for an expert of another cohort (and ids
+// outside [0, E)): such blocks leave at once, before any barrier.  weights: one device pointer per expert of the cohort
+// (experts that are tensors of their own), or null for a cohort that is one expert-shaped tensor.  ids = null: a dense call.
+struct PairSel {
+    const int32_t *ids, *slot;
+    const uint8_t *const *weights;
+    int E, R, routed_input;
+};
+
 // Dense activations: rows m0 .. m0+MB-1 of x[M, ldx] / y[M, ldy].
 template <int MB>
 __device__ __forceinline__ void dense_rows(const uint16_t *x, int64_t ldx, float *y, int64_t ldy, int M, int m0,
@@ -424,6 +435,32 @@ __device__ __forceinline__ void dense_rows(const uint16_t *x, int64_t ldx, float
         xr[m] = ok ? x + static_cast<int64_t>(m0 + m) * ldx : nullptr;
         yr[m] = ok ? y + static_cast<int64_t>(m0 + m) * ldy : nullptr;
     }
+}
+
+// Rows of a block: dense_rows, or the pair blockIdx.y of a PairSel launch (one row per block).  False: the pair belongs
+// to another cohort.  `w` is replaced by the expert's tensor where the cohort has one per expert; `local` = its index.
+template <int MB>
+__device__ __forceinline__ bool select_rows(const PairSel &sel, const uint8_t *&w, int &local, const uint16_t *x, int64_t ldx,
+                                            float *y, int64_t ldy, int M, const uint16_t *(&xr)[MB], float *(&yr)[MB]) {
+    local = 0;
+    if (!sel.ids) {
+        dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
+        return true;
+    }
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        xr[m] = nullptr;
+        yr[m] = nullptr;
+    }
+    const int p = blockIdx.y;
+    const int e = sel.ids[p];
+    const int l = (e >= 0 && e < sel.E) ? sel.slot[e] : -1;
+    if (l < 0) return false;
+    local = l;
+    if (sel.weights) w = sel.weights[l];
+    xr[0] = x + static_cast<int64_t>(sel.routed_input ? p : p / sel.R) * ldx;
+    yr[0] = y + static_cast<int64_t>(p) * ldy;
+    return true;
 }
 
 }  // namespace mfq

@@ -6,6 +6,7 @@
 //   up to kMxGemvMaxM rows: a wave per neuron     mx_matmul.cu launch_mxfp8_small_m (rows 1..8 there)
 //   more rows: fp16 copy + MFMA GEMM              mfq_decode.cpp:8760-8802 (dequantize, then the fp16 GEMM)
 #include "common.hpp"
+#include "gemv_common.hpp"
 
 namespace mfq {
 
@@ -113,12 +114,27 @@ __global__ __launch_bounds__(256) void mx_stage_f16_kernel(MxK k, uint16_t *__re
 // A lane takes 16 bytes of the neuron at a time -- 32 MXFP4 or 16 MXFP8 weights under one scale -- and the matching
 // activations of the MB rows; fp32 accumulation, one wave reduction at the end.
 template <int KIND, int XF16, int MB>
-__global__ __launch_bounds__(256) void mx_gemv_kernel(MxK k, const uint16_t *__restrict__ x, int64_t ldx, int M,
-                                                      float *__restrict__ y, int64_t ldy) {
+__global__ __launch_bounds__(256) void mx_gemv_kernel(MxK k, const uint16_t *__restrict__ x_in, int64_t ldx, int M_in,
+                                                      float *__restrict__ y_in, int64_t ldy, PairSel sel) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = blockIdx.x * 4 + wave;
     if (r >= k.nrows) return;
-    const int row = k.row0 + r, m0 = blockIdx.y * MB;
+    const uint16_t *x = x_in;
+    float *y = y_in;
+    int M = M_in, m0 = blockIdx.y * MB;
+    if (sel.ids) {  // a pair of a MoE decode step: one row, the expert's rows of the pool (nrows = rows per expert)
+        const uint16_t *xr[1];
+        float *yr[1];
+        const uint8_t *unused = nullptr;
+        int local;
+        if (!select_rows<1>(sel, unused, local, x_in, ldx, y_in, ldy, M_in, xr, yr)) return;
+        k.row0 = local * k.nrows;
+        x = xr[0];
+        y = yr[0];
+        M = 1;
+        m0 = 0;
+    }
+    const int row = k.row0 + r;
     constexpr int PER = KIND == 4 ? 32 : 16;  // weights in 16 bytes
     const int64_t row_bytes = KIND == 4 ? k.cols / 2 : k.cols;
     const uint8_t *vrow = k.values + static_cast<int64_t>(row) * row_bytes;
@@ -173,16 +189,48 @@ int mx_check(const char *what, int kind, const void *values, const void *scales,
 template <int KIND, int XF16>
 int mx_launch_gemv(const MxK &k, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy, hipStream_t st) {
     const unsigned gx = static_cast<unsigned>(ceil_div(k.nrows, 4));
-    if (M == 1) hipLaunchKernelGGL((mx_gemv_kernel<KIND, XF16, 1>), dim3(gx, 1), dim3(256), 0, st, k, x, ldx, M, y, ldy);
-    else if (M == 2) hipLaunchKernelGGL((mx_gemv_kernel<KIND, XF16, 2>), dim3(gx, 1), dim3(256), 0, st, k, x, ldx, M, y, ldy);
-    else hipLaunchKernelGGL((mx_gemv_kernel<KIND, XF16, 4>), dim3(gx, static_cast<unsigned>(ceil_div(M, 4))), dim3(256), 0, st, k, x, ldx, M, y, ldy);
+    if (M == 1) hipLaunchKernelGGL((mx_gemv_kernel<KIND, XF16, 1>), dim3(gx, 1), dim3(256), 0, st, k, x, ldx, M, y, ldy, PairSel{});
+    else if (M == 2) hipLaunchKernelGGL((mx_gemv_kernel<KIND, XF16, 2>), dim3(gx, 1), dim3(256), 0, st, k, x, ldx, M, y, ldy, PairSel{});
+    else hipLaunchKernelGGL((mx_gemv_kernel<KIND, XF16, 4>), dim3(gx, static_cast<unsigned>(ceil_div(M, 4))), dim3(256), 0, st, k, x, ldx, M, y, ldy, PairSel{});
     return check_launch("mx_gemv");
+}
+
+// the same kernel over the pairs of a MoE decode step (see PairSel); k.nrows = rows per expert of the pool
+template <int KIND, int XF16>
+int mx_launch_pairs(const MxK &k, const uint16_t *x, int64_t ldx, int n_pairs, float *y, int64_t ldy, const PairSel &sel,
+                    hipStream_t st) {
+    hipLaunchKernelGGL((mx_gemv_kernel<KIND, XF16, 1>), dim3(static_cast<unsigned>(ceil_div(k.nrows, 4)), static_cast<unsigned>(n_pairs)),
+                       dim3(256), 0, st, k, x, ldx, n_pairs, y, ldy, sel);
+    return check_launch("mx_gemv_pairs");
 }
 
 }  // namespace
 }  // namespace mfq
 
 using namespace mfq;
+
+extern "C" int mfq_hip_mx_gemv_pairs(int kind, const void *values, const void *scales, int rows, int cols, int out_per_expert,
+                                     const int32_t *expert_slot, int E, const void *x, int x_dtype, int64_t ldx, int routed_input,
+                                     const int32_t *ids, int T, int R, float *y, int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(out_per_expert > 0 && rows % out_per_expert == 0, MFQ_ERR_INVALID,
+                "mx_gemv_pairs: %d rows per expert do not divide the pool's %d", out_per_expert, rows);
+    if (int rc = mx_check("mx_gemv_pairs", kind, values, scales, rows, cols, 0, out_per_expert)) return rc;
+    MFQ_REQUIRE(kind == 4 || out_per_expert % 128 == 0, MFQ_ERR_UNSUPPORTED,
+                "mx_gemv_pairs: MXFP8 experts must be whole 128-row scale blocks, got %d rows", out_per_expert);
+    MFQ_REQUIRE(expert_slot && x && ids && y, MFQ_ERR_INVALID, "mx_gemv_pairs: null argument");
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "mx_gemv_pairs: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(T >= 0 && R >= 1 && E >= 1, MFQ_ERR_INVALID, "mx_gemv_pairs: T=%d R=%d E=%d", T, R, E);
+    MFQ_REQUIRE(static_cast<int64_t>(T) * R <= 65535, MFQ_ERR_UNSUPPORTED, "mx_gemv_pairs: %lld pairs (at most 65535 per launch)",
+                static_cast<long long>(T) * R);
+    MFQ_REQUIRE(ldx >= cols && ldy >= out_per_expert, MFQ_ERR_INVALID, "mx_gemv_pairs: ldx/ldy smaller than the tensor");
+    if (T == 0) return MFQ_OK;
+    const PairSel sel{ids, expert_slot, nullptr, E, R, routed_input ? 1 : 0};
+    const MxK k{kind, rows, cols, 0, out_per_expert, static_cast<const uint8_t *>(values), static_cast<const uint8_t *>(scales)};
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    hipStream_t st = as_stream(stream);
+    if (kind == 4) return x_dtype == MFQ_X_F16 ? mx_launch_pairs<4, 1>(k, xp, ldx, T * R, y, ldy, sel, st) : mx_launch_pairs<4, 0>(k, xp, ldx, T * R, y, ldy, sel, st);
+    return x_dtype == MFQ_X_F16 ? mx_launch_pairs<8, 1>(k, xp, ldx, T * R, y, ldy, sel, st) : mx_launch_pairs<8, 0>(k, xp, ldx, T * R, y, ldy, sel, st);
+}
 
 extern "C" int mfq_hip_mx_dequant_rows(int kind, const void *values, const void *scales, int rows, int cols, int row0,
                                        int nrows, int out_dtype, void *w_out, int64_t ld, mfq_stream_t stream) {

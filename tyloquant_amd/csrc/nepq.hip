@@ -153,18 +153,24 @@ __global__ void nepq_dequant_kernel(NepqK k, const uint8_t *__restrict__ w, int 
 // PROF: the profile (2 = S, 3 = L) as a constant -- a decoder that branches on it at run time splits every unit into
 // basic blocks the scheduler cannot mix, and the kernel spills.
 template <int XF16, int MB, int TAB_LDS, int RPB, int PROF>
-__global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t *__restrict__ w, int rb0, int row0,
+__global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t *__restrict__ w_in, int rb0, int row0,
                                                          int nrows, const uint16_t *__restrict__ x, int64_t ldx, int M,
-                                                         float *__restrict__ y, int64_t ldy, int spw) {
+                                                         float *__restrict__ y, int64_t ldy, int spw, PairSel sel) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     constexpr uint32_t MAGIC = 0x64006400u;  // fp16 (1024, 1024): digit d becomes 1024 + d
     constexpr float BIAS = 1024.f;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
-    const int rb = rb0 + blockIdx.x * RPB;
-    const int rb_last = rb0 + (nrows + 15) / 16 - 1;  // row-blocks past it repeat it; their sums are dropped
     const uint16_t *xr[MB];
     float *yr[MB];
-    dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
+    const uint8_t *w = w_in;
+    int local;
+    if (!select_rows<MB>(sel, w, local, x, ldx, y, ldy, M, xr, yr)) return;
+    if (sel.ids) {  // a pair of a MoE decode step: the expert's rows of the expert-shaped tensor (nrows = rows per expert)
+        row0 = local * nrows;
+        rb0 = row0 / 16;
+    }
+    const int rb = rb0 + blockIdx.x * RPB;
+    const int rb_last = rb0 + (nrows + 15) / 16 - 1;  // row-blocks past it repeat it; their sums are dropped
     const uint16_t *gtab = reinterpret_cast<const uint16_t *>(w + k.tables_off);
     const int ntab = k.banks * k.entries;  // u16 entries
     uint16_t *ltab = reinterpret_cast<uint16_t *>(lds);
@@ -905,7 +911,7 @@ static int nepq_launch_as(const NepqK &k, const uint8_t *w, int row0, int nrows,
     do {                                                                                                                        \
         if (int rc = nepq_allow_lds(nepq_gemv_kernel<XF16, MB, T, RPB, P>, lds)) return rc;                                     \
         hipLaunchKernelGGL((nepq_gemv_kernel<XF16, MB, T, RPB, P>), grid, block, lds, st, k, w, rb0, row0, nrows, x, ldx, M, y, \
-                           ldy, spw);                                                                                           \
+                           ldy, spw, PairSel{});                                                                                \
     } while (0)
     if (k.profile == 2) {
         if (tab_lds) MFQ_NEPQ_GEMV(1, 2); else MFQ_NEPQ_GEMV(0, 2);
@@ -914,6 +920,33 @@ static int nepq_launch_as(const NepqK &k, const uint8_t *w, int row0, int nrows,
     }
 #undef MFQ_NEPQ_GEMV
     return check_launch("nepq_gemv");
+}
+
+// the same kernel, one row and one row-block per block, over the pairs of a MoE decode step (see PairSel): the experts are
+// the row ranges of one expert-shaped tensor
+template <int XF16>
+static int nepq_launch_pairs(const NepqK &k, const uint8_t *w, int out_per_expert, const uint16_t *x, int64_t ldx, int n_pairs,
+                             float *y, int64_t ldy, const PairSel &sel, hipStream_t st) {
+    const int nrb = static_cast<int>(ceil_div(out_per_expert, 16));
+    int spw, nwaves;
+    size_t lds;
+    bool tab_lds;
+    nepq_gemv_shape(k, nrb * n_pairs, 1, 1, spw, nwaves, lds, tab_lds);
+    MFQ_REQUIRE(lds <= kNepqTableLds, MFQ_ERR_UNSUPPORTED, "nepq_gemv_pairs: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
+    const dim3 grid(static_cast<unsigned>(nrb), static_cast<unsigned>(n_pairs)), block(64 * nwaves);
+#define MFQ_NEPQ_PAIRS(T, P)                                                                                              \
+    do {                                                                                                                  \
+        if (int rc = nepq_allow_lds(nepq_gemv_kernel<XF16, 1, T, 1, P>, lds)) return rc;                                   \
+        hipLaunchKernelGGL((nepq_gemv_kernel<XF16, 1, T, 1, P>), grid, block, lds, st, k, w, 0, 0, out_per_expert, x, ldx,  \
+                           n_pairs, y, ldy, spw, sel);                                                                    \
+    } while (0)
+    if (k.profile == 2) {
+        if (tab_lds) MFQ_NEPQ_PAIRS(1, 2); else MFQ_NEPQ_PAIRS(0, 2);
+    } else {
+        if (tab_lds) MFQ_NEPQ_PAIRS(1, 3); else MFQ_NEPQ_PAIRS(0, 3);
+    }
+#undef MFQ_NEPQ_PAIRS
+    return check_launch("nepq_gemv_pairs");
 }
 template <int XF16, int MB>
 static int nepq_launch(const NepqK &k, const uint8_t *w, int row0, int nrows, const uint16_t *x, int64_t ldx, int M,
@@ -1071,6 +1104,26 @@ extern "C" int mfq_hip_nepq_gemv(const mfq_nepq_desc *d, const void *weight, int
     if (int rc = nepq_check_rows(d, row0, nrows)) return rc;
     MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= nrows, MFQ_ERR_INVALID, "nepq_gemv: ldx/ldy smaller than the tensor");
     return nepq_gemv_any(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, as_stream(stream));
+}
+
+extern "C" int mfq_hip_nepq_gemv_pairs(const mfq_nepq_desc *d, const void *weight, int out_per_expert, const int32_t *expert_slot,
+                                       int E, const void *x, int x_dtype, int64_t ldx, int routed_input, const int32_t *ids, int T,
+                                       int R, float *y, int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && weight && expert_slot && x && ids && y, MFQ_ERR_INVALID, "nepq_gemv_pairs: null argument");
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nepq_gemv_pairs: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(T >= 0 && R >= 1 && E >= 1, MFQ_ERR_INVALID, "nepq_gemv_pairs: T=%d R=%d E=%d", T, R, E);
+    MFQ_REQUIRE(out_per_expert > 0 && out_per_expert % 16 == 0 && d->rows % out_per_expert == 0, MFQ_ERR_UNSUPPORTED,
+                "nepq_gemv_pairs: %d rows per expert (a multiple of 16 that divides the tensor's %d)", out_per_expert, d->rows);
+    MFQ_REQUIRE(static_cast<int64_t>(T) * R <= 65535, MFQ_ERR_UNSUPPORTED, "nepq_gemv_pairs: %lld pairs (at most 65535 per launch)",
+                static_cast<long long>(T) * R);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= out_per_expert, MFQ_ERR_INVALID, "nepq_gemv_pairs: ldx/ldy smaller than the tensor");
+    if (T == 0) return MFQ_OK;
+    const PairSel sel{ids, expert_slot, nullptr, E, R, routed_input ? 1 : 0};
+    const NepqK k = to_k(d);
+    const uint8_t *w = static_cast<const uint8_t *>(weight);
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    return x_dtype == MFQ_X_F16 ? nepq_launch_pairs<1>(k, w, out_per_expert, xp, ldx, T * R, y, ldy, sel, as_stream(stream))
+                                : nepq_launch_pairs<0>(k, w, out_per_expert, xp, ldx, T * R, y, ldy, sel, as_stream(stream));
 }
 
 // The reference's Python policy keeps M <= 16 on the GEMV.  Two 16-row passes of the matrix-core streaming kernel cost

@@ -100,11 +100,26 @@ __global__ __launch_bounds__(256) void nint8z_dequant_f16_kernel(N8zK k, const u
 // Block = 4 waves, RW rows per wave in turn; activation rows m0 .. m0 + MB - 1 of the pass.  LDS: fp16 x [MB][K], then
 // float chunk sums [MB][K / 16].
 template <int XF16, int MB>
-__global__ __launch_bounds__(256) void nint8z_gemv_kernel(N8zK k, const uint8_t *__restrict__ w, const uint16_t *__restrict__ x,
-                                                          int64_t ldx, int M, float *__restrict__ y, int64_t ldy, int rw) {
+__global__ __launch_bounds__(256) void nint8z_gemv_kernel(N8zK k, const uint8_t *__restrict__ w_in, const uint16_t *__restrict__ x_in,
+                                                          int64_t ldx, int M_in, float *__restrict__ y_in, int64_t ldy, int rw,
+                                                          PairSel sel) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int K = k.neuron_len, m0 = blockIdx.y * MB;
+    const uint8_t *w = w_in;
+    const uint16_t *x = x_in;
+    float *y = y_in;
+    int M = M_in, m0 = blockIdx.y * MB;
+    if (sel.ids) {  // a pair of a MoE decode step: one row, the expert's own tensor
+        const uint16_t *xr[1];
+        float *yr[1];
+        int local;
+        if (!select_rows<1>(sel, w, local, x_in, ldx, y_in, ldy, M_in, xr, yr)) return;
+        x = xr[0];
+        y = yr[0];
+        M = 1;
+        m0 = 0;
+    }
+    const int K = k.neuron_len;
     uint16_t *xh = reinterpret_cast<uint16_t *>(lds);
     float *xsum = reinterpret_cast<float *>(lds + MB * K / 2);
     if (ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {  // 16-byte chunks (K is a multiple of 32)
@@ -314,10 +329,25 @@ static int nint8z_gemv_launch(const N8zK &k, const uint8_t *w, const uint16_t *x
     const dim3 grid(static_cast<unsigned>(ceil_div(k.out, 4 * rw)), static_cast<unsigned>(ceil_div(M, mb)));
     const size_t lds = static_cast<size_t>(mb) * k.neuron_len * 2 + static_cast<size_t>(mb) * (k.neuron_len / 16) * 4;
 #define MFQ_N8Z(MB)                                                                                                  \
-    if (mb == MB) hipLaunchKernelGGL((nint8z_gemv_kernel<XF16, MB>), grid, dim3(256), lds, st, k, w, x, ldx, M, y, ldy, rw);
+    if (mb == MB) hipLaunchKernelGGL((nint8z_gemv_kernel<XF16, MB>), grid, dim3(256), lds, st, k, w, x, ldx, M, y, ldy, rw, PairSel{});
     MFQ_N8Z(8) MFQ_N8Z(4) MFQ_N8Z(2) MFQ_N8Z(1)
 #undef MFQ_N8Z
     return check_launch("nint8z_gemv");
+}
+
+// the same kernel, one row per block row, over the pairs of a MoE decode step (see PairSel)
+template <int XF16>
+static int nint8z_launch_pairs(const N8zK &k, const uint16_t *x, int64_t ldx, int n_pairs, float *y, int64_t ldy, const PairSel &sel,
+                               hipStream_t st) {
+    MFQ_REQUIRE(nint8z_rows_per_pass(k.neuron_len, 1) > 0, MFQ_ERR_UNSUPPORTED, "nint8z_gemv_pairs: neuron_len %d does not fit the LDS",
+                k.neuron_len);
+    int rw = k.out / 1024;  // about four blocks per compute unit and pair
+    if (rw < 1) rw = 1;
+    const dim3 grid(static_cast<unsigned>(ceil_div(k.out, 4 * rw)), static_cast<unsigned>(n_pairs));
+    const size_t lds = static_cast<size_t>(k.neuron_len) * 2 + static_cast<size_t>(k.neuron_len / 16) * 4;
+    hipLaunchKernelGGL((nint8z_gemv_kernel<XF16, 1>), grid, dim3(256), lds, st, k, static_cast<const uint8_t *>(nullptr), x, ldx, n_pairs,
+                       y, ldy, rw, sel);
+    return check_launch("nint8z_gemv_pairs");
 }
 
 }  // namespace mfq
@@ -347,6 +377,23 @@ extern "C" int mfq_hip_nint8z_repack(const mfq_nint8z_desc *d, const void *block
     hipLaunchKernelGGL(nint8z_repack_kernel, dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, as_stream(stream), k,
                        static_cast<const uint8_t *>(blocks), static_cast<uint8_t *>(weight));
     return check_launch("nint8z_repack");
+}
+
+extern "C" int mfq_hip_nint8z_gemv_pairs(const mfq_nint8z_desc *d, const void *const *expert_weights, const int32_t *expert_slot,
+                                         int E, const void *x, int x_dtype, int64_t ldx, int routed_input, const int32_t *ids, int T,
+                                         int R, float *y, int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && expert_weights && expert_slot && x && ids && y, MFQ_ERR_INVALID, "nint8z_gemv_pairs: null argument");
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nint8z_gemv_pairs: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(T >= 0 && R >= 1 && E >= 1, MFQ_ERR_INVALID, "nint8z_gemv_pairs: T=%d R=%d E=%d", T, R, E);
+    MFQ_REQUIRE(static_cast<int64_t>(T) * R <= 65535, MFQ_ERR_UNSUPPORTED, "nint8z_gemv_pairs: %lld pairs (at most 65535 per launch)",
+                static_cast<long long>(T) * R);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nint8z_gemv_pairs: ldx/ldy smaller than the tensor");
+    if (T == 0) return MFQ_OK;
+    const PairSel sel{ids, expert_slot, reinterpret_cast<const uint8_t *const *>(expert_weights), E, R, routed_input ? 1 : 0};
+    const N8zK k = to_k(d);
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    return x_dtype == MFQ_X_F16 ? nint8z_launch_pairs<1>(k, xp, ldx, T * R, y, ldy, sel, as_stream(stream))
+                                : nint8z_launch_pairs<0>(k, xp, ldx, T * R, y, ldy, sel, as_stream(stream));
 }
 
 extern "C" int mfq_hip_nint8z_embedding(const mfq_nint8z_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,

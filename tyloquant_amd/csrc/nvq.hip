@@ -204,15 +204,17 @@ __global__ __launch_bounds__(64) void nvq_embedding_kernel(NvqK k, const uint8_t
 // ---- GEMV ------------------------------------------------------------------------------
 // LDS map (dwords): [codebook pairs: banks*entries*2][sign xor table: 128*4][lut: 16][bank: 16][x staging ...]
 template <int XF16, int MB>
-__global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *__restrict__ w,
+__global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *__restrict__ w_in,
                                                         const uint16_t *__restrict__ x, int64_t ldx, int M,
-                                                        float *__restrict__ y, int64_t ldy, int spw) {
+                                                        float *__restrict__ y, int64_t ldy, int spw, PairSel sel) {
     extern __shared__ uint32_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
     const int rb = blockIdx.x;
     const uint16_t *xr[MB];
     float *yr[MB];
-    dense_rows<MB>(x, ldx, y, ldy, M, blockIdx.y * MB, xr, yr);
+    const uint8_t *w = w_in;
+    int local;
+    if (!select_rows<MB>(sel, w, local, x, ldx, y, ldy, M, xr, yr)) return;
     const int ncb = k.banks * k.entries;
     uint32_t *cbp = lds;                 // 2 dwords per entry: (m0, m1), (m2, m3) as fp16 pairs
     uint32_t *sgx = cbp + 2 * ncb;       // 4 dwords per 7-bit mask
@@ -1376,8 +1378,21 @@ static int nvq_launch(const NvqK &k, const uint8_t *w, const uint16_t *x, int64_
     nvq_gemv_shape(k, MB, spw, nwaves, lds);
     MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nvq_gemv: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
     hipLaunchKernelGGL((nvq_gemv_kernel<XF16, MB>), dim3(k.n_rowblocks, static_cast<unsigned>(ceil_div(M, MB))),
-                       dim3(64 * nwaves), lds, st, k, w, x, ldx, M, y, ldy, spw);
+                       dim3(64 * nwaves), lds, st, k, w, x, ldx, M, y, ldy, spw, PairSel{});
     return check_launch("nvq_gemv");
+}
+
+// the same kernel, one row per block, over the pairs of a MoE decode step (see PairSel)
+template <int XF16>
+static int nvq_launch_pairs(const NvqK &k, const uint16_t *x, int64_t ldx, int n_pairs, float *y, int64_t ldy, const PairSel &sel,
+                            hipStream_t st) {
+    int spw, nwaves;
+    size_t lds;
+    nvq_gemv_shape(k, 1, spw, nwaves, lds);
+    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nvq_gemv_pairs: neuron_len %d needs %zu bytes of LDS", k.neuron_len, lds);
+    hipLaunchKernelGGL((nvq_gemv_kernel<XF16, 1>), dim3(k.n_rowblocks, static_cast<unsigned>(n_pairs)), dim3(64 * nwaves), lds, st, k,
+                       static_cast<const uint8_t *>(nullptr), x, ldx, n_pairs, y, ldy, spw, sel);
+    return check_launch("nvq_gemv_pairs");
 }
 
 static int nvq_gemv_any(const mfq_nvq_desc *d, const void *weight, const void *x, int x_dtype, int64_t ldx, int M,
@@ -1476,6 +1491,23 @@ extern "C" int mfq_hip_nvq_repack_plain(const mfq_nvq_desc *d, const void *paylo
                        static_cast<const uint8_t *>(nullptr), static_cast<const int8_t *>(grid),
                        static_cast<uint8_t *>(weight));
     return check_launch("nvq_repack_plain");
+}
+
+extern "C" int mfq_hip_nvq_gemv_pairs(const mfq_nvq_desc *d, const void *const *expert_weights, const int32_t *expert_slot, int E,
+                                      const void *x, int x_dtype, int64_t ldx, int routed_input, const int32_t *ids, int T, int R,
+                                      float *y, int64_t ldy, mfq_stream_t stream) {
+    MFQ_REQUIRE(d && expert_weights && expert_slot && x && ids && y, MFQ_ERR_INVALID, "nvq_gemv_pairs: null argument");
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvq_gemv_pairs: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(T >= 0 && R >= 1 && E >= 1, MFQ_ERR_INVALID, "nvq_gemv_pairs: T=%d R=%d E=%d", T, R, E);
+    MFQ_REQUIRE(static_cast<int64_t>(T) * R <= 65535, MFQ_ERR_UNSUPPORTED, "nvq_gemv_pairs: %lld pairs (at most 65535 per launch)",
+                static_cast<long long>(T) * R);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= d->out, MFQ_ERR_INVALID, "nvq_gemv_pairs: ldx/ldy smaller than the tensor");
+    if (T == 0) return MFQ_OK;
+    const PairSel sel{ids, expert_slot, reinterpret_cast<const uint8_t *const *>(expert_weights), E, R, routed_input ? 1 : 0};
+    const NvqK k = to_k(d);
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    return x_dtype == MFQ_X_F16 ? nvq_launch_pairs<1>(k, xp, ldx, T * R, y, ldy, sel, as_stream(stream))
+                                : nvq_launch_pairs<0>(k, xp, ldx, T * R, y, ldy, sel, as_stream(stream));
 }
 
 extern "C" int mfq_hip_nvq_embedding(const mfq_nvq_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,

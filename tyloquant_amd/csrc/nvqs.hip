@@ -292,11 +292,26 @@ __global__ __launch_bounds__(256) void nvqs_embedding_kernel(NvqsK k, const uint
 // LDS (CB_LDS): the int8 codebooks.  The activation rows are read as 16-byte chunks straight from global memory (they
 // stay in L2: every wave of the grid reads the same rows).
 template <int XF16, int MB, bool CB_LDS>
-__global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *__restrict__ w,
-                                                        const uint16_t *__restrict__ x, int64_t ldx, int M,
-                                                        float *__restrict__ y, int64_t ldy) {
+__global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *__restrict__ w_in,
+                                                        const uint16_t *__restrict__ x_in, int64_t ldx, int M_in,
+                                                        float *__restrict__ y_in, int64_t ldy, PairSel sel) {
     extern __shared__ __attribute__((aligned(16))) int8_t cbl[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint8_t *w = w_in;
+    const uint16_t *x = x_in;
+    float *y = y_in;
+    int M = M_in, m0 = blockIdx.y * MB;
+    if (sel.ids) {  // a pair of a MoE decode step: one row, the expert's own tensor
+        const uint16_t *xr[1];
+        float *yr[1];
+        int local;
+        if (!select_rows<1>(sel, w, local, x_in, ldx, y_in, ldy, M_in, xr, yr)) return;
+        if (!sel.weights) k.row0 = local * k.nrows;  // the experts are row ranges of one tensor
+        x = xr[0];
+        y = yr[0];
+        M = 1;
+        m0 = 0;
+    }
     const float *lut = nvqs_lut(k, w);
     const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
     const int8_t *cbp = reinterpret_cast<const int8_t *>(bfs + 16);
@@ -308,7 +323,6 @@ __global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *
     const int row = blockIdx.x * (blockDim.x >> 6) + wave;
     if (row >= k.nrows) return;
     const int n = k.row0 + row;
-    const int m0 = blockIdx.y * MB;
     const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[n];
     float acc[MB];
 #pragma unroll
@@ -367,10 +381,23 @@ static int nvqs_launch_gemv(const NvqsK &k, const uint8_t *w, const uint16_t *x,
     const size_t ncb = static_cast<size_t>(k.cb_bytes);
     const dim3 grid(static_cast<unsigned>(ceil_div(k.nrows, 4)), static_cast<unsigned>(ceil_div(M, MB)));
     if (ncb <= 49152 && ncb % 4 == 0)
-        hipLaunchKernelGGL((nvqs_gemv_kernel<XF16, MB, true>), grid, dim3(256), ncb, st, k, w, x, ldx, M, y, ldy);
+        hipLaunchKernelGGL((nvqs_gemv_kernel<XF16, MB, true>), grid, dim3(256), ncb, st, k, w, x, ldx, M, y, ldy, PairSel{});
     else
-        hipLaunchKernelGGL((nvqs_gemv_kernel<XF16, MB, false>), grid, dim3(256), 0, st, k, w, x, ldx, M, y, ldy);
+        hipLaunchKernelGGL((nvqs_gemv_kernel<XF16, MB, false>), grid, dim3(256), 0, st, k, w, x, ldx, M, y, ldy, PairSel{});
     return check_launch("nvqs_gemv");
+}
+
+// the same kernel, one row per block row, over the pairs of a MoE decode step (see PairSel)
+template <int XF16>
+static int nvqs_launch_pairs(const NvqsK &k, const uint8_t *none, const uint16_t *x, int64_t ldx, int n_pairs, float *y, int64_t ldy,
+                             const PairSel &sel, hipStream_t st) {
+    const size_t ncb = static_cast<size_t>(k.cb_bytes);
+    const dim3 grid(static_cast<unsigned>(ceil_div(k.nrows, 4)), static_cast<unsigned>(n_pairs));
+    if (ncb <= 49152 && ncb % 4 == 0)
+        hipLaunchKernelGGL((nvqs_gemv_kernel<XF16, 1, true>), grid, dim3(256), ncb, st, k, none, x, ldx, n_pairs, y, ldy, sel);
+    else
+        hipLaunchKernelGGL((nvqs_gemv_kernel<XF16, 1, false>), grid, dim3(256), 0, st, k, none, x, ldx, n_pairs, y, ldy, sel);
+    return check_launch("nvqs_gemv_pairs");
 }
 
 }  // namespace mfq
@@ -540,6 +567,29 @@ extern "C" int mfq_hip_nvqs_dequant_rows_f32(const mfq_nvqs_desc *d, const void 
                            ld, static_cast<float *>(nullptr), 0);
     }
     return check_launch("nvqs_dequant_f32");
+}
+
+extern "C" int mfq_hip_nvqs_gemv_pairs(const mfq_nvqs_desc *d, const void *const *expert_weights, const void *weight,
+                                       int out_per_expert, const int32_t *expert_slot, int E, const void *x, int x_dtype,
+                                       int64_t ldx, int routed_input, const int32_t *ids, int T, int R, float *y, int64_t ldy,
+                                       mfq_stream_t stream) {
+    MFQ_REQUIRE(d && (expert_weights || weight) && expert_slot && x && ids && y, MFQ_ERR_INVALID, "nvqs_gemv_pairs: null argument");
+    MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvqs_gemv_pairs: x_dtype=%d", x_dtype);
+    MFQ_REQUIRE(T >= 0 && R >= 1 && E >= 1, MFQ_ERR_INVALID, "nvqs_gemv_pairs: T=%d R=%d E=%d", T, R, E);
+    MFQ_REQUIRE(static_cast<int64_t>(T) * R <= 65535, MFQ_ERR_UNSUPPORTED, "nvqs_gemv_pairs: %lld pairs (at most 65535 per launch)",
+                static_cast<long long>(T) * R);
+    MFQ_REQUIRE(out_per_expert > 0 && (expert_weights ? out_per_expert == d->out : d->out % out_per_expert == 0), MFQ_ERR_INVALID,
+                "nvqs_gemv_pairs: %d rows per expert, the tensor has %d", out_per_expert, d->out);
+    MFQ_REQUIRE(ldx >= d->neuron_len && ldy >= out_per_expert, MFQ_ERR_INVALID, "nvqs_gemv_pairs: ldx/ldy smaller than the tensor");
+    if (T == 0) return MFQ_OK;
+    const PairSel sel{ids, expert_slot, reinterpret_cast<const uint8_t *const *>(expert_weights), E, R, routed_input ? 1 : 0};
+    NvqsK k = to_k(d);
+    k.row0 = 0;
+    k.nrows = out_per_expert;
+    const uint16_t *xp = static_cast<const uint16_t *>(x);
+    const uint8_t *w = static_cast<const uint8_t *>(weight);
+    return x_dtype == MFQ_X_F16 ? nvqs_launch_pairs<1>(k, w, xp, ldx, T * R, y, ldy, sel, as_stream(stream))
+                                : nvqs_launch_pairs<0>(k, w, xp, ldx, T * R, y, ldy, sel, as_stream(stream));
 }
 
 extern "C" int mfq_hip_nvqs_embedding(const mfq_nvqs_desc *d, const void *weight, const int64_t *ids, int n_ids, void *out,

@@ -119,6 +119,48 @@ class ForeignCohort:
             shape = (n, self.linears[0].out, self.linears[0].neuron_len)
         if shape != (n, out_per_expert, neuron_len):
             raise ValueError(f"NINTM pool tensor shape {shape} must be {(n, out_per_expert, neuron_len)}")
+        self._slot = self._wtab = None           # device tables of the one-launch decode form, built on first use
+
+    PAIRS_MAX = 64   # (token, route) pairs up to which a decode step takes one launch per cohort over all its pairs
+
+    def matmul_pairs(self, n_experts: int, x2: torch.Tensor, routed: bool, ids: torch.Tensor, T: int, R: int,
+                     flat: torch.Tensor) -> None:
+        """flat[p] = W[ids[p]] . x2[p or p // R] for the pairs routed to this cohort, in one launch that reads the routing
+        table on the device (mfq_hip_{nvq,nvqs,nepq,nint8z,mx}_gemv_pairs); the rows of other pairs are left alone."""
+        from .runtime import Nint8ZeroWeight
+        from .runtime_vq import NvqsWeight, nepq_hadamard
+        lib, dev = L.lib(), x2.device
+        if self._slot is None:
+            slot = np.full(n_experts, -1, dtype=np.int32)
+            slot[self.expert_ids] = np.arange(len(self.expert_ids), dtype=np.int32)
+            self._slot = torch.from_numpy(slot).to(dev)
+            if self.linears:
+                self._wtab = torch.tensor([q.weight.data.data_ptr() for q in self.linears], dtype=torch.int64, device=dev)
+        common = (_ptr(self._slot), n_experts)
+        if self.nepq is not None and self.nepq.rotation_block:
+            x2 = nepq_hadamard(x2, self.nepq.signs, self.nepq.rotation_block)
+        tail = (_ptr(x2), _x_dtype(x2), x2.stride(0), int(routed), _ptr(ids), T, R, _ptr(flat), flat.stride(0), _stream())
+        if self.mx is not None:
+            w = self.mx
+            L.check(lib.mfq_hip_mx_gemv_pairs(w.kind, _ptr(w.values), _ptr(w.scales), w.rows, w.neuron_len, self.out, *common, *tail))
+        elif self.nepq is not None:
+            w = self.nepq
+            if w.streams:
+                L.check(lib.mfq_hip_nvqs_gemv_pairs(C.byref(w.desc), None, _ptr(w.data), self.out, *common, *tail))
+            else:
+                L.check(lib.mfq_hip_nepq_gemv_pairs(C.byref(w.desc), _ptr(w.data), self.out, *common, *tail))
+        else:
+            w0 = self.linears[0].weight
+            if isinstance(w0, Nint8ZeroWeight):
+                L.check(lib.mfq_hip_nint8z_gemv_pairs(C.byref(w0.desc), _ptr(self._wtab), *common, *tail))
+            elif isinstance(w0, NvqsWeight):
+                L.check(lib.mfq_hip_nvqs_gemv_pairs(C.byref(w0.desc), _ptr(self._wtab), None, self.out, *common, *tail))
+            else:
+                L.check(lib.mfq_hip_nvq_gemv_pairs(C.byref(w0.desc), _ptr(self._wtab), *common, *tail))
+
+    def pairs_capable(self) -> bool:
+        """Whether matmul_pairs takes this cohort: every family has the launch; NEPQ1 experts must be whole row-blocks."""
+        return not (self.nepq is not None and not self.nepq.streams and self.out % 16)
 
     @property
     def payload_bytes(self) -> int:
@@ -219,11 +261,20 @@ class NintMoeWeight:
 
     def _add_foreign(self, x2: torch.Tensor, routed: bool, route: MoeRoutePlan, out: torch.Tensor) -> None:
         """The rows of the pairs routed to experts of other families: per expert, gather its activation rows, multiply
-        on that family's kernels, scatter into `out` [T, R, out_per_expert].  Reads the routing table on the host."""
+        on that family's kernels, scatter into `out` [T, R, out_per_expert]; reads the routing table on the host.  A
+        decode step (up to ForeignCohort.PAIRS_MAX pairs) instead takes one launch per cohort over all pairs, with the
+        routing table read on the device."""
         T, R = route.tokens, route.routes
-        ids = route.ids.reshape(T, R).cpu().numpy()
         flat = out.view(T * R, self.out_per_expert)
-        for c in self.foreign:
+        walk = list(self.foreign)
+        if T * R <= ForeignCohort.PAIRS_MAX:     # a decode step: one launch per cohort, nothing read back
+            for c in [c for c in walk if c.pairs_capable()]:
+                c.matmul_pairs(self.n_experts, x2, routed, route.ids, T, R, flat)
+                walk.remove(c)
+        if not walk:
+            return
+        ids = route.ids.reshape(T, R).cpu().numpy()
+        for c in walk:
             for local, e in enumerate(c.expert_ids):
                 t_idx, r_idx = np.nonzero(ids == e)
                 if t_idx.size == 0:
