@@ -13,15 +13,21 @@
  * row-major [M, ldy].
  *
  * Range of the activations.  The kernels multiply in fp16 (the reference's activation type).  fp16 rows are used as
- * given.  bf16 rows of any finite magnitude are taken by the NINT batch-1 / batch-2 kernels (GEMV, fused GLU, arg-max,
- * MoE decode: every K-slice of a row is scaled by a power of two before the conversion and the sums are scaled back),
- * by the NINT kernel for 3 to 16 rows that keeps the activations in LDS (groups of 32 or 16 weights and K of at most
- * eight steps of 16 groups: every row of the batch has its own scale per K-slice) and by every prefill kernel (whole
- * rows are scaled the same way), so a row of values near 1e-6 or 1e6 keeps the accuracy of a row near 1; within one
- * slice, elements more than about 2^20 below its largest magnitude lose bits.
- * The kernels in between -- the other streaming matrix-core kernels for a few to a few hundred rows, and the NVQ /
- * NEPQ / NINT8-0 batch-1 kernels -- convert bf16 without scaling: there |x| must not exceed 65504 (larger values
- * saturate), and rows whose magnitudes sit below about 1e-3 lose precision to fp16's subnormal range.
+ * given.  bf16 rows of any finite magnitude are taken by
+ *   - the NINT batch-1 / batch-2 kernels (GEMV, fused GLU, arg-max, MoE decode) and the NINT kernel for 3 to 16 rows that
+ *     keeps the activations in LDS (groups of 32 or 16 weights, K of at most eight steps of 16 groups),
+ *   - the NVQ3J kernel for one and two rows with its signed table in LDS, the generic NVQ kernel (which runs behind a MoE
+ *     decode step on an NVQ cohort), the NEPQ1 one-row kernel and the NINT8-0 streaming GEMV,
+ *   - the stream-family (E8, d4_1024, 1-bit, NEPQ0) and MX wave-per-neuron kernels up to 16 rows, which multiply in fp32,
+ *   - every prefill kernel:
+ * every K-slice of a row (the streaming GEMVs; the whole row in the NINT8-0 GEMV and the prefill kernels) is scaled by a
+ * power of two before the conversion and the sums are scaled back, so a row of values near 1e-6 or 1e6 keeps the
+ * accuracy of a row near 1; within one slice, elements more than about 2^20 below its largest magnitude lose bits.
+ * The streaming matrix-core kernels in between (NINT outside the LDS-resident shapes, NVQ on tables too large for the
+ * one-row kernel, NVQ / NEPQ / NINT8-0 from two or three rows to a few hundred) convert bf16 without scaling: there |x|
+ * must not exceed 65504 (larger values saturate), and rows whose magnitudes sit below about 1e-3 lose precision to
+ * fp16's subnormal range.  A per-slice scale costs those kernels a second pass over their activation fragments, which
+ * already are most of their traffic.
  */
 #ifndef MFQ_HIP_H
 #define MFQ_HIP_H

@@ -507,3 +507,30 @@ def test_mixed_family_decode_step_reads_the_routing_table_on_the_device():
         ref = O.moe_grouped_matmul(d2, x_d.float().cpu().numpy(), idn)
         got = y2.cpu().numpy()
         assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL * max(1.0, float(np.sqrt(np.mean(ref * ref))))
+
+
+@pytest.mark.parametrize("scale", [1e-6, 3e6])
+def test_decode_pairs_take_bf16_rows_of_any_magnitude(scale):
+    """The one-row kernels behind a decode step on cohorts of other families (NVQ, NEPQ1 and NINT8-0 rescale every bf16
+    row by a power of two before the fp16 conversion; the stream families and MX multiply in fp32): rows 1e-6 and 3e6
+    times an ordinary row come out with the relative accuracy of an ordinary one."""
+    from tyloquant_amd.runtime_moe import NintMoeWeight, build_moe_route_plan
+    rng = np.random.default_rng(79)
+    out, K, E, R, T = 32, 192, 6, 2, 3
+    def pool(ids, dtype, t):
+        return O.MoePool(np.asarray(ids, dtype=np.int32), dtype, t)
+    t = O.NintMoeTensor((E, out, K), [
+        pool([0], "NINT8-0", O.quantize_nint8_zero((rng.standard_normal((out, K)) * 0.02).astype(np.float32))),
+        pool([1, 2], "NVQ3J-512", synth.nvq_jsc_random(rng, 2 * out, K, "d4_512", 2)),
+        pool([3], "NEPQ1-S", synth.nepq_random(rng, "NEPQ1-S", 1, out, K, 3)),
+        pool([4], "NVQ1-S", synth.nvq1_random(rng, "NVQ1-S", out, K)),
+        pool([5], "MXFP4", synth.mx_random(rng, "MXFP4", out, K, 120, 124))])
+    w = NintMoeWeight.from_blob(O.pack_nint_moe(t))
+    dense = O.dequantize_expertwise(t)
+    ids = np.array([[0, 1], [2, 3], [4, 5]], dtype=np.int32)
+    x = torch.from_numpy((rng.standard_normal((T, K)) * scale).astype(np.float32)).to(torch.bfloat16)
+    got = w(x.cuda(), build_moe_route_plan(torch.from_numpy(ids).cuda(), E)).cpu().numpy()
+    ref = O.moe_grouped_matmul(dense, x.float().numpy(), ids)
+    for t_ in range(T):
+        for r in range(R):
+            assert rel_l2(got[t_, r], ref[t_, r]) < REL_TOL, (t_, r, rel_l2(got[t_, r], ref[t_, r]))

@@ -188,7 +188,8 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
     float *red = reinterpret_cast<float *>(xbase + nwaves * (MB * (npairs + 2 * ngl)));
     XRegs<MB> xg;
     stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * 24, npairs, lane, xg);
-    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane, xg);
+    float xinv[MB];  // bf16 rows are staged times a per-wave power of two; the sums are scaled back below
+    stage_x<XF16, MB, PlainBias, true>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane, xg, xinv);
     if constexpr (TAB_LDS) __syncthreads();  // the LDS table copy was made by the whole block
 
     const int r = lane & 15, kb = lane >> 4;
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(1024) void nepq_gemv_kernel(NepqK k, const uint8_t 
     for (int i = 0; i < RPB; ++i) {
         float v[MB];
 #pragma unroll
-        for (int m = 0; m < MB; ++m) v[m] = anchor[i] * acc[i][m];
+        for (int m = 0; m < MB; ++m) v[m] = anchor[i] * acc[i][m] * xinv[m];
         park_rows<MB>(v, red, i * nwaves + wave, lane);
     }
     // a row-block past the tensor's last has rows beyond nrows: flush_rows drops them

@@ -122,18 +122,49 @@ __global__ __launch_bounds__(256) void nint8z_gemv_kernel(N8zK k, const uint8_t 
     const int K = k.neuron_len;
     uint16_t *xh = reinterpret_cast<uint16_t *>(lds);
     float *xsum = reinterpret_cast<float *>(lds + MB * K / 2);
-    if (ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {  // 16-byte chunks (K is a multiple of 32)
-        const int cpr = K / 8;
+    const bool vec = ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;  // 16-byte chunks (K is a multiple of 32)
+    const int cpr = K / 8;
+    // bf16 rows: each row times the power of two that brings its largest magnitude near 2^12 (rows of any magnitude stay
+    // inside fp16's range); the sums are scaled back when they are stored
+    __shared__ uint32_t rowmax[MB];
+    float rs[MB], rinv[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) rs[m] = rinv[m] = 1.f;
+    if constexpr (!XF16) {
+        if (tid < MB) rowmax[tid] = 0u;
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            const uint16_t *xrow = x + static_cast<int64_t>(min(m0 + m, M - 1)) * ldx;
+            uint32_t mx = 0;
+            if (vec) {
+                for (int c = tid; c < cpr; c += 256) {
+                    const u32x4_t v = *reinterpret_cast<const u32x4_t *>(xrow + 8 * c);
+                    mx = absmax_bf16(absmax_bf16(absmax_bf16(absmax_bf16(mx, v.x), v.y), v.z), v.w);
+                }
+            } else {
+                for (int c = tid; c < K; c += 256) mx = absmax_bf16(mx, xrow[c]);
+            }
+            const uint32_t wm = wave_max_u32(mx);
+            if (lane == 0) atomicMax(&rowmax[m], wm);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < MB; ++m) rs[m] = slice_scale(rowmax[m], rinv[m]);
+    }
+    if (vec) {
         for (int i = tid; i < MB * cpr; i += 256) {
             const int m = i / cpr, c = i - m * cpr;
             const int row = min(m0 + m, M - 1);
-            const u32x4_t v = *reinterpret_cast<const u32x4_t *>(x + row * ldx + 8 * c);
+            const u32x4_t v = *reinterpret_cast<const u32x4_t *>(x + static_cast<int64_t>(row) * ldx + 8 * c);
             uint32_t h[4] = {v.x, v.y, v.z, v.w};
             if constexpr (!XF16) {
+                float sc = rs[0];
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    h[t] = f32_to_f16_rne(__uint_as_float(h[t] << 16)) |
-                           (static_cast<uint32_t>(f32_to_f16_rne(__uint_as_float(h[t] & 0xffff0000u))) << 16);
+                for (int mm = 1; mm < MB; ++mm)
+                    if (m == mm) sc = rs[mm];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) h[t] = to_h2_scaled(h[t], sc);
             }
             *reinterpret_cast<u32x4_t *>(xh + m * K + 8 * c) = u32x4_t{h[0], h[1], h[2], h[3]};
         }
@@ -141,8 +172,12 @@ __global__ __launch_bounds__(256) void nint8z_gemv_kernel(N8zK k, const uint8_t 
         for (int i = tid; i < MB * K; i += 256) {
             const int m = i / K, c = i - m * K;
             const int row = min(m0 + m, M - 1);
-            const uint16_t v = x[row * ldx + c];
-            xh[i] = XF16 ? v : f32_to_f16_rne(bf16_to_f32(v));
+            const uint16_t v = x[static_cast<int64_t>(row) * ldx + c];
+            float sc = rs[0];
+#pragma unroll
+            for (int mm = 1; mm < MB; ++mm)
+                if (m == mm) sc = rs[mm];
+            xh[i] = XF16 ? v : f32_to_f16_rne(bf16_to_f32(v) * sc);
         }
     }
     __syncthreads();
@@ -194,7 +229,7 @@ __global__ __launch_bounds__(256) void nint8z_gemv_kernel(N8zK k, const uint8_t 
             float v = acc[m];
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-            if (lane == 0 && m0 + m < M) y[static_cast<int64_t>(m0 + m) * ldy + row] = v;
+            if (lane == 0 && m0 + m < M) y[static_cast<int64_t>(m0 + m) * ldy + row] = v * rinv[m];
         }
     }
 }

@@ -268,7 +268,8 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
     XRegs<MB> xg;
     stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * 24, npairs, lane, xg);
     if (s0 < s1) load_step(s0, cur);
-    stage_x<XF16, MB, PlainBias>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane, xg);
+    float xinv[MB];  // bf16 rows are staged times a per-wave power of two; the sums are scaled back below
+    stage_x<XF16, MB, PlainBias, true>(xr, k.neuron_len, s0 * 16 * 24, npairs, 24, ngl, xs, xsum, lane, xg, xinv);
     __syncthreads();  // the LDS tables were filled by the whole block
 
     const int r = lane & 15, kb = lane >> 4;
@@ -314,7 +315,7 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
     const float anchor = reinterpret_cast<const float *>(w + k.anchors_off)[rb * 16 + r];
     float v[MB];
 #pragma unroll
-    for (int m = 0; m < MB; ++m) v[m] = anchor * acc[m];
+    for (int m = 0; m < MB; ++m) v[m] = anchor * acc[m] * xinv[m];
     finish_rows<MB>(v, red, wave, nwaves, lane, rb, 0, k.out, yr);
 }
 
