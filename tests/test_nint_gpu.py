@@ -355,16 +355,18 @@ def test_nint8_zero_dequant_bit_exact_and_matmul(out, K):
     x, xf = _x(rng, 40, K)                            # the streaming kernel beyond its default range
     y = R.nint8_zero_matmul(lin.weight, x, force="gemv").cpu().numpy()
     assert rel_l2(y, O.linear_forward_f64(deq, xf)) < REL_TOL
-    # bf16 rows far outside fp16's range on the streaming kernel (every row scaled by its own power of two), each row with
-    # its own magnitude, aligned and misaligned
+    # bf16 rows far outside fp16's range on the streaming kernel (every row scaled by its own power of two): one row at a
+    # time, and three rows of different magnitudes in one misaligned batch (aligned batches run on the matrix cores)
     x, xf = _x(rng, 3, K)
     sc = torch.tensor([[1e-6], [1.0], [3e6]])
     xs = (x.float().cpu() * sc).to(torch.bfloat16)
-    for xin in (xs.cuda(), torch.zeros((3, K + 3), dtype=torch.bfloat16, device="cuda")[:, 1:K + 1].copy_(xs)):
-        y = R.nint8_zero_matmul(lin.weight, xin, force="gemv").cpu().numpy()
-        ref = O.linear_forward_f64(deq, xs.float().numpy())
-        for m in range(3):
-            assert rel_l2(y[m], ref[m]) < REL_TOL, (m, rel_l2(y[m], ref[m]))
+    ref = O.linear_forward_f64(deq, xs.float().numpy())
+    ys = [R.nint8_zero_matmul(lin.weight, xs[m:m + 1].cuda(), force="gemv").cpu().numpy()[0] for m in range(3)]
+    ys3 = R.nint8_zero_matmul(lin.weight, torch.zeros((3, K + 3), dtype=torch.bfloat16, device="cuda")[:, 1:K + 1].copy_(xs),
+                              force="gemv").cpu().numpy()
+    for m in range(3):
+        assert rel_l2(ys[m], ref[m]) < REL_TOL, (m, rel_l2(ys[m], ref[m]))
+        assert rel_l2(ys3[m], ref[m]) < REL_TOL, (m, rel_l2(ys3[m], ref[m]))
 
 
 @pytest.mark.parametrize("cus,out,K", [(4, 200, 1056), (3, 96, 4096), (2, 40, 96), (64, 33, 2048)])
