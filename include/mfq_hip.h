@@ -16,8 +16,8 @@
  * given.  bf16 rows of any finite magnitude are taken by
  *   - the NINT batch-1 / batch-2 kernels (GEMV, fused GLU, arg-max, MoE decode) and the NINT kernel for 3 to 16 rows that
  *     keeps the activations in LDS (groups of 32 or 16 weights, K of at most eight steps of 16 groups),
- *   - the NVQ3J kernel for one and two rows with its signed table in LDS, the generic NVQ kernel (which runs behind a MoE
- *     decode step on an NVQ cohort), the NEPQ1 one-row kernel and the NINT8-0 streaming GEMV (one row; more rows when
+ *   - the NVQ3J kernel for one and two rows with its signed table in LDS, the NVQ kernels behind a MoE decode step on an
+ *     NVQ cohort (mfq_hip_nvq_gemv_pairs), the NEPQ1 one-row kernel and the NINT8-0 streaming GEMV (one row; more rows when
  *     the activation rows are not 16-byte aligned),
  *   - the stream-family (E8, d4_1024, 1-bit, NEPQ0) and MX wave-per-neuron kernels up to 16 rows, which multiply in fp32,
  *   - every prefill kernel:

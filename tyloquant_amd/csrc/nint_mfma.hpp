@@ -68,6 +68,18 @@ __device__ __forceinline__ u32x4_t xfrag_finish(u32x4_t v, int kpos, int K) {
     return v;
 }
 
+// xfrag_finish for a bf16 row that is multiplied by a power of two on the way to fp16 (see slice_scale)
+template <int XF16, bool ALIGN8>
+__device__ __forceinline__ u32x4_t xfrag_finish_scaled(u32x4_t v, int kpos, int K, float scale) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) v[t] = XF16 ? v[t] : to_h2_scaled(v[t], scale);
+    if constexpr (!ALIGN8) {
+        if (kpos + 4 == K) v = u32x4_t{v.z, v.w, 0u, 0u};
+    }
+    if (kpos >= K) v = u32x4_t{0u, 0u, 0u, 0u};
+    return v;
+}
+
 __device__ __forceinline__ half2_t pk_h2(float lo, float hi) {
     return __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
 }

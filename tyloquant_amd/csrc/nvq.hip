@@ -327,13 +327,29 @@ __global__ __launch_bounds__(1024) void nvq_gemv_kernel(NvqK k, const uint8_t *_
 // the fp32 accumulator.  Codes of padding groups are zero (not zero weights), so the activation fragments
 // read as zero at and beyond K.
 // LDS map (dwords): [codebook pairs: banks*entries*2][sign xor table: 512][lut pairs: 16][bank offset: 16][red]
-template <int XF16, int NB>
-__global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__restrict__ w,
-                                                       const uint16_t *__restrict__ x, int64_t ldx, int M,
-                                                       float *__restrict__ y, int64_t ldy, int spw) {
+// PAIRS: the launch runs over the pairs of a MoE decode step (see PairSel); the tile's one bf16 row is scaled per wave
+// by the power of two that brings its K-slice near 2^12 (rows of any magnitude), as in the one-row kernels.
+template <int XF16, int NB, bool PAIRS = false>
+__global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__restrict__ w_in,
+                                                       const uint16_t *__restrict__ x_in, int64_t ldx, int M_in,
+                                                       float *__restrict__ y_in, int64_t ldy, int spw, PairSel sel) {
     extern __shared__ uint32_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint8_t *w = w_in;
+    const uint16_t *x = x_in;
+    float *y = y_in;
+    int M = M_in, m0 = blockIdx.y * 16;
+    if constexpr (PAIRS) {  // a tile of one row, the expert's own tensor
+        const uint16_t *xr[1];
+        float *yr[1];
+        int local;
+        if (!select_rows<1>(sel, w, local, x_in, ldx, y_in, ldy, M_in, xr, yr)) return;
+        x = xr[0];
+        y = yr[0];
+        M = 1;
+        m0 = 0;
+    }
     const int ncb = k.banks * k.entries;
     uint32_t *cbp = lds;
     uint32_t *sgx = cbp + 2 * ncb;
@@ -364,7 +380,7 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
             bankoff[tid] = bfs[tid] * k.entries * 2;
         }
     }
-    const int rb0 = blockIdx.x * NB, m0 = blockIdx.y * 16;
+    const int rb0 = blockIdx.x * NB;
     const int tok = min(m0 + (lane & 15), M - 1);
     const uint16_t *xrow = x + static_cast<int64_t>(tok) * ldx;
     const int r = lane & 15, kb = lane >> 4;
@@ -382,6 +398,16 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
     float4_t acc[NB];
 #pragma unroll
     for (int i = 0; i < NB; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float xscale = 1.f, xinv = 1.f;
+    if constexpr (PAIRS && !XF16) {  // largest magnitude of the wave's K-slice of the row (K is a multiple of 8)
+        uint32_t mx = 0;
+        const int k0 = s0 * 16 * 24, k1 = min(k.neuron_len, (s0 + max(n, 0)) * 16 * 24);
+        for (int c = k0 + 8 * lane; c < k1; c += 512) {
+            const u32x4_t v = *reinterpret_cast<const u32x4_t *>(x + c);
+            mx = absmax_bf16(absmax_bf16(absmax_bf16(absmax_bf16(mx, v.x), v.y), v.z), v.w);
+        }
+        xscale = slice_scale(wave_max_u32(mx), xinv);
+    }
     __syncthreads();  // tables
 
     if constexpr (NB <= 2) {
@@ -417,7 +443,10 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
                 u32x4_t a[3];
 #pragma unroll
                 for (int m = 0; m < 3; ++m) {
-                    a[m] = xfrag_finish<XF16, true>(a1[m], (s0 + s) * 16 * 24 + kb * 24 + 4 * j * 24 + 8 * m, k.neuron_len);
+                    if constexpr (PAIRS)
+                        a[m] = xfrag_finish_scaled<XF16, true>(a1[m], (s0 + s) * 16 * 24 + kb * 24 + 4 * j * 24 + 8 * m, k.neuron_len, xscale);
+                    else
+                        a[m] = xfrag_finish<XF16, true>(a1[m], (s0 + s) * 16 * 24 + kb * 24 + 4 * j * 24 + 8 * m, k.neuron_len);
                     a1[m] = a2[m];
                 }
                 xfrags(4 * s + j + 2, a2);
@@ -489,7 +518,7 @@ __global__ __launch_bounds__(512) void nvq_mfma_kernel(NvqK k, const uint8_t *__
 #pragma unroll
     for (int i = 0; i < NB; ++i)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) red[((wave * NB + i) * 4 + v) * 64 + lane] = anchor[i] * acc[i][v];
+        for (int v = 0; v < 4; ++v) red[((wave * NB + i) * 4 + v) * 64 + lane] = anchor[i] * acc[i][v] * xinv;
     mfma_store_dense<NB>(red, rb0, m0, M, k.out, y, ldy);
 }
 
@@ -1212,8 +1241,24 @@ static int nvq_launch_mfma(const NvqK &k, const uint8_t *w, const uint16_t *x, i
     const size_t lds = (static_cast<size_t>(k.banks) * k.entries * 2 + 512 + 32) * 4 + static_cast<size_t>(nwaves) * NB * 1024;
     MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nvq_mfma: %zu bytes of LDS", lds);
     hipLaunchKernelGGL((nvq_mfma_kernel<XF16, NB>), dim3(static_cast<unsigned>(groups), static_cast<unsigned>(ceil_div(M, 16))),
-                       dim3(64 * nwaves), lds, st, k, w, x, ldx, M, y, ldy, spw);
+                       dim3(64 * nwaves), lds, st, k, w, x, ldx, M, y, ldy, spw, PairSel{});
     return check_launch("nvq_mfma");
+}
+
+// the same kernel, a tile of one row per block row, over the pairs of a MoE decode step (see PairSel): eight times the
+// generic kernel's rate on an expert of 2048 x 4096
+template <int XF16, int NB>
+static int nvq_launch_mfma_pairs(const NvqK &k, const uint16_t *x, int64_t ldx, int n_pairs, float *y, int64_t ldy, const PairSel &sel,
+                                 hipStream_t st) {
+    const int64_t groups = ceil_div(k.n_rowblocks, NB);
+    int spw = static_cast<int>(ceil_div(k.nsteps, 8));
+    while (spw < k.nsteps && groups * ceil_div(k.nsteps, spw) > 8192) ++spw;
+    const int nwaves = static_cast<int>(ceil_div(k.nsteps, spw));
+    const size_t lds = (static_cast<size_t>(k.banks) * k.entries * 2 + 512 + 32) * 4 + static_cast<size_t>(nwaves) * NB * 1024;
+    MFQ_REQUIRE(lds <= 65536, MFQ_ERR_UNSUPPORTED, "nvq_mfma_pairs: %zu bytes of LDS", lds);
+    hipLaunchKernelGGL((nvq_mfma_kernel<XF16, NB, true>), dim3(static_cast<unsigned>(groups), static_cast<unsigned>(n_pairs)),
+                       dim3(64 * nwaves), lds, st, k, static_cast<const uint8_t *>(nullptr), x, ldx, n_pairs, y, ldy, spw, sel);
+    return check_launch("nvq_mfma_pairs");
 }
 
 // 16-row tiles through nvq_signed_kernel: at most one block per CU and tile, each with up to six row-blocks
@@ -1507,6 +1552,16 @@ extern "C" int mfq_hip_nvq_gemv_pairs(const mfq_nvq_desc *d, const void *const *
     const PairSel sel{ids, expert_slot, reinterpret_cast<const uint8_t *const *>(expert_weights), E, R, routed_input ? 1 : 0};
     const NvqK k = to_k(d);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
+    // the matrix-core kernel where the activation rows allow 16-byte reads; else the generic kernel
+    static const int pairs_mfma = tune_env("MFQ_NVQ_PAIRS_MFMA", 1);
+    if (pairs_mfma && nvq_stream_capable(k) && ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+        const bool two = ceil_div(k.n_rowblocks, 2) * (k.nsteps < 8 ? k.nsteps : 8) * T * R >= 1024;
+        if (x_dtype == MFQ_X_F16)
+            return two ? nvq_launch_mfma_pairs<1, 2>(k, xp, ldx, T * R, y, ldy, sel, as_stream(stream))
+                       : nvq_launch_mfma_pairs<1, 1>(k, xp, ldx, T * R, y, ldy, sel, as_stream(stream));
+        return two ? nvq_launch_mfma_pairs<0, 2>(k, xp, ldx, T * R, y, ldy, sel, as_stream(stream))
+                   : nvq_launch_mfma_pairs<0, 1>(k, xp, ldx, T * R, y, ldy, sel, as_stream(stream));
+    }
     return x_dtype == MFQ_X_F16 ? nvq_launch_pairs<1>(k, xp, ldx, T * R, y, ldy, sel, as_stream(stream))
                                 : nvq_launch_pairs<0>(k, xp, ldx, T * R, y, ldy, sel, as_stream(stream));
 }

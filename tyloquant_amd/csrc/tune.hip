@@ -48,6 +48,7 @@ Knob g_knobs[] = {
     {"MFQ_MOE_PREFILL_PAIRS", "pairs per expert from which mapped MoE calls take the prefill kernel (0 = default)", 0, false},
     {"MFQ_FFN_SPIN_LIMIT", "polls after which the one-launch FFN's grid barrier gives up", 0, false},
     {"MFQ_FFN_TRACE", "1 = the one-launch FFN records per-block clocks behind its workspace", 0, false},
+    {"MFQ_NVQ_PAIRS_MFMA", "0 = a MoE decode step on an NVQ cohort always takes the generic one-row kernel", 0, false},
     {"MFQ_MOE_NB", "row-blocks per wave of the MoE streaming kernel (0 = by shape)", 0, false},
     {"MFQ_MOE_GROUPS", "bit mask of the register groups the mapped MoE prefill path launches (7 = all)", 0, false},
     {"MFQ_GLU_PREFILL_MIN_M", "rows from which the dense gate/up prefill fuses the GLU into its epilogue", 0, false},
