@@ -130,7 +130,33 @@ __global__ __launch_bounds__(256) void nint8z_gemv_kernel(N8zK k, const uint8_t 
     float rs[MB], rinv[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) rs[m] = rinv[m] = 1.f;
-    if constexpr (!XF16) {
+    // one row of up to 8192 values in 16-byte chunks: the chunks stay in registers between the maximum and the conversion
+    constexpr int HELD = 4;
+    const bool held = MB == 1 && !XF16 && vec && cpr <= HELD * 256;
+    u32x4_t keep[HELD];
+    if (held) {
+        if (tid == 0) rowmax[0] = 0u;
+        __syncthreads();
+        const uint16_t *xrow = x + static_cast<int64_t>(min(m0, M - 1)) * ldx;
+        uint32_t mx = 0;
+#pragma unroll
+        for (int j = 0; j < HELD; ++j) {
+            const int c = tid + 256 * j;
+            keep[j] = c < cpr ? *reinterpret_cast<const u32x4_t *>(xrow + 8 * c) : u32x4_t{0u, 0u, 0u, 0u};
+            mx = absmax_bf16(absmax_bf16(absmax_bf16(absmax_bf16(mx, keep[j].x), keep[j].y), keep[j].z), keep[j].w);
+        }
+        const uint32_t wm = wave_max_u32(mx);
+        if (lane == 0) atomicMax(&rowmax[0], wm);
+        __syncthreads();
+        rs[0] = slice_scale(rowmax[0], rinv[0]);
+#pragma unroll
+        for (int j = 0; j < HELD; ++j) {
+            const int c = tid + 256 * j;
+            if (c < cpr)
+                *reinterpret_cast<u32x4_t *>(xh + 8 * c) = u32x4_t{to_h2_scaled(keep[j].x, rs[0]), to_h2_scaled(keep[j].y, rs[0]),
+                                                                   to_h2_scaled(keep[j].z, rs[0]), to_h2_scaled(keep[j].w, rs[0])};
+        }
+    } else if constexpr (!XF16) {
         if (tid < MB) rowmax[tid] = 0u;
         __syncthreads();
 #pragma unroll
@@ -152,7 +178,9 @@ __global__ __launch_bounds__(256) void nint8z_gemv_kernel(N8zK k, const uint8_t 
 #pragma unroll
         for (int m = 0; m < MB; ++m) rs[m] = slice_scale(rowmax[m], rinv[m]);
     }
-    if (vec) {
+    if (held) {
+        // staged above
+    } else if (vec) {
         for (int i = tid; i < MB * cpr; i += 256) {
             const int m = i / cpr, c = i - m * cpr;
             const int row = min(m0 + m, M - 1);
