@@ -31,9 +31,10 @@ int mfq_rt_linear_dequantize(void *handle, float *out, void *stream);
  * (fp32 [M, 2 W], may be null when the fused forms apply). */
 int mfq_rt_linear_forward_glu(void *handle, const void *x, int x_dtype, int64_t ldx, int M, int gelu, void *hidden,
                               float *scratch, void *stream);
-/* embed_forward (cpp_runtime/mfq_decode.cpp:13929-13957) on a NINT table: out [n_ids, K] of out_dtype (MFQ_X_*),
- * ids device int64; and next_token_from_hidden (:14107-14130): token[m] device int64, logits fp32 [M, out] or null.
- * Both fail on a handle that does not hold a NINT tensor. */
+/* embed_forward (cpp_runtime/mfq_decode.cpp:13929-13957) on a NINT, NINT8-0 or NVQ table: out [n_ids, K] of out_dtype
+ * (MFQ_X_*), ids device int64, rows of ids outside the table are zero; NEPQ and MX tables are refused, as there.  And
+ * next_token_from_hidden (:14107-14130): token[m] device int64, logits fp32 [M, out] or null; fails on a handle that does
+ * not hold a NINT tensor. */
 int mfq_rt_linear_embedding(void *handle, const int64_t *ids, int n_ids, void *out, int out_dtype, void *stream);
 int mfq_rt_linear_argmax(void *handle, const void *x, int x_dtype, int64_t ldx, int M, int64_t *token, float *logits,
                          void *stream);
@@ -67,6 +68,9 @@ int mfq_rt_file_load_quant_linear(void *handle, const char *name, void **linear)
 
 /* NINTM expert-wise tensors and nint_moe_ffn_forward (cpp_runtime/mfq_decode.cpp:3394-3416). */
 int mfq_rt_load_nint_moe(const void *blob, size_t n, void **handle);
+/* The same with the tensor's NINTMD record from an expert overlay file (MFQ_EXPERT_OVERLAY, mfq_rt_file_open): the
+ * overlay's cohorts are appended and own the experts they list (load_nint_moe_cpu, cpp_runtime/mfq_decode.cpp:5752-5774). */
+int mfq_rt_load_nint_moe_overlay(const void *blob, size_t n, const void *overlay, size_t overlay_n, void **handle);
 void mfq_rt_free_nint_moe(void *handle);
 int mfq_rt_moe_ffn_forward(void *gate_up, void *down, const void *x, int x_dtype, int64_t ldx, int T,
                            const float *router_logits, int top_k, int topk_mode, int normalize,

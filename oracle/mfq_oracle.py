@@ -1197,10 +1197,11 @@ _NIM_HDR = struct.Struct("<4sIIII")
 _NIM_POOL = struct.Struct("<IIQQ")
 
 
-def pack_nint_moe(t: NintMoeTensor) -> bytes:
-    """mfq/formats/io.py:304-336 (NIM2)."""
+def pack_nint_moe(t: NintMoeTensor, delta: bool = False) -> bytes:
+    """mfq/formats/io.py:304-336 (NIM2).  delta: the NID2 form of an expert overlay record (dtype NINTMD): the same
+    layout, pools for some experts only (unpack_nint_moe_impl, cpp_runtime/mfq_decode.cpp:2367-2477)."""
     E, out, K = t.shape
-    parts = [_NIM_HDR.pack(b"NIM2", E, out, K, len(t.pools))]
+    parts = [_NIM_HDR.pack(b"NID2" if delta else b"NIM2", E, out, K, len(t.pools))]
     for p in t.pools:
         ids = np.ascontiguousarray(p.expert_ids, dtype=np.int32).reshape(-1)
         dtype, payload = pack_tensor(p.tensor)
@@ -1209,13 +1210,16 @@ def pack_nint_moe(t: NintMoeTensor) -> bytes:
     return b"".join(parts)
 
 
-def unpack_nint_moe(blob) -> NintMoeTensor:
-    """mfq/formats/io.py:382-446 + invariants of mfq/formats/moe.py:98-134."""
+def unpack_nint_moe(blob, allow_partial: bool = False) -> NintMoeTensor:
+    """mfq/formats/io.py:382-446 + invariants of mfq/formats/moe.py:98-134.  allow_partial: also take an expert delta
+    (magic NID2, pools for some experts only), as unpack_nint_moe_delta does (cpp_runtime/mfq_decode.cpp:2484-2487)."""
     blob = bytes(blob)
     if len(blob) < _NIM_HDR.size:
         raise ValueError("truncated NINTM header")
     magic, E, out, K, npools = _NIM_HDR.unpack_from(blob, 0)
-    if magic != b"NIM2":
+    if magic == b"NID2" and not allow_partial:
+        raise ValueError("NINTM delta cannot be loaded as a full tensor")
+    if magic not in (b"NIM2", b"NID2"):
         raise ValueError(f"invalid NINTM magic: {magic!r}")
     if npools == 0 or npools > E:
         raise ValueError("invalid NINTM pool count")
@@ -1246,9 +1250,18 @@ def unpack_nint_moe(blob) -> NintMoeTensor:
         pools.append(MoePool(ids, dtype, tensor))
     if off != len(blob):
         raise ValueError(f"invalid NINTM tail: {len(blob) - off} extra bytes")
-    if np.any(owners < 0):
+    if np.any(owners < 0) and not allow_partial:
         raise ValueError("NINTM pools do not cover all experts")
     return NintMoeTensor((E, out, K), pools)
+
+
+def apply_expert_overlay(base: NintMoeTensor, delta: NintMoeTensor) -> NintMoeTensor:
+    """load_nint_moe_cpu with an expert overlay (cpp_runtime/mfq_decode.cpp:5752-5774): the delta's pools are appended to
+    the base tensor's; an expert then belongs to the last pool that lists it (the dispatch tables are filled pool by
+    pool, :3355-3372), which dequantize_expertwise reproduces by assigning in pool order."""
+    if tuple(delta.shape) != tuple(base.shape):
+        raise ValueError("expert overlay shape mismatch")
+    return NintMoeTensor(tuple(base.shape), list(base.pools) + list(delta.pools))
 
 
 def dequantize_tensor(t) -> np.ndarray:

@@ -384,6 +384,42 @@ def test_cpp_moe_ffn_with_cohorts_of_other_families(rt, T):
     rt.mfq_rt_free_nint_moe(hd)
 
 
+def test_cpp_moe_ffn_with_an_expert_overlay(rt):
+    """An NINTMD expert overlay on the gate/up tensor (a NINT3 cohort for an expert of the NINT4 cohort and for the NVQ
+    expert, an NEPQ1-S cohort for the 1-bit expert): the layer against the oracle on the overlaid tensor, at a decode
+    step and on a mapped batch; the delta alone does not load."""
+    rng = np.random.default_rng(150)
+    E, H, W, k = 8, 192, 96, 3
+    tg, td = _mixed_moe(rng, 2 * W, H), _mixed_moe(rng, H, W)
+    delta = O.NintMoeTensor((E, 2 * W, H), [
+        O.MoePool(np.array([7, 1], dtype=np.int32), "NINT3", synth.nint_random(rng, 2 * 2 * W, H, 3, 24, 5)),
+        O.MoePool(np.array([2], dtype=np.int32), "NEPQ1-S", synth.nepq_random(rng, "NEPQ1-S", 1, 2 * W, H, 3))])
+    bg, bd, bo = O.pack_nint_moe(tg), O.pack_nint_moe(td), O.pack_nint_moe(delta, delta=True)
+    rt.mfq_rt_load_nint_moe_overlay.argtypes = [C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t, C.POINTER(C.c_void_p)]
+    hg, hd, hbad = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert rt.mfq_rt_load_nint_moe(bo, len(bo), C.byref(hbad)) != 0 and b"delta cannot be loaded" in rt.mfq_rt_last_error()
+    assert rt.mfq_rt_load_nint_moe_overlay(bg, len(bg), bo, len(bo), C.byref(hg)) == 0, rt.mfq_rt_last_error()
+    assert rt.mfq_rt_load_nint_moe(bd, len(bd), C.byref(hd)) == 0, rt.mfq_rt_last_error()
+    dg, dd = O.dequantize_expertwise(O.apply_expert_overlay(tg, delta)), O.dequantize_expertwise(td)
+    for T in (3, 40):
+        x = torch.from_numpy((rng.standard_normal((T, H)) * 3).astype(np.float32)).to(torch.bfloat16).cuda()
+        logits = rng.standard_normal((T, E)).astype(np.float32)
+        logits[0, [7, 1, 2]] += 8.0                      # the first token routes to the experts that changed hands
+        lg = torch.from_numpy(logits).cuda()
+        out = torch.empty((T, H), dtype=torch.float32, device="cuda")
+        ids = torch.empty((T, k), dtype=torch.int32, device="cuda")
+        wts = torch.empty((T, k), dtype=torch.float32, device="cuda")
+        rc = rt.mfq_rt_moe_ffn_forward(hg, hd, x.data_ptr(), 0, H, T, lg.data_ptr(), k, 3, 0, None, None, out.data_ptr(),
+                                       ids.data_ptr(), wts.data_ptr(), None)
+        assert rc == 0, rt.mfq_rt_last_error()
+        torch.cuda.synchronize()
+        ref, rids, rw = O.moe_ffn(dg, dd, x.float().cpu().numpy(), logits, k, delayed_softmax=True)
+        assert np.array_equal(ids.cpu().numpy(), rids) and set(rids[0].tolist()) == {7, 1, 2}
+        check_close(out.cpu().numpy(), ref)
+    rt.mfq_rt_free_nint_moe(hg)
+    rt.mfq_rt_free_nint_moe(hd)
+
+
 def test_cpp_nvq_ffn_swiglu_down(rt):
     """nvq_ffn_swiglu_down of the C++ runtime (joint gate/up launch, SwiGLU kernel, down projection) against the
     oracle's float64 evaluation of the dequantized weights; the hidden rows pass through fp16."""

@@ -208,6 +208,25 @@ def test_cpp_parsers_reject_malformed_headers_without_touching_the_gpu():
     struct.pack_into("<QQ", nim, 20 + 8, 2 ** 64 - 64, 128)
     msg = _rt_load_error(lib, lib.mfq_rt_load_nint_moe, bytes(nim), ctypes.c_size_t(len(nim)))
     assert "truncated NINTM v2 pool payload" in msg
+    # an expert delta (NID2) is not a tensor; as an overlay its shape must match the tensor's
+    nid = O.pack_nint_moe(O.NintMoeTensor((4, 16, 48), [O.MoePool(np.array([2], dtype=np.int32), "NINT3",
+                                                                  synth.nint_random(rng, 16, 48, 3, 24, 5))]), delta=True)
+    assert "delta cannot be loaded as a full tensor" in _rt_load_error(lib, lib.mfq_rt_load_nint_moe, nid, ctypes.c_size_t(len(nid)))
+    with pytest.raises(ValueError, match="delta cannot be loaded as a full tensor"):
+        F.parse_nintm(nid)
+    d = F.parse_nintm(nid, allow_partial=True)
+    assert [p.dtype for p in d.pools] == ["NINT3"] and d.pools[0].expert_ids.tolist() == [2]
+    back = O.unpack_nint_moe(nid, allow_partial=True)
+    over = O.apply_expert_overlay(t, back)
+    dense, base = O.dequantize_expertwise(over), O.dequantize_expertwise(t)
+    assert np.array_equal(dense[[0, 1, 3]], base[[0, 1, 3]]) and not np.array_equal(dense[2], base[2])
+    wrong = O.pack_nint_moe(O.NintMoeTensor((4, 16, 96), [O.MoePool(np.array([2], dtype=np.int32), "NINT3",
+                                                                    synth.nint_random(rng, 16, 96, 3, 24, 5))]), delta=True)
+    good = O.pack_nint_moe(t)
+    lib.mfq_rt_load_nint_moe_overlay.argtypes = [ctypes.c_char_p, ctypes.c_size_t, ctypes.c_char_p, ctypes.c_size_t,
+                                                 ctypes.POINTER(ctypes.c_void_p)]
+    assert "expert overlay shape mismatch" in _rt_load_error(lib, lib.mfq_rt_load_nint_moe_overlay, good, len(good), wrong,
+                                                             len(wrong))
 
 
 def test_mfq_directory_checks_of_the_reference_reader(tmp_path):

@@ -236,6 +236,8 @@ def test_tensor_and_expert_overlays(tmp_path, monkeypatch):
             assert bytes(st.blob("blk.0.attn_k.weight")) == TENSORS["blk.0.attn_k.weight"][1]
             assert list(st.tensor_overlays) == ["blk.0.attn_q.weight"]
             assert st.expert_overlays["blk.0.ffn_gate_up_exps.weight"].nbytes == 77
+            assert bytes(st.expert_overlay_blob("blk.0.ffn_gate_up_exps.weight")) == b"\x01" * 77
+            assert st.expert_overlay_blob("blk.0.attn_q.weight") is None
             got = {n: (d, b) for n, d, _, b in _cpp_records(lib, h)}
             assert got["blk.0.attn_q.weight"] == ("NINT5", new_q)
             assert got["blk.0.attn_k.weight"][1] == TENSORS["blk.0.attn_k.weight"][1]

@@ -534,3 +534,42 @@ def test_decode_pairs_take_bf16_rows_of_any_magnitude(scale):
     for t_ in range(T):
         for r in range(R):
             assert rel_l2(got[t_, r], ref[t_, r]) < REL_TOL, (t_, r, rel_l2(got[t_, r], ref[t_, r]))
+
+
+def test_expert_overlay_cohorts_take_over_their_experts():
+    """An NINTMD expert overlay (magic NID2: cohorts for some experts only) on a mixed-family NINTM tensor: the overlay's
+    cohorts are appended and own the experts they list -- here a NINT3 cohort takes a NINT4 expert and an NVQ expert, an
+    NEPQ1-S cohort a stream-NVQ expert.  Dequantized experts bit for bit against the oracle's overlaid tensor; a decode
+    step (one launch per cohort) and a mapped batch against the oracle's loop; the delta alone is not a tensor."""
+    from tyloquant_amd.runtime_moe import NintMoeWeight, build_moe_route_plan
+    rng = np.random.default_rng(80)
+    out, K, E, R = 32, 192, 9, 3
+    base = _mixed_family_moe(rng, out, K)
+    def pool(ids, dtype, t):
+        return O.MoePool(np.asarray(ids, dtype=np.int32), dtype, t)
+    delta = O.NintMoeTensor((E, out, K), [pool([4, 1], "NINT3", synth.nint_random(rng, 2 * out, K, 3, 24, 5)),
+                                          pool([2], "NEPQ1-S", synth.nepq_random(rng, "NEPQ1-S", 1, out, K, 3))])
+    blob, dblob = O.pack_nint_moe(base), O.pack_nint_moe(delta, delta=True)
+    assert dblob[:4] == b"NID2"
+    with pytest.raises(ValueError, match="delta cannot be loaded as a full tensor"):
+        NintMoeWeight.from_blob(dblob)
+    with pytest.raises(ValueError, match="delta cannot be loaded as a full tensor"):
+        O.unpack_nint_moe(dblob)
+    back = O.unpack_nint_moe(dblob, allow_partial=True)
+    assert [p.dtype for p in back.pools] == ["NINT3", "NEPQ1-S"] and back.pools[0].expert_ids.tolist() == [4, 1]
+    w = NintMoeWeight.from_blob(blob, expert_overlay=dblob)
+    over = O.apply_expert_overlay(base, delta)
+    dense = O.dequantize_expertwise(over)
+    assert not np.array_equal(dense, O.dequantize_expertwise(base))
+    assert np.array_equal(w.dequantize().cpu().numpy().view(np.uint32), dense.view(np.uint32))
+    assert w.expert_bits[4] == 3 and w.expert_bits[1] == 3 and w.expert_bits[0] == 4
+    with pytest.raises(ValueError, match="expert overlay shape mismatch"):
+        NintMoeWeight.from_blob(blob, expert_overlay=O.pack_nint_moe(O.NintMoeTensor((E, out, 2 * K), [pool(
+            [0], "NINT4", synth.nint_random(rng, out, 2 * K, 4, 32, 6))]), delta=True))
+    for T in (40, 2):
+        ids = np.stack([rng.choice(E, size=R, replace=False) for _ in range(T)]).astype(np.int32)
+        ids[0] = [4, 1, 2]                                # the three experts that changed hands
+        x = torch.from_numpy((rng.standard_normal((T, K)) * 0.1).astype(np.float32)).to(torch.bfloat16)
+        got = w(x.cuda(), build_moe_route_plan(torch.from_numpy(ids).cuda(), E)).cpu().numpy()
+        ref = O.moe_grouped_matmul(dense, x.float().numpy(), ids)
+        assert rel_l2(got, ref) < REL_TOL and np.abs(got - ref).max() < ABS_TOL

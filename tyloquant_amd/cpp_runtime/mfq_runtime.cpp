@@ -220,9 +220,11 @@ NepqHeader parse_nepq(const uint8_t *b, size_t n) {
     return h;
 }
 
-NintmHeader parse_nintm(const uint8_t *b, size_t n) {
+NintmHeader parse_nintm(const uint8_t *b, size_t n, bool allow_partial) {
     if (n < 20) fail("truncated NINTM header");
-    if (std::memcmp(b, "NIM2", 4) != 0) fail("invalid NINTM magic");
+    const bool delta = std::memcmp(b, "NID2", 4) == 0;
+    if (delta && !allow_partial) fail("NINTM delta cannot be loaded as a full tensor");
+    if (!delta && std::memcmp(b, "NIM2", 4) != 0) fail("invalid NINTM magic");
     NintmHeader h;
     h.n_experts = static_cast<int>(rd<uint32_t>(b, 4)); h.out_per_expert = static_cast<int>(rd<uint32_t>(b, 8));
     h.neuron_len = static_cast<int>(rd<uint32_t>(b, 12));
@@ -264,7 +266,7 @@ NintmHeader parse_nintm(const uint8_t *b, size_t n) {
         h.pools.push_back(std::move(p));
     }
     if (off != n) fail("invalid NINTM tail: " + std::to_string(n - off) + " extra bytes");
-    for (int e = 0; e < h.n_experts; ++e)
+    for (int e = 0; e < h.n_experts && !allow_partial; ++e)
         if (owner[e] < 0) fail("NINTM pools do not cover expert " + std::to_string(e));
     return h;
 }
@@ -931,18 +933,36 @@ MoeRoutePlan build_moe_route_plan(const int32_t *ids, int tokens, int routes, in
     return p;
 }
 
-NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream) {
-    const NintmHeader h = parse_nintm(blob, n);
+NintMoeWeight NintMoeWeight::from_blob(const uint8_t *base_blob, size_t n, mfq_stream_t stream, const uint8_t *overlay,
+                                       size_t overlay_n) {
+    const NintmHeader h = parse_nintm(base_blob, n);
     NintMoeWeight w;
     w.n_experts = h.n_experts; w.out_per_expert = h.out_per_expert; w.neuron_len = h.neuron_len;
+    // the cohorts of an expert overlay follow the tensor's own; the last cohort that lists an expert owns it
+    struct Cohort { const uint8_t *blob; const NintmPool *pool; };
+    std::vector<Cohort> cohorts;
+    for (const NintmPool &p : h.pools) cohorts.push_back({base_blob, &p});
+    NintmHeader d;
+    if (overlay) {
+        d = parse_nintm(overlay, overlay_n, true);
+        if (d.n_experts != h.n_experts || d.out_per_expert != h.out_per_expert || d.neuron_len != h.neuron_len)
+            fail("expert overlay shape mismatch");
+        for (const NintmPool &p : d.pools) cohorts.push_back({overlay, &p});
+    }
+    std::vector<int> owner(static_cast<size_t>(h.n_experts), -1);
+    for (size_t ci = 0; ci < cohorts.size(); ++ci)
+        for (int32_t e : cohorts[ci].pool->expert_ids) owner[static_cast<size_t>(e)] = static_cast<int>(ci);
     std::vector<int32_t> ep(h.n_experts, -1), el(h.n_experts, -1);
-    for (size_t pi = 0; pi < h.pools.size(); ++pi) {
-        const NintmPool &p = h.pools[pi];
+    for (size_t pi = 0; pi < cohorts.size(); ++pi) {
+        const NintmPool &p = *cohorts[pi].pool;
+        const uint8_t *blob = cohorts[pi].blob;
+        std::vector<uint8_t> live;
+        for (int32_t e : p.expert_ids) live.push_back(owner[static_cast<size_t>(e)] == static_cast<int>(pi) ? 1 : 0);
         if (p.runtime_bytes) fail("unexpected NINTM cohort runtime metadata");
         const std::string shape_error = "NINTM pool " + std::to_string(pi) + " tensor shape does not match its expert count";
         if (!is_nint_linear_dtype(p.dtype)) {
             MoeForeignCohort c;
-            c.dtype = p.dtype; c.expert_ids = p.expert_ids;
+            c.dtype = p.dtype; c.expert_ids = p.expert_ids; c.live = live;
             const int parts = static_cast<int>(p.expert_ids.size());
             if (is_nepq_linear_dtype(p.dtype)) {
                 c.nepq = std::make_shared<NepqWeight>(NepqWeight::from_blob(blob + p.payload_off, p.payload_bytes, nullptr, stream));
@@ -970,6 +990,7 @@ NintMoeWeight NintMoeWeight::from_blob(const uint8_t *blob, size_t n, mfq_stream
         if (pw->out() != static_cast<int64_t>(p.expert_ids.size()) * h.out_per_expert || pw->neuron_len() != h.neuron_len)
             fail(shape_error);
         for (size_t i = 0; i < p.expert_ids.size(); ++i) {
+            if (!live[i]) continue;
             ep[p.expert_ids[i]] = static_cast<int32_t>(w.pool_table.size());
             el[p.expert_ids[i]] = static_cast<int32_t>(i);
         }
@@ -1009,7 +1030,8 @@ void MoeForeignCohort::dequantize(int local, float *out, mfq_stream_t stream) co
 void MoeForeignCohort::prepare_pairs(int n_experts, int out_per_expert, mfq_stream_t stream) {
     if (nepq && !nepq->streams && out_per_expert % 16) return;  // NEPQ1 experts must be whole row-blocks
     std::vector<int32_t> slot(static_cast<size_t>(n_experts), -1);
-    for (size_t i = 0; i < expert_ids.size(); ++i) slot[static_cast<size_t>(expert_ids[i])] = static_cast<int32_t>(i);
+    for (size_t i = 0; i < expert_ids.size(); ++i)
+        if (live.empty() || live[i]) slot[static_cast<size_t>(expert_ids[i])] = static_cast<int32_t>(i);
     pair_slot.ensure(slot.size() * 4);
     hip_check(hipMemcpyAsync(pair_slot.get(), slot.data(), slot.size() * 4, hipMemcpyHostToDevice, hs(stream)), "NINTM cohort tables");
     std::vector<const void *> ptrs;
@@ -1087,6 +1109,7 @@ void NintMoeWeight::add_foreign(const void *x, int x_dtype, int64_t ldx, bool ro
     for (const MoeForeignCohort *cp : walk) {
         const MoeForeignCohort &c = *cp;
         for (size_t local = 0; local < c.expert_ids.size(); ++local) {
+            if (!c.live.empty() && !c.live[local]) continue;  // an expert overlay gave this expert to a later cohort
             const int32_t e = c.expert_ids[local];
             std::vector<int32_t> pair_rows, src_rows;
             for (int t = 0; t < T; ++t)
@@ -1883,6 +1906,12 @@ int mfq_rt_moe_cache_stats(void *cache, int64_t *out5) {
 
 int mfq_rt_load_nint_moe(const void *blob, size_t n, void **handle) {
     return guard([&] { *handle = new NintMoeWeight(NintMoeWeight::from_blob(static_cast<const uint8_t *>(blob), n)); });
+}
+int mfq_rt_load_nint_moe_overlay(const void *blob, size_t n, const void *overlay, size_t overlay_n, void **handle) {
+    return guard([&] {
+        *handle = new NintMoeWeight(NintMoeWeight::from_blob(static_cast<const uint8_t *>(blob), n, nullptr,
+                                                             static_cast<const uint8_t *>(overlay), overlay_n));
+    });
 }
 void mfq_rt_free_nint_moe(void *handle) { delete static_cast<NintMoeWeight *>(handle); }
 int mfq_rt_file_open(const char *path, const char *tensor_overlay, const char *expert_overlay, void **handle) {

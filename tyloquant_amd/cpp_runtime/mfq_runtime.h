@@ -83,7 +83,9 @@ struct NintmHeader {
 NintHeader parse_nint(const uint8_t *blob, size_t n);
 NvqHeader parse_nvq(const uint8_t *blob, size_t n);
 NepqHeader parse_nepq(const uint8_t *blob, size_t n);
-NintmHeader parse_nintm(const uint8_t *blob, size_t n);
+// allow_partial: also an expert delta (an NINTMD overlay record: magic NID2, cohorts for some experts only;
+// unpack_nint_moe_delta :2484-2487)
+NintmHeader parse_nintm(const uint8_t *blob, size_t n, bool allow_partial = false);
 
 // ---- weights ------------------------------------------------------------------------------------
 struct NintWeight {
@@ -275,6 +277,7 @@ std::vector<std::vector<uint8_t>> split_rows(const std::string &dtype, const uin
 struct MoeForeignCohort {
     std::string dtype;
     std::vector<int32_t> expert_ids;
+    std::vector<uint8_t> live;          // per expert: still owned (an expert overlay may give it to a later cohort)
     std::vector<QuantLinear> linears;   // one per expert (NVQ, 1-bit families)
     std::shared_ptr<NepqWeight> nepq;   // or the cohort as one expert-shaped tensor
     std::shared_ptr<MxWeight> mx;       // or a native MXFP4 pool: one [experts * out, K] tensor, experts = row ranges
@@ -306,7 +309,10 @@ struct NintMoeWeight {
     DeviceBuffer expert_pool, expert_local;  // int32 [E] dispatch tables
     std::vector<mfq_moe_pool> pool_table;
     mutable DeviceBuffer workspace;  // prefill path, grown on demand (do not grow it under graph capture)
-    static NintMoeWeight from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream = nullptr);
+    // overlay: the NINTMD record of the same name from an expert overlay file (MfqFile::expert_overlays): its cohorts are
+    // appended and own the experts they list (load_nint_moe_cpu :5752-5774)
+    static NintMoeWeight from_blob(const uint8_t *blob, size_t n, mfq_stream_t stream = nullptr,
+                                   const uint8_t *overlay = nullptr, size_t overlay_n = 0);
     // x: [T, K] (routed_input = false) or [T*R, K]; out: fp32 [T*R, out_per_expert]
     void forward(const void *x, int x_dtype, int64_t ldx, bool routed_input, const MoeRoutePlan &route, float *out,
                  mfq_stream_t stream = nullptr) const;

@@ -650,11 +650,15 @@ def nintm_blob(n_experts, out_per_expert, neuron_len, pools) -> bytes:
     return b"".join(parts)
 
 
-def parse_nintm(blob) -> NintmHeader:
+def parse_nintm(blob, allow_partial: bool = False) -> NintmHeader:
+    """allow_partial: also take an expert delta (an NINTMD overlay record: magic NID2, the same layout, pools for some
+    experts only -- unpack_nint_moe_impl, cpp_runtime/mfq_decode.cpp:2367-2477)."""
     if len(blob) < _NIM_HDR.size:
         raise ValueError("truncated NINTM header")
     magic, E, out, K, npools = _NIM_HDR.unpack_from(blob, 0)
-    if magic != b"NIM2":
+    if magic == b"NID2" and not allow_partial:
+        raise ValueError("NINTM delta cannot be loaded as a full tensor")
+    if magic not in (b"NIM2", b"NID2"):
         raise ValueError(f"invalid NINTM magic: {magic!r}")
     if npools == 0 or npools > E:
         raise ValueError("invalid NINTM pool count")
@@ -690,7 +694,7 @@ def parse_nintm(blob) -> NintmHeader:
     if off != len(blob):
         raise ValueError(f"invalid NINTM tail: {len(blob) - off} extra bytes")
     missing = np.flatnonzero(owners < 0)
-    if missing.size:
+    if missing.size and not allow_partial:
         raise ValueError(f"NINTM pools do not cover experts {missing[:16].tolist()}")
     return hdr
 
@@ -1009,6 +1013,13 @@ class MfqStore:
         """The record's bytes as a read-only view into the file map (no copy); valid until close()."""
         r = self.record(name)
         return memoryview(self._maps[r.source])[r.offset: r.offset + r.nbytes]
+
+    def expert_overlay_blob(self, name):
+        """The NINTMD record an expert overlay holds for NINTM tensor `name` (read_expert_overlay,
+        cpp_runtime/mfq_decode.cpp:1513-1521) as a view into its file map, or None when there is none: what
+        NintMoeWeight.from_blob takes as `expert_overlay`."""
+        r = self.expert_overlays.get(name)
+        return None if r is None else memoryview(self._maps[r.source])[r.offset: r.offset + r.nbytes]
 
     def asset_text(self, name) -> str:
         r = self.record(name)

@@ -120,6 +120,7 @@ class ForeignCohort:
         if shape != (n, out_per_expert, neuron_len):
             raise ValueError(f"NINTM pool tensor shape {shape} must be {(n, out_per_expert, neuron_len)}")
         self._slot = self._wtab = None           # device tables of the one-launch decode form, built on first use
+        self.live = np.ones(n, dtype=bool)       # experts an expert overlay has not given to a later cohort
 
     PAIRS_MAX = 64   # (token, route) pairs up to which a decode step takes one launch per cohort over all its pairs
 
@@ -132,7 +133,7 @@ class ForeignCohort:
         lib, dev = L.lib(), x2.device
         if self._slot is None:
             slot = np.full(n_experts, -1, dtype=np.int32)
-            slot[self.expert_ids] = np.arange(len(self.expert_ids), dtype=np.int32)
+            slot[self.expert_ids[self.live]] = np.arange(len(self.expert_ids), dtype=np.int32)[self.live]
             self._slot = torch.from_numpy(slot).to(dev)
             if self.linears:
                 self._wtab = torch.tensor([q.weight.data.data_ptr() for q in self.linears], dtype=torch.int64, device=dev)
@@ -189,16 +190,19 @@ class NintMoeWeight:
     """One logical [experts, out_per_expert, K] tensor made of cohorts (NINTM / NIM2).  NINT cohorts run on the grouped
     kernels; cohorts of other families (`foreign`) are added by the host, expert by expert."""
 
-    def __init__(self, n_experts, out_per_expert, neuron_len, pools, expert_ids, device, foreign=()):
+    def __init__(self, n_experts, out_per_expert, neuron_len, pools, expert_ids, device, foreign=(), pool_live=None):
+        """pool_live[i]: which experts of NINT cohort i the cohort still owns (all of them unless an expert overlay gave
+        some to a later cohort); cohorts of other families carry the same mask as `live`."""
         self.n_experts, self.out_per_expert, self.neuron_len = n_experts, out_per_expert, neuron_len
         self.pools: list[NintWeight] = pools
         self.pool_expert_ids = expert_ids
+        self.pool_live = pool_live if pool_live is not None else [np.ones(len(ids), dtype=bool) for ids in expert_ids]
         self.foreign: list[ForeignCohort] = list(foreign)
         ep = np.full(n_experts, -1, dtype=np.int32)       # -1: no NINT cohort -- the kernels leave a zero row
         el = np.full(n_experts, -1, dtype=np.int32)
-        for pi, ids in enumerate(expert_ids):
-            ep[ids] = pi
-            el[ids] = np.arange(len(ids), dtype=np.int32)
+        for pi, (ids, live) in enumerate(zip(expert_ids, self.pool_live)):
+            ep[ids[live]] = pi
+            el[ids[live]] = np.arange(len(ids), dtype=np.int32)[live]
         # device dispatch tables (initialize_nint_moe_dispatch, cpp_runtime/mfq_decode.cpp:3249-3343)
         self.expert_pool = torch.from_numpy(ep).to(device)
         self.expert_local = torch.from_numpy(el).to(device)
@@ -208,8 +212,8 @@ class NintMoeWeight:
             self._pool_array[i].weight = p.data.data_ptr()
         self._ws = _Workspace()
         self.expert_bits = np.zeros(n_experts, dtype=np.int32)
-        for pi, ids in enumerate(expert_ids):
-            self.expert_bits[ids] = pools[pi].bits
+        for pi, (ids, live) in enumerate(zip(expert_ids, self.pool_live)):
+            self.expert_bits[ids[live]] = pools[pi].bits
 
     @property
     def payload_bytes(self) -> int:
@@ -218,17 +222,29 @@ class NintMoeWeight:
     def expert_payload_bytes(self, e: int) -> float:
         pi = int(self.expert_pool[e].item())
         if pi < 0:
-            c = next(c for c in self.foreign if e in c.expert_ids)
+            c = next(c for c in self.foreign if e in c.expert_ids[c.live])
             return c.payload_bytes / len(c.expert_ids)
         return self.pools[pi].payload_bytes / len(self.pool_expert_ids[pi])
 
     @staticmethod
-    def from_blob(blob, device="cuda") -> "NintMoeWeight":
+    def from_blob(blob, device="cuda", expert_overlay=None) -> "NintMoeWeight":
+        """expert_overlay: the NINTMD record of the same name from an expert overlay file (MfqFile.expert_overlays): its
+        cohorts are appended and take over the experts they list (load_nint_moe_cpu, cpp_runtime/mfq_decode.cpp:5752-5774)."""
         h = F.parse_nintm(blob)
+        cohorts = [(blob, p) for p in h.pools]
+        if expert_overlay is not None:
+            d = F.parse_nintm(expert_overlay, allow_partial=True)
+            if (d.n_experts, d.out_per_expert, d.neuron_len) != (h.n_experts, h.out_per_expert, h.neuron_len):
+                raise ValueError("expert overlay shape mismatch")
+            cohorts += [(expert_overlay, p) for p in d.pools]
+        owner = np.full(h.n_experts, -1, dtype=np.int64)        # the last cohort that lists an expert owns it
+        for ci, (_, p) in enumerate(cohorts):
+            owner[p.expert_ids] = ci
         device = torch.device(device)
-        pools, ids = [], []
+        pools, ids, pool_live = [], [], []
         foreign = []
-        for p in h.pools:
+        for ci, (blob, p) in enumerate(cohorts):
+            live = owner[p.expert_ids] == ci
             if p.runtime_bytes:
                 raise ValueError("unexpected NINTM cohort runtime metadata")
             if not (p.dtype.startswith("NINT") and p.dtype[4:].isdigit()):
@@ -240,6 +256,7 @@ class NintMoeWeight:
                     raise NotImplementedError(f"NINTM cohort family {p.dtype} is not supported")
                 foreign.append(ForeignCohort(p.dtype, bytes(blob[p.payload_off: p.payload_off + p.payload_bytes]),
                                              p.expert_ids, h.out_per_expert, h.neuron_len, device))
+                foreign[-1].live = live
                 continue
             w = NintWeight.from_blob(bytes(blob[p.payload_off: p.payload_off + p.payload_bytes]), device)
             if w.out != len(p.expert_ids) * h.out_per_expert or w.neuron_len != h.neuron_len:
@@ -247,16 +264,19 @@ class NintMoeWeight:
                                  f"{(len(p.expert_ids) * h.out_per_expert, h.neuron_len)}")
             pools.append(w)
             ids.append(p.expert_ids)
-        return NintMoeWeight(h.n_experts, h.out_per_expert, h.neuron_len, pools, ids, device, foreign)
+            pool_live.append(live)
+        return NintMoeWeight(h.n_experts, h.out_per_expert, h.neuron_len, pools, ids, device, foreign, pool_live)
 
     def dequantize(self) -> torch.Tensor:
         out = torch.empty((self.n_experts, self.out_per_expert, self.neuron_len), dtype=torch.float32,
                           device=self.expert_pool.device)
-        for p, ids in zip(self.pools, self.pool_expert_ids):
-            out[torch.from_numpy(ids.astype(np.int64)).to(out.device)] = p.dequantize().reshape(
-                len(ids), self.out_per_expert, self.neuron_len)
+        for p, ids, live in zip(self.pools, self.pool_expert_ids, self.pool_live):
+            mask = torch.from_numpy(live).to(out.device)
+            out[torch.from_numpy(ids[live].astype(np.int64)).to(out.device)] = p.dequantize().reshape(
+                len(ids), self.out_per_expert, self.neuron_len)[mask]
         for c in self.foreign:
-            out[torch.from_numpy(c.expert_ids.astype(np.int64)).to(out.device)] = c.dequantize()
+            mask = torch.from_numpy(c.live).to(out.device)
+            out[torch.from_numpy(c.expert_ids[c.live].astype(np.int64)).to(out.device)] = c.dequantize()[mask]
         return out
 
     def _add_foreign(self, x2: torch.Tensor, routed: bool, route: MoeRoutePlan, out: torch.Tensor) -> None:
@@ -276,6 +296,8 @@ class NintMoeWeight:
         ids = route.ids.reshape(T, R).cpu().numpy()
         for c in walk:
             for local, e in enumerate(c.expert_ids):
+                if not c.live[local]:
+                    continue
                 t_idx, r_idx = np.nonzero(ids == e)
                 if t_idx.size == 0:
                     continue
