@@ -128,3 +128,36 @@ def test_mx_entry_points_check_geometry_rows_and_workspace(lib):
     assert lib.mfq_hip_mx_gemm_rows_workspace_bytes(96, 4, 16) == 0 and lib.mfq_hip_mx_gemm_rows_workspace_bytes(96, 4, 17) > 0
     assert lib.mfq_hip_mx_gemm_rows(4, FAKE, FAKE, 4, 96, 0, 4, FAKE, L.X_BF16, 96, 17, FAKE, 4, None, 0, None) == L.ERR_WORKSPACE
 
+
+
+def test_embedding_and_decode_pair_entry_points_check_their_arguments(lib):
+    """The embedding-row entry points of the NVQ / NINT8-0 tables and the per-cohort launches of a MoE decode step
+    (mfq_hip_*_gemv_pairs): null pointers, output types, strides, pair counts and expert row counts are refused before
+    anything is launched."""
+    v = L.NvqDesc()
+    assert lib.mfq_hip_nvq_plan(9, 2, 64, 96, C.byref(v)) == L.OK
+    assert lib.mfq_hip_nvq_embedding(C.byref(v), None, FAKE, 2, FAKE, L.X_F16, 96, None) == L.ERR_INVALID
+    assert lib.mfq_hip_nvq_embedding(C.byref(v), FAKE, FAKE, 2, FAKE, 9, 96, None) == L.ERR_INVALID and "out_dtype" in _msg(lib)
+    assert lib.mfq_hip_nvq_embedding(C.byref(v), FAKE, FAKE, 2, FAKE, L.X_F16, 95, None) == L.ERR_INVALID and "ldo" in _msg(lib)
+    assert lib.mfq_hip_nvq_embedding(C.byref(v), FAKE, None, 2, FAKE, L.X_F16, 96, None) == L.ERR_INVALID
+    assert lib.mfq_hip_nvq_embedding(C.byref(v), FAKE, None, 0, None, L.X_F16, 96, None) == L.OK          # no ids: nothing to do
+    z = L.Nint8zDesc()
+    assert lib.mfq_hip_nint8z_plan(64, 96, C.byref(z)) == L.OK
+    assert lib.mfq_hip_nint8z_embedding(C.byref(z), FAKE, FAKE, -1, FAKE, L.X_F16, 96, None) == L.ERR_INVALID
+    assert lib.mfq_hip_nvq_gemv_pairs(C.byref(v), None, FAKE, 8, FAKE, L.X_BF16, 96, 0, FAKE, 1, 2, FAKE, 64, None) == L.ERR_INVALID
+    assert lib.mfq_hip_nvq_gemv_pairs(C.byref(v), FAKE, FAKE, 8, FAKE, 5, 96, 0, FAKE, 1, 2, FAKE, 64, None) == L.ERR_INVALID
+    assert lib.mfq_hip_nvq_gemv_pairs(C.byref(v), FAKE, FAKE, 8, FAKE, L.X_BF16, 96, 0, FAKE, 40000, 2, FAKE, 64,
+                                      None) == L.ERR_UNSUPPORTED and "65535" in _msg(lib)
+    assert lib.mfq_hip_nvq_gemv_pairs(C.byref(v), FAKE, FAKE, 8, FAKE, L.X_BF16, 96, 0, FAKE, 1, 2, FAKE, 63, None) == L.ERR_INVALID
+    assert lib.mfq_hip_nvq_gemv_pairs(C.byref(v), FAKE, FAKE, 8, FAKE, L.X_BF16, 96, 0, FAKE, 0, 2, FAKE, 64, None) == L.OK
+    assert lib.mfq_hip_nint8z_gemv_pairs(C.byref(z), FAKE, None, 8, FAKE, L.X_BF16, 96, 0, FAKE, 1, 2, FAKE, 64, None) == L.ERR_INVALID
+    assert lib.mfq_hip_mx_gemv_pairs(4, FAKE, FAKE, 64, 96, 24, FAKE, 8, FAKE, L.X_BF16, 96, 0, FAKE, 1, 2, FAKE, 24,
+                                     None) == L.ERR_INVALID and "do not divide" in _msg(lib)
+    assert lib.mfq_hip_mx_gemv_pairs(8, FAKE, FAKE, 256, 128, 64, FAKE, 8, FAKE, L.X_BF16, 128, 0, FAKE, 1, 2, FAKE, 64,
+                                     None) == L.ERR_UNSUPPORTED and "128-row" in _msg(lib)
+    s = L.NvqsDesc()
+    assert lib.mfq_hip_nvqs_plan(8, 8, 2, 0, 64, 96, C.byref(s)) == L.OK
+    assert lib.mfq_hip_nvqs_gemv_pairs(C.byref(s), None, None, 64, FAKE, 8, FAKE, L.X_BF16, 96, 0, FAKE, 1, 2, FAKE, 64,
+                                       None) == L.ERR_INVALID
+    assert lib.mfq_hip_nvqs_gemv_pairs(C.byref(s), None, FAKE, 24, FAKE, 8, FAKE, L.X_BF16, 96, 0, FAKE, 1, 2, FAKE, 64,
+                                       None) == L.ERR_INVALID and "rows per expert" in _msg(lib)
