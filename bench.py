@@ -475,6 +475,21 @@ def main() -> int:
         del stack, proto
         torch.cuda.empty_cache()
 
+        # ---- OCP MX payloads (no BASELINE config): 12288 x 4096 MXFP4 / MXFP8 read in place, batch {1, 16} ----
+        from tyloquant_amd.runtime_mx import MxWeight, mx_matmul
+        for mx_dtype in ("MXFP4", "MXFP8"):
+            blob = synth.mx_blob(60, mx_dtype, 12288, 4096)[1]
+            mxw = [MxWeight.from_blob(mx_dtype, blob) for _ in range(8)]
+            for M in (1, 16):
+                xm = [bf16(synth.activations(rng, M, 4096)) for _ in range(8)]
+                ms = graph_ms(lambda: [mx_matmul(mxw[i], xm[i]) for i in range(8)], 5, warm=2) / 8
+                key = f"{mx_dtype.lower()}_12288x4096_M{M}"
+                extras[f"{key}_us"] = ms * 1e3
+                extras[f"{key}_gbps"] = mxw[0].payload_bytes / (ms * 1e-3) / 1e9
+                log(f"[bench] {mx_dtype} 12288x4096 M={M}: {ms * 1e3:.1f} us, {extras[f'{key}_gbps']:.0f} GB/s of payload")
+            del mxw
+        torch.cuda.empty_cache()
+
     cpu = None
     if not args.no_cpu:
         from oracle import c_oracle

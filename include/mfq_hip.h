@@ -19,7 +19,9 @@
  *   - the NVQ3J kernel for one and two rows with its signed table in LDS, the NVQ kernels behind a MoE decode step on an
  *     NVQ cohort (mfq_hip_nvq_gemv_pairs), the NEPQ1 one-row kernel and the NINT8-0 streaming GEMV (one row; more rows when
  *     the activation rows are not 16-byte aligned),
- *   - the stream-family (E8, d4_1024, 1-bit, NEPQ0) and MX wave-per-neuron kernels up to 16 rows, which multiply in fp32,
+ *   - the stream-family (E8, d4_1024, 1-bit, NEPQ0) wave-per-neuron kernels up to 16 rows, which multiply in fp32,
+ *   - the MXFP4 / MXFP8 kernels up to 256 rows, whose matrix-core products take bf16 as it is (the weights are exact in
+ *     bf16, scale included),
  *   - every prefill kernel:
  * every K-slice of a row (the streaming GEMVs; the whole row in the NINT8-0 GEMV and the prefill kernels) is scaled by a
  * power of two before the conversion and the sums are scaled back, so a row of values near 1e-6 or 1e6 keeps the
@@ -444,9 +446,12 @@ int mfq_hip_nvqs_gemm(const mfq_nvqs_desc *d, const void *weight, const void *x,
  * dequant_mxfp4_cpu, cpp_runtime/mfq_decode.cpp:1832-1947, mxfp8_dequant_kernel, mfq/kernels/cuda/mx_matmul.cu:222-240),
  * or that rounded once more to fp16 as the reference's device copy is (MFQ_X_F16); a scale byte 255 and the E4M3FN codes
  * 0x7f / 0xff give NaN.
- * mfq_hip_mx_gemm_rows: y[M, nrows] = x[M, cols] . W^T in fp32 (mxfp8_matmul_f32, mfq_decode.cpp:8784-8802): a wave
- * per neuron up to 16 rows of x (mxfp8_small_m_f32_cuda serves 1..8), above that an fp16 copy of the rows, each
- * relative to its largest scale, and the fp16 MFMA GEMM -- workspace of mfq_hip_mx_gemm_rows_workspace_bytes. */
+ * mfq_hip_mx_gemm_rows: y[M, nrows] = x[M, cols] . W^T in fp32 (mxfp8_matmul_f32, mfq_decode.cpp:8784-8802): up to 256
+ * rows of x on the matrix cores from the file's bytes (the hardware's FP4 / FP8 conversions with the E8M0 scale in
+ * their exponent operand, bf16 or fp16 MFMA by the activations' type; mxfp8_small_m_f32_cuda serves 1..8 rows) when x is
+ * 16-byte aligned with ldx % 8 == 0 -- otherwise a wave per neuron, four rows per pass; above 256 rows an fp16 copy of
+ * the rows, each relative to its largest scale, and the fp16 MFMA GEMM -- workspace of
+ * mfq_hip_mx_gemm_rows_workspace_bytes.  bf16 activations of any magnitude are taken as they are (no fp16 detour). */
 int mfq_hip_mx_dequant_rows(int kind, const void *values, const void *scales, int rows, int cols, int row0, int nrows,
                             int out_dtype, void *w_out, int64_t ld, mfq_stream_t stream);
 size_t mfq_hip_mx_gemm_rows_workspace_bytes(int cols, int nrows, int M);

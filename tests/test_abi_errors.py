@@ -125,8 +125,9 @@ def test_mx_entry_points_check_geometry_rows_and_workspace(lib):
         assert rc == L.ERR_INVALID and "outside the tensor" in _msg(lib)
     assert lib.mfq_hip_mx_gemm_rows(4, FAKE, FAKE, 4, 96, 0, 4, FAKE, L.X_F32, 96, 1, FAKE, 4, None, 0, None) == L.ERR_INVALID
     assert lib.mfq_hip_mx_gemm_rows(4, FAKE, FAKE, 4, 96, 0, 4, FAKE, L.X_BF16, 64, 1, FAKE, 4, None, 0, None) == L.ERR_INVALID
-    assert lib.mfq_hip_mx_gemm_rows_workspace_bytes(96, 4, 16) == 0 and lib.mfq_hip_mx_gemm_rows_workspace_bytes(96, 4, 17) > 0
-    assert lib.mfq_hip_mx_gemm_rows(4, FAKE, FAKE, 4, 96, 0, 4, FAKE, L.X_BF16, 96, 17, FAKE, 4, None, 0, None) == L.ERR_WORKSPACE
+    # up to 256 rows run on the tile kernels without a workspace, the fp16 copy + GEMM above needs one
+    assert lib.mfq_hip_mx_gemm_rows_workspace_bytes(96, 4, 256) == 0 and lib.mfq_hip_mx_gemm_rows_workspace_bytes(96, 4, 257) > 0
+    assert lib.mfq_hip_mx_gemm_rows(4, FAKE, FAKE, 4, 96, 0, 4, FAKE, L.X_BF16, 96, 257, FAKE, 4, None, 0, None) == L.ERR_WORKSPACE
 
 
 

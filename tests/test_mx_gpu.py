@@ -50,12 +50,53 @@ def test_mx_matmul_all_routes(dtype, rows, cols):
     assert lin.out == rows and lin.neuron_len == cols
     assert same_bits(lin.dequantize().cpu().numpy(), want)
     for M, xdt in ((1, torch.bfloat16), (2, torch.float16), (3, torch.bfloat16), (16, torch.bfloat16), (17, torch.float16),
-                   (70, torch.bfloat16)):
+                   (70, torch.bfloat16), (300, torch.bfloat16), (257, torch.float16)):   # above 256 rows: fp16 copy + GEMM
         x = torch.from_numpy(rng.standard_normal((M, cols)).astype(np.float32)).to(xdt).cuda()
         check_close(lin(x).cpu().numpy(), O.linear_forward_f64(want, x.float().cpu().numpy()))
     assert lin(torch.empty((0, cols), dtype=torch.bfloat16, device="cuda")).shape == (0, rows)
     xw = torch.from_numpy(rng.standard_normal((5, cols + 8)).astype(np.float32)).to(torch.bfloat16).cuda()[:, :cols]
     check_close(lin(xw).cpu().numpy(), O.linear_forward_f64(want, xw.float().cpu().numpy()))    # a row stride above K
+
+
+@pytest.mark.parametrize("dtype,rows,cols", [("MXFP4", 200, 2880), ("MXFP4", 48, 4096), ("MXFP8", 256, 384), ("MXFP8", 384, 2944)])
+def test_mx_matrix_core_tiles(dtype, rows, cols):
+    """The tile kernel's corners: K that ends inside a unit (2880 = 22.5 units of four scale blocks, scale rows off
+    4-byte boundaries), row counts off the 16-neuron row-blocks, tiles of 1 .. 32 rows and passes of them, both
+    activation types, rows of bf16 magnitudes fp16 cannot hold, and activations the kernel cannot take in 16-byte pieces."""
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(rows * 7 + cols)
+    t = synth.mx_random(rng, dtype, rows, cols)
+    lin = R.load_quant_linear(dtype, O.pack_mx(t))
+    want = O.dequantize_mx(t)
+    for M, xdt in ((1, torch.bfloat16), (1, torch.float16), (5, torch.bfloat16), (16, torch.float16), (31, torch.bfloat16),
+                   (32, torch.bfloat16), (33, torch.float16), (100, torch.bfloat16), (256, torch.bfloat16)):
+        x = torch.from_numpy(rng.standard_normal((M, cols)).astype(np.float32)).to(xdt).cuda()
+        check_close(lin(x).cpu().numpy(), O.linear_forward_f64(want, x.float().cpu().numpy()))
+    big = torch.from_numpy((rng.standard_normal((3, cols)) * 3.0e5).astype(np.float32)).to(torch.bfloat16).cuda()
+    check_close(lin(big).cpu().numpy() / 3.0e5, O.linear_forward_f64(want, big.float().cpu().numpy()) / 3.0e5)
+    odd = torch.from_numpy(rng.standard_normal((6, cols + 4)).astype(np.float32)).to(torch.bfloat16).cuda()[:, 4:]
+    check_close(lin(odd).cpu().numpy(), O.linear_forward_f64(want, odd.float().cpu().numpy()))
+
+
+@pytest.mark.parametrize("dtype", ["MXFP4", "MXFP8"])
+def test_mx_scale_bytes_0_and_255_in_the_matmul(dtype):
+    """E8M0 0 is 2^-127 and 255 a NaN (mx_matmul.cu:17-28): a neuron whose row holds a NaN scale comes out NaN, the
+    others are untouched; blocks under the smallest scale add nothing visible."""
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(77)
+    rows, cols = 256, 512
+    t = synth.mx_random(rng, dtype, rows, cols)
+    t.scales[0, 0] = 255
+    t.scales[-1, -1] = 0
+    lin = R.load_quant_linear(dtype, O.pack_mx(t))
+    want = O.dequantize_mx(t)
+    nan_rows = np.isnan(want).any(axis=1)
+    assert 0 < nan_rows.sum() < rows
+    for M, xdt in ((1, torch.bfloat16), (4, torch.float16), (20, torch.bfloat16)):
+        x = torch.from_numpy(rng.standard_normal((M, cols)).astype(np.float32)).to(xdt).cuda()
+        got = lin(x).cpu().numpy()
+        assert np.isnan(got[:, nan_rows]).all() and not np.isnan(got[:, ~nan_rows]).any()
+        check_close(got[:, ~nan_rows], O.linear_forward_f64(want[~nan_rows], x.float().cpu().numpy()))
 
 
 def test_mx_wide_scale_range_survives_the_fp16_copy():
@@ -67,7 +108,7 @@ def test_mx_wide_scale_range_survives_the_fp16_copy():
     t.scales[:] = np.array([[87, 100, 127, 140], [167, 150, 127, 90]], np.uint8)
     lin = R.load_quant_linear("MXFP8", O.pack_mx(t))
     want = O.dequantize_mx(t)
-    for M in (4, 40):
+    for M in (4, 40, 260):
         x = torch.from_numpy(rng.standard_normal((M, 512)).astype(np.float32)).to(torch.bfloat16).cuda()
         check_close(lin(x).cpu().numpy(), O.linear_forward_f64(want, x.float().cpu().numpy()))
 

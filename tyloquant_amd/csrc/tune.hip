@@ -48,6 +48,12 @@ Knob g_knobs[] = {
     {"MFQ_MOE_PREFILL_PAIRS", "pairs per expert from which mapped MoE calls take the prefill kernel (0 = default)", 0, false},
     {"MFQ_FFN_SPIN_LIMIT", "polls after which the one-launch FFN's grid barrier gives up", 0, false},
     {"MFQ_FFN_TRACE", "1 = the one-launch FFN records per-block clocks behind its workspace", 0, false},
+    {"MFQ_MX_TILE_OFF", "1 = MXFP4 / MXFP8 small batches on the wave-per-neuron kernel instead of the matrix-core tile kernel", 0, false},
+    {"MFQ_MX_STAGE_OFF", "1 = the MX tile kernel never stages a wave's activation slice and scales in LDS", 0, false},
+    {"MFQ_MX_STAGE_MAX_M", "rows up to which MX matmuls run as 16-row tiles with the activations staged in LDS (default 48)", 0, false},
+    {"MFQ_MX_TILE_MAX_M", "rows up to which MX matmuls run on the tile kernel before the fp16 copy + GEMM (default 256)", 0, false},
+    {"MFQ_MX_NB", "row-blocks per block of the MX tile kernel (0 = by shape)", 0, false},
+    {"MFQ_MX_WAVES", "waves per block the MX tile kernels split K over (0 = by shape)", 0, false},
     {"MFQ_NVQ_PAIRS_MFMA", "0 = a MoE decode step on an NVQ cohort always takes the generic one-row kernel", 0, false},
     {"MFQ_MOE_NB", "row-blocks per wave of the MoE streaming kernel (0 = by shape)", 0, false},
     {"MFQ_MOE_GROUPS", "bit mask of the register groups the mapped MoE prefill path launches (7 = all)", 0, false},

@@ -58,8 +58,8 @@ class MxWeight:
 
 
 def mx_matmul(w: MxWeight, x: torch.Tensor, expert: int = 0) -> torch.Tensor:
-    """x @ W^T in fp32 (mxfp8_matmul_f32, cpp_runtime/mfq_decode.cpp:8784-8802): a wave per neuron up to 16 rows, the fp16
-    copy + MFMA GEMM above."""
+    """x @ W^T in fp32 (mxfp8_matmul_f32, cpp_runtime/mfq_decode.cpp:8784-8802): the matrix-core tile kernels up to 256 rows (a
+    wave per neuron for activations they cannot read in 16-byte pieces), the fp16 copy + MFMA GEMM above."""
     row0, nrows = w._rows(expert)
     x2 = _as_2d(x, w.neuron_len)
     M = x2.shape[0]

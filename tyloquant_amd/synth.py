@@ -108,6 +108,17 @@ def nint8_zero_blob(seed, out, K):
     return "NINT8-0", head + blocks.tobytes()
 
 
+def mx_blob(seed, dtype, out, K, lo=118, hi=132):
+    """(dtype, blob) of an [out, K] MXFP4 / MXFP8 tensor drawn in the packed domain: random value bytes without the E4M3FN
+    NaN codes, E8M0 block scales within a few octaves of one (container of mfq/formats/mx.py:120-151)."""
+    rng = np.random.default_rng(seed)
+    storage, scale = F.mx_shapes(dtype, out, K)
+    values = rng.integers(0, 256, storage, dtype=np.uint8)
+    if dtype == "MXFP8":
+        values[(values & 0x7F) == 0x7F] = 0x38
+    return dtype, F.write_mx(dtype, out, K, values, rng.integers(lo, hi, scale, dtype=np.uint8))
+
+
 def nepq1_blob(seed, label, out, K, banks=16, experts=1):
     rng = np.random.default_rng(seed)
     pid = F.NEPQ_PROFILE[label]
