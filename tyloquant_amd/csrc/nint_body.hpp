@@ -441,28 +441,6 @@ __device__ __forceinline__ int gemv_red_offset(int nwaves, int mb, int spw, int 
     return nwaves * (mb * (spw * 16 * (gs / 2) + 2 * spw * 16));
 }
 
-// Tuning builds (-DMFQ_GEMV_TRACE) record the 100 MHz clock per wave at start / activations staged / each item
-// computed / end into mfq_trace_ptr[wave_global * 8 + slot].
-#ifdef MFQ_GEMV_TRACE
-__device__ long long *mfq_trace_ptr;
-// the readings stay in registers until the wave is done, so that no store sits among the loads being timed
-#define MFQ_TRACE_DECL long long trace_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#ifndef MFQ_TRACE_CLOCK
-#define MFQ_TRACE_CLOCK() __builtin_readcyclecounter()
-#endif
-#define MFQ_TRACE(slot) trace_t[slot] = MFQ_TRACE_CLOCK()
-#define MFQ_TRACE_FLUSH                                                                                             \
-    do {                                                                                                            \
-        if (mfq_trace_ptr && lane == 0)                                                                             \
-            for (int i_ = 0; i_ < 8; ++i_)                                                                          \
-                mfq_trace_ptr[(static_cast<size_t>(blockIdx.x) * (blockDim.x >> 6) + wave) * 8 + i_] = trace_t[i_]; \
-    } while (0)
-#else
-#define MFQ_TRACE_DECL
-#define MFQ_TRACE(slot) do { } while (0)
-#define MFQ_TRACE_FLUSH do { } while (0)
-#endif
-
 template <class U, int XF16, int MB, bool RING = true, bool FLUSH = true, class XP = NoXPre>
 __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__restrict__ w, int rb0, int rbw,
                                                int row_base, int out_rows, const uint16_t *const (&xr)[MB],
@@ -481,8 +459,6 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     float *red = reinterpret_cast<float *>(lds + nwaves * (MB * (npairs + 2 * ngl)));
     const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes) * rb_step;
 
-    MFQ_TRACE_DECL
-    MFQ_TRACE(0);
     XRegs<MB> xg;
     stage_x_issue<MB>(xr, k.neuron_len, s0 * 16 * GS, npairs, lane, xg);
     xp.template issue<MB>(k.neuron_len, s0 * 16 * GS, npairs, lane);
@@ -515,7 +491,6 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
     xp.template finish<XF16, MB>(xg);
     stage_x<XF16, MB, typename U::Bias, true>(xr, k.neuron_len, s0 * 16 * GS, npairs, GS, ngl, xs, xsum, lane, xg, xinv);
 
-    MFQ_TRACE(1);
     float accS[MB], accM[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) accS[m] = accM[m] = 0.f;
@@ -546,11 +521,8 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
         }
     } else if constexpr (!RING) {  // at most 3 items: everything is already requested
         MFQ_COMPUTE(q0, t0, c0)
-        MFQ_TRACE(2);
         if (items > 1) MFQ_COMPUTE(q1, t1, c1)
-        MFQ_TRACE(3);
         if (items > 2) MFQ_COMPUTE(q2, t2, c2)
-        MFQ_TRACE(4);
     } else {
         uint32_t q3[4][D], t3;
         u32x2_t c3;
@@ -568,8 +540,6 @@ __device__ __forceinline__ void nint_unit_body(const NintK &k, const uint8_t *__
 #undef MFQ_ISSUE
 #undef MFQ_COMPUTE
     if constexpr (FLUSH) flush_rows<MB>(red, nwaves, nrb, rb0, row_base, out_rows, yr);
-    MFQ_TRACE(5);
-    MFQ_TRACE_FLUSH;
 }
 
 // The same block decomposition for waves with at most three items and activations in registers (see XItem): no LDS
@@ -590,8 +560,6 @@ __device__ __forceinline__ void nint_unit_body_xreg(const NintK &k, const uint8_
     const uint32_t sb = static_cast<uint32_t>(k.step_bytes), rbb = static_cast<uint32_t>(k.rowblock_bytes) * rb_step;
     const int items = n > 0 ? nrb * n : 0;  // <= 3
 
-    MFQ_TRACE_DECL
-    MFQ_TRACE(0);
     // item t = (row-block t / n, step t % n); requests in order of use: activations, anchors, weights
     __amdgpu_buffer_rsrc_t wx[MB];
 #pragma unroll
@@ -638,7 +606,6 @@ __device__ __forceinline__ void nint_unit_body_xreg(const NintK &k, const uint8_
             xs_[m] = slice_scale(wave_max_u32(mx), xinv[m]);
         }
     }
-    MFQ_TRACE(1);
     float accS[MB], accM[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) accS[m] = accM[m] = 0.f;
@@ -672,12 +639,9 @@ __device__ __forceinline__ void nint_unit_body_xreg(const NintK &k, const uint8_
                     park_rows<MB>(v, red, irb_[t] * nwaves + wave, lane);
                 }
             }
-            MFQ_TRACE(2 + t);
         }
     }
     if constexpr (FLUSH) flush_rows<MB>(red, nwaves, nrb, rb0, row_base, out_rows, yr);
-    MFQ_TRACE(5);
-    MFQ_TRACE_FLUSH;
 }
 
 template <int BITS, int GS, int XF16, int MB, bool RING = true>
