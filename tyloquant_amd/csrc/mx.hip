@@ -630,7 +630,7 @@ static int mx_tile_max_m() {
 static bool mx_tile_eligible(const MxK &k, const void *x, int64_t ldx) {
     static const int off = tune_env("MFQ_MX_TILE_OFF", 0);
     const int64_t row_bytes = k.kind == 4 ? k.cols / 2 : k.cols;
-    return !off && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && ldx % 8 == 0 && (31 * ldx + k.cols) * 2 < (1ll << 32) &&
+    return !off && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && ldx % 8 == 0 && (31 * ldx + k.cols) * 2 < (1ll << 31) &&
            (reinterpret_cast<uintptr_t>(k.values) & 15) == 0 && 64 * row_bytes < (1ll << 31) &&
            static_cast<int64_t>(k.rows) * (k.cols / 32) < (1ll << 31);
 }

@@ -365,6 +365,222 @@ __global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *
     }
 }
 
+// ---- the 256-entry E8 codebooks (NVQ2, NVQ2J; parity or index-parity signs): one to eight rows per pass -------------
+// The generic kernel above asks for every field of every block by itself -- a few bytes per request, some fifty requests
+// per kilobyte of payload, where a compute unit keeps about 64 in flight -- and decodes a weight at a time.  Here a wave
+// copies the three stream ranges of its neurons (consecutive neurons: consecutive bits) into LDS in 16-byte pieces, one
+// to three requests per range, and a lane takes a group of 24 weights at a time: its 4-bit state, 21 sign bits and
+// three index bytes are funnel shifts over aligned LDS dwords; a block of eight weights is one 16-byte read of the
+// entry out of a table of the activations' type (bf16 or fp16: the int8 magnitudes are exact in both), one 16-byte read
+// of the eight sign bits' XOR pattern, four XORs and four packed dot products against the row's 16 bytes in LDS;
+// the group's scale multiplies the sum of its 24 products in fp32.  bf16 activations are used as they are
+// (v_dot2c_f32_bf16): no conversion and no range to mind.
+// LDS: [entries: banks * 256 * 16][sign patterns: 256 * 16][states: 16 x {anchor-free scale f32, entry base}]
+//      [rows: MB * kp * 2][per wave: index | sign | state ranges]
+template <int XF16>
+__device__ __forceinline__ float e8_dot8(u32x4_t wv, u32x4_t xv, float acc) {
+    // (the elements go through dot2's by-value parameters: a bit cast applied to a vector element directly reads element 0)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc = dot2<XF16>(wv[t], xv[t], acc);
+    return acc;
+}
+// int8 pair -> pair of the activations' type (exact)
+template <int XF16>
+__device__ __forceinline__ uint32_t e8_pair(int a, int b) {
+    if constexpr (XF16) {
+        return static_cast<uint32_t>(f32_to_f16_rne(static_cast<float>(a))) | (static_cast<uint32_t>(f32_to_f16_rne(static_cast<float>(b))) << 16);
+    } else {
+        return (__float_as_uint(static_cast<float>(a)) >> 16) | (__float_as_uint(static_cast<float>(b)) & 0xffff0000u);
+    }
+}
+constexpr int kE8Waves = 16;
+struct E8Shape {
+    int npw;            // consecutive neurons per wave
+    int kp;             // staged elements of a row: whole groups of 24
+    uint32_t cap[3];    // LDS bytes of a wave's index / sign / state range
+    uint32_t wave_bytes, lds_bytes;
+};
+template <int XF16, int MB>
+__global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const uint8_t *__restrict__ w_in,
+                                                                const uint16_t *__restrict__ x_in, int64_t ldx, int M_in,
+                                                                float *__restrict__ y_in, int64_t ldy, E8Shape sh, PairSel sel) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds32[];
+    typedef __attribute__((address_space(3))) const u32x4_t *lds_u32x4_ptr;
+    typedef __attribute__((address_space(3))) const u32x2_t *lds_u32x2_ptr;
+    typedef __attribute__((address_space(3))) const uint32_t *lds_u32_ptr;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint8_t *w = w_in;
+    const uint16_t *x = x_in;
+    float *y = y_in;
+    int M = M_in, m0 = static_cast<int>(blockIdx.y) * MB;
+    if (sel.ids) {
+        const uint16_t *xr[1];
+        float *yr[1];
+        int local;
+        if (!select_rows<1>(sel, w, local, x_in, ldx, y_in, ldy, M_in, xr, yr)) return;
+        if (!sel.weights) k.row0 = local * k.nrows;
+        x = xr[0];
+        y = yr[0];
+        M = 1;
+        m0 = 0;
+    }
+    const int ncb = k.banks * 256;
+    uint8_t *lds8 = reinterpret_cast<uint8_t *>(lds32);
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)lds8));
+    const uint32_t sgn_off = static_cast<uint32_t>(ncb) * 16u, stab_off = sgn_off + 4096u, x_off = stab_off + 128u;
+    const uint32_t row_bytes = static_cast<uint32_t>(sh.kp) * 2u;
+    const uint32_t wave_off = x_off + MB * row_bytes + static_cast<uint32_t>(wave) * sh.wave_bytes;
+
+    // ---- the wave's stream ranges: requested first, parked after the tables are written ----------------------------------
+    const int row_first = (static_cast<int>(blockIdx.x) * kE8Waves + wave) * sh.npw;  // of the launch's rows
+    const int nn = max(0, min(sh.npw, k.nrows - row_first));
+    const int64_t n0 = k.row0 + row_first;
+    // bit ranges [n0 * per, (n0 + nn) * per) of the three streams, read from 16-byte aligned addresses
+    const int64_t bit0[3] = {n0 * k.nvec * 8, n0 * k.nsign * 7, n0 * k.ng * 4};
+    const int64_t region[3] = {k.index_off, k.sign_off, k.state_off};
+    const int64_t region_bytes[3] = {k.index_bytes + 4, k.sign_bytes + 4, k.state_bytes + 4};
+    uint32_t shift[3];   // bits between the staged range's first bit and the first bit of neuron n0
+    u32x4_t piece[3][2];
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+        const int64_t a0 = (bit0[r] >> 3) & ~static_cast<int64_t>(15);
+        shift[r] = static_cast<uint32_t>(bit0[r] - a0 * 8);
+        // bytes of the region from a0 on.  A wave past the launch's last neuron has none: its window must be empty, not a
+        // negative length wrapped to 4 GiB, inside which the "no data" offset would be a real address
+        const int64_t left = nn > 0 ? region_bytes[r] - a0 : 0;
+        const __amdgpu_buffer_rsrc_t win = wave_window(w + region[r] + (nn > 0 ? a0 : 0),
+                                                       static_cast<uint32_t>(left <= 0 ? 0 : (left < (1ll << 31) ? left : (1ll << 31))));
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint32_t off = static_cast<uint32_t>(t * 64 + lane) * 16u;
+            piece[r][t] = __builtin_amdgcn_raw_buffer_load_b128(win, nn > 0 && off < sh.cap[r] ? off : kNoStep, 0, 2);
+        }
+    }
+    // ---- tables and rows (all waves): every request first, then the conversions and the LDS writes ----------------------
+    const float *lut = nvqs_lut(k, w);
+    const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+    const int8_t *cbp = reinterpret_cast<const int8_t *>(bfs + 16);
+    const int chunks = sh.kp / 8;
+    const bool vec = ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    auto x_chunk = [&](int c) -> u32x4_t {  // chunk c = (row, 8 elements) of the staged rows, zeros past M and K
+        const int m = c / chunks, j = c - m * chunks;
+        u32x4_t v = {0u, 0u, 0u, 0u};
+        if (c < MB * chunks && m0 + m < M) {
+            const uint16_t *xr = x + static_cast<int64_t>(m0 + m) * ldx + j * 8;
+            if (vec && j * 8 + 8 <= k.neuron_len) {
+                v = *reinterpret_cast<const u32x4_t *>(xr);
+            } else {
+                uint32_t h[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = j * 8 + i < k.neuron_len ? xr[i] : 0u;
+                v = u32x4_t{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+            }
+        }
+        return v;
+    };
+    auto x_park = [&](int c, u32x4_t v) {
+        const int m = c / chunks, j = c - m * chunks;
+        if (c < MB * chunks)
+            *reinterpret_cast<u32x4_t *>(lds8 + x_off + static_cast<uint32_t>(m) * row_bytes + static_cast<uint32_t>(j) * 16u) = v;
+    };
+    auto entry_park = [&](int e, u32x2_t raw) {
+        u32x4_t v;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t src = t < 2 ? raw.x : raw.y;
+            const int a = static_cast<int8_t>((src >> (16 * (t & 1))) & 0xffu), b = static_cast<int8_t>((src >> (16 * (t & 1) + 8)) & 0xffu);
+            v[t] = e8_pair<XF16>(a, b);
+        }
+        *reinterpret_cast<u32x4_t *>(lds8 + static_cast<uint32_t>(e) * 16u) = v;
+    };
+    // the first entry and the first two chunks of every thread, and the state tables, are requested together
+    const u32x2_t raw0 = tid < ncb ? *reinterpret_cast<const u32x2_t *>(cbp + static_cast<int64_t>(tid) * 8) : u32x2_t{0u, 0u};
+    const u32x4_t xc0 = x_chunk(tid), xc1 = x_chunk(tid + static_cast<int>(blockDim.x));
+    const float lutv = tid < 16 ? lut[tid] : 0.f;
+    const uint32_t bfsv = tid < 16 ? bfs[tid] : 0u;
+    if (tid < ncb) entry_park(tid, raw0);
+    for (int e = tid + blockDim.x; e < ncb; e += blockDim.x) entry_park(e, *reinterpret_cast<const u32x2_t *>(cbp + static_cast<int64_t>(e) * 8));
+    for (int e = tid; e < 256; e += blockDim.x) {
+        u32x4_t v;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) v[t] = (((e >> (2 * t)) & 1u) << 15) | (((e >> (2 * t + 1)) & 1u) << 31);
+        *reinterpret_cast<u32x4_t *>(lds8 + sgn_off + static_cast<uint32_t>(e) * 16u) = v;
+    }
+    if (tid < 16) {
+        float *st = reinterpret_cast<float *>(lds8 + stab_off);
+        st[2 * tid] = lutv;
+        reinterpret_cast<uint32_t *>(st)[2 * tid + 1] = lds_base + bfsv * 4096u;
+    }
+    x_park(tid, xc0);
+    x_park(tid + static_cast<int>(blockDim.x), xc1);
+    for (int c = tid + 2 * static_cast<int>(blockDim.x); c < MB * chunks; c += blockDim.x) x_park(c, x_chunk(c));
+    uint32_t roff[3];  // LDS byte offsets of the wave's three ranges
+    roff[0] = wave_off;
+    roff[1] = roff[0] + sh.cap[0];
+    roff[2] = roff[1] + sh.cap[1];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint32_t off = static_cast<uint32_t>(t * 64 + lane) * 16u;
+            if (off < sh.cap[r]) *reinterpret_cast<u32x4_t *>(lds8 + roff[r] + off) = piece[r][t];
+        }
+    __syncthreads();
+    // `nbits` (<= 25) bits at bit position `bit` of the range at LDS address `base`
+    auto field = [&](uint32_t base, uint32_t bit, uint32_t nbits) -> uint32_t {
+        const u32x2_t d = u32x2_t{*reinterpret_cast<lds_u32_ptr>(base + ((bit >> 5) << 2)), *reinterpret_cast<lds_u32_ptr>(base + ((bit >> 5) << 2) + 4u)};
+        return __builtin_amdgcn_alignbit(d.y, d.x, bit & 31u) & ((1u << nbits) - 1u);
+    };
+    const float *anchors = reinterpret_cast<const float *>(w + k.anchors_off);
+    for (int j = 0; j < nn; ++j) {
+        float acc[MB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[m] = 0.f;
+        const uint32_t ib = shift[0] + static_cast<uint32_t>(j) * k.nvec * 8u, sb0 = shift[1] + static_cast<uint32_t>(j) * k.nsign * 7u,
+                       tb = shift[2] + static_cast<uint32_t>(j) * k.ng * 4u;
+        for (int g = lane; g < k.ng; g += 64) {
+            const uint32_t state = field(lds_base + roff[2], tb + 4u * g, 4);
+            const uint32_t idx3 = field(lds_base + roff[0], ib + 24u * g, 24);
+            const uint32_t mask3 = field(lds_base + roff[1], sb0 + 21u * g, 21);
+            const u32x2_t se = *reinterpret_cast<lds_u32x2_ptr>(lds_base + stab_off + state * 8u);
+            float part[MB];
+#pragma unroll
+            for (int m = 0; m < MB; ++m) part[m] = 0.f;
+            // (no test for blocks past K in the last group: whatever entry and signs their bits name meets staged zeros)
+            u32x4_t wv[3];
+#pragma unroll
+            for (int b = 0; b < 3; ++b) {
+                const uint32_t idx = (idx3 >> (8 * b)) & 255u, mk = (mask3 >> (7 * b)) & 127u;
+                uint32_t last = __popc(mk) & 1u;
+                if (k.index_parity) last ^= idx >> 7;
+                const uint32_t neg = mk | (last << 7);
+                const u32x4_t ev = *reinterpret_cast<lds_u32x4_ptr>(se.y + idx * 16u);
+                const u32x4_t sv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + sgn_off + neg * 16u);
+                wv[b] = ev ^ sv;
+            }
+#pragma unroll
+            for (int m = 0; m < MB; ++m)
+#pragma unroll
+                for (int b = 0; b < 3; ++b) {
+                    const u32x4_t xv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + x_off + static_cast<uint32_t>(m) * row_bytes + static_cast<uint32_t>(3 * g + b) * 16u);
+                    part[m] = e8_dot8<XF16>(wv[b], xv, part[m]);
+                }
+            const float sc = __uint_as_float(se.x);
+#pragma unroll
+            for (int m = 0; m < MB; ++m) acc[m] = fmaf(sc, part[m], acc[m]);
+        }
+        const float anchor = anchors[n0 + j];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+            float v = acc[m];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+            if (lane == 0 && m0 + m < M) y[static_cast<int64_t>(m0 + m) * ldy + row_first + j] = v * anchor;
+        }
+    }
+}
+
 int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, const float *sa,
                 const float *sb, float *y, int64_t ldy, hipStream_t st, float *part = nullptr);
 float *dequant_gemm_part(float *wscale, int N, int K, int M);
@@ -374,6 +590,48 @@ void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&x
                         int &Kp);
 
 constexpr int kNvqsGemvMaxM = 16;  // rows up to which the weights are re-read per pass of eight rows
+
+// The E8 kernel takes the sign-stream format with 8-dimensional vectors, 256 entries per bank (index bytes), 4-bit
+// states and at most four banks, tensors whose streams fit 32-bit offsets and neurons of at most about 16000 weights (a
+// wave's index range is two 1 KB requests at most).  MB = rows per pass that fit the LDS.
+static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
+    static const int off = tune_env("MFQ_NVQS_E8_OFF", 0);
+    if (off || k.kind != 0 || k.vs != 8 || k.ib != 8 || k.entries != 256 || k.sbits != 4 || k.banks > 4 ||
+        k.index_bytes >= (1ll << 31) || k.sign_bytes >= (1ll << 31))
+        return false;
+    auto cap = [](int64_t bits) { return static_cast<uint32_t>((16 + (bits + 7) / 8 + 8 + 15) / 16 * 16); };
+    int npw = static_cast<int>(ceil_div(k.nrows, static_cast<int64_t>(gemv_cu_count()) * kE8Waves));
+    if (npw > 4) npw = 4;
+    while (npw > 1 && cap(static_cast<int64_t>(npw) * k.nvec * 8) > 2048) --npw;
+    if (cap(static_cast<int64_t>(npw) * k.nvec * 8) > 2048) return false;
+    sh.npw = npw;
+    sh.kp = k.ng * 24;
+    sh.cap[0] = cap(static_cast<int64_t>(npw) * k.nvec * 8);
+    sh.cap[1] = cap(static_cast<int64_t>(npw) * k.nsign * 7);
+    sh.cap[2] = cap(static_cast<int64_t>(npw) * k.ng * 4);
+    sh.wave_bytes = sh.cap[0] + sh.cap[1] + sh.cap[2];
+    for (mb = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1)); mb >= 1; mb >>= 1) {
+        sh.lds_bytes = static_cast<uint32_t>(k.banks) * 4096u + 4096u + 128u + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
+        if (sh.lds_bytes <= kMaxDynamicLds) return true;
+    }
+    return false;
+}
+template <int XF16>
+static int nvqs_launch_e8(const NvqsK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy, int mb,
+                          const E8Shape &sh, const PairSel &sel, int n_pairs, hipStream_t st) {
+    const dim3 grid(static_cast<unsigned>(ceil_div(k.nrows, static_cast<int64_t>(kE8Waves) * sh.npw)),
+                    static_cast<unsigned>(n_pairs ? n_pairs : ceil_div(M, mb)));
+#define MFQ_E8(MBV)                                                                                                   \
+    if (mb == MBV) {                                                                                                  \
+        auto kern = nvqs_e8_kernel<XF16, MBV>;                                                                        \
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), sh.lds_bytes, "nvqs_e8")) return rc;     \
+        hipLaunchKernelGGL(kern, grid, dim3(64 * kE8Waves), sh.lds_bytes, st, k, w, x, ldx, M, y, ldy, sh, sel);       \
+        return check_launch("nvqs_e8");                                                                               \
+    }
+    MFQ_E8(1) MFQ_E8(2) MFQ_E8(4) MFQ_E8(8)
+#undef MFQ_E8
+    return fail(MFQ_ERR_UNSUPPORTED, "nvqs_e8: %d rows per pass", mb);
+}
 
 template <int XF16, int MB>
 static int nvqs_launch_gemv(const NvqsK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
@@ -588,6 +846,13 @@ extern "C" int mfq_hip_nvqs_gemv_pairs(const mfq_nvqs_desc *d, const void *const
     k.nrows = out_per_expert;
     const uint16_t *xp = static_cast<const uint16_t *>(x);
     const uint8_t *w = static_cast<const uint8_t *>(weight);
+    {
+        int mb;
+        E8Shape sh;
+        if (nvqs_e8_shape(k, 1, mb, sh))
+            return x_dtype == MFQ_X_F16 ? nvqs_launch_e8<1>(k, w, xp, ldx, T * R, y, ldy, 1, sh, sel, T * R, as_stream(stream))
+                                        : nvqs_launch_e8<0>(k, w, xp, ldx, T * R, y, ldy, 1, sh, sel, T * R, as_stream(stream));
+    }
     return x_dtype == MFQ_X_F16 ? nvqs_launch_pairs<1>(k, w, xp, ldx, T * R, y, ldy, sel, as_stream(stream))
                                 : nvqs_launch_pairs<0>(k, w, xp, ldx, T * R, y, ldy, sel, as_stream(stream));
 }
@@ -632,6 +897,13 @@ extern "C" int mfq_hip_nvqs_gemv_rows(const mfq_nvqs_desc *d, const void *weight
     const uint8_t *w = static_cast<const uint8_t *>(weight);
     const uint16_t *xp = static_cast<const uint16_t *>(x);
     hipStream_t st = as_stream(stream);
+    {
+        int mb;
+        E8Shape sh;
+        if (nvqs_e8_shape(k, M, mb, sh))
+            return x_dtype == MFQ_X_F16 ? nvqs_launch_e8<1>(k, w, xp, ldx, M, y, ldy, mb, sh, PairSel{}, 0, st)
+                                        : nvqs_launch_e8<0>(k, w, xp, ldx, M, y, ldy, mb, sh, PairSel{}, 0, st);
+    }
     if (x_dtype == MFQ_X_F16) {
         if (M == 1) return nvqs_launch_gemv<1, 1>(k, w, xp, ldx, M, y, ldy, st);
         if (M <= 4) return nvqs_launch_gemv<1, 4>(k, w, xp, ldx, M, y, ldy, st);
