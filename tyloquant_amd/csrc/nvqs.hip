@@ -365,7 +365,7 @@ __global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *
     }
 }
 
-// ---- the 256-entry E8 codebooks (NVQ2, NVQ2J; parity or index-parity signs): one to eight rows per pass -------------
+// ---- the E8 codebooks whose tables fit the LDS (NVQ2, NVQ2J, NVQ2J-L, one bank of NVQ2J-XL): one to eight rows per pass
 // The generic kernel above asks for every field of every block by itself -- a few bytes per request, some fifty requests
 // per kilobyte of payload, where a compute unit keeps about 64 in flight -- and decodes a weight at a time.  Here a wave
 // copies the three stream ranges of its neurons (consecutive neurons: consecutive bits) into LDS in 16-byte pieces, one
@@ -375,7 +375,7 @@ __global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *
 // of the eight sign bits' XOR pattern, four XORs and four packed dot products against the row's 16 bytes in LDS;
 // the group's scale multiplies the sum of its 24 products in fp32.  bf16 activations are used as they are
 // (v_dot2c_f32_bf16): no conversion and no range to mind.
-// LDS: [entries: banks * 256 * 16][sign patterns: 256 * 16][states: 16 x {anchor-free scale f32, entry base}]
+// LDS: [entries: banks * entries * 16][sign patterns: 256 * 16][states: 16 x {anchor-free scale f32, entry base}]
 //      [rows: MB * kp * 2][per wave: index | sign | state ranges]
 template <int XF16>
 __device__ __forceinline__ float e8_dot8(u32x4_t wv, u32x4_t xv, float acc) {
@@ -425,7 +425,7 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
         M = 1;
         m0 = 0;
     }
-    const int ncb = k.banks * 256;
+    const int ncb = k.banks * k.entries;
     uint8_t *lds8 = reinterpret_cast<uint8_t *>(lds32);
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)lds8));
     const uint32_t sgn_off = static_cast<uint32_t>(ncb) * 16u, stab_off = sgn_off + 4096u, x_off = stab_off + 128u;
@@ -437,7 +437,7 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
     const int nn = max(0, min(sh.npw, k.nrows - row_first));
     const int64_t n0 = k.row0 + row_first;
     // bit ranges [n0 * per, (n0 + nn) * per) of the three streams, read from 16-byte aligned addresses
-    const int64_t bit0[3] = {n0 * k.nvec * 8, n0 * k.nsign * 7, n0 * k.ng * 4};
+    const int64_t bit0[3] = {n0 * k.nvec * k.ib, n0 * k.nsign * 7, n0 * k.ng * 4};
     const int64_t region[3] = {k.index_off, k.sign_off, k.state_off};
     const int64_t region_bytes[3] = {k.index_bytes + 4, k.sign_bytes + 4, k.state_bytes + 4};
     uint32_t shift[3];   // bits between the staged range's first bit and the first bit of neuron n0
@@ -510,7 +510,7 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
     if (tid < 16) {
         float *st = reinterpret_cast<float *>(lds8 + stab_off);
         st[2 * tid] = lutv;
-        reinterpret_cast<uint32_t *>(st)[2 * tid + 1] = lds_base + bfsv * 4096u;
+        reinterpret_cast<uint32_t *>(st)[2 * tid + 1] = lds_base + bfsv * static_cast<uint32_t>(k.entries) * 16u;
     }
     x_park(tid, xc0);
     x_park(tid + static_cast<int>(blockDim.x), xc1);
@@ -537,11 +537,19 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
         float acc[MB];
 #pragma unroll
         for (int m = 0; m < MB; ++m) acc[m] = 0.f;
-        const uint32_t ib = shift[0] + static_cast<uint32_t>(j) * k.nvec * 8u, sb0 = shift[1] + static_cast<uint32_t>(j) * k.nsign * 7u,
+        const uint32_t ib = shift[0] + static_cast<uint32_t>(j) * k.nvec * k.ib, sb0 = shift[1] + static_cast<uint32_t>(j) * k.nsign * 7u,
                        tb = shift[2] + static_cast<uint32_t>(j) * k.ng * 4u;
         for (int g = lane; g < k.ng; g += 64) {
             const uint32_t state = field(lds_base + roff[2], tb + 4u * g, 4);
-            const uint32_t idx3 = field(lds_base + roff[0], ib + 24u * g, 24);
+            // the three indices of the group: one 24-bit field of index bytes, or three fields of 10 or 12 bits
+            uint32_t ix[3];
+            if (k.ib == 8) {
+                const uint32_t idx3 = field(lds_base + roff[0], ib + 24u * g, 24);
+                ix[0] = idx3 & 255u; ix[1] = (idx3 >> 8) & 255u; ix[2] = idx3 >> 16;
+            } else {
+#pragma unroll
+                for (int b = 0; b < 3; ++b) ix[b] = field(lds_base + roff[0], ib + static_cast<uint32_t>(3 * g + b) * k.ib, k.ib);
+            }
             const uint32_t mask3 = field(lds_base + roff[1], sb0 + 21u * g, 21);
             const u32x2_t se = *reinterpret_cast<lds_u32x2_ptr>(lds_base + stab_off + state * 8u);
             float part[MB];
@@ -551,7 +559,7 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
             u32x4_t wv[3];
 #pragma unroll
             for (int b = 0; b < 3; ++b) {
-                const uint32_t idx = (idx3 >> (8 * b)) & 255u, mk = (mask3 >> (7 * b)) & 127u;
+                const uint32_t idx = ix[b], mk = (mask3 >> (7 * b)) & 127u;
                 uint32_t last = __popc(mk) & 1u;
                 if (k.index_parity) last ^= idx >> 7;
                 const uint32_t neg = mk | (last << 7);
@@ -591,27 +599,28 @@ void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&x
 
 constexpr int kNvqsGemvMaxM = 16;  // rows up to which the weights are re-read per pass of eight rows
 
-// The E8 kernel takes the sign-stream format with 8-dimensional vectors, 256 entries per bank (index bytes), 4-bit
-// states and at most four banks, tensors whose streams fit 32-bit offsets and neurons of at most about 16000 weights (a
-// wave's index range is two 1 KB requests at most).  MB = rows per pass that fit the LDS.
+// The E8 kernel takes the sign-stream format with 8-dimensional vectors, 4-bit states and tables that fit the LDS as
+// 16-byte entries (256 or 1024 entries in up to four banks, 4096 in one), tensors whose streams fit 32-bit offsets and
+// neurons of at most about 16000 weights with index bytes, 10000 with 12-bit indices (a wave's index range is two 1 KB
+// requests at most).  MB = rows per pass that fit the LDS.
 static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     static const int off = tune_env("MFQ_NVQS_E8_OFF", 0);
-    if (off || k.kind != 0 || k.vs != 8 || k.ib != 8 || k.entries != 256 || k.sbits != 4 || k.banks > 4 ||
+    if (off || k.kind != 0 || k.vs != 8 || k.ib < 8 || k.ib > 12 || k.entries != (1 << k.ib) || k.sbits != 4 || k.banks > 4 ||
         k.index_bytes >= (1ll << 31) || k.sign_bytes >= (1ll << 31))
         return false;
     auto cap = [](int64_t bits) { return static_cast<uint32_t>((16 + (bits + 7) / 8 + 8 + 15) / 16 * 16); };
     int npw = static_cast<int>(ceil_div(k.nrows, static_cast<int64_t>(gemv_cu_count()) * kE8Waves));
     if (npw > 4) npw = 4;
-    while (npw > 1 && cap(static_cast<int64_t>(npw) * k.nvec * 8) > 2048) --npw;
-    if (cap(static_cast<int64_t>(npw) * k.nvec * 8) > 2048) return false;
+    while (npw > 1 && cap(static_cast<int64_t>(npw) * k.nvec * k.ib) > 2048) --npw;
+    if (cap(static_cast<int64_t>(npw) * k.nvec * k.ib) > 2048) return false;
     sh.npw = npw;
     sh.kp = k.ng * 24;
-    sh.cap[0] = cap(static_cast<int64_t>(npw) * k.nvec * 8);
+    sh.cap[0] = cap(static_cast<int64_t>(npw) * k.nvec * k.ib);
     sh.cap[1] = cap(static_cast<int64_t>(npw) * k.nsign * 7);
     sh.cap[2] = cap(static_cast<int64_t>(npw) * k.ng * 4);
     sh.wave_bytes = sh.cap[0] + sh.cap[1] + sh.cap[2];
     for (mb = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1)); mb >= 1; mb >>= 1) {
-        sh.lds_bytes = static_cast<uint32_t>(k.banks) * 4096u + 4096u + 128u + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
+        sh.lds_bytes = static_cast<uint32_t>(k.banks) * static_cast<uint32_t>(k.entries) * 16u + 4096u + 128u + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
         if (sh.lds_bytes <= kMaxDynamicLds) return true;
     }
     return false;

@@ -48,7 +48,7 @@ Knob g_knobs[] = {
     {"MFQ_MOE_PREFILL_PAIRS", "pairs per expert from which mapped MoE calls take the prefill kernel (0 = default)", 0, false},
     {"MFQ_FFN_SPIN_LIMIT", "polls after which the one-launch FFN's grid barrier gives up", 0, false},
     {"MFQ_FFN_TRACE", "1 = the one-launch FFN records per-block clocks behind its workspace", 0, false},
-    {"MFQ_NVQS_E8_OFF", "1 = the 256-entry E8 formats (NVQ2, NVQ2J) on the generic stream kernel", 0, false},
+    {"MFQ_NVQS_E8_OFF", "1 = the E8 formats on the generic stream kernel", 0, false},
     {"MFQ_MX_TILE_OFF", "1 = MXFP4 / MXFP8 small batches on the wave-per-neuron kernel instead of the matrix-core tile kernel", 0, false},
     {"MFQ_MX_STAGE_OFF", "1 = the MX tile kernel never stages a wave's activation slice and scales in LDS", 0, false},
     {"MFQ_MX_STAGE_MAX_M", "rows up to which MX matmuls run as 16-row tiles with the activations staged in LDS (default 48)", 0, false},
