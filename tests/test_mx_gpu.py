@@ -78,6 +78,23 @@ def test_mx_matrix_core_tiles(dtype, rows, cols):
     check_close(lin(odd).cpu().numpy(), O.linear_forward_f64(want, odd.float().cpu().numpy()))
 
 
+@pytest.mark.parametrize("cus", [1, 2, 3, 5])
+@pytest.mark.parametrize("dtype,rows,cols", [("MXFP4", 200, 2880), ("MXFP4", 272, 512), ("MXFP8", 384, 640)])
+def test_mx_tiles_with_several_row_blocks_per_block(cu_count, cus, dtype, rows, cols):
+    """Blocks of two to four row-blocks (the shapes a large tensor gets) on small tensors: the grid is sized for a few
+    compute units, which makes the launcher share the staged rows between row-blocks -- whole and partial last blocks,
+    one tile, several staged tiles and the 32-row tiles."""
+    from tyloquant_amd import runtime as R
+    rng = np.random.default_rng(rows + cols + cus)
+    t = synth.mx_random(rng, dtype, rows, cols)
+    lin = R.load_quant_linear(dtype, O.pack_mx(t))
+    want = O.dequantize_mx(t)
+    cu_count(cus)
+    for M, xdt in ((1, torch.bfloat16), (6, torch.bfloat16), (16, torch.float16), (40, torch.bfloat16), (90, torch.bfloat16)):
+        x = torch.from_numpy(rng.standard_normal((M, cols)).astype(np.float32)).to(xdt).cuda()
+        check_close(lin(x).cpu().numpy(), O.linear_forward_f64(want, x.float().cpu().numpy()))
+
+
 @pytest.mark.parametrize("dtype", ["MXFP4", "MXFP8"])
 def test_mx_scale_bytes_0_and_255_in_the_matmul(dtype):
     """E8M0 0 is 2^-127 and 255 a NaN (mx_matmul.cu:17-28): a neuron whose row holds a NaN scale comes out NaN, the

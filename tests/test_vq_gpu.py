@@ -338,6 +338,27 @@ def test_multi_expert_nepq_blob_is_not_a_linear():
     assert "must hold one expert" in lib.mfq_rt_last_error().decode()
 
 
+@pytest.mark.parametrize("cus", [1, 2])
+@pytest.mark.parametrize("codebook,banks,out,K", [("e8_256", 2, 150, 120), ("e8_1024", 2, 70, 1544), ("e8_4096", 1, 97, 96)])
+def test_e8_kernel_with_several_neurons_per_wave(cu_count, cus, codebook, banks, out, K):
+    """A wave of the E8 kernel walks up to four consecutive neurons of a large tensor; sized for one or two compute
+    units, small tensors take the same shape: neurons whose stream ranges start inside a byte, waves with fewer neurons
+    than the others and waves with none, one to eight rows per pass and both activation types."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import nvq_matmul
+    rng = np.random.default_rng(70 + out + K + cus)
+    t = synth.nvq_jsc_random(rng, out, K, codebook, banks)
+    _, blob = O.pack_tensor(t)
+    lin = R.load_quant_linear(_, blob)
+    want = O.dequantize_nvq_jsc(O.unpack_nvq(blob))
+    cu_count(cus)
+    for M, xd in ((1, torch.bfloat16), (2, torch.float16), (5, torch.bfloat16), (8, torch.float16), (13, torch.bfloat16)):
+        x, xf = _x(rng, M, K, xd)
+        _check(nvq_matmul(lin.weight, x).cpu().numpy(), O.linear_forward_f64(want, xf))
+    big = torch.from_numpy((rng.standard_normal((2, K)) * 2.0e6).astype(np.float32)).to(torch.bfloat16).cuda()
+    _check(nvq_matmul(lin.weight, big).cpu().numpy() / 2.0e6, O.linear_forward_f64(want, big.float().cpu().numpy()) / 2.0e6)
+
+
 @pytest.mark.parametrize("codebook,banks,dtype", [("e8_256", 2, "NVQ2J"), ("e8_256", 4, "NVQ2J"), ("e8_1024", 2, "NVQ2J-L"),
                                                   ("e8_4096", 1, "NVQ2J-XL"), ("e8_4096", 4, "NVQ2J-XL"),
                                                   ("d4_1024", 2, "NVQ3J-L")])
