@@ -352,7 +352,7 @@ int mfq_hip_nvq_gemm(const mfq_nvq_desc *d, const void *weight, const void *x, i
  * NVQ3J-L (d4_1024), whose 10-bit indices do not fit the lane-major D4 layout above.  Group size 24, 4-bit states.
  * The device weight keeps the payload's three tensor-wide streams (4-bit state, index, 7-bit sign) as they are, with
  * the tables widened in front (float lut[16], uint32 bank_for_state[16], int8 codebooks) and fp32 anchors; fields are
- * fetched by bit offset, a wave per neuron (E8 tables of up to 64 KB -- NVQ2, NVQ2J, NVQ2J-L, one-bank NVQ2J-XL: a wave copies its neurons' bit ranges
+ * fetched by bit offset, a wave per neuron (tables of up to 64 KB -- NVQ2, NVQ2J, NVQ2J-L, one-bank NVQ2J-XL, NVQ3J-L: a wave copies its neurons' bit ranges
  * into LDS and multiplies 24 weights per lane and step, the reference's NVQ2 fast path,
  * mfq/kernels/cuda/nvq_matmul.cu:1378-1420).  Replaces the formats 2, 5, 13, 14 and 15 of unpack_nvq / NvqWeight
  * (cpp_runtime/mfq_decode.cpp:3756-4013, 4019-4150) and their nvq_gemv_ws_cuda / nvq_mmq_* / nvq_dequant_cuda calls

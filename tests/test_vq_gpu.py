@@ -339,7 +339,8 @@ def test_multi_expert_nepq_blob_is_not_a_linear():
 
 
 @pytest.mark.parametrize("cus", [1, 2])
-@pytest.mark.parametrize("codebook,banks,out,K", [("e8_256", 2, 150, 120), ("e8_1024", 2, 70, 1544), ("e8_4096", 1, 97, 96)])
+@pytest.mark.parametrize("codebook,banks,out,K", [("e8_256", 2, 150, 120), ("e8_1024", 2, 70, 1544), ("e8_4096", 1, 97, 96),
+                                                  ("d4_1024", 2, 90, 100)])
 def test_e8_kernel_with_several_neurons_per_wave(cu_count, cus, codebook, banks, out, K):
     """A wave of the E8 kernel walks up to four consecutive neurons of a large tensor; sized for one or two compute
     units, small tensors take the same shape: neurons whose stream ranges start inside a byte, waves with fewer neurons

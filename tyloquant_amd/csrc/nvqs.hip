@@ -365,7 +365,8 @@ __global__ __launch_bounds__(256) void nvqs_gemv_kernel(NvqsK k, const uint8_t *
     }
 }
 
-// ---- the E8 codebooks whose tables fit the LDS (NVQ2, NVQ2J, NVQ2J-L, one bank of NVQ2J-XL): one to eight rows per pass
+// ---- the sign-stream codebooks whose tables fit the LDS (E8: NVQ2, NVQ2J, NVQ2J-L, one bank of NVQ2J-XL; D4: NVQ3J-L): one
+// ---- to eight rows per pass
 // The generic kernel above asks for every field of every block by itself -- a few bytes per request, some fifty requests
 // per kilobyte of payload, where a compute unit keeps about 64 in flight -- and decodes a weight at a time.  Here a wave
 // copies the three stream ranges of its neurons (consecutive neurons: consecutive bits) into LDS in 16-byte pieces, one
@@ -428,7 +429,8 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
     const int ncb = k.banks * k.entries;
     uint8_t *lds8 = reinterpret_cast<uint8_t *>(lds32);
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)lds8));
-    const uint32_t sgn_off = static_cast<uint32_t>(ncb) * 16u, stab_off = sgn_off + 4096u, x_off = stab_off + 128u;
+    const uint32_t esz = static_cast<uint32_t>(k.vs) * 2u;  // bytes of a table entry: 8 (E8) or 4 (D4) values of the activations' type
+    const uint32_t sgn_off = static_cast<uint32_t>(ncb) * esz, stab_off = sgn_off + 4096u, x_off = stab_off + 128u;
     const uint32_t row_bytes = static_cast<uint32_t>(sh.kp) * 2u;
     const uint32_t wave_off = x_off + MB * row_bytes + static_cast<uint32_t>(wave) * sh.wave_bytes;
 
@@ -484,6 +486,7 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
         if (c < MB * chunks)
             *reinterpret_cast<u32x4_t *>(lds8 + x_off + static_cast<uint32_t>(m) * row_bytes + static_cast<uint32_t>(j) * 16u) = v;
     };
+    // slot e of the table: eight int8 magnitudes -- one E8 entry, or two consecutive D4 entries
     auto entry_park = [&](int e, u32x2_t raw) {
         u32x4_t v;
 #pragma unroll
@@ -494,13 +497,14 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
         }
         *reinterpret_cast<u32x4_t *>(lds8 + static_cast<uint32_t>(e) * 16u) = v;
     };
-    // the first entry and the first two chunks of every thread, and the state tables, are requested together
-    const u32x2_t raw0 = tid < ncb ? *reinterpret_cast<const u32x2_t *>(cbp + static_cast<int64_t>(tid) * 8) : u32x2_t{0u, 0u};
+    const int nslot = ncb * k.vs / 8;
+    // the first slot and the first two chunks of every thread, and the state tables, are requested together
+    const u32x2_t raw0 = tid < nslot ? *reinterpret_cast<const u32x2_t *>(cbp + static_cast<int64_t>(tid) * 8) : u32x2_t{0u, 0u};
     const u32x4_t xc0 = x_chunk(tid), xc1 = x_chunk(tid + static_cast<int>(blockDim.x));
     const float lutv = tid < 16 ? lut[tid] : 0.f;
     const uint32_t bfsv = tid < 16 ? bfs[tid] : 0u;
-    if (tid < ncb) entry_park(tid, raw0);
-    for (int e = tid + blockDim.x; e < ncb; e += blockDim.x) entry_park(e, *reinterpret_cast<const u32x2_t *>(cbp + static_cast<int64_t>(e) * 8));
+    if (tid < nslot) entry_park(tid, raw0);
+    for (int e = tid + blockDim.x; e < nslot; e += blockDim.x) entry_park(e, *reinterpret_cast<const u32x2_t *>(cbp + static_cast<int64_t>(e) * 8));
     for (int e = tid; e < 256; e += blockDim.x) {
         u32x4_t v;
 #pragma unroll
@@ -510,7 +514,7 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
     if (tid < 16) {
         float *st = reinterpret_cast<float *>(lds8 + stab_off);
         st[2 * tid] = lutv;
-        reinterpret_cast<uint32_t *>(st)[2 * tid + 1] = lds_base + bfsv * static_cast<uint32_t>(k.entries) * 16u;
+        reinterpret_cast<uint32_t *>(st)[2 * tid + 1] = lds_base + bfsv * static_cast<uint32_t>(k.entries) * esz;
     }
     x_park(tid, xc0);
     x_park(tid + static_cast<int>(blockDim.x), xc1);
@@ -541,9 +545,16 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
                        tb = shift[2] + static_cast<uint32_t>(j) * k.ng * 4u;
         for (int g = lane; g < k.ng; g += 64) {
             const uint32_t state = field(lds_base + roff[2], tb + 4u * g, 4);
-            // the three indices of the group: one 24-bit field of index bytes, or three fields of 10 or 12 bits
-            uint32_t ix[3];
-            if (k.ib == 8) {
+            // the indices of the group's three blocks: one 24-bit field of index bytes, three fields of 10 or 12 bits, or
+            // (4-dimensional vectors) two fields per block
+            uint32_t ix[3], ix2[3] = {0u, 0u, 0u};
+            if (k.vs == 4) {
+#pragma unroll
+                for (int b = 0; b < 3; ++b) {
+                    ix[b] = field(lds_base + roff[0], ib + static_cast<uint32_t>(6 * g + 2 * b) * k.ib, k.ib);
+                    ix2[b] = field(lds_base + roff[0], ib + static_cast<uint32_t>(6 * g + 2 * b + 1) * k.ib, k.ib);
+                }
+            } else if (k.ib == 8) {
                 const uint32_t idx3 = field(lds_base + roff[0], ib + 24u * g, 24);
                 ix[0] = idx3 & 255u; ix[1] = (idx3 >> 8) & 255u; ix[2] = idx3 >> 16;
             } else {
@@ -563,7 +574,13 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
                 uint32_t last = __popc(mk) & 1u;
                 if (k.index_parity) last ^= idx >> 7;
                 const uint32_t neg = mk | (last << 7);
-                const u32x4_t ev = *reinterpret_cast<lds_u32x4_ptr>(se.y + idx * 16u);
+                u32x4_t ev;
+                if (k.vs == 4) {
+                    const u32x2_t e0 = *reinterpret_cast<lds_u32x2_ptr>(se.y + idx * 8u), e1 = *reinterpret_cast<lds_u32x2_ptr>(se.y + ix2[b] * 8u);
+                    ev = u32x4_t{e0.x, e0.y, e1.x, e1.y};
+                } else {
+                    ev = *reinterpret_cast<lds_u32x4_ptr>(se.y + idx * 16u);
+                }
                 const u32x4_t sv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + sgn_off + neg * 16u);
                 wv[b] = ev ^ sv;
             }
@@ -599,13 +616,13 @@ void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&x
 
 constexpr int kNvqsGemvMaxM = 16;  // rows up to which the weights are re-read per pass of eight rows
 
-// The E8 kernel takes the sign-stream format with 8-dimensional vectors, 4-bit states and tables that fit the LDS as
-// 16-byte entries (256 or 1024 entries in up to four banks, 4096 in one), tensors whose streams fit 32-bit offsets and
+// The E8 kernel takes the sign-stream format with 8- or 4-dimensional vectors, 4-bit states and tables that fit the LDS
+// in the activations' type (E8: 256 or 1024 entries in up to four banks, 4096 in one; D4: 1024 entries), tensors whose streams fit 32-bit offsets and
 // neurons of at most about 16000 weights with index bytes, 10000 with 12-bit indices (a wave's index range is two 1 KB
 // requests at most).  MB = rows per pass that fit the LDS.
 static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     static const int off = tune_env("MFQ_NVQS_E8_OFF", 0);
-    if (off || k.kind != 0 || k.vs != 8 || k.ib < 8 || k.ib > 12 || k.entries != (1 << k.ib) || k.sbits != 4 || k.banks > 4 ||
+    if (off || k.kind != 0 || (k.vs != 8 && k.vs != 4) || k.ib < 8 || k.ib > 12 || k.entries != (1 << k.ib) || k.sbits != 4 || k.banks > 4 ||
         k.index_bytes >= (1ll << 31) || k.sign_bytes >= (1ll << 31))
         return false;
     auto cap = [](int64_t bits) { return static_cast<uint32_t>((16 + (bits + 7) / 8 + 8 + 15) / 16 * 16); };
@@ -620,7 +637,7 @@ static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     sh.cap[2] = cap(static_cast<int64_t>(npw) * k.ng * 4);
     sh.wave_bytes = sh.cap[0] + sh.cap[1] + sh.cap[2];
     for (mb = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1)); mb >= 1; mb >>= 1) {
-        sh.lds_bytes = static_cast<uint32_t>(k.banks) * static_cast<uint32_t>(k.entries) * 16u + 4096u + 128u + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
+        sh.lds_bytes = static_cast<uint32_t>(k.banks) * static_cast<uint32_t>(k.entries) * static_cast<uint32_t>(k.vs) * 2u + 4096u + 128u + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
         if (sh.lds_bytes <= kMaxDynamicLds) return true;
     }
     return false;
