@@ -14,8 +14,9 @@
  *
  * Range of the activations.  The kernels multiply in fp16 (the reference's activation type).  fp16 rows are used as
  * given.  bf16 rows of any finite magnitude are taken by
- *   - the NINT batch-1 / batch-2 kernels (GEMV, fused GLU, arg-max, MoE decode) and the NINT kernel for 3 to 16 rows that
- *     keeps the activations in LDS (groups of 32 or 16 weights, K of at most eight steps of 16 groups),
+ *   - the NINT batch-1 / batch-2 kernels (GEMV, fused GLU, arg-max, MoE decode; not NINT8-48, whose plain matmul runs on
+ *     the streaming matrix-core kernel from one row on) and the NINT kernel for 3 to 16 rows that keeps the activations
+ *     in LDS (groups of 32 or 16 weights, K of at most eight steps of 16 groups),
  *   - the NVQ3J kernel for one and two rows with its signed table in LDS, the NVQ kernels behind a MoE decode step on an
  *     NVQ cohort (mfq_hip_nvq_gemv_pairs), the NEPQ1 one-row kernel and the NINT8-0 streaming GEMV (one row; more rows when
  *     the activation rows are not 16-byte aligned),

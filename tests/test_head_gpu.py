@@ -4,15 +4,15 @@ import numpy as np
 import pytest
 
 import synth
-from conftest import ABS_TOL, REL_TOL, rel_l2
+from conftest import ABS_TOL, REL_TOL, check_close, rel_l2
 from oracle import mfq_oracle as O
 
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
 
-SPECS = [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (6, 24, 6), (8, 24, 8), (6, 26, 6)]
-FUSED = [(4, 32, 6), (4, 24, 6), (3, 24, 5), (5, 28, 7)]   # one GEMV launch that also emits the blocks' winners
-UNFUSED = [(6, 26, 6), (2, 16, 5)]                          # GEMV into the logits, then two reduction passes
+SPECS = [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (6, 24, 6), (8, 24, 8), (6, 26, 6), (8, 48, 7)]
+FUSED = [(4, 32, 6), (4, 24, 6), (3, 24, 5), (5, 28, 7), (6, 24, 7)]   # one GEMV launch that also emits the blocks' winners
+UNFUSED = [(6, 26, 6), (2, 16, 5), (8, 48, 7)]                          # GEMV into the logits, then two reduction passes
 
 
 def _load(t):
@@ -177,8 +177,7 @@ def test_lm_head_argmax_of_several_rows_and_nan(bits, gs, sb):
     assert token.shape == (1, 5) and logits.shape == (1, 5, out)
     assert torch.equal(token[0], logits[0].argmax(-1))
     ref = O.linear_forward_f64(O.dequantize_nint(t), xf)
-    assert rel_l2(logits[0].cpu().numpy(), ref) < REL_TOL
-    assert np.abs(logits[0].cpu().numpy() - ref).max() < ABS_TOL
+    check_close(logits[0].cpu().numpy(), ref)   # (packed-domain fixture: logits of order 50, the bound scales with their RMS)
     bad = torch.full((1, K), float("nan"), dtype=torch.bfloat16, device="cuda")
     assert int(R.nint_matmul_argmax(lin.weight, bad)[0]) == -1
     bad3 = torch.full((3, K), float("nan"), dtype=torch.bfloat16, device="cuda")

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 # (bits, gs, sub_bits): the production profiles plus odd ones that take the generic unit
 SPECS = [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (6, 24, 6), (8, 24, 8), (4, 16, 6), (4, 48, 6),
-         (6, 26, 6), (2, 32, 5), (5, 16, 5)]
+         (6, 26, 6), (2, 32, 5), (5, 16, 5), (6, 24, 7), (8, 48, 7)]   # the last two: the production NINT6 / NINT8 profiles
 
 
 _rand_tensor = synth.nint_random
@@ -61,7 +61,7 @@ def test_gemv_matches_oracle(bits, gs, sb, M):
 
 
 @pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (4, 16, 6), (4, 48, 6),
-                                        (2, 32, 5), (4, 32, 8)])
+                                        (2, 32, 5), (4, 32, 8), (6, 24, 7), (8, 48, 7)])
 @pytest.mark.parametrize("out,K,M", [(128, 1024, 2), (200, 2056, 16), (80, 4096, 5), (96, 1544, 17), (64, 12288, 40)])
 def test_small_batch_matrix_core_path(bits, gs, sb, out, K, M):
     """Batches of 2..64 rows stream the packed weights once per 16 rows through the MFMA kernel (K % 8 == 0,
@@ -80,7 +80,7 @@ def test_small_batch_matrix_core_path(bits, gs, sb, out, K, M):
         assert np.abs(y - ref).max() < ABS_TOL
 
 
-@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (4, 24, 6)])
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (4, 24, 6), (6, 24, 7), (8, 48, 7)])
 @pytest.mark.parametrize("out,K,M", [(128, 280, 16), (257, 224, 23), (73, 1537, 65), (512, 1024, 257)])
 def test_gemm_matches_oracle(bits, gs, sb, out, K, M):
     from tyloquant_amd import runtime as R
@@ -288,7 +288,8 @@ def test_input_gate_then_matmul(mode, K):
             assert rel_l2(y, ref) < REL_TOL and np.abs(y - ref).max() < ABS_TOL
 
 
-@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (6, 20, 6)])
+@pytest.mark.parametrize("bits,gs,sb", [(4, 32, 6), (4, 24, 6), (3, 24, 5), (2, 16, 5), (5, 28, 7), (6, 20, 6), (6, 24, 7),
+                                        (8, 48, 7)])
 @pytest.mark.parametrize("mode", [0, 1])
 def test_input_gate_inside_the_gemv(bits, gs, sb, mode):
     """One or two rows: the gate is applied by the GEMV's own activation staging (mfq_hip_nint_gemv_gate).  Against the
@@ -311,7 +312,9 @@ def test_input_gate_inside_the_gemv(bits, gs, sb, mode):
                                                     y.data_ptr(), y.stride(0), None)
                 assert rc == 0, L.lib().mfq_hip_last_error()
                 two = R.nint_matmul_input_mul(lin.weight, x, g, mode, fused=False)
-                assert torch.allclose(y, two, rtol=1e-3, atol=1e-4)
+                # (NINT8-48 takes its plain matmul on the matrix cores, where 8-bit code x 7-bit sub-scale is rounded to
+                # fp16's eleven bits: the two forms then agree to that rounding, not to the summation order)
+                assert torch.allclose(y, two, rtol=1e-3, atol=1e-4 if bits < 8 else 2e-3)
                 one = R.nint_matmul_input_mul(lin.weight, x, g, mode)
                 assert torch.equal(one, y)
                 gated = torch.from_numpy(O.input_mul(xf, gf, mode).astype(np.float32)).to(dtype).float().numpy()

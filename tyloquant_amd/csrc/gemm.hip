@@ -435,6 +435,9 @@ static bool nint_streams(const mfq_nint_desc *d, int M) {
         const int m = static_cast<int>(64.0 * tp / t64) / 16 * 16;
         stream_max = m < 32 ? 32 : (m > 512 ? 512 : m);
     }
+    // NINT8-48 streams one row-block per wave (twelve dwords a unit), 16 rows per pass: 12288 x 4096 takes 133 us at 64
+    // rows where the fp16 copy + GEMM takes 335 us at any batch up to a few hundred
+    else if (d->bits == 8) stream_max = 160;
     if (env_max > 0) stream_max = env_max;
     return M <= kGemvMaxM || (M <= stream_max && nint_stream_capable(d));
 }

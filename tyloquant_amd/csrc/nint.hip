@@ -218,15 +218,18 @@ static int launch_gemv_mb(const NintK &k, const uint8_t *w, const uint16_t *x, i
         return fail(MFQ_ERR_UNSUPPORTED, "nint_gemv: no paired kernel for NINT%d-%d", k.bits, k.gs);
     }
 #undef MFQ_PAIRED
-    if (mfma_generic_profile(k)) {
-        MFQ_XREG(MFQ_SINGLE_ARG(GenericUnit<5, 28>))
-        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, rbw)), static_cast<unsigned>(ceil_div(M, MB)));
-        if (spw * rbw <= 3)
-            MFQ_GEMV_LAUNCH((nint_gemv_natural_kernel<5, 28, XF16, MB, false>), grid, k, w, x, ldx, M, y, ldy, spw, rbw);
-        else
-            MFQ_GEMV_LAUNCH((nint_gemv_natural_kernel<5, 28, XF16, MB, true>), grid, k, w, x, ldx, M, y, ldy, spw, rbw);
-        return check_launch("nint_gemv_natural");
+#define MFQ_NATURAL(UNIT, B, G)                                                                              \
+    if (k.kind == 0 && k.bits == B && k.gs == G) {                                                           \
+        MFQ_XREG(MFQ_SINGLE_ARG(UNIT<B, G>))                                                                 \
+        const dim3 grid(static_cast<unsigned>(ceil_div(k.n_rowblocks, rbw)), static_cast<unsigned>(ceil_div(M, MB))); \
+        if (spw * rbw <= 3)                                                                                  \
+            MFQ_GEMV_LAUNCH((nint_gemv_natural_kernel<B, G, XF16, MB, false>), grid, k, w, x, ldx, M, y, ldy, spw, rbw); \
+        else                                                                                                 \
+            MFQ_GEMV_LAUNCH((nint_gemv_natural_kernel<B, G, XF16, MB, true>), grid, k, w, x, ldx, M, y, ldy, spw, rbw); \
+        return check_launch("nint_gemv_natural");                                                            \
     }
+    MFQ_GENERIC_PROFILES(MFQ_NATURAL)
+#undef MFQ_NATURAL
     const dim3 grid(k.n_rowblocks, static_cast<unsigned>(ceil_div(M, MB)));
     MFQ_GEMV_LAUNCH((nint_gemv_generic_kernel<XF16, MB>), grid, k, w, x, ldx, M, y, ldy, spw);
 #undef MFQ_GEMV_LAUNCH
@@ -278,7 +281,11 @@ static int launch_mfma_nb(const NintK &k, const uint8_t *w, const uint16_t *x, i
         MFQ_MFMA(PairedUnit, 4, 32) MFQ_MFMA(PairedUnit, 4, 24) MFQ_MFMA(PairedUnit, 4, 16) MFQ_MFMA(PairedUnit, 4, 48)
         MFQ_MFMA(PairedUnit, 3, 24) MFQ_MFMA(PairedUnit, 2, 16) MFQ_MFMA(PairedUnit, 2, 32)
     } else {
-        MFQ_MFMA(GenericUnit, 5, 28)
+        // (twelve dwords a unit: one row-block of NINT8-48 per wave; two spill and run 1.4x slower)
+        if constexpr (NB > 1) {
+            if (k.bits == 8) return launch_mfma_nb<XF16, 1>(k, w, x, ldx, M, y, ldy, st);
+        }
+        MFQ_GENERIC_PROFILES(MFQ_MFMA)
     }
 #undef MFQ_MFMA
     return fail(MFQ_ERR_UNSUPPORTED, "nint_mfma: no kernel for NINT%d-%d", k.bits, k.gs);
@@ -367,7 +374,8 @@ static int launch_mfma_resident(const NintK &k, const uint8_t *w, const uint16_t
 
 // ---- prefill: block-tiled MFMA GEMM with in-register dequantization ---------------------------
 bool nint_prefill_capable(const mfq_nint_desc *d) {
-    return (d->kind == 1 || (d->bits == 5 && d->gs == 28)) && d->neuron_len >= 8 && 4 * d->rowblock_bytes < (1ll << 31);
+    return (d->kind == 1 || (d->bits == 5 && d->gs == 28) || (d->bits == 6 && d->gs == 24)) && d->neuron_len >= 8 &&
+           4 * d->rowblock_bytes < (1ll << 31);
 }
 size_t nint_prefill_xg_bytes(const mfq_nint_desc *d, int M) { return static_cast<size_t>(M) * d->nsteps * 64; }
 
@@ -475,7 +483,7 @@ int nint_prefill(const mfq_nint_desc *d, const void *weight, const uint16_t *x16
         MFQ_PREFILL(PairedUnit, 4, 48) MFQ_PREFILL(PairedUnit, 3, 24) MFQ_PREFILL(PairedUnit, 2, 16)
         MFQ_PREFILL(PairedUnit, 2, 32)
     } else {
-        MFQ_PREFILL(GenericUnit, 5, 28)
+        MFQ_PREFILL(GenericUnit, 5, 28) MFQ_PREFILL(GenericUnit, 6, 24)
     }
 #undef MFQ_PREFILL
 #undef MFQ_PREFILL_CFG
@@ -490,7 +498,9 @@ int nint_gemv_any(const mfq_nint_desc *d, const void *weight, const void *x, int
     static const int valu_max = tune_env("MFQ_GEMV_VALU_MAX_M", 2);
     // two rows: the vector-ALU GEMV unpacks once and takes two dot products (10.6 vs 12.9 us on 12288x4096);
     // from three rows on the matrix-core kernel wins
-    if (M > valu_max && mfma_eligible(k, x, ldx)) {
+    // NINT8-48: the vector-ALU bodies hold a step of twelve-dword units per row-block and spill; the matrix-core kernel
+    // with one row-block per wave takes every batch from one row on (12288 x 4096: 28 us against 39)
+    if ((M > valu_max || k.bits == 8) && mfma_eligible(k, x, ldx)) {
         int nb, spw, nwaves, red_slots;
         size_t lds;
         if (mfma_resident_shape(k, M, nb, spw, nwaves, lds, red_slots))
@@ -619,7 +629,7 @@ static int launch_gemv_swiglu(const NintK &k, const uint8_t *w, const uint16_t *
         MFQ_SWIGLU(PairedUnit, 4, 32) MFQ_SWIGLU(PairedUnit, 4, 24) MFQ_SWIGLU(PairedUnit, 4, 16) MFQ_SWIGLU(PairedUnit, 4, 48)
         MFQ_SWIGLU(PairedUnit, 3, 24) MFQ_SWIGLU(PairedUnit, 2, 16) MFQ_SWIGLU(PairedUnit, 2, 32)
     } else {
-        MFQ_SWIGLU(GenericUnit, 5, 28)
+        MFQ_GENERIC_PROFILES(MFQ_SWIGLU)
     }
 #undef MFQ_SWIGLU
 #undef MFQ_SWIGLU_LAUNCH

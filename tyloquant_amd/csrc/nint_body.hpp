@@ -70,7 +70,11 @@ __device__ __forceinline__ uint32_t unit_code(const NintK &k, const uint32_t *q,
 }
 
 // natural-order profiles with a unit of their own (GEMV, streaming and prefill kernels)
-inline bool mfma_generic_profile(const NintK &k) { return k.kind == 0 && k.bits == 5 && k.gs == 28; }
+// (NINT5 (5,28), NINT6 (6,24) and NINT8 (8,48): the production profiles outside the paired layouts, FORMATS.md:73-79)
+inline bool mfma_generic_profile(const NintK &k) {
+    return k.kind == 0 && ((k.bits == 5 && k.gs == 28) || (k.bits == 6 && k.gs == 24) || (k.bits == 8 && k.gs == 48));
+}
+#define MFQ_GENERIC_PROFILES(X) X(GenericUnit, 5, 28) X(GenericUnit, 6, 24) X(GenericUnit, 8, 48)
 
 constexpr uint32_t kMagicH2 = 0x64006400u;  // (1024.0, 1024.0) in fp16
 constexpr int kMaxRbw = 4;                  // row-blocks one wave may walk through
@@ -203,6 +207,12 @@ struct GenericUnit {
     // dwords), a shift-or copies the second code to bit 16, one AND-OR drops the rest and adds the magic exponent.
     __device__ static __forceinline__ void unpack(const uint32_t (&q)[D], uint32_t, uint32_t (&v)[NPAIR]) {
         constexpr uint32_t M = (1u << BITS) - 1u;
+        if constexpr (BITS == 8) {  // bytes: one byte permute drops a pair into the mantissas of (1024, 1024)
+#pragma unroll
+            for (int p = 0; p < NPAIR; ++p)
+                v[p] = 2 * p >= GS ? kMagicH2 : __builtin_amdgcn_perm(q[p / 2], kMagicH2, (p & 1) ? 0x03070106u : 0x03050104u);
+            return;
+        }
 #pragma unroll
         for (int p = 0; p < NPAIR; ++p) {
             if (2 * p >= GS) {

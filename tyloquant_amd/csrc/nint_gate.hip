@@ -73,7 +73,9 @@ static int launch_gate(const NintK &k, const uint8_t *w, const uint16_t *x, int6
         MFQ_GATE_UNIT(PairedUnit, 2, 32)
         return fail(MFQ_ERR_UNSUPPORTED, "nint_gemv_gate: no paired kernel for NINT%d-%d", k.bits, k.gs);
     }
-    if (mfma_generic_profile(k)) MFQ_GATE_UNIT(GenericUnit, 5, 28)
+    if (mfma_generic_profile(k)) {
+        MFQ_GENERIC_PROFILES(MFQ_GATE_UNIT)
+    }
     const dim3 ggrid(k.n_rowblocks, static_cast<unsigned>(ceil_div(M, MB)));
     MFQ_GATE_LAUNCH((nint_gemv_gate_generic_kernel<XF16, MB>), ggrid, k, w, x, ldx, gate, ldg, mode, M, y, ldy, spw);
 #undef MFQ_GATE_UNIT

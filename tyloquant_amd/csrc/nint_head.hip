@@ -171,7 +171,9 @@ static int launch_gemv_argmax(const NintK &k, const uint8_t *w, const uint16_t *
     if (k.kind == 1) {
         MFQ_ARGMAX(PairedUnit, 4, 32) MFQ_ARGMAX(PairedUnit, 4, 24) MFQ_ARGMAX(PairedUnit, 3, 24)
     } else {
-        MFQ_ARGMAX(GenericUnit, 5, 28)
+        // (NINT8-48 takes the unfused form: its plain GEMV runs on the matrix cores, and the logits of this call are
+        // the plain GEMV's floats)
+        MFQ_ARGMAX(GenericUnit, 5, 28) MFQ_ARGMAX(GenericUnit, 6, 24)
     }
 #undef MFQ_ARGMAX
     return MFQ_OK;
