@@ -449,6 +449,30 @@ def test_one_bit_families_dequant_bit_exact_and_matmul(dtype, kw, out, K):
         _check(lin(x).cpu().numpy(), O.linear_forward_f64(want, xf))
 
 
+@pytest.mark.parametrize("cus", [1, 2])
+@pytest.mark.parametrize("dtype,kw,out,K", [("NVQ1-L", dict(state_bits=3), 150, 100), ("NVQ1-L", dict(state_bits=4), 70, 1544),
+                                            ("NVQ1-S", dict(), 97, 1544), ("NPQ0-L", dict(), 150, 120),
+                                            ("NPQ0-S", dict(), 70, 1544)])
+def test_one_bit_families_with_several_neurons_per_wave(cu_count, cus, dtype, kw, out, K):
+    """The decoders of the 1-bit families in the kernel that stages a wave's bit ranges in LDS, sized for one or two
+    compute units so that a wave walks several neurons: state fields of 2 to 4 bits and delta signs that start inside a
+    byte, waves with fewer neurons than the others and with none, one to eight rows per pass, both activation types
+    and bf16 rows far outside fp16's range."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import nvq_matmul
+    rng = np.random.default_rng(170 + out + K + cus)
+    t = synth.nvq1_random(rng, dtype, out, K, **kw) if dtype.startswith("NVQ1") else synth.npq0_random(rng, dtype, out, K)
+    _, blob = O.pack_tensor(t)
+    lin = R.load_quant_linear(dtype, blob)
+    want = O.dequantize_tensor(O.unpack_tensor(dtype, blob))
+    cu_count(cus)
+    for M, xd in ((1, torch.bfloat16), (2, torch.float16), (5, torch.bfloat16), (8, torch.float16), (16, torch.bfloat16)):
+        x, xf = _x(rng, M, K, xd)
+        _check(nvq_matmul(lin.weight, x).cpu().numpy(), O.linear_forward_f64(want, xf))
+    big = torch.from_numpy((rng.standard_normal((2, K)) * 2.0e6).astype(np.float32)).to(torch.bfloat16).cuda()
+    _check(nvq_matmul(lin.weight, big).cpu().numpy() / 2.0e6, O.linear_forward_f64(want, big.float().cpu().numpy()) / 2.0e6)
+
+
 def test_one_bit_families_reference_blobs_and_loader_errors():
     """The reference-packed blobs of the golden fixture dequantize on the device to the values the reference computed;
     malformed blobs are refused with the reference's messages before anything is uploaded."""

@@ -426,7 +426,7 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
         M = 1;
         m0 = 0;
     }
-    const int ncb = k.banks * k.entries;
+    const int ncb = k.kind == 2 ? k.cb_bytes / k.vs : k.banks * k.entries;  // table entries of vs int8 values (kind 2: 4-value entries of both sub-codebooks)
     uint8_t *lds8 = reinterpret_cast<uint8_t *>(lds32);
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)lds8));
     const uint32_t esz = static_cast<uint32_t>(k.vs) * 2u;  // bytes of a table entry: 8 (E8) or 4 (D4) values of the activations' type
@@ -439,7 +439,11 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
     const int nn = max(0, min(sh.npw, k.nrows - row_first));
     const int64_t n0 = k.row0 + row_first;
     // bit ranges [n0 * per, (n0 + nn) * per) of the three streams, read from 16-byte aligned addresses
-    const int64_t bit0[3] = {n0 * k.nvec * k.ib, n0 * k.nsign * 7, n0 * k.ng * 4};
+    // bits per neuron of the three ranges: indices, the sign stream (kind 0: 7 per block; kind 1: a delta sign per group;
+    // kind 2: none) and the states
+    const uint32_t per1 = k.kind == 0 ? static_cast<uint32_t>(k.nsign) * 7u : (k.kind == 1 ? static_cast<uint32_t>(k.ng) : 0u);
+    const uint32_t per2 = static_cast<uint32_t>(k.ng) * static_cast<uint32_t>(k.sbits);
+    const int64_t bit0[3] = {n0 * k.nvec * k.ib, n0 * static_cast<int64_t>(per1), n0 * static_cast<int64_t>(per2)};
     const int64_t region[3] = {k.index_off, k.sign_off, k.state_off};
     const int64_t region_bytes[3] = {k.index_bytes + 4, k.sign_bytes + 4, k.state_bytes + 4};
     uint32_t shift[3];   // bits between the staged range's first bit and the first bit of neuron n0
@@ -541,10 +545,46 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
         float acc[MB];
 #pragma unroll
         for (int m = 0; m < MB; ++m) acc[m] = 0.f;
-        const uint32_t ib = shift[0] + static_cast<uint32_t>(j) * k.nvec * k.ib, sb0 = shift[1] + static_cast<uint32_t>(j) * k.nsign * 7u,
-                       tb = shift[2] + static_cast<uint32_t>(j) * k.ng * 4u;
+        const uint32_t ib = shift[0] + static_cast<uint32_t>(j) * k.nvec * k.ib, sb0 = shift[1] + static_cast<uint32_t>(j) * per1,
+                       tb = shift[2] + static_cast<uint32_t>(j) * per2;
         for (int g = lane; g < k.ng; g += 64) {
-            const uint32_t state = field(lds_base + roff[2], tb + 4u * g, 4);
+            const uint32_t state = field(lds_base + roff[2], tb + static_cast<uint32_t>(k.sbits) * g, k.sbits);
+            if (k.kind != 0) {
+                // The 1-bit families.  Kind 1 (NVQ1-L / -S): w = scale * (code + d), code a ternary 8-vector of the bank the
+                // group's delta sign names, d = -delta / +delta by that sign -- the products with the codes plus d times
+                // the sum of the group's activations.  Kind 2 (NPQ0-L / -S): a block is a 4-vector of the state's first
+                // sub-codebook (index bits 0..2) beside one of its second (the bits above).
+                const u32x2_t se1 = *reinterpret_cast<lds_u32x2_ptr>(lds_base + stab_off + state * 8u);
+                uint32_t neg = 0u;
+                if (k.kind == 1) neg = field(lds_base + roff[1], sb0 + g, 1);
+                u32x4_t wv1[3];
+#pragma unroll
+                for (int b = 0; b < 3; ++b) {
+                    // (a block past the neuron's last vector meets staged zeros; entry 0 keeps its lookups inside the tables)
+                    const uint32_t idx = 3 * g + b < k.nvec ? field(lds_base + roff[0], ib + static_cast<uint32_t>(3 * g + b) * k.ib, k.ib) : 0u;
+                    if (k.kind == 1) {
+                        wv1[b] = *reinterpret_cast<lds_u32x4_ptr>(lds_base + ((k.banks == 2 ? neg : 0u) * static_cast<uint32_t>(k.entries) + idx) * 16u);
+                    } else {
+                        const u32x2_t e0 = *reinterpret_cast<lds_u32x2_ptr>(lds_base + (state * 8u + (idx & 7u)) * 8u);
+                        const u32x2_t e1 = *reinterpret_cast<lds_u32x2_ptr>(lds_base + (static_cast<uint32_t>(k.banks) * 8u + state * static_cast<uint32_t>(k.entries) + (idx >> 3)) * 8u);
+                        wv1[b] = u32x4_t{e0.x, e0.y, e1.x, e1.y};
+                    }
+                }
+                const float sc1 = __uint_as_float(se1.x), dl = neg ? -k.delta : k.delta;
+                const uint32_t ones = XF16 ? 0x3c003c00u : 0x3f803f80u;
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+                    float part1 = 0.f, xsum = 0.f;
+#pragma unroll
+                    for (int b = 0; b < 3; ++b) {
+                        const u32x4_t xv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + x_off + static_cast<uint32_t>(m) * row_bytes + static_cast<uint32_t>(3 * g + b) * 16u);
+                        part1 = e8_dot8<XF16>(wv1[b], xv, part1);
+                        if (k.kind == 1) xsum = e8_dot8<XF16>(u32x4_t{ones, ones, ones, ones}, xv, xsum);
+                    }
+                    acc[m] = fmaf(sc1, fmaf(dl, xsum, part1), acc[m]);
+                }
+                continue;
+            }
             // the indices of the group's three blocks: one 24-bit field of index bytes, three fields of 10 or 12 bits, or
             // (4-dimensional vectors) two fields per block
             uint32_t ix[3], ix2[3] = {0u, 0u, 0u};
@@ -619,12 +659,20 @@ constexpr int kNvqsGemvMaxM = 16;  // rows up to which the weights are re-read p
 // The E8 kernel takes the sign-stream format with 8- or 4-dimensional vectors, 4-bit states and tables that fit the LDS
 // in the activations' type (E8: 256 or 1024 entries in up to four banks, 4096 in one; D4: 1024 entries), tensors whose streams fit 32-bit offsets and
 // neurons of at most about 16000 weights with index bytes, 10000 with 12-bit indices (a wave's index range is two 1 KB
-// requests at most).  MB = rows per pass that fit the LDS.
+// requests at most), and the 1-bit families NVQ1-L / NVQ1-S (ternary 8-vectors, a delta sign per group) and NPQ0-L /
+// NPQ0-S (two 4-vectors per block) with their states of 2 to 4 bits.  MB = rows per pass that fit the LDS.
 static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     static const int off = tune_env("MFQ_NVQS_E8_OFF", 0);
-    if (off || k.kind != 0 || (k.vs != 8 && k.vs != 4) || k.ib < 8 || k.ib > 12 || k.entries != (1 << k.ib) || k.sbits != 4 || k.banks > 4 ||
-        k.index_bytes >= (1ll << 31) || k.sign_bytes >= (1ll << 31))
+    if (off || k.index_bytes >= (1ll << 31) || k.sign_bytes >= (1ll << 31)) return false;
+    if (k.kind == 0) {
+        if ((k.vs != 8 && k.vs != 4) || k.ib < 8 || k.ib > 12 || k.entries != (1 << k.ib) || k.sbits != 4 || k.banks > 4) return false;
+    } else if (k.kind == 1) {  // NVQ1-L / NVQ1-S: 2048 or two banks of 512 ternary 8-vectors
+        if (k.vs != 8 || k.ib < 8 || k.ib > 12 || k.entries != (1 << k.ib) || k.sbits < 2 || k.sbits > 4 || k.banks > 2) return false;
+    } else if (k.kind == 2) {  // NPQ0-L / NPQ0-S: a few dozen 4-vectors per state
+        if (k.ib < 4 || k.ib > 8 || k.entries * 8 != (1 << k.ib) || k.sbits < 2 || k.sbits > 4 || k.cb_bytes % 8 != 0) return false;
+    } else {
         return false;
+    }
     auto cap = [](int64_t bits) { return static_cast<uint32_t>((16 + (bits + 7) / 8 + 8 + 15) / 16 * 16); };
     int npw = static_cast<int>(ceil_div(k.nrows, static_cast<int64_t>(gemv_cu_count()) * kE8Waves));
     if (npw > 4) npw = 4;
@@ -633,11 +681,11 @@ static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     sh.npw = npw;
     sh.kp = k.ng * 24;
     sh.cap[0] = cap(static_cast<int64_t>(npw) * k.nvec * k.ib);
-    sh.cap[1] = cap(static_cast<int64_t>(npw) * k.nsign * 7);
-    sh.cap[2] = cap(static_cast<int64_t>(npw) * k.ng * 4);
+    sh.cap[1] = cap(static_cast<int64_t>(npw) * (k.kind == 0 ? static_cast<int64_t>(k.nsign) * 7 : (k.kind == 1 ? k.ng : 0)));
+    sh.cap[2] = cap(static_cast<int64_t>(npw) * k.ng * k.sbits);
     sh.wave_bytes = sh.cap[0] + sh.cap[1] + sh.cap[2];
     for (mb = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1)); mb >= 1; mb >>= 1) {
-        sh.lds_bytes = static_cast<uint32_t>(k.banks) * static_cast<uint32_t>(k.entries) * static_cast<uint32_t>(k.vs) * 2u + 4096u + 128u + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
+        sh.lds_bytes = (k.kind == 2 ? static_cast<uint32_t>(k.cb_bytes) : static_cast<uint32_t>(k.banks) * static_cast<uint32_t>(k.entries) * static_cast<uint32_t>(k.vs)) * 2u + 4096u + 128u + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
         if (sh.lds_bytes <= kMaxDynamicLds) return true;
     }
     return false;
