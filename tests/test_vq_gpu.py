@@ -542,6 +542,26 @@ def test_nepq0_dequant_bit_exact_and_matmul(label, E, out, K, banks):
         NepqWeight.from_blob(bytes(bad))
 
 
+@pytest.mark.parametrize("cus", [1, 2])
+@pytest.mark.parametrize("label,E,out,K,banks", [("NEPQ0-S", 2, 75, 1544, 40), ("NEPQ0-L", 3, 50, 200, 5), ("NEPQ0-L", 1, 150, 96, 1)])
+def test_nepq0_with_several_neurons_per_wave(cu_count, cus, label, E, out, K, banks):
+    """The table-pool decoder in the kernel that stages a wave's bit ranges in LDS, sized for one or two compute units:
+    experts whose first neuron starts inside a byte of the streams, waves with several neurons, with fewer and with
+    none, one to eight rows per pass, both activation types and bf16 rows far outside fp16's range."""
+    from tyloquant_amd.runtime_vq import NepqWeight, nepq_matmul
+    rng = np.random.default_rng(223 + E + out + K + cus)
+    blob = O.pack_nepq(synth.nepq_random(rng, label, E, out, K, banks))
+    w = NepqWeight.from_blob(blob)
+    want = O.dequantize_nepq(O.unpack_nepq(blob))
+    cu_count(cus)
+    for e in range(E):
+        for M, xd in ((1, torch.bfloat16), (2, torch.float16), (5, torch.bfloat16), (8, torch.float16), (16, torch.bfloat16)):
+            x, xf = _x(rng, M, K, xd)
+            _check(nepq_matmul(w, x, e).cpu().numpy(), O.linear_forward_f64(want[e], xf))
+    big = torch.from_numpy((rng.standard_normal((2, K)) * 2.0e6).astype(np.float32)).to(torch.bfloat16).cuda()
+    _check(nepq_matmul(w, big, E - 1).cpu().numpy() / 2.0e6, O.linear_forward_f64(want[E - 1], big.float().cpu().numpy()) / 2.0e6)
+
+
 @pytest.mark.parametrize("family", ["NVQ3J-512", "NEPQ0-L", "NEPQ1-S", "MXFP8"])
 def test_reserve_sizes_the_workspace_of_every_family(family):
     """QuantLinear.reserve(max_rows) on an NVQ, an NEPQ0 (bit streams in place), an NEPQ1 and an MX linear: forward() of

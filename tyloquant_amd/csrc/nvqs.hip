@@ -426,11 +426,14 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
         M = 1;
         m0 = 0;
     }
-    const int ncb = k.kind == 2 ? k.cb_bytes / k.vs : k.banks * k.entries;  // table entries of vs int8 values (kind 2: 4-value entries of both sub-codebooks)
+    // table entries of vs int8 values (kinds 2 and 3: pairs of the 4-value entries of the sub-codebooks, of every table of the pool)
+    const int ncb = k.kind == 2 ? k.cb_bytes / k.vs : (k.kind == 3 ? k.nbank * k.bank_bytes / k.vs : k.banks * k.entries);
     uint8_t *lds8 = reinterpret_cast<uint8_t *>(lds32);
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)lds8));
     const uint32_t esz = static_cast<uint32_t>(k.vs) * 2u;  // bytes of a table entry: 8 (E8) or 4 (D4) values of the activations' type
-    const uint32_t sgn_off = static_cast<uint32_t>(ncb) * esz, stab_off = sgn_off + 4096u, x_off = stab_off + 128u;
+    // (kind 3 keeps the pool's scale tables, eight floats per table, behind the state table)
+    const uint32_t sgn_off = static_cast<uint32_t>(ncb) * esz, stab_off = sgn_off + 4096u, lut3_off = stab_off + 128u,
+                   x_off = lut3_off + (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * 32u : 0u);
     const uint32_t row_bytes = static_cast<uint32_t>(sh.kp) * 2u;
     const uint32_t wave_off = x_off + MB * row_bytes + static_cast<uint32_t>(wave) * sh.wave_bytes;
 
@@ -440,8 +443,9 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
     const int64_t n0 = k.row0 + row_first;
     // bit ranges [n0 * per, (n0 + nn) * per) of the three streams, read from 16-byte aligned addresses
     // bits per neuron of the three ranges: indices, the sign stream (kind 0: 7 per block; kind 1: a delta sign per group;
-    // kind 2: none) and the states
-    const uint32_t per1 = k.kind == 0 ? static_cast<uint32_t>(k.nsign) * 7u : (k.kind == 1 ? static_cast<uint32_t>(k.ng) : 0u);
+    // kind 2: none; kind 3: a table id byte per 96 weights) and the states
+    const uint32_t per1 = k.kind == 0 ? static_cast<uint32_t>(k.nsign) * 7u
+                        : (k.kind == 1 ? static_cast<uint32_t>(k.ng) : (k.kind == 3 ? static_cast<uint32_t>(k.nsuper) * 8u : 0u));
     const uint32_t per2 = static_cast<uint32_t>(k.ng) * static_cast<uint32_t>(k.sbits);
     const int64_t bit0[3] = {n0 * k.nvec * k.ib, n0 * static_cast<int64_t>(per1), n0 * static_cast<int64_t>(per2)};
     const int64_t region[3] = {k.index_off, k.sign_off, k.state_off};
@@ -520,6 +524,10 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
         st[2 * tid] = lutv;
         reinterpret_cast<uint32_t *>(st)[2 * tid + 1] = lds_base + bfsv * static_cast<uint32_t>(k.entries) * esz;
     }
+    if (k.kind == 3) {
+        const float *lut3 = reinterpret_cast<const float *>(reinterpret_cast<const uint8_t *>(lut) + 128 + static_cast<int64_t>(k.nbank) * k.bank_bytes);
+        for (int i = tid; i < k.nbank * 8; i += blockDim.x) *reinterpret_cast<float *>(lds8 + lut3_off + static_cast<uint32_t>(i) * 4u) = lut3[i];
+    }
     x_park(tid, xc0);
     x_park(tid + static_cast<int>(blockDim.x), xc1);
     for (int c = tid + 2 * static_cast<int>(blockDim.x); c < MB * chunks; c += blockDim.x) x_park(c, x_chunk(c));
@@ -553,10 +561,18 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
                 // The 1-bit families.  Kind 1 (NVQ1-L / -S): w = scale * (code + d), code a ternary 8-vector of the bank the
                 // group's delta sign names, d = -delta / +delta by that sign -- the products with the codes plus d times
                 // the sum of the group's activations.  Kind 2 (NPQ0-L / -S): a block is a 4-vector of the state's first
-                // sub-codebook (index bits 0..2) beside one of its second (the bits above).
+                // sub-codebook (index bits 0..2) beside one of its second (the bits above).  Kind 3 (NEPQ0-S / -L): the same
+                // with a pool of tables.
                 const u32x2_t se1 = *reinterpret_cast<lds_u32x2_ptr>(lds_base + stab_off + state * 8u);
-                uint32_t neg = 0u;
+                uint32_t neg = 0u, tbase = 0u;  // tbase: LDS byte offset of the group's table
+                float sc1 = __uint_as_float(se1.x);
                 if (k.kind == 1) neg = field(lds_base + roff[1], sb0 + g, 1);
+                if (k.kind == 3) {
+                    // NEPQ0: the neuron's table of the pool for these 96 weights gives sub-codebooks and scale
+                    const uint32_t pb = min(field(lds_base + roff[1], sb0 + 8u * (static_cast<uint32_t>(g) >> 2), 8), static_cast<uint32_t>(k.nbank - 1));
+                    tbase = pb * static_cast<uint32_t>(k.bank_bytes) * 2u;
+                    sc1 = __uint_as_float(*reinterpret_cast<lds_u32_ptr>(lds_base + lut3_off + (pb * 8u + state) * 4u));
+                }
                 u32x4_t wv1[3];
 #pragma unroll
                 for (int b = 0; b < 3; ++b) {
@@ -565,12 +581,12 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
                     if (k.kind == 1) {
                         wv1[b] = *reinterpret_cast<lds_u32x4_ptr>(lds_base + ((k.banks == 2 ? neg : 0u) * static_cast<uint32_t>(k.entries) + idx) * 16u);
                     } else {
-                        const u32x2_t e0 = *reinterpret_cast<lds_u32x2_ptr>(lds_base + (state * 8u + (idx & 7u)) * 8u);
-                        const u32x2_t e1 = *reinterpret_cast<lds_u32x2_ptr>(lds_base + (static_cast<uint32_t>(k.banks) * 8u + state * static_cast<uint32_t>(k.entries) + (idx >> 3)) * 8u);
+                        const u32x2_t e0 = *reinterpret_cast<lds_u32x2_ptr>(lds_base + tbase + (state * 8u + (idx & 7u)) * 8u);
+                        const u32x2_t e1 = *reinterpret_cast<lds_u32x2_ptr>(lds_base + tbase + (static_cast<uint32_t>(k.banks) * 8u + state * static_cast<uint32_t>(k.entries) + (idx >> 3)) * 8u);
                         wv1[b] = u32x4_t{e0.x, e0.y, e1.x, e1.y};
                     }
                 }
-                const float sc1 = __uint_as_float(se1.x), dl = neg ? -k.delta : k.delta;
+                const float dl = neg ? -k.delta : k.delta;
                 const uint32_t ones = XF16 ? 0x3c003c00u : 0x3f803f80u;
 #pragma unroll
                 for (int m = 0; m < MB; ++m) {
@@ -660,7 +676,8 @@ constexpr int kNvqsGemvMaxM = 16;  // rows up to which the weights are re-read p
 // in the activations' type (E8: 256 or 1024 entries in up to four banks, 4096 in one; D4: 1024 entries), tensors whose streams fit 32-bit offsets and
 // neurons of at most about 16000 weights with index bytes, 10000 with 12-bit indices (a wave's index range is two 1 KB
 // requests at most), and the 1-bit families NVQ1-L / NVQ1-S (ternary 8-vectors, a delta sign per group) and NPQ0-L /
-// NPQ0-S (two 4-vectors per block) with their states of 2 to 4 bits.  MB = rows per pass that fit the LDS.
+// NPQ0-S (two 4-vectors per block; NEPQ0-S / NEPQ0-L: out of a pool of tables that fits the LDS) with their states of
+// 2 to 4 bits.  MB = rows per pass that fit the LDS.
 static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     static const int off = tune_env("MFQ_NVQS_E8_OFF", 0);
     if (off || k.index_bytes >= (1ll << 31) || k.sign_bytes >= (1ll << 31)) return false;
@@ -668,8 +685,9 @@ static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
         if ((k.vs != 8 && k.vs != 4) || k.ib < 8 || k.ib > 12 || k.entries != (1 << k.ib) || k.sbits != 4 || k.banks > 4) return false;
     } else if (k.kind == 1) {  // NVQ1-L / NVQ1-S: 2048 or two banks of 512 ternary 8-vectors
         if (k.vs != 8 || k.ib < 8 || k.ib > 12 || k.entries != (1 << k.ib) || k.sbits < 2 || k.sbits > 4 || k.banks > 2) return false;
-    } else if (k.kind == 2) {  // NPQ0-L / NPQ0-S: a few dozen 4-vectors per state
+    } else if (k.kind == 2 || k.kind == 3) {  // NPQ0-L / NPQ0-S: a few dozen 4-vectors per state; NEPQ0: a pool of such tables
         if (k.ib < 4 || k.ib > 8 || k.entries * 8 != (1 << k.ib) || k.sbits < 2 || k.sbits > 4 || k.cb_bytes % 8 != 0) return false;
+        if (k.kind == 3 && (k.nbank < 1 || k.nbank > 256 || k.bank_bytes % 8 != 0 || k.bank_bytes != k.banks * 32 + k.banks * k.entries * 4)) return false;
     } else {
         return false;
     }
@@ -681,11 +699,15 @@ static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     sh.npw = npw;
     sh.kp = k.ng * 24;
     sh.cap[0] = cap(static_cast<int64_t>(npw) * k.nvec * k.ib);
-    sh.cap[1] = cap(static_cast<int64_t>(npw) * (k.kind == 0 ? static_cast<int64_t>(k.nsign) * 7 : (k.kind == 1 ? k.ng : 0)));
+    sh.cap[1] = cap(static_cast<int64_t>(npw) * (k.kind == 0 ? static_cast<int64_t>(k.nsign) * 7 : (k.kind == 1 ? k.ng : (k.kind == 3 ? k.nsuper * 8 : 0))));
     sh.cap[2] = cap(static_cast<int64_t>(npw) * k.ng * k.sbits);
     sh.wave_bytes = sh.cap[0] + sh.cap[1] + sh.cap[2];
     for (mb = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1)); mb >= 1; mb >>= 1) {
-        sh.lds_bytes = (k.kind == 2 ? static_cast<uint32_t>(k.cb_bytes) : static_cast<uint32_t>(k.banks) * static_cast<uint32_t>(k.entries) * static_cast<uint32_t>(k.vs)) * 2u + 4096u + 128u + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
+        const uint32_t table = k.kind == 2 ? static_cast<uint32_t>(k.cb_bytes)
+                             : (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * static_cast<uint32_t>(k.bank_bytes)
+                                            : static_cast<uint32_t>(k.banks) * static_cast<uint32_t>(k.entries) * static_cast<uint32_t>(k.vs));
+        if (table > kMaxDynamicLds / 2) return false;
+        sh.lds_bytes = table * 2u + 4096u + 128u + (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * 32u : 0u) + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
         if (sh.lds_bytes <= kMaxDynamicLds) return true;
     }
     return false;
