@@ -21,8 +21,8 @@
  *     NVQ cohort (mfq_hip_nvq_gemv_pairs), the NEPQ1 one-row kernel and the NINT8-0 streaming GEMV (one row; more rows when
  *     the activation rows are not 16-byte aligned),
  *   - the stream-family (E8, d4_1024, 1-bit, NEPQ0) wave-per-neuron kernels up to 16 rows, which multiply in fp32, and
- *     the kernel of the E8 formats whose tables fit the LDS and of NVQ1-L / NVQ1-S / NPQ0-L / NPQ0-S / NEPQ0, whose
- *     packed dot products take bf16 as it is,
+ *     the kernels of the E8 formats whose tables fit the LDS and of NVQ1-L / NVQ1-S / NPQ0-L / NPQ0-S / NEPQ0 (packed dot
+ *     products up to four rows, matrix-core products from five to 16), which take bf16 as it is,
  *   - the MXFP4 / MXFP8 kernels up to 256 rows, whose matrix-core products take bf16 as it is (the weights are exact in
  *     bf16, scale included),
  *   - every prefill kernel:

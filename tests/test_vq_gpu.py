@@ -562,6 +562,45 @@ def test_nepq0_with_several_neurons_per_wave(cu_count, cus, label, E, out, K, ba
     _check(nepq_matmul(w, big, E - 1).cpu().numpy() / 2.0e6, O.linear_forward_f64(want[E - 1], big.float().cpu().numpy()) / 2.0e6)
 
 
+TILE_CASES = [("jsc", "e8_256", 4, 37, 1544), ("jsc", "e8_1024", 2, 70, 100), ("jsc", "e8_4096", 1, 33, 96),
+              ("jsc", "d4_1024", 2, 50, 1540), ("plain_e8", "index_parity", 0, 41, 200), ("NVQ1-L", dict(state_bits=3), 0, 37, 1540),
+              ("NVQ1-S", dict(), 0, 33, 1544), ("NPQ0-L", dict(), 0, 70, 104), ("NPQ0-S", dict(), 0, 18, 1544)]
+
+
+@pytest.mark.parametrize("kind,a,b,out,K", TILE_CASES)
+def test_stream_formats_on_the_matrix_core_tile_kernel(kind, a, b, out, K):
+    """Five to sixteen rows of the formats read in place from their bit streams run as 16-neuron tiles on the matrix
+    cores: a last tile with fewer neurons, K that ends inside a group, a block and a vector, every row count of the
+    range in both activation types, rows at a stride that is no multiple of 16 bytes (element-wise loads), and bf16 rows
+    far outside fp16's range."""
+    from tyloquant_amd import runtime as R
+    from tyloquant_amd.runtime_vq import nvq_matmul
+    rng = np.random.default_rng(310 + out + K)
+    if kind == "jsc":
+        t = synth.nvq_jsc_random(rng, out, K, a, b)
+    elif kind == "plain_e8":
+        t = synth.nvq_plain_e8_random(rng, out, K, a)
+    elif kind.startswith("NVQ1"):
+        t = synth.nvq1_random(rng, kind, out, K, **a)
+    else:
+        t = synth.npq0_random(rng, kind, out, K)
+    dtype, blob = O.pack_tensor(t)
+    lin = R.load_quant_linear(dtype, blob)
+    want = O.dequantize_tensor(O.unpack_tensor(dtype, blob))
+    for M in range(5, 17):
+        xd = torch.bfloat16 if M % 2 else torch.float16
+        x, xf = _x(rng, M, K, xd)
+        _check(nvq_matmul(lin.weight, x).cpu().numpy(), O.linear_forward_f64(want, xf))
+    wide = torch.zeros((9, K + 3), dtype=torch.bfloat16, device="cuda")
+    x, xf = _x(rng, 9, K, torch.bfloat16)
+    wide[:, 1:K + 1] = x
+    view = wide[:, 1:K + 1]
+    assert view.stride(0) == K + 3 and view.data_ptr() % 16 != 0
+    _check(nvq_matmul(lin.weight, view).cpu().numpy(), O.linear_forward_f64(want, xf))
+    big = torch.from_numpy((rng.standard_normal((7, K)) * 2.0e6).astype(np.float32)).to(torch.bfloat16).cuda()
+    _check(nvq_matmul(lin.weight, big).cpu().numpy() / 2.0e6, O.linear_forward_f64(want, big.float().cpu().numpy()) / 2.0e6)
+
+
 @pytest.mark.parametrize("family", ["NVQ3J-512", "NEPQ0-L", "NEPQ1-S", "MXFP8"])
 def test_reserve_sizes_the_workspace_of_every_family(family):
     """QuantLinear.reserve(max_rows) on an NVQ, an NEPQ0 (bit streams in place), an NEPQ1 and an MX linear: forward() of

@@ -395,6 +395,8 @@ __device__ __forceinline__ uint32_t e8_pair(int a, int b) {
     }
 }
 constexpr int kE8Waves = 16;
+// bytes staged for a bit range of `bits` bits that starts anywhere in its first 16 bytes, with room for a field's two dwords
+__host__ __device__ inline uint32_t nvqs_e8_range_bytes(int64_t bits) { return static_cast<uint32_t>((16 + (bits + 7) / 8 + 8 + 15) / 16 * 16); }
 struct E8Shape {
     int npw;            // consecutive neurons per wave
     int kp;             // staged elements of a row: whole groups of 24
@@ -662,6 +664,229 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
     }
 }
 
+
+// ---- the same formats for up to 16 rows on the matrix cores ------------------------------------------------------------
+// nvqs_e8_kernel reads a row's activations again for every block of weights, so its time grows with the rows.  Here a
+// block owns 16 consecutive neurons: their three bit ranges (contiguous in the streams) are staged whole, the waves
+// split the groups of 24 weights, and lane (n, kb) -- neuron n = lane % 16, block kb = lane / 16 of the group, the lanes
+// of kb = 3 idle -- decodes one 8-weight block, which is its B fragment of a 16 x 16 x 32 product against the rows'
+// 24 activations of the group (A fragment: row lane % 16, the same block; zeros for kb = 3).  The product's four
+// results of a lane belong to its own neuron, whose group scale it has decoded, and are scaled and added in fp32.
+// The waves' partial sums meet in LDS.  The 16 neurons of a wave read their fields at a stride of the neuron's bytes in
+// the stream -- 512 bytes of index bytes for K = 4096, one LDS bank for all of them -- so the staged copy of a range
+// skips a bank after every 2^pad bytes, with pad chosen per range so that the 16 strides spread over the banks.
+// LDS map (bytes): [entries][256 sign patterns x 16][state table 128][pool scale tables][index | sign | state ranges]
+// [partial sums: waves x 1024]
+struct E8TileShape {
+    int gpw;            // groups of 24 weights per wave
+    uint32_t cap[3];    // LDS bytes of the block's index / sign / state range, padding included
+    uint32_t pad[3];    // log2 of the bytes of a range after which its LDS copy skips a bank (31: no padding)
+    uint32_t lds_bytes;
+};
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+template <int XF16>
+__device__ __forceinline__ float4_t e8_mfma(u32x4_t a, u32x4_t b, float4_t c) {
+    if constexpr (XF16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+template <int XF16>
+__global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k, const uint8_t *__restrict__ w,
+                                                                     const uint16_t *__restrict__ x, int64_t ldx, int M,
+                                                                     float *__restrict__ y, int64_t ldy, E8TileShape sh) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds32[];
+    typedef __attribute__((address_space(3))) const u32x4_t *lds_u32x4_ptr;
+    typedef __attribute__((address_space(3))) const u32x2_t *lds_u32x2_ptr;
+    typedef __attribute__((address_space(3))) const uint32_t *lds_u32_ptr;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ncb = k.kind == 2 ? k.cb_bytes / k.vs : (k.kind == 3 ? k.nbank * k.bank_bytes / k.vs : k.banks * k.entries);
+    uint8_t *lds8 = reinterpret_cast<uint8_t *>(lds32);
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)lds8));
+    const uint32_t esz = static_cast<uint32_t>(k.vs) * 2u;
+    const uint32_t sgn_off = static_cast<uint32_t>(ncb) * esz, stab_off = sgn_off + 4096u, lut3_off = stab_off + 128u;
+    uint32_t roff[3];
+    roff[0] = lut3_off + (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * 32u : 0u);
+    roff[1] = roff[0] + sh.cap[0];
+    roff[2] = roff[1] + sh.cap[1];
+    const uint32_t red_off = roff[2] + sh.cap[2];
+
+    // ---- the block's stream ranges: 16-byte pieces, four requests of a thread in flight ----------------------------
+    const int row_first = static_cast<int>(blockIdx.x) * 16;
+    const int nn = min(16, k.nrows - row_first);  // >= 1: the grid has no block past the last neuron
+    const int64_t n0 = k.row0 + row_first;
+    const uint32_t per[3] = {static_cast<uint32_t>(k.nvec) * static_cast<uint32_t>(k.ib),
+                             k.kind == 0 ? static_cast<uint32_t>(k.nsign) * 7u
+                                         : (k.kind == 1 ? static_cast<uint32_t>(k.ng) : (k.kind == 3 ? static_cast<uint32_t>(k.nsuper) * 8u : 0u)),
+                             static_cast<uint32_t>(k.ng) * static_cast<uint32_t>(k.sbits)};
+    const int64_t region[3] = {k.index_off, k.sign_off, k.state_off};
+    const int64_t region_bytes[3] = {k.index_bytes + 4, k.sign_bytes + 4, k.state_bytes + 4};
+    uint32_t shift[3];  // bits between the staged range's first bit and the first bit of neuron n0
+    // the tables' first requests go out with the stream ranges'
+    const float *lut = nvqs_lut(k, w);
+    const uint32_t *bfs = reinterpret_cast<const uint32_t *>(lut + 16);
+    const int8_t *cbp = reinterpret_cast<const int8_t *>(bfs + 16);
+    const int nslot = ncb * k.vs / 8;  // slot e: eight int8 values -> eight values of the activations' type
+    const u32x2_t raw0 = tid < nslot ? *reinterpret_cast<const u32x2_t *>(cbp + static_cast<int64_t>(tid) * 8) : u32x2_t{0u, 0u};
+    const float lutv = lut[tid & 15];
+    const uint32_t bfsv = bfs[tid & 15];
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+        const int64_t bit0 = n0 * static_cast<int64_t>(per[r]);
+        const int64_t a0 = (bit0 >> 3) & ~static_cast<int64_t>(15);
+        shift[r] = static_cast<uint32_t>(bit0 - a0 * 8);
+        const int64_t left = region_bytes[r] - a0;
+        const __amdgpu_buffer_rsrc_t win =
+            wave_window(w + region[r] + a0, static_cast<uint32_t>(left <= 0 ? 0 : (left < (1ll << 31) ? left : (1ll << 31))));
+        const uint32_t raw = nvqs_e8_range_bytes(16ll * per[r]);  // stream bytes of the range
+        for (uint32_t p0 = static_cast<uint32_t>(tid) * 16u; p0 < raw; p0 += 4u * 64u * kE8Waves * 16u) {
+            u32x4_t piece[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t off = p0 + static_cast<uint32_t>(t) * 64u * kE8Waves * 16u;
+                piece[t] = __builtin_amdgcn_raw_buffer_load_b128(win, off < raw ? off : kNoStep, 0, 2);
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t off = p0 + static_cast<uint32_t>(t) * 64u * kE8Waves * 16u;
+                if (off < raw) {  // (a piece lies inside one padding period: they are 64 bytes and more)
+                    uint32_t *dst = reinterpret_cast<uint32_t *>(lds8 + roff[r] + off + ((off >> sh.pad[r]) << 2));
+                    dst[0] = piece[t].x; dst[1] = piece[t].y; dst[2] = piece[t].z; dst[3] = piece[t].w;
+                }
+            }
+        }
+    }
+    // ---- tables -------------------------------------------------------------------------------------------------------
+    for (int e = tid; e < nslot; e += blockDim.x) {
+        const u32x2_t raw = e == tid ? raw0 : *reinterpret_cast<const u32x2_t *>(cbp + static_cast<int64_t>(e) * 8);
+        u32x4_t v;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t src = t < 2 ? raw.x : raw.y;
+            const int a = static_cast<int8_t>((src >> (16 * (t & 1))) & 0xffu), b = static_cast<int8_t>((src >> (16 * (t & 1) + 8)) & 0xffu);
+            v[t] = e8_pair<XF16>(a, b);
+        }
+        *reinterpret_cast<u32x4_t *>(lds8 + static_cast<uint32_t>(e) * 16u) = v;
+    }
+    for (int e = tid; e < 256; e += blockDim.x) {
+        u32x4_t v;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) v[t] = (((e >> (2 * t)) & 1u) << 15) | (((e >> (2 * t + 1)) & 1u) << 31);
+        *reinterpret_cast<u32x4_t *>(lds8 + sgn_off + static_cast<uint32_t>(e) * 16u) = v;
+    }
+    if (tid < 16) {
+        float *st = reinterpret_cast<float *>(lds8 + stab_off);
+        st[2 * tid] = lutv;
+        reinterpret_cast<uint32_t *>(st)[2 * tid + 1] = lds_base + bfsv * static_cast<uint32_t>(k.entries) * esz;
+    }
+    if (k.kind == 3) {
+        const float *lut3 = reinterpret_cast<const float *>(reinterpret_cast<const uint8_t *>(lut) + 128 + static_cast<int64_t>(k.nbank) * k.bank_bytes);
+        for (int i = tid; i < k.nbank * 8; i += blockDim.x) *reinterpret_cast<float *>(lds8 + lut3_off + static_cast<uint32_t>(i) * 4u) = lut3[i];
+    }
+    __syncthreads();
+
+    // `nbits` (<= 25) bits at bit position `bit` of staged range r
+    auto field = [&](int r, uint32_t bit, uint32_t nbits) -> uint32_t {
+        const uint32_t b0 = (bit >> 5) << 2, b1 = b0 + 4u;
+        const u32x2_t d = u32x2_t{*reinterpret_cast<lds_u32_ptr>(lds_base + roff[r] + b0 + ((b0 >> sh.pad[r]) << 2)),
+                                  *reinterpret_cast<lds_u32_ptr>(lds_base + roff[r] + b1 + ((b1 >> sh.pad[r]) << 2))};
+        return __builtin_amdgcn_alignbit(d.y, d.x, bit & 31u) & ((1u << nbits) - 1u);
+    };
+    const int r16 = lane & 15, kb = lane >> 4;
+    const uint32_t nloc = static_cast<uint32_t>(min(r16, nn - 1));  // lanes past the last neuron repeat it; their sums are not stored
+    const uint32_t ixb = shift[0] + nloc * per[0], sgb = shift[1] + nloc * per[1], stb = shift[2] + nloc * per[2];
+    const bool xrow_ok = r16 < M && kb < 3;
+    const uint16_t *xr = x + static_cast<int64_t>(min(r16, M - 1)) * ldx;
+    const bool vec = ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    auto x_frag = [&](int g) -> u32x4_t {  // the row's eight activations of block kb of group g; zeros past K and for kb = 3
+        u32x4_t v = {0u, 0u, 0u, 0u};
+        const int c0 = (3 * g + kb) * 8;
+        if (xrow_ok && g < k.ng && c0 < k.neuron_len) {
+            if (vec && c0 + 8 <= k.neuron_len) {
+                v = *reinterpret_cast<const u32x4_t *>(xr + c0);
+            } else {
+                uint32_t h[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = c0 + i < k.neuron_len ? xr[c0 + i] : 0u;
+                v = u32x4_t{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+            }
+        }
+        return v;
+    };
+    const uint32_t ones = XF16 ? 0x3c003c00u : 0x3f803f80u;
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const int g0 = wave * sh.gpw, g1 = min(k.ng, g0 + sh.gpw);
+    for (int gq = g0; gq < g1; gq += 4) {
+        u32x4_t xf[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) xf[t] = x_frag(gq + t < g1 ? gq + t : k.ng);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int g = min(gq + t, g1 - 1);  // past the wave's last group: that group again, against zero activations
+            const uint32_t sb = static_cast<uint32_t>(3 * g + min(kb, 2));  // the lanes of kb = 3 meet zero activations
+            const uint32_t state = field(2, stb + static_cast<uint32_t>(k.sbits) * g, k.sbits);
+            const u32x2_t se = *reinterpret_cast<lds_u32x2_ptr>(lds_base + stab_off + state * 8u);
+            float sc = __uint_as_float(se.x);
+            u32x4_t wv;
+            float4_t part = {0.f, 0.f, 0.f, 0.f};
+            if (k.kind == 0) {
+                const uint32_t mk = field(1, sgb + 7u * sb, 7);
+                uint32_t last = __popc(mk) & 1u;
+                u32x4_t ev;
+                if (k.vs == 4) {
+                    const uint32_t i0 = field(0, ixb + (2u * sb) * k.ib, k.ib);
+                    const uint32_t i1 = 2u * sb + 1u < static_cast<uint32_t>(k.nvec) ? field(0, ixb + (2u * sb + 1u) * k.ib, k.ib) : 0u;
+                    const u32x2_t e0 = *reinterpret_cast<lds_u32x2_ptr>(se.y + i0 * 8u), e1 = *reinterpret_cast<lds_u32x2_ptr>(se.y + i1 * 8u);
+                    ev = u32x4_t{e0.x, e0.y, e1.x, e1.y};
+                } else {
+                    const uint32_t idx = field(0, ixb + sb * k.ib, k.ib);
+                    if (k.index_parity) last ^= (idx >> 7) & 1u;
+                    ev = *reinterpret_cast<lds_u32x4_ptr>(se.y + idx * 16u);
+                }
+                const u32x4_t sv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + sgn_off + (mk | (last << 7)) * 16u);
+                wv = ev ^ sv;
+            } else {
+                const uint32_t idx = sb < static_cast<uint32_t>(k.nvec) ? field(0, ixb + sb * k.ib, k.ib) : 0u;
+                if (k.kind == 1) {
+                    const uint32_t neg = field(1, sgb + g, 1);
+                    wv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + ((k.banks == 2 ? neg : 0u) * static_cast<uint32_t>(k.entries) + idx) * 16u);
+                    // w = scale * (code + d): d times the sum of the group's activations, as a product with ones
+                    const float dl = neg ? -k.delta : k.delta;
+                    const float4_t xs = e8_mfma<XF16>(xf[t], u32x4_t{ones, ones, ones, ones}, float4_t{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) part[v] = dl * xs[v];
+                } else {
+                    uint32_t tbase = 0u;
+                    if (k.kind == 3) {
+                        const uint32_t pb = min(field(1, sgb + 8u * (static_cast<uint32_t>(g) >> 2), 8), static_cast<uint32_t>(k.nbank - 1));
+                        tbase = pb * static_cast<uint32_t>(k.bank_bytes) * 2u;
+                        sc = __uint_as_float(*reinterpret_cast<lds_u32_ptr>(lds_base + lut3_off + (pb * 8u + state) * 4u));
+                    }
+                    const u32x2_t e0 = *reinterpret_cast<lds_u32x2_ptr>(lds_base + tbase + (state * 8u + (idx & 7u)) * 8u);
+                    const u32x2_t e1 = *reinterpret_cast<lds_u32x2_ptr>(lds_base + tbase + (static_cast<uint32_t>(k.banks) * 8u + state * static_cast<uint32_t>(k.entries) + (idx >> 3)) * 8u);
+                    wv = u32x4_t{e0.x, e0.y, e1.x, e1.y};
+                }
+            }
+            part = e8_mfma<XF16>(xf[t], wv, part);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[v] = fmaf(sc, part[v], acc[v]);
+        }
+    }
+    // ---- the waves' partial sums: red[wave][row][neuron] ------------------------------------------------------------
+    float *red = reinterpret_cast<float *>(lds8 + red_off);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave * 256 + (4 * kb + v) * 16 + r16] = acc[v];
+    __syncthreads();
+    if (tid < 256) {
+        const int m = tid >> 4, n = tid & 15;
+        float sum = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < kE8Waves; ++wv) sum += red[wv * 256 + tid];
+        if (m < M && n < nn) y[static_cast<int64_t>(m) * ldy + row_first + n] = sum * reinterpret_cast<const float *>(w + k.anchors_off)[n0 + n];
+    }
+}
+
 int gemm_f16_nt(const void *a, int64_t lda, const void *b, int64_t ldb, int M, int N, int K, const float *sa,
                 const float *sb, float *y, int64_t ldy, hipStream_t st, float *part = nullptr);
 float *dequant_gemm_part(float *wscale, int N, int K, int M);
@@ -678,7 +903,7 @@ constexpr int kNvqsGemvMaxM = 16;  // rows up to which the weights are re-read p
 // requests at most), and the 1-bit families NVQ1-L / NVQ1-S (ternary 8-vectors, a delta sign per group) and NPQ0-L /
 // NPQ0-S (two 4-vectors per block; NEPQ0-S / NEPQ0-L: out of a pool of tables that fits the LDS) with their states of
 // 2 to 4 bits.  MB = rows per pass that fit the LDS.
-static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
+static bool nvqs_e8_format(const NvqsK &k) {
     static const int off = tune_env("MFQ_NVQS_E8_OFF", 0);
     if (off || k.index_bytes >= (1ll << 31) || k.sign_bytes >= (1ll << 31)) return false;
     if (k.kind == 0) {
@@ -691,7 +916,20 @@ static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     } else {
         return false;
     }
-    auto cap = [](int64_t bits) { return static_cast<uint32_t>((16 + (bits + 7) / 8 + 8 + 15) / 16 * 16); };
+    return true;
+}
+static uint32_t nvqs_e8_table_bytes(const NvqsK &k) {  // the tables as int8
+    return k.kind == 2 ? static_cast<uint32_t>(k.cb_bytes)
+                       : (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * static_cast<uint32_t>(k.bank_bytes)
+                                      : static_cast<uint32_t>(k.banks) * static_cast<uint32_t>(k.entries) * static_cast<uint32_t>(k.vs));
+}
+static int64_t nvqs_e8_sign_bits(const NvqsK &k) {  // bits per neuron of the second staged range
+    return k.kind == 0 ? static_cast<int64_t>(k.nsign) * 7 : (k.kind == 1 ? k.ng : (k.kind == 3 ? k.nsuper * 8 : 0));
+}
+static uint32_t nvqs_e8_cap(int64_t bits) { return nvqs_e8_range_bytes(bits); }
+static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
+    if (!nvqs_e8_format(k)) return false;
+    auto cap = nvqs_e8_cap;
     int npw = static_cast<int>(ceil_div(k.nrows, static_cast<int64_t>(gemv_cu_count()) * kE8Waves));
     if (npw > 4) npw = 4;
     while (npw > 1 && cap(static_cast<int64_t>(npw) * k.nvec * k.ib) > 2048) --npw;
@@ -699,18 +937,55 @@ static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     sh.npw = npw;
     sh.kp = k.ng * 24;
     sh.cap[0] = cap(static_cast<int64_t>(npw) * k.nvec * k.ib);
-    sh.cap[1] = cap(static_cast<int64_t>(npw) * (k.kind == 0 ? static_cast<int64_t>(k.nsign) * 7 : (k.kind == 1 ? k.ng : (k.kind == 3 ? k.nsuper * 8 : 0))));
+    sh.cap[1] = cap(static_cast<int64_t>(npw) * nvqs_e8_sign_bits(k));
     sh.cap[2] = cap(static_cast<int64_t>(npw) * k.ng * k.sbits);
     sh.wave_bytes = sh.cap[0] + sh.cap[1] + sh.cap[2];
-    for (mb = M >= 8 ? 8 : (M >= 4 ? 4 : (M >= 2 ? 2 : 1)); mb >= 1; mb >>= 1) {
-        const uint32_t table = k.kind == 2 ? static_cast<uint32_t>(k.cb_bytes)
-                             : (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * static_cast<uint32_t>(k.bank_bytes)
-                                            : static_cast<uint32_t>(k.banks) * static_cast<uint32_t>(k.entries) * static_cast<uint32_t>(k.vs));
+    for (mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1); mb >= 1; mb >>= 1) {  // (five rows and more go to the matrix-core form)
+        const uint32_t table = nvqs_e8_table_bytes(k);
         if (table > kMaxDynamicLds / 2) return false;
         sh.lds_bytes = table * 2u + 4096u + 128u + (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * 32u : 0u) + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
         if (sh.lds_bytes <= kMaxDynamicLds) return true;
     }
     return false;
+}
+// The matrix-core form: from MFQ_NVQS_TILE_MIN_M rows on, when the 16 neurons' ranges and the tables fit the LDS.
+static bool nvqs_e8_tile_shape(const NvqsK &k, int M, E8TileShape &sh) {
+    static const int min_m = tune_env("MFQ_NVQS_TILE_MIN_M", 5);
+    if (M < min_m || M > 16 || !nvqs_e8_format(k)) return false;
+    const int64_t bits[3] = {16ll * k.nvec * k.ib, 16ll * nvqs_e8_sign_bits(k), 16ll * k.ng * k.sbits};
+    uint64_t total = static_cast<uint64_t>(nvqs_e8_table_bytes(k)) * 2u + 4096u + 128u + (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * 32u : 0u) +
+                     kE8Waves * 1024u;
+    for (int r = 0; r < 3; ++r) {
+        if (bits[r] > (1ll << 22)) return false;
+        // the padding period under which the first dwords of the 16 neurons spread best over 32 banks
+        const uint32_t raw = nvqs_e8_range_bytes(bits[r]);
+        const int periods[6] = {31, 6, 7, 8, 9, 10};
+        int best = 17;
+        for (int pi = 0; pi < 6; ++pi) {
+            int hits[32] = {0}, worst = 0;
+            for (int n = 0; n < 16; ++n) {
+                const uint32_t b = static_cast<uint32_t>(n * (bits[r] / 16) / 32) * 4u;
+                const int bank = static_cast<int>(((b + ((b >> periods[pi]) << 2)) >> 2) & 31u);
+                if (++hits[bank] > worst) worst = hits[bank];
+            }
+            if (worst < best) { best = worst; sh.pad[r] = static_cast<uint32_t>(periods[pi]); }
+        }
+        sh.cap[r] = (raw + ((raw >> sh.pad[r]) << 2) + 16u + 15u) / 16u * 16u;
+        total += sh.cap[r];
+    }
+    if (total > kMaxDynamicLds) return false;
+    sh.lds_bytes = static_cast<uint32_t>(total);
+    sh.gpw = static_cast<int>(ceil_div(k.ng, kE8Waves));
+    return true;
+}
+template <int XF16>
+static int nvqs_launch_e8_tile(const NvqsK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
+                               const E8TileShape &sh, hipStream_t st) {
+    auto kern = nvqs_e8_tile_kernel<XF16>;
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), sh.lds_bytes, "nvqs_e8_tile")) return rc;
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(ceil_div(k.nrows, 16))), dim3(64 * kE8Waves), sh.lds_bytes, st, k, w, x, ldx,
+                       M, y, ldy, sh);
+    return check_launch("nvqs_e8_tile");
 }
 template <int XF16>
 static int nvqs_launch_e8(const NvqsK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy, int mb,
@@ -724,7 +999,7 @@ static int nvqs_launch_e8(const NvqsK &k, const uint8_t *w, const uint16_t *x, i
         hipLaunchKernelGGL(kern, grid, dim3(64 * kE8Waves), sh.lds_bytes, st, k, w, x, ldx, M, y, ldy, sh, sel);       \
         return check_launch("nvqs_e8");                                                                               \
     }
-    MFQ_E8(1) MFQ_E8(2) MFQ_E8(4) MFQ_E8(8)
+    MFQ_E8(1) MFQ_E8(2) MFQ_E8(4)
 #undef MFQ_E8
     return fail(MFQ_ERR_UNSUPPORTED, "nvqs_e8: %d rows per pass", mb);
 }
@@ -994,6 +1269,10 @@ extern "C" int mfq_hip_nvqs_gemv_rows(const mfq_nvqs_desc *d, const void *weight
     const uint16_t *xp = static_cast<const uint16_t *>(x);
     hipStream_t st = as_stream(stream);
     {
+        E8TileShape ts;
+        if (nvqs_e8_tile_shape(k, M, ts))
+            return x_dtype == MFQ_X_F16 ? nvqs_launch_e8_tile<1>(k, w, xp, ldx, M, y, ldy, ts, st)
+                                        : nvqs_launch_e8_tile<0>(k, w, xp, ldx, M, y, ldy, ts, st);
         int mb;
         E8Shape sh;
         if (nvqs_e8_shape(k, M, mb, sh))
