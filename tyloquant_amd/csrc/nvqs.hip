@@ -665,14 +665,15 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
 }
 
 
-// ---- the same formats for up to 16 rows on the matrix cores ------------------------------------------------------------
+// ---- the same formats for 5 to 128 rows on the matrix cores -----------------------------------------------------------
 // nvqs_e8_kernel reads a row's activations again for every block of weights, so its time grows with the rows.  Here a
 // block owns 16 consecutive neurons: their three bit ranges (contiguous in the streams) are staged whole, the waves
 // split the groups of 24 weights, and lane (n, kb) -- neuron n = lane % 16, block kb = lane / 16 of the group, the lanes
 // of kb = 3 idle -- decodes one 8-weight block, which is its B fragment of a 16 x 16 x 32 product against the rows'
 // 24 activations of the group (A fragment: row lane % 16, the same block; zeros for kb = 3).  The product's four
 // results of a lane belong to its own neuron, whose group scale it has decoded, and are scaled and added in fp32.
-// The waves' partial sums meet in LDS.  The 16 neurons of a wave read their fields at a stride of the neuron's bytes in
+// The waves' partial sums meet in LDS.  Above 16 rows a block takes two 16-row tiles (blockIdx.y counts pairs of tiles),
+// which share every decoded fragment.  The 16 neurons of a wave read their fields at a stride of the neuron's bytes in
 // the stream -- 512 bytes of index bytes for K = 4096, one LDS bank for all of them -- so the staged copy of a range
 // skips a bank after every 2^pad bytes, with pad chosen per range so that the 16 strides spread over the banks.
 // LDS map (bytes): [entries][256 sign patterns x 16][state table 128][pool scale tables][index | sign | state ranges]
@@ -691,7 +692,7 @@ __device__ __forceinline__ float4_t e8_mfma(u32x4_t a, u32x4_t b, float4_t c) {
     else
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
-template <int XF16>
+template <int XF16, int MT>
 __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k, const uint8_t *__restrict__ w,
                                                                      const uint16_t *__restrict__ x, int64_t ldx, int M,
                                                                      float *__restrict__ y, int64_t ldy, E8TileShape sh) {
@@ -796,13 +797,14 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
     const int r16 = lane & 15, kb = lane >> 4;
     const uint32_t nloc = static_cast<uint32_t>(min(r16, nn - 1));  // lanes past the last neuron repeat it; their sums are not stored
     const uint32_t ixb = shift[0] + nloc * per[0], sgb = shift[1] + nloc * per[1], stb = shift[2] + nloc * per[2];
-    const bool xrow_ok = r16 < M && kb < 3;
-    const uint16_t *xr = x + static_cast<int64_t>(min(r16, M - 1)) * ldx;
+    const int m0 = static_cast<int>(blockIdx.y) * 16 * MT;  // the block's MT tiles of 16 rows share every decoded fragment
     const bool vec = ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
-    auto x_frag = [&](int g) -> u32x4_t {  // the row's eight activations of block kb of group g; zeros past K and for kb = 3
+    // the eight activations of block kb of group g of the lane's row in tile mt; zeros past M and K and for kb = 3
+    auto x_frag = [&](int g, int mt) -> u32x4_t {
         u32x4_t v = {0u, 0u, 0u, 0u};
-        const int c0 = (3 * g + kb) * 8;
-        if (xrow_ok && g < k.ng && c0 < k.neuron_len) {
+        const int c0 = (3 * g + kb) * 8, m = m0 + 16 * mt + r16;
+        const uint16_t *xr = x + static_cast<int64_t>(min(m, M - 1)) * ldx;
+        if (m < M && kb < 3 && g < k.ng && c0 < k.neuron_len) {
             if (vec && c0 + 8 <= k.neuron_len) {
                 v = *reinterpret_cast<const u32x4_t *>(xr + c0);
             } else {
@@ -815,21 +817,26 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
         return v;
     };
     const uint32_t ones = XF16 ? 0x3c003c00u : 0x3f803f80u;
-    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    constexpr int GT = MT == 1 ? 4 : 2;  // groups whose activations are requested together
+    float4_t acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
     const int g0 = wave * sh.gpw, g1 = min(k.ng, g0 + sh.gpw);
-    for (int gq = g0; gq < g1; gq += 4) {
-        u32x4_t xf[4];
+    for (int gq = g0; gq < g1; gq += GT) {
+        u32x4_t xf[GT][MT];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) xf[t] = x_frag(gq + t < g1 ? gq + t : k.ng);
+        for (int t = 0; t < GT; ++t)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+            for (int mt = 0; mt < MT; ++mt) xf[t][mt] = x_frag(gq + t < g1 ? gq + t : k.ng, mt);
+#pragma unroll
+        for (int t = 0; t < GT; ++t) {
             const int g = min(gq + t, g1 - 1);  // past the wave's last group: that group again, against zero activations
             const uint32_t sb = static_cast<uint32_t>(3 * g + min(kb, 2));  // the lanes of kb = 3 meet zero activations
             const uint32_t state = field(2, stb + static_cast<uint32_t>(k.sbits) * g, k.sbits);
             const u32x2_t se = *reinterpret_cast<lds_u32x2_ptr>(lds_base + stab_off + state * 8u);
             float sc = __uint_as_float(se.x);
             u32x4_t wv;
-            float4_t part = {0.f, 0.f, 0.f, 0.f};
+            float dl = 0.f;
             if (k.kind == 0) {
                 const uint32_t mk = field(1, sgb + 7u * sb, 7);
                 uint32_t last = __popc(mk) & 1u;
@@ -852,10 +859,7 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
                     const uint32_t neg = field(1, sgb + g, 1);
                     wv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + ((k.banks == 2 ? neg : 0u) * static_cast<uint32_t>(k.entries) + idx) * 16u);
                     // w = scale * (code + d): d times the sum of the group's activations, as a product with ones
-                    const float dl = neg ? -k.delta : k.delta;
-                    const float4_t xs = e8_mfma<XF16>(xf[t], u32x4_t{ones, ones, ones, ones}, float4_t{0.f, 0.f, 0.f, 0.f});
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) part[v] = dl * xs[v];
+                    dl = neg ? -k.delta : k.delta;
                 } else {
                     uint32_t tbase = 0u;
                     if (k.kind == 3) {
@@ -868,22 +872,35 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
                     wv = u32x4_t{e0.x, e0.y, e1.x, e1.y};
                 }
             }
-            part = e8_mfma<XF16>(xf[t], wv, part);
 #pragma unroll
-            for (int v = 0; v < 4; ++v) acc[v] = fmaf(sc, part[v], acc[v]);
+            for (int mt = 0; mt < MT; ++mt) {
+                float4_t part = {0.f, 0.f, 0.f, 0.f};
+                if (k.kind == 1) {
+                    const float4_t xs = e8_mfma<XF16>(xf[t][mt], u32x4_t{ones, ones, ones, ones}, float4_t{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) part[v] = dl * xs[v];
+                }
+                part = e8_mfma<XF16>(xf[t][mt], wv, part);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[mt][v] = fmaf(sc, part[v], acc[mt][v]);
+            }
         }
     }
     // ---- the waves' partial sums: red[wave][row][neuron] ------------------------------------------------------------
     float *red = reinterpret_cast<float *>(lds8 + red_off);
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave * 256 + (4 * kb + v) * 16 + r16] = acc[v];
-    __syncthreads();
-    if (tid < 256) {
-        const int m = tid >> 4, n = tid & 15;
-        float sum = 0.f;
+    for (int mt = 0; mt < MT; ++mt) {  // one tile at a time through the same 16 KB
+        if (mt > 0) __syncthreads();
 #pragma unroll
-        for (int wv = 0; wv < kE8Waves; ++wv) sum += red[wv * 256 + tid];
-        if (m < M && n < nn) y[static_cast<int64_t>(m) * ldy + row_first + n] = sum * reinterpret_cast<const float *>(w + k.anchors_off)[n0 + n];
+        for (int v = 0; v < 4; ++v) red[wave * 256 + (4 * kb + v) * 16 + r16] = acc[mt][v];
+        __syncthreads();
+        if (tid < 256) {
+            const int m = m0 + 16 * mt + (tid >> 4), n = tid & 15;
+            float sum = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < kE8Waves; ++wv) sum += red[wv * 256 + tid];
+            if (m < M && n < nn) y[static_cast<int64_t>(m) * ldy + row_first + n] = sum * reinterpret_cast<const float *>(w + k.anchors_off)[n0 + n];
+        }
     }
 }
 
@@ -896,6 +913,7 @@ void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&x
                         int &Kp);
 
 constexpr int kNvqsGemvMaxM = 16;  // rows up to which the weights are re-read per pass of eight rows
+constexpr int kNvqsTileMaxM = 128;  // rows up to which the formats of the matrix-core tile kernel stay on it
 
 // The E8 kernel takes the sign-stream format with 8- or 4-dimensional vectors, 4-bit states and tables that fit the LDS
 // in the activations' type (E8: 256 or 1024 entries in up to four banks, 4096 in one; D4: 1024 entries), tensors whose streams fit 32-bit offsets and
@@ -951,7 +969,8 @@ static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
 // The matrix-core form: from MFQ_NVQS_TILE_MIN_M rows on, when the 16 neurons' ranges and the tables fit the LDS.
 static bool nvqs_e8_tile_shape(const NvqsK &k, int M, E8TileShape &sh) {
     static const int min_m = tune_env("MFQ_NVQS_TILE_MIN_M", 5);
-    if (M < min_m || M > 16 || !nvqs_e8_format(k)) return false;
+    static const int max_m = tune_env("MFQ_NVQS_TILE_MAX_M", kNvqsTileMaxM);
+    if (M < min_m || M > max_m || !nvqs_e8_format(k)) return false;
     const int64_t bits[3] = {16ll * k.nvec * k.ib, 16ll * nvqs_e8_sign_bits(k), 16ll * k.ng * k.sbits};
     uint64_t total = static_cast<uint64_t>(nvqs_e8_table_bytes(k)) * 2u + 4096u + 128u + (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * 32u : 0u) +
                      kE8Waves * 1024u;
@@ -981,11 +1000,19 @@ static bool nvqs_e8_tile_shape(const NvqsK &k, int M, E8TileShape &sh) {
 template <int XF16>
 static int nvqs_launch_e8_tile(const NvqsK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                                const E8TileShape &sh, hipStream_t st) {
-    auto kern = nvqs_e8_tile_kernel<XF16>;
-    if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), sh.lds_bytes, "nvqs_e8_tile")) return rc;
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(ceil_div(k.nrows, 16))), dim3(64 * kE8Waves), sh.lds_bytes, st, k, w, x, ldx,
-                       M, y, ldy, sh);
-    return check_launch("nvqs_e8_tile");
+    // one or two 16-row tiles per block, which share every decoded fragment (four per block measured no faster than two
+    // blocks of two: every block reads its rows' activations again, and that traffic grows with the tiles)
+#define MFQ_E8_TILE(MTV)                                                                                              \
+    {                                                                                                                 \
+        auto kern = nvqs_e8_tile_kernel<XF16, MTV>;                                                                   \
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), sh.lds_bytes, "nvqs_e8_tile")) return rc; \
+        hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(ceil_div(k.nrows, 16)), static_cast<unsigned>(ceil_div(M, 16 * MTV))), \
+                           dim3(64 * kE8Waves), sh.lds_bytes, st, k, w, x, ldx, M, y, ldy, sh);                        \
+        return check_launch("nvqs_e8_tile");                                                                          \
+    }
+    if (M <= 16) MFQ_E8_TILE(1)
+    MFQ_E8_TILE(2)
+#undef MFQ_E8_TILE
 }
 template <int XF16>
 static int nvqs_launch_e8(const NvqsK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy, int mb,
@@ -1295,8 +1322,13 @@ extern "C" int mfq_hip_nvqs_gemv(const mfq_nvqs_desc *d, const void *weight, con
     return mfq_hip_nvqs_gemv_rows(d, weight, 0, d->out, x, x_dtype, ldx, M, y, ldy, stream);
 }
 
+// batches above the GEMV range that the matrix-core tile kernel takes (no workspace)
+static bool nvqs_tile_takes(const mfq_nvqs_desc *d, int M) {
+    E8TileShape ts;
+    return nvqs_e8_tile_shape(to_k(d), M, ts);
+}
 extern "C" size_t mfq_hip_nvqs_gemm_rows_workspace_bytes(const mfq_nvqs_desc *d, int nrows, int M) {
-    if (!d || M <= kNvqsGemvMaxM) return 0;
+    if (!d || M <= kNvqsGemvMaxM || nvqs_tile_takes(d, M)) return 0;
     return dequant_gemm_workspace(nrows, d->neuron_len, M);
 }
 extern "C" size_t mfq_hip_nvqs_gemm_workspace_bytes(const mfq_nvqs_desc *d, int M) {
@@ -1307,7 +1339,8 @@ extern "C" int mfq_hip_nvqs_gemm_rows(const mfq_nvqs_desc *d, const void *weight
                                       int x_dtype, int64_t ldx, int M, float *y, int64_t ldy, void *workspace,
                                       size_t workspace_bytes, mfq_stream_t stream) {
     MFQ_REQUIRE(d && weight && x && y, MFQ_ERR_INVALID, "nvqs_gemm: null argument");
-    if (M <= kNvqsGemvMaxM) return mfq_hip_nvqs_gemv_rows(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, stream);
+    if (M <= kNvqsGemvMaxM || nvqs_tile_takes(d, M))
+        return mfq_hip_nvqs_gemv_rows(d, weight, row0, nrows, x, x_dtype, ldx, M, y, ldy, stream);
     MFQ_REQUIRE(x_dtype == MFQ_X_BF16 || x_dtype == MFQ_X_F16, MFQ_ERR_INVALID, "nvqs_gemm: x_dtype=%d", x_dtype);
     MFQ_REQUIRE(nvqs_rows_ok(d, row0, nrows), MFQ_ERR_INVALID, "nvqs_gemm: rows [%d, %d) outside the tensor's %d", row0,
                 row0 + nrows, d->out);
