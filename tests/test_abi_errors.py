@@ -92,7 +92,7 @@ def test_row_ranges_must_lie_inside_the_tensor(lib):
         rc = lib.mfq_hip_nvqs_gemv_rows(C.byref(v), FAKE, row0, nrows, FAKE, L.X_BF16, 96, 1, FAKE, 64, None)
         assert rc == L.ERR_INVALID and "outside the tensor" in _msg(lib)
         assert lib.mfq_hip_nvqs_dequant_rows_f32(C.byref(v), FAKE, row0, nrows, FAKE, 96, None) == L.ERR_INVALID
-    assert lib.mfq_hip_nvqs_gemm_rows(C.byref(v), FAKE, 0, 32, FAKE, L.X_BF16, 96, 64, FAKE, 32, None, 0, None) == L.ERR_WORKSPACE
+    assert lib.mfq_hip_nvqs_gemm_rows(C.byref(v), FAKE, 0, 32, FAKE, L.X_BF16, 96, 200, FAKE, 32, None, 0, None) == L.ERR_WORKSPACE
 
 
 def test_moe_helpers_check_their_arguments(lib):
