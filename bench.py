@@ -489,6 +489,16 @@ def main() -> int:
                 extras[f"{key}_gbps"] = mxw[0].payload_bytes / (ms * 1e-3) / 1e9
                 log(f"[bench] {mx_dtype} 12288x4096 M={M}: {ms * 1e3:.1f} us, {extras[f'{key}_gbps']:.0f} GB/s of payload")
             del mxw
+        # ---- NVQ2J (E8 vectors, 2 bits per weight; no BASELINE config): 12288 x 4096 read in place from its bit streams ----
+        e8_blob = synth.nvq2j_blob(61, 12288, 4096)
+        e8 = [R.load_quant_linear(*e8_blob) for _ in range(4)]
+        for M in (1, 16, 64):
+            xe = [bf16(synth.activations(rng, M, 4096)) for _ in range(4)]
+            ms = graph_ms(lambda: [e8[i](xe[i]) for i in range(4)], 5, warm=2) / 4
+            extras[f"nvq2j_12288x4096_M{M}_us"] = ms * 1e3
+            extras[f"nvq2j_12288x4096_M{M}_gbps"] = e8[0].weight.payload_bytes / (ms * 1e-3) / 1e9
+            log(f"[bench] NVQ2J 12288x4096 M={M}: {ms * 1e3:.1f} us, {extras[f'nvq2j_12288x4096_M{M}_gbps']:.0f} GB/s of payload")
+        del e8
         torch.cuda.empty_cache()
 
     cpu = None

@@ -692,7 +692,9 @@ __device__ __forceinline__ float4_t e8_mfma(u32x4_t a, u32x4_t b, float4_t c) {
     else
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
-template <int XF16, int MT>
+// DEC: the block decoder -- 0: sign-stream formats with 8-dimensional vectors, 4: with 4-dimensional ones, 1: NVQ1,
+// 2: NPQ0 / NEPQ0
+template <int XF16, int MT, int DEC>
 __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k, const uint8_t *__restrict__ w,
                                                                      const uint16_t *__restrict__ x, int64_t ldx, int M,
                                                                      float *__restrict__ y, int64_t ldy, E8TileShape sh) {
@@ -754,6 +756,9 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
                 if (off < raw) {  // (a piece lies inside one padding period: they are 64 bytes and more)
                     uint32_t *dst = reinterpret_cast<uint32_t *>(lds8 + roff[r] + off + ((off >> sh.pad[r]) << 2));
                     dst[0] = piece[t].x; dst[1] = piece[t].y; dst[2] = piece[t].z; dst[3] = piece[t].w;
+                    // the skipped bank before a period holds a copy of the period's first dword: a field's two dwords
+                    // are adjacent in LDS wherever it starts
+                    if (off > 0u && (off & ((1u << sh.pad[r]) - 1u)) == 0u) dst[-1] = piece[t].x;
                 }
             }
         }
@@ -789,9 +794,8 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
 
     // `nbits` (<= 25) bits at bit position `bit` of staged range r
     auto field = [&](int r, uint32_t bit, uint32_t nbits) -> uint32_t {
-        const uint32_t b0 = (bit >> 5) << 2, b1 = b0 + 4u;
-        const u32x2_t d = u32x2_t{*reinterpret_cast<lds_u32_ptr>(lds_base + roff[r] + b0 + ((b0 >> sh.pad[r]) << 2)),
-                                  *reinterpret_cast<lds_u32_ptr>(lds_base + roff[r] + b1 + ((b1 >> sh.pad[r]) << 2))};
+        const uint32_t b0 = (bit >> 5) << 2, a = lds_base + roff[r] + b0 + ((b0 >> sh.pad[r]) << 2);
+        const u32x2_t d = u32x2_t{*reinterpret_cast<lds_u32_ptr>(a), *reinterpret_cast<lds_u32_ptr>(a + 4u)};
         return __builtin_amdgcn_alignbit(d.y, d.x, bit & 31u) & ((1u << nbits) - 1u);
     };
     const int r16 = lane & 15, kb = lane >> 4;
@@ -837,11 +841,11 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
             float sc = __uint_as_float(se.x);
             u32x4_t wv;
             float dl = 0.f;
-            if (k.kind == 0) {
+            if constexpr (DEC == 0 || DEC == 4) {
                 const uint32_t mk = field(1, sgb + 7u * sb, 7);
                 uint32_t last = __popc(mk) & 1u;
                 u32x4_t ev;
-                if (k.vs == 4) {
+                if constexpr (DEC == 4) {
                     const uint32_t i0 = field(0, ixb + (2u * sb) * k.ib, k.ib);
                     const uint32_t i1 = 2u * sb + 1u < static_cast<uint32_t>(k.nvec) ? field(0, ixb + (2u * sb + 1u) * k.ib, k.ib) : 0u;
                     const u32x2_t e0 = *reinterpret_cast<lds_u32x2_ptr>(se.y + i0 * 8u), e1 = *reinterpret_cast<lds_u32x2_ptr>(se.y + i1 * 8u);
@@ -855,7 +859,7 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
                 wv = ev ^ sv;
             } else {
                 const uint32_t idx = sb < static_cast<uint32_t>(k.nvec) ? field(0, ixb + sb * k.ib, k.ib) : 0u;
-                if (k.kind == 1) {
+                if constexpr (DEC == 1) {
                     const uint32_t neg = field(1, sgb + g, 1);
                     wv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + ((k.banks == 2 ? neg : 0u) * static_cast<uint32_t>(k.entries) + idx) * 16u);
                     // w = scale * (code + d): d times the sum of the group's activations, as a product with ones
@@ -875,7 +879,7 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 float4_t part = {0.f, 0.f, 0.f, 0.f};
-                if (k.kind == 1) {
+                if constexpr (DEC == 1) {
                     const float4_t xs = e8_mfma<XF16>(xf[t][mt], u32x4_t{ones, ones, ones, ones}, float4_t{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
                     for (int v = 0; v < 4; ++v) part[v] = dl * xs[v];
@@ -1002,16 +1006,21 @@ static int nvqs_launch_e8_tile(const NvqsK &k, const uint8_t *w, const uint16_t 
                                const E8TileShape &sh, hipStream_t st) {
     // one or two 16-row tiles per block, which share every decoded fragment (four per block measured no faster than two
     // blocks of two: every block reads its rows' activations again, and that traffic grows with the tiles)
-#define MFQ_E8_TILE(MTV)                                                                                              \
+#define MFQ_E8_TILE(MTV, DECV)                                                                                        \
     {                                                                                                                 \
-        auto kern = nvqs_e8_tile_kernel<XF16, MTV>;                                                                   \
+        auto kern = nvqs_e8_tile_kernel<XF16, MTV, DECV>;                                                             \
         if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kern), sh.lds_bytes, "nvqs_e8_tile")) return rc; \
         hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(ceil_div(k.nrows, 16)), static_cast<unsigned>(ceil_div(M, 16 * MTV))), \
                            dim3(64 * kE8Waves), sh.lds_bytes, st, k, w, x, ldx, M, y, ldy, sh);                        \
         return check_launch("nvqs_e8_tile");                                                                          \
     }
-    if (M <= 16) MFQ_E8_TILE(1)
-    MFQ_E8_TILE(2)
+#define MFQ_E8_TILE_MT(DECV) \
+    if (M <= 16) MFQ_E8_TILE(1, DECV) else MFQ_E8_TILE(2, DECV)
+    if (k.kind == 0 && k.vs == 8) MFQ_E8_TILE_MT(0)
+    if (k.kind == 0) MFQ_E8_TILE_MT(4)
+    if (k.kind == 1) MFQ_E8_TILE_MT(1)
+    MFQ_E8_TILE_MT(2)
+#undef MFQ_E8_TILE_MT
 #undef MFQ_E8_TILE
 }
 template <int XF16>

@@ -95,6 +95,19 @@ def nvq3j512_blob(seed, out, K, banks=2):
     return "NVQ3J-512", blob
 
 
+def nvq2j_blob(seed, out, K, banks=4):
+    """NVQ2J: 8-dimensional vectors out of `banks` 256-entry tables of random int8 magnitudes in [0, 7] (the reference
+    learns them from the E8 grid; a matmul's time does not depend on their values), scale LUT linspace(0.45, 1.55),
+    random state / index / sign streams (stream layout of mfq/quantize/nvq_jsc.py:1053-1079)."""
+    rng = np.random.default_rng(seed)
+    ng, nvec = math.ceil(K / 24), math.ceil(K / 8)
+    blob = F.nvq_jsc_blob(
+        "e8_256", K, rng.uniform(0.002, 0.02, out).astype(np.float32) * 0.02, np.linspace(0.45, 1.55, 16, dtype=np.float32),
+        np.arange(16) % banks, rng.integers(0, 8, (banks, 256, 8), dtype=np.int8), rng.integers(0, 16, (out, ng), dtype=np.uint8),
+        rng.integers(0, 256, (out, nvec), dtype=np.uint16), rng.integers(0, 128, (out, nvec), dtype=np.uint8))
+    return "NVQ2J", blob
+
+
 def nint8_zero_blob(seed, out, K):
     """(dtype, blob) of an [out, K] NINT8-0 tensor drawn in the packed domain: 34-byte blocks of an fp16 scale
     U(1, 3) * 1e-4 and 32 int8 codes in [-127, 127] (block layout of mfq/formats/nint8_zero.py:84-124)."""
