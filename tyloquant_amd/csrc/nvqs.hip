@@ -6,6 +6,8 @@
 // The 1-bit families ride on the same machinery: NVQ1-L / NVQ1-S (kind 1: ternary 8-dimensional codebooks, an integer
 // relative scale and a delta sign per group, the sign also choosing NVQ1-S's bank) and NPQ0-L / NPQ0-S (kind 2: two
 // 4-dimensional int8 sub-codebooks and a relative scale chosen by the group's state).
+#include <type_traits>
+
 #include "common.hpp"
 #include "gemv_common.hpp"
 #include "tune.hpp"
@@ -804,6 +806,17 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
     const int m0 = static_cast<int>(blockIdx.y) * 16 * MT;  // the block's MT tiles of 16 rows share every decoded fragment
     const bool vec = ldx % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
     // the eight activations of block kb of group g of the lane's row in tile mt; zeros past M and K and for kb = 3
+    // whole aligned vectors everywhere (the common case): one range-checked load per fragment, the "no data" offset for
+    // the fragments that are zero
+    const bool fast = vec && k.neuron_len % 8 == 0 && 32 * ldx * 2 < (1ll << 31);
+    const __amdgpu_buffer_rsrc_t xwin =
+        wave_window(reinterpret_cast<const uint8_t *>(x + static_cast<int64_t>(m0) * ldx),
+                    fast ? static_cast<uint32_t>(((min(M - m0, 16 * MT) - 1) * ldx + k.neuron_len) * 2) : 0u);
+    auto x_frag_fast = [&](int g, int mt) -> u32x4_t {
+        const int c0 = (3 * g + kb) * 8, ml = 16 * mt + r16;
+        const bool ok = m0 + ml < M && kb < 3 && c0 < k.neuron_len;  // (g past the wave's groups is passed as ng: c0 >= K)
+        return __builtin_amdgcn_raw_buffer_load_b128(xwin, ok ? static_cast<uint32_t>(ml * ldx * 2 + c0 * 2) : kNoStep, 0, 0);
+    };
     auto x_frag = [&](int g, int mt) -> u32x4_t {
         u32x4_t v = {0u, 0u, 0u, 0u};
         const int c0 = (3 * g + kb) * 8, m = m0 + 16 * mt + r16;
@@ -826,12 +839,17 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
     const int g0 = wave * sh.gpw, g1 = min(k.ng, g0 + sh.gpw);
+    auto walk = [&](auto fast_c) {
     for (int gq = g0; gq < g1; gq += GT) {
         u32x4_t xf[GT][MT];
 #pragma unroll
         for (int t = 0; t < GT; ++t)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) xf[t][mt] = x_frag(gq + t < g1 ? gq + t : k.ng, mt);
+            for (int mt = 0; mt < MT; ++mt) {
+                const int gx = gq + t < g1 ? gq + t : k.ng;
+                if constexpr (decltype(fast_c)::value) xf[t][mt] = x_frag_fast(gx, mt);
+                else xf[t][mt] = x_frag(gx, mt);
+            }
 #pragma unroll
         for (int t = 0; t < GT; ++t) {
             const int g = min(gq + t, g1 - 1);  // past the wave's last group: that group again, against zero activations
@@ -890,6 +908,9 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
             }
         }
     }
+    };
+    if (fast) walk(std::true_type{});
+    else walk(std::false_type{});
     // ---- the waves' partial sums: red[wave][row][neuron] ------------------------------------------------------------
     float *red = reinterpret_cast<float *>(lds8 + red_off);
 #pragma unroll
