@@ -383,7 +383,7 @@ def test_nvq_stream_formats_dequant_bit_exact_and_matmul(codebook, banks, dtype,
         for xd in (torch.bfloat16, torch.float16):
             x, xf = _x(rng, M, K, xd)
             _check(nvq_matmul(lin.weight, x).cpu().numpy(), O.linear_forward_f64(want, xf))
-    for M in (17, 70, 140):                      # tiles of the matrix-core kernel; above 128 rows the fp16 GEMM
+    for M in (17, 70, 200):                      # tiles of the matrix-core kernel; above 192 rows the fp16 GEMM
         x, xf = _x(rng, M, K)
         _check(lin(x).cpu().numpy(), O.linear_forward_f64(want, xf))
     xs = torch.zeros((1, K + 3), dtype=torch.bfloat16, device="cuda")[:, 1:K + 1]       # a misaligned row
@@ -444,7 +444,7 @@ def test_one_bit_families_dequant_bit_exact_and_matmul(dtype, kw, out, K):
         for xd in (torch.bfloat16, torch.float16):
             x, xf = _x(rng, M, K, xd)
             _check(nvq_matmul(lin.weight, x).cpu().numpy(), O.linear_forward_f64(want, xf))
-    for M in (17, 70, 140):                      # tiles of the matrix-core kernel; above 128 rows the fp16 GEMM
+    for M in (17, 70, 200):                      # tiles of the matrix-core kernel; above 192 rows the fp16 GEMM
         x, xf = _x(rng, M, K)
         _check(lin(x).cpu().numpy(), O.linear_forward_f64(want, xf))
 
@@ -523,7 +523,7 @@ def test_nepq0_dequant_bit_exact_and_matmul(label, E, out, K, banks):
         for M in (1, 5, 16):
             x, xf = _x(rng, M, K)
             _check(nepq_matmul(w, x, e).cpu().numpy(), O.linear_forward_f64(want[e], xf))
-        for M in (40, 140):
+        for M in (40, 200):
             x, xf = _x(rng, M, K)
             _check(nepq_matmul(w, x, e).cpu().numpy(), O.linear_forward_f64(want[e], xf))
     if E == 1:
@@ -570,7 +570,7 @@ TILE_CASES = [("jsc", "e8_256", 4, 37, 1544), ("jsc", "e8_1024", 2, 70, 100), ("
 
 @pytest.mark.parametrize("kind,a,b,out,K", TILE_CASES)
 def test_stream_formats_on_the_matrix_core_tile_kernel(kind, a, b, out, K):
-    """Five to 128 rows of the formats read in place from their bit streams run as 16-neuron tiles on the matrix
+    """Five to 192 rows of the formats read in place from their bit streams run as 16-neuron tiles on the matrix
     cores: a last tile with fewer neurons, K that ends inside a group, a block and a vector, every row count of the
     range in both activation types, rows at a stride that is no multiple of 16 bytes (element-wise loads), and bf16 rows
     far outside fp16's range."""
@@ -588,7 +588,7 @@ def test_stream_formats_on_the_matrix_core_tile_kernel(kind, a, b, out, K):
     dtype, blob = O.pack_tensor(t)
     lin = R.load_quant_linear(dtype, blob)
     want = O.dequantize_tensor(O.unpack_tensor(dtype, blob))
-    for M in list(range(5, 17)) + [17, 32, 33, 64, 100, 128, 129]:   # one or two tiles per block, several blocks of rows; 129: the fp16 GEMM
+    for M in list(range(5, 17)) + [17, 32, 33, 64, 100, 129, 192, 193]:   # one, two or four tiles per block, several sets of rows; 193: the fp16 GEMM
         xd = torch.bfloat16 if M % 2 else torch.float16
         x, xf = _x(rng, M, K, xd)
         _check(nvq_matmul(lin.weight, x).cpu().numpy(), O.linear_forward_f64(want, xf))

@@ -667,15 +667,15 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
 }
 
 
-// ---- the same formats for 5 to 128 rows on the matrix cores -----------------------------------------------------------
+// ---- the same formats for 5 to 192 rows on the matrix cores -----------------------------------------------------------
 // nvqs_e8_kernel reads a row's activations again for every block of weights, so its time grows with the rows.  Here a
 // block owns 16 consecutive neurons: their three bit ranges (contiguous in the streams) are staged whole, the waves
 // split the groups of 24 weights, and lane (n, kb) -- neuron n = lane % 16, block kb = lane / 16 of the group, the lanes
 // of kb = 3 idle -- decodes one 8-weight block, which is its B fragment of a 16 x 16 x 32 product against the rows'
 // 24 activations of the group (A fragment: row lane % 16, the same block; zeros for kb = 3).  The product's four
 // results of a lane belong to its own neuron, whose group scale it has decoded, and are scaled and added in fp32.
-// The waves' partial sums meet in LDS.  Above 16 rows a block takes two 16-row tiles (blockIdx.y counts pairs of tiles),
-// which share every decoded fragment.  The 16 neurons of a wave read their fields at a stride of the neuron's bytes in
+// The waves' partial sums meet in LDS.  Above 16 rows a block takes two or four 16-row tiles (blockIdx.y counts such
+// sets), which share every decoded fragment.  The 16 neurons of a wave read their fields at a stride of the neuron's bytes in
 // the stream -- 512 bytes of index bytes for K = 4096, one LDS bank for all of them -- so the staged copy of a range
 // skips a bank after every 2^pad bytes, with pad chosen per range so that the 16 strides spread over the banks.
 // LDS map (bytes): [entries][256 sign patterns x 16][state table 128][pool scale tables][index | sign | state ranges]
@@ -834,7 +834,7 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
         return v;
     };
     const uint32_t ones = XF16 ? 0x3c003c00u : 0x3f803f80u;
-    constexpr int GT = MT == 1 ? 4 : 2;  // groups whose activations are requested together
+    constexpr int GT = MT == 1 ? 4 : (MT == 2 ? 2 : 1);  // groups whose activations are requested together
     float4_t acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -938,7 +938,7 @@ void dequant_gemm_carve(void *ws, int N, int K, int M, uint16_t *&x16, float *&x
                         int &Kp);
 
 constexpr int kNvqsGemvMaxM = 16;  // rows up to which the weights are re-read per pass of eight rows
-constexpr int kNvqsTileMaxM = 128;  // rows up to which the formats of the matrix-core tile kernel stay on it
+constexpr int kNvqsTileMaxM = 192;  // rows up to which the formats of the matrix-core tile kernel stay on it
 
 // The E8 kernel takes the sign-stream format with 8- or 4-dimensional vectors, 4-bit states and tables that fit the LDS
 // in the activations' type (E8: 256 or 1024 entries in up to four banks, 4096 in one; D4: 1024 entries), tensors whose streams fit 32-bit offsets and
@@ -1025,8 +1025,8 @@ static bool nvqs_e8_tile_shape(const NvqsK &k, int M, E8TileShape &sh) {
 template <int XF16>
 static int nvqs_launch_e8_tile(const NvqsK &k, const uint8_t *w, const uint16_t *x, int64_t ldx, int M, float *y, int64_t ldy,
                                const E8TileShape &sh, hipStream_t st) {
-    // one or two 16-row tiles per block, which share every decoded fragment (four per block measured no faster than two
-    // blocks of two: every block reads its rows' activations again, and that traffic grows with the tiles)
+    // one, two or four 16-row tiles per block, which share every decoded fragment (with four, one group's activations
+    // are requested at a time to stay within 64 registers: two blocks of 16 waves per compute unit)
 #define MFQ_E8_TILE(MTV, DECV)                                                                                        \
     {                                                                                                                 \
         auto kern = nvqs_e8_tile_kernel<XF16, MTV, DECV>;                                                             \
@@ -1036,7 +1036,7 @@ static int nvqs_launch_e8_tile(const NvqsK &k, const uint8_t *w, const uint16_t 
         return check_launch("nvqs_e8_tile");                                                                          \
     }
 #define MFQ_E8_TILE_MT(DECV) \
-    if (M <= 16) MFQ_E8_TILE(1, DECV) else MFQ_E8_TILE(2, DECV)
+    if (M <= 16) MFQ_E8_TILE(1, DECV) else if (M <= 32) MFQ_E8_TILE(2, DECV) else MFQ_E8_TILE(4, DECV)
     if (k.kind == 0 && k.vs == 8) MFQ_E8_TILE_MT(0)
     if (k.kind == 0) MFQ_E8_TILE_MT(4)
     if (k.kind == 1) MFQ_E8_TILE_MT(1)
