@@ -839,6 +839,13 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = float4_t{0.f, 0.f, 0.f, 0.f};
     const int g0 = wave * sh.gpw, g1 = min(k.ng, g0 + sh.gpw);
+    // bit positions of the lane's fields in the wave's first group; they advance by a constant per group (a product per
+    // field and group would be a quarter-rate 64-bit multiply-add each)
+    const uint32_t kb2 = static_cast<uint32_t>(min(kb, 2));  // the lanes of kb = 3 meet zero activations
+    const uint32_t ix_inc = (DEC == 4 ? 6u : 3u) * static_cast<uint32_t>(k.ib), sg_inc = DEC == 1 ? 1u : 21u, st_inc = static_cast<uint32_t>(k.sbits);
+    uint32_t ix_bit = ixb + (DEC == 4 ? 2u : 1u) * (3u * static_cast<uint32_t>(g0) + kb2) * static_cast<uint32_t>(k.ib);
+    uint32_t sg_bit = sgb + (DEC == 1 ? static_cast<uint32_t>(g0) : 7u * (3u * static_cast<uint32_t>(g0) + kb2));
+    uint32_t st_bit = stb + st_inc * static_cast<uint32_t>(g0);
     auto walk = [&](auto fast_c) {
     for (int gq = g0; gq < g1; gq += GT) {
         u32x4_t xf[GT][MT];
@@ -853,32 +860,32 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
 #pragma unroll
         for (int t = 0; t < GT; ++t) {
             const int g = min(gq + t, g1 - 1);  // past the wave's last group: that group again, against zero activations
-            const uint32_t sb = static_cast<uint32_t>(3 * g + min(kb, 2));  // the lanes of kb = 3 meet zero activations
-            const uint32_t state = field(2, stb + static_cast<uint32_t>(k.sbits) * g, k.sbits);
+            const uint32_t sb = static_cast<uint32_t>(3 * g) + kb2;
+            const uint32_t state = field(2, st_bit, k.sbits);
             const u32x2_t se = *reinterpret_cast<lds_u32x2_ptr>(lds_base + stab_off + state * 8u);
             float sc = __uint_as_float(se.x);
             u32x4_t wv;
             float dl = 0.f;
             if constexpr (DEC == 0 || DEC == 4) {
-                const uint32_t mk = field(1, sgb + 7u * sb, 7);
+                const uint32_t mk = field(1, sg_bit, 7);
                 uint32_t last = __popc(mk) & 1u;
                 u32x4_t ev;
                 if constexpr (DEC == 4) {
-                    const uint32_t i0 = field(0, ixb + (2u * sb) * k.ib, k.ib);
-                    const uint32_t i1 = 2u * sb + 1u < static_cast<uint32_t>(k.nvec) ? field(0, ixb + (2u * sb + 1u) * k.ib, k.ib) : 0u;
+                    const uint32_t i0 = field(0, ix_bit, k.ib);
+                    const uint32_t i1 = 2u * sb + 1u < static_cast<uint32_t>(k.nvec) ? field(0, ix_bit + static_cast<uint32_t>(k.ib), k.ib) : 0u;
                     const u32x2_t e0 = *reinterpret_cast<lds_u32x2_ptr>(se.y + i0 * 8u), e1 = *reinterpret_cast<lds_u32x2_ptr>(se.y + i1 * 8u);
                     ev = u32x4_t{e0.x, e0.y, e1.x, e1.y};
                 } else {
-                    const uint32_t idx = field(0, ixb + sb * k.ib, k.ib);
+                    const uint32_t idx = field(0, ix_bit, k.ib);
                     if (k.index_parity) last ^= (idx >> 7) & 1u;
                     ev = *reinterpret_cast<lds_u32x4_ptr>(se.y + idx * 16u);
                 }
                 const u32x4_t sv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + sgn_off + (mk | (last << 7)) * 16u);
                 wv = ev ^ sv;
             } else {
-                const uint32_t idx = sb < static_cast<uint32_t>(k.nvec) ? field(0, ixb + sb * k.ib, k.ib) : 0u;
+                const uint32_t idx = sb < static_cast<uint32_t>(k.nvec) ? field(0, ix_bit, k.ib) : 0u;
                 if constexpr (DEC == 1) {
-                    const uint32_t neg = field(1, sgb + g, 1);
+                    const uint32_t neg = field(1, sg_bit, 1);
                     wv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + ((k.banks == 2 ? neg : 0u) * static_cast<uint32_t>(k.entries) + idx) * 16u);
                     // w = scale * (code + d): d times the sum of the group's activations, as a product with ones
                     dl = neg ? -k.delta : k.delta;
@@ -905,6 +912,9 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
                 part = e8_mfma<XF16>(xf[t][mt], wv, part);
 #pragma unroll
                 for (int v = 0; v < 4; ++v) acc[mt][v] = fmaf(sc, part[v], acc[mt][v]);
+            }
+            if (gq + t + 1 < g1) {  // (wave-uniform; past the wave's last group the positions stay on it)
+                ix_bit += ix_inc; sg_bit += sg_inc; st_bit += st_inc;
             }
         }
     }
