@@ -684,6 +684,7 @@ struct E8TileShape {
     int gpw;            // groups of 24 weights per wave
     uint32_t cap[3];    // LDS bytes of the block's index / sign / state range, padding included
     uint32_t pad[3];    // log2 of the bytes of a range after which its LDS copy skips a bank (31: no padding)
+    int compact;        // the table stays bytes in LDS (decoder 8)
     uint32_t lds_bytes;
 };
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -695,7 +696,11 @@ __device__ __forceinline__ float4_t e8_mfma(u32x4_t a, u32x4_t b, float4_t c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 // DEC: the block decoder -- 0: sign-stream formats with 8-dimensional vectors, 4: with 4-dimensional ones, 1: NVQ1,
-// 2: NPQ0 / NEPQ0
+// 2: NPQ0 / NEPQ0, 8: 8-dimensional vectors whose table fits the LDS only as bytes (NVQ2J-XL with several banks: 128 KB
+// of int8).  The bytes are kept with bit 7 flipped (u = v + 128, unsigned) and widened where they are used: for fp16
+// activations a byte permute builds 1024 + u and a packed subtraction of 1152 leaves v exactly; bf16 has no packed
+// arithmetic here, so the block is multiplied as u and 128 times the product of the same activations with the block's
+// signs alone is taken off (exact factors, fp32 sums).  The partial sums then reuse the ranges' LDS.
 template <int XF16, int MT, int DEC>
 __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k, const uint8_t *__restrict__ w,
                                                                      const uint16_t *__restrict__ x, int64_t ldx, int M,
@@ -709,13 +714,13 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
     const int ncb = k.kind == 2 ? k.cb_bytes / k.vs : (k.kind == 3 ? k.nbank * k.bank_bytes / k.vs : k.banks * k.entries);
     uint8_t *lds8 = reinterpret_cast<uint8_t *>(lds32);
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)lds8));
-    const uint32_t esz = static_cast<uint32_t>(k.vs) * 2u;
+    const uint32_t esz = DEC == 8 ? 8u : static_cast<uint32_t>(k.vs) * 2u;
     const uint32_t sgn_off = static_cast<uint32_t>(ncb) * esz, stab_off = sgn_off + 4096u, lut3_off = stab_off + 128u;
     uint32_t roff[3];
     roff[0] = lut3_off + (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * 32u : 0u);
     roff[1] = roff[0] + sh.cap[0];
     roff[2] = roff[1] + sh.cap[1];
-    const uint32_t red_off = roff[2] + sh.cap[2];
+    const uint32_t red_off = DEC == 8 ? roff[0] : roff[2] + sh.cap[2];
 
     // ---- the block's stream ranges: 16-byte pieces, four requests of a thread in flight ----------------------------
     const int row_first = static_cast<int>(blockIdx.x) * 16;
@@ -768,6 +773,10 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
     // ---- tables -------------------------------------------------------------------------------------------------------
     for (int e = tid; e < nslot; e += blockDim.x) {
         const u32x2_t raw = e == tid ? raw0 : *reinterpret_cast<const u32x2_t *>(cbp + static_cast<int64_t>(e) * 8);
+        if constexpr (DEC == 8) {
+            *reinterpret_cast<u32x2_t *>(lds8 + static_cast<uint32_t>(e) * 8u) = u32x2_t{raw.x ^ 0x80808080u, raw.y ^ 0x80808080u};
+            continue;
+        }
         u32x4_t v;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -866,7 +875,8 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
             float sc = __uint_as_float(se.x);
             u32x4_t wv;
             float dl = 0.f;
-            if constexpr (DEC == 0 || DEC == 4) {
+            [[maybe_unused]] u32x4_t sgn_ones = {0u, 0u, 0u, 0u};  // DEC 8, bf16: the block's signs on ones
+            if constexpr (DEC == 0 || DEC == 4 || DEC == 8) {
                 const uint32_t mk = field(1, sg_bit, 7);
                 uint32_t last = __popc(mk) & 1u;
                 u32x4_t ev;
@@ -878,10 +888,29 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
                 } else {
                     const uint32_t idx = field(0, ix_bit, k.ib);
                     if (k.index_parity) last ^= (idx >> 7) & 1u;
-                    ev = *reinterpret_cast<lds_u32x4_ptr>(se.y + idx * 16u);
+                    if constexpr (DEC == 8) {
+                        const u32x2_t q = *reinterpret_cast<lds_u32x2_ptr>(se.y + idx * 8u);
+                        const uint32_t qq[2] = {q.x, q.y};
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            if constexpr (XF16) {
+                                const half2_t bias = {static_cast<_Float16>(1152.f), static_cast<_Float16>(1152.f)};
+                                ev[2 * h] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(qq[h], 0x64006400u, 0x03050104u)) - bias);
+                                ev[2 * h + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(qq[h], 0x64006400u, 0x03070106u)) - bias);
+                            } else {
+                                const float f0 = static_cast<float>(qq[h] & 0xffu), f1 = static_cast<float>((qq[h] >> 8) & 0xffu),
+                                            f2 = static_cast<float>((qq[h] >> 16) & 0xffu), f3 = static_cast<float>(qq[h] >> 24);
+                                ev[2 * h] = (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+                                ev[2 * h + 1] = (__float_as_uint(f2) >> 16) | (__float_as_uint(f3) & 0xffff0000u);
+                            }
+                        }
+                    } else {
+                        ev = *reinterpret_cast<lds_u32x4_ptr>(se.y + idx * 16u);
+                    }
                 }
                 const u32x4_t sv = *reinterpret_cast<lds_u32x4_ptr>(lds_base + sgn_off + (mk | (last << 7)) * 16u);
                 wv = ev ^ sv;
+                if constexpr (DEC == 8 && !XF16) sgn_ones = u32x4_t{ones, ones, ones, ones} ^ sv;
             } else {
                 const uint32_t idx = sb < static_cast<uint32_t>(k.nvec) ? field(0, ix_bit, k.ib) : 0u;
                 if constexpr (DEC == 1) {
@@ -909,6 +938,11 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
 #pragma unroll
                     for (int v = 0; v < 4; ++v) part[v] = dl * xs[v];
                 }
+                if constexpr (DEC == 8 && !XF16) {
+                    const float4_t xs = e8_mfma<XF16>(xf[t][mt], sgn_ones, float4_t{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) part[v] = -128.f * xs[v];
+                }
                 part = e8_mfma<XF16>(xf[t][mt], wv, part);
 #pragma unroll
                 for (int v = 0; v < 4; ++v) acc[mt][v] = fmaf(sc, part[v], acc[mt][v]);
@@ -923,6 +957,7 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
     else walk(std::false_type{});
     // ---- the waves' partial sums: red[wave][row][neuron] ------------------------------------------------------------
     float *red = reinterpret_cast<float *>(lds8 + red_off);
+    if constexpr (DEC == 8) __syncthreads();  // the sums take the place of the ranges: every wave is done with them
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {  // one tile at a time through the same 16 KB
         if (mt > 0) __syncthreads();
@@ -1001,14 +1036,14 @@ static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     }
     return false;
 }
-// The matrix-core form: from MFQ_NVQS_TILE_MIN_M rows on, when the 16 neurons' ranges and the tables fit the LDS.
+// The matrix-core form: from MFQ_NVQS_TILE_MIN_M rows on (from one row for the tables kept as bytes), when the 16 neurons'
+// ranges and the tables fit the LDS.
 static bool nvqs_e8_tile_shape(const NvqsK &k, int M, E8TileShape &sh) {
     static const int min_m = tune_env("MFQ_NVQS_TILE_MIN_M", 5);
     static const int max_m = tune_env("MFQ_NVQS_TILE_MAX_M", kNvqsTileMaxM);
-    if (M < min_m || M > max_m || !nvqs_e8_format(k)) return false;
+    if (M < 1 || M > max_m || !nvqs_e8_format(k)) return false;
     const int64_t bits[3] = {16ll * k.nvec * k.ib, 16ll * nvqs_e8_sign_bits(k), 16ll * k.ng * k.sbits};
-    uint64_t total = static_cast<uint64_t>(nvqs_e8_table_bytes(k)) * 2u + 4096u + 128u + (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * 32u : 0u) +
-                     kE8Waves * 1024u;
+    uint64_t ranges = 0;
     for (int r = 0; r < 3; ++r) {
         if (bits[r] > (1ll << 22)) return false;
         // the padding period under which the first dwords of the 16 neurons spread best over 32 banks
@@ -1025,8 +1060,15 @@ static bool nvqs_e8_tile_shape(const NvqsK &k, int M, E8TileShape &sh) {
             if (worst < best) { best = worst; sh.pad[r] = static_cast<uint32_t>(periods[pi]); }
         }
         sh.cap[r] = (raw + ((raw >> sh.pad[r]) << 2) + 16u + 15u) / 16u * 16u;
-        total += sh.cap[r];
+        ranges += sh.cap[r];
     }
+    const uint64_t tables = 4096u + 128u + (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * 32u : 0u);
+    uint64_t total = static_cast<uint64_t>(nvqs_e8_table_bytes(k)) * 2u + tables + ranges + kE8Waves * 1024u;
+    // 8-dimensional sign-stream tables too large for the LDS in the activations' type stay bytes there and the sums
+    // reuse the ranges' place; the vector kernel cannot take those tensors, so the tile kernel does from one row on
+    sh.compact = total > kMaxDynamicLds && k.kind == 0 && k.vs == 8;
+    if (sh.compact) total = nvqs_e8_table_bytes(k) + tables + (ranges > kE8Waves * 1024u ? ranges : kE8Waves * 1024u);
+    if (!sh.compact && M < min_m) return false;
     if (total > kMaxDynamicLds) return false;
     sh.lds_bytes = static_cast<uint32_t>(total);
     sh.gpw = static_cast<int>(ceil_div(k.ng, kE8Waves));
@@ -1047,6 +1089,7 @@ static int nvqs_launch_e8_tile(const NvqsK &k, const uint8_t *w, const uint16_t 
     }
 #define MFQ_E8_TILE_MT(DECV) \
     if (M <= 16) MFQ_E8_TILE(1, DECV) else if (M <= 32) MFQ_E8_TILE(2, DECV) else MFQ_E8_TILE(4, DECV)
+    if (sh.compact) MFQ_E8_TILE_MT(8)
     if (k.kind == 0 && k.vs == 8) MFQ_E8_TILE_MT(0)
     if (k.kind == 0) MFQ_E8_TILE_MT(4)
     if (k.kind == 1) MFQ_E8_TILE_MT(1)
