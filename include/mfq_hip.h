@@ -22,7 +22,7 @@
  *     the activation rows are not 16-byte aligned),
  *   - the stream-family (E8, d4_1024, 1-bit, NEPQ0) wave-per-neuron kernels up to 16 rows, which multiply in fp32, and
  *     the kernels of the E8 formats whose tables fit the LDS and of NVQ1-L / NVQ1-S / NPQ0-L / NPQ0-S / NEPQ0 (packed dot
- *     products up to four rows, matrix-core products from five to 192), which take bf16 as it is,
+ *     products for one and two rows, matrix-core products from three to 192), which take bf16 as it is,
  *   - the MXFP4 / MXFP8 kernels up to 256 rows, whose matrix-core products take bf16 as it is (the weights are exact in
  *     bf16, scale included),
  *   - every prefill kernel:

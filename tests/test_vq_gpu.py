@@ -344,7 +344,8 @@ def test_multi_expert_nepq_blob_is_not_a_linear():
 def test_e8_kernel_with_several_neurons_per_wave(cu_count, cus, codebook, banks, out, K):
     """A wave of the E8 kernel walks up to four consecutive neurons of a large tensor; sized for one or two compute
     units, small tensors take the same shape: neurons whose stream ranges start inside a byte, waves with fewer neurons
-    than the others and waves with none, one to eight rows per pass and both activation types."""
+    than the others and waves with none, one and two rows per pass and both activation types (the larger batches of the
+    loop take the tile kernel on the same tensors)."""
     from tyloquant_amd import runtime as R
     from tyloquant_amd.runtime_vq import nvq_matmul
     rng = np.random.default_rng(70 + out + K + cus)
@@ -456,8 +457,8 @@ def test_one_bit_families_dequant_bit_exact_and_matmul(dtype, kw, out, K):
 def test_one_bit_families_with_several_neurons_per_wave(cu_count, cus, dtype, kw, out, K):
     """The decoders of the 1-bit families in the kernel that stages a wave's bit ranges in LDS, sized for one or two
     compute units so that a wave walks several neurons: state fields of 2 to 4 bits and delta signs that start inside a
-    byte, waves with fewer neurons than the others and with none, one to eight rows per pass, both activation types
-    and bf16 rows far outside fp16's range."""
+    byte, waves with fewer neurons than the others and with none, one and two rows per pass, both activation types
+    and bf16 rows far outside fp16's range (the larger batches of the loop take the tile kernel)."""
     from tyloquant_amd import runtime as R
     from tyloquant_amd.runtime_vq import nvq_matmul
     rng = np.random.default_rng(170 + out + K + cus)
@@ -548,7 +549,8 @@ def test_nepq0_dequant_bit_exact_and_matmul(label, E, out, K, banks):
 def test_nepq0_with_several_neurons_per_wave(cu_count, cus, label, E, out, K, banks):
     """The table-pool decoder in the kernel that stages a wave's bit ranges in LDS, sized for one or two compute units:
     experts whose first neuron starts inside a byte of the streams, waves with several neurons, with fewer and with
-    none, one to eight rows per pass, both activation types and bf16 rows far outside fp16's range."""
+    none, one and two rows per pass, both activation types and bf16 rows far outside fp16's range (the larger batches of
+    the loop take the tile kernel)."""
     from tyloquant_amd.runtime_vq import NepqWeight, nepq_matmul
     rng = np.random.default_rng(223 + E + out + K + cus)
     blob = O.pack_nepq(synth.nepq_random(rng, label, E, out, K, banks))
@@ -572,7 +574,7 @@ TILE_CASES = [("jsc", "e8_256", 4, 37, 1544), ("jsc", "e8_1024", 2, 70, 100), ("
 
 @pytest.mark.parametrize("kind,a,b,out,K", TILE_CASES)
 def test_stream_formats_on_the_matrix_core_tile_kernel(kind, a, b, out, K):
-    """Five to 192 rows of the formats read in place from their bit streams run as 16-neuron tiles on the matrix
+    """Three to 192 rows of the formats read in place from their bit streams run as 16-neuron tiles on the matrix
     cores: a last tile with fewer neurons, K that ends inside a group, a block and a vector, every row count of the
     range in both activation types, rows at a stride that is no multiple of 16 bytes (element-wise loads), and bf16 rows
     far outside fp16's range."""
@@ -590,7 +592,7 @@ def test_stream_formats_on_the_matrix_core_tile_kernel(kind, a, b, out, K):
     dtype, blob = O.pack_tensor(t)
     lin = R.load_quant_linear(dtype, blob)
     want = O.dequantize_tensor(O.unpack_tensor(dtype, blob))
-    for M in list(range(1 if kind == "jsc" and a == "e8_4096" and b > 1 else 5, 17)) + [17, 32, 33, 64, 100, 129, 192, 193]:   # one, two or four tiles per block, several sets of rows; 193: the fp16 GEMM
+    for M in list(range(1 if kind == "jsc" and a == "e8_4096" and b > 1 else 3, 17)) + [17, 32, 33, 64, 100, 129, 192, 193]:   # one, two or four tiles per block, several sets of rows; 193: the fp16 GEMM
         xd = torch.bfloat16 if M % 2 else torch.float16
         x, xf = _x(rng, M, K, xd)
         _check(nvq_matmul(lin.weight, x).cpu().numpy(), O.linear_forward_f64(want, xf))

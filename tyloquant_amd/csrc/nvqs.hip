@@ -667,7 +667,7 @@ __global__ __launch_bounds__(64 * kE8Waves) void nvqs_e8_kernel(NvqsK k, const u
 }
 
 
-// ---- the same formats for 5 to 192 rows on the matrix cores -----------------------------------------------------------
+// ---- the same formats for 3 to 192 rows on the matrix cores -----------------------------------------------------------
 // nvqs_e8_kernel reads a row's activations again for every block of weights, so its time grows with the rows.  Here a
 // block owns 16 consecutive neurons: their three bit ranges (contiguous in the streams) are staged whole, the waves
 // split the groups of 24 weights, and lane (n, kb) -- neuron n = lane % 16, block kb = lane / 16 of the group, the lanes
@@ -1028,7 +1028,7 @@ static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
     sh.cap[1] = cap(static_cast<int64_t>(npw) * nvqs_e8_sign_bits(k));
     sh.cap[2] = cap(static_cast<int64_t>(npw) * k.ng * k.sbits);
     sh.wave_bytes = sh.cap[0] + sh.cap[1] + sh.cap[2];
-    for (mb = M >= 4 ? 4 : (M >= 2 ? 2 : 1); mb >= 1; mb >>= 1) {  // (five rows and more go to the matrix-core form)
+    for (mb = M >= 2 ? 2 : 1; mb >= 1; mb >>= 1) {  // (three rows and more go to the matrix-core form)
         const uint32_t table = nvqs_e8_table_bytes(k);
         if (table > kMaxDynamicLds / 2) return false;
         sh.lds_bytes = table * 2u + 4096u + 128u + (k.kind == 3 ? static_cast<uint32_t>(k.nbank) * 32u : 0u) + static_cast<uint32_t>(mb) * sh.kp * 2u + kE8Waves * sh.wave_bytes;
@@ -1039,7 +1039,7 @@ static bool nvqs_e8_shape(const NvqsK &k, int M, int &mb, E8Shape &sh) {
 // The matrix-core form: from MFQ_NVQS_TILE_MIN_M rows on (from one row for the tables kept as bytes), when the 16 neurons'
 // ranges and the tables fit the LDS.
 static bool nvqs_e8_tile_shape(const NvqsK &k, int M, E8TileShape &sh) {
-    static const int min_m = tune_env("MFQ_NVQS_TILE_MIN_M", 5);
+    static const int min_m = tune_env("MFQ_NVQS_TILE_MIN_M", 3);
     static const int max_m = tune_env("MFQ_NVQS_TILE_MAX_M", kNvqsTileMaxM);
     if (M < 1 || M > max_m || !nvqs_e8_format(k)) return false;
     const int64_t bits[3] = {16ll * k.nvec * k.ib, 16ll * nvqs_e8_sign_bits(k), 16ll * k.ng * k.sbits};
@@ -1109,7 +1109,7 @@ static int nvqs_launch_e8(const NvqsK &k, const uint8_t *w, const uint16_t *x, i
         hipLaunchKernelGGL(kern, grid, dim3(64 * kE8Waves), sh.lds_bytes, st, k, w, x, ldx, M, y, ldy, sh, sel);       \
         return check_launch("nvqs_e8");                                                                               \
     }
-    MFQ_E8(1) MFQ_E8(2) MFQ_E8(4)
+    MFQ_E8(1) MFQ_E8(2)
 #undef MFQ_E8
     return fail(MFQ_ERR_UNSUPPORTED, "nvqs_e8: %d rows per pass", mb);
 }

@@ -49,7 +49,7 @@ Knob g_knobs[] = {
     {"MFQ_FFN_SPIN_LIMIT", "polls after which the one-launch FFN's grid barrier gives up", 0, false},
     {"MFQ_FFN_TRACE", "1 = the one-launch FFN records per-block clocks behind its workspace", 0, false},
     {"MFQ_NVQS_E8_OFF", "1 = the E8 formats on the generic stream kernel", 0, false},
-    {"MFQ_NVQS_TILE_MIN_M", "rows from which the stream formats whose ranges fit the LDS run on the matrix-core tile kernel (default 5)", 0, false},
+    {"MFQ_NVQS_TILE_MIN_M", "rows from which the stream formats whose ranges fit the LDS run on the matrix-core tile kernel (default 3)", 0, false},
     {"MFQ_NVQS_TILE_MAX_M", "rows up to which they stay on it before the fp16 copy + GEMM (default 192)", 0, false},
     {"MFQ_MX_TILE_OFF", "1 = MXFP4 / MXFP8 small batches on the wave-per-neuron kernel instead of the matrix-core tile kernel", 0, false},
     {"MFQ_MX_STAGE_OFF", "1 = the MX tile kernel never stages a wave's activation slice and scales in LDS", 0, false},
