@@ -741,33 +741,50 @@ __global__ __launch_bounds__(64 * kE8Waves, 8) void nvqs_e8_tile_kernel(NvqsK k,
     const u32x2_t raw0 = tid < nslot ? *reinterpret_cast<const u32x2_t *>(cbp + static_cast<int64_t>(tid) * 8) : u32x2_t{0u, 0u};
     const float lutv = lut[tid & 15];
     const uint32_t bfsv = bfs[tid & 15];
+    // the first pieces of a thread in each range (two: 32 KB of a range; one where four row tiles leave few registers) are
+    // requested together, so that the three ranges cost one round trip, not three; what a longer range has left follows
+    // in turns of four pieces
+    constexpr int HEAD = MT == 4 ? 1 : 2;
+    constexpr uint32_t kTurn = 64u * kE8Waves * 16u;  // bytes the block's threads cover with one piece each
+    __amdgpu_buffer_rsrc_t win[3];
+    uint32_t raw[3];  // stream bytes of the ranges
+    u32x4_t head[3][HEAD];
 #pragma unroll
     for (int r = 0; r < 3; ++r) {
         const int64_t bit0 = n0 * static_cast<int64_t>(per[r]);
         const int64_t a0 = (bit0 >> 3) & ~static_cast<int64_t>(15);
         shift[r] = static_cast<uint32_t>(bit0 - a0 * 8);
         const int64_t left = region_bytes[r] - a0;
-        const __amdgpu_buffer_rsrc_t win =
-            wave_window(w + region[r] + a0, static_cast<uint32_t>(left <= 0 ? 0 : (left < (1ll << 31) ? left : (1ll << 31))));
-        const uint32_t raw = nvqs_e8_range_bytes(16ll * per[r]);  // stream bytes of the range
-        for (uint32_t p0 = static_cast<uint32_t>(tid) * 16u; p0 < raw; p0 += 4u * 64u * kE8Waves * 16u) {
+        win[r] = wave_window(w + region[r] + a0, static_cast<uint32_t>(left <= 0 ? 0 : (left < (1ll << 31) ? left : (1ll << 31))));
+        raw[r] = nvqs_e8_range_bytes(16ll * per[r]);
+#pragma unroll
+        for (int t = 0; t < HEAD; ++t) {
+            const uint32_t off = static_cast<uint32_t>(tid) * 16u + static_cast<uint32_t>(t) * kTurn;
+            head[r][t] = __builtin_amdgcn_raw_buffer_load_b128(win[r], off < raw[r] ? off : kNoStep, 0, 2);
+        }
+    }
+    // a piece lies inside one padding period (they are 64 bytes and more); the skipped bank before a period holds a copy
+    // of the period's first dword, so that a field's two dwords are adjacent in LDS wherever it starts
+    auto park = [&](int r, uint32_t off, u32x4_t piece) {
+        if (off < raw[r]) {
+            uint32_t *dst = reinterpret_cast<uint32_t *>(lds8 + roff[r] + off + ((off >> sh.pad[r]) << 2));
+            dst[0] = piece.x; dst[1] = piece.y; dst[2] = piece.z; dst[3] = piece.w;
+            if (off > 0u && (off & ((1u << sh.pad[r]) - 1u)) == 0u) dst[-1] = piece.x;
+        }
+    };
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+#pragma unroll
+        for (int t = 0; t < HEAD; ++t) park(r, static_cast<uint32_t>(tid) * 16u + static_cast<uint32_t>(t) * kTurn, head[r][t]);
+        for (uint32_t p0 = static_cast<uint32_t>(tid) * 16u + HEAD * kTurn; p0 < raw[r]; p0 += 4u * kTurn) {
             u32x4_t piece[4];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                const uint32_t off = p0 + static_cast<uint32_t>(t) * 64u * kE8Waves * 16u;
-                piece[t] = __builtin_amdgcn_raw_buffer_load_b128(win, off < raw ? off : kNoStep, 0, 2);
+                const uint32_t off = p0 + static_cast<uint32_t>(t) * kTurn;
+                piece[t] = __builtin_amdgcn_raw_buffer_load_b128(win[r], off < raw[r] ? off : kNoStep, 0, 2);
             }
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const uint32_t off = p0 + static_cast<uint32_t>(t) * 64u * kE8Waves * 16u;
-                if (off < raw) {  // (a piece lies inside one padding period: they are 64 bytes and more)
-                    uint32_t *dst = reinterpret_cast<uint32_t *>(lds8 + roff[r] + off + ((off >> sh.pad[r]) << 2));
-                    dst[0] = piece[t].x; dst[1] = piece[t].y; dst[2] = piece[t].z; dst[3] = piece[t].w;
-                    // the skipped bank before a period holds a copy of the period's first dword: a field's two dwords
-                    // are adjacent in LDS wherever it starts
-                    if (off > 0u && (off & ((1u << sh.pad[r]) - 1u)) == 0u) dst[-1] = piece[t].x;
-                }
-            }
+            for (int t = 0; t < 4; ++t) park(r, p0 + static_cast<uint32_t>(t) * kTurn, piece[t]);
         }
     }
     // ---- tables -------------------------------------------------------------------------------------------------------
