@@ -432,6 +432,8 @@ int mfq_hip_nvqs_gemv_pairs(const mfq_nvqs_desc *d, const void *const *expert_we
                             int routed_input, const int32_t *ids, int T, int R, float *y, int64_t ldy, mfq_stream_t stream);
 int mfq_hip_nvqs_gemv_rows(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, const void *x, int x_dtype,
                            int64_t ldx, int M, float *y, int64_t ldy, mfq_stream_t stream);
+/* Workspace of mfq_hip_nvqs_gemm_rows for M rows: 0 for the batches that run from the bit streams (up to 16 rows, and up
+ * to 192 for the tensors whose tables and bit ranges fit the LDS), else the fp16 copies of the weights and activations. */
 size_t mfq_hip_nvqs_gemm_rows_workspace_bytes(const mfq_nvqs_desc *d, int nrows, int M);
 int mfq_hip_nvqs_gemm_rows(const mfq_nvqs_desc *d, const void *weight, int row0, int nrows, const void *x, int x_dtype,
                            int64_t ldx, int M, float *y, int64_t ldy, void *workspace, size_t workspace_bytes,
